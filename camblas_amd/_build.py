@@ -1,0 +1,90 @@
+"""Build recipe for libcamblas_hip.so (hipcc, gfx950 only) and the optional ATen tensor binding.
+
+The counterpart of the reference's scripts/build_cuda.py:68-155: the core library and the tensor
+binding land side by side in one directory (`camblas_amd/lib/`), which is where the loader looks
+when CAMBLAS_CUDA_LIBRARY is not set.
+"""
+
+import hashlib
+import json
+import os
+import subprocess
+import sys
+from concurrent.futures import ThreadPoolExecutor
+from pathlib import Path
+
+PACKAGE = Path(__file__).resolve().parent
+ROOT = PACKAGE.parent
+CSRC = PACKAGE / "csrc"
+LIB_DIR = PACKAGE / "lib"
+CORE = LIB_DIR / "libcamblas_hip.so"
+HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
+
+CORE_SOURCES = (
+    "abi.hip",
+    "planner.cpp",
+    "gemm_generic.hip",
+    "gemv_f32.hip",
+    "bgemm_tn.hip",
+    "fp8_block.hip",
+    "fusion.hip",
+    "attention_decode.hip",
+)
+
+HIP_FLAGS = [
+    "--offload-arch=gfx950",
+    "-O3",
+    "-std=c++17",
+    "-fPIC",
+    "-Wall",
+    "-Wextra",
+    "-Wno-unused-parameter",
+    # packed FP32 instructions stay disabled for all device code
+    "-Xclang",
+    "-target-feature",
+    "-Xclang",
+    "-packed-fp32-ops",
+    f"-I{ROOT / 'include'}",
+    f"-I{CSRC}",
+]
+
+
+def _run(command):
+    result = subprocess.run([str(c) for c in command], capture_output=True, text=True)
+    if result.returncode != 0:
+        sys.stderr.write(result.stdout + result.stderr)
+        raise RuntimeError("command failed: " + " ".join(str(c) for c in command))
+    return result
+
+
+def build_core(jobs=8, verbose=False):
+    """Compile every HIP translation unit for gfx950 and link libcamblas_hip.so."""
+    objects = LIB_DIR / "obj"
+    objects.mkdir(parents=True, exist_ok=True)
+
+    def compile_unit(name):
+        source = CSRC / name
+        target = objects / (source.stem + ".o")
+        language = ["-x", "hip"] if source.suffix == ".cpp" else []
+        _run([HIPCC, *HIP_FLAGS, *language, "-c", source, "-o", target])
+        if verbose:
+            print("compiled", name, flush=True)
+        return target
+
+    with ThreadPoolExecutor(max_workers=jobs) as pool:
+        built = list(pool.map(compile_unit, CORE_SOURCES))
+    _run([HIPCC, "--offload-arch=gfx950", "-shared", "-fPIC", *built, "-o", CORE,
+          "-Wl,-soname,libcamblas_hip.so"])
+    record = {
+        "library": CORE.name,
+        "sources": {
+            name: hashlib.sha256((CSRC / name).read_bytes()).hexdigest() for name in CORE_SOURCES
+        },
+        "flags": HIP_FLAGS[:-2],
+    }
+    (LIB_DIR / "build.json").write_text(json.dumps(record, indent=1))
+    return CORE
+
+
+if __name__ == "__main__":
+    print(build_core(verbose=True))

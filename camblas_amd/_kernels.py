@@ -1,0 +1,336 @@
+"""Tensor-level operators of the linear path on top of the C ABI.
+
+Host-side mirror of the reference's operator table (camblas/_kernels.py:34-59 and the binding
+functions in src/cuda/torch_bindings.cpp): same names, argument meaning and error behaviour for
+matmul / linear / rms_norm / add_rms_norm / silu_multiply / swiglu / gated_mlp / qkv_linear, plus
+the block-128 FP8 linear, rotary embedding, GQA decode attention and the decoder-layer decode step
+this backend adds. torch supplies device memory and streams only; every product and fusion runs in
+libcamblas_hip.so. Nothing here computes on the CPU or falls back to torch kernels.
+"""
+
+import ctypes as ct
+
+import torch
+
+from . import _native
+from ._native import algorithm, set_algorithm, stats, tensor_module  # noqa: F401 (re-exported)
+
+_DTYPE_CODE = {torch.float32: 0, torch.float64: 1, torch.bfloat16: 2}
+INT_MAX = 2**31 - 1
+
+
+def _require(condition, message):
+    if not condition:
+        raise RuntimeError(message)
+
+
+def _validate(tensor, reference, allow_bfloat16=True):
+    # ref: src/cuda/torch_bindings.cpp:122-138
+    allowed = (torch.float32, torch.float64) + ((torch.bfloat16,) if allow_bfloat16 else ())
+    _require(
+        tensor.is_cuda and tensor.dtype in allowed,
+        "CAMBLAS matmul requires CUDA FP32, FP64 or BF16 tensors"
+        if allow_bfloat16
+        else "CAMBLAS CUDA requires CUDA FP32 or FP64 tensors",
+    )
+    _require(
+        tensor.device == reference.device and tensor.dtype == reference.dtype,
+        "All operands must have the same device and dtype",
+    )
+    _require(all(size <= INT_MAX for size in tensor.shape), "LP64 dimension overflow")
+    _require(all(stride <= INT_MAX for stride in tensor.stride()), "LP64 stride overflow")
+
+
+def _operand(tensor):
+    """Row-major 2-D tensor -> (tensor, transpose flag, leading dimension) of the column-major view.
+
+    ref: src/cuda/torch_bindings.cpp:146-153
+    """
+    rows, columns = tensor.shape
+    stride0, stride1 = tensor.stride()
+    if stride1 == 1 and stride0 >= max(1, columns):
+        return tensor, b"N", stride0
+    if stride0 == 1 and stride1 >= max(1, rows):
+        return tensor, b"T", stride1
+    return tensor.contiguous(), b"N", max(1, columns)
+
+
+def _pointer(tensor):
+    return ct.c_void_p(tensor.data_ptr()) if tensor is not None else None
+
+
+def matmul(a, b, out=None, alpha=1.0, beta=0.0):
+    """alpha * a @ b + beta * out for 2-D FP32 or BF16 device tensors.
+
+    ref: src/cuda/torch_bindings.cpp:155-199 (row-major operands become the swapped column-major
+    call). FP64 is rejected by the library with its own message.
+    """
+    _validate(a, a)
+    _validate(b, a)
+    _require(
+        a.dim() == 2 and b.dim() == 2 and a.shape[1] == b.shape[0],
+        "matmul requires compatible rank-two operands",
+    )
+    m, k = a.shape
+    n = b.shape[1]
+    if out is not None:
+        _validate(out, a)
+        _require(
+            out.dim() == 2 and out.shape[0] == m and out.shape[1] == n and out.is_contiguous(),
+            "Output must have the product shape and contiguous row storage",
+        )
+        _require(
+            out.untyped_storage().data_ptr() != a.untyped_storage().data_ptr()
+            and out.untyped_storage().data_ptr() != b.untyped_storage().data_ptr(),
+            "GEMM output cannot alias an input",
+        )
+        c = out
+    else:
+        _require(beta == 0, "beta requires an existing output tensor")
+        c = torch.empty((m, n), dtype=a.dtype, device=a.device)
+    left, left_trans, left_ld = _operand(b)
+    right, right_trans, right_ld = _operand(a)
+    native = _native.context(a.device)
+    name = {torch.float32: "sgemm", torch.float64: "dgemm", torch.bfloat16: "bgemm"}[a.dtype]
+    scalar = ct.c_double if a.dtype == torch.float64 else ct.c_float
+    with torch.cuda.device(a.device):
+        native.call(
+            name, left_trans, right_trans, n, m, k, scalar(alpha), _pointer(left), left_ld,
+            _pointer(right), right_ld, scalar(beta), _pointer(c), max(1, n),
+        )
+    return c
+
+
+def linear(x, weight, bias=None):
+    """x @ weight.T (+ bias) with x [..., inputs] and weight [outputs, inputs].
+
+    ref: src/cuda/torch_bindings.cpp:244-270. The bias add is a torch elementwise op there as well.
+    """
+    _validate(x, x)
+    _validate(weight, x)
+    _require(
+        x.dim() >= 1 and weight.dim() == 2 and x.shape[-1] == weight.shape[1],
+        "linear requires matching input and [outputs, inputs] weight dimensions",
+    )
+    rows = 1
+    for size in x.shape[:-1]:
+        rows *= size
+    _require(rows <= INT_MAX, "LP64 flattened row overflow")
+    if bias is not None:
+        _validate(bias, x)
+        _require(
+            bias.dim() == 1 and bias.shape[0] == weight.shape[0],
+            "linear bias must have the output width",
+        )
+    result = matmul(x.reshape(rows, x.shape[-1]), weight.t())
+    if bias is not None:
+        result = result.add(bias)
+    return result.reshape(*x.shape[:-1], weight.shape[0])
+
+
+def addmm(bias, a, b, beta=1.0, alpha=1.0):
+    """beta * bias + alpha * a @ b; the bias is expanded and cloned, then updated in place.
+
+    ref: src/cuda/torch_backend.cuh:59-71
+    """
+    m, n = a.shape[0], b.shape[1]
+    if beta == 0:
+        return matmul(a, b, None, alpha, 0.0)
+    out = bias.expand(m, n).clone(memory_format=torch.contiguous_format)
+    return matmul(a, b, out, alpha, beta)
+
+
+def _elementwise_pair(gate, up, name):
+    _require(
+        gate.is_cuda and gate.dtype in (torch.float32, torch.bfloat16),
+        f"{name} requires CUDA FP32 or BF16 tensors",
+    )
+    _require(
+        up.device == gate.device and up.dtype == gate.dtype and up.shape == gate.shape,
+        f"{name} operands must share device, dtype and shape",
+    )
+    _require(gate.is_contiguous() and up.is_contiguous(), f"{name} operands must be contiguous")
+
+
+def silu_multiply(gate, up, out=None):
+    """round(silu(gate)) * up with storage rounding in between (ref: inference_fusion.cuh:19-28)."""
+    _elementwise_pair(gate, up, "silu_multiply")
+    out = torch.empty_like(gate) if out is None else out
+    _native.context(gate.device).call(
+        "silu_multiply", _DTYPE_CODE[gate.dtype], gate.numel(), _pointer(gate), _pointer(up),
+        _pointer(out),
+    )
+    return out
+
+
+def swiglu(gate, up, limit=0.0, routing=None, out=None):
+    """silu(gate) * up in FP32 with optional clamp and per-row routing (ref: :30-51)."""
+    _elementwise_pair(gate, up, "swiglu")
+    out = torch.empty_like(gate) if out is None else out
+    width = gate.shape[-1] if gate.dim() else 1
+    if routing is not None:
+        _require(
+            routing.dtype == torch.float32 and routing.is_contiguous()
+            and routing.numel() * width == gate.numel(),
+            "routing must hold one FP32 value per row",
+        )
+    _native.context(gate.device).call(
+        "swiglu", _DTYPE_CODE[gate.dtype], gate.numel(), max(1, width), ct.c_float(limit),
+        _pointer(gate), _pointer(up), _pointer(routing), _pointer(out),
+    )
+    return out
+
+
+def rms_norm(x, weight, epsilon=1e-6, round_before_weight=True):
+    """RMS normalisation over the last dimension (ref: src/cuda/torch_bindings.cpp:602-673)."""
+    _require(x.is_cuda and x.dtype in (torch.float32, torch.bfloat16), "rms_norm needs FP32/BF16")
+    _require(x.is_contiguous() and weight.is_contiguous(), "rms_norm operands must be contiguous")
+    width = x.shape[-1]
+    _require(weight.numel() == width, "rms_norm weight must match the last dimension")
+    rows = x.numel() // max(1, width)
+    out = torch.empty_like(x)
+    _native.context(x.device).call(
+        "add_rms_norm_rows", _DTYPE_CODE[x.dtype], _DTYPE_CODE[weight.dtype], rows, width,
+        ct.c_float(epsilon), int(round_before_weight), _pointer(x), None, _pointer(weight), None,
+        _pointer(out),
+    )
+    return out
+
+
+def add_rms_norm(x, residual, weight, epsilon=1e-6, round_before_weight=True):
+    """(x + residual rounded to storage, its RMS norm) (ref: torch_bindings.cpp:675-701)."""
+    _require(x.is_cuda and x.dtype in (torch.float32, torch.bfloat16), "add_rms_norm needs FP32/BF16")
+    _require(
+        residual.shape == x.shape and residual.dtype == x.dtype and residual.device == x.device,
+        "residual must match the input",
+    )
+    _require(
+        x.is_contiguous() and residual.is_contiguous() and weight.is_contiguous(),
+        "add_rms_norm operands must be contiguous",
+    )
+    width = x.shape[-1]
+    _require(weight.numel() == width, "add_rms_norm weight must match the last dimension")
+    rows = x.numel() // max(1, width)
+    added, out = torch.empty_like(x), torch.empty_like(x)
+    _native.context(x.device).call(
+        "add_rms_norm_rows", _DTYPE_CODE[x.dtype], _DTYPE_CODE[weight.dtype], rows, width,
+        ct.c_float(epsilon), int(round_before_weight), _pointer(x), _pointer(residual),
+        _pointer(weight), _pointer(added), _pointer(out),
+    )
+    return added, out
+
+
+def gated_mlp(x, gate_weight, up_weight, down_weight):
+    """down(silu_multiply(gate(x), up(x))) (ref: src/cuda/torch_bindings.cpp:703-723)."""
+    gate = linear(x, gate_weight)
+    up = linear(x, up_weight)
+    silu_multiply(gate, up, out=gate)
+    return linear(gate, down_weight)
+
+
+def qkv_linear(x, q_weight, k_weight, v_weight):
+    """Three independent linears with distinct outputs (ref: torch_bindings.cpp:725-736)."""
+    return linear(x, q_weight), linear(x, k_weight), linear(x, v_weight)
+
+
+def fp8_block_matmul(a, a_scale, weight, weight_scale, out=None):
+    """E4M3fn a [M,K] x weight [N,K]^T with 1x128 / 128x128 FP32 scales -> BF16 [M,N]."""
+    _require(a.dtype == torch.float8_e4m3fn and weight.dtype == torch.float8_e4m3fn,
+             "fp8_block_matmul requires float8_e4m3fn operands")
+    _require(a.is_cuda and a.is_contiguous() and weight.is_contiguous(), "contiguous device operands")
+    rows, inner = a.shape
+    outputs = weight.shape[0]
+    groups = inner // 128
+    _require(weight.shape[1] == inner and inner % 128 == 0, "inner must be a multiple of 128")
+    _require(
+        a_scale.dtype == torch.float32 and tuple(a_scale.shape) == (rows, groups)
+        and a_scale.is_contiguous(),
+        "activation scales must be FP32 [rows, inner/128]",
+    )
+    _require(
+        weight_scale.dtype == torch.float32
+        and tuple(weight_scale.shape) == ((outputs + 127) // 128, groups)
+        and weight_scale.is_contiguous(),
+        "weight scales must be FP32 [ceil(outputs/128), inner/128]",
+    )
+    out = torch.empty((rows, outputs), dtype=torch.bfloat16, device=a.device) if out is None else out
+    _native.context(a.device).call(
+        "fp8_block_matmul", rows, outputs, inner, _pointer(a), _pointer(a_scale), _pointer(weight),
+        _pointer(weight_scale), _pointer(out),
+    )
+    return out
+
+
+def fp8_quantise_1x128(x):
+    """BF16 [M,K] -> (E4M3fn [M,K], FP32 scales [M,K/128]) (ref: camblas/_hopper.py:82-98)."""
+    _require(x.dtype == torch.bfloat16 and x.is_cuda and x.is_contiguous() and x.dim() == 2,
+             "fp8_quantise_1x128 requires a contiguous 2-D BF16 device tensor")
+    rows, inner = x.shape
+    q = torch.empty((rows, inner), dtype=torch.float8_e4m3fn, device=x.device)
+    scale = torch.empty((rows, inner // 128), dtype=torch.float32, device=x.device)
+    _native.context(x.device).call(
+        "fp8_quantise_1x128", rows, inner, _pointer(x), _pointer(q), _pointer(scale)
+    )
+    return q, scale
+
+
+def fp8_block_linear(x, weight, weight_scale):
+    """BF16 activations quantised on the fly, then the block-scaled product."""
+    q, scale = fp8_quantise_1x128(x.reshape(-1, x.shape[-1]))
+    out = fp8_block_matmul(q, scale, weight, weight_scale)
+    return out.reshape(*x.shape[:-1], weight.shape[0])
+
+
+def rope(x, positions, theta=500000.0):
+    """In-place rotate-half rotary embedding on BF16 x [tokens, heads, dim]."""
+    _require(x.dtype == torch.bfloat16 and x.is_cuda and x.dim() == 3, "rope needs BF16 [T,H,D]")
+    _require(x.stride(2) == 1 and x.stride(1) == x.shape[2], "rope needs dense heads")
+    _require(positions.dtype == torch.int32 and positions.numel() == x.shape[0], "int32 positions")
+    tokens, heads, dim = x.shape
+    _native.context(x.device).call(
+        "rope", tokens, heads, dim, x.stride(0), ct.c_float(theta), _pointer(positions), _pointer(x)
+    )
+    return x
+
+
+def gqa_decode_attention(q, k_cache, v_cache, lengths=None, scale=None):
+    """One-token-per-sequence grouped-query attention against BF16 caches [B, C, Hkv, 128]."""
+    _require(q.dtype == torch.bfloat16 and q.is_cuda and q.dim() == 3, "q must be BF16 [B,H,D]")
+    _require(q.stride(2) == 1 and q.stride(1) == q.shape[2], "q heads must be dense")
+    _require(k_cache.is_contiguous() and v_cache.is_contiguous() and k_cache.shape == v_cache.shape,
+             "caches must be contiguous and equal-shaped")
+    batch, q_heads, dim = q.shape
+    _, context_length, kv_heads, _ = k_cache.shape
+    scale = dim**-0.5 if scale is None else scale
+    out = torch.empty((batch, q_heads, dim), dtype=torch.bfloat16, device=q.device)
+    _native.context(q.device).call(
+        "gqa_decode_attention", batch, q_heads, kv_heads, dim, context_length, _pointer(lengths),
+        ct.c_float(scale), _pointer(q), q.stride(0), _pointer(k_cache), _pointer(v_cache),
+        _pointer(out),
+    )
+    return out
+
+
+def decoder_layer_decode(hidden, residual, weights, k_cache, v_cache, positions, *, q_heads,
+                         kv_heads, head_dim=128, epsilon=1e-5, theta=500000.0):
+    """One Llama-shaped decoder layer for one new token per sequence.
+
+    residual-add + RMSNorm -> fused QKV linear -> RoPE on q and k -> cache append -> GQA decode
+    attention -> o-proj -> residual-add + RMSNorm -> SwiGLU MLP. Returns (mlp output, residual).
+    `weights` holds input_norm, qkv [ (Hq+2Hkv)*D, hidden ], o, post_norm, gate, up, down.
+    `positions` (int32 [batch]) is the cache slot the new token is written to.
+    """
+    batch = hidden.shape[0]
+    residual, normed = add_rms_norm(hidden, residual, weights["input_norm"], epsilon)
+    qkv = linear(normed, weights["qkv"]).view(batch, q_heads + 2 * kv_heads, head_dim)
+    rope(qkv[:, : q_heads + kv_heads], positions, theta)
+    q = qkv[:, :q_heads]
+    index = positions.long()
+    rows = torch.arange(batch, device=hidden.device)
+    k_cache[rows, index] = qkv[:, q_heads : q_heads + kv_heads]
+    v_cache[rows, index] = qkv[:, q_heads + kv_heads :]
+    lengths = (positions + 1).to(torch.int32)
+    attended = gqa_decode_attention(q, k_cache, v_cache, lengths)
+    projected = linear(attended.view(batch, q_heads * head_dim), weights["o"])
+    residual, normed = add_rms_norm(projected, residual, weights["post_norm"], epsilon)
+    return gated_mlp(normed, weights["gate"], weights["up"], weights["down"]), residual

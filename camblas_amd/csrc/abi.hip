@@ -1,0 +1,643 @@
+// extern "C" surface of libcamblas_hip.so: context lifetime, argument validation in the
+// reference's order, planning and dispatch. No kernel lives here.
+#include "common.hpp"
+
+#include <algorithm>
+#include <cmath>
+#include <climits>
+#include <cstring>
+#include <exception>
+#include <new>
+
+namespace camblas_hip
+{
+namespace
+{
+thread_local char creation_error[256] = "";
+}
+
+int fail(camblas_cuda_context *context, const char *operation, int code)
+{
+    char *message = context ? context->error : creation_error;
+    std::snprintf(message, 256, "%s failed (status %d)", operation, code);
+    return code > 0 ? -code : -1;
+}
+
+hipError_t reserve_scratch(camblas_cuda_context *context, size_t bytes)
+{
+    if (bytes <= context->scratch_bytes)
+        return hipSuccess;
+    hipStreamCaptureStatus capture = hipStreamCaptureStatusNone;
+    hipStreamIsCapturing(context->stream, &capture);
+    if (capture != hipStreamCaptureStatusNone)
+        return hipErrorStreamCaptureUnsupported;
+    size_t wanted = std::max(bytes, context->scratch_bytes * 2);
+    wanted = (wanted + 255) & ~size_t(255);
+    void *fresh = nullptr;
+    hipError_t status = hipMalloc(&fresh, wanted);
+    if (status != hipSuccess) {
+        (void)hipGetLastError();
+        return status;
+    }
+    // Earlier launches (possibly captured) may still reference the old arena.
+    if (context->scratch)
+        context->retired.push_back(context->scratch);
+    context->scratch = fresh;
+    context->scratch_bytes = wanted;
+    return hipSuccess;
+}
+
+namespace
+{
+// Activates the context's device for one call and restores the caller's (ref: backend.cu:913-932).
+class DeviceScope
+{
+    int previous = -1;
+    bool changed = false;
+
+  public:
+    hipError_t status;
+    explicit DeviceScope(int device) : status(hipGetDevice(&previous))
+    {
+        if (status == hipSuccess && previous != device) {
+            status = hipSetDevice(device);
+            changed = status == hipSuccess;
+        }
+    }
+    ~DeviceScope()
+    {
+        if (changed)
+            (void)hipSetDevice(previous);
+    }
+};
+
+// ref: backend.cu:934-951
+template <typename Function> int execute(camblas_cuda_context *context, Function function)
+{
+    if (!context)
+        return fail(nullptr, "missing context", 1);
+    DeviceScope device(context->device);
+    if (device.status != hipSuccess)
+        return fail(context, "activate device", device.status);
+    try {
+        return function();
+    } catch (const std::bad_alloc &) {
+        return fail(context, "host allocation", 2);
+    } catch (const std::exception &error) {
+        std::snprintf(context->error, sizeof(context->error), "host exception: %s", error.what());
+        return -1;
+    } catch (...) {
+        return fail(context, "unexpected host exception", 1);
+    }
+}
+
+bool is_n(char t) { return t == 'N' || t == 'n'; }
+bool is_t(char t) { return t == 'T' || t == 't'; }
+bool aligned(const void *p, size_t bytes) { return reinterpret_cast<uintptr_t>(p) % bytes == 0; }
+
+int unsupported(camblas_cuda_context *context, const char *what)
+{
+    if (!context)
+        return fail(nullptr, "missing context", 1);
+    std::snprintf(context->error, sizeof(context->error),
+                  "%s is not provided by the HIP linear backend", what);
+    return -1;
+}
+
+// Column-major GEMM shared by FP32/FP64 (ref: backend.cu:786-866): validation order, no-op and
+// beta-only cases, alias rejection, then the planner's choice.
+template <typename T, typename Scale, typename Launch>
+int gemm(camblas_cuda_context *context, const char *type_name, char trans_a, char trans_b, int m,
+         int n, int k, T alpha, const T *a, int lda, const T *b, int ldb, T beta, T *c, int ldc,
+         Scale scale, Launch launch)
+{
+    (void)type_name;
+    bool na = is_n(trans_a), ta = is_t(trans_a), nb = is_n(trans_b), tb = is_t(trans_b);
+    if ((!na && !ta) || (!nb && !tb) || m < 0 || n < 0 || k < 0 || lda < 1 || ldb < 1 || ldc < 1)
+        return fail(context, "invalid GEMM arguments", 1);
+    if (m == 0 || n == 0)
+        return 0;
+    if (!c || lda < std::max(1, na ? m : k) || ldb < std::max(1, nb ? k : n) || ldc < m)
+        return fail(context, "invalid device pointer or leading dimension", 1);
+    if (alpha == T(0) || k == 0) {
+        if (beta == T(1))
+            return 0;
+        hipError_t error = scale();
+        return error == hipSuccess ? 0 : fail(context, "scale output", error);
+    }
+    if (!a || !b || a == c || b == c)
+        return fail(context, "missing or aliased GEMM operand", 1);
+    return launch(ta, tb);
+}
+} // namespace
+} // namespace camblas_hip
+
+using namespace camblas_hip;
+
+extern "C" int camblas_cuda_create(int device, void *stream, camblas_cuda_context **out)
+{
+    if (!out)
+        return fail(nullptr, "missing context output", 1);
+    *out = nullptr;
+    DeviceScope scope(device);
+    if (scope.status != hipSuccess)
+        return fail(nullptr, "activate device", scope.status);
+    auto *context = new (std::nothrow) camblas_cuda_context;
+    if (!context)
+        return fail(nullptr, "context allocation", 2);
+    context->device = device;
+    context->stream = static_cast<hipStream_t>(stream);
+    hipDeviceProp_t properties;
+    hipError_t status = hipGetDeviceProperties(&properties, device);
+    if (status != hipSuccess) {
+        delete context;
+        return fail(nullptr, "device properties", status);
+    }
+    if (std::strncmp(properties.gcnArchName, "gfx950", 6) != 0) {
+        delete context;
+        std::snprintf(creation_error, sizeof(creation_error),
+                      "libcamblas_hip is built for gfx950 only; device %d is %s", device,
+                      properties.gcnArchName);
+        return -1;
+    }
+    context->compute_units = properties.multiProcessorCount;
+    *out = context;
+    return 0;
+}
+
+extern "C" int camblas_cuda_destroy(camblas_cuda_context *context)
+{
+    if (!context)
+        return 0;
+    DeviceScope scope(context->device);
+    if (scope.status != hipSuccess)
+        return fail(context, "activate device for destruction", scope.status);
+    hipError_t error = hipStreamSynchronize(context->stream);
+    if (context->scratch)
+        (void)hipFree(context->scratch);
+    for (void *allocation : context->retired)
+        (void)hipFree(allocation);
+    delete context;
+    return error == hipSuccess ? 0 : fail(nullptr, "stream completion during destruction", error);
+}
+
+extern "C" const char *camblas_cuda_error(const camblas_cuda_context *context)
+{
+    return context ? context->error : creation_error;
+}
+
+extern "C" int camblas_cuda_set_algorithm(camblas_cuda_context *context, int algorithm)
+{
+    if (!context || algorithm < CAMBLAS_CUDA_AUTO || algorithm > CAMBLAS_CUDA_STRASSEN_FOUR)
+        return fail(context, "invalid algorithm", 1);
+    context->algorithm = algorithm;
+    return 0;
+}
+
+extern "C" int camblas_cuda_sgemm(camblas_cuda_context *context, char ta, char tb, int m, int n,
+                                  int k, float alpha, const float *a, int lda, const float *b,
+                                  int ldb, float beta, float *c, int ldc)
+{
+    return execute(context, [&] {
+        return gemm<float>(
+            context, "FP32", ta, tb, m, n, k, alpha, a, lda, b, ldb, beta, c, ldc,
+            [&] { return launch_scale_f32(context->stream, m, n, beta, c, ldc); },
+            [&](bool trans_a, bool trans_b) {
+                Plan plan = make_plan(0, context->algorithm, trans_a, trans_b, m, n, k, lda, ldb,
+                                      ldc, aligned(a, 16) && aligned(b, 16), context->compute_units);
+                context->counts[plan.counter]++;
+                hipError_t error;
+                if (plan.family == FAMILY_GEMV_F32) {
+                    error = launch_gemv_f32(context->stream, m, k, alpha, a, lda, b, beta, c);
+                    return error == hipSuccess ? 0 : fail(context, "FP32 native GEMV", error);
+                }
+                error = launch_generic_f32(context->stream, trans_a, trans_b, m, n, k, alpha, a,
+                                           lda, b, ldb, beta, c, ldc);
+                return error == hipSuccess ? 0 : fail(context, "classical GEMM", error);
+            });
+    });
+}
+
+extern "C" int camblas_cuda_dgemm(camblas_cuda_context *context, char ta, char tb, int m, int n,
+                                  int k, double alpha, const double *a, int lda, const double *b,
+                                  int ldb, double beta, double *c, int ldc)
+{
+    (void)ta, (void)tb, (void)m, (void)n, (void)k, (void)alpha, (void)a, (void)lda, (void)b;
+    (void)ldb, (void)beta, (void)c, (void)ldc;
+    return unsupported(context, "FP64 GEMM");
+}
+
+extern "C" int camblas_cuda_bgemm(camblas_cuda_context *context, char trans_a, char trans_b, int m,
+                                  int n, int k, float alpha, const void *a, int lda, const void *b,
+                                  int ldb, float beta, void *c, int ldc)
+{
+    // ref: src/cuda/bfloat16.cuh:11-57
+    return execute(context, [&] {
+        bool na = is_n(trans_a), ta = is_t(trans_a), nb = is_n(trans_b), tb = is_t(trans_b);
+        if ((!na && !ta) || (!nb && !tb) || m < 0 || n < 0 || k < 0 || lda < 1 || ldb < 1 ||
+            ldc < 1)
+            return fail(context, "invalid BF16 GEMM arguments", 1);
+        if (m == 0 || n == 0)
+            return 0;
+        if (!c || lda < std::max(1, na ? m : k) || ldb < std::max(1, nb ? k : n) || ldc < m)
+            return fail(context, "invalid BF16 pointer or leading dimension", 1);
+        if (alpha == 0 || k == 0) {
+            if (beta == 1)
+                return 0;
+            hipError_t error = launch_scale_bf16(context->stream, m, n, beta, c, ldc);
+            return error == hipSuccess ? 0 : fail(context, "scale BF16 output", error);
+        }
+        if (!a || !b || a == c || b == c)
+            return fail(context, "missing or aliased BF16 GEMM operand", 1);
+        Plan plan = make_plan(2, context->algorithm, ta, tb, m, n, k, lda, ldb, ldc,
+                              aligned(a, 16) && aligned(b, 16), context->compute_units);
+        if (plan.family == FAMILY_MFMA_TN && context->override_kernel >= 0) {
+            plan.kernel = context->override_kernel;
+            if (context->override_split > 0)
+                plan.split_k = context->override_split;
+        }
+        if (plan.family == FAMILY_MFMA_TN) {
+            float *partials = nullptr;
+            if (plan.split_k > 1) {
+                hipError_t grown =
+                    reserve_scratch(context, size_t(plan.split_k) * size_t(m) * size_t(n) * 4);
+                if (grown != hipSuccess) {
+                    // cannot hold the partials (allocation failure or capture in progress):
+                    // run unsplit, and if even that is impossible use the generic kernel
+                    context->counts[5]++;
+                    plan.split_k = 1;
+                } else {
+                    partials = static_cast<float *>(context->scratch);
+                }
+            }
+            context->counts[plan.counter]++;
+            hipError_t error = launch_bgemm_tn(context->stream, plan.kernel, plan.split_k, m, n, k,
+                                               alpha, a, lda, b, ldb, beta, c, ldc, partials);
+            return error == hipSuccess ? 0 : fail(context, "BF16 MFMA GEMM", error);
+        }
+        context->counts[0]++;
+        hipError_t error = launch_generic_bf16(context->stream, ta, tb, m, n, k, alpha, a, lda, b,
+                                               ldb, beta, c, ldc);
+        return error == hipSuccess ? 0 : fail(context, "BF16 GEMM", error);
+    });
+}
+
+extern "C" int camblas_cuda_affine(camblas_cuda_context *context, int, int, int, int, const void *,
+                                   const void *, const void *, int, void *)
+{
+    return unsupported(context, "affine");
+}
+
+extern "C" int camblas_cuda_mlp(camblas_cuda_context *context, int, int, int, int, int,
+                                const void *, const void *, const void *, const void *,
+                                const void *, void *, void *)
+{
+    return unsupported(context, "MLP");
+}
+
+extern "C" int camblas_cuda_attention(camblas_cuda_context *context, int, int, int, int, int, double,
+                                      const void *, const void *, const void *, void *)
+{
+    return unsupported(context, "dense single-head attention");
+}
+
+extern "C" int camblas_cuda_mlp_backward(camblas_cuda_context *context, int, int, int, int, int,
+                                         const void *, const void *, const void *, const void *,
+                                         const void *, void *, void *, void *, void *, void *,
+                                         void *)
+{
+    return unsupported(context, "MLP backward");
+}
+
+extern "C" int camblas_cuda_silu_multiply(camblas_cuda_context *context, int dtype, uint64_t count,
+                                          const void *gate, const void *up, void *output)
+{
+    // ref: backend.cu:1119-1133
+    return execute(context, [&] {
+        if (dtype != 0 && dtype != 2)
+            return fail(context, "unsupported SiLU dtype", 1);
+        if (!count)
+            return 0;
+        if (!gate || !up || !output || count > SIZE_MAX / (dtype == 0 ? 4 : 2))
+            return fail(context, "invalid SiLU operands or length", 1);
+        hipError_t error = launch_silu_multiply(context->stream, dtype, count, gate, up, output);
+        return error == hipSuccess ? 0 : fail(context, "SiLU multiply", error);
+    });
+}
+
+extern "C" int camblas_cuda_swiglu(camblas_cuda_context *context, int dtype, uint64_t count,
+                                   int width, float limit, const void *gate, const void *up,
+                                   const float *routing, void *output)
+{
+    // ref: backend.cu:1135-1163
+    return execute(context, [&] {
+        if ((dtype != 0 && dtype != 2) || width <= 0 || count % unsigned(width) ||
+            !std::isfinite(limit) || limit < 0 || count > SIZE_MAX / (dtype == 0 ? 4 : 2))
+            return fail(context, "invalid SwiGLU dimensions or clipping limit", 1);
+        if (!count)
+            return 0;
+        unsigned alignment = dtype == 0 ? 4 : 2;
+        if (!gate || !up || !output || !aligned(gate, alignment) || !aligned(up, alignment) ||
+            !aligned(output, alignment) || (routing && (!aligned(routing, 4) || output == routing)))
+            return fail(context, "invalid SwiGLU buffers", 1);
+        hipError_t error =
+            launch_swiglu(context->stream, dtype, count, width, limit, gate, up, routing, output);
+        return error == hipSuccess ? 0 : fail(context, "SwiGLU", error);
+    });
+}
+
+extern "C" int camblas_cuda_rms_norm_decode(camblas_cuda_context *context, int dtype,
+                                            int weight_dtype, int width, float epsilon,
+                                            int round_before_weight, int descending,
+                                            const void *input, const void *weight, void *output)
+{
+    // ref: backend.cu:1363-1396
+    return execute(context, [&] {
+        if ((dtype != 0 && dtype != 2) || (weight_dtype != 0 && weight_dtype != 2) ||
+            (dtype == 0 && weight_dtype != 0) || width < 2048 || width > 65536 || width % 4 ||
+            (round_before_weight != 0 && round_before_weight != 1) ||
+            (descending != 0 && descending != 1) || !std::isfinite(epsilon) || epsilon < 0 ||
+            !input || !weight || !output || output == input || output == weight ||
+            !aligned(input, dtype == 0 ? 4 : 2) || !aligned(weight, weight_dtype == 0 ? 4 : 2) ||
+            !aligned(output, dtype == 0 ? 4 : 2))
+            return fail(context, "invalid decode RMS arguments", 1);
+        hipError_t error =
+            launch_rms_rows(context->stream, dtype, weight_dtype, 1, width, epsilon,
+                            round_before_weight != 0, input, nullptr, weight, nullptr, output);
+        return error == hipSuccess ? 0 : fail(context, "decode RMS normalisation", error);
+    });
+}
+
+extern "C" int camblas_cuda_add_rms_norm(camblas_cuda_context *context, int dtype, int width,
+                                         float epsilon, const void *input, const void *residual,
+                                         const void *weight, void *added, void *output)
+{
+    // ref: backend.cu:1398-1421
+    return execute(context, [&] {
+        if ((dtype != 0 && dtype != 2) || width < 2048 || width > 65536 || width % 4 ||
+            !std::isfinite(epsilon) || epsilon < 0 || !input || !residual || !weight || !added ||
+            !output || added == output || added == input || added == residual || added == weight ||
+            output == input || output == residual || output == weight)
+            return fail(context, "invalid residual RMS arguments", 1);
+        hipError_t error = launch_rms_rows(context->stream, dtype, dtype, 1, width, epsilon, true,
+                                           input, residual, weight, added, output);
+        return error == hipSuccess ? 0 : fail(context, "residual RMS normalisation", error);
+    });
+}
+
+extern "C" int camblas_cuda_add_rms_norm_rows(camblas_cuda_context *context, int dtype,
+                                              int weight_dtype, int rows, int width, float epsilon,
+                                              int round_before_weight, const void *input,
+                                              const void *residual, const void *weight, void *added,
+                                              void *output)
+{
+    return execute(context, [&] {
+        if ((dtype != 0 && dtype != 2) || (weight_dtype != 0 && weight_dtype != 2) ||
+            (dtype == 0 && weight_dtype != 0) || rows < 0 || width < 0 ||
+            (round_before_weight != 0 && round_before_weight != 1) || !std::isfinite(epsilon) ||
+            epsilon < 0)
+            return fail(context, "invalid residual RMS rows arguments", 1);
+        if (!rows || !width)
+            return 0;
+        if (!input || !weight || !output || output == weight || output == input ||
+            (residual && (!added || added == output || added == input || added == residual ||
+                          added == weight || output == residual)))
+            return fail(context, "invalid residual RMS rows operands", 1);
+        hipError_t error =
+            launch_rms_rows(context->stream, dtype, weight_dtype, rows, width, epsilon,
+                            round_before_weight != 0, input, residual, weight, added, output);
+        return error == hipSuccess ? 0 : fail(context, "residual RMS normalisation", error);
+    });
+}
+
+extern "C" int camblas_cuda_rms_norm(camblas_cuda_context *context, int dtype, int rows, int width,
+                                     float epsilon, const void *input, const void *weight,
+                                     void *output)
+{
+    // ref: backend.cu:1423-1439. In-place output==input is allowed there; each element is read
+    // before it is written by the same thread here as well.
+    return execute(context, [&] {
+        if ((dtype != 0 && dtype != 2) || rows < 0 || width < 0 || !std::isfinite(epsilon) ||
+            epsilon < 0)
+            return fail(context, "invalid RMS normalisation dimensions, dtype or epsilon", 1);
+        if (!rows || !width)
+            return 0;
+        if (!input || !weight || !output || output == weight)
+            return fail(context, "invalid RMS normalisation operands", 1);
+        hipError_t error = launch_rms_rows(context->stream, dtype, dtype, rows, width, epsilon, true,
+                                           input, nullptr, weight, nullptr, output);
+        return error == hipSuccess ? 0 : fail(context, "RMS normalisation", error);
+    });
+}
+
+extern "C" int camblas_cuda_bfloat16_square(camblas_cuda_context *context, uint64_t count,
+                                            const void *input, float *output)
+{
+    return execute(context, [&] {
+        if (!count)
+            return 0;
+        if (!input || !output || count > SIZE_MAX / sizeof(float))
+            return fail(context, "invalid BF16 square operands", 1);
+        hipError_t error = launch_bf16_square(context->stream, count, input, output);
+        return error == hipSuccess ? 0 : fail(context, "BF16 squares", error);
+    });
+}
+
+extern "C" int camblas_cuda_rms_scale(camblas_cuda_context *context, int dtype, uint64_t count,
+                                      int width, float epsilon, const void *input,
+                                      const void *weight, const float *means, void *output)
+{
+    // ref: backend.cu:1457-1475
+    return execute(context, [&] {
+        if ((dtype != 0 && dtype != 2) || width < 0 || !std::isfinite(epsilon) || epsilon < 0)
+            return fail(context, "invalid RMS scale dimensions, dtype or epsilon", 1);
+        if (!count)
+            return 0;
+        if (!width || count % width || count > SIZE_MAX / sizeof(float) || !input || !weight ||
+            !means || !output || output == weight)
+            return fail(context, "invalid RMS scale operands", 1);
+        hipError_t error = launch_rms_scale(context->stream, dtype, count, width, epsilon, input,
+                                            weight, means, output);
+        return error == hipSuccess ? 0 : fail(context, "RMS scaling", error);
+    });
+}
+
+extern "C" int camblas_cuda_stats(const camblas_cuda_context *context, uint64_t *counts, int length)
+{
+    if (!context || !counts || (length != 6 && length != 8))
+        return fail(nullptr, "invalid stats output", 1);
+    for (int i = 0; i < length; ++i)
+        counts[i] = context->counts[i].load(std::memory_order_relaxed);
+    return 0;
+}
+
+extern "C" int camblas_cuda_reset_stats(camblas_cuda_context *context)
+{
+    if (!context)
+        return fail(nullptr, "missing context", 1);
+    for (auto &count : context->counts)
+        count.store(0, std::memory_order_relaxed);
+    return 0;
+}
+
+// ------------------------------------------------------------------ extensions
+
+extern "C" int camblas_cuda_fp8_block_matmul(camblas_cuda_context *context, int rows, int outputs,
+                                             int inner, const void *a, const float *a_scale,
+                                             const void *w, const float *w_scale, void *out)
+{
+    return execute(context, [&] {
+        if (rows < 0 || rows > 65535 || outputs < 1 || inner < 128 || inner % 128)
+            return fail(context, "invalid FP8 block matrix dimensions", 1);
+        if (!rows)
+            return 0;
+        if (!a || !a_scale || !w || !w_scale || !out || !aligned(a, 16) || !aligned(w, 16) ||
+            !aligned(a_scale, 4) || !aligned(w_scale, 4) || !aligned(out, 2) || out == a ||
+            out == w || out == (const void *)a_scale || out == (const void *)w_scale)
+            return fail(context, "invalid FP8 block matrix buffers", 1);
+        Plan plan = make_plan(3, context->algorithm, true, false, outputs, rows, inner, inner, inner,
+                              outputs, true, context->compute_units);
+        if (context->override_kernel >= 0) {
+            plan.kernel = context->override_kernel;
+            if (context->override_split > 0)
+                plan.split_k = context->override_split;
+        }
+        float *partials = nullptr;
+        if (plan.split_k > 1) {
+            hipError_t grown = reserve_scratch(
+                context, size_t(plan.split_k) * size_t(rows) * size_t(outputs) * 4);
+            if (grown != hipSuccess) {
+                context->counts[5]++;
+                plan.split_k = 1;
+            } else {
+                partials = static_cast<float *>(context->scratch);
+            }
+        }
+        context->counts[plan.counter]++;
+        hipError_t error = launch_fp8_block(context->stream, plan.kernel, plan.split_k, rows,
+                                            outputs, inner, a, a_scale, w, w_scale, out, partials);
+        return error == hipSuccess ? 0 : fail(context, "FP8 block-scaled GEMM", error);
+    });
+}
+
+extern "C" int camblas_cuda_fp8_quantise_1x128(camblas_cuda_context *context, int rows, int inner,
+                                               const void *x, void *q, float *scale)
+{
+    return execute(context, [&] {
+        if (rows < 0 || inner < 128 || inner % 128)
+            return fail(context, "invalid FP8 quantiser dimensions", 1);
+        if (!rows)
+            return 0;
+        if (!x || !q || !scale || !aligned(x, 16) || !aligned(q, 16) || !aligned(scale, 4) ||
+            q == x)
+            return fail(context, "invalid FP8 quantiser buffers", 1);
+        hipError_t error = launch_fp8_quantise(context->stream, rows, inner, x, q, scale);
+        return error == hipSuccess ? 0 : fail(context, "FP8 activation quantisation", error);
+    });
+}
+
+extern "C" size_t camblas_cuda_fp8_block_workspace_size(int rows, int inner)
+{
+    if (rows <= 0 || inner < 128 || inner % 128)
+        return 0;
+    size_t bytes = (size_t(rows) * inner + 15) & ~size_t(15);
+    return bytes + size_t(rows) * (inner / 128) * sizeof(float);
+}
+
+extern "C" int camblas_cuda_fp8_block_linear(camblas_cuda_context *context, int rows, int outputs,
+                                             int inner, const void *x, const void *w,
+                                             const float *w_scale, void *workspace,
+                                             size_t workspace_bytes, void *out)
+{
+    if (!context)
+        return fail(nullptr, "missing context", 1);
+    if (rows < 0 || rows > 65535 || outputs < 1 || inner < 128 || inner % 128)
+        return fail(context, "invalid FP8 block matrix dimensions", 1);
+    if (!rows)
+        return 0;
+    size_t required = camblas_cuda_fp8_block_workspace_size(rows, inner);
+    if (!workspace || workspace_bytes < required || !aligned(workspace, 16) || workspace == x ||
+        workspace == w || workspace == out)
+        return fail(context, "invalid FP8 block linear workspace", 1);
+    unsigned char *q = static_cast<unsigned char *>(workspace);
+    float *scale = reinterpret_cast<float *>(q + ((size_t(rows) * inner + 15) & ~size_t(15)));
+    int status = camblas_cuda_fp8_quantise_1x128(context, rows, inner, x, q, scale);
+    if (status != 0)
+        return status;
+    return camblas_cuda_fp8_block_matmul(context, rows, outputs, inner, q, scale, w, w_scale, out);
+}
+
+extern "C" int camblas_cuda_rope(camblas_cuda_context *context, int tokens, int heads, int dim,
+                                 int token_stride, float theta, const int32_t *positions, void *x)
+{
+    return execute(context, [&] {
+        if (tokens < 0 || heads < 1 || dim < 2 || dim % 2 || token_stride < heads * dim ||
+            !std::isfinite(theta) || theta <= 0)
+            return fail(context, "invalid rotary embedding arguments", 1);
+        if (!tokens)
+            return 0;
+        if (!positions || !x || !aligned(x, 2) || !aligned(positions, 4))
+            return fail(context, "invalid rotary embedding buffers", 1);
+        hipError_t error =
+            launch_rope(context->stream, tokens, heads, dim, token_stride, theta, positions, x);
+        return error == hipSuccess ? 0 : fail(context, "rotary embedding", error);
+    });
+}
+
+extern "C" int camblas_cuda_gqa_decode_attention(camblas_cuda_context *context, int batch,
+                                                 int q_heads, int kv_heads, int dim,
+                                                 int context_length, const int32_t *lengths,
+                                                 float scale, const void *q, int q_stride,
+                                                 const void *k_cache, const void *v_cache,
+                                                 void *output)
+{
+    return execute(context, [&] {
+        if (batch < 0 || q_heads < 1 || kv_heads < 1 || q_heads % kv_heads ||
+            q_heads / kv_heads > 16 || dim != 128 || context_length < 1 ||
+            q_stride < q_heads * dim || !std::isfinite(scale))
+            return fail(context, "invalid decode attention arguments", 1);
+        if (!batch)
+            return 0;
+        if (!q || !k_cache || !v_cache || !output || !aligned(q, 16) || !aligned(k_cache, 16) ||
+            !aligned(v_cache, 16) || !aligned(output, 16) || q_stride % 8 || output == q ||
+            output == k_cache || output == v_cache)
+            return fail(context, "invalid decode attention buffers", 1);
+        int splits = 1;
+        size_t bytes = gqa_decode_scratch_bytes(batch, q_heads, dim, context_length, &splits);
+        hipError_t grown = reserve_scratch(context, bytes);
+        if (grown != hipSuccess)
+            return fail(context, "decode attention scratch", grown);
+        context->counts[6]++;
+        hipError_t error = launch_gqa_decode(context->stream, batch, q_heads, kv_heads, dim,
+                                             context_length, lengths, scale, q, q_stride, k_cache,
+                                             v_cache, output, context->scratch, splits);
+        return error == hipSuccess ? 0 : fail(context, "decode attention", error);
+    });
+}
+
+extern "C" int camblas_hip_plan_describe(int dtype, int algorithm, char trans_a, char trans_b, int m,
+                                         int n, int k, int lda, int ldb, int ldc, int aligned16,
+                                         char *text, size_t text_bytes)
+{
+    if ((dtype != 0 && dtype != 2 && dtype != 3) || (!is_n(trans_a) && !is_t(trans_a)) ||
+        (!is_n(trans_b) && !is_t(trans_b)) || m < 1 || n < 1 || k < 1)
+        return -1;
+    Plan plan = make_plan(dtype, algorithm, is_t(trans_a), is_t(trans_b), m, n, k, lda, ldb, ldc,
+                          aligned16 != 0, 256);
+    describe_plan(plan, dtype, text, text_bytes);
+    return plan.family * 100 + plan.kernel;
+}
+
+extern "C" int camblas_hip_set_plan_override(camblas_cuda_context *context, int kernel, int split_k)
+{
+    if (!context)
+        return fail(nullptr, "missing context", 1);
+    context->override_kernel = kernel;
+    context->override_split = split_k;
+    return 0;
+}
+
+extern "C" int camblas_hip_kernel_count(int dtype)
+{
+    return dtype == 2 ? tn_variant_count() : dtype == 3 ? fp8_variant_count() : 1;
+}

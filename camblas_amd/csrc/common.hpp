@@ -1,0 +1,113 @@
+// Shared declarations of libcamblas_hip.so: context, error convention, kernel launch prototypes.
+#pragma once
+
+#include "camblas_hip.h"
+
+#include <hip/hip_runtime.h>
+
+#include <atomic>
+#include <cstdint>
+#include <cstdio>
+#include <vector>
+
+// One device, one stream, scratch, counters, last error text.
+// Mirrors the role of the reference context (src/cuda/backend.cu:57-77) without vendor handles.
+struct camblas_cuda_context {
+    int device = 0;
+    int algorithm = CAMBLAS_CUDA_AUTO;
+    hipStream_t stream = nullptr;
+    int compute_units = 256;
+    void *scratch = nullptr;       // split-K partials, attention partials
+    size_t scratch_bytes = 0;
+    std::vector<void *> retired;   // superseded scratch kept alive for captured graphs
+    int override_kernel = -1;      // diagnostics: forced kernel variant
+    int override_split = 0;
+    std::atomic<uint64_t> counts[8] = {};
+    char error[256] = "";
+};
+
+namespace camblas_hip
+{
+// Formats "<operation> failed (status <code>)" into the context (or the calling thread's creation
+// buffer when context is null) and returns -code for positive codes, else -1
+// (ref: src/cuda/backend.cu:81-86).
+int fail(camblas_cuda_context *context, const char *operation, int code);
+
+// Ensures the context scratch holds at least `bytes`; refuses to grow while the stream is
+// capturing (ref: src/cuda/backend.cu:399-426). Returns hipSuccess or the failing status.
+hipError_t reserve_scratch(camblas_cuda_context *context, size_t bytes);
+
+inline hipError_t launch_status() { return hipGetLastError(); }
+
+// ---------------------------------------------------------------- planner (pure host)
+enum KernelFamily {
+    FAMILY_GENERIC = 0, // LDS-tiled VALU kernel, any transpose / leading dimension / alignment
+    FAMILY_GEMV_F32 = 1,
+    FAMILY_MFMA_TN = 2, // BF16 'T','N', K-contiguous operands, MFMA tiles staged through LDS
+    FAMILY_FP8_BLOCK = 3
+};
+
+struct Plan {
+    int family = FAMILY_GENERIC;
+    int kernel = 0;   // variant index inside the family
+    int split_k = 1;  // number of K partitions (partials reduced in fixed order)
+    int counter = 0;  // stats slot incremented at launch
+};
+
+// dtype: 0 FP32, 2 BF16, 3 FP8 block-scaled ('T','N' implied). aligned16: every operand pointer
+// is 16-byte aligned. compute_units sizes split-K. Pure function: no device access.
+Plan make_plan(int dtype, int algorithm, bool trans_a, bool trans_b, int m, int n, int k, int lda,
+               int ldb, int ldc, bool aligned16, int compute_units);
+void describe_plan(const Plan &plan, int dtype, char *text, size_t bytes);
+
+struct TnVariant {
+    const char *name;
+    int block_n, block_m, block_k, threads;
+};
+int tn_variant_count();
+const TnVariant &tn_variant(int index);
+int fp8_variant_count();
+const TnVariant &fp8_variant(int index);
+
+// ---------------------------------------------------------------- launchers (each returns a hipError_t)
+hipError_t launch_scale_f32(hipStream_t stream, int m, int n, float beta, float *c, int ldc);
+hipError_t launch_scale_bf16(hipStream_t stream, int m, int n, float beta, void *c, int ldc);
+hipError_t launch_generic_f32(hipStream_t stream, bool ta, bool tb, int m, int n, int k, float alpha,
+                              const float *a, int lda, const float *b, int ldb, float beta, float *c,
+                              int ldc);
+hipError_t launch_generic_bf16(hipStream_t stream, bool ta, bool tb, int m, int n, int k,
+                               float alpha, const void *a, int lda, const void *b, int ldb,
+                               float beta, void *c, int ldc);
+hipError_t launch_generic_f64(hipStream_t stream, bool ta, bool tb, int m, int n, int k,
+                              double alpha, const double *a, int lda, const double *b, int ldb,
+                              double beta, double *c, int ldc);
+hipError_t launch_gemv_f32(hipStream_t stream, int rows, int inner, float alpha, const float *w,
+                           int ld, const float *x, float beta, float *y);
+// y[M,N] (ldc) = alpha * x[M,K] (ldb) * W[N,K]^T (lda) + beta * y, BF16 storage.
+// partials: FP32 [split_k, M, N] when split_k > 1.
+hipError_t launch_bgemm_tn(hipStream_t stream, int variant, int split_k, int n_out, int m_rows,
+                           int k, float alpha, const void *w, int lda, const void *x, int ldb,
+                           float beta, void *y, int ldc, float *partials);
+hipError_t launch_fp8_block(hipStream_t stream, int variant, int split_k, int rows, int outputs,
+                            int inner, const void *a, const float *a_scale, const void *w,
+                            const float *w_scale, void *out, float *partials);
+hipError_t launch_fp8_quantise(hipStream_t stream, int rows, int inner, const void *x, void *q,
+                               float *scale);
+hipError_t launch_silu_multiply(hipStream_t stream, int dtype, uint64_t count, const void *gate,
+                                const void *up, void *out);
+hipError_t launch_swiglu(hipStream_t stream, int dtype, uint64_t count, int width, float limit,
+                         const void *gate, const void *up, const float *routing, void *out);
+hipError_t launch_rms_rows(hipStream_t stream, int dtype, int weight_dtype, int rows, int width,
+                           float epsilon, bool round_before_weight, const void *input,
+                           const void *residual, const void *weight, void *added, void *out);
+hipError_t launch_bf16_square(hipStream_t stream, uint64_t count, const void *input, float *out);
+hipError_t launch_rms_scale(hipStream_t stream, int dtype, uint64_t count, int width, float epsilon,
+                            const void *input, const void *weight, const float *means, void *out);
+hipError_t launch_rope(hipStream_t stream, int tokens, int heads, int dim, int token_stride,
+                       float theta, const int32_t *positions, void *x);
+size_t gqa_decode_scratch_bytes(int batch, int q_heads, int dim, int context_length, int *splits);
+hipError_t launch_gqa_decode(hipStream_t stream, int batch, int q_heads, int kv_heads, int dim,
+                             int context_length, const int32_t *lengths, float scale, const void *q,
+                             int q_stride, const void *k, const void *v, void *out, void *scratch,
+                             int splits);
+} // namespace camblas_hip

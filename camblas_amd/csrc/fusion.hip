@@ -1,0 +1,366 @@
+// Decode-layer epilogues: SiLU*up, SwiGLU, RMS normalisation (optionally fused with the residual
+// add, any number of rows), BF16 squares, RMS scaling and rotary embedding. All are bandwidth or
+// latency bound; they use 128-bit accesses where the row layout allows and FP32 arithmetic with
+// the storage roundings of the reference (src/cuda/inference_fusion.cuh:19-207).
+#include "common.hpp"
+#include "device.hpp"
+
+namespace camblas_hip
+{
+namespace
+{
+// ---------------------------------------------------------------- SiLU(gate) * up
+// round_T(g / (1 + exp(-g))) then round_T(that * u)   (ref: inference_fusion.cuh:19-28)
+template <typename T>
+__global__ void silu_multiply_kernel(size_t count, const T *gate, const T *up, T *out)
+{
+    for (size_t index = size_t(blockIdx.x) * blockDim.x + threadIdx.x; index < count;
+         index += size_t(gridDim.x) * blockDim.x) {
+        float g = storage<T>::load(gate + index);
+        float activated = storage<T>::round(g / (1.f + expf(-g)));
+        storage<T>::store(out + index, __fmul_rn(activated, storage<T>::load(up + index)));
+    }
+}
+
+// Eight BF16 per thread per step; same arithmetic.
+__global__ void silu_multiply_bf16x8_kernel(size_t vectors, const u32x4_t *gate, const u32x4_t *up,
+                                            u32x4_t *out)
+{
+    for (size_t index = size_t(blockIdx.x) * blockDim.x + threadIdx.x; index < vectors;
+         index += size_t(gridDim.x) * blockDim.x) {
+        u32x4_t g = gate[index], u = up[index], r;
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+            float g0 = __uint_as_float(g[e] << 16), g1 = __uint_as_float(g[e] & 0xffff0000u);
+            float u0 = __uint_as_float(u[e] << 16), u1 = __uint_as_float(u[e] & 0xffff0000u);
+            float a0 = bf16_bits_to_float(float_to_bf16_bits(g0 / (1.f + expf(-g0))));
+            float a1 = bf16_bits_to_float(float_to_bf16_bits(g1 / (1.f + expf(-g1))));
+            r[e] = pack_bf16x2(__fmul_rn(a0, u0), __fmul_rn(a1, u1));
+        }
+        out[index] = r;
+    }
+}
+
+// ---------------------------------------------------------------- SwiGLU
+// optional clamp with NaN-preserving compares, FP32 silu(g)*u, optional per-row routing factor,
+// one final rounding (ref: inference_fusion.cuh:30-51)
+template <typename T>
+__global__ void swiglu_kernel(size_t count, int width, float limit, const T *gate, const T *up,
+                              const float *routing, T *out)
+{
+    for (size_t index = size_t(blockIdx.x) * blockDim.x + threadIdx.x; index < count;
+         index += size_t(gridDim.x) * blockDim.x) {
+        float g = storage<T>::load(gate + index), u = storage<T>::load(up + index);
+        if (limit > 0) {
+            if (g > limit)
+                g = limit;
+            if (u > limit)
+                u = limit;
+            if (u < -limit)
+                u = -limit;
+        }
+        float value = __fmul_rn(g / (1.f + expf(-g)), u);
+        if (routing)
+            value = __fmul_rn(routing[index / size_t(width)], value);
+        storage<T>::store(out + index, value);
+    }
+}
+
+// ---------------------------------------------------------------- RMS normalisation rows
+// One workgroup per row. added = round_T(x + r) when a residual is given; scale = rsqrt(mean(v^2) +
+// eps); out = round_T(round_T(v*scale) * w) or, without intermediate rounding, round_T((v*scale)*w)
+// (ref: inference_fusion.cuh:53-86 and :136-191). The sum of squares uses a fixed order: per-thread
+// strided partial sums, a 64-lane butterfly, then the wave partials in index order.
+template <typename T, typename W>
+__global__ __launch_bounds__(256) void rms_rows_kernel(int width, float epsilon,
+                                                       bool round_before_weight, const T *input,
+                                                       const T *residual, const W *weight, T *added,
+                                                       T *out)
+{
+    __shared__ float partial[4];
+    const size_t base = size_t(blockIdx.x) * width;
+    const T *x = input + base;
+    const T *r = residual ? residual + base : nullptr;
+    float sum = 0.f;
+    for (int column = threadIdx.x; column < width; column += 256) {
+        float value = storage<T>::load(x + column);
+        if (r)
+            value = storage<T>::round(__fadd_rn(value, storage<T>::load(r + column)));
+        sum = __fadd_rn(sum, __fmul_rn(value, value));
+    }
+    sum = wave_sum(sum);
+    if (threadIdx.x % 64 == 0)
+        partial[threadIdx.x / 64] = sum;
+    __syncthreads();
+    float total = __fadd_rn(__fadd_rn(partial[0], partial[1]), __fadd_rn(partial[2], partial[3]));
+    float scale = rsqrtf(__fadd_rn(total / float(width), epsilon));
+    for (int column = threadIdx.x; column < width; column += 256) {
+        float value = storage<T>::load(x + column);
+        if (r) {
+            value = storage<T>::round(__fadd_rn(value, storage<T>::load(r + column)));
+            storage<T>::store(added + base + column, value);
+        }
+        float normalised = __fmul_rn(value, scale);
+        if (round_before_weight)
+            normalised = storage<T>::round(normalised);
+        storage<T>::store(out + base + column,
+                          __fmul_rn(normalised, storage<W>::load(weight + column)));
+    }
+}
+
+// BF16 rows whose width is a multiple of 8 and whose buffers are 16-byte aligned: the row is read
+// once with 128-bit loads and kept in registers (up to 8192 columns per 256 threads x 4 vectors;
+// wider rows loop), same arithmetic and reduction order class as above.
+template <int VECTORS, bool WEIGHT_BF16>
+__global__ __launch_bounds__(256) void rms_rows_bf16_kernel(int width, float epsilon,
+                                                            bool round_before_weight,
+                                                            const unsigned short *input,
+                                                            const unsigned short *residual,
+                                                            const void *weight,
+                                                            unsigned short *added,
+                                                            unsigned short *out)
+{
+    __shared__ float partial[4];
+    const size_t base = size_t(blockIdx.x) * width;
+    const int vectors = width / 8;
+    const u32x4_t *x = reinterpret_cast<const u32x4_t *>(input + base);
+    const u32x4_t *r = residual ? reinterpret_cast<const u32x4_t *>(residual + base) : nullptr;
+    float values[VECTORS][8];
+    float sum = 0.f;
+#pragma unroll
+    for (int v = 0; v < VECTORS; ++v) {
+        int index = v * 256 + threadIdx.x;
+        if (index < vectors) {
+            u32x4_t xv = x[index];
+            u32x4_t rv = {0u, 0u, 0u, 0u};
+            if (r)
+                rv = r[index];
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                float lo = __uint_as_float(xv[e] << 16), hi = __uint_as_float(xv[e] & 0xffff0000u);
+                if (r) {
+                    lo = bf16_bits_to_float(
+                        float_to_bf16_bits(__fadd_rn(lo, __uint_as_float(rv[e] << 16))));
+                    hi = bf16_bits_to_float(
+                        float_to_bf16_bits(__fadd_rn(hi, __uint_as_float(rv[e] & 0xffff0000u))));
+                }
+                values[v][2 * e] = lo;
+                values[v][2 * e + 1] = hi;
+                sum = __fadd_rn(sum, __fmul_rn(lo, lo));
+                sum = __fadd_rn(sum, __fmul_rn(hi, hi));
+            }
+            if (r) {
+                u32x4_t packed;
+#pragma unroll
+                for (int e = 0; e < 4; ++e)
+                    packed[e] = (__float_as_uint(values[v][2 * e]) >> 16) |
+                                (__float_as_uint(values[v][2 * e + 1]) & 0xffff0000u);
+                reinterpret_cast<u32x4_t *>(added + base)[index] = packed;
+            }
+        }
+    }
+    sum = wave_sum(sum);
+    if (threadIdx.x % 64 == 0)
+        partial[threadIdx.x / 64] = sum;
+    __syncthreads();
+    float total = __fadd_rn(__fadd_rn(partial[0], partial[1]), __fadd_rn(partial[2], partial[3]));
+    float scale = rsqrtf(__fadd_rn(total / float(width), epsilon));
+#pragma unroll
+    for (int v = 0; v < VECTORS; ++v) {
+        int index = v * 256 + threadIdx.x;
+        if (index < vectors) {
+            float w[8];
+            if constexpr (WEIGHT_BF16) {
+                u32x4_t wv = reinterpret_cast<const u32x4_t *>(weight)[index];
+#pragma unroll
+                for (int e = 0; e < 4; ++e) {
+                    w[2 * e] = __uint_as_float(wv[e] << 16);
+                    w[2 * e + 1] = __uint_as_float(wv[e] & 0xffff0000u);
+                }
+            } else {
+                const f32x4_t *wf = reinterpret_cast<const f32x4_t *>(weight) + 2 * index;
+                f32x4_t w0 = wf[0], w1 = wf[1];
+#pragma unroll
+                for (int e = 0; e < 4; ++e) {
+                    w[e] = w0[e];
+                    w[4 + e] = w1[e];
+                }
+            }
+            u32x4_t packed;
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                float n0 = __fmul_rn(values[v][2 * e], scale);
+                float n1 = __fmul_rn(values[v][2 * e + 1], scale);
+                if (round_before_weight) {
+                    n0 = bf16_bits_to_float(float_to_bf16_bits(n0));
+                    n1 = bf16_bits_to_float(float_to_bf16_bits(n1));
+                }
+                packed[e] = pack_bf16x2(__fmul_rn(n0, w[2 * e]), __fmul_rn(n1, w[2 * e + 1]));
+            }
+            reinterpret_cast<u32x4_t *>(out + base)[index] = packed;
+        }
+    }
+}
+
+// ---------------------------------------------------------------- helpers kept for the binding
+__global__ void bf16_square_kernel(size_t count, const unsigned short *input, float *out)
+{
+    for (size_t index = size_t(blockIdx.x) * blockDim.x + threadIdx.x; index < count;
+         index += size_t(gridDim.x) * blockDim.x) {
+        float value = bf16_bits_to_float(input[index]);
+        out[index] = __fmul_rn(value, value);
+    }
+}
+
+// ref: inference_fusion.cuh:106-119
+template <typename T>
+__global__ void rms_scale_kernel(size_t count, int width, float epsilon, const T *input,
+                                 const T *weight, const float *means, T *out)
+{
+    for (size_t index = size_t(blockIdx.x) * blockDim.x + threadIdx.x; index < count;
+         index += size_t(gridDim.x) * blockDim.x) {
+        float scale = rsqrtf(__fadd_rn(means[index / size_t(width)], epsilon));
+        float normalised = storage<T>::round(__fmul_rn(storage<T>::load(input + index), scale));
+        storage<T>::store(out + index,
+                          __fmul_rn(normalised, storage<T>::load(weight + index % size_t(width))));
+    }
+}
+
+// ---------------------------------------------------------------- rotary embedding
+// Rotate-half pairing (i, i + dim/2), angle = position * theta^(-2i/dim), FP32 sin/cos, one BF16
+// rounding per element. One thread per (token, head, i).
+__global__ void rope_kernel(int tokens, int heads, int dim, int token_stride, float theta,
+                            const int32_t *positions, unsigned short *x)
+{
+    const int half = dim / 2;
+    size_t index = size_t(blockIdx.x) * blockDim.x + threadIdx.x;
+    size_t count = size_t(tokens) * heads * half;
+    if (index >= count)
+        return;
+    int i = int(index % half);
+    int head = int((index / half) % heads);
+    int token = int(index / (size_t(half) * heads));
+    float frequency = exp2f(-2.f * float(i) / float(dim) * log2f(theta));
+    float angle = float(positions[token]) * frequency;
+    float s, c;
+    sincosf(angle, &s, &c);
+    unsigned short *v = x + size_t(token) * token_stride + size_t(head) * dim;
+    float lo = bf16_bits_to_float(v[i]), hi = bf16_bits_to_float(v[i + half]);
+    v[i] = float_to_bf16_bits(lo * c - hi * s);
+    v[i + half] = float_to_bf16_bits(hi * c + lo * s);
+}
+
+unsigned stride_blocks(uint64_t count)
+{
+    uint64_t blocks = (count + 255) / 256;
+    return unsigned(blocks < 65535 ? blocks : 65535);
+}
+
+bool aligned16(const void *p) { return reinterpret_cast<uintptr_t>(p) % 16 == 0; }
+} // namespace
+
+hipError_t launch_silu_multiply(hipStream_t stream, int dtype, uint64_t count, const void *gate,
+                                const void *up, void *out)
+{
+    if (dtype == 0)
+        silu_multiply_kernel<float><<<stride_blocks(count), 256, 0, stream>>>(
+            count, static_cast<const float *>(gate), static_cast<const float *>(up),
+            static_cast<float *>(out));
+    else if (count % 8 == 0 && aligned16(gate) && aligned16(up) && aligned16(out))
+        silu_multiply_bf16x8_kernel<<<stride_blocks(count / 8), 256, 0, stream>>>(
+            count / 8, static_cast<const u32x4_t *>(gate), static_cast<const u32x4_t *>(up),
+            static_cast<u32x4_t *>(out));
+    else
+        silu_multiply_kernel<bf16_storage><<<stride_blocks(count), 256, 0, stream>>>(
+            count, static_cast<const bf16_storage *>(gate), static_cast<const bf16_storage *>(up),
+            static_cast<bf16_storage *>(out));
+    return launch_status();
+}
+
+hipError_t launch_swiglu(hipStream_t stream, int dtype, uint64_t count, int width, float limit,
+                         const void *gate, const void *up, const float *routing, void *out)
+{
+    if (dtype == 0)
+        swiglu_kernel<float><<<stride_blocks(count), 256, 0, stream>>>(
+            count, width, limit, static_cast<const float *>(gate), static_cast<const float *>(up),
+            routing, static_cast<float *>(out));
+    else
+        swiglu_kernel<bf16_storage><<<stride_blocks(count), 256, 0, stream>>>(
+            count, width, limit, static_cast<const bf16_storage *>(gate),
+            static_cast<const bf16_storage *>(up), routing, static_cast<bf16_storage *>(out));
+    return launch_status();
+}
+
+hipError_t launch_rms_rows(hipStream_t stream, int dtype, int weight_dtype, int rows, int width,
+                           float epsilon, bool round_before_weight, const void *input,
+                           const void *residual, const void *weight, void *added, void *out)
+{
+    if (dtype == 0) {
+        rms_rows_kernel<float, float><<<rows, 256, 0, stream>>>(
+            width, epsilon, round_before_weight, static_cast<const float *>(input),
+            static_cast<const float *>(residual), static_cast<const float *>(weight),
+            static_cast<float *>(added), static_cast<float *>(out));
+        return launch_status();
+    }
+    const unsigned short *x = static_cast<const unsigned short *>(input);
+    const unsigned short *r = static_cast<const unsigned short *>(residual);
+    unsigned short *a = static_cast<unsigned short *>(added), *o = static_cast<unsigned short *>(out);
+    bool vector = width % 8 == 0 && width <= 8192 && aligned16(input) && aligned16(out) &&
+                  aligned16(weight) && (!residual || (aligned16(residual) && aligned16(added)));
+    if (vector && weight_dtype == 2) {
+        if (width <= 2048)
+            rms_rows_bf16_kernel<1, true>
+                <<<rows, 256, 0, stream>>>(width, epsilon, round_before_weight, x, r, weight, a, o);
+        else if (width <= 4096)
+            rms_rows_bf16_kernel<2, true>
+                <<<rows, 256, 0, stream>>>(width, epsilon, round_before_weight, x, r, weight, a, o);
+        else
+            rms_rows_bf16_kernel<4, true>
+                <<<rows, 256, 0, stream>>>(width, epsilon, round_before_weight, x, r, weight, a, o);
+    } else if (vector) {
+        rms_rows_bf16_kernel<4, false>
+            <<<rows, 256, 0, stream>>>(width, epsilon, round_before_weight, x, r, weight, a, o);
+    } else if (weight_dtype == 2) {
+        rms_rows_kernel<bf16_storage, bf16_storage><<<rows, 256, 0, stream>>>(
+            width, epsilon, round_before_weight, static_cast<const bf16_storage *>(input),
+            static_cast<const bf16_storage *>(residual), static_cast<const bf16_storage *>(weight),
+            static_cast<bf16_storage *>(added), static_cast<bf16_storage *>(out));
+    } else {
+        rms_rows_kernel<bf16_storage, float><<<rows, 256, 0, stream>>>(
+            width, epsilon, round_before_weight, static_cast<const bf16_storage *>(input),
+            static_cast<const bf16_storage *>(residual), static_cast<const float *>(weight),
+            static_cast<bf16_storage *>(added), static_cast<bf16_storage *>(out));
+    }
+    return launch_status();
+}
+
+hipError_t launch_bf16_square(hipStream_t stream, uint64_t count, const void *input, float *out)
+{
+    bf16_square_kernel<<<stride_blocks(count), 256, 0, stream>>>(
+        count, static_cast<const unsigned short *>(input), out);
+    return launch_status();
+}
+
+hipError_t launch_rms_scale(hipStream_t stream, int dtype, uint64_t count, int width, float epsilon,
+                            const void *input, const void *weight, const float *means, void *out)
+{
+    if (dtype == 0)
+        rms_scale_kernel<float><<<stride_blocks(count), 256, 0, stream>>>(
+            count, width, epsilon, static_cast<const float *>(input),
+            static_cast<const float *>(weight), means, static_cast<float *>(out));
+    else
+        rms_scale_kernel<bf16_storage><<<stride_blocks(count), 256, 0, stream>>>(
+            count, width, epsilon, static_cast<const bf16_storage *>(input),
+            static_cast<const bf16_storage *>(weight), means, static_cast<bf16_storage *>(out));
+    return launch_status();
+}
+
+hipError_t launch_rope(hipStream_t stream, int tokens, int heads, int dim, int token_stride,
+                       float theta, const int32_t *positions, void *x)
+{
+    size_t count = size_t(tokens) * heads * (dim / 2);
+    rope_kernel<<<unsigned((count + 255) / 256), 256, 0, stream>>>(
+        tokens, heads, dim, token_stride, theta, positions, static_cast<unsigned short *>(x));
+    return launch_status();
+}
+} // namespace camblas_hip

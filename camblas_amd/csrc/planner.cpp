@@ -1,0 +1,132 @@
+// GEMM planner: a pure host function from (dtype, layout, shape, leading dimensions, alignment)
+// to a kernel family, a tile variant and a split-K factor. It replaces the reference's run-time
+// plan cache and timing autotune (src/cuda/backend.cu:553-784) with a closed-form decision: no
+// device access, no stream synchronisation, identical answers for identical inputs, so a shape
+// planned during warm-up replays unchanged under graph capture.
+#include "common.hpp"
+
+#include <algorithm>
+#include <cstring>
+
+namespace camblas_hip
+{
+namespace
+{
+int ceil_div(int a, int b) { return (a + b - 1) / b; }
+
+// Work partition for the bandwidth-bound decode tiles: enough workgroups to keep about four per
+// compute unit in flight, never fewer than four K tiles per partition.
+int decode_split(int tiles, int k_tiles, int compute_units)
+{
+    int wanted = ceil_div(4 * compute_units, std::max(1, tiles));
+    int limit = std::max(1, k_tiles / 4);
+    return std::max(1, std::min(wanted, limit));
+}
+
+// Fraction of the machine a tiling keeps busy: useful tiles over whole rounds of resident
+// workgroups, times the fraction of each tile that is inside the matrix.
+double occupancy_score(int n, int m, int block_n, int block_m, int resident, int compute_units)
+{
+    double tiles = double(ceil_div(n, block_n)) * ceil_div(m, block_m);
+    double slots = double(resident) * compute_units;
+    double rounds = std::ceil(tiles / slots);
+    double fill = (double(n) * m) / (tiles * block_n * block_m);
+    return tiles / (rounds * slots) * fill;
+}
+} // namespace
+
+Plan make_plan(int dtype, int algorithm, bool trans_a, bool trans_b, int m, int n, int k, int lda,
+               int ldb, int ldc, bool aligned16, int compute_units)
+{
+    (void)ldc;
+    Plan plan;
+    if (compute_units < 1)
+        compute_units = 256;
+    if (dtype == 0) {
+        // FP32: the single-vector shortcut exists only under AUTO (ref: src/cuda/backend.cu:810-815)
+        if (algorithm == CAMBLAS_CUDA_AUTO && n == 1 && trans_a && !trans_b && m >= 1024 &&
+            k >= 4096 && k % 4 == 0 && lda % 4 == 0 && aligned16) {
+            plan.family = FAMILY_GEMV_F32;
+            plan.counter = 0;
+            return plan;
+        }
+        plan.family = FAMILY_GENERIC;
+        plan.counter = algorithm == CAMBLAS_CUDA_LT || algorithm == CAMBLAS_CUDA_AUTO ? 4 : 0;
+        return plan;
+    }
+    if (dtype == 2) {
+        const int limit = 1 << 23;
+        bool matrix_path = algorithm != CAMBLAS_CUDA_CLASSICAL && trans_a && !trans_b &&
+                           k % 8 == 0 && lda % 8 == 0 && ldb % 8 == 0 && aligned16 && lda < limit &&
+                           ldb < limit;
+        if (!matrix_path) {
+            plan.family = FAMILY_GENERIC;
+            plan.counter = 0;
+            return plan;
+        }
+        plan.family = FAMILY_MFMA_TN;
+        plan.counter = 4;
+        const int outputs = m, tokens = n;
+        if (tokens <= 32) {
+            plan.kernel = 4; // 128 x 32 x 64
+            const TnVariant &v = tn_variant(plan.kernel);
+            plan.split_k =
+                decode_split(ceil_div(outputs, v.block_n), ceil_div(k, v.block_k), compute_units);
+        } else if (tokens <= 64) {
+            plan.kernel = 3; // 128 x 64 x 64
+            const TnVariant &v = tn_variant(plan.kernel);
+            plan.split_k =
+                decode_split(ceil_div(outputs, v.block_n), ceil_div(k, v.block_k), compute_units);
+        } else {
+            // prefill: larger tiles reuse more per byte; prefer them unless a smaller tile fills
+            // the compute units noticeably better
+            double best = -1;
+            const int candidates[3] = {0, 1, 2};
+            const int resident[3] = {1, 1, 2};
+            const double weight[3] = {1.0, 0.95, 0.85};
+            for (int i = 0; i < 3; ++i) {
+                const TnVariant &v = tn_variant(candidates[i]);
+                double score = weight[i] * occupancy_score(outputs, tokens, v.block_n, v.block_m,
+                                                           resident[i], compute_units);
+                if (score > best) {
+                    best = score;
+                    plan.kernel = candidates[i];
+                }
+            }
+            plan.split_k = 1;
+        }
+        return plan;
+    }
+    // FP8 block-scaled: rows = n (tokens), outputs = m, always K-contiguous
+    plan.family = FAMILY_FP8_BLOCK;
+    plan.counter = 4;
+    plan.kernel = n <= 32 ? 1 : 0;
+    if (n <= 32) {
+        const TnVariant &v = fp8_variant(plan.kernel);
+        plan.split_k = decode_split(ceil_div(m, v.block_n), ceil_div(k, v.block_k), compute_units);
+    }
+    return plan;
+}
+
+void describe_plan(const Plan &plan, int dtype, char *text, size_t bytes)
+{
+    if (!text || !bytes)
+        return;
+    const char *type = dtype == 0 ? "f32" : dtype == 2 ? "bf16" : "fp8-block128";
+    switch (plan.family) {
+    case FAMILY_GEMV_F32:
+        std::snprintf(text, bytes, "%s gemv wave-per-row", type);
+        break;
+    case FAMILY_MFMA_TN:
+        std::snprintf(text, bytes, "%s %s split_k=%d", type, tn_variant(plan.kernel).name,
+                      plan.split_k);
+        break;
+    case FAMILY_FP8_BLOCK:
+        std::snprintf(text, bytes, "%s %s split_k=%d", type, fp8_variant(plan.kernel).name,
+                      plan.split_k);
+        break;
+    default:
+        std::snprintf(text, bytes, "%s generic 64x64x16", type);
+    }
+}
+} // namespace camblas_hip

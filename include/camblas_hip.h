@@ -1,0 +1,192 @@
+/*
+ * C ABI of libcamblas_hip.so: the MI355X (gfx950) backend for the CAMBLAS GPU linear path.
+ *
+ * The exported symbols keep the reference's names (camblas_cuda_*) and signatures so the
+ * reference's ctypes loader (camblas/_native.py:97-173) and tensor binding resolve them
+ * unchanged when CAMBLAS_CUDA_LIBRARY points at this library. Each declaration cites the reference
+ * interface it replaces as "ref: file:line" (paths relative to the reference tree). Entry points
+ * marked "extension" have no counterpart in include/camblas_cuda.h; the comment says which
+ * reference code defines their arithmetic.
+ *
+ * Conventions (ref: include/camblas_cuda.h:25-38, src/cuda/backend.cu:81-86):
+ *  - every operation returns 0 on success and a negative code on failure; the message is
+ *    available from camblas_cuda_error(context) (or camblas_cuda_error(NULL) for creation errors,
+ *    which are stored per host thread);
+ *  - one context owns one device and one HIP stream (hipStream_t passed as void*); calls enqueue
+ *    work on that stream and return; the caller keeps operands alive until the stream completes;
+ *  - a context is single-threaded and not fork-safe; use one per (thread, device, stream);
+ *  - stream capture: create contexts and run each shape once before capturing; scratch growth is
+ *    refused while the stream is capturing.
+ */
+#ifndef CAMBLAS_HIP_H
+#define CAMBLAS_HIP_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef struct camblas_cuda_context camblas_cuda_context;
+
+/* ref: include/camblas_cuda.h:14-23. On this backend AUTO and LT select the planned MFMA/GEMV
+ * kernels (counter slot 4), CLASSICAL forces the generic LDS-tiled kernel (counter slot 0), and
+ * the SYMMETRIC/STRASSEN values are accepted and executed as CLASSICAL-or-planned products with
+ * ordinary rounding (the reference documents those modes as optional accelerations). */
+enum camblas_cuda_algorithm {
+    CAMBLAS_CUDA_AUTO = 0,
+    CAMBLAS_CUDA_CLASSICAL = 1,
+    CAMBLAS_CUDA_STRASSEN = 2,
+    CAMBLAS_CUDA_LT = 3,
+    CAMBLAS_CUDA_SYMMETRIC = 4,
+    CAMBLAS_CUDA_STRASSEN_TWO = 5,
+    CAMBLAS_CUDA_STRASSEN_THREE = 6,
+    CAMBLAS_CUDA_STRASSEN_FOUR = 7
+};
+
+/* ref: include/camblas_cuda.h:39-42, src/cuda/backend.cu:954-1055 */
+int camblas_cuda_create(int device, void *stream, camblas_cuda_context **out);
+int camblas_cuda_destroy(camblas_cuda_context *context);
+const char *camblas_cuda_error(const camblas_cuda_context *context);
+int camblas_cuda_set_algorithm(camblas_cuda_context *context, int algorithm);
+
+/* Column-major C = alpha op(A) op(B) + beta C, FP32 throughout (no reduced-precision matrix
+ * path). beta==0 never reads C; output may not alias A or B; A/B may be NULL when alpha==0 or
+ * k==0. ref: include/camblas_cuda.h:44-59, src/cuda/backend.cu:786-866 (validation order) and
+ * src/cuda/decode_float.cuh:2-52 (the n==1 'T','N' GEMV shortcut under AUTO). */
+int camblas_cuda_sgemm(camblas_cuda_context *context, char trans_a, char trans_b, int m, int n,
+                       int k, float alpha, const float *a, int lda, const float *b, int ldb,
+                       float beta, float *c, int ldc);
+
+/* Same contract with BF16 storage, float alpha/beta, FP32 accumulation and one round-to-nearest
+ * conversion to BF16. ref: include/camblas_cuda.h:64-69, src/cuda/bfloat16.cuh:11-57.
+ * The linear path always arrives as ('T','N', m=out_features, n=tokens, k=in_features) with both
+ * operands K-contiguous (ref: src/cuda/torch_bindings.cpp:146-199). */
+int camblas_cuda_bgemm(camblas_cuda_context *context, char trans_a, char trans_b, int m, int n,
+                       int k, float alpha, const void *a, int lda, const void *b, int ldb,
+                       float beta, void *c, int ldc);
+
+/* ref: include/camblas_cuda.h:60-62, :71-94. Present so the reference loader, which resolves
+ * these names at load time, accepts the library; FP64 GEMM, affine/MLP, dense single-head
+ * attention and MLP backward are outside the linear path and return a negative status with the
+ * message "... is not provided by the HIP linear backend". */
+int camblas_cuda_dgemm(camblas_cuda_context *context, char trans_a, char trans_b, int m, int n,
+                       int k, double alpha, const double *a, int lda, const double *b, int ldb,
+                       double beta, double *c, int ldc);
+int camblas_cuda_affine(camblas_cuda_context *context, int dtype, int rows, int inner, int columns,
+                        const void *x, const void *weight, const void *bias, int relu,
+                        void *output);
+int camblas_cuda_mlp(camblas_cuda_context *context, int dtype, int rows, int inputs, int hidden,
+                     int outputs, const void *x, const void *w1, const void *b1, const void *w2,
+                     const void *b2, void *hidden_output, void *output);
+int camblas_cuda_attention(camblas_cuda_context *context, int dtype, int queries, int keys,
+                           int depth, int values, double scale, const void *q, const void *k,
+                           const void *v, void *output);
+int camblas_cuda_mlp_backward(camblas_cuda_context *context, int dtype, int rows, int inputs,
+                              int hidden, int outputs, const void *x, const void *w1,
+                              const void *w2, const void *hidden_output, const void *grad_output,
+                              void *grad_hidden, void *dx, void *dw1, void *db1, void *dw2,
+                              void *db2);
+
+/* SiLU(gate)*up, dtype 0 FP32 / 2 BF16, intermediate rounding to the storage type.
+ * ref: include/camblas_cuda.h:96-100, src/cuda/inference_fusion.cuh:19-28 */
+int camblas_cuda_silu_multiply(camblas_cuda_context *context, int dtype, uint64_t count,
+                               const void *gate, const void *up, void *output);
+/* ref: include/camblas_cuda.h:101-109, src/cuda/inference_fusion.cuh:30-51 */
+int camblas_cuda_swiglu(camblas_cuda_context *context, int dtype, uint64_t count, int width,
+                        float limit, const void *gate, const void *up, const float *routing,
+                        void *output);
+
+/* Row-major RMS normalisation, rounding the normalised value to storage before the weight
+ * multiply. ref: include/camblas_cuda.h:185-189, src/cuda/inference_fusion.cuh:53-86 */
+int camblas_cuda_rms_norm(camblas_cuda_context *context, int dtype, int rows, int width,
+                          float epsilon, const void *input, const void *weight, void *output);
+/* Single row, explicit rounding policy. `descending` selects a reduction order in the reference;
+ * here it is validated and otherwise has no effect (one fixed wavefront-64 order).
+ * ref: include/camblas_cuda.h:190-196, src/cuda/inference_fusion.cuh:136-191 */
+int camblas_cuda_rms_norm_decode(camblas_cuda_context *context, int dtype, int weight_dtype,
+                                 int width, float epsilon, int round_before_weight, int descending,
+                                 const void *input, const void *weight, void *output);
+/* Single-row residual add + RMS norm. ref: include/camblas_cuda.h:197-202 */
+int camblas_cuda_add_rms_norm(camblas_cuda_context *context, int dtype, int width, float epsilon,
+                              const void *input, const void *residual, const void *weight,
+                              void *added, void *output);
+/* ref: include/camblas_cuda.h:203-209, src/cuda/inference_fusion.cuh:99-119 */
+int camblas_cuda_bfloat16_square(camblas_cuda_context *context, uint64_t count, const void *input,
+                                 float *output);
+int camblas_cuda_rms_scale(camblas_cuda_context *context, int dtype, uint64_t count, int width,
+                           float epsilon, const void *input, const void *weight, const float *means,
+                           void *output);
+
+/* Host launch counters, length 6 or 8: [0] classical/generic/GEMV, [1] strassen (always 0),
+ * [2] gram (always 0), [3] affine (0), [4] planned MFMA GEMM ("lt"), [5] guard fallback
+ * (scratch could not grow: generic kernel used), [6] attention, [7] backward (0).
+ * ref: include/camblas_cuda.h:211-215, src/cuda/backend.cu:1477-1493 */
+int camblas_cuda_stats(const camblas_cuda_context *context, uint64_t *counts, int length);
+int camblas_cuda_reset_stats(camblas_cuda_context *context);
+
+/* ------------------------------------------------------------------ extensions */
+
+/* extension. FP8 E4M3fn block-scaled linear: a [rows, inner] bytes with FP32 scales
+ * [rows, inner/128] (one per 1x128 group), w [outputs, inner] bytes with FP32 scales
+ * [ceil(outputs/128), inner/128] (one per 128x128 block), BF16 out [rows, outputs].
+ * Arithmetic rule (ref: camblas/_hopper.py:118-126 and :168-182, which implement it for rows==1):
+ * per 128-wide K group the unscaled FP32 dot product, then
+ * acc = fma(dot_g, a_scale[r,g] * w_scale[n/128,g], acc) for g ascending, one BF16 rounding.
+ * inner is a positive multiple of 128, outputs >= 1, rows 0..65535; a, w 16-byte aligned. */
+int camblas_cuda_fp8_block_matmul(camblas_cuda_context *context, int rows, int outputs, int inner,
+                                  const void *a_fp8, const float *a_scale, const void *w_fp8,
+                                  const float *w_scale, void *out_bf16);
+/* extension. Dynamic 1x128 activation quantiser (ref: camblas/_hopper.py:82-98): amax =
+ * max(|x|, 1e-10) per group, scale = amax/448, q = e4m3(clamp(x * (448/amax), +-448)). */
+int camblas_cuda_fp8_quantise_1x128(camblas_cuda_context *context, int rows, int inner,
+                                    const void *x_bf16, void *q_fp8, float *scale);
+/* extension. BF16 input, quantised on the fly, then the product above. `workspace` holds the
+ * quantised activations: rows*inner bytes + rows*(inner/128) floats, 16-byte aligned. */
+size_t camblas_cuda_fp8_block_workspace_size(int rows, int inner);
+int camblas_cuda_fp8_block_linear(camblas_cuda_context *context, int rows, int outputs, int inner,
+                                  const void *x_bf16, const void *w_fp8, const float *w_scale,
+                                  void *workspace, size_t workspace_bytes, void *out_bf16);
+
+/* extension. Multi-row residual add + RMS norm with the arithmetic of camblas_cuda_add_rms_norm
+ * (ref: src/cuda/inference_fusion.cuh:136-191) applied to each of `rows` rows; residual may be
+ * NULL (plain norm, `added` ignored). weight_dtype 0 FP32 / 2 BF16. */
+int camblas_cuda_add_rms_norm_rows(camblas_cuda_context *context, int dtype, int weight_dtype,
+                                   int rows, int width, float epsilon, int round_before_weight,
+                                   const void *input, const void *residual, const void *weight,
+                                   void *added, void *output);
+
+/* extension (no reference counterpart; the reference leaves RoPE and KV-cache attention to the
+ * serving engine, configs/sglang.json:44). Rotate-half rotary embedding in place on BF16
+ * x [tokens, heads, dim] whose token stride is token_stride elements; positions int32 [tokens]. */
+int camblas_cuda_rope(camblas_cuda_context *context, int tokens, int heads, int dim,
+                      int token_stride, float theta, const int32_t *positions, void *x_bf16);
+/* extension. Grouped-query decode attention, one query per sequence: q [batch, q_heads, dim]
+ * (token stride q_stride elements), K/V caches [batch, context, kv_heads, dim] BF16, lengths int32
+ * [batch] or NULL (= context), out [batch, q_heads, dim] BF16. dim must be 128, q_heads a
+ * multiple of kv_heads with ratio <= 16. Split-K over the context with an ordered combine;
+ * partials live in context scratch. */
+int camblas_cuda_gqa_decode_attention(camblas_cuda_context *context, int batch, int q_heads,
+                                      int kv_heads, int dim, int context_length,
+                                      const int32_t *lengths, float scale, const void *q,
+                                      int q_stride, const void *k_cache, const void *v_cache,
+                                      void *output);
+
+/* extension. Planner introspection (the GPU counterpart of the reference CPU planner's
+ * camblas_plan_format, src/planner.c:654-669): writes a one-line description of the kernel the
+ * planner picks for a GEMM call into `text` and returns the kernel id (>=0) without touching a
+ * device. dtype 0 FP32, 2 BF16, 3 FP8-block. Pure host function: works without a GPU. */
+int camblas_hip_plan_describe(int dtype, int algorithm, char trans_a, char trans_b, int m, int n,
+                              int k, int lda, int ldb, int ldc, int aligned16, char *text,
+                              size_t text_bytes);
+/* extension. Diagnostics for tests and tuning: force the planner's choice for BF16/FP8 GEMMs on
+ * this context (kernel < 0 restores the planner; split_k <= 0 lets the planner choose). */
+int camblas_hip_set_plan_override(camblas_cuda_context *context, int kernel, int split_k);
+/* extension. Number of kernel variants `camblas_hip_set_plan_override` accepts for a dtype. */
+int camblas_hip_kernel_count(int dtype);
+
+#ifdef __cplusplus
+}
+#endif
+#endif

@@ -1,0 +1,199 @@
+"""BF16 GEMM through the C ABI against the CPU oracle.
+
+Strategy follows the reference's BF16 suite (tests/test_bfloat16.py:24-217, tests/test_linear.py):
+FP64 accumulation of the exact BF16 operands rounded once to BF16, exact analytic cases that prove
+FP32 accumulation and correct placement, alpha/beta and NaN semantics, padded leading dimensions,
+changed-input reruns. Tolerance: relative Frobenius error <= 1e-2 against the FP64 product (the
+measured error is about 2e-3, the BF16 output rounding). Every MFMA tile variant and split-K
+factor is forced in turn so the whole kernel table is covered, not just the planner's choice.
+"""
+
+import ctypes as ct
+
+import numpy as np
+import pytest
+import torch
+
+import oracle
+from camblas_amd import _kernels, _native
+from helpers import bf16_values, from_device_bf16, ptr, rel_frobenius, to_device_bf16
+
+pytestmark = pytest.mark.gpu
+TOLERANCE = 1e-2
+
+
+def run_bgemm(device, ta, tb, m, n, k, alpha, a, lda, b, ldb, beta, c, ldc, override=None,
+              algorithm="auto"):
+    at, bt, ct_ = (to_device_bf16(v, device) for v in (a, b, c))
+    with _native.algorithm(algorithm):
+        native = _native.context(device)
+        if override is not None:
+            native.call("hip_set_plan_override", override[0], override[1])
+        try:
+            native.call("bgemm", ta.encode(), tb.encode(), m, n, k, ct.c_float(alpha), ptr(at), lda,
+                        ptr(bt), ldb, ct.c_float(beta), ptr(ct_), ldc)
+        finally:
+            native.call("hip_set_plan_override", -1, 0)
+    torch.cuda.synchronize()
+    return from_device_bf16(ct_)
+
+
+def reference(ta, tb, m, n, k, alpha, a, lda, b, ldb, beta, c, ldc):
+    want = c.copy()
+    status, want64 = oracle.bgemm_f64(ta, tb, m, n, k, alpha, a, lda, b, ldb, beta, want, ldc,
+                                      want64=True)
+    assert status == 0
+    return want, want64
+
+
+def variant_count():
+    return _native.library().camblas_hip_kernel_count(2)
+
+
+@pytest.mark.parametrize("variant", range(8))
+@pytest.mark.parametrize("split,n_out,pad", [(1, 300, 4), (3, 300, 4), (1, 301, 4), (2, 301, 4)])
+def test_tn_every_variant(device, variant, split, n_out, pad):
+    assert variant < variant_count()
+    # N is not a multiple of any tile (301: not of 4 either, so the scalar store path runs);
+    # M=70 spans tiles; K=328 leaves a K tail
+    m_rows, k = 70, 328
+    lda, ldb, ldc = k + 8, k + 16, n_out + pad
+    w = oracle.fill_normal_bf16(20 + variant, (n_out * lda,))
+    x = oracle.fill_normal_bf16(40 + variant, (m_rows * ldb,))
+    c0 = oracle.fill_normal_bf16(60, (m_rows * ldc,))
+    for alpha, beta in ((1.0, 0.0), (0.5, -1.5)):
+        got = run_bgemm(device, "T", "N", n_out, m_rows, k, alpha, w, lda, x, ldb, beta, c0, ldc,
+                        override=(variant, split))
+        want, want64 = reference("T", "N", n_out, m_rows, k, alpha, w, lda, x, ldb, beta, c0, ldc)
+        got2d = got.reshape(m_rows, ldc)
+        error = rel_frobenius(oracle.bf16_to_f32(got2d[:, :n_out]), want64.reshape(m_rows, n_out))
+        assert error <= TOLERANCE, (variant, split, alpha, beta, error)
+        assert np.array_equal(got2d[:, n_out:], c0.reshape(m_rows, ldc)[:, n_out:])
+
+
+@pytest.mark.parametrize("tokens", [1, 8, 32, 33, 64, 65, 200])
+def test_planned_linear_shapes(device, tokens):
+    # aligned fast path as F.linear produces it; planner picks variant and split-K
+    outputs, inner = 1024 + 128, 2048
+    w = oracle.fill_normal_bf16(70, (outputs, inner), std=0.02)
+    x = oracle.fill_normal_bf16(71 + tokens, (tokens, inner))
+    native = _native.context(device)
+    native.call("reset_stats")
+    y = _kernels.linear(to_device_bf16(x, device), to_device_bf16(w, device))
+    torch.cuda.synchronize()
+    assert _native.stats(device)["lt"] == 1
+    assert rel_frobenius(bf16_values(y), oracle.linear_bf16_f64(x, w)) <= TOLERANCE
+    # changed-input rerun: nothing about the previous call may be cached
+    x2 = oracle.fill_normal_bf16(900 + tokens, (tokens, inner))
+    y2 = _kernels.linear(to_device_bf16(x2, device), to_device_bf16(w, device))
+    assert rel_frobenius(bf16_values(y2), oracle.linear_bf16_f64(x2, w)) <= TOLERANCE
+
+
+@pytest.mark.parametrize("ta", "NT")
+@pytest.mark.parametrize("tb", "NT")
+def test_generic_layouts_and_unaligned(device, ta, tb):
+    m, n, k = 45, 38, 51  # odd sizes: never eligible for the MFMA path
+    lda = (m if ta == "N" else k) + 1
+    ldb = (k if tb == "N" else n) + 3
+    ldc = m + 2
+    a = oracle.fill_normal_bf16(80, (lda * (k if ta == "N" else m),))
+    b = oracle.fill_normal_bf16(81, (ldb * (n if tb == "N" else k),))
+    c0 = oracle.fill_normal_bf16(82, (ldc * n,))
+    got = run_bgemm(device, ta, tb, m, n, k, 1.5, a, lda, b, ldb, 0.25, c0, ldc)
+    want, want64 = reference(ta, tb, m, n, k, 1.5, a, lda, b, ldb, 0.25, c0, ldc)
+    got2d = got.reshape(n, ldc)
+    assert rel_frobenius(oracle.bf16_to_f32(got2d[:, :m]), want64.reshape(n, m)) <= TOLERANCE
+    assert np.array_equal(got2d[:, m:], c0.reshape(n, ldc)[:, m:])
+
+
+def test_classical_algorithm_uses_generic_kernel(device):
+    outputs, tokens, inner = 256, 16, 256
+    w = oracle.fill_normal_bf16(83, (outputs, inner))
+    x = oracle.fill_normal_bf16(84, (tokens, inner))
+    c = np.zeros(tokens * outputs, np.uint16)
+    native = _native.context(device)
+    native.call("reset_stats")
+    got = run_bgemm(device, "T", "N", outputs, tokens, inner, 1.0, w.ravel(), inner, x.ravel(),
+                    inner, 0.0, c, outputs, algorithm="classical")
+    counts = _native.stats(device)
+    assert counts["classical"] == 1 and counts["lt"] == 0
+    assert rel_frobenius(oracle.bf16_to_f32(got).reshape(tokens, outputs),
+                         oracle.linear_bf16_f64(x, w)) <= TOLERANCE
+
+
+@pytest.mark.parametrize("override", [None, (0, 1), (4, 2)])
+def test_exact_identity_and_fp32_accumulation(device, override):
+    # identity placement (ref: tests/test_bfloat16.py:94-110): W = I gives y = x exactly
+    size = 256
+    eye = oracle.f32_to_bf16(np.eye(size, dtype=np.float32))
+    x = oracle.f32_to_bf16(np.arange(32 * size, dtype=np.float32).reshape(32, size) % 251 - 125)
+    got = run_bgemm(device, "T", "N", size, 32, size, 1.0, eye.ravel(), size, x.ravel(), size, 0.0,
+                    np.full(32 * size, 0x7FC0, np.uint16), size, override=override)
+    assert np.array_equal(got.reshape(32, size), x)
+    # [256, 1, -256] . [1, 1, 1] = 1 only when the accumulator is wider than BF16
+    w = np.zeros((size, size), np.float32)
+    w[:, 0], w[:, 1], w[:, 2] = 256.0, 1.0, -256.0
+    ones = np.zeros((8, size), np.float32)
+    ones[:, :3] = 1.0
+    got = run_bgemm(device, "T", "N", size, 8, size, 1.0, oracle.f32_to_bf16(w).ravel(), size,
+                    oracle.f32_to_bf16(ones).ravel(), size, 0.0, np.zeros(8 * size, np.uint16),
+                    size, override=override)
+    assert np.array_equal(oracle.bf16_to_f32(got), np.ones(8 * size, np.float32))
+
+
+def test_alpha_zero_beta_and_nan_semantics(device):
+    outputs, tokens, inner = 128, 8, 128
+    w = oracle.fill_normal_bf16(85, (outputs * inner,))
+    x = oracle.fill_normal_bf16(86, (tokens * inner,))
+    nan_c = np.full(tokens * outputs, 0x7FC0, np.uint16)
+    # beta == 0 never reads C
+    got = run_bgemm(device, "T", "N", outputs, tokens, inner, 1.0, w, inner, x, inner, 0.0, nan_c,
+                    outputs)
+    assert np.isfinite(oracle.bf16_to_f32(got)).all()
+    # alpha == 0, beta == 0 writes +0 without reading; beta == 1 is a no-op
+    got = run_bgemm(device, "T", "N", outputs, tokens, inner, 0.0, w, inner, x, inner, 0.0, nan_c,
+                    outputs)
+    assert not got.any()
+    c = oracle.fill_normal_bf16(87, (tokens * outputs,))
+    got = run_bgemm(device, "T", "N", outputs, tokens, inner, 0.0, w, inner, x, inner, 1.0, c,
+                    outputs)
+    assert np.array_equal(got, c)
+    got = run_bgemm(device, "T", "N", outputs, tokens, inner, 0.0, w, inner, x, inner, 0.5, c,
+                    outputs)
+    assert np.array_equal(got, oracle.f32_to_bf16(np.float32(0.5) * oracle.bf16_to_f32(c)))
+    # NaN in an operand propagates to its output row only (ref: tests/test_bfloat16.py:132-139)
+    x_nan = x.copy().reshape(tokens, inner)
+    x_nan[3, 17] = 0x7FC0
+    got = run_bgemm(device, "T", "N", outputs, tokens, inner, 1.0, w, inner, x_nan.ravel(), inner,
+                    0.0, nan_c, outputs).reshape(tokens, outputs)
+    values = oracle.bf16_to_f32(got)
+    assert np.isnan(values[3]).all() and np.isfinite(np.delete(values, 3, axis=0)).all()
+
+
+def test_addmm_beta_one_and_errors(device):
+    tokens, outputs, inner = 96, 384, 512
+    x = oracle.fill_normal_bf16(88, (tokens, inner))
+    w = oracle.fill_normal_bf16(89, (outputs, inner), std=0.02)
+    c = oracle.fill_normal_bf16(90, (tokens, outputs))
+    y = _kernels.addmm(to_device_bf16(c, device), to_device_bf16(x, device),
+                       to_device_bf16(w, device).t(), beta=1.0)
+    want = oracle.linear_bf16_f64(x, w) + oracle.bf16_to_f32(c).astype(np.float64)
+    assert rel_frobenius(bf16_values(y), want) <= TOLERANCE
+    native = _native.context(device)
+    lib = _native.library()
+    buffer = to_device_bf16(c, device)
+    status = lib.camblas_cuda_bgemm(native.handle, b"T", b"N", 8, 8, 8, 1.0, ptr(buffer), 8,
+                                    ptr(buffer), 8, 0.0, ptr(buffer), 8)
+    assert status == -1 and b"aliased BF16 GEMM operand" in lib.camblas_cuda_error(native.handle)
+    status = lib.camblas_cuda_bgemm(native.handle, b"T", b"N", 8, 8, 8, 1.0, ptr(buffer), 4,
+                                    ptr(buffer), 8, 0.0, ptr(buffer), 8)
+    assert status == -1 and b"leading dimension" in lib.camblas_cuda_error(native.handle)
+
+
+def test_long_k_llama_dims(device):
+    # down-projection depth (ref: tests/test_bfloat16.py:207-217): K = 28672
+    tokens, outputs, inner = 32, 512, 28672
+    x = oracle.fill_normal_bf16(91, (tokens, inner))
+    w = oracle.fill_normal_bf16(92, (outputs, inner), std=0.02)
+    y = _kernels.linear(to_device_bf16(x, device), to_device_bf16(w, device))
+    assert rel_frobenius(bf16_values(y), oracle.linear_bf16_f64(x, w)) <= TOLERANCE

@@ -1,0 +1,141 @@
+"""FP8 E4M3fn block-scaled linear (1x128 activation groups, 128x128 weight blocks) against the
+CPU oracle.
+
+Bars: scale/block indexing bit-exact (exact-arithmetic cases with a distinct power-of-two scale per
+block must reproduce the oracle's BF16 bits), outputs within relative Frobenius 1e-2 of the FP64
+accumulation of the dequantised operands; the ordered-FMA restatement (camblas/_hopper.py:168-182)
+is matched to within one BF16 unit in the last place on random data. Known-answer bytes follow
+tests/test_quantized.py:160-216 (0x38 = 1.0, 0x40 = 2.0, 0x30 = 0.5, 0x7f = NaN).
+"""
+
+import numpy as np
+import pytest
+import torch
+
+import oracle
+from camblas_amd import _kernels, _native
+from helpers import (bf16_ulp_distance, bf16_values, from_device_bf16, from_device_fp8, rel_frobenius,
+                     to_device_bf16, to_device_fp8)
+
+pytestmark = pytest.mark.gpu
+TOLERANCE = 1e-2
+
+
+def run(device, a, a_scale, w, w_scale, override=None):
+    native = _native.context(device)
+    if override is not None:
+        native.call("hip_set_plan_override", override[0], override[1])
+    try:
+        out = _kernels.fp8_block_matmul(
+            to_device_fp8(a, device), torch.from_numpy(a_scale).to(device),
+            to_device_fp8(w, device), torch.from_numpy(w_scale).to(device))
+        torch.cuda.synchronize()
+    finally:
+        native.call("hip_set_plan_override", -1, 0)
+    return out
+
+
+@pytest.mark.parametrize("variant", range(4))
+@pytest.mark.parametrize("split", [1, 2])
+@pytest.mark.parametrize("rows", [1, 16, 70])
+def test_random_blocks_every_variant(device, variant, split, rows):
+    outputs, inner = 300, 512  # partial last 128-row weight block, partial tiles
+    a, a_scale = oracle.fill_fp8_blocks(100 + rows, rows, inner, 1)
+    w, w_scale = oracle.fill_fp8_blocks(200, outputs, inner, 128)
+    out = run(device, a, a_scale, w, w_scale, override=(variant, split))
+    want64 = oracle.fp8_block_matmul_f64(a, a_scale, w, w_scale)
+    assert rel_frobenius(bf16_values(out), want64) <= TOLERANCE
+    if split == 1:
+        ordered = oracle.fp8_block_matmul(a, a_scale, w, w_scale)
+        distance = bf16_ulp_distance(from_device_bf16(out), ordered)
+        assert distance.max() <= 1, distance.max()
+        assert (distance == 0).mean() > 0.98
+
+
+@pytest.mark.parametrize("rows", [1, 16, 256])
+def test_planned_shapes(device, rows):
+    outputs, inner = 1536, 1024
+    a, a_scale = oracle.fill_fp8_blocks(300 + rows, rows, inner, 1)
+    w, w_scale = oracle.fill_fp8_blocks(301, outputs, inner, 128)
+    out = run(device, a, a_scale, w, w_scale)
+    assert rel_frobenius(bf16_values(out), oracle.fp8_block_matmul_f64(a, a_scale, w, w_scale)) <= TOLERANCE
+
+
+@pytest.mark.parametrize("override", [None, (0, 1), (1, 1), (2, 1), (3, 1)])
+def test_scale_indexing_is_bit_exact(device, override):
+    # every product is a small integer and every scale a distinct power of two, so the FMA chain
+    # is exact: any wrong (row, group) or (block, group) scale index changes the bits
+    rows, outputs, inner = 40, 384, 512
+    groups, blocks = inner // 128, outputs // 128
+    rng = np.random.default_rng(5)
+    small = np.array([0x00, 0x38, 0x40, 0x30, 0xB8, 0xC0], dtype=np.uint8)  # 0, 1, 2, .5, -1, -2
+    a = small[rng.integers(0, len(small), size=(rows, inner))]
+    w = small[rng.integers(0, len(small), size=(outputs, inner))]
+    a_scale = np.exp2(rng.integers(-6, 6, size=(rows, groups))).astype(np.float32)
+    w_scale = np.exp2(-(np.arange(blocks * groups).reshape(blocks, groups) % 7)).astype(np.float32)
+    out = run(device, a, a_scale, w, w_scale, override=override)
+    want = oracle.fp8_block_matmul(a, a_scale, w, w_scale)
+    assert np.array_equal(from_device_bf16(out), want)
+
+
+def test_known_answer_bytes_and_nan(device):
+    rows, outputs, inner = 2, 256, 256
+    a = np.full((rows, inner), 0x38, np.uint8)       # 1.0
+    w = np.full((outputs, inner), 0x40, np.uint8)    # 2.0
+    w[128:] = 0x30                                   # 0.5 in the second weight block
+    a_scale = np.array([[1.0, 0.5], [2.0, 2.0]], np.float32)
+    w_scale = np.array([[1.0, 1.0], [4.0, 8.0]], np.float32)
+    out = bf16_values(run(device, a, a_scale, w, w_scale))
+    # row 0: block 0 -> 128*2*(1*1) + 128*2*(0.5*1) = 384; block 1 -> 64*(1*4) + 64*(0.5*8) = 512
+    assert (out[0, :128] == 384).all() and (out[0, 128:] == 512).all()
+    # row 1: block 0 -> 2 * 128*2*(2*1) = 1024; block 1 -> 64*(2*4) + 64*(2*8) = 1536
+    assert (out[1, :128] == 1024).all() and (out[1, 128:] == 1536).all()
+    a[1, 5] = 0x7F  # NaN byte poisons its row only
+    out = bf16_values(run(device, a, a_scale, w, w_scale))
+    assert np.isnan(out[1]).all() and np.isfinite(out[0]).all()
+    # zero activations give +0
+    out = from_device_bf16(run(device, np.zeros_like(a), a_scale, w, w_scale))
+    assert not out.any()
+
+
+def test_weight_scale_doubling_doubles_output(device):
+    rows, outputs, inner = 16, 256, 384
+    a, a_scale = oracle.fill_fp8_blocks(400, rows, inner, 1)
+    w, w_scale = oracle.fill_fp8_blocks(401, outputs, inner, 128)
+    base = bf16_values(run(device, a, a_scale, w, w_scale))
+    doubled = bf16_values(run(device, a, a_scale, w, w_scale * np.float32(2)))
+    assert np.array_equal(doubled, base * 2)
+
+
+@pytest.mark.parametrize("rows,inner", [(1, 7168), (5, 256), (33, 1024)])
+def test_activation_quantiser_is_bit_exact(device, rows, inner):
+    x = oracle.fill_normal_bf16(500 + rows, (rows, inner))
+    x[0, :128] = 0  # an all-zero group keeps amax at the 1e-10 floor
+    q, scale = _kernels.fp8_quantise_1x128(to_device_bf16(x, device))
+    torch.cuda.synchronize()
+    want_q, want_scale = oracle.quantise_1x128(x)
+    assert np.array_equal(scale.cpu().numpy(), want_scale)
+    assert np.array_equal(from_device_fp8(q), want_q)
+    # invariant: the group maximum maps to +-448 exactly (byte 0x7e / 0xfe)
+    values = np.abs(oracle.e4m3_to_f32(from_device_fp8(q))).reshape(rows, inner // 128, 128)
+    assert (values.max(axis=2)[1:] == 448).all()
+
+
+def test_block_linear_with_dynamic_quantisation(device):
+    rows, outputs, inner = 16, 512, 1024
+    x = oracle.fill_normal_bf16(600, (rows, inner))
+    w, w_scale = oracle.fill_fp8_blocks(601, outputs, inner, 128)
+    out = _kernels.fp8_block_linear(to_device_bf16(x, device), to_device_fp8(w, device),
+                                    torch.from_numpy(w_scale).to(device))
+    q, scale = oracle.quantise_1x128(x)
+    assert rel_frobenius(bf16_values(out), oracle.fp8_block_matmul_f64(q, scale, w, w_scale)) <= TOLERANCE
+
+
+def test_invalid_arguments(device):
+    native = _native.context(device)
+    lib = _native.library()
+    assert lib.camblas_cuda_fp8_block_matmul(native.handle, 1, 128, 100, None, None, None, None, None) == -1
+    assert b"invalid FP8 block matrix dimensions" in lib.camblas_cuda_error(native.handle)
+    assert lib.camblas_cuda_fp8_block_matmul(native.handle, 0, 128, 128, None, None, None, None, None) == 0
+    assert lib.camblas_cuda_fp8_block_matmul(native.handle, 1, 128, 128, None, None, None, None, None) == -1
+    assert b"invalid FP8 block matrix buffers" in lib.camblas_cuda_error(native.handle)

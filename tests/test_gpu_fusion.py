@@ -1,0 +1,162 @@
+"""Decode epilogues (SiLU*up, SwiGLU, RMSNorm family, rotary embedding, GQA decode attention) and
+the decoder-layer decode step against the CPU oracle.
+
+The elementwise/RMS oracles restate src/cuda/inference_fusion.cuh; as in the reference's
+tolerance-form tests (tests/test_residual_rms.py:64-69, tests/test_inference_fusion.py:64-101) the
+GPU result may differ from the CPU one by one unit in the last place of the storage type where
+expf/rsqrt or the reduction order differ; residual sums (pure BF16 adds) must be bit-exact.
+RoPE and attention have no reference code: FP64 textbook formulas, relative Frobenius <= 1e-2.
+"""
+
+import ctypes as ct
+
+import numpy as np
+import pytest
+import torch
+
+import oracle
+from camblas_amd import _kernels, _native
+from helpers import (bf16_ulp_distance, bf16_values, from_device_bf16, ptr, rel_frobenius,
+                     to_device_bf16)
+
+pytestmark = pytest.mark.gpu
+
+
+def close_bf16(got_bits, want_bits, ulps=1, exact_fraction=0.97):
+    distance = bf16_ulp_distance(got_bits, want_bits)
+    assert distance.max() <= ulps, distance.max()
+    assert (distance == 0).mean() >= exact_fraction, (distance == 0).mean()
+
+
+@pytest.mark.parametrize("count", [8 * 1000, 1001])
+def test_silu_multiply_bf16(device, count):
+    gate = oracle.fill_normal_bf16(1, (count,), std=3.0)
+    up = oracle.fill_normal_bf16(2, (count,))
+    out = _kernels.silu_multiply(to_device_bf16(gate, device), to_device_bf16(up, device))
+    close_bf16(from_device_bf16(out), oracle.silu_multiply(2, gate, up))
+
+
+def test_silu_multiply_f32_and_in_place(device):
+    gate = oracle.fill_normal(3, (4099,), std=3.0)
+    up = oracle.fill_normal(4, (4099,))
+    g = torch.from_numpy(gate).to(device)
+    out = _kernels.silu_multiply(g, torch.from_numpy(up).to(device), out=g)
+    want = oracle.silu_multiply(0, gate, up)
+    np.testing.assert_allclose(out.cpu().numpy(), want, rtol=2e-6, atol=1e-7)
+
+
+@pytest.mark.parametrize("limit", [0.0, 1.5])
+@pytest.mark.parametrize("routed", [False, True])
+def test_swiglu_bf16(device, limit, routed):
+    rows, width = 7, 520
+    gate = oracle.fill_normal_bf16(5, (rows, width), std=2.0)
+    up = oracle.fill_normal_bf16(6, (rows, width), std=2.0)
+    routing = oracle.fill_uniform(7, (rows,), 0.1, 1.0) if routed else None
+    out = _kernels.swiglu(to_device_bf16(gate, device), to_device_bf16(up, device), limit,
+                          torch.from_numpy(routing).to(device) if routed else None)
+    close_bf16(from_device_bf16(out), oracle.swiglu(2, width, limit, gate, up, routing))
+    # NaN inputs survive the clamp (comparisons, not fmin/fmax)
+    gate[0, 0] = 0x7FC0
+    out = _kernels.swiglu(to_device_bf16(gate, device), to_device_bf16(up, device), limit)
+    assert np.isnan(bf16_values(out)[0, 0])
+
+
+@pytest.mark.parametrize("rows,width", [(32, 8192), (1, 2048), (3, 4104), (5, 1000), (2, 16384)])
+@pytest.mark.parametrize("round_before_weight", [True, False])
+def test_add_rms_norm_rows_bf16(device, rows, width, round_before_weight):
+    x = oracle.fill_normal_bf16(10, (rows, width))
+    r = oracle.fill_normal_bf16(11, (rows, width))
+    w = oracle.fill_normal_bf16(12, (width,), mean=1.0, std=0.02)
+    added, out = _kernels.add_rms_norm(to_device_bf16(x, device), to_device_bf16(r, device),
+                                       to_device_bf16(w, device), 1e-5, round_before_weight)
+    want_added, want_out = oracle.rms_norm(2, 2, 1e-5, x, w, residual=r,
+                                           round_before_weight=round_before_weight)
+    assert np.array_equal(from_device_bf16(added), want_added)
+    close_bf16(from_device_bf16(out), want_out)
+    plain = _kernels.rms_norm(to_device_bf16(x, device), to_device_bf16(w, device), 1e-5,
+                              round_before_weight)
+    close_bf16(from_device_bf16(plain),
+               oracle.rms_norm(2, 2, 1e-5, x, w, round_before_weight=round_before_weight))
+
+
+def test_reference_single_row_entry_points(device):
+    width = 4096
+    x = oracle.fill_normal_bf16(13, (1, width))
+    r = oracle.fill_normal_bf16(14, (1, width))
+    w = oracle.fill_normal_bf16(15, (width,), mean=1.0, std=0.1)
+    native = _native.context(device)
+    xt, rt, wt = (to_device_bf16(v, device) for v in (x, r, w))
+    added, out = torch.empty_like(xt), torch.empty_like(xt)
+    native.call("add_rms_norm", 2, width, ct.c_float(1e-6), ptr(xt), ptr(rt), ptr(wt), ptr(added),
+                ptr(out))
+    want_added, want_out = oracle.rms_norm(2, 2, 1e-6, x, w, residual=r)
+    assert np.array_equal(from_device_bf16(added), want_added)
+    close_bf16(from_device_bf16(out), want_out)
+    wf = torch.from_numpy(oracle.bf16_to_f32(w)).to(device)
+    native.call("rms_norm_decode", 2, 0, width, ct.c_float(1e-6), 0, 1, ptr(xt), ptr(wf), ptr(out))
+    close_bf16(from_device_bf16(out),
+               oracle.rms_norm(2, 0, 1e-6, x, oracle.bf16_to_f32(w), round_before_weight=False))
+    native.call("rms_norm", 2, 1, width, ct.c_float(1e-6), ptr(xt), ptr(wt), ptr(out))
+    close_bf16(from_device_bf16(out), oracle.rms_norm(2, 2, 1e-6, x, w))
+    lib = _native.library()
+    assert lib.camblas_cuda_add_rms_norm(native.handle, 2, 100, 1e-6, ptr(xt), ptr(rt), ptr(wt),
+                                         ptr(added), ptr(out)) == -1
+    assert b"invalid residual RMS arguments" in lib.camblas_cuda_error(native.handle)
+    # squares + scale helpers keep the framework's own mean (ref: torch_bindings.cpp:654-666)
+    squares = torch.empty((1, width), dtype=torch.float32, device=device)
+    native.call("bfloat16_square", width, ptr(xt), ptr(squares))
+    values = oracle.bf16_to_f32(x)
+    assert np.array_equal(squares.cpu().numpy(), values * values)
+    means = squares.mean(dim=1)
+    native.call("rms_scale", 2, width, width, ct.c_float(1e-6), ptr(xt), ptr(wt), ptr(means),
+                ptr(out))
+    close_bf16(from_device_bf16(out), oracle.rms_norm(2, 2, 1e-6, x, w))
+
+
+def test_rms_norm_f32(device):
+    rows, width = 4, 3000
+    x = oracle.fill_normal(16, (rows, width))
+    w = oracle.fill_normal(17, (width,), mean=1.0, std=0.1)
+    out = _kernels.rms_norm(torch.from_numpy(x).to(device), torch.from_numpy(w).to(device), 1e-6)
+    np.testing.assert_allclose(out.cpu().numpy(), oracle.rms_norm(0, 0, 1e-6, x, w), rtol=3e-6)
+
+
+def test_rope(device):
+    tokens, heads, dim = 5, 9, 128
+    x = oracle.fill_normal_bf16(20, (tokens, heads, dim))
+    positions = np.array([0, 1, 17, 2047, 100000], np.int32)
+    out = _kernels.rope(to_device_bf16(x, device), torch.from_numpy(positions).to(device), 5e5)
+    want = oracle.rope(x, positions, 5e5)
+    assert np.array_equal(from_device_bf16(out)[0], x[0])  # position 0 is the identity
+    distance = bf16_ulp_distance(from_device_bf16(out)[:3], want[:3])
+    assert distance.max() <= 1 and (distance == 0).mean() > 0.97
+    wanted = oracle.bf16_to_f32(want)
+    assert (np.abs(bf16_values(out) - wanted)[:4] <= 0.01 * np.abs(wanted[:4]) + 2e-3).all()
+    assert rel_frobenius(bf16_values(out), oracle.bf16_to_f32(want)) <= 1e-2
+
+
+@pytest.mark.parametrize("batch,q_heads,kv_heads,context", [(3, 16, 2, 700), (2, 8, 8, 256),
+                                                            (2, 12, 4, 300), (1, 64, 8, 2048)])
+def test_gqa_decode_attention(device, batch, q_heads, kv_heads, context):
+    dim = 128
+    q = oracle.fill_normal_bf16(30, (batch, q_heads, dim))
+    k = oracle.fill_normal_bf16(31, (batch, context, kv_heads, dim))
+    v = oracle.fill_normal_bf16(32, (batch, context, kv_heads, dim))
+    lengths = np.array([context, 1, 257][:batch], np.int32)
+    scale = dim**-0.5
+    out = _kernels.gqa_decode_attention(to_device_bf16(q, device), to_device_bf16(k, device),
+                                        to_device_bf16(v, device),
+                                        torch.from_numpy(lengths).to(device), scale)
+    want = oracle.gqa_decode(q, k, v, lengths, scale)
+    assert rel_frobenius(bf16_values(out), oracle.bf16_to_f32(want)) <= 1e-2
+    wanted = oracle.bf16_to_f32(want)
+    assert (np.abs(bf16_values(out) - wanted) <= 0.01 * np.abs(wanted) + 2e-3).all()
+    # a single valid position returns that value row exactly
+    if batch > 1:
+        group = q_heads // kv_heads
+        expect = np.repeat(v[1, 0], group, axis=0)
+        assert np.array_equal(from_device_bf16(out)[1], expect)
+    full = _kernels.gqa_decode_attention(to_device_bf16(q, device), to_device_bf16(k, device),
+                                         to_device_bf16(v, device), None, scale)
+    want_full = oracle.gqa_decode(q, k, v, None, scale)
+    assert rel_frobenius(bf16_values(full), oracle.bf16_to_f32(want_full)) <= 1e-2

@@ -1,0 +1,144 @@
+"""FP32 GEMM/GEMV through the C ABI against the CPU oracle.
+
+Mirrors the reference's strategy (tests/test_cuda.py:38-58, :285-354; tests/test_float_gemv.py):
+independent FP64 product, padded leading dimensions with untouched padding, beta=0 over NaN-filled
+C, alpha=0 semantics, exact analytic cases. Tolerance: relative Frobenius error <= 1e-5 against the
+FP64 accumulation.
+"""
+
+import ctypes as ct
+
+import numpy as np
+import pytest
+import torch
+
+import oracle
+from camblas_amd import _native
+from helpers import ptr, rel_frobenius
+
+pytestmark = pytest.mark.gpu
+TOLERANCE = 1e-5
+
+
+def run_sgemm(device, ta, tb, m, n, k, alpha, a, lda, b, ldb, beta, c, ldc, algorithm="auto"):
+    at, bt, ct_ = (torch.from_numpy(v).to(device) for v in (a, b, c))
+    with _native.algorithm(algorithm):
+        native = _native.context(device)
+        native.call("sgemm", ta.encode(), tb.encode(), m, n, k, ct.c_float(alpha), ptr(at), lda,
+                    ptr(bt), ldb, ct.c_float(beta), ptr(ct_), ldc)
+    torch.cuda.synchronize()
+    return ct_.cpu().numpy()
+
+
+@pytest.mark.parametrize("ta", "NT")
+@pytest.mark.parametrize("tb", "NT")
+@pytest.mark.parametrize("shape", [(37, 29, 53), (128, 96, 200), (65, 130, 17)])
+def test_sgemm_padded_alpha_beta(device, ta, tb, shape):
+    m, n, k = shape
+    lda = (m if ta == "N" else k) + 3
+    ldb = (k if tb == "N" else n) + 2
+    ldc = m + 5
+    a = oracle.fill_uniform(1, (lda * (k if ta == "N" else m),))
+    b = oracle.fill_uniform(2, (ldb * (n if tb == "N" else k),))
+    c0 = oracle.fill_uniform(3, (ldc * n,))
+    got = run_sgemm(device, ta, tb, m, n, k, 1.25, a, lda, b, ldb, -0.5, c0.copy(), ldc)
+    want = c0.copy()
+    want64 = oracle.sgemm_f64(ta, tb, m, n, k, 1.25, a, lda, b, ldb, -0.5, want, ldc, want64=True)
+    got2d, c2d = got.reshape(n, ldc), c0.reshape(n, ldc)
+    assert rel_frobenius(got2d[:, :m].ravel(), want64.reshape(n, m).ravel()) <= TOLERANCE
+    assert np.array_equal(got2d[:, m:], c2d[:, m:]), "padding rows of C were written"
+    # the reference's scalar-order result is within the same bar of the FP64 product
+    scalar = c0.copy()
+    oracle.sgemm(ta, tb, m, n, k, 1.25, a, lda, b, ldb, -0.5, scalar, ldc)
+    assert rel_frobenius(got2d[:, :m], scalar.reshape(n, ldc)[:, :m]) <= 5 * TOLERANCE
+
+
+def test_sgemm_beta_zero_ignores_nan_and_alpha_zero(device):
+    m, n, k = 70, 33, 40
+    a = oracle.fill_uniform(4, (m * k,))
+    b = oracle.fill_uniform(5, (k * n,))
+    c = np.full(m * n, np.nan, dtype=np.float32)
+    got = run_sgemm(device, "N", "N", m, n, k, 1.0, a, m, b, k, 0.0, c, m)
+    want = np.zeros(m * n, np.float32)
+    want64 = oracle.sgemm_f64("N", "N", m, n, k, 1.0, a, m, b, k, 0.0, want, m, want64=True)
+    assert np.isfinite(got).all() and rel_frobenius(got, want64) <= TOLERANCE
+    # alpha == 0: beta scaling only; beta == 0 writes zeros over NaN; beta == 1 leaves C alone
+    c = np.full(m * n, np.nan, dtype=np.float32)
+    assert not run_sgemm(device, "N", "N", m, n, k, 0.0, a, m, b, k, 0.0, c, m).any()
+    c = oracle.fill_uniform(6, (m * n,))
+    assert np.array_equal(run_sgemm(device, "N", "N", m, n, k, 0.0, a, m, b, k, 1.0, c.copy(), m), c)
+    assert np.array_equal(
+        run_sgemm(device, "N", "N", m, n, k, 0.0, a, m, b, k, 2.0, c.copy(), m), np.float32(2.0) * c
+    )
+
+
+def test_sgemm_full_precision_not_reduced(device):
+    # (1 + 2^-12)^2 needs more than a 10-bit mantissa: a reduced-precision matrix path would
+    # return exactly 1 (ref: tests/test_cuda.py:245-270)
+    m = n = k = 64
+    value = np.float32(1.0 + 2.0**-12)
+    a = np.zeros((m, k), np.float32)
+    a[np.arange(m), np.arange(m)] = value
+    b = a.copy()
+    got = run_sgemm(device, "N", "N", m, n, k, 1.0, a.ravel(), m, b.ravel(), k, 0.0,
+                    np.zeros(m * n, np.float32), m).reshape(n, m)
+    assert got[5, 5] == np.float32(value * value)
+
+
+def test_sgemm_config1_row_major_2048(device):
+    # row-major C = A.B arrives as the swapped column-major call (ref: src/cblas_shim.c:184-199)
+    size = 2048
+    a = oracle.fill_uniform(101, (size, size))
+    b = oracle.fill_uniform(102, (size, size))
+    got = run_sgemm(device, "N", "N", size, size, size, 1.0, b.ravel(), size, a.ravel(), size, 0.0,
+                    np.zeros(size * size, np.float32), size).reshape(size, size)
+    want = a.astype(np.float64) @ b.astype(np.float64)
+    assert rel_frobenius(got, want) <= TOLERANCE
+
+
+@pytest.mark.parametrize("rows,inner,pad", [(1024, 4096, 0), (1536, 4100, 8), (1027, 8192, 4)])
+def test_sgemv_shortcut(device, rows, inner, pad):
+    ld = inner + pad
+    w = oracle.fill_uniform(7, (rows, ld))
+    x = oracle.fill_uniform(8, (inner,))
+    y0 = oracle.fill_uniform(9, (rows,))
+    native = _native.context(device)
+    native.call("reset_stats")
+    got = run_sgemm(device, "T", "N", rows, 1, inner, 0.75, w.ravel(), ld, x, inner, 0.5, y0.copy(),
+                    rows)
+    want = oracle.sgemv_f64(0.75, w[:, :inner], x, 0.5, y0.copy())
+    assert rel_frobenius(got, want) <= TOLERANCE
+    assert _native.stats(device)["classical"] >= 1
+
+
+def test_sgemv_exact_cancellation(device):
+    # ref: tests/test_float_gemv.py:69-90 style: sparse rows and exact cancellation
+    rows, inner = 1024, 4096
+    w = np.zeros((rows, inner), np.float32)
+    x = np.ones(inner, np.float32)
+    w[0, 0], w[0, inner - 1] = 16777216.0, -16777216.0
+    w[0, 7] = 3.0
+    w[1, 100] = 2.5
+    w[rows - 1, inner - 1] = -4.0
+    got = run_sgemm(device, "T", "N", rows, 1, inner, 1.0, w.ravel(), inner, x, inner, 0.0,
+                    np.full(rows, np.nan, np.float32), rows)
+    want = np.zeros(rows, np.float32)
+    want[0], want[1], want[rows - 1] = 3.0, 2.5, -4.0
+    assert np.array_equal(got, want)
+
+
+def test_invalid_arguments_report_errors(device):
+    native = _native.context(device)
+    lib = _native.library()
+    status = lib.camblas_cuda_sgemm(native.handle, b"X", b"N", 1, 1, 1, 1.0, None, 1, None, 1, 0.0,
+                                    None, 1)
+    assert status == -1 and b"invalid GEMM arguments" in lib.camblas_cuda_error(native.handle)
+    status = lib.camblas_cuda_sgemm(native.handle, b"N", b"N", 4, 4, 4, 1.0, None, 4, None, 4, 0.0,
+                                    None, 4)
+    assert status == -1
+    assert b"invalid device pointer or leading dimension" in lib.camblas_cuda_error(native.handle)
+    assert lib.camblas_cuda_sgemm(native.handle, b"N", b"N", 0, 4, 4, 1.0, None, 1, None, 4, 0.0,
+                                  None, 1) == 0
+    assert lib.camblas_cuda_dgemm(native.handle, b"N", b"N", 1, 1, 1, 1.0, None, 1, None, 1, 0.0,
+                                  None, 1) == -1
+    assert b"not provided" in lib.camblas_cuda_error(native.handle)
