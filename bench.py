@@ -1,0 +1,290 @@
+"""Benchmark of the linear hot path on one MI355X.
+
+`python bench.py --gpus 1 --steps K --warmup W` prints ONE JSON line. The headline workload is the
+BF16 decode linear y = x W^T with W [28672, 8192] (Llama-70B up-projection) and x [M, 8192] for
+M in {1, 8, 32}: one "step" is one pass over the three batch sizes, each through
+camblas_cuda_bgemm('T','N') on resident operands. Three weight copies (3 x 470 MB, more than the
+256 MB last-level cache) are rotated so every launch streams its weights from HBM. `value` is the
+algorithmic HBM traffic of the timed steps divided by wall time (host clock around K steps with a
+device synchronisation on both sides).
+
+The line also carries
+  roofline      the dominant kernel (M=32 launch) timed with HIP events on the launch stream,
+  cpu_baseline  the CPU oracle port of the same BF16 linear on a bounded sample of weight rows,
+  also          the other configurations (BF16 prefill linear and addmm, FP8 block-scaled linear,
+                FP32 SGEMM, decoder-layer decode step), each with its own roofline fraction, and
+                the reference's own CPU SGEMM when oracle/_ref is present.
+"""
+
+import argparse
+import json
+import os
+import sys
+import time
+from pathlib import Path
+
+ROOT = Path(__file__).resolve().parent
+sys.path.insert(0, str(ROOT))
+
+HBM_PEAK = 8.0e12
+BF16_PEAK = 2.5e15
+FP8_PEAK = 5.0e15
+FP32_PEAK = 157.3e12
+
+OUTPUTS, INNER = 28672, 8192
+BATCHES = (1, 8, 32)
+
+
+def decode_bytes(tokens):
+    return OUTPUTS * INNER * 2 + tokens * INNER * 2 + tokens * OUTPUTS * 2
+
+
+def event_time(torch, launch, warmup, iterations):
+    """Average seconds per launch measured with events on torch's current stream, which is the
+    stream the library context enqueues on."""
+    for index in range(warmup):
+        launch(index)
+    stream = torch.cuda.current_stream()
+    start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    start.record(stream)
+    for index in range(iterations):
+        launch(index)
+    stop.record(stream)
+    stop.synchronize()
+    return start.elapsed_time(stop) * 1e-3 / iterations
+
+
+def cpu_port_baseline(budget_seconds=12.0):
+    """Time the CPU oracle's BF16 linear (FP64 accumulate, OpenMP) on a bounded sample of rows."""
+    import oracle
+
+    cores = len(os.sched_getaffinity(0))
+    tokens = 32
+    x = oracle.fill_normal_bf16(1, (tokens, INNER))
+    rows = 256
+    elapsed = 0.0
+    while True:
+        w = oracle.fill_normal_bf16(2, (rows, INNER), std=0.02)
+        out = oracle.f32_to_bf16(oracle.fill_uniform(3, (tokens, rows)) * 0)
+        begin = time.perf_counter()
+        oracle.bgemm_f64("T", "N", rows, tokens, INNER, 1.0, w, INNER, x, INNER, 0.0, out, rows)
+        elapsed = time.perf_counter() - begin
+        if elapsed * 4 > budget_seconds or rows >= OUTPUTS:
+            break
+        rows = min(OUTPUTS, rows * 4)
+    traffic = rows * INNER * 2 + tokens * INNER * 2 + tokens * rows * 2
+    return {
+        "value": round(traffic / elapsed / 1e9, 3),
+        "unit": "GB/s",
+        "cores": cores,
+        "kind": "port",
+        "sample": f"oracle_bgemm_f64 (OpenMP) on {rows} of {OUTPUTS} weight rows, M=32, K={INNER}, "
+                  f"{elapsed:.2f} s",
+    }
+
+
+def cpu_reference_sgemm():
+    """The reference's own CPU library on the FP32 2048^3 product, when it was built."""
+    import oracle
+
+    if oracle.ref() is None:
+        return None
+    size = 2048
+    a = oracle.fill_uniform(101, (size * size,))
+    b = oracle.fill_uniform(102, (size * size,))
+    c = oracle.fill_uniform(103, (size * size,)) * 0
+    threads = oracle.ref_threads_available()
+    oracle.ref_sgemm_packed(threads, "N", "N", size, size, size, 1.0, b, size, a, size, 0.0, c, size)
+    begin = time.perf_counter()
+    oracle.ref_sgemm_packed(threads, "N", "N", size, size, size, 1.0, b, size, a, size, 0.0, c, size)
+    elapsed = time.perf_counter() - begin
+    return {
+        "value": round(2.0 * size**3 / elapsed / 1e9, 2),
+        "unit": "GFLOP/s",
+        "cores": threads,
+        "kind": "reference",
+        "sample": f"camblas_sgemm shape-aware + pthread pool, 2048^3, {elapsed:.3f} s",
+    }
+
+
+def main():
+    parser = argparse.ArgumentParser()
+    parser.add_argument("--gpus", type=int, default=1)
+    parser.add_argument("--steps", type=int, default=50)
+    parser.add_argument("--warmup", type=int, default=10)
+    parser.add_argument("--skip-extras", action="store_true")
+    parser.add_argument("--skip-cpu", action="store_true")
+    args = parser.parse_args()
+    if args.gpus != 1:
+        sys.exit("bench.py: this build measures one GPU only (no collectives exist in the linear "
+                 "path); run with --gpus 1")
+
+    import torch
+
+    from camblas_amd import _kernels, _native
+
+    device = torch.device("cuda:0")
+    torch.cuda.set_device(device)
+    generator = torch.Generator(device=device).manual_seed(20261125)
+
+    def normal(shape, std=1.0, dtype=torch.bfloat16):
+        return (torch.randn(shape, device=device, generator=generator) * std).to(dtype)
+
+    weights = [normal((OUTPUTS, INNER), 0.02) for _ in range(3)]
+    inputs = {m: normal((m, INNER)) for m in BATCHES}
+    outputs = {m: torch.empty((m, OUTPUTS), dtype=torch.bfloat16, device=device) for m in BATCHES}
+
+    def step(index):
+        for position, m in enumerate(BATCHES):
+            weight = weights[(index * len(BATCHES) + position) % 3]
+            _kernels.matmul(inputs[m], weight.t(), out=outputs[m])
+
+    for index in range(args.warmup):
+        step(index)
+    torch.cuda.synchronize()
+    begin = time.perf_counter()
+    for index in range(args.steps):
+        step(index)
+    torch.cuda.synchronize()
+    elapsed = time.perf_counter() - begin
+    step_bytes = sum(decode_bytes(m) for m in BATCHES)
+    value = step_bytes * args.steps / elapsed / 1e9
+
+    # dominant kernel: the M=32 launch, timed alone with events on the launch stream
+    per_launch = {}
+    for m in BATCHES:
+        seconds = event_time(
+            torch, lambda i, m=m: _kernels.matmul(inputs[m], weights[i % 3].t(), out=outputs[m]),
+            5, 30)
+        per_launch[m] = seconds
+    _, plan_text = _native.plan_describe(2, "T", "N", OUTPUTS, 32, INNER, INNER, INNER, OUTPUTS)
+    achieved = decode_bytes(32) / per_launch[32]
+    roofline = {
+        "bound": "hbm",
+        "kernel": plan_text,
+        "achieved": round(achieved / 1e9, 1),
+        "peak": HBM_PEAK / 1e9,
+        "unit": "GB/s",
+        "frac": round(achieved / HBM_PEAK, 4),
+        "traffic": None,
+        "launch_us": round(per_launch[32] * 1e6, 2),
+    }
+
+    also = {
+        "decode_linear_us": {str(m): round(per_launch[m] * 1e6, 2) for m in BATCHES},
+        "decode_linear_gbps": {str(m): round(decode_bytes(m) / per_launch[m] / 1e9, 1)
+                               for m in BATCHES},
+    }
+    if not args.skip_extras:
+        also.update(extras(torch, _kernels, _native, device, normal))
+    result = {
+        "metric": "decode-GEMV HBM GB/s (BF16 linear W[28672,8192], M in {1,8,32}); TFLOP/s of the "
+                  "BF16/FP8 prefill linears under 'also'",
+        "value": round(value, 1),
+        "unit": "GB/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": round(elapsed / args.steps * 1e3, 4),
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "bf16",
+        "data": "synthetic",
+        "config": {
+            "workload": "BF16 decode linear y = x W^T, W [28672, 8192] ~N(0,0.02), x [M, 8192] "
+                        "~N(0,1), M in {1,8,32}, fp32 accumulate, BF16 out; 3 rotating weight "
+                        "copies (HBM-cold)",
+            "entry_point": "camblas_cuda_bgemm('T','N')",
+            "peak_fraction": round(value * 1e9 / HBM_PEAK, 4),
+        },
+        "roofline": roofline,
+        "cpu_baseline": None if args.skip_cpu else cpu_port_baseline(),
+        "also": also,
+    }
+    if not args.skip_cpu:
+        reference = cpu_reference_sgemm()
+        if reference:
+            result["also"]["cpu_reference_sgemm_2048"] = reference
+    print(json.dumps(result))
+
+
+def extras(torch, _kernels, _native, device, normal):
+    """The other configurations, each as absolute rate and fraction of its roofline."""
+    found = {}
+    # BF16 prefill linear and addmm (beta = 1)
+    tokens, outputs, inner = 4096, 10240, 8192
+    x, w = normal((tokens, inner)), normal((outputs, inner), 0.02)
+    y = torch.empty((tokens, outputs), dtype=torch.bfloat16, device=device)
+    c = normal((tokens, outputs))
+    flops = 2.0 * tokens * outputs * inner
+    seconds = event_time(torch, lambda i: _kernels.matmul(x, w.t(), out=y), 3, 10)
+    found["bf16_prefill_linear"] = {
+        "shape": [tokens, outputs, inner], "us": round(seconds * 1e6, 1),
+        "tflops": round(flops / seconds / 1e12, 1), "frac_of_2.5PF": round(flops / seconds / BF16_PEAK, 4),
+    }
+    seconds = event_time(torch, lambda i: _kernels.addmm(c, x, w.t(), beta=1.0), 3, 10)
+    found["bf16_prefill_addmm_beta1"] = {
+        "us": round(seconds * 1e6, 1), "tflops": round(flops / seconds / 1e12, 1),
+        "note": "includes the bias expand+clone copy, as in the reference binding",
+    }
+    del x, w, y, c
+    # FP8 block-scaled linear
+    outputs, inner = 18432, 7168
+    w = torch.randint(0, 0x7E, (outputs, inner), device=device, dtype=torch.uint8)
+    w = w.view(torch.float8_e4m3fn)
+    w_scale = torch.rand((outputs // 128, inner // 128), device=device) * 0.1 + 1e-4
+    fp8 = {}
+    for tokens in (1, 16, 256, 4096):
+        a = torch.randint(0, 0x7E, (tokens, inner), device=device, dtype=torch.uint8)
+        a = a.view(torch.float8_e4m3fn)
+        a_scale = torch.rand((tokens, inner // 128), device=device) * 0.1 + 1e-4
+        out = torch.empty((tokens, outputs), dtype=torch.bfloat16, device=device)
+        seconds = event_time(
+            torch, lambda i: _kernels.fp8_block_matmul(a, a_scale, w, w_scale, out=out), 3, 10)
+        flops = 2.0 * tokens * outputs * inner
+        traffic = outputs * inner + w_scale.numel() * 4 + tokens * (inner + inner // 128 * 4 + outputs * 2)
+        fp8[str(tokens)] = {
+            "us": round(seconds * 1e6, 1), "tflops": round(flops / seconds / 1e12, 1),
+            "frac_of_5PF": round(flops / seconds / FP8_PEAK, 4),
+            "gbps": round(traffic / seconds / 1e9, 1), "frac_of_8TBs": round(traffic / seconds / HBM_PEAK, 4),
+        }
+    found["fp8_block_linear_18432x7168"] = fp8
+    del w, w_scale
+    # FP32 SGEMM 2048^3 (plumbing)
+    size = 2048
+    a32 = torch.rand((size, size), device=device) * 2 - 1
+    b32 = torch.rand((size, size), device=device) * 2 - 1
+    c32 = torch.empty((size, size), device=device)
+    seconds = event_time(torch, lambda i: _kernels.matmul(a32, b32, out=c32), 3, 10)
+    found["fp32_sgemm_2048"] = {"us": round(seconds * 1e6, 1),
+                                "tflops": round(2.0 * size**3 / seconds / 1e12, 2),
+                                "frac_of_157TF": round(2.0 * size**3 / seconds / FP32_PEAK, 4)}
+    # decoder-layer decode step (Llama-3.1-70B shapes, batch 32, KV context 2048)
+    batch, hidden, q_heads, kv_heads, dim, ffn, context = 32, 8192, 64, 8, 128, 28672, 2048
+    weights = {
+        "input_norm": normal((hidden,), 0.02) + 1, "post_norm": normal((hidden,), 0.02) + 1,
+        "qkv": normal(((q_heads + 2 * kv_heads) * dim, hidden), 0.02),
+        "o": normal((hidden, q_heads * dim), 0.02), "gate": normal((ffn, hidden), 0.02),
+        "up": normal((ffn, hidden), 0.02), "down": normal((hidden, ffn), 0.02),
+    }
+    k_cache = normal((batch, context, kv_heads, dim))
+    v_cache = normal((batch, context, kv_heads, dim))
+    hidden_in, residual = normal((batch, hidden)), normal((batch, hidden))
+    positions = torch.full((batch,), context - 1, dtype=torch.int32, device=device)
+    seconds = event_time(
+        torch, lambda i: _kernels.decoder_layer_decode(
+            hidden_in, residual, weights, k_cache, v_cache, positions, q_heads=q_heads,
+            kv_heads=kv_heads, head_dim=dim), 3, 10)
+    weight_bytes = sum(v.numel() * 2 for k, v in weights.items())
+    traffic = weight_bytes + 2 * k_cache.numel() * 2 + 10e6
+    found["llama70b_layer_decode_b32_ctx2048"] = {
+        "us": round(seconds * 1e6, 1), "gbps": round(traffic / seconds / 1e9, 1),
+        "frac_of_8TBs": round(traffic / seconds / HBM_PEAK, 4),
+        "note": "eager launches (no graph); weights not rotated",
+    }
+    return found
+
+
+if __name__ == "__main__":
+    main()
