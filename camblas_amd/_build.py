@@ -26,6 +26,7 @@ CORE_SOURCES = (
     "gemm_generic.hip",
     "gemv_f32.hip",
     "bgemm_tn.hip",
+    "bgemv_stream.hip",
     "fp8_block.hip",
     "fusion.hip",
     "attention_decode.hip",

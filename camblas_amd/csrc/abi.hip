@@ -251,10 +251,26 @@ extern "C" int camblas_cuda_bgemm(camblas_cuda_context *context, char trans_a, c
             return fail(context, "missing or aliased BF16 GEMM operand", 1);
         Plan plan = make_plan(2, context->algorithm, ta, tb, m, n, k, lda, ldb, ldc,
                               aligned(a, 16) && aligned(b, 16), context->compute_units);
-        if (plan.family == FAMILY_MFMA_TN && context->override_kernel >= 0) {
-            plan.kernel = context->override_kernel;
-            if (context->override_split > 0)
-                plan.split_k = context->override_split;
+        if ((plan.family == FAMILY_MFMA_TN || plan.family == FAMILY_STREAM) &&
+            context->override_kernel >= 0) {
+            // diagnostics: 0.. selects an MFMA tile variant, 100 + 10*row_tiles + token_tiles the
+            // streaming kernel
+            if (context->override_kernel >= 100) {
+                plan.family = FAMILY_STREAM;
+                plan.kernel = context->override_kernel - 100;
+                plan.split_k = 1;
+            } else {
+                plan.family = FAMILY_MFMA_TN;
+                plan.kernel = context->override_kernel;
+                plan.split_k = context->override_split > 0 ? context->override_split : 1;
+            }
+        }
+        if (plan.family == FAMILY_STREAM) {
+            context->counts[plan.counter]++;
+            hipError_t error =
+                launch_bgemv_stream(context->stream, plan.kernel / 10, plan.kernel % 10, m, n, k,
+                                    alpha, a, lda, b, ldb, beta, c, ldc);
+            return error == hipSuccess ? 0 : fail(context, "BF16 streaming GEMV", error);
         }
         if (plan.family == FAMILY_MFMA_TN) {
             float *partials = nullptr;

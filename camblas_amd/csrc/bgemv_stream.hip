@@ -1,0 +1,268 @@
+// Bandwidth-bound BF16 decode linear y[M,N] = alpha * x[M,K] * W[N,K]^T + beta * y for small M.
+//
+// The whole cost is reading W once from HBM, so the kernel is organised around the weight stream:
+// one workgroup owns 16*NT consecutive weight rows for the whole K extent (about one workgroup per
+// compute unit for a Llama-sized projection) and marches along K in 128-element steps; all
+// workgroups advance roughly in lock step, which keeps the DRAM pages of one column block open
+// across the chip. Two K steps are in flight in registers per thread (128-bit loads, 256
+// contiguous bytes per row) while a third is multiplied, so a compute unit keeps ~2 * 16*NT * 256
+// bytes outstanding. Tiles are staged in LDS with a 16-way XOR swizzle (conflict-free 128-bit
+// stores and MFMA-layout reads). The four wavefronts split each K step four ways
+// (v_mfma_f32_16x16x32_bf16, FP32 accumulate) and their partial sums are combined in wavefront
+// order at the end, so results do not depend on scheduling. No split-K pass and no scratch.
+// Contract: ref src/cuda/bfloat16.cuh:11-57 for the ('T','N') call of a linear
+// (src/cuda/torch_bindings.cpp:146-199); the reference's own decode kernel class is
+// src/cuda/decode_float.cuh:2-52 (FP32, one vector).
+#include "common.hpp"
+#include "device.hpp"
+
+namespace camblas_hip
+{
+namespace
+{
+struct StreamParams {
+    const unsigned short *w;
+    const unsigned short *x;
+    unsigned short *y;
+    int lda, ldb, ldc;
+    int n, m, k;
+    float alpha, beta;
+    int vector_store;
+};
+
+template <int NT, int MT>
+__global__ __launch_bounds__(256) void bgemv_stream_kernel(StreamParams p)
+{
+    constexpr int ROWS = NT * 16, XROWS = MT * 16, CH = 16, BK = 128;
+    constexpr int STAGE_SLOTS = (ROWS + XROWS) * CH;
+    extern __shared__ __attribute__((aligned(16))) unsigned char lds_bytes[];
+    u32x4_t *lds = reinterpret_cast<u32x4_t *>(lds_bytes);
+
+    const int thread = threadIdx.x, lane = thread % 64, wave = thread / 64;
+    const int chunk = thread % CH, pass_row = thread / CH; // 16 lanes per 256-byte row segment
+    const int n0 = blockIdx.x * ROWS, m0 = blockIdx.y * XROWS;
+    const int k_tiles = (p.k + BK - 1) / BK;
+
+    unsigned a_off[NT], b_off[MT];
+#pragma unroll
+    for (int i = 0; i < NT; ++i) {
+        int row = n0 + i * 16 + pass_row;
+        row = row < p.n ? row : p.n - 1;
+        a_off[i] = unsigned(row - n0) * unsigned(p.lda);
+    }
+#pragma unroll
+    for (int j = 0; j < MT; ++j) {
+        int row = m0 + j * 16 + pass_row;
+        row = row < p.m ? row : p.m - 1;
+        b_off[j] = unsigned(row - m0) * unsigned(p.ldb);
+    }
+    const unsigned short *a_base = p.w + size_t(n0) * p.lda;
+    const unsigned short *b_base = p.x + size_t(m0) * p.ldb;
+    // LDS slot of this thread's chunk inside a 16-row pass; passes are 256 slots apart
+    const int store_slot = pass_row * CH + (chunk ^ pass_row);
+
+    // Loads are unconditional and the loop below has no data-dependent control flow, so the
+    // compiler can count outstanding loads exactly and wait only for the older of the two tiles in
+    // flight. A K position past the end (the K tail, or the padding tile of an odd tile count) is
+    // read from the last valid chunk instead and zeroed by a mask when it is stored to LDS.
+    u32x4_t a_reg[2][NT], b_reg[2][MT];
+    // Workgroups start at different K tiles and wrap around: if all of them swept K in lock step
+    // the chip would read one 256-byte column block of every row at a time, a 16 KB-strided
+    // pattern that lands on few HBM channels; staggering spreads the requests over all of them.
+    const int start = int(blockIdx.x % unsigned(k_tiles));
+    auto rotated = [&](int step) {
+        int tile = (step < k_tiles ? step : k_tiles - 1) + start;
+        return tile < k_tiles ? tile : tile - k_tiles;
+    };
+    auto fetch = [&](int step, u32x4_t(&a)[NT], u32x4_t(&b)[MT]) {
+        int k0 = rotated(step) * BK + chunk * 8;
+        k0 = k0 < p.k ? k0 : p.k - 8;
+#pragma unroll
+        for (int i = 0; i < NT; ++i)
+            a[i] = *reinterpret_cast<const u32x4_t *>(a_base + k0 + a_off[i]);
+#pragma unroll
+        for (int j = 0; j < MT; ++j)
+            b[j] = *reinterpret_cast<const u32x4_t *>(b_base + k0 + b_off[j]);
+    };
+    auto stash = [&](int stage, int step, const u32x4_t(&a)[NT], const u32x4_t(&b)[MT]) {
+        const unsigned mask =
+            step < k_tiles && rotated(step) * BK + chunk * 8 < p.k ? 0xffffffffu : 0u;
+        u32x4_t *base = lds + stage * STAGE_SLOTS + store_slot;
+#pragma unroll
+        for (int i = 0; i < NT; ++i)
+            base[i * 16 * CH] = a[i] & mask;
+#pragma unroll
+        for (int j = 0; j < MT; ++j)
+            base[(NT + j) * 16 * CH] = b[j] & mask;
+    };
+
+    // MFMA 16x16x32 operand positions: lane -> row lane%16, 8 K values at (wave*4 + lane/16)*8
+    const int frag_row = lane % 16;
+    const int frag_slot = frag_row * CH + ((wave * 4 + lane / 16) ^ frag_row);
+    f32x4_t acc[NT][MT];
+#pragma unroll
+    for (int i = 0; i < NT; ++i)
+#pragma unroll
+        for (int j = 0; j < MT; ++j)
+            acc[i][j] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+    auto multiply = [&](int stage) {
+        const u32x4_t *base = lds + stage * STAGE_SLOTS + frag_slot;
+        bf16x8_t b_frag[MT];
+#pragma unroll
+        for (int j = 0; j < MT; ++j)
+            b_frag[j] = __builtin_bit_cast(bf16x8_t, base[(NT + j) * 16 * CH]);
+#pragma unroll
+        for (int i = 0; i < NT; ++i) {
+            bf16x8_t a_frag = __builtin_bit_cast(bf16x8_t, base[i * 16 * CH]);
+#pragma unroll
+            for (int j = 0; j < MT; ++j)
+                acc[i][j] =
+                    __builtin_amdgcn_mfma_f32_16x16x32_bf16(a_frag, b_frag[j], acc[i][j], 0, 0, 0);
+        }
+    };
+
+    fetch(0, a_reg[0], b_reg[0]);
+    __builtin_amdgcn_sched_barrier(0);
+    fetch(1, a_reg[1], b_reg[1]);
+    // sched_barrier(0) pins the phase order: without it the scheduler interleaves the two fetches
+    // and the wait before a store to LDS degenerates to "all loads", halving the bytes in flight.
+    for (int tile = 0; tile < k_tiles; tile += 2) {
+        __builtin_amdgcn_sched_barrier(0);
+        stash(0, tile, a_reg[0], b_reg[0]);
+        __syncthreads();
+        __builtin_amdgcn_sched_barrier(0);
+        fetch(tile + 2, a_reg[0], b_reg[0]);
+        __builtin_amdgcn_sched_barrier(0);
+        multiply(0);
+        __builtin_amdgcn_sched_barrier(0);
+        stash(1, tile + 1, a_reg[1], b_reg[1]);
+        __syncthreads();
+        __builtin_amdgcn_sched_barrier(0);
+        fetch(tile + 3, a_reg[1], b_reg[1]);
+        __builtin_amdgcn_sched_barrier(0);
+        multiply(1);
+    }
+
+    // ---- combine the four K partitions in wavefront order through LDS
+    __syncthreads();
+    f32x4_t *combine = reinterpret_cast<f32x4_t *>(lds_bytes);
+#pragma unroll
+    for (int w = 0; w < 4; ++w) {
+        if (wave == w) {
+#pragma unroll
+            for (int i = 0; i < NT; ++i)
+#pragma unroll
+                for (int j = 0; j < MT; ++j) {
+                    f32x4_t *slot = combine + (i * MT + j) * 64 + lane;
+                    *slot = w == 0 ? acc[i][j] : *slot + acc[i][j];
+                }
+        }
+        __syncthreads();
+    }
+    // ---- epilogue: wavefront w writes tiles w, w+4, ...; register r of lane l is feature
+    // 4*(l/16) + r and token l%16 inside the 16x16 tile
+#pragma unroll
+    for (int index = 0; index < NT * MT; ++index) {
+        if (index % 4 != wave)
+            continue;
+        const int i = index / MT, j = index % MT;
+        const int m = m0 + j * 16 + lane % 16;
+        const int n = n0 + i * 16 + (lane / 16) * 4;
+        if (m >= p.m || n >= p.n)
+            continue;
+        f32x4_t sum = combine[index * 64 + lane];
+        float v[4] = {sum[0], sum[1], sum[2], sum[3]};
+        unsigned short *out = p.y + size_t(m) * p.ldc + n;
+        if (n + 3 < p.n && p.vector_store) {
+            if (p.beta != 0.f) {
+                u32x2_t old = *reinterpret_cast<const u32x2_t *>(out);
+                v[0] = fmaf(p.beta, __uint_as_float(old[0] << 16), p.alpha * v[0]);
+                v[1] = fmaf(p.beta, __uint_as_float(old[0] & 0xffff0000u), p.alpha * v[1]);
+                v[2] = fmaf(p.beta, __uint_as_float(old[1] << 16), p.alpha * v[2]);
+                v[3] = fmaf(p.beta, __uint_as_float(old[1] & 0xffff0000u), p.alpha * v[3]);
+            } else {
+#pragma unroll
+                for (int e = 0; e < 4; ++e)
+                    v[e] *= p.alpha;
+            }
+            u32x2_t packed = {pack_bf16x2(v[0], v[1]), pack_bf16x2(v[2], v[3])};
+            *reinterpret_cast<u32x2_t *>(out) = packed;
+        } else {
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                if (n + e >= p.n)
+                    break;
+                float value = p.alpha * v[e];
+                if (p.beta != 0.f)
+                    value = fmaf(p.beta, bf16_bits_to_float(out[e]), value);
+                out[e] = float_to_bf16_bits(value);
+            }
+        }
+    }
+}
+
+template <int NT, int MT> hipError_t launch_one(hipStream_t stream, const StreamParams &p)
+{
+    constexpr size_t lds_bytes = size_t(2) * (NT + MT) * 16 * 256;
+    auto kernel = bgemv_stream_kernel<NT, MT>;
+    static bool configured[64] = {};
+    int device = 0;
+    hipError_t status = hipGetDevice(&device);
+    if (status != hipSuccess)
+        return status;
+    if (device < 0 || device >= 64 || !configured[device]) {
+        status = hipFuncSetAttribute(reinterpret_cast<const void *>(kernel),
+                                     hipFuncAttributeMaxDynamicSharedMemorySize, int(lds_bytes));
+        if (status != hipSuccess)
+            return status;
+        if (device >= 0 && device < 64)
+            configured[device] = true;
+    }
+    dim3 grid(unsigned((p.n + NT * 16 - 1) / (NT * 16)), unsigned((p.m + MT * 16 - 1) / (MT * 16)));
+    kernel<<<grid, 256, lds_bytes, stream>>>(p);
+    return launch_status();
+}
+
+template <int MT> hipError_t launch_rows(hipStream_t stream, int row_tiles, const StreamParams &p)
+{
+    switch (row_tiles) {
+    case 1: return launch_one<1, MT>(stream, p);
+    case 2: return launch_one<2, MT>(stream, p);
+    case 3: return launch_one<3, MT>(stream, p);
+    case 4: return launch_one<4, MT>(stream, p);
+    case 5: return launch_one<5, MT>(stream, p);
+    case 6: return launch_one<6, MT>(stream, p);
+    case 7: return launch_one<7, MT>(stream, p);
+    case 8: return launch_one<8, MT>(stream, p);
+    default: return hipErrorInvalidValue;
+    }
+}
+} // namespace
+
+hipError_t launch_bgemv_stream(hipStream_t stream, int row_tiles, int token_tiles, int n_out,
+                               int m_rows, int k, float alpha, const void *w, int lda,
+                               const void *x, int ldb, float beta, void *y, int ldc)
+{
+    StreamParams p;
+    p.w = static_cast<const unsigned short *>(w);
+    p.x = static_cast<const unsigned short *>(x);
+    p.y = static_cast<unsigned short *>(y);
+    p.lda = lda;
+    p.ldb = ldb;
+    p.ldc = ldc;
+    p.n = n_out;
+    p.m = m_rows;
+    p.k = k;
+    p.alpha = alpha;
+    p.beta = beta;
+    p.vector_store = (ldc % 4 == 0) && (reinterpret_cast<uintptr_t>(y) % 8 == 0);
+    if ((m_rows + token_tiles * 16 - 1) / (token_tiles * 16) > 65535)
+        return hipErrorInvalidValue;
+    switch (token_tiles) {
+    case 1: return launch_rows<1>(stream, row_tiles, p);
+    case 2: return launch_rows<2>(stream, row_tiles, p);
+    case 4: return launch_rows<4>(stream, row_tiles, p);
+    default: return hipErrorInvalidValue;
+    }
+}
+} // namespace camblas_hip

@@ -44,12 +44,13 @@ enum KernelFamily {
     FAMILY_GENERIC = 0, // LDS-tiled VALU kernel, any transpose / leading dimension / alignment
     FAMILY_GEMV_F32 = 1,
     FAMILY_MFMA_TN = 2, // BF16 'T','N', K-contiguous operands, MFMA tiles staged through LDS
-    FAMILY_FP8_BLOCK = 3
+    FAMILY_FP8_BLOCK = 3,
+    FAMILY_STREAM = 4 // BF16 'T','N' with few tokens: weight-streaming kernel, one pass over W
 };
 
 struct Plan {
     int family = FAMILY_GENERIC;
-    int kernel = 0;   // variant index inside the family
+    int kernel = 0;   // variant index inside the family (stream family: 10*row_tiles + token_tiles)
     int split_k = 1;  // number of K partitions (partials reduced in fixed order)
     int counter = 0;  // stats slot incremented at launch
 };
@@ -88,6 +89,10 @@ hipError_t launch_gemv_f32(hipStream_t stream, int rows, int inner, float alpha,
 hipError_t launch_bgemm_tn(hipStream_t stream, int variant, int split_k, int n_out, int m_rows,
                            int k, float alpha, const void *w, int lda, const void *x, int ldb,
                            float beta, void *y, int ldc, float *partials);
+// Decode-shaped BF16 linear: each workgroup streams 16*row_tiles weight rows over the whole K.
+hipError_t launch_bgemv_stream(hipStream_t stream, int row_tiles, int token_tiles, int n_out,
+                               int m_rows, int k, float alpha, const void *w, int lda,
+                               const void *x, int ldb, float beta, void *y, int ldc);
 hipError_t launch_fp8_block(hipStream_t stream, int variant, int split_k, int rows, int outputs,
                             int inner, const void *a, const float *a_scale, const void *w,
                             const float *w_scale, void *out, float *partials);

@@ -6,6 +6,7 @@
 #include "common.hpp"
 
 #include <algorithm>
+#include <cmath>
 #include <cstring>
 
 namespace camblas_hip
@@ -21,6 +22,28 @@ int decode_split(int tiles, int k_tiles, int compute_units)
     int wanted = ceil_div(4 * compute_units, std::max(1, tiles));
     int limit = std::max(1, k_tiles / 4);
     return std::max(1, std::min(wanted, limit));
+}
+
+// Weight rows per workgroup (in units of 16) for the streaming decode kernel: the choice that
+// spreads the row tiles most evenly over the compute units; ties go to the larger block, which
+// keeps more bytes in flight per workgroup.
+int stream_row_tiles(int outputs, int compute_units)
+{
+    const int tiles = ceil_div(outputs, 16);
+    int best = 1;
+    double best_score = -1;
+    for (int candidate = 1; candidate <= 8; ++candidate) {
+        int groups = ceil_div(tiles, candidate);
+        double busiest = double(ceil_div(groups, compute_units)) * candidate;
+        double score = (double(tiles) / compute_units) / busiest;
+        if (groups < compute_units)
+            score = std::min(score, double(groups) / compute_units);
+        if (score >= best_score - 1e-9) {
+            best_score = score;
+            best = candidate;
+        }
+    }
+    return best;
 }
 
 // Fraction of the machine a tiling keeps busy: useful tiles over whole rounds of resident
@@ -67,12 +90,13 @@ Plan make_plan(int dtype, int algorithm, bool trans_a, bool trans_b, int m, int 
         plan.family = FAMILY_MFMA_TN;
         plan.counter = 4;
         const int outputs = m, tokens = n;
-        if (tokens <= 32) {
-            plan.kernel = 4; // 128 x 32 x 64
-            const TnVariant &v = tn_variant(plan.kernel);
-            plan.split_k =
-                decode_split(ceil_div(outputs, v.block_n), ceil_div(k, v.block_k), compute_units);
-        } else if (tokens <= 64) {
+        if (tokens <= 64) {
+            // decode: bandwidth-bound on W, one streaming pass, no split-K
+            plan.family = FAMILY_STREAM;
+            plan.kernel = 10 * stream_row_tiles(outputs, compute_units) +
+                          (tokens <= 16 ? 1 : tokens <= 32 ? 2 : 4);
+            plan.split_k = 1;
+        } else if (tokens <= 96) {
             plan.kernel = 3; // 128 x 64 x 64
             const TnVariant &v = tn_variant(plan.kernel);
             plan.split_k =
@@ -124,6 +148,10 @@ void describe_plan(const Plan &plan, int dtype, char *text, size_t bytes)
     case FAMILY_FP8_BLOCK:
         std::snprintf(text, bytes, "%s %s split_k=%d", type, fp8_variant(plan.kernel).name,
                       plan.split_k);
+        break;
+    case FAMILY_STREAM:
+        std::snprintf(text, bytes, "%s stream rows=%d tokens=%d k128 depth2", type,
+                      16 * (plan.kernel / 10), 16 * (plan.kernel % 10));
         break;
     default:
         std::snprintf(text, bytes, "%s generic 64x64x16", type);
