@@ -254,7 +254,7 @@ extern "C" int camblas_cuda_bgemm(camblas_cuda_context *context, char trans_a, c
         if ((plan.family == FAMILY_MFMA_TN || plan.family == FAMILY_STREAM) &&
             context->override_kernel >= 0) {
             // diagnostics: 0.. selects an MFMA tile variant, 100 + 10*row_tiles + token_tiles the
-            // streaming kernel
+            // streaming kernel (+ 100*mode)
             if (context->override_kernel >= 100) {
                 plan.family = FAMILY_STREAM;
                 plan.kernel = context->override_kernel - 100;
@@ -268,8 +268,8 @@ extern "C" int camblas_cuda_bgemm(camblas_cuda_context *context, char trans_a, c
         if (plan.family == FAMILY_STREAM) {
             context->counts[plan.counter]++;
             hipError_t error =
-                launch_bgemv_stream(context->stream, plan.kernel / 10, plan.kernel % 10, m, n, k,
-                                    alpha, a, lda, b, ldb, beta, c, ldc);
+                launch_bgemv_stream(context->stream, plan.kernel / 100, plan.kernel / 10 % 10,
+                                    plan.kernel % 10, m, n, k, alpha, a, lda, b, ldb, beta, c, ldc);
             return error == hipSuccess ? 0 : fail(context, "BF16 streaming GEMV", error);
         }
         if (plan.family == FAMILY_MFMA_TN) {

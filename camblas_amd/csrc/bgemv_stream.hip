@@ -30,16 +30,18 @@ struct StreamParams {
     int vector_store;
 };
 
-template <int NT, int MT>
-__global__ __launch_bounds__(256) void bgemv_stream_kernel(StreamParams p)
+// NT, MT: 16-row weight tiles and 16-token tiles per workgroup; WAVES wavefronts split one K step
+// of 32*WAVES elements; DEPTH K steps are in flight in registers.
+template <int NT, int MT, int WAVES, int DEPTH>
+__global__ __launch_bounds__(WAVES * 64) void bgemv_stream_kernel(StreamParams p)
 {
-    constexpr int ROWS = NT * 16, XROWS = MT * 16, CH = 16, BK = 128;
+    constexpr int ROWS = NT * 16, XROWS = MT * 16, CH = 4 * WAVES, BK = 32 * WAVES;
     constexpr int STAGE_SLOTS = (ROWS + XROWS) * CH;
     extern __shared__ __attribute__((aligned(16))) unsigned char lds_bytes[];
     u32x4_t *lds = reinterpret_cast<u32x4_t *>(lds_bytes);
 
     const int thread = threadIdx.x, lane = thread % 64, wave = thread / 64;
-    const int chunk = thread % CH, pass_row = thread / CH; // 16 lanes per 256-byte row segment
+    const int chunk = thread % CH, pass_row = thread / CH; // CH lanes per row segment, 16 rows per pass
     const int n0 = blockIdx.x * ROWS, m0 = blockIdx.y * XROWS;
     const int k_tiles = (p.k + BK - 1) / BK;
 
@@ -60,12 +62,13 @@ __global__ __launch_bounds__(256) void bgemv_stream_kernel(StreamParams p)
     const unsigned short *b_base = p.x + size_t(m0) * p.ldb;
     // LDS slot of this thread's chunk inside a 16-row pass; passes are 256 slots apart
     const int store_slot = pass_row * CH + (chunk ^ pass_row);
+    static_assert(CH == 16 || CH == 32, "XOR swizzle covers the low four chunk bits");
 
     // Loads are unconditional and the loop below has no data-dependent control flow, so the
     // compiler can count outstanding loads exactly and wait only for the older of the two tiles in
     // flight. A K position past the end (the K tail, or the padding tile of an odd tile count) is
     // read from the last valid chunk instead and zeroed by a mask when it is stored to LDS.
-    u32x4_t a_reg[2][NT], b_reg[2][MT];
+    u32x4_t a_reg[DEPTH][NT], b_reg[DEPTH][MT];
     // Workgroups start at different K tiles and wrap around: if all of them swept K in lock step
     // the chip would read one 256-byte column block of every row at a time, a 16 KB-strided
     // pattern that lands on few HBM channels; staggering spreads the requests over all of them.
@@ -121,33 +124,34 @@ __global__ __launch_bounds__(256) void bgemv_stream_kernel(StreamParams p)
         }
     };
 
-    fetch(0, a_reg[0], b_reg[0]);
-    __builtin_amdgcn_sched_barrier(0);
-    fetch(1, a_reg[1], b_reg[1]);
-    // sched_barrier(0) pins the phase order: without it the scheduler interleaves the two fetches
-    // and the wait before a store to LDS degenerates to "all loads", halving the bytes in flight.
-    for (int tile = 0; tile < k_tiles; tile += 2) {
+    // sched_barrier(0) pins the phase order (also between the prologue fetches): if the scheduler
+    // interleaves loads of different tiles, the wait before a store to LDS degenerates to "all
+    // loads" and only one tile stays in flight.
+#pragma unroll
+    for (int d = 0; d < DEPTH; ++d) {
+        fetch(d, a_reg[d], b_reg[d]);
         __builtin_amdgcn_sched_barrier(0);
-        stash(0, tile, a_reg[0], b_reg[0]);
-        __syncthreads();
-        __builtin_amdgcn_sched_barrier(0);
-        fetch(tile + 2, a_reg[0], b_reg[0]);
-        __builtin_amdgcn_sched_barrier(0);
-        multiply(0);
-        __builtin_amdgcn_sched_barrier(0);
-        stash(1, tile + 1, a_reg[1], b_reg[1]);
-        __syncthreads();
-        __builtin_amdgcn_sched_barrier(0);
-        fetch(tile + 3, a_reg[1], b_reg[1]);
-        __builtin_amdgcn_sched_barrier(0);
-        multiply(1);
+    }
+    int stage = 0;
+    for (int step = 0; step < k_tiles; step += DEPTH) {
+#pragma unroll
+        for (int d = 0; d < DEPTH; ++d) {
+            __builtin_amdgcn_sched_barrier(0);
+            stash(stage, step + d, a_reg[d], b_reg[d]);
+            __syncthreads();
+            __builtin_amdgcn_sched_barrier(0);
+            fetch(step + d + DEPTH, a_reg[d], b_reg[d]);
+            __builtin_amdgcn_sched_barrier(0);
+            multiply(stage);
+            stage ^= 1;
+        }
     }
 
-    // ---- combine the four K partitions in wavefront order through LDS
+    // ---- combine the K partitions of the wavefronts in wavefront order through LDS
     __syncthreads();
     f32x4_t *combine = reinterpret_cast<f32x4_t *>(lds_bytes);
 #pragma unroll
-    for (int w = 0; w < 4; ++w) {
+    for (int w = 0; w < WAVES; ++w) {
         if (wave == w) {
 #pragma unroll
             for (int i = 0; i < NT; ++i)
@@ -163,7 +167,7 @@ __global__ __launch_bounds__(256) void bgemv_stream_kernel(StreamParams p)
     // 4*(l/16) + r and token l%16 inside the 16x16 tile
 #pragma unroll
     for (int index = 0; index < NT * MT; ++index) {
-        if (index % 4 != wave)
+        if (index % WAVES != wave)
             continue;
         const int i = index / MT, j = index % MT;
         const int m = m0 + j * 16 + lane % 16;
@@ -201,45 +205,63 @@ __global__ __launch_bounds__(256) void bgemv_stream_kernel(StreamParams p)
     }
 }
 
-template <int NT, int MT> hipError_t launch_one(hipStream_t stream, const StreamParams &p)
+template <int NT, int MT, int WAVES, int DEPTH>
+hipError_t launch_one(hipStream_t stream, const StreamParams &p)
 {
-    constexpr size_t lds_bytes = size_t(2) * (NT + MT) * 16 * 256;
-    auto kernel = bgemv_stream_kernel<NT, MT>;
-    static bool configured[64] = {};
-    int device = 0;
-    hipError_t status = hipGetDevice(&device);
-    if (status != hipSuccess)
-        return status;
-    if (device < 0 || device >= 64 || !configured[device]) {
-        status = hipFuncSetAttribute(reinterpret_cast<const void *>(kernel),
-                                     hipFuncAttributeMaxDynamicSharedMemorySize, int(lds_bytes));
+    constexpr size_t lds_bytes = size_t(2) * (NT + MT) * 16 * (64 * WAVES);
+    if constexpr (lds_bytes > 160 * 1024) {
+        return hipErrorInvalidValue;
+    } else {
+        auto kernel = bgemv_stream_kernel<NT, MT, WAVES, DEPTH>;
+        static bool configured[64] = {};
+        int device = 0;
+        hipError_t status = hipGetDevice(&device);
         if (status != hipSuccess)
             return status;
-        if (device >= 0 && device < 64)
-            configured[device] = true;
+        if (device < 0 || device >= 64 || !configured[device]) {
+            status = hipFuncSetAttribute(reinterpret_cast<const void *>(kernel),
+                                         hipFuncAttributeMaxDynamicSharedMemorySize, int(lds_bytes));
+            if (status != hipSuccess)
+                return status;
+            if (device >= 0 && device < 64)
+                configured[device] = true;
+        }
+        dim3 grid(unsigned((p.n + NT * 16 - 1) / (NT * 16)),
+                  unsigned((p.m + MT * 16 - 1) / (MT * 16)));
+        kernel<<<grid, WAVES * 64, lds_bytes, stream>>>(p);
+        return launch_status();
     }
-    dim3 grid(unsigned((p.n + NT * 16 - 1) / (NT * 16)), unsigned((p.m + MT * 16 - 1) / (MT * 16)));
-    kernel<<<grid, 256, lds_bytes, stream>>>(p);
-    return launch_status();
 }
 
-template <int MT> hipError_t launch_rows(hipStream_t stream, int row_tiles, const StreamParams &p)
+template <int MT, int WAVES, int DEPTH>
+hipError_t launch_rows(hipStream_t stream, int row_tiles, const StreamParams &p)
 {
     switch (row_tiles) {
-    case 1: return launch_one<1, MT>(stream, p);
-    case 2: return launch_one<2, MT>(stream, p);
-    case 3: return launch_one<3, MT>(stream, p);
-    case 4: return launch_one<4, MT>(stream, p);
-    case 5: return launch_one<5, MT>(stream, p);
-    case 6: return launch_one<6, MT>(stream, p);
-    case 7: return launch_one<7, MT>(stream, p);
-    case 8: return launch_one<8, MT>(stream, p);
+    case 1: return launch_one<1, MT, WAVES, DEPTH>(stream, p);
+    case 2: return launch_one<2, MT, WAVES, DEPTH>(stream, p);
+    case 3: return launch_one<3, MT, WAVES, DEPTH>(stream, p);
+    case 4: return launch_one<4, MT, WAVES, DEPTH>(stream, p);
+    case 5: return launch_one<5, MT, WAVES, DEPTH>(stream, p);
+    case 6: return launch_one<6, MT, WAVES, DEPTH>(stream, p);
+    case 7: return launch_one<7, MT, WAVES, DEPTH>(stream, p);
+    case 8: return launch_one<8, MT, WAVES, DEPTH>(stream, p);
+    default: return hipErrorInvalidValue;
+    }
+}
+
+template <int WAVES, int DEPTH>
+hipError_t launch_tokens(hipStream_t stream, int row_tiles, int token_tiles, const StreamParams &p)
+{
+    switch (token_tiles) {
+    case 1: return launch_rows<1, WAVES, DEPTH>(stream, row_tiles, p);
+    case 2: return launch_rows<2, WAVES, DEPTH>(stream, row_tiles, p);
+    case 4: return launch_rows<4, WAVES, DEPTH>(stream, row_tiles, p);
     default: return hipErrorInvalidValue;
     }
 }
 } // namespace
 
-hipError_t launch_bgemv_stream(hipStream_t stream, int row_tiles, int token_tiles, int n_out,
+hipError_t launch_bgemv_stream(hipStream_t stream, int mode, int row_tiles, int token_tiles, int n_out,
                                int m_rows, int k, float alpha, const void *w, int lda,
                                const void *x, int ldb, float beta, void *y, int ldc)
 {
@@ -258,10 +280,11 @@ hipError_t launch_bgemv_stream(hipStream_t stream, int row_tiles, int token_tile
     p.vector_store = (ldc % 4 == 0) && (reinterpret_cast<uintptr_t>(y) % 8 == 0);
     if ((m_rows + token_tiles * 16 - 1) / (token_tiles * 16) > 65535)
         return hipErrorInvalidValue;
-    switch (token_tiles) {
-    case 1: return launch_rows<1>(stream, row_tiles, p);
-    case 2: return launch_rows<2>(stream, row_tiles, p);
-    case 4: return launch_rows<4>(stream, row_tiles, p);
+    switch (mode) {
+    case 0: return launch_tokens<4, 2>(stream, row_tiles, token_tiles, p);
+    case 1: return launch_tokens<4, 3>(stream, row_tiles, token_tiles, p);
+    case 2: return launch_tokens<8, 2>(stream, row_tiles, token_tiles, p);
+    case 3: return launch_tokens<8, 3>(stream, row_tiles, token_tiles, p);
     default: return hipErrorInvalidValue;
     }
 }

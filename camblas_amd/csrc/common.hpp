@@ -50,7 +50,7 @@ enum KernelFamily {
 
 struct Plan {
     int family = FAMILY_GENERIC;
-    int kernel = 0;   // variant index inside the family (stream family: 10*row_tiles + token_tiles)
+    int kernel = 0;   // variant index inside the family (stream family: 100*mode + 10*row_tiles + token_tiles)
     int split_k = 1;  // number of K partitions (partials reduced in fixed order)
     int counter = 0;  // stats slot incremented at launch
 };
@@ -90,7 +90,8 @@ hipError_t launch_bgemm_tn(hipStream_t stream, int variant, int split_k, int n_o
                            int k, float alpha, const void *w, int lda, const void *x, int ldb,
                            float beta, void *y, int ldc, float *partials);
 // Decode-shaped BF16 linear: each workgroup streams 16*row_tiles weight rows over the whole K.
-hipError_t launch_bgemv_stream(hipStream_t stream, int row_tiles, int token_tiles, int n_out,
+// mode: 0 = 4 wavefronts / 2 K steps in flight, 1 = 4 / 3, 2 = 8 / 2, 3 = 8 / 3.
+hipError_t launch_bgemv_stream(hipStream_t stream, int mode, int row_tiles, int token_tiles, int n_out,
                                int m_rows, int k, float alpha, const void *w, int lda,
                                const void *x, int ldb, float beta, void *y, int ldc);
 hipError_t launch_fp8_block(hipStream_t stream, int variant, int split_k, int rows, int outputs,

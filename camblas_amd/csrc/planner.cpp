@@ -150,8 +150,9 @@ void describe_plan(const Plan &plan, int dtype, char *text, size_t bytes)
                       plan.split_k);
         break;
     case FAMILY_STREAM:
-        std::snprintf(text, bytes, "%s stream rows=%d tokens=%d k128 depth2", type,
-                      16 * (plan.kernel / 10), 16 * (plan.kernel % 10));
+        std::snprintf(text, bytes, "%s stream rows=%d tokens=%d waves=%d depth=%d", type,
+                      16 * (plan.kernel / 10 % 10), 16 * (plan.kernel % 10),
+                      plan.kernel / 100 >= 2 ? 8 : 4, plan.kernel / 100 % 2 ? 3 : 2);
         break;
     default:
         std::snprintf(text, bytes, "%s generic 64x64x16", type);

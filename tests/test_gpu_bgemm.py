@@ -71,7 +71,13 @@ def test_tn_every_variant(device, variant, split, n_out, pad):
         assert np.array_equal(got2d[:, n_out:], c0.reshape(m_rows, ldc)[:, n_out:])
 
 
-STREAM_CODES = [100 + 10 * rows + tokens for rows in range(1, 9) for tokens in (1, 2, 4)]
+# 100 + 100*mode + 10*row_tiles + token_tiles; modes 2 and 3 (eight wavefronts) need
+# row_tiles + token_tiles <= 10 to fit the LDS
+STREAM_CODES = [100 + 10 * rows + tokens for rows in range(1, 9) for tokens in (1, 2, 4)] + [
+    100 + 100 * mode + 10 * rows + tokens
+    for mode in (1, 2, 3) for rows in (1, 4, 7, 8) for tokens in (1, 2, 4)
+    if mode == 1 or rows + tokens <= 10
+]
 
 
 @pytest.mark.parametrize("code", STREAM_CODES)
