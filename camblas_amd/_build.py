@@ -27,6 +27,7 @@ CORE_SOURCES = (
     "gemv_f32.hip",
     "bgemm_tn.hip",
     "bgemv_stream.hip",
+    "bgemm_dma.hip",
     "fp8_block.hip",
     "fusion.hip",
     "attention_decode.hip",

@@ -251,7 +251,10 @@ extern "C" int camblas_cuda_bgemm(camblas_cuda_context *context, char trans_a, c
             return fail(context, "missing or aliased BF16 GEMM operand", 1);
         Plan plan = make_plan(2, context->algorithm, ta, tb, m, n, k, lda, ldb, ldc,
                               aligned(a, 16) && aligned(b, 16), context->compute_units);
-        if ((plan.family == FAMILY_MFMA_TN || plan.family == FAMILY_STREAM) &&
+        if (plan.family == FAMILY_DMA && !aligned(c, 8))
+            plan.family = FAMILY_MFMA_TN; // same tile shapes, register-staged loads, scalar stores
+        if ((plan.family == FAMILY_MFMA_TN || plan.family == FAMILY_STREAM ||
+             plan.family == FAMILY_DMA) &&
             context->override_kernel >= 0) {
             // diagnostics: 0.. selects an MFMA tile variant, 100 + 10*row_tiles + token_tiles the
             // streaming kernel (+ 100*mode)
@@ -259,11 +262,21 @@ extern "C" int camblas_cuda_bgemm(camblas_cuda_context *context, char trans_a, c
                 plan.family = FAMILY_STREAM;
                 plan.kernel = context->override_kernel - 100;
                 plan.split_k = 1;
+            } else if (context->override_kernel >= 20 && context->override_kernel < 30) {
+                plan.family = FAMILY_DMA; // 20, 21, 22: direct-to-LDS tiles
+                plan.kernel = context->override_kernel - 20;
+                plan.split_k = 1;
             } else {
                 plan.family = FAMILY_MFMA_TN;
                 plan.kernel = context->override_kernel;
                 plan.split_k = context->override_split > 0 ? context->override_split : 1;
             }
+        }
+        if (plan.family == FAMILY_DMA) {
+            context->counts[plan.counter]++;
+            hipError_t error = launch_bgemm_dma(context->stream, plan.kernel, m, n, k, alpha, a, lda,
+                                                b, ldb, beta, c, ldc);
+            return error == hipSuccess ? 0 : fail(context, "BF16 MFMA GEMM (direct LDS loads)", error);
         }
         if (plan.family == FAMILY_STREAM) {
             context->counts[plan.counter]++;

@@ -1,0 +1,311 @@
+// Compute-bound BF16 prefill linear y[M,N] = alpha * x[M,K] * W[N,K]^T + beta * y: large MFMA
+// tiles fed by direct global->LDS loads.
+//
+// A workgroup of four wavefronts (2 x 2) owns a (64*TN) x (64*TM) output tile; each wavefront
+// accumulates a (32*TN) x (32*TM) block in TN*TM v_mfma_f32_32x32x16_bf16 accumulators (FP32).
+// K advances 64 elements per step through two LDS stages. The next step's operands are fetched with
+// global_load_lds_dwordx4: each lane names the 16-byte chunk of W or x that belongs in its LDS slot,
+// so the data lands in the XOR-swizzled layout the MFMA-layout reads expect without passing through
+// registers (no staging VGPRs, no ds_write). The two stages are separate LDS objects so the
+// compiler can tell the in-flight stage from the one being read. Fragments of the next 16-deep
+// step are read while the current step's MFMAs issue. Workgroups are renumbered per XCD so the
+// tiles resident on one XCD share W and x panels through its L2.
+// Shape requirements (the planner checks them): K % 64 == 0, N % 4 == 0, ldc % 4 == 0, 16-byte
+// aligned operands, 8-byte aligned y.
+// Contract: ref src/cuda/bfloat16.cuh:11-57 ('T','N' call of src/cuda/torch_bindings.cpp:155-199).
+#include "common.hpp"
+#include "device.hpp"
+
+namespace camblas_hip
+{
+namespace
+{
+struct DmaParams {
+    const unsigned short *w;
+    const unsigned short *x;
+    unsigned short *y;
+    int lda, ldb, ldc;
+    int n, m, k;
+    float alpha, beta;
+    int tiles_n, tiles_m;
+};
+
+// XOR applied to the 16-byte chunk index inside an LDS row of CH chunks: any 8 (and any 16)
+// consecutive rows land on distinct banks for a fixed logical chunk.
+template <int CH> __device__ __forceinline__ int swizzle(int row)
+{
+    if constexpr (CH == 8)
+        return ((row >> 1) & 7) ^ ((row & 1) << 2);
+    else
+        return (((row >> 2) & 1) << 1) | (((row >> 1) ^ (row >> 3)) & 1);
+}
+
+typedef __attribute__((address_space(3))) void lds_void;
+
+// 16 bytes per lane from global memory straight into LDS at `lds_base + lane*16` (the base must be
+// wave-uniform). Kept in a non-template function: inside a kernel template the host pass drops the
+// whole instantiation when it meets this target builtin.
+__device__ __forceinline__ void load_to_lds(const void *global, void *lds_base)
+{
+    __builtin_amdgcn_global_load_lds(global, (lds_void *)lds_base, 16, 0, 0);
+}
+
+// s_waitcnt vmcnt(N) with the other counters left alone (gfx9 encoding: vmcnt in bits 3:0 and
+// 15:14, expcnt 6:4, lgkmcnt 11:8).
+template <int N> __device__ __forceinline__ void wait_loads()
+{
+    __builtin_amdgcn_s_waitcnt((N & 15) | ((N >> 4) << 14) | 0x0f70);
+}
+
+// TN, TM: 32x32 MFMA tiles per wavefront along features / tokens (workgroup tile 64*TN x 64*TM);
+// BK: K elements per step (32 or 64); STAGES: LDS stages (STAGES - 1 steps are in flight).
+template <int TN, int TM, int BK, int STAGES>
+__global__ __launch_bounds__(256) void bgemm_dma_kernel(DmaParams p)
+{
+    constexpr int BN = 64 * TN, BM = 64 * TM, CH = BK / 8;
+    constexpr int ROWS_PER_LOAD = 64 / CH;               // rows one wave instruction fills
+    constexpr int A_ITERS = BN / (4 * ROWS_PER_LOAD), B_ITERS = BM / (4 * ROWS_PER_LOAD);
+    constexpr int LOADS = A_ITERS + B_ITERS;             // direct loads per wavefront and step
+    constexpr int SLOTS = (BN + BM) * CH;
+    static_assert(STAGES >= 2 && STAGES <= 4 && (BK == 32 || BK == 64), "pipeline shape");
+    static_assert(LOADS * (STAGES - 2) < 64, "vmcnt holds 6 bits");
+    // One LDS object per stage so that reads of one stage and in-flight writes of another are
+    // provably disjoint.
+    __shared__ u32x4_t stage0[SLOTS];
+    __shared__ u32x4_t stage1[SLOTS];
+    __shared__ u32x4_t stage2[STAGES > 2 ? SLOTS : 1];
+    __shared__ u32x4_t stage3[STAGES > 3 ? SLOTS : 1];
+
+    const int total = p.tiles_n * p.tiles_m;
+    int logical;
+    {
+        int b = blockIdx.x, per = total / 8, rem = total % 8, xcd = b % 8, local = b / 8;
+        logical = xcd * per + (xcd < rem ? xcd : rem) + local;
+    }
+    constexpr int GROUP = 8;
+    const int span = GROUP * p.tiles_m;
+    const int first_n = (logical / span) * GROUP;
+    const int group_size = (p.tiles_n - first_n) < GROUP ? (p.tiles_n - first_n) : GROUP;
+    const int tile_n = first_n + (logical % span) % group_size;
+    const int tile_m = (logical % span) / group_size;
+    const int n0 = tile_n * BN, m0 = tile_m * BM;
+    const int k_tiles = p.k / BK;
+
+    const int thread = threadIdx.x, lane = thread % 64, wave = thread / 64;
+    const int wn = wave % 2, wm = wave / 2;
+
+    // ---- per-lane sources of the direct loads. Wave-instruction (it, wave) fills LDS slots
+    // [(it*4 + wave)*64, +64): row = (it*4 + wave)*ROWS_PER_LOAD + lane/CH, physical chunk lane%CH,
+    // which holds logical chunk (lane%CH) ^ swizzle(row). The address is a constant uniform base
+    // plus a 32-bit per-lane byte offset that advances by 2*BK per step (scalar base + vector
+    // offset addressing, one VGPR per load).
+    unsigned a_off[A_ITERS], b_off[B_ITERS];
+#pragma unroll
+    for (int it = 0; it < A_ITERS; ++it) {
+        int row = (it * 4 + wave) * ROWS_PER_LOAD + lane / CH;
+        int chunk = (lane % CH) ^ swizzle<CH>(row);
+        int global_row = n0 + row < p.n ? n0 + row : p.n - 1;
+        a_off[it] = (unsigned(global_row - n0) * unsigned(p.lda) + unsigned(chunk * 8)) * 2u;
+    }
+#pragma unroll
+    for (int it = 0; it < B_ITERS; ++it) {
+        int row = (it * 4 + wave) * ROWS_PER_LOAD + lane / CH;
+        int chunk = (lane % CH) ^ swizzle<CH>(row);
+        int global_row = m0 + row < p.m ? m0 + row : p.m - 1;
+        b_off[it] = (unsigned(global_row - m0) * unsigned(p.ldb) + unsigned(chunk * 8)) * 2u;
+    }
+    const char *a_base = reinterpret_cast<const char *>(p.w + size_t(n0) * p.lda);
+    const char *b_base = reinterpret_cast<const char *>(p.x + size_t(m0) * p.ldb);
+    unsigned k_bytes = 0;
+    auto issue = [&](u32x4_t *stage) {
+#pragma unroll
+        for (int it = 0; it < A_ITERS; ++it)
+            load_to_lds(a_base + (a_off[it] + k_bytes), stage + (it * 4 + wave) * 64);
+#pragma unroll
+        for (int it = 0; it < B_ITERS; ++it)
+            load_to_lds(b_base + (b_off[it] + k_bytes), stage + BN * CH + (it * 4 + wave) * 64);
+        k_bytes += BK * 2;
+    };
+
+    // ---- MFMA-layout read positions
+    const int frag_row = lane % 32, half = lane / 32;
+    const int frag_swizzle = swizzle<CH>(frag_row);
+    const int a_frag_base = (wn * TN * 32 + frag_row) * CH;
+    const int b_frag_base = BN * CH + (wm * TM * 32 + frag_row) * CH;
+
+    f32x16_t acc[TN][TM];
+#pragma unroll
+    for (int i = 0; i < TN; ++i)
+#pragma unroll
+        for (int j = 0; j < TM; ++j)
+#pragma unroll
+            for (int r = 0; r < 16; ++r)
+                acc[i][j][r] = 0.f;
+
+    auto multiply = [&](const u32x4_t *stage) {
+#pragma unroll
+        for (int ks = 0; ks < BK / 16; ++ks) {
+            const int column = (ks * 2 + half) ^ frag_swizzle;
+            bf16x8_t a_frag[TN], b_frag[TM];
+#pragma unroll
+            for (int i = 0; i < TN; ++i)
+                a_frag[i] = __builtin_bit_cast(bf16x8_t, stage[a_frag_base + i * 32 * CH + column]);
+#pragma unroll
+            for (int j = 0; j < TM; ++j)
+                b_frag[j] = __builtin_bit_cast(bf16x8_t, stage[b_frag_base + j * 32 * CH + column]);
+#pragma unroll
+            for (int i = 0; i < TN; ++i)
+#pragma unroll
+                for (int j = 0; j < TM; ++j)
+                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a_frag[i], b_frag[j],
+                                                                        acc[i][j], 0, 0, 0);
+        }
+    };
+    // One pipeline step: start the loads of step (tile + STAGES - 1) into the stage that was read
+    // last, multiply the current stage, then wait until this wavefront's loads for the next step
+    // have landed (newer ones may stay in flight) and meet the other wavefronts at the barrier.
+    // Loads are issued unconditionally; steps past the end re-read the last K block into a stage
+    // nobody multiplies, which keeps the outstanding-load count fixed.
+    auto step = [&](u32x4_t *fill, const u32x4_t *current) {
+        issue(fill);
+        multiply(current);
+        wait_loads<LOADS *(STAGES - 2)>();
+        __syncthreads();
+    };
+    const unsigned last_k_bytes = unsigned(k_tiles - 1) * BK * 2;
+    auto clamp_k = [&]() { k_bytes = k_bytes < last_k_bytes ? k_bytes : last_k_bytes; };
+
+    // prologue: STAGES - 1 steps in flight, the first one complete
+    issue(stage0);
+    clamp_k();
+    if constexpr (STAGES > 2) {
+        issue(stage1);
+        clamp_k();
+    }
+    if constexpr (STAGES > 3) {
+        issue(stage2);
+        clamp_k();
+    }
+    wait_loads<LOADS *(STAGES - 2)>();
+    __syncthreads();
+    for (int tile = 0; tile < k_tiles; tile += STAGES) {
+        if constexpr (STAGES == 2) {
+            step(stage1, stage0);
+            clamp_k();
+            if (tile + 1 < k_tiles)
+                step(stage0, stage1);
+            clamp_k();
+        } else if constexpr (STAGES == 3) {
+            step(stage2, stage0);
+            clamp_k();
+            if (tile + 1 < k_tiles)
+                step(stage0, stage1);
+            clamp_k();
+            if (tile + 2 < k_tiles)
+                step(stage1, stage2);
+            clamp_k();
+        } else {
+            step(stage3, stage0);
+            clamp_k();
+            if (tile + 1 < k_tiles)
+                step(stage0, stage1);
+            clamp_k();
+            if (tile + 2 < k_tiles)
+                step(stage1, stage2);
+            clamp_k();
+            if (tile + 3 < k_tiles)
+                step(stage2, stage3);
+            clamp_k();
+        }
+    }
+    wait_loads<0>(); // drain the padding loads before the LDS is released
+
+    // ---- epilogue. Accumulator register 4q+e of lane l is feature 8q + 4*(l/32) + e, token l%32.
+    const bool with_beta = p.beta != 0.f;
+#pragma unroll
+    for (int j = 0; j < TM; ++j) {
+        const int m = m0 + (wm * TM + j) * 32 + frag_row;
+        unsigned short *row = p.y + size_t(m) * p.ldc + n0 + wn * TN * 32 + half * 4;
+#pragma unroll
+        for (int i = 0; i < TN; ++i) {
+            __builtin_amdgcn_sched_barrier(0); // keep one accumulator tile live at a time
+#pragma unroll
+            for (int q = 0; q < 4; ++q) {
+                const int offset = i * 32 + q * 8;
+                if (m < p.m && n0 + wn * TN * 32 + half * 4 + offset < p.n) {
+                    float v0 = p.alpha * acc[i][j][q * 4], v1 = p.alpha * acc[i][j][q * 4 + 1];
+                    float v2 = p.alpha * acc[i][j][q * 4 + 2], v3 = p.alpha * acc[i][j][q * 4 + 3];
+                    if (with_beta) {
+                        u32x2_t old = *reinterpret_cast<const u32x2_t *>(row + offset);
+                        v0 = fmaf(p.beta, __uint_as_float(old[0] << 16), v0);
+                        v1 = fmaf(p.beta, __uint_as_float(old[0] & 0xffff0000u), v1);
+                        v2 = fmaf(p.beta, __uint_as_float(old[1] << 16), v2);
+                        v3 = fmaf(p.beta, __uint_as_float(old[1] & 0xffff0000u), v3);
+                    }
+                    u32x2_t packed = {pack_bf16x2(v0, v1), pack_bf16x2(v2, v3)};
+                    *reinterpret_cast<u32x2_t *>(row + offset) = packed;
+                }
+            }
+        }
+    }
+}
+
+template <int TN, int TM, int BK, int STAGES> hipError_t launch_dma(hipStream_t stream, DmaParams p)
+{
+    if (p.k % BK)
+        return hipErrorInvalidValue;
+    p.tiles_n = (p.n + 64 * TN - 1) / (64 * TN);
+    p.tiles_m = (p.m + 64 * TM - 1) / (64 * TM);
+    if (size_t(p.tiles_n) * size_t(p.tiles_m) > 0x7fffffffu)
+        return hipErrorInvalidValue;
+    bgemm_dma_kernel<TN, TM, BK, STAGES>
+        <<<unsigned(p.tiles_n) * unsigned(p.tiles_m), 256, 0, stream>>>(p);
+    return launch_status();
+}
+
+const TnVariant variants[] = {
+    {"dma256x256x32s4", 256, 256, 32, 256}, {"dma256x128x64s3", 256, 128, 64, 256},
+    {"dma128x128x64s2", 128, 128, 64, 256}, {"dma256x256x32s3", 256, 256, 32, 256},
+    {"dma256x128x64s2", 256, 128, 64, 256}, {"dma128x128x64s3", 128, 128, 64, 256},
+    {"dma256x128x32s4", 256, 128, 32, 256}, {"dma128x128x32s4", 128, 128, 32, 256},
+};
+} // namespace
+
+int dma_variant_count() { return int(sizeof(variants) / sizeof(variants[0])); }
+const TnVariant &dma_variant(int index) { return variants[index]; }
+
+hipError_t launch_bgemm_dma(hipStream_t stream, int variant, int n_out, int m_rows, int k,
+                            float alpha, const void *w, int lda, const void *x, int ldb, float beta,
+                            void *y, int ldc)
+{
+    if (k % 64 || n_out % 4 || ldc % 4 || reinterpret_cast<uintptr_t>(y) % 8)
+        return hipErrorInvalidValue;
+    // per-lane byte offsets are 32-bit: 256 rows of the widest operand plus the K extent must fit
+    if ((size_t(256) * size_t(lda > ldb ? lda : ldb) + size_t(k)) * 2 >= (size_t(1) << 32))
+        return hipErrorInvalidValue;
+    DmaParams p;
+    p.w = static_cast<const unsigned short *>(w);
+    p.x = static_cast<const unsigned short *>(x);
+    p.y = static_cast<unsigned short *>(y);
+    p.lda = lda;
+    p.ldb = ldb;
+    p.ldc = ldc;
+    p.n = n_out;
+    p.m = m_rows;
+    p.k = k;
+    p.alpha = alpha;
+    p.beta = beta;
+    p.tiles_n = p.tiles_m = 0;
+    switch (variant) {
+    case 0: return launch_dma<4, 4, 32, 4>(stream, p);
+    case 1: return launch_dma<4, 2, 64, 3>(stream, p);
+    case 2: return launch_dma<2, 2, 64, 2>(stream, p);
+    case 3: return launch_dma<4, 4, 32, 3>(stream, p);
+    case 4: return launch_dma<4, 2, 64, 2>(stream, p);
+    case 5: return launch_dma<2, 2, 64, 3>(stream, p);
+    case 6: return launch_dma<4, 2, 32, 4>(stream, p);
+    case 7: return launch_dma<2, 2, 32, 4>(stream, p);
+    default: return hipErrorInvalidValue;
+    }
+}
+} // namespace camblas_hip

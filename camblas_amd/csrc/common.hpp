@@ -45,7 +45,8 @@ enum KernelFamily {
     FAMILY_GEMV_F32 = 1,
     FAMILY_MFMA_TN = 2, // BF16 'T','N', K-contiguous operands, MFMA tiles staged through LDS
     FAMILY_FP8_BLOCK = 3,
-    FAMILY_STREAM = 4 // BF16 'T','N' with few tokens: weight-streaming kernel, one pass over W
+    FAMILY_STREAM = 4, // BF16 'T','N' with few tokens: weight-streaming kernel, one pass over W
+    FAMILY_DMA = 5     // BF16 'T','N' prefill: large MFMA tiles fed by direct global->LDS loads
 };
 
 struct Plan {
@@ -67,6 +68,8 @@ struct TnVariant {
 };
 int tn_variant_count();
 const TnVariant &tn_variant(int index);
+int dma_variant_count();
+const TnVariant &dma_variant(int index);
 int fp8_variant_count();
 const TnVariant &fp8_variant(int index);
 
@@ -89,6 +92,11 @@ hipError_t launch_gemv_f32(hipStream_t stream, int rows, int inner, float alpha,
 hipError_t launch_bgemm_tn(hipStream_t stream, int variant, int split_k, int n_out, int m_rows,
                            int k, float alpha, const void *w, int lda, const void *x, int ldb,
                            float beta, void *y, int ldc, float *partials);
+// Prefill BF16 linear with direct-to-LDS operand loads; variants are listed by dma_variant().
+// Needs k % 64 == 0, n_out % 4 == 0, ldc % 4 == 0, y 8-byte aligned.
+hipError_t launch_bgemm_dma(hipStream_t stream, int variant, int n_out, int m_rows, int k,
+                            float alpha, const void *w, int lda, const void *x, int ldb, float beta,
+                            void *y, int ldc);
 // Decode-shaped BF16 linear: each workgroup streams 16*row_tiles weight rows over the whole K.
 // mode: 0 = 4 wavefronts / 2 K steps in flight, 1 = 4 / 3, 2 = 8 / 2, 3 = 8 / 3.
 hipError_t launch_bgemv_stream(hipStream_t stream, int mode, int row_tiles, int token_tiles, int n_out,

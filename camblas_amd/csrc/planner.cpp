@@ -61,8 +61,7 @@ double occupancy_score(int n, int m, int block_n, int block_m, int resident, int
 Plan make_plan(int dtype, int algorithm, bool trans_a, bool trans_b, int m, int n, int k, int lda,
                int ldb, int ldc, bool aligned16, int compute_units)
 {
-    (void)ldc;
-    Plan plan;
+        Plan plan;
     if (compute_units < 1)
         compute_units = 256;
     if (dtype == 0) {
@@ -118,6 +117,10 @@ Plan make_plan(int dtype, int algorithm, bool trans_a, bool trans_b, int m, int 
                 }
             }
             plan.split_k = 1;
+            if (k % 64 == 0 && outputs % 4 == 0 && ldc % 4 == 0 && lda < (1 << 22) && ldb < (1 << 22)) {
+                // same tile choice with operands streamed straight into LDS
+                plan.family = FAMILY_DMA;
+            }
         }
         return plan;
     }
@@ -148,6 +151,9 @@ void describe_plan(const Plan &plan, int dtype, char *text, size_t bytes)
     case FAMILY_FP8_BLOCK:
         std::snprintf(text, bytes, "%s %s split_k=%d", type, fp8_variant(plan.kernel).name,
                       plan.split_k);
+        break;
+    case FAMILY_DMA:
+        std::snprintf(text, bytes, "%s %s", type, dma_variant(plan.kernel).name);
         break;
     case FAMILY_STREAM:
         std::snprintf(text, bytes, "%s stream rows=%d tokens=%d waves=%d depth=%d", type,

@@ -100,6 +100,25 @@ def test_streaming_kernel_every_variant(device, code, n_out, m_rows, pad):
         assert np.array_equal(got2d[:, n_out:], c0.reshape(m_rows, ldc)[:, n_out:])
 
 
+@pytest.mark.parametrize("code", range(20, 28))
+@pytest.mark.parametrize("n_out,m_rows,k", [(300, 70, 320), (512, 256, 64), (260, 513, 448)])
+def test_direct_lds_load_kernel(device, code, n_out, m_rows, k):
+    # direct global->LDS tiles: ragged N and M (partial tiles, clamped rows), odd and even numbers
+    # of 64-deep K steps, padded operand rows
+    lda, ldb, ldc = k + 8, k + 16, n_out + 4
+    w = oracle.fill_normal_bf16(220 + code, (n_out * lda,))
+    x = oracle.fill_normal_bf16(240 + code, (m_rows * ldb,))
+    c0 = oracle.fill_normal_bf16(260, (m_rows * ldc,))
+    for alpha, beta in ((1.0, 0.0), (0.5, -1.5)):
+        got = run_bgemm(device, "T", "N", n_out, m_rows, k, alpha, w, lda, x, ldb, beta, c0, ldc,
+                        override=(code, 1))
+        want, want64 = reference("T", "N", n_out, m_rows, k, alpha, w, lda, x, ldb, beta, c0, ldc)
+        got2d = got.reshape(m_rows, ldc)
+        error = rel_frobenius(oracle.bf16_to_f32(got2d[:, :n_out]), want64.reshape(m_rows, n_out))
+        assert error <= TOLERANCE, (code, alpha, beta, error)
+        assert np.array_equal(got2d[:, n_out:], c0.reshape(m_rows, ldc)[:, n_out:])
+
+
 @pytest.mark.parametrize("tokens", [1, 8, 32, 33, 64, 65, 200])
 def test_planned_linear_shapes(device, tokens):
     # aligned fast path as F.linear produces it; planner picks variant and split-K
@@ -150,7 +169,7 @@ def test_classical_algorithm_uses_generic_kernel(device):
                          oracle.linear_bf16_f64(x, w)) <= TOLERANCE
 
 
-@pytest.mark.parametrize("override", [None, (0, 1), (4, 2), (172, 1)])
+@pytest.mark.parametrize("override", [None, (0, 1), (4, 2), (172, 1), (20, 1), (22, 1)])
 def test_exact_identity_and_fp32_accumulation(device, override):
     # identity placement (ref: tests/test_bfloat16.py:94-110): W = I gives y = x exactly
     size = 256
