@@ -262,8 +262,8 @@ extern "C" int camblas_cuda_bgemm(camblas_cuda_context *context, char trans_a, c
                 plan.family = FAMILY_STREAM;
                 plan.kernel = context->override_kernel - 100;
                 plan.split_k = 1;
-            } else if (context->override_kernel >= 20 && context->override_kernel < 30) {
-                plan.family = FAMILY_DMA; // 20, 21, 22: direct-to-LDS tiles
+            } else if (context->override_kernel >= 20 && context->override_kernel < 60) {
+                plan.family = FAMILY_DMA; // 20..59: direct-to-LDS tile variants
                 plan.kernel = context->override_kernel - 20;
                 plan.split_k = 1;
             } else {

@@ -42,12 +42,25 @@ template <int CH> __device__ __forceinline__ int swizzle(int row)
 
 typedef __attribute__((address_space(3))) void lds_void;
 
-// 16 bytes per lane from global memory straight into LDS at `lds_base + lane*16` (the base must be
-// wave-uniform). Kept in a non-template function: inside a kernel template the host pass drops the
-// whole instantiation when it meets this target builtin.
-__device__ __forceinline__ void load_to_lds(const void *global, void *lds_base)
+// 16 bytes per lane from a buffer resource straight into LDS at `lds_base + lane*16` (the base
+// must be wave-uniform): buffer_load_dwordx4 ... offen lds. The source byte address is the
+// resource base + per-lane `lane_offset` + wave-uniform `step_offset`; bytes past the resource's
+// extent read as zero instead of faulting. A buffer load is used rather than global_load_lds
+// because the compiler treats the latter as a flat access that may also touch LDS, after which it
+// degrades every LDS wait in the loop to "wait for everything". Kept in a non-template function:
+// inside a kernel template the host pass drops the whole instantiation when it meets a target
+// builtin.
+__device__ __forceinline__ void load_to_lds(__amdgpu_buffer_rsrc_t resource, unsigned lane_offset,
+                                            unsigned step_offset, void *lds_base)
 {
-    __builtin_amdgcn_global_load_lds(global, (lds_void *)lds_base, 16, 0, 0);
+    __builtin_amdgcn_raw_ptr_buffer_load_lds(resource, (lds_void *)lds_base, 16, lane_offset,
+                                             step_offset, 0, 0);
+}
+
+// Raw buffer resource over `bytes` bytes starting at `base` (gfx9 descriptor word 3: 32-bit data).
+__device__ __forceinline__ __amdgpu_buffer_rsrc_t make_resource(const void *base, unsigned bytes)
+{
+    return __builtin_amdgcn_make_buffer_rsrc(const_cast<void *>(base), 0, int(bytes), 0x00020000);
 }
 
 // s_waitcnt vmcnt(N) with the other counters left alone (gfx9 encoding: vmcnt in bits 3:0 and
@@ -57,14 +70,17 @@ template <int N> __device__ __forceinline__ void wait_loads()
     __builtin_amdgcn_s_waitcnt((N & 15) | ((N >> 4) << 14) | 0x0f70);
 }
 
-// TN, TM: 32x32 MFMA tiles per wavefront along features / tokens (workgroup tile 64*TN x 64*TM);
-// BK: K elements per step (32 or 64); STAGES: LDS stages (STAGES - 1 steps are in flight).
-template <int TN, int TM, int BK, int STAGES>
-__global__ __launch_bounds__(256) void bgemm_dma_kernel(DmaParams p)
+// TN, TM: 32x32 MFMA tiles per wavefront along features / tokens; the workgroup has 2 x WM
+// wavefronts and owns a (64*TN) x (32*WM*TM) tile; BK: K elements per step (32 or 64); STAGES: LDS
+// stages (STAGES - 1 steps are in flight).
+template <int TN, int TM, int WM, int BK, int STAGES>
+__global__ __launch_bounds__(128 * WM) void bgemm_dma_kernel(DmaParams p)
 {
-    constexpr int BN = 64 * TN, BM = 64 * TM, CH = BK / 8;
+    constexpr int WAVES = 2 * WM;
+    constexpr int BN = 64 * TN, BM = 32 * WM * TM, CH = BK / 8;
     constexpr int ROWS_PER_LOAD = 64 / CH;               // rows one wave instruction fills
-    constexpr int A_ITERS = BN / (4 * ROWS_PER_LOAD), B_ITERS = BM / (4 * ROWS_PER_LOAD);
+    constexpr int A_ITERS = BN / (WAVES * ROWS_PER_LOAD), B_ITERS = BM / (WAVES * ROWS_PER_LOAD);
+    static_assert(A_ITERS >= 1 && B_ITERS >= 1 && (BK / 16) % 2 == 0, "load and fragment tiling");
     constexpr int LOADS = A_ITERS + B_ITERS;             // direct loads per wavefront and step
     constexpr int SLOTS = (BN + BM) * CH;
     static_assert(STAGES >= 2 && STAGES <= 4 && (BK == 32 || BK == 64), "pipeline shape");
@@ -92,38 +108,42 @@ __global__ __launch_bounds__(256) void bgemm_dma_kernel(DmaParams p)
     const int k_tiles = p.k / BK;
 
     const int thread = threadIdx.x, lane = thread % 64, wave = thread / 64;
-    const int wn = wave % 2, wm = wave / 2;
+    const int wn = wave % 2, wm = wave / 2; // 2 x WM wavefront grid
 
     // ---- per-lane sources of the direct loads. Wave-instruction (it, wave) fills LDS slots
-    // [(it*4 + wave)*64, +64): row = (it*4 + wave)*ROWS_PER_LOAD + lane/CH, physical chunk lane%CH,
-    // which holds logical chunk (lane%CH) ^ swizzle(row). The address is a constant uniform base
-    // plus a 32-bit per-lane byte offset that advances by 2*BK per step (scalar base + vector
-    // offset addressing, one VGPR per load).
+    // [(it*WAVES + wave)*64, +64): row = (it*WAVES + wave)*ROWS_PER_LOAD + lane/CH, chunk lane%CH,
+    // which holds logical chunk (lane%CH) ^ swizzle(row). The address is the tile's buffer
+    // resource plus a constant 32-bit per-lane byte offset plus a scalar offset that advances by
+    // 2*BK per step: one VGPR per load and no vector arithmetic in the loop.
     unsigned a_off[A_ITERS], b_off[B_ITERS];
 #pragma unroll
     for (int it = 0; it < A_ITERS; ++it) {
-        int row = (it * 4 + wave) * ROWS_PER_LOAD + lane / CH;
+        int row = (it * WAVES + wave) * ROWS_PER_LOAD + lane / CH;
         int chunk = (lane % CH) ^ swizzle<CH>(row);
         int global_row = n0 + row < p.n ? n0 + row : p.n - 1;
         a_off[it] = (unsigned(global_row - n0) * unsigned(p.lda) + unsigned(chunk * 8)) * 2u;
     }
 #pragma unroll
     for (int it = 0; it < B_ITERS; ++it) {
-        int row = (it * 4 + wave) * ROWS_PER_LOAD + lane / CH;
+        int row = (it * WAVES + wave) * ROWS_PER_LOAD + lane / CH;
         int chunk = (lane % CH) ^ swizzle<CH>(row);
         int global_row = m0 + row < p.m ? m0 + row : p.m - 1;
         b_off[it] = (unsigned(global_row - m0) * unsigned(p.ldb) + unsigned(chunk * 8)) * 2u;
     }
-    const char *a_base = reinterpret_cast<const char *>(p.w + size_t(n0) * p.lda);
-    const char *b_base = reinterpret_cast<const char *>(p.x + size_t(m0) * p.ldb);
+    // One resource per operand, covering exactly the rows of this tile that exist.
+    const int a_rows = p.n - n0 < BN ? p.n - n0 : BN, b_rows = p.m - m0 < BM ? p.m - m0 : BM;
+    const __amdgpu_buffer_rsrc_t a_resource = make_resource(
+        p.w + size_t(n0) * p.lda, (unsigned(a_rows - 1) * unsigned(p.lda) + unsigned(p.k)) * 2u);
+    const __amdgpu_buffer_rsrc_t b_resource = make_resource(
+        p.x + size_t(m0) * p.ldb, (unsigned(b_rows - 1) * unsigned(p.ldb) + unsigned(p.k)) * 2u);
     unsigned k_bytes = 0;
     auto issue = [&](u32x4_t *stage) {
 #pragma unroll
         for (int it = 0; it < A_ITERS; ++it)
-            load_to_lds(a_base + (a_off[it] + k_bytes), stage + (it * 4 + wave) * 64);
+            load_to_lds(a_resource, a_off[it], k_bytes, stage + (it * WAVES + wave) * 64);
 #pragma unroll
         for (int it = 0; it < B_ITERS; ++it)
-            load_to_lds(b_base + (b_off[it] + k_bytes), stage + BN * CH + (it * 4 + wave) * 64);
+            load_to_lds(b_resource, b_off[it], k_bytes, stage + BN * CH + (it * WAVES + wave) * 64);
         k_bytes += BK * 2;
     };
 
@@ -142,35 +162,55 @@ __global__ __launch_bounds__(256) void bgemm_dma_kernel(DmaParams p)
             for (int r = 0; r < 16; ++r)
                 acc[i][j][r] = 0.f;
 
-    auto multiply = [&](const u32x4_t *stage) {
+    // Fragment registers are double-buffered across the 16-deep sub-steps: while the MFMAs of one
+    // sub-step issue, the operands of the next are already on their way from LDS. The last
+    // sub-step of a K step overlaps with the first fragment reads of the next stage, which become
+    // legal once this wavefront's loads for that stage have landed and all wavefronts have met at
+    // the barrier (which also tells everyone that the current stage may be overwritten).
+    bf16x8_t a_frag[2][TN], b_frag[2][TM];
+    auto read = [&](const u32x4_t *stage, int ks, bf16x8_t(&a)[TN], bf16x8_t(&b)[TM]) {
+        const int column = (ks * 2 + half) ^ frag_swizzle;
 #pragma unroll
-        for (int ks = 0; ks < BK / 16; ++ks) {
-            const int column = (ks * 2 + half) ^ frag_swizzle;
-            bf16x8_t a_frag[TN], b_frag[TM];
+        for (int i = 0; i < TN; ++i)
+            a[i] = __builtin_bit_cast(bf16x8_t, stage[a_frag_base + i * 32 * CH + column]);
 #pragma unroll
-            for (int i = 0; i < TN; ++i)
-                a_frag[i] = __builtin_bit_cast(bf16x8_t, stage[a_frag_base + i * 32 * CH + column]);
+        for (int j = 0; j < TM; ++j)
+            b[j] = __builtin_bit_cast(bf16x8_t, stage[b_frag_base + j * 32 * CH + column]);
+    };
+    auto mfma = [&](const bf16x8_t(&a)[TN], const bf16x8_t(&b)[TM]) {
+#pragma unroll
+        for (int i = 0; i < TN; ++i)
 #pragma unroll
             for (int j = 0; j < TM; ++j)
-                b_frag[j] = __builtin_bit_cast(bf16x8_t, stage[b_frag_base + j * 32 * CH + column]);
-#pragma unroll
-            for (int i = 0; i < TN; ++i)
-#pragma unroll
-                for (int j = 0; j < TM; ++j)
-                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a_frag[i], b_frag[j],
-                                                                        acc[i][j], 0, 0, 0);
-        }
+                acc[i][j] =
+                    __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[i], b[j], acc[i][j], 0, 0, 0);
     };
+    constexpr int KS = BK / 16;
     // One pipeline step: start the loads of step (tile + STAGES - 1) into the stage that was read
-    // last, multiply the current stage, then wait until this wavefront's loads for the next step
-    // have landed (newer ones may stay in flight) and meet the other wavefronts at the barrier.
-    // Loads are issued unconditionally; steps past the end re-read the last K block into a stage
-    // nobody multiplies, which keeps the outstanding-load count fixed.
-    auto step = [&](u32x4_t *fill, const u32x4_t *current) {
+    // last, run the sub-steps of the current stage, and hand over to `next`. Loads are issued
+    // unconditionally; steps past the end re-read the last K block into a stage nobody multiplies,
+    // which keeps the outstanding-load count fixed.
+    // sched_barrier(0) pins this order; left alone, the scheduler sinks the direct loads to the
+    // end of the step and moves every fragment read next to its first use, which exposes both
+    // latencies.
+    auto step = [&](u32x4_t *fill, const u32x4_t *current, const u32x4_t *next) {
+        __builtin_amdgcn_sched_barrier(0);
         issue(fill);
-        multiply(current);
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int ks = 0; ks + 1 < KS; ++ks) {
+            read(current, ks + 1, a_frag[(ks + 1) & 1], b_frag[(ks + 1) & 1]);
+            __builtin_amdgcn_sched_barrier(0);
+            mfma(a_frag[ks & 1], b_frag[ks & 1]);
+            __builtin_amdgcn_sched_barrier(0);
+        }
         wait_loads<LOADS *(STAGES - 2)>();
         __syncthreads();
+        __builtin_amdgcn_sched_barrier(0);
+        read(next, 0, a_frag[0], b_frag[0]);
+        __builtin_amdgcn_sched_barrier(0);
+        mfma(a_frag[(KS - 1) & 1], b_frag[(KS - 1) & 1]);
+        __builtin_amdgcn_sched_barrier(0);
     };
     const unsigned last_k_bytes = unsigned(k_tiles - 1) * BK * 2;
     auto clamp_k = [&]() { k_bytes = k_bytes < last_k_bytes ? k_bytes : last_k_bytes; };
@@ -188,33 +228,34 @@ __global__ __launch_bounds__(256) void bgemm_dma_kernel(DmaParams p)
     }
     wait_loads<LOADS *(STAGES - 2)>();
     __syncthreads();
+    read(stage0, 0, a_frag[0], b_frag[0]);
     for (int tile = 0; tile < k_tiles; tile += STAGES) {
         if constexpr (STAGES == 2) {
-            step(stage1, stage0);
+            step(stage1, stage0, stage1);
             clamp_k();
             if (tile + 1 < k_tiles)
-                step(stage0, stage1);
+                step(stage0, stage1, stage0);
             clamp_k();
         } else if constexpr (STAGES == 3) {
-            step(stage2, stage0);
+            step(stage2, stage0, stage1);
             clamp_k();
             if (tile + 1 < k_tiles)
-                step(stage0, stage1);
+                step(stage0, stage1, stage2);
             clamp_k();
             if (tile + 2 < k_tiles)
-                step(stage1, stage2);
+                step(stage1, stage2, stage0);
             clamp_k();
         } else {
-            step(stage3, stage0);
+            step(stage3, stage0, stage1);
             clamp_k();
             if (tile + 1 < k_tiles)
-                step(stage0, stage1);
+                step(stage0, stage1, stage2);
             clamp_k();
             if (tile + 2 < k_tiles)
-                step(stage1, stage2);
+                step(stage1, stage2, stage3);
             clamp_k();
             if (tile + 3 < k_tiles)
-                step(stage2, stage3);
+                step(stage2, stage3, stage0);
             clamp_k();
         }
     }
@@ -250,24 +291,28 @@ __global__ __launch_bounds__(256) void bgemm_dma_kernel(DmaParams p)
     }
 }
 
-template <int TN, int TM, int BK, int STAGES> hipError_t launch_dma(hipStream_t stream, DmaParams p)
+template <int TN, int TM, int WM, int BK, int STAGES>
+hipError_t launch_dma(hipStream_t stream, DmaParams p)
 {
+    constexpr int BN = 64 * TN, BM = 32 * WM * TM;
     if (p.k % BK)
         return hipErrorInvalidValue;
-    p.tiles_n = (p.n + 64 * TN - 1) / (64 * TN);
-    p.tiles_m = (p.m + 64 * TM - 1) / (64 * TM);
+    p.tiles_n = (p.n + BN - 1) / BN;
+    p.tiles_m = (p.m + BM - 1) / BM;
     if (size_t(p.tiles_n) * size_t(p.tiles_m) > 0x7fffffffu)
         return hipErrorInvalidValue;
-    bgemm_dma_kernel<TN, TM, BK, STAGES>
-        <<<unsigned(p.tiles_n) * unsigned(p.tiles_m), 256, 0, stream>>>(p);
+    bgemm_dma_kernel<TN, TM, WM, BK, STAGES>
+        <<<unsigned(p.tiles_n) * unsigned(p.tiles_m), 128 * WM, 0, stream>>>(p);
     return launch_status();
 }
 
 const TnVariant variants[] = {
-    {"dma256x256x32s4", 256, 256, 32, 256}, {"dma256x128x64s3", 256, 128, 64, 256},
-    {"dma128x128x64s2", 128, 128, 64, 256}, {"dma256x256x32s3", 256, 256, 32, 256},
-    {"dma256x128x64s2", 256, 128, 64, 256}, {"dma128x128x64s3", 128, 128, 64, 256},
-    {"dma256x128x32s4", 256, 128, 32, 256}, {"dma128x128x32s4", 128, 128, 32, 256},
+    {"dma256x256x32s4w4", 256, 256, 32, 256}, {"dma256x128x64s3w4", 256, 128, 64, 256},
+    {"dma128x128x64s2w4", 128, 128, 64, 256}, {"dma256x256x32s3w4", 256, 256, 32, 256},
+    {"dma256x128x64s2w4", 256, 128, 64, 256}, {"dma128x128x64s3w4", 128, 128, 64, 256},
+    {"dma256x256x64s2w8", 256, 256, 64, 512}, {"dma256x256x32s4w8", 256, 256, 32, 512},
+    {"dma256x128x64s3w8", 256, 128, 64, 512}, {"dma128x256x64s3w8", 128, 256, 64, 512},
+    {"dma320x256x64s2w8", 320, 256, 64, 512}, {"dma192x256x64s2w8", 192, 256, 64, 512},
 };
 } // namespace
 
@@ -297,14 +342,18 @@ hipError_t launch_bgemm_dma(hipStream_t stream, int variant, int n_out, int m_ro
     p.beta = beta;
     p.tiles_n = p.tiles_m = 0;
     switch (variant) {
-    case 0: return launch_dma<4, 4, 32, 4>(stream, p);
-    case 1: return launch_dma<4, 2, 64, 3>(stream, p);
-    case 2: return launch_dma<2, 2, 64, 2>(stream, p);
-    case 3: return launch_dma<4, 4, 32, 3>(stream, p);
-    case 4: return launch_dma<4, 2, 64, 2>(stream, p);
-    case 5: return launch_dma<2, 2, 64, 3>(stream, p);
-    case 6: return launch_dma<4, 2, 32, 4>(stream, p);
-    case 7: return launch_dma<2, 2, 32, 4>(stream, p);
+    case 0: return launch_dma<4, 4, 2, 32, 4>(stream, p);
+    case 1: return launch_dma<4, 2, 2, 64, 3>(stream, p);
+    case 2: return launch_dma<2, 2, 2, 64, 2>(stream, p);
+    case 3: return launch_dma<4, 4, 2, 32, 3>(stream, p);
+    case 4: return launch_dma<4, 2, 2, 64, 2>(stream, p);
+    case 5: return launch_dma<2, 2, 2, 64, 3>(stream, p);
+    case 6: return launch_dma<4, 2, 4, 64, 2>(stream, p);
+    case 7: return launch_dma<4, 2, 4, 32, 4>(stream, p);
+    case 8: return launch_dma<4, 1, 4, 64, 3>(stream, p);
+    case 9: return launch_dma<2, 2, 4, 64, 3>(stream, p);
+    case 10: return launch_dma<5, 2, 4, 64, 2>(stream, p);
+    case 11: return launch_dma<3, 2, 4, 64, 2>(stream, p);
     default: return hipErrorInvalidValue;
     }
 }

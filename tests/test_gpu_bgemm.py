@@ -100,7 +100,7 @@ def test_streaming_kernel_every_variant(device, code, n_out, m_rows, pad):
         assert np.array_equal(got2d[:, n_out:], c0.reshape(m_rows, ldc)[:, n_out:])
 
 
-@pytest.mark.parametrize("code", range(20, 28))
+@pytest.mark.parametrize("code", range(20, 32))
 @pytest.mark.parametrize("n_out,m_rows,k", [(300, 70, 320), (512, 256, 64), (260, 513, 448)])
 def test_direct_lds_load_kernel(device, code, n_out, m_rows, k):
     # direct global->LDS tiles: ragged N and M (partial tiles, clamped rows), odd and even numbers
