@@ -80,7 +80,9 @@ __global__ __launch_bounds__(128 * WM) void bgemm_dma_kernel(DmaParams p)
     constexpr int BN = 64 * TN, BM = 32 * WM * TM, CH = BK / 8;
     constexpr int ROWS_PER_LOAD = 64 / CH;               // rows one wave instruction fills
     constexpr int A_ITERS = BN / (WAVES * ROWS_PER_LOAD), B_ITERS = BM / (WAVES * ROWS_PER_LOAD);
-    static_assert(A_ITERS >= 1 && B_ITERS >= 1 && (BK / 16) % 2 == 0, "load and fragment tiling");
+    static_assert(BN % (WAVES * ROWS_PER_LOAD) == 0 && BM % (WAVES * ROWS_PER_LOAD) == 0 &&
+                      (BK / 16) % 2 == 0,
+                  "every wavefront issues whole loads; fragment buffers alternate evenly");
     constexpr int LOADS = A_ITERS + B_ITERS;             // direct loads per wavefront and step
     constexpr int SLOTS = (BN + BM) * CH;
     static_assert(STAGES >= 2 && STAGES <= 4 && (BK == 32 || BK == 64), "pipeline shape");

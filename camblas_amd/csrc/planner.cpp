@@ -103,24 +103,42 @@ Plan make_plan(int dtype, int algorithm, bool trans_a, bool trans_b, int m, int 
         } else {
             // prefill: larger tiles reuse more per byte; prefer them unless a smaller tile fills
             // the compute units noticeably better
+            const bool direct = k % 64 == 0 && outputs % 4 == 0 && ldc % 4 == 0 &&
+                                lda < (1 << 22) && ldb < (1 << 22);
             double best = -1;
-            const int candidates[3] = {0, 1, 2};
-            const int resident[3] = {1, 1, 2};
-            const double weight[3] = {1.0, 0.95, 0.85};
-            for (int i = 0; i < 3; ++i) {
-                const TnVariant &v = tn_variant(candidates[i]);
-                double score = weight[i] * occupancy_score(outputs, tokens, v.block_n, v.block_m,
-                                                           resident[i], compute_units);
-                if (score > best) {
-                    best = score;
-                    plan.kernel = candidates[i];
+            if (direct) {
+                // direct-to-LDS tiles: {variant, resident workgroups per CU, relative efficiency}
+                const struct {
+                    int variant, resident;
+                    double weight;
+                } candidates[] = {{10, 1, 1.0}, {6, 1, 0.93}, {11, 1, 0.88}, {9, 1, 0.85}, {2, 2, 0.8}};
+                plan.family = FAMILY_DMA;
+                for (const auto &candidate : candidates) {
+                    const TnVariant &v = dma_variant(candidate.variant);
+                    double score = candidate.weight * occupancy_score(outputs, tokens, v.block_n,
+                                                                      v.block_m, candidate.resident,
+                                                                      compute_units);
+                    if (score > best) {
+                        best = score;
+                        plan.kernel = candidate.variant;
+                    }
+                }
+            } else {
+                const int candidates[3] = {0, 1, 2};
+                const int resident[3] = {1, 1, 2};
+                const double weight[3] = {0.5, 0.95, 1.0};
+                for (int i = 0; i < 3; ++i) {
+                    const TnVariant &v = tn_variant(candidates[i]);
+                    double score = weight[i] * occupancy_score(outputs, tokens, v.block_n,
+                                                               v.block_m, resident[i],
+                                                               compute_units);
+                    if (score > best) {
+                        best = score;
+                        plan.kernel = candidates[i];
+                    }
                 }
             }
             plan.split_k = 1;
-            if (k % 64 == 0 && outputs % 4 == 0 && ldc % 4 == 0 && lda < (1 << 22) && ldb < (1 << 22)) {
-                // same tile choice with operands streamed straight into LDS
-                plan.family = FAMILY_DMA;
-            }
         }
         return plan;
     }
