@@ -61,25 +61,23 @@ def cpu_port_baseline(budget_seconds=12.0):
     cores = len(os.sched_getaffinity(0))
     tokens = 32
     x = oracle.fill_normal_bf16(1, (tokens, INNER))
-    rows = 256
-    elapsed = 0.0
-    while True:
-        w = oracle.fill_normal_bf16(2, (rows, INNER), std=0.02)
-        out = oracle.f32_to_bf16(oracle.fill_uniform(3, (tokens, rows)) * 0)
+    rows = 4096
+    w = oracle.fill_normal_bf16(2, (rows, INNER), std=0.02)
+    out = oracle.f32_to_bf16(oracle.fill_uniform(3, (tokens, rows)) * 0)
+    elapsed, passes = 0.0, 0
+    while elapsed < budget_seconds and passes < 64:
         begin = time.perf_counter()
         oracle.bgemm_f64("T", "N", rows, tokens, INNER, 1.0, w, INNER, x, INNER, 0.0, out, rows)
-        elapsed = time.perf_counter() - begin
-        if elapsed * 4 > budget_seconds or rows >= OUTPUTS:
-            break
-        rows = min(OUTPUTS, rows * 4)
-    traffic = rows * INNER * 2 + tokens * INNER * 2 + tokens * rows * 2
+        elapsed += time.perf_counter() - begin
+        passes += 1
+    traffic = passes * (rows * INNER * 2 + tokens * INNER * 2 + tokens * rows * 2)
     return {
         "value": round(traffic / elapsed / 1e9, 3),
         "unit": "GB/s",
         "cores": cores,
         "kind": "port",
-        "sample": f"oracle_bgemm_f64 (OpenMP) on {rows} of {OUTPUTS} weight rows, M=32, K={INNER}, "
-                  f"{elapsed:.2f} s",
+        "sample": f"oracle_bgemm_f64 (OpenMP, FP64 accumulate) on {rows} of {OUTPUTS} weight rows "
+                  f"x {passes} passes, M=32, K={INNER}, {elapsed:.1f} s",
     }
 
 
@@ -114,6 +112,8 @@ def main():
     parser.add_argument("--warmup", type=int, default=10)
     parser.add_argument("--skip-extras", action="store_true")
     parser.add_argument("--skip-cpu", action="store_true")
+    parser.add_argument("--only", choices=("decode1", "decode8", "decode32", "prefill", "copy"),
+                        help="profiling aid: launch just this kernel --steps times, print nothing")
     args = parser.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this build measures one GPU only (no collectives exist in the linear "
@@ -133,6 +133,10 @@ def main():
     weights = [normal((OUTPUTS, INNER), 0.02) for _ in range(3)]
     inputs = {m: normal((m, INNER)) for m in BATCHES}
     outputs = {m: torch.empty((m, OUTPUTS), dtype=torch.bfloat16, device=device) for m in BATCHES}
+
+    if args.only:
+        profile_only(args, torch, _kernels, _native, device, normal, weights, inputs, outputs)
+        return
 
     def step(index):
         for position, m in enumerate(BATCHES):
@@ -166,7 +170,7 @@ def main():
         "peak": HBM_PEAK / 1e9,
         "unit": "GB/s",
         "frac": round(achieved / HBM_PEAK, 4),
-        "traffic": None,
+        "traffic": measured_traffic(),
         "launch_us": round(per_launch[32] * 1e6, 2),
     }
 
@@ -207,6 +211,47 @@ def main():
         if reference:
             result["also"]["cpu_reference_sgemm_2048"] = reference
     print(json.dumps(result))
+
+
+def measured_traffic():
+    """HBM bytes per M=32 launch from the committed counter profile (FETCH_SIZE + WRITE_SIZE, each
+    scaled by the copy-probe calibration), or None when that profile has not been taken."""
+    path = ROOT / "profiles" / "bgemv_stream_decode_m32_hbm_traffic.txt"
+    if not path.is_file():
+        return None
+    for line in path.read_text().splitlines():
+        if line.startswith("traffic_bytes_per_launch:"):
+            return int(float(line.split(":", 1)[1]))
+    return None
+
+
+def profile_only(args, torch, _kernels, _native, device, normal, weights, inputs, outputs):
+    """Launch one kernel repeatedly under an external profiler."""
+    import ctypes as ct
+
+    if args.only.startswith("decode"):
+        m = int(args.only[6:])
+
+        def launch(i):
+            _kernels.matmul(inputs[m], weights[i % 3].t(), out=outputs[m])
+    elif args.only == "copy":
+        size = OUTPUTS * INNER * 2
+        source, target = weights[0], weights[1]
+        native = _native.context(device)
+
+        def launch(i):
+            native.call("hip_copy_probe", size, ct.c_void_p(source.data_ptr()),
+                        ct.c_void_p(target.data_ptr()))
+    else:
+        tokens, features = 4096, 10240
+        x, w = normal((tokens, INNER)), normal((features, INNER), 0.02)
+        y = torch.empty((tokens, features), dtype=torch.bfloat16, device=device)
+
+        def launch(i):
+            _kernels.matmul(x, w.t(), out=y)
+    for index in range(args.warmup + args.steps):
+        launch(index)
+    torch.cuda.synchronize()
 
 
 def extras(torch, _kernels, _native, device, normal):

@@ -666,6 +666,20 @@ extern "C" int camblas_hip_set_plan_override(camblas_cuda_context *context, int 
     return 0;
 }
 
+extern "C" int camblas_hip_copy_probe(camblas_cuda_context *context, size_t bytes, const void *source,
+                                      void *destination)
+{
+    return execute(context, [&] {
+        if (bytes % 16 || !source || !destination || !aligned(source, 16) ||
+            !aligned(destination, 16))
+            return fail(context, "invalid copy probe arguments", 1);
+        if (!bytes)
+            return 0;
+        hipError_t error = launch_copy_probe(context->stream, bytes, source, destination);
+        return error == hipSuccess ? 0 : fail(context, "copy probe", error);
+    });
+}
+
 extern "C" int camblas_hip_kernel_count(int dtype)
 {
     return dtype == 2 ? tn_variant_count() : dtype == 3 ? fp8_variant_count() : 1;

@@ -117,6 +117,7 @@ hipError_t launch_rms_rows(hipStream_t stream, int dtype, int weight_dtype, int 
 hipError_t launch_bf16_square(hipStream_t stream, uint64_t count, const void *input, float *out);
 hipError_t launch_rms_scale(hipStream_t stream, int dtype, uint64_t count, int width, float epsilon,
                             const void *input, const void *weight, const float *means, void *out);
+hipError_t launch_copy_probe(hipStream_t stream, size_t bytes, const void *source, void *destination);
 hipError_t launch_rope(hipStream_t stream, int tokens, int heads, int dim, int token_stride,
                        float theta, const int32_t *positions, void *x);
 size_t gqa_decode_scratch_bytes(int batch, int q_heads, int dim, int context_length, int *splits);

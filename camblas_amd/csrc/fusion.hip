@@ -250,6 +250,14 @@ __global__ void rope_kernel(int tokens, int heads, int dim, int token_stride, fl
     v[i + half] = float_to_bf16_bits(hi * c + lo * s);
 }
 
+// Plain 16-byte-per-thread copy: the known-traffic kernel used to calibrate the HBM byte counters.
+__global__ void copy_probe_kernel(size_t vectors, const u32x4_t *source, u32x4_t *destination)
+{
+    for (size_t index = size_t(blockIdx.x) * blockDim.x + threadIdx.x; index < vectors;
+         index += size_t(gridDim.x) * blockDim.x)
+        destination[index] = source[index];
+}
+
 unsigned stride_blocks(uint64_t count)
 {
     uint64_t blocks = (count + 255) / 256;
@@ -352,6 +360,13 @@ hipError_t launch_rms_scale(hipStream_t stream, int dtype, uint64_t count, int w
         rms_scale_kernel<bf16_storage><<<stride_blocks(count), 256, 0, stream>>>(
             count, width, epsilon, static_cast<const bf16_storage *>(input),
             static_cast<const bf16_storage *>(weight), means, static_cast<bf16_storage *>(out));
+    return launch_status();
+}
+
+hipError_t launch_copy_probe(hipStream_t stream, size_t bytes, const void *source, void *destination)
+{
+    copy_probe_kernel<<<2048, 256, 0, stream>>>(bytes / 16, static_cast<const u32x4_t *>(source),
+                                                static_cast<u32x4_t *>(destination));
     return launch_status();
 }
 

@@ -183,6 +183,11 @@ int camblas_hip_plan_describe(int dtype, int algorithm, char trans_a, char trans
 /* extension. Diagnostics for tests and tuning: force the planner's choice for BF16/FP8 GEMMs on
  * this context (kernel < 0 restores the planner; split_k <= 0 lets the planner choose). */
 int camblas_hip_set_plan_override(camblas_cuda_context *context, int kernel, int split_k);
+/* extension. Diagnostics: copies `bytes` (a multiple of 16, 16-byte aligned buffers) with a plain
+ * grid-stride kernel. A launch of known HBM traffic (bytes read + bytes written) against which
+ * the hardware byte counters are calibrated. */
+int camblas_hip_copy_probe(camblas_cuda_context *context, size_t bytes, const void *source,
+                           void *destination);
 /* extension. Number of kernel variants `camblas_hip_set_plan_override` accepts for a dtype. */
 int camblas_hip_kernel_count(int dtype);
 
