@@ -80,12 +80,15 @@ __global__ __launch_bounds__(WAVES * 64) void bgemv_stream_kernel(StreamParams p
     auto fetch = [&](int step, u32x4_t(&a)[NT], u32x4_t(&b)[MT]) {
         int k0 = rotated(step) * BK + chunk * 8;
         k0 = k0 < p.k ? k0 : p.k - 8;
+        // padding steps past the end (their data is masked away) all read one cached line
+        const unsigned live = step < k_tiles ? 0xffffffffu : 0u;
+        k0 &= int(live);
 #pragma unroll
         for (int i = 0; i < NT; ++i)
-            a[i] = *reinterpret_cast<const u32x4_t *>(a_base + k0 + a_off[i]);
+            a[i] = *reinterpret_cast<const u32x4_t *>(a_base + k0 + (a_off[i] & live));
 #pragma unroll
         for (int j = 0; j < MT; ++j)
-            b[j] = *reinterpret_cast<const u32x4_t *>(b_base + k0 + b_off[j]);
+            b[j] = *reinterpret_cast<const u32x4_t *>(b_base + k0 + (b_off[j] & live));
     };
     auto stash = [&](int stage, int step, const u32x4_t(&a)[NT], const u32x4_t(&b)[MT]) {
         const unsigned mask =

@@ -1,0 +1,119 @@
+"""Host-side checks that need no GPU: the C-ABI library loads and exports every symbol the header
+declares and every symbol the reference's loader resolves, the planner (a pure host function)
+makes the documented choices, the Python surface mirrors the reference's contract, and bench.py
+refuses more than one GPU."""
+
+import ctypes as ct
+import os
+import re
+import subprocess
+import sys
+from pathlib import Path
+
+import pytest
+import torch
+
+from camblas_amd import _kernels, _native
+
+ROOT = Path(__file__).resolve().parents[1]
+HEADER = (ROOT / "include" / "camblas_hip.h").read_text()
+
+
+def declared_symbols():
+    names = re.findall(r"\b(camblas_(?:cuda|hip)_[a-z0-9_]+)\s*\(", HEADER)
+    return sorted(set(names))
+
+
+def test_library_exports_every_declared_symbol():
+    lib = ct.CDLL(str(_native.library_path()))
+    names = declared_symbols()
+    assert len(names) >= 30
+    for name in names:
+        assert hasattr(lib, name), name
+
+
+def test_reference_loader_contract_symbols_present():
+    # the names the reference's ctypes loader resolves at load time (camblas/_native.py:97-173);
+    # only bgemm is optional there
+    lib = _native.library()
+    for name in ("create", "destroy", "error", "set_algorithm", "stats", "reset_stats", "affine",
+                 "mlp", "sgemm", "dgemm", "bgemm", "attention"):
+        assert hasattr(lib, "camblas_cuda_" + name)
+    # every Python-side signature names an exported symbol
+    for name in _native.SIGNATURES:
+        assert hasattr(lib, _native.symbol_name(name)), name
+
+
+def test_null_context_and_stats_errors_without_a_device():
+    lib = _native.library()
+    assert lib.camblas_cuda_destroy(None) == 0
+    assert lib.camblas_cuda_set_algorithm(None, 0) == -1
+    assert b"invalid algorithm failed (status 1)" in lib.camblas_cuda_error(None)
+    assert lib.camblas_cuda_sgemm(None, b"N", b"N", 1, 1, 1, 1.0, None, 1, None, 1, 0.0, None, 1) == -1
+    assert b"missing context" in lib.camblas_cuda_error(None)
+    counts = (ct.c_uint64 * 8)()
+    assert lib.camblas_cuda_stats(None, counts, 8) == -1
+    assert lib.camblas_cuda_fp8_block_workspace_size(4, 256) == 4 * 256 + 4 * 2 * 4
+    assert lib.camblas_cuda_fp8_block_workspace_size(4, 100) == 0
+
+
+def test_planner_choices_for_the_baseline_shapes():
+    describe = _native.plan_describe
+    # decode linears: weight-streaming kernel, one workgroup per compute unit for the up-projection
+    code, text = describe(2, "T", "N", 28672, 32, 8192, 8192, 8192, 28672)
+    assert code // 100 == 4 and "stream rows=112 tokens=32" in text
+    assert "tokens=16" in describe(2, "T", "N", 28672, 1, 8192, 8192, 8192, 28672)[1]
+    assert "rows=32" in describe(2, "T", "N", 8192, 32, 28672, 28672, 28672, 8192)[1]
+    # prefill: direct-to-LDS MFMA tile that divides 10240 x 4096 into exactly two waves of tiles
+    code, text = describe(2, "T", "N", 10240, 4096, 8192, 8192, 8192, 10240)
+    assert code // 100 == 5 and "dma320x256" in text
+    # K not a multiple of 64: register-staged MFMA tiles; unaligned or other layouts: generic
+    assert describe(2, "T", "N", 10240, 4096, 8200, 8200, 8200, 10240)[0] // 100 == 2
+    assert describe(2, "T", "N", 1024, 64, 1001, 1001, 1001, 1024)[0] // 100 == 0
+    assert describe(2, "N", "N", 1024, 64, 1024, 1024, 1024, 1024)[0] // 100 == 0
+    assert describe(2, "T", "N", 1024, 64, 1024, 1024, 1024, 1024, aligned16=False)[0] // 100 == 0
+    assert describe(2, "T", "N", 1024, 64, 1024, 1024, 1024, 1024, algorithm="classical")[0] // 100 == 0
+    # FP32: single-vector shortcut only under auto (ref: src/cuda/backend.cu:810-815)
+    assert describe(0, "T", "N", 4096, 1, 4096, 4096, 4096, 4096)[0] // 100 == 1
+    assert describe(0, "T", "N", 4096, 1, 4096, 4096, 4096, 4096, algorithm="lt")[0] // 100 == 0
+    assert describe(0, "T", "N", 1000, 1, 4096, 4096, 4096, 1000)[0] // 100 == 0
+    assert describe(0, "N", "N", 2048, 2048, 2048, 2048, 2048, 2048)[0] // 100 == 0
+    # the plan is a pure function of its arguments
+    assert describe(3, "T", "N", 18432, 16, 7168, 7168, 7168, 18432) == describe(
+        3, "T", "N", 18432, 16, 7168, 7168, 7168, 18432)
+
+
+def test_operand_layout_mapping():
+    # ref: src/cuda/torch_bindings.cpp:146-153
+    base = torch.zeros(6, 8)
+    assert _kernels._operand(base)[1:] == (b"N", 8)
+    assert _kernels._operand(base.t())[1:] == (b"T", 8)
+    assert _kernels._operand(base[:, :5])[1:] == (b"N", 8)          # padded rows keep their stride
+    assert _kernels._operand(base[:, ::2])[1:] == (b"N", 4)         # neither: made contiguous
+    assert _kernels._operand(torch.zeros(1, 8))[1:] == (b"N", 8)
+    assert _kernels._operand(torch.zeros(8, 1).t())[1:] == (b"T", 1)        # [1, 8] view of a column
+
+
+def test_python_surface_contract(monkeypatch):
+    assert _native.ALGORITHMS["lt"] == 3 and _native.COUNTERS[4] == "lt"
+    with pytest.raises(ValueError):
+        _native.set_algorithm("fastest")
+    import camblas_amd
+
+    monkeypatch.delenv("CAMBLAS_ENABLE", raising=False)
+    assert camblas_amd._autoload() is None  # disabled processes touch nothing
+    with pytest.raises(RuntimeError):
+        _kernels.matmul(torch.zeros(2, 2), torch.zeros(2, 2))  # CPU tensors are rejected, no fallback
+
+
+def test_missing_library_fails_loudly(tmp_path):
+    code = "from camblas_amd import _native; _native.library()"
+    env = dict(os.environ, CAMBLAS_CUDA_LIBRARY=str(tmp_path / "absent.so"), PYTHONPATH=str(ROOT))
+    result = subprocess.run([sys.executable, "-c", code], capture_output=True, text=True, env=env)
+    assert result.returncode != 0 and "libcamblas_hip.so not found" in result.stderr
+
+
+def test_bench_refuses_more_than_one_gpu():
+    result = subprocess.run([sys.executable, str(ROOT / "bench.py"), "--gpus", "2"],
+                            capture_output=True, text=True)
+    assert result.returncode != 0 and "one GPU" in result.stderr
