@@ -29,6 +29,7 @@ CORE_SOURCES = (
     "bgemv_stream.hip",
     "bgemm_dma.hip",
     "fp8_block.hip",
+    "fp8_dma.hip",
     "fusion.hip",
     "attention_decode.hip",
 )

@@ -526,10 +526,26 @@ extern "C" int camblas_cuda_fp8_block_matmul(camblas_cuda_context *context, int 
             return fail(context, "invalid FP8 block matrix buffers", 1);
         Plan plan = make_plan(3, context->algorithm, true, false, outputs, rows, inner, inner, inner,
                               outputs, true, context->compute_units);
+        if (plan.family == FAMILY_FP8_DMA && !aligned(out, 8))
+            plan = Plan{FAMILY_FP8_BLOCK, 0, 1, 4};
         if (context->override_kernel >= 0) {
-            plan.kernel = context->override_kernel;
-            if (context->override_split > 0)
-                plan.split_k = context->override_split;
+            // diagnostics: 0.. register-staged variants (with split-K), 20.. direct-to-LDS variants
+            if (context->override_kernel >= 20) {
+                plan.family = FAMILY_FP8_DMA;
+                plan.kernel = context->override_kernel - 20;
+                plan.split_k = 1;
+            } else {
+                plan.family = FAMILY_FP8_BLOCK;
+                plan.kernel = context->override_kernel;
+                plan.split_k = context->override_split > 0 ? context->override_split : 1;
+            }
+        }
+        if (plan.family == FAMILY_FP8_DMA) {
+            context->counts[plan.counter]++;
+            hipError_t error = launch_fp8_dma(context->stream, plan.kernel, rows, outputs, inner, a,
+                                              a_scale, w, w_scale, out);
+            return error == hipSuccess ? 0
+                                       : fail(context, "FP8 block-scaled GEMM (direct LDS loads)", error);
         }
         float *partials = nullptr;
         if (plan.split_k > 1) {

@@ -15,6 +15,7 @@
 // Contract: ref src/cuda/bfloat16.cuh:11-57 ('T','N' call of src/cuda/torch_bindings.cpp:155-199).
 #include "common.hpp"
 #include "device.hpp"
+#include "dma.hpp"
 
 namespace camblas_hip
 {
@@ -29,46 +30,6 @@ struct DmaParams {
     float alpha, beta;
     int tiles_n, tiles_m;
 };
-
-// XOR applied to the 16-byte chunk index inside an LDS row of CH chunks: any 8 (and any 16)
-// consecutive rows land on distinct banks for a fixed logical chunk.
-template <int CH> __device__ __forceinline__ int swizzle(int row)
-{
-    if constexpr (CH == 8)
-        return ((row >> 1) & 7) ^ ((row & 1) << 2);
-    else
-        return (((row >> 2) & 1) << 1) | (((row >> 1) ^ (row >> 3)) & 1);
-}
-
-typedef __attribute__((address_space(3))) void lds_void;
-
-// 16 bytes per lane from a buffer resource straight into LDS at `lds_base + lane*16` (the base
-// must be wave-uniform): buffer_load_dwordx4 ... offen lds. The source byte address is the
-// resource base + per-lane `lane_offset` + wave-uniform `step_offset`; bytes past the resource's
-// extent read as zero instead of faulting. A buffer load is used rather than global_load_lds
-// because the compiler treats the latter as a flat access that may also touch LDS, after which it
-// degrades every LDS wait in the loop to "wait for everything". Kept in a non-template function:
-// inside a kernel template the host pass drops the whole instantiation when it meets a target
-// builtin.
-__device__ __forceinline__ void load_to_lds(__amdgpu_buffer_rsrc_t resource, unsigned lane_offset,
-                                            unsigned step_offset, void *lds_base)
-{
-    __builtin_amdgcn_raw_ptr_buffer_load_lds(resource, (lds_void *)lds_base, 16, lane_offset,
-                                             step_offset, 0, 0);
-}
-
-// Raw buffer resource over `bytes` bytes starting at `base` (gfx9 descriptor word 3: 32-bit data).
-__device__ __forceinline__ __amdgpu_buffer_rsrc_t make_resource(const void *base, unsigned bytes)
-{
-    return __builtin_amdgcn_make_buffer_rsrc(const_cast<void *>(base), 0, int(bytes), 0x00020000);
-}
-
-// s_waitcnt vmcnt(N) with the other counters left alone (gfx9 encoding: vmcnt in bits 3:0 and
-// 15:14, expcnt 6:4, lgkmcnt 11:8).
-template <int N> __device__ __forceinline__ void wait_loads()
-{
-    __builtin_amdgcn_s_waitcnt((N & 15) | ((N >> 4) << 14) | 0x0f70);
-}
 
 // TN, TM: 32x32 MFMA tiles per wavefront along features / tokens; the workgroup has 2 x WM
 // wavefronts and owns a (64*TN) x (32*WM*TM) tile; BK: K elements per step (32 or 64); STAGES: LDS
@@ -94,18 +55,8 @@ __global__ __launch_bounds__(128 * WM) void bgemm_dma_kernel(DmaParams p)
     __shared__ u32x4_t stage2[STAGES > 2 ? SLOTS : 1];
     __shared__ u32x4_t stage3[STAGES > 3 ? SLOTS : 1];
 
-    const int total = p.tiles_n * p.tiles_m;
-    int logical;
-    {
-        int b = blockIdx.x, per = total / 8, rem = total % 8, xcd = b % 8, local = b / 8;
-        logical = xcd * per + (xcd < rem ? xcd : rem) + local;
-    }
-    constexpr int GROUP = 8;
-    const int span = GROUP * p.tiles_m;
-    const int first_n = (logical / span) * GROUP;
-    const int group_size = (p.tiles_n - first_n) < GROUP ? (p.tiles_n - first_n) : GROUP;
-    const int tile_n = first_n + (logical % span) % group_size;
-    const int tile_m = (logical % span) / group_size;
+    int tile_n, tile_m;
+    xcd_tile(int(blockIdx.x), p.tiles_n, p.tiles_m, tile_n, tile_m);
     const int n0 = tile_n * BN, m0 = tile_m * BM;
     const int k_tiles = p.k / BK;
 
@@ -121,14 +72,14 @@ __global__ __launch_bounds__(128 * WM) void bgemm_dma_kernel(DmaParams p)
 #pragma unroll
     for (int it = 0; it < A_ITERS; ++it) {
         int row = (it * WAVES + wave) * ROWS_PER_LOAD + lane / CH;
-        int chunk = (lane % CH) ^ swizzle<CH>(row);
+        int chunk = (lane % CH) ^ lds_swizzle<CH>(row);
         int global_row = n0 + row < p.n ? n0 + row : p.n - 1;
         a_off[it] = (unsigned(global_row - n0) * unsigned(p.lda) + unsigned(chunk * 8)) * 2u;
     }
 #pragma unroll
     for (int it = 0; it < B_ITERS; ++it) {
         int row = (it * WAVES + wave) * ROWS_PER_LOAD + lane / CH;
-        int chunk = (lane % CH) ^ swizzle<CH>(row);
+        int chunk = (lane % CH) ^ lds_swizzle<CH>(row);
         int global_row = m0 + row < p.m ? m0 + row : p.m - 1;
         b_off[it] = (unsigned(global_row - m0) * unsigned(p.ldb) + unsigned(chunk * 8)) * 2u;
     }
@@ -151,7 +102,7 @@ __global__ __launch_bounds__(128 * WM) void bgemm_dma_kernel(DmaParams p)
 
     // ---- MFMA-layout read positions
     const int frag_row = lane % 32, half = lane / 32;
-    const int frag_swizzle = swizzle<CH>(frag_row);
+    const int frag_swizzle = lds_swizzle<CH>(frag_row);
     const int a_frag_base = (wn * TN * 32 + frag_row) * CH;
     const int b_frag_base = BN * CH + (wm * TM * 32 + frag_row) * CH;
 

@@ -46,7 +46,8 @@ enum KernelFamily {
     FAMILY_MFMA_TN = 2, // BF16 'T','N', K-contiguous operands, MFMA tiles staged through LDS
     FAMILY_FP8_BLOCK = 3,
     FAMILY_STREAM = 4, // BF16 'T','N' with few tokens: weight-streaming kernel, one pass over W
-    FAMILY_DMA = 5     // BF16 'T','N' prefill: large MFMA tiles fed by direct global->LDS loads
+    FAMILY_DMA = 5,    // BF16 'T','N' prefill: large MFMA tiles fed by direct global->LDS loads
+    FAMILY_FP8_DMA = 6 // FP8 block-scaled prefill: the same structure with one scale group per step
 };
 
 struct Plan {
@@ -70,6 +71,8 @@ int tn_variant_count();
 const TnVariant &tn_variant(int index);
 int dma_variant_count();
 const TnVariant &dma_variant(int index);
+int fp8_dma_variant_count();
+const TnVariant &fp8_dma_variant(int index);
 int fp8_variant_count();
 const TnVariant &fp8_variant(int index);
 
@@ -105,6 +108,10 @@ hipError_t launch_bgemv_stream(hipStream_t stream, int mode, int row_tiles, int 
 hipError_t launch_fp8_block(hipStream_t stream, int variant, int split_k, int rows, int outputs,
                             int inner, const void *a, const float *a_scale, const void *w,
                             const float *w_scale, void *out, float *partials);
+// Prefill FP8 block-scaled linear with direct-to-LDS loads; needs outputs % 4 == 0.
+hipError_t launch_fp8_dma(hipStream_t stream, int variant, int rows, int outputs, int inner,
+                          const void *a, const float *a_scale, const void *w, const float *w_scale,
+                          void *out);
 hipError_t launch_fp8_quantise(hipStream_t stream, int rows, int inner, const void *x, void *q,
                                float *scale);
 hipError_t launch_silu_multiply(hipStream_t stream, int dtype, uint64_t count, const void *gate,

@@ -1,0 +1,66 @@
+// Helpers shared by the kernels that fill LDS tiles with direct loads (buffer_load ... lds).
+#pragma once
+
+#include "device.hpp"
+
+namespace camblas_hip
+{
+// XOR applied to the 16-byte chunk index inside an LDS row of CH chunks: any 8 (and any 16)
+// consecutive rows land on distinct banks for a fixed logical chunk, for 128-bit accesses.
+template <int CH> __device__ __forceinline__ int lds_swizzle(int row)
+{
+    if constexpr (CH == 8)
+        return ((row >> 1) & 7) ^ ((row & 1) << 2);
+    else if constexpr (CH == 16)
+        return row & 15;
+    else
+        return (((row >> 2) & 1) << 1) | (((row >> 1) ^ (row >> 3)) & 1);
+}
+
+typedef __attribute__((address_space(3))) void lds_void_t;
+
+// 16 bytes per lane from a buffer resource straight into LDS at `lds_base + lane*16` (the base
+// must be wave-uniform): buffer_load_dwordx4 ... offen lds. The source byte address is the
+// resource base + per-lane `lane_offset` + wave-uniform `step_offset`; bytes past the resource's
+// extent read as zero instead of faulting. A buffer load is used rather than global_load_lds
+// because the compiler treats the latter as a flat access that may also touch LDS, after which it
+// degrades every LDS wait in the loop to "wait for everything". Kept in a non-template function:
+// inside a kernel template the host pass drops the whole instantiation when it meets a target
+// builtin.
+__device__ __forceinline__ void load_to_lds(__amdgpu_buffer_rsrc_t resource, unsigned lane_offset,
+                                            unsigned step_offset, void *lds_base)
+{
+    __builtin_amdgcn_raw_ptr_buffer_load_lds(resource, (lds_void_t *)lds_base, 16, lane_offset,
+                                             step_offset, 0, 0);
+}
+
+// Raw buffer resource over `bytes` bytes starting at `base` (gfx9 descriptor word 3: 32-bit data).
+__device__ __forceinline__ __amdgpu_buffer_rsrc_t make_resource(const void *base, unsigned bytes)
+{
+    return __builtin_amdgcn_make_buffer_rsrc(const_cast<void *>(base), 0, int(bytes), 0x00020000);
+}
+
+// s_waitcnt vmcnt(N) with the other counters left alone (gfx9 encoding: vmcnt in bits 3:0 and
+// 15:14, expcnt 6:4, lgkmcnt 11:8).
+template <int N> __device__ __forceinline__ void wait_loads()
+{
+    static_assert(N >= 0 && N < 64, "vmcnt holds 6 bits");
+    __builtin_amdgcn_s_waitcnt((N & 15) | ((N >> 4) << 14) | 0x0f70);
+}
+
+// Workgroup index -> output tile: consecutive workgroups go to different XCDs, so each XCD is given
+// a contiguous range of logical tile numbers, and logical numbers walk the tile grid in groups of
+// eight feature tiles so that the tiles resident on one XCD share operand panels through its L2.
+__device__ __forceinline__ void xcd_tile(int block, int tiles_n, int tiles_m, int &tile_n, int &tile_m)
+{
+    const int total = tiles_n * tiles_m;
+    const int per = total / 8, rem = total % 8, xcd = block % 8, local = block / 8;
+    const int logical = xcd * per + (xcd < rem ? xcd : rem) + local;
+    constexpr int GROUP = 8;
+    const int span = GROUP * tiles_m;
+    const int first_n = (logical / span) * GROUP;
+    const int group_size = (tiles_n - first_n) < GROUP ? (tiles_n - first_n) : GROUP;
+    tile_n = first_n + (logical % span) % group_size;
+    tile_m = (logical % span) / group_size;
+}
+} // namespace camblas_hip

@@ -143,12 +143,33 @@ Plan make_plan(int dtype, int algorithm, bool trans_a, bool trans_b, int m, int 
         return plan;
     }
     // FP8 block-scaled: rows = n (tokens), outputs = m, always K-contiguous
-    plan.family = FAMILY_FP8_BLOCK;
     plan.counter = 4;
-    plan.kernel = n <= 32 ? 1 : 0;
     if (n <= 32) {
+        plan.family = FAMILY_FP8_BLOCK;
+        plan.kernel = 1;
         const TnVariant &v = fp8_variant(plan.kernel);
         plan.split_k = decode_split(ceil_div(m, v.block_n), ceil_div(k, v.block_k), compute_units);
+        return plan;
+    }
+    if (m % 4 != 0 || k >= (1 << 24)) {
+        plan.family = FAMILY_FP8_BLOCK;
+        plan.kernel = 0;
+        return plan;
+    }
+    plan.family = FAMILY_FP8_DMA;
+    const struct {
+        int variant, resident;
+        double weight;
+    } candidates[] = {{1, 1, 1.0}, {3, 1, 0.9}};
+    double best = -1;
+    for (const auto &candidate : candidates) {
+        const TnVariant &v = fp8_dma_variant(candidate.variant);
+        double score = candidate.weight * occupancy_score(m, n, v.block_n, v.block_m,
+                                                          candidate.resident, compute_units);
+        if (score > best) {
+            best = score;
+            plan.kernel = candidate.variant;
+        }
     }
     return plan;
 }
@@ -169,6 +190,9 @@ void describe_plan(const Plan &plan, int dtype, char *text, size_t bytes)
     case FAMILY_FP8_BLOCK:
         std::snprintf(text, bytes, "%s %s split_k=%d", type, fp8_variant(plan.kernel).name,
                       plan.split_k);
+        break;
+    case FAMILY_FP8_DMA:
+        std::snprintf(text, bytes, "%s %s", type, fp8_dma_variant(plan.kernel).name);
         break;
     case FAMILY_DMA:
         std::snprintf(text, bytes, "%s %s", type, dma_variant(plan.kernel).name);

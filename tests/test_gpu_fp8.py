@@ -56,6 +56,21 @@ def test_random_blocks_every_variant(device, variant, split, rows):
         assert (np.abs(bf16_values(out) - wanted) <= bound).all()
 
 
+@pytest.mark.parametrize("code", [20, 21, 22, 23])
+@pytest.mark.parametrize("rows,outputs,inner", [(70, 300, 512), (256, 512, 128), (513, 260, 896)])
+def test_direct_lds_load_variants(device, code, rows, outputs, inner):
+    # partial tiles in both directions, a partial last weight-scale block, odd and even numbers of
+    # K groups; the ordered chain is the same as the oracle's, so results agree to one BF16 unit
+    a, a_scale = oracle.fill_fp8_blocks(700 + rows, rows, inner, 1)
+    w, w_scale = oracle.fill_fp8_blocks(701, outputs, inner, 128)
+    out = run(device, a, a_scale, w, w_scale, override=(code, 1))
+    want64 = oracle.fp8_block_matmul_f64(a, a_scale, w, w_scale)
+    assert rel_frobenius(bf16_values(out), want64) <= TOLERANCE
+    ordered = oracle.bf16_to_f32(oracle.fp8_block_matmul(a, a_scale, w, w_scale))
+    bound = 2.0**-7 * np.abs(ordered) + 1e-4 * np.abs(want64).max()
+    assert (np.abs(bf16_values(out) - ordered) <= bound).all()
+
+
 @pytest.mark.parametrize("rows", [1, 16, 256])
 def test_planned_shapes(device, rows):
     outputs, inner = 1536, 1024
@@ -65,7 +80,7 @@ def test_planned_shapes(device, rows):
     assert rel_frobenius(bf16_values(out), oracle.fp8_block_matmul_f64(a, a_scale, w, w_scale)) <= TOLERANCE
 
 
-@pytest.mark.parametrize("override", [None, (0, 1), (1, 1), (2, 1), (3, 1)])
+@pytest.mark.parametrize("override", [None, (0, 1), (1, 1), (2, 1), (3, 1), (20, 1), (21, 1), (22, 1), (23, 1)])
 def test_scale_indexing_is_bit_exact(device, override):
     # every product is a small integer and every scale a distinct power of two, so the FMA chain
     # is exact: any wrong (row, group) or (block, group) scale index changes the bits
