@@ -29,7 +29,7 @@ __global__ __launch_bounds__(WAVES * 64) void gqa_partition_kernel(
     const unsigned short *v_cache, float *part_o, float *part_m, float *part_l, int splits,
     int group)
 {
-    __shared__ float score[G][CHUNK];
+    __shared__ __attribute__((aligned(16))) float score[G][CHUNK];
     __shared__ float reduce[WAVES][G][DIM];
     const int split = blockIdx.x, kvh = blockIdx.y, b = blockIdx.z;
     const int thread = threadIdx.x, lane = thread % 64, wave = thread / 64;
@@ -84,9 +84,7 @@ __global__ __launch_bounds__(WAVES * 64) void gqa_partition_kernel(
             }
 #pragma unroll
             for (int h = 0; h < G; ++h)
-#pragma unroll
-                for (int offset = 8; offset; offset >>= 1)
-                    dot[h] += __shfl_xor(dot[h], offset, 64);
+                dot[h] = row16_sum(dot[h]);
             int position = p0 + u * 4 + sub;
             if (position < count) {
 #pragma unroll
@@ -132,16 +130,24 @@ __global__ __launch_bounds__(WAVES * 64) void gqa_partition_kernel(
             raw[u] = *reinterpret_cast<const unsigned *>(v_base + size_t(position) * row_stride +
                                                          lane * 2);
         }
+        // weights of four consecutive positions per head in one 128-bit LDS read; positions past
+        // the end of the partition contribute nothing
+        f32x4_t weight[G];
+#pragma unroll
+        for (int h = 0; h < G; ++h) {
+            weight[h] = *reinterpret_cast<const f32x4_t *>(&score[h][p0]);
+#pragma unroll
+            for (int u = 1; u < 4; ++u)
+                if (p0 + u >= count)
+                    weight[h][u] = 0.f;
+        }
 #pragma unroll
         for (int u = 0; u < 4; ++u) {
-            if (p0 + u < count) {
-                float lo = __uint_as_float(raw[u] << 16), hi = __uint_as_float(raw[u] & 0xffff0000u);
+            float lo = __uint_as_float(raw[u] << 16), hi = __uint_as_float(raw[u] & 0xffff0000u);
 #pragma unroll
-                for (int h = 0; h < G; ++h) {
-                    float weight = score[h][p0 + u];
-                    acc[h][0] = fmaf(weight, lo, acc[h][0]);
-                    acc[h][1] = fmaf(weight, hi, acc[h][1]);
-                }
+            for (int h = 0; h < G; ++h) {
+                acc[h][0] = fmaf(weight[h][u], lo, acc[h][0]);
+                acc[h][1] = fmaf(weight[h][u], hi, acc[h][1]);
             }
         }
     }

@@ -71,20 +71,52 @@ template <> struct storage<bf16_storage> {
     }
 };
 
+// Cross-lane moves inside the vector ALU (DPP), no LDS traffic. CONTROL: 0xB1 swaps neighbours
+// (lane ^ 1), 0x4E swaps pairs (lane ^ 2), 0x141 mirrors each group of 8, 0x140 mirrors each row of
+// 16 lanes.
+template <int CONTROL> __device__ __forceinline__ float dpp_move(float value)
+{
+    return __builtin_bit_cast(
+        float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, value), CONTROL, 0xf, 0xf, true));
+}
+
+// Sum over each aligned group of 16 lanes; every lane of the group receives the total. Fixed order:
+// neighbours, pairs, then the two mirrored halves.
+__device__ __forceinline__ float row16_sum(float value)
+{
+    value += dpp_move<0xB1>(value);
+    value += dpp_move<0x4E>(value);
+    value += dpp_move<0x141>(value);
+    value += dpp_move<0x140>(value);
+    return value;
+}
+
+__device__ __forceinline__ float row16_max(float value)
+{
+    value = fmaxf(value, dpp_move<0xB1>(value));
+    value = fmaxf(value, dpp_move<0x4E>(value));
+    value = fmaxf(value, dpp_move<0x141>(value));
+    value = fmaxf(value, dpp_move<0x140>(value));
+    return value;
+}
+
+__device__ __forceinline__ float lane_value(float value, int lane)
+{
+    return __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, value), lane));
+}
+
 // Sum across the 64 lanes of a wavefront in a fixed order; every lane receives the total.
 __device__ __forceinline__ float wave_sum(float value)
 {
-#pragma unroll
-    for (int offset = 32; offset; offset >>= 1)
-        value += __shfl_xor(value, offset, 64);
-    return value;
+    value = row16_sum(value);
+    return (lane_value(value, 0) + lane_value(value, 16)) +
+           (lane_value(value, 32) + lane_value(value, 48));
 }
 
 __device__ __forceinline__ float wave_max(float value)
 {
-#pragma unroll
-    for (int offset = 32; offset; offset >>= 1)
-        value = fmaxf(value, __shfl_xor(value, offset, 64));
-    return value;
+    value = row16_max(value);
+    return fmaxf(fmaxf(lane_value(value, 0), lane_value(value, 16)),
+                 fmaxf(lane_value(value, 32), lane_value(value, 48)));
 }
 } // namespace camblas_hip

@@ -146,7 +146,7 @@ Plan make_plan(int dtype, int algorithm, bool trans_a, bool trans_b, int m, int 
     plan.counter = 4;
     if (n <= 32) {
         plan.family = FAMILY_FP8_BLOCK;
-        plan.kernel = 1;
+        plan.kernel = 3; // 64 x 32 tiles, split-K: the most workgroups in flight for the weight stream
         const TnVariant &v = fp8_variant(plan.kernel);
         plan.split_k = decode_split(ceil_div(m, v.block_n), ceil_div(k, v.block_k), compute_units);
         return plan;

@@ -111,20 +111,21 @@ def test_sgemv_shortcut(device, rows, inner, pad):
     assert _native.stats(device)["classical"] >= 1
 
 
-def test_sgemv_exact_cancellation(device):
-    # ref: tests/test_float_gemv.py:69-90 style: sparse rows and exact cancellation
-    rows, inner = 1024, 4096
+def test_sgemv_exact_sparse_and_cancellation(device):
+    # ref: tests/test_float_gemv.py:69-90: one-hot rows select single inputs exactly, and
+    # 256 + 1 - 256 = 1 in full FP32 in any summation order
+    rows, inner = 1024, 8192
     w = np.zeros((rows, inner), np.float32)
-    x = np.ones(inner, np.float32)
-    w[0, 0], w[0, inner - 1] = 16777216.0, -16777216.0
-    w[0, 7] = 3.0
-    w[1, 100] = 2.5
-    w[rows - 1, inner - 1] = -4.0
+    w[np.arange(rows), np.arange(rows) * 7] = 1
+    x = np.arange(inner, dtype=np.float32)
     got = run_sgemm(device, "T", "N", rows, 1, inner, 1.0, w.ravel(), inner, x, inner, 0.0,
                     np.full(rows, np.nan, np.float32), rows)
-    want = np.zeros(rows, np.float32)
-    want[0], want[1], want[rows - 1] = 3.0, 2.5, -4.0
-    assert np.array_equal(got, want)
+    assert np.array_equal(got, x[np.arange(rows) * 7])
+    w[:] = 0
+    w[:, 0], w[:, 8], w[:, 16] = 256, 1, -256
+    got = run_sgemm(device, "T", "N", rows, 1, inner, 1.0, w.ravel(), inner,
+                    np.ones(inner, np.float32), inner, 0.0, np.full(rows, np.nan, np.float32), rows)
+    assert np.array_equal(got, np.ones(rows, np.float32))
 
 
 def test_invalid_arguments_report_errors(device):
