@@ -311,26 +311,38 @@ def gqa_decode_attention(q, k_cache, v_cache, lengths=None, scale=None):
     return out
 
 
-def decoder_layer_decode(hidden, residual, weights, k_cache, v_cache, positions, *, q_heads,
-                         kv_heads, head_dim=128, epsilon=1e-5, theta=500000.0):
+def kv_append(k_new, v_new, k_cache, v_cache, positions):
+    """Write the new token's K/V heads [B, Hkv, D] (views of a fused activation are fine) into the
+    caches [B, C, Hkv, D] at positions[B]."""
+    batch, kv_heads, dim = k_new.shape
+    _require(k_new.stride(2) == 1 and k_new.stride(1) == dim and v_new.stride(1) == dim
+             and k_new.stride(0) == v_new.stride(0), "new K/V heads must be dense rows of one stride")
+    _require(k_cache.is_contiguous() and v_cache.is_contiguous(), "caches must be contiguous")
+    _native.context(k_new.device).call(
+        "kv_append", batch, kv_heads, dim, k_cache.shape[1], _pointer(positions), _pointer(k_new),
+        _pointer(v_new), k_new.stride(0), _pointer(k_cache), _pointer(v_cache),
+    )
+
+
+def decoder_layer_decode(hidden, residual, weights, k_cache, v_cache, positions, lengths, *,
+                         q_heads, kv_heads, head_dim=128, epsilon=1e-5, theta=500000.0):
     """One Llama-shaped decoder layer for one new token per sequence.
 
     residual-add + RMSNorm -> fused QKV linear -> RoPE on q and k -> cache append -> GQA decode
     attention -> o-proj -> residual-add + RMSNorm -> SwiGLU MLP. Returns (mlp output, residual).
     `weights` holds input_norm, qkv [ (Hq+2Hkv)*D, hidden ], o, post_norm, gate, up, down.
-    `positions` (int32 [batch]) is the cache slot the new token is written to.
+    `positions` (int32 [batch]) is the cache slot the new token is written to and rotated for;
+    `lengths` (int32 [batch]) the number of valid cache positions afterwards (positions + 1).
+    Every step is a call into libcamblas_hip.so, so the whole function can be captured in a graph
+    after one warm-up call on the capture stream.
     """
     batch = hidden.shape[0]
     residual, normed = add_rms_norm(hidden, residual, weights["input_norm"], epsilon)
     qkv = linear(normed, weights["qkv"]).view(batch, q_heads + 2 * kv_heads, head_dim)
     rope(qkv[:, : q_heads + kv_heads], positions, theta)
-    q = qkv[:, :q_heads]
-    index = positions.long()
-    rows = torch.arange(batch, device=hidden.device)
-    k_cache[rows, index] = qkv[:, q_heads : q_heads + kv_heads]
-    v_cache[rows, index] = qkv[:, q_heads + kv_heads :]
-    lengths = (positions + 1).to(torch.int32)
-    attended = gqa_decode_attention(q, k_cache, v_cache, lengths)
+    kv_append(qkv[:, q_heads : q_heads + kv_heads], qkv[:, q_heads + kv_heads :], k_cache, v_cache,
+              positions)
+    attended = gqa_decode_attention(qkv[:, :q_heads], k_cache, v_cache, lengths)
     projected = linear(attended.view(batch, q_heads * head_dim), weights["o"])
     residual, normed = add_rms_norm(projected, residual, weights["post_norm"], epsilon)
     return gated_mlp(normed, weights["gate"], weights["up"], weights["down"]), residual

@@ -629,6 +629,27 @@ extern "C" int camblas_cuda_rope(camblas_cuda_context *context, int tokens, int 
     });
 }
 
+extern "C" int camblas_cuda_kv_append(camblas_cuda_context *context, int batch, int kv_heads, int dim,
+                                      int context_length, const int32_t *positions,
+                                      const void *k_new, const void *v_new, int token_stride,
+                                      void *k_cache, void *v_cache)
+{
+    return execute(context, [&] {
+        if (batch < 0 || kv_heads < 1 || dim < 8 || dim % 8 || context_length < 1 ||
+            token_stride < kv_heads * dim || token_stride % 8)
+            return fail(context, "invalid cache append arguments", 1);
+        if (!batch)
+            return 0;
+        if (!positions || !k_new || !v_new || !k_cache || !v_cache || !aligned(k_new, 16) ||
+            !aligned(v_new, 16) || !aligned(k_cache, 16) || !aligned(v_cache, 16) ||
+            k_cache == v_cache)
+            return fail(context, "invalid cache append buffers", 1);
+        hipError_t error = launch_kv_append(context->stream, batch, kv_heads, dim, context_length,
+                                            positions, k_new, v_new, token_stride, k_cache, v_cache);
+        return error == hipSuccess ? 0 : fail(context, "cache append", error);
+    });
+}
+
 extern "C" int camblas_cuda_gqa_decode_attention(camblas_cuda_context *context, int batch,
                                                  int q_heads, int kv_heads, int dim,
                                                  int context_length, const int32_t *lengths,

@@ -124,6 +124,9 @@ hipError_t launch_rms_rows(hipStream_t stream, int dtype, int weight_dtype, int 
 hipError_t launch_bf16_square(hipStream_t stream, uint64_t count, const void *input, float *out);
 hipError_t launch_rms_scale(hipStream_t stream, int dtype, uint64_t count, int width, float epsilon,
                             const void *input, const void *weight, const float *means, void *out);
+hipError_t launch_kv_append(hipStream_t stream, int batch, int kv_heads, int dim, int context_length,
+                            const int32_t *positions, const void *k_new, const void *v_new,
+                            int token_stride, void *k_cache, void *v_cache);
 hipError_t launch_copy_probe(hipStream_t stream, size_t bytes, const void *source, void *destination);
 hipError_t launch_rope(hipStream_t stream, int tokens, int heads, int dim, int token_stride,
                        float theta, const int32_t *positions, void *x);

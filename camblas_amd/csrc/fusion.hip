@@ -258,6 +258,28 @@ __global__ void copy_probe_kernel(size_t vectors, const u32x4_t *source, u32x4_t
         destination[index] = source[index];
 }
 
+// Writes the new token's K and V heads (taken from a fused QKV activation row) into the caches at
+// each sequence's position: 16 bytes per thread.
+__global__ void kv_append_kernel(int batch, int kv_heads, int dim, int context_length,
+                                 const int32_t *positions, const unsigned short *k_new,
+                                 const unsigned short *v_new, int token_stride,
+                                 unsigned short *k_cache, unsigned short *v_cache)
+{
+    const int vectors = kv_heads * dim / 8;
+    size_t index = size_t(blockIdx.x) * blockDim.x + threadIdx.x;
+    if (index >= size_t(batch) * vectors)
+        return;
+    const int b = int(index / vectors), v = int(index % vectors);
+    const int position = positions[b];
+    if (position < 0 || position >= context_length)
+        return;
+    const size_t target = ((size_t(b) * context_length + position) * kv_heads * dim) / 8 + v;
+    reinterpret_cast<u32x4_t *>(k_cache)[target] =
+        reinterpret_cast<const u32x4_t *>(k_new + size_t(b) * token_stride)[v];
+    reinterpret_cast<u32x4_t *>(v_cache)[target] =
+        reinterpret_cast<const u32x4_t *>(v_new + size_t(b) * token_stride)[v];
+}
+
 unsigned stride_blocks(uint64_t count)
 {
     uint64_t blocks = (count + 255) / 256;
@@ -360,6 +382,18 @@ hipError_t launch_rms_scale(hipStream_t stream, int dtype, uint64_t count, int w
         rms_scale_kernel<bf16_storage><<<stride_blocks(count), 256, 0, stream>>>(
             count, width, epsilon, static_cast<const bf16_storage *>(input),
             static_cast<const bf16_storage *>(weight), means, static_cast<bf16_storage *>(out));
+    return launch_status();
+}
+
+hipError_t launch_kv_append(hipStream_t stream, int batch, int kv_heads, int dim, int context_length,
+                            const int32_t *positions, const void *k_new, const void *v_new,
+                            int token_stride, void *k_cache, void *v_cache)
+{
+    size_t count = size_t(batch) * kv_heads * dim / 8;
+    kv_append_kernel<<<unsigned((count + 255) / 256), 256, 0, stream>>>(
+        batch, kv_heads, dim, context_length, positions, static_cast<const unsigned short *>(k_new),
+        static_cast<const unsigned short *>(v_new), token_stride,
+        static_cast<unsigned short *>(k_cache), static_cast<unsigned short *>(v_cache));
     return launch_status();
 }
 

@@ -162,6 +162,13 @@ int camblas_cuda_add_rms_norm_rows(camblas_cuda_context *context, int dtype, int
  * x [tokens, heads, dim] whose token stride is token_stride elements; positions int32 [tokens]. */
 int camblas_cuda_rope(camblas_cuda_context *context, int tokens, int heads, int dim,
                       int token_stride, float theta, const int32_t *positions, void *x_bf16);
+/* extension (no reference counterpart). Writes each sequence's new K and V heads, rows of k_new /
+ * v_new [batch, kv_heads*dim] with row stride token_stride elements (e.g. slices of a fused QKV
+ * activation), into the caches [batch, context, kv_heads, dim] at positions[batch]; positions
+ * outside [0, context) are skipped. dim % 8 == 0, 16-byte aligned buffers. */
+int camblas_cuda_kv_append(camblas_cuda_context *context, int batch, int kv_heads, int dim,
+                           int context_length, const int32_t *positions, const void *k_new,
+                           const void *v_new, int token_stride, void *k_cache, void *v_cache);
 /* extension. Grouped-query decode attention, one query per sequence: q [batch, q_heads, dim]
  * (token stride q_stride elements), K/V caches [batch, context, kv_heads, dim] BF16, lengths int32
  * [batch] or NULL (= context), out [batch, q_heads, dim] BF16. dim must be 128, q_heads a
