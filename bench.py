@@ -112,7 +112,8 @@ def main():
     parser.add_argument("--warmup", type=int, default=10)
     parser.add_argument("--skip-extras", action="store_true")
     parser.add_argument("--skip-cpu", action="store_true")
-    parser.add_argument("--only", choices=("decode1", "decode8", "decode32", "prefill", "copy"),
+    parser.add_argument("--only", choices=("decode1", "decode8", "decode32", "prefill", "copy", "fp8m1", "fp8m16",
+                                 "fp8m256", "fp8m4096", "attention", "layer"),
                         help="profiling aid: launch just this kernel --steps times, print nothing")
     args = parser.parse_args()
     if args.gpus != 1:
@@ -242,6 +243,21 @@ def profile_only(args, torch, _kernels, _native, device, normal, weights, inputs
         def launch(i):
             native.call("hip_copy_probe", size, ct.c_void_p(source.data_ptr()),
                         ct.c_void_p(target.data_ptr()))
+    elif args.only.startswith("fp8m"):
+        tokens, features, inner = int(args.only[4:]), 18432, 7168
+        w = torch.randint(0, 0x7E, (features, inner), device=device, dtype=torch.uint8)
+        w = w.view(torch.float8_e4m3fn)
+        w_scale = torch.rand((features // 128, inner // 128), device=device) * 0.1 + 1e-4
+        a = torch.randint(0, 0x7E, (tokens, inner), device=device, dtype=torch.uint8)
+        a = a.view(torch.float8_e4m3fn)
+        a_scale = torch.rand((tokens, inner // 128), device=device) * 0.1 + 1e-4
+        out = torch.empty((tokens, features), dtype=torch.bfloat16, device=device)
+
+        def launch(i):
+            _kernels.fp8_block_matmul(a, a_scale, w, w_scale, out=out)
+    elif args.only in ("attention", "layer"):
+        layer, attention = layer_step(torch, _kernels, device, normal)
+        launch = (lambda i: layer()) if args.only == "layer" else (lambda i: attention())
     else:
         tokens, features = 4096, 10240
         x, w = normal((tokens, INNER)), normal((features, INNER), 0.02)
@@ -252,6 +268,38 @@ def profile_only(args, torch, _kernels, _native, device, normal, weights, inputs
     for index in range(args.warmup + args.steps):
         launch(index)
     torch.cuda.synchronize()
+
+
+KV_BYTES = 2 * 32 * 2048 * 8 * 128 * 2
+LAYER_BYTES = 2 * (10240 * 8192 + 8192 * 8192 + 3 * 28672 * 8192) + KV_BYTES + 10e6
+
+
+def layer_step(torch, _kernels, device, normal):
+    """Llama-3.1-70B decoder-layer shapes at batch 32 and KV context 2048, random-init weights, all
+    positions at the last slot; returns closures running the whole step and the attention alone."""
+    batch, hidden, q_heads, kv_heads, dim, ffn, context = 32, 8192, 64, 8, 128, 28672, 2048
+    weights = {
+        "input_norm": normal((hidden,), 0.02) + 1, "post_norm": normal((hidden,), 0.02) + 1,
+        "qkv": normal(((q_heads + 2 * kv_heads) * dim, hidden), 0.02),
+        "o": normal((hidden, q_heads * dim), 0.02), "gate": normal((ffn, hidden), 0.02),
+        "up": normal((ffn, hidden), 0.02), "down": normal((hidden, ffn), 0.02),
+    }
+    k_cache = normal((batch, context, kv_heads, dim))
+    v_cache = normal((batch, context, kv_heads, dim))
+    hidden_in, residual = normal((batch, hidden)), normal((batch, hidden))
+    positions = torch.full((batch,), context - 1, dtype=torch.int32, device=device)
+    lengths = positions + 1
+    q = normal((batch, q_heads, dim))
+
+    def step():
+        return _kernels.decoder_layer_decode(
+            hidden_in, residual, weights, k_cache, v_cache, positions, lengths, q_heads=q_heads,
+            kv_heads=kv_heads, head_dim=dim)
+
+    def attention():
+        return _kernels.gqa_decode_attention(q, k_cache, v_cache, lengths)
+
+    return step, attention
 
 
 def extras(torch, _kernels, _native, device, normal):
@@ -306,23 +354,10 @@ def extras(torch, _kernels, _native, device, normal):
                                 "tflops": round(2.0 * size**3 / seconds / 1e12, 2),
                                 "frac_of_157TF": round(2.0 * size**3 / seconds / FP32_PEAK, 4)}
     # decoder-layer decode step (Llama-3.1-70B shapes, batch 32, KV context 2048)
-    batch, hidden, q_heads, kv_heads, dim, ffn, context = 32, 8192, 64, 8, 128, 28672, 2048
-    weights = {
-        "input_norm": normal((hidden,), 0.02) + 1, "post_norm": normal((hidden,), 0.02) + 1,
-        "qkv": normal(((q_heads + 2 * kv_heads) * dim, hidden), 0.02),
-        "o": normal((hidden, q_heads * dim), 0.02), "gate": normal((ffn, hidden), 0.02),
-        "up": normal((ffn, hidden), 0.02), "down": normal((hidden, ffn), 0.02),
-    }
-    k_cache = normal((batch, context, kv_heads, dim))
-    v_cache = normal((batch, context, kv_heads, dim))
-    hidden_in, residual = normal((batch, hidden)), normal((batch, hidden))
-    positions = torch.full((batch,), context - 1, dtype=torch.int32, device=device)
-    lengths = positions + 1
+    step, attention = layer_step(torch, _kernels, device, normal)
 
     def layer(i):
-        return _kernels.decoder_layer_decode(
-            hidden_in, residual, weights, k_cache, v_cache, positions, lengths, q_heads=q_heads,
-            kv_heads=kv_heads, head_dim=dim)
+        return step()
 
     eager = event_time(torch, layer, 3, 10)
     # the same step replayed from a captured graph (capture on a side stream after a warm-up there)
@@ -336,8 +371,12 @@ def extras(torch, _kernels, _native, device, normal):
     with torch.cuda.graph(graph, stream=side):
         layer(0)
     replayed = event_time(torch, lambda i: graph.replay(), 3, 20)
-    weight_bytes = sum(v.numel() * 2 for k, v in weights.items())
-    traffic = weight_bytes + 2 * k_cache.numel() * 2 + 10e6
+    traffic = LAYER_BYTES
+    seconds = event_time(torch, lambda i: attention(), 3, 20)
+    found["gqa_decode_attention_b32_ctx2048"] = {
+        "us": round(seconds * 1e6, 1), "gbps": round(KV_BYTES / seconds / 1e9, 1),
+        "frac_of_8TBs": round(KV_BYTES / seconds / HBM_PEAK, 4),
+    }
     found["llama70b_layer_decode_b32_ctx2048"] = {
         "eager_us": round(eager * 1e6, 1), "graph_us": round(replayed * 1e6, 1),
         "gbps": round(traffic / replayed / 1e9, 1),

@@ -691,7 +691,7 @@ extern "C" int camblas_hip_plan_describe(int dtype, int algorithm, char trans_a,
     Plan plan = make_plan(dtype, algorithm, is_t(trans_a), is_t(trans_b), m, n, k, lda, ldb, ldc,
                           aligned16 != 0, 256);
     describe_plan(plan, dtype, text, text_bytes);
-    return plan.family * 100 + plan.kernel;
+    return plan.family * 1000 + plan.kernel;
 }
 
 extern "C" int camblas_hip_set_plan_override(camblas_cuda_context *context, int kernel, int split_k)

@@ -2,14 +2,15 @@
 //
 // The whole cost is reading W once from HBM, so the kernel is organised around the weight stream:
 // one workgroup owns 16*NT consecutive weight rows for the whole K extent (about one workgroup per
-// compute unit for a Llama-sized projection) and marches along K in 128-element steps; all
-// workgroups advance roughly in lock step, which keeps the DRAM pages of one column block open
-// across the chip. Two K steps are in flight in registers per thread (128-bit loads, 256
-// contiguous bytes per row) while a third is multiplied, so a compute unit keeps ~2 * 16*NT * 256
-// bytes outstanding. Tiles are staged in LDS with a 16-way XOR swizzle (conflict-free 128-bit
-// stores and MFMA-layout reads). The four wavefronts split each K step four ways
-// (v_mfma_f32_16x16x32_bf16, FP32 accumulate) and their partial sums are combined in wavefront
-// order at the end, so results do not depend on scheduling. No split-K pass and no scratch.
+// compute unit for a Llama-sized projection) and marches along K in steps of KT 128-element
+// blocks. Two K steps are in flight in registers per thread (128-bit loads, 256 contiguous bytes
+// per row and block) while a third is multiplied, so a compute unit keeps 2 * 16*NT * KT * 256
+// bytes outstanding; KT grows as NT shrinks (projections with few output rows) so that this stays
+// near 64 KB, which is what it takes to cover the HBM latency at full bandwidth. Tiles are staged
+// in LDS with a 16-way XOR swizzle (conflict-free 128-bit stores and MFMA-layout reads). The four
+// wavefronts split each 128-element block four ways (v_mfma_f32_16x16x32_bf16, FP32 accumulate)
+// and their partial sums are combined in wavefront order at the end, so results do not depend on
+// scheduling. No split-K pass and no scratch.
 // Contract: ref src/cuda/bfloat16.cuh:11-57 for the ('T','N') call of a linear
 // (src/cuda/torch_bindings.cpp:146-199); the reference's own decode kernel class is
 // src/cuda/decode_float.cuh:2-52 (FP32, one vector).
@@ -30,20 +31,22 @@ struct StreamParams {
     int vector_store;
 };
 
-// NT, MT: 16-row weight tiles and 16-token tiles per workgroup; WAVES wavefronts split one K step
-// of 32*WAVES elements; DEPTH K steps are in flight in registers.
-template <int NT, int MT, int WAVES, int DEPTH>
+constexpr int WAVES = 4, DEPTH = 2;
+
+// NT, MT: 16-row weight tiles and 16-token tiles per workgroup; a K step is KT blocks of 32*WAVES
+// elements, each block split over the WAVES wavefronts; DEPTH K steps are in flight in registers.
+template <int NT, int MT, int KT>
 __global__ __launch_bounds__(WAVES * 64) void bgemv_stream_kernel(StreamParams p)
 {
     constexpr int ROWS = NT * 16, XROWS = MT * 16, CH = 4 * WAVES, BK = 32 * WAVES;
-    constexpr int STAGE_SLOTS = (ROWS + XROWS) * CH;
+    constexpr int BLOCK_SLOTS = (ROWS + XROWS) * CH, STAGE_SLOTS = BLOCK_SLOTS * KT;
     extern __shared__ __attribute__((aligned(16))) unsigned char lds_bytes[];
     u32x4_t *lds = reinterpret_cast<u32x4_t *>(lds_bytes);
 
     const int thread = threadIdx.x, lane = thread % 64, wave = thread / 64;
     const int chunk = thread % CH, pass_row = thread / CH; // CH lanes per row segment, 16 rows per pass
     const int n0 = blockIdx.x * ROWS, m0 = blockIdx.y * XROWS;
-    const int k_tiles = (p.k + BK - 1) / BK;
+    const int k_tiles = (p.k + BK * KT - 1) / (BK * KT);
 
     unsigned a_off[NT], b_off[MT];
 #pragma unroll
@@ -68,38 +71,45 @@ __global__ __launch_bounds__(WAVES * 64) void bgemv_stream_kernel(StreamParams p
     // compiler can count outstanding loads exactly and wait only for the older of the two tiles in
     // flight. A K position past the end (the K tail, or the padding tile of an odd tile count) is
     // read from the last valid chunk instead and zeroed by a mask when it is stored to LDS.
-    u32x4_t a_reg[DEPTH][NT], b_reg[DEPTH][MT];
+    u32x4_t a_reg[DEPTH][KT][NT], b_reg[DEPTH][KT][MT];
     // Workgroups start at different K tiles and wrap around: if all of them swept K in lock step
-    // the chip would read one 256-byte column block of every row at a time, a 16 KB-strided
-    // pattern that lands on few HBM channels; staggering spreads the requests over all of them.
+    // the chip would read one column block of every row at a time, a pattern strided by the row
+    // pitch that lands on few HBM channels; staggering spreads the requests over all of them.
     const int start = int(blockIdx.x % unsigned(k_tiles));
     auto rotated = [&](int step) {
         int tile = (step < k_tiles ? step : k_tiles - 1) + start;
         return tile < k_tiles ? tile : tile - k_tiles;
     };
-    auto fetch = [&](int step, u32x4_t(&a)[NT], u32x4_t(&b)[MT]) {
-        int k0 = rotated(step) * BK + chunk * 8;
-        k0 = k0 < p.k ? k0 : p.k - 8;
+    auto fetch = [&](int step, u32x4_t(&a)[KT][NT], u32x4_t(&b)[KT][MT]) {
         // padding steps past the end (their data is masked away) all read one cached line
         const unsigned live = step < k_tiles ? 0xffffffffu : 0u;
-        k0 &= int(live);
+        const int tile_k = rotated(step) * (BK * KT) + chunk * 8;
 #pragma unroll
-        for (int i = 0; i < NT; ++i)
-            a[i] = *reinterpret_cast<const u32x4_t *>(a_base + k0 + (a_off[i] & live));
+        for (int t = 0; t < KT; ++t) {
+            int k0 = tile_k + t * BK;
+            k0 = k0 < p.k ? k0 : p.k - 8;
+            k0 &= int(live);
 #pragma unroll
-        for (int j = 0; j < MT; ++j)
-            b[j] = *reinterpret_cast<const u32x4_t *>(b_base + k0 + (b_off[j] & live));
+            for (int i = 0; i < NT; ++i)
+                a[t][i] = *reinterpret_cast<const u32x4_t *>(a_base + k0 + (a_off[i] & live));
+#pragma unroll
+            for (int j = 0; j < MT; ++j)
+                b[t][j] = *reinterpret_cast<const u32x4_t *>(b_base + k0 + (b_off[j] & live));
+        }
     };
-    auto stash = [&](int stage, int step, const u32x4_t(&a)[NT], const u32x4_t(&b)[MT]) {
-        const unsigned mask =
-            step < k_tiles && rotated(step) * BK + chunk * 8 < p.k ? 0xffffffffu : 0u;
-        u32x4_t *base = lds + stage * STAGE_SLOTS + store_slot;
+    auto stash = [&](int stage, int step, const u32x4_t(&a)[KT][NT], const u32x4_t(&b)[KT][MT]) {
+        const int tile_k = rotated(step) * (BK * KT) + chunk * 8;
 #pragma unroll
-        for (int i = 0; i < NT; ++i)
-            base[i * 16 * CH] = a[i] & mask;
+        for (int t = 0; t < KT; ++t) {
+            const unsigned mask = step < k_tiles && tile_k + t * BK < p.k ? 0xffffffffu : 0u;
+            u32x4_t *base = lds + stage * STAGE_SLOTS + t * BLOCK_SLOTS + store_slot;
 #pragma unroll
-        for (int j = 0; j < MT; ++j)
-            base[(NT + j) * 16 * CH] = b[j] & mask;
+            for (int i = 0; i < NT; ++i)
+                base[i * 16 * CH] = a[t][i] & mask;
+#pragma unroll
+            for (int j = 0; j < MT; ++j)
+                base[(NT + j) * 16 * CH] = b[t][j] & mask;
+        }
     };
 
     // MFMA 16x16x32 operand positions: lane -> row lane%16, 8 K values at (wave*4 + lane/16)*8
@@ -112,18 +122,21 @@ __global__ __launch_bounds__(WAVES * 64) void bgemv_stream_kernel(StreamParams p
         for (int j = 0; j < MT; ++j)
             acc[i][j] = f32x4_t{0.f, 0.f, 0.f, 0.f};
     auto multiply = [&](int stage) {
-        const u32x4_t *base = lds + stage * STAGE_SLOTS + frag_slot;
-        bf16x8_t b_frag[MT];
 #pragma unroll
-        for (int j = 0; j < MT; ++j)
-            b_frag[j] = __builtin_bit_cast(bf16x8_t, base[(NT + j) * 16 * CH]);
-#pragma unroll
-        for (int i = 0; i < NT; ++i) {
-            bf16x8_t a_frag = __builtin_bit_cast(bf16x8_t, base[i * 16 * CH]);
+        for (int t = 0; t < KT; ++t) {
+            const u32x4_t *base = lds + stage * STAGE_SLOTS + t * BLOCK_SLOTS + frag_slot;
+            bf16x8_t b_frag[MT];
 #pragma unroll
             for (int j = 0; j < MT; ++j)
-                acc[i][j] =
-                    __builtin_amdgcn_mfma_f32_16x16x32_bf16(a_frag, b_frag[j], acc[i][j], 0, 0, 0);
+                b_frag[j] = __builtin_bit_cast(bf16x8_t, base[(NT + j) * 16 * CH]);
+#pragma unroll
+            for (int i = 0; i < NT; ++i) {
+                bf16x8_t a_frag = __builtin_bit_cast(bf16x8_t, base[i * 16 * CH]);
+#pragma unroll
+                for (int j = 0; j < MT; ++j)
+                    acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a_frag, b_frag[j],
+                                                                        acc[i][j], 0, 0, 0);
+            }
         }
     };
 
@@ -208,14 +221,15 @@ __global__ __launch_bounds__(WAVES * 64) void bgemv_stream_kernel(StreamParams p
     }
 }
 
-template <int NT, int MT, int WAVES, int DEPTH>
+template <int NT, int MT, int KT>
 hipError_t launch_one(hipStream_t stream, const StreamParams &p)
 {
-    constexpr size_t lds_bytes = size_t(2) * (NT + MT) * 16 * (64 * WAVES);
-    if constexpr (lds_bytes > 160 * 1024) {
+    constexpr size_t lds_bytes = size_t(2) * KT * (NT + MT) * 16 * (64 * WAVES);
+    // combined limits: the tiles in flight fit the register file, a stage pair fits the LDS
+    if constexpr (NT * KT > 8 || lds_bytes > 128 * 1024) {
         return hipErrorInvalidValue;
     } else {
-        auto kernel = bgemv_stream_kernel<NT, MT, WAVES, DEPTH>;
+        auto kernel = bgemv_stream_kernel<NT, MT, KT>;
         static bool configured[64] = {};
         int device = 0;
         hipError_t status = hipGetDevice(&device);
@@ -236,35 +250,35 @@ hipError_t launch_one(hipStream_t stream, const StreamParams &p)
     }
 }
 
-template <int MT, int WAVES, int DEPTH>
+template <int MT, int KT>
 hipError_t launch_rows(hipStream_t stream, int row_tiles, const StreamParams &p)
 {
     switch (row_tiles) {
-    case 1: return launch_one<1, MT, WAVES, DEPTH>(stream, p);
-    case 2: return launch_one<2, MT, WAVES, DEPTH>(stream, p);
-    case 3: return launch_one<3, MT, WAVES, DEPTH>(stream, p);
-    case 4: return launch_one<4, MT, WAVES, DEPTH>(stream, p);
-    case 5: return launch_one<5, MT, WAVES, DEPTH>(stream, p);
-    case 6: return launch_one<6, MT, WAVES, DEPTH>(stream, p);
-    case 7: return launch_one<7, MT, WAVES, DEPTH>(stream, p);
-    case 8: return launch_one<8, MT, WAVES, DEPTH>(stream, p);
+    case 1: return launch_one<1, MT, KT>(stream, p);
+    case 2: return launch_one<2, MT, KT>(stream, p);
+    case 3: return launch_one<3, MT, KT>(stream, p);
+    case 4: return launch_one<4, MT, KT>(stream, p);
+    case 5: return launch_one<5, MT, KT>(stream, p);
+    case 6: return launch_one<6, MT, KT>(stream, p);
+    case 7: return launch_one<7, MT, KT>(stream, p);
+    case 8: return launch_one<8, MT, KT>(stream, p);
     default: return hipErrorInvalidValue;
     }
 }
 
-template <int WAVES, int DEPTH>
+template <int KT>
 hipError_t launch_tokens(hipStream_t stream, int row_tiles, int token_tiles, const StreamParams &p)
 {
     switch (token_tiles) {
-    case 1: return launch_rows<1, WAVES, DEPTH>(stream, row_tiles, p);
-    case 2: return launch_rows<2, WAVES, DEPTH>(stream, row_tiles, p);
-    case 4: return launch_rows<4, WAVES, DEPTH>(stream, row_tiles, p);
+    case 1: return launch_rows<1, KT>(stream, row_tiles, p);
+    case 2: return launch_rows<2, KT>(stream, row_tiles, p);
+    case 4: return launch_rows<4, KT>(stream, row_tiles, p);
     default: return hipErrorInvalidValue;
     }
 }
 } // namespace
 
-hipError_t launch_bgemv_stream(hipStream_t stream, int mode, int row_tiles, int token_tiles, int n_out,
+hipError_t launch_bgemv_stream(hipStream_t stream, int depth_log2, int row_tiles, int token_tiles, int n_out,
                                int m_rows, int k, float alpha, const void *w, int lda,
                                const void *x, int ldb, float beta, void *y, int ldc)
 {
@@ -283,11 +297,11 @@ hipError_t launch_bgemv_stream(hipStream_t stream, int mode, int row_tiles, int 
     p.vector_store = (ldc % 4 == 0) && (reinterpret_cast<uintptr_t>(y) % 8 == 0);
     if ((m_rows + token_tiles * 16 - 1) / (token_tiles * 16) > 65535)
         return hipErrorInvalidValue;
-    switch (mode) {
-    case 0: return launch_tokens<4, 2>(stream, row_tiles, token_tiles, p);
-    case 1: return launch_tokens<4, 3>(stream, row_tiles, token_tiles, p);
-    case 2: return launch_tokens<8, 2>(stream, row_tiles, token_tiles, p);
-    case 3: return launch_tokens<8, 3>(stream, row_tiles, token_tiles, p);
+    switch (depth_log2) {
+    case 0: return launch_tokens<1>(stream, row_tiles, token_tiles, p);
+    case 1: return launch_tokens<2>(stream, row_tiles, token_tiles, p);
+    case 2: return launch_tokens<4>(stream, row_tiles, token_tiles, p);
+    case 3: return launch_tokens<8>(stream, row_tiles, token_tiles, p);
     default: return hipErrorInvalidValue;
     }
 }

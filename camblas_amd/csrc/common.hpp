@@ -52,7 +52,7 @@ enum KernelFamily {
 
 struct Plan {
     int family = FAMILY_GENERIC;
-    int kernel = 0;   // variant index inside the family (stream family: 100*mode + 10*row_tiles + token_tiles)
+    int kernel = 0;   // variant index inside the family (stream family: 100*log2(K blocks per step) + 10*row_tiles + token_tiles)
     int split_k = 1;  // number of K partitions (partials reduced in fixed order)
     int counter = 0;  // stats slot incremented at launch
 };
@@ -101,8 +101,9 @@ hipError_t launch_bgemm_dma(hipStream_t stream, int variant, int n_out, int m_ro
                             float alpha, const void *w, int lda, const void *x, int ldb, float beta,
                             void *y, int ldc);
 // Decode-shaped BF16 linear: each workgroup streams 16*row_tiles weight rows over the whole K.
-// mode: 0 = 4 wavefronts / 2 K steps in flight, 1 = 4 / 3, 2 = 8 / 2, 3 = 8 / 3.
-hipError_t launch_bgemv_stream(hipStream_t stream, int mode, int row_tiles, int token_tiles, int n_out,
+// depth_log2: a K step is 2^depth_log2 blocks of 128 elements (0..3); row_tiles << depth_log2 <= 8
+// and (row_tiles + token_tiles) << depth_log2 <= 16 or the launch is refused.
+hipError_t launch_bgemv_stream(hipStream_t stream, int depth_log2, int row_tiles, int token_tiles, int n_out,
                                int m_rows, int k, float alpha, const void *w, int lda,
                                const void *x, int ldb, float beta, void *y, int ldc);
 hipError_t launch_fp8_block(hipStream_t stream, int variant, int split_k, int rows, int outputs,

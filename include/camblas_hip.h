@@ -182,7 +182,7 @@ int camblas_cuda_gqa_decode_attention(camblas_cuda_context *context, int batch, 
 
 /* extension. Planner introspection (the GPU counterpart of the reference CPU planner's
  * camblas_plan_format, src/planner.c:654-669): writes a one-line description of the kernel the
- * planner picks for a GEMM call into `text` and returns the kernel id (>=0) without touching a
+ * planner picks for a GEMM call into `text` and returns 1000 * family + variant (>=0) without touching a
  * device. dtype 0 FP32, 2 BF16, 3 FP8-block. Pure host function: works without a GPU. */
 int camblas_hip_plan_describe(int dtype, int algorithm, char trans_a, char trans_b, int m, int n,
                               int k, int lda, int ldb, int ldc, int aligned16, char *text,

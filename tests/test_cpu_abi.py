@@ -61,23 +61,23 @@ def test_planner_choices_for_the_baseline_shapes():
     describe = _native.plan_describe
     # decode linears: weight-streaming kernel, one workgroup per compute unit for the up-projection
     code, text = describe(2, "T", "N", 28672, 32, 8192, 8192, 8192, 28672)
-    assert code // 100 == 4 and "stream rows=112 tokens=32" in text
+    assert code // 1000 == 4 and "stream rows=112 tokens=32" in text
     assert "tokens=16" in describe(2, "T", "N", 28672, 1, 8192, 8192, 8192, 28672)[1]
     assert "rows=32" in describe(2, "T", "N", 8192, 32, 28672, 28672, 28672, 8192)[1]
     # prefill: direct-to-LDS MFMA tile that divides 10240 x 4096 into exactly two waves of tiles
     code, text = describe(2, "T", "N", 10240, 4096, 8192, 8192, 8192, 10240)
-    assert code // 100 == 5 and "dma320x256" in text
+    assert code // 1000 == 5 and "dma320x256" in text
     # K not a multiple of 64: register-staged MFMA tiles; unaligned or other layouts: generic
-    assert describe(2, "T", "N", 10240, 4096, 8200, 8200, 8200, 10240)[0] // 100 == 2
-    assert describe(2, "T", "N", 1024, 64, 1001, 1001, 1001, 1024)[0] // 100 == 0
-    assert describe(2, "N", "N", 1024, 64, 1024, 1024, 1024, 1024)[0] // 100 == 0
-    assert describe(2, "T", "N", 1024, 64, 1024, 1024, 1024, 1024, aligned16=False)[0] // 100 == 0
-    assert describe(2, "T", "N", 1024, 64, 1024, 1024, 1024, 1024, algorithm="classical")[0] // 100 == 0
+    assert describe(2, "T", "N", 10240, 4096, 8200, 8200, 8200, 10240)[0] // 1000 == 2
+    assert describe(2, "T", "N", 1024, 64, 1001, 1001, 1001, 1024)[0] // 1000 == 0
+    assert describe(2, "N", "N", 1024, 64, 1024, 1024, 1024, 1024)[0] // 1000 == 0
+    assert describe(2, "T", "N", 1024, 64, 1024, 1024, 1024, 1024, aligned16=False)[0] // 1000 == 0
+    assert describe(2, "T", "N", 1024, 64, 1024, 1024, 1024, 1024, algorithm="classical")[0] // 1000 == 0
     # FP32: single-vector shortcut only under auto (ref: src/cuda/backend.cu:810-815)
-    assert describe(0, "T", "N", 4096, 1, 4096, 4096, 4096, 4096)[0] // 100 == 1
-    assert describe(0, "T", "N", 4096, 1, 4096, 4096, 4096, 4096, algorithm="lt")[0] // 100 == 0
-    assert describe(0, "T", "N", 1000, 1, 4096, 4096, 4096, 1000)[0] // 100 == 0
-    assert describe(0, "N", "N", 2048, 2048, 2048, 2048, 2048, 2048)[0] // 100 == 0
+    assert describe(0, "T", "N", 4096, 1, 4096, 4096, 4096, 4096)[0] // 1000 == 1
+    assert describe(0, "T", "N", 4096, 1, 4096, 4096, 4096, 4096, algorithm="lt")[0] // 1000 == 0
+    assert describe(0, "T", "N", 1000, 1, 4096, 4096, 4096, 1000)[0] // 1000 == 0
+    assert describe(0, "N", "N", 2048, 2048, 2048, 2048, 2048, 2048)[0] // 1000 == 0
     # the plan is a pure function of its arguments
     assert describe(3, "T", "N", 18432, 16, 7168, 7168, 7168, 18432) == describe(
         3, "T", "N", 18432, 16, 7168, 7168, 7168, 18432)

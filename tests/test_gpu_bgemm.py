@@ -71,12 +71,12 @@ def test_tn_every_variant(device, variant, split, n_out, pad):
         assert np.array_equal(got2d[:, n_out:], c0.reshape(m_rows, ldc)[:, n_out:])
 
 
-# 100 + 100*mode + 10*row_tiles + token_tiles; modes 2 and 3 (eight wavefronts) need
-# row_tiles + token_tiles <= 10 to fit the LDS
-STREAM_CODES = [100 + 10 * rows + tokens for rows in range(1, 9) for tokens in (1, 2, 4)] + [
-    100 + 100 * mode + 10 * rows + tokens
-    for mode in (1, 2, 3) for rows in (1, 4, 7, 8) for tokens in (1, 2, 4)
-    if mode == 1 or rows + tokens <= 10
+# 100 + 100*log2(K blocks per step) + 10*row_tiles + token_tiles; the blocks are limited by
+# row_tiles * blocks <= 8 and (row_tiles + token_tiles) * blocks <= 16
+STREAM_CODES = [
+    100 + 100 * depth + 10 * rows + tokens
+    for depth in (0, 1, 2, 3) for rows in range(1, 9) for tokens in (1, 2, 4)
+    if (rows << depth) <= 8 and ((rows + tokens) << depth) <= 16
 ]
 
 
