@@ -5,14 +5,21 @@
 // arithmetic is the textbook softmax(scale * q k^T) v with FP32 accumulation and an online-softmax
 // merge of the context partitions.
 //
-// Partition kernel, one workgroup per (partition, kv head, sequence), 4 wavefronts:
-//   1. scores: 16 lanes share one cache row (16-byte loads, 256 contiguous bytes per row), every
-//      lane multiplies its 8 dims with all query heads of the group, 4 butterfly steps finish the
-//      dot products; scores go to LDS.
-//   2. per-head maximum and exponentials in LDS (one wavefront per head).
-//   3. values: a lane owns two output dims, wavefronts stride over positions, the four wavefront
-//      partial sums are added in index order.
-// The kernel is bound by the cache read (2 * context * 256 bytes per kv head and sequence).
+// Partition kernel, one workgroup per (256 positions, kv head, sequence); each of its 4 wavefronts
+// owns 64 positions and runs both products on the matrix cores (v_mfma_f32_16x16x32_bf16), with the
+// query heads of the group padded to 16:
+//   scores  S[position, head] = K[position, :] . Q[head, :]    A = K rows (16-byte loads), B = Q
+//   output  O[head, dim]      = P[head, position] . V[position, dim]
+// The score tile leaves the first product with lane l holding head l%16 and four positions, which
+// is already the A-operand layout of the second product once the K index of that product is
+// *defined* as the position order the lane holds; V has to follow the same order. V is read with
+// 16-byte loads (a lane takes dims 8m..8m+7 of its eight positions, 16 lanes cover one 256-byte
+// row) and transposed in registers with byte permutes into eight B operands, one per dim offset
+// w, so that output column m of product w is dim 8m + w.
+// All K, V and Q loads of a wavefront are issued before the first product, which keeps about
+// 32 KB per wavefront in flight. The wavefronts' partial (max, sum, O) are merged through LDS in
+// wavefront order. The kernel is bound by the cache read (2 * context * 256 bytes per kv head
+// and sequence).
 #include "common.hpp"
 #include "device.hpp"
 
@@ -20,150 +27,158 @@ namespace camblas_hip
 {
 namespace
 {
-constexpr int DIM = 128, CHUNK = 256, WAVES = 4;
+constexpr int DIM = 128, CHUNK = 256, WAVES = 4, WAVE_POSITIONS = CHUNK / WAVES, HEADS = 16;
 
-template <int G>
+__device__ __forceinline__ float swap_lanes(float value, int mask)
+{
+    return __shfl_xor(value, mask, 64);
+}
+
 __global__ __launch_bounds__(WAVES * 64) void gqa_partition_kernel(
     int q_heads, int kv_heads, int context_length, const int32_t *lengths, float scale,
     const unsigned short *q, int q_stride, const unsigned short *k_cache,
     const unsigned short *v_cache, float *part_o, float *part_m, float *part_l, int splits,
     int group)
 {
-    __shared__ __attribute__((aligned(16))) float score[G][CHUNK];
-    __shared__ float reduce[WAVES][G][DIM];
+    __shared__ __attribute__((aligned(16))) float wave_o[WAVES][HEADS][DIM];
+    __shared__ float wave_m[WAVES][HEADS], wave_l[WAVES][HEADS];
     const int split = blockIdx.x, kvh = blockIdx.y, b = blockIdx.z;
     const int thread = threadIdx.x, lane = thread % 64, wave = thread / 64;
+    const int m = lane % 16, j = lane / 16;
     const int length = lengths ? min(max(lengths[b], 0), context_length) : context_length;
-    const int begin = split * CHUNK;
-    const int count = min(CHUNK, length - begin); // may be <= 0: empty partition
+    const int begin = split * CHUNK + wave * WAVE_POSITIONS;
+    const int count = min(WAVE_POSITIONS, length - begin); // may be <= 0: nothing for this wave
     const size_t row_stride = size_t(kv_heads) * DIM;
     const unsigned short *k_base =
         k_cache + (size_t(b) * context_length + begin) * row_stride + size_t(kvh) * DIM;
     const unsigned short *v_base =
         v_cache + (size_t(b) * context_length + begin) * row_stride + size_t(kvh) * DIM;
 
-    // ---- 1. scores
-    const int part = lane % 16, sub = lane / 16;
-    float qv[G][8];
+    f32x4_t acc[8];
 #pragma unroll
-    for (int h = 0; h < G; ++h) {
-        int head = kvh * group + (h < group ? h : group - 1);
-        u32x4_t raw = *reinterpret_cast<const u32x4_t *>(q + size_t(b) * q_stride +
-                                                         size_t(head) * DIM + part * 8);
+    for (int w = 0; w < 8; ++w)
+        acc[w] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+    float top = -INFINITY, total = 0.f;
+    if (count > 0) { // uniform over the wavefront
+        // ---- loads: Q (head m, dims 32s + 8j ..), K (position 16t + m, same dims),
+        // V (position 32u + 16(e/4) + 4j + e%4, dims 8m ..); rows past the end repeat the last one
+        const int head = kvh * group + (m < group ? m : group - 1);
+        const unsigned short *q_row = q + size_t(b) * q_stride + size_t(head) * DIM + 8 * j;
+        bf16x8_t q_frag[4], k_frag[4][4];
+        u32x4_t v_rows[2][8];
 #pragma unroll
-        for (int e = 0; e < 4; ++e) {
-            qv[h][2 * e] = __uint_as_float(raw[e] << 16) * scale;
-            qv[h][2 * e + 1] = __uint_as_float(raw[e] & 0xffff0000u) * scale;
-        }
-    }
-    for (int p0 = wave * 16; p0 < count; p0 += WAVES * 16) {
-        u32x4_t rows[4];
+        for (int s = 0; s < 4; ++s)
+            q_frag[s] = *reinterpret_cast<const bf16x8_t *>(q_row + 32 * s);
 #pragma unroll
-        for (int u = 0; u < 4; ++u) {
-            int position = p0 + u * 4 + sub;
+        for (int t = 0; t < 4; ++t) {
+            int position = 16 * t + m;
             position = position < count ? position : count - 1;
-            rows[u] = *reinterpret_cast<const u32x4_t *>(k_base + size_t(position) * row_stride +
-                                                         part * 8);
+            const unsigned short *row = k_base + size_t(position) * row_stride + 8 * j;
+#pragma unroll
+            for (int s = 0; s < 4; ++s)
+                k_frag[t][s] = *reinterpret_cast<const bf16x8_t *>(row + 32 * s);
         }
 #pragma unroll
-        for (int u = 0; u < 4; ++u) {
-            float kv[8];
+        for (int u = 0; u < 2; ++u)
 #pragma unroll
-            for (int e = 0; e < 4; ++e) {
-                kv[2 * e] = __uint_as_float(rows[u][e] << 16);
-                kv[2 * e + 1] = __uint_as_float(rows[u][e] & 0xffff0000u);
+            for (int e = 0; e < 8; ++e) {
+                int position = 32 * u + 16 * (e / 4) + 4 * j + e % 4;
+                position = position < count ? position : count - 1;
+                v_rows[u][e] =
+                    *reinterpret_cast<const u32x4_t *>(v_base + size_t(position) * row_stride + 8 * m);
             }
-            float dot[G];
-#pragma unroll
-            for (int h = 0; h < G; ++h) {
-                float sum = 0.f;
-#pragma unroll
-                for (int e = 0; e < 8; ++e)
-                    sum = fmaf(qv[h][e], kv[e], sum);
-                dot[h] = sum;
-            }
-#pragma unroll
-            for (int h = 0; h < G; ++h)
-                dot[h] = row16_sum(dot[h]);
-            int position = p0 + u * 4 + sub;
-            if (position < count) {
-#pragma unroll
-                for (int h = 0; h < G; ++h)
-                    if (part == h % 16)
-                        score[h][position] = dot[h];
-            }
-        }
-    }
-    __syncthreads();
 
-    // ---- 2. per-head maximum, exponentials, sum (wavefront w owns heads w, w+4, ...)
-    for (int h = wave; h < G; h += WAVES) {
-        float top = -INFINITY;
-        for (int position = lane; position < count; position += 64)
-            top = fmaxf(top, score[h][position]);
-        top = wave_max(top);
-        float total = 0.f;
-        for (int position = lane; position < count; position += 64) {
-            float e = __expf(score[h][position] - top);
-            score[h][position] = e;
-            total += e;
+        // ---- scores: register r of tile t is position 16t + 4j + r, head m
+        f32x4_t score[4];
+#pragma unroll
+        for (int t = 0; t < 4; ++t) {
+            score[t] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+            for (int s = 0; s < 4; ++s)
+                score[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(k_frag[t][s], q_frag[s], score[t],
+                                                                   0, 0, 0);
         }
-        total = wave_sum(total);
-        if (lane == 0 && h < group) {
-            size_t index = (size_t(b) * q_heads + kvh * group + h) * splits + split;
-            part_m[index] = top;
-            part_l[index] = total;
-        }
-    }
-    __syncthreads();
+#pragma unroll
+        for (int t = 0; t < 4; ++t)
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+                float value = 16 * t + 4 * j + r < count ? score[t][r] * scale : -INFINITY;
+                score[t][r] = value;
+                top = fmaxf(top, value);
+            }
+        // the four lanes m, m+16, m+32, m+48 share a head; position 0 is always valid, so the
+        // maximum is finite
+        top = fmaxf(top, swap_lanes(top, 16));
+        top = fmaxf(top, swap_lanes(top, 32));
+#pragma unroll
+        for (int t = 0; t < 4; ++t)
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+                float e = __expf(score[t][r] - top);
+                score[t][r] = e;
+                total += e;
+            }
+        total += swap_lanes(total, 16);
+        total += swap_lanes(total, 32);
 
-    // ---- 3. values: lane owns dims 2*lane, 2*lane+1
-    float acc[G][2];
+        // ---- output: K index 8j + e of product u is position 32u + 16(e/4) + 4j + e%4
 #pragma unroll
-    for (int h = 0; h < G; ++h)
-        acc[h][0] = acc[h][1] = 0.f;
-    for (int p0 = wave * 4; p0 < count; p0 += WAVES * 4) {
-        unsigned raw[4];
+        for (int u = 0; u < 2; ++u) {
+            u32x4_t weights = {pack_bf16x2(score[2 * u][0], score[2 * u][1]),
+                               pack_bf16x2(score[2 * u][2], score[2 * u][3]),
+                               pack_bf16x2(score[2 * u + 1][0], score[2 * u + 1][1]),
+                               pack_bf16x2(score[2 * u + 1][2], score[2 * u + 1][3])};
+            bf16x8_t p_frag = __builtin_bit_cast(bf16x8_t, weights);
 #pragma unroll
-        for (int u = 0; u < 4; ++u) {
-            int position = p0 + u < count ? p0 + u : count - 1;
-            raw[u] = *reinterpret_cast<const unsigned *>(v_base + size_t(position) * row_stride +
-                                                         lane * 2);
-        }
-        // weights of four consecutive positions per head in one 128-bit LDS read; positions past
-        // the end of the partition contribute nothing
-        f32x4_t weight[G];
+            for (int pair = 0; pair < 4; ++pair) {
+                u32x4_t even, odd; // dims 8m + 2 pair and 8m + 2 pair + 1 of the eight positions
 #pragma unroll
-        for (int h = 0; h < G; ++h) {
-            weight[h] = *reinterpret_cast<const f32x4_t *>(&score[h][p0]);
-#pragma unroll
-            for (int u = 1; u < 4; ++u)
-                if (p0 + u >= count)
-                    weight[h][u] = 0.f;
-        }
-#pragma unroll
-        for (int u = 0; u < 4; ++u) {
-            float lo = __uint_as_float(raw[u] << 16), hi = __uint_as_float(raw[u] & 0xffff0000u);
-#pragma unroll
-            for (int h = 0; h < G; ++h) {
-                acc[h][0] = fmaf(weight[h][u], lo, acc[h][0]);
-                acc[h][1] = fmaf(weight[h][u], hi, acc[h][1]);
+                for (int c = 0; c < 4; ++c) {
+                    unsigned lo = v_rows[u][2 * c][pair], hi = v_rows[u][2 * c + 1][pair];
+                    even[c] = __builtin_amdgcn_perm(hi, lo, 0x05040100u);
+                    odd[c] = __builtin_amdgcn_perm(hi, lo, 0x07060302u);
+                }
+                acc[2 * pair] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(
+                    p_frag, __builtin_bit_cast(bf16x8_t, even), acc[2 * pair], 0, 0, 0);
+                acc[2 * pair + 1] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(
+                    p_frag, __builtin_bit_cast(bf16x8_t, odd), acc[2 * pair + 1], 0, 0, 0);
             }
         }
     }
+
+    // ---- merge the wavefronts: register r of acc[w] is head 4j + r, dim 8m + w
+    if (j == 0) {
+        wave_m[wave][m] = top;
+        wave_l[wave][m] = total;
+    }
 #pragma unroll
-    for (int h = 0; h < G; ++h) {
-        reduce[wave][h][lane * 2] = acc[h][0];
-        reduce[wave][h][lane * 2 + 1] = acc[h][1];
+    for (int r = 0; r < 4; ++r) {
+        float *row = &wave_o[wave][4 * j + r][8 * m];
+        *reinterpret_cast<f32x4_t *>(row) = f32x4_t{acc[0][r], acc[1][r], acc[2][r], acc[3][r]};
+        *reinterpret_cast<f32x4_t *>(row + 4) = f32x4_t{acc[4][r], acc[5][r], acc[6][r], acc[7][r]};
     }
     __syncthreads();
     for (int index = thread; index < group * DIM; index += WAVES * 64) {
-        int h = index / DIM, d = index % DIM;
-        float sum = reduce[0][h][d];
+        const int h = index / DIM, d = index % DIM;
+        float best = wave_m[0][h];
 #pragma unroll
         for (int w = 1; w < WAVES; ++w)
-            sum += reduce[w][h][d];
-        part_o[((size_t(b) * q_heads + kvh * group + h) * splits + split) * DIM + d] = sum;
+            best = fmaxf(best, wave_m[w][h]);
+        float numerator = 0.f, denominator = 0.f;
+        if (best > -INFINITY) {
+#pragma unroll
+            for (int w = 0; w < WAVES; ++w) {
+                float factor = __expf(wave_m[w][h] - best); // 0 for a wavefront without positions
+                numerator = fmaf(factor, wave_o[w][h][d], numerator);
+                denominator = fmaf(factor, wave_l[w][h], denominator);
+            }
+        }
+        const size_t row = (size_t(b) * q_heads + kvh * group + h) * splits + split;
+        part_o[row * DIM + d] = numerator;
+        if (d == 0) {
+            part_m[row] = best;
+            part_l[row] = denominator;
+        }
     }
 }
 
@@ -205,9 +220,10 @@ hipError_t launch_gqa_decode(hipStream_t stream, int batch, int q_heads, int kv_
                              int q_stride, const void *k, const void *v, void *out, void *scratch,
                              int splits)
 {
-    if (dim != DIM || splits > 65535 || kv_heads > 65535 || batch > 65535)
+    const int group = kv_heads > 0 ? q_heads / kv_heads : 0;
+    if (dim != DIM || splits > 65535 || kv_heads > 65535 || batch > 65535 || group < 1 ||
+        group > HEADS)
         return hipErrorInvalidValue;
-    const int group = q_heads / kv_heads;
     size_t rows = size_t(batch) * q_heads * splits;
     float *part_o = static_cast<float *>(scratch);
     float *part_m = part_o + rows * DIM;
@@ -216,21 +232,9 @@ hipError_t launch_gqa_decode(hipStream_t stream, int batch, int q_heads, int kv_
     const unsigned short *qp = static_cast<const unsigned short *>(q);
     const unsigned short *kp = static_cast<const unsigned short *>(k);
     const unsigned short *vp = static_cast<const unsigned short *>(v);
-#define CAMBLAS_LAUNCH_GQA(G)                                                                      \
-    gqa_partition_kernel<G><<<grid, WAVES * 64, 0, stream>>>(                                      \
-        q_heads, kv_heads, context_length, lengths, scale, qp, q_stride, kp, vp, part_o, part_m,   \
-        part_l, splits, group)
-    if (group <= 1)
-        CAMBLAS_LAUNCH_GQA(1);
-    else if (group <= 2)
-        CAMBLAS_LAUNCH_GQA(2);
-    else if (group <= 4)
-        CAMBLAS_LAUNCH_GQA(4);
-    else if (group <= 8)
-        CAMBLAS_LAUNCH_GQA(8);
-    else
-        CAMBLAS_LAUNCH_GQA(16);
-#undef CAMBLAS_LAUNCH_GQA
+    gqa_partition_kernel<<<grid, WAVES * 64, 0, stream>>>(q_heads, kv_heads, context_length, lengths,
+                                                          scale, qp, q_stride, kp, vp, part_o, part_m,
+                                                          part_l, splits, group);
     hipError_t status = launch_status();
     if (status != hipSuccess)
         return status;

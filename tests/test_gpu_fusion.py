@@ -136,7 +136,8 @@ def test_rope(device):
 
 
 @pytest.mark.parametrize("batch,q_heads,kv_heads,context", [(3, 16, 2, 700), (2, 8, 8, 256),
-                                                            (2, 12, 4, 300), (1, 64, 8, 2048)])
+                                                            (2, 12, 4, 300), (1, 64, 8, 2048),
+                                                            (3, 32, 2, 520), (2, 5, 5, 65)])
 def test_gqa_decode_attention(device, batch, q_heads, kv_heads, context):
     dim = 128
     q = oracle.fill_normal_bf16(30, (batch, q_heads, dim))
@@ -160,3 +161,20 @@ def test_gqa_decode_attention(device, batch, q_heads, kv_heads, context):
                                          to_device_bf16(v, device), None, scale)
     want_full = oracle.gqa_decode(q, k, v, None, scale)
     assert rel_frobenius(bf16_values(full), oracle.bf16_to_f32(want_full)) <= 1e-2
+
+
+def test_gqa_decode_attention_empty_and_partial_partitions(device):
+    # lengths 0 (no position: zeros), 64 and 65 (wavefront boundary), 256 and 259 (partition boundary)
+    batch, q_heads, kv_heads, context, dim = 5, 16, 2, 600, 128
+    q = oracle.fill_normal_bf16(40, (batch, q_heads, dim))
+    k = oracle.fill_normal_bf16(41, (batch, context, kv_heads, dim))
+    v = oracle.fill_normal_bf16(42, (batch, context, kv_heads, dim))
+    lengths = np.array([0, 64, 65, 256, 259], np.int32)
+    out = _kernels.gqa_decode_attention(to_device_bf16(q, device), to_device_bf16(k, device),
+                                        to_device_bf16(v, device),
+                                        torch.from_numpy(lengths).to(device), dim**-0.5)
+    want = oracle.gqa_decode(q, k, v, np.maximum(lengths, 1), dim**-0.5)
+    got = from_device_bf16(out)
+    assert not got[0].any()
+    wanted = oracle.bf16_to_f32(want)[1:]
+    assert (np.abs(bf16_values(out)[1:] - wanted) <= 0.01 * np.abs(wanted) + 2e-3).all()
