@@ -19,7 +19,7 @@ def _autoload():
     module = tensor_module()
     if module is None or not hasattr(module, "install_torch_backend"):
         raise RuntimeError(
-            "Build the tensor binding with `python -m camblas_amd._build --torch` first"
+            "Build the tensor binding with `python camblas_amd/_build.py` first"
         )
     name = os.environ.get(
         "CAMBLAS_CUDA_ALGORITHM", os.environ.get("CAMBLAS_SGLANG_ALGORITHM", "lt")

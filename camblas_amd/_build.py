@@ -89,5 +89,35 @@ def build_core(jobs=8, verbose=False):
     return CORE
 
 
+def build_tensor_binding():
+    """Compile csrc/tensor_binding.cpp (host code only: ATen + pybind11 + the C ABI) into
+    lib/_camblas_cuda_torch<ext>.so, linked against libcamblas_hip.so beside it."""
+    import sysconfig
+
+    import torch
+    from torch.utils import cpp_extension
+
+    torch_lib = Path(torch.__file__).resolve().parent / "lib"
+    suffix = sysconfig.get_config_var("EXT_SUFFIX") or ".so"
+    target = LIB_DIR / ("_camblas_cuda_torch" + suffix)
+    includes = [f"-I{path}" for path in cpp_extension.include_paths()]
+    includes += [f"-I{sysconfig.get_paths()['include']}", "-I/opt/rocm/include",
+                 f"-I{ROOT / 'include'}"]
+    abi = int(torch._C._GLIBCXX_USE_CXX11_ABI)
+    command = [
+        os.environ.get("CXX", "g++"), "-O2", "-std=c++17", "-fPIC", "-shared", "-Wall",
+        "-Wno-unused-function", "-Wno-deprecated-declarations", "-D__HIP_PLATFORM_AMD__=1",
+        "-DUSE_ROCM=1", f"-D_GLIBCXX_USE_CXX11_ABI={abi}", "-DTORCH_API_INCLUDE_EXTENSION_H",
+        "-DTORCH_EXTENSION_NAME=_camblas_cuda_torch", *includes, CSRC / "tensor_binding.cpp",
+        "-o", target, f"-L{LIB_DIR}", "-lcamblas_hip", f"-L{torch_lib}", "-ltorch_python",
+        "-ltorch", "-ltorch_cpu", "-ltorch_hip", "-lc10", "-lc10_hip", "-L/opt/rocm/lib",
+        "-lamdhip64", "-Wl,-rpath,$ORIGIN", f"-Wl,-rpath,{torch_lib}",
+    ]
+    _run(command)
+    return target
+
+
 if __name__ == "__main__":
     print(build_core(verbose=True))
+    if "--no-binding" not in sys.argv:
+        print(build_tensor_binding())

@@ -222,9 +222,19 @@ extern "C" int camblas_cuda_dgemm(camblas_cuda_context *context, char ta, char t
                                   int k, double alpha, const double *a, int lda, const double *b,
                                   int ldb, double beta, double *c, int ldc)
 {
-    (void)ta, (void)tb, (void)m, (void)n, (void)k, (void)alpha, (void)a, (void)lda, (void)b;
-    (void)ldb, (void)beta, (void)c, (void)ldc;
-    return unsupported(context, "FP64 GEMM");
+    // ref: src/cuda/backend.cu:1066-1073; FP64 has no matrix-core path here, every layout runs the
+    // LDS-tiled FMA kernel
+    return execute(context, [&] {
+        return gemm<double>(
+            context, "FP64", ta, tb, m, n, k, alpha, a, lda, b, ldb, beta, c, ldc,
+            [&] { return launch_scale_f64(context->stream, m, n, beta, c, ldc); },
+            [&](bool trans_a, bool trans_b) {
+                context->counts[0]++;
+                hipError_t error = launch_generic_f64(context->stream, trans_a, trans_b, m, n, k,
+                                                      alpha, a, lda, b, ldb, beta, c, ldc);
+                return error == hipSuccess ? 0 : fail(context, "classical FP64 GEMM", error);
+            });
+    });
 }
 
 extern "C" int camblas_cuda_bgemm(camblas_cuda_context *context, char trans_a, char trans_b, int m,

@@ -79,6 +79,7 @@ const TnVariant &fp8_variant(int index);
 // ---------------------------------------------------------------- launchers (each returns a hipError_t)
 hipError_t launch_scale_f32(hipStream_t stream, int m, int n, float beta, float *c, int ldc);
 hipError_t launch_scale_bf16(hipStream_t stream, int m, int n, float beta, void *c, int ldc);
+hipError_t launch_scale_f64(hipStream_t stream, int m, int n, double beta, double *c, int ldc);
 hipError_t launch_generic_f32(hipStream_t stream, bool ta, bool tb, int m, int n, int k, float alpha,
                               const float *a, int lda, const float *b, int ldb, float beta, float *c,
                               int ldc);

@@ -129,6 +129,13 @@ hipError_t launch_scale_f32(hipStream_t stream, int m, int n, float beta, float 
     return launch_status();
 }
 
+hipError_t launch_scale_f64(hipStream_t stream, int m, int n, double beta, double *c, int ldc)
+{
+    scale_kernel<double>
+        <<<unsigned((size_t(m) * n + 255) / 256), 256, 0, stream>>>(m, n, beta, c, ldc);
+    return launch_status();
+}
+
 hipError_t launch_scale_bf16(hipStream_t stream, int m, int n, float beta, void *c, int ldc)
 {
     scale_kernel<bf16_storage><<<unsigned((size_t(m) * n + 255) / 256), 256, 0, stream>>>(

@@ -67,13 +67,16 @@ int camblas_cuda_bgemm(camblas_cuda_context *context, char trans_a, char trans_b
                        int k, float alpha, const void *a, int lda, const void *b, int ldb,
                        float beta, void *c, int ldc);
 
-/* ref: include/camblas_cuda.h:60-62, :71-94. Present so the reference loader, which resolves
- * these names at load time, accepts the library; FP64 GEMM, affine/MLP, dense single-head
- * attention and MLP backward are outside the linear path and return a negative status with the
- * message "... is not provided by the HIP linear backend". */
+/* Same contract in FP64 (ref: include/camblas_cuda.h:60-62, src/cuda/backend.cu:1066-1073):
+ * LDS-tiled FMA kernel for every layout, no matrix-core path. */
 int camblas_cuda_dgemm(camblas_cuda_context *context, char trans_a, char trans_b, int m, int n,
                        int k, double alpha, const double *a, int lda, const double *b, int ldb,
                        double beta, double *c, int ldc);
+
+/* ref: include/camblas_cuda.h:71-94. Present so the reference loader, which resolves these names
+ * at load time, accepts the library; affine/MLP, dense single-head attention and MLP backward
+ * are outside the linear path and return a negative status with the message
+ * "... is not provided by the HIP linear backend". */
 int camblas_cuda_affine(camblas_cuda_context *context, int dtype, int rows, int inner, int columns,
                         const void *x, const void *weight, const void *bias, int relu,
                         void *output);

@@ -117,3 +117,18 @@ def test_bench_refuses_more_than_one_gpu():
     result = subprocess.run([sys.executable, str(ROOT / "bench.py"), "--gpus", "2"],
                             capture_output=True, text=True)
     assert result.returncode != 0 and "one GPU" in result.stderr
+
+
+def test_tensor_binding_loads_and_exports_the_reference_surface():
+    # names the reference's Python layer looks up on its compiled binding
+    # (ref: src/cuda/torch_bindings.cpp:1194-1294, camblas/_native.py:278-283, :327-336)
+    module = _native.tensor_module()
+    assert module is not None, "camblas_amd/lib/_camblas_cuda_torch*.so is not built"
+    for name in ("install_torch_backend", "set_default_algorithm", "stats", "stats_all", "close",
+                 "matmul", "matmul_public", "linear_public", "qkv_linear", "gated_mlp",
+                 "silu_multiply", "swiglu", "rms_norm", "add_rms_norm", "fp8_block_matmul"):
+        assert callable(getattr(module, name)), name
+    import torch
+
+    with pytest.raises(ValueError, match="GPU"):
+        module.matmul_public(torch.zeros(2, 2), torch.zeros(2, 2))

@@ -142,4 +142,29 @@ def test_invalid_arguments_report_errors(device):
                                   None, 1) == 0
     assert lib.camblas_cuda_dgemm(native.handle, b"N", b"N", 1, 1, 1, 1.0, None, 1, None, 1, 0.0,
                                   None, 1) == -1
+    assert b"invalid device pointer" in lib.camblas_cuda_error(native.handle)
+    assert lib.camblas_cuda_affine(native.handle, 0, 1, 1, 1, None, None, None, 0, None) == -1
     assert b"not provided" in lib.camblas_cuda_error(native.handle)
+
+
+@pytest.mark.parametrize("ta", "NT")
+@pytest.mark.parametrize("tb", "NT")
+def test_dgemm_matches_float64_product(device, ta, tb):
+    # FP64 storage and accumulation: the only difference from numpy's product is summation order
+    m, n, k = 67, 45, 130
+    lda, ldb, ldc = (m if ta == "N" else k) + 1, (k if tb == "N" else n) + 2, m + 3
+    a = oracle.fill_uniform(31, (lda * (k if ta == "N" else m),)).astype(np.float64)
+    b = oracle.fill_uniform(32, (ldb * (n if tb == "N" else k),)).astype(np.float64)
+    c0 = oracle.fill_uniform(33, (ldc * n,)).astype(np.float64)
+    at, bt, ct_ = (torch.from_numpy(v).to(device) for v in (a, b, c0.copy()))
+    _native.context(device).call("dgemm", ta.encode(), tb.encode(), m, n, k, ct.c_double(0.75),
+                                 ptr(at), lda, ptr(bt), ldb, ct.c_double(-2.0), ptr(ct_), ldc)
+    torch.cuda.synchronize()
+    got = ct_.cpu().numpy().reshape(n, ldc)
+    left = a.reshape(-1, lda)[:, : (m if ta == "N" else k)]   # column-major storage, rows = columns
+    left = left.T if ta == "N" else left                       # -> [m, k]
+    right = b.reshape(-1, ldb)[:, : (k if tb == "N" else n)]
+    right = right.T if tb == "N" else right                    # -> [k, n]
+    want = 0.75 * (left @ right) - 2.0 * c0.reshape(n, ldc)[:, :m].T
+    assert rel_frobenius(got[:, :m].T, want) <= 1e-13
+    assert np.array_equal(got[:, m:], c0.reshape(n, ldc)[:, m:])

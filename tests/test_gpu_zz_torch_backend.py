@@ -1,0 +1,196 @@
+"""The compiled ATen binding (_camblas_cuda_torch) on the GPU: explicit products with transpose
+views, out/alpha/beta and autograd, the linear wrapper, and the dispatcher override of
+torch.mm / mm.out / addmm with its fall-back rules (ref: src/cuda/torch_bindings.cpp:146-271,
+src/cuda/torch_backend.cuh:7-88; strategy of tests/test_torch_backend.py and tests/test_linear.py
+in the reference: FP64 product of the same operands, tolerance by storage type, dispatch counters).
+
+This file sorts last on purpose: installing the backend cannot be undone inside a process.
+Tolerances: relative Frobenius <= 1e-5 (FP32), 1e-12 (FP64), 1e-2 (BF16) against the FP64 product.
+"""
+
+import pytest
+import torch
+import torch.nn.functional as F
+
+from camblas_amd import _native
+
+pytestmark = pytest.mark.gpu
+BAR = {torch.float32: 1e-5, torch.float64: 1e-12, torch.bfloat16: 1e-2}
+
+
+@pytest.fixture(scope="module")
+def binding():
+    module = _native.tensor_module()
+    assert module is not None, "camblas_amd/lib/_camblas_cuda_torch*.so is not built"
+    return module
+
+
+def error(got, want):
+    got, want = got.double(), want.double()
+    return ((got - want).norm() / want.norm().clamp_min(1e-300)).item()
+
+
+def randn(shape, dtype, device, seed):
+    generator = torch.Generator(device="cpu").manual_seed(seed)
+    return torch.randn(shape, generator=generator, dtype=torch.float64).to(dtype).to(device)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float64, torch.bfloat16])
+@pytest.mark.parametrize("views", ["nn", "tn", "nt", "strided"])
+def test_matmul_public_layouts(binding, device, dtype, views):
+    m, k, n = 45, 96, 70
+    a = randn((m, k), dtype, device, 1)
+    b = randn((k, n), dtype, device, 2)
+    if views == "tn":
+        a = randn((k, m), dtype, device, 1).t()
+    elif views == "nt":
+        b = randn((n, k), dtype, device, 2).t()
+    elif views == "strided":
+        a = randn((m, 2 * k), dtype, device, 1)[:, ::2]      # neither stride is 1: copied
+        b = randn((k, n + 8), dtype, device, 2)[:, :n]        # padded rows: used in place
+    got = binding.matmul_public(a, b)
+    assert got.shape == (m, n) and got.dtype == dtype and got.is_contiguous()
+    assert error(got, a.double() @ b.double()) <= BAR[dtype]
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_matmul_public_out_alpha_beta(binding, device, dtype):
+    a, b = randn((33, 64), dtype, device, 3), randn((64, 40), dtype, device, 4)
+    c = randn((33, 40), dtype, device, 5)
+    want = 0.5 * (a.double() @ b.double()) - 1.5 * c.double()
+    version = c._version
+    out = binding.matmul_public(a, b, out=c, alpha=0.5, beta=-1.5)
+    assert out.data_ptr() == c.data_ptr() and c._version == version + 1
+    assert error(c, want) <= BAR[dtype]
+    with pytest.raises(ValueError, match="alias"):
+        binding.matmul_public(a, b, out=a.view(-1)[: 33 * 40].view(33, 40))
+    with pytest.raises(ValueError, match="beta requires"):
+        binding.matmul_public(a, b, beta=1.0)
+    with pytest.raises(ValueError, match="same device and dtype"):
+        binding.matmul_public(a, b.float() if dtype != torch.float32 else b.double())
+    with pytest.raises(ValueError, match="GPU"):
+        binding.matmul_public(a.cpu(), b.cpu())
+
+
+def test_matmul_public_autograd(binding, device):
+    a = randn((24, 48), torch.float32, device, 6).requires_grad_()
+    b = randn((48, 16), torch.float32, device, 7).requires_grad_()
+    g = randn((24, 16), torch.float32, device, 8)
+    binding.matmul_public(a, b).backward(g)
+    assert error(a.grad, g.double() @ b.detach().double().t()) <= 1e-5
+    assert error(b.grad, a.detach().double().t() @ g.double()) <= 1e-5
+    with pytest.raises(ValueError, match="Autograd matmul"):
+        binding.matmul_public(a, b, alpha=2.0)
+    # second derivative goes through the same entry
+    a2 = randn((6, 5), torch.float64, device, 9).requires_grad_()
+    b2 = randn((5, 4), torch.float64, device, 10).requires_grad_()
+    assert torch.autograd.gradcheck(lambda u, v: binding.matmul_public(u, v), (a2, b2))
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_linear_public(binding, device, dtype):
+    x = randn((3, 5, 256), dtype, device, 11)
+    w = randn((72, 256), dtype, device, 12)
+    bias = randn((72,), dtype, device, 13)
+    got = binding.linear_public(x, w, bias)
+    assert got.shape == (3, 5, 72)
+    want = x.double() @ w.double().t() + bias.double()
+    assert error(got, want) <= 1.5 * BAR[dtype]
+    assert error(binding.linear_public(x[0, 0], w), x[0, 0].double() @ w.double().t()) <= BAR[dtype]
+    with pytest.raises(ValueError, match="linear requires"):
+        binding.linear_public(x, w[:, :100])
+
+
+def test_fusion_entries(binding, device):
+    x = randn((7, 512), torch.bfloat16, device, 14)
+    gate_w, up_w = randn((384, 512), torch.bfloat16, device, 15) * 0.05, randn((384, 512), torch.bfloat16, device, 16) * 0.05
+    down_w = randn((512, 384), torch.bfloat16, device, 17) * 0.05
+    gate, up = x.double() @ gate_w.double().t(), x.double() @ up_w.double().t()
+    want = (F.silu(gate) * up) @ down_w.double().t()
+    assert error(binding.gated_mlp(x, gate_w, up_w, down_w), want) <= 2e-2
+    q, k, v = binding.qkv_linear(x, gate_w, up_w, gate_w)
+    assert error(q, gate) <= 1e-2 and error(k, up) <= 1e-2 and torch.equal(q, v)
+    weight = randn((512,), torch.bfloat16, device, 18) * 0.1 + 1
+    residual = randn((7, 512), torch.bfloat16, device, 19)
+    added, normed = binding.add_rms_norm(x, residual, weight, 1e-5)
+    assert torch.equal(added, x + residual)
+    a64 = added.double()
+    want = a64 * torch.rsqrt((a64 * a64).mean(-1, keepdim=True) + 1e-5) * weight.double()
+    assert error(normed, want) <= 1e-2
+    assert error(binding.rms_norm(added, weight, 1e-5), want) <= 1e-2
+    assert error(binding.silu_multiply(x, residual), F.silu(x.double()) * residual.double()) <= 1e-2
+    assert error(binding.swiglu(x, residual), F.silu(x.double()) * residual.double()) <= 1e-2
+    with pytest.raises(ValueError, match="inference only"):
+        binding.silu_multiply(x.clone().requires_grad_(), residual)
+
+
+def test_backend_override_routes_and_falls_back(binding, device):
+    binding.install_torch_backend(_native.ALGORITHMS["lt"])
+    binding.install_torch_backend(_native.ALGORITHMS["lt"])  # idempotent
+
+    def dispatched(run):
+        before = sum(binding.stats_all(device.index or 0, False).values())
+        result = run()
+        torch.cuda.synchronize()
+        return result, sum(binding.stats_all(device.index or 0, False).values()) - before
+
+    # BF16 and FP32 products, transposed views, F.linear with and without bias
+    a, b = randn((64, 256), torch.bfloat16, device, 20), randn((256, 48), torch.bfloat16, device, 21)
+    got, count = dispatched(lambda: torch.mm(a, b))
+    assert count == 1 and error(got, a.double() @ b.double()) <= 1e-2
+    w, bias = randn((48, 256), torch.bfloat16, device, 22), randn((48,), torch.bfloat16, device, 23)
+    got, count = dispatched(lambda: F.linear(a.view(4, 16, 256), w, bias))
+    assert count == 1 and got.shape == (4, 16, 48)
+    assert error(got, a.double().view(4, 16, 256) @ w.double().t() + bias.double()) <= 1e-2
+    got, count = dispatched(lambda: a @ w.t())
+    assert count == 1 and error(got, a.double() @ w.double().t()) <= 1e-2
+    previous = torch.backends.cuda.matmul.allow_tf32
+    try:
+        torch.backends.cuda.matmul.allow_tf32 = False
+        a32, b32 = randn((50, 80), torch.float32, device, 24), randn((80, 30), torch.float32, device, 25)
+        got, count = dispatched(lambda: torch.mm(a32, b32))
+        assert count == 1 and error(got, a32.double() @ b32.double()) <= 1e-5
+        out = torch.empty((50, 30), device=device)
+        _, count = dispatched(lambda: torch.mm(a32, b32, out=out))
+        assert count == 1 and error(out, a32.double() @ b32.double()) <= 1e-5
+        # addmm: beta scales the broadcast bias; beta = 0 never reads it
+        row = randn((30,), torch.float32, device, 26)
+        got, count = dispatched(lambda: torch.addmm(row, a32, b32, beta=0.5, alpha=2.0))
+        assert count == 1 and error(got, 2.0 * (a32.double() @ b32.double()) + 0.5 * row.double()) <= 1e-5
+        poisoned = torch.full((50, 30), float("nan"), device=device)
+        got, count = dispatched(lambda: torch.addmm(poisoned, a32, b32, beta=0.0))
+        assert count == 1 and torch.isfinite(got).all()
+        # autograd derives its products from mm, so they are routed as well
+        left = a32.clone().requires_grad_()
+        _, count = dispatched(lambda: torch.mm(left, b32).sum().backward())
+        assert count == 2 and error(left.grad, torch.ones(50, 30, device=device).double() @ b32.double().t()) <= 1e-5
+        # fall-backs keep ATen's result and do not touch the library: reduced-precision FP32
+        # allowed by the caller, other dtypes, empty operands
+        torch.backends.cuda.matmul.allow_tf32 = True
+        got, count = dispatched(lambda: torch.mm(a32, b32))
+        assert count == 0 and error(got, a32.double() @ b32.double()) <= 1e-2
+        torch.backends.cuda.matmul.allow_tf32 = False
+        half = a32.half()
+        got, count = dispatched(lambda: torch.mm(half, b32.half()))
+        assert count == 0 and got.dtype == torch.float16
+        got, count = dispatched(lambda: torch.mm(a32[:0], b32))
+        assert count == 0 and got.shape == (0, 30)
+        got, count = dispatched(lambda: torch.mm(a32[:, :0], b32[:0]))
+        assert count == 0 and got.shape == (50, 30) and not got.any()
+    finally:
+        torch.backends.cuda.matmul.allow_tf32 = previous
+
+
+def test_stats_and_close(binding, device):
+    index = device.index or 0
+    a, b = randn((32, 64), torch.bfloat16, device, 30), randn((64, 32), torch.bfloat16, device, 31)
+    binding.stats(index, True, 0)
+    binding.matmul_public(a, b)
+    counts = binding.stats(index, False, 0)
+    assert set(counts) == set(_native.COUNTERS) and sum(counts.values()) == 1
+    assert sum(binding.stats(index, True, 0).values()) == 1
+    assert sum(binding.stats(index, False, 0).values()) == 0
+    binding.close()
+    torch.cuda.synchronize()
+    # contexts are recreated on demand after close
+    assert error(binding.matmul_public(a, b), a.double() @ b.double()) <= 1e-2
