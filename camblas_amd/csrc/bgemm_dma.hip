@@ -157,9 +157,7 @@ __global__ __launch_bounds__(128 * WM) void bgemm_dma_kernel(DmaParams p)
             mfma(a_frag[ks & 1], b_frag[ks & 1]);
             __builtin_amdgcn_sched_barrier(0);
         }
-        wait_loads<LOADS *(STAGES - 2)>();
-        __syncthreads();
-        __builtin_amdgcn_sched_barrier(0);
+        pipeline_barrier<LOADS *(STAGES - 2)>();
         read(next, 0, a_frag[0], b_frag[0]);
         __builtin_amdgcn_sched_barrier(0);
         mfma(a_frag[(KS - 1) & 1], b_frag[(KS - 1) & 1]);
@@ -179,8 +177,7 @@ __global__ __launch_bounds__(128 * WM) void bgemm_dma_kernel(DmaParams p)
         issue(stage2);
         clamp_k();
     }
-    wait_loads<LOADS *(STAGES - 2)>();
-    __syncthreads();
+    pipeline_barrier<LOADS *(STAGES - 2)>();
     read(stage0, 0, a_frag[0], b_frag[0]);
     for (int tile = 0; tile < k_tiles; tile += STAGES) {
         if constexpr (STAGES == 2) {

@@ -48,6 +48,21 @@ template <int N> __device__ __forceinline__ void wait_loads()
     __builtin_amdgcn_s_waitcnt((N & 15) | ((N >> 4) << 14) | 0x0f70);
 }
 
+// End of a pipeline step: wait until at most N of this wavefront's loads (the newest ones, filling
+// a stage nobody reads yet) are outstanding and its own LDS reads have returned, then meet the
+// other wavefronts. __syncthreads() cannot be used here: its release fence makes the compiler wait
+// for every outstanding load, LDS fills included, which collapses a deeper pipeline to two stages.
+// What the barrier has to order is covered by the explicit wait: fills of the stage read next
+// were issued a full step earlier and are complete; reads of the stage refilled next are complete.
+template <int N> __device__ __forceinline__ void pipeline_barrier()
+{
+    static_assert(N >= 0 && N < 64, "vmcnt holds 6 bits");
+    __builtin_amdgcn_sched_barrier(0);
+    __builtin_amdgcn_s_waitcnt((N & 15) | ((N >> 4) << 14) | 0x0070); // vmcnt(N) lgkmcnt(0)
+    __builtin_amdgcn_s_barrier();
+    __builtin_amdgcn_sched_barrier(0);
+}
+
 // Workgroup index -> output tile: consecutive workgroups go to different XCDs, so each XCD is given
 // a contiguous range of logical tile numbers, and logical numbers walk the tile grid in groups of
 // eight feature tiles so that the tiles resident on one XCD share operand panels through its L2.

@@ -8,12 +8,13 @@
 // A workgroup of 2 x WM wavefronts owns a 256 x (32*WM*TM) output tile; each wavefront owns 128
 // weight rows (exactly one 128-row scale block) by 32*TM tokens. One K step is one scale group:
 // 128 bytes per row, the same LDS geometry (8 chunks of 16 bytes, XOR swizzle) as a 64-deep BF16
-// step, two stages filled by buffer_load ... lds. A group's dot product is two
+// step, STAGES stages filled by buffer_load ... lds STAGES-1 groups ahead (one group of matrix
+// work is shorter than the memory latency, so two stages leave the matrix cores waiting for
+// loads). A group's dot product is two
 // v_mfma_scale_f32_32x32x64_f8f6f4 (unit hardware scales) into a zeroed temporary; the scaled
 // accumulate of one 32x32 tile runs on the vector ALU while the matrix cores work on the next tile.
-// Weight scales for 64 consecutive groups are fetched with one coalesced load and broadcast with
-// v_readlane, activation scales are one 4-byte load per lane, token tile and step, fetched a step
-// ahead.
+// The weight scale of a group (one per wavefront: its 128 rows lie in one scale block) and the
+// activation scales (one per lane and token tile) are 4-byte loads fetched a group ahead.
 #include "common.hpp"
 #include "device.hpp"
 #include "dma.hpp"
@@ -32,17 +33,19 @@ struct Fp8DmaParams {
     int tiles_n, tiles_m;
 };
 
-template <int TM, int WM>
+template <int TM, int WM, int STAGES>
 __global__ __launch_bounds__(128 * WM) void fp8_dma_kernel(Fp8DmaParams p)
 {
+    static_assert(STAGES == 2 || STAGES == 3, "two or three LDS stages");
     constexpr int TN = 4, WAVES = 2 * WM, CH = 8, BK = 128;
     constexpr int BN = 64 * TN, BM = 32 * WM * TM;
     constexpr int ROWS_PER_LOAD = 8;
     constexpr int A_ITERS = BN / (WAVES * ROWS_PER_LOAD), B_ITERS = BM / (WAVES * ROWS_PER_LOAD);
-    constexpr int SLOTS = (BN + BM) * CH;
+    constexpr int SLOTS = (BN + BM) * CH, LOADS = A_ITERS + B_ITERS;
     static_assert(BN % (WAVES * ROWS_PER_LOAD) == 0 && BM % (WAVES * ROWS_PER_LOAD) == 0, "loads");
     __shared__ u32x4_t stage0[SLOTS];
     __shared__ u32x4_t stage1[SLOTS];
+    __shared__ u32x4_t stage2[STAGES > 2 ? SLOTS : 1];
 
     int tile_n, tile_m;
     xcd_tile(int(blockIdx.x), p.tiles_n, p.tiles_m, tile_n, tile_m);
@@ -50,21 +53,16 @@ __global__ __launch_bounds__(128 * WM) void fp8_dma_kernel(Fp8DmaParams p)
     const int thread = threadIdx.x, lane = thread % 64, wave = thread / 64;
     const int wn = wave % 2, wm = wave / 2;
 
-    unsigned a_off[A_ITERS], b_off[B_ITERS];
-#pragma unroll
-    for (int it = 0; it < A_ITERS; ++it) {
-        int row = (it * WAVES + wave) * ROWS_PER_LOAD + lane / CH;
-        int chunk = (lane % CH) ^ lds_swizzle<CH>(row);
-        int global_row = n0 + row < p.n ? n0 + row : p.n - 1;
-        a_off[it] = unsigned(global_row - n0) * unsigned(p.k) + unsigned(chunk * 16);
-    }
-#pragma unroll
-    for (int it = 0; it < B_ITERS; ++it) {
-        int row = (it * WAVES + wave) * ROWS_PER_LOAD + lane / CH;
-        int chunk = (lane % CH) ^ lds_swizzle<CH>(row);
-        int global_row = m0 + row < p.m ? m0 + row : p.m - 1;
-        b_off[it] = unsigned(global_row - m0) * unsigned(p.k) + unsigned(chunk * 16);
-    }
+    // Lane -> (row inside an 8-row load, swizzled 16-byte chunk). Successive loads of a thread are
+    // WAVES*8 rows apart, which leaves the swizzle unchanged (it depends on row bits 0..3 only and
+    // WAVES*8 is a multiple of 16), so one lane offset serves all of them and the row advance goes
+    // into the scalar offset. Rows past the end of the matrix are outside the buffer resource and
+    // read as zero.
+    static_assert((WAVES * ROWS_PER_LOAD) % 16 == 0, "row step keeps the swizzle");
+    const int load_row = wave * ROWS_PER_LOAD + lane / CH;
+    const unsigned lane_off =
+        unsigned(load_row) * unsigned(p.k) + unsigned(((lane % CH) ^ lds_swizzle<CH>(load_row)) * 16);
+    const unsigned row_step = unsigned(WAVES * ROWS_PER_LOAD) * unsigned(p.k);
     const int a_rows = p.n - n0 < BN ? p.n - n0 : BN, b_rows = p.m - m0 < BM ? p.m - m0 : BM;
     const __amdgpu_buffer_rsrc_t a_resource =
         make_resource(p.w + size_t(n0) * p.k, unsigned(a_rows) * unsigned(p.k));
@@ -72,27 +70,32 @@ __global__ __launch_bounds__(128 * WM) void fp8_dma_kernel(Fp8DmaParams p)
         make_resource(p.a + size_t(m0) * p.k, unsigned(b_rows) * unsigned(p.k));
     const unsigned last_k_bytes = unsigned(p.groups - 1) * BK;
     unsigned k_bytes = 0;
+    // Load number `index` (0 .. LOADS-1) of the group at k_bytes; advance() moves to the next group.
+    auto issue_one = [&](u32x4_t *stage, int index) {
+        if (index < A_ITERS)
+            load_to_lds(a_resource, lane_off, k_bytes + unsigned(index) * row_step,
+                        stage + (index * WAVES + wave) * 64);
+        else
+            load_to_lds(b_resource, lane_off, k_bytes + unsigned(index - A_ITERS) * row_step,
+                        stage + BN * CH + ((index - A_ITERS) * WAVES + wave) * 64);
+    };
+    auto advance = [&]() { k_bytes = k_bytes + BK < last_k_bytes ? k_bytes + BK : last_k_bytes; };
     auto issue = [&](u32x4_t *stage) {
 #pragma unroll
-        for (int it = 0; it < A_ITERS; ++it)
-            load_to_lds(a_resource, a_off[it], k_bytes, stage + (it * WAVES + wave) * 64);
-#pragma unroll
-        for (int it = 0; it < B_ITERS; ++it)
-            load_to_lds(b_resource, b_off[it], k_bytes, stage + BN * CH + (it * WAVES + wave) * 64);
-        k_bytes = k_bytes + BK < last_k_bytes ? k_bytes + BK : last_k_bytes;
+        for (int index = 0; index < LOADS; ++index)
+            issue_one(stage, index);
+        advance();
     };
 
-    // ---- scales. The wavefront's 128 weight rows lie in one scale block: lane l holds the scale
-    // of group (64*window + l); v_readlane broadcasts the current one. Activation scales: one per
-    // lane (token = lane % 32) and token tile, loaded one step ahead.
+    // ---- scales. The wavefront's 128 weight rows lie in one scale block, so its weight scale is
+    // one value per group (every lane loads the same address); activation scales are one per lane
+    // (token = lane % 32) and token tile. Both are loaded one group ahead, unconditionally: a load
+    // under a branch would make the compiler wait for every outstanding load, the LDS fills
+    // included.
     const int frag_row = lane % 32, half = lane / 32;
     int block = (n0 + wn * 128) / 128;
     block = block < p.scale_blocks ? block : p.scale_blocks - 1;
     const float *ws_row = p.w_scale + size_t(block) * p.groups;
-    auto load_ws = [&](int window) {
-        int g = window * 64 + lane;
-        return ws_row[g < p.groups ? g : p.groups - 1];
-    };
     const float *as_ptr[TM];
 #pragma unroll
     for (int j = 0; j < TM; ++j) {
@@ -120,21 +123,22 @@ __global__ __launch_bounds__(128 * WM) void fp8_dma_kernel(Fp8DmaParams p)
         return i32x8_t{int(lo[0]), int(lo[1]), int(lo[2]), int(lo[3]),
                        int(hi[0]), int(hi[1]), int(hi[2]), int(hi[3])};
     };
-    // One K group. All fragments are read first; then the tiles are walked in a software pipeline:
-    // the two MFMAs of tile t+1 are issued before the 16 scaled accumulates of tile t, so the vector
-    // ALU work of one tile runs while the matrix cores execute the next (sched_barrier pins it).
-    auto multiply = [&](const u32x4_t *stage, const float (&as_now)[TM], float ws_now) {
-        i32x8_t a_frag[TN][2], b_frag[TM][2];
+    // One K group. The token fragments are read once; the weight fragments are streamed one
+    // 32-row tile ahead (two register buffers), and the tiles are walked in a software pipeline: the
+    // two MFMAs of tile t are issued, then a share of the LDS fills for the group STAGES-1 ahead,
+    // then the 16 scaled accumulates of tile t-1, so that the vector ALU work and the load issue of
+    // one tile run while the matrix cores execute the next (sched_barrier pins it).
+    auto multiply = [&](const u32x4_t *stage, u32x4_t *fill, const float (&as_now)[TM],
+                        float ws_now) {
+        constexpr int TILES = TN * TM, SHARE = (LOADS + TILES - 1) / TILES;
+        i32x8_t a_frag[2][2], b_frag[TM][2];
 #pragma unroll
         for (int j = 0; j < TM; ++j) {
             b_frag[j][0] = fragment(stage, b_frag_base + j * 32 * CH, 0);
             b_frag[j][1] = fragment(stage, b_frag_base + j * 32 * CH, 1);
         }
-#pragma unroll
-        for (int i = 0; i < TN; ++i) {
-            a_frag[i][0] = fragment(stage, a_frag_base + i * 32 * CH, 0);
-            a_frag[i][1] = fragment(stage, a_frag_base + i * 32 * CH, 1);
-        }
+        a_frag[0][0] = fragment(stage, a_frag_base, 0);
+        a_frag[0][1] = fragment(stage, a_frag_base, 1);
         float scale[TM];
 #pragma unroll
         for (int j = 0; j < TM; ++j)
@@ -145,10 +149,10 @@ __global__ __launch_bounds__(128 * WM) void fp8_dma_kernel(Fp8DmaParams p)
 #pragma unroll
             for (int r = 0; r < 16; ++r)
                 d[r] = 0.f;
-            d = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(a_frag[i][0], b_frag[j][0], d, 0, 0,
-                                                                0, UNIT, 0, UNIT);
-            d = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(a_frag[i][1], b_frag[j][1], d, 0, 0,
-                                                                0, UNIT, 0, UNIT);
+            d = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(a_frag[i & 1][0], b_frag[j][0], d, 0,
+                                                                0, 0, UNIT, 0, UNIT);
+            d = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(a_frag[i & 1][1], b_frag[j][1], d, 0,
+                                                                0, 0, UNIT, 0, UNIT);
         };
         auto accumulate = [&](int tile, const f32x16_t &d) {
             const int i = tile / TM, j = tile % TM;
@@ -156,59 +160,76 @@ __global__ __launch_bounds__(128 * WM) void fp8_dma_kernel(Fp8DmaParams p)
             for (int r = 0; r < 16; ++r)
                 acc[i][j][r] = fmaf(d[r], scale[j], acc[i][j][r]);
         };
-        __builtin_amdgcn_sched_barrier(0);
-        product(0, dot[0]);
 #pragma unroll
-        for (int tile = 1; tile < TN * TM; ++tile) {
+        for (int tile = 0; tile < TILES; ++tile) {
+            __builtin_amdgcn_sched_barrier(0);
+            if (tile % TM == 0 && tile / TM + 1 < TN) { // next weight tile into the other buffer
+                const int row = tile / TM + 1;
+                a_frag[row & 1][0] = fragment(stage, a_frag_base + row * 32 * CH, 0);
+                a_frag[row & 1][1] = fragment(stage, a_frag_base + row * 32 * CH, 1);
+            }
             __builtin_amdgcn_sched_barrier(0);
             product(tile, dot[tile & 1]);
             __builtin_amdgcn_sched_barrier(0);
-            accumulate(tile - 1, dot[(tile - 1) & 1]);
+#pragma unroll
+            for (int index = tile * SHARE; index < (tile + 1) * SHARE && index < LOADS; ++index)
+                issue_one(fill, index);
+            __builtin_amdgcn_sched_barrier(0);
+            if (tile > 0)
+                accumulate(tile - 1, dot[(tile - 1) & 1]);
         }
         __builtin_amdgcn_sched_barrier(0);
-        accumulate(TN * TM - 1, dot[(TN * TM - 1) & 1]);
+        advance();
+        accumulate(TILES - 1, dot[(TILES - 1) & 1]);
         __builtin_amdgcn_sched_barrier(0);
     };
 
-    float ws_window = load_ws(0);
+    float ws_now = ws_row[0], ws_next;
     float as_now[TM], as_next[TM];
 #pragma unroll
     for (int j = 0; j < TM; ++j)
         as_now[j] = as_ptr[j][0];
+    // One group: start the loads of the group STAGES-1 ahead into the stage that was read last,
+    // multiply the current stage, then wait until only the newest loads are still in flight.
+    auto step = [&](int g, const u32x4_t *current, u32x4_t *fill) {
+        const int next = g + 1 < p.groups ? g + 1 : p.groups - 1;
+        ws_next = ws_row[next];
+#pragma unroll
+        for (int j = 0; j < TM; ++j)
+            as_next[j] = as_ptr[j][next];
+        __builtin_amdgcn_sched_barrier(0);
+        multiply(current, fill, as_now, ws_now);
+        ws_now = ws_next;
+#pragma unroll
+        for (int j = 0; j < TM; ++j)
+            as_now[j] = as_next[j];
+        pipeline_barrier<(STAGES - 2) * LOADS>();
+    };
     issue(stage0);
-    wait_loads<0>();
-    __syncthreads();
-    for (int g = 0; g < p.groups; g += 2) {
-        // even group: stage0 is current
-        {
-            const int next = g + 1 < p.groups ? g + 1 : p.groups - 1;
-#pragma unroll
-            for (int j = 0; j < TM; ++j)
-                as_next[j] = as_ptr[j][next];
-            __builtin_amdgcn_sched_barrier(0);
-            issue(stage1);
-            __builtin_amdgcn_sched_barrier(0);
-            float ws_now = __builtin_bit_cast(
-                float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, ws_window), g & 63));
-            multiply(stage0, as_now, ws_now);
-            wait_loads<0>();
-            __syncthreads();
+    if constexpr (STAGES == 3) {
+        __builtin_amdgcn_sched_barrier(0);
+        issue(stage1);
+    }
+    pipeline_barrier<(STAGES - 2) * LOADS>();
+    // whole rounds of STAGES groups run without a branch between the steps; the remainder follows
+    int g = 0;
+    if constexpr (STAGES == 2) {
+        for (; g + 2 <= p.groups; g += 2) {
+            step(g, stage0, stage1);
+            step(g + 1, stage1, stage0);
         }
-        if (g + 1 < p.groups) {
-            const int next = g + 2 < p.groups ? g + 2 : p.groups - 1;
-#pragma unroll
-            for (int j = 0; j < TM; ++j)
-                as_now[j] = as_ptr[j][next];
-            __builtin_amdgcn_sched_barrier(0);
-            issue(stage0);
-            __builtin_amdgcn_sched_barrier(0);
-            float ws_now = __builtin_bit_cast(
-                float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, ws_window), (g + 1) & 63));
-            multiply(stage1, as_next, ws_now);
-            if (((g + 2) & 63) == 0) // the next group starts a new window of 64 weight scales
-                ws_window = load_ws((g + 2) / 64);
-            wait_loads<0>();
-            __syncthreads();
+        if (g < p.groups)
+            step(g, stage0, stage1);
+    } else {
+        for (; g + 3 <= p.groups; g += 3) {
+            step(g, stage0, stage2);
+            step(g + 1, stage1, stage0);
+            step(g + 2, stage2, stage1);
+        }
+        if (g < p.groups) {
+            step(g, stage0, stage2);
+            if (g + 1 < p.groups)
+                step(g + 1, stage1, stage0);
         }
     }
     wait_loads<0>();
@@ -234,14 +255,15 @@ __global__ __launch_bounds__(128 * WM) void fp8_dma_kernel(Fp8DmaParams p)
     }
 }
 
-template <int TM, int WM> hipError_t launch_one(hipStream_t stream, Fp8DmaParams p)
+template <int TM, int WM, int STAGES> hipError_t launch_one(hipStream_t stream, Fp8DmaParams p)
 {
     constexpr int BN = 256, BM = 32 * WM * TM;
     p.tiles_n = (p.n + BN - 1) / BN;
     p.tiles_m = (p.m + BM - 1) / BM;
     if (size_t(p.tiles_n) * size_t(p.tiles_m) > 0x7fffffffu)
         return hipErrorInvalidValue;
-    fp8_dma_kernel<TM, WM><<<unsigned(p.tiles_n) * unsigned(p.tiles_m), 128 * WM, 0, stream>>>(p);
+    fp8_dma_kernel<TM, WM, STAGES>
+        <<<unsigned(p.tiles_n) * unsigned(p.tiles_m), 128 * WM, 0, stream>>>(p);
     return launch_status();
 }
 
@@ -250,6 +272,9 @@ const TnVariant variants[] = {
     {"fp8dma256x128x128w8", 256, 128, 128, 512},
     {"fp8dma256x128x128w4", 256, 128, 128, 256},
     {"fp8dma256x64x128w4", 256, 64, 128, 256},
+    {"fp8dma256x128x128s3w8", 256, 128, 128, 512},
+    {"fp8dma256x128x128s3w4", 256, 128, 128, 256},
+    {"fp8dma256x64x128s3w4", 256, 64, 128, 256},
 };
 } // namespace
 
@@ -278,10 +303,13 @@ hipError_t launch_fp8_dma(hipStream_t stream, int variant, int rows, int outputs
     p.scale_blocks = (outputs + 127) / 128;
     p.tiles_n = p.tiles_m = 0;
     switch (variant) {
-    case 0: return launch_one<2, 4>(stream, p);
-    case 1: return launch_one<1, 4>(stream, p);
-    case 2: return launch_one<2, 2>(stream, p);
-    case 3: return launch_one<1, 2>(stream, p);
+    case 0: return launch_one<2, 4, 2>(stream, p);
+    case 1: return launch_one<1, 4, 2>(stream, p);
+    case 2: return launch_one<2, 2, 2>(stream, p);
+    case 3: return launch_one<1, 2, 2>(stream, p);
+    case 4: return launch_one<1, 4, 3>(stream, p);
+    case 5: return launch_one<2, 2, 3>(stream, p);
+    case 6: return launch_one<1, 2, 3>(stream, p);
     default: return hipErrorInvalidValue;
     }
 }

@@ -171,7 +171,7 @@ Plan make_plan(int dtype, int algorithm, bool trans_a, bool trans_b, int m, int 
     const struct {
         int variant, resident;
         double weight;
-    } candidates[] = {{1, 1, 1.0}, {3, 1, 0.9}};
+    } candidates[] = {{4, 1, 1.0}, {3, 1, 0.9}};
     double best = -1;
     for (const auto &candidate : candidates) {
         const TnVariant &v = fp8_dma_variant(candidate.variant);

@@ -56,7 +56,7 @@ def test_random_blocks_every_variant(device, variant, split, rows):
         assert (np.abs(bf16_values(out) - wanted) <= bound).all()
 
 
-@pytest.mark.parametrize("code", [20, 21, 22, 23])
+@pytest.mark.parametrize("code", [20, 21, 22, 23, 24, 25, 26])
 @pytest.mark.parametrize("rows,outputs,inner", [(70, 300, 512), (256, 512, 128), (513, 260, 896)])
 def test_direct_lds_load_variants(device, code, rows, outputs, inner):
     # partial tiles in both directions, a partial last weight-scale block, odd and even numbers of
@@ -80,7 +80,7 @@ def test_planned_shapes(device, rows):
     assert rel_frobenius(bf16_values(out), oracle.fp8_block_matmul_f64(a, a_scale, w, w_scale)) <= TOLERANCE
 
 
-@pytest.mark.parametrize("override", [None, (0, 1), (1, 1), (2, 1), (3, 1), (20, 1), (21, 1), (22, 1), (23, 1)])
+@pytest.mark.parametrize("override", [None, (0, 1), (1, 1), (2, 1), (3, 1), (20, 1), (21, 1), (22, 1), (23, 1), (24, 1), (25, 1), (26, 1)])
 def test_scale_indexing_is_bit_exact(device, override):
     # every product is a small integer and every scale a distinct power of two, so the FMA chain
     # is exact: any wrong (row, group) or (block, group) scale index changes the bits
