@@ -311,7 +311,7 @@ def extras(torch, _kernels, _native, device, normal):
     y = torch.empty((tokens, outputs), dtype=torch.bfloat16, device=device)
     c = normal((tokens, outputs))
     flops = 2.0 * tokens * outputs * inner
-    seconds = event_time(torch, lambda i: _kernels.matmul(x, w.t(), out=y), 3, 10)
+    seconds = event_time(torch, lambda i: _kernels.matmul(x, w.t(), out=y), 10, 20)
     found["bf16_prefill_linear"] = {
         "shape": [tokens, outputs, inner], "us": round(seconds * 1e6, 1),
         "tflops": round(flops / seconds / 1e12, 1), "frac_of_2.5PF": round(flops / seconds / BF16_PEAK, 4),
@@ -334,7 +334,7 @@ def extras(torch, _kernels, _native, device, normal):
         a_scale = torch.rand((tokens, inner // 128), device=device) * 0.1 + 1e-4
         out = torch.empty((tokens, outputs), dtype=torch.bfloat16, device=device)
         seconds = event_time(
-            torch, lambda i: _kernels.fp8_block_matmul(a, a_scale, w, w_scale, out=out), 3, 10)
+            torch, lambda i: _kernels.fp8_block_matmul(a, a_scale, w, w_scale, out=out), 10, 20)
         flops = 2.0 * tokens * outputs * inner
         traffic = outputs * inner + w_scale.numel() * 4 + tokens * (inner + inner // 128 * 4 + outputs * 2)
         fp8[str(tokens)] = {
