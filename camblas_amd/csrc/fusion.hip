@@ -109,10 +109,12 @@ __global__ __launch_bounds__(256) void rms_rows_kernel(int width, float epsilon,
 }
 
 // BF16 rows whose width is a multiple of 8 and whose buffers are 16-byte aligned: the row is read
-// once with 128-bit loads and kept in registers (up to 8192 columns per 256 threads x 4 vectors;
-// wider rows loop), same arithmetic and reduction order class as above.
-template <int VECTORS, bool WEIGHT_BF16>
-__global__ __launch_bounds__(256) void rms_rows_bf16_kernel(int width, float epsilon,
+// once with 128-bit loads and kept in registers (THREADS x VECTORS vectors of 8 columns), same
+// arithmetic and reduction order class as above. Decode batches have few rows, so a row is spread
+// over up to 1024 threads to keep the dependent chain per thread short, and the weights are
+// fetched before the reduction so that their latency overlaps it.
+template <int VECTORS, bool WEIGHT_BF16, int THREADS>
+__global__ __launch_bounds__(THREADS) void rms_rows_bf16_kernel(int width, float epsilon,
                                                             bool round_before_weight,
                                                             const unsigned short *input,
                                                             const unsigned short *residual,
@@ -120,7 +122,7 @@ __global__ __launch_bounds__(256) void rms_rows_bf16_kernel(int width, float eps
                                                             unsigned short *added,
                                                             unsigned short *out)
 {
-    __shared__ float partial[4];
+    __shared__ float partial[THREADS / 64];
     const size_t base = size_t(blockIdx.x) * width;
     const int vectors = width / 8;
     const u32x4_t *x = reinterpret_cast<const u32x4_t *>(input + base);
@@ -129,7 +131,7 @@ __global__ __launch_bounds__(256) void rms_rows_bf16_kernel(int width, float eps
     float sum = 0.f;
 #pragma unroll
     for (int v = 0; v < VECTORS; ++v) {
-        int index = v * 256 + threadIdx.x;
+        int index = v * THREADS + threadIdx.x;
         if (index < vectors) {
             u32x4_t xv = x[index];
             u32x4_t rv = {0u, 0u, 0u, 0u};
@@ -159,33 +161,42 @@ __global__ __launch_bounds__(256) void rms_rows_bf16_kernel(int width, float eps
             }
         }
     }
+    // weights of this thread's columns, requested before the reduction
+    float w[VECTORS][8];
+#pragma unroll
+    for (int v = 0; v < VECTORS; ++v) {
+        int index = v * THREADS + threadIdx.x;
+        index = index < vectors ? index : vectors - 1;
+        if constexpr (WEIGHT_BF16) {
+            u32x4_t wv = reinterpret_cast<const u32x4_t *>(weight)[index];
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                w[v][2 * e] = __uint_as_float(wv[e] << 16);
+                w[v][2 * e + 1] = __uint_as_float(wv[e] & 0xffff0000u);
+            }
+        } else {
+            const f32x4_t *wf = reinterpret_cast<const f32x4_t *>(weight) + 2 * index;
+            f32x4_t w0 = wf[0], w1 = wf[1];
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                w[v][e] = w0[e];
+                w[v][4 + e] = w1[e];
+            }
+        }
+    }
     sum = wave_sum(sum);
     if (threadIdx.x % 64 == 0)
         partial[threadIdx.x / 64] = sum;
     __syncthreads();
-    float total = __fadd_rn(__fadd_rn(partial[0], partial[1]), __fadd_rn(partial[2], partial[3]));
+    float total = partial[0];
+#pragma unroll
+    for (int part = 1; part < THREADS / 64; ++part)
+        total = __fadd_rn(total, partial[part]);
     float scale = rsqrtf(__fadd_rn(total / float(width), epsilon));
 #pragma unroll
     for (int v = 0; v < VECTORS; ++v) {
-        int index = v * 256 + threadIdx.x;
+        int index = v * THREADS + threadIdx.x;
         if (index < vectors) {
-            float w[8];
-            if constexpr (WEIGHT_BF16) {
-                u32x4_t wv = reinterpret_cast<const u32x4_t *>(weight)[index];
-#pragma unroll
-                for (int e = 0; e < 4; ++e) {
-                    w[2 * e] = __uint_as_float(wv[e] << 16);
-                    w[2 * e + 1] = __uint_as_float(wv[e] & 0xffff0000u);
-                }
-            } else {
-                const f32x4_t *wf = reinterpret_cast<const f32x4_t *>(weight) + 2 * index;
-                f32x4_t w0 = wf[0], w1 = wf[1];
-#pragma unroll
-                for (int e = 0; e < 4; ++e) {
-                    w[e] = w0[e];
-                    w[4 + e] = w1[e];
-                }
-            }
             u32x4_t packed;
 #pragma unroll
             for (int e = 0; e < 4; ++e) {
@@ -195,7 +206,7 @@ __global__ __launch_bounds__(256) void rms_rows_bf16_kernel(int width, float eps
                     n0 = bf16_bits_to_float(float_to_bf16_bits(n0));
                     n1 = bf16_bits_to_float(float_to_bf16_bits(n1));
                 }
-                packed[e] = pack_bf16x2(__fmul_rn(n0, w[2 * e]), __fmul_rn(n1, w[2 * e + 1]));
+                packed[e] = pack_bf16x2(__fmul_rn(n0, w[v][2 * e]), __fmul_rn(n1, w[v][2 * e + 1]));
             }
             reinterpret_cast<u32x4_t *>(out + base)[index] = packed;
         }
@@ -335,21 +346,30 @@ hipError_t launch_rms_rows(hipStream_t stream, int dtype, int weight_dtype, int 
     const unsigned short *x = static_cast<const unsigned short *>(input);
     const unsigned short *r = static_cast<const unsigned short *>(residual);
     unsigned short *a = static_cast<unsigned short *>(added), *o = static_cast<unsigned short *>(out);
-    bool vector = width % 8 == 0 && width <= 8192 && aligned16(input) && aligned16(out) &&
+    bool vector = width % 8 == 0 && width <= 32768 && aligned16(input) && aligned16(out) &&
                   aligned16(weight) && (!residual || (aligned16(residual) && aligned16(added)));
-    if (vector && weight_dtype == 2) {
-        if (width <= 2048)
-            rms_rows_bf16_kernel<1, true>
-                <<<rows, 256, 0, stream>>>(width, epsilon, round_before_weight, x, r, weight, a, o);
-        else if (width <= 4096)
-            rms_rows_bf16_kernel<2, true>
-                <<<rows, 256, 0, stream>>>(width, epsilon, round_before_weight, x, r, weight, a, o);
-        else
-            rms_rows_bf16_kernel<4, true>
-                <<<rows, 256, 0, stream>>>(width, epsilon, round_before_weight, x, r, weight, a, o);
-    } else if (vector) {
-        rms_rows_bf16_kernel<4, false>
-            <<<rows, 256, 0, stream>>>(width, epsilon, round_before_weight, x, r, weight, a, o);
+#define CAMBLAS_RMS_ROWS(VECTORS, BF16_WEIGHT, THREADS)                                            \
+    rms_rows_bf16_kernel<VECTORS, BF16_WEIGHT, THREADS>                                            \
+        <<<rows, THREADS, 0, stream>>>(width, epsilon, round_before_weight, x, r, weight, a, o)
+    if (vector) {
+        const bool bf16_weight = weight_dtype == 2;
+        if (width <= 2048) {
+            if (bf16_weight)
+                CAMBLAS_RMS_ROWS(1, true, 256);
+            else
+                CAMBLAS_RMS_ROWS(1, false, 256);
+        } else if (width <= 8192) {
+            if (bf16_weight)
+                CAMBLAS_RMS_ROWS(1, true, 1024);
+            else
+                CAMBLAS_RMS_ROWS(1, false, 1024);
+        } else {
+            if (bf16_weight)
+                CAMBLAS_RMS_ROWS(4, true, 1024);
+            else
+                CAMBLAS_RMS_ROWS(4, false, 1024);
+        }
+#undef CAMBLAS_RMS_ROWS
     } else if (weight_dtype == 2) {
         rms_rows_kernel<bf16_storage, bf16_storage><<<rows, 256, 0, stream>>>(
             width, epsilon, round_before_weight, static_cast<const bf16_storage *>(input),

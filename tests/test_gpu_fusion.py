@@ -61,7 +61,8 @@ def test_swiglu_bf16(device, limit, routed):
     assert np.isnan(bf16_values(out)[0, 0])
 
 
-@pytest.mark.parametrize("rows,width", [(32, 8192), (1, 2048), (3, 4104), (5, 1000), (2, 16384)])
+@pytest.mark.parametrize("rows,width", [(32, 8192), (1, 2048), (3, 4104), (5, 1000), (2, 16384),
+                                        (2, 32768), (1, 40008)])
 @pytest.mark.parametrize("round_before_weight", [True, False])
 def test_add_rms_norm_rows_bf16(device, rows, width, round_before_weight):
     x = oracle.fill_normal_bf16(10, (rows, width))
