@@ -324,11 +324,27 @@ def kv_append(k_new, v_new, k_cache, v_cache, positions):
     )
 
 
+def rope_kv_append(qkv, positions, k_cache, v_cache, *, q_heads, kv_heads, theta=500000.0):
+    """rope() on the q and k heads of a fused QKV activation [B, Hq + 2 Hkv, D] and kv_append() of
+    its k and v heads, in one launch."""
+    _require(qkv.dtype == torch.bfloat16 and qkv.is_cuda and qkv.dim() == 3
+             and qkv.shape[1] == q_heads + 2 * kv_heads, "qkv must be BF16 [B, Hq + 2 Hkv, D]")
+    _require(qkv.stride(2) == 1 and qkv.stride(1) == qkv.shape[2], "qkv heads must be dense")
+    _require(k_cache.is_contiguous() and v_cache.is_contiguous() and k_cache.shape == v_cache.shape
+             and k_cache.shape[2:] == (kv_heads, qkv.shape[2]), "caches must be [B, C, Hkv, D]")
+    _native.context(qkv.device).call(
+        "rope_kv_append", qkv.shape[0], q_heads, kv_heads, qkv.shape[2], qkv.stride(0),
+        ct.c_float(theta), _pointer(positions), _pointer(qkv), k_cache.shape[1], _pointer(k_cache),
+        _pointer(v_cache),
+    )
+    return qkv
+
+
 def decoder_layer_decode(hidden, residual, weights, k_cache, v_cache, positions, lengths, *,
                          q_heads, kv_heads, head_dim=128, epsilon=1e-5, theta=500000.0):
     """One Llama-shaped decoder layer for one new token per sequence.
 
-    residual-add + RMSNorm -> fused QKV linear -> RoPE on q and k -> cache append -> GQA decode
+    residual-add + RMSNorm -> fused QKV linear -> RoPE on q and k with cache append -> GQA decode
     attention -> o-proj -> residual-add + RMSNorm -> SwiGLU MLP. Returns (mlp output, residual).
     `weights` holds input_norm, qkv [ (Hq+2Hkv)*D, hidden ], o, post_norm, gate, up, down.
     `positions` (int32 [batch]) is the cache slot the new token is written to and rotated for;
@@ -339,9 +355,7 @@ def decoder_layer_decode(hidden, residual, weights, k_cache, v_cache, positions,
     batch = hidden.shape[0]
     residual, normed = add_rms_norm(hidden, residual, weights["input_norm"], epsilon)
     qkv = linear(normed, weights["qkv"]).view(batch, q_heads + 2 * kv_heads, head_dim)
-    rope(qkv[:, : q_heads + kv_heads], positions, theta)
-    kv_append(qkv[:, q_heads : q_heads + kv_heads], qkv[:, q_heads + kv_heads :], k_cache, v_cache,
-              positions)
+    rope_kv_append(qkv, positions, k_cache, v_cache, q_heads=q_heads, kv_heads=kv_heads, theta=theta)
     attended = gqa_decode_attention(qkv[:, :q_heads], k_cache, v_cache, lengths)
     projected = linear(attended.view(batch, q_heads * head_dim), weights["o"])
     residual, normed = add_rms_norm(projected, residual, weights["post_norm"], epsilon)

@@ -660,6 +660,27 @@ extern "C" int camblas_cuda_kv_append(camblas_cuda_context *context, int batch, 
     });
 }
 
+extern "C" int camblas_cuda_rope_kv_append(camblas_cuda_context *context, int batch, int q_heads,
+                                           int kv_heads, int dim, int token_stride, float theta,
+                                           const int32_t *positions, void *qkv, int context_length,
+                                           void *k_cache, void *v_cache)
+{
+    return execute(context, [&] {
+        if (batch < 0 || q_heads < 1 || kv_heads < 1 || dim < 2 || dim % 2 || context_length < 1 ||
+            token_stride < (q_heads + 2 * kv_heads) * dim || !std::isfinite(theta) || theta <= 0)
+            return fail(context, "invalid rotary cache append arguments", 1);
+        if (!batch)
+            return 0;
+        if (!positions || !qkv || !k_cache || !v_cache || k_cache == v_cache || !aligned(qkv, 2) ||
+            !aligned(k_cache, 2) || !aligned(v_cache, 2) || !aligned(positions, 4))
+            return fail(context, "invalid rotary cache append buffers", 1);
+        hipError_t error =
+            launch_rope_kv_append(context->stream, batch, q_heads, kv_heads, dim, token_stride,
+                                  theta, positions, qkv, context_length, k_cache, v_cache);
+        return error == hipSuccess ? 0 : fail(context, "rotary cache append", error);
+    });
+}
+
 extern "C" int camblas_cuda_gqa_decode_attention(camblas_cuda_context *context, int batch,
                                                  int q_heads, int kv_heads, int dim,
                                                  int context_length, const int32_t *lengths,

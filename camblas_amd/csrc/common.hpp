@@ -130,6 +130,9 @@ hipError_t launch_kv_append(hipStream_t stream, int batch, int kv_heads, int dim
                             const int32_t *positions, const void *k_new, const void *v_new,
                             int token_stride, void *k_cache, void *v_cache);
 hipError_t launch_copy_probe(hipStream_t stream, size_t bytes, const void *source, void *destination);
+hipError_t launch_rope_kv_append(hipStream_t stream, int batch, int q_heads, int kv_heads, int dim,
+                                 int token_stride, float theta, const int32_t *positions, void *qkv,
+                                 int context_length, void *k_cache, void *v_cache);
 hipError_t launch_rope(hipStream_t stream, int tokens, int heads, int dim, int token_stride,
                        float theta, const int32_t *positions, void *x);
 size_t gqa_decode_scratch_bytes(int batch, int q_heads, int dim, int context_length, int *splits);

@@ -240,6 +240,17 @@ __global__ void rms_scale_kernel(size_t count, int width, float epsilon, const T
 // ---------------------------------------------------------------- rotary embedding
 // Rotate-half pairing (i, i + dim/2), angle = position * theta^(-2i/dim), FP32 sin/cos, one BF16
 // rounding per element. One thread per (token, head, i).
+__device__ __forceinline__ void rotate_pair(float position, int i, int dim, float theta, float lo,
+                                            float hi, unsigned short &out_lo, unsigned short &out_hi)
+{
+    float frequency = exp2f(-2.f * float(i) / float(dim) * log2f(theta));
+    float angle = position * frequency;
+    float s, c;
+    sincosf(angle, &s, &c);
+    out_lo = float_to_bf16_bits(lo * c - hi * s);
+    out_hi = float_to_bf16_bits(hi * c + lo * s);
+}
+
 __global__ void rope_kernel(int tokens, int heads, int dim, int token_stride, float theta,
                             const int32_t *positions, unsigned short *x)
 {
@@ -251,14 +262,47 @@ __global__ void rope_kernel(int tokens, int heads, int dim, int token_stride, fl
     int i = int(index % half);
     int head = int((index / half) % heads);
     int token = int(index / (size_t(half) * heads));
-    float frequency = exp2f(-2.f * float(i) / float(dim) * log2f(theta));
-    float angle = float(positions[token]) * frequency;
-    float s, c;
-    sincosf(angle, &s, &c);
     unsigned short *v = x + size_t(token) * token_stride + size_t(head) * dim;
-    float lo = bf16_bits_to_float(v[i]), hi = bf16_bits_to_float(v[i + half]);
-    v[i] = float_to_bf16_bits(lo * c - hi * s);
-    v[i + half] = float_to_bf16_bits(hi * c + lo * s);
+    rotate_pair(float(positions[token]), i, dim, theta, bf16_bits_to_float(v[i]),
+                bf16_bits_to_float(v[i + half]), v[i], v[i + half]);
+}
+
+// Decode-step form of the two kernels above and below in one launch: a fused QKV activation row
+// [q heads | k heads | v heads] per sequence; q and k heads are rotated in place, the rotated k
+// heads and the v heads are also written to the caches at positions[b] (skipped when outside the
+// cache). One thread per (sequence, head, i); same arithmetic as rope_kernel, bit for bit.
+__global__ void rope_kv_append_kernel(int batch, int q_heads, int kv_heads, int dim,
+                                      int token_stride, float theta, const int32_t *positions,
+                                      unsigned short *qkv, int context_length,
+                                      unsigned short *k_cache, unsigned short *v_cache)
+{
+    const int half = dim / 2, heads = q_heads + 2 * kv_heads;
+    size_t index = size_t(blockIdx.x) * blockDim.x + threadIdx.x;
+    if (index >= size_t(batch) * heads * half)
+        return;
+    const int i = int(index % half);
+    const int head = int((index / half) % heads);
+    const int b = int(index / (size_t(half) * heads));
+    const int position = positions[b];
+    const bool cached = position >= 0 && position < context_length;
+    unsigned short *v = qkv + size_t(b) * token_stride + size_t(head) * dim;
+    unsigned short lo = v[i], hi = v[i + half];
+    unsigned short *cache = nullptr;
+    if (head < q_heads + kv_heads) {
+        rotate_pair(float(position), i, dim, theta, bf16_bits_to_float(lo), bf16_bits_to_float(hi),
+                    lo, hi);
+        v[i] = lo;
+        v[i + half] = hi;
+        if (head >= q_heads)
+            cache = k_cache + ((size_t(b) * context_length + position) * kv_heads + (head - q_heads)) * dim;
+    } else {
+        cache = v_cache + ((size_t(b) * context_length + position) * kv_heads +
+                           (head - q_heads - kv_heads)) * dim;
+    }
+    if (cache && cached) {
+        cache[i] = lo;
+        cache[i + half] = hi;
+    }
 }
 
 // Plain 16-byte-per-thread copy: the known-traffic kernel used to calibrate the HBM byte counters.
@@ -421,6 +465,18 @@ hipError_t launch_copy_probe(hipStream_t stream, size_t bytes, const void *sourc
 {
     copy_probe_kernel<<<2048, 256, 0, stream>>>(bytes / 16, static_cast<const u32x4_t *>(source),
                                                 static_cast<u32x4_t *>(destination));
+    return launch_status();
+}
+
+hipError_t launch_rope_kv_append(hipStream_t stream, int batch, int q_heads, int kv_heads, int dim,
+                                 int token_stride, float theta, const int32_t *positions, void *qkv,
+                                 int context_length, void *k_cache, void *v_cache)
+{
+    size_t count = size_t(batch) * (q_heads + 2 * kv_heads) * (dim / 2);
+    rope_kv_append_kernel<<<unsigned((count + 255) / 256), 256, 0, stream>>>(
+        batch, q_heads, kv_heads, dim, token_stride, theta, positions,
+        static_cast<unsigned short *>(qkv), context_length, static_cast<unsigned short *>(k_cache),
+        static_cast<unsigned short *>(v_cache));
     return launch_status();
 }
 

@@ -172,6 +172,12 @@ int camblas_cuda_rope(camblas_cuda_context *context, int tokens, int heads, int 
 int camblas_cuda_kv_append(camblas_cuda_context *context, int batch, int kv_heads, int dim,
                            int context_length, const int32_t *positions, const void *k_new,
                            const void *v_new, int token_stride, void *k_cache, void *v_cache);
+/* extension (no reference counterpart). camblas_cuda_rope on the q and k heads of a fused QKV
+ * activation [batch, (q_heads + 2*kv_heads)*dim] (row stride token_stride) followed by
+ * camblas_cuda_kv_append of its k and v heads, in one launch and with the same results. */
+int camblas_cuda_rope_kv_append(camblas_cuda_context *context, int batch, int q_heads, int kv_heads,
+                                int dim, int token_stride, float theta, const int32_t *positions,
+                                void *qkv_bf16, int context_length, void *k_cache, void *v_cache);
 /* extension. Grouped-query decode attention, one query per sequence: q [batch, q_heads, dim]
  * (token stride q_stride elements), K/V caches [batch, context, kv_heads, dim] BF16, lengths int32
  * [batch] or NULL (= context), out [batch, q_heads, dim] BF16. dim must be 128, q_heads a

@@ -179,3 +179,26 @@ def test_gqa_decode_attention_empty_and_partial_partitions(device):
     assert not got[0].any()
     wanted = oracle.bf16_to_f32(want)[1:]
     assert (np.abs(bf16_values(out)[1:] - wanted) <= 0.01 * np.abs(wanted) + 2e-3).all()
+
+
+def test_rope_kv_append_equals_rope_then_append(device):
+    # the fused launch must give bit-identical activations and caches, including a sequence whose
+    # position lies outside the cache (rotated, not written)
+    batch, q_heads, kv_heads, dim, context = 4, 6, 2, 128, 40
+    qkv = oracle.fill_normal_bf16(50, (batch, q_heads + 2 * kv_heads, dim))
+    k_cache = oracle.fill_normal_bf16(51, (batch, context, kv_heads, dim))
+    v_cache = oracle.fill_normal_bf16(52, (batch, context, kv_heads, dim))
+    positions = torch.tensor([0, 39, 17, 40], dtype=torch.int32, device=device)
+    fused, kf, vf = (to_device_bf16(t, device) for t in (qkv, k_cache, v_cache))
+    _kernels.rope_kv_append(fused, positions, kf, vf, q_heads=q_heads, kv_heads=kv_heads)
+    split, ks, vs = (to_device_bf16(t, device) for t in (qkv, k_cache, v_cache))
+    _kernels.rope(split[:, : q_heads + kv_heads], positions)
+    _kernels.kv_append(split[:, q_heads : q_heads + kv_heads], split[:, q_heads + kv_heads :], ks, vs,
+                       positions)
+    torch.cuda.synchronize()
+    assert np.array_equal(from_device_bf16(fused), from_device_bf16(split))
+    assert np.array_equal(from_device_bf16(kf), from_device_bf16(ks))
+    assert np.array_equal(from_device_bf16(vf), from_device_bf16(vs))
+    assert np.array_equal(from_device_bf16(kf)[3], k_cache[3])  # position 40 is outside the cache
+    want = oracle.rope(qkv[:, : q_heads + kv_heads], positions.cpu().numpy(), 5e5)
+    assert rel_frobenius(bf16_values(fused[:, : q_heads + kv_heads]), oracle.bf16_to_f32(want)) <= 1e-2
