@@ -245,8 +245,9 @@ def profile_only(args, torch, _kernels, _native, device, normal, weights, inputs
                         ct.c_void_p(target.data_ptr()))
     elif args.only.startswith("fp8m"):
         tokens, features, inner = int(args.only[4:]), 18432, 7168
-        w = torch.randint(0, 0x7E, (features, inner), device=device, dtype=torch.uint8)
-        w = w.view(torch.float8_e4m3fn)
+        rotate = 3 if tokens <= 256 else 1
+        copies = [torch.randint(0, 0x7E, (features, inner), device=device, dtype=torch.uint8)
+                  .view(torch.float8_e4m3fn) for _ in range(rotate)]
         w_scale = torch.rand((features // 128, inner // 128), device=device) * 0.1 + 1e-4
         a = torch.randint(0, 0x7E, (tokens, inner), device=device, dtype=torch.uint8)
         a = a.view(torch.float8_e4m3fn)
@@ -254,7 +255,7 @@ def profile_only(args, torch, _kernels, _native, device, normal, weights, inputs
         out = torch.empty((tokens, features), dtype=torch.bfloat16, device=device)
 
         def launch(i):
-            _kernels.fp8_block_matmul(a, a_scale, w, w_scale, out=out)
+            _kernels.fp8_block_matmul(a, a_scale, copies[i % rotate], w_scale, out=out)
     elif args.only in ("attention", "layer"):
         layer, attention = layer_step(torch, _kernels, device, normal)
         launch = (lambda i: layer()) if args.only == "layer" else (lambda i: attention())
@@ -290,6 +291,10 @@ def layer_step(torch, _kernels, device, normal):
     positions = torch.full((batch,), context - 1, dtype=torch.int32, device=device)
     lengths = positions + 1
     q = normal((batch, q_heads, dim))
+    # the attention alone is timed over three rotating caches (805 MB) so that it reads HBM
+    caches = [(k_cache, v_cache)] + [(normal((batch, context, kv_heads, dim)),
+                                      normal((batch, context, kv_heads, dim))) for _ in range(2)]
+    turn = [0]
 
     def step():
         return _kernels.decoder_layer_decode(
@@ -297,7 +302,8 @@ def layer_step(torch, _kernels, device, normal):
             kv_heads=kv_heads, head_dim=dim)
 
     def attention():
-        return _kernels.gqa_decode_attention(q, k_cache, v_cache, lengths)
+        turn[0] = (turn[0] + 1) % 3
+        return _kernels.gqa_decode_attention(q, caches[turn[0]][0], caches[turn[0]][1], lengths)
 
     return step, attention
 
@@ -322,10 +328,11 @@ def extras(torch, _kernels, _native, device, normal):
         "note": "includes the bias expand+clone copy, as in the reference binding",
     }
     del x, w, y, c
-    # FP8 block-scaled linear
+    # FP8 block-scaled linear; the decode sizes rotate three weight copies (396 MB) so that the
+    # weights come from HBM rather than from the 256 MB last-level cache
     outputs, inner = 18432, 7168
-    w = torch.randint(0, 0x7E, (outputs, inner), device=device, dtype=torch.uint8)
-    w = w.view(torch.float8_e4m3fn)
+    copies = [torch.randint(0, 0x7E, (outputs, inner), device=device, dtype=torch.uint8)
+              .view(torch.float8_e4m3fn) for _ in range(3)]
     w_scale = torch.rand((outputs // 128, inner // 128), device=device) * 0.1 + 1e-4
     fp8 = {}
     for tokens in (1, 16, 256, 4096):
@@ -333,8 +340,10 @@ def extras(torch, _kernels, _native, device, normal):
         a = a.view(torch.float8_e4m3fn)
         a_scale = torch.rand((tokens, inner // 128), device=device) * 0.1 + 1e-4
         out = torch.empty((tokens, outputs), dtype=torch.bfloat16, device=device)
+        rotate = 3 if tokens <= 256 else 1
         seconds = event_time(
-            torch, lambda i: _kernels.fp8_block_matmul(a, a_scale, w, w_scale, out=out), 10, 20)
+            torch, lambda i: _kernels.fp8_block_matmul(a, a_scale, copies[i % rotate], w_scale,
+                                                       out=out), 10, 20)
         flops = 2.0 * tokens * outputs * inner
         traffic = outputs * inner + w_scale.numel() * 4 + tokens * (inner + inner // 128 * 4 + outputs * 2)
         fp8[str(tokens)] = {
@@ -343,7 +352,7 @@ def extras(torch, _kernels, _native, device, normal):
             "gbps": round(traffic / seconds / 1e9, 1), "frac_of_8TBs": round(traffic / seconds / HBM_PEAK, 4),
         }
     found["fp8_block_linear_18432x7168"] = fp8
-    del w, w_scale
+    del copies, w_scale
     # FP32 SGEMM 2048^3 (plumbing)
     size = 2048
     a32 = torch.rand((size, size), device=device) * 2 - 1

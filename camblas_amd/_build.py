@@ -30,6 +30,7 @@ CORE_SOURCES = (
     "bgemm_dma.hip",
     "fp8_block.hip",
     "fp8_dma.hip",
+    "fp8_stream.hip",
     "fusion.hip",
     "attention_decode.hip",
 )

@@ -539,8 +539,13 @@ extern "C" int camblas_cuda_fp8_block_matmul(camblas_cuda_context *context, int 
         if (plan.family == FAMILY_FP8_DMA && !aligned(out, 8))
             plan = Plan{FAMILY_FP8_BLOCK, 0, 1, 4};
         if (context->override_kernel >= 0) {
-            // diagnostics: 0.. register-staged variants (with split-K), 20.. direct-to-LDS variants
-            if (context->override_kernel >= 20) {
+            // diagnostics: 0.. register-staged variants (with split-K), 20.. direct-to-LDS variants,
+            // 100 + 10*row_tiles + token_tiles the streaming kernel
+            if (context->override_kernel >= 100) {
+                plan.family = FAMILY_FP8_STREAM;
+                plan.kernel = context->override_kernel - 100;
+                plan.split_k = 1;
+            } else if (context->override_kernel >= 20) {
                 plan.family = FAMILY_FP8_DMA;
                 plan.kernel = context->override_kernel - 20;
                 plan.split_k = 1;
@@ -549,6 +554,12 @@ extern "C" int camblas_cuda_fp8_block_matmul(camblas_cuda_context *context, int 
                 plan.kernel = context->override_kernel;
                 plan.split_k = context->override_split > 0 ? context->override_split : 1;
             }
+        }
+        if (plan.family == FAMILY_FP8_STREAM) {
+            context->counts[plan.counter]++;
+            hipError_t error = launch_fp8_stream(context->stream, plan.kernel / 10, plan.kernel % 10,
+                                                 rows, outputs, inner, a, a_scale, w, w_scale, out);
+            return error == hipSuccess ? 0 : fail(context, "FP8 block-scaled streaming GEMV", error);
         }
         if (plan.family == FAMILY_FP8_DMA) {
             context->counts[plan.counter]++;

@@ -84,8 +84,10 @@ __global__ __launch_bounds__(WAVES * 64) void gqa_partition_kernel(
             for (int e = 0; e < 8; ++e) {
                 int position = 32 * u + 16 * (e / 4) + 4 * j + e % 4;
                 position = position < count ? position : count - 1;
-                v_rows[u][e] =
-                    *reinterpret_cast<const u32x4_t *>(v_base + size_t(position) * row_stride + 8 * m);
+                // a V row is consumed whole by one load (16 lanes x 16 bytes) and read once: it
+                // bypasses cache allocation; a K row is covered by four loads and stays cacheable
+                v_rows[u][e] = __builtin_nontemporal_load(reinterpret_cast<const u32x4_t *>(
+                    v_base + size_t(position) * row_stride + 8 * m));
             }
 
         // ---- scores: register r of tile t is position 16t + 4j + r, head m

@@ -47,7 +47,8 @@ enum KernelFamily {
     FAMILY_FP8_BLOCK = 3,
     FAMILY_STREAM = 4, // BF16 'T','N' with few tokens: weight-streaming kernel, one pass over W
     FAMILY_DMA = 5,    // BF16 'T','N' prefill: large MFMA tiles fed by direct global->LDS loads
-    FAMILY_FP8_DMA = 6 // FP8 block-scaled prefill: the same structure with one scale group per step
+    FAMILY_FP8_DMA = 6, // FP8 block-scaled prefill: the same structure with one scale group per step
+    FAMILY_FP8_STREAM = 7 // FP8 block-scaled decode: weight-streaming kernel (10*row_tiles + token_tiles)
 };
 
 struct Plan {
@@ -114,6 +115,10 @@ hipError_t launch_fp8_block(hipStream_t stream, int variant, int split_k, int ro
 hipError_t launch_fp8_dma(hipStream_t stream, int variant, int rows, int outputs, int inner,
                           const void *a, const float *a_scale, const void *w, const float *w_scale,
                           void *out);
+// row_tiles 1..8 (16 weight rows each), token_tiles 1, 2 or 4 (16 tokens each).
+hipError_t launch_fp8_stream(hipStream_t stream, int row_tiles, int token_tiles, int rows, int outputs,
+                             int inner, const void *a, const float *a_scale, const void *w,
+                             const float *w_scale, void *out);
 hipError_t launch_fp8_quantise(hipStream_t stream, int rows, int inner, const void *x, void *q,
                                float *scale);
 hipError_t launch_silu_multiply(hipStream_t stream, int dtype, uint64_t count, const void *gate,

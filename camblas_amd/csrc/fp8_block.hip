@@ -31,6 +31,17 @@ struct Fp8Params {
 
 __device__ __forceinline__ int swizzle8(int row) { return ((row >> 1) & 7) ^ ((row & 1) << 2); }
 
+// Weight bytes: a tile with at most 32 tokens belongs to a decode-sized call whose weights are read
+// exactly once, so they are loaded non-temporally (they do not displace the activations and
+// scales in the caches); larger token tiles re-read the weights through L2 and load them normally.
+template <bool STREAMED> __device__ __forceinline__ u32x4_t weight_load(const unsigned char *address)
+{
+    if constexpr (STREAMED)
+        return __builtin_nontemporal_load(reinterpret_cast<const u32x4_t *>(address));
+    else
+        return *reinterpret_cast<const u32x4_t *>(address);
+}
+
 template <int BN, int BM, int WN, int WM>
 __global__ __launch_bounds__(WN *WM * 64) void fp8_block_kernel(Fp8Params p)
 {
@@ -109,7 +120,7 @@ __global__ __launch_bounds__(WN *WM * 64) void fp8_block_kernel(Fp8Params p)
         const size_t k0 = size_t(g) * BK;
 #pragma unroll
         for (int it = 0; it < A_ITERS; ++it)
-            a_reg[it] = *reinterpret_cast<const u32x4_t *>(a_base + k0 + a_off[it]);
+            a_reg[it] = weight_load<BM <= 32>(a_base + k0 + a_off[it]);
 #pragma unroll
         for (int it = 0; it < B_ITERS; ++it)
             b_reg[it] = *reinterpret_cast<const u32x4_t *>(b_base + k0 + b_off[it]);

@@ -1,0 +1,281 @@
+// Bandwidth-bound FP8 E4M3fn block-scaled decode linear (few tokens): out[M,N] =
+// sum_g (a[M,g] . w[N,g]) * a_scale[M,g] * w_scale[N/128,g], 1x128 activation groups, 128x128
+// weight blocks, FP32 scales, BF16 out. Rule: ref camblas/_hopper.py:118-126 and :168-182 (which
+// covers one token); here up to 64 tokens share one pass over the weights.
+//
+// The whole cost is reading W once, so the kernel is the FP8 sibling of the BF16 weight-streaming
+// kernel: a workgroup owns 16*NT consecutive weight rows for the whole K extent, no split-K pass
+// and no scratch. One K group (128 bytes per row) is exactly one v_mfma_scale_f32_16x16x128_f8f6f4
+// per 16x16 output tile. The four wavefronts take groups g = 4s + wave and never synchronise in
+// the loop: a wavefront loads its group of a 16-row tile with two 128-bit loads per lane in which
+// eight lanes cover one whole 128-byte line (loading straight in the MFMA operand layout would
+// touch every line from eight different quarter-wave passes, which the L1 tag pipeline cannot
+// sustain), transposes it to the operand layout (row lane%16, 32 bytes lane/16) through a private,
+// XOR-swizzled 2 KB LDS patch, which needs no barrier because LDS operations of one wavefront
+// execute in order, and multiplies. Each wavefront keeps the ascending fma chain
+// acc = fma(dot_g, a_s * w_s, acc) over its own groups (hardware block scales are set to one: the
+// scales here are FP32), and the four partial sums are added in wavefront order at the end, so
+// results do not depend on scheduling. Weight loads are non-temporal (read once); two or three
+// groups are in flight per wavefront.
+#include "common.hpp"
+#include "device.hpp"
+
+namespace camblas_hip
+{
+namespace
+{
+struct Fp8StreamParams {
+    const unsigned char *w;
+    const unsigned char *a;
+    const float *w_scale;
+    const float *a_scale;
+    unsigned short *out;
+    int n, m, k, groups, scale_blocks;
+};
+
+constexpr int WAVES = 4, GROUP = 128;
+constexpr int UNIT = 0x7f7f7f7f; // E8M0 exponent 127 = scale 1.0 in every byte
+
+// NT, MT: 16-row weight tiles and 16-token tiles per workgroup.
+template <int NT, int MT>
+__global__ __launch_bounds__(WAVES * 64) void fp8_stream_kernel(Fp8StreamParams p)
+{
+    // groups in flight per wavefront: three while the operand registers allow it
+    constexpr int DEPTH = NT + MT <= 6 ? 3 : 2;
+    constexpr int TILES = NT + MT; // weight tiles, then token tiles
+    __shared__ __attribute__((aligned(16))) u32x4_t patch[WAVES][TILES][128];
+    __shared__ __attribute__((aligned(16))) f32x4_t combine[NT * MT * 64];
+    const int thread = threadIdx.x, lane = thread % 64, wave = thread / 64;
+    const int row = lane % 16, chunk = lane / 16; // operand row / token, 32-byte chunk of the group
+    const int load_row = lane / 8, piece = lane % 8; // load layout: 8 lanes per 128-byte line
+    const int n0 = blockIdx.x * (NT * 16), m0 = blockIdx.y * (MT * 16);
+    const int steps = (p.groups + WAVES - 1) / WAVES; // groups per wavefront, padded
+
+    // tile t < NT: weight rows n0 + 16 t ..; tile NT + j: tokens m0 + 16 j ..; half h: rows 8h ..
+    const unsigned char *source[TILES][2];
+    const float *ws_ptr[NT], *as_ptr[MT];
+#pragma unroll
+    for (int h = 0; h < 2; ++h) {
+#pragma unroll
+        for (int i = 0; i < NT; ++i) {
+            int n = n0 + i * 16 + h * 8 + load_row;
+            n = n < p.n ? n : p.n - 1;
+            source[i][h] = p.w + size_t(n) * p.k + piece * 16;
+        }
+#pragma unroll
+        for (int j = 0; j < MT; ++j) {
+            int m = m0 + j * 16 + h * 8 + load_row;
+            m = m < p.m ? m : p.m - 1;
+            source[NT + j][h] = p.a + size_t(m) * p.k + piece * 16;
+        }
+    }
+#pragma unroll
+    for (int i = 0; i < NT; ++i) {
+        int block = (n0 + i * 16) / 128;
+        block = block < p.scale_blocks ? block : p.scale_blocks - 1;
+        ws_ptr[i] = p.w_scale + size_t(block) * p.groups;
+    }
+#pragma unroll
+    for (int j = 0; j < MT; ++j) {
+        int m = m0 + j * 16 + row;
+        m = m < p.m ? m : p.m - 1;
+        as_ptr[j] = p.a_scale + size_t(m) * p.groups;
+    }
+    // LDS patch of one tile: 16 rows x 8 pieces of 16 bytes, piece index XORed with row bits 1..3,
+    // which makes both the line-shaped stores and the operand-shaped loads conflict-free
+    auto slot = [](int r, int q) { return r * 8 + (q ^ ((r >> 1) & 7)); };
+    const int store_slot[2] = {slot(load_row, piece), slot(load_row + 8, piece)};
+    const int read_slot[2] = {slot(row, 2 * chunk), slot(row, 2 * chunk + 1)};
+
+    // Workgroups start at different groups and wrap around, which spreads the row-pitch-strided
+    // requests of the chip over all HBM channels. Steps past the end (the padding of the last
+    // round of four groups, and the DEPTH prefetches beyond the loop) re-read the last group and
+    // are given a zero scale.
+    const int start = int(blockIdx.x % unsigned(steps));
+    auto group_of = [&](int step) {
+        int rotated = (step < steps ? step : steps - 1) + start;
+        rotated = rotated < steps ? rotated : rotated - steps;
+        return rotated * WAVES + wave;
+    };
+    u32x4_t raw[DEPTH][TILES][2];
+    float ws_reg[DEPTH][NT], as_reg[DEPTH][MT], live_reg[DEPTH];
+    // Nothing in a fetch may use a loaded value (that would wait for the loads just issued): a dead
+    // step is remembered as a zero factor and applied to the scale when the group is multiplied.
+    auto fetch = [&](int step, u32x4_t(&data)[TILES][2], float(&ws)[NT], float(&as)[MT],
+                     float &live) {
+        int g = group_of(step);
+        live = step < steps && g < p.groups ? 1.f : 0.f;
+        g = g < p.groups ? g : p.groups - 1;
+        const size_t offset = size_t(g) * GROUP;
+#pragma unroll
+        for (int t = 0; t < TILES; ++t)
+#pragma unroll
+            for (int h = 0; h < 2; ++h) {
+                const u32x4_t *address = reinterpret_cast<const u32x4_t *>(source[t][h] + offset);
+                data[t][h] = t < NT ? __builtin_nontemporal_load(address) : *address;
+            }
+#pragma unroll
+        for (int i = 0; i < NT; ++i)
+            ws[i] = ws_ptr[i][g];
+#pragma unroll
+        for (int j = 0; j < MT; ++j)
+            as[j] = as_ptr[j][g];
+    };
+
+    f32x4_t acc[NT][MT];
+#pragma unroll
+    for (int i = 0; i < NT; ++i)
+#pragma unroll
+        for (int j = 0; j < MT; ++j)
+            acc[i][j] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+    auto multiply = [&](const u32x4_t(&data)[TILES][2], const float(&ws)[NT], const float(&as)[MT],
+                        float live) {
+        u32x4_t *mine = &patch[wave][0][0];
+#pragma unroll
+        for (int t = 0; t < TILES; ++t) {
+            mine[t * 128 + store_slot[0]] = data[t][0];
+            mine[t * 128 + store_slot[1]] = data[t][1];
+        }
+        // other lanes' stores are read below: keep the compiler from moving the loads up (the
+        // hardware executes one wavefront's LDS operations in order)
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+        i32x8_t operand[TILES];
+#pragma unroll
+        for (int t = 0; t < TILES; ++t) {
+            u32x4_t lo = mine[t * 128 + read_slot[0]], hi = mine[t * 128 + read_slot[1]];
+            operand[t] = i32x8_t{int(lo[0]), int(lo[1]), int(lo[2]), int(lo[3]),
+                                 int(hi[0]), int(hi[1]), int(hi[2]), int(hi[3])};
+        }
+#pragma unroll
+        for (int i = 0; i < NT; ++i)
+#pragma unroll
+            for (int j = 0; j < MT; ++j) {
+                f32x4_t dot = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(
+                    operand[i], operand[NT + j], f32x4_t{0.f, 0.f, 0.f, 0.f}, 0, 0, 0, UNIT, 0, UNIT);
+                const float scale = __fmul_rn(as[j], ws[i]) * live;
+#pragma unroll
+                for (int r = 0; r < 4; ++r)
+                    acc[i][j][r] = fmaf(dot[r], scale, acc[i][j][r]);
+            }
+        // the next group's stores must not overtake these loads in the compiler either
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+    };
+
+    // sched_barrier(0) keeps the fetches of different steps apart so that the wait before a
+    // multiply covers only the oldest of the groups in flight
+#pragma unroll
+    for (int d = 0; d < DEPTH; ++d) {
+        fetch(d, raw[d], ws_reg[d], as_reg[d], live_reg[d]);
+        __builtin_amdgcn_sched_barrier(0);
+    }
+    for (int step = 0; step < steps; step += DEPTH) {
+#pragma unroll
+        for (int d = 0; d < DEPTH; ++d) {
+            __builtin_amdgcn_sched_barrier(0);
+            multiply(raw[d], ws_reg[d], as_reg[d], live_reg[d]);
+            __builtin_amdgcn_sched_barrier(0);
+            fetch(step + d + DEPTH, raw[d], ws_reg[d], as_reg[d], live_reg[d]);
+        }
+    }
+    __syncthreads();
+
+    // ---- add the four wavefronts' partial sums in wavefront order through LDS
+#pragma unroll
+    for (int w = 0; w < WAVES; ++w) {
+        if (wave == w) {
+#pragma unroll
+            for (int i = 0; i < NT; ++i)
+#pragma unroll
+                for (int j = 0; j < MT; ++j) {
+                    f32x4_t *slot = combine + (i * MT + j) * 64 + lane;
+                    *slot = w == 0 ? acc[i][j] : *slot + acc[i][j];
+                }
+        }
+        __syncthreads();
+    }
+    // ---- epilogue: wavefront w writes tiles w, w+4, ...; register r of lane l is feature
+    // 4*(l/16) + r and token l%16 inside the 16x16 tile
+    const bool vector_store = p.n % 4 == 0 && reinterpret_cast<uintptr_t>(p.out) % 8 == 0;
+#pragma unroll
+    for (int index = 0; index < NT * MT; ++index) {
+        if (index % WAVES != wave)
+            continue;
+        const int i = index / MT, j = index % MT;
+        const int m = m0 + j * 16 + row;
+        const int n = n0 + i * 16 + chunk * 4;
+        if (m >= p.m || n >= p.n)
+            continue;
+        f32x4_t sum = combine[index * 64 + lane];
+        unsigned short *out = p.out + size_t(m) * p.n + n;
+        if (n + 3 < p.n && vector_store) {
+            u32x2_t packed = {pack_bf16x2(sum[0], sum[1]), pack_bf16x2(sum[2], sum[3])};
+            *reinterpret_cast<u32x2_t *>(out) = packed;
+        } else {
+#pragma unroll
+            for (int e = 0; e < 4; ++e)
+                if (n + e < p.n)
+                    out[e] = float_to_bf16_bits(sum[e]);
+        }
+    }
+}
+
+template <int NT, int MT> hipError_t launch_one(hipStream_t stream, const Fp8StreamParams &p)
+{
+    // the prefetch registers grow with NT + MT: keep both groups in flight inside the register file
+    if constexpr (NT * MT > 16 || NT + MT > 10) {
+        return hipErrorInvalidValue;
+    } else {
+        dim3 grid(unsigned((p.n + NT * 16 - 1) / (NT * 16)), unsigned((p.m + MT * 16 - 1) / (MT * 16)));
+        fp8_stream_kernel<NT, MT><<<grid, WAVES * 64, 0, stream>>>(p);
+        return launch_status();
+    }
+}
+
+template <int MT> hipError_t launch_rows(hipStream_t stream, int row_tiles, const Fp8StreamParams &p)
+{
+    switch (row_tiles) {
+    case 1: return launch_one<1, MT>(stream, p);
+    case 2: return launch_one<2, MT>(stream, p);
+    case 3: return launch_one<3, MT>(stream, p);
+    case 4: return launch_one<4, MT>(stream, p);
+    case 5: return launch_one<5, MT>(stream, p);
+    case 6: return launch_one<6, MT>(stream, p);
+    case 7: return launch_one<7, MT>(stream, p);
+    case 8: return launch_one<8, MT>(stream, p);
+    default: return hipErrorInvalidValue;
+    }
+}
+} // namespace
+
+// row_tiles 1..8 (16 weight rows each), token_tiles 1, 2 or 4 (16 tokens each); a, w 16-byte
+// aligned, inner a multiple of 128.
+hipError_t launch_fp8_stream(hipStream_t stream, int row_tiles, int token_tiles, int rows, int outputs,
+                             int inner, const void *a, const float *a_scale, const void *w,
+                             const float *w_scale, void *out)
+{
+    if (inner % GROUP || inner < GROUP || rows < 1 || outputs < 1)
+        return hipErrorInvalidValue;
+    if ((rows + token_tiles * 16 - 1) / (token_tiles * 16) > 65535)
+        return hipErrorInvalidValue;
+    Fp8StreamParams p;
+    p.w = static_cast<const unsigned char *>(w);
+    p.a = static_cast<const unsigned char *>(a);
+    p.w_scale = w_scale;
+    p.a_scale = a_scale;
+    p.out = static_cast<unsigned short *>(out);
+    p.n = outputs;
+    p.m = rows;
+    p.k = inner;
+    p.groups = inner / GROUP;
+    p.scale_blocks = (outputs + 127) / 128;
+    switch (token_tiles) {
+    case 1: return launch_rows<1>(stream, row_tiles, p);
+    case 2: return launch_rows<2>(stream, row_tiles, p);
+    case 4: return launch_rows<4>(stream, row_tiles, p);
+    default: return hipErrorInvalidValue;
+    }
+}
+} // namespace camblas_hip

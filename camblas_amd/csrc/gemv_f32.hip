@@ -38,8 +38,8 @@ __global__ __launch_bounds__(WAVES * 64) void gemv_f32_kernel(int rows, int inne
         f32x4_t a0[ROWS_PER_WAVE], a1[ROWS_PER_WAVE];
 #pragma unroll
         for (int r = 0; r < ROWS_PER_WAVE; ++r) {
-            a0[r] = wv[r][index];
-            a1[r] = wv[r][index + 64];
+            a0[r] = __builtin_nontemporal_load(wv[r] + index); // W is read exactly once
+            a1[r] = __builtin_nontemporal_load(wv[r] + index + 64);
         }
 #pragma unroll
         for (int r = 0; r < ROWS_PER_WAVE; ++r)
@@ -53,7 +53,7 @@ __global__ __launch_bounds__(WAVES * 64) void gemv_f32_kernel(int rows, int inne
         f32x4_t b0 = xv[index];
 #pragma unroll
         for (int r = 0; r < ROWS_PER_WAVE; ++r) {
-            f32x4_t a0 = wv[r][index];
+            f32x4_t a0 = __builtin_nontemporal_load(wv[r] + index);
 #pragma unroll
             for (int e = 0; e < 4; ++e)
                 acc[r][0] = fmaf(a0[e], b0[e], acc[r][0]);

@@ -46,6 +46,26 @@ int stream_row_tiles(int outputs, int compute_units)
     return best;
 }
 
+// Weight rows per workgroup (in units of 16) for the FP8 streaming kernel. Several of its
+// workgroups can share a compute unit, so the time follows the busiest compute unit's share of the
+// traffic: workgroups per compute unit times the bytes one workgroup moves, the weight rows from
+// HBM plus the token tiles, which every workgroup re-reads through L2 (counted at half weight).
+int fp8_stream_row_tiles(int outputs, int token_tiles, int compute_units, int limit)
+{
+    const int tiles = ceil_div(outputs, 16);
+    int best = 1;
+    double best_cost = 1e300;
+    for (int candidate = 1; candidate <= limit; ++candidate) {
+        int groups = ceil_div(tiles, candidate);
+        double cost = double(ceil_div(groups, compute_units)) * (candidate + 0.5 * token_tiles);
+        if (cost <= best_cost + 1e-9) {
+            best_cost = cost;
+            best = candidate;
+        }
+    }
+    return best;
+}
+
 // 128-element K blocks per step of the streaming kernel, as a power of two. Workgroups with few
 // weight rows (projections with few outputs) take two blocks per step so that enough bytes are in
 // flight per compute unit; measured on 8192- and 10240-row projections, two blocks beat one by
@@ -155,7 +175,18 @@ Plan make_plan(int dtype, int algorithm, bool trans_a, bool trans_b, int m, int 
     }
     // FP8 block-scaled: rows = n (tokens), outputs = m, always K-contiguous
     plan.counter = 4;
-    if (n <= 32) {
+    if (n > 8 && n <= 64) {
+        // decode batches: one streaming pass over the weights, whole K per workgroup; the row
+        // tiles are limited by the operand registers (row_tiles * token_tiles <= 16, sum <= 10)
+        const int token_tiles = n <= 16 ? 1 : n <= 32 ? 2 : 4;
+        const int limit = std::min(16 / token_tiles, 10 - token_tiles);
+        plan.family = FAMILY_FP8_STREAM;
+        plan.kernel =
+            10 * fp8_stream_row_tiles(m, token_tiles, compute_units, std::min(8, limit)) + token_tiles;
+        return plan;
+    }
+    if (n <= 8) {
+        // a handful of tokens: small tiles with split-K put the most workgroups on the weight stream
         plan.family = FAMILY_FP8_BLOCK;
         plan.kernel = 3; // 64 x 32 tiles, split-K: the most workgroups in flight for the weight stream
         const TnVariant &v = fp8_variant(plan.kernel);
@@ -204,6 +235,10 @@ void describe_plan(const Plan &plan, int dtype, char *text, size_t bytes)
         break;
     case FAMILY_FP8_DMA:
         std::snprintf(text, bytes, "%s %s", type, fp8_dma_variant(plan.kernel).name);
+        break;
+    case FAMILY_FP8_STREAM:
+        std::snprintf(text, bytes, "%s stream rows=%d tokens=%d", type, 16 * (plan.kernel / 10),
+                      16 * (plan.kernel % 10));
         break;
     case FAMILY_DMA:
         std::snprintf(text, bytes, "%s %s", type, dma_variant(plan.kernel).name);

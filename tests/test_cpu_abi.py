@@ -78,6 +78,13 @@ def test_planner_choices_for_the_baseline_shapes():
     assert describe(0, "T", "N", 4096, 1, 4096, 4096, 4096, 4096, algorithm="lt")[0] // 1000 == 0
     assert describe(0, "T", "N", 1000, 1, 4096, 4096, 4096, 1000)[0] // 1000 == 0
     assert describe(0, "N", "N", 2048, 2048, 2048, 2048, 2048, 2048)[0] // 1000 == 0
+    # FP8: split-K tiles for a few tokens, the streaming kernel for decode batches, direct-to-LDS
+    # tiles for prefill
+    assert describe(3, "T", "N", 18432, 1, 7168, 7168, 7168, 18432)[0] // 1000 == 3
+    code, text = describe(3, "T", "N", 18432, 16, 7168, 7168, 7168, 18432)
+    assert code // 1000 == 7 and "stream rows=80 tokens=16" in text
+    assert "rows=48 tokens=64" in describe(3, "T", "N", 18432, 64, 7168, 7168, 7168, 18432)[1]
+    assert describe(3, "T", "N", 18432, 4096, 7168, 7168, 7168, 18432)[0] // 1000 == 6
     # the plan is a pure function of its arguments
     assert describe(3, "T", "N", 18432, 16, 7168, 7168, 7168, 18432) == describe(
         3, "T", "N", 18432, 16, 7168, 7168, 7168, 18432)

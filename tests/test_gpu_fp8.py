@@ -56,6 +56,28 @@ def test_random_blocks_every_variant(device, variant, split, rows):
         assert (np.abs(bf16_values(out) - wanted) <= bound).all()
 
 
+# 100 + 10*row_tiles + token_tiles: the weight-streaming decode kernel
+FP8_STREAM_CODES = [100 + 10 * rows + tokens for rows in range(1, 9) for tokens in (1, 2, 4)
+                    if rows * tokens <= 16 and rows + tokens <= 10]
+
+
+@pytest.mark.parametrize("code", FP8_STREAM_CODES)
+@pytest.mark.parametrize("rows,outputs,inner", [(1, 300, 512), (20, 258, 896), (70, 131, 1280)])
+def test_streaming_decode_variants(device, code, rows, outputs, inner):
+    # ragged weight rows (partial 16-row tile, partial 128-row scale block, output counts that are
+    # not multiples of four), token counts that underfill and span the token tiles, group counts
+    # that are not multiples of the four wavefronts; the sum order differs from the oracle's single
+    # chain (four interleaved chains), so results agree to the tolerance form, not bit for bit
+    a, a_scale = oracle.fill_fp8_blocks(300 + rows, rows, inner, 1)
+    w, w_scale = oracle.fill_fp8_blocks(301, outputs, inner, 128)
+    out = run(device, a, a_scale, w, w_scale, override=(code, 1))
+    want64 = oracle.fp8_block_matmul_f64(a, a_scale, w, w_scale)
+    assert rel_frobenius(bf16_values(out), want64) <= TOLERANCE
+    wanted = oracle.bf16_to_f32(oracle.f32_to_bf16(want64.astype(np.float32)))
+    bound = 2.0**-7 * np.abs(wanted) + 1e-4 * np.abs(want64).max()
+    assert (np.abs(bf16_values(out) - wanted) <= bound).all()
+
+
 @pytest.mark.parametrize("code", [20, 21, 22, 23, 24, 25, 26])
 @pytest.mark.parametrize("rows,outputs,inner", [(70, 300, 512), (256, 512, 128), (513, 260, 896)])
 def test_direct_lds_load_variants(device, code, rows, outputs, inner):
@@ -80,7 +102,8 @@ def test_planned_shapes(device, rows):
     assert rel_frobenius(bf16_values(out), oracle.fp8_block_matmul_f64(a, a_scale, w, w_scale)) <= TOLERANCE
 
 
-@pytest.mark.parametrize("override", [None, (0, 1), (1, 1), (2, 1), (3, 1), (20, 1), (21, 1), (22, 1), (23, 1), (24, 1), (25, 1), (26, 1)])
+@pytest.mark.parametrize("override", [None, (0, 1), (1, 1), (2, 1), (3, 1), (20, 1), (21, 1), (22, 1), (23, 1), (24, 1), (25, 1), (26, 1),
+                                      (111, 1), (152, 1), (134, 1)])
 def test_scale_indexing_is_bit_exact(device, override):
     # every product is a small integer and every scale a distinct power of two, so the FMA chain
     # is exact: any wrong (row, group) or (block, group) scale index changes the bits
