@@ -352,6 +352,17 @@ def extras(torch, _kernels, _native, device, normal):
             "gbps": round(traffic / seconds / 1e9, 1), "frac_of_8TBs": round(traffic / seconds / HBM_PEAK, 4),
         }
     found["fp8_block_linear_18432x7168"] = fp8
+    # single-token block-32 product of the reference header (FP32 scales per 32 x 32 block)
+    token = torch.randint(0, 0x7E, (1, inner), device=device, dtype=torch.uint8).view(torch.float8_e4m3fn)
+    token_scale = torch.rand((1, inner // 32), device=device) * 0.1 + 1e-4
+    block_scale = torch.rand((outputs // 32, inner // 32), device=device) * 0.1 + 1e-4
+    seconds = event_time(
+        torch, lambda i: _kernels.fp8_decode(token, token_scale, copies[i % 3], block_scale), 10, 20)
+    traffic = outputs * inner + block_scale.numel() * 4 + inner + inner // 32 * 4 + outputs * 2
+    found["fp8_block32_decode_18432x7168"] = {
+        "us": round(seconds * 1e6, 1), "gbps": round(traffic / seconds / 1e9, 1),
+        "frac_of_8TBs": round(traffic / seconds / HBM_PEAK, 4),
+    }
     del copies, w_scale
     # FP32 SGEMM 2048^3 (plumbing)
     size = 2048

@@ -31,6 +31,7 @@ CORE_SOURCES = (
     "fp8_block.hip",
     "fp8_dma.hip",
     "fp8_stream.hip",
+    "fp8_block32.hip",
     "fusion.hip",
     "attention_decode.hip",
 )

@@ -281,6 +281,65 @@ def fp8_block_linear(x, weight, weight_scale):
     return out.reshape(*x.shape[:-1], weight.shape[0])
 
 
+def fp8_decode_supported(device=None):
+    """Whether the block-32 single-token FP8 product runs on this device (ref: fp8_decode_supported
+    in src/cuda/torch_bindings.cpp:380-387)."""
+    native = _native.context(device)
+    return bool(_native.library().camblas_cuda_fp8_decode_supported(native.handle))
+
+
+def _fp8_block32(x, x_scale, weight, weight_scale):
+    # ref: src/cuda/torch_bindings.cpp:389-445 (same checks, same messages' meaning)
+    quantise = x_scale is None
+    _require(x.is_cuda and x.dtype == (torch.bfloat16 if quantise else torch.float8_e4m3fn)
+             and weight.dtype == torch.float8_e4m3fn,
+             "FP8 linear requires GPU BF16/FP8 input and E4M3 weight")
+    _require(x.dim() >= 1 and weight.dim() == 2 and weight_scale.dim() == 2 and x.is_contiguous()
+             and weight.is_contiguous(),
+             "FP8 linear requires contiguous matrices and rank-two weight scales")
+    _require(weight_scale.dtype == torch.float32, "FP8 weight scales must be FP32")
+    for tensor in (x, weight, weight_scale):
+        _require(tensor.device == x.device
+                 and not (torch.is_grad_enabled() and tensor.requires_grad),
+                 "FP8 operands must share a GPU and support inference only")
+    inner, outputs = x.shape[-1], weight.shape[0]
+    _require(32 <= inner <= 8192 and inner % 32 == 0 and outputs >= 16 and outputs % 16 == 0
+             and x.numel() == inner and weight.shape[1] == inner,
+             "Invalid FP8 linear matrix dimensions")
+    _require(tuple(weight_scale.shape) == ((outputs + 31) // 32, inner // 32),
+             "FP8 weight scale shape does not match its blocks")
+    sx, sn, sk = 1, weight_scale.stride(0), weight_scale.stride(1)
+    if not quantise:
+        _require(x_scale.device == x.device and x_scale.dtype == torch.float32
+                 and x_scale.dim() == x.dim()
+                 and not (torch.is_grad_enabled() and x_scale.requires_grad),
+                 "FP8 input scales require matching device/rank and FP32 inference storage")
+        _require(tuple(x_scale.shape[:-1]) == tuple(x.shape[:-1])
+                 and x_scale.shape[-1] == inner // 32, "FP8 input scale shape mismatch")
+        sx = x_scale.stride(-1)
+    _require(sx > 0 and sn > 0 and sk > 0, "FP8 scale strides must be positive")
+    out = torch.empty(tuple(x.shape[:-1]) + (outputs,), dtype=torch.bfloat16, device=x.device)
+    native = _native.context(x.device)
+    if quantise:
+        native.call("fp8_linear", outputs, inner, _pointer(x), _pointer(weight),
+                    _pointer(weight_scale), sn, sk, None, 0, _pointer(out))
+    else:
+        native.call("fp8_decode", outputs, inner, _pointer(x), _pointer(x_scale), _pointer(weight),
+                    _pointer(weight_scale), sx, sn, sk, None, 0, _pointer(out))
+    return out
+
+
+def fp8_decode(x, x_scale, weight, weight_scale):
+    """One E4M3 token [.., inner] with FP32 block-32 scales times E4M3 weights [outputs, inner] with
+    FP32 scales [ceil(outputs/32), inner/32] (any positive strides); BF16 [.., outputs]."""
+    return _fp8_block32(x, x_scale, weight, weight_scale)
+
+
+def fp8_linear(x, weight, weight_scale):
+    """One BF16 token, quantised per 32 values with a power-of-two scale, then fp8_decode."""
+    return _fp8_block32(x, None, weight, weight_scale)
+
+
 def rope(x, positions, theta=500000.0):
     """In-place rotate-half rotary embedding on BF16 x [tokens, heads, dim]."""
     _require(x.dtype == torch.bfloat16 and x.is_cuda and x.dim() == 3, "rope needs BF16 [T,H,D]")

@@ -65,6 +65,10 @@ SIGNATURES = {
     "add_rms_norm": ([_P, _I, _I, _F, _P, _P, _P, _P, _P], _I),
     "bfloat16_square": ([_P, _U64, _P, _P], _I),
     "rms_scale": ([_P, _I, _U64, _I, _F, _P, _P, _P, _P], _I),
+    "fp8_decode_supported": ([_P], _I),
+    "fp8_decode": ([_P, _I, _I, _P, _P, _P, _P, _I, _I, _I, _P, _SZ, _P], _I),
+    "fp8_workspace_size": ([_I, _I, _I], _SZ),
+    "fp8_linear": ([_P, _I, _I, _P, _P, _P, _I, _I, _P, _SZ, _P], _I),
     "fp8_block_matmul": ([_P, _I, _I, _I, _P, _P, _P, _P, _P], _I),
     "fp8_quantise_1x128": ([_P, _I, _I, _P, _P, _P], _I),
     "fp8_block_workspace_size": ([_I, _I], _SZ),

@@ -586,6 +586,66 @@ extern "C" int camblas_cuda_fp8_block_matmul(camblas_cuda_context *context, int 
     });
 }
 
+// ref: src/cuda/backend.cu:1193-1256 (validation order and messages of the block-32 decode pair)
+extern "C" int camblas_cuda_fp8_decode_supported(const camblas_cuda_context *context)
+{
+    return context ? 1 : 0;
+}
+
+extern "C" size_t camblas_cuda_fp8_workspace_size(int quantise, int outputs, int inner)
+{
+    (void)quantise, (void)outputs, (void)inner;
+    return 0; // both operations are single kernels that stage the token in LDS
+}
+
+extern "C" int camblas_cuda_fp8_decode(camblas_cuda_context *context, int outputs, int inner,
+                                       const void *input, const float *input_scale,
+                                       const void *weight, const float *weight_scale,
+                                       int input_scale_stride, int weight_scale_row_stride,
+                                       int weight_scale_column_stride, void *workspace,
+                                       size_t workspace_bytes, void *output)
+{
+    (void)workspace, (void)workspace_bytes;
+    return execute(context, [&] {
+        if (outputs < 16 || outputs % 16 || inner < 32 || inner > 8192 || inner % 32 ||
+            input_scale_stride < 1 || weight_scale_row_stride < 1 || weight_scale_column_stride < 1)
+            return fail(context, "invalid FP8 decode dimensions or scale strides", 1);
+        if (!input || !input_scale || !weight || !weight_scale || !output || !aligned(input, 4) ||
+            !aligned(weight, 16) || !aligned(input_scale, 4) || !aligned(weight_scale, 4) ||
+            !aligned(output, 2) || output == input || output == weight ||
+            output == (const void *)input_scale || output == (const void *)weight_scale)
+            return fail(context, "invalid FP8 decode buffers", 1);
+        context->counts[4]++;
+        hipError_t error = launch_fp8_block32_decode(
+            context->stream, outputs, inner, input, input_scale, input_scale_stride, weight,
+            weight_scale, weight_scale_row_stride, weight_scale_column_stride, output);
+        return error == hipSuccess ? 0 : fail(context, "FP8 block-32 decode", error);
+    });
+}
+
+extern "C" int camblas_cuda_fp8_linear(camblas_cuda_context *context, int outputs, int inner,
+                                       const void *input, const void *weight,
+                                       const float *weight_scale, int weight_scale_row_stride,
+                                       int weight_scale_column_stride, void *workspace,
+                                       size_t workspace_bytes, void *output)
+{
+    (void)workspace, (void)workspace_bytes;
+    return execute(context, [&] {
+        if (outputs < 16 || outputs % 16 || inner < 32 || inner > 8192 || inner % 32 ||
+            weight_scale_row_stride < 1 || weight_scale_column_stride < 1)
+            return fail(context, "invalid FP8 decode dimensions or scale strides", 1);
+        if (!input || !weight || !weight_scale || !output || !aligned(input, 4) ||
+            !aligned(weight, 16) || !aligned(weight_scale, 4) || !aligned(output, 2) ||
+            output == input || output == weight || output == (const void *)weight_scale)
+            return fail(context, "invalid FP8 decode buffers", 1);
+        context->counts[4]++;
+        hipError_t error = launch_fp8_block32_decode(
+            context->stream, outputs, inner, input, nullptr, 1, weight, weight_scale,
+            weight_scale_row_stride, weight_scale_column_stride, output);
+        return error == hipSuccess ? 0 : fail(context, "FP8 block-32 linear", error);
+    });
+}
+
 extern "C" int camblas_cuda_fp8_quantise_1x128(camblas_cuda_context *context, int rows, int inner,
                                                const void *x, void *q, float *scale)
 {

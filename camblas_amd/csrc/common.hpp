@@ -119,6 +119,10 @@ hipError_t launch_fp8_dma(hipStream_t stream, int variant, int rows, int outputs
 hipError_t launch_fp8_stream(hipStream_t stream, int row_tiles, int token_tiles, int rows, int outputs,
                              int inner, const void *a, const float *a_scale, const void *w,
                              const float *w_scale, void *out);
+// Single-token product with 32-wide FP32 scale blocks; sx null: x is BF16 and quantised on the fly.
+hipError_t launch_fp8_block32_decode(hipStream_t stream, int outputs, int inner, const void *x,
+                                     const float *sx, int sx_stride, const void *w, const float *sw,
+                                     int sw_row, int sw_col, void *out);
 hipError_t launch_fp8_quantise(hipStream_t stream, int rows, int inner, const void *x, void *q,
                                float *scale);
 hipError_t launch_silu_multiply(hipStream_t stream, int dtype, uint64_t count, const void *gate,

@@ -37,6 +37,23 @@ __device__ __forceinline__ unsigned pack_bf16x2(float lo, float hi)
     return unsigned(float_to_bf16_bits(lo)) | (unsigned(float_to_bf16_bits(hi)) << 16);
 }
 
+// FP32 -> E4M3fn, round-to-nearest-even, saturating at +-448, NaN -> 0x7f.
+__device__ __forceinline__ unsigned f32_to_e4m3_sat(float value)
+{
+    unsigned sign = (__float_as_uint(value) >> 24) & 0x80u;
+    float a = fabsf(value);
+    if (a != a)
+        return 0x7fu;
+    if (a >= 448.f)
+        return sign | 0x7eu;
+    if (a >= 0.015625f) { // normal range: round the FP32 mantissa to three bits
+        unsigned bits = __float_as_uint(a);
+        bits += 0x7ffffu + ((bits >> 20) & 1u);
+        return sign | ((((bits >> 23) - 120u) << 3) | ((bits >> 20) & 7u));
+    }
+    return sign | unsigned(__float2int_rn(a * 512.f)); // subnormals: multiples of 2^-9
+}
+
 // Storage traits: T is float, double or bf16_storage (a 16-bit wrapper).
 struct bf16_storage {
     unsigned short bits;

@@ -279,23 +279,6 @@ __global__ void fp8_splitk_reduce_kernel(size_t count, int splits, const float *
     out[index] = float_to_bf16_bits(sum);
 }
 
-// FP32 -> E4M3fn, round-to-nearest-even, saturating at +-448, NaN -> 0x7f.
-__device__ __forceinline__ unsigned f32_to_e4m3_sat(float value)
-{
-    unsigned sign = (__float_as_uint(value) >> 24) & 0x80u;
-    float a = fabsf(value);
-    if (a != a)
-        return 0x7fu;
-    if (a >= 448.f)
-        return sign | 0x7eu;
-    if (a >= 0.015625f) { // normal range: round the FP32 mantissa to three bits
-        unsigned bits = __float_as_uint(a);
-        bits += 0x7ffffu + ((bits >> 20) & 1u);
-        return sign | ((((bits >> 23) - 120u) << 3) | ((bits >> 20) & 7u));
-    }
-    return sign | unsigned(__float2int_rn(a * 512.f)); // subnormals: multiples of 2^-9
-}
-
 // Dynamic 1x128 quantiser (ref: camblas/_hopper.py:82-98). Sixteen lanes own one group (8 values
 // each); four groups per wavefront.
 __global__ __launch_bounds__(256) void fp8_quantise_kernel(int rows, int inner,

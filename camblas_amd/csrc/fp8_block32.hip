@@ -1,0 +1,202 @@
+// Single-token FP8 E4M3fn decode product with 32-wide scale blocks: out[n] = sum over blocks b of
+// (w[n, b] . x[b]) * sw[n/32, b] * sx[b], FP32 scales with element strides, BF16 out
+// (contract: ref include/camblas_cuda.h:124-155, src/cuda/backend.cu:1193-1256; arithmetic:
+// src/cuda/fp8_decode.cuh:150-157, sum = fma(dot_b * sw, sx, sum) for b ascending; the optional
+// activation quantiser: src/cuda/fp8_decode.cuh:58-72, scale = 2^ceil(log2(amax / 448))).
+//
+// Bandwidth-bound on W. A wavefront owns 16 weight rows for the whole K extent and keeps the
+// reference's single ascending chain per row; there is no cross-wavefront sum and no scratch.
+// One 128-byte step of a row holds four scale blocks, which one
+// v_mfma_scale_f32_16x16x128_f8f6f4 separates: in its operand layout lane group c = lane/16
+// supplies K bytes 32c .. 32c+31, i.e. exactly block c, so a B operand that carries x's block c in
+// column c and zeros elsewhere makes output column c the dot product of block c alone. The lane
+// that owns column c multiplies by its weight scale, the four products are gathered into column 0
+// with row shifts (DPP) and chained there. W is loaded with eight lanes per 128-byte line
+// (non-temporal, eight steps in flight per wavefront) and transposed to the operand layout
+// through a private swizzled LDS patch, as in the 128-block streaming kernel.
+#include "common.hpp"
+#include "device.hpp"
+
+namespace camblas_hip
+{
+namespace
+{
+struct Block32Params {
+    const unsigned char *w;
+    const void *x;    // E4M3 bytes, or BF16 when the kernel quantises
+    const float *sx;  // unused when the kernel quantises
+    const float *sw;
+    unsigned short *out;
+    int n, k, sx_stride, sw_row, sw_col;
+};
+
+constexpr int WAVES = 4, DEPTH = 8, STEP = 128, MAX_K = 8192;
+constexpr int UNIT = 0x7f7f7f7f; // E8M0 exponent 127 = scale 1.0 in every byte
+
+template <bool QUANTISE>
+__global__ __launch_bounds__(WAVES * 64) void fp8_block32_decode_kernel(Block32Params p)
+{
+    // x and its scales, zero-padded to a whole number of DEPTH-step rounds
+    __shared__ __attribute__((aligned(16))) unsigned x_words[MAX_K / 4];
+    __shared__ __attribute__((aligned(16))) float x_scale[MAX_K / 32];
+    __shared__ __attribute__((aligned(16))) u32x4_t patch[WAVES][128];
+    const int thread = threadIdx.x, lane = thread % 64, wave = thread / 64;
+    const int blocks = p.k / 32, steps = (p.k + STEP - 1) / STEP;
+    const int rounds = (steps + DEPTH - 1) / DEPTH, padded_steps = rounds * DEPTH;
+
+    if constexpr (QUANTISE) {
+        const unsigned *source = static_cast<const unsigned *>(p.x); // BF16 pairs
+        for (int b = thread; b < padded_steps * 4; b += WAVES * 64) {
+            float value[32];
+            float amax = 1e-10f;
+            if (b < blocks) {
+#pragma unroll
+                for (int e = 0; e < 16; ++e) {
+                    unsigned pair = source[b * 16 + e];
+                    value[2 * e] = __uint_as_float(pair << 16);
+                    value[2 * e + 1] = __uint_as_float(pair & 0xffff0000u);
+                    amax = fmaxf(amax, fmaxf(fabsf(value[2 * e]), fabsf(value[2 * e + 1])));
+                }
+                // power of two not below amax / 448: exponent of the product, plus one unless it
+                // is already a power of two
+                unsigned bits = __float_as_uint(__fmul_rn(amax, 1.f / 448.f));
+                int exponent = int((bits >> 23) & 255u) - 127 + int((bits & 0x7fffffu) != 0);
+                x_scale[b] = __uint_as_float(unsigned(exponent + 127) << 23);
+                float multiplier = __uint_as_float(unsigned(127 - exponent) << 23);
+#pragma unroll
+                for (int word = 0; word < 8; ++word) {
+                    unsigned packed = 0;
+#pragma unroll
+                    for (int e = 0; e < 4; ++e)
+                        packed |= f32_to_e4m3_sat(fminf(__fmul_rn(value[4 * word + e], multiplier), 448.f))
+                                  << (8 * e);
+                    x_words[b * 8 + word] = packed;
+                }
+            } else {
+                x_scale[b] = 0.f;
+#pragma unroll
+                for (int word = 0; word < 8; ++word)
+                    x_words[b * 8 + word] = 0u;
+            }
+        }
+    } else {
+        const unsigned *source = static_cast<const unsigned *>(p.x);
+        for (int word = thread; word < padded_steps * 32; word += WAVES * 64)
+            x_words[word] = word < p.k / 4 ? source[word] : 0u;
+        for (int b = thread; b < padded_steps * 4; b += WAVES * 64)
+            x_scale[b] = b < blocks ? p.sx[size_t(b) * p.sx_stride] : 0.f;
+    }
+    __syncthreads();
+
+    const int first_row = (blockIdx.x * WAVES + wave) * 16;
+    if (first_row >= p.n)
+        return; // no barrier below this point
+    const int column = lane % 16, chunk = lane / 16; // operand column / row, 32-byte chunk = block
+    const int load_row = lane / 8, piece = lane % 8; // load layout: 8 lanes per 128-byte line
+    const unsigned char *row_base[2] = {p.w + size_t(first_row + load_row) * p.k,
+                                        p.w + size_t(first_row + 8 + load_row) * p.k};
+    const float *sw_row = p.sw + size_t(first_row / 32) * p.sw_row;
+    auto slot = [](int r, int q) { return r * 8 + (q ^ ((r >> 1) & 7)); };
+    const int store_slot[2] = {slot(load_row, piece), slot(load_row + 8, piece)};
+    const int read_slot[2] = {slot(column, 2 * chunk), slot(column, 2 * chunk + 1)};
+    u32x4_t *mine = &patch[wave][0];
+
+    // Loads only (nothing here may use a loaded value). Bytes past the end of a row in a partial
+    // last step, and whole steps past the end, re-read the row's last 16 bytes: x is zero there.
+    u32x4_t raw[DEPTH][2];
+    float sw_reg[DEPTH];
+    auto fetch = [&](int step, u32x4_t(&data)[2], float &scale) {
+        int offset = step * STEP + piece * 16;
+        offset = offset < p.k ? offset : p.k - 16;
+        data[0] = __builtin_nontemporal_load(reinterpret_cast<const u32x4_t *>(row_base[0] + offset));
+        data[1] = __builtin_nontemporal_load(reinterpret_cast<const u32x4_t *>(row_base[1] + offset));
+        int b = step * 4 + (column & 3);
+        b = b < blocks ? b : blocks - 1;
+        scale = sw_row[size_t(b) * p.sw_col];
+    };
+    float sum[4] = {0.f, 0.f, 0.f, 0.f};
+    auto multiply = [&](int step, const u32x4_t(&data)[2], float scale) {
+        mine[store_slot[0]] = data[0];
+        mine[store_slot[1]] = data[1];
+        // other lanes' stores are read below: keep the compiler from moving the loads up (the
+        // hardware executes one wavefront's LDS operations in order)
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+        u32x4_t lo = mine[read_slot[0]], hi = mine[read_slot[1]];
+        const u32x4_t *x_step = reinterpret_cast<const u32x4_t *>(x_words) + step * 8 + chunk * 2;
+        u32x4_t x_lo = x_step[0], x_hi = x_step[1];
+        const unsigned keep = column == chunk ? 0xffffffffu : 0u; // block c only in column c
+        i32x8_t a = {int(lo[0]), int(lo[1]), int(lo[2]), int(lo[3]),
+                     int(hi[0]), int(hi[1]), int(hi[2]), int(hi[3])};
+        i32x8_t b = {int(x_lo[0] & keep), int(x_lo[1] & keep), int(x_lo[2] & keep), int(x_lo[3] & keep),
+                     int(x_hi[0] & keep), int(x_hi[1] & keep), int(x_hi[2] & keep), int(x_hi[3] & keep)};
+        f32x4_t dot = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(
+            a, b, f32x4_t{0.f, 0.f, 0.f, 0.f}, 0, 0, 0, UNIT, 0, UNIT);
+        const f32x4_t scales = *reinterpret_cast<const f32x4_t *>(x_scale + step * 4);
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+            // column c holds block c of row 4*chunk + r; bring blocks 1..3 to column 0 and chain
+            const float scaled = __fmul_rn(dot[r], scale);
+            const float block1 = dpp_move<0x101>(scaled), block2 = dpp_move<0x102>(scaled),
+                        block3 = dpp_move<0x103>(scaled);
+            sum[r] = fmaf(scaled, scales[0], sum[r]);
+            sum[r] = fmaf(block1, scales[1], sum[r]);
+            sum[r] = fmaf(block2, scales[2], sum[r]);
+            sum[r] = fmaf(block3, scales[3], sum[r]);
+        }
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+    };
+
+#pragma unroll
+    for (int d = 0; d < DEPTH; ++d) {
+        fetch(d, raw[d], sw_reg[d]);
+        __builtin_amdgcn_sched_barrier(0);
+    }
+    for (int step = 0; step < padded_steps; step += DEPTH) {
+#pragma unroll
+        for (int d = 0; d < DEPTH; ++d) {
+            __builtin_amdgcn_sched_barrier(0);
+            multiply(step + d, raw[d], sw_reg[d]);
+            __builtin_amdgcn_sched_barrier(0);
+            fetch(step + d + DEPTH, raw[d], sw_reg[d]);
+        }
+    }
+    if (column == 0) {
+        unsigned short *out = p.out + first_row + chunk * 4;
+#pragma unroll
+        for (int r = 0; r < 4; ++r)
+            out[r] = float_to_bf16_bits(sum[r]);
+    }
+}
+} // namespace
+
+// x: E4M3 bytes with FP32 scales sx (element stride sx_stride), or BF16 quantised on the fly when
+// sx is null. outputs a positive multiple of 16, inner a multiple of 32 in [32, 8192], w 16-byte
+// and x 4-byte aligned.
+hipError_t launch_fp8_block32_decode(hipStream_t stream, int outputs, int inner, const void *x,
+                                     const float *sx, int sx_stride, const void *w, const float *sw,
+                                     int sw_row, int sw_col, void *out)
+{
+    if (outputs < 16 || outputs % 16 || inner < 32 || inner > MAX_K || inner % 32)
+        return hipErrorInvalidValue;
+    Block32Params p;
+    p.w = static_cast<const unsigned char *>(w);
+    p.x = x;
+    p.sx = sx;
+    p.sw = sw;
+    p.out = static_cast<unsigned short *>(out);
+    p.n = outputs;
+    p.k = inner;
+    p.sx_stride = sx_stride;
+    p.sw_row = sw_row;
+    p.sw_col = sw_col;
+    const unsigned grid = unsigned((outputs + WAVES * 16 - 1) / (WAVES * 16));
+    if (sx)
+        fp8_block32_decode_kernel<false><<<grid, WAVES * 64, 0, stream>>>(p);
+    else
+        fp8_block32_decode_kernel<true><<<grid, WAVES * 64, 0, stream>>>(p);
+    return launch_status();
+}
+} // namespace camblas_hip

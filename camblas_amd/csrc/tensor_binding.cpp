@@ -15,6 +15,7 @@
 #include <ATen/Context.h>
 #include <c10/core/DeviceGuard.h>
 #include <c10/core/GradMode.h>
+#include <c10/hip/HIPFunctions.h>
 #include <c10/hip/HIPStream.h>
 
 #include <hip/hip_runtime_api.h>
@@ -544,6 +545,74 @@ Tensor fp8_block_matmul_public(const Tensor &a, const Tensor &a_scale, const Ten
     return result;
 }
 
+// Single-token FP8 product with 32-wide FP32 scale blocks; without input scales the BF16 token is
+// quantised on the fly (ref: src/cuda/torch_bindings.cpp:380-458).
+bool fp8_decode_supported_public(int device)
+{
+    same_process();
+    if (device < 0)
+        device = int(c10::hip::current_device());
+    c10::DeviceGuard guard(c10::Device(c10::kCUDA, c10::DeviceIndex(device)));
+    return camblas_cuda_fp8_decode_supported(context_for(device, default_algorithm)) != 0;
+}
+
+Tensor fp8_block32_product(const Tensor &x, const std::optional<Tensor> &x_scale,
+                           const Tensor &weight, const Tensor &weight_scale)
+{
+    same_process();
+    const bool quantise = !x_scale.has_value();
+    require(x.is_cuda() && x.scalar_type() == (quantise ? at::kBFloat16 : at::kFloat8_e4m3fn) &&
+                weight.scalar_type() == at::kFloat8_e4m3fn,
+            "FP8 linear requires GPU BF16/FP8 input and E4M3 weight");
+    require(x.dim() >= 1 && weight.dim() == 2 && weight_scale.dim() == 2 && x.is_contiguous() &&
+                weight.is_contiguous(),
+            "FP8 linear requires contiguous matrices and rank-two weight scales");
+    require(weight_scale.scalar_type() == at::kFloat, "FP8 weight scales must be FP32");
+    for (const Tensor *tensor : {&x, &weight, &weight_scale}) {
+        require(tensor->device() == x.device() &&
+                    (!c10::GradMode::is_enabled() || !tensor->requires_grad()),
+                "FP8 operands must share a GPU and support inference only");
+        for (int64_t size : tensor->sizes())
+            require(size <= INT_MAX, "LP64 dimension overflow");
+    }
+    const int64_t inner = x.size(-1), outputs = weight.size(0);
+    require(inner >= 32 && inner <= 8192 && inner % 32 == 0 && outputs >= 16 && outputs % 16 == 0 &&
+                x.numel() == inner && weight.size(1) == inner,
+            "Invalid FP8 linear matrix dimensions");
+    require(weight_scale.size(0) == (outputs + 31) / 32 && weight_scale.size(1) == inner / 32,
+            "FP8 weight scale shape does not match its blocks");
+    int64_t sx = 1;
+    const int64_t sn = weight_scale.stride(0), sk = weight_scale.stride(1);
+    if (!quantise) {
+        require(x_scale->device() == x.device() && x_scale->scalar_type() == at::kFloat &&
+                    x_scale->dim() == x.dim() &&
+                    (!c10::GradMode::is_enabled() || !x_scale->requires_grad()),
+                "FP8 input scales require matching device/rank and FP32 inference storage");
+        for (int64_t index = 0; index + 1 < x.dim(); ++index)
+            require(x_scale->size(index) == x.size(index), "FP8 input scale shape mismatch");
+        require(x_scale->size(-1) == inner / 32, "FP8 input scale shape mismatch");
+        sx = x_scale->stride(-1);
+    }
+    require(sx > 0 && sx <= INT_MAX && sn > 0 && sn <= INT_MAX && sk > 0 && sk <= INT_MAX,
+            "FP8 scale strides must be positive LP64 values");
+    c10::DeviceGuard guard(x.device());
+    camblas_cuda_context *context = context_for(x.get_device(), default_algorithm);
+    auto shape = x.sizes().vec();
+    shape.back() = outputs;
+    Tensor result = at::empty(shape, x.options().dtype(at::kBFloat16));
+    const int status =
+        quantise ? camblas_cuda_fp8_linear(context, int(outputs), int(inner), x.const_data_ptr(),
+                                           weight.const_data_ptr(),
+                                           weight_scale.const_data_ptr<float>(), int(sn), int(sk),
+                                           nullptr, 0, result.mutable_data_ptr())
+                 : camblas_cuda_fp8_decode(context, int(outputs), int(inner), x.const_data_ptr(),
+                                           x_scale->const_data_ptr<float>(), weight.const_data_ptr(),
+                                           weight_scale.const_data_ptr<float>(), int(sx), int(sn),
+                                           int(sk), nullptr, 0, result.mutable_data_ptr());
+    succeed(status, context);
+    return result;
+}
+
 // ---------------------------------------------------------------------------- ATen backend
 // Re-route aten::mm / mm.out / addmm on the GPU dispatch key. Anything the library does not take
 // goes to ATen's own GPU implementation through the at::cuda:: entry points, which bypass the
@@ -671,6 +740,24 @@ PYBIND11_MODULE(_camblas_cuda_torch, module)
                py::arg("input_scale"), py::arg("weight"), py::arg("weight_scale"),
                "Multiply E4M3fn activations (1x128 FP32 scales) by E4M3fn weights (128x128 FP32 "
                "scales), returning BF16.");
+    module.def("fp8_decode_supported", &fp8_decode_supported_public, py::arg("device") = -1,
+               "Return whether this build and device support the block-32 FP8 decode product.");
+    module.def(
+        "fp8_decode",
+        [](const Tensor &x, const Tensor &x_scale, const Tensor &weight, const Tensor &weight_scale) {
+            return fp8_block32_product(x, x_scale, weight, weight_scale);
+        },
+        py::arg("input"), py::arg("input_scale"), py::arg("weight"), py::arg("weight_scale"),
+        "Multiply one block32 E4M3 token by E4M3 weights, using FP32 scales and ordered FP32 "
+        "accumulation; positive scale strides are allowed.");
+    module.def(
+        "fp8_linear",
+        [](const Tensor &x, const Tensor &weight, const Tensor &weight_scale) {
+            return fp8_block32_product(x, std::nullopt, weight, weight_scale);
+        },
+        py::arg("input"), py::arg("weight"), py::arg("weight_scale"),
+        "Quantise one finite BF16 token to block32 E4M3 with power-of-two FP32 scales and "
+        "multiply E4M3 weights with ordered FP32 accumulation.");
     module.def("stats", &stats);
     module.def("stats_all", &stats_all);
     module.def("close", &close_all);

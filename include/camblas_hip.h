@@ -129,6 +129,27 @@ int camblas_cuda_rms_scale(camblas_cuda_context *context, int dtype, uint64_t co
 int camblas_cuda_stats(const camblas_cuda_context *context, uint64_t *counts, int length);
 int camblas_cuda_reset_stats(camblas_cuda_context *context);
 
+/* Single-token FP8 E4M3 [inner] times contiguous [outputs, inner] weights with 32-wide scale
+ * blocks: FP32 input scales [inner/32] and weight scales [ceil(outputs/32), inner/32] with
+ * positive element strides; sum = fma(dot_b * weight_scale, input_scale, sum) for b ascending, BF16
+ * out [outputs]. inner a multiple of 32 in [32, 8192], outputs a positive multiple of 16.
+ * ref: include/camblas_cuda.h:124-155, src/cuda/backend.cu:1193-1256, src/cuda/fp8_decode.cuh:150-157.
+ * camblas_cuda_fp8_linear takes a BF16 token and quantises it per block with the power-of-two
+ * scale 2^ceil(log2(max(|x|, 1e-10) / 448)) (ref: src/cuda/fp8_decode.cuh:58-72). Both run as one
+ * kernel: the workspace query returns 0 and the workspace arguments are ignored. The weight must be
+ * 16-byte aligned here (the reference asks for 4). */
+int camblas_cuda_fp8_decode_supported(const camblas_cuda_context *context);
+int camblas_cuda_fp8_decode(camblas_cuda_context *context, int outputs, int inner,
+                            const void *input, const float *input_scale, const void *weight,
+                            const float *weight_scale, int input_scale_stride,
+                            int weight_scale_row_stride, int weight_scale_column_stride,
+                            void *workspace, size_t workspace_bytes, void *output);
+size_t camblas_cuda_fp8_workspace_size(int quantise, int outputs, int inner);
+int camblas_cuda_fp8_linear(camblas_cuda_context *context, int outputs, int inner,
+                            const void *input, const void *weight, const float *weight_scale,
+                            int weight_scale_row_stride, int weight_scale_column_stride,
+                            void *workspace, size_t workspace_bytes, void *output);
+
 /* ------------------------------------------------------------------ extensions */
 
 /* extension. FP8 E4M3fn block-scaled linear: a [rows, inner] bytes with FP32 scales

@@ -149,6 +149,30 @@ def quantise_1x128(x_bits):
     return q, scale
 
 
+def quantise_block32(x_bits):
+    """Power-of-two block-32 quantiser for one BF16 token [inner]: (E4M3 bytes, FP32 scales)."""
+    x_bits = np.ascontiguousarray(x_bits, dtype=np.uint16).reshape(-1)
+    q = np.empty(x_bits.size, dtype=np.uint8)
+    scale = np.empty(x_bits.size // 32, dtype=np.float32)
+    lib().oracle_quantise_block32(x_bits.size, _ptr(x_bits), _ptr(q), _ptr(scale))
+    return q, scale
+
+
+def fp8_block32_decode(x, sx, w, sw):
+    """Single-token block-32 product; sx [inner/32] and sw [ceil(outputs/32), inner/32] may be
+    strided views (their element strides are passed on)."""
+    outputs, inner = w.shape
+    assert sx.ndim == 1 and sw.ndim == 2 and sx.dtype == np.float32 and sw.dtype == np.float32
+    out = np.empty(outputs, dtype=np.uint16)
+    x = np.ascontiguousarray(x, dtype=np.uint8).reshape(-1)
+    w = np.ascontiguousarray(w, dtype=np.uint8)
+    status = lib().oracle_fp8_block32_decode(
+        outputs, inner, _ptr(x), ct.c_void_p(sx.ctypes.data), sx.strides[0] // 4, _ptr(w),
+        ct.c_void_p(sw.ctypes.data), sw.strides[0] // 4, sw.strides[1] // 4, _ptr(out))
+    assert status == 0
+    return out
+
+
 def fp8_block_matmul(a, a_scale, w, w_scale, want32=False):
     rows, inner = a.shape
     outputs = w.shape[0]

@@ -258,6 +258,61 @@ void oracle_quantise_1x128(int rows, int inner, const uint16_t *x_bf16, uint8_t 
         }
 }
 
+/* Power-of-two block-32 activation quantiser of src/cuda/fp8_decode.cuh:58-72: per 32 values
+ * amax = max(|x|, 1e-10); bits of fl(amax * (1/448)); exponent = biased exponent - 127, plus one
+ * unless the mantissa is zero; scale = 2^exponent; q = e4m3(min(x * 2^-exponent, 448)) with a
+ * saturating finite conversion (which caps the negative side). The same integer recipe is
+ * restated on the CPU in the reference's tests/test_sglang.py:423-445. */
+void oracle_quantise_block32(int inner, const uint16_t *x_bf16, uint8_t *q, float *scale)
+{
+    for (int b = 0; b < inner / 32; ++b) {
+        float amax = 1e-10f;
+        for (int i = 0; i < 32; ++i) {
+            float v = fabsf(bf16_to_f32(x_bf16[b * 32 + i]));
+            if (v > amax)
+                amax = v;
+        }
+        float raw = amax * (1.0f / 448.0f);
+        uint32_t bits;
+        memcpy(&bits, &raw, 4);
+        int exponent = (int)((bits >> 23) & 255u) - 127 + ((bits & 0x7fffffu) != 0);
+        scale[b] = ldexpf(1.0f, exponent);
+        for (int i = 0; i < 32; ++i) {
+            float v = ldexpf(bf16_to_f32(x_bf16[b * 32 + i]), -exponent);
+            q[b * 32 + i] = f32_to_e4m3_sat(fminf(v, 448.f));
+        }
+    }
+}
+
+/* Single-token block-32 product of src/cuda/fp8_decode.cuh:150-157 for every output row n:
+ *     sum = 0;  for b ascending:  sum = fmaf(fl(dot_b * sw[n/32, b]), sx[b], sum)
+ * then one RN rounding to BF16. dot_b (32 products of two E4M3 values) is formed exactly in
+ * FP64 and rounded once to FP32. Scales are addressed with element strides as in
+ * include/camblas_cuda.h:124-137. */
+int oracle_fp8_block32_decode(int outputs, int inner, const uint8_t *x, const float *sx,
+                              int sx_stride, const uint8_t *w, const float *sw, int sw_row,
+                              int sw_col, uint16_t *out)
+{
+    if (outputs < 1 || inner < 32 || inner % 32)
+        return -1;
+    float table[256];
+    for (int i = 0; i < 256; ++i)
+        table[i] = e4m3_to_f32((uint8_t)i);
+#pragma omp parallel for schedule(static)
+    for (int n = 0; n < outputs; ++n) {
+        float sum = 0.f;
+        for (int b = 0; b < inner / 32; ++b) {
+            double dot = 0.0;
+            for (int i = 0; i < 32; ++i)
+                dot += (double)table[w[(size_t)n * inner + b * 32 + i]] * (double)table[x[b * 32 + i]];
+            float scaled = (float)dot * sw[(size_t)(n / 32) * sw_row + (size_t)b * sw_col];
+            sum = fmaf(scaled, sx[(size_t)b * sx_stride], sum);
+        }
+        out[n] = f32_to_bf16(sum);
+    }
+    return 0;
+}
+
 /* Block-scaled product rule of camblas/_hopper.py:118-126 (unscaled per-group dot, stored FP32)
  * and :168-182 (ordered reduction): for each output (r, n)
  *     acc = 0;  for g ascending:  acc = fmaf(dot_g, a_scale[r,g] * w_scale[n/128, g], acc)

@@ -133,7 +133,8 @@ def test_tensor_binding_loads_and_exports_the_reference_surface():
     assert module is not None, "camblas_amd/lib/_camblas_cuda_torch*.so is not built"
     for name in ("install_torch_backend", "set_default_algorithm", "stats", "stats_all", "close",
                  "matmul", "matmul_public", "linear_public", "qkv_linear", "gated_mlp",
-                 "silu_multiply", "swiglu", "rms_norm", "add_rms_norm", "fp8_block_matmul"):
+                 "silu_multiply", "swiglu", "rms_norm", "add_rms_norm", "fp8_block_matmul",
+                 "fp8_decode_supported", "fp8_decode", "fp8_linear"):
         assert callable(getattr(module, name)), name
     import torch
 

@@ -205,6 +205,63 @@ def test_activation_quantiser_invariants():
     assert np.abs(decoded * scale[..., None] - values).max() <= np.abs(values).max() * 2.0**-4
 
 
+def test_block32_decode_rule_and_power_of_two_quantiser():
+    # product: pure-Python chain on a small case, strided scales, the reference's known answers
+    # (ref: tests/test_quantized.py:160-216: ones times twos with sx = 0.5, sw = 2, last row block
+    # doubled -> 2k and 4k; NaN weights -> NaN)
+    outputs, inner = 48, 96
+    rng = np.random.default_rng(21)
+    x = rng.integers(0, 0x7F, inner, dtype=np.uint8)
+    w = rng.integers(0, 0x7F, (outputs, inner), dtype=np.uint8) | (rng.integers(0, 2, (outputs, inner), dtype=np.uint8) << 7)
+    w[w == 0xFF] = 0x80
+    sx_storage = rng.uniform(0.001, 0.08, (inner // 32, 4)).astype(np.float32)
+    sx = sx_storage[:, 0]                                     # padded: element stride 4
+    sw = np.asfortranarray(rng.uniform(0.5, 2.0, (2, inner // 32)).astype(np.float32))  # column-major
+    got = oracle.fp8_block32_decode(x, sx, w, sw)
+    table = oracle.e4m3_to_f32(np.arange(256, dtype=np.uint8)).astype(np.float64)
+    for n in range(outputs):
+        total = np.float32(0)
+        for b in range(inner // 32):
+            dot = np.float32(sum(table[w[n, b * 32 + i]] * table[x[b * 32 + i]] for i in range(32)))
+            scaled = np.float32(dot * sw[n // 32, b])
+            total = np.float32(math.fma(float(scaled), float(sx[b]), float(total))) if hasattr(math, "fma") \
+                else np.float32(np.float64(scaled) * np.float64(sx[b]) + np.float64(total))
+        assert oracle.f32_to_bf16(np.float32([total]))[0] == got[n], n
+    k = 5120
+    ones, twos = np.full(k, 0x38, np.uint8), np.full((1152, k), 0x40, np.uint8)
+    sw = np.full((36, k // 32), 2, np.float32)
+    sw[-1] *= 2
+    out = oracle.bf16_to_f32(oracle.fp8_block32_decode(ones, np.full(k // 32, 0.5, np.float32), twos, sw))
+    assert (out[:-32] == 2 * k).all() and (out[-32:] == 4 * k).all()
+    twos[7, 100] = 0x7F
+    out = oracle.bf16_to_f32(oracle.fp8_block32_decode(ones, np.full(k // 32, 0.5, np.float32), twos, sw))
+    assert np.isnan(out[7]) and np.isfinite(np.delete(out, 7)).all()
+
+    # quantiser: the scale is the smallest power of two not below amax / 448, the bytes are the
+    # nearest E4M3 values of x / scale (ties to even), found by search rather than by the encoder
+    x_bits = oracle.fill_normal_bf16(22, (256,), std=3.0)
+    x_bits[32:64] = oracle.f32_to_bf16(np.float32([448.0 * 2.0**-3] * 32))     # amax/448 exactly a power of two
+    x_bits[64:96] = 0
+    q, scale = oracle.quantise_block32(x_bits)
+    values = oracle.bf16_to_f32(x_bits).astype(np.float64).reshape(8, 32)
+    amax = np.maximum(np.abs(values).max(axis=1), 1e-10)
+    # the reference takes the exponent of fl32(amax * fl32(1/448)); evaluate that product exactly
+    raw = (amax.astype(np.float32) * np.float32(1 / 448)).astype(np.float64)
+    want_scale = 2.0 ** np.ceil(np.log2(raw))
+    assert np.array_equal(scale.astype(np.float64), want_scale)
+    assert scale[1] == 2.0**-3 and scale[2] == 2.0 ** math.ceil(math.log2(np.float32(1e-10) * np.float32(1 / 448)))
+    finite = np.where(~np.isnan(table))[0]
+    for b in range(8):
+        for i in range(32):
+            target = min(values[b, i] / want_scale[b], 448.0)
+            target = max(target, -448.0)
+            distance = np.abs(table[finite] - target)
+            best = finite[distance == distance.min()]
+            if len(best) > 1:                      # tie (or +-0): even mantissa wins
+                best = [c for c in best if c % 2 == 0 and (target != 0 or c == (0x80 if np.signbit(values[b, i]) else 0))] or best
+            assert q[b * 32 + i] in best, (b, i, target, q[b * 32 + i], best)
+
+
 # ---------------------------------------------------------------- decode epilogues
 
 def test_rms_silu_swiglu_closed_forms():

@@ -181,3 +181,119 @@ def test_invalid_arguments(device):
     assert lib.camblas_cuda_fp8_block_matmul(native.handle, 0, 128, 128, None, None, None, None, None) == 0
     assert lib.camblas_cuda_fp8_block_matmul(native.handle, 1, 128, 128, None, None, None, None, None) == -1
     assert b"invalid FP8 block matrix buffers" in lib.camblas_cuda_error(native.handle)
+
+
+# ---------------------------------------------------------------- block-32 single-token decode
+def block32_operands(seed, outputs, inner):
+    rng = np.random.default_rng(seed)
+    x = rng.integers(0, 0x7F, inner, dtype=np.uint8) | (rng.integers(0, 2, inner, dtype=np.uint8) << 7)
+    w = rng.integers(0, 0x7F, (outputs, inner), dtype=np.uint8) | (rng.integers(0, 2, (outputs, inner), dtype=np.uint8) << 7)
+    x[x == 0xFF] = 0x80
+    w[w == 0xFF] = 0x80
+    sx = rng.uniform(0.001, 0.08, inner // 32).astype(np.float32)
+    sw = rng.uniform(0.002, 0.05, ((outputs + 31) // 32, inner // 32)).astype(np.float32)
+    return x, sx, w, sw
+
+
+def fp8_tensor(array, device):
+    return torch.from_numpy(array).to(device).view(torch.float8_e4m3fn)
+
+
+@pytest.mark.parametrize("outputs,inner", [(48, 96), (16, 32), (1152, 5120), (5120, 576), (18432, 7168),
+                                           (80, 8192)])
+def test_block32_decode_matches_ordered_oracle(device, outputs, inner):
+    # ref strategy: tests/test_quantized.py:160-216 and tests/test_sglang.py:375-398; sizes cover
+    # partial 128-byte steps (inner % 128 != 0), a partial last 32-row scale block and a partial
+    # last workgroup. Same ordered chain as the oracle: only the rounding of a block's dot product
+    # inside the matrix core may differ.
+    x, sx, w, sw = block32_operands(400 + outputs, outputs, inner)
+    out = _kernels.fp8_decode(fp8_tensor(x, device).view(1, -1), torch.from_numpy(sx).to(device).view(1, -1),
+                              fp8_tensor(w, device), torch.from_numpy(sw).to(device))
+    torch.cuda.synchronize()
+    assert out.shape == (1, outputs)
+    want = oracle.fp8_block32_decode(x, sx, w, sw)
+    got = from_device_bf16(out)[0]
+    assert (bf16_ulp_distance(got, want) == 0).mean() > 0.9
+    wanted = oracle.bf16_to_f32(want)
+    assert (np.abs(bf16_values(out)[0] - wanted) <= 2.0**-7 * np.abs(wanted) + 1e-4 * np.abs(wanted).max()).all()
+    # padded (element stride 4) input scales and column-major weight scales give the same bits
+    storage = torch.zeros((inner // 32, 4), device=device)
+    storage[:, 0] = torch.from_numpy(sx).to(device)
+    strided = _kernels.fp8_decode(fp8_tensor(x, device).view(1, -1), storage[:, 0].view(1, -1),
+                                  fp8_tensor(w, device), torch.from_numpy(sw).to(device).T.contiguous().T)
+    assert torch.equal(strided.view(torch.int16), out.view(torch.int16))
+
+
+def test_block32_known_answers_graph_and_nan(device):
+    # ref: tests/test_quantized.py:160-216 — exact expected values, a captured graph that sees later
+    # in-place updates of its operands, NaN propagation
+    for fused, n, k in ((False, 48, 96), (True, 48, 96), (False, 1152, 5120), (True, 1152, 5120),
+                        (True, 5120, 576)):
+        x = torch.zeros(1, k, device=device).to(torch.bfloat16 if fused else torch.float8_e4m3fn)
+        weight = torch.ones(n, k, device=device).to(torch.float8_e4m3fn)
+        sx = torch.ones(1, k // 32, device=device)
+        sw = torch.ones((n + 31) // 32, k // 32, device=device)
+        sw[-1].mul_(2)
+
+        def product():
+            return _kernels.fp8_linear(x, weight, sw) if fused else _kernels.fp8_decode(x, sx, weight, sw)
+
+        stream = torch.cuda.Stream(device=device)
+        stream.wait_stream(torch.cuda.current_stream(device))
+        with torch.inference_mode(), torch.cuda.stream(stream):
+            before = product()
+            graph = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(graph, stream=stream):
+                output = product()
+            if fused:
+                x.fill_(0.5)
+            else:
+                x.view(torch.uint8).fill_(0x38)
+            weight.view(torch.uint8).fill_(0x40)
+            sx.mul_(0.5)
+            sw.mul_(2)
+            graph.replay()
+        stream.synchronize()
+        expected = torch.full((1, n), float(k * 2), dtype=torch.bfloat16)
+        # fused: 0.5 quantises exactly (256 * 2^-9), which equals the split case's 1.0 * 0.5
+        expected[:, ((n + 31) // 32 - 1) * 32:] *= 2
+        assert torch.equal(output.cpu().view(torch.int16), expected.view(torch.int16)), (fused, n, k)
+        assert (before == 0).all()
+        weight.view(torch.uint8).fill_(0x7F)
+        with torch.inference_mode():
+            assert product().isnan().all()
+
+
+@pytest.mark.parametrize("inner,std", [(7168, 0.75), (576, 80.0), (8192, 1e-3)])
+def test_block32_fused_quantiser_is_bit_exact(device, inner, std):
+    # the fused kernel quantises in LDS and then runs the same product: its output must equal the
+    # product of the oracle-quantised token bit for bit, which pins bytes and power-of-two scales
+    outputs = 256
+    _, _, w, sw = block32_operands(500 + inner, outputs, inner)
+    x_bits = oracle.fill_normal_bf16(501 + inner, (inner,), std=std)
+    x_bits[:32] = 0
+    q, scale = oracle.quantise_block32(x_bits)
+    assert (np.log2(scale) % 1 == 0).all()
+    fused = _kernels.fp8_linear(to_device_bf16(x_bits.reshape(1, -1), device), fp8_tensor(w, device),
+                                torch.from_numpy(sw).to(device))
+    split = _kernels.fp8_decode(fp8_tensor(q, device).view(1, -1), torch.from_numpy(scale).to(device).view(1, -1),
+                                fp8_tensor(w, device), torch.from_numpy(sw).to(device))
+    assert torch.equal(fused.view(torch.int16), split.view(torch.int16))
+
+
+def test_block32_invalid_arguments(device):
+    x, sx, w, sw = block32_operands(600, 48, 96)
+    xt, wt = fp8_tensor(x, device).view(1, -1), fp8_tensor(w, device)
+    sxt, swt = torch.from_numpy(sx).to(device).view(1, -1), torch.from_numpy(sw).to(device)
+    assert _kernels.fp8_decode_supported(device)
+    for operands in ((xt.expand(2, -1).contiguous(), sxt.expand(2, -1).contiguous(), wt, swt),
+                     (xt, sxt[:, :2], wt, swt), (xt, sxt[:, :1].expand_as(sxt), wt, swt),
+                     (xt, sxt, wt[:40], swt), (xt, sxt, wt, swt[:, :2])):
+        with pytest.raises(RuntimeError):
+            _kernels.fp8_decode(*operands)
+    native, lib = _native.context(device), _native.library()
+    status = lib.camblas_cuda_fp8_decode(native.handle, 40, 96, None, None, None, None, 1, 1, 1, None, 0, None)
+    assert status == -1 and b"invalid FP8 decode dimensions" in lib.camblas_cuda_error(native.handle)
+    status = lib.camblas_cuda_fp8_decode(native.handle, 48, 96, None, None, None, None, 1, 1, 1, None, 0, None)
+    assert status == -1 and b"invalid FP8 decode buffers" in lib.camblas_cuda_error(native.handle)
+    assert lib.camblas_cuda_fp8_workspace_size(0, 48, 96) == 0 == lib.camblas_cuda_fp8_workspace_size(1, 48, 96)

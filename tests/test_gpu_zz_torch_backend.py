@@ -124,6 +124,33 @@ def test_fusion_entries(binding, device):
         binding.silu_multiply(x.clone().requires_grad_(), residual)
 
 
+def test_block32_fp8_entries(binding, device):
+    # the binding's fp8_decode / fp8_linear against the ctypes path (same library entry points) and
+    # the reference's argument errors (ref: tests/test_quantized.py:218-240)
+    from camblas_amd import _kernels
+
+    assert binding.fp8_decode_supported(device.index or 0) and binding.fp8_decode_supported()
+    n, k = 64, 256
+    x = (torch.randn(1, k, device=device) * 2).to(torch.float8_e4m3fn)
+    w = torch.randn(n, k, device=device).to(torch.float8_e4m3fn)
+    sx = torch.rand(1, k // 32, device=device) + 0.5
+    sw = torch.rand(n // 32, k // 32, device=device) + 0.5
+    assert torch.equal(binding.fp8_decode(x, sx, w, sw), _kernels.fp8_decode(x, sx, w, sw))
+    token = torch.randn(1, k, device=device).bfloat16()
+    assert torch.equal(binding.fp8_linear(token, w, sw), _kernels.fp8_linear(token, w, sw))
+    dequantised = (x.float().view(-1, 32) * sx.view(-1, 1)).view(1, k).double() @ (
+        w.float().view(n // 32, 32, k // 32, 32) * sw.view(n // 32, 1, k // 32, 1)).view(n, k).double().t()
+    assert error(binding.fp8_decode(x, sx, w, sw), dequantised) <= 1e-2
+    for operands in ((x.expand(2, -1).contiguous(), sx.expand(2, -1).contiguous(), w, sw),
+                     (x, sx[:, :2], w, sw), (x, sx[:, :1].expand_as(sx), w, sw)):
+        with pytest.raises(ValueError):
+            binding.fp8_decode(*operands)
+    for operands in ((token.expand(2, -1).contiguous(), w, sw), (token, w, sw[:, :2]),
+                     (token.clone().requires_grad_(), w, sw)):
+        with pytest.raises(ValueError):
+            binding.fp8_linear(*operands)
+
+
 def test_backend_override_routes_and_falls_back(binding, device):
     binding.install_torch_backend(_native.ALGORITHMS["lt"])
     binding.install_torch_backend(_native.ALGORITHMS["lt"])  # idempotent
