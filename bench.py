@@ -363,6 +363,26 @@ def extras(torch, _kernels, _native, device, normal):
         "us": round(seconds * 1e6, 1), "gbps": round(traffic / seconds / 1e9, 1),
         "frac_of_8TBs": round(traffic / seconds / HBM_PEAK, 4),
     }
+    # E8M0 block-scaled (microscaling) decode products of the reference header: E4M3 and packed E2M1
+    # weights [18432, 7168], 16 tokens, rotating weight copies
+    mx = {}
+    tokens = 16
+    a = torch.randint(0, 0x7E, (tokens, inner), device=device, dtype=torch.uint8).view(torch.float8_e4m3fn)
+    a_scale = torch.randint(120, 130, (tokens, inner // 32), device=device, dtype=torch.uint8)
+    for name, packed in (("e4m3", False), ("e2m1", True)):
+        if packed:
+            weights = [torch.randint(0, 256, (outputs, inner // 2), device=device, dtype=torch.uint8)
+                       for _ in range(3)]
+            scale = torch.randint(120, 130, (outputs, inner // 32), device=device, dtype=torch.uint8)
+        else:
+            weights = copies
+            scale = torch.randint(120, 130, (outputs // 32, inner // 32), device=device, dtype=torch.uint8)
+        seconds = event_time(
+            torch, lambda i: _kernels.quantized_matmul(a, a_scale, weights[i % 3], scale), 10, 20)
+        traffic = weights[0].numel() + scale.numel() + tokens * (inner + inner // 32 + outputs * 2)
+        mx[name] = {"us": round(seconds * 1e6, 1), "gbps": round(traffic / seconds / 1e9, 1),
+                    "frac_of_8TBs": round(traffic / seconds / HBM_PEAK, 4)}
+    found["mx_quantized_matmul_m16_18432x7168"] = mx
     del copies, w_scale
     # FP32 SGEMM 2048^3 (plumbing)
     size = 2048

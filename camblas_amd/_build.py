@@ -32,6 +32,8 @@ CORE_SOURCES = (
     "fp8_dma.hip",
     "fp8_stream.hip",
     "fp8_block32.hip",
+    "mx_matmul.hip",
+    "routing.hip",
     "fusion.hip",
     "attention_decode.hip",
 )

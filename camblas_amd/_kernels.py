@@ -281,6 +281,93 @@ def fp8_block_linear(x, weight, weight_scale):
     return out.reshape(*x.shape[:-1], weight.shape[0])
 
 
+def _bytes(tensor):
+    return tensor if tensor.dtype == torch.uint8 else tensor.view(torch.uint8)
+
+
+def quantized_matmul(x, x_scale, weight, weight_scale, *, activation_block=32):
+    """E8M0 block-scaled linear (ref: quantized_matmul_public, src/cuda/torch_bindings.cpp:328-378):
+    x E4M3 [.., inner] with scales [.., inner/activation_block]; weight E4M3 [outputs, inner] with
+    scales [ceil(outputs/32), inner/32], or packed E2M1 [outputs, inner/2] (uint8 or
+    float4_e2m1fn_x2) with scales [outputs, inner/32]. Returns BF16 [.., outputs]."""
+    packed = weight.dtype != torch.float8_e4m3fn
+    _require(x.is_cuda and x.dtype == torch.float8_e4m3fn and x.is_contiguous()
+             and weight.is_contiguous() and x_scale.is_contiguous() and weight_scale.is_contiguous(),
+             "quantized matmul requires contiguous GPU operands with E4M3 input")
+    _require(not torch.is_grad_enabled() or not any(t.requires_grad for t in (x, x_scale, weight_scale)),
+             "quantized matmul supports inference only")
+    inner = x.shape[-1]
+    rows = x.numel() // max(inner, 1)
+    outputs = weight.shape[0]
+    _require(weight.dim() == 2 and weight.shape[1] * (2 if packed else 1) == inner
+             and inner % 32 == 0 and outputs % 8 == 0 and outputs >= 8
+             and activation_block in ((32, 128) if packed else (32,)) and inner % activation_block == 0,
+             "Invalid quantized matrix dimensions")
+    _require(x_scale.numel() == rows * (inner // activation_block)
+             and tuple(weight_scale.shape) == ((outputs if packed else (outputs + 31) // 32), inner // 32),
+             "Quantized scale shapes do not match their blocks")
+    out = torch.empty(tuple(x.shape[:-1]) + (outputs,), dtype=torch.bfloat16, device=x.device)
+    _native.context(x.device).call(
+        "quantized_matmul", int(packed), rows, outputs, inner, activation_block, _pointer(x),
+        _pointer(_bytes(x_scale)), _pointer(_bytes(weight)), _pointer(_bytes(weight_scale)),
+        _pointer(out))
+    return out
+
+
+def grouped_quantized_matmul(x, x_scale, metadata, active, counts, *, outputs, packed,
+                             activation_block=32):
+    """Batched E8M0 block-scaled products (ref: include/camblas_cuda.h:156-167): x E4M3
+    [groups, rows, inner]; metadata uint64 [weight_groups, 2] (weight, scale addresses); active and
+    counts int32 [groups]. Returns BF16 [groups, rows, outputs]; inactive groups and padding rows
+    are zero."""
+    groups, rows, inner = x.shape
+    _require(x.is_contiguous() and x_scale.is_contiguous() and metadata.dtype in (torch.int64, torch.uint64)
+             and metadata.dim() == 2 and metadata.shape[1] == 2 and active.dtype == torch.int32
+             and counts.dtype == torch.int32 and active.numel() == groups == counts.numel(),
+             "Invalid grouped operands")
+    out = torch.empty((groups, rows, outputs), dtype=torch.bfloat16, device=x.device)
+    _native.context(x.device).call(
+        "grouped_quantized_matmul", int(packed), groups, metadata.shape[0], rows, outputs, inner,
+        activation_block, _pointer(x), _pointer(_bytes(x_scale)), _pointer(metadata),
+        _pointer(active), _pointer(counts), _pointer(out))
+    return out
+
+
+def route_groups(experts, active, *, first_expert=0, rows):
+    """Slots, reverse mapping and counts for expert/choice IDs (ref: route_groups_public,
+    src/cuda/torch_bindings.cpp:465-530): experts int64 [tokens, choices], active int32 [groups].
+    Excess rows are discarded and unassigned slots are -1; runs on the current stream."""
+    _require(experts.is_cuda and experts.dtype == torch.int64 and experts.dim() == 2
+             and experts.is_contiguous() and active.dtype == torch.int32 and active.dim() == 1
+             and active.is_contiguous() and active.device == experts.device,
+             "routing needs contiguous GPU int64 expert IDs [tokens, choices] and int32 active IDs")
+    tokens, choices = experts.shape
+    groups = active.numel()
+    counts = torch.empty(groups, dtype=torch.int32, device=experts.device)
+    slots = torch.empty((groups, rows), dtype=torch.int32, device=experts.device)
+    reverse = torch.empty((tokens, max(choices, 1)), dtype=torch.int32, device=experts.device)
+    _native.context(experts.device).call(
+        "route_groups", tokens, choices, first_expert, groups, rows, _pointer(experts),
+        _pointer(active), _pointer(counts), _pointer(slots), _pointer(reverse))
+    return slots, reverse, counts
+
+
+def reduce_groups(grouped, experts, reverse):
+    """Sum BF16 contributions [grouped_rows, width] into FP32 [tokens, width] in expert/choice
+    order (ref: reduce_groups_public, src/cuda/torch_bindings.cpp:532-600)."""
+    _require(grouped.is_cuda and grouped.dtype == torch.bfloat16 and grouped.dim() == 2
+             and grouped.is_contiguous() and experts.dtype == torch.int64 and experts.is_contiguous()
+             and reverse.dtype == torch.int32 and reverse.is_contiguous()
+             and reverse.shape == experts.shape,
+             "grouped reduction needs contiguous BF16 rows, int64 experts and int32 reverse")
+    tokens, choices = experts.shape
+    out = torch.empty((tokens, grouped.shape[1]), dtype=torch.float32, device=grouped.device)
+    _native.context(grouped.device).call(
+        "reduce_groups", tokens, choices, grouped.shape[1], grouped.shape[0], _pointer(experts),
+        _pointer(reverse), _pointer(grouped), _pointer(out))
+    return out
+
+
 def fp8_decode_supported(device=None):
     """Whether the block-32 single-token FP8 product runs on this device (ref: fp8_decode_supported
     in src/cuda/torch_bindings.cpp:380-387)."""

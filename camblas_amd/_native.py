@@ -65,6 +65,10 @@ SIGNATURES = {
     "add_rms_norm": ([_P, _I, _I, _F, _P, _P, _P, _P, _P], _I),
     "bfloat16_square": ([_P, _U64, _P, _P], _I),
     "rms_scale": ([_P, _I, _U64, _I, _F, _P, _P, _P, _P], _I),
+    "quantized_matmul": ([_P, _I, _I, _I, _I, _I, _P, _P, _P, _P, _P], _I),
+    "route_groups": ([_P, _I, _I, _I, _I, _I, _P, _P, _P, _P, _P], _I),
+    "reduce_groups": ([_P, _I, _I, _I, _I, _P, _P, _P, _P], _I),
+    "grouped_quantized_matmul": ([_P, _I, _I, _I, _I, _I, _I, _I, _P, _P, _P, _P, _P, _P], _I),
     "fp8_decode_supported": ([_P], _I),
     "fp8_decode": ([_P, _I, _I, _P, _P, _P, _P, _I, _I, _I, _P, _SZ, _P], _I),
     "fp8_workspace_size": ([_I, _I, _I], _SZ),

@@ -586,6 +586,107 @@ extern "C" int camblas_cuda_fp8_block_matmul(camblas_cuda_context *context, int 
     });
 }
 
+// ref: src/cuda/backend.cu:1165-1191
+extern "C" int camblas_cuda_quantized_matmul(camblas_cuda_context *context, int packed, int rows,
+                                             int outputs, int inner, int activation_block,
+                                             const void *input, const void *input_scale,
+                                             const void *weight, const void *weight_scale,
+                                             void *output)
+{
+    return execute(context, [&] {
+        if ((packed != 0 && packed != 1) || rows < 0 || rows > 65535 || outputs < 8 ||
+            outputs % 8 || inner < 32 || inner % 32 ||
+            (activation_block != 32 && activation_block != 128) || inner % activation_block ||
+            (!packed && activation_block != 32))
+            return fail(context, "invalid quantized matrix dimensions", 1);
+        if (!rows)
+            return 0;
+        if (!input || !input_scale || !weight || !weight_scale || !output || !aligned(input, 16) ||
+            !aligned(weight, 16) || !aligned(output, 2) || output == input ||
+            output == input_scale || output == weight || output == weight_scale)
+            return fail(context, "invalid quantized matrix buffers", 1);
+        context->counts[4]++;
+        hipError_t error = launch_mx_matmul(context->stream, packed != 0, 0, 0, rows, outputs, inner,
+                                            activation_block, input, input_scale, weight,
+                                            weight_scale, nullptr, nullptr, nullptr, output);
+        return error == hipSuccess ? 0 : fail(context, "quantized matrix multiplication", error);
+    });
+}
+
+// ref: src/cuda/backend.cu:1258-1303. The kernel writes the zeros of inactive groups and padding
+// rows itself, so no memset node is needed (the call can be captured in a graph).
+extern "C" int camblas_cuda_grouped_quantized_matmul(camblas_cuda_context *context, int packed,
+                                                     int groups, int weight_groups, int rows,
+                                                     int outputs, int inner, int activation_block,
+                                                     const void *input, const void *input_scale,
+                                                     const void *metadata, const void *active,
+                                                     const void *counts, void *output)
+{
+    return execute(context, [&] {
+        if ((packed != 0 && packed != 1) || groups < 0 || groups > 65535 || weight_groups < 1 ||
+            weight_groups > 65535 || rows < 0 || rows > 65535 || outputs < 8 || outputs % 8 ||
+            inner < 32 || inner % 32 ||
+            (activation_block != 32 && !(packed && activation_block == 128)) ||
+            inner % activation_block ||
+            uint64_t(groups) * uint64_t(rows) > SIZE_MAX / (uint64_t(outputs) * 2))
+            return fail(context, "invalid grouped matrix dimensions", 1);
+        if (!groups || !rows)
+            return 0;
+        if (!input || !input_scale || !metadata || !active || !counts || !output ||
+            !aligned(input, 16) || !aligned(metadata, 8) || !aligned(active, 4) ||
+            !aligned(counts, 4) || !aligned(output, 2) || output == input ||
+            output == input_scale || output == metadata || output == active || output == counts)
+            return fail(context, "invalid grouped matrix buffers", 1);
+        context->counts[4]++;
+        hipError_t error = launch_mx_matmul(context->stream, packed != 0, groups, weight_groups, rows,
+                                            outputs, inner, activation_block, input, input_scale,
+                                            nullptr, nullptr, metadata, active, counts, output);
+        return error == hipSuccess ? 0 : fail(context, "grouped multiplication", error);
+    });
+}
+
+// ref: src/cuda/backend.cu:1306-1337
+extern "C" int camblas_cuda_route_groups(camblas_cuda_context *context, int tokens, int choices,
+                                         int first_expert, int groups, int rows,
+                                         const void *experts, const void *active, void *counts,
+                                         void *slots, void *reverse)
+{
+    return execute(context, [&] {
+        if (tokens < 0 || choices < 1 || choices > 64 || first_expert < 0 || groups < 1 ||
+            groups > 65535 || rows < 1 || rows > 65535 || int64_t(tokens) * choices > INT_MAX ||
+            int64_t(groups) * rows > INT_MAX || !counts || !slots ||
+            (tokens && (!experts || !reverse)) || !active || !aligned(experts, 8) ||
+            !aligned(active, 4) || !aligned(counts, 4) || !aligned(slots, 4) ||
+            !aligned(reverse, 4) || counts == active || slots == active || reverse == active ||
+            counts == experts || slots == experts || (reverse && reverse == experts) ||
+            counts == slots || counts == reverse || slots == reverse)
+            return fail(context, "invalid routing dimensions or buffers", 1);
+        hipError_t error = launch_route_groups(context->stream, tokens, choices, first_expert, groups,
+                                               rows, experts, active, counts, slots, reverse);
+        return error == hipSuccess ? 0 : fail(context, "expert routing", error);
+    });
+}
+
+// ref: src/cuda/backend.cu:1339-1361
+extern "C" int camblas_cuda_reduce_groups(camblas_cuda_context *context, int tokens, int choices,
+                                          int width, int grouped_rows, const void *experts,
+                                          const void *reverse, const void *input, void *output)
+{
+    return execute(context, [&] {
+        if (tokens < 0 || choices < 1 || choices > 64 || width < 1 || grouped_rows < 0 ||
+            int64_t(tokens) * choices > INT_MAX || (grouped_rows && !input) ||
+            (tokens && (!experts || !reverse || !output)) || !aligned(experts, 8) ||
+            !aligned(reverse, 4) || !aligned(input, 2) || !aligned(output, 4) ||
+            (tokens && (output == experts || output == reverse || output == input)))
+            return fail(context, "invalid grouped reduction arguments", 1);
+        if (!tokens)
+            return 0;
+        hipError_t error = launch_reduce_groups(context->stream, tokens, choices, width, grouped_rows,
+                                                experts, reverse, input, output);
+        return error == hipSuccess ? 0 : fail(context, "grouped reduction", error);
+    });
+}
+
 // ref: src/cuda/backend.cu:1193-1256 (validation order and messages of the block-32 decode pair)
 extern "C" int camblas_cuda_fp8_decode_supported(const camblas_cuda_context *context)
 {

@@ -123,6 +123,18 @@ hipError_t launch_fp8_stream(hipStream_t stream, int row_tiles, int token_tiles,
 hipError_t launch_fp8_block32_decode(hipStream_t stream, int outputs, int inner, const void *x,
                                      const float *sx, int sx_stride, const void *w, const float *sw,
                                      int sw_row, int sw_col, void *out);
+// E8M0 block-scaled product (E4M3 or packed E2M1 weights); groups == 0 plain, >= 1 grouped.
+hipError_t launch_mx_matmul(hipStream_t stream, bool packed, int groups, int weight_groups, int rows,
+                            int outputs, int inner, int activation_block, const void *input,
+                            const void *input_scale, const void *weight, const void *weight_scale,
+                            const void *metadata, const void *active, const void *counts, void *out);
+// Mixture-of-experts routing helpers.
+hipError_t launch_route_groups(hipStream_t stream, int tokens, int choices, int first_expert,
+                               int groups, int rows, const void *experts, const void *active,
+                               void *counts, void *slots, void *reverse);
+hipError_t launch_reduce_groups(hipStream_t stream, int tokens, int choices, int width,
+                                int grouped_rows, const void *experts, const void *reverse,
+                                const void *input, void *output);
 hipError_t launch_fp8_quantise(hipStream_t stream, int rows, int inner, const void *x, void *q,
                                float *scale);
 hipError_t launch_silu_multiply(hipStream_t stream, int dtype, uint64_t count, const void *gate,

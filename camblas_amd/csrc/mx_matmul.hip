@@ -1,0 +1,348 @@
+// Block-scaled (microscaling) linear with E8M0 scales: out[M,N] = x[M,K] . w[N,K]^T, x E4M3 with one
+// E8M0 scale per 32 (or 128) inputs, w either E4M3 with one scale per 32 x 32 block or packed E2M1
+// (two values per byte, low nibble first) with one scale per row and 32 inputs, FP32 accumulation,
+// BF16 out; plus the grouped form that picks weights per group from a device table (contract: ref
+// include/camblas_cuda.h:110-167, src/cuda/backend.cu:1165-1191, :1258-1303; value semantics pinned
+// by the byte decoder of the reference's tests/test_quantized.py:12-50: a scale byte e means
+// 2^(e-127), 255 means NaN).
+//
+// This is the operation gfx950's v_mfma_scale_f32_16x16x128_f8f6f4 implements natively: every lane
+// supplies 32 consecutive K elements of its row (E4M3 or E2M1, chosen per operand) together with
+// one E8M0 scale byte, and the instruction accumulates the scaled products in FP32. One 128-input
+// group is one instruction per 16 x 16 tile, with no vector-ALU arithmetic at all.
+//
+// Operand layout of the instruction, as measured with single-element probes: call the 128 K
+// positions of a group p and its four 32-input blocks b = p/32. A lane group c = lane/16 of a
+// 4-bit operand holds positions 32c .. 32c+31; a lane group of an 8-bit operand holds positions
+// 16c .. 16c+15 in its first 16 bytes and 64+16c .. 64+16c+15 in its second 16 bytes; and the scale
+// byte supplied by lane group b applies to block b of that lane's row, whichever lanes hold the
+// block's data. The loads below follow exactly this (an 8-bit lane reads two 16-byte pieces 64
+// bytes apart), so one instruction handles E2M1 weights against E4M3 inputs with independent
+// 32-input scales on both sides.
+//
+// The kernel streams the weights like the other decode kernels: a workgroup owns 16*NT weight rows
+// for the whole K extent and up to 16*MT tokens, its four wavefronts take groups g = 4s + wave,
+// load their group of a tile with whole-line 128-bit loads (non-temporal), transpose it to the
+// operand layout through a private swizzled LDS patch (no barrier: LDS operations of one wavefront
+// execute in order) and the four partial sums are added in wavefront order at the end.
+#include "common.hpp"
+#include "device.hpp"
+
+namespace camblas_hip
+{
+namespace
+{
+struct MxParams {
+    const unsigned char *input;
+    const unsigned char *input_scale;
+    const unsigned char *weight;
+    const unsigned char *weight_scale;
+    unsigned short *out;
+    int rows, outputs, inner, scale_shift; // activation scale covers 32 << scale_shift inputs
+    // grouped form
+    const unsigned long long *metadata;
+    const int32_t *active, *counts;
+    int weight_groups;
+};
+
+constexpr int WAVES = 4, GROUP = 128;
+
+template <bool PACKED, bool GROUPED, int NT, int MT>
+__global__ __launch_bounds__(WAVES * 64) void mx_stream_kernel(MxParams p)
+{
+    constexpr int DEPTH = NT + MT <= 6 ? 3 : 2;
+    constexpr int LOADS = PACKED ? 1 : 2;             // 16-byte loads per lane, weight tile and group
+    constexpr int ROW_BYTES = PACKED ? 64 : 128;      // weight bytes per row and group
+    __shared__ __attribute__((aligned(16))) u32x4_t patch[WAVES][NT][PACKED ? 64 : 128];
+    __shared__ __attribute__((aligned(16))) f32x4_t combine[NT * MT * 64];
+    const int thread = threadIdx.x, lane = thread % 64, wave = thread / 64;
+    const int row = lane % 16, chunk = lane / 16; // operand row / token, 32-input chunk of the group
+    const int n0 = blockIdx.x * (NT * 16), m0 = blockIdx.y * (MT * 16);
+    const int blocks = p.inner / 32, groups = (p.inner + GROUP - 1) / GROUP;
+    const int steps = (groups + WAVES - 1) / WAVES;
+    const size_t weight_pitch = PACKED ? size_t(p.inner) / 2 : size_t(p.inner);
+
+    const unsigned char *input = p.input, *input_scale = p.input_scale, *weight = p.weight,
+                        *weight_scale = p.weight_scale;
+    unsigned short *out = p.out;
+    int valid_rows = p.rows;
+    if constexpr (GROUPED) {
+        // ref: include/camblas_cuda.h:156-167 — weights come from a device table indexed by
+        // active[group]; invalid indices and rows at or beyond counts[group] produce zeros
+        const int group = blockIdx.z;
+        const int index = p.active[group];
+        const int count = p.counts[group];
+        valid_rows = index >= 0 && index < p.weight_groups ? min(max(count, 0), p.rows) : 0;
+        input += size_t(group) * p.rows * p.inner;
+        input_scale += size_t(group) * p.rows * (p.inner >> (5 + p.scale_shift));
+        out += size_t(group) * p.rows * p.outputs;
+        if (m0 >= valid_rows) { // nothing to multiply: this tile of the output is zero
+            for (int index2 = thread; index2 < MT * 16 * NT * 16; index2 += WAVES * 64) {
+                const int m = m0 + index2 / (NT * 16), n = n0 + index2 % (NT * 16);
+                if (m < p.rows && n < p.outputs)
+                    out[size_t(m) * p.outputs + n] = 0;
+            }
+            return;
+        }
+        weight = reinterpret_cast<const unsigned char *>(p.metadata[2 * size_t(index)]);
+        weight_scale = reinterpret_cast<const unsigned char *>(p.metadata[2 * size_t(index) + 1]);
+    }
+
+    // ---- per-lane sources. Weight tile loads: 8 (E4M3) or 4 (E2M1) lanes per row segment.
+    constexpr int LANES_PER_ROW = PACKED ? 4 : 8;
+    const int load_row = lane / LANES_PER_ROW, piece = lane % LANES_PER_ROW;
+    const unsigned char *w_source[NT][LOADS];
+    const unsigned char *ws_source[NT];
+#pragma unroll
+    for (int i = 0; i < NT; ++i) {
+#pragma unroll
+        for (int h = 0; h < LOADS; ++h) {
+            int n = n0 + i * 16 + h * 8 + load_row; // LOADS == 1: 16 rows in one load
+            n = n < p.outputs ? n : p.outputs - 1;
+            w_source[i][h] = weight + size_t(n) * weight_pitch;
+        }
+        int n = n0 + i * 16 + row;
+        n = n < p.outputs ? n : p.outputs - 1;
+        // E4M3 weights: one scale per 32 x 32 block; E2M1 weights: one per row and 32 inputs
+        ws_source[i] = weight_scale + size_t(PACKED ? n : n / 32) * blocks;
+    }
+    const unsigned char *x_source[MT], *xs_source[MT];
+#pragma unroll
+    for (int j = 0; j < MT; ++j) {
+        int m = m0 + j * 16 + row;
+        m = m < valid_rows ? m : valid_rows - 1;
+        x_source[j] = input + size_t(m) * p.inner;
+        xs_source[j] = input_scale + size_t(m) * (blocks >> p.scale_shift);
+    }
+    // LDS patch of one weight tile, XOR-swizzled so that the line-shaped stores and the
+    // operand-shaped loads are both conflict-free
+    auto slot = [](int r, int q) {
+        return PACKED ? r * 4 + (q ^ ((r >> 2) & 3)) : r * 8 + (q ^ ((r >> 1) & 7));
+    };
+    int store_slot[LOADS], read_slot[LOADS];
+#pragma unroll
+    for (int h = 0; h < LOADS; ++h) {
+        store_slot[h] = slot(load_row + 8 * h, piece);
+        read_slot[h] = PACKED ? slot(row, chunk) : slot(row, chunk + 4 * h); // pieces c and 4 + c
+    }
+
+    // Workgroups start at different groups and wrap around (spreads the row-pitch-strided requests
+    // over the HBM channels). Steps past the end re-read the last group with zeroed activations.
+    const int start = int(blockIdx.x % unsigned(steps));
+    auto group_of = [&](int step) {
+        int rotated = (step < steps ? step : steps - 1) + start;
+        rotated = rotated < steps ? rotated : rotated - steps;
+        return rotated * WAVES + wave;
+    };
+    u32x4_t w_raw[DEPTH][NT][LOADS], x_raw[DEPTH][MT][2];
+    unsigned ws_raw[DEPTH][NT], xs_raw[DEPTH][MT], keep_raw[DEPTH][2];
+    // Loads only: nothing here may use a loaded value, or the wait would cover the newest loads.
+    auto fetch = [&](int step, u32x4_t(&w)[NT][LOADS], u32x4_t(&x)[MT][2], unsigned(&ws)[NT],
+                     unsigned(&xs)[MT], unsigned(&keep)[2]) {
+        int g = group_of(step);
+        const bool live = step < steps && g < groups;
+        g = g < groups ? g : groups - 1;
+        int block = g * 4 + chunk; // the 32-input block whose scales this lane supplies
+        block = block < blocks ? block : blocks - 1;
+        // the lane's two 16-byte input pieces: positions 16c.. (block c/2) and 64+16c.. (block 2+c/2)
+        int half_offset[2] = {g * GROUP + chunk * 16, g * GROUP + 64 + chunk * 16};
+#pragma unroll
+        for (int h = 0; h < 2; ++h) {
+            keep[h] = live && half_offset[h] < p.inner ? 0xffffffffu : 0u;
+            half_offset[h] = half_offset[h] < p.inner ? half_offset[h] : p.inner - 16;
+        }
+#pragma unroll
+        for (int i = 0; i < NT; ++i) {
+#pragma unroll
+            for (int h = 0; h < LOADS; ++h) {
+                // bytes past the end of the row in a partial last group re-read its last 16 bytes
+                size_t offset = size_t(g) * ROW_BYTES + piece * 16;
+                offset = offset < weight_pitch ? offset : weight_pitch - 16;
+                w[i][h] = __builtin_nontemporal_load(
+                    reinterpret_cast<const u32x4_t *>(w_source[i][h] + offset));
+            }
+            ws[i] = ws_source[i][block];
+        }
+#pragma unroll
+        for (int j = 0; j < MT; ++j) {
+#pragma unroll
+            for (int h = 0; h < 2; ++h)
+                x[j][h] = *reinterpret_cast<const u32x4_t *>(x_source[j] + half_offset[h]);
+            xs[j] = xs_source[j][block >> p.scale_shift];
+        }
+    };
+
+    f32x4_t acc[NT][MT];
+#pragma unroll
+    for (int i = 0; i < NT; ++i)
+#pragma unroll
+        for (int j = 0; j < MT; ++j)
+            acc[i][j] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+    auto multiply = [&](const u32x4_t(&w)[NT][LOADS], const u32x4_t(&x)[MT][2],
+                        const unsigned(&ws)[NT], const unsigned(&xs)[MT], const unsigned(&keep)[2]) {
+        u32x4_t *mine = &patch[wave][0][0];
+        constexpr int TILE = PACKED ? 64 : 128;
+#pragma unroll
+        for (int i = 0; i < NT; ++i)
+#pragma unroll
+            for (int h = 0; h < LOADS; ++h)
+                mine[i * TILE + store_slot[h]] = w[i][h];
+        // other lanes' stores are read below: keep the compiler from moving the loads up
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+        i32x8_t a[NT];
+#pragma unroll
+        for (int i = 0; i < NT; ++i) {
+            u32x4_t lo = mine[i * TILE + read_slot[0]];
+            u32x4_t hi = PACKED ? u32x4_t{0u, 0u, 0u, 0u} : mine[i * TILE + read_slot[LOADS - 1]];
+            a[i] = i32x8_t{int(lo[0]), int(lo[1]), int(lo[2]), int(lo[3]),
+                           int(hi[0]), int(hi[1]), int(hi[2]), int(hi[3])};
+        }
+        // inputs past the end of K (and of dead steps) are zero
+#pragma unroll
+        for (int j = 0; j < MT; ++j) {
+            const u32x4_t lo = x[j][0] & keep[0], hi = x[j][1] & keep[1];
+            const i32x8_t b = {int(lo[0]), int(lo[1]), int(lo[2]), int(lo[3]),
+                               int(hi[0]), int(hi[1]), int(hi[2]), int(hi[3])};
+#pragma unroll
+            for (int i = 0; i < NT; ++i)
+                acc[i][j] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(
+                    a[i], b, acc[i][j], PACKED ? 4 : 0, 0, 0, int(ws[i]), 0, int(xs[j]));
+        }
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+    };
+
+#pragma unroll
+    for (int d = 0; d < DEPTH; ++d) {
+        fetch(d, w_raw[d], x_raw[d], ws_raw[d], xs_raw[d], keep_raw[d]);
+        __builtin_amdgcn_sched_barrier(0);
+    }
+    for (int step = 0; step < steps; step += DEPTH) {
+#pragma unroll
+        for (int d = 0; d < DEPTH; ++d) {
+            __builtin_amdgcn_sched_barrier(0);
+            multiply(w_raw[d], x_raw[d], ws_raw[d], xs_raw[d], keep_raw[d]);
+            __builtin_amdgcn_sched_barrier(0);
+            fetch(step + d + DEPTH, w_raw[d], x_raw[d], ws_raw[d], xs_raw[d], keep_raw[d]);
+        }
+    }
+    __syncthreads();
+
+    // ---- add the four wavefronts' partial sums in wavefront order through LDS
+#pragma unroll
+    for (int w = 0; w < WAVES; ++w) {
+        if (wave == w) {
+#pragma unroll
+            for (int i = 0; i < NT; ++i)
+#pragma unroll
+                for (int j = 0; j < MT; ++j) {
+                    f32x4_t *cell = combine + (i * MT + j) * 64 + lane;
+                    *cell = w == 0 ? acc[i][j] : *cell + acc[i][j];
+                }
+        }
+        __syncthreads();
+    }
+    // ---- epilogue: register r of lane l is feature 4*(l/16) + r and token l%16 of the tile
+#pragma unroll
+    for (int index = 0; index < NT * MT; ++index) {
+        if (index % WAVES != wave)
+            continue;
+        const int i = index / MT, j = index % MT;
+        const int m = m0 + j * 16 + row;
+        const int n = n0 + i * 16 + chunk * 4;
+        if (m >= p.rows || n >= p.outputs)
+            continue;
+        f32x4_t sum = combine[index * 64 + lane];
+        unsigned short *target = out + size_t(m) * p.outputs + n;
+        const bool zero = GROUPED && m >= valid_rows; // padding rows of a group
+        // outputs is a multiple of eight, so the four features are all inside the matrix
+#pragma unroll
+        for (int e = 0; e < 4; ++e)
+            target[e] = zero ? (unsigned short)0 : float_to_bf16_bits(sum[e]);
+    }
+}
+
+template <bool PACKED, bool GROUPED, int NT, int MT>
+hipError_t launch_one(hipStream_t stream, const MxParams &p, int groups)
+{
+    if constexpr (NT * MT > 16 || NT + MT > 10) {
+        return hipErrorInvalidValue;
+    } else {
+        dim3 grid(unsigned((p.outputs + NT * 16 - 1) / (NT * 16)),
+                  unsigned((p.rows + MT * 16 - 1) / (MT * 16)), unsigned(groups));
+        mx_stream_kernel<PACKED, GROUPED, NT, MT><<<grid, WAVES * 64, 0, stream>>>(p);
+        return launch_status();
+    }
+}
+
+template <bool PACKED, bool GROUPED>
+hipError_t launch_shape(hipStream_t stream, const MxParams &p, int groups)
+{
+    // token tiles by row count; weight-row tiles so that about one workgroup lands on each compute
+    // unit (decode-sized calls: the kernel is bound by the weight stream)
+    const int token_tiles = p.rows <= 16 ? 1 : p.rows <= 32 ? 2 : 4;
+    const int tiles = (p.outputs + 15) / 16;
+    int row_tiles = 1;
+    for (int candidate = token_tiles == 4 ? 4 : 8; candidate > 1; --candidate)
+        if (tiles / candidate >= 192) {
+            row_tiles = candidate;
+            break;
+        }
+#define CAMBLAS_MX(NT, MT) launch_one<PACKED, GROUPED, NT, MT>(stream, p, groups)
+    switch (token_tiles * 10 + row_tiles) {
+    case 11: return CAMBLAS_MX(1, 1);
+    case 12: return CAMBLAS_MX(2, 1);
+    case 13: return CAMBLAS_MX(3, 1);
+    case 14: return CAMBLAS_MX(4, 1);
+    case 15: return CAMBLAS_MX(5, 1);
+    case 16: return CAMBLAS_MX(6, 1);
+    case 17: return CAMBLAS_MX(7, 1);
+    case 18: return CAMBLAS_MX(8, 1);
+    case 21: return CAMBLAS_MX(1, 2);
+    case 22: return CAMBLAS_MX(2, 2);
+    case 23: return CAMBLAS_MX(3, 2);
+    case 24: return CAMBLAS_MX(4, 2);
+    case 25: return CAMBLAS_MX(5, 2);
+    case 26: return CAMBLAS_MX(6, 2);
+    case 27: return CAMBLAS_MX(7, 2);
+    case 28: return CAMBLAS_MX(8, 2);
+    case 41: return CAMBLAS_MX(1, 4);
+    case 42: return CAMBLAS_MX(2, 4);
+    case 43: return CAMBLAS_MX(3, 4);
+    default: return CAMBLAS_MX(4, 4);
+    }
+#undef CAMBLAS_MX
+}
+} // namespace
+
+// groups == 0: plain product (weight, weight_scale given); groups >= 1: grouped product (metadata,
+// active, counts given). activation_block 32 or 128. Weights 16-byte aligned.
+hipError_t launch_mx_matmul(hipStream_t stream, bool packed, int groups, int weight_groups, int rows,
+                            int outputs, int inner, int activation_block, const void *input,
+                            const void *input_scale, const void *weight, const void *weight_scale,
+                            const void *metadata, const void *active, const void *counts, void *out)
+{
+    MxParams p;
+    p.input = static_cast<const unsigned char *>(input);
+    p.input_scale = static_cast<const unsigned char *>(input_scale);
+    p.weight = static_cast<const unsigned char *>(weight);
+    p.weight_scale = static_cast<const unsigned char *>(weight_scale);
+    p.out = static_cast<unsigned short *>(out);
+    p.rows = rows;
+    p.outputs = outputs;
+    p.inner = inner;
+    p.scale_shift = activation_block == 128 ? 2 : 0;
+    p.metadata = static_cast<const unsigned long long *>(metadata);
+    p.active = static_cast<const int32_t *>(active);
+    p.counts = static_cast<const int32_t *>(counts);
+    p.weight_groups = weight_groups;
+    if ((rows + 15) / 16 > 65535 || groups > 65535)
+        return hipErrorInvalidValue;
+    if (groups == 0)
+        return packed ? launch_shape<true, false>(stream, p, 1) : launch_shape<false, false>(stream, p, 1);
+    return packed ? launch_shape<true, true>(stream, p, groups)
+                  : launch_shape<false, true>(stream, p, groups);
+}
+} // namespace camblas_hip

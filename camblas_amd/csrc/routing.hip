@@ -1,0 +1,169 @@
+// Mixture-of-experts routing helpers (contract: ref include/camblas_cuda.h:168-185,
+// src/cuda/backend.cu:1306-1361, src/cuda/routing.cuh:1-56).
+//
+// route_groups: expert IDs [tokens, choices] (int64) -> for every local group (active[g] is the
+// local expert ID it serves, the first group wins for duplicates) the list of (token, choice)
+// slots routed to it, `rows` at most, and for every slot its position in that list. The reference
+// hands rows out with an atomic counter, so its row order inside a group depends on scheduling;
+// here a group's rows are assigned in ascending slot order (one workgroup per group, ballot
+// prefix sums), which is one of the orders the contract allows and makes the result reproducible.
+// counts[g] is the number of slots routed to the group, including those beyond `rows`.
+//
+// reduce_groups: out[token, :] = sum over the token's choices, in ascending (expert ID, choice)
+// order, of the BF16 row reverse[token, choice] of the grouped matrix, accumulated in FP32.
+#include "common.hpp"
+#include "device.hpp"
+
+#include <climits>
+
+namespace camblas_hip
+{
+namespace
+{
+constexpr int THREADS = 256;
+
+__global__ __launch_bounds__(THREADS) void route_fill_kernel(int groups, size_t slot_cells,
+                                                             size_t reverse_cells, int32_t *counts,
+                                                             int32_t *slots, int32_t *reverse)
+{
+    const size_t stride = size_t(gridDim.x) * blockDim.x;
+    const size_t first = size_t(blockIdx.x) * blockDim.x + threadIdx.x;
+    for (size_t index = first; index < size_t(groups); index += stride)
+        counts[index] = 0;
+    for (size_t index = first; index < slot_cells; index += stride)
+        slots[index] = -1;
+    for (size_t index = first; index < reverse_cells; index += stride)
+        reverse[index] = -1;
+}
+
+__global__ __launch_bounds__(THREADS) void route_assign_kernel(int slot_count, int first_expert,
+                                                               int rows, const int64_t *experts,
+                                                               const int32_t *active, int32_t *counts,
+                                                               int32_t *slots, int32_t *reverse)
+{
+    __shared__ int wave_total[THREADS / 64];
+    __shared__ int earlier;
+    const int group = blockIdx.x, thread = threadIdx.x, lane = thread % 64, wave = thread / 64;
+    const int local = active[group];
+    // duplicate active IDs select their first group: a later one receives nothing
+    if (thread == 0)
+        earlier = 0;
+    __syncthreads();
+    for (int other = thread; other < group; other += THREADS)
+        if (active[other] == local)
+            earlier = 1;
+    __syncthreads();
+    if (earlier)
+        return; // counts[group] stays 0, slots stay -1
+    int assigned = 0; // uniform over the workgroup
+    for (int base = 0; base < slot_count; base += THREADS) {
+        const int slot = base + thread;
+        bool mine = false;
+        if (slot < slot_count) {
+            const int64_t expert = experts[slot];
+            mine = expert >= first_expert && expert < INT_MAX && int(expert) - first_expert == local;
+        }
+        const unsigned long long ballot = __ballot(mine);
+        const int before = __popcll(ballot & ((1ull << lane) - 1ull));
+        if (lane == 0)
+            wave_total[wave] = __popcll(ballot);
+        __syncthreads();
+        int offset = assigned, total = 0;
+#pragma unroll
+        for (int w = 0; w < THREADS / 64; ++w) {
+            if (w < wave)
+                offset += wave_total[w];
+            total += wave_total[w];
+        }
+        const int row = offset + before;
+        if (mine && row < rows) {
+            slots[size_t(group) * rows + row] = slot;
+            reverse[slot] = group * rows + row;
+        }
+        assigned += total;
+        __syncthreads();
+    }
+    if (thread == 0)
+        counts[group] = assigned;
+}
+
+// One workgroup per token: the choices are ranked by (expert ID, choice) once, then every thread
+// sums its columns in that order.
+__global__ __launch_bounds__(THREADS) void reduce_groups_kernel(int choices, int width,
+                                                                int grouped_rows,
+                                                                const int64_t *experts,
+                                                                const int32_t *reverse,
+                                                                const unsigned short *input,
+                                                                float *output)
+{
+    __shared__ int ordered_row[64];
+    __shared__ int ordered_count;
+    const int token = blockIdx.x, thread = threadIdx.x;
+    const int64_t *mine = experts + size_t(token) * choices;
+    if (thread < 64)
+        ordered_row[thread] = -1;
+    __syncthreads();
+    if (thread < choices) {
+        const int64_t expert = mine[thread];
+        const bool valid = expert >= 0 && expert < INT_MAX;
+        int rank = 0, valid_total = 0;
+        for (int other = 0; other < choices; ++other) {
+            const int64_t theirs = mine[other];
+            const bool theirs_valid = theirs >= 0 && theirs < INT_MAX;
+            valid_total += theirs_valid;
+            rank += theirs_valid && (theirs < expert || (theirs == expert && other < thread));
+        }
+        if (valid) {
+            const int row = reverse[size_t(token) * choices + thread];
+            ordered_row[rank] = row >= 0 && row < grouped_rows ? row : -1;
+        }
+        if (thread == 0)
+            ordered_count = valid_total;
+    }
+    __syncthreads();
+    const int count = ordered_count;
+    for (int column = thread; column < width; column += THREADS) {
+        float sum = 0.f;
+        for (int step = 0; step < count; ++step) {
+            const int row = ordered_row[step];
+            if (row >= 0)
+                sum = __fadd_rn(sum, bf16_bits_to_float(input[size_t(row) * width + column]));
+        }
+        output[size_t(token) * width + column] = sum;
+    }
+}
+} // namespace
+
+hipError_t launch_route_groups(hipStream_t stream, int tokens, int choices, int first_expert,
+                               int groups, int rows, const void *experts, const void *active,
+                               void *counts, void *slots, void *reverse)
+{
+    const size_t slot_cells = size_t(groups) * rows, reverse_cells = size_t(tokens) * choices;
+    const size_t cells = slot_cells > reverse_cells ? slot_cells : reverse_cells;
+    const unsigned blocks = unsigned(std::min<size_t>((cells + THREADS - 1) / THREADS + 1, 4096));
+    // a fill kernel rather than memset nodes, so that the call can be captured in a graph
+    route_fill_kernel<<<blocks, THREADS, 0, stream>>>(groups, slot_cells, reverse_cells,
+                                                      static_cast<int32_t *>(counts),
+                                                      static_cast<int32_t *>(slots),
+                                                      static_cast<int32_t *>(reverse));
+    hipError_t status = launch_status();
+    if (status != hipSuccess || !tokens)
+        return status;
+    route_assign_kernel<<<unsigned(groups), THREADS, 0, stream>>>(
+        tokens * choices, first_expert, rows, static_cast<const int64_t *>(experts),
+        static_cast<const int32_t *>(active), static_cast<int32_t *>(counts),
+        static_cast<int32_t *>(slots), static_cast<int32_t *>(reverse));
+    return launch_status();
+}
+
+hipError_t launch_reduce_groups(hipStream_t stream, int tokens, int choices, int width,
+                                int grouped_rows, const void *experts, const void *reverse,
+                                const void *input, void *output)
+{
+    reduce_groups_kernel<<<unsigned(tokens), THREADS, 0, stream>>>(
+        choices, width, grouped_rows, static_cast<const int64_t *>(experts),
+        static_cast<const int32_t *>(reverse), static_cast<const unsigned short *>(input),
+        static_cast<float *>(output));
+    return launch_status();
+}
+} // namespace camblas_hip

@@ -613,6 +613,204 @@ Tensor fp8_block32_product(const Tensor &x, const std::optional<Tensor> &x_scale
     return result;
 }
 
+// E8M0 block-scaled products and mixture-of-experts routing
+// (ref: src/cuda/torch_bindings.cpp:328-378, :462-600).
+void check_quantized_operand(const Tensor &tensor, const Tensor &like)
+{
+    require(tensor.device() == like.device() && tensor.is_contiguous(),
+            "Quantized operands must be contiguous and on the same GPU");
+    require(!c10::GradMode::is_enabled() || !tensor.requires_grad(),
+            "Quantized multiplication supports inference only");
+    for (int64_t size : tensor.sizes())
+        require(size <= INT_MAX, "LP64 dimension overflow");
+}
+
+Tensor quantized_matmul_public(const Tensor &x, const Tensor &x_scale, const Tensor &weight,
+                               const Tensor &weight_scale, int activation_block)
+{
+    same_process();
+    require(x.is_cuda() && x.scalar_type() == at::kFloat8_e4m3fn, "Quantized input must be GPU FP8 E4M3");
+    const bool packed = weight.scalar_type() == at::ScalarType::Float4_e2m1fn_x2;
+    require(packed || weight.scalar_type() == at::kFloat8_e4m3fn,
+            "Quantized weight must be FP8 E4M3 or packed FP4 E2M1");
+    require(x_scale.scalar_type() == at::ScalarType::Float8_e8m0fnu &&
+                weight_scale.scalar_type() == at::ScalarType::Float8_e8m0fnu,
+            "Quantized scales must be E8M0");
+    for (const Tensor *tensor : {&x, &x_scale, &weight, &weight_scale})
+        check_quantized_operand(*tensor, x);
+    require(x.dim() >= 1 && weight.dim() == 2 && x_scale.dim() == x.dim() && weight_scale.dim() == 2,
+            "Quantized matrix and scale ranks do not match");
+    const int64_t inner = x.size(-1), outputs = weight.size(0);
+    int64_t rows = 1;
+    require(inner >= 32 && inner % 32 == 0 && outputs >= 8 && outputs % 8 == 0 &&
+                weight.size(1) == inner / (packed ? 2 : 1) &&
+                (activation_block == 32 || (packed && activation_block == 128)) &&
+                inner % activation_block == 0,
+            "Invalid quantized matrix dimensions or activation block");
+    for (int64_t index = 0; index + 1 < x.dim(); ++index) {
+        require(x_scale.size(index) == x.size(index), "Input scale shape mismatch");
+        require(rows <= 65535 / std::max<int64_t>(1, x.size(index)),
+                "Quantized multiplication supports at most 65535 rows");
+        rows *= x.size(index);
+    }
+    require(x_scale.size(-1) == inner / activation_block &&
+                weight_scale.size(0) == (packed ? outputs : (outputs + 31) / 32) &&
+                weight_scale.size(1) == inner / 32,
+            "Quantized scale shapes do not match their blocks");
+    c10::DeviceGuard guard(x.device());
+    auto shape = x.sizes().vec();
+    shape.back() = outputs;
+    Tensor result = at::empty(shape, x.options().dtype(at::kBFloat16));
+    camblas_cuda_context *context = context_for(x.get_device(), default_algorithm);
+    succeed(camblas_cuda_quantized_matmul(context, packed, int(rows), int(outputs), int(inner),
+                                          activation_block, x.const_data_ptr(),
+                                          x_scale.const_data_ptr(), weight.const_data_ptr(),
+                                          weight_scale.const_data_ptr(), result.mutable_data_ptr()),
+            context);
+    return result;
+}
+
+// Keeps the weight and scale tensors of every expert alive and their addresses in a device table;
+// in-place updates of the values are seen by later calls, a relocated storage is refused.
+struct QuantizedGroups {
+    std::vector<Tensor> weights, scales;
+    Tensor table; // int64 [groups, 2] on the device
+    int outputs = 0, inner = 0;
+    bool packed = false, trainable = false;
+
+    QuantizedGroups(const std::vector<Tensor> &group_weights, const std::vector<Tensor> &group_scales)
+    {
+        same_process();
+        require(!group_weights.empty() && group_weights.size() <= 65535 &&
+                    group_weights.size() == group_scales.size(),
+                "Supply matching non-empty weight and scale groups");
+        const Tensor &first = group_weights[0];
+        require(first.is_cuda() && first.dim() == 2, "Grouped weights must be GPU matrices");
+        packed = first.scalar_type() == at::ScalarType::Float4_e2m1fn_x2;
+        require(packed || first.scalar_type() == at::kFloat8_e4m3fn,
+                "Grouped weights require FP8 or packed FP4 storage");
+        require(first.size(0) >= 8 && first.size(0) <= INT_MAX && first.size(0) % 8 == 0 &&
+                    first.size(1) >= (packed ? 16 : 32) && first.size(1) <= INT_MAX / (packed ? 2 : 1),
+                "Invalid grouped weight dimensions");
+        outputs = int(first.size(0));
+        inner = int(first.size(1)) * (packed ? 2 : 1);
+        require(inner % 32 == 0, "Grouped inner dimension must be a multiple of 32");
+        Tensor host = at::empty({int64_t(group_weights.size()), 2},
+                                at::TensorOptions().device(at::kCPU).dtype(at::kLong));
+        int64_t *addresses = host.mutable_data_ptr<int64_t>();
+        for (size_t index = 0; index < group_weights.size(); ++index) {
+            const Tensor &w = group_weights[index], &s = group_scales[index];
+            require(w.device() == first.device() && w.scalar_type() == first.scalar_type() &&
+                        w.sizes() == first.sizes() && w.is_contiguous() &&
+                        uintptr_t(w.const_data_ptr()) % 16 == 0 && s.device() == first.device() &&
+                        s.scalar_type() == at::ScalarType::Float8_e8m0fnu && s.dim() == 2 &&
+                        s.size(0) == (packed ? outputs : (outputs + 31LL) / 32) &&
+                        s.size(1) == inner / 32 && s.is_contiguous(),
+                    "Grouped weight shapes, dtypes, devices or scales differ");
+            trainable |= w.requires_grad() || s.requires_grad();
+            weights.push_back(w.detach());
+            scales.push_back(s.detach());
+            addresses[2 * index] = int64_t(uintptr_t(w.const_data_ptr()));
+            addresses[2 * index + 1] = int64_t(uintptr_t(s.const_data_ptr()));
+        }
+        c10::DeviceGuard guard(first.device());
+        table = host.to(first.device());
+        host_table = host;
+    }
+
+    Tensor matmul(const Tensor &x, const Tensor &x_scale, const Tensor &active, const Tensor &counts,
+                  int activation_block)
+    {
+        same_process();
+        require(!c10::GradMode::is_enabled() || (!trainable && !x.requires_grad()),
+                "Grouped multiplication supports inference only");
+        require(x.device() == table.device() && x.scalar_type() == at::kFloat8_e4m3fn &&
+                    x.dim() == 3 && x.size(0) <= 65535 && x.size(1) <= 65535 && x.size(2) == inner &&
+                    (activation_block == 32 || (packed && activation_block == 128)) &&
+                    inner % activation_block == 0,
+                "Invalid grouped input dimensions or activation block");
+        require(x_scale.device() == x.device() &&
+                    x_scale.scalar_type() == at::ScalarType::Float8_e8m0fnu && x_scale.dim() == 3 &&
+                    x_scale.size(0) == x.size(0) && x_scale.size(1) == x.size(1) &&
+                    x_scale.size(2) == inner / activation_block,
+                "Grouped input scale shape or dtype mismatch");
+        for (const Tensor *index : {&active, &counts})
+            require(index->device() == x.device() && index->scalar_type() == at::kInt &&
+                        index->dim() == 1 && index->numel() == x.size(0),
+                    "Grouped indices/counts require one GPU int32 value per group");
+        for (const Tensor *value : {&x, &x_scale, &active, &counts})
+            require(value->is_contiguous(), "Grouped operands must be contiguous");
+        const int64_t *addresses = host_table.const_data_ptr<int64_t>();
+        for (size_t index = 0; index < weights.size(); ++index)
+            require(int64_t(uintptr_t(weights[index].const_data_ptr())) == addresses[2 * index] &&
+                        int64_t(uintptr_t(scales[index].const_data_ptr())) == addresses[2 * index + 1],
+                    "Captured weight storage changed; recreate the group");
+        c10::DeviceGuard guard(x.device());
+        Tensor result = at::empty({x.size(0), x.size(1), outputs}, x.options().dtype(at::kBFloat16));
+        camblas_cuda_context *context = context_for(x.get_device(), default_algorithm);
+        succeed(camblas_cuda_grouped_quantized_matmul(
+                    context, packed, int(x.size(0)), int(weights.size()), int(x.size(1)), outputs,
+                    inner, activation_block, x.const_data_ptr(), x_scale.const_data_ptr(),
+                    table.const_data_ptr(), active.const_data_ptr(), counts.const_data_ptr(),
+                    result.mutable_data_ptr()),
+                context);
+        return result;
+    }
+
+  private:
+    Tensor host_table;
+};
+
+std::tuple<Tensor, Tensor, Tensor> route_groups_public(const Tensor &experts, const Tensor &active,
+                                                       int first_expert, int rows)
+{
+    same_process();
+    require(experts.is_cuda() && experts.scalar_type() == at::kLong && experts.dim() == 2 &&
+                experts.is_contiguous() && experts.size(0) <= INT_MAX && experts.size(1) >= 1 &&
+                experts.size(1) <= 64 && experts.numel() <= INT_MAX &&
+                active.device() == experts.device() && active.scalar_type() == at::kInt &&
+                active.dim() == 1 && active.is_contiguous() && active.numel() >= 1 &&
+                active.numel() <= 65535 && rows >= 1 && rows <= 65535 &&
+                active.numel() * rows <= INT_MAX && first_expert >= 0,
+            "Invalid expert routing dimensions, indices or devices");
+    c10::DeviceGuard guard(experts.device());
+    Tensor counts = at::empty({active.numel()}, active.options());
+    Tensor slots = at::empty({active.numel(), rows}, active.options());
+    Tensor reverse = at::empty(experts.sizes(), active.options());
+    camblas_cuda_context *context = context_for(experts.get_device(), default_algorithm);
+    succeed(camblas_cuda_route_groups(context, int(experts.size(0)), int(experts.size(1)),
+                                      first_expert, int(active.numel()), rows,
+                                      experts.const_data_ptr(), active.const_data_ptr(),
+                                      counts.mutable_data_ptr(), slots.mutable_data_ptr(),
+                                      reverse.mutable_data_ptr()),
+            context);
+    return std::make_tuple(slots, reverse, counts);
+}
+
+Tensor reduce_groups_public(const Tensor &input, const Tensor &experts, const Tensor &reverse)
+{
+    same_process();
+    require(input.is_cuda() && input.scalar_type() == at::kBFloat16 && input.dim() == 3 &&
+                input.is_contiguous() && input.size(0) * input.size(1) <= INT_MAX &&
+                input.size(2) >= 1 && input.size(2) <= INT_MAX &&
+                experts.device() == input.device() && experts.scalar_type() == at::kLong &&
+                experts.dim() == 2 && experts.is_contiguous() && experts.size(0) <= INT_MAX &&
+                experts.size(1) >= 1 && experts.size(1) <= 64 && experts.numel() <= INT_MAX &&
+                reverse.device() == input.device() && reverse.scalar_type() == at::kInt &&
+                reverse.sizes() == experts.sizes() && reverse.is_contiguous() &&
+                (!c10::GradMode::is_enabled() || !input.requires_grad()),
+            "Invalid grouped reduction shapes, types, devices or gradients");
+    c10::DeviceGuard guard(input.device());
+    Tensor result = at::empty({experts.size(0), input.size(2)}, input.options().dtype(at::kFloat));
+    camblas_cuda_context *context = context_for(input.get_device(), default_algorithm);
+    succeed(camblas_cuda_reduce_groups(context, int(experts.size(0)), int(experts.size(1)),
+                                       int(input.size(2)), int(input.size(0) * input.size(1)),
+                                       experts.const_data_ptr(), reverse.const_data_ptr(),
+                                       input.const_data_ptr(), result.mutable_data_ptr()),
+            context);
+    return result;
+}
+
 // ---------------------------------------------------------------------------- ATen backend
 // Re-route aten::mm / mm.out / addmm on the GPU dispatch key. Anything the library does not take
 // goes to ATen's own GPU implementation through the at::cuda:: entry points, which bypass the
@@ -740,6 +938,30 @@ PYBIND11_MODULE(_camblas_cuda_torch, module)
                py::arg("input_scale"), py::arg("weight"), py::arg("weight_scale"),
                "Multiply E4M3fn activations (1x128 FP32 scales) by E4M3fn weights (128x128 FP32 "
                "scales), returning BF16.");
+    module.attr("quantized_tile_rows") = 16;
+    py::class_<QuantizedGroups>(module, "QuantizedGroups",
+                                "Capture GPU quantized weight storages and retain their lifetimes. "
+                                "In-place value updates are visible; recreate the group after "
+                                "storage relocation.")
+        .def(py::init<const std::vector<Tensor> &, const std::vector<Tensor> &>(), py::arg("weights"),
+             py::arg("scales"))
+        .def("matmul", &QuantizedGroups::matmul, py::arg("input"), py::arg("input_scale"),
+             py::arg("active"), py::arg("counts"), py::kw_only(), py::arg("activation_block") = 32,
+             "Multiply [groups,rows,inner] FP8 input with selected captured weights. Invalid "
+             "active indices and padding return zero; counts clip to [0,rows]. Inference only.");
+    module.def("route_groups", &route_groups_public, py::arg("experts"), py::arg("active"),
+               py::kw_only(), py::arg("first_expert") = 0, py::arg("rows"),
+               "Return slots, reverse mapping and counts for expert/choice IDs. Excess rows are "
+               "discarded and unassigned slots are -1; execution uses the active stream.");
+    module.def("reduce_groups", &reduce_groups_public, py::arg("input"), py::arg("experts"),
+               py::arg("reverse"),
+               "Sum BF16 contributions into FP32 in expert/choice order. Invalid IDs/rows are "
+               "ignored; requires inference and contiguous GPU tensors.");
+    module.def("quantized_matmul", &quantized_matmul_public, py::arg("input"), py::arg("input_scale"),
+               py::arg("weight"), py::arg("weight_scale"), py::kw_only(),
+               py::arg("activation_block") = 32,
+               "Multiply block-scaled FP8 input by FP8 or packed FP4 weights, returning BF16. "
+               "Requires contiguous GPU operands and E8M0 scales.");
     module.def("fp8_decode_supported", &fp8_decode_supported_public, py::arg("device") = -1,
                "Return whether this build and device support the block-32 FP8 decode product.");
     module.def(

@@ -129,6 +129,46 @@ int camblas_cuda_rms_scale(camblas_cuda_context *context, int dtype, uint64_t co
 int camblas_cuda_stats(const camblas_cuda_context *context, uint64_t *counts, int length);
 int camblas_cuda_reset_stats(camblas_cuda_context *context);
 
+/* Row-major FP8 E4M3 input [rows, inner] times weight [outputs, inner]^T with E8M0 block scales,
+ * FP32 accumulation, BF16 [rows, outputs]. packed=1: weights are E2M1 nibbles, low/high order,
+ * [outputs, inner/2] with scales [outputs, inner/32]; packed=0: E4M3 bytes with scales
+ * [ceil(outputs/32), inner/32]. Input scales are [rows, inner/activation_block]; activation_block
+ * is 32 (both) or 128 (E2M1 only). outputs a positive multiple of eight, inner of 32, rows
+ * 0..65535. ref: include/camblas_cuda.h:110-123, src/cuda/backend.cu:1165-1191. Runs on the
+ * scaled matrix-core instruction of gfx950, which applies the E8M0 scales itself. Input and weight
+ * must be 16-byte aligned here (the reference asks for 4 and 2/4). */
+int camblas_cuda_quantized_matmul(camblas_cuda_context *context, int packed, int rows, int outputs,
+                                  int inner, int activation_block, const void *input,
+                                  const void *input_scale, const void *weight,
+                                  const void *weight_scale, void *output);
+/* Batched form: input [groups, rows, inner], output [groups, rows, outputs]; metadata is device
+ * uint64 [weight_groups, 2] holding weight / scale addresses in the layouts above; active and
+ * counts are device int32 [groups]. Invalid active indices produce zeros, counts are clipped to
+ * [0, rows], padding rows are zeroed. ref: include/camblas_cuda.h:156-167,
+ * src/cuda/backend.cu:1258-1303. */
+int camblas_cuda_grouped_quantized_matmul(camblas_cuda_context *context, int packed, int groups,
+                                          int weight_groups, int rows, int outputs, int inner,
+                                          int activation_block, const void *input,
+                                          const void *input_scale, const void *metadata,
+                                          const void *active, const void *counts, void *output);
+
+/* Route int64 expert IDs [tokens, choices] to local int32 active IDs [groups]: initialises counts
+ * [groups], slots [groups, rows] and reverse [tokens, choices]; unassigned slots / reverse are -1,
+ * rows beyond `rows` are discarded (counts still counts them), duplicate active IDs select their
+ * first group, IDs outside [first_expert, INT_MAX) are ignored.
+ * ref: include/camblas_cuda.h:168-176, src/cuda/backend.cu:1306-1337. Rows of a group are handed
+ * out in ascending slot order (the reference's order depends on its atomic counter). */
+int camblas_cuda_route_groups(camblas_cuda_context *context, int tokens, int choices,
+                              int first_expert, int groups, int rows, const void *experts,
+                              const void *active, void *counts, void *slots, void *reverse);
+/* Sum BF16 grouped rows in ascending expert-ID / choice order into FP32 [tokens, width]; reverse
+ * maps [tokens, choices] to rows of input [grouped_rows, width]; negative or out-of-range expert
+ * IDs and rows are ignored; choices is 1..64.
+ * ref: include/camblas_cuda.h:177-185, src/cuda/backend.cu:1339-1361. */
+int camblas_cuda_reduce_groups(camblas_cuda_context *context, int tokens, int choices, int width,
+                               int grouped_rows, const void *experts, const void *reverse,
+                               const void *input, void *output);
+
 /* Single-token FP8 E4M3 [inner] times contiguous [outputs, inner] weights with 32-wide scale
  * blocks: FP32 input scales [inner/32] and weight scales [ceil(outputs/32), inner/32] with
  * positive element strides; sum = fma(dot_b * weight_scale, input_scale, sum) for b ascending, BF16

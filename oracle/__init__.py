@@ -173,6 +173,78 @@ def fp8_block32_decode(x, sx, w, sw):
     return out
 
 
+E2M1_VALUES = np.array([0, 0.5, 1, 1.5, 2, 3, 4, 6, -0.0, -0.5, -1, -1.5, -2, -3, -4, -6], np.float64)
+
+
+def mx_dequantise(data, scales, block, packed=False, weight=False):
+    """FP64 values of E8M0 block-scaled storage (byte decoder of the reference's
+    tests/test_quantized.py:12-50, restated in numpy): `data` holds E4M3 bytes [r, k] or, when
+    packed, E2M1 nibbles [r, k/2] in low/high order; a scale byte e stands for 2^(e-127) and 255
+    for NaN; scales are [r, k/block], or [ceil(r/32), k/32] for E4M3 weights (weight=True)."""
+    raw = np.ascontiguousarray(data, dtype=np.uint8)
+    if packed:
+        values = E2M1_VALUES[np.stack((raw & 15, raw >> 4), -1).reshape(raw.shape[0], -1)]
+    else:
+        values = e4m3_to_f32(raw).astype(np.float64)
+    exponents = np.ascontiguousarray(scales, dtype=np.uint8).astype(np.int64)
+    powers = np.ldexp(1.0, exponents - 127)
+    powers[exponents == 255] = np.nan
+    if weight and not packed:
+        powers = np.repeat(powers, 32, axis=0)[: values.shape[0]]
+    return values * np.repeat(powers, block, axis=-1)
+
+
+def mx_matmul_f64(x, sx, w, sw, activation_block=32, packed=False):
+    """FP64 product of the dequantised operands: the yardstick for the E8M0 block-scaled linear."""
+    with np.errstate(invalid="ignore"):
+        return mx_dequantise(x, sx, activation_block) @ mx_dequantise(w, sw, 32, packed, True).T
+
+
+def route_groups(experts, active, first_expert, rows):
+    """Expert routing of include/camblas_cuda.h:168-176 in the reference (kernel:
+    src/cuda/routing.cuh:2-24), with a group's rows assigned in ascending slot order:
+    returns (counts [groups], slots [groups, rows], reverse [tokens, choices])."""
+    experts = np.asarray(experts, dtype=np.int64)
+    active = np.asarray(active, dtype=np.int32)
+    groups = active.size
+    counts = np.zeros(groups, np.int32)
+    slots = np.full((groups, rows), -1, np.int32)
+    reverse = np.full(experts.shape, -1, np.int32)
+    flat_reverse = reverse.reshape(-1)
+    for slot, expert in enumerate(experts.reshape(-1)):
+        if expert < first_expert or expert >= 2**31 - 1:
+            continue
+        local = int(expert) - first_expert
+        matches = np.nonzero(active == local)[0]
+        if matches.size == 0:
+            continue
+        group = int(matches[0])             # duplicate active IDs select their first group
+        row = int(counts[group])
+        counts[group] += 1
+        if row < rows:
+            slots[group, row] = slot
+            flat_reverse[slot] = group * rows + row
+    return counts, slots, reverse
+
+
+def reduce_groups(grouped_bits, experts, reverse):
+    """FP32 sums of BF16 grouped rows per token in ascending (expert ID, choice) order
+    (ref: include/camblas_cuda.h:177-185, src/cuda/routing.cuh:26-56); float32 [tokens, width]."""
+    experts = np.asarray(experts, dtype=np.int64)
+    reverse = np.asarray(reverse, dtype=np.int32)
+    values = bf16_to_f32(np.asarray(grouped_bits, dtype=np.uint16))
+    tokens, choices = experts.shape
+    out = np.zeros((tokens, values.shape[1]), np.float32)
+    for token in range(tokens):
+        order = sorted((int(experts[token, c]), c) for c in range(choices)
+                       if 0 <= experts[token, c] < 2**31 - 1)
+        for _, choice in order:
+            row = int(reverse[token, choice])
+            if 0 <= row < values.shape[0]:
+                out[token] = out[token] + values[row]      # float32 add, one rounding per step
+    return out
+
+
 def fp8_block_matmul(a, a_scale, w, w_scale, want32=False):
     rows, inner = a.shape
     outputs = w.shape[0]

@@ -134,7 +134,8 @@ def test_tensor_binding_loads_and_exports_the_reference_surface():
     for name in ("install_torch_backend", "set_default_algorithm", "stats", "stats_all", "close",
                  "matmul", "matmul_public", "linear_public", "qkv_linear", "gated_mlp",
                  "silu_multiply", "swiglu", "rms_norm", "add_rms_norm", "fp8_block_matmul",
-                 "fp8_decode_supported", "fp8_decode", "fp8_linear"):
+                 "fp8_decode_supported", "fp8_decode", "fp8_linear", "quantized_matmul",
+                 "QuantizedGroups", "route_groups", "reduce_groups"):
         assert callable(getattr(module, name)), name
     import torch
 

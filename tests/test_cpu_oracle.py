@@ -262,6 +262,47 @@ def test_block32_decode_rule_and_power_of_two_quantiser():
             assert q[b * 32 + i] in best, (b, i, target, q[b * 32 + i], best)
 
 
+def test_mx_byte_decoder():
+    # E2M1: (-1)^s * 2^(e-1) * (1 + m/2) for e > 0, m/2 for e == 0 (OCP microscaling formats);
+    # E8M0: 2^(e-127), 255 is NaN; packed order low nibble first; E4M3 weight scales cover 32 rows
+    for code in range(16):
+        sign, exponent, mantissa = code >> 3, (code >> 1) & 3, code & 1
+        value = (mantissa / 2 if exponent == 0 else 2.0 ** (exponent - 1) * (1 + mantissa / 2)) * (-1) ** sign
+        assert oracle.E2M1_VALUES[code] == value and np.signbit(oracle.E2M1_VALUES[code]) == bool(sign)
+    packed = np.array([[0x21, 0xF7]], np.uint8)                  # nibbles 1, 2, 7, 15
+    scales = np.array([[126]], np.uint8)                          # 2^-1 over the one block of 32... (4 here)
+    assert np.array_equal(oracle.mx_dequantise(packed, scales, 4, packed=True), [[0.25, 0.5, 3.0, -3.0]])
+    bytes_ = np.array([[0x38, 0x40], [0x30, 0xB8]], np.uint8)     # 1, 2 / 0.5, -1
+    assert np.array_equal(oracle.mx_dequantise(bytes_, np.array([[0], [254]], np.uint8), 2),
+                          [[2.0**-127, 2.0**-126], [2.0**126, -(2.0**127)]])
+    assert np.isnan(oracle.mx_dequantise(bytes_, np.array([[255], [127]], np.uint8), 2)[0]).all()
+    rows = np.full((40, 32), 0x38, np.uint8)
+    block_scales = np.array([[127], [128]], np.uint8)             # rows 0..31 and 32..39
+    values = oracle.mx_dequantise(rows, block_scales, 32, weight=True)
+    assert (values[:32] == 1).all() and (values[32:] == 2).all()
+    ones = np.full((3, 64), 0x38, np.uint8)
+    product = oracle.mx_matmul_f64(ones, np.full((3, 2), 128, np.uint8), rows[:, :32].repeat(2, axis=1),
+                                   np.array([[127, 127], [128, 128]], np.uint8))
+    assert (product[:, :32] == 128).all() and (product[:, 32:] == 256).all()
+
+
+def test_routing_oracle_hand_worked_case():
+    # tokens x choices = 3 x 2, groups serve local experts [1, 0, 1]: the duplicate (third group)
+    # gets nothing; expert 7 has no group; -1 and 2^40 are ignored; rows = 2 discards a third row
+    experts = np.array([[11, 10], [11, 17], [-1, 11]], np.int64)     # first_expert = 10
+    counts, slots, reverse = oracle.route_groups(experts, [1, 0, 1], 10, 2)
+    assert counts.tolist() == [3, 1, 0]
+    assert slots.tolist() == [[0, 2], [1, -1], [-1, -1]]
+    assert reverse.tolist() == [[0, 2], [1, -1], [-1, -1]]
+    # reduce: token 0 visits experts in ascending ID order (10 then 11): rows 2 then 0
+    grouped = oracle.f32_to_bf16(np.float32([[1, 2**-20], [100, 100], [2**24, 1]]))
+    out = oracle.reduce_groups(grouped, experts[:1], np.array([[0, 2]], np.int32))
+    assert out.tolist() == [[np.float32(2**24) + np.float32(1), np.float32(1) + np.float32(2**-20)]]
+    assert out[0, 0] == 2**24       # one FP32 rounding per step
+    out = oracle.reduce_groups(grouped, np.array([[10, 11]], np.int64), np.array([[0, 2]], np.int32))
+    assert out[0, 0] == 2**24 and out[0, 1] == np.float32(1) + np.float32(2**-20)
+
+
 # ---------------------------------------------------------------- decode epilogues
 
 def test_rms_silu_swiglu_closed_forms():

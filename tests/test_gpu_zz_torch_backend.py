@@ -151,6 +151,54 @@ def test_block32_fp8_entries(binding, device):
             binding.fp8_linear(*operands)
 
 
+def test_quantized_groups_route_multiply_reduce(binding, device):
+    # an expert-parallel slice end to end through the binding (ref: tests/test_quantized.py:324-472
+    # strategy: route, grouped product, ordered reduction, each against an independent restatement)
+    import numpy as np
+
+    import oracle
+
+    tokens, choices, experts_total, rows, inner, outputs = 12, 2, 6, 8, 128, 64
+    generator = torch.Generator(device="cpu").manual_seed(5)
+    chosen = torch.stack([torch.randperm(experts_total, generator=generator)[:choices]
+                          for _ in range(tokens)]).to(device)                      # int64 [tokens, choices]
+    active = torch.tensor([4, 1, 3], dtype=torch.int32, device=device)             # local experts served
+    slots, reverse, counts = binding.route_groups(chosen, active, first_expert=0, rows=rows)
+    want_counts, want_slots, want_reverse = oracle.route_groups(chosen.cpu().numpy(), active.cpu().numpy(), 0, rows)
+    assert np.array_equal(slots.cpu().numpy(), want_slots) and np.array_equal(counts.cpu().numpy(), want_counts)
+    assert np.array_equal(reverse.cpu().numpy(), want_reverse)
+
+    hidden = (torch.randn(tokens, inner, generator=generator) * 4).to(torch.float8_e4m3fn).to(device)
+    gathered = torch.zeros((3, rows, inner), dtype=torch.float8_e4m3fn, device=device)
+    valid = slots >= 0
+    gathered.view(torch.uint8)[valid] = hidden.view(torch.uint8)[torch.div(slots[valid], choices, rounding_mode="floor").long()]
+    gathered_scale = torch.full((3, rows, inner // 32), 127, dtype=torch.uint8, device=device).view(torch.float8_e8m0fnu)
+    weights = [(torch.randn(outputs, inner, generator=generator) * 2).to(torch.float8_e4m3fn).to(device)
+               for _ in range(experts_total)]
+    scales = [torch.randint(124, 129, (outputs // 32, inner // 32), generator=generator, dtype=torch.uint8)
+              .to(device).view(torch.float8_e8m0fnu) for _ in range(experts_total)]
+    group = binding.QuantizedGroups(weights, scales)
+    products = group.matmul(gathered, gathered_scale, active, torch.clamp(counts, max=rows))
+    assert products.shape == (3, rows, outputs) and products.dtype == torch.bfloat16
+    for g, expert in enumerate(active.tolist()):
+        count = min(int(counts[g]), rows)
+        want = oracle.mx_matmul_f64(gathered[g].view(torch.uint8).cpu().numpy(), gathered_scale[g].view(torch.uint8).cpu().numpy(),
+                                    weights[expert].view(torch.uint8).cpu().numpy(), scales[expert].view(torch.uint8).cpu().numpy())
+        got = products[g].float().cpu().numpy()
+        assert (np.abs(got[:count] - want[:count]) <= 0.02 + 0.008 * np.abs(want[:count])).all()
+        assert not got[count:].any()
+    single = binding.quantized_matmul(gathered[0], gathered_scale[0], weights[4], scales[4])
+    assert torch.equal(single[: int(counts[0])], products[0][: int(counts[0])])
+    summed = binding.reduce_groups(products, chosen, reverse)
+    want_sum = oracle.reduce_groups(products.view(torch.int16).cpu().numpy().view(np.uint16).reshape(-1, outputs),
+                                    chosen.cpu().numpy(), reverse.cpu().numpy())
+    assert np.array_equal(summed.cpu().numpy(), want_sum)
+    with pytest.raises(ValueError):
+        binding.quantized_matmul(gathered[0], gathered_scale[0], weights[4], scales[4], activation_block=128)
+    with pytest.raises(ValueError):
+        binding.route_groups(chosen.int(), active, first_expert=0, rows=rows)
+
+
 def test_backend_override_routes_and_falls_back(binding, device):
     binding.install_torch_backend(_native.ALGORITHMS["lt"])
     binding.install_torch_backend(_native.ALGORITHMS["lt"])  # idempotent
