@@ -371,14 +371,16 @@ def extras(torch, _kernels, _native, device, normal):
     a_scale = torch.randint(120, 130, (tokens, inner // 32), device=device, dtype=torch.uint8)
     for name, packed in (("e4m3", False), ("e2m1", True)):
         if packed:
+            # six copies: three of them (198 MB) would fit the 256 MB last-level cache
             weights = [torch.randint(0, 256, (outputs, inner // 2), device=device, dtype=torch.uint8)
-                       for _ in range(3)]
+                       for _ in range(6)]
             scale = torch.randint(120, 130, (outputs, inner // 32), device=device, dtype=torch.uint8)
         else:
             weights = copies
             scale = torch.randint(120, 130, (outputs // 32, inner // 32), device=device, dtype=torch.uint8)
         seconds = event_time(
-            torch, lambda i: _kernels.quantized_matmul(a, a_scale, weights[i % 3], scale), 10, 20)
+            torch, lambda i: _kernels.quantized_matmul(a, a_scale, weights[i % len(weights)], scale),
+            10, 20)
         traffic = weights[0].numel() + scale.numel() + tokens * (inner + inner // 32 + outputs * 2)
         mx[name] = {"us": round(seconds * 1e6, 1), "gbps": round(traffic / seconds / 1e9, 1),
                     "frac_of_8TBs": round(traffic / seconds / HBM_PEAK, 4)}

@@ -21,12 +21,14 @@
 // 32-input scales on both sides.
 //
 // The kernel streams the weights like the other decode kernels: a workgroup owns 16*NT weight rows
-// for the whole K extent and up to 16*MT tokens, its four wavefronts take groups g = 4s + wave,
-// load their group of a tile with whole-line 128-bit loads (non-temporal), transpose it to the
+// for the whole K extent and up to 16*MT tokens, its four wavefronts take 128-byte spans of the
+// rows in turn (span 4s + wave: one group of E4M3 weights, two of E2M1), load their span of a tile
+// with whole-line 128-bit loads (non-temporal), transpose it to the
 // operand layout through a private swizzled LDS patch (no barrier: LDS operations of one wavefront
 // execute in order) and the four partial sums are added in wavefront order at the end.
 #include "common.hpp"
 #include "device.hpp"
+#include "dma.hpp"
 
 namespace camblas_hip
 {
@@ -46,20 +48,31 @@ struct MxParams {
 };
 
 constexpr int WAVES = 4, GROUP = 128;
+// Per-row weight scales (E2M1 weights) of a workgroup's rows are one contiguous byte range; when it
+// fits this many bytes it is copied to LDS once with coalesced loads instead of being gathered a
+// byte per lane and step (16 cache lines per gather for 64 useful bytes).
+constexpr int STAGED_SCALE_BYTES = 32768;
+constexpr int STAGE_PIECES = STAGED_SCALE_BYTES / 16 / (WAVES * 64) + 1; // 16-byte pieces per thread
 
-template <bool PACKED, bool GROUPED, int NT, int MT>
+template <bool PACKED, bool GROUPED, bool STAGED, int NT, int MT>
 __global__ __launch_bounds__(WAVES * 64) void mx_stream_kernel(MxParams p)
 {
-    constexpr int DEPTH = NT + MT <= 6 ? 3 : 2;
-    constexpr int LOADS = PACKED ? 1 : 2;             // 16-byte loads per lane, weight tile and group
-    constexpr int ROW_BYTES = PACKED ? 64 : 128;      // weight bytes per row and group
-    __shared__ __attribute__((aligned(16))) u32x4_t patch[WAVES][NT][PACKED ? 64 : 128];
+    static_assert(PACKED || !STAGED, "only per-row scales are staged");
+    // A step of a wavefront covers one 128-byte line of every weight row: one 128-input group of
+    // E4M3 weights, two consecutive groups of packed E2M1 weights (a half-line step would leave the
+    // other half of each line to another wavefront's request).
+    constexpr int SUB = PACKED ? 2 : 1;
+    constexpr int STEP_INPUTS = GROUP * SUB;
+    constexpr int DEPTH = NT + MT * SUB <= 6 ? 3 : 2; // steps in flight, by registers per step
+    __shared__ __attribute__((aligned(16))) u32x4_t patch[WAVES][NT][128];
+    __shared__ __attribute__((aligned(16))) u32x4_t x_patch[WAVES][MT][128];
     __shared__ __attribute__((aligned(16))) f32x4_t combine[NT * MT * 64];
+    __shared__ __attribute__((aligned(16))) unsigned char staged[STAGED ? STAGED_SCALE_BYTES + 16 : 16];
     const int thread = threadIdx.x, lane = thread % 64, wave = thread / 64;
     const int row = lane % 16, chunk = lane / 16; // operand row / token, 32-input chunk of the group
     const int n0 = blockIdx.x * (NT * 16), m0 = blockIdx.y * (MT * 16);
-    const int blocks = p.inner / 32, groups = (p.inner + GROUP - 1) / GROUP;
-    const int steps = (groups + WAVES - 1) / WAVES;
+    const int blocks = p.inner / 32, spans = (p.inner + STEP_INPUTS - 1) / STEP_INPUTS;
+    const int steps = (spans + WAVES - 1) / WAVES; // spans per wavefront, padded
     const size_t weight_pitch = PACKED ? size_t(p.inner) / 2 : size_t(p.inner);
 
     const unsigned char *input = p.input, *input_scale = p.input_scale, *weight = p.weight,
@@ -88,16 +101,17 @@ __global__ __launch_bounds__(WAVES * 64) void mx_stream_kernel(MxParams p)
         weight_scale = reinterpret_cast<const unsigned char *>(p.metadata[2 * size_t(index) + 1]);
     }
 
-    // ---- per-lane sources. Weight tile loads: 8 (E4M3) or 4 (E2M1) lanes per row segment.
-    constexpr int LANES_PER_ROW = PACKED ? 4 : 8;
-    const int load_row = lane / LANES_PER_ROW, piece = lane % LANES_PER_ROW;
-    const unsigned char *w_source[NT][LOADS];
-    const unsigned char *ws_source[NT];
+    // ---- per-lane sources. Tiles of 16 rows x 128 bytes (weights and inputs alike) are loaded with
+    // eight lanes per line, two loads per lane (rows r and r + 8), and transposed to the operand
+    // layout through LDS: loading them straight in the operand layout would touch every line from
+    // eight quarter-wave passes.
+    const int load_row = lane / 8, piece = lane % 8;
+    const unsigned char *w_source[NT][2], *ws_source[NT];
 #pragma unroll
     for (int i = 0; i < NT; ++i) {
 #pragma unroll
-        for (int h = 0; h < LOADS; ++h) {
-            int n = n0 + i * 16 + h * 8 + load_row; // LOADS == 1: 16 rows in one load
+        for (int h = 0; h < 2; ++h) {
+            int n = n0 + i * 16 + h * 8 + load_row;
             n = n < p.outputs ? n : p.outputs - 1;
             w_source[i][h] = weight + size_t(n) * weight_pitch;
         }
@@ -106,71 +120,99 @@ __global__ __launch_bounds__(WAVES * 64) void mx_stream_kernel(MxParams p)
         // E4M3 weights: one scale per 32 x 32 block; E2M1 weights: one per row and 32 inputs
         ws_source[i] = weight_scale + size_t(PACKED ? n : n / 32) * blocks;
     }
-    const unsigned char *x_source[MT], *xs_source[MT];
+    const unsigned char *x_source[MT][2], *xs_source[MT];
 #pragma unroll
     for (int j = 0; j < MT; ++j) {
+#pragma unroll
+        for (int h = 0; h < 2; ++h) {
+            int m = m0 + j * 16 + h * 8 + load_row;
+            m = m < valid_rows ? m : valid_rows - 1;
+            x_source[j][h] = input + size_t(m) * p.inner;
+        }
         int m = m0 + j * 16 + row;
         m = m < valid_rows ? m : valid_rows - 1;
-        x_source[j] = input + size_t(m) * p.inner;
         xs_source[j] = input_scale + size_t(m) * (blocks >> p.scale_shift);
     }
-    // LDS patch of one weight tile, XOR-swizzled so that the line-shaped stores and the
-    // operand-shaped loads are both conflict-free
-    auto slot = [](int r, int q) {
-        return PACKED ? r * 4 + (q ^ ((r >> 2) & 3)) : r * 8 + (q ^ ((r >> 1) & 7));
-    };
-    int store_slot[LOADS], read_slot[LOADS];
-#pragma unroll
-    for (int h = 0; h < LOADS; ++h) {
-        store_slot[h] = slot(load_row + 8 * h, piece);
-        read_slot[h] = PACKED ? slot(row, chunk) : slot(row, chunk + 4 * h); // pieces c and 4 + c
-    }
+    // LDS patch of one tile, XOR-swizzled so that the line-shaped stores and the operand-shaped
+    // loads are both conflict-free. An 8-bit operand of lane group c is pieces c and 4 + c of the
+    // line (the instruction's layout); of a 4-bit line, piece c is the operand of the first group
+    // and piece 4 + c that of the second: the same two reads serve both formats.
+    auto slot = [](int r, int q) { return r * 8 + (q ^ ((r >> 1) & 7)); };
+    const int store_slot[2] = {slot(load_row, piece), slot(load_row + 8, piece)};
+    const int read_slot[2] = {slot(row, chunk), slot(row, chunk + 4)};
 
-    // Workgroups start at different groups and wrap around (spreads the row-pitch-strided requests
-    // over the HBM channels). Steps past the end re-read the last group with zeroed activations.
+    // Workgroups start at different spans and wrap around (spreads the row-pitch-strided requests
+    // over the HBM channels). Steps past the end re-read the last span with zeroed activations.
     const int start = int(blockIdx.x % unsigned(steps));
-    auto group_of = [&](int step) {
-        int rotated = (step < steps ? step : steps - 1) + start;
+    auto span_of = [&](int step) {
+        step = step < steps ? step : steps - 1;
+        int rotated = step + start;
         rotated = rotated < steps ? rotated : rotated - steps;
         return rotated * WAVES + wave;
     };
-    u32x4_t w_raw[DEPTH][NT][LOADS], x_raw[DEPTH][MT][2];
-    unsigned ws_raw[DEPTH][NT], xs_raw[DEPTH][MT], keep_raw[DEPTH][2];
+    u32x4_t w_raw[DEPTH][NT][2], x_raw[DEPTH][MT][SUB][2];
+    unsigned ws_raw[DEPTH][NT][SUB], xs_raw[DEPTH][MT][SUB], keep_raw[DEPTH][SUB][2];
     // Loads only: nothing here may use a loaded value, or the wait would cover the newest loads.
-    auto fetch = [&](int step, u32x4_t(&w)[NT][LOADS], u32x4_t(&x)[MT][2], unsigned(&ws)[NT],
-                     unsigned(&xs)[MT], unsigned(&keep)[2]) {
-        int g = group_of(step);
-        const bool live = step < steps && g < groups;
-        g = g < groups ? g : groups - 1;
-        int block = g * 4 + chunk; // the 32-input block whose scales this lane supplies
-        block = block < blocks ? block : blocks - 1;
-        // the lane's two 16-byte input pieces: positions 16c.. (block c/2) and 64+16c.. (block 2+c/2)
-        int half_offset[2] = {g * GROUP + chunk * 16, g * GROUP + 64 + chunk * 16};
+    auto fetch = [&](int step, u32x4_t(&w)[NT][2], u32x4_t(&x)[MT][SUB][2], unsigned(&ws)[NT][SUB],
+                     unsigned(&xs)[MT][SUB], unsigned(&keep)[SUB][2]) {
+        int g = span_of(step);
+        const bool live = step < steps && g < spans;
+        g = g < spans ? g : spans - 1;
+        // bytes past the end of a row in a partial last span re-read the row's last 16 bytes
+        size_t w_offset = size_t(g) * 128 + piece * 16;
+        w_offset = w_offset < weight_pitch ? w_offset : weight_pitch - 16;
 #pragma unroll
-        for (int h = 0; h < 2; ++h) {
-            keep[h] = live && half_offset[h] < p.inner ? 0xffffffffu : 0u;
-            half_offset[h] = half_offset[h] < p.inner ? half_offset[h] : p.inner - 16;
-        }
-#pragma unroll
-        for (int i = 0; i < NT; ++i) {
-#pragma unroll
-            for (int h = 0; h < LOADS; ++h) {
-                // bytes past the end of the row in a partial last group re-read its last 16 bytes
-                size_t offset = size_t(g) * ROW_BYTES + piece * 16;
-                offset = offset < weight_pitch ? offset : weight_pitch - 16;
-                w[i][h] = __builtin_nontemporal_load(
-                    reinterpret_cast<const u32x4_t *>(w_source[i][h] + offset));
-            }
-            ws[i] = ws_source[i][block];
-        }
-#pragma unroll
-        for (int j = 0; j < MT; ++j) {
+        for (int i = 0; i < NT; ++i)
 #pragma unroll
             for (int h = 0; h < 2; ++h)
-                x[j][h] = *reinterpret_cast<const u32x4_t *>(x_source[j] + half_offset[h]);
-            xs[j] = xs_source[j][block >> p.scale_shift];
+                w[i][h] = __builtin_nontemporal_load(
+                    reinterpret_cast<const u32x4_t *>(w_source[i][h] + w_offset));
+#pragma unroll
+        for (int s = 0; s < SUB; ++s) {
+            const int first = g * STEP_INPUTS + s * GROUP; // first input of the 128-input group
+            int block = first / 32 + chunk; // the 32-input block whose scales this lane supplies
+            block = block < blocks ? block : blocks - 1;
+            // the operand's two 16-byte input pieces are positions 16c.. and 64+16c.. of the group
+#pragma unroll
+            for (int h = 0; h < 2; ++h)
+                keep[s][h] = live && first + 64 * h + chunk * 16 < p.inner ? 0xffffffffu : 0u;
+            int x_offset = first + piece * 16;
+            x_offset = x_offset < p.inner ? x_offset : p.inner - 16;
+#pragma unroll
+            for (int i = 0; i < NT; ++i) {
+                if constexpr (STAGED)
+                    ws[i][s] = unsigned(block); // read from LDS at multiply time
+                else
+                    ws[i][s] = ws_source[i][block];
+            }
+#pragma unroll
+            for (int j = 0; j < MT; ++j) {
+#pragma unroll
+                for (int h = 0; h < 2; ++h)
+                    x[j][s][h] = *reinterpret_cast<const u32x4_t *>(x_source[j][h] + x_offset);
+                xs[j][s] = xs_source[j][block >> p.scale_shift];
+            }
         }
     };
+
+    // Staged scales: the byte range of rows n0 .. n0 + 16*NT - 1 (cut at the matrix end), widened to
+    // whole aligned 16-byte pieces (a piece holding one valid byte lies inside that byte's page).
+    // The loads go out before the first weight loads and are stored once those are in flight.
+    u32x4_t stage_raw[STAGE_PIECES];
+    int staged_shift = 0, stage_pieces = 0;
+    if constexpr (STAGED) {
+        const unsigned char *first = weight_scale + size_t(n0) * blocks;
+        const int length = min(NT * 16, p.outputs - n0) * blocks;
+        staged_shift = int(reinterpret_cast<uintptr_t>(first) & 15);
+        stage_pieces = (staged_shift + length + 15) / 16;
+        const u32x4_t *pieces = reinterpret_cast<const u32x4_t *>(first - staged_shift);
+#pragma unroll
+        for (int e = 0; e < STAGE_PIECES; ++e) {
+            const int index = thread + e * (WAVES * 64);
+            stage_raw[e] = pieces[index < stage_pieces ? index : stage_pieces - 1];
+        }
+        __builtin_amdgcn_sched_barrier(0);
+    }
 
     f32x4_t acc[NT][MT];
 #pragma unroll
@@ -178,46 +220,80 @@ __global__ __launch_bounds__(WAVES * 64) void mx_stream_kernel(MxParams p)
 #pragma unroll
         for (int j = 0; j < MT; ++j)
             acc[i][j] = f32x4_t{0.f, 0.f, 0.f, 0.f};
-    auto multiply = [&](const u32x4_t(&w)[NT][LOADS], const u32x4_t(&x)[MT][2],
-                        const unsigned(&ws)[NT], const unsigned(&xs)[MT], const unsigned(&keep)[2]) {
+    auto multiply = [&](const u32x4_t(&w)[NT][2], const u32x4_t(&x)[MT][SUB][2],
+                        const unsigned(&ws)[NT][SUB], const unsigned(&xs)[MT][SUB],
+                        const unsigned(&keep)[SUB][2]) {
         u32x4_t *mine = &patch[wave][0][0];
-        constexpr int TILE = PACKED ? 64 : 128;
+        u32x4_t *mine_x = &x_patch[wave][0][0];
 #pragma unroll
         for (int i = 0; i < NT; ++i)
 #pragma unroll
-            for (int h = 0; h < LOADS; ++h)
-                mine[i * TILE + store_slot[h]] = w[i][h];
-        // other lanes' stores are read below: keep the compiler from moving the loads up
-        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-        __builtin_amdgcn_wave_barrier();
-        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
-        i32x8_t a[NT];
+            for (int h = 0; h < 2; ++h)
+                mine[i * 128 + store_slot[h]] = w[i][h];
+        u32x4_t w_lo[NT], w_hi[NT];
 #pragma unroll
-        for (int i = 0; i < NT; ++i) {
-            u32x4_t lo = mine[i * TILE + read_slot[0]];
-            u32x4_t hi = PACKED ? u32x4_t{0u, 0u, 0u, 0u} : mine[i * TILE + read_slot[LOADS - 1]];
-            a[i] = i32x8_t{int(lo[0]), int(lo[1]), int(lo[2]), int(lo[3]),
-                           int(hi[0]), int(hi[1]), int(hi[2]), int(hi[3])};
-        }
-        // inputs past the end of K (and of dead steps) are zero
+        for (int s = 0; s < SUB; ++s) {
 #pragma unroll
-        for (int j = 0; j < MT; ++j) {
-            const u32x4_t lo = x[j][0] & keep[0], hi = x[j][1] & keep[1];
-            const i32x8_t b = {int(lo[0]), int(lo[1]), int(lo[2]), int(lo[3]),
+            for (int j = 0; j < MT; ++j)
+#pragma unroll
+                for (int h = 0; h < 2; ++h)
+                    mine_x[j * 128 + store_slot[h]] = x[j][s][h];
+            // other lanes' stores are read below: keep the compiler from moving the loads up
+            __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+            __builtin_amdgcn_wave_barrier();
+            __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+            if (s == 0) {
+#pragma unroll
+                for (int i = 0; i < NT; ++i) {
+                    w_lo[i] = mine[i * 128 + read_slot[0]];
+                    w_hi[i] = mine[i * 128 + read_slot[1]];
+                }
+            }
+            i32x8_t a[NT];
+#pragma unroll
+            for (int i = 0; i < NT; ++i) {
+                const u32x4_t lo = PACKED && s == 1 ? w_hi[i] : w_lo[i];
+                const u32x4_t hi = PACKED ? u32x4_t{0u, 0u, 0u, 0u} : w_hi[i];
+                a[i] = i32x8_t{int(lo[0]), int(lo[1]), int(lo[2]), int(lo[3]),
                                int(hi[0]), int(hi[1]), int(hi[2]), int(hi[3])};
+            }
+            unsigned w_scale[NT];
 #pragma unroll
             for (int i = 0; i < NT; ++i)
-                acc[i][j] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(
-                    a[i], b, acc[i][j], PACKED ? 4 : 0, 0, 0, int(ws[i]), 0, int(xs[j]));
+                w_scale[i] = STAGED ? unsigned(staged[staged_shift + (i * 16 + row) * blocks + int(ws[i][s])])
+                                    : ws[i][s];
+            // inputs past the end of K (and of dead steps) are zero
+#pragma unroll
+            for (int j = 0; j < MT; ++j) {
+                const u32x4_t lo = mine_x[j * 128 + read_slot[0]] & keep[s][0],
+                              hi = mine_x[j * 128 + read_slot[1]] & keep[s][1];
+                const i32x8_t b = {int(lo[0]), int(lo[1]), int(lo[2]), int(lo[3]),
+                                   int(hi[0]), int(hi[1]), int(hi[2]), int(hi[3])};
+#pragma unroll
+                for (int i = 0; i < NT; ++i)
+                    acc[i][j] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(
+                        a[i], b, acc[i][j], PACKED ? 4 : 0, 0, 0, int(w_scale[i]), 0, int(xs[j][s]));
+            }
+            // the patches are overwritten next: order the reads above before those stores
+            __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+            __builtin_amdgcn_wave_barrier();
         }
-        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-        __builtin_amdgcn_wave_barrier();
     };
 
 #pragma unroll
     for (int d = 0; d < DEPTH; ++d) {
         fetch(d, w_raw[d], x_raw[d], ws_raw[d], xs_raw[d], keep_raw[d]);
         __builtin_amdgcn_sched_barrier(0);
+    }
+    if constexpr (STAGED) {
+#pragma unroll
+        for (int e = 0; e < STAGE_PIECES; ++e) {
+            const int index = thread + e * (WAVES * 64);
+            if (index < stage_pieces)
+                reinterpret_cast<u32x4_t *>(staged)[index] = stage_raw[e];
+        }
+        // not __syncthreads(): its fence would wait for every weight load issued above
+        pipeline_barrier<63>();
     }
     for (int step = 0; step < steps; step += DEPTH) {
 #pragma unroll
@@ -267,12 +343,15 @@ __global__ __launch_bounds__(WAVES * 64) void mx_stream_kernel(MxParams p)
 template <bool PACKED, bool GROUPED, int NT, int MT>
 hipError_t launch_one(hipStream_t stream, const MxParams &p, int groups)
 {
-    if constexpr (NT * MT > 16 || NT + MT > 10) {
+    if constexpr (NT * MT > 16 || NT + MT * (PACKED ? 2 : 1) > 10) {
         return hipErrorInvalidValue;
     } else {
         dim3 grid(unsigned((p.outputs + NT * 16 - 1) / (NT * 16)),
                   unsigned((p.rows + MT * 16 - 1) / (MT * 16)), unsigned(groups));
-        mx_stream_kernel<PACKED, GROUPED, NT, MT><<<grid, WAVES * 64, 0, stream>>>(p);
+        if (PACKED && NT * 16 * (p.inner / 32) <= STAGED_SCALE_BYTES)
+            mx_stream_kernel<PACKED, GROUPED, PACKED, NT, MT><<<grid, WAVES * 64, 0, stream>>>(p);
+        else
+            mx_stream_kernel<PACKED, GROUPED, false, NT, MT><<<grid, WAVES * 64, 0, stream>>>(p);
         return launch_status();
     }
 }
@@ -282,10 +361,12 @@ hipError_t launch_shape(hipStream_t stream, const MxParams &p, int groups)
 {
     // token tiles by row count; weight-row tiles so that about one workgroup lands on each compute
     // unit (decode-sized calls: the kernel is bound by the weight stream)
-    const int token_tiles = p.rows <= 16 ? 1 : p.rows <= 32 ? 2 : 4;
+    // (E2M1 steps hold twice the input tiles: four token tiles would not fit the register file)
+    const int token_tiles = p.rows <= 16 ? 1 : p.rows <= 32 || PACKED ? 2 : 4;
     const int tiles = (p.outputs + 15) / 16;
     int row_tiles = 1;
-    for (int candidate = token_tiles == 4 ? 4 : 8; candidate > 1; --candidate)
+    const int most = PACKED ? (token_tiles == 2 ? 6 : 8) : (token_tiles == 4 ? 4 : 8);
+    for (int candidate = most; candidate > 1; --candidate)
         if (tiles / candidate >= 192) {
             row_tiles = candidate;
             break;

@@ -65,6 +65,37 @@ def test_random_operands_and_individual_mutations(device, packed, rows, outputs,
 
 
 @pytest.mark.parametrize("packed", [False, True])
+@pytest.mark.parametrize("rows,outputs,inner", [(16, 18440, 256), (20, 18440, 160), (40, 12296, 96)])
+def test_wide_workgroups_and_unaligned_scales(device, packed, rows, outputs, inner):
+    # enough outputs for workgroups of several row tiles, a last workgroup that is cut short, and
+    # scale arrays that start at an odd address (they are byte arrays: nothing aligns them)
+    x, sx, weight, sw = operands(4100 + rows, rows, outputs, inner, packed, 32)
+    xt = torch.from_numpy(x).to(device).view(torch.float8_e4m3fn)
+    wt = torch.from_numpy(weight).to(device)
+    if not packed:
+        wt = wt.view(torch.float8_e4m3fn)
+
+    def shifted(array, shift):
+        buffer = torch.zeros(array.size + 16, dtype=torch.uint8, device=device)
+        view = buffer[shift:shift + array.size].view(array.shape)
+        view.copy_(torch.from_numpy(array).to(device))
+        return view
+
+    out = _kernels.quantized_matmul(xt, shifted(sx, 3), wt, shifted(sw, 5), activation_block=32)
+    torch.cuda.synchronize()
+    got = bf16_values(out)
+    xd = oracle.mx_dequantise(x, sx, 32)
+    wd = oracle.mx_dequantise(weight, sw, 32, packed, True)
+    want = xd @ wd.T
+    # Among 300 000 outputs a few sums cancel to nearly nothing, so the reference's fixed absolute
+    # tolerance gives way to one that follows the size of the terms: FP32 accumulation may lose
+    # 2^-13 of the sum of the products' magnitudes (measured worst case about 2^-15).
+    magnitude = np.abs(xd) @ np.abs(wd).T
+    assert (np.abs(got - want) <= 0.008 * np.abs(want) + magnitude * 2.0 ** -13).all()
+    assert np.linalg.norm(got - want) <= 4e-3 * np.linalg.norm(want)
+
+
+@pytest.mark.parametrize("packed", [False, True])
 @pytest.mark.parametrize("rows", [1, 8, 17])
 def test_scale_extremes_and_nan(device, packed, rows):
     # ones times ones with unit weight scales: exact for input scales 2^-127, 1, 2^127 and NaN for
