@@ -41,6 +41,7 @@ struct MxParams {
     const unsigned char *weight_scale;
     unsigned short *out;
     int rows, outputs, inner, scale_shift; // activation scale covers 32 << scale_shift inputs
+    bool out_aligned;                      // out is 8-byte aligned: four features go out in one store
     // grouped form
     const unsigned long long *metadata;
     const int32_t *active, *counts;
@@ -64,9 +65,10 @@ __global__ __launch_bounds__(WAVES * 64) void mx_stream_kernel(MxParams p)
     constexpr int SUB = PACKED ? 2 : 1;
     constexpr int STEP_INPUTS = GROUP * SUB;
     constexpr int DEPTH = NT + MT * SUB <= 6 ? 3 : 2; // steps in flight, by registers per step
-    __shared__ __attribute__((aligned(16))) u32x4_t patch[WAVES][NT][128];
-    __shared__ __attribute__((aligned(16))) u32x4_t x_patch[WAVES][MT][128];
-    __shared__ __attribute__((aligned(16))) f32x4_t combine[NT * MT * 64];
+    // per wavefront: NT weight tiles and MT input tiles of 16 x 128 bytes; after the last step the
+    // same memory holds the wavefront's partial sums
+    __shared__ __attribute__((aligned(16))) u32x4_t tiles[WAVES][NT + MT][128];
+    static_assert(NT * MT * 64 <= (NT + MT) * 128, "partial sums must fit the wavefront's tile memory");
     __shared__ __attribute__((aligned(16))) unsigned char staged[STAGED ? STAGED_SCALE_BYTES + 16 : 16];
     const int thread = threadIdx.x, lane = thread % 64, wave = thread / 64;
     const int row = lane % 16, chunk = lane / 16; // operand row / token, 32-input chunk of the group
@@ -223,8 +225,8 @@ __global__ __launch_bounds__(WAVES * 64) void mx_stream_kernel(MxParams p)
     auto multiply = [&](const u32x4_t(&w)[NT][2], const u32x4_t(&x)[MT][SUB][2],
                         const unsigned(&ws)[NT][SUB], const unsigned(&xs)[MT][SUB],
                         const unsigned(&keep)[SUB][2]) {
-        u32x4_t *mine = &patch[wave][0][0];
-        u32x4_t *mine_x = &x_patch[wave][0][0];
+        u32x4_t *mine = &tiles[wave][0][0];
+        u32x4_t *mine_x = &tiles[wave][NT][0];
 #pragma unroll
         for (int i = 0; i < NT; ++i)
 #pragma unroll
@@ -304,23 +306,16 @@ __global__ __launch_bounds__(WAVES * 64) void mx_stream_kernel(MxParams p)
             fetch(step + d + DEPTH, w_raw[d], x_raw[d], ws_raw[d], xs_raw[d], keep_raw[d]);
         }
     }
+    // ---- every wavefront parks its partial sums in its own tile memory (nobody else reads that),
+    // one barrier, then tile t is summed in wavefront order 0, 1, 2, 3 by wavefront t % 4 and
+    // written. Register r of lane l is feature 4*(l/16) + r and token l%16 of the tile.
+    f32x4_t *parked = reinterpret_cast<f32x4_t *>(&tiles[wave][0][0]);
+#pragma unroll
+    for (int i = 0; i < NT; ++i)
+#pragma unroll
+        for (int j = 0; j < MT; ++j)
+            parked[(i * MT + j) * 64 + lane] = acc[i][j];
     __syncthreads();
-
-    // ---- add the four wavefronts' partial sums in wavefront order through LDS
-#pragma unroll
-    for (int w = 0; w < WAVES; ++w) {
-        if (wave == w) {
-#pragma unroll
-            for (int i = 0; i < NT; ++i)
-#pragma unroll
-                for (int j = 0; j < MT; ++j) {
-                    f32x4_t *cell = combine + (i * MT + j) * 64 + lane;
-                    *cell = w == 0 ? acc[i][j] : *cell + acc[i][j];
-                }
-        }
-        __syncthreads();
-    }
-    // ---- epilogue: register r of lane l is feature 4*(l/16) + r and token l%16 of the tile
 #pragma unroll
     for (int index = 0; index < NT * MT; ++index) {
         if (index % WAVES != wave)
@@ -330,13 +325,25 @@ __global__ __launch_bounds__(WAVES * 64) void mx_stream_kernel(MxParams p)
         const int n = n0 + i * 16 + chunk * 4;
         if (m >= p.rows || n >= p.outputs)
             continue;
-        f32x4_t sum = combine[index * 64 + lane];
-        unsigned short *target = out + size_t(m) * p.outputs + n;
+        f32x4_t sum = reinterpret_cast<const f32x4_t *>(&tiles[0][0][0])[index * 64 + lane];
+#pragma unroll
+        for (int w = 1; w < WAVES; ++w)
+            sum = sum + reinterpret_cast<const f32x4_t *>(&tiles[w][0][0])[index * 64 + lane];
         const bool zero = GROUPED && m >= valid_rows; // padding rows of a group
         // outputs is a multiple of eight, so the four features are all inside the matrix
+        unsigned short bits[4];
 #pragma unroll
         for (int e = 0; e < 4; ++e)
-            target[e] = zero ? (unsigned short)0 : float_to_bf16_bits(sum[e]);
+            bits[e] = zero ? (unsigned short)0 : float_to_bf16_bits(sum[e]);
+        unsigned short *target = out + size_t(m) * p.outputs + n;
+        if (p.out_aligned) {
+            *reinterpret_cast<u32x2_t *>(target) =
+                u32x2_t{bits[0] | unsigned(bits[1]) << 16, bits[2] | unsigned(bits[3]) << 16};
+        } else {
+#pragma unroll
+            for (int e = 0; e < 4; ++e)
+                target[e] = bits[e];
+        }
     }
 }
 
@@ -415,6 +422,7 @@ hipError_t launch_mx_matmul(hipStream_t stream, bool packed, int groups, int wei
     p.outputs = outputs;
     p.inner = inner;
     p.scale_shift = activation_block == 128 ? 2 : 0;
+    p.out_aligned = reinterpret_cast<uintptr_t>(out) % 8 == 0;
     p.metadata = static_cast<const unsigned long long *>(metadata);
     p.active = static_cast<const int32_t *>(active);
     p.counts = static_cast<const int32_t *>(counts);
