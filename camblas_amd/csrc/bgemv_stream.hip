@@ -167,22 +167,17 @@ __global__ __launch_bounds__(WAVES * 64) void bgemv_stream_kernel(StreamParams p
         }
     }
 
-    // ---- combine the K partitions of the wavefronts in wavefront order through LDS
+    // ---- combine the K partitions of the wavefronts: each parks its partial sums in a region of
+    // its own, and after one barrier tile t is summed in wavefront order 0, 1, 2, 3 by wavefront t % 4
     __syncthreads();
+    // (the launcher sizes the dynamic LDS for the larger of the two uses)
     f32x4_t *combine = reinterpret_cast<f32x4_t *>(lds_bytes);
 #pragma unroll
-    for (int w = 0; w < WAVES; ++w) {
-        if (wave == w) {
+    for (int i = 0; i < NT; ++i)
 #pragma unroll
-            for (int i = 0; i < NT; ++i)
-#pragma unroll
-                for (int j = 0; j < MT; ++j) {
-                    f32x4_t *slot = combine + (i * MT + j) * 64 + lane;
-                    *slot = w == 0 ? acc[i][j] : *slot + acc[i][j];
-                }
-        }
-        __syncthreads();
-    }
+        for (int j = 0; j < MT; ++j)
+            combine[((wave * NT + i) * MT + j) * 64 + lane] = acc[i][j];
+    __syncthreads();
     // ---- epilogue: wavefront w writes tiles w, w+4, ...; register r of lane l is feature
     // 4*(l/16) + r and token l%16 inside the 16x16 tile
 #pragma unroll
@@ -195,6 +190,9 @@ __global__ __launch_bounds__(WAVES * 64) void bgemv_stream_kernel(StreamParams p
         if (m >= p.m || n >= p.n)
             continue;
         f32x4_t sum = combine[index * 64 + lane];
+#pragma unroll
+        for (int w = 1; w < WAVES; ++w)
+            sum = sum + combine[(w * NT * MT + index) * 64 + lane];
         float v[4] = {sum[0], sum[1], sum[2], sum[3]};
         unsigned short *out = p.y + size_t(m) * p.ldc + n;
         if (n + 3 < p.n && p.vector_store) {
@@ -228,7 +226,9 @@ __global__ __launch_bounds__(WAVES * 64) void bgemv_stream_kernel(StreamParams p
 template <int NT, int MT, int KT>
 hipError_t launch_one(hipStream_t stream, const StreamParams &p)
 {
-    constexpr size_t lds_bytes = size_t(2) * KT * (NT + MT) * 16 * (64 * WAVES);
+    constexpr size_t stage_bytes = size_t(2) * KT * (NT + MT) * 16 * (64 * WAVES);
+    constexpr size_t parked_bytes = size_t(WAVES) * NT * MT * 64 * 16; // partial sums at the end
+    constexpr size_t lds_bytes = stage_bytes > parked_bytes ? stage_bytes : parked_bytes;
     // combined limits: the tiles in flight fit the register file, a stage pair fits the LDS
     if constexpr (NT * KT > 8 || lds_bytes > 128 * 1024) {
         return hipErrorInvalidValue;

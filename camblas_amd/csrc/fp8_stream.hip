@@ -44,7 +44,8 @@ __global__ __launch_bounds__(WAVES * 64) void fp8_stream_kernel(Fp8StreamParams 
     constexpr int DEPTH = NT + MT <= 6 ? 3 : 2;
     constexpr int TILES = NT + MT; // weight tiles, then token tiles
     __shared__ __attribute__((aligned(16))) u32x4_t patch[WAVES][TILES][128];
-    __shared__ __attribute__((aligned(16))) f32x4_t combine[NT * MT * 64];
+    // after the last step the wavefront's patches hold its partial sums instead
+    static_assert(NT * MT * 64 <= TILES * 128, "partial sums must fit the wavefront's patches");
     const int thread = threadIdx.x, lane = thread % 64, wave = thread / 64;
     const int row = lane % 16, chunk = lane / 16; // operand row / token, 32-byte chunk of the group
     const int load_row = lane / 8, piece = lane % 8; // load layout: 8 lanes per 128-byte line
@@ -180,22 +181,15 @@ __global__ __launch_bounds__(WAVES * 64) void fp8_stream_kernel(Fp8StreamParams 
             fetch(step + d + DEPTH, raw[d], ws_reg[d], as_reg[d], live_reg[d]);
         }
     }
+    // ---- every wavefront parks its partial sums in its own patches (nobody else reads those);
+    // after one barrier tile t is summed in wavefront order 0, 1, 2, 3 by wavefront t % 4
+    f32x4_t *parked = reinterpret_cast<f32x4_t *>(&patch[wave][0][0]);
+#pragma unroll
+    for (int i = 0; i < NT; ++i)
+#pragma unroll
+        for (int j = 0; j < MT; ++j)
+            parked[(i * MT + j) * 64 + lane] = acc[i][j];
     __syncthreads();
-
-    // ---- add the four wavefronts' partial sums in wavefront order through LDS
-#pragma unroll
-    for (int w = 0; w < WAVES; ++w) {
-        if (wave == w) {
-#pragma unroll
-            for (int i = 0; i < NT; ++i)
-#pragma unroll
-                for (int j = 0; j < MT; ++j) {
-                    f32x4_t *slot = combine + (i * MT + j) * 64 + lane;
-                    *slot = w == 0 ? acc[i][j] : *slot + acc[i][j];
-                }
-        }
-        __syncthreads();
-    }
     // ---- epilogue: wavefront w writes tiles w, w+4, ...; register r of lane l is feature
     // 4*(l/16) + r and token l%16 inside the 16x16 tile
     const bool vector_store = p.n % 4 == 0 && reinterpret_cast<uintptr_t>(p.out) % 8 == 0;
@@ -208,7 +202,10 @@ __global__ __launch_bounds__(WAVES * 64) void fp8_stream_kernel(Fp8StreamParams 
         const int n = n0 + i * 16 + chunk * 4;
         if (m >= p.m || n >= p.n)
             continue;
-        f32x4_t sum = combine[index * 64 + lane];
+        f32x4_t sum = reinterpret_cast<const f32x4_t *>(&patch[0][0][0])[index * 64 + lane];
+#pragma unroll
+        for (int w = 1; w < WAVES; ++w)
+            sum = sum + reinterpret_cast<const f32x4_t *>(&patch[w][0][0])[index * 64 + lane];
         unsigned short *out = p.out + size_t(m) * p.n + n;
         if (n + 3 < p.n && vector_store) {
             u32x2_t packed = {pack_bf16x2(sum[0], sum[1]), pack_bf16x2(sum[2], sum[3])};
