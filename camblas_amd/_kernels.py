@@ -63,7 +63,7 @@ def matmul(a, b, out=None, alpha=1.0, beta=0.0):
     """alpha * a @ b + beta * out for 2-D FP32 or BF16 device tensors.
 
     ref: src/cuda/torch_bindings.cpp:155-199 (row-major operands become the swapped column-major
-    call). FP64 is rejected by the library with its own message.
+    call).
     """
     _validate(a, a)
     _validate(b, a)
@@ -138,6 +138,176 @@ def addmm(bias, a, b, beta=1.0, alpha=1.0):
         return matmul(a, b, None, alpha, 0.0)
     out = bias.expand(m, n).clone(memory_format=torch.contiguous_format)
     return matmul(a, b, out, alpha, beta)
+
+
+def _dense(tensor, reference):
+    _validate(tensor, reference, allow_bfloat16=False)
+    return tensor.contiguous()
+
+
+def _affine_forward(x, weight, bias, relu, out=None):
+    # ref: affine, src/cuda/torch_bindings.cpp:737-771
+    x, weight, bias = _dense(x, x), _dense(weight, x), _dense(bias, x)
+    _require(x.dim() == 2 and weight.dim() == 2 and bias.dim() == 1 and x.shape[1] == weight.shape[0]
+             and weight.shape[1] == bias.shape[0], "Invalid affine operand shapes")
+    rows, inner = x.shape
+    columns = weight.shape[1]
+    if out is not None:
+        _validate(out, x, allow_bfloat16=False)
+        _require(out.dim() == 2 and tuple(out.shape) == (rows, columns) and out.is_contiguous(),
+                 "Invalid affine output shape or strides")
+        storage = out.untyped_storage().data_ptr()
+        _require(all(storage != t.untyped_storage().data_ptr() for t in (x, weight, bias)),
+                 "Affine output cannot alias an input")
+    else:
+        out = torch.empty((rows, columns), dtype=x.dtype, device=x.device)
+    with torch.cuda.device(x.device):
+        _native.context(x.device).call("affine", _DTYPE_CODE[x.dtype], rows, inner, columns, _pointer(x),
+                                       _pointer(weight), _pointer(bias), int(bool(relu)), _pointer(out))
+    return out
+
+
+class _Affine(torch.autograd.Function):
+    """ref: AffineAutograd, src/cuda/torch_bindings.cpp:773-801 — the gradients are products through
+    this library; with ReLU the incoming gradient is masked where the output is not positive."""
+
+    @staticmethod
+    def forward(ctx, x, weight, bias, relu):
+        output = _affine_forward(x, weight, bias, relu)
+        ctx.save_for_backward(x, weight, output)
+        ctx.relu = relu
+        return output
+
+    @staticmethod
+    def backward(ctx, gradient):
+        x, weight, output = ctx.saved_tensors
+        if ctx.relu:
+            gradient = torch.where(output <= 0, torch.zeros_like(gradient), gradient)
+        dx = matmul_autograd(gradient, weight.t()) if ctx.needs_input_grad[0] else None
+        dw = matmul_autograd(x.t(), gradient) if ctx.needs_input_grad[1] else None
+        db = gradient.sum(0) if ctx.needs_input_grad[2] else None
+        return dx, dw, db, None
+
+
+class _Matmul(torch.autograd.Function):
+    """a @ b with both gradients as products of this library (ref: MatmulAutograd,
+    src/cuda/torch_bindings.cpp:201-242); differentiable to any order."""
+
+    @staticmethod
+    def forward(ctx, a, b):
+        ctx.save_for_backward(a, b)
+        return matmul(a, b)
+
+    @staticmethod
+    def backward(ctx, gradient):
+        a, b = ctx.saved_tensors
+        da = matmul_autograd(gradient, b.t()) if ctx.needs_input_grad[0] else None
+        db = matmul_autograd(a.t(), gradient) if ctx.needs_input_grad[1] else None
+        return da, db
+
+
+def matmul_autograd(a, b):
+    """matmul that records gradients when any operand needs them."""
+    if torch.is_grad_enabled() and (a.requires_grad or b.requires_grad):
+        return _Matmul.apply(a, b)
+    return matmul(a, b)
+
+
+def affine(x, weight, bias, relu=False, out=None):
+    """x @ weight + bias with optional ReLU for FP32 / FP64 (ref: affine_public,
+    src/cuda/torch_bindings.cpp:803-813; C entry include/camblas_cuda.h:71-75)."""
+    if torch.is_grad_enabled() and any(t.requires_grad for t in (x, weight, bias)):
+        _require(out is None, "Autograd affine does not support an out tensor")
+        return _Affine.apply(x, weight, bias, bool(relu))
+    return _affine_forward(x, weight, bias, relu, out)
+
+
+def _mlp_forward(x, w1, b1, w2, b2):
+    # ref: mlp, src/cuda/torch_bindings.cpp:815-841; returns (output, hidden activations)
+    x, w1, b1, w2, b2 = (_dense(t, x) for t in (x, w1, b1, w2, b2))
+    _require(x.dim() == 2 and w1.dim() == 2 and w2.dim() == 2 and b1.dim() == 1 and b2.dim() == 1
+             and x.shape[1] == w1.shape[0] and w1.shape[1] == w2.shape[0]
+             and b1.shape[0] == w1.shape[1] and b2.shape[0] == w2.shape[1], "Invalid MLP operand shapes")
+    rows, inputs = x.shape
+    hidden, outputs = w2.shape
+    h = torch.empty((rows, hidden), dtype=x.dtype, device=x.device)
+    out = torch.empty((rows, outputs), dtype=x.dtype, device=x.device)
+    with torch.cuda.device(x.device):
+        _native.context(x.device).call("mlp", _DTYPE_CODE[x.dtype], rows, inputs, hidden, outputs,
+                                       _pointer(x), _pointer(w1), _pointer(b1), _pointer(w2), _pointer(b2),
+                                       _pointer(h), _pointer(out))
+    return out, h
+
+
+def mlp_backward(x, w1, w2, hidden, gradient, needed=(True,) * 5):
+    """Gradients (dx, dw1, db1, dw2, db2) of mlp; entries not `needed` are None
+    (ref: mlp_backward_tensors, src/cuda/torch_bindings.cpp:925-966; C entry
+    include/camblas_cuda.h:87-94)."""
+    x, w1, w2, hidden, gradient = (_dense(t, x) for t in (x, w1, w2, hidden, gradient))
+    _require(x.dim() == 2 and w1.dim() == 2 and w2.dim() == 2 and hidden.dim() == 2 and gradient.dim() == 2
+             and x.shape[1] == w1.shape[0] and w1.shape[1] == w2.shape[0]
+             and tuple(hidden.shape) == (x.shape[0], w1.shape[1])
+             and tuple(gradient.shape) == (x.shape[0], w2.shape[1]), "Invalid backward operand shapes")
+    rows, inputs = x.shape
+    width, outputs = w2.shape
+
+    def empty(wanted, *shape):
+        return torch.empty(shape, dtype=x.dtype, device=x.device) if wanted else None
+
+    dh = empty(any(needed[:3]), rows, width)
+    dx, dw1, db1 = empty(needed[0], rows, inputs), empty(needed[1], inputs, width), empty(needed[2], width)
+    dw2, db2 = empty(needed[3], width, outputs), empty(needed[4], outputs)
+    with torch.cuda.device(x.device):
+        _native.context(x.device).call(
+            "mlp_backward", _DTYPE_CODE[x.dtype], rows, inputs, width, outputs, _pointer(x), _pointer(w1),
+            _pointer(w2), _pointer(hidden), _pointer(gradient), _pointer(dh), _pointer(dx), _pointer(dw1),
+            _pointer(db1), _pointer(dw2), _pointer(db2))
+    return dx, dw1, db1, dw2, db2
+
+
+class _Mlp(torch.autograd.Function):
+    """ref: MlpAutograd, src/cuda/torch_bindings.cpp:978-1002 — first derivatives only."""
+
+    @staticmethod
+    def forward(ctx, x, w1, b1, w2, b2):
+        output, hidden = _mlp_forward(x, w1, b1, w2, b2)
+        ctx.save_for_backward(x, w1, w2, hidden)
+        return output
+
+    @staticmethod
+    @torch.autograd.function.once_differentiable
+    def backward(ctx, gradient):
+        x, w1, w2, hidden = ctx.saved_tensors
+        return mlp_backward(x, w1, w2, hidden, gradient, tuple(ctx.needs_input_grad[:5]))
+
+
+def mlp(x, w1, b1, w2, b2):
+    """relu(x @ w1 + b1) @ w2 + b2 for FP32 / FP64 (ref: mlp_public,
+    src/cuda/torch_bindings.cpp:1003-1014; C entry include/camblas_cuda.h:76-78)."""
+    if torch.is_grad_enabled() and any(t.requires_grad for t in (x, w1, b1, w2, b2)):
+        return _Mlp.apply(x, w1, b1, w2, b2)
+    return _mlp_forward(x, w1, b1, w2, b2)[0]
+
+
+def attention(q, k, v, scale=None):
+    """softmax(scale * q @ k.T) @ v, dense and single-head, FP32 / FP64 (ref: attention_public,
+    src/cuda/torch_bindings.cpp:903-923; C entry include/camblas_cuda.h:80-85). With gradients
+    enabled the result is composed from differentiable products, as the reference does."""
+    _require(q.dim() == 2 and (scale is not None or q.shape[1] > 0),
+             "Attention requires a rank-two query and positive depth for the default scale")
+    value = float(scale) if scale is not None else 1.0 / float(q.shape[1]) ** 0.5
+    if torch.is_grad_enabled() and any(t.requires_grad for t in (q, k, v)):
+        scores = matmul_autograd(q, k.t()).mul(value)
+        return matmul_autograd(torch.softmax(scores, -1), v)
+    q, k, v = _dense(q, q), _dense(k, q), _dense(v, q)
+    _require(k.dim() == 2 and v.dim() == 2 and q.shape[1] == k.shape[1] and k.shape[0] == v.shape[0],
+             "Invalid attention operand shapes")
+    out = torch.empty((q.shape[0], v.shape[1]), dtype=q.dtype, device=q.device)
+    with torch.cuda.device(q.device):
+        _native.context(q.device).call("attention", _DTYPE_CODE[q.dtype], q.shape[0], k.shape[0],
+                                       q.shape[1], v.shape[1], ct.c_double(value), _pointer(q), _pointer(k),
+                                       _pointer(v), _pointer(out))
+    return out
 
 
 def _elementwise_pair(gate, up, name):

@@ -3,6 +3,7 @@
 #include "common.hpp"
 
 #include <algorithm>
+#include <limits>
 #include <cmath>
 #include <climits>
 #include <cstring>
@@ -95,15 +96,6 @@ bool is_n(char t) { return t == 'N' || t == 'n'; }
 bool is_t(char t) { return t == 'T' || t == 't'; }
 bool aligned(const void *p, size_t bytes) { return reinterpret_cast<uintptr_t>(p) % bytes == 0; }
 
-int unsupported(camblas_cuda_context *context, const char *what)
-{
-    if (!context)
-        return fail(nullptr, "missing context", 1);
-    std::snprintf(context->error, sizeof(context->error),
-                  "%s is not provided by the HIP linear backend", what);
-    return -1;
-}
-
 // Column-major GEMM shared by FP32/FP64 (ref: backend.cu:786-866): validation order, no-op and
 // beta-only cases, alias rejection, then the planner's choice.
 template <typename T, typename Scale, typename Launch>
@@ -194,27 +186,174 @@ extern "C" int camblas_cuda_set_algorithm(camblas_cuda_context *context, int alg
     return 0;
 }
 
+namespace camblas_hip
+{
+namespace
+{
+// FP32 / FP64 column-major GEMM on the context's stream, without the device scope: shared by the
+// public entry points and by the dense helpers below.
+int dense_gemm(camblas_cuda_context *context, char ta, char tb, int m, int n, int k, float alpha,
+               const float *a, int lda, const float *b, int ldb, float beta, float *c, int ldc)
+{
+    return gemm<float>(
+        context, "FP32", ta, tb, m, n, k, alpha, a, lda, b, ldb, beta, c, ldc,
+        [&] { return launch_scale_f32(context->stream, m, n, beta, c, ldc); },
+        [&](bool trans_a, bool trans_b) {
+            Plan plan = make_plan(0, context->algorithm, trans_a, trans_b, m, n, k, lda, ldb, ldc,
+                                  aligned(a, 16) && aligned(b, 16), context->compute_units);
+            context->counts[plan.counter]++;
+            hipError_t error;
+            if (plan.family == FAMILY_GEMV_F32) {
+                error = launch_gemv_f32(context->stream, m, k, alpha, a, lda, b, beta, c);
+                return error == hipSuccess ? 0 : fail(context, "FP32 native GEMV", error);
+            }
+            error = launch_generic_f32(context->stream, trans_a, trans_b, m, n, k, alpha, a, lda, b,
+                                       ldb, beta, c, ldc);
+            return error == hipSuccess ? 0 : fail(context, "classical GEMM", error);
+        });
+}
+
+// ref: src/cuda/backend.cu:1066-1073; FP64 has no matrix-core path here, every layout runs the
+// LDS-tiled FMA kernel
+int dense_gemm(camblas_cuda_context *context, char ta, char tb, int m, int n, int k, double alpha,
+               const double *a, int lda, const double *b, int ldb, double beta, double *c, int ldc)
+{
+    return gemm<double>(
+        context, "FP64", ta, tb, m, n, k, alpha, a, lda, b, ldb, beta, c, ldc,
+        [&] { return launch_scale_f64(context->stream, m, n, beta, c, ldc); },
+        [&](bool trans_a, bool trans_b) {
+            context->counts[0]++;
+            hipError_t error = launch_generic_f64(context->stream, trans_a, trans_b, m, n, k, alpha,
+                                                  a, lda, b, ldb, beta, c, ldc);
+            return error == hipSuccess ? 0 : fail(context, "classical FP64 GEMM", error);
+        });
+}
+
+// Row-major out[rows, columns] = x[rows, inner] . weight[inner, columns] + bias, optional ReLU
+// (ref: src/cuda/backend.cu:871-905): as a column-major product out^T = weight^T-view . x^T-view,
+// then one bias/activation pass.
+template <typename T>
+int affine(camblas_cuda_context *context, int rows, int inner, int columns, const T *x, const T *weight,
+           const T *bias, bool relu, T *output)
+{
+    if (rows < 0 || inner < 0 || columns < 0)
+        return fail(context, "invalid affine dimensions", 1);
+    if (rows == 0 || columns == 0)
+        return 0;
+    if (!output || !bias || (inner > 0 && (!x || !weight)))
+        return fail(context, "missing affine operand", 1);
+    context->counts[3]++;
+    int result = dense_gemm(context, 'N', 'N', columns, rows, inner, T(1), weight, std::max(1, columns),
+                            x, std::max(1, inner), T(0), output, columns);
+    if (result != 0)
+        return result;
+    hipError_t error = launch_bias_activation(context->stream, sizeof(T) == 4 ? 0 : 1, output, bias,
+                                              size_t(rows) * columns, columns, relu);
+    return error == hipSuccess ? 0 : fail(context, "bias/activation", error);
+}
+
+// softmax(scale . q k^T) v with the scores in context scratch (ref: src/cuda/fusion.cuh:95-157).
+template <typename T>
+int dense_attention(camblas_cuda_context *context, int queries, int keys, int depth, int values, T scale,
+                    const T *q, const T *k, const T *v, T *output)
+{
+    if (queries < 0 || keys < 0 || depth < 0 || values < 0)
+        return fail(context, "invalid attention dimensions", 1);
+    if (queries == 0 || values == 0)
+        return 0;
+    if (!output || (depth > 0 && !q) || (keys > 0 && depth > 0 && !k) || (keys > 0 && !v))
+        return fail(context, "missing attention operand", 1);
+    if (keys > 0 && size_t(queries) > std::numeric_limits<size_t>::max() / sizeof(T) / size_t(keys))
+        return fail(context, "attention scratch size overflow", 2);
+    context->counts[6]++;
+    hipError_t error = reserve_scratch(context, size_t(queries) * keys * sizeof(T));
+    if (error != hipSuccess)
+        return fail(context, "attention scratch", error);
+    T *scores = static_cast<T *>(context->scratch);
+    // scores[queries, keys] = q k^T (keys == 0: nothing to do; the product below then zeroes out)
+    int result = dense_gemm(context, 'T', 'N', keys, queries, depth, T(1), k, std::max(1, depth), q,
+                            std::max(1, depth), T(0), scores, std::max(1, keys));
+    if (result != 0)
+        return result;
+    error = launch_softmax_rows(context->stream, sizeof(T) == 4 ? 0 : 1, scores, queries, keys,
+                                double(scale));
+    if (error != hipSuccess)
+        return fail(context, "attention softmax", error);
+    return dense_gemm(context, 'N', 'N', values, queries, keys, T(1), v, std::max(1, values), scores,
+                      std::max(1, keys), T(0), output, std::max(1, values));
+}
+
+// Gradients of output = relu(x w1 + b1) w2 + b2 (ref: src/cuda/fusion.cuh:207-275). Null gradient
+// pointers are skipped; grad_hidden is scratch of the caller, left holding the masked gradient.
+template <typename T>
+int mlp_backward(camblas_cuda_context *context, int rows, int inputs, int hidden, int outputs, const T *x,
+                 const T *w1, const T *w2, const T *h, const T *grad, T *dh, T *dx, T *dw1, T *db1,
+                 T *dw2, T *db2)
+{
+    if (rows < 0 || inputs < 0 || hidden < 0 || outputs < 0)
+        return fail(context, "invalid backward dimensions", 1);
+    const bool first_layer = dx || dw1 || db1;
+    if ((rows > 0 && outputs > 0 && !grad) || (rows > 0 && hidden > 0 && first_layer && (!dh || !h)))
+        return fail(context, "missing backward operand", 1);
+    context->counts[7]++;
+    const int dtype = sizeof(T) == 4 ? 0 : 1;
+    // column sums run over chunks of 128 rows; more than one chunk goes through context scratch
+    const int chunks = int(std::min<size_t>(65535, std::max<size_t>(1, (size_t(rows) + 127) / 128)));
+    const int chunk_rows = std::max(1, int((int64_t(rows) + chunks - 1) / chunks));
+    T *partial = nullptr;
+    if (chunks > 1 && ((db2 && outputs > 0) || (db1 && hidden > 0))) {
+        hipError_t error =
+            reserve_scratch(context, size_t(chunks) * std::max(hidden, outputs) * sizeof(T));
+        if (error != hipSuccess)
+            return fail(context, "backward scratch", error);
+        partial = static_cast<T *>(context->scratch);
+    }
+    int result = 0;
+    if (dw2) { // dw2[hidden, outputs] = h^T grad
+        result = dense_gemm(context, 'N', 'T', outputs, hidden, rows, T(1), grad, std::max(1, outputs), h,
+                            std::max(1, hidden), T(0), dw2, std::max(1, outputs));
+        if (result != 0)
+            return result;
+    }
+    if (db2 && outputs > 0) {
+        hipError_t error = launch_column_sums(context->stream, dtype, false, const_cast<T *>(grad),
+                                              nullptr, rows, outputs, chunks, chunk_rows, partial, db2);
+        if (error != hipSuccess)
+            return fail(context, "backward bias", error);
+    }
+    if (!first_layer)
+        return 0;
+    // dh[rows, hidden] = grad w2^T, masked by the ReLU (h > 0), summed over rows for db1
+    result = dense_gemm(context, 'T', 'N', hidden, rows, outputs, T(1), w2, std::max(1, outputs), grad,
+                        std::max(1, outputs), T(0), dh, std::max(1, hidden));
+    if (result != 0)
+        return result;
+    if (hidden > 0) {
+        hipError_t error = launch_column_sums(context->stream, dtype, true, dh, h, rows, hidden, chunks,
+                                              chunk_rows, db1 ? partial : nullptr, db1);
+        if (error != hipSuccess)
+            return fail(context, "backward activation", error);
+    }
+    if (dw1) { // dw1[inputs, hidden] = x^T dh
+        result = dense_gemm(context, 'N', 'T', hidden, inputs, rows, T(1), dh, std::max(1, hidden), x,
+                            std::max(1, inputs), T(0), dw1, std::max(1, hidden));
+        if (result != 0)
+            return result;
+    }
+    if (dx) // dx[rows, inputs] = dh w1^T
+        result = dense_gemm(context, 'T', 'N', inputs, rows, hidden, T(1), w1, std::max(1, hidden), dh,
+                            std::max(1, hidden), T(0), dx, std::max(1, inputs));
+    return result;
+}
+} // namespace
+} // namespace camblas_hip
+
 extern "C" int camblas_cuda_sgemm(camblas_cuda_context *context, char ta, char tb, int m, int n,
                                   int k, float alpha, const float *a, int lda, const float *b,
                                   int ldb, float beta, float *c, int ldc)
 {
     return execute(context, [&] {
-        return gemm<float>(
-            context, "FP32", ta, tb, m, n, k, alpha, a, lda, b, ldb, beta, c, ldc,
-            [&] { return launch_scale_f32(context->stream, m, n, beta, c, ldc); },
-            [&](bool trans_a, bool trans_b) {
-                Plan plan = make_plan(0, context->algorithm, trans_a, trans_b, m, n, k, lda, ldb,
-                                      ldc, aligned(a, 16) && aligned(b, 16), context->compute_units);
-                context->counts[plan.counter]++;
-                hipError_t error;
-                if (plan.family == FAMILY_GEMV_F32) {
-                    error = launch_gemv_f32(context->stream, m, k, alpha, a, lda, b, beta, c);
-                    return error == hipSuccess ? 0 : fail(context, "FP32 native GEMV", error);
-                }
-                error = launch_generic_f32(context->stream, trans_a, trans_b, m, n, k, alpha, a,
-                                           lda, b, ldb, beta, c, ldc);
-                return error == hipSuccess ? 0 : fail(context, "classical GEMM", error);
-            });
+        return dense_gemm(context, ta, tb, m, n, k, alpha, a, lda, b, ldb, beta, c, ldc);
     });
 }
 
@@ -222,18 +361,8 @@ extern "C" int camblas_cuda_dgemm(camblas_cuda_context *context, char ta, char t
                                   int k, double alpha, const double *a, int lda, const double *b,
                                   int ldb, double beta, double *c, int ldc)
 {
-    // ref: src/cuda/backend.cu:1066-1073; FP64 has no matrix-core path here, every layout runs the
-    // LDS-tiled FMA kernel
     return execute(context, [&] {
-        return gemm<double>(
-            context, "FP64", ta, tb, m, n, k, alpha, a, lda, b, ldb, beta, c, ldc,
-            [&] { return launch_scale_f64(context->stream, m, n, beta, c, ldc); },
-            [&](bool trans_a, bool trans_b) {
-                context->counts[0]++;
-                hipError_t error = launch_generic_f64(context->stream, trans_a, trans_b, m, n, k,
-                                                      alpha, a, lda, b, ldb, beta, c, ldc);
-                return error == hipSuccess ? 0 : fail(context, "classical FP64 GEMM", error);
-            });
+        return dense_gemm(context, ta, tb, m, n, k, alpha, a, lda, b, ldb, beta, c, ldc);
     });
 }
 
@@ -321,31 +450,85 @@ extern "C" int camblas_cuda_bgemm(camblas_cuda_context *context, char trans_a, c
     });
 }
 
-extern "C" int camblas_cuda_affine(camblas_cuda_context *context, int, int, int, int, const void *,
-                                   const void *, const void *, int, void *)
+extern "C" int camblas_cuda_affine(camblas_cuda_context *context, int dtype, int rows, int inner,
+                                   int columns, const void *x, const void *weight, const void *bias,
+                                   int relu, void *output)
 {
-    return unsupported(context, "affine");
+    // ref: src/cuda/backend.cu:1086-1101
+    return execute(context, [&] {
+        if (dtype == 0)
+            return affine(context, rows, inner, columns, static_cast<const float *>(x),
+                          static_cast<const float *>(weight), static_cast<const float *>(bias),
+                          relu != 0, static_cast<float *>(output));
+        if (dtype == 1)
+            return affine(context, rows, inner, columns, static_cast<const double *>(x),
+                          static_cast<const double *>(weight), static_cast<const double *>(bias),
+                          relu != 0, static_cast<double *>(output));
+        return fail(context, "unsupported affine dtype", 1);
+    });
 }
 
-extern "C" int camblas_cuda_mlp(camblas_cuda_context *context, int, int, int, int, int,
-                                const void *, const void *, const void *, const void *,
-                                const void *, void *, void *)
+extern "C" int camblas_cuda_mlp(camblas_cuda_context *context, int dtype, int rows, int inputs,
+                                int hidden, int outputs, const void *x, const void *w1,
+                                const void *b1, const void *w2, const void *b2, void *hidden_output,
+                                void *output)
 {
-    return unsupported(context, "MLP");
+    // ref: src/cuda/backend.cu:1103-1117 — two affine layers, the first with ReLU; the hidden
+    // activations are an output of their own and may not share storage with the result
+    if (rows < 0 || inputs < 0 || hidden < 0 || outputs < 0 ||
+        (rows > 0 && hidden > 0 && hidden_output == output))
+        return fail(context, "invalid MLP dimensions or aliased outputs", 1);
+    int result =
+        camblas_cuda_affine(context, dtype, rows, inputs, hidden, x, w1, b1, 1, hidden_output);
+    if (result != 0)
+        return result;
+    return camblas_cuda_affine(context, dtype, rows, hidden, outputs, hidden_output, w2, b2, 0, output);
 }
 
-extern "C" int camblas_cuda_attention(camblas_cuda_context *context, int, int, int, int, int, double,
-                                      const void *, const void *, const void *, void *)
+extern "C" int camblas_cuda_attention(camblas_cuda_context *context, int dtype, int queries, int keys,
+                                      int depth, int values, double scale, const void *q,
+                                      const void *k, const void *v, void *output)
 {
-    return unsupported(context, "dense single-head attention");
+    // ref: src/cuda/backend.cu:1495-1510
+    return execute(context, [&] {
+        if (dtype == 0)
+            return dense_attention(context, queries, keys, depth, values, float(scale),
+                                   static_cast<const float *>(q), static_cast<const float *>(k),
+                                   static_cast<const float *>(v), static_cast<float *>(output));
+        if (dtype == 1)
+            return dense_attention(context, queries, keys, depth, values, scale,
+                                   static_cast<const double *>(q), static_cast<const double *>(k),
+                                   static_cast<const double *>(v), static_cast<double *>(output));
+        return fail(context, "unsupported attention dtype", 1);
+    });
 }
 
-extern "C" int camblas_cuda_mlp_backward(camblas_cuda_context *context, int, int, int, int, int,
-                                         const void *, const void *, const void *, const void *,
-                                         const void *, void *, void *, void *, void *, void *,
-                                         void *)
+extern "C" int camblas_cuda_mlp_backward(camblas_cuda_context *context, int dtype, int rows,
+                                         int inputs, int hidden, int outputs, const void *x,
+                                         const void *w1, const void *w2, const void *hidden_output,
+                                         const void *grad_output, void *grad_hidden, void *dx,
+                                         void *dw1, void *db1, void *dw2, void *db2)
 {
-    return unsupported(context, "MLP backward");
+    // ref: src/cuda/backend.cu:1512-1535
+    return execute(context, [&] {
+        if (dtype == 0)
+            return mlp_backward(context, rows, inputs, hidden, outputs, static_cast<const float *>(x),
+                                static_cast<const float *>(w1), static_cast<const float *>(w2),
+                                static_cast<const float *>(hidden_output),
+                                static_cast<const float *>(grad_output),
+                                static_cast<float *>(grad_hidden), static_cast<float *>(dx),
+                                static_cast<float *>(dw1), static_cast<float *>(db1),
+                                static_cast<float *>(dw2), static_cast<float *>(db2));
+        if (dtype == 1)
+            return mlp_backward(context, rows, inputs, hidden, outputs, static_cast<const double *>(x),
+                                static_cast<const double *>(w1), static_cast<const double *>(w2),
+                                static_cast<const double *>(hidden_output),
+                                static_cast<const double *>(grad_output),
+                                static_cast<double *>(grad_hidden), static_cast<double *>(dx),
+                                static_cast<double *>(dw1), static_cast<double *>(db1),
+                                static_cast<double *>(dw2), static_cast<double *>(db2));
+        return fail(context, "unsupported backward dtype", 1);
+    });
 }
 
 extern "C" int camblas_cuda_silu_multiply(camblas_cuda_context *context, int dtype, uint64_t count,

@@ -135,6 +135,16 @@ hipError_t launch_route_groups(hipStream_t stream, int tokens, int choices, int 
 hipError_t launch_reduce_groups(hipStream_t stream, int tokens, int choices, int width,
                                 int grouped_rows, const void *experts, const void *reverse,
                                 const void *input, void *output);
+// Dense helpers (dtype 0 FP32, 1 FP64): bias + optional ReLU over a row-major [count/columns, columns]
+// matrix; in-place softmax(scale * row); column sums in `chunks` row chunks (partial: [chunks, columns]
+// scratch when chunks > 1), optionally zeroing grad where activation <= 0 first.
+hipError_t launch_bias_activation(hipStream_t stream, int dtype, void *out, const void *bias,
+                                  size_t count, int columns, bool relu);
+hipError_t launch_softmax_rows(hipStream_t stream, int dtype, void *scores, int rows, int columns,
+                               double scale);
+hipError_t launch_column_sums(hipStream_t stream, int dtype, bool mask, void *grad,
+                              const void *activation, int rows, int columns, int chunks,
+                              int chunk_rows, void *partial, void *sums);
 hipError_t launch_fp8_quantise(hipStream_t stream, int rows, int inner, const void *x, void *q,
                                float *scale);
 hipError_t launch_silu_multiply(hipStream_t stream, int dtype, uint64_t count, const void *gate,

@@ -21,6 +21,7 @@
 #include <hip/hip_runtime_api.h>
 #include <unistd.h>
 
+#include <array>
 #include <cfloat>
 #include <climits>
 #include <cmath>
@@ -337,6 +338,238 @@ Tensor matmul_public(const Tensor &a, const Tensor &b, const std::optional<Tenso
         return MatmulFunction::apply(a, b, int64_t(algorithm));
     }
     return matmul(a, b, output, alpha, beta, algorithm);
+}
+
+// ---------------------------------------------------------------------------- dense helpers
+// x W + bias with optional ReLU, FP32 / FP64 (ref: src/cuda/torch_bindings.cpp:737-771).
+Tensor affine(const Tensor &x, const Tensor &weight, const Tensor &bias, bool relu,
+              const std::optional<Tensor> &output, int algorithm)
+{
+    check_tensor(x, x, false);
+    check_tensor(weight, x, false);
+    check_tensor(bias, x, false);
+    require(x.dim() == 2 && weight.dim() == 2 && bias.dim() == 1 && x.size(1) == weight.size(0) &&
+                weight.size(1) == bias.size(0),
+            "Invalid affine operand shapes");
+    c10::DeviceGuard guard(x.device());
+    const int rows = int(x.size(0)), inner = int(x.size(1)), columns = int(weight.size(1));
+    Tensor c;
+    if (output) {
+        c = *output;
+        check_tensor(c, x, false);
+        require(!c10::GradMode::is_enabled() || !c.requires_grad(),
+                "Autograd affine does not support an out tensor requiring gradients");
+        require(c.dim() == 2 && c.size(0) == rows && c.size(1) == columns && c.is_contiguous(),
+                "Invalid affine output shape or strides");
+        require(!c.is_alias_of(x) && !c.is_alias_of(weight) && !c.is_alias_of(bias),
+                "Affine output cannot alias an input");
+    } else {
+        c = at::empty({rows, columns}, x.options());
+    }
+    Tensor xc = x.contiguous(), wc = weight.contiguous(), bc = bias.contiguous();
+    camblas_cuda_context *context = context_for(x.get_device(), algorithm);
+    succeed(camblas_cuda_affine(context, x.scalar_type() == at::kDouble, rows, inner, columns,
+                                xc.const_data_ptr(), wc.const_data_ptr(), bc.const_data_ptr(), relu,
+                                c.mutable_data_ptr()),
+            context);
+    if (output && !c.is_inference())
+        torch::autograd::impl::bump_version(c);
+    return c;
+}
+
+// Gradients as products through matmul_public, so higher derivatives build a graph; with ReLU
+// the incoming gradient is zeroed where the output is not positive
+// (ref: src/cuda/torch_bindings.cpp:773-801).
+struct AffineFunction : torch::autograd::Function<AffineFunction> {
+    static Tensor forward(torch::autograd::AutogradContext *state, const Tensor &x,
+                          const Tensor &weight, const Tensor &bias, bool relu, int64_t algorithm)
+    {
+        Tensor output = affine(x, weight, bias, relu, std::nullopt, int(algorithm));
+        state->save_for_backward({x, weight, output});
+        state->saved_data["relu"] = relu;
+        state->saved_data["algorithm"] = algorithm;
+        return output;
+    }
+    static torch::autograd::variable_list backward(torch::autograd::AutogradContext *state,
+                                                   torch::autograd::variable_list gradients)
+    {
+        auto saved = state->get_saved_variables();
+        const int algorithm = int(state->saved_data["algorithm"].toInt());
+        Tensor gradient = gradients[0], dx, dw, db;
+        if (state->saved_data["relu"].toBool())
+            gradient = at::where(saved[2].le(0), 0, gradient);
+        if (state->needs_input_grad(0))
+            dx = matmul_public(gradient, saved[1].t(), std::nullopt, 1, 0, algorithm);
+        if (state->needs_input_grad(1))
+            dw = matmul_public(saved[0].t(), gradient, std::nullopt, 1, 0, algorithm);
+        if (state->needs_input_grad(2))
+            db = gradient.sum(at::IntArrayRef{0});
+        return {dx, dw, db, Tensor(), Tensor()};
+    }
+};
+
+Tensor affine_public(const Tensor &x, const Tensor &weight, const Tensor &bias, bool relu,
+                     int algorithm)
+{
+    same_process();
+    if (algorithm < 0)
+        algorithm = default_algorithm;
+    if (c10::GradMode::is_enabled() &&
+        (x.requires_grad() || weight.requires_grad() || bias.requires_grad()))
+        return AffineFunction::apply(x, weight, bias, relu, int64_t(algorithm));
+    return affine(x, weight, bias, relu, std::nullopt, algorithm);
+}
+
+// relu(x w1 + b1) w2 + b2; returns (output, hidden activations)
+// (ref: src/cuda/torch_bindings.cpp:815-841).
+std::pair<Tensor, Tensor> mlp(const Tensor &x, const Tensor &w1, const Tensor &b1, const Tensor &w2,
+                              const Tensor &b2, int algorithm)
+{
+    for (const Tensor *tensor : {&x, &w1, &b1, &w2, &b2})
+        check_tensor(*tensor, x, false);
+    require(x.dim() == 2 && w1.dim() == 2 && w2.dim() == 2 && b1.dim() == 1 && b2.dim() == 1 &&
+                x.size(1) == w1.size(0) && w1.size(1) == w2.size(0) && b1.size(0) == w1.size(1) &&
+                b2.size(0) == w2.size(1),
+            "Invalid MLP operand shapes");
+    c10::DeviceGuard guard(x.device());
+    const int rows = int(x.size(0)), inputs = int(x.size(1));
+    const int hidden = int(w1.size(1)), outputs = int(w2.size(1));
+    Tensor h = at::empty({rows, hidden}, x.options()), c = at::empty({rows, outputs}, x.options());
+    Tensor xc = x.contiguous(), w1c = w1.contiguous(), b1c = b1.contiguous();
+    Tensor w2c = w2.contiguous(), b2c = b2.contiguous();
+    camblas_cuda_context *context = context_for(x.get_device(), algorithm);
+    succeed(camblas_cuda_mlp(context, x.scalar_type() == at::kDouble, rows, inputs, hidden, outputs,
+                             xc.const_data_ptr(), w1c.const_data_ptr(), b1c.const_data_ptr(),
+                             w2c.const_data_ptr(), b2c.const_data_ptr(), h.mutable_data_ptr(),
+                             c.mutable_data_ptr()),
+            context);
+    return {c, h};
+}
+
+// (dx, dw1, db1, dw2, db2); entries not needed stay undefined
+// (ref: src/cuda/torch_bindings.cpp:925-966).
+std::array<Tensor, 5> mlp_backward_tensors(const Tensor &x, const Tensor &w1, const Tensor &w2,
+                                           const Tensor &h, const Tensor &gradient,
+                                           const std::array<bool, 5> &needed, int algorithm)
+{
+    for (const Tensor *tensor : {&x, &w1, &w2, &h, &gradient})
+        check_tensor(*tensor, x, false);
+    require(x.dim() == 2 && w1.dim() == 2 && w2.dim() == 2 && h.dim() == 2 && gradient.dim() == 2 &&
+                x.size(1) == w1.size(0) && w1.size(1) == w2.size(0) && h.size(0) == x.size(0) &&
+                h.size(1) == w1.size(1) && gradient.size(0) == x.size(0) &&
+                gradient.size(1) == w2.size(1),
+            "Invalid backward operand shapes");
+    c10::DeviceGuard guard(x.device());
+    const int rows = int(x.size(0)), inputs = int(x.size(1));
+    const int hidden = int(w1.size(1)), outputs = int(w2.size(1));
+    Tensor xc = x.contiguous(), w1c = w1.contiguous(), w2c = w2.contiguous();
+    Tensor hc = h.contiguous(), gc = gradient.contiguous();
+    Tensor dh, dx, dw1, db1, dw2, db2;
+    if (needed[0] || needed[1] || needed[2])
+        dh = at::empty({rows, hidden}, x.options());
+    if (needed[0])
+        dx = at::empty({rows, inputs}, x.options());
+    if (needed[1])
+        dw1 = at::empty({inputs, hidden}, x.options());
+    if (needed[2])
+        db1 = at::empty({hidden}, x.options());
+    if (needed[3])
+        dw2 = at::empty({hidden, outputs}, x.options());
+    if (needed[4])
+        db2 = at::empty({outputs}, x.options());
+    auto pointer = [](Tensor &tensor) { return tensor.defined() ? tensor.mutable_data_ptr() : nullptr; };
+    camblas_cuda_context *context = context_for(x.get_device(), algorithm);
+    succeed(camblas_cuda_mlp_backward(context, x.scalar_type() == at::kDouble, rows, inputs, hidden,
+                                      outputs, xc.const_data_ptr(), w1c.const_data_ptr(),
+                                      w2c.const_data_ptr(), hc.const_data_ptr(), gc.const_data_ptr(),
+                                      pointer(dh), pointer(dx), pointer(dw1), pointer(db1),
+                                      pointer(dw2), pointer(db2)),
+            context);
+    return {dx, dw1, db1, dw2, db2};
+}
+
+py::tuple mlp_backward_public(const Tensor &x, const Tensor &w1, const Tensor &w2, const Tensor &h,
+                              const Tensor &gradient, const std::array<bool, 5> &needed,
+                              int algorithm)
+{
+    same_process();
+    auto gradients = mlp_backward_tensors(x, w1, w2, h, gradient, needed,
+                                          algorithm < 0 ? default_algorithm : algorithm);
+    py::tuple result(5);
+    for (int i = 0; i < 5; ++i)
+        result[i] = needed[i] ? py::cast(gradients[i]) : py::none();
+    return result;
+}
+
+// First derivatives only (ref: src/cuda/torch_bindings.cpp:978-1002).
+struct MlpFunction : torch::autograd::Function<MlpFunction> {
+    static Tensor forward(torch::autograd::AutogradContext *state, const Tensor &x, const Tensor &w1,
+                          const Tensor &b1, const Tensor &w2, const Tensor &b2, int64_t algorithm)
+    {
+        auto output = mlp(x, w1, b1, w2, b2, int(algorithm));
+        state->save_for_backward({x, w1, w2, output.second});
+        state->saved_data["algorithm"] = algorithm;
+        return output.first;
+    }
+    static torch::autograd::variable_list backward(torch::autograd::AutogradContext *state,
+                                                   torch::autograd::variable_list gradients)
+    {
+        TORCH_CHECK(!c10::GradMode::is_enabled(),
+                    "MLP supports first derivatives; use two affine calls for higher derivatives");
+        auto saved = state->get_saved_variables();
+        const int algorithm = int(state->saved_data["algorithm"].toInt());
+        std::array<bool, 5> needed;
+        for (int i = 0; i < 5; ++i)
+            needed[i] = state->needs_input_grad(i);
+        auto result =
+            mlp_backward_tensors(saved[0], saved[1], saved[2], saved[3], gradients[0], needed, algorithm);
+        return {result[0], result[1], result[2], result[3], result[4], Tensor()};
+    }
+};
+
+Tensor mlp_public(const Tensor &x, const Tensor &w1, const Tensor &b1, const Tensor &w2,
+                  const Tensor &b2, int algorithm)
+{
+    same_process();
+    if (algorithm < 0)
+        algorithm = default_algorithm;
+    if (c10::GradMode::is_enabled() && (x.requires_grad() || w1.requires_grad() || b1.requires_grad() ||
+                                        w2.requires_grad() || b2.requires_grad()))
+        return MlpFunction::apply(x, w1, b1, w2, b2, int64_t(algorithm));
+    return mlp(x, w1, b1, w2, b2, algorithm).first;
+}
+
+// softmax(scale q k^T) v, dense and single-head; with gradients enabled it is composed from
+// differentiable products (ref: src/cuda/torch_bindings.cpp:880-923).
+Tensor attention_public(const Tensor &q, const Tensor &k, const Tensor &v,
+                        const std::optional<double> &scale, int algorithm)
+{
+    same_process();
+    require(q.dim() == 2 && (scale || q.size(1) > 0),
+            "Attention requires a rank-two query and positive depth for the default scale");
+    const double value = scale ? *scale : 1 / std::sqrt(double(q.size(1)));
+    if (algorithm < 0)
+        algorithm = default_algorithm;
+    if (c10::GradMode::is_enabled() && (q.requires_grad() || k.requires_grad() || v.requires_grad())) {
+        Tensor scores = matmul_public(q, k.t(), std::nullopt, 1, 0, algorithm).mul(value);
+        return matmul_public(at::softmax(scores, -1, std::nullopt), v, std::nullopt, 1, 0, algorithm);
+    }
+    check_tensor(q, q, false);
+    check_tensor(k, q, false);
+    check_tensor(v, q, false);
+    require(k.dim() == 2 && v.dim() == 2 && q.size(1) == k.size(1) && k.size(0) == v.size(0),
+            "Invalid attention operand shapes");
+    c10::DeviceGuard guard(q.device());
+    const int queries = int(q.size(0)), keys = int(k.size(0)), depth = int(q.size(1)),
+              values = int(v.size(1));
+    Tensor qc = q.contiguous(), kc = k.contiguous(), vc = v.contiguous();
+    Tensor output = at::empty({queries, values}, q.options());
+    camblas_cuda_context *context = context_for(q.get_device(), algorithm);
+    succeed(camblas_cuda_attention(context, q.scalar_type() == at::kDouble, queries, keys, depth, values,
+                                   value, qc.const_data_ptr(), kc.const_data_ptr(), vc.const_data_ptr(),
+                                   output.mutable_data_ptr()),
+            context);
+    return output;
 }
 
 // y = x W^T (+ bias) for W [outputs, inputs]; leading dimensions of x are flattened
@@ -914,6 +1147,30 @@ PYBIND11_MODULE(_camblas_cuda_torch, module)
                py::arg("out") = py::none(), py::arg("alpha") = 1., py::arg("beta") = 0.,
                py::arg("algorithm") = -1,
                "Multiply two GPU matrices (FP32, FP64 or BF16) with transpose views and autograd.");
+    module.def("affine_public", &affine_public, py::arg("x"), py::arg("weight"), py::arg("bias"),
+               py::kw_only(), py::arg("relu") = false, py::arg("algorithm") = -1);
+    module.def("mlp_public", &mlp_public, py::arg("x"), py::arg("w1"), py::arg("b1"), py::arg("w2"),
+               py::arg("b2"), py::kw_only(), py::arg("algorithm") = -1);
+    module.def("mlp_backward", &mlp_backward_public, py::arg("x"), py::arg("w1"), py::arg("w2"),
+               py::arg("hidden"), py::arg("gradient"), py::arg("needed"), py::arg("algorithm") = -1);
+    module.def(
+        "mlp",
+        [](const Tensor &x, const Tensor &w1, const Tensor &b1, const Tensor &w2, const Tensor &b2,
+           int algorithm) {
+            same_process();
+            return mlp(x, w1, b1, w2, b2, algorithm < 0 ? default_algorithm : algorithm);
+        },
+        py::arg("x"), py::arg("w1"), py::arg("b1"), py::arg("w2"), py::arg("b2"),
+        py::arg("algorithm") = -1);
+    module.def(
+        "attention",
+        [](const Tensor &q, const Tensor &k, const Tensor &v, double scale, int algorithm) {
+            c10::AutoGradMode inference(false);
+            return attention_public(q, k, v, scale, algorithm);
+        },
+        py::arg("q"), py::arg("k"), py::arg("v"), py::arg("scale"), py::arg("algorithm") = -1);
+    module.def("attention_public", &attention_public, py::arg("q"), py::arg("k"), py::arg("v"),
+               py::kw_only(), py::arg("scale") = py::none(), py::arg("algorithm") = -1);
     module.def("linear_public", &linear_public, py::arg("input"), py::arg("weight"),
                py::arg("bias") = py::none(), py::kw_only(), py::arg("algorithm") = -1,
                "Apply a linear transform with [outputs, inputs] weights and autograd.");

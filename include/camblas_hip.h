@@ -73,10 +73,22 @@ int camblas_cuda_dgemm(camblas_cuda_context *context, char trans_a, char trans_b
                        int k, double alpha, const double *a, int lda, const double *b, int ldb,
                        double beta, double *c, int ldc);
 
-/* ref: include/camblas_cuda.h:71-94. Present so the reference loader, which resolves these names
- * at load time, accepts the library; affine/MLP, dense single-head attention and MLP backward
- * are outside the linear path and return a negative status with the message
- * "... is not provided by the HIP linear backend". */
+/* Dense FP32 / FP64 helpers (dtype 0 FP32, 1 FP64), all arrays row-major, contiguous and owned by
+ * the caller. Products run through the same GEMM as sgemm / dgemm; the elementwise and reduction
+ * passes have a fixed order, so results repeat bit for bit.
+ * affine: output[rows, columns] = x[rows, inner] . weight[inner, columns] + bias[columns], then
+ *   ReLU when relu != 0 (NaN stays NaN). rows == 0 or columns == 0 succeeds without touching
+ *   anything; inner == 0 yields the bias (x and weight may be null).
+ *   ref: include/camblas_cuda.h:71-75, src/cuda/backend.cu:871-905, :1086-1101.
+ * mlp: hidden_output = relu(x . w1 + b1), output = hidden_output . w2 + b2; the two outputs may not
+ *   share storage. ref: include/camblas_cuda.h:76-78, src/cuda/backend.cu:1103-1117.
+ * attention: output[queries, values] = softmax(scale . q k^T) v, single head, no mask; the scores
+ *   live in context scratch (growth is refused during stream capture); keys == 0 gives zeros.
+ *   ref: include/camblas_cuda.h:80-85, src/cuda/fusion.cuh:95-157, backend.cu:1495-1510.
+ * mlp_backward: gradients of mlp; every non-null gradient pointer is filled; grad_hidden
+ *   [rows, hidden] is caller scratch, required when dx, dw1 or db1 is requested.
+ *   ref: include/camblas_cuda.h:87-94, src/cuda/fusion.cuh:207-275, backend.cu:1512-1535.
+ * Launch counters: affine -> slot 3, attention -> slot 6, mlp_backward -> slot 7. */
 int camblas_cuda_affine(camblas_cuda_context *context, int dtype, int rows, int inner, int columns,
                         const void *x, const void *weight, const void *bias, int relu,
                         void *output);

@@ -1,0 +1,212 @@
+"""Dense FP32 / FP64 helpers of the C ABI: affine, MLP, MLP gradients, single-head attention.
+
+Strategy and tolerances of the reference's tests/test_cuda.py (:38-58 assert_close: rtol 1e-5 /
+atol 3e-6 for FP32, 2e-13 / 3e-14 for FP64, NaN equal; :356-435 affine and MLP with changed inputs
+and exceptional values; :677-755 attention with unequal lengths, no keys, NaN queries and the
+register / loop boundaries of the softmax; :1264-1283 gradient subsets), with torch's CPU FP64
+arithmetic as the yardstick.
+"""
+
+import ctypes as ct
+
+import pytest
+import torch
+
+from camblas_amd import _kernels, _native
+
+pytestmark = pytest.mark.gpu
+
+DTYPES = [torch.float32, torch.float64]
+
+
+def close(actual, expected):
+    rtol, atol = (1e-5, 3e-6) if actual.dtype == torch.float32 else (2e-13, 3e-14)
+    torch.testing.assert_close(actual.cpu(), expected.to(actual.dtype).cpu(), rtol=rtol, atol=atol,
+                               equal_nan=True)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_affine_and_mlp_values_and_all_gradients(device, dtype):
+    torch.manual_seed(73013)
+    shapes = ((11, 17), (17, 23), (23,), (23, 13), (13,))
+    host = [torch.randn(shape, dtype=torch.float64) for shape in shapes]
+    inputs = [t.to(device=device, dtype=dtype).requires_grad_() for t in host]
+    wanted = [t.to(dtype).double().requires_grad_() for t in host]
+    x, w1, b1, w2, b2 = wanted
+    expected = torch.relu(x @ w1 + b1) @ w2 + b2
+    actual = _kernels.mlp(*inputs)
+    close(actual, expected)
+    weight = torch.randn(expected.shape, dtype=torch.float64)
+    (actual * weight.to(device=device, dtype=dtype)).sum().backward()
+    (expected * weight.to(dtype).double()).sum().backward()
+    for tensor, oracle in zip(inputs, wanted):
+        close(tensor.grad, oracle.grad)
+    for relu in (False, True):
+        x, w1, b1 = (t.detach().clone().requires_grad_() for t in inputs[:3])
+        xr, wr, br = (t.detach().double().cpu().requires_grad_() for t in (x, w1, b1))
+        expected = xr @ wr + br
+        if relu:
+            expected = torch.relu(expected)
+        actual = _kernels.affine(x, w1, b1, relu=relu)
+        close(actual, expected)
+        actual.square().sum().backward()
+        expected.square().sum().backward()
+        for tensor, oracle in ((x, xr), (w1, wr), (b1, br)):
+            close(tensor.grad, oracle.grad)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("rows,inner,columns", [(1, 17, 23), (13, 17, 1), (13, 17, 23), (130, 70, 65)])
+def test_affine_changed_inputs_and_exceptional_values(device, dtype, rows, inner, columns):
+    torch.manual_seed(705537)
+    x = torch.randn((rows, inner), dtype=dtype) * 0.1
+    weight = torch.randn((inner, columns), dtype=dtype) * 0.1
+    bias = torch.randn((columns,), dtype=dtype) * 0.1
+    for relu in (False, True, False):
+        for changed in (False, True):
+            ax = x + (0.03 if changed else 0)
+            aw = weight * (0.7 if changed else 1)
+            ab = bias + (0.04 if changed else 0)
+            expected = ax.double() @ aw.double() + ab.double()
+            if relu:
+                expected = torch.relu(expected)
+            close(_kernels.affine(ax.to(device), aw.to(device), ab.to(device), relu=relu), expected)
+    for value in (float("nan"), float("inf"), -float("inf")):
+        for operand in range(3):
+            tensors = [x.clone(), weight.clone(), bias.clone()]
+            tensors[operand].reshape(-1)[0] = value
+            expected = tensors[0].double() @ tensors[1].double() + tensors[2].double()
+            for relu in (False, True):
+                close(_kernels.affine(*(t.to(device) for t in tensors), relu=relu),
+                      torch.relu(expected) if relu else expected)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_attention_lengths_no_keys_and_nan(device, dtype):
+    torch.manual_seed(20261004)
+    q = torch.randn((13, 17), dtype=dtype)
+    k = torch.randn((19, 17), dtype=dtype)
+    v = torch.randn((19, 23), dtype=dtype)
+    for scale in (0.25, -0.5, 0):
+        expected = torch.softmax((q.double() @ k.double().T) * scale, dim=-1) @ v.double()
+        close(_kernels.attention(q.to(device), k.to(device), v.to(device), scale=scale), expected)
+    expected = torch.softmax((q.double() @ k.double().T) / 17 ** 0.5, dim=-1) @ v.double()
+    close(_kernels.attention(q.to(device), k.to(device), v.to(device)), expected)
+    none = _kernels.attention(q.to(device), torch.empty((0, 17), dtype=dtype, device=device),
+                              torch.empty((0, 23), dtype=dtype, device=device))
+    assert torch.equal(none, torch.zeros((13, 23), dtype=dtype, device=device))
+    q[0, 0] = float("nan")
+    expected = torch.softmax((q.double() @ k.double().T) * 0, dim=-1) @ v.double()
+    close(_kernels.attention(q.to(device), k.to(device), v.to(device), scale=0), expected)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("keys", [1, 17, 255, 256, 257, 511, 512, 513, 1023, 1024, 1025, 2047, 2048, 2049,
+                                  4095, 4096, 4097])
+def test_attention_row_width_boundaries(device, dtype, keys):
+    torch.manual_seed(717 + keys)
+    q = torch.randn((7, 17), dtype=dtype) * 0.1
+    k = torch.randn((keys, 17), dtype=dtype) * 0.1
+    v = torch.randn((keys, 23), dtype=dtype) * 0.1
+    for scale in (0.25, -0.5, 0, 256):
+        expected = torch.softmax((q.double() @ k.double().T) * scale, dim=-1) @ v.double()
+        close(_kernels.attention(q.to(device), k.to(device), v.to(device), scale=scale), expected)
+    q.add_(0.03)
+    v.mul_(0.7)
+    expected = torch.softmax((q.double() @ k.double().T) * 0.25, dim=-1) @ v.double()
+    close(_kernels.attention(q.to(device), k.to(device), v.to(device), scale=0.25), expected)
+    if keys in (257, 1025, 4096, 4097):
+        q[0, 0] = float("nan")
+        expected = torch.softmax((q.double() @ k.double().T) * 0, dim=-1) @ v.double()
+        close(_kernels.attention(q.to(device), k.to(device), v.to(device), scale=0), expected)
+
+
+def test_attention_gradients(device):
+    torch.manual_seed(842)
+    q = torch.randn((3, 4), device=device, dtype=torch.float64, requires_grad=True)
+    k = torch.randn((5, 4), device=device, dtype=torch.float64, requires_grad=True)
+    v = torch.randn((5, 2), device=device, dtype=torch.float64, requires_grad=True)
+    assert torch.autograd.gradcheck(_kernels.attention, (q, k, v))
+
+
+@pytest.mark.parametrize("index", range(5))
+def test_mlp_single_requested_gradient(device, index):
+    torch.manual_seed(413 + index)
+    shapes = ((5, 7), (7, 11), (11,), (11, 3), (3,))
+    inputs = [torch.randn(s, device=device, dtype=torch.float64).requires_grad_(i == index)
+              for i, s in enumerate(shapes)]
+    wanted = [t.detach().cpu().clone().requires_grad_(i == index) for i, t in enumerate(inputs)]
+    x, w1, b1, w2, b2 = wanted
+    expected = torch.relu(x @ w1 + b1) @ w2 + b2
+    actual = _kernels.mlp(*inputs)
+    actual.sum().backward()
+    expected.sum().backward()
+    close(inputs[index].grad, wanted[index].grad)
+    assert all(t.grad is None for i, t in enumerate(inputs) if i != index)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("rows", [1, 127, 128, 129, 700])
+def test_mlp_backward_row_chunks_repeat_bitwise(device, dtype, rows):
+    # more than 128 rows: the bias gradients are summed in row chunks through context scratch
+    torch.manual_seed(rows)
+    x = torch.randn((rows, 19), dtype=dtype, device=device)
+    w1 = torch.randn((19, 70), dtype=dtype, device=device)
+    w2 = torch.randn((70, 9), dtype=dtype, device=device)
+    hidden = torch.relu(torch.randn((rows, 70), dtype=dtype, device=device))
+    gradient = torch.randn((rows, 9), dtype=dtype, device=device)
+    first = _kernels.mlp_backward(x, w1, w2, hidden, gradient)
+    again = _kernels.mlp_backward(x, w1, w2, hidden, gradient)
+    g, h = gradient.double().cpu(), hidden.double().cpu()
+    dh = (g @ w2.double().cpu().T) * (h > 0)
+    expected = (dh @ w1.double().cpu().T, x.double().cpu().T @ dh, dh.sum(0), h.T @ g, g.sum(0))
+    for got, repeat, want in zip(first, again, expected):
+        assert torch.equal(got, repeat)
+        rtol, atol = (2e-5, 2e-5) if dtype == torch.float32 else (2e-13, 1e-12)
+        torch.testing.assert_close(got.cpu(), want.to(dtype), rtol=rtol, atol=atol)
+    only = _kernels.mlp_backward(x, w1, w2, hidden, gradient, (False, False, False, True, True))
+    assert only[:3] == (None, None, None) and torch.equal(only[3], first[3]) and torch.equal(only[4], first[4])
+
+
+def test_c_abi_validation_counters_and_empty_shapes(device):
+    native = _native.context(device)
+    library = _native.library()
+    handle = native.handle
+    buffer = torch.zeros(64, dtype=torch.float32, device=device)
+    p = ct.c_void_p(buffer.data_ptr())
+    before = _native.stats(device)
+    # negative sizes, unknown dtype, missing operands, aliased MLP outputs
+    assert library.camblas_cuda_affine(handle, 0, -1, 2, 2, p, p, p, 0, p) != 0
+    assert b"affine" in library.camblas_cuda_error(handle)
+    assert library.camblas_cuda_affine(handle, 2, 2, 2, 2, p, p, p, 0, p) != 0
+    assert library.camblas_cuda_affine(handle, 0, 2, 2, 2, p, p, None, 0, p) != 0
+    assert library.camblas_cuda_affine(handle, 0, 2, 2, 2, None, p, p, 0, p) != 0
+    assert library.camblas_cuda_mlp(handle, 0, 2, 2, 2, 2, p, p, p, p, p, p, p) != 0
+    assert b"alias" in library.camblas_cuda_error(handle)
+    assert library.camblas_cuda_attention(handle, 0, 2, -2, 2, 2, ct.c_double(1), p, p, p, p) != 0
+    assert library.camblas_cuda_attention(handle, 3, 2, 2, 2, 2, ct.c_double(1), p, p, p, p) != 0
+    assert library.camblas_cuda_attention(handle, 0, 2, 2, 2, 2, ct.c_double(1), p, p, None, p) != 0
+    assert library.camblas_cuda_mlp_backward(handle, 0, 2, 2, 2, 2, p, p, p, p, None, p, p, p, p, p, p) != 0
+    assert library.camblas_cuda_mlp_backward(handle, 0, 2, 2, 2, 2, p, p, p, p, p, None, p, None, None, None, None) != 0
+    # empty shapes succeed without touching anything
+    assert library.camblas_cuda_affine(handle, 0, 0, 2, 2, None, None, None, 0, None) == 0
+    assert library.camblas_cuda_attention(handle, 1, 0, 2, 2, 2, ct.c_double(1), None, None, None, None) == 0
+    # inner == 0: the result is the bias (x and weight may be absent)
+    bias = torch.tensor([1.0, -2.0, 3.0], device=device)
+    out = torch.full((2, 3), 7.0, device=device)
+    assert library.camblas_cuda_affine(handle, 0, 2, 0, 3, None, None, ct.c_void_p(bias.data_ptr()), 1,
+                                       ct.c_void_p(out.data_ptr())) == 0
+    torch.cuda.synchronize()
+    assert torch.equal(out, torch.relu(bias).expand(2, 3))
+    middle = _native.stats(device)
+    assert middle["affine"] == before["affine"] + 1
+    x = torch.randn((4, 5), device=device)
+    _kernels.mlp(x, torch.randn((5, 6), device=device), torch.randn(6, device=device),
+                 torch.randn((6, 3), device=device), torch.randn(3, device=device))
+    _kernels.attention(x, x, x)
+    _kernels.mlp_backward(x, torch.randn((5, 6), device=device), torch.randn((6, 3), device=device),
+                          torch.randn((4, 6), device=device), torch.randn((4, 3), device=device))
+    after = _native.stats(device)
+    assert after["affine"] == middle["affine"] + 2
+    assert after["attention"] == middle["attention"] + 1
+    assert after["backward"] == middle["backward"] + 1

@@ -144,7 +144,7 @@ def test_invalid_arguments_report_errors(device):
                                   None, 1) == -1
     assert b"invalid device pointer" in lib.camblas_cuda_error(native.handle)
     assert lib.camblas_cuda_affine(native.handle, 0, 1, 1, 1, None, None, None, 0, None) == -1
-    assert b"not provided" in lib.camblas_cuda_error(native.handle)
+    assert b"missing affine operand" in lib.camblas_cuda_error(native.handle)
 
 
 @pytest.mark.parametrize("ta", "NT")

@@ -87,6 +87,50 @@ def test_matmul_public_autograd(binding, device):
     assert torch.autograd.gradcheck(lambda u, v: binding.matmul_public(u, v), (a2, b2))
 
 
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float64])
+def test_dense_helpers_with_gradients(binding, device, dtype):
+    # affine / MLP / attention of the binding against CPU FP64 autograd
+    # (ref: tests/test_cuda.py:356-378, :485-509, :677-698, :1264-1283)
+    tight = dict(rtol=1e-5, atol=3e-6) if dtype == torch.float32 else dict(rtol=2e-13, atol=3e-14)
+    shapes = ((11, 17), (17, 23), (23,), (23, 13), (13,))
+    inputs = [randn(shape, dtype, device, 40 + i).requires_grad_() for i, shape in enumerate(shapes)]
+    wanted = [t.detach().double().cpu().requires_grad_() for t in inputs]
+    x, w1, b1, w2, b2 = wanted
+    expected = torch.relu(x @ w1 + b1) @ w2 + b2
+    actual = binding.mlp_public(*inputs)
+    torch.testing.assert_close(actual.cpu(), expected.to(dtype), **tight)
+    actual.square().sum().backward()
+    expected.square().sum().backward()
+    for tensor, oracle in zip(inputs, wanted):
+        torch.testing.assert_close(tensor.grad.cpu(), oracle.grad.to(dtype), **tight)
+    output, hidden = binding.mlp(*(t.detach() for t in inputs))
+    torch.testing.assert_close(hidden.cpu(), torch.relu(x @ w1 + b1).detach().to(dtype), **tight)
+    only = binding.mlp_backward(inputs[0].detach(), inputs[1].detach(), inputs[3].detach(), hidden,
+                                torch.ones_like(output), [False, False, True, False, True])
+    assert only[0] is None and only[1] is None and only[3] is None
+    torch.testing.assert_close(only[4].cpu(), torch.full((13,), 11.0, dtype=dtype), **tight)
+    for relu in (False, True):
+        got = binding.affine_public(inputs[0].detach(), inputs[1].detach(), inputs[2].detach(), relu=relu)
+        want = (x @ w1 + b1).detach()
+        torch.testing.assert_close(got.cpu(), (torch.relu(want) if relu else want).to(dtype), **tight)
+    q, k, v = (randn(shape, dtype, device, 50 + i) for i, shape in enumerate(((13, 17), (19, 17), (19, 23))))
+    want = torch.softmax(q.double().cpu() @ k.double().cpu().T / 17 ** 0.5, -1) @ v.double().cpu()
+    torch.testing.assert_close(binding.attention_public(q, k, v).cpu(), want.to(dtype), **tight)
+    torch.testing.assert_close(binding.attention(q, k, v, 0.25).cpu(),
+                               (torch.softmax(q.double().cpu() @ k.double().cpu().T * 0.25, -1)
+                                @ v.double().cpu()).to(dtype), **tight)
+    if dtype == torch.float64:
+        small = [randn(shape, dtype, device, 60 + i).requires_grad_() for i, shape in
+                 enumerate(((3, 4), (4, 5), (5,)))]
+        assert torch.autograd.gradcheck(lambda a, b, c: binding.affine_public(a, b, c, relu=True), small)
+        assert torch.autograd.gradgradcheck(lambda a, b, c: binding.affine_public(a, b, c), small)
+        qkv = [randn(shape, dtype, device, 70 + i).requires_grad_() for i, shape in
+               enumerate(((3, 4), (5, 4), (5, 2)))]
+        assert torch.autograd.gradcheck(lambda a, b, c: binding.attention_public(a, b, c), qkv)
+    with pytest.raises(ValueError, match="affine"):
+        binding.affine_public(inputs[0], inputs[1].t(), inputs[2])
+
+
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 def test_linear_public(binding, device, dtype):
     x = randn((3, 5, 256), dtype, device, 11)
