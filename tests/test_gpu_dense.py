@@ -19,8 +19,10 @@ pytestmark = pytest.mark.gpu
 DTYPES = [torch.float32, torch.float64]
 
 
-def close(actual, expected):
+def close(actual, expected, magnitude=1.0):
+    # magnitude: size of the terms behind an output, where sums of large terms nearly cancel
     rtol, atol = (1e-5, 3e-6) if actual.dtype == torch.float32 else (2e-13, 3e-14)
+    atol *= magnitude
     torch.testing.assert_close(actual.cpu(), expected.to(actual.dtype).cpu(), rtol=rtol, atol=atol,
                                equal_nan=True)
 
@@ -210,3 +212,99 @@ def test_c_abi_validation_counters_and_empty_shapes(device):
     assert after["affine"] == middle["affine"] + 2
     assert after["attention"] == middle["attention"] + 1
     assert after["backward"] == middle["backward"] + 1
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_captured_attention_survives_scratch_growth(device, dtype):
+    # a captured graph keeps using the score storage it was captured with after a larger call has
+    # made the context allocate a new one (ref: tests/test_cuda.py:511-538)
+    torch.manual_seed(3)
+    stream = torch.cuda.Stream()
+    stream.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(stream):
+        q = torch.randn((17, 16), device=device, dtype=dtype)
+        k = torch.randn((513, 16), device=device, dtype=dtype)
+        v = torch.randn((513, 13), device=device, dtype=dtype)
+        for _ in range(3):
+            _kernels.attention(q, k, v)
+    stream.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph, stream=stream):
+        captured = _kernels.attention(q, k, v)
+    with torch.cuda.stream(stream):
+        larger = [torch.randn(shape, device=device, dtype=dtype) for shape in ((129, 16), (4097, 16), (4097, 13))]
+        _kernels.attention(*larger)
+        for _ in range(3):
+            q.add_(0.1)
+            v.mul_(0.9)
+            graph.replay()
+            stream.synchronize()
+            expected = torch.softmax((q.double().cpu() @ k.double().cpu().T) / 4, dim=-1) @ v.double().cpu()
+            close(captured, expected)
+    stream.synchronize()
+    torch.cuda.current_stream().wait_stream(stream)
+    graph.reset()
+
+
+def test_scratch_growth_is_refused_during_capture(device):
+    # (ref: src/cuda/backend.cu:399-426) a first large call inside a capture cannot allocate
+    stream = torch.cuda.Stream()
+    stream.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(stream):
+        q = torch.randn((8, 16), device=device)
+        _kernels.attention(q, q, q)  # creates the context of this stream
+        big_q = torch.randn((3000, 16), device=device)
+        big_k = torch.randn((3100, 16), device=device)
+    stream.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with pytest.raises(RuntimeError, match="scratch"):
+        with torch.cuda.graph(graph, stream=stream):
+            _kernels.attention(big_q, big_k, big_k)
+    torch.cuda.synchronize()
+    with torch.cuda.stream(stream):
+        out = _kernels.attention(big_q, big_k, big_k)  # fine outside a capture
+    stream.synchronize()
+    assert torch.isfinite(out).all()
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_captured_mlp_training_step_replays_with_changed_inputs(device, dtype):
+    # forward and backward captured once, replayed after the inputs change and after a larger call
+    # has grown the context's scratch (ref: tests/test_cuda.py:540-583)
+    torch.manual_seed(4)
+    shapes = ((129, 17), (17, 23), (23,), (23, 13), (13,))
+    stream = torch.cuda.Stream()
+    stream.wait_stream(torch.cuda.current_stream())
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.stream(stream):
+        inputs = [torch.randn(shape, device=device, dtype=dtype, requires_grad=True) for shape in shapes]
+        for _ in range(3):
+            for value in inputs:
+                value.grad = None
+            _kernels.mlp(*inputs).square().mean().backward()
+        for value in inputs:
+            value.grad = None
+        with torch.cuda.graph(graph, stream=stream):
+            output = _kernels.mlp(*inputs)
+            output.square().mean().backward()
+        larger = [torch.randn(shape, device=device, dtype=dtype, requires_grad=True)
+                  for shape in ((513, 17), (17, 23), (23,), (23, 13), (13,))]
+        _kernels.mlp(*larger).square().mean().backward()
+        for _ in range(3):
+            with torch.no_grad():
+                inputs[0].add_(0.03)
+                inputs[1].mul_(0.9)
+                inputs[2].sub_(0.01)
+            graph.replay()
+            stream.synchronize()
+            wanted = [value.detach().double().cpu().requires_grad_(True) for value in inputs]
+            x, w1, b1, w2, b2 = wanted
+            expected = torch.relu(x @ w1 + b1) @ w2 + b2
+            expected.square().mean().backward()
+            # outputs of size 30 from 23 terms: the absolute tolerance follows that size
+            close(output.detach(), expected.detach(), magnitude=10)
+            for actual, desired in zip(inputs, wanted):
+                close(actual.grad, desired.grad, magnitude=10)
+    torch.cuda.current_stream().wait_stream(stream)
+    torch.cuda.synchronize()
+    graph.reset()
