@@ -1,0 +1,146 @@
+"""SGLang plugin mirror on the GPU: each around-hook is called the way SGLang's registry would call
+it (original callable first), inside and outside its guard. Routed results are compared with the
+oracle or an FP64 product; everything outside a guard must reach the original untouched; the
+dispatch counters follow camblas/sglang.py:11-19 of the reference."""
+
+import types
+
+import numpy as np
+import pytest
+import torch
+
+import oracle
+from camblas_amd import _kernels, sglang as plugin
+from helpers import bf16_values, rel_frobenius, to_device_bf16, to_device_fp8
+
+pytestmark = pytest.mark.gpu
+
+
+class Original:
+    """Stands for SGLang's own function: records that it was reached."""
+
+    def __init__(self):
+        self.calls = []
+
+    def __call__(self, *arguments):
+        self.calls.append(arguments)
+        return "original"
+
+
+def delta(before, name):
+    return plugin.dispatch_counts().get(name, 0) - before.get(name, 0)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_linear_hook_routes_and_falls_back(device, dtype):
+    hook = plugin.build_hooks({"linear"})[plugin.LINEAR_TARGET]
+    assert set(plugin.build_hooks({"linear"})) == {plugin.LINEAR_TARGET}
+    generator = torch.Generator().manual_seed(11)
+    x = torch.randn((3, 5, 256), generator=generator).to(dtype).to(device)
+    weight = (torch.randn((96, 256), generator=generator) * 0.05).to(dtype).to(device)
+    bias = torch.randn((96,), generator=generator).to(dtype).to(device)
+    layer = types.SimpleNamespace(weight=weight)
+    original, before = Original(), plugin.dispatch_counts()
+    for b in (None, bias):
+        out = hook(original, object(), layer, x, b)
+        want = x.double().cpu() @ weight.double().cpu().T + (0 if b is None else b.double().cpu())
+        assert out.shape == (3, 5, 96) and out.dtype == dtype
+        assert rel_frobenius(out.double().cpu().numpy(), want.numpy()) <= (1e-5 if dtype == torch.float32 else 1e-2)
+    assert delta(before, "linear") == 2 and not original.calls
+    # outside the guard: CPU tensors, mixed dtypes, strided input, FP16, gradients wanted
+    refused = [
+        (x.cpu(), types.SimpleNamespace(weight=weight.cpu()), None),
+        (x, types.SimpleNamespace(weight=weight.double()), None),
+        (x.transpose(0, 1), layer, None),
+        (x.half(), types.SimpleNamespace(weight=weight.half()), None),
+        (x[0, 0], layer, None),
+    ]
+    for value, owner, b in refused:
+        assert hook(original, "method", owner, value, b) == "original"
+    with torch.enable_grad():
+        wanted = x.float().requires_grad_() if dtype == torch.float32 else x.clone().requires_grad_()
+        assert hook(original, "method", layer, wanted, None) == "original"
+    assert len(original.calls) == len(refused) + 1 and delta(before, "linear") == 2
+    assert original.calls[0][0] == "method"
+
+
+@pytest.mark.parametrize("rows", [1, 5, 200])
+def test_fp8_block128_hook(device, rows):
+    hooks = plugin.build_hooks({"fp8"})
+    assert set(hooks) == {plugin.FP8_BLOCK128_TARGET, plugin.FP8_BLOCK32_PRODUCT_TARGET,
+                          plugin.FP8_BLOCK32_LINEAR_TARGET}
+    hook = hooks[plugin.FP8_BLOCK128_TARGET]
+    outputs, inner = 640, 1024
+    x = oracle.fill_normal_bf16(910 + rows, (rows, inner))
+    w, w_scale = oracle.fill_fp8_blocks(911, outputs, inner, 128)
+    xt, wt, st = to_device_bf16(x, device), to_device_fp8(w, device), torch.from_numpy(w_scale).to(device)
+    original, before = Original(), plugin.dispatch_counts()
+    # like the reference's, this guard wants gradient mode off altogether (SGLang serves that way)
+    assert hook(original, xt.view(1, rows, inner), wt, [128, 128], st) == "original"
+    del original.calls[:]
+    torch.set_grad_enabled(False)
+    try:
+        block128_checks(hook, original, before, device, rows, outputs, inner, x, w, w_scale, xt, wt, st)
+    finally:
+        torch.set_grad_enabled(True)
+
+
+def block128_checks(hook, original, before, device, rows, outputs, inner, x, w, w_scale, xt, wt, st):
+    out = hook(original, xt.view(1, rows, inner), wt, [128, 128], st)
+    assert out.shape == (1, rows, outputs) and out.dtype == torch.bfloat16
+    q, scale = oracle.quantise_1x128(x)
+    assert rel_frobenius(bf16_values(out).reshape(rows, outputs),
+                         oracle.fp8_block_matmul_f64(q, scale, w, w_scale)) <= 1e-2
+    assert delta(before, "fp8") == 1 and delta(before, "fp8_dense_block128") == 1 and not original.calls
+    # other block sizes, given input scales, a bias, FP16 activations, a wrong scale grid: original
+    assert hook(original, xt, wt, [64, 64], st) == "original"
+    assert hook(original, xt, wt, [128, 128], st, torch.ones((rows, inner // 128), device=device)) == "original"
+    assert hook(original, xt, wt, [128, 128], st, None, torch.zeros(outputs, device=device)) == "original"
+    assert hook(original, xt.half(), wt, [128, 128], st) == "original"
+    assert hook(original, xt, wt, [128, 128], st[:, :-1].contiguous()) == "original"
+    assert len(original.calls) == 5 and delta(before, "fp8") == 1
+    assert len(original.calls[1]) == 6  # all six arguments are forwarded
+
+
+def block32_case(seed, outputs, inner):
+    rng = np.random.default_rng(seed)
+    x = oracle.f32_to_e4m3((rng.standard_normal(inner) * 4).astype(np.float32))
+    w = oracle.f32_to_e4m3((rng.standard_normal((outputs, inner)) * 4).astype(np.float32))
+    sx = np.exp2(rng.integers(-6, 2, inner // 32)).astype(np.float32)
+    sw = rng.uniform(0.01, 0.1, ((outputs + 31) // 32, inner // 32)).astype(np.float32)
+    return x, sx, w, sw
+
+
+def test_fp8_block32_hooks(device):
+    hooks = plugin.build_hooks({"fp8"})
+    product, linear = hooks[plugin.FP8_BLOCK32_PRODUCT_TARGET], hooks[plugin.FP8_BLOCK32_LINEAR_TARGET]
+    outputs, inner = 1152, 5120
+    x, sx, w, sw = block32_case(77, outputs, inner)
+    A = to_device_fp8(x, device).view(1, inner)
+    As = torch.from_numpy(sx).to(device).view(1, -1)
+    B, Bs = to_device_fp8(w, device), torch.from_numpy(sw).to(device)
+    original, before = Original(), plugin.dispatch_counts()
+    out = product(original, A, B, As, Bs, [32, 32], torch.bfloat16)
+    want = oracle.bf16_to_f32(oracle.fp8_block32_decode(x, sx, w, sw))
+    assert out.shape == (1, outputs)
+    assert (np.abs(bf16_values(out)[0] - want) <= 2.0 ** -7 * np.abs(want) + 1e-4 * np.abs(want).max()).all()
+    assert delta(before, "fp8") == 1 and delta(before, f"fp8_decode:{outputs},{inner}") == 1
+    # FP16 output (SGLang's default), two rows, another block size: original
+    assert product(original, A, B, As, Bs, [32, 32]) == "original"
+    two = torch.cat([A, A])
+    assert product(original, two, B, torch.cat([As, As]), Bs, [32, 32], torch.bfloat16) == "original"
+    assert product(original, A, B, As, Bs, [128, 128], torch.bfloat16) == "original"
+    assert len(original.calls) == 3 and len(original.calls[0]) == 6
+
+    activations = oracle.fill_normal_bf16(78, (1, inner), std=3.0)
+    xt = to_device_bf16(activations, device)
+    out = linear(original, xt, B, [32, 32], Bs, None, None, True, None)
+    q, scale = oracle.quantise_block32(activations[0])
+    want = oracle.bf16_to_f32(oracle.fp8_block32_decode(q, scale, w, sw))
+    assert (np.abs(bf16_values(out)[0] - want) <= 2.0 ** -7 * np.abs(want) + 1e-4 * np.abs(want).max()).all()
+    assert delta(before, "fp8_linear") == 1 and delta(before, f"fp8_linear:{outputs},{inner}") == 1
+    assert delta(before, "fp8") == 2
+    # without the power-of-two activation-scale policy the original quantiser must run
+    assert linear(original, xt, B, [32, 32], Bs, None, None, False, None) == "original"
+    assert linear(original, xt, B, [32, 32], Bs, torch.ones(1, device=device), None, True, None) == "original"
+    assert len(original.calls) == 5 and len(original.calls[-1]) == 8
