@@ -5,8 +5,9 @@
 // unscaled FP32 dot product on the matrix cores, then acc = fma(dot_g, a_s * w_s, acc) for g
 // ascending with a_s * w_s rounded to FP32 first, one BF16 rounding at the end.
 //
-// A workgroup of 2 x WM wavefronts owns a 256 x (32*WM*TM) output tile; each wavefront owns 128
-// weight rows (exactly one 128-row scale block) by 32*TM tokens. One K step is one scale group:
+// A workgroup of 2 x WM wavefronts owns a (64*TN) x (32*WM*TM) output tile; each wavefront owns
+// 32*TN weight rows (TN = 4: exactly one 128-row scale block; TN = 3 gives 192-row tiles, whose
+// count fills the compute units better for some shapes) by 32*TM tokens. One K step is one scale group:
 // 128 bytes per row, the same LDS geometry (8 chunks of 16 bytes, XOR swizzle) as a 64-deep BF16
 // step, STAGES stages filled by buffer_load ... lds STAGES-1 groups ahead (one group of matrix
 // work is shorter than the memory latency, so two stages leave the matrix cores waiting for
@@ -33,11 +34,14 @@ struct Fp8DmaParams {
     int tiles_n, tiles_m;
 };
 
-template <int TM, int WM, int STAGES>
+template <int TM, int WM, int STAGES, int TN>
 __global__ __launch_bounds__(128 * WM) void fp8_dma_kernel(Fp8DmaParams p)
 {
     static_assert(STAGES == 2 || STAGES == 3, "two or three LDS stages");
-    constexpr int TN = 4, WAVES = 2 * WM, CH = 8, BK = 128;
+    constexpr int WAVES = 2 * WM, CH = 8, BK = 128;
+    // weight scales per wavefront and group: one when its rows are one scale block, else one per
+    // 32-row tile (a 32-row tile never straddles a 128-row block)
+    constexpr int WS = TN == 4 ? 1 : TN;
     constexpr int BN = 64 * TN, BM = 32 * WM * TM;
     constexpr int ROWS_PER_LOAD = 8;
     constexpr int A_ITERS = BN / (WAVES * ROWS_PER_LOAD), B_ITERS = BM / (WAVES * ROWS_PER_LOAD);
@@ -87,15 +91,19 @@ __global__ __launch_bounds__(128 * WM) void fp8_dma_kernel(Fp8DmaParams p)
         advance();
     };
 
-    // ---- scales. The wavefront's 128 weight rows lie in one scale block, so its weight scale is
-    // one value per group (every lane loads the same address); activation scales are one per lane
+    // ---- scales. Weight scales are one value per group and scale block of the wavefront's rows
+    // (every lane loads the same address); activation scales are one per lane
     // (token = lane % 32) and token tile. Both are loaded one group ahead, unconditionally: a load
     // under a branch would make the compiler wait for every outstanding load, the LDS fills
     // included.
     const int frag_row = lane % 32, half = lane / 32;
-    int block = (n0 + wn * 128) / 128;
-    block = block < p.scale_blocks ? block : p.scale_blocks - 1;
-    const float *ws_row = p.w_scale + size_t(block) * p.groups;
+    const float *ws_row[WS];
+#pragma unroll
+    for (int s = 0; s < WS; ++s) {
+        int block = (n0 + wn * TN * 32 + s * 32) / 128;
+        block = block < p.scale_blocks ? block : p.scale_blocks - 1;
+        ws_row[s] = p.w_scale + size_t(block) * p.groups;
+    }
     const float *as_ptr[TM];
 #pragma unroll
     for (int j = 0; j < TM; ++j) {
@@ -129,7 +137,7 @@ __global__ __launch_bounds__(128 * WM) void fp8_dma_kernel(Fp8DmaParams p)
     // then the 16 scaled accumulates of tile t-1, so that the vector ALU work and the load issue of
     // one tile run while the matrix cores execute the next (sched_barrier pins it).
     auto multiply = [&](const u32x4_t *stage, u32x4_t *fill, const float (&as_now)[TM],
-                        float ws_now) {
+                        const float (&ws_now)[WS]) {
         constexpr int TILES = TN * TM, SHARE = (LOADS + TILES - 1) / TILES;
         i32x8_t a_frag[2][2], b_frag[TM][2];
 #pragma unroll
@@ -139,10 +147,12 @@ __global__ __launch_bounds__(128 * WM) void fp8_dma_kernel(Fp8DmaParams p)
         }
         a_frag[0][0] = fragment(stage, a_frag_base, 0);
         a_frag[0][1] = fragment(stage, a_frag_base, 1);
-        float scale[TM];
+        float scale[WS][TM];
 #pragma unroll
-        for (int j = 0; j < TM; ++j)
-            scale[j] = __fmul_rn(as_now[j], ws_now);
+        for (int s = 0; s < WS; ++s)
+#pragma unroll
+            for (int j = 0; j < TM; ++j)
+                scale[s][j] = __fmul_rn(as_now[j], ws_now[s]);
         f32x16_t dot[2];
         auto product = [&](int tile, f32x16_t &d) {
             const int i = tile / TM, j = tile % TM;
@@ -158,7 +168,7 @@ __global__ __launch_bounds__(128 * WM) void fp8_dma_kernel(Fp8DmaParams p)
             const int i = tile / TM, j = tile % TM;
 #pragma unroll
             for (int r = 0; r < 16; ++r)
-                acc[i][j][r] = fmaf(d[r], scale[j], acc[i][j][r]);
+                acc[i][j][r] = fmaf(d[r], scale[WS == 1 ? 0 : i][j], acc[i][j][r]);
         };
 #pragma unroll
         for (int tile = 0; tile < TILES; ++tile) {
@@ -184,7 +194,10 @@ __global__ __launch_bounds__(128 * WM) void fp8_dma_kernel(Fp8DmaParams p)
         __builtin_amdgcn_sched_barrier(0);
     };
 
-    float ws_now = ws_row[0], ws_next;
+    float ws_now[WS], ws_next[WS];
+#pragma unroll
+    for (int s = 0; s < WS; ++s)
+        ws_now[s] = ws_row[s][0];
     float as_now[TM], as_next[TM];
 #pragma unroll
     for (int j = 0; j < TM; ++j)
@@ -193,13 +206,17 @@ __global__ __launch_bounds__(128 * WM) void fp8_dma_kernel(Fp8DmaParams p)
     // multiply the current stage, then wait until only the newest loads are still in flight.
     auto step = [&](int g, const u32x4_t *current, u32x4_t *fill) {
         const int next = g + 1 < p.groups ? g + 1 : p.groups - 1;
-        ws_next = ws_row[next];
+#pragma unroll
+        for (int s = 0; s < WS; ++s)
+            ws_next[s] = ws_row[s][next];
 #pragma unroll
         for (int j = 0; j < TM; ++j)
             as_next[j] = as_ptr[j][next];
         __builtin_amdgcn_sched_barrier(0);
         multiply(current, fill, as_now, ws_now);
-        ws_now = ws_next;
+#pragma unroll
+        for (int s = 0; s < WS; ++s)
+            ws_now[s] = ws_next[s];
 #pragma unroll
         for (int j = 0; j < TM; ++j)
             as_now[j] = as_next[j];
@@ -255,14 +272,15 @@ __global__ __launch_bounds__(128 * WM) void fp8_dma_kernel(Fp8DmaParams p)
     }
 }
 
-template <int TM, int WM, int STAGES> hipError_t launch_one(hipStream_t stream, Fp8DmaParams p)
+template <int TM, int WM, int STAGES, int TN = 4>
+hipError_t launch_one(hipStream_t stream, Fp8DmaParams p)
 {
-    constexpr int BN = 256, BM = 32 * WM * TM;
+    constexpr int BN = 64 * TN, BM = 32 * WM * TM;
     p.tiles_n = (p.n + BN - 1) / BN;
     p.tiles_m = (p.m + BM - 1) / BM;
     if (size_t(p.tiles_n) * size_t(p.tiles_m) > 0x7fffffffu)
         return hipErrorInvalidValue;
-    fp8_dma_kernel<TM, WM, STAGES>
+    fp8_dma_kernel<TM, WM, STAGES, TN>
         <<<unsigned(p.tiles_n) * unsigned(p.tiles_m), 128 * WM, 0, stream>>>(p);
     return launch_status();
 }
@@ -275,6 +293,9 @@ const TnVariant variants[] = {
     {"fp8dma256x128x128s3w8", 256, 128, 128, 512},
     {"fp8dma256x128x128s3w4", 256, 128, 128, 256},
     {"fp8dma256x64x128s3w4", 256, 64, 128, 256},
+    {"fp8dma192x128x128s3w8", 192, 128, 128, 512},
+    {"fp8dma192x256x128w8", 192, 256, 128, 512},
+    {"fp8dma192x64x128s3w4", 192, 64, 128, 256},
 };
 } // namespace
 
@@ -310,6 +331,9 @@ hipError_t launch_fp8_dma(hipStream_t stream, int variant, int rows, int outputs
     case 4: return launch_one<1, 4, 3>(stream, p);
     case 5: return launch_one<2, 2, 3>(stream, p);
     case 6: return launch_one<1, 2, 3>(stream, p);
+    case 7: return launch_one<1, 4, 3, 3>(stream, p);
+    case 8: return launch_one<2, 4, 2, 3>(stream, p);
+    case 9: return launch_one<1, 2, 3, 3>(stream, p);
     default: return hipErrorInvalidValue;
     }
 }

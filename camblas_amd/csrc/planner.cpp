@@ -202,7 +202,10 @@ Plan make_plan(int dtype, int algorithm, bool trans_a, bool trans_b, int m, int 
     const struct {
         int variant, resident;
         double weight;
-    } candidates[] = {{4, 1, 1.0}, {3, 1, 0.9}};
+    } candidates[] = {{0, 1, 1.04}, {8, 1, 1.02}, {4, 1, 1.0}, {7, 1, 0.92}, {6, 1, 0.75}, {9, 1, 0.64}};
+    // {256, 192} x {256, 128, 64} tiles, one workgroup per compute unit. What decides between them
+    // is how full the last round of workgroups is (18432 outputs are 72 tiles of 256 rows or 96 of
+    // 192); the weights are the measured per-flop efficiency of each tile at equal occupancy.
     double best = -1;
     for (const auto &candidate : candidates) {
         const TnVariant &v = fp8_dma_variant(candidate.variant);
