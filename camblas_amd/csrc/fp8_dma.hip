@@ -37,6 +37,7 @@ struct Fp8DmaParams {
 template <int TM, int WM, int STAGES, int TN>
 __global__ __launch_bounds__(128 * WM) void fp8_dma_kernel(Fp8DmaParams p)
 {
+    // (a fourth stage was measured: no gain, the kernel is not limited by bytes in flight)
     static_assert(STAGES == 2 || STAGES == 3, "two or three LDS stages");
     constexpr int WAVES = 2 * WM, CH = 8, BK = 128;
     // weight scales per wavefront and group: one when its rows are one scale block, else one per
@@ -47,9 +48,7 @@ __global__ __launch_bounds__(128 * WM) void fp8_dma_kernel(Fp8DmaParams p)
     constexpr int A_ITERS = BN / (WAVES * ROWS_PER_LOAD), B_ITERS = BM / (WAVES * ROWS_PER_LOAD);
     constexpr int SLOTS = (BN + BM) * CH, LOADS = A_ITERS + B_ITERS;
     static_assert(BN % (WAVES * ROWS_PER_LOAD) == 0 && BM % (WAVES * ROWS_PER_LOAD) == 0, "loads");
-    __shared__ u32x4_t stage0[SLOTS];
-    __shared__ u32x4_t stage1[SLOTS];
-    __shared__ u32x4_t stage2[STAGES > 2 ? SLOTS : 1];
+    __shared__ u32x4_t stages[STAGES][SLOTS];
 
     int tile_n, tile_m;
     xcd_tile(int(blockIdx.x), p.tiles_n, p.tiles_m, tile_n, tile_m);
@@ -222,33 +221,25 @@ __global__ __launch_bounds__(128 * WM) void fp8_dma_kernel(Fp8DmaParams p)
             as_now[j] = as_next[j];
         pipeline_barrier<(STAGES - 2) * LOADS>();
     };
-    issue(stage0);
-    if constexpr (STAGES == 3) {
+    // Group g is read from stage g % STAGES while group g + STAGES - 1 is loaded into the stage
+    // that was read last.
+#pragma unroll
+    for (int s = 0; s + 1 < STAGES; ++s) {
         __builtin_amdgcn_sched_barrier(0);
-        issue(stage1);
+        issue(stages[s]);
     }
     pipeline_barrier<(STAGES - 2) * LOADS>();
     // whole rounds of STAGES groups run without a branch between the steps; the remainder follows
     int g = 0;
-    if constexpr (STAGES == 2) {
-        for (; g + 2 <= p.groups; g += 2) {
-            step(g, stage0, stage1);
-            step(g + 1, stage1, stage0);
-        }
-        if (g < p.groups)
-            step(g, stage0, stage1);
-    } else {
-        for (; g + 3 <= p.groups; g += 3) {
-            step(g, stage0, stage2);
-            step(g + 1, stage1, stage0);
-            step(g + 2, stage2, stage1);
-        }
-        if (g < p.groups) {
-            step(g, stage0, stage2);
-            if (g + 1 < p.groups)
-                step(g + 1, stage1, stage0);
-        }
+    for (; g + STAGES <= p.groups; g += STAGES) {
+#pragma unroll
+        for (int s = 0; s < STAGES; ++s)
+            step(g + s, stages[s], stages[(s + STAGES - 1) % STAGES]);
     }
+#pragma unroll
+    for (int s = 0; s + 1 < STAGES; ++s)
+        if (g + s < p.groups)
+            step(g + s, stages[s], stages[(s + STAGES - 1) % STAGES]);
     wait_loads<0>();
 
     // ---- epilogue: accumulator register 4q+e of lane l is feature 8q + 4*(l/32) + e, token l%32

@@ -78,7 +78,7 @@ def test_streaming_decode_variants(device, code, rows, outputs, inner):
     assert (np.abs(bf16_values(out) - wanted) <= bound).all()
 
 
-@pytest.mark.parametrize("code", [20, 21, 22, 23, 24, 25, 26, 27, 28, 29])
+@pytest.mark.parametrize("code", list(range(20, 30)))
 @pytest.mark.parametrize("rows,outputs,inner", [(70, 300, 512), (256, 512, 128), (513, 260, 896)])
 def test_direct_lds_load_variants(device, code, rows, outputs, inner):
     # partial tiles in both directions, a partial last weight-scale block, odd and even numbers of
