@@ -33,7 +33,7 @@ CORE_SOURCES = (
     "fp8_stream.hip",
     "fp8_block32.hip",
     "mx_matmul.hip",
-    "routing.hip", "dense_ops.hip",
+    "routing.hip", "dense_ops.hip", "sgemm_mfma.hip",
     "fusion.hip",
     "attention_decode.hip",
 )

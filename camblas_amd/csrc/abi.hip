@@ -207,8 +207,16 @@ int dense_gemm(camblas_cuda_context *context, char ta, char tb, int m, int n, in
                 error = launch_gemv_f32(context->stream, m, k, alpha, a, lda, b, beta, c);
                 return error == hipSuccess ? 0 : fail(context, "FP32 native GEMV", error);
             }
-            error = launch_generic_f32(context->stream, trans_a, trans_b, m, n, k, alpha, a, lda, b,
-                                       ldb, beta, c, ldc);
+            if (context->override_kernel >= 0) { // diagnostics: 0 vector-ALU tiles, 1 / 2 matrix-core tiles
+                plan.family = context->override_kernel >= 1 ? FAMILY_MFMA_F32 : FAMILY_GENERIC;
+                plan.kernel = context->override_kernel == 2 ? 1 : 0;
+            }
+            if (plan.family == FAMILY_MFMA_F32)
+                error = launch_sgemm_mfma(context->stream, plan.kernel == 0, trans_a, trans_b, m, n, k,
+                                          alpha, a, lda, b, ldb, beta, c, ldc);
+            else
+                error = launch_generic_f32(context->stream, trans_a, trans_b, m, n, k, alpha, a, lda,
+                                           b, ldb, beta, c, ldc);
             return error == hipSuccess ? 0 : fail(context, "classical GEMM", error);
         });
 }

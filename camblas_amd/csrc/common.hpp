@@ -48,7 +48,8 @@ enum KernelFamily {
     FAMILY_STREAM = 4, // BF16 'T','N' with few tokens: weight-streaming kernel, one pass over W
     FAMILY_DMA = 5,    // BF16 'T','N' prefill: large MFMA tiles fed by direct global->LDS loads
     FAMILY_FP8_DMA = 6, // FP8 block-scaled prefill: the same structure with one scale group per step
-    FAMILY_FP8_STREAM = 7 // FP8 block-scaled decode: weight-streaming kernel (10*row_tiles + token_tiles)
+    FAMILY_FP8_STREAM = 7, // FP8 block-scaled decode: weight-streaming kernel (10*row_tiles + token_tiles)
+    FAMILY_MFMA_F32 = 8    // FP32, any layout: 128 x 128 tiles on the FP32 matrix-core instruction
 };
 
 struct Plan {
@@ -84,6 +85,10 @@ hipError_t launch_scale_f64(hipStream_t stream, int m, int n, double beta, doubl
 hipError_t launch_generic_f32(hipStream_t stream, bool ta, bool tb, int m, int n, int k, float alpha,
                               const float *a, int lda, const float *b, int ldb, float beta, float *c,
                               int ldc);
+// wide: 128 x 128 output tiles per workgroup, else 128 x 64
+hipError_t launch_sgemm_mfma(hipStream_t stream, bool wide, bool ta, bool tb, int m, int n, int k,
+                             float alpha, const float *a, int lda, const float *b, int ldb, float beta,
+                             float *c, int ldc);
 hipError_t launch_generic_bf16(hipStream_t stream, bool ta, bool tb, int m, int n, int k,
                                float alpha, const void *a, int lda, const void *b, int ldb,
                                float beta, void *c, int ldc);

@@ -20,20 +20,29 @@ pytestmark = pytest.mark.gpu
 TOLERANCE = 1e-5
 
 
-def run_sgemm(device, ta, tb, m, n, k, alpha, a, lda, b, ldb, beta, c, ldc, algorithm="auto"):
+KERNEL = {"planner": -1, "vector": 0, "matrix": 1, "matrix64": 2}  # FP32 kernels (forced for the test)
+
+
+def run_sgemm(device, ta, tb, m, n, k, alpha, a, lda, b, ldb, beta, c, ldc, algorithm="auto",
+              kernel="planner"):
     at, bt, ct_ = (torch.from_numpy(v).to(device) for v in (a, b, c))
     with _native.algorithm(algorithm):
         native = _native.context(device)
-        native.call("sgemm", ta.encode(), tb.encode(), m, n, k, ct.c_float(alpha), ptr(at), lda,
-                    ptr(bt), ldb, ct.c_float(beta), ptr(ct_), ldc)
+        native.call("hip_set_plan_override", KERNEL[kernel], 0)
+        try:
+            native.call("sgemm", ta.encode(), tb.encode(), m, n, k, ct.c_float(alpha), ptr(at), lda,
+                        ptr(bt), ldb, ct.c_float(beta), ptr(ct_), ldc)
+        finally:
+            native.call("hip_set_plan_override", -1, 0)
     torch.cuda.synchronize()
     return ct_.cpu().numpy()
 
 
+@pytest.mark.parametrize("kernel", ["vector", "matrix", "matrix64"])
 @pytest.mark.parametrize("ta", "NT")
 @pytest.mark.parametrize("tb", "NT")
-@pytest.mark.parametrize("shape", [(37, 29, 53), (128, 96, 200), (65, 130, 17)])
-def test_sgemm_padded_alpha_beta(device, ta, tb, shape):
+@pytest.mark.parametrize("shape", [(37, 29, 53), (128, 96, 200), (65, 130, 17), (259, 140, 33)])
+def test_sgemm_padded_alpha_beta(device, kernel, ta, tb, shape):
     m, n, k = shape
     lda = (m if ta == "N" else k) + 3
     ldb = (k if tb == "N" else n) + 2
@@ -41,7 +50,7 @@ def test_sgemm_padded_alpha_beta(device, ta, tb, shape):
     a = oracle.fill_uniform(1, (lda * (k if ta == "N" else m),))
     b = oracle.fill_uniform(2, (ldb * (n if tb == "N" else k),))
     c0 = oracle.fill_uniform(3, (ldc * n,))
-    got = run_sgemm(device, ta, tb, m, n, k, 1.25, a, lda, b, ldb, -0.5, c0.copy(), ldc)
+    got = run_sgemm(device, ta, tb, m, n, k, 1.25, a, lda, b, ldb, -0.5, c0.copy(), ldc, kernel=kernel)
     want = c0.copy()
     want64 = oracle.sgemm_f64(ta, tb, m, n, k, 1.25, a, lda, b, ldb, -0.5, want, ldc, want64=True)
     got2d, c2d = got.reshape(n, ldc), c0.reshape(n, ldc)
@@ -57,11 +66,12 @@ def test_sgemm_beta_zero_ignores_nan_and_alpha_zero(device):
     m, n, k = 70, 33, 40
     a = oracle.fill_uniform(4, (m * k,))
     b = oracle.fill_uniform(5, (k * n,))
-    c = np.full(m * n, np.nan, dtype=np.float32)
-    got = run_sgemm(device, "N", "N", m, n, k, 1.0, a, m, b, k, 0.0, c, m)
     want = np.zeros(m * n, np.float32)
     want64 = oracle.sgemm_f64("N", "N", m, n, k, 1.0, a, m, b, k, 0.0, want, m, want64=True)
-    assert np.isfinite(got).all() and rel_frobenius(got, want64) <= TOLERANCE
+    for kernel in ("vector", "matrix", "matrix64"):
+        c = np.full(m * n, np.nan, dtype=np.float32)
+        got = run_sgemm(device, "N", "N", m, n, k, 1.0, a, m, b, k, 0.0, c, m, kernel=kernel)
+        assert np.isfinite(got).all() and rel_frobenius(got, want64) <= TOLERANCE
     # alpha == 0: beta scaling only; beta == 0 writes zeros over NaN; beta == 1 leaves C alone
     c = np.full(m * n, np.nan, dtype=np.float32)
     assert not run_sgemm(device, "N", "N", m, n, k, 0.0, a, m, b, k, 0.0, c, m).any()
@@ -72,7 +82,8 @@ def test_sgemm_beta_zero_ignores_nan_and_alpha_zero(device):
     )
 
 
-def test_sgemm_full_precision_not_reduced(device):
+@pytest.mark.parametrize("kernel", ["vector", "matrix", "matrix64"])
+def test_sgemm_full_precision_not_reduced(device, kernel):
     # (1 + 2^-12)^2 needs more than a 10-bit mantissa: a reduced-precision matrix path would
     # return exactly 1 (ref: tests/test_cuda.py:245-270)
     m = n = k = 64
@@ -81,8 +92,16 @@ def test_sgemm_full_precision_not_reduced(device):
     a[np.arange(m), np.arange(m)] = value
     b = a.copy()
     got = run_sgemm(device, "N", "N", m, n, k, 1.0, a.ravel(), m, b.ravel(), k, 0.0,
-                    np.zeros(m * n, np.float32), m).reshape(n, m)
+                    np.zeros(m * n, np.float32), m, kernel=kernel).reshape(n, m)
     assert got[5, 5] == np.float32(value * value)
+    # and a sum that needs all 24 bits: 2^12 + 1 + 2^-11 terms in one dot product
+    a = np.zeros((m, k), np.float32)
+    b = np.zeros((k, n), np.float32)
+    a[3, :3] = (4096.0, 1.0, 1.0)
+    b[:3, 7] = (1.0, 1.0, 2.0**-11)
+    got = run_sgemm(device, "T", "T", m, n, k, 1.0, a.ravel(), k, b.ravel(), n, 0.0,
+                    np.zeros(m * n, np.float32), m, kernel=kernel).reshape(n, m)
+    assert got[7, 3] == np.float32(4097.0 + 2.0**-11)
 
 
 def test_sgemm_config1_row_major_2048(device):
