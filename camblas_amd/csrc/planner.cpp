@@ -237,7 +237,7 @@ void describe_plan(const Plan &plan, int dtype, char *text, size_t bytes)
         std::snprintf(text, bytes, "%s gemv wave-per-row", type);
         break;
     case FAMILY_MFMA_F32:
-        std::snprintf(text, bytes, "%s mfma %s", type, plan.kernel == 0 ? "128x128x16" : "128x64x16");
+        std::snprintf(text, bytes, "%s mfma %s", type, plan.kernel == 0 ? "128x128x32" : "128x64x32");
         break;
     case FAMILY_MFMA_TN:
         std::snprintf(text, bytes, "%s %s split_k=%d", type, tn_variant(plan.kernel).name,

@@ -4,11 +4,11 @@
 // Contract: ref src/cuda/backend.cu:786-866 (validation is done by the caller in abi.hip).
 //
 // A workgroup of four wavefronts owns a 128 x 128 tile of C, a wavefront 64 x 64 of it as 2 x 2
-// MFMA tiles (64 accumulator registers). K is walked 16 deep: the operands of a step are loaded
+// MFMA tiles (64 accumulator registers). K is walked 32 deep: the operands of a step are loaded
 // element-wise with bounds checks (that is what makes every layout and ragged edge work), kept in
 // registers while the previous step is multiplied, and laid out in LDS so that the operand reads
-// (lane -> row lane%32, K index lane/32) are conflict-free: K-major [16][128+32] for an operand
-// whose rows are contiguous in memory, row-major [128][17] for a transposed one.
+// (lane -> row lane%32, K index lane/32) are conflict-free: K-major [32][128+32] for an operand
+// whose rows are contiguous in memory, row-major [128][33] for a transposed one.
 #include "common.hpp"
 #include "device.hpp"
 
@@ -16,7 +16,7 @@ namespace camblas_hip
 {
 namespace
 {
-constexpr int TILE = 128, DEPTH = 16, THREADS = 256;
+constexpr int TILE = 128, DEPTH = 32, THREADS = 256;
 constexpr int K_MAJOR_PITCH = TILE + 32, ROW_MAJOR_PITCH = DEPTH + 1;
 constexpr int TILE_WORDS = DEPTH * K_MAJOR_PITCH; // >= TILE * ROW_MAJOR_PITCH
 static_assert(TILE * ROW_MAJOR_PITCH <= TILE_WORDS, "one buffer serves both layouts");

@@ -78,8 +78,8 @@ def test_planner_choices_for_the_baseline_shapes():
     assert describe(0, "T", "N", 4096, 1, 4096, 4096, 4096, 4096, algorithm="lt")[0] // 1000 == 0
     assert describe(0, "T", "N", 1000, 1, 4096, 4096, 4096, 1000)[0] // 1000 == 0
     # FP32 products: matrix-core tiles, 128 x 64 until every compute unit gets two 128 x 128 tiles
-    assert describe(0, "N", "N", 2048, 2048, 2048, 2048, 2048, 2048) == (8001, "f32 mfma 128x64x16")
-    assert describe(0, "T", "N", 4096, 4096, 4096, 4096, 4096, 4096) == (8000, "f32 mfma 128x128x16")
+    assert describe(0, "N", "N", 2048, 2048, 2048, 2048, 2048, 2048) == (8001, "f32 mfma 128x64x32")
+    assert describe(0, "T", "N", 4096, 4096, 4096, 4096, 4096, 4096) == (8000, "f32 mfma 128x128x32")
     assert describe(0, "N", "N", 2048, 16, 2048, 2048, 2048, 2048)[0] // 1000 == 0
     # FP8: split-K tiles for a few tokens, the streaming kernel for decode batches, direct-to-LDS
     # tiles for prefill
