@@ -134,11 +134,18 @@ Plan make_plan(int dtype, int algorithm, bool trans_a, bool trans_b, int m, int 
             plan.kernel = 100 * stream_depth_log2(row_tiles, token_tiles, k) + 10 * row_tiles +
                           token_tiles;
             plan.split_k = 1;
-        } else if (tokens <= 96) {
-            plan.kernel = 3; // 128 x 64 x 64
-            const TnVariant &v = tn_variant(plan.kernel);
-            plan.split_k =
-                decode_split(ceil_div(outputs, v.block_n), ceil_div(k, v.block_k), compute_units);
+        } else if (ceil_div(outputs, 128) * ceil_div(tokens, 128) * 2 <= compute_units) {
+            // few output tiles (a narrow projection, a small batch): 128 x 128 register-staged
+            // tiles with K divided over workgroups, the largest power-of-two split that keeps the
+            // grid within two workgroups per compute unit and at least 512 of K per partition
+            // (measured against the direct-to-LDS tiles: [8192, 28672] x 128 tokens 120 vs 314 us,
+            // x 256 tokens 181 vs 313 us; [8192, 8192] x 128 tokens 42 vs 71 us)
+            plan.kernel = 2;
+            const int tiles = ceil_div(outputs, 128) * ceil_div(tokens, 128);
+            plan.split_k = 1;
+            while (plan.split_k < 16 && tiles * plan.split_k * 2 <= 2 * compute_units &&
+                   k / (plan.split_k * 2) >= 512)
+                plan.split_k *= 2;
         } else {
             // prefill: larger tiles reuse more per byte; prefer them unless a smaller tile fills
             // the compute units noticeably better
@@ -150,7 +157,7 @@ Plan make_plan(int dtype, int algorithm, bool trans_a, bool trans_b, int m, int 
                 const struct {
                     int variant, resident;
                     double weight;
-                } candidates[] = {{10, 1, 1.0}, {6, 1, 0.93}, {11, 1, 0.88}, {9, 1, 0.85}, {2, 2, 0.8}};
+                } candidates[] = {{10, 1, 1.0}, {6, 1, 0.93}, {11, 1, 0.88}, {9, 1, 0.85}, {5, 1, 0.8}};
                 plan.family = FAMILY_DMA;
                 for (const auto &candidate : candidates) {
                     const TnVariant &v = dma_variant(candidate.variant);
