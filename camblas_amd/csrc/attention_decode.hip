@@ -191,17 +191,43 @@ __global__ __launch_bounds__(DIM) void gqa_combine_kernel(int splits, const floa
 {
     const size_t row = blockIdx.x; // b * q_heads + head
     const int d = threadIdx.x;
+    // Partitions are taken eight at a time with all loads of a batch issued before any is used
+    // (a loop of dependent scalar loads would pay the memory latency once per partition); indices
+    // past the end are clamped and masked. The order of the sums is the partition order.
+    constexpr int BATCH = 8;
+    const float *row_m = part_m + row * splits, *row_l = part_l + row * splits;
+    const float *row_o = part_o + row * splits * DIM + d;
     float top = -INFINITY;
-    for (int s = 0; s < splits; ++s)
-        if (part_l[row * splits + s] > 0.f)
-            top = fmaxf(top, part_m[row * splits + s]);
+    for (int s0 = 0; s0 < splits; s0 += BATCH) {
+        float l[BATCH], m[BATCH];
+#pragma unroll
+        for (int i = 0; i < BATCH; ++i) {
+            const int s = s0 + i < splits ? s0 + i : splits - 1;
+            l[i] = row_l[s];
+            m[i] = row_m[s];
+        }
+#pragma unroll
+        for (int i = 0; i < BATCH; ++i)
+            if (s0 + i < splits && l[i] > 0.f)
+                top = fmaxf(top, m[i]);
+    }
     float numerator = 0.f, denominator = 0.f;
-    for (int s = 0; s < splits; ++s) {
-        float l = part_l[row * splits + s];
-        if (l > 0.f) {
-            float factor = __expf(part_m[row * splits + s] - top);
-            numerator = fmaf(factor, part_o[(row * splits + s) * DIM + d], numerator);
-            denominator = fmaf(factor, l, denominator);
+    for (int s0 = 0; s0 < splits; s0 += BATCH) {
+        float l[BATCH], m[BATCH], o[BATCH];
+#pragma unroll
+        for (int i = 0; i < BATCH; ++i) {
+            const int s = s0 + i < splits ? s0 + i : splits - 1;
+            l[i] = row_l[s];
+            m[i] = row_m[s];
+            o[i] = row_o[size_t(s) * DIM];
+        }
+#pragma unroll
+        for (int i = 0; i < BATCH; ++i) {
+            if (s0 + i < splits && l[i] > 0.f) {
+                const float factor = __expf(m[i] - top);
+                numerator = fmaf(factor, o[i], numerator);
+                denominator = fmaf(factor, l[i], denominator);
+            }
         }
     }
     out[row * DIM + d] = float_to_bf16_bits(denominator > 0.f ? numerator / denominator : 0.f);
