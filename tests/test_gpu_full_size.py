@@ -1,0 +1,146 @@
+"""The headline configurations at their full sizes, checked through properties that do not need a
+full-size CPU product: sampled outputs against the oracle's FP64 accumulation (the sample covers
+the first and last rows, tile seams and random positions), exact power-of-two scaling, token
+permutation, independence of a token's result from its neighbours, zero and NaN propagation.
+
+Shapes: BF16 decode x [M in {1, 8, 32}, 8192] . W [28672, 8192]^T; BF16 prefill x [4096, 8192] .
+W [10240, 8192]^T with and without beta = 1; FP8 block-scaled A [M in {1, 16, 256, 4096}, 7168] .
+W [18432, 7168]^T with 1x128 / 128x128 FP32 scales. Tolerances are the small-size tests': relative
+Frobenius error <= 1e-2 against FP64 accumulation, and an element-wise bound of one BF16 rounding
+plus 1e-4 of the largest output.
+"""
+
+import numpy as np
+import pytest
+import torch
+
+import oracle
+from camblas_amd import _kernels
+from helpers import bf16_values, from_device_bf16, from_device_fp8, rel_frobenius
+
+pytestmark = pytest.mark.gpu
+TOLERANCE = 1e-2
+
+
+def sample(count, size, seed, seams=()):
+    """Sorted sample of indices below `size`: both ends, the seams given, and random ones."""
+    rng = np.random.default_rng(seed)
+    fixed = [0, 1, size - 2, size - 1] + [s + d for s in seams for d in (-1, 0) if 0 < s + d < size]
+    picked = set(int(i) for i in fixed if 0 <= i < size)
+    while len(picked) < min(count, size):
+        picked.add(int(rng.integers(0, size)))
+    return np.array(sorted(picked))
+
+
+def close_to(got, want64):
+    assert rel_frobenius(got, want64) <= TOLERANCE
+    wanted = oracle.bf16_to_f32(oracle.f32_to_bf16(want64.astype(np.float32)))
+    bound = 2.0 ** -7 * np.abs(wanted) + 1e-4 * np.abs(want64).max()
+    assert (np.abs(got - wanted) <= bound).all()
+
+
+def bf16_normal(shape, std, seed, device):
+    generator = torch.Generator(device=device).manual_seed(seed)
+    return (torch.randn(shape, generator=generator, device=device) * std).bfloat16()
+
+
+@pytest.fixture(scope="module")
+def up_projection(device):
+    return bf16_normal((28672, 8192), 0.02, 9001, device)
+
+
+@pytest.mark.parametrize("tokens", [1, 8, 32])
+def test_bf16_decode_linear_28672x8192(device, up_projection, tokens):
+    w = up_projection
+    x = bf16_normal((tokens, 8192), 1.0, 9002 + tokens, device)
+    y = _kernels.linear(x, w)
+    assert y.shape == (tokens, 28672) and y.dtype == torch.bfloat16
+    # sampled output features (rows of W): the workgroup seams at multiples of 112 rows included
+    rows = sample(96, 28672, 1, seams=(112, 224, 28560, 14336))
+    want = oracle.linear_bf16_f64(from_device_bf16(x), from_device_bf16(w[torch.from_numpy(rows).to(device)]))
+    close_to(bf16_values(y)[:, rows], want)
+    # scaling the input by a power of two scales every output exactly
+    assert torch.equal(_kernels.linear(x * 4, w), y * 4)
+    # a token's result depends on that token only: reversed batch, and the token alone
+    if tokens > 1:
+        assert torch.equal(_kernels.linear(x.flip(0).contiguous(), w), y.flip(0))
+        alone = _kernels.linear(x[tokens - 1:].contiguous(), w)
+        assert rel_frobenius(bf16_values(alone), bf16_values(y[tokens - 1:]).astype(np.float64)) <= 1e-2
+    # zero input gives +0 everywhere; a NaN in one token poisons exactly that token
+    assert not _kernels.linear(torch.zeros_like(x), w).view(torch.int16).any()
+    poisoned = x.clone()
+    poisoned[tokens - 1, 4097] = float("nan")
+    out = _kernels.linear(poisoned, w)
+    assert torch.isnan(out[tokens - 1]).all() and torch.equal(out[: tokens - 1], y[: tokens - 1])
+
+
+def test_bf16_prefill_linear_4096x10240x8192(device):
+    w = bf16_normal((10240, 8192), 0.02, 9101, device)
+    x = bf16_normal((4096, 8192), 1.0, 9102, device)
+    y = _kernels.linear(x, w)
+    # sampled tokens against FP64, all 10240 features each (tile seams at 256 tokens / 320 rows)
+    tokens = sample(12, 4096, 2, seams=(256, 2048, 3840))
+    index = torch.from_numpy(tokens).to(device)
+    want = oracle.linear_bf16_f64(from_device_bf16(x[index]), from_device_bf16(w))
+    close_to(bf16_values(y[index]), want)
+    assert torch.equal(_kernels.linear(x * 0.5, w), y * 0.5)
+    # addmm with beta = 1 on a full-size C ~ N(0, 1): sampled tokens again
+    c = bf16_normal((4096, 10240), 1.0, 9103, device)
+    out = _kernels.matmul(x, w.t(), out=c.clone(), alpha=1.0, beta=1.0)
+    want = want + bf16_values(c[index]).astype(np.float64)
+    close_to(bf16_values(out[index]), want)
+    # the same tokens as a small batch through the decode kernel agree to rounding
+    small = _kernels.linear(x[index[:8]].contiguous(), w)
+    assert rel_frobenius(bf16_values(small), bf16_values(y[index[:8]]).astype(np.float64)) <= 1e-2
+
+
+@pytest.fixture(scope="module")
+def fp8_weights(device):
+    generator = torch.Generator(device=device).manual_seed(9201)
+    # every byte pattern except the two NaN encodings
+    w = torch.randint(0, 255, (18432, 7168), generator=generator, device=device, dtype=torch.uint8)
+    w[w == 0x7F] = 0x7E
+    scale = torch.exp(torch.empty((144, 56), device=device).uniform_(np.log(1e-4), np.log(1e-1), generator=generator))
+    return w.view(torch.float8_e4m3fn), scale
+
+
+@pytest.mark.parametrize("tokens", [1, 16, 256, 4096])
+def test_fp8_block_linear_18432x7168(device, fp8_weights, tokens):
+    w, w_scale = fp8_weights
+    generator = torch.Generator(device=device).manual_seed(9300 + tokens)
+    a = torch.randint(0, 255, (tokens, 7168), generator=generator, device=device, dtype=torch.uint8)
+    a[a == 0x7F] = 0x7E
+    a = a.view(torch.float8_e4m3fn)
+    a_scale = torch.exp(torch.empty((tokens, 56), device=device).uniform_(np.log(1e-4), np.log(1e-1), generator=generator))
+    out = _kernels.fp8_block_matmul(a, a_scale, w, w_scale)
+    assert out.shape == (tokens, 18432) and out.dtype == torch.bfloat16
+    # sampled tokens (all features) against the FP64 product of the dequantised operands
+    picked = sample(4, tokens, 3, seams=(128, 256))
+    index = torch.from_numpy(picked).to(device)
+    want = oracle.fp8_block_matmul_f64(from_device_fp8(a[index]), a_scale[index].cpu().numpy(),
+                                       from_device_fp8(w), w_scale.cpu().numpy())
+    close_to(bf16_values(out[index]), want)
+    # doubling every weight scale doubles every output exactly; so does doubling a token's scales
+    assert torch.equal(_kernels.fp8_block_matmul(a, a_scale, w, w_scale * 2), out * 2)
+    assert torch.equal(_kernels.fp8_block_matmul(a, a_scale * 0.5, w, w_scale), out * 0.5)
+    # bit-exact block indexing: zeroing one 128 x 128 weight-scale block changes exactly the 128
+    # features of that block row (and only through K group 17)
+    masked = w_scale.clone()
+    masked[77, 17] = 0
+    changed = _kernels.fp8_block_matmul(a, a_scale, w, masked)
+    differs = (changed.view(torch.int16) != out.view(torch.int16)).any(0).cpu().numpy()
+    assert not differs[: 77 * 128].any() and not differs[78 * 128:].any() and differs[77 * 128: 78 * 128].any()
+    # ... and zeroing one token's scale of group 17 changes exactly that token
+    masked = a_scale.clone()
+    masked[picked[-1], 17] = 0
+    changed = _kernels.fp8_block_matmul(a, masked, w, w_scale)
+    differs = (changed.view(torch.int16) != out.view(torch.int16)).any(1).cpu().numpy()
+    assert differs[picked[-1]] and differs.sum() == 1
+    # zero activations give +0; a NaN byte poisons exactly its token
+    zero = torch.zeros_like(a.view(torch.uint8)).view(torch.float8_e4m3fn)
+    assert not _kernels.fp8_block_matmul(zero, a_scale, w, w_scale).view(torch.int16).any()
+    poisoned = a.view(torch.uint8).clone()
+    poisoned[tokens - 1, 5000] = 0x7F
+    result = _kernels.fp8_block_matmul(poisoned.view(torch.float8_e4m3fn), a_scale, w, w_scale)
+    assert torch.isnan(result[tokens - 1]).all()
+    assert torch.equal(result[: tokens - 1].view(torch.int16), out[: tokens - 1].view(torch.int16))
