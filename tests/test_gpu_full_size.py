@@ -3,6 +3,9 @@ full-size CPU product: sampled outputs against the oracle's FP64 accumulation (t
 the first and last rows, tile seams and random positions), exact power-of-two scaling, token
 permutation, independence of a token's result from its neighbours, zero and NaN propagation.
 
+Also the decoder-layer decode step at its full size (batch 32, hidden 8192, 64 query / 8 KV heads of
+128, FFN 28672, context 2048) against the whole oracle pipeline.
+
 Shapes: BF16 decode x [M in {1, 8, 32}, 8192] . W [28672, 8192]^T; BF16 prefill x [4096, 8192] .
 W [10240, 8192]^T with and without beta = 1; FP8 block-scaled A [M in {1, 16, 256, 4096}, 7168] .
 W [18432, 7168]^T with 1x128 / 128x128 FP32 scales. Tolerances are the small-size tests': relative
@@ -144,3 +147,43 @@ def test_fp8_block_linear_18432x7168(device, fp8_weights, tokens):
     result = _kernels.fp8_block_matmul(poisoned.view(torch.float8_e4m3fn), a_scale, w, w_scale)
     assert torch.isnan(result[tokens - 1]).all()
     assert torch.equal(result[: tokens - 1].view(torch.int16), out[: tokens - 1].view(torch.int16))
+
+
+def test_decoder_layer_decode_llama70b_shape(device):
+    # the oracle pipeline of the reduced-size layer test, at the size the benchmark runs
+    from test_gpu_layer import device_layer, oracle_layer
+
+    batch, hidden_size, q_heads, kv_heads, dim, ffn, context = 32, 8192, 64, 8, 128, 28672, 2048
+
+    def bits(shape, std, seed, mean=0.0):
+        generator = torch.Generator(device=device).manual_seed(seed)
+        values = torch.randn(shape, generator=generator, device=device) * std + mean
+        return from_device_bf16(values.bfloat16())
+
+    weights = {
+        "input_norm": bits((hidden_size,), 0.02, 9401, 1.0),
+        "post_norm": bits((hidden_size,), 0.02, 9402, 1.0),
+        "qkv": bits(((q_heads + 2 * kv_heads) * dim, hidden_size), 0.02, 9403),
+        "o": bits((hidden_size, q_heads * dim), 0.02, 9404),
+        "gate": bits((ffn, hidden_size), 0.02, 9405),
+        "up": bits((ffn, hidden_size), 0.02, 9406),
+        "down": bits((hidden_size, ffn), 0.02, 9407),
+    }
+    hidden, residual = bits((batch, hidden_size), 1.0, 9408), bits((batch, hidden_size), 1.0, 9409)
+    k_cache = bits((batch, context, kv_heads, dim), 1.0, 9410)
+    v_cache = bits((batch, context, kv_heads, dim), 1.0, 9411)
+    # the benchmark's last slot for most sequences, shorter histories for a few
+    positions = np.full(batch, context - 1, np.int32)
+    positions[:4] = (0, 255, 256, 1000)
+    inputs = (weights, hidden, residual, k_cache, v_cache, positions)
+    want_out, want_res, want_k, want_v = oracle_layer(*inputs)
+    out, res, kc, vc = device_layer(device, *inputs)
+    assert rel_frobenius(bf16_values(res), oracle.bf16_to_f32(want_res)) <= 1e-2
+    assert rel_frobenius(bf16_values(out), oracle.bf16_to_f32(want_out)) <= 2e-2
+    untouched = np.ones((batch, context), bool)
+    untouched[np.arange(batch), positions] = False
+    assert np.array_equal(from_device_bf16(kc)[untouched], k_cache[untouched])
+    assert np.array_equal(from_device_bf16(vc)[untouched], v_cache[untouched])
+    appended = (np.arange(batch), positions)
+    assert rel_frobenius(bf16_values(kc)[appended], oracle.bf16_to_f32(want_k)[appended]) <= 1e-2
+    assert rel_frobenius(bf16_values(vc)[appended], oracle.bf16_to_f32(want_v)[appended]) <= 1e-2

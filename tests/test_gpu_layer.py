@@ -44,6 +44,10 @@ def make_inputs(seed):
 
 
 def oracle_layer(weights, hidden, residual, k_cache, v_cache, positions):
+    # sizes come from the operands, so the same pipeline serves the full-size configuration
+    BATCH, HIDDEN = hidden.shape
+    KV_HEADS, DIM = k_cache.shape[2:]
+    Q_HEADS = weights["qkv"].shape[0] // DIM - 2 * KV_HEADS
     k_cache, v_cache = k_cache.copy(), v_cache.copy()
     residual, normed = oracle.rms_norm(2, 2, 1e-5, hidden, weights["input_norm"], residual=residual)
     qkv = bf16_linear(normed, weights["qkv"]).reshape(BATCH, Q_HEADS + 2 * KV_HEADS, DIM)
@@ -60,6 +64,8 @@ def oracle_layer(weights, hidden, residual, k_cache, v_cache, positions):
 
 
 def device_layer(device, weights, hidden, residual, k_cache, v_cache, positions):
+    KV_HEADS, DIM = k_cache.shape[2:]
+    Q_HEADS = weights["qkv"].shape[0] // DIM - 2 * KV_HEADS
     w = {name: to_device_bf16(value, device) for name, value in weights.items()}
     kc, vc = to_device_bf16(k_cache, device), to_device_bf16(v_cache, device)
     pos = torch.from_numpy(positions).to(device)
