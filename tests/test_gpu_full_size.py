@@ -187,3 +187,36 @@ def test_decoder_layer_decode_llama70b_shape(device):
     appended = (np.arange(batch), positions)
     assert rel_frobenius(bf16_values(kc)[appended], oracle.bf16_to_f32(want_k)[appended]) <= 1e-2
     assert rel_frobenius(bf16_values(vc)[appended], oracle.bf16_to_f32(want_v)[appended]) <= 1e-2
+
+
+@pytest.mark.parametrize("packed", [False, True])
+def test_e8m0_product_18432x7168(device, packed):
+    # the benchmarked microscaling shape: 16 tokens, weights [18432, 7168] E4M3 (scales per 32 x 32
+    # block) or packed E2M1 (scales per row and 32 inputs); sampled 32-row blocks against FP64
+    outputs, inner, tokens = 18432, 7168, 16
+    generator = torch.Generator(device=device).manual_seed(9500 + packed)
+    x = torch.randint(0, 255, (tokens, inner), generator=generator, device=device, dtype=torch.uint8)
+    x[x == 0x7F] = 0x7E
+    sx = torch.randint(120, 130, (tokens, inner // 32), generator=generator, device=device, dtype=torch.uint8)
+    if packed:
+        w = torch.randint(0, 256, (outputs, inner // 2), generator=generator, device=device, dtype=torch.uint8)
+        sw = torch.randint(118, 128, (outputs, inner // 32), generator=generator, device=device, dtype=torch.uint8)
+    else:
+        w = torch.randint(0, 255, (outputs, inner), generator=generator, device=device, dtype=torch.uint8)
+        w[w == 0x7F] = 0x7E
+        sw = torch.randint(118, 128, (outputs // 32, inner // 32), generator=generator, device=device, dtype=torch.uint8)
+    weight = w if packed else w.view(torch.float8_e4m3fn)
+    out = _kernels.quantized_matmul(x.view(torch.float8_e4m3fn), sx, weight, sw)
+    assert out.shape == (tokens, outputs)
+    blocks = sample(10, outputs // 32, 4, seams=(3, 288))  # workgroup seams at multiples of 96 rows
+    rows = (blocks[:, None] * 32 + np.arange(32)).ravel()
+    index = torch.from_numpy(rows).to(device)
+    scale_rows = sw[index] if packed else sw[torch.from_numpy(blocks).to(device)]
+    xd = oracle.mx_dequantise(x.cpu().numpy(), sx.cpu().numpy(), 32)
+    wd = oracle.mx_dequantise(w[index].cpu().numpy(), scale_rows.cpu().numpy(), 32, packed, True)
+    want = xd @ wd.T
+    got = bf16_values(out)[:, rows]
+    assert rel_frobenius(got, want) <= 4e-3
+    assert (np.abs(got - want) <= 0.008 * np.abs(want) + (np.abs(xd) @ np.abs(wd).T) * 2.0 ** -13).all()
+    # one more on every input scale doubles every output exactly (E8M0 scales are powers of two)
+    assert torch.equal(_kernels.quantized_matmul(x.view(torch.float8_e4m3fn), sx + 1, weight, sw), out * 2)
