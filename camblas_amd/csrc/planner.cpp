@@ -126,7 +126,9 @@ Plan make_plan(int dtype, int algorithm, bool trans_a, bool trans_b, int m, int 
         plan.family = FAMILY_MFMA_TN;
         plan.counter = 4;
         const int outputs = m, tokens = n;
-        if (tokens <= 64) {
+        // narrow projection: its 128-row tiles occupy at most half of the compute units
+        const bool narrow = ceil_div(outputs, 128) * 2 <= compute_units;
+        if (tokens <= 32 || (tokens <= 64 && !narrow)) {
             // decode: bandwidth-bound on W, one streaming pass, no split-K
             plan.family = FAMILY_STREAM;
             const int row_tiles = stream_row_tiles(outputs, compute_units);
@@ -134,6 +136,17 @@ Plan make_plan(int dtype, int algorithm, bool trans_a, bool trans_b, int m, int 
             plan.kernel = 100 * stream_depth_log2(row_tiles, token_tiles, k) + 10 * row_tiles +
                           token_tiles;
             plan.split_k = 1;
+        } else if (tokens <= 64) {
+            // 33..64 tokens on a narrow projection: the streaming kernel would have 32-48 weight
+            // rows per workgroup and re-read as many token rows through L2; 128 x 64 register-staged
+            // tiles with K divided over up to 2.5 workgroups per compute unit are 15-30 % faster
+            // (measured: [8192, 28672] 89-98 vs 118-137 us, [8192, 8192] 29-32 vs 36-40 us)
+            plan.kernel = 3;
+            const int tiles = ceil_div(outputs, 128);
+            plan.split_k = 1;
+            while (plan.split_k < 16 && tiles * plan.split_k * 2 * 2 <= 5 * compute_units &&
+                   k / (plan.split_k * 2) >= 512)
+                plan.split_k *= 2;
         } else if (ceil_div(outputs, 128) * ceil_div(tokens, 128) * 2 <= compute_units) {
             // few output tiles (a narrow projection, a small batch): 128 x 128 register-staged
             // tiles with K divided over workgroups, the largest power-of-two split that keeps the
