@@ -145,3 +145,16 @@ def test_tensor_binding_loads_and_exports_the_reference_surface():
 
     with pytest.raises(ValueError, match="GPU"):
         module.matmul_public(torch.zeros(2, 2), torch.zeros(2, 2))
+
+
+def test_contexts_inherited_through_fork_are_refused(monkeypatch):
+    # ref: camblas/_native.py:266-268 — the check is on the process id, before any device call
+    import os
+    import types
+
+    table = _native._LOCAL.__dict__.setdefault("contexts", {})
+    inherited = types.SimpleNamespace(pid=os.getpid() + 1, handle=1, set_algorithm=lambda name: None)
+    monkeypatch.setitem(table, (0, 4242), inherited)
+    monkeypatch.setattr(torch.cuda, "current_stream", lambda device=None: types.SimpleNamespace(cuda_stream=4242))
+    with pytest.raises(RuntimeError, match="fork"):
+        _native.context(0)
