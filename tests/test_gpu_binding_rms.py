@@ -1,0 +1,153 @@
+"""Single-row and multi-row RMS normalisation of the binding against torch's own FP32 arithmetic
+on the GPU, after the reference's tests/test_decode_rms.py:19-118 and tests/test_residual_rms.py:
+every supported width, changed values, three epsilons, graph replay, final-only rounding with BF16
+and FP32 weights, and the C entry point on a context of its own with alias rejection.
+
+The reference asks for bit equality with torch, which it gets by copying ATen's reduction tree.
+The kernels here reduce in their own fixed order, so the mean of squares can differ from torch's
+in its last bits. The bar for BF16 storage is at most one unit in the last place on every element
+and bit equality on at least 99 % of them; FP32 storage shows the summation order directly and is
+held to eight units in the last place (1e-6 relative).
+"""
+
+import ctypes
+
+import pytest
+import torch
+
+from camblas_amd import _native
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def binding():
+    module = _native.tensor_module()
+    assert module is not None
+    return module
+
+
+def ulps(actual, expected):
+    """Distance in units in the last place of the storage type (both finite, same sign assumed)."""
+    if actual.dtype == torch.bfloat16:
+        a, b = actual.view(torch.int16).int(), expected.view(torch.int16).int()
+    else:
+        a, b = actual.view(torch.int32).long(), expected.view(torch.int32).long()
+    return (a - b).abs()
+
+
+def assert_matches_torch(actual, expected):
+    distance = ulps(actual.contiguous(), expected.contiguous())
+    if actual.dtype == torch.bfloat16:
+        assert distance.max().item() <= 1
+        assert (distance == 0).float().mean().item() >= 0.99
+    else:
+        assert distance.max().item() <= 8
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("width", [2048, 2052, 4096, 8192, 16384, 32768, 65536])
+def test_single_row_all_widths_and_changed_values(binding, device, dtype, width):
+    torch.manual_seed(20261004)
+    with torch.inference_mode():
+        x = torch.randn((1, 1, width), device=device, dtype=dtype)
+        weight = torch.randn(width, device=device, dtype=dtype)
+        for changed in (False, True):
+            if changed:
+                x.mul_(-0.5).add_(0.125)
+                weight.mul_(-0.5).add_(0.125)
+            for epsilon in (0, 1e-6, 0.01):
+                value = x.float()
+                variance = value.pow(2).mean(-1, keepdim=True)
+                expected = weight * (value * torch.rsqrt(variance + epsilon)).to(dtype)
+                assert_matches_torch(binding.rms_norm(x, weight, epsilon), expected)
+
+
+def test_single_row_graph_replay(binding, device):
+    with torch.no_grad():
+        x = torch.randn((1, 1, 8192), device=device, dtype=torch.bfloat16)
+        weight = torch.randn(8192, device=device, dtype=x.dtype)
+        stream = torch.cuda.Stream(device=device)
+        stream.wait_stream(torch.cuda.current_stream(device))
+        with torch.cuda.stream(stream):
+            for _ in range(3):
+                binding.rms_norm(x, weight, 1e-6)
+            graph = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(graph, stream=stream):
+                output = binding.rms_norm(x, weight, 1e-6)
+            for _ in range(3):
+                x.mul_(-0.5).add_(0.125)
+                weight.mul_(-0.5)
+                graph.replay()
+                stream.synchronize()
+                expected = weight * (x.float() * torch.rsqrt(x.float().pow(2).mean(-1, keepdim=True) + 1e-6)).to(x.dtype)
+                assert_matches_torch(output, expected)
+        graph.reset()
+
+
+@pytest.mark.parametrize("width", [128, 2048, 5120, 8192, 20480, 65536])
+@pytest.mark.parametrize("rows", [1, 3])
+@pytest.mark.parametrize("weight_type", [torch.bfloat16, torch.float32])
+def test_final_only_rounding(binding, device, width, rows, weight_type):
+    torch.manual_seed(20261004)
+    with torch.inference_mode():
+        x = torch.randn((rows, width), device=device, dtype=torch.bfloat16) / 8
+        weight = torch.randn(width, device=device, dtype=weight_type) / 8
+        for changed in ("original", "input", "weight"):
+            if changed == "input":
+                x.mul_(-0.5).add_(0.125)
+            elif changed == "weight":
+                weight.mul_(-0.5)
+            for epsilon in (0, 1e-20, 1e-6):
+                values = x.float()
+                expected = (weight.float() * (values * (values.square().mean(-1, keepdim=True) + epsilon).rsqrt())
+                            ).to(torch.bfloat16)
+                actual = binding.rms_norm(x, weight, epsilon, round_before_weight=False)
+                assert_matches_torch(actual, expected)
+                host = x.cpu().double()
+                independent = weight.cpu().double() * host * (host.square().mean(-1, keepdim=True) + epsilon).rsqrt()
+                torch.testing.assert_close(actual.cpu().double(), independent, rtol=0.008, atol=1e-4)
+
+
+def test_c_entry_on_its_own_context_rejects_aliases(device):
+    # ref: tests/test_residual_rms.py:123-192
+    library = _native.library()
+    function = library.camblas_cuda_add_rms_norm
+    original_device = torch.cuda.current_device()
+    stream = torch.cuda.Stream(device=device)
+    context = ctypes.c_void_p()
+    assert library.camblas_cuda_create(device.index or 0, ctypes.c_void_p(stream.cuda_stream),
+                                       ctypes.byref(context)) == 0
+    try:
+        with torch.no_grad():
+            x = torch.randn(2048, device=device)
+            residual, weight = torch.randn_like(x), torch.randn_like(x)
+            added, output = torch.empty_like(x), torch.empty_like(x)
+            stream.wait_stream(torch.cuda.current_stream(device))
+            pointers = [ctypes.c_void_p(t.data_ptr()) for t in (x, residual, weight, added, output)]
+            arguments = [context, 0, 2048, ctypes.c_float(1e-6)] + pointers
+            for changed in (False, True):
+                if changed:
+                    x.mul_(-0.5)
+                    residual.add_(0.125)
+                    weight.mul_(-0.5)
+                    stream.wait_stream(torch.cuda.current_stream(device))
+                assert function(*arguments) == 0
+                stream.synchronize()
+                expected_sum = (x.cpu().double() + residual.cpu().double()).float()
+                torch.testing.assert_close(added.cpu(), expected_sum, rtol=0, atol=0)
+                value = expected_sum.double()
+                expected = weight.cpu().double() * value * (value.square().mean() + 1e-6).rsqrt()
+                torch.testing.assert_close(output.cpu().double(), expected, rtol=2e-5, atol=2e-5)
+            before = x.cpu().clone()
+            invalid = list(arguments)
+            invalid[-1] = pointers[0]  # output aliases the input
+            assert function(*invalid) != 0
+            invalid = list(arguments)
+            invalid[2] = 2049  # not a multiple of four
+            assert function(*invalid) != 0
+            torch.cuda.synchronize()
+            torch.testing.assert_close(x.cpu(), before, rtol=0, atol=0)
+            assert torch.cuda.current_device() == original_device
+    finally:
+        assert library.camblas_cuda_destroy(context) == 0
