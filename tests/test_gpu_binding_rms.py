@@ -151,3 +151,67 @@ def test_c_entry_on_its_own_context_rejects_aliases(device):
             assert torch.cuda.current_device() == original_device
     finally:
         assert library.camblas_cuda_destroy(context) == 0
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("shape", [(1, 1, 2048), (1, 1, 2052), (1, 1, 8192), (1, 1, 65536), (2, 3, 127),
+                                   (1, 1, 4095)])
+def test_add_rms_norm_outputs_changed_inputs_and_boundaries(binding, device, dtype, shape):
+    # ref: tests/test_residual_rms.py:22-89
+    torch.manual_seed(20261004)
+    with torch.inference_mode():
+        x = torch.randn(shape, device=device, dtype=dtype) / 4
+        residual = torch.randn(shape, device=device, dtype=dtype) / 4
+        weight = torch.randn(shape[-1], device=device, dtype=dtype) / 4
+        for changed in (False, True):
+            if changed:
+                x.mul_(-0.5).add_(0.125)
+                residual.add_(0.25)
+                weight.mul_(-0.5)
+            added, output = binding.add_rms_norm(x, residual, weight, 1e-6)
+            expected_added = (x.cpu().double() + residual.cpu().double()).to(dtype)
+            torch.testing.assert_close(added.cpu(), expected_added, rtol=0, atol=0)
+            reference = expected_added.double()
+            expected = (weight.cpu().double() * (reference * torch.rsqrt(
+                reference.square().mean(-1, keepdim=True) + 1e-6)).to(dtype).double()).to(dtype)
+            torch.testing.assert_close(output.cpu(), expected,
+                                       rtol=0.02 if dtype == torch.bfloat16 else 2e-5,
+                                       atol=0.002 if dtype == torch.bfloat16 else 2e-6)
+            value = added.float()
+            exact = weight * (value * torch.rsqrt(value.square().mean(-1, keepdim=True) + 1e-6)).to(dtype)
+            assert_matches_torch(output, exact)
+            assert added.data_ptr() != x.data_ptr() and output.data_ptr() != added.data_ptr()
+        with pytest.raises(ValueError):
+            binding.add_rms_norm(x, residual, weight, -1)
+        with pytest.raises(ValueError):
+            binding.add_rms_norm(x, residual[..., :3], weight, 1e-6)
+    with pytest.raises(ValueError):
+        binding.add_rms_norm(x.float().clone().requires_grad_(), residual.float(), weight.float(), 1e-6)
+
+
+def test_add_rms_norm_graph_replay(binding, device):
+    # ref: tests/test_residual_rms.py:92-121
+    with torch.no_grad():
+        x = torch.randn((1, 1, 8192), device=device, dtype=torch.bfloat16)
+        residual = torch.randn_like(x)
+        weight = torch.randn(8192, device=device, dtype=x.dtype)
+        stream = torch.cuda.Stream(device=device)
+        stream.wait_stream(torch.cuda.current_stream(device))
+        with torch.cuda.stream(stream):
+            for _ in range(3):
+                binding.add_rms_norm(x, residual, weight, 1e-6)
+            graph = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(graph, stream=stream):
+                added, output = binding.add_rms_norm(x, residual, weight, 1e-6)
+            for _ in range(3):
+                x.add_(0.125)
+                residual.mul_(-0.5)
+                weight.mul_(-0.5)
+                graph.replay()
+                stream.synchronize()
+                expected_added = x + residual
+                torch.testing.assert_close(added, expected_added, rtol=0, atol=0)
+                value = expected_added.float()
+                expected = weight * (value * torch.rsqrt(value.square().mean(-1, keepdim=True) + 1e-6)).to(x.dtype)
+                assert_matches_torch(output, expected)
+        graph.reset()
