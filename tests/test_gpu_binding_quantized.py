@@ -148,3 +148,50 @@ def test_c_entry_dimensions_alignment_aliases_and_empty_rows(device):
         assert call(dimensions, pointers[:4] + [pointer]) != 0
     assert call(dimensions, pointers) == 0
     torch.cuda.synchronize()
+
+
+@pytest.mark.parametrize("shape", [(1152, 5120), (1792, 5120), (4096, 1280), (5120, 2048), (5120, 576),
+                                   (8192, 1280), (25600, 6144)])
+@pytest.mark.parametrize("sample", [0, 1])
+def test_block32_products_on_the_plugin_shapes(binding, device, shape, sample):
+    # ref: tests/test_sglang.py:361-470 without its Triton yardstick: power-of-two block scales,
+    # padded / column-major scale storage, the fused BF16 quantiser against the CPU recipe
+    # (scale = smallest power of two >= amax/448), selected outputs rebuilt in FP64 and held to
+    # the reference's rounding unit max(|value|, 1) / 128
+    n, k = shape
+    torch.manual_seed(413 + sample)
+    a = (torch.randn(1, k, device=device) * 0.75).to(torch.float8_e4m3fn)
+    b = (torch.randn(n, k, device=device) * 0.6).to(torch.float8_e4m3fn)
+    a_scale = (2.0 ** torch.randint(-3, 2, (1, k // 32), device=device)).float()
+    b_scale = (2.0 ** torch.randint(-3, 2, (n // 32, k // 32), device=device)).float()
+    if sample == 1:
+        storage = torch.empty((k // 32, 4), device=device)
+        a_scale = storage[:, 0].view(1, -1)
+        a_scale.uniform_(0.001, 0.08)
+        b_scale = b_scale.T.contiguous().T
+
+    def rebuilt(actual, a, a_scale):
+        indices = torch.arange(0, n, max(1, n // 16), device=device)[:16]
+        decoded_a = a.float().cpu().double() * a_scale.cpu().double().repeat_interleave(32, dim=1)
+        decoded_b = b.index_select(0, indices).float().cpu().double()
+        decoded_b *= b_scale.index_select(0, indices // 32).cpu().double().repeat_interleave(32, dim=1)
+        reference = decoded_a @ decoded_b.T
+        received = actual.index_select(1, indices).float().cpu()
+        assert ((reference - received).abs() <= reference.abs().clamp_min(1.0) / 128).all()
+
+    native = binding.fp8_decode(a, a_scale, b, b_scale)
+    assert native.shape == (1, n) and native.dtype == torch.bfloat16
+    rebuilt(native, a, a_scale)
+    if k <= 8192:
+        bf16 = (torch.randn(1, k, device=device) * (80 if sample else 0.75)).to(torch.bfloat16)
+        fused = binding.fp8_linear(bf16, b, b_scale)
+        values = bf16.float().cpu().view(1, k // 32, 32)
+        raw = values.abs().amax(-1).clamp_min(1.0e-10) * (1.0 / 448.0)
+        bits = raw.view(torch.int32).long()
+        exponent = ((bits >> 23) & 255) - 127 + ((bits & 0x7FFFFF) != 0)
+        cpu_scales = torch.ldexp(torch.ones_like(raw), exponent.int())
+        cpu_q = (values / cpu_scales.unsqueeze(-1)).reshape(1, k).to(torch.float8_e4m3fn)
+        # the fused kernel must equal the two-step path on the CPU-quantised token bit for bit
+        two_step = binding.fp8_decode(cpu_q.to(device), cpu_scales.to(device), b, b_scale)
+        assert torch.equal(fused.view(torch.int16), two_step.view(torch.int16))
+        rebuilt(fused, cpu_q.to(device), cpu_scales.to(device))
