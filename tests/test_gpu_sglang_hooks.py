@@ -144,3 +144,23 @@ def test_fp8_block32_hooks(device):
     assert linear(original, xt, B, [32, 32], Bs, None, None, False, None) == "original"
     assert linear(original, xt, B, [32, 32], Bs, torch.ones(1, device=device), None, True, None) == "original"
     assert len(original.calls) == 5 and len(original.calls[-1]) == 8
+
+
+@pytest.mark.parametrize("shape", [(2048, 4096), (3392, 6144)])
+@pytest.mark.parametrize("magnitude", [0.75, 80.0])
+def test_fp8_block128_hook_on_the_reference_shapes(device, shape, magnitude):
+    # ref: tests/test_sglang.py:74-117 — one BF16 token, dynamic 1x128 quantisation, a weight whose
+    # row count is not a multiple of the 128-row scale block; FP64 product of the oracle-quantised
+    # token as the yardstick (the reference compares with SGLang's own kernel bit for bit)
+    outputs, inner = shape
+    hook = plugin.build_hooks({"fp8"})[plugin.FP8_BLOCK128_TARGET]
+    x = oracle.fill_normal_bf16(717, (1, inner), std=magnitude)
+    w, w_scale = oracle.fill_fp8_blocks(718, outputs, inner, 128)
+    w_scale = (w_scale * 1.25).astype(np.float32)
+    original = Original()
+    with torch.no_grad():
+        out = hook(original, to_device_bf16(x, device), to_device_fp8(w, device), [128, 128],
+                   torch.from_numpy(w_scale).to(device))
+    assert not original.calls and out.shape == (1, outputs)
+    q, scale = oracle.quantise_1x128(x)
+    assert rel_frobenius(bf16_values(out), oracle.fp8_block_matmul_f64(q, scale, w, w_scale)) <= 1e-2
