@@ -187,3 +187,37 @@ def test_dgemm_matches_float64_product(device, ta, tb):
     want = 0.75 * (left @ right) - 2.0 * c0.reshape(n, ldc)[:, :m].T
     assert rel_frobenius(got[:, :m].T, want) <= 1e-13
     assert np.array_equal(got[:, m:], c0.reshape(n, ldc)[:, m:])
+
+
+@pytest.mark.parametrize("kernel", ["vector", "matrix", "matrix64"])
+@pytest.mark.parametrize("shape", [(67, 45, 130), (200, 131, 257), (129, 64, 1024)])
+def test_sgemm_exact_rank_two_integer_identity(device, kernel, shape):
+    # ref: tests/test_mlp_packing.py:120-207 — A = u v^T + p q^T and B = r s^T + t w^T make A B four
+    # outer products of small integers: every product and every partial sum is exact in FP32, so
+    # any summation order must give the same bits, and a wrong index shows up exactly
+    m, n, k = shape
+    i, j, depth = np.arange(m), np.arange(n), np.arange(k)
+    v, q, r, t = depth % 5 - 2, depth % 11 - 5, depth % 13 - 6, depth % 3 - 1
+    products = [int(np.sum(x * y)) for x, y in ((v, r), (v, t), (q, r), (q, t))]
+    for ta in "NT":
+        for tb in "NT":
+            for change, (alpha, beta) in enumerate([(1.0, 0.0), (0.5, -0.25), (-1.0, 1.0)]):
+                u, p = i % 7 - 3 + change, i % 3 - 1 - change
+                s, w = j % 5 - 2 - change, j % 7 - 3 + change
+                left = (u[:, None] * v + p[:, None] * q).astype(np.float32)       # [m, k]
+                right = (r[:, None] * s + t[:, None] * w).astype(np.float32)      # [k, n]
+                lda, ldb, ldc = (m if ta == "N" else k) + 3, (k if tb == "N" else n) + 5, m + 7
+                a = np.full(lda * (k if ta == "N" else m), -73.0, np.float32)
+                b = np.full(ldb * (n if tb == "N" else k), -73.0, np.float32)
+                # column-major storage: element (x, y) of the stored matrix at x + y * ld
+                stored_a = left if ta == "N" else left.T
+                stored_b = right if tb == "N" else right.T
+                a.reshape(-1, lda)[:, : stored_a.shape[0]] = stored_a.T
+                b.reshape(-1, ldb)[:, : stored_b.shape[0]] = stored_b.T
+                c = np.full(ldc * n, np.nan if beta == 0 else 2.0, np.float32)
+                c.reshape(n, ldc)[:, m:] = -73.0
+                got = run_sgemm(device, ta, tb, m, n, k, alpha, a, lda, b, ldb, beta, c, ldc, kernel=kernel)
+                expected = alpha * (products[0] * u[:, None] * s + products[1] * u[:, None] * w
+                                    + products[2] * p[:, None] * s + products[3] * p[:, None] * w) + beta * 2.0
+                assert np.array_equal(got.reshape(n, ldc)[:, :m].T, expected.astype(np.float32)), (ta, tb, change)
+                assert (got.reshape(n, ldc)[:, m:] == -73.0).all()
