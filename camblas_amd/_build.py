@@ -33,6 +33,7 @@ CORE_SOURCES = (
     "fp8_stream.hip",
     "fp8_block32.hip",
     "mx_matmul.hip",
+    "mx_dma.hip",
     "routing.hip", "dense_ops.hip", "sgemm_mfma.hip",
     "fusion.hip",
     "attention_decode.hip",

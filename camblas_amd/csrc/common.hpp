@@ -129,10 +129,19 @@ hipError_t launch_fp8_block32_decode(hipStream_t stream, int outputs, int inner,
                                      const float *sx, int sx_stride, const void *w, const float *sw,
                                      int sw_row, int sw_col, void *out);
 // E8M0 block-scaled product (E4M3 or packed E2M1 weights); groups == 0 plain, >= 1 grouped.
-hipError_t launch_mx_matmul(hipStream_t stream, bool packed, int groups, int weight_groups, int rows,
-                            int outputs, int inner, int activation_block, const void *input,
+// kernel: -1 chooses by shape; 0 the weight-streaming kernel; 20 + v the prefill kernel variant v.
+hipError_t launch_mx_matmul(hipStream_t stream, int kernel, bool packed, int groups, int weight_groups,
+                            int rows, int outputs, int inner, int activation_block, const void *input,
                             const void *input_scale, const void *weight, const void *weight_scale,
                             const void *metadata, const void *active, const void *counts, void *out);
+// Prefill-sized E8M0 product (hardware-scaled matrix instructions, operands loaded straight into
+// LDS); needs inner % 128 == 0, 16-byte aligned operands and an 8-byte aligned output.
+int mx_dma_variant_count();
+bool mx_dma_supported(int outputs, int inner, const void *input, const void *weight, const void *out);
+hipError_t launch_mx_dma(hipStream_t stream, int variant, bool packed, int groups, int weight_groups,
+                         int rows, int outputs, int inner, int activation_block, const void *input,
+                         const void *input_scale, const void *weight, const void *weight_scale,
+                         const void *metadata, const void *active, const void *counts, void *out);
 // Mixture-of-experts routing helpers.
 hipError_t launch_route_groups(hipStream_t stream, int tokens, int choices, int first_expert,
                                int groups, int rows, const void *experts, const void *active,

@@ -34,6 +34,14 @@ __device__ __forceinline__ void load_to_lds(__amdgpu_buffer_rsrc_t resource, uns
                                              step_offset, 0, 0);
 }
 
+// The same with 4 bytes per lane: LDS gets 64 consecutive words at `lds_base`.
+__device__ __forceinline__ void load_word_to_lds(__amdgpu_buffer_rsrc_t resource, unsigned lane_offset,
+                                                 unsigned step_offset, void *lds_base)
+{
+    __builtin_amdgcn_raw_ptr_buffer_load_lds(resource, (lds_void_t *)lds_base, 4, lane_offset,
+                                             step_offset, 0, 0);
+}
+
 // Raw buffer resource over `bytes` bytes starting at `base` (gfx9 descriptor word 3: 32-bit data).
 __device__ __forceinline__ __amdgpu_buffer_rsrc_t make_resource(const void *base, unsigned bytes)
 {

@@ -1,0 +1,467 @@
+// Prefill-sized E8M0 block-scaled product on the gfx950 matrix cores with hardware scales:
+// out[M,N] = x[M,K] . w[N,K]^T, x E4M3 with one E8M0 scale per 32 (or 128) inputs, w E4M3 with one
+// scale per 32 x 32 block or packed E2M1 with one scale per row and 32 inputs, BF16 out; plain and
+// grouped (contract: ref include/camblas_cuda.h:110-167, src/cuda/backend.cu:1165-1191, :1258-1303;
+// value semantics: tests/test_quantized.py:12-50 of the reference).
+//
+// v_mfma_scale_f32_32x32x64_f8f6f4 multiplies a 32 x 64 by a 64 x 32 tile and applies one E8M0 scale
+// per row and 32 inputs on either side, so the whole scaling rule is inside the instruction and the
+// accumulators are never touched by the vector ALU. Operand layout (checked against a host product
+// of random operands and scales): of the 64 K positions of one instruction, lane group c = lane/32
+// of an 8-bit operand holds positions 16c..16c+15 in its first 16 bytes and 32+16c..32+16c+15 in
+// its second 16 bytes; a 4-bit operand holds positions 32c..32c+31 in its first 16 bytes; the scale
+// byte supplied by lane group g applies to positions 32g..32g+31 of that lane's row.
+//
+// Structure: as the FP32-scaled FP8 prefill kernel. A workgroup of 2 x WM wavefronts owns
+// (64*TN) weight rows x (32*WM*TM) tokens, a K step is 128 inputs (128 bytes of an E4M3 row, 64 of
+// an E2M1 row), operands go straight from memory into XOR-swizzled LDS stages STAGES-1 steps ahead
+// (buffer_load ... lds; rows outside the matrix read as zero). The four scale bytes of a row and
+// step are one 32-bit word, read from the address rounded down to four bytes; v_alignbyte of two
+// consecutive words undoes any misalignment of the scale pointer, which is the same for every row
+// because a scale row is a multiple of four bytes long. E4M3 weights have one scale row per 32
+// weight rows, so a tile's word is one address for the whole wavefront and is loaded into
+// registers two steps ahead, like the per-token words. E2M1 weights have one scale row per weight
+// row: there the words of all rows of the workgroup (and of its tokens) are gathered once per step
+// into the LDS stage, 64 rows per wavefront load, instead of once per wavefront that uses them.
+#include "common.hpp"
+#include "device.hpp"
+#include "dma.hpp"
+
+namespace camblas_hip
+{
+namespace
+{
+struct MxDmaParams {
+    const unsigned char *input, *input_scale, *weight, *weight_scale;
+    unsigned short *out;
+    int rows, outputs, inner, steps; // steps = inner / 128
+    int tiles_n, tiles_m;
+    // grouped form
+    const unsigned long long *metadata;
+    const int32_t *active, *counts;
+    int weight_groups;
+};
+
+__device__ __forceinline__ unsigned scale_word(const unsigned char *base, int index)
+{
+    return *reinterpret_cast<const unsigned *>(base + size_t(index) * 4);
+}
+
+__device__ __forceinline__ unsigned long long uniform(unsigned long long value)
+{
+    const unsigned lo = __builtin_amdgcn_readfirstlane(unsigned(value));
+    const unsigned hi = __builtin_amdgcn_readfirstlane(unsigned(value >> 32));
+    return (static_cast<unsigned long long>(hi) << 32) | lo;
+}
+
+// WIDE_X: one activation scale per 128 inputs (one byte per step) instead of one per 32
+template <bool PACKED, bool WIDE_X, bool GROUPED, int TN, int TM, int WM, int STAGES>
+__global__ __launch_bounds__(128 * WM) void mx_dma_kernel(MxDmaParams p)
+{
+    static_assert(STAGES == 2 || STAGES == 3, "two or three LDS stages");
+    static_assert(PACKED || !WIDE_X, "128-input activation scales go with E2M1 weights only");
+    constexpr int WAVES = 2 * WM, BK = 128;
+    constexpr int CHW = PACKED ? 4 : 8, CHX = 8;        // 16-byte chunks of a row per step
+    constexpr int W_ROWS = 64 / CHW, X_ROWS = 64 / CHX; // rows covered by one wavefront load
+    constexpr int BN = 64 * TN, BM = 32 * WM * TM;
+    constexpr int A_ITERS = BN / (WAVES * W_ROWS), B_ITERS = BM / (WAVES * X_ROWS);
+    static_assert(BN % (WAVES * W_ROWS) == 0 && BM % (WAVES * X_ROWS) == 0, "loads");
+    static_assert((WAVES * W_ROWS) % 16 == 0 && (WAVES * X_ROWS) % 16 == 0, "row step keeps the swizzle");
+    constexpr int W_SLOTS = BN * CHW, SLOTS = W_SLOTS + BM * CHX, LOADS = A_ITERS + B_ITERS;
+    // scale words that travel through LDS: those of the weight rows and, unless the tokens have
+    // one scale byte per step, of the token rows
+    constexpr bool STAGED = PACKED;
+    constexpr int STAGED_ROWS = STAGED ? BN + (WIDE_X ? 0 : BM) : 0;
+    constexpr int SCALE_WAVES = STAGED ? STAGED_ROWS / 64 : 1;
+    static_assert(!STAGED || (STAGES == 3 && STAGED_ROWS % 64 == 0 && SCALE_WAVES <= WAVES),
+                  "one wavefront load stages the scale words of 64 rows");
+    __shared__ u32x4_t stages[STAGES][SLOTS];
+    // (an array of its own: all its reads share one address register and differ by immediates)
+    __shared__ u32x4_t scale_stages[STAGES][STAGED ? STAGED_ROWS / 4 : 1];
+
+    int tile_n, tile_m;
+    xcd_tile(int(blockIdx.x), p.tiles_n, p.tiles_m, tile_n, tile_m);
+    const int n0 = tile_n * BN, m0 = tile_m * BM;
+    const int thread = threadIdx.x, lane = thread % 64, wave = thread / 64;
+    const int wn = wave % 2, wm = wave / 2;
+    const int scale_pitch = p.inner / 32; // bytes of a row of 32-input scales: a multiple of four
+
+    const unsigned char *input = p.input, *input_scale = p.input_scale, *weight = p.weight,
+                        *weight_scale = p.weight_scale;
+    unsigned short *out = p.out;
+    int valid_rows = p.rows;
+    if constexpr (GROUPED) {
+        // ref: include/camblas_cuda.h:156-167 — weights come from a device table indexed by
+        // active[group]; invalid indices and rows at or beyond counts[group] produce zeros
+        // (values that are the same for the whole workgroup are moved to scalar registers)
+        const int group = blockIdx.y;
+        const int index = __builtin_amdgcn_readfirstlane(p.active[group]);
+        const int count = __builtin_amdgcn_readfirstlane(p.counts[group]);
+        valid_rows = index >= 0 && index < p.weight_groups ? min(max(count, 0), p.rows) : 0;
+        input += size_t(group) * p.rows * p.inner;
+        input_scale += size_t(group) * p.rows * (WIDE_X ? p.steps : scale_pitch);
+        out += size_t(group) * p.rows * p.outputs;
+        if (m0 >= valid_rows) { // nothing to multiply: this tile of the output is zero
+            for (int item = thread; item < BM * (BN / 4); item += 128 * WM) {
+                const int m = m0 + item / (BN / 4), n = n0 + (item % (BN / 4)) * 4;
+                if (m < p.rows && n < p.outputs)
+                    *reinterpret_cast<u32x2_t *>(out + size_t(m) * p.outputs + n) = u32x2_t{0u, 0u};
+            }
+            return;
+        }
+        weight = reinterpret_cast<const unsigned char *>(uniform(p.metadata[2 * size_t(index)]));
+        weight_scale = reinterpret_cast<const unsigned char *>(uniform(p.metadata[2 * size_t(index) + 1]));
+    }
+
+    // ---- operand loads. Lane -> (row inside one wavefront load, swizzled chunk); successive loads
+    // of a thread are WAVES*rows apart, which leaves the swizzle unchanged, so one lane offset
+    // serves all of them and the row advance goes into the wave-uniform offset.
+    const unsigned w_pitch = PACKED ? unsigned(p.inner) / 2 : unsigned(p.inner);
+    const int w_load_row = wave * W_ROWS + lane / CHW, x_load_row = wave * X_ROWS + lane / CHX;
+    const unsigned w_lane_off =
+        unsigned(w_load_row) * w_pitch + unsigned(((lane % CHW) ^ lds_swizzle<CHW>(w_load_row)) * 16);
+    const unsigned x_lane_off = unsigned(x_load_row) * unsigned(p.inner) +
+                                unsigned(((lane % CHX) ^ lds_swizzle<CHX>(x_load_row)) * 16);
+    const unsigned w_row_step = unsigned(WAVES * W_ROWS) * w_pitch;
+    const unsigned x_row_step = unsigned(WAVES * X_ROWS) * unsigned(p.inner);
+    const int w_rows = p.outputs - n0 < BN ? p.outputs - n0 : BN;
+    const int x_rows = valid_rows - m0 < BM ? valid_rows - m0 : BM;
+    const __amdgpu_buffer_rsrc_t w_resource =
+        make_resource(weight + size_t(n0) * w_pitch, unsigned(w_rows) * w_pitch);
+    const __amdgpu_buffer_rsrc_t x_resource =
+        make_resource(input + size_t(m0) * p.inner, unsigned(x_rows) * unsigned(p.inner));
+    constexpr unsigned W_STEP_BYTES = PACKED ? BK / 2 : BK;
+    const int last_step = p.steps - 1;
+    int load_step = 0;
+    auto issue_one = [&](u32x4_t *stage, int index) {
+        if (index < A_ITERS)
+            load_to_lds(w_resource, w_lane_off,
+                        unsigned(load_step) * W_STEP_BYTES + unsigned(index) * w_row_step,
+                        stage + (index * WAVES + wave) * 64);
+        else
+            load_to_lds(x_resource, x_lane_off,
+                        unsigned(load_step) * BK + unsigned(index - A_ITERS) * x_row_step,
+                        stage + W_SLOTS + ((index - A_ITERS) * WAVES + wave) * 64);
+    };
+    auto advance = [&]() { load_step = load_step < last_step ? load_step + 1 : last_step; };
+    auto issue = [&](u32x4_t *stage) {
+#pragma unroll
+        for (int index = 0; index < LOADS; ++index)
+            issue_one(stage, index);
+        advance();
+    };
+
+    // ---- scales: per lane (operand row lane%32) one 32-bit word per 32-row tile and step, read
+    // from the 4-byte aligned address at or below the row's scales. Register path: loaded
+    // unconditionally two steps ahead (a load under a branch would make the compiler wait for the
+    // LDS fills as well).
+    const int frag_row = lane % 32, half = lane / 32;
+    const unsigned w_skew = unsigned(reinterpret_cast<uintptr_t>(weight_scale)) & 3u;
+    const unsigned x_skew = WIDE_X ? 0u : unsigned(reinterpret_cast<uintptr_t>(input_scale)) & 3u;
+    const int w_last_word = p.steps - 1 + (w_skew != 0), x_last_word = p.steps - 1 + (x_skew != 0);
+    unsigned ws_offset[TN], xs_offset[TM]; // bytes from (scale pointer - skew): rows * pitch < 2^32
+#pragma unroll
+    for (int i = 0; i < TN; ++i) {
+        int n = n0 + (wn * TN + i) * 32;
+        n = n < p.outputs ? n : p.outputs - 1;
+        ws_offset[i] = unsigned(n / 32) * unsigned(scale_pitch); // (register path: E4M3 weights)
+    }
+#pragma unroll
+    for (int j = 0; j < TM; ++j) {
+        int m = m0 + (wm * TM + j) * 32 + frag_row;
+        m = m < valid_rows ? m : valid_rows - 1;
+        xs_offset[j] = unsigned(m) * unsigned(WIDE_X ? p.steps : scale_pitch);
+    }
+    unsigned ws_now[TN], ws_next[TN], ws_load[TN], xs_now[TM], xs_next[TM], xs_load[TM];
+    auto fetch_scales = [&](int step, unsigned (&w)[TN], unsigned (&x)[TM]) {
+        const int w_word = step < w_last_word ? step : w_last_word;
+        const int x_word = step < x_last_word ? step : x_last_word;
+        if constexpr (!STAGED) {
+#pragma unroll
+            for (int i = 0; i < TN; ++i)
+                w[i] = scale_word(weight_scale - w_skew + ws_offset[i], w_word);
+        }
+        if constexpr (!STAGED && !WIDE_X) {
+#pragma unroll
+            for (int j = 0; j < TM; ++j)
+                x[j] = scale_word(input_scale - x_skew + xs_offset[j], x_word);
+        }
+    };
+    // one scale byte per token and step: no second word is needed, so one step ahead is enough
+    auto fetch_token_bytes = [&](int step, unsigned (&x)[TM]) {
+        const int x_byte = step < last_step ? step : last_step;
+        if constexpr (WIDE_X) {
+#pragma unroll
+            for (int j = 0; j < TM; ++j)
+                x[j] = unsigned(input_scale[xs_offset[j] + unsigned(x_byte)]);
+        }
+    };
+    // LDS path: wavefront w gathers the words of scale rows 64*w .. 64*w+63 of the list (weight
+    // rows of the tile, then its token rows) into the words behind the stage's operand tiles.
+    // Wavefronts beyond the list repeat the load of another one (same data to the same place)
+    // rather than branch around a load.
+    const int scale_wave = wave % SCALE_WAVES;
+    const bool scale_of_weights = scale_wave * 64 < BN; // wave-uniform
+    const int scale_last_word = scale_of_weights ? w_last_word : x_last_word;
+    unsigned scale_lane_off = 0;
+    int scale_step = 0;
+    __amdgpu_buffer_rsrc_t scale_resource = w_resource;
+    if constexpr (STAGED) {
+        const int listed = scale_wave * 64 + lane;
+        int row = scale_of_weights ? n0 + listed : m0 + listed - BN;
+        const int rows = scale_of_weights ? p.outputs : valid_rows;
+        row = row < rows ? row : rows - 1;
+        scale_lane_off = unsigned(row) * unsigned(scale_pitch);
+        const unsigned skew = scale_of_weights ? w_skew : x_skew;
+        scale_resource =
+            make_resource((scale_of_weights ? weight_scale : input_scale) - skew,
+                          unsigned(rows) * unsigned(scale_pitch) + (skew ? 4u : 0u));
+    }
+    auto issue_scales = [&](u32x4_t *stage) {
+        if constexpr (STAGED) {
+            load_word_to_lds(scale_resource, scale_lane_off, unsigned(scale_step) * 4u,
+                             stage + scale_wave * 16);
+            scale_step = scale_step < scale_last_word ? scale_step + 1 : scale_last_word;
+        }
+    };
+    auto read_scales = [&](const u32x4_t *stage, unsigned (&w)[TN], unsigned (&x)[TM]) {
+        const unsigned *words = reinterpret_cast<const unsigned *>(stage);
+#pragma unroll
+        for (int i = 0; i < TN; ++i)
+            w[i] = words[(wn * TN + i) * 32 + frag_row];
+        if constexpr (!WIDE_X) {
+#pragma unroll
+            for (int j = 0; j < TM; ++j)
+                x[j] = words[BN + (wm * TM + j) * 32 + frag_row];
+        }
+    };
+
+    const int w_swizzle = lds_swizzle<CHW>(frag_row), x_swizzle = lds_swizzle<CHX>(frag_row);
+    const int w_frag_base = (wn * TN * 32 + frag_row) * CHW;
+    const int x_frag_base = W_SLOTS + (wm * TM * 32 + frag_row) * CHX;
+    f32x16_t acc[TN][TM];
+#pragma unroll
+    for (int i = 0; i < TN; ++i)
+#pragma unroll
+        for (int j = 0; j < TM; ++j)
+#pragma unroll
+            for (int r = 0; r < 16; ++r)
+                acc[i][j][r] = 0.f;
+
+    // operand of the instruction that covers inputs 64*ks .. 64*ks+63 of the step
+    auto fragment8 = [&](const u32x4_t *stage, int base, int swizzle, int ks) {
+        const u32x4_t lo = stage[base + ((ks * 4 + half) ^ swizzle)];
+        const u32x4_t hi = stage[base + ((ks * 4 + 2 + half) ^ swizzle)];
+        return i32x8_t{int(lo[0]), int(lo[1]), int(lo[2]), int(lo[3]),
+                       int(hi[0]), int(hi[1]), int(hi[2]), int(hi[3])};
+    };
+    auto fragment4 = [&](const u32x4_t *stage, int base, int swizzle, int ks) {
+        const u32x4_t lo = stage[base + ((ks * 2 + half) ^ swizzle)];
+        return i32x8_t{int(lo[0]), int(lo[1]), int(lo[2]), int(lo[3]), 0, 0, 0, 0};
+    };
+    auto weight_fragment = [&](const u32x4_t *stage, int tile, int ks) {
+        if constexpr (PACKED)
+            return fragment4(stage, w_frag_base + tile * 32 * CHW, w_swizzle, ks);
+        else
+            return fragment8(stage, w_frag_base + tile * 32 * CHW, w_swizzle, ks);
+    };
+
+    // One K step, as two halves of 64 inputs: the token fragments of a half are read once, the
+    // weight fragments (one per 32-row tile) one instruction group ahead into the other of two
+    // register buffers; the fills of the stage STAGES-1 ahead are issued between the matrix
+    // instructions.
+    auto multiply = [&](const u32x4_t *stage, u32x4_t *fill, const unsigned (&w_scale)[TN],
+                        const unsigned (&x_scale)[TM]) {
+        constexpr int OPS = TN * 2 * TM, SHARE = (LOADS + OPS - 1) / OPS;
+        i32x8_t w_frag[2], x_frag[TM];
+        w_frag[0] = weight_fragment(stage, 0, 0);
+#pragma unroll
+        for (int op = 0; op < OPS; ++op) {
+            const int part = op / TM, ks = part / TN, i = part % TN, j = op % TM;
+            __builtin_amdgcn_sched_barrier(0);
+            if (op % (TN * TM) == 0) {
+#pragma unroll
+                for (int t = 0; t < TM; ++t)
+                    x_frag[t] = fragment8(stage, x_frag_base + t * 32 * CHX, x_swizzle, ks);
+            }
+            if (j == 0 && part + 1 < TN * 2)
+                w_frag[(part + 1) & 1] = weight_fragment(stage, (part + 1) % TN, (part + 1) / TN);
+            __builtin_amdgcn_sched_barrier(0);
+            if (ks == 0) // (the byte selects are immediates of the instruction)
+                acc[i][j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(
+                    w_frag[part & 1], x_frag[j], acc[i][j], PACKED ? 4 : 0, 0, 0, int(w_scale[i]), 0,
+                    int(x_scale[j]));
+            else
+                acc[i][j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(
+                    w_frag[part & 1], x_frag[j], acc[i][j], PACKED ? 4 : 0, 0, 2, int(w_scale[i]),
+                    WIDE_X ? 0 : 2, int(x_scale[j]));
+            __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+            for (int index = op * SHARE; index < (op + 1) * SHARE && index < LOADS; ++index)
+                issue_one(fill, index);
+        }
+        __builtin_amdgcn_sched_barrier(0);
+        advance();
+    };
+
+    // The scale byte of this lane's block (lane group g supplies the scale of inputs 32g..32g+31 of
+    // an instruction) is byte 2*ks + half of the step's word: the word is shifted by `half` bytes
+    // and the instruction's byte select takes byte 2*ks.
+    auto step = [&](int g, int s, const u32x4_t *current, u32x4_t *fill) {
+        if constexpr (STAGED) {
+            // words of step g + 2, ahead of its operand fills; words of step g + 1, gathered a step ago
+            issue_scales(scale_stages[(s + STAGES - 1) % STAGES]);
+            read_scales(scale_stages[(s + 1) % STAGES], ws_next, xs_next);
+        }
+        fetch_scales(g + 2, ws_load, xs_load);
+        fetch_token_bytes(g + 1, xs_next);
+        unsigned w_scale[TN], x_scale[TM];
+#pragma unroll
+        for (int i = 0; i < TN; ++i)
+            w_scale[i] = __builtin_amdgcn_alignbyte(ws_next[i], ws_now[i], w_skew) >> (8 * half);
+#pragma unroll
+        for (int j = 0; j < TM; ++j)
+            x_scale[j] = WIDE_X ? xs_now[j]
+                                : __builtin_amdgcn_alignbyte(xs_next[j], xs_now[j], x_skew) >> (8 * half);
+        __builtin_amdgcn_sched_barrier(0);
+        multiply(current, fill, w_scale, x_scale);
+#pragma unroll
+        for (int i = 0; i < TN; ++i) {
+            ws_now[i] = ws_next[i];
+            if constexpr (!STAGED)
+                ws_next[i] = ws_load[i];
+        }
+#pragma unroll
+        for (int j = 0; j < TM; ++j) {
+            xs_now[j] = xs_next[j];
+            if constexpr (!STAGED && !WIDE_X)
+                xs_next[j] = xs_load[j];
+        }
+        pipeline_barrier<(STAGES - 2) * LOADS>();
+    };
+
+    fetch_scales(0, ws_now, xs_now);
+    fetch_scales(1, ws_next, xs_next);
+    fetch_token_bytes(0, xs_now);
+#pragma unroll
+    for (int s = 0; s + 1 < STAGES; ++s) {
+        __builtin_amdgcn_sched_barrier(0);
+        issue_scales(scale_stages[s]);
+        issue(stages[s]);
+    }
+    pipeline_barrier<(STAGES - 2) * LOADS>();
+    if constexpr (STAGED)
+        read_scales(scale_stages[0], ws_now, xs_now);
+    // whole rounds of STAGES steps run without a branch between the steps; the remainder follows
+    int g = 0;
+    for (; g + STAGES <= p.steps; g += STAGES) {
+#pragma unroll
+        for (int s = 0; s < STAGES; ++s)
+            step(g + s, s, stages[s], stages[(s + STAGES - 1) % STAGES]);
+    }
+#pragma unroll
+    for (int s = 0; s + 1 < STAGES; ++s)
+        if (g + s < p.steps)
+            step(g + s, s, stages[s], stages[(s + STAGES - 1) % STAGES]);
+    wait_loads<0>();
+
+    // ---- epilogue: accumulator register 4q+e of lane l is feature 8q + 4*(l/32) + e, token l%32
+#pragma unroll
+    for (int j = 0; j < TM; ++j) {
+        const int m = m0 + (wm * TM + j) * 32 + frag_row;
+        const bool live = !GROUPED || m < valid_rows; // padding rows of a group are written as zeros
+        unsigned short *row = out + size_t(m) * p.outputs + n0 + wn * TN * 32 + half * 4;
+#pragma unroll
+        for (int i = 0; i < TN; ++i) {
+            __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+            for (int q = 0; q < 4; ++q) {
+                const int offset = i * 32 + q * 8;
+                if (m < p.rows && n0 + wn * TN * 32 + half * 4 + offset < p.outputs) {
+                    u32x2_t packed = {pack_bf16x2(acc[i][j][q * 4], acc[i][j][q * 4 + 1]),
+                                      pack_bf16x2(acc[i][j][q * 4 + 2], acc[i][j][q * 4 + 3])};
+                    if (!live)
+                        packed = u32x2_t{0u, 0u};
+                    *reinterpret_cast<u32x2_t *>(row + offset) = packed;
+                }
+            }
+        }
+    }
+}
+
+template <bool PACKED, bool WIDE_X, bool GROUPED, int TN, int TM, int WM, int STAGES>
+hipError_t launch_one(hipStream_t stream, MxDmaParams p, int groups)
+{
+    constexpr int BN = 64 * TN, BM = 32 * WM * TM;
+    p.tiles_n = (p.outputs + BN - 1) / BN;
+    p.tiles_m = (p.rows + BM - 1) / BM;
+    if (size_t(p.tiles_n) * size_t(p.tiles_m) > 0x7fffffffu || groups > 65535)
+        return hipErrorInvalidValue;
+    dim3 grid(unsigned(p.tiles_n) * unsigned(p.tiles_m), unsigned(groups));
+    mx_dma_kernel<PACKED, WIDE_X, GROUPED, TN, TM, WM, STAGES><<<grid, 128 * WM, 0, stream>>>(p);
+    return launch_status();
+}
+
+// variant 0: 256 weight rows x 256 tokens (two stages for E4M3 weights, three for E2M1);
+// variant 1: 256 x 128, three stages
+template <bool PACKED, bool WIDE_X, bool GROUPED>
+hipError_t launch_variant(hipStream_t stream, const MxDmaParams &p, int groups, int variant)
+{
+    switch (variant) {
+    case 0: return launch_one<PACKED, WIDE_X, GROUPED, 4, 2, 4, PACKED ? 3 : 2>(stream, p, groups);
+    case 1: return launch_one<PACKED, WIDE_X, GROUPED, 4, 1, 4, 3>(stream, p, groups);
+    default: return hipErrorInvalidValue;
+    }
+}
+} // namespace
+
+int mx_dma_variant_count() { return 2; }
+
+// The prefill kernel's conditions: K a multiple of 128, 16-byte aligned operands, an 8-byte aligned
+// output (scale pointers may have any alignment).
+bool mx_dma_supported(int outputs, int inner, const void *input, const void *weight, const void *out)
+{
+    // (32-bit byte offsets: a 256-row operand tile, and the scale bytes of all rows of an operand)
+    return inner % 128 == 0 && outputs % 4 == 0 && size_t(256) * size_t(inner) < (size_t(1) << 32) &&
+           (size_t(outputs) + 65536) * size_t(inner / 32) < (size_t(1) << 32) &&
+           reinterpret_cast<uintptr_t>(out) % 8 == 0 && reinterpret_cast<uintptr_t>(input) % 16 == 0 &&
+           reinterpret_cast<uintptr_t>(weight) % 16 == 0;
+}
+
+// groups == 0: plain product; >= 1: grouped (weights and their scales from the device table)
+hipError_t launch_mx_dma(hipStream_t stream, int variant, bool packed, int groups, int weight_groups,
+                         int rows, int outputs, int inner, int activation_block, const void *input,
+                         const void *input_scale, const void *weight, const void *weight_scale,
+                         const void *metadata, const void *active, const void *counts, void *out)
+{
+    if (!mx_dma_supported(outputs, inner, input, weight, out) ||
+        (activation_block != 32 && !(packed && activation_block == 128)))
+        return hipErrorInvalidValue;
+    MxDmaParams p;
+    p.input = static_cast<const unsigned char *>(input);
+    p.input_scale = static_cast<const unsigned char *>(input_scale);
+    p.weight = static_cast<const unsigned char *>(weight);
+    p.weight_scale = static_cast<const unsigned char *>(weight_scale);
+    p.out = static_cast<unsigned short *>(out);
+    p.rows = rows;
+    p.outputs = outputs;
+    p.inner = inner;
+    p.steps = inner / 128;
+    p.tiles_n = p.tiles_m = 0;
+    p.metadata = static_cast<const unsigned long long *>(metadata);
+    p.active = static_cast<const int32_t *>(active);
+    p.counts = static_cast<const int32_t *>(counts);
+    p.weight_groups = weight_groups;
+    const bool wide = activation_block == 128;
+    if (groups == 0) {
+        if (!packed)
+            return launch_variant<false, false, false>(stream, p, 1, variant);
+        return wide ? launch_variant<true, true, false>(stream, p, 1, variant)
+                    : launch_variant<true, false, false>(stream, p, 1, variant);
+    }
+    if (!packed)
+        return launch_variant<false, false, true>(stream, p, groups, variant);
+    return wide ? launch_variant<true, true, true>(stream, p, groups, variant)
+                : launch_variant<true, false, true>(stream, p, groups, variant);
+}
+} // namespace camblas_hip

@@ -407,11 +407,29 @@ hipError_t launch_shape(hipStream_t stream, const MxParams &p, int groups)
 
 // groups == 0: plain product (weight, weight_scale given); groups >= 1: grouped product (metadata,
 // active, counts given). activation_block 32 or 128. Weights 16-byte aligned.
-hipError_t launch_mx_matmul(hipStream_t stream, bool packed, int groups, int weight_groups, int rows,
-                            int outputs, int inner, int activation_block, const void *input,
+hipError_t launch_mx_matmul(hipStream_t stream, int kernel, bool packed, int groups, int weight_groups,
+                            int rows, int outputs, int inner, int activation_block, const void *input,
                             const void *input_scale, const void *weight, const void *weight_scale,
                             const void *metadata, const void *active, const void *counts, void *out)
 {
+    // Above 64 rows the streaming kernel would read the weights once per 32- or 64-token slab; the
+    // prefill kernel tiles both operands instead (grouped weights come from the device table and
+    // are 16-byte aligned by contract, so only the host-visible pointers are checked here).
+    const void *checked_weight = groups == 0 ? weight : nullptr;
+    if (kernel >= 20)
+        return launch_mx_dma(stream, kernel - 20, packed, groups, weight_groups, rows, outputs, inner,
+                             activation_block, input, input_scale, weight, weight_scale, metadata,
+                             active, counts, out);
+    if (kernel < 0 && rows > 64 && mx_dma_supported(outputs, inner, input, checked_weight, out)) {
+        // 256 x 256 tiles do the most work per byte moved through LDS, 256 x 128 tiles give twice
+        // the workgroups: the large tile when its token extent is used and the chip still fills
+        const long long wide_tiles = static_cast<long long>((outputs + 255) / 256) * ((rows + 255) / 256) *
+                                     (groups > 0 ? groups : 1);
+        const int variant = rows > 256 || (rows > 128 && wide_tiles >= 512) ? 0 : 1;
+        return launch_mx_dma(stream, variant, packed, groups, weight_groups, rows, outputs, inner,
+                             activation_block, input, input_scale, weight, weight_scale, metadata,
+                             active, counts, out);
+    }
     MxParams p;
     p.input = static_cast<const unsigned char *>(input);
     p.input_scale = static_cast<const unsigned char *>(input_scale);
