@@ -113,7 +113,8 @@ def main():
     parser.add_argument("--skip-extras", action="store_true")
     parser.add_argument("--skip-cpu", action="store_true")
     parser.add_argument("--only", choices=("decode1", "decode8", "decode32", "prefill", "copy", "fp8m1", "fp8m16",
-                                 "fp8m256", "fp8m4096", "attention", "layer"),
+                                 "fp8m256", "fp8m4096", "mxe4m3m4096", "mxe2m1m4096", "attention",
+                                 "layer"),
                         help="profiling aid: launch just this kernel --steps times, print nothing")
     args = parser.parse_args()
     if args.gpus != 1:
@@ -256,6 +257,12 @@ def profile_only(args, torch, _kernels, _native, device, normal, weights, inputs
 
         def launch(i):
             _kernels.fp8_block_matmul(a, a_scale, copies[i % rotate], w_scale, out=out)
+    elif args.only.startswith("mx"):
+        packed, tokens, features, inner = args.only.startswith("mxe2m1"), 4096, 18432, 7168
+        w, scale, a, a_scale = mx_operands(torch, device, packed, tokens, features, inner)
+
+        def launch(i):
+            _kernels.quantized_matmul(a, a_scale, w, scale)
     elif args.only in ("attention", "layer"):
         layer, attention = layer_step(torch, _kernels, device, normal)
         launch = (lambda i: layer()) if args.only == "layer" else (lambda i: attention())
@@ -269,6 +276,20 @@ def profile_only(args, torch, _kernels, _native, device, normal, weights, inputs
     for index in range(args.warmup + args.steps):
         launch(index)
     torch.cuda.synchronize()
+
+
+def mx_operands(torch, device, packed, tokens, features, inner):
+    """Random E8M0 block-scaled operands: weights [features, inner] E4M3 (scales per 32 x 32 block) or
+    packed E2M1 (scales per row and 32 inputs), E4M3 tokens with one scale per 32 inputs."""
+    if packed:
+        w = torch.randint(0, 256, (features, inner // 2), device=device, dtype=torch.uint8)
+        scale = torch.randint(120, 130, (features, inner // 32), device=device, dtype=torch.uint8)
+    else:
+        w = torch.randint(0, 0x7E, (features, inner), device=device, dtype=torch.uint8).view(torch.float8_e4m3fn)
+        scale = torch.randint(120, 130, (features // 32, inner // 32), device=device, dtype=torch.uint8)
+    a = torch.randint(0, 0x7E, (tokens, inner), device=device, dtype=torch.uint8).view(torch.float8_e4m3fn)
+    a_scale = torch.randint(120, 130, (tokens, inner // 32), device=device, dtype=torch.uint8)
+    return w, scale, a, a_scale
 
 
 KV_BYTES = 2 * 32 * 2048 * 8 * 128 * 2
@@ -385,6 +406,16 @@ def extras(torch, _kernels, _native, device, normal):
         mx[name] = {"us": round(seconds * 1e6, 1), "gbps": round(traffic / seconds / 1e9, 1),
                     "frac_of_8TBs": round(traffic / seconds / HBM_PEAK, 4)}
     found["mx_quantized_matmul_m16_18432x7168"] = mx
+    # the same products at 4096 tokens (tiled kernel, hardware-scaled matrix instructions)
+    mx = {}
+    for name, packed in (("e4m3", False), ("e2m1", True)):
+        w, scale, a, a_scale = mx_operands(torch, device, packed, 4096, outputs, inner)
+        seconds = event_time(torch, lambda i: _kernels.quantized_matmul(a, a_scale, w, scale), 3, 10)
+        flops = 2.0 * 4096 * outputs * inner
+        mx[name] = {"us": round(seconds * 1e6, 1), "tflops": round(flops / seconds / 1e12, 1),
+                    "frac_of_5PF": round(flops / seconds / FP8_PEAK, 4)}
+        del w, scale, a, a_scale
+    found["mx_quantized_matmul_m4096_18432x7168"] = mx
     del copies, w_scale
     # FP32 SGEMM 2048^3 (plumbing)
     size = 2048

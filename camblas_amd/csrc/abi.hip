@@ -797,10 +797,10 @@ extern "C" int camblas_cuda_quantized_matmul(camblas_cuda_context *context, int 
             output == input_scale || output == weight || output == weight_scale)
             return fail(context, "invalid quantized matrix buffers", 1);
         context->counts[4]++;
-        hipError_t error = launch_mx_matmul(context->stream, context->override_kernel, packed != 0,
-                                            0, 0, rows, outputs, inner, activation_block, input,
-                                            input_scale, weight, weight_scale, nullptr, nullptr,
-                                            nullptr, output);
+        hipError_t error = launch_mx_matmul(context->stream, context->override_kernel,
+                                            context->compute_units, packed != 0, 0, 0, rows,
+                                            outputs, inner, activation_block, input, input_scale,
+                                            weight, weight_scale, nullptr, nullptr, nullptr, output);
         return error == hipSuccess ? 0 : fail(context, "quantized matrix multiplication", error);
     });
 }
@@ -830,10 +830,11 @@ extern "C" int camblas_cuda_grouped_quantized_matmul(camblas_cuda_context *conte
             output == input_scale || output == metadata || output == active || output == counts)
             return fail(context, "invalid grouped matrix buffers", 1);
         context->counts[4]++;
-        hipError_t error = launch_mx_matmul(context->stream, context->override_kernel, packed != 0,
-                                            groups, weight_groups, rows, outputs, inner,
-                                            activation_block, input, input_scale, nullptr, nullptr,
-                                            metadata, active, counts, output);
+        hipError_t error = launch_mx_matmul(context->stream, context->override_kernel,
+                                            context->compute_units, packed != 0, groups,
+                                            weight_groups, rows, outputs, inner, activation_block,
+                                            input, input_scale, nullptr, nullptr, metadata, active,
+                                            counts, output);
         return error == hipSuccess ? 0 : fail(context, "grouped multiplication", error);
     });
 }

@@ -130,8 +130,9 @@ hipError_t launch_fp8_block32_decode(hipStream_t stream, int outputs, int inner,
                                      int sw_row, int sw_col, void *out);
 // E8M0 block-scaled product (E4M3 or packed E2M1 weights); groups == 0 plain, >= 1 grouped.
 // kernel: -1 chooses by shape; 0 the weight-streaming kernel; 20 + v the prefill kernel variant v.
-hipError_t launch_mx_matmul(hipStream_t stream, int kernel, bool packed, int groups, int weight_groups,
-                            int rows, int outputs, int inner, int activation_block, const void *input,
+hipError_t launch_mx_matmul(hipStream_t stream, int kernel, int compute_units, bool packed, int groups,
+                            int weight_groups, int rows, int outputs, int inner,
+                            int activation_block, const void *input,
                             const void *input_scale, const void *weight, const void *weight_scale,
                             const void *metadata, const void *active, const void *counts, void *out);
 // Prefill-sized E8M0 product (hardware-scaled matrix instructions, operands loaded straight into

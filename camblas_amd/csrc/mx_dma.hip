@@ -55,9 +55,10 @@ __device__ __forceinline__ unsigned long long uniform(unsigned long long value)
 }
 
 // WIDE_X: one activation scale per 128 inputs (one byte per step) instead of one per 32
-template <bool PACKED, bool WIDE_X, bool GROUPED, int TN, int TM, int WM, int STAGES>
+template <bool PACKED, bool WIDE_X, bool GROUPED, int TN, int TM, int WM, int STAGES, int RING>
 __global__ __launch_bounds__(128 * WM) void mx_dma_kernel(MxDmaParams p)
 {
+    static_assert(RING >= 2 && RING <= 4, "weight fragments in flight");
     static_assert(STAGES == 2 || STAGES == 3, "two or three LDS stages");
     static_assert(PACKED || !WIDE_X, "128-input activation scales go with E2M1 weights only");
     constexpr int WAVES = 2 * WM, BK = 128;
@@ -266,39 +267,54 @@ __global__ __launch_bounds__(128 * WM) void mx_dma_kernel(MxDmaParams p)
             return fragment8(stage, w_frag_base + tile * 32 * CHW, w_swizzle, ks);
     };
 
-    // One K step, as two halves of 64 inputs: the token fragments of a half are read once, the
-    // weight fragments (one per 32-row tile) one instruction group ahead into the other of two
-    // register buffers; the fills of the stage STAGES-1 ahead are issued between the matrix
-    // instructions.
+    // One K step, as two halves of 64 inputs. LDS reads return long after one or two matrix
+    // instructions have issued, so the weight fragments (one per 32-row tile and half) are read
+    // RING-1 fragments ahead of their use into a ring of register buffers, and the token
+    // fragments of the second half while the first half is multiplied; the fills of the stage
+    // STAGES-1 ahead are issued between the matrix instructions.
     auto multiply = [&](const u32x4_t *stage, u32x4_t *fill, const unsigned (&w_scale)[TN],
                         const unsigned (&x_scale)[TM]) {
-        constexpr int OPS = TN * 2 * TM, SHARE = (LOADS + OPS - 1) / OPS;
-        i32x8_t w_frag[2], x_frag[TM];
-        w_frag[0] = weight_fragment(stage, 0, 0);
+        constexpr int PARTS = TN * 2, OPS = PARTS * TM;
+        static_assert(LOADS <= OPS, "at most one fill per matrix instruction");
+        // (a ring of two leaves no registers for both halves' token fragments: there the second
+        // half's are read into the first half's registers when the first half is done)
+        constexpr int XB = RING > 2 ? 2 : 1;
+        i32x8_t w_frag[RING], x_frag[XB][TM];
+#pragma unroll
+        for (int t = 0; t < TM; ++t)
+            x_frag[0][t] = fragment8(stage, x_frag_base + t * 32 * CHX, x_swizzle, 0);
+#pragma unroll
+        for (int part = 0; part < RING - 1 && part < PARTS; ++part)
+            w_frag[part] = weight_fragment(stage, part % TN, part / TN);
 #pragma unroll
         for (int op = 0; op < OPS; ++op) {
             const int part = op / TM, ks = part / TN, i = part % TN, j = op % TM;
             __builtin_amdgcn_sched_barrier(0);
-            if (op % (TN * TM) == 0) {
+            if (j == 0 && part + RING - 1 < PARTS)
+                w_frag[(part + RING - 1) % RING] =
+                    weight_fragment(stage, (part + RING - 1) % TN, (part + RING - 1) / TN);
+            if (op == (XB == 2 ? TM : OPS / 2)) { // second half's tokens: read during the first half
 #pragma unroll
                 for (int t = 0; t < TM; ++t)
-                    x_frag[t] = fragment8(stage, x_frag_base + t * 32 * CHX, x_swizzle, ks);
+                    x_frag[XB - 1][t] = fragment8(stage, x_frag_base + t * 32 * CHX, x_swizzle, 1);
             }
-            if (j == 0 && part + 1 < TN * 2)
-                w_frag[(part + 1) & 1] = weight_fragment(stage, (part + 1) % TN, (part + 1) / TN);
             __builtin_amdgcn_sched_barrier(0);
             if (ks == 0) // (the byte selects are immediates of the instruction)
                 acc[i][j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(
-                    w_frag[part & 1], x_frag[j], acc[i][j], PACKED ? 4 : 0, 0, 0, int(w_scale[i]), 0,
-                    int(x_scale[j]));
+                    w_frag[part % RING], x_frag[0][j], acc[i][j], PACKED ? 4 : 0, 0, 0, int(w_scale[i]),
+                    0, int(x_scale[j]));
             else
                 acc[i][j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(
-                    w_frag[part & 1], x_frag[j], acc[i][j], PACKED ? 4 : 0, 0, 2, int(w_scale[i]),
+                    w_frag[part % RING], x_frag[XB - 1][j], acc[i][j], PACKED ? 4 : 0, 0, 2, int(w_scale[i]),
                     WIDE_X ? 0 : 2, int(x_scale[j]));
             __builtin_amdgcn_sched_barrier(0);
+            // One fill per matrix instruction from the start of the step; the short steps of the
+            // 128-token tile spread them evenly instead (measured: 10 % faster there, slower for
+            // the long steps).
 #pragma unroll
-            for (int index = op * SHARE; index < (op + 1) * SHARE && index < LOADS; ++index)
-                issue_one(fill, index);
+            for (int index = 0; index < LOADS; ++index)
+                if ((STAGES == 3 && TM == 1 ? index * OPS / LOADS : index) == op)
+                    issue_one(fill, index);
         }
         __builtin_amdgcn_sched_barrier(0);
         advance();
@@ -389,7 +405,7 @@ __global__ __launch_bounds__(128 * WM) void mx_dma_kernel(MxDmaParams p)
     }
 }
 
-template <bool PACKED, bool WIDE_X, bool GROUPED, int TN, int TM, int WM, int STAGES>
+template <bool PACKED, bool WIDE_X, bool GROUPED, int TN, int TM, int WM, int STAGES, int RING>
 hipError_t launch_one(hipStream_t stream, MxDmaParams p, int groups)
 {
     constexpr int BN = 64 * TN, BM = 32 * WM * TM;
@@ -398,24 +414,30 @@ hipError_t launch_one(hipStream_t stream, MxDmaParams p, int groups)
     if (size_t(p.tiles_n) * size_t(p.tiles_m) > 0x7fffffffu || groups > 65535)
         return hipErrorInvalidValue;
     dim3 grid(unsigned(p.tiles_n) * unsigned(p.tiles_m), unsigned(groups));
-    mx_dma_kernel<PACKED, WIDE_X, GROUPED, TN, TM, WM, STAGES><<<grid, 128 * WM, 0, stream>>>(p);
+    mx_dma_kernel<PACKED, WIDE_X, GROUPED, TN, TM, WM, STAGES, RING>
+        <<<grid, 128 * WM, 0, stream>>>(p);
     return launch_status();
 }
 
 // variant 0: 256 weight rows x 256 tokens (two stages for E4M3 weights, three for E2M1);
-// variant 1: 256 x 128, three stages
+// variant 1: 256 x 128, three stages; variant 2: 192 x 256, two stages, E4M3 weights only (a
+// wavefront load covers 16 rows of packed weights: 192 rows are not a whole number of rounds)
 template <bool PACKED, bool WIDE_X, bool GROUPED>
 hipError_t launch_variant(hipStream_t stream, const MxDmaParams &p, int groups, int variant)
 {
     switch (variant) {
-    case 0: return launch_one<PACKED, WIDE_X, GROUPED, 4, 2, 4, PACKED ? 3 : 2>(stream, p, groups);
-    case 1: return launch_one<PACKED, WIDE_X, GROUPED, 4, 1, 4, 3>(stream, p, groups);
+    case 0: return launch_one<PACKED, WIDE_X, GROUPED, 4, 2, 4, PACKED ? 3 : 2, PACKED ? 2 : 3>(stream, p, groups);
+    case 1: return launch_one<PACKED, WIDE_X, GROUPED, 4, 1, 4, 3, 4>(stream, p, groups);
+    case 2:
+        if constexpr (!PACKED)
+            return launch_one<false, false, GROUPED, 3, 2, 4, 2, 3>(stream, p, groups);
+        return hipErrorInvalidValue;
     default: return hipErrorInvalidValue;
     }
 }
 } // namespace
 
-int mx_dma_variant_count() { return 2; }
+int mx_dma_variant_count() { return 3; }
 
 // The prefill kernel's conditions: K a multiple of 128, 16-byte aligned operands, an 8-byte aligned
 // output (scale pointers may have any alignment).

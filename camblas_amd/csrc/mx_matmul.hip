@@ -407,8 +407,9 @@ hipError_t launch_shape(hipStream_t stream, const MxParams &p, int groups)
 
 // groups == 0: plain product (weight, weight_scale given); groups >= 1: grouped product (metadata,
 // active, counts given). activation_block 32 or 128. Weights 16-byte aligned.
-hipError_t launch_mx_matmul(hipStream_t stream, int kernel, bool packed, int groups, int weight_groups,
-                            int rows, int outputs, int inner, int activation_block, const void *input,
+hipError_t launch_mx_matmul(hipStream_t stream, int kernel, int compute_units, bool packed, int groups,
+                            int weight_groups, int rows, int outputs, int inner,
+                            int activation_block, const void *input,
                             const void *input_scale, const void *weight, const void *weight_scale,
                             const void *metadata, const void *active, const void *counts, void *out)
 {
@@ -421,11 +422,16 @@ hipError_t launch_mx_matmul(hipStream_t stream, int kernel, bool packed, int gro
                              activation_block, input, input_scale, weight, weight_scale, metadata,
                              active, counts, out);
     if (kernel < 0 && rows > 64 && mx_dma_supported(outputs, inner, input, checked_weight, out)) {
-        // 256 x 256 tiles do the most work per byte moved through LDS, 256 x 128 tiles give twice
-        // the workgroups: the large tile when its token extent is used and the chip still fills
-        const long long wide_tiles = static_cast<long long>((outputs + 255) / 256) * ((rows + 255) / 256) *
-                                     (groups > 0 ? groups : 1);
-        const int variant = rows > 256 || (rows > 128 && wide_tiles >= 512) ? 0 : 1;
+        // 256 x 256 tiles do the most work per byte moved through LDS; 256 x 128 tiles cost 0.57 of
+        // one (0.6 with packed weights, whose scales are gathered per row) and fill the chip
+        // when the large ones leave compute units idle: the fewer weighted rounds win.
+        const long long batches = groups > 0 ? groups : 1, panels = (outputs + 255) / 256;
+        const long long wide = panels * ((rows + 255) / 256) * batches;
+        const long long narrow = panels * ((rows + 127) / 128) * batches;
+        const double wide_cost = double((wide + compute_units - 1) / compute_units);
+        const double narrow_cost =
+            double((narrow + compute_units - 1) / compute_units) * (packed ? 0.6 : 0.57);
+        const int variant = rows > 128 && wide_cost <= narrow_cost ? 0 : 1;
         return launch_mx_dma(stream, variant, packed, groups, weight_groups, rows, outputs, inner,
                              activation_block, input, input_scale, weight, weight_scale, metadata,
                              active, counts, out);

@@ -148,7 +148,9 @@ int camblas_cuda_reset_stats(camblas_cuda_context *context);
  * is 32 (both) or 128 (E2M1 only). outputs a positive multiple of eight, inner of 32, rows
  * 0..65535. ref: include/camblas_cuda.h:110-123, src/cuda/backend.cu:1165-1191. Runs on the
  * scaled matrix-core instruction of gfx950, which applies the E8M0 scales itself. Input and weight
- * must be 16-byte aligned here (the reference asks for 4 and 2/4). */
+ * must be 16-byte aligned here (the reference asks for 4 and 2/4); the scale arrays may start at
+ * any byte. Up to 64 rows a weight-streaming kernel runs; above that, when inner is a multiple of
+ * 128 and the output is 8-byte aligned, a kernel that tiles both operands through LDS. */
 int camblas_cuda_quantized_matmul(camblas_cuda_context *context, int packed, int rows, int outputs,
                                   int inner, int activation_block, const void *input,
                                   const void *input_scale, const void *weight,
@@ -270,7 +272,10 @@ int camblas_hip_plan_describe(int dtype, int algorithm, char trans_a, char trans
                               int k, int lda, int ldb, int ldc, int aligned16, char *text,
                               size_t text_bytes);
 /* extension. Diagnostics for tests and tuning: force the planner's choice for BF16/FP8 GEMMs on
- * this context (kernel < 0 restores the planner; split_k <= 0 lets the planner choose). */
+ * this context (kernel < 0 restores the planner; split_k <= 0 lets the planner choose). For the
+ * E8M0 products: 0 the weight-streaming kernel, 20 / 21 / 22 the tiled kernel with 256 x 256,
+ * 256 x 128 and (E4M3 weights only) 192 x 256 tiles; a forced kernel that cannot run the call
+ * makes the call fail. */
 int camblas_hip_set_plan_override(camblas_cuda_context *context, int kernel, int split_k);
 /* extension. Diagnostics: copies `bytes` (a multiple of 16, 16-byte aligned buffers) with a plain
  * grid-stride kernel. A launch of known HBM traffic (bytes read + bytes written) against which
