@@ -367,14 +367,15 @@ template <bool PACKED, bool GROUPED>
 hipError_t launch_shape(hipStream_t stream, const MxParams &p, int groups)
 {
     // token tiles by row count; weight-row tiles so that about one workgroup lands on each compute
-    // unit (decode-sized calls: the kernel is bound by the weight stream)
+    // unit, all groups counted (decode-sized calls: the kernel is bound by the weight stream, and a
+    // workgroup of few rows spends most of its time in its fixed start and end)
     // (E2M1 steps hold twice the input tiles: four token tiles would not fit the register file)
     const int token_tiles = p.rows <= 16 ? 1 : p.rows <= 32 || PACKED ? 2 : 4;
     const int tiles = (p.outputs + 15) / 16;
     int row_tiles = 1;
     const int most = PACKED ? (token_tiles == 2 ? 6 : 8) : (token_tiles == 4 ? 4 : 8);
     for (int candidate = most; candidate > 1; --candidate)
-        if (tiles / candidate >= 192) {
+        if (static_cast<long long>(tiles / candidate) * groups >= 192) {
             row_tiles = candidate;
             break;
         }
@@ -413,25 +414,29 @@ hipError_t launch_mx_matmul(hipStream_t stream, int kernel, int compute_units, b
                             const void *input_scale, const void *weight, const void *weight_scale,
                             const void *metadata, const void *active, const void *counts, void *out)
 {
-    // Above 64 rows the streaming kernel would read the weights once per 32- or 64-token slab; the
-    // prefill kernel tiles both operands instead (grouped weights come from the device table and
-    // are 16-byte aligned by contract, so only the host-visible pointers are checked here).
+    // Above 32 rows the streaming kernel reads the weights once per 32-token slab; the tiled kernel
+    // reads them once per 128 or 256 tokens (grouped weights come from the device table and are
+    // 16-byte aligned by contract, so only the host-visible pointers are checked here). Measured
+    // crossover: 33 rows, except a single product with packed weights (65).
     const void *checked_weight = groups == 0 ? weight : nullptr;
     if (kernel >= 20)
         return launch_mx_dma(stream, kernel - 20, packed, groups, weight_groups, rows, outputs, inner,
                              activation_block, input, input_scale, weight, weight_scale, metadata,
                              active, counts, out);
-    if (kernel < 0 && rows > 64 && mx_dma_supported(outputs, inner, input, checked_weight, out)) {
-        // 256 x 256 tiles do the most work per byte moved through LDS; 256 x 128 tiles cost 0.57 of
-        // one (0.6 with packed weights, whose scales are gathered per row) and fill the chip
-        // when the large ones leave compute units idle: the fewer weighted rounds win.
-        const long long batches = groups > 0 ? groups : 1, panels = (outputs + 255) / 256;
-        const long long wide = panels * ((rows + 255) / 256) * batches;
-        const long long narrow = panels * ((rows + 127) / 128) * batches;
-        const double wide_cost = double((wide + compute_units - 1) / compute_units);
-        const double narrow_cost =
-            double((narrow + compute_units - 1) / compute_units) * (packed ? 0.6 : 0.57);
-        const int variant = rows > 128 && wide_cost <= narrow_cost ? 0 : 1;
+    const int most_streamed = packed && groups <= 1 ? 64 : 32;
+    if (kernel < 0 && rows > most_streamed &&
+        mx_dma_supported(outputs, inner, input, checked_weight, out)) {
+        // 256 x 256 tiles do the most work per byte moved through LDS; a 256 x 128 tile costs 0.57
+        // of one (0.6 with packed weights, whose scales are gathered per row), a 192 x 256 tile
+        // (E4M3 weights) 0.84, and the smaller tiles fill the chip when the large ones leave
+        // compute units idle: the fewest weighted rounds win.
+        const long long batches = groups > 0 ? groups : 1, token_tiles = (rows + 255) / 256;
+        auto rounds = [&](long long tiles) { return double((tiles * batches + compute_units - 1) / compute_units); };
+        const double wide = rows > 128 ? rounds((outputs + 255) / 256 * token_tiles) : 1e30;
+        const double narrow = rounds(static_cast<long long>((outputs + 255) / 256) * ((rows + 127) / 128)) *
+                              (packed ? 0.6 : 0.57);
+        const double flat = rows > 128 && !packed ? rounds((outputs + 191) / 192 * token_tiles) * 0.84 : 1e30;
+        const int variant = wide <= narrow && wide <= flat ? 0 : flat < narrow ? 2 : 1;
         return launch_mx_dma(stream, variant, packed, groups, weight_groups, rows, outputs, inner,
                              activation_block, input, input_scale, weight, weight_scale, metadata,
                              active, counts, out);

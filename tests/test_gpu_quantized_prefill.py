@@ -1,4 +1,4 @@
-"""E8M0 block-scaled products at prefill row counts (more than 64 rows: the tiled kernel that uses
+"""E8M0 block-scaled products at prefill row counts (more than 32 rows: the tiled kernel that uses
 the matrix cores' hardware scales), through the C ABI, against the independent FP64 byte decoder
 of the oracle. Strategy of the reference's tests/test_quantized.py:110-158 and :243-320 (every
 operand mutated separately, scale extremes and NaN, grouped weights with clipped counts), plus
@@ -66,13 +66,15 @@ def close(got, x, sx, weight, sw, packed, block):
     assert np.linalg.norm(got - want) <= 4e-3 * np.linalg.norm(want)
 
 
-@pytest.mark.parametrize("kernel", ["auto", "tile256x256", "tile256x128", "tile192x256"])
-@pytest.mark.parametrize("packed,block", [(False, 32), (True, 32), (True, 128)])
-@pytest.mark.parametrize("rows,outputs,inner", [(65, 264, 256), (128, 520, 384), (300, 776, 1024),
-                                               (513, 40, 128)])
+# (the 192-row tile exists for E4M3 weights only)
+FORMATS = [(kernel, packed, block) for kernel in ("auto", "tile256x256", "tile256x128", "tile192x256")
+           for packed, block in ((False, 32), (True, 32), (True, 128)) if not (packed and kernel == "tile192x256")]
+
+
+@pytest.mark.parametrize("kernel,packed,block", FORMATS)
+@pytest.mark.parametrize("rows,outputs,inner", [(33, 264, 256), (65, 264, 256), (128, 520, 384),
+                                               (300, 776, 1024), (513, 40, 128)])
 def test_random_operands_and_individual_mutations(device, kernel, packed, block, rows, outputs, inner):
-    if packed and kernel == "tile192x256":
-        pytest.skip("the 192-row tile exists for E4M3 weights only")
     x, sx, weight, sw = operands(900 + rows, rows, outputs, inner, packed, block)
     for changed in ("original", "input", "weight", "input_scale", "weight_scale"):
         if changed == "input":
@@ -88,12 +90,9 @@ def test_random_operands_and_individual_mutations(device, kernel, packed, block,
         close(run(device, x, sx, weight, sw, packed, block, kernel), x, sx, weight, sw, packed, block)
 
 
-@pytest.mark.parametrize("kernel", ["tile256x256", "tile256x128", "tile192x256"])
-@pytest.mark.parametrize("packed,block", [(False, 32), (True, 32), (True, 128)])
+@pytest.mark.parametrize("kernel,packed,block", [f for f in FORMATS if f[0] != "auto"])
 @pytest.mark.parametrize("shifts", [(0, 0), (1, 3), (2, 1), (3, 2)])
 def test_exact_products_with_every_scale_alignment(device, kernel, packed, block, shifts):
-    if packed and kernel == "tile192x256":
-        pytest.skip("the 192-row tile exists for E4M3 weights only")
     # Inputs in {0, +-0.5, +-1, +-2}, weights in {0, +-0.5 .. +-2} (E2M1: any nibble up to 2), scales
     # 2^-2 .. 2^2 drawn per block: every product is a multiple of 2^-6 below 2^6 and a sum of 640 of
     # them is exact in FP32, so the result must be the BF16 rounding of the exact product, and a
