@@ -426,6 +426,22 @@ def extras(torch, _kernels, _native, device, normal):
     found["fp32_sgemm_2048"] = {"us": round(seconds * 1e6, 1),
                                 "tflops": round(2.0 * size**3 / seconds / 1e12, 2),
                                 "frac_of_157TF": round(2.0 * size**3 / seconds / FP32_PEAK, 4)}
+    # FP64 DGEMM 4096^3 (plumbing), through the C entry point
+    import ctypes as ct
+
+    size = 4096
+    a64 = torch.rand((size, size), device=device, dtype=torch.float64) * 2 - 1
+    b64 = torch.rand((size, size), device=device, dtype=torch.float64) * 2 - 1
+    c64 = torch.empty((size, size), device=device, dtype=torch.float64)
+    native = _native.context(device)
+    seconds = event_time(
+        torch, lambda i: native.call("dgemm", b"N", b"N", size, size, size, ct.c_double(1.0),
+                                     ct.c_void_p(a64.data_ptr()), size, ct.c_void_p(b64.data_ptr()), size,
+                                     ct.c_double(0.0), ct.c_void_p(c64.data_ptr()), size), 2, 5)
+    found["fp64_dgemm_4096"] = {"us": round(seconds * 1e6, 1),
+                                "tflops": round(2.0 * size**3 / seconds / 1e12, 2),
+                                "frac_of_78.6TF": round(2.0 * size**3 / seconds / 78.6e12, 4)}
+    del a64, b64, c64
     # decoder-layer decode step (Llama-3.1-70B shapes, batch 32, KV context 2048)
     step, attention = layer_step(torch, _kernels, device, normal)
 

@@ -34,7 +34,7 @@ CORE_SOURCES = (
     "fp8_block32.hip",
     "mx_matmul.hip",
     "mx_dma.hip",
-    "routing.hip", "dense_ops.hip", "sgemm_mfma.hip",
+    "routing.hip", "dense_ops.hip", "sgemm_mfma.hip", "dgemm_mfma.hip",
     "fusion.hip",
     "attention_decode.hip",
 )

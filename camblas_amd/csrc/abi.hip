@@ -221,8 +221,8 @@ int dense_gemm(camblas_cuda_context *context, char ta, char tb, int m, int n, in
         });
 }
 
-// ref: src/cuda/backend.cu:1066-1073; FP64 has no matrix-core path here, every layout runs the
-// LDS-tiled FMA kernel
+// ref: src/cuda/backend.cu:1066-1073; products with at least one 16 x 16 x 4 matrix-core tile in
+// every dimension run on the matrix cores, smaller ones on the LDS-tiled FMA kernel
 int dense_gemm(camblas_cuda_context *context, char ta, char tb, int m, int n, int k, double alpha,
                const double *a, int lda, const double *b, int ldb, double beta, double *c, int ldc)
 {
@@ -231,8 +231,14 @@ int dense_gemm(camblas_cuda_context *context, char ta, char tb, int m, int n, in
         [&] { return launch_scale_f64(context->stream, m, n, beta, c, ldc); },
         [&](bool trans_a, bool trans_b) {
             context->counts[0]++;
-            hipError_t error = launch_generic_f64(context->stream, trans_a, trans_b, m, n, k, alpha,
-                                                  a, lda, b, ldb, beta, c, ldc);
+            bool matrix = m >= 16 && n >= 16 && k >= 4;
+            if (context->override_kernel >= 0) // diagnostics: 0 vector-ALU tiles, else matrix-core tiles
+                matrix = context->override_kernel >= 1;
+            hipError_t error =
+                matrix ? launch_dgemm_mfma(context->stream, trans_a, trans_b, m, n, k, alpha, a, lda, b,
+                                           ldb, beta, c, ldc)
+                       : launch_generic_f64(context->stream, trans_a, trans_b, m, n, k, alpha, a, lda,
+                                            b, ldb, beta, c, ldc);
             return error == hipSuccess ? 0 : fail(context, "classical FP64 GEMM", error);
         });
 }

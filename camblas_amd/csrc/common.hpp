@@ -89,6 +89,9 @@ hipError_t launch_generic_f32(hipStream_t stream, bool ta, bool tb, int m, int n
 hipError_t launch_sgemm_mfma(hipStream_t stream, bool wide, bool ta, bool tb, int m, int n, int k,
                              float alpha, const float *a, int lda, const float *b, int ldb, float beta,
                              float *c, int ldc);
+hipError_t launch_dgemm_mfma(hipStream_t stream, bool ta, bool tb, int m, int n, int k, double alpha,
+                             const double *a, int lda, const double *b, int ldb, double beta, double *c,
+                             int ldc);
 hipError_t launch_generic_bf16(hipStream_t stream, bool ta, bool tb, int m, int n, int k,
                                float alpha, const void *a, int lda, const void *b, int ldb,
                                float beta, void *c, int ldc);

@@ -1,0 +1,143 @@
+// FP64 column-major GEMM on the matrix cores: C = alpha * op(A) op(B) + beta * C for any transpose,
+// leading dimension and alignment (v_mfma_f64_16x16x4_f64: IEEE double multiply-add).
+// Contract: ref src/cuda/backend.cu:1066-1073 (validation is done by the caller in abi.hip).
+//
+// The structure of the FP32 kernel with the shapes of the FP64 instruction: a workgroup of four
+// wavefronts owns a 128 x 128 tile of C, a wavefront 64 x 64 of it as 4 x 4 tiles of 16 x 16 (64
+// accumulator doubles per lane). K is walked 16 deep: the operands of a step are loaded
+// element-wise with bounds checks (every layout and ragged edge), kept in registers while the
+// previous step is multiplied, and laid out in LDS so that the operand reads (lane -> row lane%16,
+// K index lane/16) do not collide: K-major [16][128+16] for an operand whose rows are contiguous
+// in memory, row-major [128][17] for a transposed one.
+#include "common.hpp"
+#include "device.hpp"
+
+namespace camblas_hip
+{
+namespace
+{
+typedef double f64x4_t __attribute__((ext_vector_type(4)));
+
+constexpr int TILE = 128, DEPTH = 16, THREADS = 256;
+constexpr int K_MAJOR_PITCH = TILE + 16, ROW_MAJOR_PITCH = DEPTH + 1;
+constexpr int TILE_WORDS = DEPTH * K_MAJOR_PITCH; // >= TILE * ROW_MAJOR_PITCH
+static_assert(TILE * ROW_MAJOR_PITCH <= TILE_WORDS, "one buffer serves both layouts");
+
+// LDS index of element (row r of the tile, K index l) of an operand; CONTIGUOUS_K: K is the
+// contiguous index in memory (a transposed A, an untransposed B)
+template <bool CONTIGUOUS_K> __device__ __forceinline__ int lds_index(int r, int l)
+{
+    return CONTIGUOUS_K ? r * ROW_MAJOR_PITCH + l : l * K_MAJOR_PITCH + r;
+}
+
+template <bool TA, bool TB>
+__global__ __launch_bounds__(THREADS, 2) void dgemm_mfma_kernel(int m, int n, int k, double alpha,
+                                                             const double *a, int lda, const double *b,
+                                                             int ldb, double beta, double *c, int ldc)
+{
+    __shared__ double tile_a[TILE_WORDS];
+    __shared__ double tile_b[TILE_WORDS];
+    const int thread = threadIdx.x, lane = thread % 64, wave = thread / 64;
+    constexpr int PER_THREAD = TILE * DEPTH / THREADS;
+    const int row0 = blockIdx.x * TILE, col0 = blockIdx.y * TILE;
+    // A(i, l) is a[i + l*lda] ('N', rows contiguous) or a[l + i*lda] ('T', K contiguous);
+    // B(l, j) is b[l + j*ldb] ('N', K contiguous) or b[j + l*ldb] ('T', columns contiguous).
+    // Element e of a step goes to the thread so that consecutive threads read consecutive memory.
+    double next_a[PER_THREAD], next_b[PER_THREAD];
+    auto fetch = [&](int l0) {
+#pragma unroll
+        for (int s = 0; s < PER_THREAD; ++s) {
+            const int e = s * THREADS + thread;
+            const int ai = TA ? e / DEPTH : e % TILE, al = TA ? e % DEPTH : e / TILE;
+            const int gi = row0 + ai, gl = l0 + al;
+            next_a[s] = gi < m && gl < k ? (TA ? a[gl + size_t(gi) * lda] : a[gi + size_t(gl) * lda]) : 0.0;
+            const int bj = TB ? e % TILE : e / DEPTH, bl = TB ? e / TILE : e % DEPTH;
+            const int gj = col0 + bj, hl = l0 + bl;
+            next_b[s] = gj < n && hl < k ? (TB ? b[gj + size_t(hl) * ldb] : b[hl + size_t(gj) * ldb]) : 0.0;
+        }
+    };
+    auto stash = [&]() {
+#pragma unroll
+        for (int s = 0; s < PER_THREAD; ++s) {
+            const int e = s * THREADS + thread;
+            const int ai = TA ? e / DEPTH : e % TILE, al = TA ? e % DEPTH : e / TILE;
+            tile_a[lds_index<TA>(ai, al)] = next_a[s];
+            const int bj = TB ? e % TILE : e / DEPTH, bl = TB ? e / TILE : e % DEPTH;
+            tile_b[lds_index<!TB>(bj, bl)] = next_b[s];
+        }
+    };
+
+    const int wave_i = (wave % 2) * 64, wave_j = (wave / 2) * 64;
+    const int frag_row = lane % 16, frag_k = lane / 16;
+    f64x4_t acc[4][4];
+#pragma unroll
+    for (int x = 0; x < 4; ++x)
+#pragma unroll
+        for (int y = 0; y < 4; ++y)
+            acc[x][y] = f64x4_t{0.0, 0.0, 0.0, 0.0};
+
+    fetch(0);
+    for (int l0 = 0; l0 < k; l0 += DEPTH) {
+        stash();
+        __syncthreads();
+        if (l0 + DEPTH < k)
+            fetch(l0 + DEPTH);
+#pragma unroll
+        for (int s = 0; s < DEPTH / 4; ++s) {
+            double av[4], bv[4];
+#pragma unroll
+            for (int x = 0; x < 4; ++x)
+                av[x] = tile_a[lds_index<TA>(wave_i + x * 16 + frag_row, 4 * s + frag_k)];
+#pragma unroll
+            for (int y = 0; y < 4; ++y)
+                bv[y] = tile_b[lds_index<!TB>(wave_j + y * 16 + frag_row, 4 * s + frag_k)];
+#pragma unroll
+            for (int x = 0; x < 4; ++x)
+#pragma unroll
+                for (int y = 0; y < 4; ++y)
+                    acc[x][y] = __builtin_amdgcn_mfma_f64_16x16x4f64(av[x], bv[y], acc[x][y], 0, 0, 0);
+        }
+        __syncthreads();
+    }
+
+    // accumulator element e of lane l: row 4*e + l/16, column l%16 of the 16 x 16 tile (found with
+    // an identity product; the FP32 16 x 16 instructions use 4*(l/16) + e instead)
+#pragma unroll
+    for (int y = 0; y < 4; ++y) {
+        const int j = col0 + wave_j + y * 16 + frag_row;
+        if (j >= n)
+            continue;
+#pragma unroll
+        for (int x = 0; x < 4; ++x) {
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                const int i = row0 + wave_i + x * 16 + 4 * e + frag_k;
+                if (i >= m)
+                    continue;
+                double *out = c + i + size_t(j) * ldc;
+                const double value = alpha * acc[x][y][e];
+                *out = beta != 0.0 ? fma(beta, *out, value) : value;
+            }
+        }
+    }
+}
+} // namespace
+
+hipError_t launch_dgemm_mfma(hipStream_t stream, bool ta, bool tb, int m, int n, int k, double alpha,
+                             const double *a, int lda, const double *b, int ldb, double beta, double *c,
+                             int ldc)
+{
+    dim3 grid((m + TILE - 1) / TILE, (n + TILE - 1) / TILE);
+    if (grid.y > 65535u)
+        return hipErrorInvalidValue;
+    if (!ta && !tb)
+        dgemm_mfma_kernel<false, false><<<grid, THREADS, 0, stream>>>(m, n, k, alpha, a, lda, b, ldb, beta, c, ldc);
+    else if (!ta && tb)
+        dgemm_mfma_kernel<false, true><<<grid, THREADS, 0, stream>>>(m, n, k, alpha, a, lda, b, ldb, beta, c, ldc);
+    else if (ta && !tb)
+        dgemm_mfma_kernel<true, false><<<grid, THREADS, 0, stream>>>(m, n, k, alpha, a, lda, b, ldb, beta, c, ldc);
+    else
+        dgemm_mfma_kernel<true, true><<<grid, THREADS, 0, stream>>>(m, n, k, alpha, a, lda, b, ldb, beta, c, ldc);
+    return launch_status();
+}
+} // namespace camblas_hip

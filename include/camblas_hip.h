@@ -68,7 +68,8 @@ int camblas_cuda_bgemm(camblas_cuda_context *context, char trans_a, char trans_b
                        float beta, void *c, int ldc);
 
 /* Same contract in FP64 (ref: include/camblas_cuda.h:60-62, src/cuda/backend.cu:1066-1073):
- * LDS-tiled FMA kernel for every layout, no matrix-core path. */
+ * FP64 matrix-core tiles for every layout (IEEE double multiply-add); products with m or n below
+ * 16 run an LDS-tiled FMA kernel. */
 int camblas_cuda_dgemm(camblas_cuda_context *context, char trans_a, char trans_b, int m, int n,
                        int k, double alpha, const double *a, int lda, const double *b, int ldb,
                        double beta, double *c, int ldc);

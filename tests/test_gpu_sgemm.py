@@ -166,20 +166,32 @@ def test_invalid_arguments_report_errors(device):
     assert b"missing affine operand" in lib.camblas_cuda_error(native.handle)
 
 
+def run_dgemm(device, ta, tb, m, n, k, alpha, a, lda, b, ldb, beta, c, ldc, kernel="planner"):
+    at, bt, ct_ = (torch.from_numpy(v).to(device) for v in (a, b, c))
+    native = _native.context(device)
+    native.call("hip_set_plan_override", KERNEL[kernel], 0)
+    try:
+        native.call("dgemm", ta.encode(), tb.encode(), m, n, k, ct.c_double(alpha), ptr(at), lda,
+                    ptr(bt), ldb, ct.c_double(beta), ptr(ct_), ldc)
+    finally:
+        native.call("hip_set_plan_override", -1, 0)
+    torch.cuda.synchronize()
+    return ct_.cpu().numpy()
+
+
+@pytest.mark.parametrize("kernel", ["planner", "vector", "matrix"])
 @pytest.mark.parametrize("ta", "NT")
 @pytest.mark.parametrize("tb", "NT")
-def test_dgemm_matches_float64_product(device, ta, tb):
+@pytest.mark.parametrize("shape", [(67, 45, 130), (16, 16, 4), (129, 257, 19), (300, 140, 64)])
+def test_dgemm_matches_float64_product(device, kernel, ta, tb, shape):
     # FP64 storage and accumulation: the only difference from numpy's product is summation order
-    m, n, k = 67, 45, 130
+    # (vector: LDS-tiled FMA kernel; matrix: v_mfma_f64_16x16x4 tiles; the planner picks by size)
+    m, n, k = shape
     lda, ldb, ldc = (m if ta == "N" else k) + 1, (k if tb == "N" else n) + 2, m + 3
     a = oracle.fill_uniform(31, (lda * (k if ta == "N" else m),)).astype(np.float64)
     b = oracle.fill_uniform(32, (ldb * (n if tb == "N" else k),)).astype(np.float64)
     c0 = oracle.fill_uniform(33, (ldc * n,)).astype(np.float64)
-    at, bt, ct_ = (torch.from_numpy(v).to(device) for v in (a, b, c0.copy()))
-    _native.context(device).call("dgemm", ta.encode(), tb.encode(), m, n, k, ct.c_double(0.75),
-                                 ptr(at), lda, ptr(bt), ldb, ct.c_double(-2.0), ptr(ct_), ldc)
-    torch.cuda.synchronize()
-    got = ct_.cpu().numpy().reshape(n, ldc)
+    got = run_dgemm(device, ta, tb, m, n, k, 0.75, a, lda, b, ldb, -2.0, c0.copy(), ldc, kernel).reshape(n, ldc)
     left = a.reshape(-1, lda)[:, : (m if ta == "N" else k)]   # column-major storage, rows = columns
     left = left.T if ta == "N" else left                       # -> [m, k]
     right = b.reshape(-1, ldb)[:, : (k if tb == "N" else n)]
@@ -187,6 +199,17 @@ def test_dgemm_matches_float64_product(device, ta, tb):
     want = 0.75 * (left @ right) - 2.0 * c0.reshape(n, ldc)[:, :m].T
     assert rel_frobenius(got[:, :m].T, want) <= 1e-13
     assert np.array_equal(got[:, m:], c0.reshape(n, ldc)[:, m:])
+
+
+@pytest.mark.parametrize("kernel", ["vector", "matrix"])
+def test_dgemm_beta_zero_ignores_nan_and_keeps_full_precision(device, kernel):
+    # beta = 0 must not read C; 1 + 2^-40 squared keeps its 2^-39 term only in full FP64 arithmetic
+    m, n, k = 48, 33, 20
+    a = np.full(m * k, 1.0 + 2.0 ** -40)
+    b = np.full(k * n, 1.0 + 2.0 ** -40)
+    c = np.full(m * n, np.nan)
+    got = run_dgemm(device, "N", "N", m, n, k, 1.0, a, m, b, k, 0.0, c, m, kernel)
+    assert np.array_equal(got, np.full(m * n, k * (1.0 + 2.0 ** -39 + 2.0 ** -80)))
 
 
 @pytest.mark.parametrize("kernel", ["vector", "matrix", "matrix64"])
