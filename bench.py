@@ -426,14 +426,32 @@ def extras(torch, _kernels, _native, device, normal):
     found["fp32_sgemm_2048"] = {"us": round(seconds * 1e6, 1),
                                 "tflops": round(2.0 * size**3 / seconds / 1e12, 2),
                                 "frac_of_157TF": round(2.0 * size**3 / seconds / FP32_PEAK, 4)}
-    # FP64 DGEMM 4096^3 (plumbing), through the C entry point
+    # what the matrix cores sustain: independent matrix instructions with no memory traffic (the
+    # part's clock under matrix load included), the ceiling the prefill rates are read against
     import ctypes as ct
+
+    native = _native.context(device)
+    sink = torch.empty(4096 * 512, dtype=torch.float32, device=device)
+    flops = ct.c_double(0.0)
+    sustained = {}
+    # (rounds sized for launches of 2-3 ms, long enough for the clock to settle)
+    for name, kind, rounds in (("bf16_32x32x16", 0, 16000), ("e4m3_scaled_32x32x64", 1, 8000),
+                               ("e2m1_x_e4m3_scaled_32x32x64", 2, 8000), ("fp32_32x32x2", 3, 8000)):
+        entry = {}
+        for operands, constant in (("varied", 0), ("constant", 1)):
+            seconds = event_time(
+                torch, lambda i: native.call("hip_matrix_probe", kind, rounds, constant,
+                                             ct.c_void_p(sink.data_ptr()), sink.numel() * 4, ct.byref(flops)),
+                2, 5)
+            entry[operands + "_operands_tflops"] = round(flops.value / seconds / 1e12, 1)
+        sustained[name] = entry
+    found["matrix_instruction_issue_rate"] = sustained
+    # FP64 DGEMM 4096^3 (plumbing), through the C entry point
 
     size = 4096
     a64 = torch.rand((size, size), device=device, dtype=torch.float64) * 2 - 1
     b64 = torch.rand((size, size), device=device, dtype=torch.float64) * 2 - 1
     c64 = torch.empty((size, size), device=device, dtype=torch.float64)
-    native = _native.context(device)
     seconds = event_time(
         torch, lambda i: native.call("dgemm", b"N", b"N", size, size, size, ct.c_double(1.0),
                                      ct.c_void_p(a64.data_ptr()), size, ct.c_void_p(b64.data_ptr()), size,

@@ -36,6 +36,7 @@ CORE_SOURCES = (
     "mx_dma.hip",
     "routing.hip", "dense_ops.hip", "sgemm_mfma.hip", "dgemm_mfma.hip",
     "fusion.hip",
+    "probes.hip",
     "attention_decode.hip",
 )
 

@@ -1120,6 +1120,21 @@ extern "C" int camblas_hip_copy_probe(camblas_cuda_context *context, size_t byte
     });
 }
 
+extern "C" int camblas_hip_matrix_probe(camblas_cuda_context *context, int kind, int rounds,
+                                        int constant_operands, void *sink, size_t sink_bytes,
+                                        double *flops)
+{
+    return execute(context, [&] {
+        const size_t needed = size_t(context->compute_units) * 512 * sizeof(float);
+        if (kind < 0 || kind > 3 || rounds < 1 || !sink || !flops || !aligned(sink, 4) ||
+            sink_bytes < needed)
+            return fail(context, "invalid matrix probe arguments", 1);
+        hipError_t error = launch_matrix_probe(context->stream, kind, context->compute_units, rounds,
+                                               constant_operands != 0, static_cast<float *>(sink), flops);
+        return error == hipSuccess ? 0 : fail(context, "matrix probe", error);
+    });
+}
+
 extern "C" int camblas_hip_kernel_count(int dtype)
 {
     return dtype == 2 ? tn_variant_count() : dtype == 3 ? fp8_variant_count() : 1;

@@ -178,6 +178,10 @@ hipError_t launch_rms_scale(hipStream_t stream, int dtype, uint64_t count, int w
 hipError_t launch_kv_append(hipStream_t stream, int batch, int kv_heads, int dim, int context_length,
                             const int32_t *positions, const void *k_new, const void *v_new,
                             int token_stride, void *k_cache, void *v_cache);
+// kind: 0 BF16 32x32x16, 1 E4M3 x E4M3 and 2 E2M1 x E4M3 scaled 32x32x64, 3 FP32 32x32x2; one
+// workgroup of eight wavefronts per entry of `workgroups`, rounds * 8 instructions per wavefront.
+hipError_t launch_matrix_probe(hipStream_t stream, int kind, int workgroups, int rounds, int constant,
+                               float *sink, double *flops);
 hipError_t launch_copy_probe(hipStream_t stream, size_t bytes, const void *source, void *destination);
 hipError_t launch_rope_kv_append(hipStream_t stream, int batch, int q_heads, int kv_heads, int dim,
                                  int token_stride, float theta, const int32_t *positions, void *qkv,

@@ -148,3 +148,32 @@ print('ok')
     result = subprocess.run([sys.executable, "-c", code], cwd=ROOT, capture_output=True, text=True,
                             timeout=120)
     assert result.returncode == 0 and "ok" in result.stdout, result.stdout + result.stderr
+
+
+@pytest.mark.parametrize("kind,per_round", [(0, 16.0), (1, 64.0), (2, 48.0), (3, 2.0)])
+def test_matrix_probe_counts_its_work(device, kind, per_round):
+    # the calibration launch for the matrix cores: with the value 1 in every operand lane each
+    # accumulator element grows by the instruction's K per round (E2M1 reads the byte 0x38 as the
+    # nibbles -0 and 1.5: 32 * 1.5), so a lane's sum over 8 accumulators x 16 elements is exact,
+    # and the reported operation count is compute units * 8 wavefronts * rounds * 8 instructions
+    import ctypes as ct
+
+    native, lib = _native.context(device), _native.library()
+    units = torch.cuda.get_device_properties(device).multi_processor_count
+    sink = torch.zeros(units * 512, dtype=torch.float32, device=device)
+    flops = ct.c_double(0.0)
+    rounds = 25
+    native.call("hip_matrix_probe", kind, rounds, 1, ct.c_void_p(sink.data_ptr()), sink.numel() * 4, ct.byref(flops))
+    torch.cuda.synchronize()
+    assert (sink == 128 * rounds * per_round).all()
+    k = {0: 16, 1: 64, 2: 64, 3: 2}[kind]
+    assert flops.value == 2.0 * 32 * 32 * k * units * 8 * rounds * 8
+    native.call("hip_matrix_probe", kind, rounds, 0, ct.c_void_p(sink.data_ptr()), sink.numel() * 4, ct.byref(flops))
+    torch.cuda.synchronize()
+    assert torch.isfinite(sink).all() and (sink != 0).any()
+    status = lib.camblas_cuda_error  # (error text after a refused call)
+    assert lib.camblas_hip_matrix_probe(native.handle, 9, rounds, 0, ct.c_void_p(sink.data_ptr()),
+                                        sink.numel() * 4, ct.byref(flops)) == -1
+    assert b"invalid matrix probe arguments" in status(native.handle)
+    assert lib.camblas_hip_matrix_probe(native.handle, 0, rounds, 0, ct.c_void_p(sink.data_ptr()), 16,
+                                        ct.byref(flops)) == -1
