@@ -426,6 +426,25 @@ def extras(torch, _kernels, _native, device, normal):
     found["fp32_sgemm_2048"] = {"us": round(seconds * 1e6, 1),
                                 "tflops": round(2.0 * size**3 / seconds / 1e12, 2),
                                 "frac_of_157TF": round(2.0 * size**3 / seconds / FP32_PEAK, 4)}
+    # single-token FP8 expert step at the shapes of the reference's hook: 9 of 289 experts, gate/up
+    # [1024, 4096] and down [4096, 512] per expert; the chosen experts rotate so that weights come from HBM
+    experts, hidden, width, choices = 289, 4096, 512, 9
+    w1 = torch.randint(0, 0x7E, (experts, 2 * width, hidden), device=device, dtype=torch.uint8).view(torch.float8_e4m3fn)
+    w2 = torch.randint(0, 0x7E, (experts, hidden, width), device=device, dtype=torch.uint8).view(torch.float8_e4m3fn)
+    s1 = torch.rand((experts, 2 * width // 128, hidden // 128), device=device) * 0.001 + 0.001
+    s2 = torch.rand((experts, hidden // 128, width // 128), device=device) * 0.001 + 0.001
+    token = normal((1, hidden))
+    routing = torch.linspace(0.05, 1.0, choices, device=device)
+    chosen = [torch.arange(choices * i, choices * i + choices, device=device, dtype=torch.int32) for i in range(32)]
+    result = torch.empty((1, hidden), dtype=torch.bfloat16, device=device)
+    seconds = event_time(
+        torch, lambda i: _kernels.fp8_moe_decode(token, w1, w2, s1, s2, chosen[i % 32], routing, factor=2.5,
+                                                 out=result), 10, 40)
+    traffic = choices * (2 * width * hidden + hidden * width)
+    found["fp8_moe_decode_9_of_289_experts"] = {
+        "us": round(seconds * 1e6, 1), "gbps": round(traffic / seconds / 1e9, 1),
+        "note": "two launches; bound by launch and latency, not bandwidth"}
+    del w1, w2, s1, s2
     # what the matrix cores sustain: independent matrix instructions with no memory traffic (the
     # part's clock under matrix load included), the ceiling the prefill rates are read against
     import ctypes as ct

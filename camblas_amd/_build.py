@@ -32,6 +32,7 @@ CORE_SOURCES = (
     "fp8_dma.hip",
     "fp8_stream.hip",
     "fp8_block32.hip",
+    "fp8_moe.hip",
     "mx_matmul.hip",
     "mx_dma.hip",
     "routing.hip", "dense_ops.hip", "sgemm_mfma.hip", "dgemm_mfma.hip",

@@ -451,6 +451,40 @@ def fp8_block_linear(x, weight, weight_scale):
     return out.reshape(*x.shape[:-1], weight.shape[0])
 
 
+def fp8_moe_decode(x, w1, w2, w1_scale, w2_scale, expert_ids, routing, *, factor=1.0, out=None):
+    """One BF16 token [1, hidden] through a block-scaled FP8 mixture-of-experts layer
+    (ref: camblas/_hopper.py:329-401 `fused`): w1 E4M3 [experts, 2*width, hidden] (gate rows, then
+    up rows), w2 E4M3 [experts, hidden_out, width], FP32 scales per 128 x 128 block, expert_ids
+    int32 and routing FP32 with at most 16 entries. Returns BF16 [1, hidden_out]; `out` may be x."""
+    experts, doubled, hidden = w1.shape
+    hidden_out, width = w2.shape[1], w2.shape[2]
+    choices = expert_ids.numel()
+    _require(x.is_cuda and x.dtype == torch.bfloat16 and x.numel() == hidden and x.is_contiguous()
+             and w1.dtype == w2.dtype == torch.float8_e4m3fn and w1.is_contiguous() and w2.is_contiguous()
+             and w2.shape[0] == experts and doubled == 2 * width,
+             "FP8 expert step needs one contiguous BF16 token and E4M3 weights [experts, 2*width, hidden] / [experts, hidden_out, width]")
+    _require(hidden % 128 == 0 and width % 128 == 0 and hidden_out % 16 == 0 and 1 <= choices <= 16,
+             "FP8 expert step needs hidden and width in multiples of 128, outputs of 16 and 1..16 choices")
+    _require(w1_scale.dtype == w2_scale.dtype == torch.float32 and w1_scale.is_contiguous()
+             and w2_scale.is_contiguous()
+             and tuple(w1_scale.shape) == (experts, doubled // 128, hidden // 128)
+             and tuple(w2_scale.shape) == (experts, (hidden_out + 127) // 128, width // 128),
+             "FP8 expert scale shapes do not match their 128 x 128 blocks")
+    _require(expert_ids.dtype == torch.int32 and routing.dtype == torch.float32
+             and routing.numel() == choices and expert_ids.is_contiguous() and routing.is_contiguous()
+             and all(t.device == x.device for t in (w1, w2, w1_scale, w2_scale, expert_ids, routing)),
+             "FP8 expert step needs int32 expert IDs and FP32 routing weights on the token's device")
+    if out is None:
+        out = torch.empty((1, hidden_out), dtype=torch.bfloat16, device=x.device)
+    _require(out.dtype == torch.bfloat16 and out.numel() == hidden_out and out.is_contiguous()
+             and out.device == x.device, "FP8 expert output must be contiguous BF16 [1, hidden_out]")
+    _native.context(x.device).call(
+        "fp8_moe_decode", experts, choices, hidden, width, hidden_out, _pointer(x), _pointer(w1),
+        _pointer(w1_scale), _pointer(w2), _pointer(w2_scale), _pointer(expert_ids), _pointer(routing),
+        float(factor), _pointer(out))
+    return out
+
+
 def _bytes(tensor):
     return tensor if tensor.dtype == torch.uint8 else tensor.view(torch.uint8)
 

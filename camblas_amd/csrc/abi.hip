@@ -994,6 +994,35 @@ extern "C" int camblas_cuda_fp8_block_linear(camblas_cuda_context *context, int 
     return camblas_cuda_fp8_block_matmul(context, rows, outputs, inner, q, scale, w, w_scale, out);
 }
 
+// One token through a block-scaled FP8 mixture-of-experts layer (rule of camblas/_hopper.py:329-401,
+// which the reference reaches from Python only; here it is an entry point like the other products).
+extern "C" int camblas_cuda_fp8_moe_decode(camblas_cuda_context *context, int experts, int choices,
+                                           int hidden, int width, int hidden_out, const void *x,
+                                           const void *w1, const float *w1_scale, const void *w2,
+                                           const float *w2_scale, const int32_t *expert_ids,
+                                           const float *routing, float factor, void *output)
+{
+    return execute(context, [&] {
+        if (experts < 1 || choices < 1 || choices > 16 || hidden < 128 || hidden % 128 ||
+            width < 128 || width % 128 || hidden_out < 16 || hidden_out % 16 ||
+            choices * (width / 128) > 960 || !std::isfinite(factor))
+            return fail(context, "invalid FP8 expert dimensions", 1);
+        if (!x || !w1 || !w1_scale || !w2 || !w2_scale || !expert_ids || !routing || !output ||
+            !aligned(x, 16) || !aligned(w1, 16) || !aligned(w2, 16) || !aligned(w1_scale, 4) ||
+            !aligned(w2_scale, 4) || !aligned(expert_ids, 4) || !aligned(routing, 4) ||
+            !aligned(output, 2) || output == w1 || output == w2)
+            return fail(context, "invalid FP8 expert buffers", 1);
+        hipError_t grown = reserve_scratch(context, fp8_moe_decode_scratch_bytes(choices, width));
+        if (grown != hipSuccess)
+            return fail(context, "FP8 expert scratch", grown);
+        context->counts[4]++;
+        hipError_t error = launch_fp8_moe_decode(context->stream, experts, choices, hidden, width,
+                                                 hidden_out, x, w1, w1_scale, w2, w2_scale, expert_ids,
+                                                 routing, factor, context->scratch, output);
+        return error == hipSuccess ? 0 : fail(context, "FP8 expert step", error);
+    });
+}
+
 extern "C" int camblas_cuda_rope(camblas_cuda_context *context, int tokens, int heads, int dim,
                                  int token_stride, float theta, const int32_t *positions, void *x)
 {

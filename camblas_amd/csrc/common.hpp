@@ -131,6 +131,13 @@ hipError_t launch_fp8_stream(hipStream_t stream, int row_tiles, int token_tiles,
 hipError_t launch_fp8_block32_decode(hipStream_t stream, int outputs, int inner, const void *x,
                                      const float *sx, int sx_stride, const void *w, const float *sw,
                                      int sw_row, int sw_col, void *out);
+// One token through an FP8 (1x128 . 128x128 scales) mixture-of-experts layer: gate/up products,
+// clipped SiLU-multiply, down products, routed sum. scratch: fp8_moe_decode_scratch_bytes().
+size_t fp8_moe_decode_scratch_bytes(int choices, int width);
+hipError_t launch_fp8_moe_decode(hipStream_t stream, int experts, int choices, int hidden, int width,
+                                 int hidden_out, const void *x, const void *w1, const float *s1,
+                                 const void *w2, const float *s2, const int32_t *ids,
+                                 const float *routing, float factor, void *scratch, void *out);
 // E8M0 block-scaled product (E4M3 or packed E2M1 weights); groups == 0 plain, >= 1 grouped.
 // kernel: -1 chooses by shape; 0 the weight-streaming kernel; 20 + v the prefill kernel variant v.
 hipError_t launch_mx_matmul(hipStream_t stream, int kernel, int compute_units, bool packed, int groups,

@@ -37,21 +37,26 @@ __device__ __forceinline__ unsigned pack_bf16x2(float lo, float hi)
     return unsigned(float_to_bf16_bits(lo)) | (unsigned(float_to_bf16_bits(hi)) << 16);
 }
 
-// FP32 -> E4M3fn, round-to-nearest-even, saturating at +-448, NaN -> 0x7f.
+// FP32 -> E4M3fn, round-to-nearest-even, saturating at +-448, NaN -> 0x7f: the conversion
+// instruction of gfx950 (OCP formats) after a clamp; the comparisons of the clamp keep NaN.
 __device__ __forceinline__ unsigned f32_to_e4m3_sat(float value)
 {
-    unsigned sign = (__float_as_uint(value) >> 24) & 0x80u;
-    float a = fabsf(value);
-    if (a != a)
-        return 0x7fu;
-    if (a >= 448.f)
-        return sign | 0x7eu;
-    if (a >= 0.015625f) { // normal range: round the FP32 mantissa to three bits
-        unsigned bits = __float_as_uint(a);
-        bits += 0x7ffffu + ((bits >> 20) & 1u);
-        return sign | ((((bits >> 23) - 120u) << 3) | ((bits >> 20) & 7u));
-    }
-    return sign | unsigned(__float2int_rn(a * 512.f)); // subnormals: multiples of 2^-9
+    const float clamped = value > 448.f ? 448.f : value < -448.f ? -448.f : value;
+    const unsigned code = unsigned(__builtin_amdgcn_cvt_pk_fp8_f32(clamped, clamped, 0, false)) & 0xffu;
+    return (code & 0x7fu) == 0x7fu ? 0x7fu : code;
+}
+
+// two values at once: low byte from `first`, next byte from `second`
+__device__ __forceinline__ unsigned f32x2_to_e4m3_sat(float first, float second)
+{
+    const float a = first > 448.f ? 448.f : first < -448.f ? -448.f : first;
+    const float b = second > 448.f ? 448.f : second < -448.f ? -448.f : second;
+    unsigned codes = unsigned(__builtin_amdgcn_cvt_pk_fp8_f32(a, b, 0, false)) & 0xffffu;
+    if ((codes & 0x7fu) == 0x7fu)
+        codes &= 0xff7fu;
+    if ((codes & 0x7f00u) == 0x7f00u)
+        codes &= 0x7fffu;
+    return codes;
 }
 
 // Storage traits: T is float, double or bf16_storage (a 16-bit wrapper).

@@ -13,9 +13,11 @@ What differs from the reference, on purpose: its block-128 FP8 guard admits one 
 of eleven weight shapes, because its kernel is a single-token Triton kernel for Hopper; the kernels
 here cover any token count and any [N, K] with K a multiple of 128, so the guard checks layout and
 dtypes only. The block-32 guards keep the single-token rule (that is what the entry points
-compute) but drop the shape list for the same reason. The reference's Hopper-only hooks (the
-[2, 1, 128] batched BF16 product, the fused 289-expert FP8 MoE step and the Triton tile tables of
-CAMBLAS_SGLANG_FP8_TILES) have no counterpart and are not registered.
+compute) but drop the shape list for the same reason. The fused single-token FP8 expert step
+keeps every condition of the reference on the runner configuration and drops only the fixed
+289-expert shapes: any expert count and any widths in multiples of 128 with at most 16 choices.
+The reference's remaining Hopper-only hooks (the [2, 1, 128] batched BF16 product and the Triton
+tile tables of CAMBLAS_SGLANG_FP8_TILES) have no counterpart and are not registered.
 
 The hook bodies are plain functions of (original, *arguments) returned by `build_hooks`, so they
 can be exercised without SGLang; `install` only hands them to the registry.
@@ -30,6 +32,7 @@ FP8_BLOCK128_TARGET = ("sglang.srt.layers.quantization.fp8_utils."
                        "deepgemm_w8a8_block_fp8_linear_with_fallback")
 FP8_BLOCK32_PRODUCT_TARGET = "sglang.kernels.ops.quantization.fp8_kernel.w8a8_block_fp8_matmul_triton"
 FP8_BLOCK32_LINEAR_TARGET = "sglang.srt.layers.quantization.fp8_utils.triton_w8a8_block_fp8_linear"
+FP8_MOE_TARGET = "sglang.srt.layers.moe.moe_runner.triton_utils.fused_moe.fused_experts"
 MOE_ALIGN_TARGET = ("sglang.srt.layers.moe.moe_runner.triton_utils."
                     "moe_align_block_size.moe_align_block_size")
 OPERATIONS = ("linear", "fp8")
@@ -155,12 +158,48 @@ def build_hooks(selected):
         return original(input, weight, block_size, weight_scale, input_scale, bias, act_scale_ue8m0,
                         weight_bf16)
 
+    def fp8_moe_fused(original, hidden_states, w1, w2, topk_output, moe_runner_config, *args, **kwargs):
+        # ref: camblas/sglang.py:340-455; one token, silu-gated experts with the limit 10, FP8
+        # weights with 128 x 128 block scales, no biases, zero points or static activation scales
+        cfg = moe_runner_config
+        ids, routing = topk_output.topk_ids, topk_output.topk_weights
+        scales = (kwargs.get("w1_scale"), kwargs.get("w2_scale"))
+        if (not args and not _tracing() and hidden_states.is_cuda and hidden_states.dtype == torch.bfloat16
+                and hidden_states.ndim == 2 and hidden_states.shape[0] == 1
+                and w1.ndim == 3 and w2.ndim == 3 and w1.dtype == w2.dtype == torch.float8_e4m3fn
+                and w1.shape[0] == w2.shape[0] and w1.shape[2] == hidden_states.shape[1] == w2.shape[1]
+                and w1.shape[1] == 2 * w2.shape[2] and w1.shape[2] % 128 == 0 and w2.shape[2] % 128 == 0
+                and cfg.activation == "silu" and cfg.is_gated and not cfg.no_combine
+                and not cfg.apply_router_weight_on_input and cfg.swiglu_limit == 10
+                and cfg.gemm1_alpha is None and cfg.gemm1_clamp_limit is None
+                and cfg.num_experts == cfg.num_local_experts == w1.shape[0]
+                and kwargs.get("use_fp8_w8a8") and kwargs.get("block_shape") == [128, 128]
+                and not any(kwargs.get(k, False) for k in ("use_int8_w8a8", "use_int8_w8a16", "use_int4_w4a16",
+                                                           "per_channel_quant", "fuse_swiglu_interleaved"))
+                and all(kwargs.get(k) is None for k in ("b1", "b2", "w1_zp", "w2_zp", "a1_scale", "a2_scale", "a1_q"))
+                and ids.dtype == torch.int32 and ids.ndim == 2 and ids.shape[0] == 1 and 1 <= ids.shape[1] <= 16
+                and routing.dtype == torch.float32 and routing.shape == ids.shape
+                and all(t is not None and t.dtype == torch.float32 for t in scales)
+                and tuple(scales[0].shape) == (w1.shape[0], w1.shape[1] // 128, w1.shape[2] // 128)
+                and tuple(scales[1].shape) == (w2.shape[0], w2.shape[1] // 128, w2.shape[2] // 128)
+                and all(t.is_contiguous() and t.device == hidden_states.device
+                        for t in (hidden_states, w1, w2, ids, routing, *scales))
+                and not torch.is_grad_enabled()):
+            output = hidden_states if cfg.inplace else torch.empty_like(hidden_states)
+            factor = 1.0 if cfg.routed_scaling_factor is None else cfg.routed_scaling_factor
+            _kernels.fp8_moe_decode(hidden_states, w1, w2, scales[0], scales[1], ids, routing,
+                                    factor=factor, out=output)
+            _count("fp8", "fp8_moe")
+            return output
+        return original(hidden_states, w1, w2, topk_output, moe_runner_config, *args, **kwargs)
+
     if "linear" in selected:
         hooks[LINEAR_TARGET] = linear
     if "fp8" in selected:
         hooks[FP8_BLOCK128_TARGET] = fp8_block128
         hooks[FP8_BLOCK32_PRODUCT_TARGET] = fp8_block32_product
         hooks[FP8_BLOCK32_LINEAR_TARGET] = fp8_block32_linear
+        hooks[FP8_MOE_TARGET] = fp8_moe_fused
     return hooks
 
 

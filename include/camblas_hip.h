@@ -265,6 +265,23 @@ int camblas_cuda_gqa_decode_attention(camblas_cuda_context *context, int batch, 
                                       int q_stride, const void *k_cache, const void *v_cache,
                                       void *output);
 
+/* extension (the reference runs this step from Python on Triton kernels, camblas/_hopper.py:329-401,
+ * behind its SGLang hook camblas/sglang.py:340-455; here it is an entry point like the other
+ * products). One BF16 token x [hidden] through a mixture-of-experts layer with E4M3 weights and
+ * FP32 scales per 128 x 128 block: w1 [experts, 2*width, hidden] (gate rows, then up rows) with
+ * w1_scale [experts, 2*width/128, hidden/128], w2 [experts, hidden_out, width] with w2_scale
+ * [experts, ceil(hidden_out/128), width/128], expert_ids int32 [choices] and routing FP32
+ * [choices] on the device. Per choice: x quantised per 128 inputs (amax/448), gate/up product
+ * rounded to BF16, silu(min(gate, 10)) * clamp(up, -10, 10) rounded to BF16 and quantised per 128,
+ * down product times the routing weight rounded to BF16; the choices are summed in order and the
+ * sum times `factor` is rounded to BF16 into output [hidden_out], which may be x itself.
+ * hidden and width multiples of 128, hidden_out of 16, 1..16 choices. Uses context scratch. */
+int camblas_cuda_fp8_moe_decode(camblas_cuda_context *context, int experts, int choices, int hidden,
+                                int width, int hidden_out, const void *x, const void *w1,
+                                const float *w1_scale, const void *w2, const float *w2_scale,
+                                const int32_t *expert_ids, const float *routing, float factor,
+                                void *output);
+
 /* extension. Planner introspection (the GPU counterpart of the reference CPU planner's
  * camblas_plan_format, src/planner.c:654-669): writes a one-line description of the kernel the
  * planner picks for a GEMM call into `text` and returns 1000 * family + variant (>=0) without touching a

@@ -267,6 +267,28 @@ def fp8_block_matmul_f64(a, a_scale, w, w_scale):
     return out
 
 
+def fp8_moe_decode_f64(x_bits, w1, s1, w2, s2, ids, routing, factor, limit=10.0):
+    """One BF16 token through the reference's FP8 mixture-of-experts step with FP64 dot products
+    and the reference's rounding points (camblas/_hopper.py:329-401 `fused`: dynamic 1x128
+    quantiser :82-98, ordered scaled products :118-126 and :168-182, clipped SiLU-multiply rounded
+    to BF16 :65-80, routing, BF16 rounding and ordered expert sum :305-326). Returns FP64
+    [hidden_out], before the final BF16 rounding. Built from the pinned `quantise_1x128` and
+    `fp8_block_matmul_f64`; the steps added here are pinned by tests/test_cpu_fp8_moe.py."""
+    width = w1.shape[1] // 2
+    q, scale = quantise_1x128(np.asarray(x_bits, dtype=np.uint16).reshape(1, -1))
+    total = np.zeros(w2.shape[1], dtype=np.float32)
+    for choice, expert in enumerate(np.asarray(ids).reshape(-1)):
+        up = fp8_block_matmul_f64(q, scale, w1[expert], s1[expert])[0]
+        up = bf16_to_f32(f32_to_bf16(up.astype(np.float32))).astype(np.float64)
+        gate, value = np.minimum(up[:width], limit), np.clip(up[width:], -limit, limit)
+        act = f32_to_bf16((gate / (1.0 + np.exp(-gate)) * value).astype(np.float32))
+        q2, scale2 = quantise_1x128(act.reshape(1, -1))
+        down = fp8_block_matmul_f64(q2, scale2, w2[expert], s2[expert])[0]
+        routed = (down * np.float64(np.float32(routing.reshape(-1)[choice]))).astype(np.float32)
+        total = total + bf16_to_f32(f32_to_bf16(routed))  # FP32 sum of BF16 values, choice order
+    return total.astype(np.float64) * float(factor)
+
+
 # ------------------------------------------------------------------ decode epilogues
 
 

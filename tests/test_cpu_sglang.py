@@ -109,6 +109,8 @@ def test_hook_targets_are_the_reference_ones():
     assert plugin.FP8_BLOCK32_PRODUCT_TARGET.endswith("w8a8_block_fp8_matmul_triton")
     assert plugin.FP8_BLOCK32_LINEAR_TARGET.endswith("triton_w8a8_block_fp8_linear")
     assert plugin.MOE_ALIGN_TARGET.endswith("moe_align_block_size.moe_align_block_size")
+    # ref: camblas/sglang.py:452-456
+    assert plugin.FP8_MOE_TARGET == "sglang.srt.layers.moe.moe_runner.triton_utils.fused_moe.fused_experts"
 
 
 def test_stable_moe_hook_only_reorders_prefill():

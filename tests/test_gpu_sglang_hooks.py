@@ -68,7 +68,7 @@ def test_linear_hook_routes_and_falls_back(device, dtype):
 def test_fp8_block128_hook(device, rows):
     hooks = plugin.build_hooks({"fp8"})
     assert set(hooks) == {plugin.FP8_BLOCK128_TARGET, plugin.FP8_BLOCK32_PRODUCT_TARGET,
-                          plugin.FP8_BLOCK32_LINEAR_TARGET}
+                          plugin.FP8_BLOCK32_LINEAR_TARGET, plugin.FP8_MOE_TARGET}
     hook = hooks[plugin.FP8_BLOCK128_TARGET]
     outputs, inner = 640, 1024
     x = oracle.fill_normal_bf16(910 + rows, (rows, inner))
@@ -164,3 +164,77 @@ def test_fp8_block128_hook_on_the_reference_shapes(device, shape, magnitude):
     assert not original.calls and out.shape == (1, outputs)
     q, scale = oracle.quantise_1x128(x)
     assert rel_frobenius(bf16_values(out), oracle.fp8_block_matmul_f64(q, scale, w, w_scale)) <= 1e-2
+
+
+def moe_configuration(experts, **changes):
+    """The runner configuration the reference's guard accepts (camblas/sglang.py:376-396)."""
+    fields = dict(activation="silu", is_gated=True, no_combine=False, apply_router_weight_on_input=False,
+                  swiglu_limit=10, gemm1_alpha=None, gemm1_clamp_limit=None, num_experts=experts,
+                  num_local_experts=experts, inplace=False, routed_scaling_factor=2.5)
+    fields.update(changes)
+    return types.SimpleNamespace(**fields)
+
+
+def test_fp8_moe_hook(device):
+    # ref: camblas/sglang.py:340-455 — the single-token FP8 expert step behind
+    # fused_moe.fused_experts: routed inside the guard (also in place), the original outside it
+    hooks = plugin.build_hooks({"fp8"})
+    hook = hooks[plugin.FP8_MOE_TARGET]
+    experts, choices, hidden, width = 12, 9, 512, 256
+    rng = np.random.default_rng(3)
+    x = oracle.f32_to_bf16((rng.standard_normal(hidden) * 3).astype(np.float32))
+    w1 = oracle.f32_to_e4m3((rng.standard_normal((experts, 2 * width, hidden)) * 0.6).astype(np.float32))
+    w2 = oracle.f32_to_e4m3((rng.standard_normal((experts, hidden, width)) * 0.6).astype(np.float32))
+    s1 = (rng.random((experts, 2 * width // 128, hidden // 128)) * 0.002 + 0.001).astype(np.float32)
+    s2 = (rng.random((experts, hidden // 128, width // 128)) * 0.002 + 0.001).astype(np.float32)
+    ids = rng.permutation(experts)[:choices].astype(np.int32)
+    routing = np.linspace(0.05, 1.0, choices).astype(np.float32)
+    want = oracle.fp8_moe_decode_f64(x, w1, s1, w2, s2, ids, routing, 2.5)
+
+    xt = to_device_bf16(x.reshape(1, -1), device)
+    w1t, w2t = to_device_fp8(w1, device), to_device_fp8(w2, device)
+    topk = types.SimpleNamespace(topk_ids=torch.from_numpy(ids).to(device).view(1, -1),
+                                 topk_weights=torch.from_numpy(routing).to(device).view(1, -1))
+    keywords = dict(w1_scale=torch.from_numpy(s1).to(device), w2_scale=torch.from_numpy(s2).to(device),
+                    use_fp8_w8a8=True, block_shape=[128, 128])
+    original, before = Original(), plugin.dispatch_counts()
+
+    class KeywordOriginal(Original):
+        def __call__(self, *arguments, **kwargs):
+            return super().__call__(*arguments)
+
+    original = KeywordOriginal()
+    with torch.no_grad():
+        out = hook(original, xt, w1t, w2t, topk, moe_configuration(experts), **keywords)
+        assert out is not xt and out.shape == (1, hidden) and out.dtype == torch.bfloat16
+        assert rel_frobenius(bf16_values(out)[0], want) <= 1e-2
+        same = xt.clone()
+        inplace = hook(original, same, w1t, w2t, topk, moe_configuration(experts, inplace=True), **keywords)
+        assert inplace is same and torch.equal(inplace, out)
+        unscaled = hook(original, xt, w1t, w2t, topk, moe_configuration(experts, routed_scaling_factor=None), **keywords)
+        assert rel_frobenius(bf16_values(unscaled)[0], want / 2.5) <= 1e-2
+        assert delta(before, "fp8") == 3 and delta(before, "fp8_moe") == 3 and not original.calls
+        # outside the guard: two tokens, another activation or limit, router weights on the input,
+        # a bias, a static activation scale, another block shape, int64 expert IDs, 17 choices,
+        # experts sharded over ranks, extra positional arguments
+        two = torch.cat([xt, xt])
+        refused = [
+            ((two, w1t, w2t, topk, moe_configuration(experts)), keywords),
+            ((xt, w1t, w2t, topk, moe_configuration(experts, activation="gelu")), keywords),
+            ((xt, w1t, w2t, topk, moe_configuration(experts, swiglu_limit=7)), keywords),
+            ((xt, w1t, w2t, topk, moe_configuration(experts, apply_router_weight_on_input=True)), keywords),
+            ((xt, w1t, w2t, topk, moe_configuration(experts, num_local_experts=experts // 2)), keywords),
+            ((xt, w1t, w2t, topk, moe_configuration(experts)), dict(keywords, b1=keywords["w1_scale"])),
+            ((xt, w1t, w2t, topk, moe_configuration(experts)), dict(keywords, a1_scale=keywords["w1_scale"])),
+            ((xt, w1t, w2t, topk, moe_configuration(experts)), dict(keywords, block_shape=[64, 64])),
+            ((xt, w1t, w2t, types.SimpleNamespace(topk_ids=topk.topk_ids.long(), topk_weights=topk.topk_weights),
+              moe_configuration(experts)), keywords),
+            ((xt, w1t, w2t, types.SimpleNamespace(topk_ids=torch.zeros((1, 17), dtype=torch.int32, device=device),
+                                                  topk_weights=torch.ones((1, 17), device=device)),
+              moe_configuration(experts)), keywords),
+            ((xt, w1t, w2t, topk, moe_configuration(experts), "extra"), keywords),
+        ]
+        for arguments, kwargs in refused:
+            assert hook(original, *arguments, **kwargs) == "original"
+    assert hook(original, xt, w1t, w2t, topk, moe_configuration(experts), **keywords) == "original"  # grad mode on
+    assert len(original.calls) == len(refused) + 1 and delta(before, "fp8_moe") == 3
