@@ -121,3 +121,41 @@ def test_invalid_arguments(device):
         case = make_case(1, 2, 1, 128, 128, 16, 1.0)
         x, w1, s1, w2, s2, ids, routing = case
         run(device, (x, w1, s1, w2, s2, np.zeros(17, np.int32), np.ones(17, np.float32)), 1.0)
+
+
+def test_captured_step_replays_with_changed_token_and_choices(device):
+    # the two launches captured once in a graph and replayed after the token, the chosen experts and
+    # the routing weights change in place; every replay equals the eager call bit for bit (the step
+    # has no reductions whose order depends on timing), with other work between the replays
+    x, w1, s1, w2, s2, ids, routing = make_case(61, 24, 8, 512, 256, 512, 2.0, [5, 0, 23, 7, 11, 2, 19, 13])
+    stream = torch.cuda.Stream()
+    stream.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(stream):
+        xt = torch.from_numpy(x.view(np.int16)).to(device).view(torch.bfloat16).reshape(1, -1)
+        tensors = [torch.from_numpy(w1).to(device).view(torch.float8_e4m3fn),
+                   torch.from_numpy(w2).to(device).view(torch.float8_e4m3fn),
+                   torch.from_numpy(s1).to(device), torch.from_numpy(s2).to(device)]
+        ids_t, routing_t = torch.from_numpy(ids).to(device), torch.from_numpy(routing).to(device)
+        out = torch.empty((1, 512), dtype=torch.bfloat16, device=device)
+        for _ in range(2):  # creates the stream's context and its scratch outside the capture
+            _kernels.fp8_moe_decode(xt, *tensors, ids_t, routing_t, factor=1.5, out=out)
+    stream.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph, stream=stream):
+        _kernels.fp8_moe_decode(xt, *tensors, ids_t, routing_t, factor=1.5, out=out)
+    with torch.cuda.stream(stream):
+        for round_ in range(3):
+            xt.mul_(-0.75)
+            ids_t.copy_((ids_t + 3 + round_) % 24)
+            routing_t.mul_(1.25)
+            graph.replay()
+            stream.synchronize()
+            eager = _kernels.fp8_moe_decode(xt, *tensors, ids_t, routing_t, factor=1.5)
+            stream.synchronize()
+            assert torch.equal(out, eager)
+    want = oracle.fp8_moe_decode_f64(oracle.f32_to_bf16(xt.float().cpu().numpy()[0]), w1, s1, w2, s2,
+                                     ids_t.cpu().numpy(), routing_t.cpu().numpy(), 1.5)
+    assert rel_frobenius(bf16_values(out)[0], want) <= 1e-2
+    torch.cuda.current_stream().wait_stream(stream)
+    torch.cuda.synchronize()
+    graph.reset()
