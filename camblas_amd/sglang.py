@@ -16,8 +16,10 @@ dtypes only. The block-32 guards keep the single-token rule (that is what the en
 compute) but drop the shape list for the same reason. The fused single-token FP8 expert step
 keeps every condition of the reference on the runner configuration and drops only the fixed
 289-expert shapes: any expert count and any widths in multiples of 128 with at most 16 choices.
-The reference's remaining Hopper-only hooks (the [2, 1, 128] batched BF16 product and the Triton
-tile tables of CAMBLAS_SGLANG_FP8_TILES) have no counterpart and are not registered.
+The batched BF16 projection hook takes any [batch, rows, inner] x [batch, outputs, inner] with
+at most 16 batches (one product per batch) instead of the single [2, 1, 128] x [2, 2048, 128]
+shape. The Triton tile tables of CAMBLAS_SGLANG_FP8_TILES configure SGLang's own Triton kernels
+and have no counterpart.
 
 The hook bodies are plain functions of (original, *arguments) returned by `build_hooks`, so they
 can be exercised without SGLang; `install` only hands them to the registry.
@@ -28,6 +30,7 @@ import os
 _calls = {}
 
 LINEAR_TARGET = "sglang.srt.layers.quantization.unquant.UnquantizedLinearMethod.apply"
+BATCHED_LINEAR_TARGET = "sglang.srt.layers.linear.ColumnParallelBatchedLinear.forward"
 FP8_BLOCK128_TARGET = ("sglang.srt.layers.quantization.fp8_utils."
                        "deepgemm_w8a8_block_fp8_linear_with_fallback")
 FP8_BLOCK32_PRODUCT_TARGET = "sglang.kernels.ops.quantization.fp8_kernel.w8a8_block_fp8_matmul_triton"
@@ -102,6 +105,23 @@ def build_hooks(selected):
             _count("linear")
             return _kernels.linear(x, weight, bias)
         return original(method, layer, x, bias)
+
+    def batched(original, layer, input):
+        # ref: camblas/sglang.py:294-336; FP32 accumulation, one BF16 rounding
+        weight = layer.weight
+        if (input.is_cuda and input.ndim == 3 and weight.ndim == 3 and 1 <= input.shape[0] <= 16
+                and input.shape[0] == weight.shape[0] and input.shape[2] == weight.shape[2]
+                and input.shape[1] >= 1 and input.dtype == weight.dtype == torch.bfloat16
+                and input.is_contiguous() and weight.is_contiguous() and weight.device == input.device
+                and not torch.is_grad_enabled() and not _tracing()
+                and not torch.backends.cuda.matmul.allow_bf16_reduced_precision_reduction):
+            output = torch.empty((input.shape[0], input.shape[1], weight.shape[1]), dtype=torch.bfloat16,
+                                 device=input.device)
+            for index in range(input.shape[0]):
+                _kernels.matmul(input[index], weight[index].t(), out=output[index])
+            _count("bmm")
+            return output
+        return original(layer, input)
 
     def fp8_block128(original, input, weight, block_size, weight_scale, input_scale=None, bias=None):
         # ref: camblas/sglang.py:472-544; dynamic 1x128 activation quantisation, any row count
@@ -195,6 +215,7 @@ def build_hooks(selected):
 
     if "linear" in selected:
         hooks[LINEAR_TARGET] = linear
+        hooks[BATCHED_LINEAR_TARGET] = batched
     if "fp8" in selected:
         hooks[FP8_BLOCK128_TARGET] = fp8_block128
         hooks[FP8_BLOCK32_PRODUCT_TARGET] = fp8_block32_product
@@ -238,6 +259,14 @@ def install():
         return
     from . import _kernels
 
-    _kernels.set_algorithm(os.environ.get("CAMBLAS_SGLANG_ALGORITHM", "auto"))
+    algorithm = os.environ.get("CAMBLAS_SGLANG_ALGORITHM", "auto")
+    _kernels.set_algorithm(algorithm)
+    if "linear" in selected:
+        # torch.mm / addmm / F.linear outside the hooked method as well (ref: camblas/sglang.py:245-248)
+        from . import _native
+
+        module = _native.tensor_module()
+        if module is not None and hasattr(module, "install_torch_backend"):
+            module.install_torch_backend(_native.ALGORITHMS[algorithm])
     for target, function in build_hooks(selected).items():
         HookRegistry.register(target, function, HookType.AROUND)

@@ -93,10 +93,20 @@ def test_install_registers_the_reference_hook_targets(registry, monkeypatch):
                                                                  for name in sorted(selected)})
     from camblas_amd import _kernels
 
-    chosen = []
+    chosen, installed = [], []
     monkeypatch.setattr(_kernels, "set_algorithm", chosen.append)
+    # "linear" also routes torch.mm / addmm / F.linear through the library (ref: camblas/sglang.py:245-248)
+    from camblas_amd import _native
+    import types
+
+    monkeypatch.setattr(_native, "tensor_module",
+                        lambda: types.SimpleNamespace(install_torch_backend=installed.append))
     plugin.install()
     assert [t for t, _, _ in registry] == ["fp8", "linear"] and chosen == ["auto"]
+    assert installed == [_native.ALGORITHMS["auto"]]
+    monkeypatch.setenv("CAMBLAS_SGLANG_OPS", "fp8")
+    plugin.install()
+    assert installed == [_native.ALGORITHMS["auto"]]  # not without "linear"
     monkeypatch.setenv("CAMBLAS_SGLANG_OPS", "bmm")
     with pytest.raises(ValueError):
         plugin.install()
@@ -105,6 +115,7 @@ def test_install_registers_the_reference_hook_targets(registry, monkeypatch):
 def test_hook_targets_are_the_reference_ones():
     # ref: camblas/sglang.py:287-291, :540-544, :641-645, :742-746, :192-196
     assert plugin.LINEAR_TARGET.endswith("UnquantizedLinearMethod.apply")
+    assert plugin.BATCHED_LINEAR_TARGET == "sglang.srt.layers.linear.ColumnParallelBatchedLinear.forward"
     assert plugin.FP8_BLOCK128_TARGET.endswith("deepgemm_w8a8_block_fp8_linear_with_fallback")
     assert plugin.FP8_BLOCK32_PRODUCT_TARGET.endswith("w8a8_block_fp8_matmul_triton")
     assert plugin.FP8_BLOCK32_LINEAR_TARGET.endswith("triton_w8a8_block_fp8_linear")

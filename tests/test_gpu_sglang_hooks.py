@@ -34,7 +34,7 @@ def delta(before, name):
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 def test_linear_hook_routes_and_falls_back(device, dtype):
     hook = plugin.build_hooks({"linear"})[plugin.LINEAR_TARGET]
-    assert set(plugin.build_hooks({"linear"})) == {plugin.LINEAR_TARGET}
+    assert set(plugin.build_hooks({"linear"})) == {plugin.LINEAR_TARGET, plugin.BATCHED_LINEAR_TARGET}
     generator = torch.Generator().manual_seed(11)
     x = torch.randn((3, 5, 256), generator=generator).to(dtype).to(device)
     weight = (torch.randn((96, 256), generator=generator) * 0.05).to(dtype).to(device)
@@ -238,3 +238,48 @@ def test_fp8_moe_hook(device):
             assert hook(original, *arguments, **kwargs) == "original"
     assert hook(original, xt, w1t, w2t, topk, moe_configuration(experts), **keywords) == "original"  # grad mode on
     assert len(original.calls) == len(refused) + 1 and delta(before, "fp8_moe") == 3
+
+
+@pytest.mark.parametrize("batch,rows,inner,outputs", [(2, 1, 128, 2048), (3, 5, 256, 520), (16, 2, 64, 24)])
+def test_batched_linear_hook(device, batch, rows, inner, outputs):
+    # ref: camblas/sglang.py:294-336 (its single shape is the first case): BF16 projections per batch
+    # with FP32 accumulation and one rounding; anything else reaches the original
+    hook = plugin.build_hooks({"linear"})[plugin.BATCHED_LINEAR_TARGET]
+    generator = torch.Generator().manual_seed(21 + batch)
+    x = torch.randn((batch, rows, inner), generator=generator).to(torch.bfloat16).to(device)
+    weight = (torch.randn((batch, outputs, inner), generator=generator) * 0.1).to(torch.bfloat16).to(device)
+    layer = types.SimpleNamespace(weight=weight)
+    original, before = Original(), plugin.dispatch_counts()
+    # the hook serves callers that asked for full-precision BF16 reductions (torch's default allows
+    # reduced precision; the reference's guard, and this one, then leave the product to the original)
+    previous = torch.backends.cuda.matmul.allow_bf16_reduced_precision_reduction
+    torch.backends.cuda.matmul.allow_bf16_reduced_precision_reduction = False
+    try:
+        routed_and_refused(hook, original, before, layer, x, weight, batch, rows, inner, outputs)
+    finally:
+        torch.backends.cuda.matmul.allow_bf16_reduced_precision_reduction = previous
+
+
+def routed_and_refused(hook, original, before, layer, x, weight, batch, rows, inner, outputs):
+    with torch.no_grad():
+        out = hook(original, layer, x)
+        assert out.shape == (batch, rows, outputs) and out.dtype == torch.bfloat16
+        want = torch.einsum("brk,bnk->brn", x.double().cpu(), weight.double().cpu())
+        assert rel_frobenius(out.double().cpu().numpy(), want.numpy()) <= 1e-2
+        assert delta(before, "bmm") == 1 and not original.calls
+        refused = [
+            (types.SimpleNamespace(weight=weight.float()), x.float()),
+            (types.SimpleNamespace(weight=weight[:, :, : inner // 2]), x[:, :, : inner // 2]),   # strided
+            (types.SimpleNamespace(weight=weight[0]), x),
+            (types.SimpleNamespace(weight=weight[:1]), x),
+            (types.SimpleNamespace(weight=weight.cpu()), x.cpu()),
+        ]
+        for owner, value in refused:
+            assert hook(original, owner, value) == "original"
+        torch.backends.cuda.matmul.allow_bf16_reduced_precision_reduction = True
+        try:
+            assert hook(original, layer, x) == "original"
+        finally:
+            torch.backends.cuda.matmul.allow_bf16_reduced_precision_reduction = False
+    assert hook(original, layer, x) == "original"  # grad mode on
+    assert len(original.calls) == len(refused) + 2 and delta(before, "bmm") == 1
