@@ -113,7 +113,7 @@ def main():
     parser.add_argument("--skip-extras", action="store_true")
     parser.add_argument("--skip-cpu", action="store_true")
     parser.add_argument("--only", choices=("decode1", "decode8", "decode32", "prefill", "copy", "fp8m1", "fp8m16",
-                                 "fp8m256", "fp8m4096", "mxe4m3m4096", "mxe2m1m4096", "attention",
+                                 "fp8m256", "fp8m4096", "mxe4m3m4096", "mxe2m1m4096", "fp8moe", "attention",
                                  "layer"),
                         help="profiling aid: launch just this kernel --steps times, print nothing")
     args = parser.parse_args()
@@ -244,7 +244,7 @@ def profile_only(args, torch, _kernels, _native, device, normal, weights, inputs
         def launch(i):
             native.call("hip_copy_probe", size, ct.c_void_p(source.data_ptr()),
                         ct.c_void_p(target.data_ptr()))
-    elif args.only.startswith("fp8m"):
+    elif args.only.startswith("fp8m") and args.only != "fp8moe":
         tokens, features, inner = int(args.only[4:]), 18432, 7168
         rotate = 3 if tokens <= 256 else 1
         copies = [torch.randint(0, 0x7E, (features, inner), device=device, dtype=torch.uint8)
@@ -257,6 +257,11 @@ def profile_only(args, torch, _kernels, _native, device, normal, weights, inputs
 
         def launch(i):
             _kernels.fp8_block_matmul(a, a_scale, copies[i % rotate], w_scale, out=out)
+    elif args.only == "fp8moe":
+        step = moe_step(torch, _kernels, device, normal)
+
+        def launch(i):
+            step(i)
     elif args.only.startswith("mx"):
         packed, tokens, features, inner = args.only.startswith("mxe2m1"), 4096, 18432, 7168
         w, scale, a, a_scale = mx_operands(torch, device, packed, tokens, features, inner)
@@ -276,6 +281,25 @@ def profile_only(args, torch, _kernels, _native, device, normal, weights, inputs
     for index in range(args.warmup + args.steps):
         launch(index)
     torch.cuda.synchronize()
+
+
+MOE_SHAPE = (289, 4096, 512, 9)  # experts, hidden, expert width, choices per token
+
+
+def moe_step(torch, _kernels, device, normal):
+    """Single-token FP8 expert step at the shapes of the reference's hook: 9 of 289 experts, gate/up
+    [1024, 4096] and down [4096, 512] per expert; the chosen experts rotate over 32 disjoint sets so
+    that the weights come from HBM."""
+    experts, hidden, width, choices = MOE_SHAPE
+    w1 = torch.randint(0, 0x7E, (experts, 2 * width, hidden), device=device, dtype=torch.uint8).view(torch.float8_e4m3fn)
+    w2 = torch.randint(0, 0x7E, (experts, hidden, width), device=device, dtype=torch.uint8).view(torch.float8_e4m3fn)
+    s1 = torch.rand((experts, 2 * width // 128, hidden // 128), device=device) * 0.001 + 0.001
+    s2 = torch.rand((experts, hidden // 128, width // 128), device=device) * 0.001 + 0.001
+    token = normal((1, hidden))
+    routing = torch.linspace(0.05, 1.0, choices, device=device)
+    chosen = [torch.arange(choices * i, choices * i + choices, device=device, dtype=torch.int32) for i in range(32)]
+    result = torch.empty((1, hidden), dtype=torch.bfloat16, device=device)
+    return lambda i: _kernels.fp8_moe_decode(token, w1, w2, s1, s2, chosen[i % 32], routing, factor=2.5, out=result)
 
 
 def mx_operands(torch, device, packed, tokens, features, inner):
@@ -426,25 +450,15 @@ def extras(torch, _kernels, _native, device, normal):
     found["fp32_sgemm_2048"] = {"us": round(seconds * 1e6, 1),
                                 "tflops": round(2.0 * size**3 / seconds / 1e12, 2),
                                 "frac_of_157TF": round(2.0 * size**3 / seconds / FP32_PEAK, 4)}
-    # single-token FP8 expert step at the shapes of the reference's hook: 9 of 289 experts, gate/up
-    # [1024, 4096] and down [4096, 512] per expert; the chosen experts rotate so that weights come from HBM
-    experts, hidden, width, choices = 289, 4096, 512, 9
-    w1 = torch.randint(0, 0x7E, (experts, 2 * width, hidden), device=device, dtype=torch.uint8).view(torch.float8_e4m3fn)
-    w2 = torch.randint(0, 0x7E, (experts, hidden, width), device=device, dtype=torch.uint8).view(torch.float8_e4m3fn)
-    s1 = torch.rand((experts, 2 * width // 128, hidden // 128), device=device) * 0.001 + 0.001
-    s2 = torch.rand((experts, hidden // 128, width // 128), device=device) * 0.001 + 0.001
-    token = normal((1, hidden))
-    routing = torch.linspace(0.05, 1.0, choices, device=device)
-    chosen = [torch.arange(choices * i, choices * i + choices, device=device, dtype=torch.int32) for i in range(32)]
-    result = torch.empty((1, hidden), dtype=torch.bfloat16, device=device)
-    seconds = event_time(
-        torch, lambda i: _kernels.fp8_moe_decode(token, w1, w2, s1, s2, chosen[i % 32], routing, factor=2.5,
-                                                 out=result), 10, 40)
+    # single-token FP8 expert step (9 of 289 experts, rotating sets)
+    experts, hidden, width, choices = MOE_SHAPE
+    step = moe_step(torch, _kernels, device, normal)
+    seconds = event_time(torch, step, 10, 40)
     traffic = choices * (2 * width * hidden + hidden * width)
     found["fp8_moe_decode_9_of_289_experts"] = {
         "us": round(seconds * 1e6, 1), "gbps": round(traffic / seconds / 1e9, 1),
         "note": "two launches; bound by launch and latency, not bandwidth"}
-    del w1, w2, s1, s2
+    del step
     # what the matrix cores sustain: independent matrix instructions with no memory traffic (the
     # part's clock under matrix load included), the ceiling the prefill rates are read against
     import ctypes as ct
