@@ -223,3 +223,56 @@ def test_e8m0_product_18432x7168(device, packed, tokens):
     assert (np.abs(got - want) <= 0.008 * np.abs(want) + (np.abs(xd) @ np.abs(wd).T) * 2.0 ** -13).all()
     # one more on every input scale doubles every output exactly (E8M0 scales are powers of two)
     assert torch.equal(_kernels.quantized_matmul(x.view(torch.float8_e4m3fn), sx + 1, weight, sw), out * 2)
+
+
+@pytest.mark.parametrize("packed", [False, True])
+def test_grouped_e8m0_products_at_an_expert_layer_size(device, packed):
+    # a mixture-of-experts prefill: 8 groups of up to 300 rows through experts of [4096, 7168]
+    # (gate and up of a 2048-wide expert), weights chosen through the device table; sampled rows
+    # and outputs against FP64, zeros for clipped rows and invalid experts, exact doubling
+    groups, weight_groups, rows, outputs, inner = 8, 5, 300, 4096, 7168
+    generator = torch.Generator(device=device).manual_seed(9700 + packed)
+    x = torch.randint(0, 255, (groups, rows, inner), generator=generator, device=device, dtype=torch.uint8)
+    x[x == 0x7F] = 0x7E
+    sx = torch.randint(120, 130, (groups, rows, inner // 32), generator=generator, device=device, dtype=torch.uint8)
+    weights, scales = [], []
+    for _ in range(weight_groups):
+        if packed:
+            weights.append(torch.randint(0, 256, (outputs, inner // 2), generator=generator, device=device, dtype=torch.uint8))
+            scales.append(torch.randint(118, 128, (outputs, inner // 32), generator=generator, device=device, dtype=torch.uint8))
+        else:
+            w = torch.randint(0, 255, (outputs, inner), generator=generator, device=device, dtype=torch.uint8)
+            w[w == 0x7F] = 0x7E
+            weights.append(w)
+            scales.append(torch.randint(118, 128, (outputs // 32, inner // 32), generator=generator, device=device, dtype=torch.uint8))
+    metadata = torch.tensor([[w.data_ptr(), s.data_ptr()] for w, s in zip(weights, scales)],
+                            dtype=torch.int64, device=device)
+    active_host, counts_host = [4, 0, 2, 9, 1, 3, 0, -1], [300, 17, 256, 300, 0, 129, 999, 300]
+    active = torch.tensor(active_host, dtype=torch.int32, device=device)
+    counts = torch.tensor(counts_host, dtype=torch.int32, device=device)
+    xt = x.view(torch.float8_e4m3fn)
+    out = _kernels.grouped_quantized_matmul(xt, sx, metadata, active, counts, outputs=outputs, packed=packed)
+    assert out.shape == (groups, rows, outputs)
+    got_all = bf16_values(out)
+    blocks = sample(6, outputs // 32, 11, seams=(8,))   # tile seams at multiples of 256 rows
+    columns = (blocks[:, None] * 32 + np.arange(32)).ravel()
+    for g, (index, count) in enumerate(zip(active_host, counts_host)):
+        if not 0 <= index < weight_groups:
+            assert not got_all[g].any()
+            continue
+        count = min(max(count, 0), rows)
+        assert not got_all[g, count:].any()
+        if count == 0:
+            continue
+        picked = np.unique(np.concatenate([np.arange(0, count, 41), [count - 1], np.arange(126, 131) % count]))
+        xd = oracle.mx_dequantise(x[g].cpu().numpy()[picked], sx[g].cpu().numpy()[picked], 32)
+        w_rows = weights[index][torch.from_numpy(columns).to(device)].cpu().numpy()
+        s_rows = scales[index][torch.from_numpy(columns if packed else blocks).to(device)].cpu().numpy()
+        wd = oracle.mx_dequantise(w_rows, s_rows, 32, packed, True)
+        want = xd @ wd.T
+        got = got_all[g][np.ix_(picked, columns)]
+        assert rel_frobenius(got, want) <= 4e-3
+        assert (np.abs(got - want) <= 0.008 * np.abs(want) + (np.abs(xd) @ np.abs(wd).T) * 2.0 ** -13).all()
+    # one more on every input scale doubles every output exactly (E8M0 scales are powers of two)
+    assert torch.equal(_kernels.grouped_quantized_matmul(xt, sx + 1, metadata, active, counts, outputs=outputs,
+                                                         packed=packed), out * 2)
