@@ -1147,6 +1147,10 @@ PYBIND11_MODULE(_camblas_cuda_torch, module)
                py::arg("out") = py::none(), py::arg("alpha") = 1., py::arg("beta") = 0.,
                py::arg("algorithm") = -1,
                "Multiply two GPU matrices (FP32, FP64 or BF16) with transpose views and autograd.");
+    module.def("affine", [](const Tensor &x, const Tensor &weight, const Tensor &bias, bool relu,
+                            const std::optional<Tensor> &output, int algorithm) {
+        return affine(x, weight, bias, relu, output, algorithm < 0 ? default_algorithm : algorithm);
+    });
     module.def("affine_public", &affine_public, py::arg("x"), py::arg("weight"), py::arg("bias"),
                py::kw_only(), py::arg("relu") = false, py::arg("algorithm") = -1);
     module.def("mlp_public", &mlp_public, py::arg("x"), py::arg("w1"), py::arg("b1"), py::arg("w2"),

@@ -138,7 +138,7 @@ def test_tensor_binding_loads_and_exports_the_reference_surface():
                  "matmul", "matmul_public", "linear_public", "qkv_linear", "gated_mlp",
                  "silu_multiply", "swiglu", "rms_norm", "add_rms_norm", "fp8_block_matmul",
                  "fp8_decode_supported", "fp8_decode", "fp8_linear", "quantized_matmul",
-                 "QuantizedGroups", "route_groups", "reduce_groups", "affine_public", "mlp_public",
+                 "QuantizedGroups", "route_groups", "reduce_groups", "affine", "affine_public", "mlp_public",
                  "mlp", "mlp_backward", "attention_public", "attention"):
         assert callable(getattr(module, name)), name
     import torch

@@ -308,3 +308,21 @@ def test_captured_mlp_training_step_replays_with_changed_inputs(device, dtype):
     torch.cuda.current_stream().wait_stream(stream)
     torch.cuda.synchronize()
     graph.reset()
+
+
+def test_raw_affine_binding_writes_into_the_given_output(device):
+    # the positional entry the reference's Python layer binds beside the autograd form
+    # (ref: src/cuda/torch_bindings.cpp:738-775, :1227): x, weight, bias, relu, output, algorithm
+    from camblas_amd import _native
+
+    module = _native.tensor_module()
+    generator = torch.Generator().manual_seed(12)
+    x = torch.randn((9, 33), generator=generator).to(device)
+    weight = torch.randn((33, 21), generator=generator).to(device)
+    bias = torch.randn((21,), generator=generator).to(device)
+    out = torch.full((9, 21), float("nan"), device=device)
+    returned = module.affine(x, weight, bias, True, out, -1)
+    assert returned.data_ptr() == out.data_ptr()
+    close(out, torch.relu(x.double().cpu() @ weight.double().cpu() + bias.double().cpu()))
+    fresh = module.affine(x, weight, bias, False, None, -1)
+    close(fresh, x.double().cpu() @ weight.double().cpu() + bias.double().cpu())
