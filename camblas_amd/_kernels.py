@@ -710,3 +710,14 @@ def decoder_layer_decode(hidden, residual, weights, k_cache, v_cache, positions,
     projected = linear(attended.view(batch, q_heads * head_dim), weights["o"])
     residual, normed = add_rms_norm(projected, residual, weights["post_norm"], epsilon)
     return gated_mlp(normed, weights["gate"], weights["up"], weights["down"]), residual
+
+
+def __getattr__(name):
+    """`QuantizedGroups` (captured expert weights, ref: camblas/_kernels.py:55) lives in the tensor
+    binding; it is looked up on first use so that importing this module needs no built binding."""
+    if name == "QuantizedGroups":
+        module = _native.tensor_module()
+        if module is None or not hasattr(module, "QuantizedGroups"):
+            raise RuntimeError("QuantizedGroups requires the tensor binding (python camblas_amd/_build.py)")
+        return module.QuantizedGroups
+    raise AttributeError(name)

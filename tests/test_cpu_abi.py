@@ -143,6 +143,11 @@ def test_tensor_binding_loads_and_exports_the_reference_surface():
         assert callable(getattr(module, name)), name
     import torch
 
+    from camblas_amd import _kernels
+
+    assert _kernels.QuantizedGroups is module.QuantizedGroups
+    with pytest.raises(AttributeError):
+        _kernels.no_such_operation
     with pytest.raises(ValueError, match="GPU"):
         module.matmul_public(torch.zeros(2, 2), torch.zeros(2, 2))
 
