@@ -116,6 +116,35 @@ def test_python_surface_contract(monkeypatch):
         _kernels.matmul(torch.zeros(2, 2), torch.zeros(2, 2))  # CPU tensors are rejected, no fallback
 
 
+def test_autoload_environment_contract(monkeypatch):
+    # ref: camblas/__init__.py:6-29 — CAMBLAS_ENABLE=1 installs the backend with the policy named by
+    # CAMBLAS_CUDA_ALGORITHM, else CAMBLAS_SGLANG_ALGORITHM, else "lt"; a missing binding is a
+    # RuntimeError, an unknown policy a ValueError
+    import types
+
+    import camblas_amd
+
+    installed = []
+    monkeypatch.setattr(_native, "tensor_module",
+                        lambda: types.SimpleNamespace(install_torch_backend=installed.append))
+    monkeypatch.setenv("CAMBLAS_ENABLE", "1")
+    for variable in ("CAMBLAS_CUDA_ALGORITHM", "CAMBLAS_SGLANG_ALGORITHM"):
+        monkeypatch.delenv(variable, raising=False)
+    camblas_amd._autoload()
+    monkeypatch.setenv("CAMBLAS_SGLANG_ALGORITHM", "classical")
+    camblas_amd._autoload()
+    monkeypatch.setenv("CAMBLAS_CUDA_ALGORITHM", "auto")
+    camblas_amd._autoload()
+    assert installed == [_native.ALGORITHMS["lt"], _native.ALGORITHMS["classical"], _native.ALGORITHMS["auto"]]
+    monkeypatch.setenv("CAMBLAS_CUDA_ALGORITHM", "fastest")
+    with pytest.raises(ValueError, match="Unknown CAMBLAS CUDA algorithm"):
+        camblas_amd._autoload()
+    monkeypatch.setattr(_native, "tensor_module", lambda: None)
+    with pytest.raises(RuntimeError, match="tensor binding"):
+        camblas_amd._autoload()
+    assert len(installed) == 3
+
+
 def test_missing_library_fails_loudly(tmp_path):
     code = "from camblas_amd import _native; _native.library()"
     env = dict(os.environ, CAMBLAS_CUDA_LIBRARY=str(tmp_path / "absent.so"), PYTHONPATH=str(ROOT))
