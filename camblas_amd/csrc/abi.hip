@@ -1005,7 +1005,7 @@ extern "C" int camblas_cuda_fp8_moe_decode(camblas_cuda_context *context, int ex
     return execute(context, [&] {
         if (experts < 1 || choices < 1 || choices > 16 || hidden < 128 || hidden % 128 ||
             width < 128 || width % 128 || hidden_out < 16 || hidden_out % 16 ||
-            choices * (width / 128) > 960 || !std::isfinite(factor))
+            choices * (width / 128) > 512 || !std::isfinite(factor)) // (LDS of the second launch)
             return fail(context, "invalid FP8 expert dimensions", 1);
         if (!x || !w1 || !w1_scale || !w2 || !w2_scale || !expert_ids || !routing || !output ||
             !aligned(x, 16) || !aligned(w1, 16) || !aligned(w2, 16) || !aligned(w1_scale, 4) ||

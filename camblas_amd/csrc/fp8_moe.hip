@@ -324,8 +324,9 @@ hipError_t launch_fp8_moe_decode(hipStream_t stream, int experts, int choices, i
     if (error != hipSuccess)
         return error;
     const int pairs = choices * (width / 128);
+    // dynamic LDS beside 18 KB of static LDS, inside the 64 KB a launch gets without asking for more
     const size_t lds = size_t(pairs) * (MOE_ROWS + 1) * sizeof(float);
-    if (lds > 64 * 1024)
+    if (pairs > 512)
         return hipErrorInvalidValue;
     moe_down_kernel<<<unsigned(hidden_out / MOE_ROWS), MOE_THREADS, lds, stream>>>(p);
     return launch_status();

@@ -275,7 +275,8 @@ int camblas_cuda_gqa_decode_attention(camblas_cuda_context *context, int batch, 
  * rounded to BF16, silu(min(gate, 10)) * clamp(up, -10, 10) rounded to BF16 and quantised per 128,
  * down product times the routing weight rounded to BF16; the choices are summed in order and the
  * sum times `factor` is rounded to BF16 into output [hidden_out], which may be x itself.
- * hidden and width multiples of 128, hidden_out of 16, 1..16 choices. Uses context scratch. */
+ * hidden and width multiples of 128, hidden_out of 16, 1..16 choices, choices * width / 128 at
+ * most 512. Uses context scratch. */
 int camblas_cuda_fp8_moe_decode(camblas_cuda_context *context, int experts, int choices, int hidden,
                                 int width, int hidden_out, const void *x, const void *w1,
                                 const float *w1_scale, const void *w2, const float *w2_scale,

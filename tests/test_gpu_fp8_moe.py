@@ -109,7 +109,7 @@ def test_invalid_arguments(device):
     buffer = torch.zeros(4096, dtype=torch.uint8, device=device)
     p = ct.c_void_p(buffer.data_ptr())
     for arguments in ((0, 1, 128, 128, 16), (1, 0, 128, 128, 16), (1, 17, 128, 128, 16), (1, 1, 64, 128, 16),
-                      (1, 1, 128, 192, 16), (1, 1, 128, 128, 24)):
+                      (1, 1, 128, 192, 16), (1, 1, 128, 128, 24), (1, 16, 128, 4224, 16)):
         status = lib.camblas_cuda_fp8_moe_decode(native.handle, *arguments, p, p, p, p, p, p, p, 1.0, p)
         assert status == -1 and b"invalid FP8 expert dimensions" in lib.camblas_cuda_error(native.handle)
     status = lib.camblas_cuda_fp8_moe_decode(native.handle, 1, 1, 128, 128, 16, None, p, p, p, p, p, p, 1.0, p)
@@ -159,3 +159,11 @@ def test_captured_step_replays_with_changed_token_and_choices(device):
     torch.cuda.current_stream().wait_stream(stream)
     torch.cuda.synchronize()
     graph.reset()
+
+
+def test_largest_intermediate_width(device):
+    # 16 choices of 4096-wide experts: 512 (choice, group) pairs, the most the second launch holds
+    case = make_case(91, 16, 16, 128, 4096, 32, 1.0)
+    want = oracle.fp8_moe_decode_f64(*case, 1.0)
+    got = bf16_values(run(device, case, 1.0))[0]
+    assert rel_frobenius(got, want) <= 1e-2
