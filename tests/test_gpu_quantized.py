@@ -156,6 +156,39 @@ def test_grouped_products(device, packed):
         assert not got[g, count:].any()
 
 
+@pytest.mark.parametrize("packed", [False, True])
+def test_grouped_decode_with_many_groups_uses_wide_workgroups(device, packed):
+    # 40 groups of a few rows: the streaming kernel sizes its workgroups with all groups counted
+    # (eight 16-row tiles each here, the last workgroup of a group cut short at 1032 outputs)
+    groups, weight_groups, rows, outputs, inner = 40, 4, 5, 1032, 256
+    rng = np.random.default_rng(29)
+    x = oracle.f32_to_e4m3((rng.standard_normal((groups, rows, inner)) * 8).astype(np.float32))
+    sx = rng.integers(122, 129, (groups, rows, inner // 32), dtype=np.uint8)
+    weights, scales = [], []
+    for g in range(weight_groups):
+        _, _, w, sw = operands(820 + g, 1, outputs, inner, packed, 32)
+        weights.append(torch.from_numpy(w).to(device))
+        scales.append(torch.from_numpy(sw).to(device))
+    metadata = torch.tensor([[w.data_ptr(), s.data_ptr()] for w, s in zip(weights, scales)],
+                            dtype=torch.int64, device=device)
+    active_host = [int(v) for v in rng.integers(-1, weight_groups + 1, groups)]
+    counts_host = [int(v) for v in rng.integers(0, rows + 2, groups)]
+    out = _kernels.grouped_quantized_matmul(
+        torch.from_numpy(x).to(device).view(torch.float8_e4m3fn), torch.from_numpy(sx).to(device), metadata,
+        torch.tensor(active_host, dtype=torch.int32, device=device),
+        torch.tensor(counts_host, dtype=torch.int32, device=device), outputs=outputs, packed=packed)
+    torch.cuda.synchronize()
+    got = bf16_values(out)
+    for g, (index, count) in enumerate(zip(active_host, counts_host)):
+        if not 0 <= index < weight_groups:
+            assert not got[g].any()
+            continue
+        count = min(max(count, 0), rows)
+        want = oracle.mx_matmul_f64(x[g], sx[g], weights[index].cpu().numpy(), scales[index].cpu().numpy(), 32, packed)
+        assert (np.abs(got[g, :count] - want[:count]) <= 0.02 + 0.008 * np.abs(want[:count])).all()
+        assert not got[g, count:].any()
+
+
 def test_invalid_arguments(device):
     native, lib = _native.context(device), _native.library()
     for arguments in ((2, 1, 8, 32, 32), (0, 1, 12, 32, 32), (0, 1, 8, 48, 32), (0, 1, 8, 128, 128),
