@@ -421,7 +421,8 @@ hipError_t launch_one(hipStream_t stream, MxDmaParams p, int groups)
 
 // variant 0: 256 weight rows x 256 tokens (two stages for E4M3 weights, three for E2M1);
 // variant 1: 256 x 128, three stages; variant 2: 192 x 256, two stages, E4M3 weights only (a
-// wavefront load covers 16 rows of packed weights: 192 rows are not a whole number of rounds)
+// wavefront load covers 16 rows of packed weights: 192 rows are not a whole number of rounds);
+// variant 3: 128 x 128, three stages (twice the workgroups of variant 1 for small products)
 template <bool PACKED, bool WIDE_X, bool GROUPED>
 hipError_t launch_variant(hipStream_t stream, const MxDmaParams &p, int groups, int variant)
 {
@@ -432,12 +433,13 @@ hipError_t launch_variant(hipStream_t stream, const MxDmaParams &p, int groups, 
         if constexpr (!PACKED)
             return launch_one<false, false, GROUPED, 3, 2, 4, 2, 3>(stream, p, groups);
         return hipErrorInvalidValue;
+    case 3: return launch_one<PACKED, WIDE_X, GROUPED, 2, 1, 4, 3, 4>(stream, p, groups);
     default: return hipErrorInvalidValue;
     }
 }
 } // namespace
 
-int mx_dma_variant_count() { return 3; }
+int mx_dma_variant_count() { return 4; }
 
 // The prefill kernel's conditions: K a multiple of 128, 16-byte aligned operands, an 8-byte aligned
 // output (scale pointers may have any alignment).

@@ -417,26 +417,33 @@ hipError_t launch_mx_matmul(hipStream_t stream, int kernel, int compute_units, b
     // Above 32 rows the streaming kernel reads the weights once per 32-token slab; the tiled kernel
     // reads them once per 128 or 256 tokens (grouped weights come from the device table and are
     // 16-byte aligned by contract, so only the host-visible pointers are checked here). Measured
-    // crossover: 33 rows, except a single product with packed weights (65).
+    // crossover: 33 rows.
     const void *checked_weight = groups == 0 ? weight : nullptr;
     if (kernel >= 20)
         return launch_mx_dma(stream, kernel - 20, packed, groups, weight_groups, rows, outputs, inner,
                              activation_block, input, input_scale, weight, weight_scale, metadata,
                              active, counts, out);
-    const int most_streamed = packed && groups <= 1 ? 64 : 32;
-    if (kernel < 0 && rows > most_streamed &&
-        mx_dma_supported(outputs, inner, input, checked_weight, out)) {
-        // 256 x 256 tiles do the most work per byte moved through LDS; a 256 x 128 tile costs 0.57
-        // of one (0.6 with packed weights, whose scales are gathered per row), a 192 x 256 tile
-        // (E4M3 weights) 0.84, and the smaller tiles fill the chip when the large ones leave
-        // compute units idle: the fewest weighted rounds win.
-        const long long batches = groups > 0 ? groups : 1, token_tiles = (rows + 255) / 256;
+    if (kernel < 0 && rows > 32 && mx_dma_supported(outputs, inner, input, checked_weight, out)) {
+        // 256 x 256 tiles do the most work per byte moved through LDS; the smaller tiles cost more
+        // per output (a 256 x 128 tile 0.57 of a large one, 0.6 with packed weights whose scales
+        // are gathered per row; a 192 x 256 tile, E4M3 weights only, 0.84; a 128 x 128 tile 0.43 /
+        // 0.45) but fill the chip when the large ones leave compute units idle: the fewest
+        // weighted rounds win (weights fitted to [18432, 7168] at 48 to 8192 rows).
+        const long long batches = groups > 0 ? groups : 1;
         auto rounds = [&](long long tiles) { return double((tiles * batches + compute_units - 1) / compute_units); };
-        const double wide = rows > 128 ? rounds((outputs + 255) / 256 * token_tiles) : 1e30;
-        const double narrow = rounds(static_cast<long long>((outputs + 255) / 256) * ((rows + 127) / 128)) *
-                              (packed ? 0.6 : 0.57);
-        const double flat = rows > 128 && !packed ? rounds((outputs + 191) / 192 * token_tiles) * 0.84 : 1e30;
-        const int variant = wide <= narrow && wide <= flat ? 0 : flat < narrow ? 2 : 1;
+        auto tiles = [&](int tile_outputs, int tile_rows) {
+            return static_cast<long long>((outputs + tile_outputs - 1) / tile_outputs) * ((rows + tile_rows - 1) / tile_rows);
+        };
+        const double cost[4] = {
+            rows > 128 ? rounds(tiles(256, 256)) : 1e30,
+            rounds(tiles(256, 128)) * (packed ? 0.6 : 0.57),
+            rows > 128 && !packed ? rounds(tiles(192, 256)) * 0.84 : 1e30,
+            rounds(tiles(128, 128)) * (packed ? 0.45 : 0.43),
+        };
+        int variant = 0;
+        for (int candidate = 1; candidate < 4; ++candidate)
+            if (cost[candidate] < cost[variant])
+                variant = candidate;
         return launch_mx_dma(stream, variant, packed, groups, weight_groups, rows, outputs, inner,
                              activation_block, input, input_scale, weight, weight_scale, metadata,
                              active, counts, out);

@@ -292,9 +292,9 @@ int camblas_hip_plan_describe(int dtype, int algorithm, char trans_a, char trans
                               size_t text_bytes);
 /* extension. Diagnostics for tests and tuning: force the planner's choice for BF16/FP8 GEMMs on
  * this context (kernel < 0 restores the planner; split_k <= 0 lets the planner choose). For the
- * E8M0 products: 0 the weight-streaming kernel, 20 / 21 / 22 the tiled kernel with 256 x 256,
- * 256 x 128 and (E4M3 weights only) 192 x 256 tiles; a forced kernel that cannot run the call
- * makes the call fail. */
+ * E8M0 products: 0 the weight-streaming kernel, 20 / 21 / 22 / 23 the tiled kernel with
+ * 256 x 256, 256 x 128, (E4M3 weights only) 192 x 256 and 128 x 128 tiles; a forced kernel that
+ * cannot run the call makes the call fail. */
 int camblas_hip_set_plan_override(camblas_cuda_context *context, int kernel, int split_k);
 /* extension. Diagnostics: copies `bytes` (a multiple of 16, 16-byte aligned buffers) with a plain
  * grid-stride kernel. A launch of known HBM traffic (bytes read + bytes written) against which

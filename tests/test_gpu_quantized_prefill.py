@@ -15,7 +15,7 @@ from helpers import bf16_values
 
 pytestmark = pytest.mark.gpu
 
-KERNELS = {"auto": -1, "stream": 0, "tile256x256": 20, "tile256x128": 21, "tile192x256": 22}
+KERNELS = {"auto": -1, "stream": 0, "tile256x256": 20, "tile256x128": 21, "tile192x256": 22, "tile128x128": 23}
 
 
 def operands(seed, rows, outputs, inner, packed, block):
@@ -67,7 +67,7 @@ def close(got, x, sx, weight, sw, packed, block):
 
 
 # (the 192-row tile exists for E4M3 weights only)
-FORMATS = [(kernel, packed, block) for kernel in ("auto", "tile256x256", "tile256x128", "tile192x256")
+FORMATS = [(kernel, packed, block) for kernel in ("auto", "tile256x256", "tile256x128", "tile192x256", "tile128x128")
            for packed, block in ((False, 32), (True, 32), (True, 128)) if not (packed and kernel == "tile192x256")]
 
 
@@ -126,7 +126,7 @@ def test_tiled_and_streaming_kernels_agree(device, packed):
     assert (np.abs(tiled - streamed) <= 0.008 * np.abs(streamed) + magnitude * 2.0 ** -13).all()
 
 
-@pytest.mark.parametrize("kernel", ["tile256x256", "tile256x128"])
+@pytest.mark.parametrize("kernel", ["tile256x256", "tile256x128", "tile128x128"])
 @pytest.mark.parametrize("packed", [False, True])
 def test_scale_extremes_and_nan(device, kernel, packed):
     # ones times ones with unit weight scales: exact for input scales 2^-127, 1, 2^127 and NaN for
@@ -159,7 +159,7 @@ def test_scale_extremes_and_nan(device, kernel, packed):
         assert np.isnan(got[:, 263]).all() and (np.delete(got, 263, axis=1) == inner).all()
 
 
-@pytest.mark.parametrize("kernel", ["auto", "tile256x256", "tile256x128"])
+@pytest.mark.parametrize("kernel", ["auto", "tile256x256", "tile256x128", "tile128x128"])
 @pytest.mark.parametrize("packed,block", [(False, 32), (True, 32), (True, 128)])
 def test_grouped_products(device, kernel, packed, block):
     # ref: include/camblas_cuda.h:156-167 — weights chosen per group through a device table, an
