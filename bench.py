@@ -493,6 +493,25 @@ def extras(torch, _kernels, _native, device, normal):
                                 "tflops": round(2.0 * size**3 / seconds / 1e12, 2),
                                 "frac_of_78.6TF": round(2.0 * size**3 / seconds / 78.6e12, 4)}
     del a64, b64, c64
+    # FP32 SGEMM 8192^3: the ordinary kernel and the default policy (two Strassen levels from 8192;
+    # its time includes the guard's stream synchronisation), flops counted as 2 n^3 for both
+    size = 8192
+    a32 = torch.rand((size, size), device=device, dtype=torch.float32) * 2 - 1
+    b32 = torch.rand((size, size), device=device, dtype=torch.float32) * 2 - 1
+    c32 = torch.empty((size, size), device=device, dtype=torch.float32)
+    entry = {}
+    for policy in ("classical", "auto"):
+        with _native.algorithm(policy):
+            policy_context = _native.context(device)
+            seconds = event_time(
+                torch, lambda i: policy_context.call(
+                    "sgemm", b"N", b"N", size, size, size, ct.c_float(1.0), ct.c_void_p(a32.data_ptr()), size,
+                    ct.c_void_p(b32.data_ptr()), size, ct.c_float(0.0), ct.c_void_p(c32.data_ptr()), size), 1, 3)
+        entry[policy] = {"ms": round(seconds * 1e3, 2),
+                         "tflops_equivalent": round(2.0 * size**3 / seconds / 1e12, 1)}
+    _native.context(device)  # back to the thread's policy
+    found["fp32_sgemm_8192"] = entry
+    del a32, b32, c32
     # decoder-layer decode step (Llama-3.1-70B shapes, batch 32, KV context 2048)
     step, attention = layer_step(torch, _kernels, device, normal)
 

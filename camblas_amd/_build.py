@@ -35,7 +35,7 @@ CORE_SOURCES = (
     "fp8_moe.hip",
     "mx_matmul.hip",
     "mx_dma.hip",
-    "routing.hip", "dense_ops.hip", "sgemm_mfma.hip", "dgemm_mfma.hip",
+    "routing.hip", "dense_ops.hip", "sgemm_mfma.hip", "dgemm_mfma.hip", "strassen.hip",
     "fusion.hip",
     "probes.hip",
     "attention_decode.hip",

@@ -190,6 +190,16 @@ namespace camblas_hip
 {
 namespace
 {
+// Depth of the Strassen recursion for this product under the context's policy, 0 for none: square
+// untransposed products of even size from 256 under an explicit Strassen policy, from 8192 under
+// the default one (ref: src/cuda/backend.cu:843-853).
+int square_strassen_levels(const camblas_cuda_context *context, bool trans_a, bool trans_b, int m, int n, int k)
+{
+    if (trans_a || trans_b || m != n || n != k || n % 2 != 0 || n < 256)
+        return 0;
+    return strassen_levels(context->algorithm, n);
+}
+
 // FP32 / FP64 column-major GEMM on the context's stream, without the device scope: shared by the
 // public entry points and by the dense helpers below.
 int dense_gemm(camblas_cuda_context *context, char ta, char tb, int m, int n, int k, float alpha,
@@ -199,6 +209,11 @@ int dense_gemm(camblas_cuda_context *context, char ta, char tb, int m, int n, in
         context, "FP32", ta, tb, m, n, k, alpha, a, lda, b, ldb, beta, c, ldc,
         [&] { return launch_scale_f32(context->stream, m, n, beta, c, ldc); },
         [&](bool trans_a, bool trans_b) {
+            if (int levels = square_strassen_levels(context, trans_a, trans_b, m, n, k)) {
+                const int outcome = strassen_gemm(context, levels, n, alpha, a, lda, b, ldb, beta, c, ldc);
+                if (outcome != STRASSEN_FALL_BACK && outcome != STRASSEN_NOT_ELIGIBLE)
+                    return outcome;
+            }
             Plan plan = make_plan(0, context->algorithm, trans_a, trans_b, m, n, k, lda, ldb, ldc,
                                   aligned(a, 16) && aligned(b, 16), context->compute_units);
             context->counts[plan.counter]++;
@@ -230,6 +245,11 @@ int dense_gemm(camblas_cuda_context *context, char ta, char tb, int m, int n, in
         context, "FP64", ta, tb, m, n, k, alpha, a, lda, b, ldb, beta, c, ldc,
         [&] { return launch_scale_f64(context->stream, m, n, beta, c, ldc); },
         [&](bool trans_a, bool trans_b) {
+            if (int levels = square_strassen_levels(context, trans_a, trans_b, m, n, k)) {
+                const int outcome = strassen_gemm(context, levels, n, alpha, a, lda, b, ldb, beta, c, ldc);
+                if (outcome != STRASSEN_FALL_BACK && outcome != STRASSEN_NOT_ELIGIBLE)
+                    return outcome;
+            }
             context->counts[0]++;
             bool matrix = m >= 16 && n >= 16 && k >= 4;
             if (context->override_kernel >= 0) // diagnostics: 0 vector-ALU tiles, else matrix-core tiles

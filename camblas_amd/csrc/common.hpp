@@ -86,12 +86,23 @@ hipError_t launch_generic_f32(hipStream_t stream, bool ta, bool tb, int m, int n
                               const float *a, int lda, const float *b, int ldb, float beta, float *c,
                               int ldc);
 // wide: 128 x 128 output tiles per workgroup, else 128 x 64
+// batches > 1: that many independent products, operands and outputs batch_stride elements apart
 hipError_t launch_sgemm_mfma(hipStream_t stream, bool wide, bool ta, bool tb, int m, int n, int k,
                              float alpha, const float *a, int lda, const float *b, int ldb, float beta,
-                             float *c, int ldc);
+                             float *c, int ldc, int batches = 1, size_t batch_stride = 0);
 hipError_t launch_dgemm_mfma(hipStream_t stream, bool ta, bool tb, int m, int n, int k, double alpha,
                              const double *a, int lda, const double *b, int ldb, double beta, double *c,
-                             int ldc);
+                             int ldc, int batches = 1, size_t batch_stride = 0);
+// Strassen policies for square 'N','N' products (strassen.hip). strassen_levels: recursion depth of
+// a policy for size n (0: the policy does not apply). strassen_gemm returns STRASSEN_DONE,
+// STRASSEN_FALL_BACK (guard raised or no scratch: counted, the caller runs the ordinary kernel),
+// STRASSEN_NOT_ELIGIBLE (capture, operands in scratch, non-finite alpha: nothing counted), or a
+// negative status after fail().
+enum { STRASSEN_DONE = 0, STRASSEN_FALL_BACK = 1, STRASSEN_NOT_ELIGIBLE = 2 };
+int strassen_levels(int algorithm, int n);
+template <typename T>
+int strassen_gemm(camblas_cuda_context *context, int levels, int n, T alpha, const T *a, int lda, const T *b,
+                  int ldb, T beta, T *c, int ldc);
 hipError_t launch_generic_bf16(hipStream_t stream, bool ta, bool tb, int m, int n, int k,
                                float alpha, const void *a, int lda, const void *b, int ldb,
                                float beta, void *c, int ldc);

@@ -33,8 +33,12 @@ template <bool CONTIGUOUS_K> __device__ __forceinline__ int lds_index(int r, int
 template <bool TA, bool TB>
 __global__ __launch_bounds__(THREADS, 2) void dgemm_mfma_kernel(int m, int n, int k, double alpha,
                                                              const double *a, int lda, const double *b,
-                                                             int ldb, double beta, double *c, int ldc)
+                                                             int ldb, double beta, double *c, int ldc,
+                                                             size_t batch_stride)
 {
+    a += blockIdx.z * batch_stride; // one independent product per grid z-slice
+    b += blockIdx.z * batch_stride;
+    c += blockIdx.z * batch_stride;
     __shared__ double tile_a[TILE_WORDS];
     __shared__ double tile_b[TILE_WORDS];
     const int thread = threadIdx.x, lane = thread % 64, wave = thread / 64;
@@ -125,19 +129,19 @@ __global__ __launch_bounds__(THREADS, 2) void dgemm_mfma_kernel(int m, int n, in
 
 hipError_t launch_dgemm_mfma(hipStream_t stream, bool ta, bool tb, int m, int n, int k, double alpha,
                              const double *a, int lda, const double *b, int ldb, double beta, double *c,
-                             int ldc)
+                             int ldc, int batches, size_t batch_stride)
 {
-    dim3 grid((m + TILE - 1) / TILE, (n + TILE - 1) / TILE);
-    if (grid.y > 65535u)
+    dim3 grid((m + TILE - 1) / TILE, (n + TILE - 1) / TILE, batches);
+    if (grid.y > 65535u || batches < 1 || batches > 65535)
         return hipErrorInvalidValue;
     if (!ta && !tb)
-        dgemm_mfma_kernel<false, false><<<grid, THREADS, 0, stream>>>(m, n, k, alpha, a, lda, b, ldb, beta, c, ldc);
+        dgemm_mfma_kernel<false, false><<<grid, THREADS, 0, stream>>>(m, n, k, alpha, a, lda, b, ldb, beta, c, ldc, batch_stride);
     else if (!ta && tb)
-        dgemm_mfma_kernel<false, true><<<grid, THREADS, 0, stream>>>(m, n, k, alpha, a, lda, b, ldb, beta, c, ldc);
+        dgemm_mfma_kernel<false, true><<<grid, THREADS, 0, stream>>>(m, n, k, alpha, a, lda, b, ldb, beta, c, ldc, batch_stride);
     else if (ta && !tb)
-        dgemm_mfma_kernel<true, false><<<grid, THREADS, 0, stream>>>(m, n, k, alpha, a, lda, b, ldb, beta, c, ldc);
+        dgemm_mfma_kernel<true, false><<<grid, THREADS, 0, stream>>>(m, n, k, alpha, a, lda, b, ldb, beta, c, ldc, batch_stride);
     else
-        dgemm_mfma_kernel<true, true><<<grid, THREADS, 0, stream>>>(m, n, k, alpha, a, lda, b, ldb, beta, c, ldc);
+        dgemm_mfma_kernel<true, true><<<grid, THREADS, 0, stream>>>(m, n, k, alpha, a, lda, b, ldb, beta, c, ldc, batch_stride);
     return launch_status();
 }
 } // namespace camblas_hip

@@ -33,8 +33,12 @@ template <bool CONTIGUOUS_K> __device__ __forceinline__ int lds_word(int r, int 
 template <bool TA, bool TB, int COLUMNS>
 __global__ __launch_bounds__(THREADS) void sgemm_mfma_kernel(int m, int n, int k, float alpha,
                                                              const float *a, int lda, const float *b,
-                                                             int ldb, float beta, float *c, int ldc)
+                                                             int ldb, float beta, float *c, int ldc,
+                                                             size_t batch_stride)
 {
+    a += blockIdx.z * batch_stride; // one independent product per grid z-slice
+    b += blockIdx.z * batch_stride;
+    c += blockIdx.z * batch_stride;
     __shared__ float tile_a[TILE_WORDS];
     __shared__ float tile_b[TILE_WORDS];
     const int thread = threadIdx.x, lane = thread % 64, wave = thread / 64;
@@ -154,19 +158,20 @@ __global__ __launch_bounds__(THREADS) void sgemm_mfma_kernel(int m, int n, int k
 
 template <int COLUMNS>
 hipError_t launch_columns(hipStream_t stream, bool ta, bool tb, int m, int n, int k, float alpha,
-                          const float *a, int lda, const float *b, int ldb, float beta, float *c, int ldc)
+                          const float *a, int lda, const float *b, int ldb, float beta, float *c, int ldc,
+                          int batches, size_t batch_stride)
 {
-    dim3 grid((m + TILE - 1) / TILE, (n + COLUMNS - 1) / COLUMNS);
-    if (grid.y > 65535u)
+    dim3 grid((m + TILE - 1) / TILE, (n + COLUMNS - 1) / COLUMNS, batches);
+    if (grid.y > 65535u || batches < 1 || batches > 65535)
         return hipErrorInvalidValue;
     if (!ta && !tb)
-        sgemm_mfma_kernel<false, false, COLUMNS><<<grid, THREADS, 0, stream>>>(m, n, k, alpha, a, lda, b, ldb, beta, c, ldc);
+        sgemm_mfma_kernel<false, false, COLUMNS><<<grid, THREADS, 0, stream>>>(m, n, k, alpha, a, lda, b, ldb, beta, c, ldc, batch_stride);
     else if (!ta && tb)
-        sgemm_mfma_kernel<false, true, COLUMNS><<<grid, THREADS, 0, stream>>>(m, n, k, alpha, a, lda, b, ldb, beta, c, ldc);
+        sgemm_mfma_kernel<false, true, COLUMNS><<<grid, THREADS, 0, stream>>>(m, n, k, alpha, a, lda, b, ldb, beta, c, ldc, batch_stride);
     else if (ta && !tb)
-        sgemm_mfma_kernel<true, false, COLUMNS><<<grid, THREADS, 0, stream>>>(m, n, k, alpha, a, lda, b, ldb, beta, c, ldc);
+        sgemm_mfma_kernel<true, false, COLUMNS><<<grid, THREADS, 0, stream>>>(m, n, k, alpha, a, lda, b, ldb, beta, c, ldc, batch_stride);
     else
-        sgemm_mfma_kernel<true, true, COLUMNS><<<grid, THREADS, 0, stream>>>(m, n, k, alpha, a, lda, b, ldb, beta, c, ldc);
+        sgemm_mfma_kernel<true, true, COLUMNS><<<grid, THREADS, 0, stream>>>(m, n, k, alpha, a, lda, b, ldb, beta, c, ldc, batch_stride);
     return launch_status();
 }
 } // namespace
@@ -174,9 +179,11 @@ hipError_t launch_columns(hipStream_t stream, bool ta, bool tb, int m, int n, in
 // wide: 128 x 128 tiles, else 128 x 64
 hipError_t launch_sgemm_mfma(hipStream_t stream, bool wide, bool ta, bool tb, int m, int n, int k,
                              float alpha, const float *a, int lda, const float *b, int ldb, float beta,
-                             float *c, int ldc)
+                             float *c, int ldc, int batches, size_t batch_stride)
 {
-    return wide ? launch_columns<128>(stream, ta, tb, m, n, k, alpha, a, lda, b, ldb, beta, c, ldc)
-                : launch_columns<64>(stream, ta, tb, m, n, k, alpha, a, lda, b, ldb, beta, c, ldc);
+    return wide ? launch_columns<128>(stream, ta, tb, m, n, k, alpha, a, lda, b, ldb, beta, c, ldc, batches,
+                                      batch_stride)
+                : launch_columns<64>(stream, ta, tb, m, n, k, alpha, a, lda, b, ldb, beta, c, ldc, batches,
+                                     batch_stride);
 }
 } // namespace camblas_hip

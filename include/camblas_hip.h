@@ -31,9 +31,18 @@ extern "C" {
 typedef struct camblas_cuda_context camblas_cuda_context;
 
 /* ref: include/camblas_cuda.h:14-23. On this backend AUTO and LT select the planned MFMA/GEMV
- * kernels (counter slot 4), CLASSICAL forces the generic LDS-tiled kernel (counter slot 0), and
- * the SYMMETRIC/STRASSEN values are accepted and executed as CLASSICAL-or-planned products with
- * ordinary rounding (the reference documents those modes as optional accelerations). */
+ * kernels (counter slot 4), CLASSICAL counts in slot 0 (and for BF16 forces the generic LDS-tiled
+ * kernel), SYMMETRIC is accepted and executed as an ordinary product.
+ * STRASSEN / _TWO / _THREE / _FOUR apply to sgemm and dgemm of square 'N','N' products of even
+ * size from 256 (ref: src/cuda/backend.cu:442-551, :836-853): one to four levels of Strassen's
+ * seven-product recursion, as deep as n stays divisible by two and the leaves keep 32 rows, the 7^L
+ * leaf products in one batched matrix-core launch (counter slot 1). The first pass checks the
+ * operands: a NaN, an infinity or a magnitude above sqrt(max / (16 4^L n max(1, |alpha|))) sends the
+ * call to the ordinary kernel instead (counter slot 5), as does a scratch allocation failure, which
+ * first tries fewer levels. That check is one stream synchronisation per call, so the policy is
+ * skipped while the stream is capturing, and for operands inside the context's scratch. AUTO uses
+ * two levels from n = 8192, where they are measured 10-20 % faster than the ordinary kernel.
+ * Every other product under these policies runs the ordinary kernels with ordinary rounding. */
 enum camblas_cuda_algorithm {
     CAMBLAS_CUDA_AUTO = 0,
     CAMBLAS_CUDA_CLASSICAL = 1,
