@@ -200,6 +200,24 @@ int square_strassen_levels(const camblas_cuda_context *context, bool trans_a, bo
     return strassen_levels(context->algorithm, n);
 }
 
+// The symmetric policy applies to a product of a matrix with its own transpose that overwrites C
+// (ref: src/cuda/backend.cu:819-835): only the tiles on and below the diagonal are computed, the
+// upper triangle is a copy of the lower one, so C is symmetric bit for bit.
+bool symmetric_gram(const camblas_cuda_context *context, bool trans_a, bool trans_b, int m, int n,
+                    const void *a, int lda, const void *b, int ldb, bool overwrite)
+{
+    return context->algorithm == CAMBLAS_CUDA_SYMMETRIC && a == b && trans_a != trans_b && m == n &&
+           lda == ldb && overwrite;
+}
+
+// Tile width of the FP32 lower-triangle product: 128 x 128 once the tiles that reach the diagonal
+// number two per compute unit, else 128 x 64 (the rule of the full product)
+bool gram_prefers_wide_tiles(int n, int compute_units)
+{
+    const double rows = (n + 127) / 128;
+    return rows * (rows + 1) / 2 >= 2.0 * compute_units;
+}
+
 // FP32 / FP64 column-major GEMM on the context's stream, without the device scope: shared by the
 // public entry points and by the dense helpers below.
 int dense_gemm(camblas_cuda_context *context, char ta, char tb, int m, int n, int k, float alpha,
@@ -209,6 +227,19 @@ int dense_gemm(camblas_cuda_context *context, char ta, char tb, int m, int n, in
         context, "FP32", ta, tb, m, n, k, alpha, a, lda, b, ldb, beta, c, ldc,
         [&] { return launch_scale_f32(context->stream, m, n, beta, c, ldc); },
         [&](bool trans_a, bool trans_b) {
+            if (symmetric_gram(context, trans_a, trans_b, m, n, a, lda, b, ldb, beta == 0.f)) {
+                context->counts[2]++;
+                hipError_t error =
+                    m >= 32 && k >= 16
+                        ? launch_sgemm_mfma(context->stream, gram_prefers_wide_tiles(m, context->compute_units),
+                                            trans_a, trans_b, m, n, k, alpha, a, lda, b, ldb, beta, c, ldc, 1, 0, true)
+                        : launch_generic_f32(context->stream, trans_a, trans_b, m, n, k, alpha, a, lda, b, ldb,
+                                             beta, c, ldc);
+                if (error != hipSuccess)
+                    return fail(context, "symmetric Gram", error);
+                error = launch_mirror_lower(context->stream, 0, n, c, ldc);
+                return error == hipSuccess ? 0 : fail(context, "Gram mirroring", error);
+            }
             if (int levels = square_strassen_levels(context, trans_a, trans_b, m, n, k)) {
                 const int outcome = strassen_gemm(context, levels, n, alpha, a, lda, b, ldb, beta, c, ldc);
                 if (outcome != STRASSEN_FALL_BACK && outcome != STRASSEN_NOT_ELIGIBLE)
@@ -245,6 +276,19 @@ int dense_gemm(camblas_cuda_context *context, char ta, char tb, int m, int n, in
         context, "FP64", ta, tb, m, n, k, alpha, a, lda, b, ldb, beta, c, ldc,
         [&] { return launch_scale_f64(context->stream, m, n, beta, c, ldc); },
         [&](bool trans_a, bool trans_b) {
+            if (symmetric_gram(context, trans_a, trans_b, m, n, a, lda, b, ldb, beta == 0.0)) {
+                context->counts[2]++;
+                hipError_t error =
+                    m >= 16 && k >= 4
+                        ? launch_dgemm_mfma(context->stream, trans_a, trans_b, m, n, k, alpha, a, lda, b, ldb, beta,
+                                            c, ldc, 1, 0, true)
+                        : launch_generic_f64(context->stream, trans_a, trans_b, m, n, k, alpha, a, lda, b, ldb,
+                                             beta, c, ldc);
+                if (error != hipSuccess)
+                    return fail(context, "symmetric Gram", error);
+                error = launch_mirror_lower(context->stream, 1, n, c, ldc);
+                return error == hipSuccess ? 0 : fail(context, "Gram mirroring", error);
+            }
             if (int levels = square_strassen_levels(context, trans_a, trans_b, m, n, k)) {
                 const int outcome = strassen_gemm(context, levels, n, alpha, a, lda, b, ldb, beta, c, ldc);
                 if (outcome != STRASSEN_FALL_BACK && outcome != STRASSEN_NOT_ELIGIBLE)

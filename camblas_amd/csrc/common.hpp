@@ -86,13 +86,18 @@ hipError_t launch_generic_f32(hipStream_t stream, bool ta, bool tb, int m, int n
                               const float *a, int lda, const float *b, int ldb, float beta, float *c,
                               int ldc);
 // wide: 128 x 128 output tiles per workgroup, else 128 x 64
-// batches > 1: that many independent products, operands and outputs batch_stride elements apart
+// batches > 1: that many independent products, operands and outputs batch_stride elements apart;
+// lower_only (square outputs): only the tiles that reach the diagonal run, as a one-dimensional grid
+// (the caller mirrors the lower triangle)
 hipError_t launch_sgemm_mfma(hipStream_t stream, bool wide, bool ta, bool tb, int m, int n, int k,
                              float alpha, const float *a, int lda, const float *b, int ldb, float beta,
-                             float *c, int ldc, int batches = 1, size_t batch_stride = 0);
+                             float *c, int ldc, int batches = 1, size_t batch_stride = 0,
+                             bool lower_only = false);
 hipError_t launch_dgemm_mfma(hipStream_t stream, bool ta, bool tb, int m, int n, int k, double alpha,
                              const double *a, int lda, const double *b, int ldb, double beta, double *c,
-                             int ldc, int batches = 1, size_t batch_stride = 0);
+                             int ldc, int batches = 1, size_t batch_stride = 0, bool lower_only = false);
+// c[row, column] = c[column, row] for row < column of a column-major n x n matrix (dtype 0 FP32, 1 FP64)
+hipError_t launch_mirror_lower(hipStream_t stream, int dtype, int n, void *c, int ldc);
 // Strassen policies for square 'N','N' products (strassen.hip). strassen_levels: recursion depth of
 // a policy for size n (0: the policy does not apply). strassen_gemm returns STRASSEN_DONE,
 // STRASSEN_FALL_BACK (guard raised or no scratch: counted, the caller runs the ordinary kernel),

@@ -217,7 +217,45 @@ hipError_t column_sums(hipStream_t stream, bool mask, T *grad, const T *activati
         partial, chunks, columns, sums);
     return launch_status();
 }
+
+// Upper tile (ti, tj), ti <= tj, of a column-major matrix from the transposed lower tile (tj, ti):
+// both the reads and the writes run along columns, the transposition happens in LDS.
+constexpr int MIRROR_TILE = 32;
+template <typename T>
+__global__ __launch_bounds__(MIRROR_TILE * 8) void mirror_lower_kernel(int n, T *c, size_t ldc)
+{
+    __shared__ T tile[MIRROR_TILE][MIRROR_TILE + 1];
+    const int ti = blockIdx.x, tj = blockIdx.y;
+    if (ti > tj)
+        return;
+    for (int y = threadIdx.y; y < MIRROR_TILE; y += 8) {
+        const int row = tj * MIRROR_TILE + threadIdx.x, column = ti * MIRROR_TILE + y; // lower source
+        if (row < n && column < n)
+            tile[y][threadIdx.x] = c[row + column * ldc];
+    }
+    __syncthreads();
+    for (int y = threadIdx.y; y < MIRROR_TILE; y += 8) {
+        const int row = ti * MIRROR_TILE + threadIdx.x, column = tj * MIRROR_TILE + y; // upper target
+        if (row < column && column < n)
+            c[row + column * ldc] = tile[threadIdx.x][y];
+    }
+}
 } // namespace
+
+hipError_t launch_mirror_lower(hipStream_t stream, int dtype, int n, void *c, int ldc)
+{
+    if (n < 2)
+        return hipSuccess;
+    const unsigned tiles = unsigned((n + MIRROR_TILE - 1) / MIRROR_TILE);
+    if (tiles > 65535u)
+        return hipErrorInvalidValue;
+    dim3 grid(tiles, tiles), block(MIRROR_TILE, 8);
+    if (dtype == 0)
+        mirror_lower_kernel<<<grid, block, 0, stream>>>(n, static_cast<float *>(c), size_t(ldc));
+    else
+        mirror_lower_kernel<<<grid, block, 0, stream>>>(n, static_cast<double *>(c), size_t(ldc));
+    return launch_status();
+}
 
 hipError_t launch_bias_activation(hipStream_t stream, int dtype, void *out, const void *bias,
                                   size_t count, int columns, bool relu)

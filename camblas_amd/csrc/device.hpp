@@ -141,4 +141,27 @@ __device__ __forceinline__ float wave_max(float value)
     return fmaxf(fmaxf(lane_value(value, 0), lane_value(value, 16)),
                  fmaxf(lane_value(value, 32), lane_value(value, 48)));
 }
+// Tile of a lower-triangle launch: workgroup t of a one-dimensional grid owns column tile j of row
+// tile i, the tiles of a row (those that reach the diagonal: (i + 1) * TILE / COLUMNS of them)
+// numbered before those of the next row. Returns false for a tile beyond the last column.
+template <int TILE_ROWS, int TILE_COLUMNS>
+__device__ __forceinline__ bool lower_tile(unsigned t, int n, int &row0, int &col0)
+{
+    constexpr unsigned PER_ROW = TILE_ROWS / TILE_COLUMNS; // column tiles added by every row tile
+    int i = int((sqrtf(8.f * float(t / PER_ROW) + 1.f) - 1.f) * 0.5f);
+    while (PER_ROW * unsigned(i + 1) * unsigned(i + 2) / 2 <= t)
+        ++i;
+    while (PER_ROW * unsigned(i) * unsigned(i + 1) / 2 > t)
+        --i;
+    row0 = i * TILE_ROWS;
+    col0 = int(t - PER_ROW * unsigned(i) * unsigned(i + 1) / 2) * TILE_COLUMNS;
+    return col0 < n;
+}
+
+// workgroups of a lower-triangle launch over an n x n output
+template <int TILE_ROWS, int TILE_COLUMNS> inline unsigned lower_tile_count(int n)
+{
+    const unsigned rows = unsigned((n + TILE_ROWS - 1) / TILE_ROWS);
+    return TILE_ROWS / TILE_COLUMNS * rows * (rows + 1) / 2;
+}
 } // namespace camblas_hip

@@ -34,8 +34,12 @@ template <bool TA, bool TB>
 __global__ __launch_bounds__(THREADS, 2) void dgemm_mfma_kernel(int m, int n, int k, double alpha,
                                                              const double *a, int lda, const double *b,
                                                              int ldb, double beta, double *c, int ldc,
-                                                             size_t batch_stride)
+                                                             size_t batch_stride, bool lower_only)
 {
+    // a symmetric product: only the tiles that reach the diagonal, the rest is the mirroring pass
+    int row0 = blockIdx.x * TILE, col0 = blockIdx.y * TILE;
+    if (lower_only && !lower_tile<TILE, TILE>(blockIdx.x, n, row0, col0))
+        return;
     a += blockIdx.z * batch_stride; // one independent product per grid z-slice
     b += blockIdx.z * batch_stride;
     c += blockIdx.z * batch_stride;
@@ -43,7 +47,6 @@ __global__ __launch_bounds__(THREADS, 2) void dgemm_mfma_kernel(int m, int n, in
     __shared__ double tile_b[TILE_WORDS];
     const int thread = threadIdx.x, lane = thread % 64, wave = thread / 64;
     constexpr int PER_THREAD = TILE * DEPTH / THREADS;
-    const int row0 = blockIdx.x * TILE, col0 = blockIdx.y * TILE;
     // A(i, l) is a[i + l*lda] ('N', rows contiguous) or a[l + i*lda] ('T', K contiguous);
     // B(l, j) is b[l + j*ldb] ('N', K contiguous) or b[j + l*ldb] ('T', columns contiguous).
     // Element e of a step goes to the thread so that consecutive threads read consecutive memory.
@@ -129,19 +132,21 @@ __global__ __launch_bounds__(THREADS, 2) void dgemm_mfma_kernel(int m, int n, in
 
 hipError_t launch_dgemm_mfma(hipStream_t stream, bool ta, bool tb, int m, int n, int k, double alpha,
                              const double *a, int lda, const double *b, int ldb, double beta, double *c,
-                             int ldc, int batches, size_t batch_stride)
+                             int ldc, int batches, size_t batch_stride, bool lower_only)
 {
     dim3 grid((m + TILE - 1) / TILE, (n + TILE - 1) / TILE, batches);
+    if (lower_only)
+        grid = dim3(lower_tile_count<TILE, TILE>(n), 1, batches);
     if (grid.y > 65535u || batches < 1 || batches > 65535)
         return hipErrorInvalidValue;
     if (!ta && !tb)
-        dgemm_mfma_kernel<false, false><<<grid, THREADS, 0, stream>>>(m, n, k, alpha, a, lda, b, ldb, beta, c, ldc, batch_stride);
+        dgemm_mfma_kernel<false, false><<<grid, THREADS, 0, stream>>>(m, n, k, alpha, a, lda, b, ldb, beta, c, ldc, batch_stride, lower_only);
     else if (!ta && tb)
-        dgemm_mfma_kernel<false, true><<<grid, THREADS, 0, stream>>>(m, n, k, alpha, a, lda, b, ldb, beta, c, ldc, batch_stride);
+        dgemm_mfma_kernel<false, true><<<grid, THREADS, 0, stream>>>(m, n, k, alpha, a, lda, b, ldb, beta, c, ldc, batch_stride, lower_only);
     else if (ta && !tb)
-        dgemm_mfma_kernel<true, false><<<grid, THREADS, 0, stream>>>(m, n, k, alpha, a, lda, b, ldb, beta, c, ldc, batch_stride);
+        dgemm_mfma_kernel<true, false><<<grid, THREADS, 0, stream>>>(m, n, k, alpha, a, lda, b, ldb, beta, c, ldc, batch_stride, lower_only);
     else
-        dgemm_mfma_kernel<true, true><<<grid, THREADS, 0, stream>>>(m, n, k, alpha, a, lda, b, ldb, beta, c, ldc, batch_stride);
+        dgemm_mfma_kernel<true, true><<<grid, THREADS, 0, stream>>>(m, n, k, alpha, a, lda, b, ldb, beta, c, ldc, batch_stride, lower_only);
     return launch_status();
 }
 } // namespace camblas_hip

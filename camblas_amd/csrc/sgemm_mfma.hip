@@ -34,8 +34,12 @@ template <bool TA, bool TB, int COLUMNS>
 __global__ __launch_bounds__(THREADS) void sgemm_mfma_kernel(int m, int n, int k, float alpha,
                                                              const float *a, int lda, const float *b,
                                                              int ldb, float beta, float *c, int ldc,
-                                                             size_t batch_stride)
+                                                             size_t batch_stride, bool lower_only)
 {
+    // a symmetric product: only the tiles that reach the diagonal, the rest is the mirroring pass
+    int row0 = blockIdx.x * TILE, col0 = blockIdx.y * COLUMNS;
+    if (lower_only && !lower_tile<TILE, COLUMNS>(blockIdx.x, n, row0, col0))
+        return;
     a += blockIdx.z * batch_stride; // one independent product per grid z-slice
     b += blockIdx.z * batch_stride;
     c += blockIdx.z * batch_stride;
@@ -44,7 +48,6 @@ __global__ __launch_bounds__(THREADS) void sgemm_mfma_kernel(int m, int n, int k
     const int thread = threadIdx.x, lane = thread % 64, wave = thread / 64;
     constexpr int A_PER_THREAD = TILE * DEPTH / THREADS, B_PER_THREAD = COLUMNS * DEPTH / THREADS;
     constexpr int WJ = COLUMNS / 64; // 32-column MFMA tiles per wavefront
-    const int row0 = blockIdx.x * TILE, col0 = blockIdx.y * COLUMNS;
     // A(i, l) is a[i + l*lda] ('N', rows contiguous) or a[l + i*lda] ('T', K contiguous);
     // B(l, j) is b[l + j*ldb] ('N', K contiguous) or b[j + l*ldb] ('T', columns contiguous).
     // Element e of a step goes to the thread so that consecutive threads read consecutive memory.
@@ -159,19 +162,21 @@ __global__ __launch_bounds__(THREADS) void sgemm_mfma_kernel(int m, int n, int k
 template <int COLUMNS>
 hipError_t launch_columns(hipStream_t stream, bool ta, bool tb, int m, int n, int k, float alpha,
                           const float *a, int lda, const float *b, int ldb, float beta, float *c, int ldc,
-                          int batches, size_t batch_stride)
+                          int batches, size_t batch_stride, bool lower_only)
 {
     dim3 grid((m + TILE - 1) / TILE, (n + COLUMNS - 1) / COLUMNS, batches);
+    if (lower_only)
+        grid = dim3(lower_tile_count<TILE, COLUMNS>(n), 1, batches);
     if (grid.y > 65535u || batches < 1 || batches > 65535)
         return hipErrorInvalidValue;
     if (!ta && !tb)
-        sgemm_mfma_kernel<false, false, COLUMNS><<<grid, THREADS, 0, stream>>>(m, n, k, alpha, a, lda, b, ldb, beta, c, ldc, batch_stride);
+        sgemm_mfma_kernel<false, false, COLUMNS><<<grid, THREADS, 0, stream>>>(m, n, k, alpha, a, lda, b, ldb, beta, c, ldc, batch_stride, lower_only);
     else if (!ta && tb)
-        sgemm_mfma_kernel<false, true, COLUMNS><<<grid, THREADS, 0, stream>>>(m, n, k, alpha, a, lda, b, ldb, beta, c, ldc, batch_stride);
+        sgemm_mfma_kernel<false, true, COLUMNS><<<grid, THREADS, 0, stream>>>(m, n, k, alpha, a, lda, b, ldb, beta, c, ldc, batch_stride, lower_only);
     else if (ta && !tb)
-        sgemm_mfma_kernel<true, false, COLUMNS><<<grid, THREADS, 0, stream>>>(m, n, k, alpha, a, lda, b, ldb, beta, c, ldc, batch_stride);
+        sgemm_mfma_kernel<true, false, COLUMNS><<<grid, THREADS, 0, stream>>>(m, n, k, alpha, a, lda, b, ldb, beta, c, ldc, batch_stride, lower_only);
     else
-        sgemm_mfma_kernel<true, true, COLUMNS><<<grid, THREADS, 0, stream>>>(m, n, k, alpha, a, lda, b, ldb, beta, c, ldc, batch_stride);
+        sgemm_mfma_kernel<true, true, COLUMNS><<<grid, THREADS, 0, stream>>>(m, n, k, alpha, a, lda, b, ldb, beta, c, ldc, batch_stride, lower_only);
     return launch_status();
 }
 } // namespace
@@ -179,11 +184,11 @@ hipError_t launch_columns(hipStream_t stream, bool ta, bool tb, int m, int n, in
 // wide: 128 x 128 tiles, else 128 x 64
 hipError_t launch_sgemm_mfma(hipStream_t stream, bool wide, bool ta, bool tb, int m, int n, int k,
                              float alpha, const float *a, int lda, const float *b, int ldb, float beta,
-                             float *c, int ldc, int batches, size_t batch_stride)
+                             float *c, int ldc, int batches, size_t batch_stride, bool lower_only)
 {
     return wide ? launch_columns<128>(stream, ta, tb, m, n, k, alpha, a, lda, b, ldb, beta, c, ldc, batches,
-                                      batch_stride)
+                                      batch_stride, lower_only)
                 : launch_columns<64>(stream, ta, tb, m, n, k, alpha, a, lda, b, ldb, beta, c, ldc, batches,
-                                     batch_stride);
+                                     batch_stride, lower_only);
 }
 } // namespace camblas_hip

@@ -32,7 +32,10 @@ typedef struct camblas_cuda_context camblas_cuda_context;
 
 /* ref: include/camblas_cuda.h:14-23. On this backend AUTO and LT select the planned MFMA/GEMV
  * kernels (counter slot 4), CLASSICAL counts in slot 0 (and for BF16 forces the generic LDS-tiled
- * kernel), SYMMETRIC is accepted and executed as an ordinary product.
+ * kernel). Under SYMMETRIC an sgemm / dgemm call with a == b, opposite transposes, m == n,
+ * lda == ldb and beta == 0 (a matrix times its own transpose; ref: src/cuda/backend.cu:819-835)
+ * computes only the tiles that reach the diagonal and copies the lower triangle into the upper one,
+ * so C equals its transpose bit for bit (counter slot 2); every other call is an ordinary product.
  * STRASSEN / _TWO / _THREE / _FOUR apply to sgemm and dgemm of square 'N','N' products of even
  * size from 256 (ref: src/cuda/backend.cu:442-551, :836-853): one to four levels of Strassen's
  * seven-product recursion, as deep as n stays divisible by two and the leaves keep 32 rows, the 7^L
