@@ -164,11 +164,16 @@ int strassen_gemm(camblas_cuda_context *context, int levels, int n, T alpha, con
         in_scratch(a) || in_scratch(b) || in_scratch(c))
         return STRASSEN_NOT_ELIGIBLE;
 
-    // scratch for L levels; an allocation failure drops a level (counted once as a guard fallback)
+    // scratch for L levels; an allocation failure drops a level (counted once as a guard fallback).
+    // The default policy was not asked for by name, so it never grows the scratch beyond 16 GiB:
+    // it drops levels, or leaves the product to the ordinary kernel, without counting anything.
+    constexpr size_t DEFAULT_POLICY_LIMIT = size_t(16) << 30;
     bool counted = false;
     size_t leaves = 0, leaf_elements = 0, spare_elements = 0;
     for (;; --levels) {
         if (levels == 0) {
+            if (!counted && context->algorithm == CAMBLAS_CUDA_AUTO)
+                return STRASSEN_NOT_ELIGIBLE;
             if (!counted)
                 context->counts[5]++;
             return STRASSEN_FALL_BACK;
@@ -177,8 +182,10 @@ int strassen_gemm(camblas_cuda_context *context, int levels, int n, T alpha, con
         leaves = power_of_seven(levels);
         leaf_elements = leaves * leaf * leaf;
         spare_elements = levels > 1 ? power_of_seven(levels - 1) * (2 * leaf) * (2 * leaf) : 0;
-        const hipError_t status =
-            reserve_scratch(context, FLAG_BYTES + (3 * leaf_elements + spare_elements) * sizeof(T));
+        const size_t bytes = FLAG_BYTES + (3 * leaf_elements + spare_elements) * sizeof(T);
+        if (context->algorithm == CAMBLAS_CUDA_AUTO && bytes > DEFAULT_POLICY_LIMIT)
+            continue;
+        const hipError_t status = reserve_scratch(context, bytes);
         if (status == hipSuccess)
             break;
         if (status != hipErrorOutOfMemory)

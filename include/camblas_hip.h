@@ -44,7 +44,9 @@ typedef struct camblas_cuda_context camblas_cuda_context;
  * call to the ordinary kernel instead (counter slot 5), as does a scratch allocation failure, which
  * first tries fewer levels. That check is one stream synchronisation per call, so the policy is
  * skipped while the stream is capturing, and for operands inside the context's scratch. AUTO uses
- * two levels from n = 8192, where they are measured 10-20 % faster than the ordinary kernel.
+ * two levels from n = 8192, where they are measured 10-20 % faster than the ordinary kernel, and
+ * fewer (or none) where the scratch would exceed 16 GiB; a named policy takes what it needs:
+ * (3 (7/4)^L + (7/4)^(L-1)) n^2 elements, kept by the context like all of its scratch.
  * Every other product under these policies runs the ordinary kernels with ordinary rounding. */
 enum camblas_cuda_algorithm {
     CAMBLAS_CUDA_AUTO = 0,
