@@ -201,6 +201,50 @@ def test_grouped_products(device, kernel, packed, block):
         assert not got[g, count:].any()
 
 
+@pytest.mark.parametrize("kernel", ["tile256x128", "tile128x128"])
+@pytest.mark.parametrize("packed", [False, True])
+def test_grouped_products_many_groups_skewed_counts(device, kernel, packed):
+    """150 groups (three 64-lane chunks of the tile numbering) with a capacity of several token tiles
+    and counts from none to all of it, negative and oversized included: every tile with work is
+    computed for the right group, every other tile of the capacity is zero."""
+    groups, weight_groups, rows, outputs, inner = 150, 5, 300, 136, 128
+    rng = np.random.default_rng(23)
+    x = oracle.f32_to_e4m3((rng.standard_normal((groups, rows, inner)) * 8).astype(np.float32))
+    sx = rng.integers(124, 129, (groups, rows, inner // 32), dtype=np.uint8)
+    counts_host = rng.choice([-3, 0, 1, 40, 127, 128, 129, 255, 256, 257, 300, 4000], size=groups).tolist()
+    active_host = rng.integers(-1, weight_groups + 1, size=groups).tolist()
+    weights, scales = [], []
+    for g in range(weight_groups):
+        _, _, w, sw = operands(900 + g, 1, outputs, inner, packed, 32)
+        weights.append(torch.from_numpy(w).to(device))
+        scales.append(torch.from_numpy(sw).to(device))
+    metadata = torch.tensor([[w.data_ptr(), s.data_ptr()] for w, s in zip(weights, scales)],
+                            dtype=torch.int64, device=device)
+    active = torch.tensor(active_host, dtype=torch.int32, device=device)
+    counts = torch.tensor(counts_host, dtype=torch.int32, device=device)
+    native = _native.context(device)
+    native.call("hip_set_plan_override", KERNELS[kernel], 0)
+    try:
+        out = _kernels.grouped_quantized_matmul(
+            torch.from_numpy(x).to(device).view(torch.float8_e4m3fn), torch.from_numpy(sx).to(device),
+            metadata, active, counts, outputs=outputs, packed=packed, activation_block=32)
+        torch.cuda.synchronize()
+    finally:
+        native.call("hip_set_plan_override", -1, 0)
+    got = bf16_values(out)
+    checked = 0
+    for g, (index, count) in enumerate(zip(active_host, counts_host)):
+        count = min(max(count, 0), rows) if 0 <= index < weight_groups else 0
+        assert not got[g, count:].any(), g
+        if count and checked < 40:  # the CPU product of every group would take minutes
+            close(got[g, :count], x[g, :count], sx[g, :count], weights[index].cpu().numpy(),
+                  scales[index].cpu().numpy(), packed, 32)
+            checked += 1
+        elif count:
+            assert got[g, :count].any(), g
+    assert checked == 40
+
+
 def test_forced_tile_kernel_refuses_what_it_cannot_run(device):
     # K that is not a multiple of 128 belongs to the streaming kernel; forcing the tiled one fails
     x, sx, weight, sw = operands(5, 70, 40, 160, False, 32)
