@@ -42,10 +42,17 @@ __global__ __launch_bounds__(WAVES * 64) void gqa_partition_kernel(
 {
     __shared__ __attribute__((aligned(16))) float wave_o[WAVES][HEADS][DIM];
     __shared__ float wave_m[WAVES][HEADS], wave_l[WAVES][HEADS];
-    const int split = blockIdx.x, kvh = blockIdx.y, b = blockIdx.z;
+    // Consecutive workgroups go to consecutive XCDs, so with the partition as the fast grid index
+    // and a partition count that is a multiple of eight, partition s of every sequence and head
+    // would run on XCD s % 8: sequences much shorter than the cache would keep one or two XCDs
+    // busy and leave the rest idle. The partition index is rotated by the (head, sequence) number.
+    const int kvh = blockIdx.y, b = blockIdx.z;
+    const int split = int((blockIdx.x + blockIdx.y + blockIdx.z * gridDim.y) % gridDim.x);
     const int thread = threadIdx.x, lane = thread % 64, wave = thread / 64;
     const int m = lane % 16, j = lane / 16;
     const int length = lengths ? min(max(lengths[b], 0), context_length) : context_length;
+    if (split * CHUNK >= length)
+        return; // past the sequence: the combine never reads this partition (uniform, before any barrier)
     const int begin = split * CHUNK + wave * WAVE_POSITIONS;
     const int count = min(WAVE_POSITIONS, length - begin); // may be <= 0: nothing for this wave
     const size_t row_stride = size_t(kv_heads) * DIM;
@@ -185,18 +192,23 @@ __global__ __launch_bounds__(WAVES * 64) void gqa_partition_kernel(
 }
 
 // out[b, head, :] = sum_s exp(m_s - M) o_s / sum_s exp(m_s - M) l_s, partitions in index order.
-__global__ __launch_bounds__(DIM) void gqa_combine_kernel(int splits, const float *part_o,
+// Only the partitions that hold positions of the sequence are read: the others were never written.
+__global__ __launch_bounds__(DIM) void gqa_combine_kernel(int partitions, int q_heads, int context_length,
+                                                          const int32_t *lengths, const float *part_o,
                                                           const float *part_m, const float *part_l,
                                                           unsigned short *out)
 {
     const size_t row = blockIdx.x; // b * q_heads + head
     const int d = threadIdx.x;
+    const int b = int(row / q_heads);
+    const int length = lengths ? min(max(lengths[b], 0), context_length) : context_length;
+    const int splits = min(partitions, (length + CHUNK - 1) / CHUNK);
     // Partitions are taken eight at a time with all loads of a batch issued before any is used
     // (a loop of dependent scalar loads would pay the memory latency once per partition); indices
     // past the end are clamped and masked. The order of the sums is the partition order.
     constexpr int BATCH = 8;
-    const float *row_m = part_m + row * splits, *row_l = part_l + row * splits;
-    const float *row_o = part_o + row * splits * DIM + d;
+    const float *row_m = part_m + row * partitions, *row_l = part_l + row * partitions;
+    const float *row_o = part_o + row * partitions * DIM + d;
     float top = -INFINITY;
     for (int s0 = 0; s0 < splits; s0 += BATCH) {
         float l[BATCH], m[BATCH];
@@ -267,7 +279,7 @@ hipError_t launch_gqa_decode(hipStream_t stream, int batch, int q_heads, int kv_
     if (status != hipSuccess)
         return status;
     gqa_combine_kernel<<<unsigned(size_t(batch) * q_heads), DIM, 0, stream>>>(
-        splits, part_o, part_m, part_l, static_cast<unsigned short *>(out));
+        splits, q_heads, context_length, lengths, part_o, part_m, part_l, static_cast<unsigned short *>(out));
     return launch_status();
 }
 } // namespace camblas_hip

@@ -181,6 +181,26 @@ def test_gqa_decode_attention_empty_and_partial_partitions(device):
     assert (np.abs(bf16_values(out)[1:] - wanted) <= 0.01 * np.abs(wanted) + 2e-3).all()
 
 
+def test_gqa_decode_attention_short_sequences_in_a_long_cache(device):
+    """Sixteen partitions per sequence, of which a sequence uses none to all: partitions past a
+    sequence's length are neither computed nor read, whatever an earlier call left in the scratch
+    (a first call with NaN queries over the whole cache leaves NaN in every partition record)."""
+    batch, q_heads, kv_heads, context, dim = 6, 16, 2, 4096, 128
+    q = oracle.fill_normal_bf16(43, (batch, q_heads, dim))
+    k = oracle.fill_normal_bf16(44, (batch, context, kv_heads, dim))
+    v = oracle.fill_normal_bf16(45, (batch, context, kv_heads, dim))
+    k_device, v_device = to_device_bf16(k, device), to_device_bf16(v, device)
+    poison = torch.full((batch, q_heads, dim), float("nan"), dtype=torch.bfloat16, device=device)
+    _kernels.gqa_decode_attention(poison, k_device, v_device, None, dim**-0.5)
+    lengths = np.array([0, 1, 255, 700, 2049, 4096], np.int32)
+    out = _kernels.gqa_decode_attention(to_device_bf16(q, device), k_device, v_device,
+                                        torch.from_numpy(lengths).to(device), dim**-0.5)
+    want = oracle.gqa_decode(q, k, v, np.maximum(lengths, 1), dim**-0.5)
+    assert not from_device_bf16(out)[0].any()
+    wanted = oracle.bf16_to_f32(want)[1:]
+    assert (np.abs(bf16_values(out)[1:] - wanted) <= 0.01 * np.abs(wanted) + 2e-3).all()
+
+
 def test_rope_kv_append_equals_rope_then_append(device):
     # the fused launch must give bit-identical activations and caches, including a sequence whose
     # position lies outside the cache (rotated, not written)
