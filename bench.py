@@ -440,6 +440,39 @@ def extras(torch, _kernels, _native, device, normal):
                     "frac_of_5PF": round(flops / seconds / FP8_PEAK, 4)}
         del w, scale, a, a_scale
     found["mx_quantized_matmul_m4096_18432x7168"] = mx
+    # the grouped form as an MoE prefill meets it: 32 experts of [4096, 7168] with a capacity of 1024
+    # rows each, every expert a quarter full (the rest of the capacity comes back as zeros)
+    experts, capacity, features, inner = 32, 1024, 4096, 7168
+    grouped = {}
+    for name, packed in (("e4m3_weights", False), ("e2m1_weights", True)):
+        parts = [mx_operands(torch, device, packed, 1, features, inner)[:2] for _ in range(experts)]
+        table = torch.tensor([[w.data_ptr(), scale.data_ptr()] for w, scale in parts], dtype=torch.int64,
+                             device=device)
+        tokens = torch.randint(0, 0x7E, (experts, capacity, inner), device=device,
+                               dtype=torch.uint8).view(torch.float8_e4m3fn)
+        token_scale = torch.randint(120, 130, (experts, capacity, inner // 32), device=device, dtype=torch.uint8)
+        order = torch.arange(experts, dtype=torch.int32, device=device)
+        for label, fill in (("full", capacity), ("quarter_full", capacity // 4)):
+            counts = torch.full((experts,), fill, dtype=torch.int32, device=device)
+            seconds = event_time(
+                torch, lambda i: _kernels.grouped_quantized_matmul(tokens, token_scale, table, order, counts,
+                                                                   outputs=features, packed=packed), 2, 5)
+            grouped[name + "_" + label] = {
+                "us": round(seconds * 1e6, 1),
+                "useful_pflops": round(2.0 * experts * fill * features * inner / seconds / 1e15, 3)}
+        del parts, table, tokens, token_scale
+    found["mx_grouped_32_experts_4096x7168_capacity_1024"] = grouped
+    # decode attention when the cache is larger than the sequences: 32 sequences of 512 positions in a
+    # cache of 8192 (64 query heads, 8 KV heads of 128)
+    cache_k = normal((32, 8192, 8, 128))
+    cache_v = normal((32, 8192, 8, 128))
+    query = normal((32, 64, 128))
+    live = torch.full((32,), 512, dtype=torch.int32, device=device)
+    seconds = event_time(torch, lambda i: _kernels.gqa_decode_attention(query, cache_k, cache_v, live), 3, 10)
+    found["gqa_decode_512_live_of_8192"] = {
+        "us": round(seconds * 1e6, 1),
+        "tb_per_s_of_live_cache": round(2 * 32 * 512 * 8 * 128 * 2 / seconds / 1e12, 2)}
+    del cache_k, cache_v, query
     del copies, w_scale
     # FP32 SGEMM 2048^3 (plumbing)
     size = 2048
