@@ -153,6 +153,14 @@ extern "C" int camblas_cuda_create(int device, void *stream, camblas_cuda_contex
         return -1;
     }
     context->compute_units = properties.multiProcessorCount;
+    // the allocation-free attention entry point's fixed array: find this device's copy now, so
+    // that the entry point itself never has to ask the runtime
+    void *resident = nullptr;
+    status = gqa_resident_scratch(device, &resident);
+    if (status != hipSuccess) {
+        delete context;
+        return fail(nullptr, "resident scratch address", status);
+    }
     *out = context;
     return 0;
 }
@@ -1146,6 +1154,40 @@ extern "C" int camblas_cuda_rope_kv_append(camblas_cuda_context *context, int ba
     });
 }
 
+namespace camblas_hip
+{
+namespace
+{
+// Shared by the two decode-attention entry points: argument checks, then the launch with the
+// partials wherever `partials_for(bytes, &where)` puts them.
+template <typename Partials>
+int gqa_decode(camblas_cuda_context *context, int batch, int q_heads, int kv_heads, int dim,
+               int context_length, const int32_t *lengths, float scale, const void *q, int q_stride,
+               const void *k_cache, const void *v_cache, void *output, Partials partials_for)
+{
+    if (batch < 0 || q_heads < 1 || kv_heads < 1 || q_heads % kv_heads || q_heads / kv_heads > 16 ||
+        dim != 128 || context_length < 1 || q_stride < q_heads * dim || !std::isfinite(scale))
+        return fail(context, "invalid decode attention arguments", 1);
+    if (!batch)
+        return 0;
+    if (!q || !k_cache || !v_cache || !output || !aligned(q, 16) || !aligned(k_cache, 16) ||
+        !aligned(v_cache, 16) || !aligned(output, 16) || q_stride % 8 || output == q ||
+        output == k_cache || output == v_cache)
+        return fail(context, "invalid decode attention buffers", 1);
+    int splits = 1;
+    const size_t bytes = gqa_decode_scratch_bytes(batch, q_heads, dim, context_length, &splits);
+    void *partials = nullptr;
+    if (int refused = partials_for(bytes, &partials))
+        return refused;
+    context->counts[6]++;
+    hipError_t error =
+        launch_gqa_decode(context->stream, batch, q_heads, kv_heads, dim, context_length, lengths,
+                          scale, q, q_stride, k_cache, v_cache, output, partials, splits);
+    return error == hipSuccess ? 0 : fail(context, "decode attention", error);
+}
+} // namespace
+} // namespace camblas_hip
+
 extern "C" int camblas_cuda_gqa_decode_attention(camblas_cuda_context *context, int batch,
                                                  int q_heads, int kv_heads, int dim,
                                                  int context_length, const int32_t *lengths,
@@ -1154,26 +1196,46 @@ extern "C" int camblas_cuda_gqa_decode_attention(camblas_cuda_context *context, 
                                                  void *output)
 {
     return execute(context, [&] {
-        if (batch < 0 || q_heads < 1 || kv_heads < 1 || q_heads % kv_heads ||
-            q_heads / kv_heads > 16 || dim != 128 || context_length < 1 ||
-            q_stride < q_heads * dim || !std::isfinite(scale))
-            return fail(context, "invalid decode attention arguments", 1);
-        if (!batch)
-            return 0;
-        if (!q || !k_cache || !v_cache || !output || !aligned(q, 16) || !aligned(k_cache, 16) ||
-            !aligned(v_cache, 16) || !aligned(output, 16) || q_stride % 8 || output == q ||
-            output == k_cache || output == v_cache)
-            return fail(context, "invalid decode attention buffers", 1);
-        int splits = 1;
-        size_t bytes = gqa_decode_scratch_bytes(batch, q_heads, dim, context_length, &splits);
-        hipError_t grown = reserve_scratch(context, bytes);
-        if (grown != hipSuccess)
-            return fail(context, "decode attention scratch", grown);
-        context->counts[6]++;
-        hipError_t error = launch_gqa_decode(context->stream, batch, q_heads, kv_heads, dim,
-                                             context_length, lengths, scale, q, q_stride, k_cache,
-                                             v_cache, output, context->scratch, splits);
-        return error == hipSuccess ? 0 : fail(context, "decode attention", error);
+        return gqa_decode(context, batch, q_heads, kv_heads, dim, context_length, lengths, scale, q,
+                          q_stride, k_cache, v_cache, output, [&](size_t bytes, void **where) {
+                              hipError_t grown = reserve_scratch(context, bytes);
+                              if (grown != hipSuccess)
+                                  return fail(context, "decode attention scratch", grown);
+                              *where = context->scratch;
+                              return 0;
+                          });
+    });
+}
+
+extern "C" size_t camblas_cuda_gqa_decode_attention_noalloc_limit(void)
+{
+    return gqa_resident_scratch_bytes();
+}
+
+// The same kernels with the partials in the library's fixed device array: no hipMalloc, no
+// hipFree, no context scratch. Calls that overlap on one GPU share that array and race.
+extern "C" int camblas_cuda_gqa_decode_attention_noalloc(camblas_cuda_context *context, int batch,
+                                                         int q_heads, int kv_heads, int dim,
+                                                         int context_length, const int32_t *lengths,
+                                                         float scale, const void *q, int q_stride,
+                                                         const void *k_cache, const void *v_cache,
+                                                         void *output)
+{
+    return execute(context, [&] {
+        return gqa_decode(context, batch, q_heads, kv_heads, dim, context_length, lengths, scale, q,
+                          q_stride, k_cache, v_cache, output, [&](size_t bytes, void **where) {
+                              if (bytes > gqa_resident_scratch_bytes()) {
+                                  std::snprintf(context->error, sizeof(context->error),
+                                                "decode attention needs %zu bytes of partials; the "
+                                                "allocation-free entry point holds %zu",
+                                                bytes, gqa_resident_scratch_bytes());
+                                  return -1;
+                              }
+                              hipError_t found = gqa_resident_scratch(context->device, where);
+                              return found == hipSuccess
+                                         ? 0
+                                         : fail(context, "resident decode attention partials", found);
+                          });
     });
 }
 

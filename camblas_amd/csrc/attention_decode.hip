@@ -23,11 +23,22 @@
 #include "common.hpp"
 #include "device.hpp"
 
+#include <atomic>
+
 namespace camblas_hip
 {
 namespace
 {
 constexpr int DIM = 128, CHUNK = 256, WAVES = 4, WAVE_POSITIONS = CHUNK / WAVES, HEADS = 16;
+
+// Partials of the allocation-free entry point: one fixed array in the library's device image, so
+// every GPU that loads the library holds its own 16 MiB copy until the process ends. The name is
+// a host-side stand-in, not a device address: host code only ever uses the per-device address
+// that hipGetSymbolAddress returned (resident_partials below).
+constexpr size_t RESIDENT_BYTES = size_t(16) << 20;
+constexpr int MAX_DEVICES = 64;
+static __device__ __align__(256) unsigned char scratch[RESIDENT_BYTES];
+std::atomic<void *> resident_address[MAX_DEVICES] = {};
 
 __device__ __forceinline__ float swap_lanes(float value, int mask)
 {
@@ -255,9 +266,34 @@ size_t gqa_decode_scratch_bytes(int batch, int q_heads, int dim, int context_len
     return rows * (size_t(dim) + 2) * sizeof(float);
 }
 
+size_t gqa_resident_scratch_bytes() { return RESIDENT_BYTES; }
+
+// Address of this device's copy of the fixed partials array. `device` must be the current device
+// (every entry point runs under the context's device scope). Resolved once per device; later
+// calls are one atomic load and touch no runtime API.
+hipError_t gqa_resident_scratch(int device, void **address)
+{
+    *address = nullptr;
+    if (device < 0 || device >= MAX_DEVICES)
+        return hipErrorInvalidDevice;
+    void *known = resident_address[device].load(std::memory_order_acquire);
+    if (!known) {
+        hipError_t status = hipGetSymbolAddress(&known, HIP_SYMBOL(scratch));
+        if (status != hipSuccess) {
+            (void)hipGetLastError();
+            return status;
+        }
+        if (!known)
+            return hipErrorInvalidSymbol;
+        resident_address[device].store(known, std::memory_order_release);
+    }
+    *address = known;
+    return hipSuccess;
+}
+
 hipError_t launch_gqa_decode(hipStream_t stream, int batch, int q_heads, int kv_heads, int dim,
                              int context_length, const int32_t *lengths, float scale, const void *q,
-                             int q_stride, const void *k, const void *v, void *out, void *scratch,
+                             int q_stride, const void *k, const void *v, void *out, void *partials,
                              int splits)
 {
     const int group = kv_heads > 0 ? q_heads / kv_heads : 0;
@@ -265,7 +301,7 @@ hipError_t launch_gqa_decode(hipStream_t stream, int batch, int q_heads, int kv_
         group > HEADS)
         return hipErrorInvalidValue;
     size_t rows = size_t(batch) * q_heads * splits;
-    float *part_o = static_cast<float *>(scratch);
+    float *part_o = static_cast<float *>(partials);
     float *part_m = part_o + rows * DIM;
     float *part_l = part_m + rows;
     dim3 grid(splits, kv_heads, batch);

@@ -212,8 +212,12 @@ hipError_t launch_rope_kv_append(hipStream_t stream, int batch, int q_heads, int
 hipError_t launch_rope(hipStream_t stream, int tokens, int heads, int dim, int token_stride,
                        float theta, const int32_t *positions, void *x);
 size_t gqa_decode_scratch_bytes(int batch, int q_heads, int dim, int context_length, int *splits);
+// Fixed device array for the allocation-free attention entry point: its size, and its address on
+// `device` (which must be current; resolved with hipGetSymbolAddress on first use per device).
+size_t gqa_resident_scratch_bytes();
+hipError_t gqa_resident_scratch(int device, void **address);
 hipError_t launch_gqa_decode(hipStream_t stream, int batch, int q_heads, int kv_heads, int dim,
                              int context_length, const int32_t *lengths, float scale, const void *q,
-                             int q_stride, const void *k, const void *v, void *out, void *scratch,
+                             int q_stride, const void *k, const void *v, void *out, void *partials,
                              int splits);
 } // namespace camblas_hip

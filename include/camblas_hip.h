@@ -278,6 +278,22 @@ int camblas_cuda_gqa_decode_attention(camblas_cuda_context *context, int batch, 
                                       const int32_t *lengths, float scale, const void *q,
                                       int q_stride, const void *k_cache, const void *v_cache,
                                       void *output);
+/* No counterpart in the reference. camblas_cuda_gqa_decode_attention for callers that cannot
+ * allocate device memory (code under HIP graph capture on a context that has not grown its scratch
+ * yet, tight serving loops, harnesses that forbid hipMalloc): same arguments, same kernels, same
+ * results, but the split partials live in a fixed 16 MiB device array inside the library instead
+ * of context scratch, and the call performs no hipMalloc / hipFree. A call whose partials
+ * (batch * q_heads * ceil(context_length / 256) * 520 bytes) exceed
+ * camblas_cuda_gqa_decode_attention_noalloc_limit() fails with a message and launches nothing.
+ * Every GPU holds one such array for the life of the process and all contexts on that GPU share
+ * it: calls that overlap in time on one GPU (different streams or threads) race. Nothing in it
+ * has to start at zero: each call writes every partial it later reads. */
+int camblas_cuda_gqa_decode_attention_noalloc(camblas_cuda_context *context, int batch, int q_heads,
+                                              int kv_heads, int dim, int context_length,
+                                              const int32_t *lengths, float scale, const void *q,
+                                              int q_stride, const void *k_cache,
+                                              const void *v_cache, void *output);
+size_t camblas_cuda_gqa_decode_attention_noalloc_limit(void);
 
 /* extension (the reference runs this step from Python on Triton kernels, camblas/_hopper.py:329-401,
  * behind its SGLang hook camblas/sglang.py:340-455; here it is an entry point like the other
