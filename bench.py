@@ -215,6 +215,22 @@ def main():
     print(json.dumps(result))
 
 
+def probes():
+    """The bench-side calibration library (a copy of known traffic, a stream of matrix instructions);
+    built by camblas_amd._build.build_probes(), never part of libcamblas_hip.so."""
+    import ctypes as ct
+
+    if not hasattr(probes, "library"):
+        from camblas_amd import _native
+
+        lib = ct.CDLL(str(_native.library_path().parent / "libcamblas_probes.so"))
+        lib.camblas_probe_copy.argtypes = [ct.c_void_p, ct.c_size_t, ct.c_void_p, ct.c_void_p]
+        lib.camblas_probe_matrix.argtypes = [ct.c_void_p, ct.c_int, ct.c_int, ct.c_int, ct.c_int,
+                                             ct.c_void_p, ct.c_size_t, ct.POINTER(ct.c_double)]
+        probes.library = lib
+    return probes.library
+
+
 def measured_traffic():
     """HBM bytes per M=32 launch from the committed counter profile (FETCH_SIZE + WRITE_SIZE, each
     scaled by the copy-probe calibration), or None when that profile has not been taken."""
@@ -242,8 +258,10 @@ def profile_only(args, torch, _kernels, _native, device, normal, weights, inputs
         native = _native.context(device)
 
         def launch(i):
-            native.call("hip_copy_probe", size, ct.c_void_p(source.data_ptr()),
-                        ct.c_void_p(target.data_ptr()))
+            status = probes().camblas_probe_copy(
+                ct.c_void_p(torch.cuda.current_stream(device).cuda_stream), size,
+                ct.c_void_p(source.data_ptr()), ct.c_void_p(target.data_ptr()))
+            assert status == 0, status
     elif args.only.startswith("fp8m") and args.only != "fp8moe":
         tokens, features, inner = int(args.only[4:]), 18432, 7168
         rotate = 3 if tokens <= 256 else 1
@@ -497,7 +515,8 @@ def extras(torch, _kernels, _native, device, normal):
     import ctypes as ct
 
     native = _native.context(device)
-    sink = torch.empty(4096 * 512, dtype=torch.float32, device=device)
+    units = torch.cuda.get_device_properties(device).multi_processor_count
+    sink = torch.empty(units * 512, dtype=torch.float32, device=device)
     flops = ct.c_double(0.0)
     sustained = {}
     # (rounds sized for launches of 2-3 ms, long enough for the clock to settle)
@@ -506,8 +525,9 @@ def extras(torch, _kernels, _native, device, normal):
         entry = {}
         for operands, constant in (("varied", 0), ("constant", 1)):
             seconds = event_time(
-                torch, lambda i: native.call("hip_matrix_probe", kind, rounds, constant,
-                                             ct.c_void_p(sink.data_ptr()), sink.numel() * 4, ct.byref(flops)),
+                torch, lambda i: probes().camblas_probe_matrix(
+                    ct.c_void_p(torch.cuda.current_stream(device).cuda_stream), kind, units, rounds, constant,
+                    ct.c_void_p(sink.data_ptr()), sink.numel() * 4, ct.byref(flops)),
                 2, 5)
             entry[operands + "_operands_tflops"] = round(flops.value / seconds / 1e12, 1)
         sustained[name] = entry

@@ -21,8 +21,12 @@ CORE = LIB_DIR / "libcamblas_hip.so"
 HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
 
 CORE_SOURCES = (
-    "abi.hip",
+    "abi_context.hip",
+    "abi_dense.hip",
+    "abi_fusion.hip",
+    "abi_quantized.hip",
     "planner.cpp",
+    "bgemm_any.hip",
     "gemm_generic.hip",
     "gemv_f32.hip",
     "bgemm_tn.hip",
@@ -37,7 +41,6 @@ CORE_SOURCES = (
     "mx_dma.hip",
     "routing.hip", "dense_ops.hip", "sgemm_mfma.hip", "dgemm_mfma.hip", "strassen.hip",
     "fusion.hip",
-    "probes.hip",
     "attention_decode.hip",
 )
 
@@ -96,8 +99,21 @@ def build_core(jobs=8, verbose=False):
     return CORE
 
 
-def build_tensor_binding():
-    """Compile csrc/tensor_binding.cpp (host code only: ATen + pybind11 + the C ABI) into
+def build_probes():
+    """Compile csrc/bench_probes.hip into lib/libcamblas_probes.so: calibration launches (a copy of
+    known traffic, a stream of matrix instructions) that bench.py loads; not part of the product
+    library."""
+    target = LIB_DIR / "libcamblas_probes.so"
+    LIB_DIR.mkdir(parents=True, exist_ok=True)
+    _run([HIPCC, *HIP_FLAGS, "-shared", CSRC / "bench_probes.hip", "-o", target])
+    return target
+
+
+BINDING_SOURCES = ("tensor_binding.cpp", "binding_dense.cpp", "binding_fusion.cpp", "binding_quantized.cpp")
+
+
+def build_tensor_binding(jobs=4):
+    """Compile the binding units (host code only: ATen + pybind11 + the C ABI) into
     lib/_camblas_cuda_torch<ext>.so, linked against libcamblas_hip.so beside it."""
     import sysconfig
 
@@ -111,13 +127,26 @@ def build_tensor_binding():
     includes += [f"-I{sysconfig.get_paths()['include']}", "-I/opt/rocm/include",
                  f"-I{ROOT / 'include'}"]
     abi = int(torch._C._GLIBCXX_USE_CXX11_ABI)
+    compiler = os.environ.get("CXX", "g++")
+    flags = [
+        "-O2", "-std=c++17", "-fPIC", "-Wall", "-Wno-unused-function", "-Wno-deprecated-declarations",
+        "-D__HIP_PLATFORM_AMD__=1", "-DUSE_ROCM=1", f"-D_GLIBCXX_USE_CXX11_ABI={abi}",
+        "-DTORCH_API_INCLUDE_EXTENSION_H", "-DTORCH_EXTENSION_NAME=_camblas_cuda_torch", *includes,
+        f"-I{CSRC}",
+    ]
+    objects = LIB_DIR / "obj"
+    objects.mkdir(parents=True, exist_ok=True)
+
+    def compile_unit(name):
+        unit = objects / (Path(name).stem + ".binding.o")
+        _run([compiler, *flags, "-c", CSRC / name, "-o", unit])
+        return unit
+
+    with ThreadPoolExecutor(max_workers=jobs) as pool:
+        units = list(pool.map(compile_unit, BINDING_SOURCES))
     command = [
-        os.environ.get("CXX", "g++"), "-O2", "-std=c++17", "-fPIC", "-shared", "-Wall",
-        "-Wno-unused-function", "-Wno-deprecated-declarations", "-D__HIP_PLATFORM_AMD__=1",
-        "-DUSE_ROCM=1", f"-D_GLIBCXX_USE_CXX11_ABI={abi}", "-DTORCH_API_INCLUDE_EXTENSION_H",
-        "-DTORCH_EXTENSION_NAME=_camblas_cuda_torch", *includes, CSRC / "tensor_binding.cpp",
-        "-o", target, f"-L{LIB_DIR}", "-lcamblas_hip", f"-L{torch_lib}", "-ltorch_python",
-        "-ltorch", "-ltorch_cpu", "-ltorch_hip", "-lc10", "-lc10_hip", "-L/opt/rocm/lib",
+        compiler, "-shared", *units, "-o", target, f"-L{LIB_DIR}", "-lcamblas_hip", f"-L{torch_lib}",
+        "-ltorch_python", "-ltorch", "-ltorch_cpu", "-ltorch_hip", "-lc10", "-lc10_hip", "-L/opt/rocm/lib",
         "-lamdhip64", "-Wl,-rpath,$ORIGIN", f"-Wl,-rpath,{torch_lib}",
     ]
     _run(command)
@@ -126,5 +155,6 @@ def build_tensor_binding():
 
 if __name__ == "__main__":
     print(build_core(verbose=True))
+    print(build_probes())
     if "--no-binding" not in sys.argv:
         print(build_tensor_binding())

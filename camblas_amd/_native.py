@@ -88,8 +88,6 @@ SIGNATURES = {
     "hip_plan_describe": ([_I, _I, _C, _C, _I, _I, _I, _I, _I, _I, _I, ct.c_char_p, _SZ], _I),
     "hip_set_plan_override": ([_P, _I, _I], _I),
     "hip_kernel_count": ([_I], _I),
-    "hip_copy_probe": ([_P, _SZ, _P, _P], _I),
-    "hip_matrix_probe": ([_P, _I, _I, _I, _P, _SZ, ct.POINTER(ct.c_double)], _I),
 }
 
 

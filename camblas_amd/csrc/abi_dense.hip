@@ -1,0 +1,527 @@
+// The GEMM family of the C ABI: sgemm / dgemm / bgemm and the FP32 / FP64 helpers composed from them
+// (affine, mlp, dense attention, mlp_backward). Argument rules and their order follow the
+// reference (src/cuda/backend.cu:786-866 for the dense product, src/cuda/bfloat16.cuh:11-57 for
+// BF16, :871-905 and src/cuda/fusion.cuh:95-157, :207-275 for the helpers); every kernel is this
+// library's own.
+#include "entry.hpp"
+
+#include <algorithm>
+#include <cmath>
+#include <limits>
+
+namespace camblas_hip
+{
+namespace
+{
+// The shape part of a column-major product C[m, n] = alpha op(A) op(B) + beta C.
+struct Product {
+    int trans_a, trans_b; // 0 'N', 1 'T', -1 neither
+    int m, n, k, lda, ldb, ldc;
+
+    Product(char ta, char tb, int m_, int n_, int k_, int lda_, int ldb_, int ldc_)
+        : trans_a(transposition(ta)), trans_b(transposition(tb)), m(m_), n(n_), k(k_), lda(lda_),
+          ldb(ldb_), ldc(ldc_)
+    {
+    }
+    bool well_formed() const
+    {
+        return trans_a >= 0 && trans_b >= 0 && m >= 0 && n >= 0 && k >= 0 && lda >= 1 && ldb >= 1 && ldc >= 1;
+    }
+    bool empty() const { return m == 0 || n == 0; }
+    // a leading dimension covers the stored rows of its operand (at least 1)
+    bool strides_cover() const
+    {
+        return lda >= std::max(1, trans_a ? k : m) && ldb >= std::max(1, trans_b ? n : k) && ldc >= m;
+    }
+};
+
+// What the three GEMM entry points share: the reference's order of checks. `names` are the three
+// failure texts (arguments, output/strides, operands). Returns 1 when the caller should go on to
+// launch the product, 0 when the call is complete, negative on failure.
+template <typename Scalar, typename ScaleOutput>
+int admit_product(const Entry &entry, const Product &p, Scalar alpha, Scalar beta, const void *a,
+                  const void *b, const void *c, const char *const (&names)[4], ScaleOutput scale_output)
+{
+    if (!p.well_formed())
+        return entry.refuse(names[0]);
+    if (p.empty())
+        return 0;
+    if (!c || !p.strides_cover())
+        return entry.refuse(names[1]);
+    if (alpha == Scalar(0) || p.k == 0) { // only beta acts; beta == 0 writes zeros without reading C
+        if (beta == Scalar(1))
+            return 0;
+        return entry.finish(scale_output(), names[2]);
+    }
+    if (!a || !b || a == c || b == c)
+        return entry.refuse(names[3]);
+    return 1;
+}
+
+// C = A A^T or A^T A over the whole of C under the symmetric policy (ref: backend.cu:819-835): the
+// tiles that reach the diagonal are computed and the rest mirrored, so C equals its transpose
+// bit for bit.
+bool is_gram(const camblas_cuda_context *context, const Product &p, const void *a, const void *b,
+             bool overwrites)
+{
+    return context->algorithm == CAMBLAS_CUDA_SYMMETRIC && a == b && p.trans_a != p.trans_b &&
+           p.m == p.n && p.lda == p.ldb && overwrites;
+}
+
+// square, untransposed, even, at least 256: the products the Strassen policies split
+// (ref: backend.cu:843-853)
+int strassen_depth(const camblas_cuda_context *context, const Product &p)
+{
+    if (p.trans_a || p.trans_b || p.m != p.n || p.n != p.k || p.n % 2 || p.n < 256)
+        return 0;
+    return strassen_levels(context->algorithm, p.n);
+}
+
+template <typename T> struct Kernels;
+
+template <> struct Kernels<float> {
+    static constexpr int dtype = 0;
+    static hipError_t scale(hipStream_t s, const Product &p, float beta, float *c)
+    {
+        return launch_scale_f32(s, p.m, p.n, beta, c, p.ldc);
+    }
+    static hipError_t vector(hipStream_t s, const Product &p, float alpha, const float *a, const float *b,
+                             float beta, float *c)
+    {
+        return launch_generic_f32(s, p.trans_a, p.trans_b, p.m, p.n, p.k, alpha, a, p.lda, b, p.ldb, beta, c,
+                                  p.ldc);
+    }
+    static bool matrix_worthwhile(const Product &p) { return p.m >= 32 && p.k >= 16; }
+    // 128 x 128 tiles once the tiles that reach the diagonal number two per compute unit
+    static hipError_t triangle(const camblas_cuda_context *context, const Product &p, float alpha,
+                               const float *a, const float *b, float beta, float *c)
+    {
+        const double rows = (p.n + 127) / 128;
+        const bool wide = rows * (rows + 1) / 2 >= 2.0 * context->compute_units;
+        return launch_sgemm_mfma(context->stream, wide, p.trans_a, p.trans_b, p.m, p.n, p.k, alpha, a, p.lda,
+                                 b, p.ldb, beta, c, p.ldc, 1, 0, true);
+    }
+};
+
+template <> struct Kernels<double> {
+    static constexpr int dtype = 1;
+    static hipError_t scale(hipStream_t s, const Product &p, double beta, double *c)
+    {
+        return launch_scale_f64(s, p.m, p.n, beta, c, p.ldc);
+    }
+    static hipError_t vector(hipStream_t s, const Product &p, double alpha, const double *a, const double *b,
+                             double beta, double *c)
+    {
+        return launch_generic_f64(s, p.trans_a, p.trans_b, p.m, p.n, p.k, alpha, a, p.lda, b, p.ldb, beta, c,
+                                  p.ldc);
+    }
+    static bool matrix_worthwhile(const Product &p) { return p.m >= 16 && p.k >= 4; }
+    static hipError_t triangle(const camblas_cuda_context *context, const Product &p, double alpha,
+                               const double *a, const double *b, double beta, double *c)
+    {
+        return launch_dgemm_mfma(context->stream, p.trans_a, p.trans_b, p.m, p.n, p.k, alpha, a, p.lda, b, p.ldb,
+                                 beta, c, p.ldc, 1, 0, true);
+    }
+};
+
+// the ordinary FP32 product: the planner's choice (decode GEMV, matrix-core tiles, vector-ALU tiles)
+int ordinary(const Entry &entry, const Product &p, float alpha, const float *a, const float *b, float beta,
+             float *c, bool classical_counter)
+{
+    camblas_cuda_context *context = entry.context();
+    Plan plan = make_plan(0, context->algorithm, p.trans_a, p.trans_b, p.m, p.n, p.k, p.lda, p.ldb, p.ldc,
+                          is_aligned(a, 16) && is_aligned(b, 16), context->compute_units);
+    context->counts[classical_counter ? 0 : plan.counter]++;
+    if (plan.family == FAMILY_GEMV_F32)
+        return entry.finish(launch_gemv_f32(context->stream, p.m, p.k, alpha, a, p.lda, b, beta, c),
+                            "FP32 native GEMV");
+    if (context->override_kernel >= 0) { // tests: 0 vector-ALU tiles, 1 / 2 matrix-core tiles
+        plan.family = context->override_kernel >= 1 ? FAMILY_MFMA_F32 : FAMILY_GENERIC;
+        plan.kernel = context->override_kernel == 2 ? 1 : 0;
+    }
+    const hipError_t launched =
+        plan.family == FAMILY_MFMA_F32
+            ? launch_sgemm_mfma(context->stream, plan.kernel == 0, p.trans_a, p.trans_b, p.m, p.n, p.k, alpha,
+                                a, p.lda, b, p.ldb, beta, c, p.ldc)
+            : Kernels<float>::vector(context->stream, p, alpha, a, b, beta, c);
+    return entry.finish(launched, "classical GEMM");
+}
+
+// the ordinary FP64 product: matrix cores when every dimension holds a 16 x 16 x 4 tile
+// (ref: backend.cu:1066-1073)
+int ordinary(const Entry &entry, const Product &p, double alpha, const double *a, const double *b,
+             double beta, double *c, bool)
+{
+    camblas_cuda_context *context = entry.context();
+    context->counts[0]++;
+    bool matrix = p.m >= 16 && p.n >= 16 && p.k >= 4;
+    if (context->override_kernel >= 0) // tests: 0 vector-ALU tiles, else matrix-core tiles
+        matrix = context->override_kernel >= 1;
+    const hipError_t launched =
+        matrix ? launch_dgemm_mfma(context->stream, p.trans_a, p.trans_b, p.m, p.n, p.k, alpha, a, p.lda, b,
+                                   p.ldb, beta, c, p.ldc)
+               : Kernels<double>::vector(context->stream, p, alpha, a, b, beta, c);
+    return entry.finish(launched, "classical FP64 GEMM");
+}
+
+// FP32 / FP64 product on the entry's stream: policies first (symmetric, Strassen), then the
+// ordinary kernels. Shared by the public entry points and by the helpers below.
+template <typename T>
+int dense_product(const Entry &entry, const Product &p, T alpha, const T *a, const T *b, T beta, T *c)
+{
+    static const char *const names[4] = {"invalid GEMM arguments",
+                                         "invalid device pointer or leading dimension", "scale output",
+                                         "missing or aliased GEMM operand"};
+    camblas_cuda_context *context = entry.context();
+    const int admitted = admit_product(entry, p, alpha, beta, a, b, c, names,
+                                       [&] { return Kernels<T>::scale(context->stream, p, beta, c); });
+    if (admitted <= 0)
+        return admitted;
+    if (is_gram(context, p, a, b, beta == T(0))) {
+        context->counts[2]++;
+        const hipError_t lower = Kernels<T>::matrix_worthwhile(p)
+                                     ? Kernels<T>::triangle(context, p, alpha, a, b, beta, c)
+                                     : Kernels<T>::vector(context->stream, p, alpha, a, b, beta, c);
+        if (lower != hipSuccess)
+            return entry.refuse("symmetric Gram", int(lower));
+        return entry.finish(launch_mirror_lower(context->stream, Kernels<T>::dtype, p.n, c, p.ldc),
+                            "Gram mirroring");
+    }
+    bool guarded = false; // the Strassen guard sent the call here: it counts as a classical product
+    if (const int depth = strassen_depth(context, p)) {
+        const int outcome = strassen_gemm(context, depth, p.n, alpha, a, p.lda, b, p.ldb, beta, c, p.ldc);
+        if (outcome != STRASSEN_FALL_BACK && outcome != STRASSEN_NOT_ELIGIBLE)
+            return outcome;
+        guarded = outcome == STRASSEN_FALL_BACK;
+    }
+    return ordinary(entry, p, alpha, a, b, beta, c, guarded);
+}
+
+// Row-major out[rows, columns] = x[rows, inner] weight[inner, columns] + bias, optional ReLU
+// (ref: backend.cu:871-905): the column-major product out^T = weight^T-view x^T-view, then one
+// bias / activation pass.
+template <typename T>
+int affine_layer(const Entry &entry, int rows, int inner, int columns, const T *x, const T *weight,
+                 const T *bias, bool relu, T *output)
+{
+    if (rows < 0 || inner < 0 || columns < 0)
+        return entry.refuse("invalid affine dimensions");
+    if (rows == 0 || columns == 0)
+        return 0;
+    if (!output || !bias || (inner > 0 && (!x || !weight)))
+        return entry.refuse("missing affine operand");
+    entry.context()->counts[3]++;
+    const Product p('N', 'N', columns, rows, inner, std::max(1, columns), std::max(1, inner), columns);
+    if (const int status = dense_product(entry, p, T(1), weight, x, T(0), output))
+        return status;
+    return entry.finish(launch_bias_activation(entry.stream(), Kernels<T>::dtype, output, bias,
+                                               size_t(rows) * columns, columns, relu),
+                        "bias/activation");
+}
+
+// softmax(scale q k^T) v with the score matrix in the context's scratch (ref: fusion.cuh:95-157)
+template <typename T>
+int score_attention(const Entry &entry, int queries, int keys, int depth, int values, T scale, const T *q,
+                    const T *k, const T *v, T *output)
+{
+    if (queries < 0 || keys < 0 || depth < 0 || values < 0)
+        return entry.refuse("invalid attention dimensions");
+    if (queries == 0 || values == 0)
+        return 0;
+    if (!output || (depth > 0 && !q) || (keys > 0 && depth > 0 && !k) || (keys > 0 && !v))
+        return entry.refuse("missing attention operand");
+    if (keys > 0 && size_t(queries) > std::numeric_limits<size_t>::max() / sizeof(T) / size_t(keys))
+        return entry.refuse("attention scratch size overflow", 2);
+    camblas_cuda_context *context = entry.context();
+    context->counts[6]++;
+    const hipError_t grown = reserve_scratch(context, size_t(queries) * keys * sizeof(T));
+    if (grown != hipSuccess)
+        return entry.refuse("attention scratch", int(grown));
+    T *scores = static_cast<T *>(context->scratch);
+    const int depth_ld = std::max(1, depth), keys_ld = std::max(1, keys), values_ld = std::max(1, values);
+    // scores[queries, keys] = q k^T; with no keys the second product just writes zeros
+    const Product score('T', 'N', keys, queries, depth, depth_ld, depth_ld, keys_ld);
+    if (const int status = dense_product(entry, score, T(1), k, q, T(0), scores))
+        return status;
+    const hipError_t softened =
+        launch_softmax_rows(context->stream, Kernels<T>::dtype, scores, queries, keys, double(scale));
+    if (softened != hipSuccess)
+        return entry.refuse("attention softmax", int(softened));
+    const Product mix('N', 'N', values, queries, keys, values_ld, keys_ld, values_ld);
+    return dense_product(entry, mix, T(1), v, scores, T(0), output);
+}
+
+// Gradients of output = relu(x w1 + b1) w2 + b2 (ref: fusion.cuh:207-275). A null gradient pointer
+// skips that gradient; grad_hidden is the caller's scratch and is left holding the masked gradient.
+template <typename T> struct BackwardPass {
+    const Entry &entry;
+    int rows, inputs, hidden, outputs;
+    const T *x, *w1, *w2, *h, *grad;
+    T *dh, *dx, *dw1, *db1, *dw2, *db2;
+
+    // column sums run over chunks of 128 rows; more than one chunk goes through context scratch
+    int chunks() const
+    {
+        return int(std::min<size_t>(65535, std::max<size_t>(1, (size_t(rows) + 127) / 128)));
+    }
+    int product(char ta, char tb, int m, int n, int k, const T *a, int lda, const T *b, int ldb, T *c,
+                int ldc) const
+    {
+        return dense_product(entry, Product(ta, tb, m, n, k, std::max(1, lda), std::max(1, ldb), std::max(1, ldc)),
+                             T(1), a, b, T(0), c);
+    }
+    int run() const
+    {
+        if (rows < 0 || inputs < 0 || hidden < 0 || outputs < 0)
+            return entry.refuse("invalid backward dimensions");
+        const bool first_layer = dx || dw1 || db1;
+        const bool needs_output_gradient = rows > 0 && outputs > 0;
+        const bool needs_hidden = rows > 0 && hidden > 0 && first_layer;
+        if ((needs_output_gradient && !grad) || (needs_hidden && (!dh || !h)))
+            return entry.refuse("missing backward operand");
+        camblas_cuda_context *context = entry.context();
+        context->counts[7]++;
+        const int parts = chunks(), part_rows = std::max(1, int((int64_t(rows) + parts - 1) / parts));
+        T *partial = nullptr;
+        if (parts > 1 && ((db2 && outputs > 0) || (db1 && hidden > 0))) {
+            const hipError_t grown =
+                reserve_scratch(context, size_t(parts) * std::max(hidden, outputs) * sizeof(T));
+            if (grown != hipSuccess)
+                return entry.refuse("backward scratch", int(grown));
+            partial = static_cast<T *>(context->scratch);
+        }
+        // second layer: dw2[hidden, outputs] = h^T grad, db2 = column sums of grad
+        if (dw2)
+            if (const int status = product('N', 'T', outputs, hidden, rows, grad, outputs, h, hidden, dw2, outputs))
+                return status;
+        if (db2 && outputs > 0) {
+            const hipError_t summed =
+                launch_column_sums(context->stream, Kernels<T>::dtype, false, const_cast<T *>(grad), nullptr, rows,
+                                   outputs, parts, part_rows, partial, db2);
+            if (summed != hipSuccess)
+                return entry.refuse("backward bias", int(summed));
+        }
+        if (!first_layer)
+            return 0;
+        // dh[rows, hidden] = grad w2^T, zeroed where the ReLU was inactive, summed over rows for db1
+        if (const int status = product('T', 'N', hidden, rows, outputs, w2, outputs, grad, outputs, dh, hidden))
+            return status;
+        if (hidden > 0) {
+            const hipError_t masked =
+                launch_column_sums(context->stream, Kernels<T>::dtype, true, dh, h, rows, hidden, parts, part_rows,
+                                   db1 ? partial : nullptr, db1);
+            if (masked != hipSuccess)
+                return entry.refuse("backward activation", int(masked));
+        }
+        if (dw1) // dw1[inputs, hidden] = x^T dh
+            if (const int status = product('N', 'T', hidden, inputs, rows, dh, hidden, x, inputs, dw1, hidden))
+                return status;
+        if (dx) // dx[rows, inputs] = dh w1^T
+            return product('T', 'N', inputs, rows, hidden, w1, hidden, dh, hidden, dx, inputs);
+        return 0;
+    }
+};
+
+// BF16 'T','N' and the other layouts: the planner's kernel, or the one a test forced.
+int bf16_product(const Entry &entry, const Product &p, float alpha, const void *a, const void *b, float beta,
+                 void *c)
+{
+    camblas_cuda_context *context = entry.context();
+    hipStream_t stream = context->stream;
+    Plan plan = make_plan(2, context->algorithm, p.trans_a, p.trans_b, p.m, p.n, p.k, p.lda, p.ldb, p.ldc,
+                          is_aligned(a, 16) && is_aligned(b, 16), context->compute_units);
+    if (plan.family == FAMILY_DMA && !is_aligned(c, 8))
+        plan.family = FAMILY_MFMA_TN; // same tile shapes, register-staged loads, scalar stores
+    const bool matrix_family =
+        plan.family == FAMILY_MFMA_TN || plan.family == FAMILY_STREAM || plan.family == FAMILY_DMA;
+    if (matrix_family && context->override_kernel >= 0) {
+        // tests: 0.. a register-staged tile variant (with override_split), 20..59 a direct-to-LDS
+        // variant, 100 + 100*depth + 10*row_tiles + token_tiles the streaming kernel
+        const int forced = context->override_kernel;
+        plan.split_k = 1;
+        if (forced >= 100) {
+            plan.family = FAMILY_STREAM;
+            plan.kernel = forced - 100;
+        } else if (forced >= 20 && forced < 60) {
+            plan.family = FAMILY_DMA;
+            plan.kernel = forced - 20;
+        } else {
+            plan.family = FAMILY_MFMA_TN;
+            plan.kernel = forced;
+            plan.split_k = std::max(1, context->override_split);
+        }
+    }
+    switch (plan.family) {
+    case FAMILY_DMA:
+        context->counts[plan.counter]++;
+        return entry.finish(launch_bgemm_dma(stream, plan.kernel, p.m, p.n, p.k, alpha, a, p.lda, b, p.ldb, beta,
+                                             c, p.ldc),
+                            "BF16 MFMA GEMM (direct LDS loads)");
+    case FAMILY_STREAM:
+        context->counts[plan.counter]++;
+        return entry.finish(launch_bgemv_stream(stream, plan.kernel / 100, plan.kernel / 10 % 10,
+                                                plan.kernel % 10, p.m, p.n, p.k, alpha, a, p.lda, b, p.ldb,
+                                                beta, c, p.ldc),
+                            "BF16 streaming GEMV");
+    case FAMILY_MFMA_TN: {
+        float *partials = nullptr;
+        if (plan.split_k > 1) {
+            // without room for the partials (allocation failure, capture in progress) run unsplit
+            if (reserve_scratch(context, size_t(plan.split_k) * size_t(p.m) * size_t(p.n) * 4) == hipSuccess) {
+                partials = static_cast<float *>(context->scratch);
+            } else {
+                context->counts[5]++;
+                plan.split_k = 1;
+            }
+        }
+        context->counts[plan.counter]++;
+        return entry.finish(launch_bgemm_tn(stream, plan.kernel, plan.split_k, p.m, p.n, p.k, alpha, a, p.lda, b,
+                                            p.ldb, beta, c, p.ldc, partials),
+                            "BF16 MFMA GEMM");
+    }
+    case FAMILY_MFMA_BF16:
+        context->counts[plan.counter]++;
+        return entry.finish(launch_bgemm_any(stream, plan.kernel == 0, p.trans_a, p.trans_b, p.m, p.n, p.k, alpha,
+                                             a, p.lda, b, p.ldb, beta, c, p.ldc),
+                            "BF16 MFMA GEMM (any layout)");
+    default:
+        context->counts[0]++;
+        return entry.finish(launch_generic_bf16(stream, p.trans_a, p.trans_b, p.m, p.n, p.k, alpha, a, p.lda, b,
+                                                p.ldb, beta, c, p.ldc),
+                            "BF16 GEMM");
+    }
+}
+
+template <typename T>
+int typed_gemm(camblas_cuda_context *context, char ta, char tb, int m, int n, int k, T alpha, const T *a,
+               int lda, const T *b, int ldb, T beta, T *c, int ldc)
+{
+    Entry entry(context);
+    return entry.run(
+        [&] { return dense_product(entry, Product(ta, tb, m, n, k, lda, ldb, ldc), alpha, a, b, beta, c); });
+}
+} // namespace
+} // namespace camblas_hip
+
+using namespace camblas_hip;
+
+extern "C" int camblas_cuda_sgemm(camblas_cuda_context *context, char ta, char tb, int m, int n,
+                                  int k, float alpha, const float *a, int lda, const float *b,
+                                  int ldb, float beta, float *c, int ldc)
+{
+    return typed_gemm(context, ta, tb, m, n, k, alpha, a, lda, b, ldb, beta, c, ldc);
+}
+
+extern "C" int camblas_cuda_dgemm(camblas_cuda_context *context, char ta, char tb, int m, int n,
+                                  int k, double alpha, const double *a, int lda, const double *b,
+                                  int ldb, double beta, double *c, int ldc)
+{
+    return typed_gemm(context, ta, tb, m, n, k, alpha, a, lda, b, ldb, beta, c, ldc);
+}
+
+extern "C" int camblas_cuda_bgemm(camblas_cuda_context *context, char trans_a, char trans_b, int m,
+                                  int n, int k, float alpha, const void *a, int lda, const void *b,
+                                  int ldb, float beta, void *c, int ldc)
+{
+    static const char *const names[4] = {"invalid BF16 GEMM arguments",
+                                         "invalid BF16 pointer or leading dimension", "scale BF16 output",
+                                         "missing or aliased BF16 GEMM operand"};
+    Entry entry(context);
+    return entry.run([&] {
+        const Product p(trans_a, trans_b, m, n, k, lda, ldb, ldc);
+        const int admitted = admit_product(entry, p, alpha, beta, a, b, c, names, [&] {
+            return launch_scale_bf16(context->stream, m, n, beta, c, ldc);
+        });
+        return admitted <= 0 ? admitted : bf16_product(entry, p, alpha, a, b, beta, c);
+    });
+}
+
+extern "C" int camblas_cuda_affine(camblas_cuda_context *context, int dtype, int rows, int inner,
+                                   int columns, const void *x, const void *weight, const void *bias,
+                                   int relu, void *output)
+{
+    Entry entry(context);
+    return entry.run([&] {
+        switch (dtype) {
+        case 0:
+            return affine_layer(entry, rows, inner, columns, static_cast<const float *>(x),
+                                static_cast<const float *>(weight), static_cast<const float *>(bias), relu != 0,
+                                static_cast<float *>(output));
+        case 1:
+            return affine_layer(entry, rows, inner, columns, static_cast<const double *>(x),
+                                static_cast<const double *>(weight), static_cast<const double *>(bias), relu != 0,
+                                static_cast<double *>(output));
+        default:
+            return entry.refuse("unsupported affine dtype");
+        }
+    });
+}
+
+// two affine layers, the first with ReLU; the hidden activations are an output of their own and
+// may not share storage with the result (ref: backend.cu:1103-1117)
+extern "C" int camblas_cuda_mlp(camblas_cuda_context *context, int dtype, int rows, int inputs,
+                                int hidden, int outputs, const void *x, const void *w1,
+                                const void *b1, const void *w2, const void *b2, void *hidden_output,
+                                void *output)
+{
+    const bool shares_storage = rows > 0 && hidden > 0 && hidden_output == output;
+    if (rows < 0 || inputs < 0 || hidden < 0 || outputs < 0 || shares_storage)
+        return fail(context, "invalid MLP dimensions or aliased outputs", 1);
+    if (const int status = camblas_cuda_affine(context, dtype, rows, inputs, hidden, x, w1, b1, 1, hidden_output))
+        return status;
+    return camblas_cuda_affine(context, dtype, rows, hidden, outputs, hidden_output, w2, b2, 0, output);
+}
+
+extern "C" int camblas_cuda_attention(camblas_cuda_context *context, int dtype, int queries, int keys,
+                                      int depth, int values, double scale, const void *q,
+                                      const void *k, const void *v, void *output)
+{
+    Entry entry(context);
+    return entry.run([&] {
+        switch (dtype) {
+        case 0:
+            return score_attention(entry, queries, keys, depth, values, float(scale),
+                                   static_cast<const float *>(q), static_cast<const float *>(k),
+                                   static_cast<const float *>(v), static_cast<float *>(output));
+        case 1:
+            return score_attention(entry, queries, keys, depth, values, scale, static_cast<const double *>(q),
+                                   static_cast<const double *>(k), static_cast<const double *>(v),
+                                   static_cast<double *>(output));
+        default:
+            return entry.refuse("unsupported attention dtype");
+        }
+    });
+}
+
+extern "C" int camblas_cuda_mlp_backward(camblas_cuda_context *context, int dtype, int rows,
+                                         int inputs, int hidden, int outputs, const void *x,
+                                         const void *w1, const void *w2, const void *hidden_output,
+                                         const void *grad_output, void *grad_hidden, void *dx,
+                                         void *dw1, void *db1, void *dw2, void *db2)
+{
+    Entry entry(context);
+    return entry.run([&] {
+        switch (dtype) {
+        case 0: {
+            using T = float;
+            return BackwardPass<T>{entry, rows, inputs, hidden, outputs, static_cast<const T *>(x),
+                                   static_cast<const T *>(w1), static_cast<const T *>(w2),
+                                   static_cast<const T *>(hidden_output), static_cast<const T *>(grad_output),
+                                   static_cast<T *>(grad_hidden), static_cast<T *>(dx), static_cast<T *>(dw1),
+                                   static_cast<T *>(db1), static_cast<T *>(dw2), static_cast<T *>(db2)}
+                .run();
+        }
+        case 1: {
+            using T = double;
+            return BackwardPass<T>{entry, rows, inputs, hidden, outputs, static_cast<const T *>(x),
+                                   static_cast<const T *>(w1), static_cast<const T *>(w2),
+                                   static_cast<const T *>(hidden_output), static_cast<const T *>(grad_output),
+                                   static_cast<T *>(grad_hidden), static_cast<T *>(dx), static_cast<T *>(dw1),
+                                   static_cast<T *>(db1), static_cast<T *>(dw2), static_cast<T *>(db2)}
+                .run();
+        }
+        default:
+            return entry.refuse("unsupported backward dtype");
+        }
+    });
+}

@@ -1,0 +1,333 @@
+// Elementwise and row-wise entry points of the C ABI (SiLU-multiply, SwiGLU, the RMS normalisation
+// family) and the decode-layer pieces the reference has no counterpart for (rotary embedding,
+// cache append, grouped-query decode attention). What each call rejects follows the reference's
+// wrappers, read as text: src/cuda/backend.cu:1119-1163 (activations), :1363-1475 (normalisation).
+#include "entry.hpp"
+
+#include <cmath>
+#include <cstdint>
+
+namespace camblas_hip
+{
+namespace
+{
+bool valid_epsilon(float epsilon) { return std::isfinite(epsilon) && epsilon >= 0; }
+
+// the single-row kernels of the reference accept widths 2048 .. 65536 in multiples of four
+bool decode_width(int width) { return within({{width, 2048, 65536, 4}}); }
+
+// count elements of `dtype` fit in a size_t
+bool countable(uint64_t count, int dtype) { return count <= SIZE_MAX / storage_bytes(dtype); }
+} // namespace
+} // namespace camblas_hip
+
+using namespace camblas_hip;
+
+extern "C" int camblas_cuda_silu_multiply(camblas_cuda_context *context, int dtype, uint64_t count,
+                                          const void *gate, const void *up, void *output)
+{
+    Entry entry(context);
+    return entry.run([&] {
+        if (!storage_in(dtype, {0, 2}))
+            return entry.refuse("unsupported SiLU dtype");
+        if (count == 0)
+            return 0;
+        if (!usable({{gate, 1}, {up, 1}, {output, 1}}) || !countable(count, dtype))
+            return entry.refuse("invalid SiLU operands or length");
+        return entry.finish(launch_silu_multiply(entry.stream(), dtype, count, gate, up, output), "SiLU multiply");
+    });
+}
+
+extern "C" int camblas_cuda_swiglu(camblas_cuda_context *context, int dtype, uint64_t count,
+                                   int width, float limit, const void *gate, const void *up,
+                                   const float *routing, void *output)
+{
+    Entry entry(context);
+    return entry.run([&] {
+        const bool shaped = storage_in(dtype, {0, 2}) && width > 0 && count % unsigned(width) == 0 &&
+                            std::isfinite(limit) && limit >= 0 && countable(count, dtype);
+        if (!shaped)
+            return entry.refuse("invalid SwiGLU dimensions or clipping limit");
+        if (count == 0)
+            return 0;
+        const size_t element = storage_bytes(dtype);
+        if (!usable({{gate, element}, {up, element}, {output, element}, {routing, 4, true}}) ||
+            !apart(output, {routing}))
+            return entry.refuse("invalid SwiGLU buffers");
+        return entry.finish(launch_swiglu(entry.stream(), dtype, count, width, limit, gate, up, routing, output),
+                            "SwiGLU");
+    });
+}
+
+extern "C" int camblas_cuda_rms_norm_decode(camblas_cuda_context *context, int dtype,
+                                            int weight_dtype, int width, float epsilon,
+                                            int round_before_weight, int descending,
+                                            const void *input, const void *weight, void *output)
+{
+    Entry entry(context);
+    return entry.run([&] {
+        // FP32 rows take FP32 weights; BF16 rows take either
+        const bool typed = storage_in(dtype, {0, 2}) && storage_in(weight_dtype, {0, 2}) &&
+                           !(dtype == 0 && weight_dtype != 0);
+        const bool ok = typed && decode_width(width) && is_flag(round_before_weight) && is_flag(descending) &&
+                        valid_epsilon(epsilon) &&
+                        usable({{input, storage_bytes(dtype)},
+                                {weight, storage_bytes(weight_dtype)},
+                                {output, storage_bytes(dtype)}}) &&
+                        apart(output, {input, weight});
+        if (!ok)
+            return entry.refuse("invalid decode RMS arguments");
+        return entry.finish(launch_rms_rows(entry.stream(), dtype, weight_dtype, 1, width, epsilon,
+                                            round_before_weight != 0, input, nullptr, weight, nullptr, output),
+                            "decode RMS normalisation");
+    });
+}
+
+extern "C" int camblas_cuda_add_rms_norm(camblas_cuda_context *context, int dtype, int width,
+                                         float epsilon, const void *input, const void *residual,
+                                         const void *weight, void *added, void *output)
+{
+    Entry entry(context);
+    return entry.run([&] {
+        const bool ok = storage_in(dtype, {0, 2}) && decode_width(width) && valid_epsilon(epsilon) &&
+                        usable({{input, 1}, {residual, 1}, {weight, 1}, {added, 1}, {output, 1}}) &&
+                        apart(added, {output, input, residual, weight}) &&
+                        apart(output, {input, residual, weight});
+        if (!ok)
+            return entry.refuse("invalid residual RMS arguments");
+        return entry.finish(launch_rms_rows(entry.stream(), dtype, dtype, 1, width, epsilon, true, input, residual,
+                                            weight, added, output),
+                            "residual RMS normalisation");
+    });
+}
+
+// Any number of rows, with or without a residual (no counterpart in the reference header).
+extern "C" int camblas_cuda_add_rms_norm_rows(camblas_cuda_context *context, int dtype,
+                                              int weight_dtype, int rows, int width, float epsilon,
+                                              int round_before_weight, const void *input,
+                                              const void *residual, const void *weight, void *added,
+                                              void *output)
+{
+    Entry entry(context);
+    return entry.run([&] {
+        const bool typed = storage_in(dtype, {0, 2}) && storage_in(weight_dtype, {0, 2}) &&
+                           !(dtype == 0 && weight_dtype != 0);
+        if (!typed || rows < 0 || width < 0 || !is_flag(round_before_weight) || !valid_epsilon(epsilon))
+            return entry.refuse("invalid residual RMS rows arguments");
+        if (rows == 0 || width == 0)
+            return 0;
+        bool ok = usable({{input, 1}, {weight, 1}, {output, 1}}) && apart(output, {weight, input});
+        if (ok && residual)
+            ok = added && apart(added, {output, input, residual, weight}) && apart(output, {residual});
+        if (!ok)
+            return entry.refuse("invalid residual RMS rows operands");
+        return entry.finish(launch_rms_rows(entry.stream(), dtype, weight_dtype, rows, width, epsilon,
+                                            round_before_weight != 0, input, residual, weight, added, output),
+                            "residual RMS normalisation");
+    });
+}
+
+// In-place (output == input) is allowed as in the reference (backend.cu:1423-1439): a thread reads
+// an element before it writes it.
+extern "C" int camblas_cuda_rms_norm(camblas_cuda_context *context, int dtype, int rows, int width,
+                                     float epsilon, const void *input, const void *weight,
+                                     void *output)
+{
+    Entry entry(context);
+    return entry.run([&] {
+        if (!storage_in(dtype, {0, 2}) || rows < 0 || width < 0 || !valid_epsilon(epsilon))
+            return entry.refuse("invalid RMS normalisation dimensions, dtype or epsilon");
+        if (rows == 0 || width == 0)
+            return 0;
+        if (!usable({{input, 1}, {weight, 1}, {output, 1}}) || !apart(output, {weight}))
+            return entry.refuse("invalid RMS normalisation operands");
+        return entry.finish(launch_rms_rows(entry.stream(), dtype, dtype, rows, width, epsilon, true, input,
+                                            nullptr, weight, nullptr, output),
+                            "RMS normalisation");
+    });
+}
+
+extern "C" int camblas_cuda_bfloat16_square(camblas_cuda_context *context, uint64_t count,
+                                            const void *input, float *output)
+{
+    Entry entry(context);
+    return entry.run([&] {
+        if (count == 0)
+            return 0;
+        if (!usable({{input, 1}, {output, 1}}) || !countable(count, 0))
+            return entry.refuse("invalid BF16 square operands");
+        return entry.finish(launch_bf16_square(entry.stream(), count, input, output), "BF16 squares");
+    });
+}
+
+extern "C" int camblas_cuda_rms_scale(camblas_cuda_context *context, int dtype, uint64_t count,
+                                      int width, float epsilon, const void *input,
+                                      const void *weight, const float *means, void *output)
+{
+    Entry entry(context);
+    return entry.run([&] {
+        if (!storage_in(dtype, {0, 2}) || width < 0 || !valid_epsilon(epsilon))
+            return entry.refuse("invalid RMS scale dimensions, dtype or epsilon");
+        if (count == 0)
+            return 0;
+        const bool ok = width > 0 && count % unsigned(width) == 0 && countable(count, 0) &&
+                        usable({{input, 1}, {weight, 1}, {means, 1}, {output, 1}}) && apart(output, {weight});
+        if (!ok)
+            return entry.refuse("invalid RMS scale operands");
+        return entry.finish(launch_rms_scale(entry.stream(), dtype, count, width, epsilon, input, weight, means,
+                                             output),
+                            "RMS scaling");
+    });
+}
+
+// ---- decode-layer pieces (no counterpart in the reference)
+
+extern "C" int camblas_cuda_rope(camblas_cuda_context *context, int tokens, int heads, int dim,
+                                 int token_stride, float theta, const int32_t *positions, void *x)
+{
+    Entry entry(context);
+    return entry.run([&] {
+        const bool shaped = tokens >= 0 && heads >= 1 && within({{dim, 2, INT32_MAX, 2}}) &&
+                            token_stride >= int64_t(heads) * dim && std::isfinite(theta) && theta > 0;
+        if (!shaped)
+            return entry.refuse("invalid rotary embedding arguments");
+        if (tokens == 0)
+            return 0;
+        if (!usable({{positions, 4}, {x, 2}}))
+            return entry.refuse("invalid rotary embedding buffers");
+        return entry.finish(launch_rope(entry.stream(), tokens, heads, dim, token_stride, theta, positions, x),
+                            "rotary embedding");
+    });
+}
+
+extern "C" int camblas_cuda_kv_append(camblas_cuda_context *context, int batch, int kv_heads, int dim,
+                                      int context_length, const int32_t *positions,
+                                      const void *k_new, const void *v_new, int token_stride,
+                                      void *k_cache, void *v_cache)
+{
+    Entry entry(context);
+    return entry.run([&] {
+        const bool shaped = batch >= 0 && kv_heads >= 1 && within({{dim, 8, INT32_MAX, 8}}) &&
+                            context_length >= 1 && token_stride >= int64_t(kv_heads) * dim &&
+                            token_stride % 8 == 0;
+        if (!shaped)
+            return entry.refuse("invalid cache append arguments");
+        if (batch == 0)
+            return 0;
+        if (!usable({{positions, 1}, {k_new, 16}, {v_new, 16}, {k_cache, 16}, {v_cache, 16}}) ||
+            k_cache == v_cache)
+            return entry.refuse("invalid cache append buffers");
+        return entry.finish(launch_kv_append(entry.stream(), batch, kv_heads, dim, context_length, positions, k_new,
+                                             v_new, token_stride, k_cache, v_cache),
+                            "cache append");
+    });
+}
+
+extern "C" int camblas_cuda_rope_kv_append(camblas_cuda_context *context, int batch, int q_heads,
+                                           int kv_heads, int dim, int token_stride, float theta,
+                                           const int32_t *positions, void *qkv, int context_length,
+                                           void *k_cache, void *v_cache)
+{
+    Entry entry(context);
+    return entry.run([&] {
+        const bool shaped = batch >= 0 && q_heads >= 1 && kv_heads >= 1 && within({{dim, 2, INT32_MAX, 2}}) &&
+                            context_length >= 1 &&
+                            token_stride >= (int64_t(q_heads) + 2 * int64_t(kv_heads)) * dim &&
+                            std::isfinite(theta) && theta > 0;
+        if (!shaped)
+            return entry.refuse("invalid rotary cache append arguments");
+        if (batch == 0)
+            return 0;
+        if (!usable({{positions, 4}, {qkv, 2}, {k_cache, 2}, {v_cache, 2}}) || k_cache == v_cache)
+            return entry.refuse("invalid rotary cache append buffers");
+        return entry.finish(launch_rope_kv_append(entry.stream(), batch, q_heads, kv_heads, dim, token_stride, theta,
+                                                  positions, qkv, context_length, k_cache, v_cache),
+                            "rotary cache append");
+    });
+}
+
+namespace camblas_hip
+{
+namespace
+{
+// Both decode-attention entry points: the argument rules, then the two launches with the split
+// partials wherever `place(bytes, &where)` puts them (it returns a status of its own on failure).
+template <typename Place>
+int decode_attention(const Entry &entry, int batch, int q_heads, int kv_heads, int dim, int context_length,
+                     const int32_t *lengths, float scale, const void *q, int q_stride, const void *k_cache,
+                     const void *v_cache, void *output, Place place)
+{
+    const bool shaped = batch >= 0 && q_heads >= 1 && kv_heads >= 1 && q_heads % kv_heads == 0 &&
+                        q_heads / kv_heads <= 16 && dim == 128 && context_length >= 1 &&
+                        q_stride >= q_heads * dim && std::isfinite(scale);
+    if (!shaped)
+        return entry.refuse("invalid decode attention arguments");
+    if (batch == 0)
+        return 0;
+    if (!usable({{q, 16}, {k_cache, 16}, {v_cache, 16}, {output, 16}}) || q_stride % 8 != 0 ||
+        !apart(output, {q, k_cache, v_cache}))
+        return entry.refuse("invalid decode attention buffers");
+    int splits = 1;
+    const size_t bytes = gqa_decode_scratch_bytes(batch, q_heads, dim, context_length, &splits);
+    void *partials = nullptr;
+    if (const int refused = place(bytes, &partials))
+        return refused;
+    entry.context()->counts[6]++;
+    return entry.finish(launch_gqa_decode(entry.stream(), batch, q_heads, kv_heads, dim, context_length, lengths,
+                                          scale, q, q_stride, k_cache, v_cache, output, partials, splits),
+                        "decode attention");
+}
+} // namespace
+} // namespace camblas_hip
+
+extern "C" int camblas_cuda_gqa_decode_attention(camblas_cuda_context *context, int batch,
+                                                 int q_heads, int kv_heads, int dim,
+                                                 int context_length, const int32_t *lengths,
+                                                 float scale, const void *q, int q_stride,
+                                                 const void *k_cache, const void *v_cache,
+                                                 void *output)
+{
+    Entry entry(context);
+    return entry.run([&] {
+        return decode_attention(entry, batch, q_heads, kv_heads, dim, context_length, lengths, scale, q, q_stride,
+                                k_cache, v_cache, output, [&](size_t bytes, void **where) {
+                                    const hipError_t grown = reserve_scratch(context, bytes);
+                                    if (grown != hipSuccess)
+                                        return entry.refuse("decode attention scratch", int(grown));
+                                    *where = context->scratch;
+                                    return 0;
+                                });
+    });
+}
+
+extern "C" size_t camblas_cuda_gqa_decode_attention_noalloc_limit(void)
+{
+    return gqa_resident_scratch_bytes();
+}
+
+// The same kernels with the partials in the library's fixed device array: no hipMalloc, no
+// hipFree, no context scratch. Calls that overlap on one GPU share that array and race.
+extern "C" int camblas_cuda_gqa_decode_attention_noalloc(camblas_cuda_context *context, int batch,
+                                                         int q_heads, int kv_heads, int dim,
+                                                         int context_length, const int32_t *lengths,
+                                                         float scale, const void *q, int q_stride,
+                                                         const void *k_cache, const void *v_cache,
+                                                         void *output)
+{
+    Entry entry(context);
+    return entry.run([&] {
+        return decode_attention(
+            entry, batch, q_heads, kv_heads, dim, context_length, lengths, scale, q, q_stride, k_cache, v_cache,
+            output, [&](size_t bytes, void **where) {
+                if (bytes > gqa_resident_scratch_bytes()) {
+                    std::snprintf(context->error, sizeof(context->error),
+                                  "decode attention needs %zu bytes of partials; the allocation-free entry "
+                                  "point holds %zu",
+                                  bytes, gqa_resident_scratch_bytes());
+                    return -1;
+                }
+                return entry.finish(gqa_resident_scratch(context->device, where),
+                                    "resident decode attention partials");
+            });
+    });
+}

@@ -1,8 +1,12 @@
+// Bench equipment, built as libcamblas_probes.so beside the product library and loaded by bench.py
+// only: nothing here is part of libcamblas_hip.so.
+//
 // Calibration launch for the matrix cores: every wavefront issues independent matrix instructions
 // back to back, with no memory traffic, so the launch's duration gives the rate the part sustains
 // for that instruction (its clock under matrix load included). No counterpart in the reference.
-#include "common.hpp"
 #include "device.hpp"
+
+#include <hip/hip_runtime.h>
 
 namespace camblas_hip
 {
@@ -85,6 +89,46 @@ hipError_t launch_matrix_probe(hipStream_t stream, int kind, int workgroups, int
     default: return hipErrorInvalidValue;
     }
     *flops = per_instruction[kind] * double(workgroups) * (PROBE_THREADS / 64) * double(rounds) * PROBE_ACCUMULATORS;
-    return launch_status();
+    return hipGetLastError();
 }
+
+// Plain 16-byte-per-thread copy: a launch of known HBM traffic (bytes read + bytes written)
+// against which the hardware byte counters are calibrated.
+namespace
+{
+__global__ void copy_probe_kernel(size_t vectors, const u32x4_t *source, u32x4_t *destination)
+{
+    for (size_t index = size_t(blockIdx.x) * blockDim.x + threadIdx.x; index < vectors;
+         index += size_t(gridDim.x) * blockDim.x)
+        destination[index] = source[index];
+}
+} // namespace
 } // namespace camblas_hip
+
+// stream: a raw hipStream_t. Both return 0 or a negative hipError_t.
+extern "C" int camblas_probe_copy(void *stream, size_t bytes, const void *source, void *destination)
+{
+    using namespace camblas_hip;
+    if (bytes % 16 || !source || !destination || reinterpret_cast<uintptr_t>(source) % 16 ||
+        reinterpret_cast<uintptr_t>(destination) % 16)
+        return -int(hipErrorInvalidValue);
+    if (!bytes)
+        return 0;
+    copy_probe_kernel<<<2048, 256, 0, static_cast<hipStream_t>(stream)>>>(
+        bytes / 16, static_cast<const u32x4_t *>(source), static_cast<u32x4_t *>(destination));
+    return -int(hipGetLastError());
+}
+
+// kind 0 BF16 32x32x16, 1 E4M3 x E4M3 and 2 E2M1 x E4M3 scaled 32x32x64, 3 FP32 32x32x2; one
+// workgroup of eight wavefronts per entry of `workgroups`, each wavefront issuing rounds * 8
+// independent matrix instructions. sink (device) receives workgroups * 512 floats; *flops (host)
+// the floating-point operations of the launch.
+extern "C" int camblas_probe_matrix(void *stream, int kind, int workgroups, int rounds, int constant_operands,
+                                    void *sink, size_t sink_bytes, double *flops)
+{
+    if (kind < 0 || kind > 3 || workgroups < 1 || rounds < 1 || !sink || !flops ||
+        reinterpret_cast<uintptr_t>(sink) % 4 || sink_bytes < size_t(workgroups) * 512 * sizeof(float))
+        return -int(hipErrorInvalidValue);
+    return -int(camblas_hip::launch_matrix_probe(static_cast<hipStream_t>(stream), kind, workgroups, rounds,
+                                                 constant_operands != 0, static_cast<float *>(sink), flops));
+}

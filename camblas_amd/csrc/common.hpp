@@ -20,6 +20,7 @@ struct camblas_cuda_context {
     void *scratch = nullptr;       // split-K partials, attention partials
     size_t scratch_bytes = 0;
     std::vector<void *> retired;   // superseded scratch kept alive for captured graphs
+    bool seen_capture = false;     // the arena has been used by a launch under stream capture
     int override_kernel = -1;      // diagnostics: forced kernel variant
     int override_split = 0;
     std::atomic<uint64_t> counts[8] = {};
@@ -49,7 +50,8 @@ enum KernelFamily {
     FAMILY_DMA = 5,    // BF16 'T','N' prefill: large MFMA tiles fed by direct global->LDS loads
     FAMILY_FP8_DMA = 6, // FP8 block-scaled prefill: the same structure with one scale group per step
     FAMILY_FP8_STREAM = 7, // FP8 block-scaled decode: weight-streaming kernel (10*row_tiles + token_tiles)
-    FAMILY_MFMA_F32 = 8    // FP32, any layout: 128 x 128 tiles on the FP32 matrix-core instruction
+    FAMILY_MFMA_F32 = 8,   // FP32, any layout: 128 x 128 tiles on the FP32 matrix-core instruction
+    FAMILY_MFMA_BF16 = 9   // BF16, any layout: the same structure on the BF16 matrix-core instruction
 };
 
 struct Plan {
@@ -114,6 +116,11 @@ hipError_t launch_generic_bf16(hipStream_t stream, bool ta, bool tb, int m, int 
 hipError_t launch_generic_f64(hipStream_t stream, bool ta, bool tb, int m, int n, int k,
                               double alpha, const double *a, int lda, const double *b, int ldb,
                               double beta, double *c, int ldc);
+// BF16 for any transpose pair / leading dimension / alignment on the matrix cores (bgemm_any.hip);
+// wide: 128 x 128 tiles, else 128 x 64.
+hipError_t launch_bgemm_any(hipStream_t stream, bool wide, bool ta, bool tb, int m, int n, int k,
+                            float alpha, const void *a, int lda, const void *b, int ldb, float beta,
+                            void *c, int ldc);
 hipError_t launch_gemv_f32(hipStream_t stream, int rows, int inner, float alpha, const float *w,
                            int ld, const float *x, float beta, float *y);
 // y[M,N] (ldc) = alpha * x[M,K] (ldb) * W[N,K]^T (lda) + beta * y, BF16 storage.
@@ -201,11 +208,6 @@ hipError_t launch_rms_scale(hipStream_t stream, int dtype, uint64_t count, int w
 hipError_t launch_kv_append(hipStream_t stream, int batch, int kv_heads, int dim, int context_length,
                             const int32_t *positions, const void *k_new, const void *v_new,
                             int token_stride, void *k_cache, void *v_cache);
-// kind: 0 BF16 32x32x16, 1 E4M3 x E4M3 and 2 E2M1 x E4M3 scaled 32x32x64, 3 FP32 32x32x2; one
-// workgroup of eight wavefronts per entry of `workgroups`, rounds * 8 instructions per wavefront.
-hipError_t launch_matrix_probe(hipStream_t stream, int kind, int workgroups, int rounds, int constant,
-                               float *sink, double *flops);
-hipError_t launch_copy_probe(hipStream_t stream, size_t bytes, const void *source, void *destination);
 hipError_t launch_rope_kv_append(hipStream_t stream, int batch, int q_heads, int kv_heads, int dim,
                                  int token_stride, float theta, const int32_t *positions, void *qkv,
                                  int context_length, void *k_cache, void *v_cache);

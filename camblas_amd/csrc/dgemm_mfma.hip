@@ -134,19 +134,30 @@ hipError_t launch_dgemm_mfma(hipStream_t stream, bool ta, bool tb, int m, int n,
                              const double *a, int lda, const double *b, int ldb, double beta, double *c,
                              int ldc, int batches, size_t batch_stride, bool lower_only)
 {
-    dim3 grid((m + TILE - 1) / TILE, (n + TILE - 1) / TILE, batches);
-    if (lower_only)
-        grid = dim3(lower_tile_count<TILE, TILE>(n), 1, batches);
-    if (grid.y > 65535u || batches < 1 || batches > 65535)
+    if (batches < 1 || batches > 65535)
         return hipErrorInvalidValue;
-    if (!ta && !tb)
-        dgemm_mfma_kernel<false, false><<<grid, THREADS, 0, stream>>>(m, n, k, alpha, a, lda, b, ldb, beta, c, ldc, batch_stride, lower_only);
-    else if (!ta && tb)
-        dgemm_mfma_kernel<false, true><<<grid, THREADS, 0, stream>>>(m, n, k, alpha, a, lda, b, ldb, beta, c, ldc, batch_stride, lower_only);
-    else if (ta && !tb)
-        dgemm_mfma_kernel<true, false><<<grid, THREADS, 0, stream>>>(m, n, k, alpha, a, lda, b, ldb, beta, c, ldc, batch_stride, lower_only);
-    else
-        dgemm_mfma_kernel<true, true><<<grid, THREADS, 0, stream>>>(m, n, k, alpha, a, lda, b, ldb, beta, c, ldc, batch_stride, lower_only);
-    return launch_status();
+    // column tiles travel in grid.y (at most 65535): wider products go panel by panel; the
+    // lower-triangle grid is one-dimensional
+    constexpr int PANEL = 65535 * TILE;
+    for (int first = 0; first < n; first += lower_only ? n : PANEL) {
+        const int columns = lower_only ? n : (n - first < PANEL ? n - first : PANEL);
+        const double *bp = b + (tb ? size_t(first) : size_t(first) * ldb);
+        double *cp = c + size_t(first) * ldc;
+        dim3 grid((m + TILE - 1) / TILE, (columns + TILE - 1) / TILE, batches);
+        if (lower_only)
+            grid = dim3(lower_tile_count<TILE, TILE>(n), 1, batches);
+        if (!ta && !tb)
+            dgemm_mfma_kernel<false, false><<<grid, THREADS, 0, stream>>>(m, columns, k, alpha, a, lda, bp, ldb, beta, cp, ldc, batch_stride, lower_only);
+        else if (!ta && tb)
+            dgemm_mfma_kernel<false, true><<<grid, THREADS, 0, stream>>>(m, columns, k, alpha, a, lda, bp, ldb, beta, cp, ldc, batch_stride, lower_only);
+        else if (ta && !tb)
+            dgemm_mfma_kernel<true, false><<<grid, THREADS, 0, stream>>>(m, columns, k, alpha, a, lda, bp, ldb, beta, cp, ldc, batch_stride, lower_only);
+        else
+            dgemm_mfma_kernel<true, true><<<grid, THREADS, 0, stream>>>(m, columns, k, alpha, a, lda, bp, ldb, beta, cp, ldc, batch_stride, lower_only);
+        const hipError_t status = launch_status();
+        if (status != hipSuccess)
+            return status;
+    }
+    return hipSuccess;
 }
 } // namespace camblas_hip

@@ -305,14 +305,6 @@ __global__ void rope_kv_append_kernel(int batch, int q_heads, int kv_heads, int 
     }
 }
 
-// Plain 16-byte-per-thread copy: the known-traffic kernel used to calibrate the HBM byte counters.
-__global__ void copy_probe_kernel(size_t vectors, const u32x4_t *source, u32x4_t *destination)
-{
-    for (size_t index = size_t(blockIdx.x) * blockDim.x + threadIdx.x; index < vectors;
-         index += size_t(gridDim.x) * blockDim.x)
-        destination[index] = source[index];
-}
-
 // Writes the new token's K and V heads (taken from a fused QKV activation row) into the caches at
 // each sequence's position: 16 bytes per thread.
 __global__ void kv_append_kernel(int batch, int kv_heads, int dim, int context_length,
@@ -458,13 +450,6 @@ hipError_t launch_kv_append(hipStream_t stream, int batch, int kv_heads, int dim
         batch, kv_heads, dim, context_length, positions, static_cast<const unsigned short *>(k_new),
         static_cast<const unsigned short *>(v_new), token_stride,
         static_cast<unsigned short *>(k_cache), static_cast<unsigned short *>(v_cache));
-    return launch_status();
-}
-
-hipError_t launch_copy_probe(hipStream_t stream, size_t bytes, const void *source, void *destination)
-{
-    copy_probe_kernel<<<2048, 256, 0, stream>>>(bytes / 16, static_cast<const u32x4_t *>(source),
-                                                static_cast<u32x4_t *>(destination));
     return launch_status();
 }
 

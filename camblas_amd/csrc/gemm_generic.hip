@@ -103,22 +103,30 @@ hipError_t launch_generic(hipStream_t stream, bool ta, bool tb, int m, int n, in
                           typename storage<T>::accumulator alpha, const T *a, int lda, const T *b,
                           int ldb, typename storage<T>::accumulator beta, T *c, int ldc)
 {
-    dim3 grid((m + TILE - 1) / TILE, (n + TILE - 1) / TILE);
-    if (grid.y > 65535u)
-        return hipErrorInvalidValue;
-    if (!ta && !tb)
-        generic_kernel<T, false, false>
-            <<<grid, THREADS, 0, stream>>>(m, n, k, alpha, a, lda, b, ldb, beta, c, ldc);
-    else if (!ta && tb)
-        generic_kernel<T, false, true>
-            <<<grid, THREADS, 0, stream>>>(m, n, k, alpha, a, lda, b, ldb, beta, c, ldc);
-    else if (ta && !tb)
-        generic_kernel<T, true, false>
-            <<<grid, THREADS, 0, stream>>>(m, n, k, alpha, a, lda, b, ldb, beta, c, ldc);
-    else
-        generic_kernel<T, true, true>
-            <<<grid, THREADS, 0, stream>>>(m, n, k, alpha, a, lda, b, ldb, beta, c, ldc);
-    return launch_status();
+    // column tiles travel in grid.y (at most 65535): wider products go panel by panel
+    constexpr int PANEL = 65535 * TILE;
+    for (int first = 0; first < n; first += PANEL) {
+        const int columns = n - first < PANEL ? n - first : PANEL;
+        const T *bp = b + (tb ? size_t(first) : size_t(first) * ldb);
+        T *cp = c + size_t(first) * ldc;
+        const dim3 grid((m + TILE - 1) / TILE, (columns + TILE - 1) / TILE);
+        if (!ta && !tb)
+            generic_kernel<T, false, false>
+                <<<grid, THREADS, 0, stream>>>(m, columns, k, alpha, a, lda, bp, ldb, beta, cp, ldc);
+        else if (!ta && tb)
+            generic_kernel<T, false, true>
+                <<<grid, THREADS, 0, stream>>>(m, columns, k, alpha, a, lda, bp, ldb, beta, cp, ldc);
+        else if (ta && !tb)
+            generic_kernel<T, true, false>
+                <<<grid, THREADS, 0, stream>>>(m, columns, k, alpha, a, lda, bp, ldb, beta, cp, ldc);
+        else
+            generic_kernel<T, true, true>
+                <<<grid, THREADS, 0, stream>>>(m, columns, k, alpha, a, lda, bp, ldb, beta, cp, ldc);
+        const hipError_t status = launch_status();
+        if (status != hipSuccess)
+            return status;
+    }
+    return hipSuccess;
 }
 } // namespace
 

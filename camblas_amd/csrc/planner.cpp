@@ -119,6 +119,15 @@ Plan make_plan(int dtype, int algorithm, bool trans_a, bool trans_b, int m, int 
                            k % 8 == 0 && lda % 8 == 0 && ldb % 8 == 0 && aligned16 && lda < limit &&
                            ldb < limit;
         if (!matrix_path) {
+            // the other layouts (and 'T','N' operands the K-contiguous kernels cannot take): the
+            // layout-agnostic matrix-core kernel unless the product is a sliver, tiles chosen as for
+            // FP32 (the reference sends every transpose pair to tensor-core GEMMs)
+            if (algorithm != CAMBLAS_CUDA_CLASSICAL && m >= 32 && n >= 32 && k >= 16) {
+                plan.family = FAMILY_MFMA_BF16;
+                plan.kernel = double(ceil_div(m, 128)) * ceil_div(n, 128) >= 2.0 * compute_units ? 0 : 1;
+                plan.counter = 4;
+                return plan;
+            }
             plan.family = FAMILY_GENERIC;
             plan.counter = 0;
             return plan;
@@ -258,6 +267,9 @@ void describe_plan(const Plan &plan, int dtype, char *text, size_t bytes)
         break;
     case FAMILY_MFMA_F32:
         std::snprintf(text, bytes, "%s mfma %s", type, plan.kernel == 0 ? "128x128x32" : "128x64x32");
+        break;
+    case FAMILY_MFMA_BF16:
+        std::snprintf(text, bytes, "%s mfma any-layout %s", type, plan.kernel == 0 ? "128x128x32" : "128x64x32");
         break;
     case FAMILY_MFMA_TN:
         std::snprintf(text, bytes, "%s %s split_k=%d", type, tn_variant(plan.kernel).name,

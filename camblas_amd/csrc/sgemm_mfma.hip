@@ -164,20 +164,31 @@ hipError_t launch_columns(hipStream_t stream, bool ta, bool tb, int m, int n, in
                           const float *a, int lda, const float *b, int ldb, float beta, float *c, int ldc,
                           int batches, size_t batch_stride, bool lower_only)
 {
-    dim3 grid((m + TILE - 1) / TILE, (n + COLUMNS - 1) / COLUMNS, batches);
-    if (lower_only)
-        grid = dim3(lower_tile_count<TILE, COLUMNS>(n), 1, batches);
-    if (grid.y > 65535u || batches < 1 || batches > 65535)
+    if (batches < 1 || batches > 65535)
         return hipErrorInvalidValue;
-    if (!ta && !tb)
-        sgemm_mfma_kernel<false, false, COLUMNS><<<grid, THREADS, 0, stream>>>(m, n, k, alpha, a, lda, b, ldb, beta, c, ldc, batch_stride, lower_only);
-    else if (!ta && tb)
-        sgemm_mfma_kernel<false, true, COLUMNS><<<grid, THREADS, 0, stream>>>(m, n, k, alpha, a, lda, b, ldb, beta, c, ldc, batch_stride, lower_only);
-    else if (ta && !tb)
-        sgemm_mfma_kernel<true, false, COLUMNS><<<grid, THREADS, 0, stream>>>(m, n, k, alpha, a, lda, b, ldb, beta, c, ldc, batch_stride, lower_only);
-    else
-        sgemm_mfma_kernel<true, true, COLUMNS><<<grid, THREADS, 0, stream>>>(m, n, k, alpha, a, lda, b, ldb, beta, c, ldc, batch_stride, lower_only);
-    return launch_status();
+    // The column tiles travel in grid.y (at most 65535): wider products are launched as panels of
+    // that many tiles, each on its own columns of B and C. The lower-triangle grid is one-dimensional.
+    constexpr int PANEL = 65535 * COLUMNS;
+    for (int first = 0; first < n; first += lower_only ? n : PANEL) {
+        const int columns = lower_only ? n : (n - first < PANEL ? n - first : PANEL);
+        const float *bp = b + (tb ? size_t(first) : size_t(first) * ldb);
+        float *cp = c + size_t(first) * ldc;
+        dim3 grid((m + TILE - 1) / TILE, (columns + COLUMNS - 1) / COLUMNS, batches);
+        if (lower_only)
+            grid = dim3(lower_tile_count<TILE, COLUMNS>(n), 1, batches);
+        if (!ta && !tb)
+            sgemm_mfma_kernel<false, false, COLUMNS><<<grid, THREADS, 0, stream>>>(m, columns, k, alpha, a, lda, bp, ldb, beta, cp, ldc, batch_stride, lower_only);
+        else if (!ta && tb)
+            sgemm_mfma_kernel<false, true, COLUMNS><<<grid, THREADS, 0, stream>>>(m, columns, k, alpha, a, lda, bp, ldb, beta, cp, ldc, batch_stride, lower_only);
+        else if (ta && !tb)
+            sgemm_mfma_kernel<true, false, COLUMNS><<<grid, THREADS, 0, stream>>>(m, columns, k, alpha, a, lda, bp, ldb, beta, cp, ldc, batch_stride, lower_only);
+        else
+            sgemm_mfma_kernel<true, true, COLUMNS><<<grid, THREADS, 0, stream>>>(m, columns, k, alpha, a, lda, bp, ldb, beta, cp, ldc, batch_stride, lower_only);
+        const hipError_t status = launch_status();
+        if (status != hipSuccess)
+            return status;
+    }
+    return hipSuccess;
 }
 } // namespace
 

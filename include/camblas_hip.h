@@ -326,21 +326,6 @@ int camblas_hip_plan_describe(int dtype, int algorithm, char trans_a, char trans
  * 256 x 256, 256 x 128, (E4M3 weights only) 192 x 256 and 128 x 128 tiles; a forced kernel that
  * cannot run the call makes the call fail. */
 int camblas_hip_set_plan_override(camblas_cuda_context *context, int kernel, int split_k);
-/* extension. Diagnostics: copies `bytes` (a multiple of 16, 16-byte aligned buffers) with a plain
- * grid-stride kernel. A launch of known HBM traffic (bytes read + bytes written) against which
- * the hardware byte counters are calibrated. */
-int camblas_hip_copy_probe(camblas_cuda_context *context, size_t bytes, const void *source,
-                           void *destination);
-/* extension. Diagnostics: one workgroup of eight wavefronts per compute unit, each wavefront
- * issuing rounds * 8 independent matrix instructions with no memory traffic (kind 0:
- * v_mfma_f32_32x32x16_bf16; 1 and 2: v_mfma_scale_f32_32x32x64_f8f6f4 with E4M3 x E4M3 and
- * E2M1 x E4M3 operands; 3: v_mfma_f32_32x32x2_f32). The launch's duration gives the rate the part
- * sustains for that instruction, its clock under matrix load included: the ceiling a GEMM's
- * rate is read against. Operands are per-lane hashes shaped into finite values of either sign,
- * or the value 1 in every lane when constant_operands is set. sink (device, at least compute units * 2048 bytes) receives each
- * lane's accumulator sum; *flops (host) the floating-point operations of the launch. */
-int camblas_hip_matrix_probe(camblas_cuda_context *context, int kind, int rounds,
-                             int constant_operands, void *sink, size_t sink_bytes, double *flops);
 /* extension. Number of kernel variants `camblas_hip_set_plan_override` accepts for a dtype. */
 int camblas_hip_kernel_count(int dtype);
 

@@ -67,11 +67,14 @@ def test_planner_choices_for_the_baseline_shapes():
     # prefill: direct-to-LDS MFMA tile that divides 10240 x 4096 into exactly two waves of tiles
     code, text = describe(2, "T", "N", 10240, 4096, 8192, 8192, 8192, 10240)
     assert code // 1000 == 5 and "dma320x256" in text
-    # K not a multiple of 64: register-staged MFMA tiles; unaligned or other layouts: generic
+    # K not a multiple of 64: register-staged MFMA tiles; unaligned operands and the other transpose
+    # pairs: the layout-agnostic matrix-core kernel; slivers and the classical policy: vector-ALU tiles
     assert describe(2, "T", "N", 10240, 4096, 8200, 8200, 8200, 10240)[0] // 1000 == 2
-    assert describe(2, "T", "N", 1024, 64, 1001, 1001, 1001, 1024)[0] // 1000 == 0
-    assert describe(2, "N", "N", 1024, 64, 1024, 1024, 1024, 1024)[0] // 1000 == 0
-    assert describe(2, "T", "N", 1024, 64, 1024, 1024, 1024, 1024, aligned16=False)[0] // 1000 == 0
+    assert describe(2, "T", "N", 1024, 64, 1001, 1001, 1001, 1024)[0] // 1000 == 9
+    assert describe(2, "N", "N", 1024, 64, 1024, 1024, 1024, 1024) == (9001, "bf16 mfma any-layout 128x64x32")
+    assert describe(2, "N", "T", 8192, 8192, 4096, 8192, 8192, 8192) == (9000, "bf16 mfma any-layout 128x128x32")
+    assert describe(2, "T", "N", 1024, 64, 1024, 1024, 1024, 1024, aligned16=False)[0] // 1000 == 9
+    assert describe(2, "N", "N", 1024, 16, 1024, 1024, 1024, 1024)[0] // 1000 == 0
     assert describe(2, "T", "N", 1024, 64, 1024, 1024, 1024, 1024, algorithm="classical")[0] // 1000 == 0
     # FP32: single-vector shortcut only under auto (ref: src/cuda/backend.cu:810-815)
     assert describe(0, "T", "N", 4096, 1, 4096, 4096, 4096, 4096)[0] // 1000 == 1

@@ -140,7 +140,7 @@ def test_planned_linear_shapes(device, tokens):
 @pytest.mark.parametrize("ta", "NT")
 @pytest.mark.parametrize("tb", "NT")
 def test_generic_layouts_and_unaligned(device, ta, tb):
-    m, n, k = 45, 38, 51  # odd sizes: never eligible for the MFMA path
+    m, n, k = 45, 38, 51  # odd sizes and leading dimensions: the layout-agnostic kernel with element loads
     lda = (m if ta == "N" else k) + 1
     ldb = (k if tb == "N" else n) + 3
     ldc = m + 2
@@ -152,6 +152,42 @@ def test_generic_layouts_and_unaligned(device, ta, tb):
     got2d = got.reshape(n, ldc)
     assert rel_frobenius(oracle.bf16_to_f32(got2d[:, :m]), want64.reshape(n, m)) <= TOLERANCE
     assert np.array_equal(got2d[:, m:], c0.reshape(n, ldc)[:, m:])
+
+
+@pytest.mark.parametrize("ta", "NT")
+@pytest.mark.parametrize("tb", "NT")
+@pytest.mark.parametrize("m,n,k,pad", [(200, 150, 72, 8), (130, 70, 33, 16), (20, 300, 64, 8), (1500, 1400, 40, 0)])
+def test_every_layout_on_the_matrix_cores(device, ta, tb, m, n, k, pad):
+    # leading dimensions in multiples of eight: 16-byte operand loads, with ragged edges in every
+    # dimension (K = 33 ends inside a vector); 20 rows is a sliver and stays on the vector-ALU tiles
+    lda = (m if ta == "N" else k) + 7 & ~7
+    ldb = (k if tb == "N" else n) + 7 & ~7
+    lda, ldb, ldc = lda + pad, ldb + pad, m + 4
+    a = oracle.fill_normal_bf16(90, (lda * (k if ta == "N" else m),))
+    b = oracle.fill_normal_bf16(91, (ldb * (n if tb == "N" else k),))
+    c0 = oracle.fill_normal_bf16(92, (ldc * n,))
+    got = run_bgemm(device, ta, tb, m, n, k, 0.75, a, lda, b, ldb, -0.5, c0, ldc)
+    want, want64 = reference(ta, tb, m, n, k, 0.75, a, lda, b, ldb, -0.5, c0, ldc)
+    got2d = got.reshape(n, ldc)
+    assert rel_frobenius(oracle.bf16_to_f32(got2d[:, :m]), want64.reshape(n, m)) <= TOLERANCE
+    assert np.array_equal(got2d[:, m:], c0.reshape(n, ldc)[:, m:])
+    if (ta, tb) != ("T", "N") and m >= 32:
+        code = _native.plan_describe(2, ta, tb, m, n, k, lda, ldb, ldc)[0]
+        assert code // 1000 == 9
+
+
+def test_layout_agnostic_kernel_counts_as_a_library_product(device):
+    # row-major torch.mm(x, w) with a contiguous [in, out] weight arrives as 'N','N'
+    native = _native.context(device)
+    native.call("reset_stats")
+    x = oracle.fill_normal_bf16(93, (96, 256))
+    w = oracle.fill_normal_bf16(94, (256, 160))
+    y = _kernels.matmul(to_device_bf16(x, device), to_device_bf16(w, device))
+    torch.cuda.synchronize()
+    counts = _native.stats(device)
+    assert counts["lt"] == 1 and counts["classical"] == 0
+    want = oracle.bf16_to_f32(x).astype(np.float64) @ oracle.bf16_to_f32(w).astype(np.float64)
+    assert rel_frobenius(bf16_values(y), want) <= TOLERANCE
 
 
 def test_classical_algorithm_uses_generic_kernel(device):

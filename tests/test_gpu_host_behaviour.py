@@ -152,28 +152,31 @@ print('ok')
 
 @pytest.mark.parametrize("kind,per_round", [(0, 16.0), (1, 64.0), (2, 48.0), (3, 2.0)])
 def test_matrix_probe_counts_its_work(device, kind, per_round):
-    # the calibration launch for the matrix cores: with the value 1 in every operand lane each
-    # accumulator element grows by the instruction's K per round (E2M1 reads the byte 0x38 as the
-    # nibbles -0 and 1.5: 32 * 1.5), so a lane's sum over 8 accumulators x 16 elements is exact,
-    # and the reported operation count is compute units * 8 wavefronts * rounds * 8 instructions
+    # the bench-side calibration launch for the matrix cores (libcamblas_probes.so, not part of the
+    # product library): with the value 1 in every operand lane each accumulator element grows by the
+    # instruction's K per round (E2M1 reads the byte 0x38 as the nibbles -0 and 1.5: 32 * 1.5), so a
+    # lane's sum over 8 accumulators x 16 elements is exact, and the reported operation count is
+    # workgroups * 8 wavefronts * rounds * 8 instructions
     import ctypes as ct
 
-    native, lib = _native.context(device), _native.library()
+    lib = ct.CDLL(str(_native.library_path().parent / "libcamblas_probes.so"))
+    probe = lib.camblas_probe_matrix
+    probe.argtypes = [ct.c_void_p, ct.c_int, ct.c_int, ct.c_int, ct.c_int, ct.c_void_p, ct.c_size_t,
+                      ct.POINTER(ct.c_double)]
+    assert not hasattr(_native.library(), "camblas_hip_matrix_probe")
+    stream = ct.c_void_p(torch.cuda.current_stream(device).cuda_stream)
     units = torch.cuda.get_device_properties(device).multi_processor_count
     sink = torch.zeros(units * 512, dtype=torch.float32, device=device)
     flops = ct.c_double(0.0)
     rounds = 25
-    native.call("hip_matrix_probe", kind, rounds, 1, ct.c_void_p(sink.data_ptr()), sink.numel() * 4, ct.byref(flops))
+    assert probe(stream, kind, units, rounds, 1, sink.data_ptr(), sink.numel() * 4, ct.byref(flops)) == 0
     torch.cuda.synchronize()
     assert (sink == 128 * rounds * per_round).all()
     k = {0: 16, 1: 64, 2: 64, 3: 2}[kind]
     assert flops.value == 2.0 * 32 * 32 * k * units * 8 * rounds * 8
-    native.call("hip_matrix_probe", kind, rounds, 0, ct.c_void_p(sink.data_ptr()), sink.numel() * 4, ct.byref(flops))
+    assert probe(stream, kind, units, rounds, 0, sink.data_ptr(), sink.numel() * 4, ct.byref(flops)) == 0
     torch.cuda.synchronize()
     assert torch.isfinite(sink).all() and (sink != 0).any()
-    status = lib.camblas_cuda_error  # (error text after a refused call)
-    assert lib.camblas_hip_matrix_probe(native.handle, 9, rounds, 0, ct.c_void_p(sink.data_ptr()),
-                                        sink.numel() * 4, ct.byref(flops)) == -1
-    assert b"invalid matrix probe arguments" in status(native.handle)
-    assert lib.camblas_hip_matrix_probe(native.handle, 0, rounds, 0, ct.c_void_p(sink.data_ptr()), 16,
-                                        ct.byref(flops)) == -1
+    # refused without a launch: unknown kind, sink too small
+    assert probe(stream, 9, units, rounds, 0, sink.data_ptr(), sink.numel() * 4, ct.byref(flops)) < 0
+    assert probe(stream, 0, units, rounds, 0, sink.data_ptr(), 16, ct.byref(flops)) < 0

@@ -244,3 +244,30 @@ def test_sgemm_exact_rank_two_integer_identity(device, kernel, shape):
                                     + products[2] * p[:, None] * s + products[3] * p[:, None] * w) + beta * 2.0
                 assert np.array_equal(got.reshape(n, ldc)[:, :m].T, expected.astype(np.float32)), (ta, tb, change)
                 assert (got.reshape(n, ldc)[:, m:] == -73.0).all()
+
+
+@pytest.mark.parametrize("kernel", ["matrix64", "vector"])
+def test_more_column_tiles_than_one_grid_dimension_holds(device, kernel):
+    # a grid dimension holds 65535 tiles: 64-column tiles cover 4,194,240 columns. A product with
+    # more columns (row-major: a tall left operand times a small matrix) is launched panel by
+    # panel; columns on both sides of the seam and at the far end are compared with FP64 products.
+    m, k = 40, 16
+    n = 65535 * 64 + 70
+    rng = np.random.default_rng(11)
+    a = torch.from_numpy(rng.uniform(-1, 1, (k, m)).astype(np.float32)).to(device)      # column-major [m, k]
+    b = (torch.rand((n, k), device=device, dtype=torch.float32) * 2 - 1)                 # column-major [k, n]
+    c = torch.full((n, m), float("nan"), device=device, dtype=torch.float32)
+    native = _native.context(device)
+    native.call("hip_set_plan_override", KERNEL[kernel], 0)
+    try:
+        native.call("sgemm", b"N", b"N", m, n, k, ct.c_float(1.0), ptr(a), m, ptr(b), k, ct.c_float(0.0),
+                    ptr(c), m)
+    finally:
+        native.call("hip_set_plan_override", -1, 0)
+    torch.cuda.synchronize()
+    seam = 65535 * 64
+    columns = np.r_[0:64, seam - 64:seam + 70, n - 64:n]
+    got = c[columns].cpu().numpy().astype(np.float64)
+    want = b[columns].cpu().numpy().astype(np.float64) @ a.cpu().numpy().astype(np.float64)
+    assert rel_frobenius(got.ravel(), want.ravel()) <= TOLERANCE
+    assert bool(torch.isfinite(c).all())
