@@ -234,19 +234,10 @@ hipError_t launch_one(hipStream_t stream, const StreamParams &p)
         return hipErrorInvalidValue;
     } else {
         auto kernel = bgemv_stream_kernel<NT, MT, KT>;
-        static bool configured[64] = {};
-        int device = 0;
-        hipError_t status = hipGetDevice(&device);
+        static LdsLimitFlags limits; // (one per instantiation)
+        const hipError_t status = raise_lds_limit(limits, reinterpret_cast<const void *>(kernel), lds_bytes);
         if (status != hipSuccess)
             return status;
-        if (device < 0 || device >= 64 || !configured[device]) {
-            status = hipFuncSetAttribute(reinterpret_cast<const void *>(kernel),
-                                         hipFuncAttributeMaxDynamicSharedMemorySize, int(lds_bytes));
-            if (status != hipSuccess)
-                return status;
-            if (device >= 0 && device < 64)
-                configured[device] = true;
-        }
         dim3 grid(unsigned((p.n + NT * 16 - 1) / (NT * 16)),
                   unsigned((p.m + MT * 16 - 1) / (MT * 16)));
         kernel<<<grid, WAVES * 64, lds_bytes, stream>>>(p);

@@ -40,6 +40,29 @@ hipError_t reserve_scratch(camblas_cuda_context *context, size_t bytes);
 
 inline hipError_t launch_status() { return hipGetLastError(); }
 
+// Per kernel instantiation and device: which devices have had the kernel's dynamic LDS limit raised.
+// Contexts on different host threads may launch the same kernel at the same time, so the flags are
+// atomic; setting the attribute twice is harmless, so no lock is needed.
+struct LdsLimitFlags {
+    std::atomic<bool> raised[64] = {};
+};
+
+// Raises `kernel`'s dynamic shared memory limit to `bytes` once per device (the current one).
+inline hipError_t raise_lds_limit(LdsLimitFlags &flags, const void *kernel, size_t bytes)
+{
+    int device = 0;
+    hipError_t status = hipGetDevice(&device);
+    if (status != hipSuccess)
+        return status;
+    const bool tracked = device >= 0 && device < 64;
+    if (tracked && flags.raised[device].load(std::memory_order_acquire))
+        return hipSuccess;
+    status = hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, int(bytes));
+    if (status == hipSuccess && tracked)
+        flags.raised[device].store(true, std::memory_order_release);
+    return status;
+}
+
 // ---------------------------------------------------------------- planner (pure host)
 enum KernelFamily {
     FAMILY_GENERIC = 0, // LDS-tiled VALU kernel, any transpose / leading dimension / alignment

@@ -321,19 +321,10 @@ hipError_t launch_variant(hipStream_t stream, const Fp8Params &p, int split_k)
 {
     constexpr size_t lds_bytes = size_t(2) * (BN + BM) * 128;
     auto kernel = fp8_block_kernel<BN, BM, WN, WM>;
-    static bool configured[64] = {};
-    int device = 0;
-    hipError_t status = hipGetDevice(&device);
+    static LdsLimitFlags limits; // (one per instantiation)
+    const hipError_t status = raise_lds_limit(limits, reinterpret_cast<const void *>(kernel), lds_bytes);
     if (status != hipSuccess)
         return status;
-    if (device < 0 || device >= 64 || !configured[device]) {
-        status = hipFuncSetAttribute(reinterpret_cast<const void *>(kernel),
-                                     hipFuncAttributeMaxDynamicSharedMemorySize, int(lds_bytes));
-        if (status != hipSuccess)
-            return status;
-        if (device >= 0 && device < 64)
-            configured[device] = true;
-    }
     dim3 grid(unsigned(p.tiles_n) * unsigned(p.tiles_m), unsigned(split_k));
     kernel<<<grid, WN * WM * 64, lds_bytes, stream>>>(p);
     return launch_status();

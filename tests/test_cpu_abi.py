@@ -195,3 +195,21 @@ def test_contexts_inherited_through_fork_are_refused(monkeypatch):
     monkeypatch.setattr(torch.cuda, "current_stream", lambda device=None: types.SimpleNamespace(cuda_stream=4242))
     with pytest.raises(RuntimeError, match="fork"):
         _native.context(0)
+
+
+def test_plugin_entry_points_are_registered():
+    # pyproject.toml and the hand-written dist-info at the repository root both name the two plugin
+    # groups the reference registers (ref: pyproject.toml:12-16); importlib.metadata finds the
+    # dist-info for any process that has the repository root on its module search path
+    from importlib.metadata import entry_points
+
+    sys.path.insert(0, str(ROOT))
+    try:
+        found = {(group, entry.name, entry.value) for group in ("torch.backends", "sglang.srt.plugins")
+                 for entry in entry_points(group=group)}
+    finally:
+        sys.path.remove(str(ROOT))
+    assert ("torch.backends", "camblas", "camblas_amd:_autoload") in found
+    assert ("sglang.srt.plugins", "camblas", "camblas_amd.sglang:install") in found
+    text = (ROOT / "pyproject.toml").read_text()
+    assert 'camblas = "camblas_amd:_autoload"' in text and 'camblas = "camblas_amd.sglang:install"' in text

@@ -205,6 +205,32 @@ def test_activation_quantiser_invariants():
     assert np.abs(decoded * scale[..., None] - values).max() <= np.abs(values).max() * 2.0**-4
 
 
+def test_activation_quantiser_bytes_match_an_independent_codec():
+    # The bytes, not just their invariants: torch's E4M3fn conversion (a third-party codec, round to
+    # nearest even) applied to clamp(x * fl(448 / amax), +-448) evaluated in FP32 by torch. A
+    # round-half-away encoder, a division by the scale instead of the multiplication by the
+    # reciprocal, or a missing clamp each change bytes here. Constructed ties: with amax = 448 the
+    # factor is exactly 1, so values halfway between two E4M3 neighbours (17 between 16 and 18,
+    # 19 between 18 and 20, 0.0009765625 * 1.5 ... in the subnormal range) must go to the even code.
+    rng = np.random.default_rng(77)
+    x = oracle.fill_normal_bf16(78, (6, 512))
+    ties = np.float32([448, 17, 19, 21, 23, -17, -19, 34, 38, 208, 240, 2.0**-9 * 1.5, 2.0**-9 * 2.5,
+                       2.0**-10, -(2.0**-9) * 0.5, 416 + 16, 0.0, 1.0625, 1.1875])
+    x[0, : ties.size] = oracle.f32_to_bf16(ties)
+    x[0, ties.size:128] = 0
+    x[1, 128:256] = oracle.f32_to_bf16(rng.uniform(-3e-5, 3e-5, 128).astype(np.float32))  # tiny group
+    x[2, :128] = oracle.f32_to_bf16(np.full(128, 1e30, np.float32))                         # huge group
+    q, scale = oracle.quantise_1x128(x)
+    values = torch.from_numpy(oracle.bf16_to_f32(x)).reshape(6, 4, 128)
+    amax = values.abs().amax(dim=2, keepdim=True).clamp_min(1e-10)
+    factor = torch.tensor(448.0, dtype=torch.float32) / amax
+    want = torch.clamp(values * factor, -448.0, 448.0).to(torch.float8_e4m3fn).view(torch.uint8)
+    assert np.array_equal(q.reshape(6, 4, 128), want.numpy())
+    assert np.array_equal(scale.reshape(6, 4, 1), (amax * torch.tensor(1 / 448, dtype=torch.float32)).numpy())
+    # the constructed ties, spelled out: 17 -> 16 (0x58), 19 -> 20 (0x5a), 21 -> 20, 23 -> 24 (0x5c)
+    assert list(q[0, 1:5]) == [0x58, 0x5A, 0x5A, 0x5C]
+
+
 def test_block32_decode_rule_and_power_of_two_quantiser():
     # product: pure-Python chain on a small case, strided scales, the reference's known answers
     # (ref: tests/test_quantized.py:160-216: ones times twos with sx = 0.5, sw = 2, last row block
