@@ -390,8 +390,37 @@ def add_rms_norm(x, residual, weight, epsilon=1e-6, round_before_weight=True):
     return added, out
 
 
+def gated_linear(x, gate_weight, up_weight):
+    """silu_multiply(gate(x), up(x)) for a BF16 decode batch x [rows <= 64, inner] in one pass over both
+    weight matrices [outputs, inner]; the same rounding points as the three separate calls."""
+    _require(x.dtype == gate_weight.dtype == up_weight.dtype == torch.bfloat16 and x.is_cuda,
+             "gated_linear takes BF16 device tensors")
+    _require(x.dim() == 2 and gate_weight.dim() == 2 and gate_weight.shape == up_weight.shape
+             and x.shape[1] == gate_weight.shape[1] and x.shape[0] <= 64, "gated_linear shapes")
+    _require(x.stride(1) == 1 and gate_weight.stride(1) == 1 and up_weight.stride(1) == 1
+             and gate_weight.stride(0) == up_weight.stride(0), "gated_linear needs row-major operands")
+    rows, inner = x.shape
+    outputs = gate_weight.shape[0]
+    out = torch.empty((rows, outputs), dtype=torch.bfloat16, device=x.device)
+    _native.context(x.device).call(
+        "bf16_gated_linear", rows, outputs, inner, _pointer(x), x.stride(0), _pointer(gate_weight),
+        _pointer(up_weight), gate_weight.stride(0), _pointer(out), outputs)
+    return out
+
+
+def _gated_linear_takes(x, gate_weight, up_weight):
+    return (x.dtype == torch.bfloat16 and x.dim() == 2 and 0 < x.shape[0] <= 64 and x.stride(1) == 1
+            and gate_weight.stride(1) == 1 and up_weight.stride(1) == 1
+            and gate_weight.stride(0) == up_weight.stride(0)
+            and all(t.data_ptr() % 16 == 0 for t in (x, gate_weight, up_weight))
+            and all(s % 8 == 0 for s in (x.shape[1], x.stride(0), gate_weight.stride(0))))
+
+
 def gated_mlp(x, gate_weight, up_weight, down_weight):
-    """down(silu_multiply(gate(x), up(x))) (ref: src/cuda/torch_bindings.cpp:703-723)."""
+    """down(silu_multiply(gate(x), up(x))) (ref: src/cuda/torch_bindings.cpp:703-723). A BF16 decode
+    batch takes the one-pass front end; anything else the three separate calls."""
+    if _gated_linear_takes(x, gate_weight, up_weight):
+        return linear(gated_linear(x, gate_weight, up_weight), down_weight)
     gate = linear(x, gate_weight)
     up = linear(x, up_weight)
     silu_multiply(gate, up, out=gate)
@@ -463,7 +492,8 @@ def fp8_moe_decode(x, w1, w2, w1_scale, w2_scale, expert_ids, routing, *, factor
              and w1.dtype == w2.dtype == torch.float8_e4m3fn and w1.is_contiguous() and w2.is_contiguous()
              and w2.shape[0] == experts and doubled == 2 * width,
              "FP8 expert step needs one contiguous BF16 token and E4M3 weights [experts, 2*width, hidden] / [experts, hidden_out, width]")
-    _require(hidden % 128 == 0 and width % 128 == 0 and hidden_out % 16 == 0 and 1 <= choices <= 16,
+    _require(hidden % 128 == 0 and width % 128 == 0 and hidden_out % 16 == 0 and 1 <= choices <= 16
+             and choices * (width // 128) <= 512,
              "FP8 expert step needs hidden and width in multiples of 128, outputs of 16 and 1..16 choices")
     _require(w1_scale.dtype == w2_scale.dtype == torch.float32 and w1_scale.is_contiguous()
              and w2_scale.is_contiguous()

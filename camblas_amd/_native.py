@@ -84,6 +84,7 @@ SIGNATURES = {
     "gqa_decode_attention": ([_P, _I, _I, _I, _I, _I, _P, _F, _P, _I, _P, _P, _P], _I),
     "gqa_decode_attention_noalloc": ([_P, _I, _I, _I, _I, _I, _P, _F, _P, _I, _P, _P, _P], _I),
     "gqa_decode_attention_noalloc_limit": ([], _SZ),
+    "bf16_gated_linear": ([_P, _I, _I, _I, _P, _I, _P, _P, _I, _P, _I], _I),
     "fp8_moe_decode": ([_P, _I, _I, _I, _I, _I, _P, _P, _P, _P, _P, _P, _P, _F, _P], _I),
     "hip_plan_describe": ([_I, _I, _C, _C, _I, _I, _I, _I, _I, _I, _I, ct.c_char_p, _SZ], _I),
     "hip_set_plan_override": ([_P, _I, _I], _I),

@@ -180,6 +180,37 @@ extern "C" int camblas_cuda_rms_scale(camblas_cuda_context *context, int dtype, 
     });
 }
 
+// The front end of a gated MLP for a decode batch, out = silu_multiply(x gate^T, x up^T), as one
+// streaming pass over both weight matrices. The reference composes it from two linears and
+// camblas_cuda_silu_multiply in its binding (src/cuda/torch_bindings.cpp:703-723); the rounding
+// points here are the same (both products and the activation are rounded to BF16).
+extern "C" int camblas_cuda_bf16_gated_linear(camblas_cuda_context *context, int rows, int outputs, int inner,
+                                              const void *x, int ldx, const void *gate, const void *up,
+                                              int ldw, void *out, int ldo)
+{
+    Entry entry(context);
+    return entry.run([&] {
+        if (!within({{rows, 0, 64, 1}, {outputs, 0, INT32_MAX, 1}, {inner, 8, (1 << 23) - 8, 8}, {ldx, inner, (1 << 23) - 8, 8},
+                     {ldw, inner, (1 << 23) - 8, 8}, {ldo, outputs, INT32_MAX, 1}}))
+            return entry.refuse("invalid gated linear dimensions");
+        if (rows == 0 || outputs == 0)
+            return 0;
+        if (!usable({{x, 16}, {gate, 16}, {up, 16}, {out, 2}}) || !apart(out, {x, gate, up}))
+            return entry.refuse("invalid gated linear buffers");
+        const int token_tiles = rows <= 16 ? 1 : rows <= 32 ? 2 : 4;
+        // the widest workgroups that still leave one and a half per compute unit (or a test's choice)
+        int pair_tiles = 4;
+        while (pair_tiles > 1 && (outputs + 16 * pair_tiles - 1) / (16 * pair_tiles) * 2 < 3 * context->compute_units)
+            --pair_tiles;
+        if (context->override_kernel >= 1 && context->override_kernel <= 4)
+            pair_tiles = context->override_kernel;
+        context->counts[4]++;
+        return entry.finish(launch_gated_stream(context->stream, pair_tiles, token_tiles, outputs, rows, inner,
+                                                gate, up, ldw, x, ldx, out, ldo),
+                            "BF16 gated streaming linear");
+    });
+}
+
 // ---- decode-layer pieces (no counterpart in the reference)
 
 extern "C" int camblas_cuda_rope(camblas_cuda_context *context, int tokens, int heads, int dim,

@@ -23,6 +23,7 @@ namespace
 {
 struct StreamParams {
     const unsigned short *w;
+    const unsigned short *w2; // gated form: the "up" weights (w holds the "gate" weights)
     const unsigned short *x;
     unsigned short *y;
     int lda, ldb, ldc;
@@ -35,11 +36,20 @@ constexpr int WAVES = 4, DEPTH = 2;
 
 // NT, MT: 16-row weight tiles and 16-token tiles per workgroup; a K step is KT blocks of 32*WAVES
 // elements, each block split over the WAVES wavefronts; DEPTH K steps are in flight in registers.
-template <int NT, int MT, int KT>
+//
+// GATED: the gated-MLP front end in one pass. The workgroup's first NT/2 tiles are rows of the gate
+// weights, the other NT/2 the SAME rows of the up weights, and the epilogue writes
+// round(round(silu(g)) * u) for g = round(alpha * x Wg^T), u = round(alpha * x Wu^T): the two
+// linears and the SiLU-multiply of the reference's gated MLP (src/cuda/torch_bindings.cpp:703-723,
+// src/cuda/inference_fusion.cuh:19-28) with the same rounding points, without the two
+// activations' round trip through memory and without two of the three launches.
+template <int NT, int MT, int KT, bool GATED>
 __global__ __launch_bounds__(WAVES * 64) void bgemv_stream_kernel(StreamParams p)
 {
-    constexpr int ROWS = NT * 16, XROWS = MT * 16, CH = 4 * WAVES, BK = 32 * WAVES;
-    constexpr int BLOCK_SLOTS = (ROWS + XROWS) * CH, STAGE_SLOTS = BLOCK_SLOTS * KT;
+    static_assert(!GATED || NT % 2 == 0, "gate and up tiles come in pairs");
+    constexpr int HALF = GATED ? NT / 2 : NT; // distinct 16-row blocks of output rows
+    constexpr int ROWS = HALF * 16, XROWS = MT * 16, CH = 4 * WAVES, BK = 32 * WAVES;
+    constexpr int BLOCK_SLOTS = (NT * 16 + XROWS) * CH, STAGE_SLOTS = BLOCK_SLOTS * KT;
     extern __shared__ __attribute__((aligned(16))) unsigned char lds_bytes[];
     u32x4_t *lds = reinterpret_cast<u32x4_t *>(lds_bytes);
 
@@ -51,7 +61,7 @@ __global__ __launch_bounds__(WAVES * 64) void bgemv_stream_kernel(StreamParams p
     unsigned a_off[NT], b_off[MT];
 #pragma unroll
     for (int i = 0; i < NT; ++i) {
-        int row = n0 + i * 16 + pass_row;
+        int row = n0 + (i % HALF) * 16 + pass_row;
         row = row < p.n ? row : p.n - 1;
         a_off[i] = unsigned(row - n0) * unsigned(p.lda);
     }
@@ -62,6 +72,7 @@ __global__ __launch_bounds__(WAVES * 64) void bgemv_stream_kernel(StreamParams p
         b_off[j] = unsigned(row - m0) * unsigned(p.ldb);
     }
     const unsigned short *a_base = p.w + size_t(n0) * p.lda;
+    const unsigned short *a2_base = GATED ? p.w2 + size_t(n0) * p.lda : a_base;
     const unsigned short *b_base = p.x + size_t(m0) * p.ldb;
     // LDS slot of this thread's chunk inside a 16-row pass; passes are 256 slots apart
     const int store_slot = pass_row * CH + (chunk ^ pass_row);
@@ -94,8 +105,8 @@ __global__ __launch_bounds__(WAVES * 64) void bgemv_stream_kernel(StreamParams p
             k0 &= int(live);
 #pragma unroll
             for (int i = 0; i < NT; ++i)
-                a[t][i] = __builtin_nontemporal_load(
-                    reinterpret_cast<const u32x4_t *>(a_base + k0 + (a_off[i] & live)));
+                a[t][i] = __builtin_nontemporal_load(reinterpret_cast<const u32x4_t *>(
+                    (i < HALF ? a_base : a2_base) + k0 + (a_off[i] & live)));
 #pragma unroll
             for (int j = 0; j < MT; ++j)
                 b[t][j] = *reinterpret_cast<const u32x4_t *>(b_base + k0 + (b_off[j] & live));
@@ -180,8 +191,15 @@ __global__ __launch_bounds__(WAVES * 64) void bgemv_stream_kernel(StreamParams p
     __syncthreads();
     // ---- epilogue: wavefront w writes tiles w, w+4, ...; register r of lane l is feature
     // 4*(l/16) + r and token l%16 inside the 16x16 tile
+    auto summed = [&](int index) {
+        f32x4_t sum = combine[index * 64 + lane];
 #pragma unroll
-    for (int index = 0; index < NT * MT; ++index) {
+        for (int w = 1; w < WAVES; ++w)
+            sum = sum + combine[(w * NT * MT + index) * 64 + lane];
+        return sum;
+    };
+#pragma unroll
+    for (int index = 0; index < HALF * MT; ++index) {
         if (index % WAVES != wave)
             continue;
         const int i = index / MT, j = index % MT;
@@ -189,12 +207,28 @@ __global__ __launch_bounds__(WAVES * 64) void bgemv_stream_kernel(StreamParams p
         const int n = n0 + i * 16 + (lane / 16) * 4;
         if (m >= p.m || n >= p.n)
             continue;
-        f32x4_t sum = combine[index * 64 + lane];
-#pragma unroll
-        for (int w = 1; w < WAVES; ++w)
-            sum = sum + combine[(w * NT * MT + index) * 64 + lane];
+        const f32x4_t sum = summed(index);
         float v[4] = {sum[0], sum[1], sum[2], sum[3]};
         unsigned short *out = p.y + size_t(m) * p.ldc + n;
+        if constexpr (GATED) {
+            const f32x4_t raised = summed((i + HALF) * MT + j);
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                const float g = bf16_bits_to_float(float_to_bf16_bits(p.alpha * v[e]));
+                const float u = bf16_bits_to_float(float_to_bf16_bits(p.alpha * raised[e]));
+                const float activated = bf16_bits_to_float(float_to_bf16_bits(g / (1.f + expf(-g))));
+                v[e] = __fmul_rn(activated, u);
+            }
+            if (n + 3 < p.n && p.vector_store) {
+                *reinterpret_cast<u32x2_t *>(out) = u32x2_t{pack_bf16x2(v[0], v[1]), pack_bf16x2(v[2], v[3])};
+            } else {
+#pragma unroll
+                for (int e = 0; e < 4; ++e)
+                    if (n + e < p.n)
+                        out[e] = float_to_bf16_bits(v[e]);
+            }
+            continue;
+        }
         if (n + 3 < p.n && p.vector_store) {
             if (p.beta != 0.f) {
                 u32x2_t old = *reinterpret_cast<const u32x2_t *>(out);
@@ -223,7 +257,7 @@ __global__ __launch_bounds__(WAVES * 64) void bgemv_stream_kernel(StreamParams p
     }
 }
 
-template <int NT, int MT, int KT>
+template <int NT, int MT, int KT, bool GATED = false>
 hipError_t launch_one(hipStream_t stream, const StreamParams &p)
 {
     constexpr size_t stage_bytes = size_t(2) * KT * (NT + MT) * 16 * (64 * WAVES);
@@ -233,13 +267,13 @@ hipError_t launch_one(hipStream_t stream, const StreamParams &p)
     if constexpr (NT * KT > 8 || lds_bytes > 128 * 1024) {
         return hipErrorInvalidValue;
     } else {
-        auto kernel = bgemv_stream_kernel<NT, MT, KT>;
+        auto kernel = bgemv_stream_kernel<NT, MT, KT, GATED>;
         static LdsLimitFlags limits; // (one per instantiation)
         const hipError_t status = raise_lds_limit(limits, reinterpret_cast<const void *>(kernel), lds_bytes);
         if (status != hipSuccess)
             return status;
-        dim3 grid(unsigned((p.n + NT * 16 - 1) / (NT * 16)),
-                  unsigned((p.m + MT * 16 - 1) / (MT * 16)));
+        constexpr int rows = (GATED ? NT / 2 : NT) * 16;
+        dim3 grid(unsigned((p.n + rows - 1) / rows), unsigned((p.m + MT * 16 - 1) / (MT * 16)));
         kernel<<<grid, WAVES * 64, lds_bytes, stream>>>(p);
         return launch_status();
     }
@@ -273,12 +307,53 @@ hipError_t launch_tokens(hipStream_t stream, int row_tiles, int token_tiles, con
 }
 } // namespace
 
+// Gated form: out[m, n] = round(round(silu(g)) * u) with g = round(x Wg^T), u = round(x Wu^T); a
+// workgroup owns 16 * pair_tiles output rows (that many gate rows and the same up rows) over the
+// whole K. pair_tiles 1..4, token_tiles 1, 2 or 4.
+hipError_t launch_gated_stream(hipStream_t stream, int pair_tiles, int token_tiles, int n_out, int m_rows,
+                               int k, const void *gate, const void *up, int lda, const void *x, int ldb,
+                               void *y, int ldc)
+{
+    StreamParams p;
+    p.w = static_cast<const unsigned short *>(gate);
+    p.w2 = static_cast<const unsigned short *>(up);
+    p.x = static_cast<const unsigned short *>(x);
+    p.y = static_cast<unsigned short *>(y);
+    p.lda = lda;
+    p.ldb = ldb;
+    p.ldc = ldc;
+    p.n = n_out;
+    p.m = m_rows;
+    p.k = k;
+    p.alpha = 1.f;
+    p.beta = 0.f;
+    p.vector_store = (ldc % 4 == 0) && (reinterpret_cast<uintptr_t>(y) % 8 == 0);
+    if ((m_rows + token_tiles * 16 - 1) / (token_tiles * 16) > 65535)
+        return hipErrorInvalidValue;
+    switch (token_tiles * 10 + pair_tiles) {
+    case 11: return launch_one<2, 1, 1, true>(stream, p);
+    case 12: return launch_one<4, 1, 1, true>(stream, p);
+    case 13: return launch_one<6, 1, 1, true>(stream, p);
+    case 14: return launch_one<8, 1, 1, true>(stream, p);
+    case 21: return launch_one<2, 2, 1, true>(stream, p);
+    case 22: return launch_one<4, 2, 1, true>(stream, p);
+    case 23: return launch_one<6, 2, 1, true>(stream, p);
+    case 24: return launch_one<8, 2, 1, true>(stream, p);
+    case 41: return launch_one<2, 4, 1, true>(stream, p);
+    case 42: return launch_one<4, 4, 1, true>(stream, p);
+    case 43: return launch_one<6, 4, 1, true>(stream, p);
+    case 44: return launch_one<8, 4, 1, true>(stream, p);
+    default: return hipErrorInvalidValue;
+    }
+}
+
 hipError_t launch_bgemv_stream(hipStream_t stream, int depth_log2, int row_tiles, int token_tiles, int n_out,
                                int m_rows, int k, float alpha, const void *w, int lda,
                                const void *x, int ldb, float beta, void *y, int ldc)
 {
     StreamParams p;
     p.w = static_cast<const unsigned short *>(w);
+    p.w2 = nullptr;
     p.x = static_cast<const unsigned short *>(x);
     p.y = static_cast<unsigned short *>(y);
     p.lda = lda;

@@ -162,6 +162,12 @@ hipError_t launch_bgemm_dma(hipStream_t stream, int variant, int n_out, int m_ro
 hipError_t launch_bgemv_stream(hipStream_t stream, int depth_log2, int row_tiles, int token_tiles, int n_out,
                                int m_rows, int k, float alpha, const void *w, int lda,
                                const void *x, int ldb, float beta, void *y, int ldc);
+// The gated-MLP front end for decode batches in one pass over both weight matrices:
+// y = round(round(silu(g)) * u), g = round(x gate^T), u = round(x up^T). pair_tiles 1..4 (16 output
+// rows each: that many gate rows and the same up rows per workgroup), token_tiles 1, 2 or 4.
+hipError_t launch_gated_stream(hipStream_t stream, int pair_tiles, int token_tiles, int n_out, int m_rows,
+                               int k, const void *gate, const void *up, int lda, const void *x, int ldb,
+                               void *y, int ldc);
 hipError_t launch_fp8_block(hipStream_t stream, int variant, int split_k, int rows, int outputs,
                             int inner, const void *a, const float *a_scale, const void *w,
                             const float *w_scale, void *out, float *partials);

@@ -129,7 +129,7 @@ def build_hooks(selected):
                 and input.dtype == torch.bfloat16 and weight.dtype == torch.float8_e4m3fn
                 and list(block_size) == [128, 128] and weight_scale.dtype == torch.float32
                 and input.shape[-1] == weight.shape[1] and weight.shape[1] % 128 == 0
-                and input.numel() > 0
+                and input.numel() > 0 and input.numel() // input.shape[-1] <= 65535
                 and tuple(weight_scale.shape) == ((weight.shape[0] + 127) // 128, weight.shape[1] // 128)
                 and input_scale is None and bias is None
                 and all(t.is_contiguous() and t.device == input.device
@@ -198,6 +198,7 @@ def build_hooks(selected):
                                                            "per_channel_quant", "fuse_swiglu_interleaved"))
                 and all(kwargs.get(k) is None for k in ("b1", "b2", "w1_zp", "w2_zp", "a1_scale", "a2_scale", "a1_q"))
                 and ids.dtype == torch.int32 and ids.ndim == 2 and ids.shape[0] == 1 and 1 <= ids.shape[1] <= 16
+                and ids.shape[1] * (w2.shape[2] // 128) <= 512
                 and routing.dtype == torch.float32 and routing.shape == ids.shape
                 and all(t is not None and t.dtype == torch.float32 for t in scales)
                 and tuple(scales[0].shape) == (w1.shape[0], w1.shape[1] // 128, w1.shape[2] // 128)

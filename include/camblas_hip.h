@@ -255,6 +255,17 @@ int camblas_cuda_add_rms_norm_rows(camblas_cuda_context *context, int dtype, int
  * x [tokens, heads, dim] whose token stride is token_stride elements; positions int32 [tokens]. */
 int camblas_cuda_rope(camblas_cuda_context *context, int tokens, int heads, int dim,
                       int token_stride, float theta, const int32_t *positions, void *x_bf16);
+/* extension. The front end of a gated MLP for a decode batch (at most 64 rows) in one streaming pass
+ * over both weight matrices: out[rows, outputs] = silu_multiply(x gate^T, x up^T), BF16 storage,
+ * FP32 accumulation, with the rounding points of the composition the reference's binding makes from
+ * two linears and camblas_cuda_silu_multiply (src/cuda/torch_bindings.cpp:703-723,
+ * src/cuda/inference_fusion.cuh:19-28): g = bf16(x gate^T), u = bf16(x up^T),
+ * out = bf16(bf16(silu(g)) * u). x [rows, inner] with row stride ldx, gate and up [outputs, inner]
+ * with row stride ldw, out with row stride ldo (elements). inner, ldx and ldw multiples of 8;
+ * x, gate, up 16-byte aligned. More than 64 rows are refused: compose the three calls instead. */
+int camblas_cuda_bf16_gated_linear(camblas_cuda_context *context, int rows, int outputs, int inner,
+                                   const void *x, int ldx, const void *gate, const void *up, int ldw,
+                                   void *out, int ldo);
 /* extension (no reference counterpart). Writes each sequence's new K and V heads, rows of k_new /
  * v_new [batch, kv_heads*dim] with row stride token_stride elements (e.g. slices of a fused QKV
  * activation), into the caches [batch, context, kv_heads, dim] at positions[batch]; positions

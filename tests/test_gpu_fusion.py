@@ -222,3 +222,52 @@ def test_rope_kv_append_equals_rope_then_append(device):
     assert np.array_equal(from_device_bf16(kf)[3], k_cache[3])  # position 40 is outside the cache
     want = oracle.rope(qkv[:, : q_heads + kv_heads], positions.cpu().numpy(), 5e5)
     assert rel_frobenius(bf16_values(fused[:, : q_heads + kv_heads]), oracle.bf16_to_f32(want)) <= 1e-2
+
+
+@pytest.mark.parametrize("rows,outputs,inner,pairs", [(1, 100, 256, None), (7, 130, 264, 1), (32, 300, 512, 2),
+                                                        (33, 70, 136, 3), (64, 257, 1024, 4), (32, 1024, 2048, None)])
+def test_gated_linear_equals_the_three_call_composition(device, rows, outputs, inner, pairs):
+    # one pass over both weight matrices against linear, linear, silu_multiply: the rounding points
+    # are the same and only the order of the FP32 sums inside a product may differ (the planner is
+    # free to give the separate products another kernel), so the two agree to a few BF16 units in
+    # a few places; and the oracle's composition holds within the BF16 bar
+    from camblas_amd import _native
+
+    x = oracle.fill_normal_bf16(500 + rows, (rows, inner))
+    gate = oracle.fill_normal_bf16(501, (outputs, inner), std=0.05)
+    up = oracle.fill_normal_bf16(502, (outputs, inner), std=0.05)
+    xt, gt, ut = (to_device_bf16(v, device) for v in (x, gate, up))
+    native = _native.context(device)
+    if pairs is not None:
+        native.call("hip_set_plan_override", pairs, 0)
+    try:
+        fused = _kernels.gated_linear(xt, gt, ut)
+    finally:
+        native.call("hip_set_plan_override", -1, 0)
+    g, u = _kernels.linear(xt, gt), _kernels.linear(xt, ut)
+    composed = _kernels.silu_multiply(g, u)
+    torch.cuda.synchronize()
+    assert rel_frobenius(bf16_values(fused), bf16_values(composed)) <= 4e-3
+    want_g = oracle.f32_to_bf16(oracle.linear_bf16_f64(x, gate).astype(np.float32))
+    want_u = oracle.f32_to_bf16(oracle.linear_bf16_f64(x, up).astype(np.float32))
+    want = oracle.bf16_to_f32(oracle.silu_multiply(2, want_g, want_u))
+    assert rel_frobenius(bf16_values(fused), want) <= 2e-2  # two BF16-rounded products, then two roundings
+
+
+def test_gated_linear_refuses_what_it_does_not_take(device):
+    import ctypes as ct
+
+    from camblas_amd import _native
+    from helpers import ptr
+
+    native, lib = _native.context(device), _native.library()
+    x = torch.zeros((65, 64), dtype=torch.bfloat16, device=device)
+    w = torch.zeros((32, 64), dtype=torch.bfloat16, device=device)
+    out = torch.zeros((65, 32), dtype=torch.bfloat16, device=device)
+    call = lib.camblas_cuda_bf16_gated_linear
+    assert call(native.handle, 65, 32, 64, ptr(x), 64, ptr(w), ptr(w), 64, ptr(out), 32) == -1
+    assert b"invalid gated linear dimensions" in lib.camblas_cuda_error(native.handle)
+    assert call(native.handle, 8, 32, 60, ptr(x), 64, ptr(w), ptr(w), 64, ptr(out), 32) == -1
+    assert call(native.handle, 8, 32, 64, ptr(x), 64, ptr(w), ptr(w), 64, ptr(x), 32) == -1
+    assert b"invalid gated linear buffers" in lib.camblas_cuda_error(native.handle)
+    assert call(native.handle, 0, 32, 64, None, 64, None, None, 64, None, 32) == 0

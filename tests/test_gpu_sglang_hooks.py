@@ -283,3 +283,40 @@ def routed_and_refused(hook, original, before, layer, x, weight, batch, rows, in
             torch.backends.cuda.matmul.allow_bf16_reduced_precision_reduction = False
     assert hook(original, layer, x) == "original"  # grad mode on
     assert len(original.calls) == len(refused) + 2 and delta(before, "bmm") == 1
+
+
+def test_hooks_leave_what_the_entry_points_refuse_to_the_original(device):
+    # the guards stop where the C entry points do: more than 65535 rows for the block-128 product,
+    # more than 512 (choice, 128-wide group) pairs for the fused expert step; both must reach
+    # SGLang's own function instead of raising inside the hook
+    hooks = plugin.build_hooks({"fp8"})
+    original = Original()
+    rows, outputs, inner = 65536, 128, 128
+    x = torch.zeros((rows, inner), dtype=torch.bfloat16, device=device)
+    w = torch.zeros((outputs, inner), dtype=torch.uint8, device=device).view(torch.float8_e4m3fn)
+    scale = torch.ones((1, 1), dtype=torch.float32, device=device)
+    with torch.no_grad():
+        assert hooks[plugin.FP8_BLOCK128_TARGET](original, x, w, [128, 128], scale) == "original"
+        out = hooks[plugin.FP8_BLOCK128_TARGET](original, x[:65535], w, [128, 128], scale)
+    assert out.shape == (65535, outputs) and len(original.calls) == 1
+
+    class KeywordOriginal(Original):
+        def __call__(self, *arguments, **kwargs):
+            return super().__call__(*arguments)
+
+    original = KeywordOriginal()
+    experts, choices, hidden, width = 16, 16, 128, 128 * 33        # 16 * 33 = 528 pairs
+    xt = torch.zeros((1, hidden), dtype=torch.bfloat16, device=device)
+    w1 = torch.zeros((experts, 2 * width, hidden), dtype=torch.uint8, device=device).view(torch.float8_e4m3fn)
+    w2 = torch.zeros((experts, hidden, width), dtype=torch.uint8, device=device).view(torch.float8_e4m3fn)
+    topk = types.SimpleNamespace(topk_ids=torch.arange(choices, dtype=torch.int32, device=device).view(1, -1),
+                                 topk_weights=torch.ones((1, choices), dtype=torch.float32, device=device))
+    keywords = dict(w1_scale=torch.ones((experts, 2 * width // 128, 1), device=device),
+                    w2_scale=torch.ones((experts, 1, width // 128), device=device),
+                    use_fp8_w8a8=True, block_shape=[128, 128])
+    with torch.no_grad():
+        assert hooks[plugin.FP8_MOE_TARGET](original, xt, w1, w2, topk, moe_configuration(experts), **keywords) == "original"
+        with pytest.raises(RuntimeError):
+            _kernels.fp8_moe_decode(xt, w1, w2, keywords["w1_scale"], keywords["w2_scale"],
+                                    topk.topk_ids.view(-1), topk.topk_weights.view(-1))
+    assert len(original.calls) == 1
