@@ -388,7 +388,13 @@ def extras(torch, _kernels, _native, device, normal):
     seconds = event_time(torch, lambda i: _kernels.addmm(c, x, w.t(), beta=1.0), 3, 10)
     found["bf16_prefill_addmm_beta1"] = {
         "us": round(seconds * 1e6, 1), "tflops": round(flops / seconds / 1e12, 1),
-        "note": "includes the bias expand+clone copy, as in the reference binding",
+        "note": "full [tokens, outputs] addend read by the product's epilogue (no expand+clone copy)",
+    }
+    row = normal((outputs,))
+    seconds = event_time(torch, lambda i: _kernels.addmm(row, x, w.t(), beta=1.0), 3, 10)
+    found["bf16_prefill_addmm_bias_row"] = {
+        "us": round(seconds * 1e6, 1), "tflops": round(flops / seconds / 1e12, 1),
+        "note": "[outputs] bias row of a linear layer, read by the product's epilogue",
     }
     del x, w, y, c
     # FP8 block-scaled linear; the decode sizes rotate three weight copies (396 MB) so that the

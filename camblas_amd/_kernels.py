@@ -128,14 +128,43 @@ def linear(x, weight, bias=None):
     return result.reshape(*x.shape[:-1], weight.shape[0])
 
 
-def addmm(bias, a, b, beta=1.0, alpha=1.0):
-    """beta * bias + alpha * a @ b; the bias is expanded and cloned, then updated in place.
+def _epilogue_addend(bias, a, rows, columns):
+    """(pointer holder, row pitch) of a BF16 bias the product can read where it lies, else None:
+    one row for all output rows ([n], [1, n]) or a full [rows, n] matrix, unit stride along n."""
+    if (a.dtype != torch.bfloat16 or bias.dtype != torch.bfloat16 or bias.device != a.device or bias.dim() not in (1, 2)
+            or bias.shape[-1] != columns or (columns > 1 and bias.stride(-1) != 1)):
+        return None
+    if bias.dim() == 1 or bias.shape[0] == 1:
+        return bias, 0
+    if bias.shape[0] != rows or (rows > 1 and bias.stride(0) < columns):
+        return None
+    return bias, (bias.stride(0) if rows > 1 else 0)
 
-    ref: src/cuda/torch_backend.cuh:59-71
+
+def addmm(bias, a, b, beta=1.0, alpha=1.0):
+    """beta * bias + alpha * a @ b, rounded once.
+
+    A BF16 bias row or matrix with unit stride along the output features is read by the product's
+    epilogue (camblas_cuda_bgemm_add); any other broadcast form is expanded and cloned, then updated
+    in place, as the reference does for every form (ref: src/cuda/torch_backend.cuh:59-71).
     """
     m, n = a.shape[0], b.shape[1]
     if beta == 0:
         return matmul(a, b, None, alpha, 0.0)
+    addend = _epilogue_addend(bias, a, m, n) if m > 0 and n > 0 and a.shape[1] > 0 else None
+    if addend is not None:
+        _validate(a, a)
+        _validate(b, a)
+        _require(a.dim() == 2 and b.dim() == 2 and a.shape[1] == b.shape[0],
+                 "matmul requires compatible rank-two operands")
+        out = torch.empty((m, n), dtype=a.dtype, device=a.device)
+        left, left_trans, left_ld = _operand(b)
+        right, right_trans, right_ld = _operand(a)
+        with torch.cuda.device(a.device):
+            _native.context(a.device).call(
+                "bgemm_add", left_trans, right_trans, n, m, a.shape[1], ct.c_float(alpha), _pointer(left), left_ld,
+                _pointer(right), right_ld, ct.c_float(beta), _pointer(addend[0]), addend[1], _pointer(out), max(1, n))
+        return out
     out = bias.expand(m, n).clone(memory_format=torch.contiguous_format)
     return matmul(a, b, out, alpha, beta)
 

@@ -54,6 +54,7 @@ SIGNATURES = {
     "sgemm": (_gemm(_F), _I),
     "dgemm": (_gemm(_D), _I),
     "bgemm": (_gemm(_F), _I),
+    "bgemm_add": ([_P, _C, _C, _I, _I, _I, _F, _P, _I, _P, _I, _F, _P, _I, _P, _I], _I),
     "affine": ([_P, _I, _I, _I, _I, _P, _P, _P, _I, _P], _I),
     "mlp": ([_P, _I, _I, _I, _I, _I, _P, _P, _P, _P, _P, _P, _P], _I),
     "attention": ([_P, _I, _I, _I, _I, _I, _D, _P, _P, _P, _P], _I),

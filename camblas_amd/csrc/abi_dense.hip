@@ -323,14 +323,16 @@ template <typename T> struct BackwardPass {
 };
 
 // BF16 'T','N' and the other layouts: the planner's kernel, or the one a test forced.
+// `source`: where the beta term is read from when that is not C itself (see BetaSource). The
+// K-contiguous families read it in their epilogues; for the others it is first spread over C.
 int bf16_product(const Entry &entry, const Product &p, float alpha, const void *a, const void *b, float beta,
-                 void *c)
+                 void *c, BetaSource source = {})
 {
     camblas_cuda_context *context = entry.context();
     hipStream_t stream = context->stream;
     Plan plan = make_plan(2, context->algorithm, p.trans_a, p.trans_b, p.m, p.n, p.k, p.lda, p.ldb, p.ldc,
                           is_aligned(a, 16) && is_aligned(b, 16), context->compute_units);
-    if (plan.family == FAMILY_DMA && !is_aligned(c, 8))
+    if (plan.family == FAMILY_DMA && (!is_aligned(c, 8) || !is_aligned(source.z, 8) || source.ldz % 4))
         plan.family = FAMILY_MFMA_TN; // same tile shapes, register-staged loads, scalar stores
     const bool matrix_family =
         plan.family == FAMILY_MFMA_TN || plan.family == FAMILY_STREAM || plan.family == FAMILY_DMA;
@@ -351,17 +353,25 @@ int bf16_product(const Entry &entry, const Product &p, float alpha, const void *
             plan.split_k = std::max(1, context->override_split);
         }
     }
+    const bool in_epilogue =
+        plan.family == FAMILY_MFMA_TN || plan.family == FAMILY_STREAM || plan.family == FAMILY_DMA;
+    if (source.z && !in_epilogue) {
+        const hipError_t spread = launch_spread_bf16(stream, p.m, p.n, source.z, source.ldz, c, p.ldc);
+        if (spread != hipSuccess)
+            return entry.finish(spread, "BF16 GEMM addend");
+        source = BetaSource{};
+    }
     switch (plan.family) {
     case FAMILY_DMA:
         context->counts[plan.counter]++;
         return entry.finish(launch_bgemm_dma(stream, plan.kernel, p.m, p.n, p.k, alpha, a, p.lda, b, p.ldb, beta,
-                                             c, p.ldc),
+                                             c, p.ldc, source),
                             "BF16 MFMA GEMM (direct LDS loads)");
     case FAMILY_STREAM:
         context->counts[plan.counter]++;
         return entry.finish(launch_bgemv_stream(stream, plan.kernel / 100, plan.kernel / 10 % 10,
                                                 plan.kernel % 10, p.m, p.n, p.k, alpha, a, p.lda, b, p.ldb,
-                                                beta, c, p.ldc),
+                                                beta, c, p.ldc, source),
                             "BF16 streaming GEMV");
     case FAMILY_MFMA_TN: {
         float *partials = nullptr;
@@ -376,7 +386,7 @@ int bf16_product(const Entry &entry, const Product &p, float alpha, const void *
         }
         context->counts[plan.counter]++;
         return entry.finish(launch_bgemm_tn(stream, plan.kernel, plan.split_k, p.m, p.n, p.k, alpha, a, p.lda, b,
-                                            p.ldb, beta, c, p.ldc, partials),
+                                            p.ldb, beta, c, p.ldc, partials, source),
                             "BF16 MFMA GEMM");
     }
     case FAMILY_MFMA_BF16:
@@ -433,6 +443,46 @@ extern "C" int camblas_cuda_bgemm(camblas_cuda_context *context, char trans_a, c
             return launch_scale_bf16(context->stream, m, n, beta, c, ldc);
         });
         return admitted <= 0 ? admitted : bf16_product(entry, p, alpha, a, b, beta, c);
+    });
+}
+
+// C = alpha op(A) op(B) + beta Z with the addend Z apart from C: an m x n matrix with leading
+// dimension ldz >= m, or one column of m values repeated n times (ldz == 0), which is the bias row
+// of a linear layer seen column-major. What aten::addmm needs without first spreading the bias
+// over the output (the reference spreads it: src/cuda/torch_backend.cuh:60-88).
+extern "C" int camblas_cuda_bgemm_add(camblas_cuda_context *context, char trans_a, char trans_b, int m,
+                                      int n, int k, float alpha, const void *a, int lda, const void *b,
+                                      int ldb, float beta, const void *z, int ldz, void *c, int ldc)
+{
+    if (beta == 0.f) // Z is never read
+        return camblas_cuda_bgemm(context, trans_a, trans_b, m, n, k, alpha, a, lda, b, ldb, 0.f, c, ldc);
+    static const char *const names[4] = {"invalid BF16 GEMM arguments",
+                                         "invalid BF16 pointer or leading dimension", "scale BF16 output",
+                                         "missing or aliased BF16 GEMM operand"};
+    Entry entry(context);
+    return entry.run([&] {
+        const Product p(trans_a, trans_b, m, n, k, lda, ldb, ldc);
+        if (!p.well_formed() || ldz < 0)
+            return entry.refuse(names[0]);
+        if (p.empty())
+            return 0;
+        if (!c || !z || !p.strides_cover() || (ldz != 0 && ldz < m))
+            return entry.refuse(names[1]);
+        // the two stored extents may not overlap: C is written while Z is still being read
+        const char *z_first = static_cast<const char *>(z), *c_first = static_cast<const char *>(c);
+        const size_t z_bytes = (size_t(ldz) * size_t(n - 1) + size_t(m)) * 2;
+        const size_t c_bytes = (size_t(ldc) * size_t(n - 1) + size_t(m)) * 2;
+        if (z_first < c_first + c_bytes && c_first < z_first + z_bytes)
+            return entry.refuse(names[3]);
+        if (alpha == 0.f || k == 0) { // only beta acts
+            const hipError_t spread = launch_spread_bf16(context->stream, m, n, z, ldz, c, ldc);
+            if (spread != hipSuccess)
+                return entry.finish(spread, "BF16 GEMM addend");
+            return beta == 1.f ? 0 : entry.finish(launch_scale_bf16(context->stream, m, n, beta, c, ldc), names[2]);
+        }
+        if (!a || !b || a == c || b == c)
+            return entry.refuse(names[3]);
+        return bf16_product(entry, p, alpha, a, b, beta, c, BetaSource{z, ldz});
     });
 }
 

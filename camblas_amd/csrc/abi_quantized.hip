@@ -33,15 +33,12 @@ Plan fp8_plan(const camblas_cuda_context *context, int rows, int outputs, int in
     if (forced >= 100) {
         plan.family = FAMILY_FP8_STREAM;
         plan.kernel = forced - 100;
-    } else if (forced >= 20) {
-        plan.family = FAMILY_FP8_DMA;
-        plan.kernel = forced - 20;
-    } else {
-        plan.family = FAMILY_FP8_BLOCK;
-        plan.kernel = forced;
-        if (context->override_split > 0)
-            plan.split_k = context->override_split;
+        return plan;
     }
+    plan.family = forced >= 20 ? FAMILY_FP8_DMA : FAMILY_FP8_BLOCK;
+    plan.kernel = forced >= 20 ? forced - 20 : forced;
+    if (context->override_split > 0)
+        plan.split_k = std::min(context->override_split, inner / 128);
     return plan;
 }
 
@@ -88,12 +85,6 @@ extern "C" int camblas_cuda_fp8_block_matmul(camblas_cuda_context *context, int 
                                                   a, a_scale, w, w_scale, out),
                                 "FP8 block-scaled streaming GEMV");
         }
-        if (plan.family == FAMILY_FP8_DMA) {
-            context->counts[plan.counter]++;
-            return entry.finish(launch_fp8_dma(stream, plan.kernel, rows, outputs, inner, a, a_scale, w, w_scale,
-                                               out),
-                                "FP8 block-scaled GEMM (direct LDS loads)");
-        }
         float *partials = nullptr;
         if (plan.split_k > 1) {
             // without room for the partials (allocation failure, capture in progress) run unsplit
@@ -106,6 +97,10 @@ extern "C" int camblas_cuda_fp8_block_matmul(camblas_cuda_context *context, int 
             }
         }
         context->counts[plan.counter]++;
+        if (plan.family == FAMILY_FP8_DMA)
+            return entry.finish(launch_fp8_dma(stream, plan.kernel, plan.split_k, rows, outputs, inner, a, a_scale,
+                                               w, w_scale, out, partials),
+                                "FP8 block-scaled GEMM (direct LDS loads)");
         return entry.finish(launch_fp8_block(stream, plan.kernel, plan.split_k, rows, outputs, inner, a, a_scale,
                                              w, w_scale, out, partials),
                             "FP8 block-scaled GEMM");

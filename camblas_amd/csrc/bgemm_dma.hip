@@ -25,7 +25,8 @@ struct DmaParams {
     const unsigned short *w;
     const unsigned short *x;
     unsigned short *y;
-    int lda, ldb, ldc;
+    const unsigned short *z; // what beta multiplies: z[token * ldz + feature] (y and ldc by default)
+    int lda, ldb, ldc, ldz;
     int n, m, k;
     float alpha, beta;
     int tiles_n, tiles_m;
@@ -224,6 +225,7 @@ __global__ __launch_bounds__(128 * WM) void bgemm_dma_kernel(DmaParams p)
     for (int j = 0; j < TM; ++j) {
         const int m = m0 + (wm * TM + j) * 32 + frag_row;
         unsigned short *row = p.y + size_t(m) * p.ldc + n0 + wn * TN * 32 + half * 4;
+        const unsigned short *source = p.z + size_t(m) * p.ldz + n0 + wn * TN * 32 + half * 4;
 #pragma unroll
         for (int i = 0; i < TN; ++i) {
             __builtin_amdgcn_sched_barrier(0); // keep one accumulator tile live at a time
@@ -234,7 +236,7 @@ __global__ __launch_bounds__(128 * WM) void bgemm_dma_kernel(DmaParams p)
                     float v0 = p.alpha * acc[i][j][q * 4], v1 = p.alpha * acc[i][j][q * 4 + 1];
                     float v2 = p.alpha * acc[i][j][q * 4 + 2], v3 = p.alpha * acc[i][j][q * 4 + 3];
                     if (with_beta) {
-                        u32x2_t old = *reinterpret_cast<const u32x2_t *>(row + offset);
+                        u32x2_t old = *reinterpret_cast<const u32x2_t *>(source + offset);
                         v0 = fmaf(p.beta, __uint_as_float(old[0] << 16), v0);
                         v1 = fmaf(p.beta, __uint_as_float(old[0] & 0xffff0000u), v1);
                         v2 = fmaf(p.beta, __uint_as_float(old[1] << 16), v2);
@@ -278,9 +280,11 @@ const TnVariant &dma_variant(int index) { return variants[index]; }
 
 hipError_t launch_bgemm_dma(hipStream_t stream, int variant, int n_out, int m_rows, int k,
                             float alpha, const void *w, int lda, const void *x, int ldb, float beta,
-                            void *y, int ldc)
+                            void *y, int ldc, const BetaSource &source)
 {
     if (k % 64 || n_out % 4 || ldc % 4 || reinterpret_cast<uintptr_t>(y) % 8)
+        return hipErrorInvalidValue;
+    if (source.z && (source.ldz % 4 || reinterpret_cast<uintptr_t>(source.z) % 8))
         return hipErrorInvalidValue;
     // per-lane byte offsets are 32-bit: 256 rows of the widest operand plus the K extent must fit
     if ((size_t(256) * size_t(lda > ldb ? lda : ldb) + size_t(k)) * 2 >= (size_t(1) << 32))
@@ -292,6 +296,8 @@ hipError_t launch_bgemm_dma(hipStream_t stream, int variant, int n_out, int m_ro
     p.lda = lda;
     p.ldb = ldb;
     p.ldc = ldc;
+    p.z = source.z ? static_cast<const unsigned short *>(source.z) : p.y;
+    p.ldz = source.z ? source.ldz : ldc;
     p.n = n_out;
     p.m = m_rows;
     p.k = k;

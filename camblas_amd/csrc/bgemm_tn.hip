@@ -30,7 +30,9 @@ struct TnParams {
     int n, m, k;
     float alpha, beta;
     int tiles_n, tiles_m, k_per_split;
-    int vector_store; // y rows allow 8-byte stores (ldc % 4 == 0, y 8-byte aligned)
+    int vector_store; // y (and z) rows allow 8-byte accesses (ldc, ldz % 4 == 0, 8-byte aligned)
+    const unsigned short *z; // what beta multiplies: z[token * ldz + feature] (y and ldc by default)
+    int ldz;
 };
 
 // XOR applied to the 16-byte chunk index inside an LDS row. With CH chunks per row the pattern
@@ -226,9 +228,10 @@ __global__ __launch_bounds__(WN *WM * 64) void bgemm_tn_kernel(TnParams p)
                     continue;
                 }
                 unsigned short *out = p.y + size_t(m) * p.ldc + n;
+                const unsigned short *source = p.z + size_t(m) * p.ldz + n;
                 if (n + 3 < p.n && p.vector_store) {
                     if (p.beta != 0.f) {
-                        u32x2_t old = *reinterpret_cast<const u32x2_t *>(out);
+                        u32x2_t old = *reinterpret_cast<const u32x2_t *>(source);
                         v[0] = fmaf(p.beta, __uint_as_float(old[0] << 16), p.alpha * v[0]);
                         v[1] = fmaf(p.beta, __uint_as_float(old[0] & 0xffff0000u), p.alpha * v[1]);
                         v[2] = fmaf(p.beta, __uint_as_float(old[1] << 16), p.alpha * v[2]);
@@ -247,7 +250,7 @@ __global__ __launch_bounds__(WN *WM * 64) void bgemm_tn_kernel(TnParams p)
                             break;
                         float value = p.alpha * v[e];
                         if (p.beta != 0.f)
-                            value = fmaf(p.beta, bf16_bits_to_float(out[e]), value);
+                            value = fmaf(p.beta, bf16_bits_to_float(source[e]), value);
                         out[e] = float_to_bf16_bits(value);
                     }
                 }
@@ -255,10 +258,11 @@ __global__ __launch_bounds__(WN *WM * 64) void bgemm_tn_kernel(TnParams p)
         }
 }
 
-// Ordered split-K reduction: y = alpha * (p_0 + p_1 + ...) + beta * y, partials added in index
+// Ordered split-K reduction: y = alpha * (p_0 + p_1 + ...) + beta * z, partials added in index
 // order so the result does not depend on scheduling.
 __global__ void splitk_reduce_kernel(int m, int n, int splits, float alpha, float beta,
-                                     const float *partials, unsigned short *y, int ldc)
+                                     const float *partials, unsigned short *y, int ldc,
+                                     const unsigned short *z, int ldz)
 {
     size_t index = size_t(blockIdx.x) * blockDim.x + threadIdx.x;
     size_t count = size_t(m) * n;
@@ -270,7 +274,7 @@ __global__ void splitk_reduce_kernel(int m, int n, int splits, float alpha, floa
     unsigned short *out = y + (index / n) * size_t(ldc) + index % n;
     float value = alpha * sum;
     if (beta != 0.f)
-        value = fmaf(beta, bf16_bits_to_float(*out), value);
+        value = fmaf(beta, bf16_bits_to_float(z[(index / n) * size_t(ldz) + index % n]), value);
     *out = float_to_bf16_bits(value);
 }
 
@@ -301,7 +305,7 @@ const TnVariant &tn_variant(int index) { return variants[index]; }
 
 hipError_t launch_bgemm_tn(hipStream_t stream, int variant, int split_k, int n_out, int m_rows,
                            int k, float alpha, const void *w, int lda, const void *x, int ldb,
-                           float beta, void *y, int ldc, float *partials)
+                           float beta, void *y, int ldc, float *partials, const BetaSource &source)
 {
     if (variant < 0 || variant >= tn_variant_count() || split_k < 1 || split_k > 65535)
         return hipErrorInvalidValue;
@@ -325,7 +329,10 @@ hipError_t launch_bgemm_tn(hipStream_t stream, int variant, int split_k, int n_o
     int tiles_per_split = (k_tiles + split_k - 1) / split_k;
     split_k = (k_tiles + tiles_per_split - 1) / tiles_per_split; // no empty partitions
     p.k_per_split = tiles_per_split * v.block_k;
-    p.vector_store = (ldc % 4 == 0) && (reinterpret_cast<uintptr_t>(y) % 8 == 0);
+    p.z = source.z ? static_cast<const unsigned short *>(source.z) : p.y;
+    p.ldz = source.z ? source.ldz : ldc;
+    p.vector_store = ldc % 4 == 0 && reinterpret_cast<uintptr_t>(y) % 8 == 0 && p.ldz % 4 == 0 &&
+                     reinterpret_cast<uintptr_t>(p.z) % 8 == 0;
     if (split_k > 1 && !partials)
         return hipErrorInvalidValue;
     if (size_t(p.tiles_n) * size_t(p.tiles_m) > 0x7fffffffu)
@@ -345,7 +352,7 @@ hipError_t launch_bgemm_tn(hipStream_t stream, int variant, int split_k, int n_o
         return status;
     size_t count = size_t(m_rows) * n_out;
     splitk_reduce_kernel<<<unsigned((count + 255) / 256), 256, 0, stream>>>(
-        m_rows, n_out, split_k, alpha, beta, partials, static_cast<unsigned short *>(y), ldc);
+        m_rows, n_out, split_k, alpha, beta, partials, static_cast<unsigned short *>(y), ldc, p.z, p.ldz);
     return launch_status();
 }
 } // namespace camblas_hip

@@ -26,10 +26,11 @@ struct StreamParams {
     const unsigned short *w2; // gated form: the "up" weights (w holds the "gate" weights)
     const unsigned short *x;
     unsigned short *y;
-    int lda, ldb, ldc;
+    const unsigned short *z; // what beta multiplies: z[token * ldz + feature] (y and ldc by default)
+    int lda, ldb, ldc, ldz;
     int n, m, k;
     float alpha, beta;
-    int vector_store;
+    int vector_store; // 8-byte accesses to y (and z) rows are aligned
 };
 
 constexpr int WAVES = 4, DEPTH = 2;
@@ -229,9 +230,10 @@ __global__ __launch_bounds__(WAVES * 64) void bgemv_stream_kernel(StreamParams p
             }
             continue;
         }
+        const unsigned short *source = p.z + size_t(m) * p.ldz + n;
         if (n + 3 < p.n && p.vector_store) {
             if (p.beta != 0.f) {
-                u32x2_t old = *reinterpret_cast<const u32x2_t *>(out);
+                u32x2_t old = *reinterpret_cast<const u32x2_t *>(source);
                 v[0] = fmaf(p.beta, __uint_as_float(old[0] << 16), p.alpha * v[0]);
                 v[1] = fmaf(p.beta, __uint_as_float(old[0] & 0xffff0000u), p.alpha * v[1]);
                 v[2] = fmaf(p.beta, __uint_as_float(old[1] << 16), p.alpha * v[2]);
@@ -250,7 +252,7 @@ __global__ __launch_bounds__(WAVES * 64) void bgemv_stream_kernel(StreamParams p
                     break;
                 float value = p.alpha * v[e];
                 if (p.beta != 0.f)
-                    value = fmaf(p.beta, bf16_bits_to_float(out[e]), value);
+                    value = fmaf(p.beta, bf16_bits_to_float(source[e]), value);
                 out[e] = float_to_bf16_bits(value);
             }
         }
@@ -322,6 +324,8 @@ hipError_t launch_gated_stream(hipStream_t stream, int pair_tiles, int token_til
     p.lda = lda;
     p.ldb = ldb;
     p.ldc = ldc;
+    p.z = p.y;
+    p.ldz = ldc;
     p.n = n_out;
     p.m = m_rows;
     p.k = k;
@@ -349,7 +353,8 @@ hipError_t launch_gated_stream(hipStream_t stream, int pair_tiles, int token_til
 
 hipError_t launch_bgemv_stream(hipStream_t stream, int depth_log2, int row_tiles, int token_tiles, int n_out,
                                int m_rows, int k, float alpha, const void *w, int lda,
-                               const void *x, int ldb, float beta, void *y, int ldc)
+                               const void *x, int ldb, float beta, void *y, int ldc,
+                               const BetaSource &source)
 {
     StreamParams p;
     p.w = static_cast<const unsigned short *>(w);
@@ -359,12 +364,15 @@ hipError_t launch_bgemv_stream(hipStream_t stream, int depth_log2, int row_tiles
     p.lda = lda;
     p.ldb = ldb;
     p.ldc = ldc;
+    p.z = source.z ? static_cast<const unsigned short *>(source.z) : p.y;
+    p.ldz = source.z ? source.ldz : ldc;
     p.n = n_out;
     p.m = m_rows;
     p.k = k;
     p.alpha = alpha;
     p.beta = beta;
-    p.vector_store = (ldc % 4 == 0) && (reinterpret_cast<uintptr_t>(y) % 8 == 0);
+    p.vector_store = ldc % 4 == 0 && reinterpret_cast<uintptr_t>(y) % 8 == 0 && p.ldz % 4 == 0 &&
+                     reinterpret_cast<uintptr_t>(p.z) % 8 == 0;
     if ((m_rows + token_tiles * 16 - 1) / (token_tiles * 16) > 65535)
         return hipErrorInvalidValue;
     switch (depth_log2) {

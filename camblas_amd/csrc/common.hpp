@@ -106,6 +106,8 @@ const TnVariant &fp8_variant(int index);
 // ---------------------------------------------------------------- launchers (each returns a hipError_t)
 hipError_t launch_scale_f32(hipStream_t stream, int m, int n, float beta, float *c, int ldc);
 hipError_t launch_scale_bf16(hipStream_t stream, int m, int n, float beta, void *c, int ldc);
+// c[i + j*ldc] = z[i + j*ldz] for BF16 storage; ldz == 0 repeats one column of m values
+hipError_t launch_spread_bf16(hipStream_t stream, int m, int n, const void *z, int ldz, void *c, int ldc);
 hipError_t launch_scale_f64(hipStream_t stream, int m, int n, double beta, double *c, int ldc);
 hipError_t launch_generic_f32(hipStream_t stream, bool ta, bool tb, int m, int n, int k, float alpha,
                               const float *a, int lda, const float *b, int ldb, float beta, float *c,
@@ -146,22 +148,30 @@ hipError_t launch_bgemm_any(hipStream_t stream, bool wide, bool ta, bool tb, int
                             void *c, int ldc);
 hipError_t launch_gemv_f32(hipStream_t stream, int rows, int inner, float alpha, const float *w,
                            int ld, const float *x, float beta, float *y);
-// y[M,N] (ldc) = alpha * x[M,K] (ldb) * W[N,K]^T (lda) + beta * y, BF16 storage.
+// Where the beta term of a BF16 linear is read from: by default the output itself; otherwise
+// z[token * ldz + feature] with ldz == 0 for one row broadcast over the tokens (a bias vector).
+// z must not overlap the output.
+struct BetaSource {
+    const void *z = nullptr;
+    int ldz = 0;
+};
+// y[M,N] (ldc) = alpha * x[M,K] (ldb) * W[N,K]^T (lda) + beta * (source or y), BF16 storage.
 // partials: FP32 [split_k, M, N] when split_k > 1.
 hipError_t launch_bgemm_tn(hipStream_t stream, int variant, int split_k, int n_out, int m_rows,
                            int k, float alpha, const void *w, int lda, const void *x, int ldb,
-                           float beta, void *y, int ldc, float *partials);
+                           float beta, void *y, int ldc, float *partials, const BetaSource &source = {});
 // Prefill BF16 linear with direct-to-LDS operand loads; variants are listed by dma_variant().
-// Needs k % 64 == 0, n_out % 4 == 0, ldc % 4 == 0, y 8-byte aligned.
+// Needs k % 64 == 0, n_out % 4 == 0, ldc % 4 == 0, y 8-byte aligned (and the same of a beta source).
 hipError_t launch_bgemm_dma(hipStream_t stream, int variant, int n_out, int m_rows, int k,
                             float alpha, const void *w, int lda, const void *x, int ldb, float beta,
-                            void *y, int ldc);
+                            void *y, int ldc, const BetaSource &source = {});
 // Decode-shaped BF16 linear: each workgroup streams 16*row_tiles weight rows over the whole K.
 // depth_log2: a K step is 2^depth_log2 blocks of 128 elements (0..3); row_tiles << depth_log2 <= 8
 // and (row_tiles + token_tiles) << depth_log2 <= 16 or the launch is refused.
 hipError_t launch_bgemv_stream(hipStream_t stream, int depth_log2, int row_tiles, int token_tiles, int n_out,
                                int m_rows, int k, float alpha, const void *w, int lda,
-                               const void *x, int ldb, float beta, void *y, int ldc);
+                               const void *x, int ldb, float beta, void *y, int ldc,
+                               const BetaSource &source = {});
 // The gated-MLP front end for decode batches in one pass over both weight matrices:
 // y = round(round(silu(g)) * u), g = round(x gate^T), u = round(x up^T). pair_tiles 1..4 (16 output
 // rows each: that many gate rows and the same up rows per workgroup), token_tiles 1, 2 or 4.
@@ -172,9 +182,12 @@ hipError_t launch_fp8_block(hipStream_t stream, int variant, int split_k, int ro
                             int inner, const void *a, const float *a_scale, const void *w,
                             const float *w_scale, void *out, float *partials);
 // Prefill FP8 block-scaled linear with direct-to-LDS loads; needs outputs % 4 == 0.
-hipError_t launch_fp8_dma(hipStream_t stream, int variant, int rows, int outputs, int inner,
+// split_k > 1: K groups divided over that many workgroups per tile, FP32 planes in `partials`
+// ([split_k, rows, outputs]) summed in index order.
+hipError_t launch_fp8_dma(hipStream_t stream, int variant, int split_k, int rows, int outputs, int inner,
                           const void *a, const float *a_scale, const void *w, const float *w_scale,
-                          void *out);
+                          void *out, float *partials);
+hipError_t launch_fp8_split_sum(hipStream_t stream, int splits, size_t count, const float *partials, void *out);
 // row_tiles 1..8 (16 weight rows each), token_tiles 1, 2 or 4 (16 tokens each).
 hipError_t launch_fp8_stream(hipStream_t stream, int row_tiles, int token_tiles, int rows, int outputs,
                              int inner, const void *a, const float *a_scale, const void *w,

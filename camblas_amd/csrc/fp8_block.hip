@@ -378,9 +378,14 @@ hipError_t launch_fp8_block(hipStream_t stream, int variant, int split_k, int ro
     }
     if (status != hipSuccess || split_k == 1)
         return status;
-    size_t count = size_t(rows) * outputs;
+    return launch_fp8_split_sum(stream, split_k, size_t(rows) * outputs, partials, out);
+}
+
+// out[i] = bf16(partials[0][i] + partials[1][i] + ...), planes of `count` FP32 sums in index order
+hipError_t launch_fp8_split_sum(hipStream_t stream, int splits, size_t count, const float *partials, void *out)
+{
     fp8_splitk_reduce_kernel<<<unsigned((count + 255) / 256), 256, 0, stream>>>(
-        count, split_k, partials, static_cast<unsigned short *>(out));
+        count, splits, partials, static_cast<unsigned short *>(out));
     return launch_status();
 }
 

@@ -30,14 +30,17 @@ struct Fp8DmaParams {
     const float *w_scale;
     const float *a_scale;
     unsigned short *out;
+    float *partials; // FP32 [splits, m, n] when the K groups are divided over blockIdx.y, else null
     int n, m, k, groups, scale_blocks;
     int tiles_n, tiles_m;
+    int split_groups; // K groups per blockIdx.y (all of them without a split)
 };
 
 template <int TM, int WM, int STAGES, int TN>
 __global__ __launch_bounds__(128 * WM) void fp8_dma_kernel(Fp8DmaParams p)
 {
-    // (a fourth stage was measured: no gain, the kernel is not limited by bytes in flight)
+    // (a fourth and a fifth stage were measured, with few and with many tokens: no gain, the kernel
+    // is not limited by bytes in flight)
     static_assert(STAGES == 2 || STAGES == 3, "two or three LDS stages");
     constexpr int WAVES = 2 * WM, CH = 8, BK = 128;
     // weight scales per wavefront and group: one when its rows are one scale block, else one per
@@ -71,8 +74,11 @@ __global__ __launch_bounds__(128 * WM) void fp8_dma_kernel(Fp8DmaParams p)
         make_resource(p.w + size_t(n0) * p.k, unsigned(a_rows) * unsigned(p.k));
     const __amdgpu_buffer_rsrc_t b_resource =
         make_resource(p.a + size_t(m0) * p.k, unsigned(b_rows) * unsigned(p.k));
-    const unsigned last_k_bytes = unsigned(p.groups - 1) * BK;
-    unsigned k_bytes = 0;
+    // this workgroup's share of the K groups: [first_group, first_group + group_count)
+    const int first_group = int(blockIdx.y) * p.split_groups;
+    const int group_count = p.groups - first_group < p.split_groups ? p.groups - first_group : p.split_groups;
+    const unsigned last_k_bytes = unsigned(first_group + group_count - 1) * BK;
+    unsigned k_bytes = unsigned(first_group) * BK;
     // Load number `index` (0 .. LOADS-1) of the group at k_bytes; advance() moves to the next group.
     auto issue_one = [&](u32x4_t *stage, int index) {
         if (index < A_ITERS)
@@ -101,14 +107,14 @@ __global__ __launch_bounds__(128 * WM) void fp8_dma_kernel(Fp8DmaParams p)
     for (int s = 0; s < WS; ++s) {
         int block = (n0 + wn * TN * 32 + s * 32) / 128;
         block = block < p.scale_blocks ? block : p.scale_blocks - 1;
-        ws_row[s] = p.w_scale + size_t(block) * p.groups;
+        ws_row[s] = p.w_scale + size_t(block) * p.groups + first_group;
     }
     const float *as_ptr[TM];
 #pragma unroll
     for (int j = 0; j < TM; ++j) {
         int m = m0 + (wm * TM + j) * 32 + frag_row;
         m = m < p.m ? m : p.m - 1;
-        as_ptr[j] = p.a_scale + size_t(m) * p.groups;
+        as_ptr[j] = p.a_scale + size_t(m) * p.groups + first_group;
     }
 
     const int frag_swizzle = lds_swizzle<CH>(frag_row);
@@ -204,7 +210,7 @@ __global__ __launch_bounds__(128 * WM) void fp8_dma_kernel(Fp8DmaParams p)
     // One group: start the loads of the group STAGES-1 ahead into the stage that was read last,
     // multiply the current stage, then wait until only the newest loads are still in flight.
     auto step = [&](int g, const u32x4_t *current, u32x4_t *fill) {
-        const int next = g + 1 < p.groups ? g + 1 : p.groups - 1;
+        const int next = g + 1 < group_count ? g + 1 : group_count - 1;
 #pragma unroll
         for (int s = 0; s < WS; ++s)
             ws_next[s] = ws_row[s][next];
@@ -231,18 +237,36 @@ __global__ __launch_bounds__(128 * WM) void fp8_dma_kernel(Fp8DmaParams p)
     pipeline_barrier<(STAGES - 2) * LOADS>();
     // whole rounds of STAGES groups run without a branch between the steps; the remainder follows
     int g = 0;
-    for (; g + STAGES <= p.groups; g += STAGES) {
+    for (; g + STAGES <= group_count; g += STAGES) {
 #pragma unroll
         for (int s = 0; s < STAGES; ++s)
             step(g + s, stages[s], stages[(s + STAGES - 1) % STAGES]);
     }
 #pragma unroll
     for (int s = 0; s + 1 < STAGES; ++s)
-        if (g + s < p.groups)
+        if (g + s < group_count)
             step(g + s, stages[s], stages[(s + STAGES - 1) % STAGES]);
     wait_loads<0>();
 
     // ---- epilogue: accumulator register 4q+e of lane l is feature 8q + 4*(l/32) + e, token l%32
+    if (p.partials) { // a share of the K groups: FP32 sums for the ordered reduction
+        float *plane = p.partials + size_t(blockIdx.y) * size_t(p.m) * size_t(p.n);
+#pragma unroll
+        for (int j = 0; j < TM; ++j) {
+            const int m = m0 + (wm * TM + j) * 32 + frag_row;
+            float *row = plane + size_t(m) * p.n + n0 + wn * TN * 32 + half * 4;
+#pragma unroll
+            for (int i = 0; i < TN; ++i)
+#pragma unroll
+                for (int q = 0; q < 4; ++q) {
+                    const int offset = i * 32 + q * 8;
+                    if (m < p.m && n0 + wn * TN * 32 + half * 4 + offset < p.n)
+                        *reinterpret_cast<f32x4_t *>(row + offset) = f32x4_t{
+                            acc[i][j][q * 4], acc[i][j][q * 4 + 1], acc[i][j][q * 4 + 2], acc[i][j][q * 4 + 3]};
+                }
+        }
+        return;
+    }
 #pragma unroll
     for (int j = 0; j < TM; ++j) {
         const int m = m0 + (wm * TM + j) * 32 + frag_row;
@@ -264,7 +288,7 @@ __global__ __launch_bounds__(128 * WM) void fp8_dma_kernel(Fp8DmaParams p)
 }
 
 template <int TM, int WM, int STAGES, int TN = 4>
-hipError_t launch_one(hipStream_t stream, Fp8DmaParams p)
+hipError_t launch_one(hipStream_t stream, Fp8DmaParams p, int splits)
 {
     constexpr int BN = 64 * TN, BM = 32 * WM * TM;
     p.tiles_n = (p.n + BN - 1) / BN;
@@ -272,7 +296,7 @@ hipError_t launch_one(hipStream_t stream, Fp8DmaParams p)
     if (size_t(p.tiles_n) * size_t(p.tiles_m) > 0x7fffffffu)
         return hipErrorInvalidValue;
     fp8_dma_kernel<TM, WM, STAGES, TN>
-        <<<unsigned(p.tiles_n) * unsigned(p.tiles_m), 128 * WM, 0, stream>>>(p);
+        <<<dim3(unsigned(p.tiles_n) * unsigned(p.tiles_m), unsigned(splits)), 128 * WM, 0, stream>>>(p);
     return launch_status();
 }
 
@@ -294,11 +318,18 @@ int fp8_dma_variant_count() { return int(sizeof(variants) / sizeof(variants[0]))
 const TnVariant &fp8_dma_variant(int index) { return variants[index]; }
 
 // Needs outputs % 4 == 0 (8-byte BF16 stores) and 16-byte aligned a, w (rows are multiples of 128).
-hipError_t launch_fp8_dma(hipStream_t stream, int variant, int rows, int outputs, int inner,
+// With split_k > 1 the K groups are divided evenly over that many workgroups per tile, each writes
+// an FP32 plane of `partials` ([split_k, rows, outputs], 16-byte aligned) and the planes are summed
+// in index order before the one BF16 rounding: few tokens leave most compute units without a tile
+// otherwise (256 tokens by 18432 outputs are 72 tiles of 256 x 256).
+hipError_t launch_fp8_dma(hipStream_t stream, int variant, int split_k, int rows, int outputs, int inner,
                           const void *a, const float *a_scale, const void *w, const float *w_scale,
-                          void *out)
+                          void *out, float *partials)
 {
     if (outputs % 4 || inner % 128 || reinterpret_cast<uintptr_t>(out) % 8)
+        return hipErrorInvalidValue;
+    if (split_k < 1 || split_k > 64 || split_k > inner / 128 || (split_k > 1 && !partials) ||
+        reinterpret_cast<uintptr_t>(partials) % 16)
         return hipErrorInvalidValue;
     if (size_t(256) * size_t(inner) >= (size_t(1) << 32))
         return hipErrorInvalidValue;
@@ -314,18 +345,26 @@ hipError_t launch_fp8_dma(hipStream_t stream, int variant, int rows, int outputs
     p.groups = inner / 128;
     p.scale_blocks = (outputs + 127) / 128;
     p.tiles_n = p.tiles_m = 0;
+    p.split_groups = (p.groups + split_k - 1) / split_k;
+    // every blockIdx.y must own at least one group
+    const int splits = (p.groups + p.split_groups - 1) / p.split_groups;
+    p.partials = splits > 1 ? partials : nullptr;
+    hipError_t status;
     switch (variant) {
-    case 0: return launch_one<2, 4, 2>(stream, p);
-    case 1: return launch_one<1, 4, 2>(stream, p);
-    case 2: return launch_one<2, 2, 2>(stream, p);
-    case 3: return launch_one<1, 2, 2>(stream, p);
-    case 4: return launch_one<1, 4, 3>(stream, p);
-    case 5: return launch_one<2, 2, 3>(stream, p);
-    case 6: return launch_one<1, 2, 3>(stream, p);
-    case 7: return launch_one<1, 4, 3, 3>(stream, p);
-    case 8: return launch_one<2, 4, 2, 3>(stream, p);
-    case 9: return launch_one<1, 2, 3, 3>(stream, p);
+    case 0: status = launch_one<2, 4, 2>(stream, p, splits); break;
+    case 1: status = launch_one<1, 4, 2>(stream, p, splits); break;
+    case 2: status = launch_one<2, 2, 2>(stream, p, splits); break;
+    case 3: status = launch_one<1, 2, 2>(stream, p, splits); break;
+    case 4: status = launch_one<1, 4, 3>(stream, p, splits); break;
+    case 5: status = launch_one<2, 2, 3>(stream, p, splits); break;
+    case 6: status = launch_one<1, 2, 3>(stream, p, splits); break;
+    case 7: status = launch_one<1, 4, 3, 3>(stream, p, splits); break;
+    case 8: status = launch_one<2, 4, 2, 3>(stream, p, splits); break;
+    case 9: status = launch_one<1, 2, 3, 3>(stream, p, splits); break;
     default: return hipErrorInvalidValue;
     }
+    if (status != hipSuccess || splits == 1)
+        return status;
+    return launch_fp8_split_sum(stream, splits, size_t(rows) * size_t(outputs), partials, out);
 }
 } // namespace camblas_hip

@@ -26,6 +26,15 @@ __global__ void scale_kernel(int m, int n, typename storage<T>::accumulator beta
     storage<T>::store(out, beta == acc_t(0) ? acc_t(0) : beta * storage<T>::load(out));
 }
 
+// c[i + j*ldc] = z[i + j*ldz], 2-byte elements; ldz == 0 repeats one column
+__global__ void spread_kernel(int m, int n, const unsigned short *z, int ldz, unsigned short *c, int ldc)
+{
+    size_t index = size_t(blockIdx.x) * blockDim.x + threadIdx.x;
+    if (index >= size_t(m) * n)
+        return;
+    c[index % m + (index / m) * size_t(ldc)] = z[index % m + (index / m) * size_t(ldz)];
+}
+
 // TA/TB: operand stored transposed. A tile element (i, l) is a[i + l*lda] (N) or a[l + i*lda] (T);
 // the thread->element map makes the memory-contiguous index the fastest-varying lane index.
 template <typename T, bool TA, bool TB>
@@ -148,6 +157,13 @@ hipError_t launch_scale_bf16(hipStream_t stream, int m, int n, float beta, void 
 {
     scale_kernel<bf16_storage><<<unsigned((size_t(m) * n + 255) / 256), 256, 0, stream>>>(
         m, n, beta, static_cast<bf16_storage *>(c), ldc);
+    return launch_status();
+}
+
+hipError_t launch_spread_bf16(hipStream_t stream, int m, int n, const void *z, int ldz, void *c, int ldc)
+{
+    spread_kernel<<<unsigned((size_t(m) * n + 255) / 256), 256, 0, stream>>>(
+        m, n, static_cast<const unsigned short *>(z), ldz, static_cast<unsigned short *>(c), ldc);
     return launch_status();
 }
 

@@ -442,6 +442,40 @@ Tensor &backend_mm_out(const Tensor &a, const Tensor &b, Tensor &out)
     return out;
 }
 
+// A BF16 bias the product's epilogue can read where it lies: one row for every output row ([n] or
+// [1, n]) or a full [rows, n] matrix, with unit stride along n. `pitch` is the row stride in
+// elements, 0 for the repeated row.
+struct Addend {
+    const void *data = nullptr;
+    int pitch = 0;
+};
+
+Addend epilogue_addend(const Tensor &bias, int64_t rows, int64_t columns)
+{
+    if (bias.scalar_type() != at::kBFloat16 || bias.dim() < 1 || bias.size(-1) != columns ||
+        (columns > 1 && bias.stride(-1) != 1))
+        return {};
+    if (bias.dim() == 1 || bias.size(0) == 1)
+        return {bias.const_data_ptr(), 0};
+    if (rows > 1 && bias.stride(0) < columns)
+        return {};
+    return {bias.const_data_ptr(), rows > 1 ? int(bias.stride(0)) : 0};
+}
+
+// out = alpha * a b + beta * addend into a fresh tensor, the addend read by the product itself
+Tensor bf16_product_adding(const Addend &addend, const Tensor &a, const Tensor &b, double alpha, double beta)
+{
+    const int rows = int(a.size(0)), inner = int(a.size(1)), columns = int(b.size(1));
+    Tensor result = at::empty({rows, columns}, a.options());
+    const AbiOperand first(b), second(a);
+    camblas_cuda_context *context = context_for(a.get_device(), backend_algorithm);
+    succeed(camblas_cuda_bgemm_add(context, first.flag, second.flag, columns, rows, inner, float(alpha), first.data(),
+                                   first.leading, second.data(), second.leading, float(beta), addend.data,
+                                   addend.pitch, result.mutable_data_ptr(), std::max(columns, 1)),
+            context);
+    return result;
+}
+
 Tensor backend_addmm(const Tensor &bias, const Tensor &a, const Tensor &b, const at::Scalar &beta,
                      const at::Scalar &alpha)
 {
@@ -452,6 +486,11 @@ Tensor backend_addmm(const Tensor &bias, const Tensor &a, const Tensor &b, const
     c10::DeviceGuard guard(a.device());
     const double keep = beta.toDouble();
     const std::vector<int64_t> shape = {a.size(0), b.size(1)};
+    if (keep != 0 && a.numel() > 0 && b.numel() > 0) {
+        const Addend addend = epilogue_addend(bias, shape[0], shape[1]);
+        if (addend.data)
+            return bf16_product_adding(addend, a, b, alpha.toDouble(), keep);
+    }
     // beta == 0 never reads the bias (NaN-safe); otherwise the product accumulates onto a copy of it
     Tensor out = keep == 0 ? at::empty(shape, a.options()) : bias.expand(shape).clone(at::MemoryFormat::Contiguous);
     return matmul(a, b, out, alpha.toDouble(), keep, backend_algorithm, false);

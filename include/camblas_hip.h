@@ -81,6 +81,17 @@ int camblas_cuda_bgemm(camblas_cuda_context *context, char trans_a, char trans_b
                        int k, float alpha, const void *a, int lda, const void *b, int ldb,
                        float beta, void *c, int ldc);
 
+/* C = alpha op(A) op(B) + beta Z with the addend Z stored apart from C: an m x n column-major matrix
+ * with leading dimension ldz >= m, or, with ldz == 0, one column of m values added to every column
+ * of the product (the bias row of a linear layer as the 'T','N' mapping above sees it). Z is never
+ * read when beta == 0 and may not overlap C; everything else as camblas_cuda_bgemm. No counterpart
+ * in the reference header: its aten::addmm first copies the broadcast bias into the output and then
+ * runs the beta form (ref: src/cuda/torch_backend.cuh:60-88), which costs one write and one read
+ * of the whole output. */
+int camblas_cuda_bgemm_add(camblas_cuda_context *context, char trans_a, char trans_b, int m, int n,
+                           int k, float alpha, const void *a, int lda, const void *b, int ldb,
+                           float beta, const void *z, int ldz, void *c, int ldc);
+
 /* Same contract in FP64 (ref: include/camblas_cuda.h:60-62, src/cuda/backend.cu:1066-1073):
  * FP64 matrix-core tiles for every layout (IEEE double multiply-add); products with m or n below
  * 16 run an LDS-tiled FMA kernel. */

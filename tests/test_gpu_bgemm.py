@@ -274,6 +274,23 @@ def test_addmm_beta_one_and_errors(device):
     assert status == -1 and b"leading dimension" in lib.camblas_cuda_error(native.handle)
 
 
+@pytest.mark.parametrize("form", ["row", "row matrix", "pitched", "column", "fp32"])
+def test_addmm_bias_forms(device, form):
+    tokens, outputs, inner = 40, 264, 320
+    x = oracle.fill_normal_bf16(92, (tokens, inner))
+    w = oracle.fill_normal_bf16(93, (outputs, inner), std=0.05)
+    wide = to_device_bf16(oracle.fill_normal_bf16(94, (tokens, 2 * outputs)), device)
+    xt, wt = to_device_bf16(x, device), to_device_bf16(w, device)
+    if form == "fp32":  # FP32 operands never take the BF16 epilogue route
+        xt, wt, wide = xt.float(), wt.float(), wide.float()
+    bias = {"row": wide[0, :outputs], "row matrix": wide[1:2, :outputs], "pitched": wide[:, outputs:],
+            "column": wide[:, :1], "fp32": wide[0, :outputs]}[form]
+    y = _kernels.addmm(bias, xt, wt.t(), beta=-0.5, alpha=1.25)
+    torch.cuda.synchronize()
+    want = 1.25 * oracle.linear_bf16_f64(x, w) - 0.5 * bias.double().cpu().numpy()
+    assert rel_frobenius(y.double().cpu().numpy(), want) <= (1e-5 if form == "fp32" else TOLERANCE)
+
+
 def test_long_k_llama_dims(device):
     # down-projection depth (ref: tests/test_bfloat16.py:207-217): K = 28672
     tokens, outputs, inner = 32, 512, 28672
@@ -281,3 +298,94 @@ def test_long_k_llama_dims(device):
     w = oracle.fill_normal_bf16(92, (outputs, inner), std=0.02)
     y = _kernels.linear(to_device_bf16(x, device), to_device_bf16(w, device))
     assert rel_frobenius(bf16_values(y), oracle.linear_bf16_f64(x, w)) <= TOLERANCE
+
+
+def run_bgemm_add(device, ta, tb, m, n, k, alpha, a, lda, b, ldb, beta, z, ldz, c, ldc, override=None,
+                  z_offset=0):
+    at, bt, ct_ = (to_device_bf16(v, device) for v in (a, b, c))
+    zt = to_device_bf16(np.concatenate([np.zeros(z_offset, dtype=np.uint16), z]), device)
+    native = _native.context(device)
+    if override is not None:
+        native.call("hip_set_plan_override", override[0], override[1])
+    try:
+        native.call("bgemm_add", ta.encode(), tb.encode(), m, n, k, ct.c_float(alpha), ptr(at), lda, ptr(bt), ldb,
+                    ct.c_float(beta), ct.c_void_p(zt.data_ptr() + 2 * z_offset), ldz, ptr(ct_), ldc)
+    finally:
+        native.call("hip_set_plan_override", -1, 0)
+    torch.cuda.synchronize()
+    return from_device_bf16(ct_)
+
+
+def spread(z, ldz, m, n, c, ldc):
+    """The addend laid over a copy of C: what the reference's addmm does before its beta product."""
+    start = c.copy()
+    for j in range(n):
+        start[j * ldc:j * ldc + m] = z[j * ldz:j * ldz + m]
+    return start
+
+
+@pytest.mark.parametrize("ta,tb,m,n,k,override", [
+    ("T", "N", 300, 70, 328, (3, 1)),      # register-staged tiles
+    ("T", "N", 300, 70, 328, (1, 3)),      # ... with a split K and the ordered reduction
+    ("T", "N", 301, 9, 328, (121, 1)),     # streaming kernel, scalar stores
+    ("T", "N", 512, 256, 320, (21, 1)),    # direct-to-LDS tiles
+    ("T", "N", 1024, 40, 512, None),       # the planner's choice for a decode batch
+    ("N", "N", 200, 150, 72, None),        # any-layout matrix-core kernel: addend spread first
+    ("N", "T", 9, 7, 5, None),             # generic kernel: addend spread first
+])
+@pytest.mark.parametrize("ldz_kind", ["row", "matrix"])
+def test_addend_apart_from_the_output(device, ta, tb, m, n, k, override, ldz_kind):
+    # C = alpha A B + beta Z equals, bit for bit, the beta form run on a C that holds Z: the same
+    # kernel computes both, only the address its epilogue reads differs. And both hold the FP64 bar.
+    rng = np.random.default_rng(m + n + k)
+    lda = (k if ta == "T" else m) + 8
+    ldb = (n if tb == "T" else k) + 8
+    ldc = m + 4
+    a = oracle.fill_normal_bf16(41, (lda * (m if ta == "T" else k),))
+    b = oracle.fill_normal_bf16(42, (ldb * (k if tb == "T" else n),))
+    c = oracle.fill_normal_bf16(43, (ldc * n,))
+    ldz = 0 if ldz_kind == "row" else m + 12
+    z = oracle.fill_normal_bf16(44, (max(ldz, m) * n,))
+    alpha, beta = 0.75, -1.5
+    got = run_bgemm_add(device, ta, tb, m, n, k, alpha, a, lda, b, ldb, beta, z, ldz, c, ldc, override)
+    start = spread(z, ldz, m, n, c, ldc)
+    composed = run_bgemm(device, ta, tb, m, n, k, alpha, a, lda, b, ldb, beta, start, ldc, override)
+    assert np.array_equal(got, composed)
+    want, want64 = reference(ta, tb, m, n, k, alpha, a, lda, b, ldb, beta, start, ldc)
+    got2d = got.reshape(n, ldc)
+    assert rel_frobenius(oracle.bf16_to_f32(got2d[:, :m]), want64.reshape(n, m)) <= TOLERANCE
+    assert np.array_equal(got2d[:, m:], c.reshape(n, ldc)[:, m:])  # the padding of C is left alone
+
+
+def test_addend_that_is_not_eight_byte_aligned(device):
+    # the direct-to-LDS family reads the addend eight bytes at a time; an odd element offset sends
+    # the product to the register-staged family, which must still give the FP64-bar answer
+    m, n, k = 512, 256, 320
+    a = oracle.fill_normal_bf16(51, (k * m,))
+    b = oracle.fill_normal_bf16(52, (k * n,))
+    z = oracle.fill_normal_bf16(53, (m,))
+    c = np.zeros(m * n, dtype=np.uint16)
+    got = run_bgemm_add(device, "T", "N", m, n, k, 1.0, a, k, b, k, 1.0, z, 0, c, m, z_offset=1)
+    want, want64 = reference("T", "N", m, n, k, 1.0, a, k, b, k, 1.0, spread(z, 0, m, n, c, m), m)
+    assert rel_frobenius(oracle.bf16_to_f32(got).reshape(n, m), want64.reshape(n, m)) <= TOLERANCE
+
+
+def test_addend_argument_checks(device):
+    native, lib = _native.context(device), _native.library()
+    m, n, k = 64, 8, 32
+    a = torch.zeros(m * k, dtype=torch.bfloat16, device=device)
+    b = torch.zeros(n * k, dtype=torch.bfloat16, device=device)
+    c = torch.ones(m * n + m, dtype=torch.bfloat16, device=device)
+    z = torch.full((m * n,), 2.0, dtype=torch.bfloat16, device=device)
+    call = lambda *args: lib.camblas_cuda_bgemm_add(native.handle, b"T", b"N", m, n, k, *args)
+    one = ct.c_float(1.0)
+    assert call(one, ptr(a), k, ptr(b), k, one, ptr(z), m - 1, ptr(c), m) == -1          # ldz below m
+    assert call(one, ptr(a), k, ptr(b), k, one, None, 0, ptr(c), m) == -1                # missing addend
+    assert call(one, ptr(a), k, ptr(b), k, one, ct.c_void_p(c.data_ptr() + 2 * m), m, ptr(c), m) == -1  # overlaps C
+    assert b"aliased" in lib.camblas_cuda_error(native.handle)
+    assert call(one, ptr(a), k, ptr(b), k, ct.c_float(0.0), None, 0, ptr(c), m) == 0     # beta 0: never read
+    torch.cuda.synchronize()
+    assert float(c[:m * n].float().abs().max()) == 0.0
+    assert call(ct.c_float(0.0), None, k, None, k, ct.c_float(0.5), ptr(z), 0, ptr(c), m) == 0  # only beta acts
+    torch.cuda.synchronize()
+    assert torch.equal(c[:m * n].float(), torch.ones(m * n, device=device))

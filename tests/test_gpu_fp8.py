@@ -93,7 +93,23 @@ def test_direct_lds_load_variants(device, code, rows, outputs, inner):
     assert (np.abs(bf16_values(out) - ordered) <= bound).all()
 
 
-@pytest.mark.parametrize("rows", [1, 16, 256])
+@pytest.mark.parametrize("code,split", [(20, 2), (24, 3), (27, 2), (29, 7), (26, 64)])
+@pytest.mark.parametrize("rows,outputs,inner", [(70, 300, 896), (129, 516, 1792)])
+def test_direct_lds_loads_with_divided_k_groups(device, code, split, rows, outputs, inner):
+    # the K groups of a tile shared by several workgroups (uneven shares, more shares asked for than
+    # groups exist) and summed in share order: the FMA chain is cut into `split` chains, so the
+    # FP64 bar applies and the ordered oracle holds to one BF16 unit plus the FP32 re-association
+    a, a_scale = oracle.fill_fp8_blocks(720 + rows, rows, inner, 1)
+    w, w_scale = oracle.fill_fp8_blocks(721, outputs, inner, 128)
+    out = run(device, a, a_scale, w, w_scale, override=(code, split))
+    want64 = oracle.fp8_block_matmul_f64(a, a_scale, w, w_scale)
+    assert rel_frobenius(bf16_values(out), want64) <= TOLERANCE
+    wanted = oracle.bf16_to_f32(oracle.f32_to_bf16(want64.astype(np.float32)))
+    bound = 2.0**-7 * np.abs(wanted) + 1e-4 * np.abs(want64).max()
+    assert (np.abs(bf16_values(out) - wanted) <= bound).all()
+
+
+@pytest.mark.parametrize("rows", [1, 16, 96, 256])
 def test_planned_shapes(device, rows):
     outputs, inner = 1536, 1024
     a, a_scale = oracle.fill_fp8_blocks(300 + rows, rows, inner, 1)
@@ -103,7 +119,7 @@ def test_planned_shapes(device, rows):
 
 
 @pytest.mark.parametrize("override", [None, (0, 1), (1, 1), (2, 1), (3, 1), (20, 1), (21, 1), (22, 1), (23, 1), (24, 1), (25, 1), (26, 1),
-                                      (111, 1), (152, 1), (134, 1)])
+                                      (24, 3), (28, 4), (111, 1), (152, 1), (134, 1)])
 def test_scale_indexing_is_bit_exact(device, override):
     # every product is a small integer and every scale a distinct power of two, so the FMA chain
     # is exact: any wrong (row, group) or (block, group) scale index changes the bits

@@ -263,6 +263,19 @@ def test_backend_override_routes_and_falls_back(binding, device):
     assert error(got, a.double().view(4, 16, 256) @ w.double().t() + bias.double()) <= 1e-2
     got, count = dispatched(lambda: a @ w.t())
     assert count == 1 and error(got, a.double() @ w.double().t()) <= 1e-2
+    # BF16 addmm for every way a bias broadcasts: rows and full matrices with unit stride along the
+    # output features are read by the product itself, the other forms are spread over the output
+    # first; either way one product is counted and alpha * a b + beta * bias is rounded once
+    product = a.double() @ w.double().t()
+    wide = randn((64, 96), torch.bfloat16, device, 27)
+    forms = {"row": bias, "row matrix": bias.view(1, 48), "full": wide[:, :48].contiguous(), "pitched": wide[:, 48:],
+             "column": wide[:, :1], "scalar": wide[0, 0], "strided": wide.t()[:48, :1].t().expand(64, 48)}
+    for name, form in forms.items():
+        got, count = dispatched(lambda: torch.addmm(form, a, w.t(), beta=0.5, alpha=2.0))
+        assert count == 1, name
+        want = 2.0 * product + 0.5 * form.double()
+        assert error(got, want) <= 1e-2, name
+        assert (got.float() - want.float()).abs().max() <= 2.0**-7 * want.abs().max(), name
     previous = torch.backends.cuda.matmul.allow_tf32
     try:
         torch.backends.cuda.matmul.allow_tf32 = False
