@@ -8,18 +8,28 @@ camblas_cuda_bgemm('T','N') on resident operands. Three weight copies (3 x 470 M
 algorithmic HBM traffic of the timed steps divided by wall time (host clock around K steps with a
 device synchronisation on both sides).
 
+When the K timed steps last less than 200 ms the same loop is timed once more over enough steps to
+fill 200 ms and both figures are reported (`config.long_run`).
+
 The line also carries
-  roofline      the dominant kernel (M=32 launch) timed with HIP events on the launch stream,
-  cpu_baseline  the CPU oracle port of the same BF16 linear on a bounded sample of weight rows,
+  roofline      the dominant kernel (M=32 launch) timed with HIP events on the launch stream; its
+                `traffic` is measured live: two child runs of this file under `rocprofv3 --pmc`
+                (FETCH_SIZE, then WRITE_SIZE), each holding a plain copy of known size to scale by,
+  cpu_baseline  PyTorch's own CPU BF16 F.linear on the same shape, all host threads of this process,
   also          the other configurations (BF16 prefill linear and addmm, FP8 block-scaled linear,
-                FP32 SGEMM, decoder-layer decode step), each with its own roofline fraction, and
-                the reference's own CPU SGEMM when oracle/_ref is present.
+                E8M0 products, FP32 SGEMM, decode attention, decoder-layer decode step), each with
+                a `roofline` object of its own; PyTorch's CPU FP8 dequantise-then-mm; the CPU
+                oracle port; the reference's own CPU SGEMM when oracle/_ref is present.
 """
 
 import argparse
+import csv
 import json
 import os
+import shutil
+import subprocess
 import sys
+import tempfile
 import time
 from pathlib import Path
 
@@ -30,6 +40,20 @@ HBM_PEAK = 8.0e12
 BF16_PEAK = 2.5e15
 FP8_PEAK = 5.0e15
 FP32_PEAK = 157.3e12
+FP64_PEAK = 78.6e12
+PEAKS = {"hbm": (HBM_PEAK, 1e9, "GB/s"), "mfma bf16": (BF16_PEAK, 1e12, "TFLOP/s"),
+         "mfma fp8": (FP8_PEAK, 1e12, "TFLOP/s"), "mfma fp32": (FP32_PEAK, 1e12, "TFLOP/s"),
+         "mfma fp64": (FP64_PEAK, 1e12, "TFLOP/s")}
+LONG_REGION = 0.2  # seconds of wall clock the headline loop should fill
+
+
+def roofline_of(bound, amount, seconds):
+    """The roofline object of one configuration: `amount` algorithmic bytes (bound "hbm") or flops
+    (bound "mfma <type>") per launch over the launch time measured with events."""
+    peak, unit_scale, unit = PEAKS[bound]
+    return {"bound": bound.split()[0], "algorithmic": int(amount), "achieved": round(amount / seconds / unit_scale, 1),
+            "peak": peak / unit_scale, "unit": unit, "frac": round(amount / seconds / peak, 4),
+            "launch_us": round(seconds * 1e6, 2)}
 
 OUTPUTS, INNER = 28672, 8192
 BATCHES = (1, 8, 32)
@@ -54,7 +78,75 @@ def event_time(torch, launch, warmup, iterations):
     return start.elapsed_time(stop) * 1e-3 / iterations
 
 
-def cpu_port_baseline(budget_seconds=12.0):
+def host_threads():
+    return len(os.sched_getaffinity(0))
+
+
+def cpu_torch_linear(budget_seconds=10.0):
+    """PyTorch's CPU BF16 F.linear on the headline shape (M = 32, W [28672, 8192]) with every host
+    thread this process may use: what a user without the GPU library would run."""
+    import torch
+    import torch.nn.functional as F
+
+    torch.set_num_threads(host_threads())
+    tokens = 32
+    generator = torch.Generator().manual_seed(7)
+    w = (torch.randn((OUTPUTS, INNER), generator=generator) * 0.02).to(torch.bfloat16)
+    x = torch.randn((tokens, INNER), generator=generator).to(torch.bfloat16)
+    F.linear(x, w)
+    elapsed, passes = 0.0, 0
+    while elapsed < budget_seconds and passes < 1000:
+        begin = time.perf_counter()
+        F.linear(x, w)
+        elapsed += time.perf_counter() - begin
+        passes += 1
+    return {
+        "value": round(passes * decode_bytes(tokens) / elapsed / 1e9, 3),
+        "unit": "GB/s",
+        "cores": host_threads(),
+        "kind": "torch-cpu",
+        "sample": f"torch.nn.functional.linear, BF16, x [32, {INNER}] W [{OUTPUTS}, {INNER}] (the whole M=32 "
+                  f"launch), torch.set_num_threads({host_threads()}), {passes} passes in {elapsed:.1f} s",
+    }
+
+
+def cpu_torch_fp8(budget_seconds=8.0):
+    """PyTorch's CPU route for the FP8 block-scaled linear at 16 tokens: dequantise both operands
+    to FP32 with their block scales, then mm: the plain PyTorch formulation of the same product."""
+    import torch
+
+    torch.set_num_threads(host_threads())
+    tokens, outputs, inner = 16, 18432, 7168
+    generator = torch.Generator().manual_seed(8)
+    w = torch.randint(0, 0x7E, (outputs, inner), generator=generator, dtype=torch.uint8).view(torch.float8_e4m3fn)
+    a = torch.randint(0, 0x7E, (tokens, inner), generator=generator, dtype=torch.uint8).view(torch.float8_e4m3fn)
+    w_scale = torch.rand((outputs // 128, inner // 128), generator=generator) * 0.1 + 1e-4
+    a_scale = torch.rand((tokens, inner // 128), generator=generator) * 0.1 + 1e-4
+
+    def once():
+        wide = w.to(torch.float32).view(outputs // 128, 128, inner // 128, 128) * w_scale[:, None, :, None]
+        rows = a.to(torch.float32).view(tokens, inner // 128, 128) * a_scale[:, :, None]
+        return (rows.view(tokens, inner) @ wide.view(outputs, inner).t()).to(torch.bfloat16)
+
+    once()
+    elapsed, passes = 0.0, 0
+    while elapsed < budget_seconds and passes < 1000:
+        begin = time.perf_counter()
+        once()
+        elapsed += time.perf_counter() - begin
+        passes += 1
+    traffic = outputs * inner + w_scale.numel() * 4 + tokens * (inner + inner // 128 * 4 + outputs * 2)
+    return {
+        "value": round(passes * traffic / elapsed / 1e9, 3),
+        "unit": "GB/s",
+        "cores": host_threads(),
+        "kind": "torch-cpu",
+        "sample": f"E4M3 -> FP32 dequantise with the 1x128 / 128x128 scales, then torch.mm, 16 tokens x "
+                  f"[{outputs}, {inner}], torch.set_num_threads({host_threads()}), {passes} passes in {elapsed:.1f} s",
+    }
+
+
+def cpu_port_baseline(budget_seconds=6.0):
     """Time the CPU oracle's BF16 linear (FP64 accumulate, OpenMP) on a bounded sample of rows."""
     import oracle
 
@@ -108,13 +200,14 @@ def cpu_reference_sgemm():
 def main():
     parser = argparse.ArgumentParser()
     parser.add_argument("--gpus", type=int, default=1)
-    parser.add_argument("--steps", type=int, default=50)
-    parser.add_argument("--warmup", type=int, default=10)
+    parser.add_argument("--steps", type=int, default=1000)
+    parser.add_argument("--warmup", type=int, default=50)
     parser.add_argument("--skip-extras", action="store_true")
     parser.add_argument("--skip-cpu", action="store_true")
-    parser.add_argument("--only", choices=("decode1", "decode8", "decode32", "prefill", "copy", "fp8m1", "fp8m16",
-                                 "fp8m256", "fp8m4096", "mxe4m3m4096", "mxe2m1m4096", "fp8moe", "attention",
-                                 "layer"),
+    parser.add_argument("--skip-traffic", action="store_true", help="do not run the rocprofv3 counter passes")
+    parser.add_argument("--only", choices=("decode1", "decode8", "decode32", "prefill", "prefillnn", "copy", "traffic",
+                                 "fp8m1", "fp8m16", "fp8m256", "fp8m4096", "fp8block32", "mxe4m3m16", "mxe2m1m16",
+                                 "mxe4m3m4096", "mxe2m1m4096", "fp8moe", "attention", "layer", "sgemm2048"),
                         help="profiling aid: launch just this kernel --steps times, print nothing")
     args = parser.parse_args()
     if args.gpus != 1:
@@ -145,16 +238,25 @@ def main():
             weight = weights[(index * len(BATCHES) + position) % 3]
             _kernels.matmul(inputs[m], weight.t(), out=outputs[m])
 
+    def timed(steps):
+        torch.cuda.synchronize()
+        begin = time.perf_counter()
+        for index in range(steps):
+            step(index)
+        torch.cuda.synchronize()
+        return time.perf_counter() - begin
+
     for index in range(args.warmup):
         step(index)
-    torch.cuda.synchronize()
-    begin = time.perf_counter()
-    for index in range(args.steps):
-        step(index)
-    torch.cuda.synchronize()
-    elapsed = time.perf_counter() - begin
+    elapsed = timed(args.steps)
     step_bytes = sum(decode_bytes(m) for m in BATCHES)
     value = step_bytes * args.steps / elapsed / 1e9
+    long_run = None
+    if elapsed < LONG_REGION:  # too short a region for a wall clock: time a longer one as well
+        long_steps = int(LONG_REGION * 1.1 / (elapsed / max(args.steps, 1))) + 1
+        long_elapsed = timed(long_steps)
+        long_run = {"steps": long_steps, "ms": round(long_elapsed * 1e3, 2),
+                    "value": round(step_bytes * long_steps / long_elapsed / 1e9, 1)}
 
     # dominant kernel: the M=32 launch, timed alone with events on the launch stream
     per_launch = {}
@@ -172,7 +274,7 @@ def main():
         "peak": HBM_PEAK / 1e9,
         "unit": "GB/s",
         "frac": round(achieved / HBM_PEAK, 4),
-        "traffic": measured_traffic(),
+        "traffic": None,
         "launch_us": round(per_launch[32] * 1e6, 2),
     }
 
@@ -183,6 +285,10 @@ def main():
     }
     if not args.skip_extras:
         also.update(extras(torch, _kernels, _native, device, normal))
+    if not args.skip_traffic:  # after every timed launch of this process: the child runs leave the GPU idle
+        counters = measured_traffic()
+        roofline["traffic"] = counters.pop("traffic")
+        roofline["traffic_source"] = counters
     result = {
         "metric": "decode-GEMV HBM GB/s (BF16 linear W[28672,8192], M in {1,8,32}); TFLOP/s of the "
                   "BF16/FP8 prefill linears under 'also'",
@@ -203,15 +309,19 @@ def main():
                         "copies (HBM-cold)",
             "entry_point": "camblas_cuda_bgemm('T','N')",
             "peak_fraction": round(value * 1e9 / HBM_PEAK, 4),
+            "timed_region_ms": round(elapsed * 1e3, 2),
+            "long_run": long_run,
         },
         "roofline": roofline,
-        "cpu_baseline": None if args.skip_cpu else cpu_port_baseline(),
+        "cpu_baseline": None if args.skip_cpu else cpu_torch_linear(),
         "also": also,
     }
     if not args.skip_cpu:
+        also["cpu_torch_fp8_dequantise_mm_m16"] = cpu_torch_fp8()
+        also["cpu_oracle_port_bf16_linear"] = cpu_port_baseline()
         reference = cpu_reference_sgemm()
         if reference:
-            result["also"]["cpu_reference_sgemm_2048"] = reference
+            also["cpu_reference_sgemm_2048"] = reference
     print(json.dumps(result))
 
 
@@ -231,16 +341,51 @@ def probes():
     return probes.library
 
 
+def counter_pass(counter):
+    """One child run of this file under `rocprofv3 --pmc <counter>`: mean KiB per dispatch of the
+    copy probe and of the M = 32 decode kernel."""
+    tool = shutil.which("rocprofv3") or "/opt/rocm/bin/rocprofv3"
+    with tempfile.TemporaryDirectory(prefix="camblas_pmc_", dir="/tmp") as directory:
+        command = [tool, "--pmc", counter, "--output-format", "csv", "-d", directory, "-o", "t", "--",
+                   sys.executable, str(ROOT / "bench.py"), "--only", "traffic", "--steps", "6", "--warmup", "0"]
+        environment = dict(os.environ, TMPDIR="/tmp")
+        subprocess.run(command, cwd=directory, env=environment, stdout=subprocess.DEVNULL, stderr=subprocess.DEVNULL,
+                       timeout=180, check=True)
+        sums, counts = {"copy": 0.0, "decode": 0.0}, {"copy": 0, "decode": 0}
+        for path in Path(directory).rglob("*counter_collection.csv"):
+            with open(path, newline="") as handle:
+                for row in csv.DictReader(handle):
+                    if row.get("Counter_Name") != counter:
+                        continue
+                    name = row.get("Kernel_Name", "")
+                    kind = "copy" if "copy_probe" in name else "decode" if "bgemv_stream" in name else None
+                    if kind:
+                        sums[kind] += float(row["Counter_Value"])
+                        counts[kind] += 1
+        if not counts["copy"] or not counts["decode"]:
+            raise RuntimeError("no counter rows for the copy probe or the decode kernel")
+        return sums["copy"] / counts["copy"], sums["decode"] / counts["decode"]
+
+
 def measured_traffic():
-    """HBM bytes per M=32 launch from the committed counter profile (FETCH_SIZE + WRITE_SIZE, each
-    scaled by the copy-probe calibration), or None when that profile has not been taken."""
-    path = ROOT / "profiles" / "bgemv_stream_decode_m32_hbm_traffic.txt"
-    if not path.is_file():
-        return None
-    for line in path.read_text().splitlines():
-        if line.startswith("traffic_bytes_per_launch:"):
-            return int(float(line.split(":", 1)[1]))
-    return None
+    """HBM bytes of one M = 32 launch from the L2-to-fabric byte counters, measured now: FETCH_SIZE and
+    WRITE_SIZE (KiB per dispatch) each in a run of its own, each scaled by what the same counter
+    reads for a plain copy of COPY_BYTES in that run. {"traffic": None, ...} when the profiler is
+    missing or a pass fails."""
+    try:
+        copy_fetch, decode_fetch = counter_pass("FETCH_SIZE")
+        copy_write, decode_write = counter_pass("WRITE_SIZE")
+    except (OSError, subprocess.SubprocessError, RuntimeError, KeyError, ValueError) as problem:
+        return {"traffic": None, "problem": str(problem)[:200]}
+    kib = COPY_BYTES / 1024
+    fetch_factor, write_factor = kib / copy_fetch, kib / copy_write
+    traffic = (decode_fetch * fetch_factor + decode_write * write_factor) * 1024
+    return {"traffic": int(traffic), "fetch_kib": round(decode_fetch, 1), "write_kib": round(decode_write, 1),
+            "fetch_factor": round(fetch_factor, 4), "write_factor": round(write_factor, 4),
+            "copy_bytes_each_way": COPY_BYTES, "algorithmic": decode_bytes(32)}
+
+
+COPY_BYTES = 448 << 20
 
 
 def profile_only(args, torch, _kernels, _native, device, normal, weights, inputs, outputs):
@@ -252,16 +397,17 @@ def profile_only(args, torch, _kernels, _native, device, normal, weights, inputs
 
         def launch(i):
             _kernels.matmul(inputs[m], weights[i % 3].t(), out=outputs[m])
-    elif args.only == "copy":
-        size = OUTPUTS * INNER * 2
+    elif args.only in ("copy", "traffic"):
         source, target = weights[0], weights[1]
-        native = _native.context(device)
+        also_decode = args.only == "traffic"  # the counter passes want both kernels in one run
 
         def launch(i):
             status = probes().camblas_probe_copy(
-                ct.c_void_p(torch.cuda.current_stream(device).cuda_stream), size,
+                ct.c_void_p(torch.cuda.current_stream(device).cuda_stream), COPY_BYTES,
                 ct.c_void_p(source.data_ptr()), ct.c_void_p(target.data_ptr()))
             assert status == 0, status
+            if also_decode:
+                _kernels.matmul(inputs[32], weights[2].t(), out=outputs[32])
     elif args.only.startswith("fp8m") and args.only != "fp8moe":
         tokens, features, inner = int(args.only[4:]), 18432, 7168
         rotate = 3 if tokens <= 256 else 1
@@ -280,12 +426,38 @@ def profile_only(args, torch, _kernels, _native, device, normal, weights, inputs
 
         def launch(i):
             step(i)
-    elif args.only.startswith("mx"):
-        packed, tokens, features, inner = args.only.startswith("mxe2m1"), 4096, 18432, 7168
-        w, scale, a, a_scale = mx_operands(torch, device, packed, tokens, features, inner)
+    elif args.only == "fp8block32":
+        features, inner = 18432, 7168
+        copies = [torch.randint(0, 0x7E, (features, inner), device=device, dtype=torch.uint8)
+                  .view(torch.float8_e4m3fn) for _ in range(3)]
+        token = torch.randint(0, 0x7E, (1, inner), device=device, dtype=torch.uint8).view(torch.float8_e4m3fn)
+        token_scale = torch.rand((1, inner // 32), device=device) * 0.1 + 1e-4
+        block_scale = torch.rand((features // 32, inner // 32), device=device) * 0.1 + 1e-4
 
         def launch(i):
+            _kernels.fp8_decode(token, token_scale, copies[i % 3], block_scale)
+    elif args.only.startswith("mx"):
+        packed, tokens, features, inner = args.only.startswith("mxe2m1"), int(args.only[7:]), 18432, 7168
+        rotate = 1 if tokens > 256 else 6 if packed else 3  # few tokens: weights from HBM, not the last-level cache
+        sets = [mx_operands(torch, device, packed, tokens, features, inner) for _ in range(rotate)]
+
+        def launch(i):
+            w, scale, a, a_scale = sets[i % rotate]
             _kernels.quantized_matmul(a, a_scale, w, scale)
+    elif args.only == "sgemm2048":
+        size = 2048
+        a32, b32 = torch.rand((size, size), device=device) * 2 - 1, torch.rand((size, size), device=device) * 2 - 1
+        c32 = torch.empty((size, size), device=device)
+
+        def launch(i):
+            _kernels.matmul(a32, b32, out=c32)
+    elif args.only == "prefillnn":
+        size = 4096
+        x, w = normal((size, size)), normal((size, size), 0.02)
+        y = torch.empty((size, size), dtype=torch.bfloat16, device=device)
+
+        def launch(i):
+            _kernels.matmul(x, w, out=y)
     elif args.only in ("attention", "layer"):
         layer, attention = layer_step(torch, _kernels, device, normal)
         launch = (lambda i: layer()) if args.only == "layer" else (lambda i: attention())
@@ -380,23 +552,36 @@ def extras(torch, _kernels, _native, device, normal):
     y = torch.empty((tokens, outputs), dtype=torch.bfloat16, device=device)
     c = normal((tokens, outputs))
     flops = 2.0 * tokens * outputs * inner
-    seconds = event_time(torch, lambda i: _kernels.matmul(x, w.t(), out=y), 10, 20)
+    # (matrix-bound lines run 50 + 100 launches: the first launches after a memory-bound phase run at a
+    # lower clock, which a short loop would fold into the average)
+    seconds = event_time(torch, lambda i: _kernels.matmul(x, w.t(), out=y), 50, 100)
     found["bf16_prefill_linear"] = {
         "shape": [tokens, outputs, inner], "us": round(seconds * 1e6, 1),
-        "tflops": round(flops / seconds / 1e12, 1), "frac_of_2.5PF": round(flops / seconds / BF16_PEAK, 4),
+        "tflops": round(flops / seconds / 1e12, 1), "roofline": roofline_of("mfma bf16", flops, seconds),
     }
-    seconds = event_time(torch, lambda i: _kernels.addmm(c, x, w.t(), beta=1.0), 3, 10)
+    seconds = event_time(torch, lambda i: _kernels.addmm(c, x, w.t(), beta=1.0), 10, 50)
     found["bf16_prefill_addmm_beta1"] = {
         "us": round(seconds * 1e6, 1), "tflops": round(flops / seconds / 1e12, 1),
+        "roofline": roofline_of("mfma bf16", flops, seconds),
         "note": "full [tokens, outputs] addend read by the product's epilogue (no expand+clone copy)",
     }
     row = normal((outputs,))
-    seconds = event_time(torch, lambda i: _kernels.addmm(row, x, w.t(), beta=1.0), 3, 10)
+    seconds = event_time(torch, lambda i: _kernels.addmm(row, x, w.t(), beta=1.0), 10, 50)
     found["bf16_prefill_addmm_bias_row"] = {
         "us": round(seconds * 1e6, 1), "tflops": round(flops / seconds / 1e12, 1),
+        "roofline": roofline_of("mfma bf16", flops, seconds),
         "note": "[outputs] bias row of a linear layer, read by the product's epilogue",
     }
-    del x, w, y, c
+    del x, w, y, c, row
+    # BF16 product with neither operand K-contiguous (row-major a @ b, 'N','N'): the layout-agnostic
+    # matrix-core kernel
+    size = 4096
+    x, w = normal((size, size)), normal((size, size), 0.02)
+    y = torch.empty((size, size), dtype=torch.bfloat16, device=device)
+    seconds = event_time(torch, lambda i: _kernels.matmul(x, w, out=y), 10, 30)
+    found["bf16_matmul_nn_4096"] = {"us": round(seconds * 1e6, 1),
+                                    "roofline": roofline_of("mfma bf16", 2.0 * size**3, seconds)}
+    del x, w, y
     # FP8 block-scaled linear; the decode sizes rotate three weight copies (396 MB) so that the
     # weights come from HBM rather than from the 256 MB last-level cache
     outputs, inner = 18432, 7168
@@ -412,13 +597,14 @@ def extras(torch, _kernels, _native, device, normal):
         rotate = 3 if tokens <= 256 else 1
         seconds = event_time(
             torch, lambda i: _kernels.fp8_block_matmul(a, a_scale, copies[i % rotate], w_scale,
-                                                       out=out), 10, 20)
+                                                       out=out), *((50, 100) if tokens >= 4096 else (20, 60)))
         flops = 2.0 * tokens * outputs * inner
         traffic = outputs * inner + w_scale.numel() * 4 + tokens * (inner + inner // 128 * 4 + outputs * 2)
+        # few tokens stream the weights once (HBM roofline); 4096 tokens are matrix-core work
+        bound = ("mfma fp8", flops) if flops / FP8_PEAK > traffic / HBM_PEAK else ("hbm", traffic)
         fp8[str(tokens)] = {
             "us": round(seconds * 1e6, 1), "tflops": round(flops / seconds / 1e12, 1),
-            "frac_of_5PF": round(flops / seconds / FP8_PEAK, 4),
-            "gbps": round(traffic / seconds / 1e9, 1), "frac_of_8TBs": round(traffic / seconds / HBM_PEAK, 4),
+            "gbps": round(traffic / seconds / 1e9, 1), "roofline": roofline_of(*bound, seconds),
         }
     found["fp8_block_linear_18432x7168"] = fp8
     # single-token block-32 product of the reference header (FP32 scales per 32 x 32 block)
@@ -430,7 +616,7 @@ def extras(torch, _kernels, _native, device, normal):
     traffic = outputs * inner + block_scale.numel() * 4 + inner + inner // 32 * 4 + outputs * 2
     found["fp8_block32_decode_18432x7168"] = {
         "us": round(seconds * 1e6, 1), "gbps": round(traffic / seconds / 1e9, 1),
-        "frac_of_8TBs": round(traffic / seconds / HBM_PEAK, 4),
+        "roofline": roofline_of("hbm", traffic, seconds),
     }
     # E8M0 block-scaled (microscaling) decode products of the reference header: E4M3 and packed E2M1
     # weights [18432, 7168], 16 tokens, rotating weight copies
@@ -452,16 +638,16 @@ def extras(torch, _kernels, _native, device, normal):
             10, 20)
         traffic = weights[0].numel() + scale.numel() + tokens * (inner + inner // 32 + outputs * 2)
         mx[name] = {"us": round(seconds * 1e6, 1), "gbps": round(traffic / seconds / 1e9, 1),
-                    "frac_of_8TBs": round(traffic / seconds / HBM_PEAK, 4)}
+                    "roofline": roofline_of("hbm", traffic, seconds)}
     found["mx_quantized_matmul_m16_18432x7168"] = mx
     # the same products at 4096 tokens (tiled kernel, hardware-scaled matrix instructions)
     mx = {}
     for name, packed in (("e4m3", False), ("e2m1", True)):
         w, scale, a, a_scale = mx_operands(torch, device, packed, 4096, outputs, inner)
-        seconds = event_time(torch, lambda i: _kernels.quantized_matmul(a, a_scale, w, scale), 3, 10)
+        seconds = event_time(torch, lambda i: _kernels.quantized_matmul(a, a_scale, w, scale), 50, 100)
         flops = 2.0 * 4096 * outputs * inner
         mx[name] = {"us": round(seconds * 1e6, 1), "tflops": round(flops / seconds / 1e12, 1),
-                    "frac_of_5PF": round(flops / seconds / FP8_PEAK, 4)}
+                    "roofline": roofline_of("mfma fp8", flops, seconds)}
         del w, scale, a, a_scale
     found["mx_quantized_matmul_m4096_18432x7168"] = mx
     # the grouped form as an MoE prefill meets it: 32 experts of [4096, 7168] with a capacity of 1024
@@ -483,7 +669,7 @@ def extras(torch, _kernels, _native, device, normal):
                                                                    outputs=features, packed=packed), 2, 5)
             grouped[name + "_" + label] = {
                 "us": round(seconds * 1e6, 1),
-                "useful_pflops": round(2.0 * experts * fill * features * inner / seconds / 1e15, 3)}
+                "roofline": roofline_of("mfma fp8", 2.0 * experts * fill * features * inner, seconds)}
         del parts, table, tokens, token_scale
     found["mx_grouped_32_experts_4096x7168_capacity_1024"] = grouped
     # decode attention when the cache is larger than the sequences: 32 sequences of 512 positions in a
@@ -494,8 +680,7 @@ def extras(torch, _kernels, _native, device, normal):
     live = torch.full((32,), 512, dtype=torch.int32, device=device)
     seconds = event_time(torch, lambda i: _kernels.gqa_decode_attention(query, cache_k, cache_v, live), 3, 10)
     found["gqa_decode_512_live_of_8192"] = {
-        "us": round(seconds * 1e6, 1),
-        "tb_per_s_of_live_cache": round(2 * 32 * 512 * 8 * 128 * 2 / seconds / 1e12, 2)}
+        "us": round(seconds * 1e6, 1), "roofline": roofline_of("hbm", 2 * 32 * 512 * 8 * 128 * 2, seconds)}
     del cache_k, cache_v, query
     del copies, w_scale
     # FP32 SGEMM 2048^3 (plumbing)
@@ -503,17 +688,16 @@ def extras(torch, _kernels, _native, device, normal):
     a32 = torch.rand((size, size), device=device) * 2 - 1
     b32 = torch.rand((size, size), device=device) * 2 - 1
     c32 = torch.empty((size, size), device=device)
-    seconds = event_time(torch, lambda i: _kernels.matmul(a32, b32, out=c32), 3, 10)
+    seconds = event_time(torch, lambda i: _kernels.matmul(a32, b32, out=c32), 20, 60)
     found["fp32_sgemm_2048"] = {"us": round(seconds * 1e6, 1),
-                                "tflops": round(2.0 * size**3 / seconds / 1e12, 2),
-                                "frac_of_157TF": round(2.0 * size**3 / seconds / FP32_PEAK, 4)}
+                                "roofline": roofline_of("mfma fp32", 2.0 * size**3, seconds)}
     # single-token FP8 expert step (9 of 289 experts, rotating sets)
     experts, hidden, width, choices = MOE_SHAPE
     step = moe_step(torch, _kernels, device, normal)
     seconds = event_time(torch, step, 10, 40)
     traffic = choices * (2 * width * hidden + hidden * width)
     found["fp8_moe_decode_9_of_289_experts"] = {
-        "us": round(seconds * 1e6, 1), "gbps": round(traffic / seconds / 1e9, 1),
+        "us": round(seconds * 1e6, 1), "roofline": roofline_of("hbm", traffic, seconds),
         "note": "two launches; bound by launch and latency, not bandwidth"}
     del step
     # what the matrix cores sustain: independent matrix instructions with no memory traffic (the
@@ -549,8 +733,7 @@ def extras(torch, _kernels, _native, device, normal):
                                      ct.c_void_p(a64.data_ptr()), size, ct.c_void_p(b64.data_ptr()), size,
                                      ct.c_double(0.0), ct.c_void_p(c64.data_ptr()), size), 2, 5)
     found["fp64_dgemm_4096"] = {"us": round(seconds * 1e6, 1),
-                                "tflops": round(2.0 * size**3 / seconds / 1e12, 2),
-                                "frac_of_78.6TF": round(2.0 * size**3 / seconds / 78.6e12, 4)}
+                                "roofline": roofline_of("mfma fp64", 2.0 * size**3, seconds)}
     del a64, b64, c64
     # FP32 SGEMM 8192^3: the ordinary kernel and the default policy (two Strassen levels from 8192;
     # its time includes the guard's stream synchronisation), flops counted as 2 n^3 for both
@@ -567,7 +750,7 @@ def extras(torch, _kernels, _native, device, normal):
                     "sgemm", b"N", b"N", size, size, size, ct.c_float(1.0), ct.c_void_p(a32.data_ptr()), size,
                     ct.c_void_p(b32.data_ptr()), size, ct.c_float(0.0), ct.c_void_p(c32.data_ptr()), size), 1, 3)
         entry[policy] = {"ms": round(seconds * 1e3, 2),
-                         "tflops_equivalent": round(2.0 * size**3 / seconds / 1e12, 1)}
+                         "roofline": roofline_of("mfma fp32", 2.0 * size**3, seconds)}
     _native.context(device)  # back to the thread's policy
     found["fp32_sgemm_8192"] = entry
     del a32, b32, c32
@@ -577,7 +760,7 @@ def extras(torch, _kernels, _native, device, normal):
     def layer(i):
         return step()
 
-    eager = event_time(torch, layer, 3, 10)
+    eager = event_time(torch, layer, 10, 50)
     # the same step replayed from a captured graph (capture on a side stream after a warm-up there)
     side = torch.cuda.Stream()
     side.wait_stream(torch.cuda.current_stream())
@@ -589,18 +772,25 @@ def extras(torch, _kernels, _native, device, normal):
     with torch.cuda.graph(graph, stream=side):
         layer(0)
     replayed = event_time(torch, lambda i: graph.replay(), 3, 20)
+    # a model replays all of its layers from one graph: eight steps in one graph show how much of a
+    # replay is paid per launch of a graph rather than per kernel in it
+    layers = 8
+    stack = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(stack, stream=side):
+        for _ in range(layers):
+            layer(0)
+    stacked = event_time(torch, lambda i: stack.replay(), 2, 10) / layers
     traffic = LAYER_BYTES
     seconds = event_time(torch, lambda i: attention(), 3, 20)
     found["gqa_decode_attention_b32_ctx2048"] = {
-        "us": round(seconds * 1e6, 1), "gbps": round(KV_BYTES / seconds / 1e9, 1),
-        "frac_of_8TBs": round(KV_BYTES / seconds / HBM_PEAK, 4),
+        "us": round(seconds * 1e6, 1), "roofline": roofline_of("hbm", KV_BYTES, seconds),
     }
     found["llama70b_layer_decode_b32_ctx2048"] = {
         "eager_us": round(eager * 1e6, 1), "graph_us": round(replayed * 1e6, 1),
-        "gbps": round(traffic / min(eager, replayed) / 1e9, 1),
-        "frac_of_8TBs": round(traffic / min(eager, replayed) / HBM_PEAK, 4),
-        "note": "one layer, 10 library calls; rate from the faster of stream launches and graph replay "
-                "(both are device-bound); weights not rotated (1.7 GB per layer, beyond the "
+        "graph_of_8_steps_us_per_step": round(stacked * 1e6, 1),
+        "roofline": roofline_of("hbm", traffic, min(eager, replayed, stacked)),
+        "note": "one layer, 9 library calls; rate from the fastest of stream launches, a one-step graph and an "
+                "eight-step graph (all device-bound); weights not rotated (1.7 GB per layer, beyond the "
                 "256 MB last-level cache)",
     }
     return found
