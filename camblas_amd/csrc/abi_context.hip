@@ -64,6 +64,26 @@ hipError_t reserve_scratch(camblas_cuda_context *context, size_t bytes)
     return hipSuccess;
 }
 
+hipError_t reserve_arrivals(camblas_cuda_context *context)
+{
+    if (context->arrivals)
+        return hipSuccess;
+    if (stream_is_capturing(context->stream))
+        return hipErrorStreamCaptureUnsupported;
+    void *counters = nullptr;
+    hipError_t status = hipMalloc(&counters, STREAM_ARRIVAL_SLOTS * sizeof(unsigned));
+    if (status == hipSuccess)
+        status = hipMemsetAsync(counters, 0, STREAM_ARRIVAL_SLOTS * sizeof(unsigned), context->stream);
+    if (status != hipSuccess) {
+        (void)hipGetLastError();
+        if (counters)
+            (void)hipFree(counters);
+        return status;
+    }
+    context->arrivals = static_cast<unsigned *>(counters);
+    return hipSuccess;
+}
+
 } // namespace camblas_hip
 
 using namespace camblas_hip;
@@ -125,6 +145,8 @@ extern "C" int camblas_cuda_destroy(camblas_cuda_context *context)
         const hipError_t drained = hipStreamSynchronize(context->stream);
         if (context->scratch)
             (void)hipFree(context->scratch);
+        if (context->arrivals)
+            (void)hipFree(context->arrivals);
         for (void *arena : context->retired)
             (void)hipFree(arena);
         delete context;

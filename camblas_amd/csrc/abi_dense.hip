@@ -322,37 +322,13 @@ template <typename T> struct BackwardPass {
     }
 };
 
-// BF16 'T','N' and the other layouts: the planner's kernel, or the one a test forced.
-// `source`: where the beta term is read from when that is not C itself (see BetaSource). The
-// K-contiguous families read it in their epilogues; for the others it is first spread over C.
-int bf16_product(const Entry &entry, const Product &p, float alpha, const void *a, const void *b, float beta,
-                 void *c, BetaSource source = {})
+// Launches one planned BF16 product. `reserved`: FP32 room for a split K that the caller already
+// holds inside the context's arena (null: reserve it here).
+int launch_bf16_plan(const Entry &entry, Plan plan, const Product &p, float alpha, const void *a, const void *b,
+                     float beta, void *c, BetaSource source, float *reserved)
 {
     camblas_cuda_context *context = entry.context();
     hipStream_t stream = context->stream;
-    Plan plan = make_plan(2, context->algorithm, p.trans_a, p.trans_b, p.m, p.n, p.k, p.lda, p.ldb, p.ldc,
-                          is_aligned(a, 16) && is_aligned(b, 16), context->compute_units);
-    if (plan.family == FAMILY_DMA && (!is_aligned(c, 8) || !is_aligned(source.z, 8) || source.ldz % 4))
-        plan.family = FAMILY_MFMA_TN; // same tile shapes, register-staged loads, scalar stores
-    const bool matrix_family =
-        plan.family == FAMILY_MFMA_TN || plan.family == FAMILY_STREAM || plan.family == FAMILY_DMA;
-    if (matrix_family && context->override_kernel >= 0) {
-        // tests: 0.. a register-staged tile variant (with override_split), 20..59 a direct-to-LDS
-        // variant, 100 + 100*depth + 10*row_tiles + token_tiles the streaming kernel
-        const int forced = context->override_kernel;
-        plan.split_k = 1;
-        if (forced >= 100) {
-            plan.family = FAMILY_STREAM;
-            plan.kernel = forced - 100;
-        } else if (forced >= 20 && forced < 60) {
-            plan.family = FAMILY_DMA;
-            plan.kernel = forced - 20;
-        } else {
-            plan.family = FAMILY_MFMA_TN;
-            plan.kernel = forced;
-            plan.split_k = std::max(1, context->override_split);
-        }
-    }
     const bool in_epilogue =
         plan.family == FAMILY_MFMA_TN || plan.family == FAMILY_STREAM || plan.family == FAMILY_DMA;
     if (source.z && !in_epilogue) {
@@ -367,15 +343,30 @@ int bf16_product(const Entry &entry, const Product &p, float alpha, const void *
         return entry.finish(launch_bgemm_dma(stream, plan.kernel, p.m, p.n, p.k, alpha, a, p.lda, b, p.ldb, beta,
                                              c, p.ldc, source),
                             "BF16 MFMA GEMM (direct LDS loads)");
-    case FAMILY_STREAM:
+    case FAMILY_STREAM: {
+        StreamShares shares;
+        if (plan.split_k > 1) {
+            // K divided over several workgroups per tile needs FP32 planes and zeroed counters;
+            // without them (allocation failure, capture in progress) the undivided choice runs
+            const size_t bytes = stream_partial_bytes(plan.kernel / 10 % 10, plan.kernel % 10, p.m, p.n, plan.split_k);
+            if (reserve_arrivals(context) == hipSuccess &&
+                (reserved || reserve_scratch(context, bytes) == hipSuccess)) {
+                float *planes = reserved ? reserved : static_cast<float *>(context->scratch);
+                shares = StreamShares{plan.split_k, planes, context->arrivals};
+            } else {
+                context->counts[5]++;
+                plan.kernel = undivided_stream_kernel(p.m, p.n, p.k, context->compute_units);
+            }
+        }
         context->counts[plan.counter]++;
         return entry.finish(launch_bgemv_stream(stream, plan.kernel / 100, plan.kernel / 10 % 10,
                                                 plan.kernel % 10, p.m, p.n, p.k, alpha, a, p.lda, b, p.ldb,
-                                                beta, c, p.ldc, source),
+                                                beta, c, p.ldc, source, shares),
                             "BF16 streaming GEMV");
+    }
     case FAMILY_MFMA_TN: {
-        float *partials = nullptr;
-        if (plan.split_k > 1) {
+        float *partials = reserved;
+        if (plan.split_k > 1 && !partials) {
             // without room for the partials (allocation failure, capture in progress) run unsplit
             if (reserve_scratch(context, size_t(plan.split_k) * size_t(p.m) * size_t(p.n) * 4) == hipSuccess) {
                 partials = static_cast<float *>(context->scratch);
@@ -400,6 +391,98 @@ int bf16_product(const Entry &entry, const Product &p, float alpha, const void *
                                                 p.ldb, beta, c, p.ldc),
                             "BF16 GEMM");
     }
+}
+
+// A large product whose operands are not both K-contiguous: the ones that are not are first copied
+// transposed into the arena, after which the product is the linear-layer shape and runs on the
+// direct-to-LDS tiles: measured 132 against 557 us at 4096^3 and 19 against 25 us at 512^3, the
+// cost being one extra pass over each copied operand. Returns 1 when the arena could not hold the
+// copies.
+constexpr double TRANSPOSE_WORTHWHILE_FLOPS = 2.5e8; // about 512^3: below, the extra launches cost more
+int bf16_product_transposing(const Entry &entry, const Product &p, float alpha, const void *a, const void *b,
+                             float beta, void *c, const BetaSource &source)
+{
+    camblas_cuda_context *context = entry.context();
+    hipStream_t stream = context->stream;
+    const auto padded = [](size_t elements) { return (elements * 2 + 255) / 256 * 256; };
+    const size_t a_bytes = p.trans_a ? 0 : padded(size_t(p.m) * p.k);
+    const size_t b_bytes = p.trans_b ? padded(size_t(p.n) * p.k) : 0;
+    Product q = p;
+    q.trans_a = 1, q.trans_b = 0;
+    q.lda = p.trans_a ? p.lda : p.k;
+    q.ldb = p.trans_b ? p.k : p.ldb;
+    const bool aligned = (!p.trans_a || is_aligned(a, 16)) && (p.trans_b || is_aligned(b, 16));
+    Plan plan = make_plan(2, context->algorithm, 1, 0, q.m, q.n, q.k, q.lda, q.ldb, q.ldc, aligned,
+                          context->compute_units);
+    if (plan.family == FAMILY_DMA && (!is_aligned(c, 8) || !is_aligned(source.z, 8) || source.ldz % 4))
+        plan.family = FAMILY_MFMA_TN;
+    size_t partial_bytes = 0; // room for a divided K, held in the same arena behind the copies
+    if (plan.split_k > 1 && plan.family == FAMILY_MFMA_TN)
+        partial_bytes = size_t(plan.split_k) * size_t(p.m) * size_t(p.n) * 4;
+    else if (plan.split_k > 1 && plan.family == FAMILY_STREAM)
+        partial_bytes = stream_partial_bytes(plan.kernel / 10 % 10, plan.kernel % 10, p.m, p.n, plan.split_k);
+    if (reserve_scratch(context, a_bytes + b_bytes + partial_bytes) != hipSuccess)
+        return 1;
+    char *arena = static_cast<char *>(context->scratch);
+    if (!p.trans_a) { // a[i + l*lda] -> [i*k + l]
+        const hipError_t status = launch_transpose_bf16(stream, p.k, p.m, a, p.lda, arena, p.k);
+        if (status != hipSuccess)
+            return entry.finish(status, "BF16 operand transposition");
+        a = arena;
+    }
+    if (p.trans_b) { // b[j + l*ldb] -> [j*k + l]
+        const hipError_t status = launch_transpose_bf16(stream, p.k, p.n, b, p.ldb, arena + a_bytes, p.k);
+        if (status != hipSuccess)
+            return entry.finish(status, "BF16 operand transposition");
+        b = arena + a_bytes;
+    }
+    float *reserved = partial_bytes ? reinterpret_cast<float *>(arena + a_bytes + b_bytes) : nullptr;
+    return launch_bf16_plan(entry, plan, q, alpha, a, b, beta, c, source, reserved);
+}
+
+// BF16 'T','N' and the other layouts: the planner's kernel, or the one a test forced.
+// `source`: where the beta term is read from when that is not C itself (see BetaSource). The
+// K-contiguous families read it in their epilogues; for the others it is first spread over C.
+int bf16_product(const Entry &entry, const Product &p, float alpha, const void *a, const void *b, float beta,
+                 void *c, BetaSource source = {})
+{
+    camblas_cuda_context *context = entry.context();
+    Plan plan = make_plan(2, context->algorithm, p.trans_a, p.trans_b, p.m, p.n, p.k, p.lda, p.ldb, p.ldc,
+                          is_aligned(a, 16) && is_aligned(b, 16), context->compute_units);
+    if (plan.family == FAMILY_DMA && (!is_aligned(c, 8) || !is_aligned(source.z, 8) || source.ldz % 4))
+        plan.family = FAMILY_MFMA_TN; // same tile shapes, register-staged loads, scalar stores
+    const int forced = context->override_kernel;
+    if (plan.family == FAMILY_MFMA_BF16) {
+        // tests: 60 keeps the layout-agnostic kernel, 61 takes the transposing route whatever the size
+        const bool worthwhile = 2.0 * p.m * p.n * p.k >= TRANSPOSE_WORTHWHILE_FLOPS;
+        if (forced == 61 || (forced != 60 && worthwhile)) {
+            const int status = bf16_product_transposing(entry, p, alpha, a, b, beta, c, source);
+            if (status <= 0)
+                return status;
+            context->counts[5]++; // no room for the copies: the layout-agnostic kernel after all
+        }
+        return launch_bf16_plan(entry, plan, p, alpha, a, b, beta, c, source, nullptr);
+    }
+    const bool matrix_family =
+        plan.family == FAMILY_MFMA_TN || plan.family == FAMILY_STREAM || plan.family == FAMILY_DMA;
+    if (matrix_family && forced >= 0) {
+        // tests: 0.. a register-staged tile variant (with override_split), 20..59 a direct-to-LDS
+        // variant, 100 + 100*depth + 10*row_tiles + token_tiles the streaming kernel
+        plan.split_k = 1;
+        if (forced >= 100) {
+            plan.family = FAMILY_STREAM;
+            plan.kernel = forced - 100;
+            plan.split_k = std::max(1, context->override_split);
+        } else if (forced >= 20 && forced < 60) {
+            plan.family = FAMILY_DMA;
+            plan.kernel = forced - 20;
+        } else {
+            plan.family = FAMILY_MFMA_TN;
+            plan.kernel = forced;
+            plan.split_k = std::max(1, context->override_split);
+        }
+    }
+    return launch_bf16_plan(entry, plan, p, alpha, a, b, beta, c, source, nullptr);
 }
 
 template <typename T>

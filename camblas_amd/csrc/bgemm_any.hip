@@ -239,7 +239,80 @@ hipError_t launch_columns(hipStream_t stream, bool ta, bool tb, int m, int n, in
     return launch_layout<true, true, COLUMNS>(stream, vector, grid, m, n, k, alpha, a, lda, b, ldb, beta, c, ldc,
                                               int(row_tiles));
 }
+// dst[c * ld_dst + r] = src[r * ld_src + c] for a 2-byte element matrix of `rows` strided rows and
+// `cols` contiguous columns: 64 x 64 tiles through LDS, 8-byte global accesses on both sides when
+// VECTOR (tile rows start 8-byte aligned on both sides), else element by element. The LDS pitch of
+// 65 elements makes both the row-wise writes and the column-wise reads conflict-poor.
+template <bool VECTOR>
+__global__ __launch_bounds__(256) void transpose_bf16_kernel(int rows, int cols, const unsigned short *src,
+                                                              int ld_src, unsigned short *dst, int ld_dst,
+                                                              int col_tiles)
+{
+    constexpr int TILE = 64, PITCH = TILE + 1;
+    __shared__ unsigned short tile[TILE * PITCH];
+    const int r0 = int(blockIdx.x / col_tiles) * TILE, c0 = int(blockIdx.x % col_tiles) * TILE;
+    const int thread = threadIdx.x, quad = thread % 16, line = thread / 16;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        const int r = line + 16 * i, c = quad * 4;
+        unsigned short v[4] = {0, 0, 0, 0};
+        if (r0 + r < rows) {
+            const unsigned short *from = src + size_t(r0 + r) * ld_src + c0 + c;
+            if (VECTOR && c0 + c + 3 < cols) {
+                const u32x2_t packed = *reinterpret_cast<const u32x2_t *>(from);
+                v[0] = packed[0] & 0xffffu, v[1] = packed[0] >> 16, v[2] = packed[1] & 0xffffu, v[3] = packed[1] >> 16;
+            } else {
+#pragma unroll
+                for (int e = 0; e < 4; ++e)
+                    if (c0 + c + e < cols)
+                        v[e] = from[e];
+            }
+        }
+#pragma unroll
+        for (int e = 0; e < 4; ++e)
+            tile[r * PITCH + c + e] = v[e];
+    }
+    __syncthreads();
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        const int c = line + 16 * i, r = quad * 4; // output row c0 + c, output columns r0 + r ..
+        if (c0 + c >= cols)
+            continue;
+        unsigned short v[4];
+#pragma unroll
+        for (int e = 0; e < 4; ++e)
+            v[e] = tile[(r + e) * PITCH + c];
+        unsigned short *to = dst + size_t(c0 + c) * ld_dst + r0 + r;
+        if (VECTOR && r0 + r + 3 < rows) {
+            *reinterpret_cast<u32x2_t *>(to) = u32x2_t{unsigned(v[0]) | unsigned(v[1]) << 16,
+                                                       unsigned(v[2]) | unsigned(v[3]) << 16};
+        } else {
+#pragma unroll
+            for (int e = 0; e < 4; ++e)
+                if (r0 + r + e < rows)
+                    to[e] = v[e];
+        }
+    }
+}
 } // namespace
+
+hipError_t launch_transpose_bf16(hipStream_t stream, int rows, int cols, const void *src, int ld_src, void *dst,
+                                 int ld_dst)
+{
+    const size_t row_tiles = (size_t(rows) + 63) / 64, col_tiles = (size_t(cols) + 63) / 64;
+    if (rows < 1 || cols < 1 || row_tiles * col_tiles > 0x7fffffffu)
+        return hipErrorInvalidValue;
+    const bool vector = ld_src % 4 == 0 && ld_dst % 4 == 0 && reinterpret_cast<uintptr_t>(src) % 8 == 0 &&
+                        reinterpret_cast<uintptr_t>(dst) % 8 == 0;
+    const unsigned short *from = static_cast<const unsigned short *>(src);
+    unsigned short *to = static_cast<unsigned short *>(dst);
+    const unsigned grid = unsigned(row_tiles * col_tiles);
+    if (vector)
+        transpose_bf16_kernel<true><<<grid, 256, 0, stream>>>(rows, cols, from, ld_src, to, ld_dst, int(col_tiles));
+    else
+        transpose_bf16_kernel<false><<<grid, 256, 0, stream>>>(rows, cols, from, ld_src, to, ld_dst, int(col_tiles));
+    return launch_status();
+}
 
 // wide: 128 x 128 tiles, else 128 x 64
 hipError_t launch_bgemm_any(hipStream_t stream, bool wide, bool ta, bool tb, int m, int n, int k, float alpha,

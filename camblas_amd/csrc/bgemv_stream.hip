@@ -16,6 +16,7 @@
 // src/cuda/decode_float.cuh:2-52 (FP32, one vector).
 #include "common.hpp"
 #include "device.hpp"
+#include "dma.hpp"
 
 namespace camblas_hip
 {
@@ -31,9 +32,25 @@ struct StreamParams {
     int n, m, k;
     float alpha, beta;
     int vector_store; // 8-byte accesses to y (and z) rows are aligned
+    // K divided over gridDim.z workgroups per output tile: FP32 planes [gridDim.z, m, n] and one
+    // arrival counter per (blockIdx.x, blockIdx.y), zero before and after every launch
+    float *partials;
+    unsigned *arrivals;
 };
 
 constexpr int WAVES = 4, DEPTH = 2;
+
+// 16 bytes per lane written to / read from the point of coherence of the whole device (cache
+// policy bit 4, "sc1": device scope on gfx950), byte offset inside a buffer resource. Kept out of
+// the kernel template: the host pass drops a template instantiation that meets a target builtin.
+__device__ __forceinline__ void store_device_scope(__amdgpu_buffer_rsrc_t resource, unsigned offset, f32x4_t value)
+{
+    __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(u32x4_t, value), resource, int(offset), 0, 0x10);
+}
+__device__ __forceinline__ f32x4_t load_device_scope(__amdgpu_buffer_rsrc_t resource, unsigned offset)
+{
+    return __builtin_bit_cast(f32x4_t, __builtin_amdgcn_raw_buffer_load_b128(resource, int(offset), 0, 0x10));
+}
 
 // NT, MT: 16-row weight tiles and 16-token tiles per workgroup; a K step is KT blocks of 32*WAVES
 // elements, each block split over the WAVES wavefronts; DEPTH K steps are in flight in registers.
@@ -57,7 +74,12 @@ __global__ __launch_bounds__(WAVES * 64) void bgemv_stream_kernel(StreamParams p
     const int thread = threadIdx.x, lane = thread % 64, wave = thread / 64;
     const int chunk = thread % CH, pass_row = thread / CH; // CH lanes per row segment, 16 rows per pass
     const int n0 = blockIdx.x * ROWS, m0 = blockIdx.y * XROWS;
-    const int k_tiles = (p.k + BK * KT - 1) / (BK * KT);
+    // this workgroup's K steps: [first_tile, first_tile + k_tiles) of all_tiles (all of them unless
+    // the launch divides K over blockIdx.z; the launcher leaves no share empty)
+    const int all_tiles = (p.k + BK * KT - 1) / (BK * KT);
+    const int share = (all_tiles + int(gridDim.z) - 1) / int(gridDim.z);
+    const int first_tile = int(blockIdx.z) * share;
+    const int k_tiles = all_tiles - first_tile < share ? all_tiles - first_tile : share;
 
     unsigned a_off[NT], b_off[MT];
 #pragma unroll
@@ -90,7 +112,7 @@ __global__ __launch_bounds__(WAVES * 64) void bgemv_stream_kernel(StreamParams p
     const int start = int(blockIdx.x % unsigned(k_tiles));
     auto rotated = [&](int step) {
         int tile = (step < k_tiles ? step : k_tiles - 1) + start;
-        return tile < k_tiles ? tile : tile - k_tiles;
+        return first_tile + (tile < k_tiles ? tile : tile - k_tiles);
     };
     // W is read exactly once, so its loads are non-temporal: they bypass the cache allocation that
     // a 470 MB stream would otherwise keep evicting (measured: 5.7 -> 6.3 TB/s); x is re-read by
@@ -199,6 +221,44 @@ __global__ __launch_bounds__(WAVES * 64) void bgemv_stream_kernel(StreamParams p
             sum = sum + combine[(w * NT * MT + index) * 64 + lane];
         return sum;
     };
+    // ---- K divided over several workgroups: every workgroup parks its sums in its own FP32 plane;
+    // the one that arrives last (a counter per output tile) adds the planes in index order, so the
+    // result does not depend on which workgroup that was, and writes the output.
+    const bool divided = !GATED && gridDim.z > 1;
+    // a plane holds, per output tile of a workgroup, 64 lanes x 4 sums in the accumulator's own
+    // layout: whole wavefronts store and load 1 KB runs
+    constexpr unsigned TILE_BYTES = 64 * 16, GROUP_BYTES = unsigned(HALF * MT) * TILE_BYTES;
+    const size_t plane_bytes = size_t(gridDim.x) * gridDim.y * GROUP_BYTES;
+    const char *group = reinterpret_cast<const char *>(p.partials) +
+                        (size_t(blockIdx.y) * gridDim.x + blockIdx.x) * GROUP_BYTES;
+    if (divided) {
+        const __amdgpu_buffer_rsrc_t mine = make_resource(group + blockIdx.z * plane_bytes, GROUP_BYTES);
+#pragma unroll
+        for (int index = 0; index < HALF * MT; ++index) {
+            if (index % WAVES != wave)
+                continue;
+            const f32x4_t sum = summed(index);
+            store_device_scope(mine, unsigned(index) * TILE_BYTES + unsigned(lane) * 16, sum);
+        }
+        // The planes are written and read with device-scope accesses, which go to the point where
+        // all XCDs agree instead of staying in one XCD's L2, so no cache has to be written back or
+        // invalidated (a device-scope fence per workgroup was measured at +20 us on a 70 us
+        // launch). The barrier waits until this workgroup's stores have been acknowledged there;
+        // only then is the arrival counted.
+        __syncthreads(); // (also: every wavefront is done with `combine`)
+        unsigned *flag = reinterpret_cast<unsigned *>(lds_bytes);
+        if (thread == 0) {
+            unsigned *counter = p.arrivals + size_t(blockIdx.y) * gridDim.x + blockIdx.x;
+            const unsigned before = __hip_atomic_fetch_add(counter, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            const unsigned last = before + 1 == gridDim.z ? 1u : 0u;
+            if (last) // nobody else touches it any more: ready for the next launch
+                __hip_atomic_store(counter, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            *flag = last;
+        }
+        __syncthreads();
+        if (*flag == 0)
+            return;
+    }
 #pragma unroll
     for (int index = 0; index < HALF * MT; ++index) {
         if (index % WAVES != wave)
@@ -206,9 +266,17 @@ __global__ __launch_bounds__(WAVES * 64) void bgemv_stream_kernel(StreamParams p
         const int i = index / MT, j = index % MT;
         const int m = m0 + j * 16 + lane % 16;
         const int n = n0 + i * 16 + (lane / 16) * 4;
+        f32x4_t sum;
+        if (divided) { // (before the bounds check: the loads are whole-wavefront)
+            sum = f32x4_t{0.f, 0.f, 0.f, 0.f};
+            for (unsigned z = 0; z < gridDim.z; ++z)
+                sum = sum + load_device_scope(make_resource(group + z * plane_bytes, GROUP_BYTES),
+                                              unsigned(index) * TILE_BYTES + unsigned(lane) * 16);
+        } else {
+            sum = summed(index);
+        }
         if (m >= p.m || n >= p.n)
             continue;
-        const f32x4_t sum = summed(index);
         float v[4] = {sum[0], sum[1], sum[2], sum[3]};
         unsigned short *out = p.y + size_t(m) * p.ldc + n;
         if constexpr (GATED) {
@@ -260,7 +328,7 @@ __global__ __launch_bounds__(WAVES * 64) void bgemv_stream_kernel(StreamParams p
 }
 
 template <int NT, int MT, int KT, bool GATED = false>
-hipError_t launch_one(hipStream_t stream, const StreamParams &p)
+hipError_t launch_one(hipStream_t stream, const StreamParams &p, int shares = 1)
 {
     constexpr size_t stage_bytes = size_t(2) * KT * (NT + MT) * 16 * (64 * WAVES);
     constexpr size_t parked_bytes = size_t(WAVES) * NT * MT * 64 * 16; // partial sums at the end
@@ -275,39 +343,52 @@ hipError_t launch_one(hipStream_t stream, const StreamParams &p)
         if (status != hipSuccess)
             return status;
         constexpr int rows = (GATED ? NT / 2 : NT) * 16;
-        dim3 grid(unsigned((p.n + rows - 1) / rows), unsigned((p.m + MT * 16 - 1) / (MT * 16)));
+        // every share of a divided K holds at least one K step
+        const int all_tiles = (p.k + 32 * WAVES * KT - 1) / (32 * WAVES * KT);
+        const int share = (all_tiles + shares - 1) / shares;
+        shares = (all_tiles + share - 1) / share;
+        dim3 grid(unsigned((p.n + rows - 1) / rows), unsigned((p.m + MT * 16 - 1) / (MT * 16)), unsigned(shares));
+        if (shares > 1 && (GATED || !p.partials || !p.arrivals || size_t(grid.x) * grid.y > STREAM_ARRIVAL_SLOTS))
+            return hipErrorInvalidValue;
         kernel<<<grid, WAVES * 64, lds_bytes, stream>>>(p);
         return launch_status();
     }
 }
 
 template <int MT, int KT>
-hipError_t launch_rows(hipStream_t stream, int row_tiles, const StreamParams &p)
+hipError_t launch_rows(hipStream_t stream, int row_tiles, const StreamParams &p, int shares)
 {
     switch (row_tiles) {
-    case 1: return launch_one<1, MT, KT>(stream, p);
-    case 2: return launch_one<2, MT, KT>(stream, p);
-    case 3: return launch_one<3, MT, KT>(stream, p);
-    case 4: return launch_one<4, MT, KT>(stream, p);
-    case 5: return launch_one<5, MT, KT>(stream, p);
-    case 6: return launch_one<6, MT, KT>(stream, p);
-    case 7: return launch_one<7, MT, KT>(stream, p);
-    case 8: return launch_one<8, MT, KT>(stream, p);
+    case 1: return launch_one<1, MT, KT>(stream, p, shares);
+    case 2: return launch_one<2, MT, KT>(stream, p, shares);
+    case 3: return launch_one<3, MT, KT>(stream, p, shares);
+    case 4: return launch_one<4, MT, KT>(stream, p, shares);
+    case 5: return launch_one<5, MT, KT>(stream, p, shares);
+    case 6: return launch_one<6, MT, KT>(stream, p, shares);
+    case 7: return launch_one<7, MT, KT>(stream, p, shares);
+    case 8: return launch_one<8, MT, KT>(stream, p, shares);
     default: return hipErrorInvalidValue;
     }
 }
 
 template <int KT>
-hipError_t launch_tokens(hipStream_t stream, int row_tiles, int token_tiles, const StreamParams &p)
+hipError_t launch_tokens(hipStream_t stream, int row_tiles, int token_tiles, const StreamParams &p, int shares)
 {
     switch (token_tiles) {
-    case 1: return launch_rows<1, KT>(stream, row_tiles, p);
-    case 2: return launch_rows<2, KT>(stream, row_tiles, p);
-    case 4: return launch_rows<4, KT>(stream, row_tiles, p);
+    case 1: return launch_rows<1, KT>(stream, row_tiles, p, shares);
+    case 2: return launch_rows<2, KT>(stream, row_tiles, p, shares);
+    case 4: return launch_rows<4, KT>(stream, row_tiles, p, shares);
     default: return hipErrorInvalidValue;
     }
 }
 } // namespace
+
+size_t stream_partial_bytes(int row_tiles, int token_tiles, int n_out, int m_rows, int shares)
+{
+    const size_t groups = size_t((n_out + row_tiles * 16 - 1) / (row_tiles * 16)) *
+                          size_t((m_rows + token_tiles * 16 - 1) / (token_tiles * 16));
+    return size_t(shares) * groups * size_t(row_tiles) * size_t(token_tiles) * 1024;
+}
 
 // Gated form: out[m, n] = round(round(silu(g)) * u) with g = round(x Wg^T), u = round(x Wu^T); a
 // workgroup owns 16 * pair_tiles output rows (that many gate rows and the same up rows) over the
@@ -332,6 +413,8 @@ hipError_t launch_gated_stream(hipStream_t stream, int pair_tiles, int token_til
     p.alpha = 1.f;
     p.beta = 0.f;
     p.vector_store = (ldc % 4 == 0) && (reinterpret_cast<uintptr_t>(y) % 8 == 0);
+    p.partials = nullptr;
+    p.arrivals = nullptr;
     if ((m_rows + token_tiles * 16 - 1) / (token_tiles * 16) > 65535)
         return hipErrorInvalidValue;
     switch (token_tiles * 10 + pair_tiles) {
@@ -354,7 +437,7 @@ hipError_t launch_gated_stream(hipStream_t stream, int pair_tiles, int token_til
 hipError_t launch_bgemv_stream(hipStream_t stream, int depth_log2, int row_tiles, int token_tiles, int n_out,
                                int m_rows, int k, float alpha, const void *w, int lda,
                                const void *x, int ldb, float beta, void *y, int ldc,
-                               const BetaSource &source)
+                               const BetaSource &source, const StreamShares &shares)
 {
     StreamParams p;
     p.w = static_cast<const unsigned short *>(w);
@@ -373,13 +456,15 @@ hipError_t launch_bgemv_stream(hipStream_t stream, int depth_log2, int row_tiles
     p.beta = beta;
     p.vector_store = ldc % 4 == 0 && reinterpret_cast<uintptr_t>(y) % 8 == 0 && p.ldz % 4 == 0 &&
                      reinterpret_cast<uintptr_t>(p.z) % 8 == 0;
-    if ((m_rows + token_tiles * 16 - 1) / (token_tiles * 16) > 65535)
+    p.partials = shares.partials;
+    p.arrivals = shares.arrivals;
+    if ((m_rows + token_tiles * 16 - 1) / (token_tiles * 16) > 65535 || shares.count < 1 || shares.count > 64)
         return hipErrorInvalidValue;
     switch (depth_log2) {
-    case 0: return launch_tokens<1>(stream, row_tiles, token_tiles, p);
-    case 1: return launch_tokens<2>(stream, row_tiles, token_tiles, p);
-    case 2: return launch_tokens<4>(stream, row_tiles, token_tiles, p);
-    case 3: return launch_tokens<8>(stream, row_tiles, token_tiles, p);
+    case 0: return launch_tokens<1>(stream, row_tiles, token_tiles, p, shares.count);
+    case 1: return launch_tokens<2>(stream, row_tiles, token_tiles, p, shares.count);
+    case 2: return launch_tokens<4>(stream, row_tiles, token_tiles, p, shares.count);
+    case 3: return launch_tokens<8>(stream, row_tiles, token_tiles, p, shares.count);
     default: return hipErrorInvalidValue;
     }
 }

@@ -21,6 +21,7 @@ struct camblas_cuda_context {
     size_t scratch_bytes = 0;
     std::vector<void *> retired;   // superseded scratch kept alive for captured graphs
     bool seen_capture = false;     // the arena has been used by a launch under stream capture
+    unsigned *arrivals = nullptr;  // zeroed counters of the divided-K streaming kernel (made on first use)
     int override_kernel = -1;      // diagnostics: forced kernel variant
     int override_split = 0;
     std::atomic<uint64_t> counts[8] = {};
@@ -37,6 +38,9 @@ int fail(camblas_cuda_context *context, const char *operation, int code);
 // Ensures the context scratch holds at least `bytes`; refuses to grow while the stream is
 // capturing (ref: src/cuda/backend.cu:399-426). Returns hipSuccess or the failing status.
 hipError_t reserve_scratch(camblas_cuda_context *context, size_t bytes);
+// The context's arrival counters (STREAM_ARRIVAL_SLOTS of them, zero between launches), made and
+// cleared on first use; never under stream capture.
+hipError_t reserve_arrivals(camblas_cuda_context *context);
 
 inline hipError_t launch_status() { return hipGetLastError(); }
 
@@ -146,6 +150,9 @@ hipError_t launch_generic_f64(hipStream_t stream, bool ta, bool tb, int m, int n
 hipError_t launch_bgemm_any(hipStream_t stream, bool wide, bool ta, bool tb, int m, int n, int k,
                             float alpha, const void *a, int lda, const void *b, int ldb, float beta,
                             void *c, int ldc);
+// dst[c * ld_dst + r] = src[r * ld_src + c], BF16 storage, `cols` the contiguous extent of src
+hipError_t launch_transpose_bf16(hipStream_t stream, int rows, int cols, const void *src, int ld_src, void *dst,
+                                 int ld_dst);
 hipError_t launch_gemv_f32(hipStream_t stream, int rows, int inner, float alpha, const float *w,
                            int ld, const float *x, float beta, float *y);
 // Where the beta term of a BF16 linear is read from: by default the output itself; otherwise
@@ -168,10 +175,22 @@ hipError_t launch_bgemm_dma(hipStream_t stream, int variant, int n_out, int m_ro
 // Decode-shaped BF16 linear: each workgroup streams 16*row_tiles weight rows over the whole K.
 // depth_log2: a K step is 2^depth_log2 blocks of 128 elements (0..3); row_tiles << depth_log2 <= 8
 // and (row_tiles + token_tiles) << depth_log2 <= 16 or the launch is refused.
+// shares: with count > 1 the K extent is divided over that many workgroups per output tile; each
+// parks FP32 sums in its plane of `partials` (stream_partial_bytes() in all, 16-byte aligned) and
+// the last to arrive adds the planes in index order. `arrivals` holds STREAM_ARRIVAL_SLOTS counters that are zero between
+// launches (the kernel leaves them so); one per output tile is used.
+constexpr size_t STREAM_ARRIVAL_SLOTS = 4096;
+size_t stream_partial_bytes(int row_tiles, int token_tiles, int n_out, int m_rows, int shares);
+struct StreamShares {
+    int count = 1;
+    float *partials = nullptr;
+    unsigned *arrivals = nullptr;
+};
+int undivided_stream_kernel(int outputs, int tokens, int k, int compute_units);
 hipError_t launch_bgemv_stream(hipStream_t stream, int depth_log2, int row_tiles, int token_tiles, int n_out,
                                int m_rows, int k, float alpha, const void *w, int lda,
                                const void *x, int ldb, float beta, void *y, int ldc,
-                               const BetaSource &source = {});
+                               const BetaSource &source = {}, const StreamShares &shares = {});
 // The gated-MLP front end for decode batches in one pass over both weight matrices:
 // y = round(round(silu(g)) * u), g = round(x gate^T), u = round(x up^T). pair_tiles 1..4 (16 output
 // rows each: that many gate rows and the same up rows per workgroup), token_tiles 1, 2 or 4.

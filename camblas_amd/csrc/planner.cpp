@@ -140,11 +140,21 @@ Plan make_plan(int dtype, int algorithm, bool trans_a, bool trans_b, int m, int 
         if (tokens <= 32 || (tokens <= 64 && !narrow)) {
             // decode: bandwidth-bound on W, one streaming pass, no split-K
             plan.family = FAMILY_STREAM;
-            const int row_tiles = stream_row_tiles(outputs, compute_units);
-            const int token_tiles = tokens <= 16 ? 1 : tokens <= 32 ? 2 : 4;
-            plan.kernel = 100 * stream_depth_log2(row_tiles, token_tiles, k) + 10 * row_tiles +
-                          token_tiles;
+            plan.kernel = undivided_stream_kernel(outputs, tokens, k, compute_units);
             plan.split_k = 1;
+            // Few output rows and a long K (a down projection): one workgroup per compute unit
+            // would own 32-48 weight rows and re-read as many token rows through L2. Two
+            // workgroups per output tile, each with half of K and twice the rows, keep the same
+            // number of workgroups with half the token traffic (measured at 32 tokens:
+            // [8192, 28672] 77 against 85-90 us, [10240, 8192] 30.5 against 33, [8192, 8192] even;
+            // up to 16 tokens the token rows are half as many and only K beyond 12288 gains).
+            const int row_tiles = plan.kernel / 10 % 10, token_tiles = plan.kernel % 10;
+            const int wider = std::min(8, ceil_div(2 * ceil_div(outputs, 16), compute_units));
+            const bool long_enough = token_tiles >= 2 ? k >= 8192 : k >= 12288;
+            if (row_tiles <= 3 && long_enough && wider > row_tiles && wider + token_tiles <= 16) {
+                plan.kernel = 10 * wider + token_tiles;
+                plan.split_k = 2;
+            }
         } else if (tokens <= 64) {
             // 33..64 tokens on a narrow projection: the streaming kernel would have 32-48 weight
             // rows per workgroup and re-read as many token rows through L2; 128 x 64 register-staged
@@ -264,6 +274,14 @@ Plan make_plan(int dtype, int algorithm, bool trans_a, bool trans_b, int m, int 
     return plan;
 }
 
+// The streaming kernel's variant code when every workgroup takes the whole K extent.
+int undivided_stream_kernel(int outputs, int tokens, int k, int compute_units)
+{
+    const int row_tiles = stream_row_tiles(outputs, compute_units);
+    const int token_tiles = tokens <= 16 ? 1 : tokens <= 32 ? 2 : 4;
+    return 100 * stream_depth_log2(row_tiles, token_tiles, k) + 10 * row_tiles + token_tiles;
+}
+
 void describe_plan(const Plan &plan, int dtype, char *text, size_t bytes)
 {
     if (!text || !bytes)
@@ -298,9 +316,9 @@ void describe_plan(const Plan &plan, int dtype, char *text, size_t bytes)
         std::snprintf(text, bytes, "%s %s", type, dma_variant(plan.kernel).name);
         break;
     case FAMILY_STREAM:
-        std::snprintf(text, bytes, "%s stream rows=%d tokens=%d k_step=%d", type,
+        std::snprintf(text, bytes, "%s stream rows=%d tokens=%d k_step=%d k_shares=%d", type,
                       16 * (plan.kernel / 10 % 10), 16 * (plan.kernel % 10),
-                      128 << (plan.kernel / 100));
+                      128 << (plan.kernel / 100), plan.split_k);
         break;
     default:
         std::snprintf(text, bytes, "%s generic 64x64x16", type);

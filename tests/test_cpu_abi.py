@@ -63,7 +63,10 @@ def test_planner_choices_for_the_baseline_shapes():
     code, text = describe(2, "T", "N", 28672, 32, 8192, 8192, 8192, 28672)
     assert code // 1000 == 4 and "stream rows=112 tokens=32" in text
     assert "tokens=16" in describe(2, "T", "N", 28672, 1, 8192, 8192, 8192, 28672)[1]
-    assert "rows=32" in describe(2, "T", "N", 8192, 32, 28672, 28672, 28672, 8192)[1]
+    # the down projection (few rows, long K): 64-row tiles, K divided over two workgroups per tile;
+    # a single token on a short K keeps the undivided 32-row tiles
+    assert "rows=64 tokens=32 k_step=128 k_shares=2" in describe(2, "T", "N", 8192, 32, 28672, 28672, 28672, 8192)[1]
+    assert "rows=32 tokens=16 k_step=256 k_shares=1" in describe(2, "T", "N", 8192, 1, 8192, 8192, 8192, 8192)[1]
     # prefill: direct-to-LDS MFMA tile that divides 10240 x 4096 into exactly two waves of tiles
     code, text = describe(2, "T", "N", 10240, 4096, 8192, 8192, 8192, 10240)
     assert code // 1000 == 5 and "dma320x256" in text

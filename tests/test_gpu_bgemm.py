@@ -176,6 +176,44 @@ def test_every_layout_on_the_matrix_cores(device, ta, tb, m, n, k, pad):
         assert code // 1000 == 9
 
 
+@pytest.mark.parametrize("ta,tb", [("N", "N"), ("N", "T"), ("T", "T")])
+@pytest.mark.parametrize("m,n,k,pad", [(200, 150, 72, 8), (130, 70, 33, 1), (300, 260, 320, 0)])
+def test_operands_transposed_into_the_linear_shape(device, ta, tb, m, n, k, pad):
+    # the route large products of these layouts take, forced at sizes the oracle finishes quickly:
+    # the operands that are not K-contiguous are copied transposed (odd leading dimensions take the
+    # element-wise copy, ragged edges in both directions) and the product runs as 'T','N'
+    lda = (m if ta == "N" else k) + pad
+    ldb = (k if tb == "N" else n) + pad
+    ldc = m + 4
+    a = oracle.fill_normal_bf16(95, (lda * (k if ta == "N" else m),))
+    b = oracle.fill_normal_bf16(96, (ldb * (n if tb == "N" else k),))
+    c0 = oracle.fill_normal_bf16(97, (ldc * n,))
+    got = run_bgemm(device, ta, tb, m, n, k, 0.75, a, lda, b, ldb, -0.5, c0, ldc, override=(61, 0))
+    want, want64 = reference(ta, tb, m, n, k, 0.75, a, lda, b, ldb, -0.5, c0, ldc)
+    got2d = got.reshape(n, ldc)
+    assert rel_frobenius(oracle.bf16_to_f32(got2d[:, :m]), want64.reshape(n, m)) <= TOLERANCE
+    assert np.array_equal(got2d[:, m:], c0.reshape(n, ldc)[:, m:])
+
+
+def test_large_product_of_another_layout_agrees_with_the_layout_agnostic_kernel(device):
+    # 1664 x 1600 x 1600 is well past the size from which the planner transposes; the layout-agnostic
+    # kernel (forced) is the check, both within the BF16 bar of each other
+    m, n, k = 1664, 1600, 1600
+    a = oracle.fill_normal_bf16(98, (m * k,))
+    b = oracle.fill_normal_bf16(99, (k * n,))
+    c0 = np.zeros(m * n, np.uint16)
+    native = _native.context(device)
+    native.call("reset_stats")
+    routed = run_bgemm(device, "N", "N", m, n, k, 1.0, a, m, b, k, 0.0, c0, m)
+    assert _native.stats(device)["lt"] == 1
+    direct = run_bgemm(device, "N", "N", m, n, k, 1.0, a, m, b, k, 0.0, c0, m, override=(60, 0))
+    assert rel_frobenius(oracle.bf16_to_f32(routed), oracle.bf16_to_f32(direct).astype(np.float64)) <= 4e-3
+    rows = np.arange(0, m, 97)  # sampled rows of C against FP64
+    a2, b2 = oracle.bf16_to_f32(a).reshape(k, m).astype(np.float64), oracle.bf16_to_f32(b).reshape(n, k).astype(np.float64)
+    want = (b2 @ a2[:, rows]).astype(np.float64)  # [n, rows]
+    assert rel_frobenius(oracle.bf16_to_f32(routed).reshape(n, m)[:, rows], want) <= TOLERANCE
+
+
 def test_layout_agnostic_kernel_counts_as_a_library_product(device):
     # row-major torch.mm(x, w) with a contiguous [in, out] weight arrives as 'N','N'
     native = _native.context(device)
@@ -389,3 +427,27 @@ def test_addend_argument_checks(device):
     assert call(ct.c_float(0.0), None, k, None, k, ct.c_float(0.5), ptr(z), 0, ptr(c), m) == 0  # only beta acts
     torch.cuda.synchronize()
     assert torch.equal(c[:m * n].float(), torch.ones(m * n, device=device))
+
+
+@pytest.mark.parametrize("n_out,m_rows,k,code,shares", [
+    (300, 32, 2048, 142, 2),    # 64-row tiles, two shares, ragged rows
+    (301, 9, 1664, 121, 3),     # odd N: element-wise partial planes and stores; 13 K steps in three shares
+    (512, 32, 4096, 182, 4),    # 128-row tiles
+    (256, 64, 1024, 234, 64),   # more shares asked for than K steps exist (k_step 256: four steps)
+    (113, 1, 1280, 111, 5),
+])
+def test_streaming_kernel_with_k_divided_over_workgroups(device, n_out, m_rows, k, code, shares):
+    # each share parks FP32 sums, the last workgroup to arrive adds the planes in index order: run
+    # twice (the counters must be back at zero) with alpha and beta, against the FP64 product; the
+    # second run must reproduce the first bit for bit whatever the arrival order was
+    lda, ldb, ldc = k + 8, k + 16, n_out + 4
+    w = oracle.fill_normal_bf16(60, (n_out * lda,))
+    x = oracle.fill_normal_bf16(61, (m_rows * ldb,))
+    c0 = oracle.fill_normal_bf16(62, (m_rows * ldc,))
+    first = run_bgemm(device, "T", "N", n_out, m_rows, k, 0.5, w, lda, x, ldb, 2.0, c0, ldc, override=(code, shares))
+    again = run_bgemm(device, "T", "N", n_out, m_rows, k, 0.5, w, lda, x, ldb, 2.0, c0, ldc, override=(code, shares))
+    assert np.array_equal(first, again)
+    want, want64 = reference("T", "N", n_out, m_rows, k, 0.5, w, lda, x, ldb, 2.0, c0, ldc)
+    got2d = first.reshape(m_rows, ldc)
+    assert rel_frobenius(oracle.bf16_to_f32(got2d[:, :n_out]), want64.reshape(m_rows, n_out)) <= TOLERANCE
+    assert np.array_equal(got2d[:, n_out:], c0.reshape(m_rows, ldc)[:, n_out:])
