@@ -234,8 +234,10 @@ int oracle_bgemm_f64(char ta, char tb, int m, int n, int k, float alpha, const u
 /* Dynamic 1x128 activation quantiser (camblas/_hopper.py:82-98): per group of 128 values,
  * amax = max(|x|, 1e-10); scale = amax * (1/448) in FP32; q = e4m3(clamp(x * inv, +-448)) with
  * inv = 448/amax. The reference computes inv with an approximate reciprocal-divide instruction;
- * this restatement uses the IEEE quotient, so FP8 bytes at exact rounding ties are
- * "parity unpinned" against the reference (everything else here is pinned by invariants). */
+ * this restatement uses the IEEE quotient, so FP8 bytes at exact rounding ties of that
+ * reciprocal are "parity unpinned" against the reference. The bytes themselves are pinned: the
+ * tests recompute x * inv in numpy and convert it with PyTorch's CPU float8_e4m3fn cast, which
+ * must give the same byte for every element. */
 void oracle_quantise_1x128(int rows, int inner, const uint16_t *x_bf16, uint8_t *q, float *scale)
 {
     int groups = inner / 128;
