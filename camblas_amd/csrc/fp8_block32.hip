@@ -16,6 +16,7 @@
 // through a private swizzled LDS patch, as in the 128-block streaming kernel.
 #include "common.hpp"
 #include "device.hpp"
+#include "dma.hpp"
 
 namespace camblas_hip
 {
@@ -44,15 +45,72 @@ __global__ __launch_bounds__(WAVES * 64) void fp8_block32_decode_kernel(Block32P
     const int blocks = p.k / 32, steps = (p.k + STEP - 1) / STEP;
     const int rounds = (steps + DEPTH - 1) / DEPTH, padded_steps = rounds * DEPTH;
 
+    // ---- addresses first, so that the weight stream can start before the token is staged. A
+    // wavefront past the last row keeps valid addresses (row 0) and leaves after the barrier.
+    const bool owns_rows = (blockIdx.x * WAVES + wave) * 16 < p.n;
+    const int first_row = owns_rows ? (blockIdx.x * WAVES + wave) * 16 : 0;
+    const int column = lane % 16, chunk = lane / 16; // operand column / row, 32-byte chunk = block
+    const int load_row = lane / 8, piece = lane % 8; // load layout: 8 lanes per 128-byte line
+    const unsigned char *row_base[2] = {p.w + size_t(first_row + load_row) * p.k,
+                                        p.w + size_t(first_row + 8 + load_row) * p.k};
+    const float *sw_row = p.sw + size_t(first_row / 32) * p.sw_row;
+    auto slot = [](int r, int q) { return r * 8 + (q ^ ((r >> 1) & 7)); };
+    const int store_slot[2] = {slot(load_row, piece), slot(load_row + 8, piece)};
+    const int read_slot[2] = {slot(column, 2 * chunk), slot(column, 2 * chunk + 1)};
+    u32x4_t *mine = &patch[wave][0];
+
+    // Loads only (nothing here may use a loaded value). Bytes past the end of a row in a partial
+    // last step, and whole steps past the end, re-read the row's last 16 bytes: x is zero there.
+    u32x4_t raw[DEPTH][2];
+    float sw_reg[DEPTH];
+    auto fetch = [&](int step, u32x4_t(&data)[2], float &scale) {
+        int offset = step * STEP + piece * 16;
+        offset = offset < p.k ? offset : p.k - 16;
+        data[0] = __builtin_nontemporal_load(reinterpret_cast<const u32x4_t *>(row_base[0] + offset));
+        data[1] = __builtin_nontemporal_load(reinterpret_cast<const u32x4_t *>(row_base[1] + offset));
+        int b = step * 4 + (column & 3);
+        b = b < blocks ? b : blocks - 1;
+        scale = sw_row[size_t(b) * p.sw_col];
+    };
+
+    // ---- the token: its loads are issued first, the first DEPTH weight steps right behind them,
+    // and only then are the token's values used (loads return in order, so waiting for the token
+    // does not wait for the weights): the weight stream's first latency overlaps the staging.
+    // Every loop below has a fixed trip count (MAX_K bounds it) so that the compiler can count the
+    // loads in flight instead of waiting for all of them.
+    static_assert(MAX_K / 32 <= WAVES * 64, "one 32-value block per thread");
+    constexpr int WORDS_PER_THREAD = MAX_K / 4 / (WAVES * 64);
+    const unsigned *source = static_cast<const unsigned *>(p.x);
+    unsigned staged[QUANTISE ? 16 : WORDS_PER_THREAD];
+    float staged_scale = 0.f;
     if constexpr (QUANTISE) {
-        const unsigned *source = static_cast<const unsigned *>(p.x); // BF16 pairs
-        for (int b = thread; b < padded_steps * 4; b += WAVES * 64) {
+        const int b = thread < blocks ? thread : blocks - 1; // BF16 pairs of block `thread`
+#pragma unroll
+        for (int e = 0; e < 16; ++e)
+            staged[e] = source[b * 16 + e];
+    } else {
+#pragma unroll
+        for (int i = 0; i < WORDS_PER_THREAD; ++i) {
+            const int word = thread + i * WAVES * 64;
+            staged[i] = source[word < p.k / 4 ? word : p.k / 4 - 1];
+        }
+        staged_scale = p.sx[size_t(thread < blocks ? thread : blocks - 1) * p.sx_stride];
+    }
+    __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+    for (int d = 0; d < DEPTH; ++d) {
+        fetch(d, raw[d], sw_reg[d]);
+        __builtin_amdgcn_sched_barrier(0);
+    }
+    if constexpr (QUANTISE) {
+        const int b = thread;
+        if (b < padded_steps * 4) {
             float value[32];
             float amax = 1e-10f;
             if (b < blocks) {
 #pragma unroll
                 for (int e = 0; e < 16; ++e) {
-                    unsigned pair = source[b * 16 + e];
+                    const unsigned pair = staged[e];
                     value[2 * e] = __uint_as_float(pair << 16);
                     value[2 * e + 1] = __uint_as_float(pair & 0xffff0000u);
                     amax = fmaxf(amax, fmaxf(fabsf(value[2 * e]), fabsf(value[2 * e + 1])));
@@ -80,40 +138,21 @@ __global__ __launch_bounds__(WAVES * 64) void fp8_block32_decode_kernel(Block32P
             }
         }
     } else {
-        const unsigned *source = static_cast<const unsigned *>(p.x);
-        for (int word = thread; word < padded_steps * 32; word += WAVES * 64)
-            x_words[word] = word < p.k / 4 ? source[word] : 0u;
-        for (int b = thread; b < padded_steps * 4; b += WAVES * 64)
-            x_scale[b] = b < blocks ? p.sx[size_t(b) * p.sx_stride] : 0.f;
+#pragma unroll
+        for (int i = 0; i < WORDS_PER_THREAD; ++i) {
+            const int word = thread + i * WAVES * 64;
+            if (word < padded_steps * 32)
+                x_words[word] = word < p.k / 4 ? staged[i] : 0u;
+        }
+        if (thread < padded_steps * 4)
+            x_scale[thread] = thread < blocks ? staged_scale : 0.f;
     }
-    __syncthreads();
-
-    const int first_row = (blockIdx.x * WAVES + wave) * 16;
-    if (first_row >= p.n)
+    // (not __syncthreads(): its fence would wait for every weight load issued above; the LDS
+    // stores are waited for explicitly, the weight loads stay in flight)
+    pipeline_barrier<63>();
+    if (!owns_rows)
         return; // no barrier below this point
-    const int column = lane % 16, chunk = lane / 16; // operand column / row, 32-byte chunk = block
-    const int load_row = lane / 8, piece = lane % 8; // load layout: 8 lanes per 128-byte line
-    const unsigned char *row_base[2] = {p.w + size_t(first_row + load_row) * p.k,
-                                        p.w + size_t(first_row + 8 + load_row) * p.k};
-    const float *sw_row = p.sw + size_t(first_row / 32) * p.sw_row;
-    auto slot = [](int r, int q) { return r * 8 + (q ^ ((r >> 1) & 7)); };
-    const int store_slot[2] = {slot(load_row, piece), slot(load_row + 8, piece)};
-    const int read_slot[2] = {slot(column, 2 * chunk), slot(column, 2 * chunk + 1)};
-    u32x4_t *mine = &patch[wave][0];
 
-    // Loads only (nothing here may use a loaded value). Bytes past the end of a row in a partial
-    // last step, and whole steps past the end, re-read the row's last 16 bytes: x is zero there.
-    u32x4_t raw[DEPTH][2];
-    float sw_reg[DEPTH];
-    auto fetch = [&](int step, u32x4_t(&data)[2], float &scale) {
-        int offset = step * STEP + piece * 16;
-        offset = offset < p.k ? offset : p.k - 16;
-        data[0] = __builtin_nontemporal_load(reinterpret_cast<const u32x4_t *>(row_base[0] + offset));
-        data[1] = __builtin_nontemporal_load(reinterpret_cast<const u32x4_t *>(row_base[1] + offset));
-        int b = step * 4 + (column & 3);
-        b = b < blocks ? b : blocks - 1;
-        scale = sw_row[size_t(b) * p.sw_col];
-    };
     float sum[4] = {0.f, 0.f, 0.f, 0.f};
     auto multiply = [&](int step, const u32x4_t(&data)[2], float scale) {
         mine[store_slot[0]] = data[0];
@@ -149,11 +188,6 @@ __global__ __launch_bounds__(WAVES * 64) void fp8_block32_decode_kernel(Block32P
         __builtin_amdgcn_wave_barrier();
     };
 
-#pragma unroll
-    for (int d = 0; d < DEPTH; ++d) {
-        fetch(d, raw[d], sw_reg[d]);
-        __builtin_amdgcn_sched_barrier(0);
-    }
     for (int step = 0; step < padded_steps; step += DEPTH) {
 #pragma unroll
         for (int d = 0; d < DEPTH; ++d) {

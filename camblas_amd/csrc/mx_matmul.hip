@@ -64,6 +64,8 @@ __global__ __launch_bounds__(WAVES * 64) void mx_stream_kernel(MxParams p)
     // other half of each line to another wavefront's request).
     constexpr int SUB = PACKED ? 2 : 1;
     constexpr int STEP_INPUTS = GROUP * SUB;
+    // (deeper queues for workgroups of few rows were measured: no gain, few rows per workgroup
+    // lose to the per-workgroup start and end whatever the queue depth)
     constexpr int DEPTH = NT + MT * SUB <= 6 ? 3 : 2; // steps in flight, by registers per step
     // per wavefront: NT weight tiles and MT input tiles of 16 x 128 bytes; after the last step the
     // same memory holds the wavefront's partial sums
@@ -364,7 +366,7 @@ hipError_t launch_one(hipStream_t stream, const MxParams &p, int groups)
 }
 
 template <bool PACKED, bool GROUPED>
-hipError_t launch_shape(hipStream_t stream, const MxParams &p, int groups)
+hipError_t launch_shape(hipStream_t stream, const MxParams &p, int groups, int forced_row_tiles)
 {
     // token tiles by row count; weight-row tiles so that about one workgroup lands on each compute
     // unit, all groups counted (decode-sized calls: the kernel is bound by the weight stream, and a
@@ -375,10 +377,12 @@ hipError_t launch_shape(hipStream_t stream, const MxParams &p, int groups)
     int row_tiles = 1;
     const int most = PACKED ? (token_tiles == 2 ? 6 : 8) : (token_tiles == 4 ? 4 : 8);
     for (int candidate = most; candidate > 1; --candidate)
-        if (static_cast<long long>(tiles / candidate) * groups >= 192) {
+        if (static_cast<long long>(tiles / candidate) * groups >= 224) {
             row_tiles = candidate;
             break;
         }
+    if (forced_row_tiles >= 1 && forced_row_tiles <= most)
+        row_tiles = forced_row_tiles;
 #define CAMBLAS_MX(NT, MT) launch_one<PACKED, GROUPED, NT, MT>(stream, p, groups)
     switch (token_tiles * 10 + row_tiles) {
     case 11: return CAMBLAS_MX(1, 1);
@@ -466,8 +470,8 @@ hipError_t launch_mx_matmul(hipStream_t stream, int kernel, int compute_units, b
     if ((rows + 15) / 16 > 65535 || groups > 65535)
         return hipErrorInvalidValue;
     if (groups == 0)
-        return packed ? launch_shape<true, false>(stream, p, 1) : launch_shape<false, false>(stream, p, 1);
-    return packed ? launch_shape<true, true>(stream, p, groups)
-                  : launch_shape<false, true>(stream, p, groups);
+        return packed ? launch_shape<true, false>(stream, p, 1, kernel) : launch_shape<false, false>(stream, p, 1, kernel);
+    return packed ? launch_shape<true, true>(stream, p, groups, kernel)
+                  : launch_shape<false, true>(stream, p, groups, kernel);
 }
 } // namespace camblas_hip
