@@ -451,3 +451,53 @@ def test_streaming_kernel_with_k_divided_over_workgroups(device, n_out, m_rows, 
     got2d = first.reshape(m_rows, ldc)
     assert rel_frobenius(oracle.bf16_to_f32(got2d[:, :n_out]), want64.reshape(m_rows, n_out)) <= TOLERANCE
     assert np.array_equal(got2d[:, n_out:], c0.reshape(m_rows, ldc)[:, n_out:])
+
+
+def test_divided_k_linear_under_graph_capture(device):
+    # a down-projection-shaped linear ([8192, 8192] weights, 32 tokens) takes the divided-K route of
+    # the streaming kernel. Captured after a warm-up it must replay bit-equal to the eager result
+    # (the arrival counters are back at zero after every launch); captured on a context that has
+    # never run it, the planes and counters cannot be made during the capture and the undivided
+    # kernel must run instead, counted as a fallback, with the same answer to the BF16 bar.
+    outputs, tokens, inner = 8192, 32, 8192
+    assert "k_shares=2" in _native.plan_describe(2, "T", "N", outputs, tokens, inner, inner, inner, outputs)[1]
+    generator = torch.Generator(device=device).manual_seed(77)
+    w = (torch.randn((outputs, inner), device=device, generator=generator) * 0.02).to(torch.bfloat16)
+    x = torch.randn((tokens, inner), device=device, generator=generator).to(torch.bfloat16)
+    eager = _kernels.matmul(x, w.t())
+    torch.cuda.synchronize()
+    rows = torch.arange(0, outputs, 251, device=device)
+    want = x.double() @ w[rows].double().t()
+    assert float((eager[:, rows].double() - want).norm() / want.norm()) <= TOLERANCE
+
+    warm = torch.cuda.Stream()
+    warm.wait_stream(torch.cuda.current_stream())
+    out = torch.empty_like(eager)
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.stream(warm):
+        _kernels.matmul(x, w.t(), out=out)  # this stream's context makes its planes and counters
+        warm.synchronize()
+        with torch.cuda.graph(graph, stream=warm):
+            _kernels.matmul(x, w.t(), out=out)
+    for _ in range(3):
+        out.zero_()
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(out, eager)
+    graph.reset()
+
+    cold = torch.cuda.Stream()
+    cold.wait_stream(torch.cuda.current_stream())
+    small = torch.ones((4, 64), device=device, dtype=torch.bfloat16)
+    with torch.cuda.stream(cold):
+        _kernels.matmul(small, small.t())  # creates the context of this stream, nothing more
+        cold.synchronize()
+        before = _native.stats(device)["guard_fallback"]
+        with torch.cuda.graph(graph, stream=cold):
+            _kernels.matmul(x, w.t(), out=out)
+        assert _native.stats(device)["guard_fallback"] == before + 1
+    out.zero_()
+    graph.replay()
+    torch.cuda.synchronize()
+    assert float((out.double() - eager.double()).norm() / eager.double().norm()) <= 4e-3
+    graph.reset()
