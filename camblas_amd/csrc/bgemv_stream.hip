@@ -40,18 +40,6 @@ struct StreamParams {
 
 constexpr int WAVES = 4, DEPTH = 2;
 
-// 16 bytes per lane written to / read from the point of coherence of the whole device (cache
-// policy bit 4, "sc1": device scope on gfx950), byte offset inside a buffer resource. Kept out of
-// the kernel template: the host pass drops a template instantiation that meets a target builtin.
-__device__ __forceinline__ void store_device_scope(__amdgpu_buffer_rsrc_t resource, unsigned offset, f32x4_t value)
-{
-    __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(u32x4_t, value), resource, int(offset), 0, 0x10);
-}
-__device__ __forceinline__ f32x4_t load_device_scope(__amdgpu_buffer_rsrc_t resource, unsigned offset)
-{
-    return __builtin_bit_cast(f32x4_t, __builtin_amdgcn_raw_buffer_load_b128(resource, int(offset), 0, 0x10));
-}
-
 // NT, MT: 16-row weight tiles and 16-token tiles per workgroup; a K step is KT blocks of 32*WAVES
 // elements, each block split over the WAVES wavefronts; DEPTH K steps are in flight in registers.
 //

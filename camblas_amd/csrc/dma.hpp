@@ -48,6 +48,22 @@ __device__ __forceinline__ __amdgpu_buffer_rsrc_t make_resource(const void *base
     return __builtin_amdgcn_make_buffer_rsrc(const_cast<void *>(base), 0, int(bytes), 0x00020000);
 }
 
+// 16 bytes per lane written to / read from the point of coherence of the whole device (cache
+// policy bit 4, "sc1": device scope on gfx950) at a byte offset inside a buffer resource. Data that
+// workgroups on different XCDs hand to each other travels this way, because an ordinary store
+// stays in the writer's XCD-local L2 until a release fence writes that whole cache back (and the
+// reader needs an acquire fence that invalidates its own): measured +20 to +40 us per launch.
+// Kept out of kernel templates: the host pass drops a template instantiation that meets a target
+// builtin.
+__device__ __forceinline__ void store_device_scope(__amdgpu_buffer_rsrc_t resource, unsigned offset, f32x4_t value)
+{
+    __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(u32x4_t, value), resource, int(offset), 0, 0x10);
+}
+__device__ __forceinline__ f32x4_t load_device_scope(__amdgpu_buffer_rsrc_t resource, unsigned offset)
+{
+    return __builtin_bit_cast(f32x4_t, __builtin_amdgcn_raw_buffer_load_b128(resource, int(offset), 0, 0x10));
+}
+
 // s_waitcnt vmcnt(N) with the other counters left alone (gfx9 encoding: vmcnt in bits 3:0 and
 // 15:14, expcnt 6:4, lgkmcnt 11:8).
 template <int N> __device__ __forceinline__ void wait_loads()
