@@ -149,6 +149,31 @@ def test_fp8_block_linear_18432x7168(device, fp8_weights, tokens):
     assert torch.equal(result[: tokens - 1].view(torch.int16), out[: tokens - 1].view(torch.int16))
 
 
+@pytest.mark.parametrize("tokens", [16, 4096])
+def test_fp8_block_linear_on_the_distribution_the_configuration_states(device, tokens):
+    # the configuration's own draw: x ~ N(0, 1) in BF16, quantised by the library's dynamic 1 x 128
+    # quantiser; W ~ N(0, 0.02) quantised per 128 x 128 block to E4M3 with scale = amax / 448 (here
+    # with PyTorch's own cast, an independent codec). Checked twice: against the FP64 product of the
+    # dequantised operands (the kernel's own bar) and against the FP64 product of the unquantised
+    # operands, where only the quantisation error of two 3-bit mantissas remains (about 4 %).
+    outputs, inner = 18432, 7168
+    x = bf16_normal((tokens, inner), 1.0, 9400 + tokens, device)
+    w32 = bf16_normal((outputs, inner), 0.02, 9401, device).float()
+    blocks = w32.view(outputs // 128, 128, inner // 128, 128)
+    w_scale = (blocks.abs().amax(dim=(1, 3)) / 448.0).clamp_min(1e-12)
+    w = (blocks / w_scale[:, None, :, None]).clamp(-448, 448).view(outputs, inner).to(torch.float8_e4m3fn)
+    q, a_scale = _kernels.fp8_quantise_1x128(x)
+    out = _kernels.fp8_block_matmul(q, a_scale, w, w_scale)
+    assert torch.equal(out, _kernels.fp8_block_linear(x, w, w_scale))
+    picked = sample(4, tokens, 5, seams=(128, 256))
+    index = torch.from_numpy(picked).to(device)
+    want = oracle.fp8_block_matmul_f64(from_device_fp8(q[index]), a_scale[index].cpu().numpy(),
+                                       from_device_fp8(w), w_scale.cpu().numpy())
+    close_to(bf16_values(out[index]), want)
+    unquantised = (x[index].double() @ w32.double().t()).cpu().numpy()
+    assert rel_frobenius(bf16_values(out[index]), unquantised) <= 6e-2
+
+
 def test_decoder_layer_decode_llama70b_shape(device):
     # the oracle pipeline of the reduced-size layer test, at the size the benchmark runs
     from test_gpu_layer import device_layer, oracle_layer
