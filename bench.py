@@ -207,7 +207,7 @@ def main():
     parser.add_argument("--skip-traffic", action="store_true", help="do not run the rocprofv3 counter passes")
     parser.add_argument("--only", choices=("decode1", "decode8", "decode32", "prefill", "prefillnn", "copy", "traffic",
                                  "fp8m1", "fp8m16", "fp8m256", "fp8m4096", "fp8block32", "mxe4m3m16", "mxe2m1m16",
-                                 "mxe4m3m4096", "mxe2m1m4096", "fp8moe", "attention", "layer", "sgemm2048"),
+                                 "mxe4m3m4096", "mxe2m1m4096", "fp8moe", "attention", "layer", "layergraph", "sgemm2048"),
                         help="profiling aid: launch just this kernel --steps times, print nothing")
     args = parser.parse_args()
     if args.gpus != 1:
@@ -461,6 +461,20 @@ def profile_only(args, torch, _kernels, _native, device, normal, weights, inputs
     elif args.only in ("attention", "layer"):
         layer, attention = layer_step(torch, _kernels, device, normal)
         launch = (lambda i: layer()) if args.only == "layer" else (lambda i: attention())
+    elif args.only == "layergraph":  # the layer step replayed from a one-step graph
+        layer, _ = layer_step(torch, _kernels, device, normal)
+        side = torch.cuda.Stream()
+        side.wait_stream(torch.cuda.current_stream())
+        with torch.cuda.stream(side):
+            layer()
+        torch.cuda.current_stream().wait_stream(side)
+        torch.cuda.synchronize()
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph, stream=side):
+            layer()
+
+        def launch(i):
+            graph.replay()
     else:
         tokens, features = 4096, 10240
         x, w = normal((tokens, INNER)), normal((features, INNER), 0.02)
@@ -771,7 +785,7 @@ def extras(torch, _kernels, _native, device, normal):
     graph = torch.cuda.CUDAGraph()
     with torch.cuda.graph(graph, stream=side):
         layer(0)
-    replayed = event_time(torch, lambda i: graph.replay(), 3, 20)
+    replayed = event_time(torch, lambda i: graph.replay(), 20, 100)
     # a model replays all of its layers from one graph: eight steps in one graph show how much of a
     # replay is paid per launch of a graph rather than per kernel in it
     layers = 8
@@ -779,7 +793,7 @@ def extras(torch, _kernels, _native, device, normal):
     with torch.cuda.graph(stack, stream=side):
         for _ in range(layers):
             layer(0)
-    stacked = event_time(torch, lambda i: stack.replay(), 2, 10) / layers
+    stacked = event_time(torch, lambda i: stack.replay(), 5, 20) / layers
     traffic = LAYER_BYTES
     seconds = event_time(torch, lambda i: attention(), 3, 20)
     found["gqa_decode_attention_b32_ctx2048"] = {
