@@ -501,3 +501,24 @@ def test_divided_k_linear_under_graph_capture(device):
     torch.cuda.synchronize()
     assert float((out.double() - eager.double()).norm() / eager.double().norm()) <= 4e-3
     graph.reset()
+
+
+def test_divided_k_result_does_not_depend_on_arrival_order(device):
+    # the down projection of the 70B layer, two hundred launches on the same operands: whichever
+    # workgroup of a tile arrives last, the planes are added in index order, so every launch must
+    # reproduce the first bit for bit (and the counters must have returned to zero each time)
+    outputs, tokens, inner = 8192, 32, 28672
+    assert "k_shares=2" in _native.plan_describe(2, "T", "N", outputs, tokens, inner, inner, inner, outputs)[1]
+    generator = torch.Generator(device=device).manual_seed(78)
+    w = (torch.randn((outputs, inner), device=device, generator=generator) * 0.02).to(torch.bfloat16)
+    x = torch.randn((tokens, inner), device=device, generator=generator).to(torch.bfloat16)
+    first = _kernels.matmul(x, w.t())
+    out = torch.empty_like(first)
+    mismatches = 0
+    for _ in range(200):
+        _kernels.matmul(x, w.t(), out=out)
+        mismatches += int(not torch.equal(out, first))
+    assert mismatches == 0
+    rows = torch.arange(0, outputs, 257, device=device)
+    want = x.double() @ w[rows].double().t()
+    assert float((first[:, rows].double() - want).norm() / want.norm()) <= TOLERANCE
