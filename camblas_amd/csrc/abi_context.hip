@@ -54,9 +54,10 @@ hipError_t reserve_scratch(camblas_cuda_context *context, size_t bytes)
         return status;
     }
     if (context->scratch) {
-        if (context->seen_capture || hipStreamSynchronize(context->stream) != hipSuccess)
+        if (context->seen_capture || hipStreamSynchronize(context->stream) != hipSuccess) {
             context->retired.push_back(context->scratch);
-        else
+            context->retired_bytes += context->scratch_bytes;
+        } else
             (void)hipFree(context->scratch);
     }
     context->scratch = arena;

@@ -20,6 +20,7 @@ struct camblas_cuda_context {
     void *scratch = nullptr;       // split-K partials, attention partials
     size_t scratch_bytes = 0;
     std::vector<void *> retired;   // superseded scratch kept alive for captured graphs
+    size_t retired_bytes = 0;      // what those arenas hold together
     bool seen_capture = false;     // the arena has been used by a launch under stream capture
     unsigned *arrivals = nullptr;  // zeroed counters of the divided-K streaming kernel (made on first use)
     int override_kernel = -1;      // diagnostics: forced kernel variant

@@ -165,8 +165,9 @@ int strassen_gemm(camblas_cuda_context *context, int levels, int n, T alpha, con
         return STRASSEN_NOT_ELIGIBLE;
 
     // scratch for L levels; an allocation failure drops a level (counted once as a guard fallback).
-    // The default policy was not asked for by name, so it never grows the scratch beyond 16 GiB:
-    // it drops levels, or leaves the product to the ordinary kernel, without counting anything.
+    // The default policy was not asked for by name, so it never grows the scratch beyond 16 GiB
+    // (arenas kept alive for captured graphs included): it drops levels, or leaves the product to
+    // the ordinary kernel, without counting anything.
     constexpr size_t DEFAULT_POLICY_LIMIT = size_t(16) << 30;
     bool counted = false;
     size_t leaves = 0, leaf_elements = 0, spare_elements = 0;
@@ -183,7 +184,8 @@ int strassen_gemm(camblas_cuda_context *context, int levels, int n, T alpha, con
         leaf_elements = leaves * leaf * leaf;
         spare_elements = levels > 1 ? power_of_seven(levels - 1) * (2 * leaf) * (2 * leaf) : 0;
         const size_t bytes = FLAG_BYTES + (3 * leaf_elements + spare_elements) * sizeof(T);
-        if (context->algorithm == CAMBLAS_CUDA_AUTO && bytes > DEFAULT_POLICY_LIMIT)
+        if (context->algorithm == CAMBLAS_CUDA_AUTO && bytes > context->scratch_bytes &&
+            bytes + context->retired_bytes > DEFAULT_POLICY_LIMIT)
             continue;
         const hipError_t status = reserve_scratch(context, bytes);
         if (status == hipSuccess)
