@@ -92,9 +92,30 @@ def test_bf16_prefill_linear_4096x10240x8192(device):
     out = _kernels.matmul(x, w.t(), out=c.clone(), alpha=1.0, beta=1.0)
     want = want + bf16_values(c[index]).astype(np.float64)
     close_to(bf16_values(out[index]), want)
+    # the addend read by the epilogue instead of first being cloned into the output: a full matrix
+    # must reproduce the in-place form bit for bit, a bias row must hold the FP64 bar
+    assert torch.equal(_kernels.addmm(c, x, w.t(), beta=1.0), out)
+    row = bf16_normal((10240,), 1.0, 9104, device)
+    biased = _kernels.addmm(row, x, w.t(), beta=1.0)
+    close_to(bf16_values(biased[index]), want - bf16_values(c[index]).astype(np.float64) + bf16_values(row).astype(np.float64))
     # the same tokens as a small batch through the decode kernel agree to rounding
     small = _kernels.linear(x[index[:8]].contiguous(), w)
     assert rel_frobenius(bf16_values(small), bf16_values(y[index[:8]]).astype(np.float64)) <= 1e-2
+
+
+def test_bf16_row_major_product_4096_cubed(device):
+    # torch.mm(a, b) with a contiguous right operand ('N','N' through the ABI): the operand that is
+    # not K-contiguous is transposed into the arena and the product runs on the linear-layer tiles.
+    # Sampled rows against FP64; the transposed view of the same data ('T','N' directly, no copy)
+    # must give the same bits, since the same kernel then multiplies the same K-contiguous rows.
+    a = bf16_normal((4096, 4096), 1.0, 9110, device)
+    b = bf16_normal((4096, 4096), 0.02, 9111, device)
+    y = _kernels.matmul(a, b)
+    rows = sample(10, 4096, 4, seams=(256, 2048))
+    index = torch.from_numpy(rows).to(device)
+    want = (a[index].double() @ b.double()).cpu().numpy()
+    close_to(bf16_values(y[index]), want)
+    assert torch.equal(_kernels.matmul(a, b.t().contiguous().t()), y)
 
 
 @pytest.fixture(scope="module")
