@@ -1,7 +1,7 @@
 """What the library does when hipMalloc fails (ref: tests/test_cuda.py:124-226 with its
 tests/cuda_fail_alloc.c, and the fallback logic of src/cuda/backend.cu:470-485).
 
-A preloaded interposer (tests/support/fail_next_hipmalloc.c, compiled here with cc) makes exactly
+A preloaded interposer (tests/support/fail_next_hipmalloc.c, compiled by the build step or here with cc) makes exactly
 one hipMalloc return hipErrorOutOfMemory on demand. It runs in a child process of its own; no
 kernel misbehaves, an API call returns an error code. Routes covered:
   * scratch growth of an entry point that cannot do without it (dense attention): status -2, the
@@ -106,12 +106,15 @@ print("allocation failure routes ok")
 
 
 def test_allocation_failure_routes(tmp_path):
-    compiler = shutil.which("cc") or shutil.which("gcc")
-    if not compiler:
-        pytest.skip("no C compiler for the interposer")
-    shim = tmp_path / "fail_next_hipmalloc.so"
-    subprocess.run([compiler, "-shared", "-fPIC", str(ROOT / "tests/support/fail_next_hipmalloc.c"), "-ldl",
-                    "-o", str(shim)], check=True, capture_output=True, text=True)
+    # the build step leaves the interposer beside its source; without that it is compiled here
+    shim = ROOT / "tests/support/fail_next_hipmalloc.so"
+    if not shim.is_file():
+        compiler = shutil.which("cc") or shutil.which("gcc")
+        if not compiler:
+            pytest.skip("no C compiler for the interposer")
+        shim = tmp_path / "fail_next_hipmalloc.so"
+        subprocess.run([compiler, "-shared", "-fPIC", str(ROOT / "tests/support/fail_next_hipmalloc.c"), "-ldl",
+                        "-o", str(shim)], check=True, capture_output=True, text=True)
     environment = dict(os.environ)
     # ours goes in front of whatever is preloaded already; nothing is removed
     existing = environment.get("LD_PRELOAD", "")
