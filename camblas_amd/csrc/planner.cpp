@@ -155,11 +155,21 @@ Plan make_plan(int dtype, int algorithm, bool trans_a, bool trans_b, int m, int 
                 plan.kernel = 10 * wider + token_tiles;
                 plan.split_k = 2;
             }
+        } else if (tokens <= 64 && k >= 8192 &&
+                   ceil_div(2 * ceil_div(outputs, 16), compute_units) >= (tokens >= 40 ? 5 : 6)) {
+            // 33..64 tokens on a projection of 10240 to 16384 rows: the streaming kernel with K
+            // divided over two workgroups per tile and 80 to 128 rows each (one workgroup per
+            // compute unit) beats the register-staged tiles below by 15-25 % from 12288 rows on
+            // (measured: [12288, 8192] 46-48 vs 55-58 us, [16384, 8192] 58-59 vs 71-74,
+            // [12288, 16384] 79-81 vs 100-106) and from 40 tokens at 10240 rows (40-41 vs 43-48)
+            plan.family = FAMILY_STREAM;
+            plan.kernel = 10 * std::min(8, ceil_div(2 * ceil_div(outputs, 16), compute_units)) + 4;
+            plan.split_k = 2;
         } else if (tokens <= 64) {
-            // 33..64 tokens on a narrow projection: the streaming kernel would have 32-48 weight
-            // rows per workgroup and re-read as many token rows through L2; 128 x 64 register-staged
-            // tiles with K divided over up to 2.5 workgroups per compute unit are 15-30 % faster
-            // (measured: [8192, 28672] 89-98 vs 118-137 us, [8192, 8192] 29-32 vs 36-40 us)
+            // 33..64 tokens on a narrow projection: the undivided streaming kernel would have 32-48
+            // weight rows per workgroup and re-read as many token rows through L2; 128 x 64
+            // register-staged tiles with K divided over up to 2.5 workgroups per compute unit are
+            // 15-30 % faster (measured: [8192, 28672] 89-98 vs 118-137 us, [8192, 8192] 29-32 vs 36-40 us)
             plan.kernel = 3;
             const int tiles = ceil_div(outputs, 128);
             plan.split_k = 1;

@@ -522,3 +522,22 @@ def test_divided_k_result_does_not_depend_on_arrival_order(device):
     rows = torch.arange(0, outputs, 257, device=device)
     want = x.double() @ w[rows].double().t()
     assert float((first[:, rows].double() - want).norm() / want.norm()) <= TOLERANCE
+
+
+@pytest.mark.parametrize("outputs,tokens", [(12288, 33), (10240, 48), (16384, 64)])
+def test_mid_width_projection_at_33_to_64_tokens(device, outputs, tokens):
+    # the planner sends these to the streaming kernel with K divided over two workgroups per tile
+    # (four token tiles, 80 to 128 rows per workgroup); sampled output rows against FP64
+    inner = 8192
+    text = _native.plan_describe(2, "T", "N", outputs, tokens, inner, inner, inner, outputs)[1]
+    assert "stream" in text and "tokens=64" in text and "k_shares=2" in text, text
+    generator = torch.Generator(device=device).manual_seed(outputs + tokens)
+    w = (torch.randn((outputs, inner), device=device, generator=generator) * 0.02).to(torch.bfloat16)
+    x = torch.randn((tokens, inner), device=device, generator=generator).to(torch.bfloat16)
+    y = _kernels.matmul(x, w.t())
+    rows = torch.cat([torch.arange(0, outputs, 509, device=device), torch.tensor([outputs - 1], device=device)])
+    want = x.double() @ w[rows].double().t()
+    got = y[:, rows].double()
+    assert float((got - want).norm() / want.norm()) <= TOLERANCE
+    bound = 2.0**-7 * want.abs() + 1e-4 * want.abs().max()
+    assert bool(((got - want).abs() <= bound).all())
