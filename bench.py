@@ -207,7 +207,7 @@ def main():
     parser.add_argument("--skip-traffic", action="store_true", help="do not run the rocprofv3 counter passes")
     parser.add_argument("--only", choices=("decode1", "decode8", "decode32", "prefill", "prefillnn", "copy", "traffic",
                                  "fp8m1", "fp8m16", "fp8m256", "fp8m4096", "fp8block32", "mxe4m3m16", "mxe2m1m16",
-                                 "mxe4m3m4096", "mxe2m1m4096", "fp8moe", "attention", "layer", "layergraph", "sgemm2048"),
+                                 "mxe4m3m4096", "mxe2m1m4096", "fp8moe", "attention", "layer", "layergraph", "sgemm2048", "dgemm4096"),
                         help="profiling aid: launch just this kernel --steps times, print nothing")
     args = parser.parse_args()
     if args.gpus != 1:
@@ -451,6 +451,14 @@ def profile_only(args, torch, _kernels, _native, device, normal, weights, inputs
 
         def launch(i):
             _kernels.matmul(a32, b32, out=c32)
+    elif args.only == "dgemm4096":
+        size = 4096
+        a64 = torch.rand((size, size), device=device, dtype=torch.float64) * 2 - 1
+        b64 = torch.rand((size, size), device=device, dtype=torch.float64) * 2 - 1
+        c64 = torch.empty((size, size), device=device, dtype=torch.float64)
+
+        def launch(i):
+            _kernels.matmul(a64, b64, out=c64)
     elif args.only == "prefillnn":
         size = 4096
         x, w = normal((size, size)), normal((size, size), 0.02)
