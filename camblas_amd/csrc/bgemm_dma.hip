@@ -220,33 +220,65 @@ __global__ __launch_bounds__(128 * WM) void bgemm_dma_kernel(DmaParams p)
     wait_loads<0>(); // drain the padding loads before the LDS is released
 
     // ---- epilogue. Accumulator register 4q+e of lane l is feature 8q + 4*(l/32) + e, token l%32.
-    const bool with_beta = p.beta != 0.f;
-#pragma unroll
-    for (int j = 0; j < TM; ++j) {
+    const int first_feature = n0 + wn * TN * 32 + half * 4;
+    auto store_tile = [&](int i, int j, const u32x2_t (&old)[4], bool with_beta) {
         const int m = m0 + (wm * TM + j) * 32 + frag_row;
-        unsigned short *row = p.y + size_t(m) * p.ldc + n0 + wn * TN * 32 + half * 4;
-        const unsigned short *source = p.z + size_t(m) * p.ldz + n0 + wn * TN * 32 + half * 4;
+        unsigned short *row = p.y + size_t(m) * p.ldc + first_feature;
 #pragma unroll
-        for (int i = 0; i < TN; ++i) {
-            __builtin_amdgcn_sched_barrier(0); // keep one accumulator tile live at a time
-#pragma unroll
-            for (int q = 0; q < 4; ++q) {
-                const int offset = i * 32 + q * 8;
-                if (m < p.m && n0 + wn * TN * 32 + half * 4 + offset < p.n) {
-                    float v0 = p.alpha * acc[i][j][q * 4], v1 = p.alpha * acc[i][j][q * 4 + 1];
-                    float v2 = p.alpha * acc[i][j][q * 4 + 2], v3 = p.alpha * acc[i][j][q * 4 + 3];
-                    if (with_beta) {
-                        u32x2_t old = *reinterpret_cast<const u32x2_t *>(source + offset);
-                        v0 = fmaf(p.beta, __uint_as_float(old[0] << 16), v0);
-                        v1 = fmaf(p.beta, __uint_as_float(old[0] & 0xffff0000u), v1);
-                        v2 = fmaf(p.beta, __uint_as_float(old[1] << 16), v2);
-                        v3 = fmaf(p.beta, __uint_as_float(old[1] & 0xffff0000u), v3);
-                    }
-                    u32x2_t packed = {pack_bf16x2(v0, v1), pack_bf16x2(v2, v3)};
-                    *reinterpret_cast<u32x2_t *>(row + offset) = packed;
+        for (int q = 0; q < 4; ++q) {
+            const int offset = i * 32 + q * 8;
+            if (m < p.m && first_feature + offset < p.n) {
+                float v0 = p.alpha * acc[i][j][q * 4], v1 = p.alpha * acc[i][j][q * 4 + 1];
+                float v2 = p.alpha * acc[i][j][q * 4 + 2], v3 = p.alpha * acc[i][j][q * 4 + 3];
+                if (with_beta) {
+                    v0 = fmaf(p.beta, __uint_as_float(old[q][0] << 16), v0);
+                    v1 = fmaf(p.beta, __uint_as_float(old[q][0] & 0xffff0000u), v1);
+                    v2 = fmaf(p.beta, __uint_as_float(old[q][1] << 16), v2);
+                    v3 = fmaf(p.beta, __uint_as_float(old[q][1] & 0xffff0000u), v3);
                 }
+                u32x2_t packed = {pack_bf16x2(v0, v1), pack_bf16x2(v2, v3)};
+                *reinterpret_cast<u32x2_t *>(row + offset) = packed;
             }
         }
+    };
+    if (p.beta == 0.f) {
+        const u32x2_t nothing[4] = {};
+#pragma unroll
+        for (int j = 0; j < TM; ++j)
+#pragma unroll
+            for (int i = 0; i < TN; ++i) {
+                __builtin_amdgcn_sched_barrier(0); // keep one accumulator tile live at a time
+                store_tile(i, j, nothing, false);
+            }
+        return;
+    }
+    // beta term: the addend of tile t + 1 is fetched while tile t is scaled and stored (one load
+    // latency per tile would otherwise be exposed twenty times: measured +56 us on a 506 us product,
+    // +29 us with the fetch one tile ahead, no better two tiles ahead). The loads are unconditional: a
+    // position outside the matrix reads the first element of a valid row instead and is not used.
+    constexpr int AHEAD = 1;
+    u32x2_t old[AHEAD + 1][4];
+    auto fetch_tile = [&](int t, u32x2_t (&into)[4]) {
+        const int i = t % TN, j = t / TN;
+        int m = m0 + (wm * TM + j) * 32 + frag_row;
+        m = m < p.m ? m : p.m - 1;
+        const unsigned short *source = p.z + size_t(m) * p.ldz;
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+            const int feature = first_feature + i * 32 + q * 8;
+            into[q] = *reinterpret_cast<const u32x2_t *>(source + (feature < p.n ? feature : 0));
+        }
+    };
+#pragma unroll
+    for (int t = 0; t < AHEAD && t < TN * TM; ++t)
+        fetch_tile(t, old[t]);
+#pragma unroll
+    for (int t = 0; t < TN * TM; ++t) {
+        __builtin_amdgcn_sched_barrier(0);
+        if (t + AHEAD < TN * TM)
+            fetch_tile(t + AHEAD, old[(t + AHEAD) % (AHEAD + 1)]);
+        __builtin_amdgcn_sched_barrier(0);
+        store_tile(t % TN, t / TN, old[t % (AHEAD + 1)], true);
     }
 }
 
