@@ -64,6 +64,68 @@ __device__ __forceinline__ f32x4_t load_device_scope(__amdgpu_buffer_rsrc_t reso
     return __builtin_bit_cast(f32x4_t, __builtin_amdgcn_raw_buffer_load_b128(resource, int(offset), 0, 0x10));
 }
 
+// The same two loads outside the compiler's bookkeeping of memory operations (it then neither
+// counts them nor makes later LDS reads wait for them): for data that is read with
+// lds_read_unordered after a wait the caller places. M0 is put back as it was. The loads still
+// count in vmcnt, which only makes waits the compiler computes for its own loads stricter.
+__device__ __forceinline__ void load_to_lds_untracked(__amdgpu_buffer_rsrc_t resource, unsigned lane_offset,
+                                                      unsigned step_offset, const void *lds_base)
+{
+    const unsigned address = __builtin_amdgcn_readfirstlane(static_cast<unsigned>(reinterpret_cast<uintptr_t>(lds_base)));
+    unsigned saved;
+    asm volatile("s_mov_b32 %0, m0\n\ts_mov_b32 m0, %1\n\ts_nop 0\n\t"
+                 "buffer_load_dwordx4 %2, %3, %4 offen lds\n\ts_mov_b32 m0, %0"
+                 : "=&s"(saved)
+                 : "s"(address), "v"(lane_offset), "s"(resource), "s"(step_offset)
+                 : "memory");
+}
+__device__ __forceinline__ void load_word_to_lds_untracked(__amdgpu_buffer_rsrc_t resource, unsigned lane_offset,
+                                                           unsigned step_offset, const void *lds_base)
+{
+    const unsigned address = __builtin_amdgcn_readfirstlane(static_cast<unsigned>(reinterpret_cast<uintptr_t>(lds_base)));
+    unsigned saved;
+    asm volatile("s_mov_b32 %0, m0\n\ts_mov_b32 m0, %1\n\ts_nop 0\n\t"
+                 "buffer_load_dword %2, %3, %4 offen lds\n\ts_mov_b32 m0, %0"
+                 : "=&s"(saved)
+                 : "s"(address), "v"(lane_offset), "s"(resource), "s"(step_offset)
+                 : "memory");
+}
+
+// One float from LDS, outside the compiler's bookkeeping of memory operations: it neither waits for
+// outstanding direct-to-LDS loads before the read nor for the read before the value is used. The
+// caller orders both: the data was complete at an earlier barrier, and an s_waitcnt lgkmcnt(0)
+// (pipeline_barrier has one) followed by tie_after_wait lies between this read and the first use;
+// keep the two a few instructions apart, so that the register is not copied or spilled in between.
+__device__ __forceinline__ float lds_read_unordered(const float *address)
+{
+    float value;
+    asm volatile("ds_read_b32 %0, %1" : "=v"(value) : "v"(static_cast<unsigned>(reinterpret_cast<uintptr_t>(address))));
+    return value;
+}
+// Placed right after the wait that covers lds_read_unordered results: no use of the values can
+// move above this point.
+template <int A, int B> __device__ __forceinline__ void tie_after_wait(float (&first)[A], float (&second)[B])
+{
+#pragma unroll
+    for (int i = 0; i < A; ++i)
+        asm volatile("" : "+v"(first[i]));
+#pragma unroll
+    for (int i = 0; i < B; ++i)
+        asm volatile("" : "+v"(second[i]));
+}
+
+// p[index] for a pointer that is the same in every lane of the wavefront (the caller's promise),
+// read-only for the whole launch: a scalar load, which leaves the vector memory counter and the
+// path into the compute unit's vector cache alone.
+__device__ __forceinline__ float uniform_load(const float *p, int index)
+{
+    typedef const __attribute__((address_space(4))) float *constant_pointer;
+    const uintptr_t address = reinterpret_cast<uintptr_t>(p);
+    const unsigned low = __builtin_amdgcn_readfirstlane(unsigned(address));
+    const unsigned high = __builtin_amdgcn_readfirstlane(unsigned(address >> 32));
+    return reinterpret_cast<constant_pointer>((uintptr_t(high) << 32) | low)[index];
+}
+
 // s_waitcnt vmcnt(N) with the other counters left alone (gfx9 encoding: vmcnt in bits 3:0 and
 // 15:14, expcnt 6:4, lgkmcnt 11:8).
 template <int N> __device__ __forceinline__ void wait_loads()

@@ -14,8 +14,9 @@
 // loads). A group's dot product is two
 // v_mfma_scale_f32_32x32x64_f8f6f4 (unit hardware scales) into a zeroed temporary; the scaled
 // accumulate of one 32x32 tile runs on the vector ALU while the matrix cores work on the next tile.
-// The weight scale of a group (one per wavefront: its 128 rows lie in one scale block) and the
-// activation scales (one per lane and token tile) are 4-byte loads fetched a group ahead.
+// The scales reach the lanes through LDS as well: slabs of eight groups per token (and per weight
+// block) are copied in with direct-to-LDS loads once per round of six or eight groups, and a lane
+// reads the next group's scales from there at the end of a step.
 #include "common.hpp"
 #include "device.hpp"
 #include "dma.hpp"
@@ -51,7 +52,11 @@ __global__ __launch_bounds__(128 * WM) void fp8_dma_kernel(Fp8DmaParams p)
     constexpr int A_ITERS = BN / (WAVES * ROWS_PER_LOAD), B_ITERS = BM / (WAVES * ROWS_PER_LOAD);
     constexpr int SLOTS = (BN + BM) * CH, LOADS = A_ITERS + B_ITERS;
     static_assert(BN % (WAVES * ROWS_PER_LOAD) == 0 && BM % (WAVES * ROWS_PER_LOAD) == 0, "loads");
-    __shared__ u32x4_t stages[STAGES][SLOTS];
+    // Scale slabs (below) behind the stages, in the same array: BM / 32 KB for two buffers of
+    // activation scales, then two buffers of 64 weight scales.
+    constexpr int SLAB_SLOTS = BM / 32 * 64, WEIGHT_SLAB_SLOTS = 16;
+    __shared__ u32x4_t lds[STAGES * SLOTS + 2 * SLAB_SLOTS + 2 * WEIGHT_SLAB_SLOTS];
+    auto stage_at = [&](int index) { return lds + index * SLOTS; };
 
     int tile_n, tile_m;
     xcd_tile(int(blockIdx.x), p.tiles_n, p.tiles_m, tile_n, tile_m);
@@ -96,26 +101,83 @@ __global__ __launch_bounds__(128 * WM) void fp8_dma_kernel(Fp8DmaParams p)
         advance();
     };
 
-    // ---- scales. Weight scales are one value per group and scale block of the wavefront's rows
-    // (every lane loads the same address); activation scales are one per lane
-    // (token = lane % 32) and token tile. Both are loaded one group ahead, unconditionally: a load
-    // under a branch would make the compiler wait for every outstanding load, the LDS fills
-    // included.
+    // ---- scales. The activation scales are one per token and group, rows of `groups` floats per
+    // token. If every lane fetched its token's scale of the next group into a register (a cache
+    // line per lane, the same line again for each of the 32 groups it holds), the kernel would lose
+    // 6 % at 4096 tokens and 16 % at 256 (measured). Instead each wavefront copies, once per PERIOD
+    // groups, 16 bytes per lane (four consecutive groups of a token, the two lanes of a token side
+    // by side in memory) straight into LDS: lane l of loader w holds groups 4 * (l / 32) .. + 3 of
+    // the slab for token 32 * w + l % 32, and a lane reads its tokens' scales from there (tokens 16
+    // apart share a bank: two-way at worst). Slab number i holds SLAB_GROUPS groups from group
+    // i * PERIOD of this workgroup's share on (PERIOD: the largest multiple of STAGES within
+    // SLAB_GROUPS, so that a slab begins where a round of stages begins) and is loaded when slab
+    // i - 1 comes into use, into the buffer that slab i - 2 has left.
+    // Both the slab loads and the reads are kept out of the compiler's bookkeeping
+    // (load_to_lds_untracked, lds_read_unordered): when it sees an LDS read that a direct-to-LDS
+    // load might have written, it waits for every outstanding load, the stage fills included, in
+    // the middle of a step, which cost all of the gain. The order is by construction: a slab load
+    // is older than the fills of the step that follows, so that step's wait covers it PERIOD - 1
+    // steps before the slab is first read; a read is issued a few instructions before the step's
+    // wait and its value is used after it.
     const int frag_row = lane % 32, half = lane / 32;
-    const float *ws_row[WS];
-#pragma unroll
-    for (int s = 0; s < WS; ++s) {
-        int block = (n0 + wn * TN * 32 + s * 32) / 128;
-        block = block < p.scale_blocks ? block : p.scale_blocks - 1;
-        ws_row[s] = p.w_scale + size_t(block) * p.groups + first_group;
-    }
-    const float *as_ptr[TM];
+    constexpr int LANES_PER_TOKEN = 2, SLAB_GROUPS = 4 * LANES_PER_TOKEN;
+    constexpr int TOKENS_PER_WAVE = 64 / LANES_PER_TOKEN, LOADERS = BM / TOKENS_PER_WAVE;
+    constexpr int PERIOD = SLAB_GROUPS / STAGES * STAGES;
+    // (with 32 tokens per wavefront tile and one token tile per wavefront, two wavefronts load the
+    // same piece: same bytes to the same place)
+    static_assert(WAVES % LOADERS == 0 && PERIOD >= 3, "every wavefront loads one piece of a slab");
+    static_assert(LOADERS * 64 == SLAB_SLOTS, "slab size");
+    auto slab_at = [&](int index) { return lds + STAGES * SLOTS + (index & 1) * SLAB_SLOTS; };
+    const int loader = __builtin_amdgcn_readfirstlane(wave) % LOADERS;
+    const __amdgpu_buffer_rsrc_t scale_resource =
+        make_resource(p.a_scale + size_t(m0) * p.groups, unsigned(b_rows) * unsigned(p.groups) * 4u);
+    const int slab_token = loader * TOKENS_PER_WAVE + lane % TOKENS_PER_WAVE;
+    const unsigned slab_lane_off =
+        (unsigned(slab_token < b_rows ? slab_token : b_rows - 1) * unsigned(p.groups) +
+         unsigned(lane / TOKENS_PER_WAVE) * 4u) * 4u;
+    // bytes past the end of the scales read as zero and are never used
+    auto load_slab = [&](int slab) {
+        load_to_lds_untracked(scale_resource, slab_lane_off, unsigned(first_group + slab * PERIOD) * 4u,
+                              slab_at(slab) + loader * 64);
+    };
+    int as_index[TM]; // float index of this lane's token inside a slab buffer (part 0, word 0)
 #pragma unroll
     for (int j = 0; j < TM; ++j) {
-        int m = m0 + (wm * TM + j) * 32 + frag_row;
-        m = m < p.m ? m : p.m - 1;
-        as_ptr[j] = p.a_scale + size_t(m) * p.groups + first_group;
+        const int token = (wm * TM + j) * 32 + frag_row;
+        as_index[j] = ((token / TOKENS_PER_WAVE) * 64 + token % TOKENS_PER_WAVE) * 4;
     }
+    // (read with lds_read_unordered: the compiler would otherwise wait for every outstanding
+    // direct-to-LDS load before a read of memory that such a load may write)
+    auto activation_scale = [&](int j, int group) { // group counted from first_group
+        const float *slab = reinterpret_cast<const float *>(slab_at(group / PERIOD));
+        const int position = group % PERIOD;
+        return lds_read_unordered(slab + as_index[j] + position / 4 * (TOKENS_PER_WAVE * 4) + position % 4);
+    };
+    // The weight scales travel the same way: the tile's rows lie in at most four 128-row blocks,
+    // and lane l of one 4-byte-per-lane load brings group l % 8 of the slab for block l / 8 (every
+    // wavefront issues the same load: same bytes to the same place).
+    static_assert(SLAB_GROUPS == 8 && BN <= 7 * 128, "eight blocks of eight groups per load");
+    auto weight_slab_at = [&](int index) {
+        return reinterpret_cast<float *>(lds + STAGES * SLOTS + 2 * SLAB_SLOTS + (index & 1) * WEIGHT_SLAB_SLOTS);
+    };
+    const int first_block = n0 / 128;
+    const __amdgpu_buffer_rsrc_t weight_scale_resource =
+        make_resource(p.w_scale + size_t(first_block) * p.groups,
+                      unsigned(p.scale_blocks - first_block < 8 ? p.scale_blocks - first_block : 8) *
+                          unsigned(p.groups) * 4u);
+    const unsigned weight_slab_lane_off = (unsigned(lane / 8) * unsigned(p.groups) + unsigned(lane % 8)) * 4u;
+    int ws_index[WS];
+#pragma unroll
+    for (int s = 0; s < WS; ++s)
+        ws_index[s] = ((n0 + wn * TN * 32 + s * 32) / 128 - first_block) * 8;
+    auto weight_scale = [&](int s, int group) { // group counted from first_group
+        return lds_read_unordered(weight_slab_at(group / PERIOD) + ws_index[s] + group % PERIOD);
+    };
+    auto load_slabs = [&](int slab) {
+        load_slab(slab);
+        load_word_to_lds_untracked(weight_scale_resource, weight_slab_lane_off,
+                                   unsigned(first_group + slab * PERIOD) * 4u, weight_slab_at(slab));
+    };
 
     const int frag_swizzle = lds_swizzle<CH>(frag_row);
     const int a_frag_base = (wn * TN * 32 + frag_row) * CH;
@@ -199,53 +261,57 @@ __global__ __launch_bounds__(128 * WM) void fp8_dma_kernel(Fp8DmaParams p)
         __builtin_amdgcn_sched_barrier(0);
     };
 
-    float ws_now[WS], ws_next[WS];
-#pragma unroll
-    for (int s = 0; s < WS; ++s)
-        ws_now[s] = ws_row[s][0];
-    float as_now[TM], as_next[TM];
-#pragma unroll
-    for (int j = 0; j < TM; ++j)
-        as_now[j] = as_ptr[j][0];
+    float ws_now[WS], as_now[TM];
     // One group: start the loads of the group STAGES-1 ahead into the stage that was read last,
-    // multiply the current stage, then wait until only the newest loads are still in flight.
+    // multiply the current stage, read the next group's scales, then wait until only the newest
+    // loads are still in flight (the wait also covers the scale reads).
     auto step = [&](int g, const u32x4_t *current, u32x4_t *fill) {
         const int next = g + 1 < group_count ? g + 1 : group_count - 1;
-#pragma unroll
-        for (int s = 0; s < WS; ++s)
-            ws_next[s] = ws_row[s][next];
-#pragma unroll
-        for (int j = 0; j < TM; ++j)
-            as_next[j] = as_ptr[j][next];
         __builtin_amdgcn_sched_barrier(0);
         multiply(current, fill, as_now, ws_now);
 #pragma unroll
         for (int s = 0; s < WS; ++s)
-            ws_now[s] = ws_next[s];
+            ws_now[s] = weight_scale(s, next);
 #pragma unroll
         for (int j = 0; j < TM; ++j)
-            as_now[j] = as_next[j];
+            as_now[j] = activation_scale(j, next);
         pipeline_barrier<(STAGES - 2) * LOADS>();
+        tie_after_wait(ws_now, as_now);
     };
     // Group g is read from stage g % STAGES while group g + STAGES - 1 is loaded into the stage
     // that was read last.
+    load_slabs(0); // (the oldest loads: complete at the first wait)
 #pragma unroll
     for (int s = 0; s + 1 < STAGES; ++s) {
         __builtin_amdgcn_sched_barrier(0);
-        issue(stages[s]);
+        issue(stage_at(s));
     }
     pipeline_barrier<(STAGES - 2) * LOADS>();
+#pragma unroll
+    for (int s = 0; s < WS; ++s)
+        ws_now[s] = weight_scale(s, 0);
+#pragma unroll
+    for (int j = 0; j < TM; ++j)
+        as_now[j] = activation_scale(j, 0);
+    __builtin_amdgcn_s_waitcnt(0xc07f); // lgkmcnt(0)
+    tie_after_wait(ws_now, as_now);
     // whole rounds of STAGES groups run without a branch between the steps; the remainder follows
     int g = 0;
-    for (; g + STAGES <= group_count; g += STAGES) {
+    for (int slab = 1; g + STAGES <= group_count; ++slab) {
+        // (older than the fills of the step that follows: landed at that step's wait, PERIOD - 1
+        // steps before its first scale is read)
+        load_slabs(slab);
+        const int end = slab * PERIOD < group_count ? slab * PERIOD : group_count;
+        for (; g + STAGES <= end; g += STAGES) {
 #pragma unroll
-        for (int s = 0; s < STAGES; ++s)
-            step(g + s, stages[s], stages[(s + STAGES - 1) % STAGES]);
+            for (int s = 0; s < STAGES; ++s)
+                step(g + s, stage_at(s), stage_at((s + STAGES - 1) % STAGES));
+        }
     }
 #pragma unroll
     for (int s = 0; s + 1 < STAGES; ++s)
         if (g + s < group_count)
-            step(g + s, stages[s], stages[(s + STAGES - 1) % STAGES]);
+            step(g + s, stage_at(s), stage_at((s + STAGES - 1) % STAGES));
     wait_loads<0>();
 
     // ---- epilogue: accumulator register 4q+e of lane l is feature 8q + 4*(l/32) + e, token l%32

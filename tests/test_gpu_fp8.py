@@ -136,6 +136,25 @@ def test_scale_indexing_is_bit_exact(device, override):
     assert np.array_equal(from_device_bf16(out), want)
 
 
+@pytest.mark.parametrize("override", [(code, 1) for code in range(20, 30)] + [(24, 3), (27, 2), (28, 5), (20, 4)])
+def test_scale_indexing_over_many_groups_is_bit_exact(device, override):
+    # the same exact arithmetic over 29 K groups (an odd number: token rows of scales start at
+    # every alignment; several rounds of the kernels' eight-group scale slabs, the last one partial),
+    # with partial tiles of tokens and outputs and a partial last weight-scale block; every
+    # (token, group) and (block, group) scale is a power of two chosen so that a wrong index changes bits
+    rows, outputs, inner = 300, 452, 29 * 128
+    groups, blocks = inner // 128, (outputs + 127) // 128
+    rng = np.random.default_rng(6)
+    small = np.array([0x00, 0x38, 0x40, 0x30, 0xB8, 0xC0], dtype=np.uint8)  # 0, 1, 2, .5, -1, -2
+    a = small[rng.integers(0, len(small), size=(rows, inner))]
+    w = small[rng.integers(0, len(small), size=(outputs, inner))]
+    a_scale = np.exp2(rng.integers(-5, 5, size=(rows, groups))).astype(np.float32)
+    w_scale = np.exp2(-((np.arange(blocks * groups).reshape(blocks, groups) * 5) % 7)).astype(np.float32)
+    out = run(device, a, a_scale, w, w_scale, override=override)
+    want = oracle.fp8_block_matmul(a, a_scale, w, w_scale)
+    assert np.array_equal(from_device_bf16(out), want)
+
+
 def test_known_answer_bytes_and_nan(device):
     rows, outputs, inner = 2, 256, 256
     a = np.full((rows, inner), 0x38, np.uint8)       # 1.0
