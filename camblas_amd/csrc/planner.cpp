@@ -256,29 +256,39 @@ Plan make_plan(int dtype, int algorithm, bool trans_a, bool trans_b, int m, int 
         return plan;
     }
     plan.family = FAMILY_FP8_DMA;
-    if (n <= 128 && ceil_div(m, 256) * 3 <= compute_units && k >= 12 * 128) {
-        // at most one tile of tokens and few tiles of outputs (18432 outputs are 72): three
-        // workgroups share a tile's K groups; measured 40 against 44 us at 96 tokens, 45 against
-        // 48 at 128, and no gain from 256 tokens on
-        plan.kernel = 4;
-        plan.split_k = 3;
-        return plan;
-    }
+    // {256, 192} x {256, 128, 64} tiles, one workgroup per compute unit, the K groups of a tile
+    // divided over up to eight workgroups when the tiles alone leave compute units empty (FP32
+    // planes summed in share order by a second launch). Each choice is priced in microseconds:
+    // rounds of workgroups x K groups per workgroup x the measured time of one group of that tile
+    // with the machine full (18432 x 7168 at 4096 tokens), plus what dividing costs. Checked
+    // against sweeps of every tile and split on [18432, 7168], [7168, 18432], [4096, 7168],
+    // [2048, 7168], [7168, 2048] and [24576, 1536] from 72 to 4096 tokens: the choice is the
+    // measured best or within a few per cent of it (e.g. [7168, 18432] at 256 tokens 60 us with
+    // 256 x 128 tiles in four shares against 98 undivided; [4096, 7168] at 256 tokens 24 against 38).
     const struct {
-        int variant, resident;
-        double weight;
-    } candidates[] = {{0, 1, 1.04}, {8, 1, 1.02}, {4, 1, 1.0}, {7, 1, 0.92}, {6, 1, 0.75}, {9, 1, 0.64}};
-    // {256, 192} x {256, 128, 64} tiles, one workgroup per compute unit. What decides between them
-    // is how full the last round of workgroups is (18432 outputs are 72 tiles of 256 rows or 96 of
-    // 192); the weights are the measured per-flop efficiency of each tile at equal occupancy.
-    double best = -1;
+        int variant;
+        double group_us;
+    } candidates[] = {{0, 2.10}, {8, 1.55}, {4, 1.12}, {7, 0.90}, {6, 0.80}, {9, 0.67}};
+    const int groups = k / 128;
+    double best = 1e30;
     for (const auto &candidate : candidates) {
         const TnVariant &v = fp8_dma_variant(candidate.variant);
-        double score = candidate.weight * occupancy_score(m, n, v.block_n, v.block_m,
-                                                          candidate.resident, compute_units);
-        if (score > best) {
-            best = score;
-            plan.kernel = candidate.variant;
+        const int tiles = ceil_div(m, v.block_n) * ceil_div(n, v.block_m);
+        // shares: as many as keep the grid within one round, at least six groups each
+        const int limit = std::max(1, std::min({8, groups / 6, compute_units / std::max(1, tiles)}));
+        for (int shares = 1; shares <= limit; ++shares) {
+            const int steps = ceil_div(groups, shares);
+            if (shares > 1 && ceil_div(groups, steps) != shares)
+                continue; // (the launcher would use fewer)
+            const double rounds = double(ceil_div(tiles * shares, compute_units));
+            double cost = rounds * steps * candidate.group_us;
+            if (shares > 1) // a second launch, and the planes written and read once
+                cost += 5.0 + 2.0 * shares * double(m) * n * 4.0 / 4.0e6;
+            if (cost < best) {
+                best = cost;
+                plan.kernel = candidate.variant;
+                plan.split_k = shares;
+            }
         }
     }
     return plan;
