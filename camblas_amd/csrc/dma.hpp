@@ -64,30 +64,41 @@ __device__ __forceinline__ f32x4_t load_device_scope(__amdgpu_buffer_rsrc_t reso
     return __builtin_bit_cast(f32x4_t, __builtin_amdgcn_raw_buffer_load_b128(resource, int(offset), 0, 0x10));
 }
 
-// The same two loads outside the compiler's bookkeeping of memory operations (it then neither
-// counts them nor makes later LDS reads wait for them): for data that is read with
+// Raw buffer descriptor (gfx9 V#: base address, stride 0, `bytes` records, 32-bit data) as four
+// words in scalar registers, for the loads below. `base` and `bytes` must be the same in every lane.
+__device__ __forceinline__ u32x4_t uniform_descriptor(const void *base, unsigned bytes)
+{
+    const uintptr_t address = reinterpret_cast<uintptr_t>(base);
+    return u32x4_t{unsigned(__builtin_amdgcn_readfirstlane(unsigned(address))),
+                   unsigned(__builtin_amdgcn_readfirstlane(unsigned(address >> 32) & 0xffffu)),
+                   unsigned(__builtin_amdgcn_readfirstlane(bytes)), 0x00020000u};
+}
+// load_to_lds / load_word_to_lds outside the compiler's bookkeeping of memory operations (it then
+// neither counts them nor makes later LDS reads wait for them): for data that is read with
 // lds_read_unordered after a wait the caller places. M0 is put back as it was. The loads still
 // count in vmcnt, which only makes waits the compiler computes for its own loads stricter.
-__device__ __forceinline__ void load_to_lds_untracked(__amdgpu_buffer_rsrc_t resource, unsigned lane_offset,
+__device__ __forceinline__ void load_to_lds_untracked(u32x4_t descriptor, unsigned lane_offset,
                                                       unsigned step_offset, const void *lds_base)
 {
     const unsigned address = __builtin_amdgcn_readfirstlane(static_cast<unsigned>(reinterpret_cast<uintptr_t>(lds_base)));
+    const unsigned step = __builtin_amdgcn_readfirstlane(step_offset);
     unsigned saved;
     asm volatile("s_mov_b32 %0, m0\n\ts_mov_b32 m0, %1\n\ts_nop 0\n\t"
                  "buffer_load_dwordx4 %2, %3, %4 offen lds\n\ts_mov_b32 m0, %0"
                  : "=&s"(saved)
-                 : "s"(address), "v"(lane_offset), "s"(resource), "s"(step_offset)
+                 : "s"(address), "v"(lane_offset), "s"(descriptor), "s"(step)
                  : "memory");
 }
-__device__ __forceinline__ void load_word_to_lds_untracked(__amdgpu_buffer_rsrc_t resource, unsigned lane_offset,
+__device__ __forceinline__ void load_word_to_lds_untracked(u32x4_t descriptor, unsigned lane_offset,
                                                            unsigned step_offset, const void *lds_base)
 {
     const unsigned address = __builtin_amdgcn_readfirstlane(static_cast<unsigned>(reinterpret_cast<uintptr_t>(lds_base)));
+    const unsigned step = __builtin_amdgcn_readfirstlane(step_offset);
     unsigned saved;
     asm volatile("s_mov_b32 %0, m0\n\ts_mov_b32 m0, %1\n\ts_nop 0\n\t"
                  "buffer_load_dword %2, %3, %4 offen lds\n\ts_mov_b32 m0, %0"
                  : "=&s"(saved)
-                 : "s"(address), "v"(lane_offset), "s"(resource), "s"(step_offset)
+                 : "s"(address), "v"(lane_offset), "s"(descriptor), "s"(step)
                  : "memory");
 }
 
@@ -96,15 +107,16 @@ __device__ __forceinline__ void load_word_to_lds_untracked(__amdgpu_buffer_rsrc_
 // caller orders both: the data was complete at an earlier barrier, and an s_waitcnt lgkmcnt(0)
 // (pipeline_barrier has one) followed by tie_after_wait lies between this read and the first use;
 // keep the two a few instructions apart, so that the register is not copied or spilled in between.
-__device__ __forceinline__ float lds_read_unordered(const float *address)
+template <typename T> __device__ __forceinline__ T lds_read_unordered(const T *address)
 {
-    float value;
+    static_assert(sizeof(T) == 4, "one 32-bit LDS read");
+    T value;
     asm volatile("ds_read_b32 %0, %1" : "=v"(value) : "v"(static_cast<unsigned>(reinterpret_cast<uintptr_t>(address))));
     return value;
 }
 // Placed right after the wait that covers lds_read_unordered results: no use of the values can
 // move above this point.
-template <int A, int B> __device__ __forceinline__ void tie_after_wait(float (&first)[A], float (&second)[B])
+template <typename T, int A, int B> __device__ __forceinline__ void tie_after_wait(T (&first)[A], T (&second)[B])
 {
 #pragma unroll
     for (int i = 0; i < A; ++i)

@@ -129,8 +129,8 @@ __global__ __launch_bounds__(128 * WM) void fp8_dma_kernel(Fp8DmaParams p)
     static_assert(LOADERS * 64 == SLAB_SLOTS, "slab size");
     auto slab_at = [&](int index) { return lds + STAGES * SLOTS + (index & 1) * SLAB_SLOTS; };
     const int loader = __builtin_amdgcn_readfirstlane(wave) % LOADERS;
-    const __amdgpu_buffer_rsrc_t scale_resource =
-        make_resource(p.a_scale + size_t(m0) * p.groups, unsigned(b_rows) * unsigned(p.groups) * 4u);
+    const u32x4_t scale_resource =
+        uniform_descriptor(p.a_scale + size_t(m0) * p.groups, unsigned(b_rows) * unsigned(p.groups) * 4u);
     const int slab_token = loader * TOKENS_PER_WAVE + lane % TOKENS_PER_WAVE;
     const unsigned slab_lane_off =
         (unsigned(slab_token < b_rows ? slab_token : b_rows - 1) * unsigned(p.groups) +
@@ -161,8 +161,8 @@ __global__ __launch_bounds__(128 * WM) void fp8_dma_kernel(Fp8DmaParams p)
         return reinterpret_cast<float *>(lds + STAGES * SLOTS + 2 * SLAB_SLOTS + (index & 1) * WEIGHT_SLAB_SLOTS);
     };
     const int first_block = n0 / 128;
-    const __amdgpu_buffer_rsrc_t weight_scale_resource =
-        make_resource(p.w_scale + size_t(first_block) * p.groups,
+    const u32x4_t weight_scale_resource =
+        uniform_descriptor(p.w_scale + size_t(first_block) * p.groups,
                       unsigned(p.scale_blocks - first_block < 8 ? p.scale_blocks - first_block : 8) *
                           unsigned(p.groups) * 4u);
     const unsigned weight_slab_lane_off = (unsigned(lane / 8) * unsigned(p.groups) + unsigned(lane % 8)) * 4u;

@@ -18,11 +18,13 @@
 // (buffer_load ... lds; rows outside the matrix read as zero). The four scale bytes of a row and
 // step are one 32-bit word, read from the address rounded down to four bytes; v_alignbyte of two
 // consecutive words undoes any misalignment of the scale pointer, which is the same for every row
-// because a scale row is a multiple of four bytes long. E4M3 weights have one scale row per 32
-// weight rows, so a tile's word is one address for the whole wavefront and is loaded into
-// registers two steps ahead, like the per-token words. E2M1 weights have one scale row per weight
-// row: there the words of all rows of the workgroup (and of its tokens) are gathered once per step
-// into the LDS stage, 64 rows per wavefront load, instead of once per wavefront that uses them.
+// because a scale row is a multiple of four bytes long. The words reach the lanes through LDS slabs:
+// once per round of three or four steps every wavefront copies, with one direct-to-LDS load, the
+// next four words of 64 scale rows (16 bytes per lane: the rows of the tile's E2M1 weights and of its
+// tokens; for E4M3 weights the tile's 32-row blocks, one word per lane), and a lane reads the word
+// of its row two steps ahead of its use. A lane that fetched its row's word for every step itself
+// would request a cache line per lane and step, the same line for 32 steps (measured 7 to 25 % of
+// the kernel). Tokens with one scale byte per 128 inputs keep a byte load per lane and step.
 #include "common.hpp"
 #include "device.hpp"
 #include "dma.hpp"
@@ -41,11 +43,6 @@ struct MxDmaParams {
     const int32_t *active, *counts;
     int weight_groups, groups;
 };
-
-__device__ __forceinline__ unsigned scale_word(const unsigned char *base, int index)
-{
-    return *reinterpret_cast<const unsigned *>(base + size_t(index) * 4);
-}
 
 __device__ __forceinline__ unsigned long long uniform(unsigned long long value)
 {
@@ -136,16 +133,19 @@ __global__ __launch_bounds__(128 * WM) void mx_dma_kernel(MxDmaParams p)
     static_assert(BN % (WAVES * W_ROWS) == 0 && BM % (WAVES * X_ROWS) == 0, "loads");
     static_assert((WAVES * W_ROWS) % 16 == 0 && (WAVES * X_ROWS) % 16 == 0, "row step keeps the swizzle");
     constexpr int W_SLOTS = BN * CHW, SLOTS = W_SLOTS + BM * CHX, LOADS = A_ITERS + B_ITERS;
-    // scale words that travel through LDS: those of the weight rows and, unless the tokens have
-    // one scale byte per step, of the token rows
-    constexpr bool STAGED = PACKED;
-    constexpr int STAGED_ROWS = STAGED ? BN + (WIDE_X ? 0 : BM) : 0;
-    constexpr int SCALE_WAVES = STAGED ? STAGED_ROWS / 64 : 1;
-    static_assert(!STAGED || (STAGES == 3 && STAGED_ROWS % 64 == 0 && SCALE_WAVES <= WAVES),
-                  "one wavefront load stages the scale words of 64 rows");
-    __shared__ u32x4_t stages[STAGES][SLOTS];
-    // (an array of its own: all its reads share one address register and differ by immediates)
-    __shared__ u32x4_t scale_stages[STAGES][STAGED ? STAGED_ROWS / 4 : 1];
+    // scale rows whose words travel through LDS slabs: the weight rows when every row has its own
+    // scales (E2M1), the token rows unless the tokens have one scale byte per step; for E4M3 weights
+    // the tile's 32-row blocks have a small slab of their own
+    constexpr int SLAB_ROWS = (PACKED ? BN : 0) + (WIDE_X ? 0 : BM);
+    constexpr int PIECES = SLAB_ROWS / 64; // 64 rows per wavefront load, 16 bytes (four steps) per row
+    constexpr int PERIOD = STAGES == 3 ? 3 : 4; // steps between slabs: a whole number of rounds
+    constexpr int BLOCK_SLAB = PACKED ? 0 : 16; // u32x4 of the block slab: 16 blocks x 4 words
+    static_assert(SLAB_ROWS % 64 == 0 && (PACKED ? BN : 0) % 64 == 0 && PIECES <= WAVES && BN / 32 <= 16,
+                  "one load per wavefront and slab");
+    __shared__ u32x4_t lds[STAGES * SLOTS + 2 * SLAB_ROWS + 2 * BLOCK_SLAB];
+    auto stage_at = [&](int index) { return lds + index * SLOTS; };
+    auto slab_at = [&](int slab) { return lds + STAGES * SLOTS + (slab & 1) * SLAB_ROWS; };
+    auto block_slab_at = [&](int slab) { return lds + STAGES * SLOTS + 2 * SLAB_ROWS + (slab & 1) * BLOCK_SLAB; };
 
     const int thread = threadIdx.x, lane = thread % 64, wave = thread / 64;
     int tile_n, tile_m, group = 0;
@@ -236,88 +236,78 @@ __global__ __launch_bounds__(128 * WM) void mx_dma_kernel(MxDmaParams p)
         advance();
     };
 
-    // ---- scales: per lane (operand row lane%32) one 32-bit word per 32-row tile and step, read
-    // from the 4-byte aligned address at or below the row's scales. Register path: loaded
-    // unconditionally two steps ahead (a load under a branch would make the compiler wait for the
-    // LDS fills as well).
+    // ---- scales: per lane (operand row lane%32) one 32-bit word per 32-row tile and step, taken
+    // from the 4-byte aligned address at or below the row's scales. Slab number i holds words
+    // PERIOD * i .. PERIOD * i + 3 of every listed row (weight rows of the tile first, then its token
+    // rows), lane l of piece q the row 64 q + l; it is loaded when slab i - 1 comes into use, into
+    // the buffer that slab i - 2 has left. Loads and reads are kept out of the compiler's
+    // bookkeeping (it would make every LDS read that such a load might have written wait for all
+    // outstanding loads, the stage fills included): a slab load is older than the fills of the step
+    // that follows, whose wait therefore covers it, at least two steps before its first word is
+    // read; a word is read a few instructions before a step's wait and used after it.
     const int frag_row = lane % 32, half = lane / 32;
     const unsigned w_skew = unsigned(reinterpret_cast<uintptr_t>(weight_scale)) & 3u;
     const unsigned x_skew = WIDE_X ? 0u : unsigned(reinterpret_cast<uintptr_t>(input_scale)) & 3u;
-    const int w_last_word = p.steps - 1 + (w_skew != 0), x_last_word = p.steps - 1 + (x_skew != 0);
-    unsigned ws_offset[TN], xs_offset[TM]; // bytes from (scale pointer - skew): rows * pitch < 2^32
-#pragma unroll
-    for (int i = 0; i < TN; ++i) {
-        int n = n0 + (wn * TN + i) * 32;
-        n = n < p.outputs ? n : p.outputs - 1;
-        ws_offset[i] = unsigned(n / 32) * unsigned(scale_pitch); // (register path: E4M3 weights)
+    const int piece = __builtin_amdgcn_readfirstlane(wave) % (PIECES > 0 ? PIECES : 1);
+    const bool piece_of_weights = PACKED && piece * 64 < BN; // wave-uniform
+    unsigned slab_lane_off = 0;
+    u32x4_t slab_resource = {0u, 0u, 0u, 0u};
+    if constexpr (PIECES > 0) {
+        const int listed = piece * 64 + lane;
+        int row = piece_of_weights ? n0 + listed : m0 + listed - (PACKED ? BN : 0);
+        const int rows = piece_of_weights ? p.outputs : valid_rows;
+        row = row < rows ? row : rows - 1;
+        slab_lane_off = unsigned(row) * unsigned(scale_pitch);
+        const unsigned skew = piece_of_weights ? w_skew : x_skew;
+        slab_resource = uniform_descriptor((piece_of_weights ? weight_scale : input_scale) - skew,
+                                           unsigned(rows) * unsigned(scale_pitch) + (skew ? 4u : 0u));
     }
+    // E4M3 weights: one scale row per 32 weight rows; lane l brings word l % 4 of the slab for the
+    // tile's block l / 4 (every wavefront issues the same load: same bytes to the same place)
+    const int block_rows = (p.outputs + 31) / 32;
+    const int lane_block = n0 / 32 + lane / 4 < block_rows ? n0 / 32 + lane / 4 : block_rows - 1;
+    const unsigned block_lane_off = unsigned(lane_block) * unsigned(scale_pitch) + unsigned(lane % 4) * 4u;
+    const u32x4_t block_resource =
+        uniform_descriptor(weight_scale - w_skew, unsigned(block_rows) * unsigned(scale_pitch) + (w_skew ? 4u : 0u));
+    auto load_slabs = [&](int slab) {
+        if constexpr (PIECES > 0)
+            load_to_lds_untracked(slab_resource, slab_lane_off, unsigned(slab * PERIOD) * 4u,
+                                  slab_at(slab) + piece * 64);
+        if constexpr (!PACKED)
+            load_word_to_lds_untracked(block_resource, block_lane_off, unsigned(slab * PERIOD) * 4u,
+                                       block_slab_at(slab));
+    };
+    int ws_index[TN], xs_index[TM]; // word index of this lane's row inside a slab buffer
+#pragma unroll
+    for (int i = 0; i < TN; ++i)
+        ws_index[i] = PACKED ? ((wn * TN + i) * 32 + frag_row) * 4 : (wn * TN + i) * 4;
+#pragma unroll
+    for (int j = 0; j < TM; ++j)
+        xs_index[j] = ((PACKED ? BN : 0) + (wm * TM + j) * 32 + frag_row) * 4;
+    // word number `step` of the weight tile i / token tile j (reads of steps past the end return
+    // words that are never used)
+    auto weight_word = [&](int i, int step) {
+        const unsigned *words = reinterpret_cast<const unsigned *>(PACKED ? slab_at(step / PERIOD) : block_slab_at(step / PERIOD));
+        return lds_read_unordered(words + ws_index[i] + step % PERIOD);
+    };
+    auto token_word = [&](int j, int step) {
+        const unsigned *words = reinterpret_cast<const unsigned *>(slab_at(step / PERIOD));
+        return lds_read_unordered(words + xs_index[j] + step % PERIOD);
+    };
+    unsigned xs_byte_offset[TM]; // one scale byte per token and step: loaded a step ahead
 #pragma unroll
     for (int j = 0; j < TM; ++j) {
         int m = m0 + (wm * TM + j) * 32 + frag_row;
         m = m < valid_rows ? m : valid_rows - 1;
-        xs_offset[j] = unsigned(m) * unsigned(WIDE_X ? p.steps : scale_pitch);
+        xs_byte_offset[j] = unsigned(m) * unsigned(p.steps);
     }
-    unsigned ws_now[TN], ws_next[TN], ws_load[TN], xs_now[TM], xs_next[TM], xs_load[TM];
-    auto fetch_scales = [&](int step, unsigned (&w)[TN], unsigned (&x)[TM]) {
-        const int w_word = step < w_last_word ? step : w_last_word;
-        const int x_word = step < x_last_word ? step : x_last_word;
-        if constexpr (!STAGED) {
-#pragma unroll
-            for (int i = 0; i < TN; ++i)
-                w[i] = scale_word(weight_scale - w_skew + ws_offset[i], w_word);
-        }
-        if constexpr (!STAGED && !WIDE_X) {
-#pragma unroll
-            for (int j = 0; j < TM; ++j)
-                x[j] = scale_word(input_scale - x_skew + xs_offset[j], x_word);
-        }
-    };
-    // one scale byte per token and step: no second word is needed, so one step ahead is enough
+    unsigned ws_now[TN], ws_next[TN], xs_now[TM], xs_next[TM];
     auto fetch_token_bytes = [&](int step, unsigned (&x)[TM]) {
         const int x_byte = step < last_step ? step : last_step;
         if constexpr (WIDE_X) {
 #pragma unroll
             for (int j = 0; j < TM; ++j)
-                x[j] = unsigned(input_scale[xs_offset[j] + unsigned(x_byte)]);
-        }
-    };
-    // LDS path: wavefront w gathers the words of scale rows 64*w .. 64*w+63 of the list (weight
-    // rows of the tile, then its token rows) into the words behind the stage's operand tiles.
-    // Wavefronts beyond the list repeat the load of another one (same data to the same place)
-    // rather than branch around a load.
-    const int scale_wave = wave % SCALE_WAVES;
-    const bool scale_of_weights = scale_wave * 64 < BN; // wave-uniform
-    const int scale_last_word = scale_of_weights ? w_last_word : x_last_word;
-    unsigned scale_lane_off = 0;
-    int scale_step = 0;
-    __amdgpu_buffer_rsrc_t scale_resource = w_resource;
-    if constexpr (STAGED) {
-        const int listed = scale_wave * 64 + lane;
-        int row = scale_of_weights ? n0 + listed : m0 + listed - BN;
-        const int rows = scale_of_weights ? p.outputs : valid_rows;
-        row = row < rows ? row : rows - 1;
-        scale_lane_off = unsigned(row) * unsigned(scale_pitch);
-        const unsigned skew = scale_of_weights ? w_skew : x_skew;
-        scale_resource =
-            make_resource((scale_of_weights ? weight_scale : input_scale) - skew,
-                          unsigned(rows) * unsigned(scale_pitch) + (skew ? 4u : 0u));
-    }
-    auto issue_scales = [&](u32x4_t *stage) {
-        if constexpr (STAGED) {
-            load_word_to_lds(scale_resource, scale_lane_off, unsigned(scale_step) * 4u,
-                             stage + scale_wave * 16);
-            scale_step = scale_step < scale_last_word ? scale_step + 1 : scale_last_word;
-        }
-    };
-    auto read_scales = [&](const u32x4_t *stage, unsigned (&w)[TN], unsigned (&x)[TM]) {
-        const unsigned *words = reinterpret_cast<const unsigned *>(stage);
-#pragma unroll
-        for (int i = 0; i < TN; ++i)
-            w[i] = words[(wn * TN + i) * 32 + frag_row];
-        if constexpr (!WIDE_X) {
-#pragma unroll
-            for (int j = 0; j < TM; ++j)
-                x[j] = words[BN + (wm * TM + j) * 32 + frag_row];
+                x[j] = unsigned(input_scale[xs_byte_offset[j] + unsigned(x_byte)]);
         }
     };
 
@@ -407,13 +397,7 @@ __global__ __launch_bounds__(128 * WM) void mx_dma_kernel(MxDmaParams p)
     // The scale byte of this lane's block (lane group g supplies the scale of inputs 32g..32g+31 of
     // an instruction) is byte 2*ks + half of the step's word: the word is shifted by `half` bytes
     // and the instruction's byte select takes byte 2*ks.
-    auto step = [&](int g, int s, const u32x4_t *current, u32x4_t *fill) {
-        if constexpr (STAGED) {
-            // words of step g + 2, ahead of its operand fills; words of step g + 1, gathered a step ago
-            issue_scales(scale_stages[(s + STAGES - 1) % STAGES]);
-            read_scales(scale_stages[(s + 1) % STAGES], ws_next, xs_next);
-        }
-        fetch_scales(g + 2, ws_load, xs_load);
+    auto step = [&](int g, const u32x4_t *current, u32x4_t *fill) {
         fetch_token_bytes(g + 1, xs_next);
         unsigned w_scale[TN], x_scale[TM];
 #pragma unroll
@@ -425,44 +409,69 @@ __global__ __launch_bounds__(128 * WM) void mx_dma_kernel(MxDmaParams p)
                                 : __builtin_amdgcn_alignbyte(xs_next[j], xs_now[j], x_skew) >> (8 * half);
         __builtin_amdgcn_sched_barrier(0);
         multiply(current, fill, w_scale, x_scale);
+        // words of step g + 2 (their slab landed at an earlier step's wait); this step's wait
+        // covers the reads
+        unsigned ws_load[TN], xs_load[TM];
+#pragma unroll
+        for (int i = 0; i < TN; ++i)
+            ws_load[i] = weight_word(i, g + 2);
+#pragma unroll
+        for (int j = 0; j < TM; ++j)
+            xs_load[j] = WIDE_X ? xs_next[j] : token_word(j, g + 2);
+        pipeline_barrier<(STAGES - 2) * LOADS>();
+        tie_after_wait(ws_load, xs_load);
 #pragma unroll
         for (int i = 0; i < TN; ++i) {
             ws_now[i] = ws_next[i];
-            if constexpr (!STAGED)
-                ws_next[i] = ws_load[i];
+            ws_next[i] = ws_load[i];
         }
 #pragma unroll
         for (int j = 0; j < TM; ++j) {
             xs_now[j] = xs_next[j];
-            if constexpr (!STAGED && !WIDE_X)
+            if constexpr (!WIDE_X)
                 xs_next[j] = xs_load[j];
         }
-        pipeline_barrier<(STAGES - 2) * LOADS>();
     };
 
-    fetch_scales(0, ws_now, xs_now);
-    fetch_scales(1, ws_next, xs_next);
+    load_slabs(0); // (the oldest loads: complete at the first wait)
     fetch_token_bytes(0, xs_now);
 #pragma unroll
     for (int s = 0; s + 1 < STAGES; ++s) {
         __builtin_amdgcn_sched_barrier(0);
-        issue_scales(scale_stages[s]);
-        issue(stages[s]);
+        issue(stage_at(s));
     }
     pipeline_barrier<(STAGES - 2) * LOADS>();
-    if constexpr (STAGED)
-        read_scales(scale_stages[0], ws_now, xs_now);
+#pragma unroll
+    for (int i = 0; i < TN; ++i) {
+        ws_now[i] = weight_word(i, 0);
+        ws_next[i] = weight_word(i, 1);
+    }
+    if constexpr (!WIDE_X) {
+#pragma unroll
+        for (int j = 0; j < TM; ++j) {
+            xs_now[j] = token_word(j, 0);
+            xs_next[j] = token_word(j, 1);
+        }
+    }
+    __builtin_amdgcn_s_waitcnt(0xc07f); // lgkmcnt(0)
+    tie_after_wait(ws_now, ws_next);
+    if constexpr (!WIDE_X)
+        tie_after_wait(xs_now, xs_next);
     // whole rounds of STAGES steps run without a branch between the steps; the remainder follows
     int g = 0;
-    for (; g + STAGES <= p.steps; g += STAGES) {
+    for (int slab = 1; g + STAGES <= p.steps; ++slab) {
+        load_slabs(slab);
+        const int end = slab * PERIOD < p.steps ? slab * PERIOD : p.steps;
+        for (; g + STAGES <= end; g += STAGES) {
 #pragma unroll
-        for (int s = 0; s < STAGES; ++s)
-            step(g + s, s, stages[s], stages[(s + STAGES - 1) % STAGES]);
+            for (int s = 0; s < STAGES; ++s)
+                step(g + s, stage_at(s), stage_at((s + STAGES - 1) % STAGES));
+        }
     }
 #pragma unroll
     for (int s = 0; s + 1 < STAGES; ++s)
         if (g + s < p.steps)
-            step(g + s, s, stages[s], stages[(s + STAGES - 1) % STAGES]);
+            step(g + s, stage_at(s), stage_at((s + STAGES - 1) % STAGES));
     wait_loads<0>();
 
     // ---- epilogue: accumulator register 4q+e of lane l is feature 8q + 4*(l/32) + e, token l%32
