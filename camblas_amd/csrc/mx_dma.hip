@@ -522,7 +522,7 @@ template <bool PACKED, bool WIDE_X, bool GROUPED>
 hipError_t launch_variant(hipStream_t stream, const MxDmaParams &p, int groups, int variant)
 {
     switch (variant) {
-    case 0: return launch_one<PACKED, WIDE_X, GROUPED, 4, 2, 4, PACKED ? 3 : 2, PACKED ? 2 : 3>(stream, p, groups);
+    case 0: return launch_one<PACKED, WIDE_X, GROUPED, 4, 2, 4, PACKED ? 3 : 2, PACKED || GROUPED ? 2 : 3>(stream, p, groups);
     case 1: return launch_one<PACKED, WIDE_X, GROUPED, 4, 1, 4, 3, 4>(stream, p, groups);
     case 2:
         if constexpr (!PACKED)
