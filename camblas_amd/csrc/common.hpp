@@ -181,6 +181,9 @@ hipError_t launch_bgemm_dma(hipStream_t stream, int variant, int n_out, int m_ro
 // the last to arrive adds the planes in index order. `arrivals` holds STREAM_ARRIVAL_SLOTS counters that are zero between
 // launches (the kernel leaves them so); one per output tile is used.
 constexpr size_t STREAM_ARRIVAL_SLOTS = 4096;
+// The FP8 streaming kernel keeps a row of K / 128 scales per token in LDS: rows of this many floats
+// (whole 64-float loads, odd so that tokens fall on different banks), at most 192 groups (K <= 24576).
+constexpr int STREAM_SCALE_PITCH = 193, STREAM_SCALE_GROUPS = 192;
 size_t stream_partial_bytes(int row_tiles, int token_tiles, int n_out, int m_rows, int shares);
 struct StreamShares {
     int count = 1;

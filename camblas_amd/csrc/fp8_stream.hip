@@ -19,6 +19,7 @@
 // groups are in flight per wavefront.
 #include "common.hpp"
 #include "device.hpp"
+#include "dma.hpp"
 
 namespace camblas_hip
 {
@@ -44,6 +45,12 @@ __global__ __launch_bounds__(WAVES * 64) void fp8_stream_kernel(Fp8StreamParams 
     constexpr int DEPTH = NT + MT <= 6 ? 3 : 2;
     constexpr int TILES = NT + MT; // weight tiles, then token tiles
     __shared__ __attribute__((aligned(16))) u32x4_t patch[WAVES][TILES][128];
+    // The scales of the workgroup's tokens (one row of `groups` floats per token) and of the two
+    // 128-row weight blocks its rows can lie in, copied to LDS once: a lane that fetched its
+    // token's scale for every group itself would request a cache line per lane and group, the same
+    // line for 32 groups (measured: 8 % of the launch at 32 tokens, 22 % at 64).
+    constexpr int SCALE_ROWS = MT * 16 + 2, SCALE_PITCH = STREAM_SCALE_PITCH;
+    __shared__ float scale_table[SCALE_ROWS * SCALE_PITCH];
     // after the last step the wavefront's patches hold its partial sums instead
     static_assert(NT * MT * 64 <= TILES * 128, "partial sums must fit the wavefront's patches");
     const int thread = threadIdx.x, lane = thread % 64, wave = thread / 64;
@@ -54,7 +61,6 @@ __global__ __launch_bounds__(WAVES * 64) void fp8_stream_kernel(Fp8StreamParams 
 
     // tile t < NT: weight rows n0 + 16 t ..; tile NT + j: tokens m0 + 16 j ..; half h: rows 8h ..
     const unsigned char *source[TILES][2];
-    const float *ws_ptr[NT], *as_ptr[MT];
 #pragma unroll
     for (int h = 0; h < 2; ++h) {
 #pragma unroll
@@ -70,17 +76,31 @@ __global__ __launch_bounds__(WAVES * 64) void fp8_stream_kernel(Fp8StreamParams 
             source[NT + j][h] = p.a + size_t(m) * p.k + piece * 16;
         }
     }
+    // rows of the scale table: tokens m0 .., then the weight blocks first_block and first_block + 1
+    const int first_block = n0 / 128;
+    int ws_row[NT], as_row[MT];
 #pragma unroll
-    for (int i = 0; i < NT; ++i) {
-        int block = (n0 + i * 16) / 128;
-        block = block < p.scale_blocks ? block : p.scale_blocks - 1;
-        ws_ptr[i] = p.w_scale + size_t(block) * p.groups;
-    }
+    for (int i = 0; i < NT; ++i)
+        ws_row[i] = (MT * 16 + (n0 + i * 16) / 128 - first_block) * SCALE_PITCH;
 #pragma unroll
-    for (int j = 0; j < MT; ++j) {
-        int m = m0 + j * 16 + row;
-        m = m < p.m ? m : p.m - 1;
-        as_ptr[j] = p.a_scale + size_t(m) * p.groups;
+    for (int j = 0; j < MT; ++j)
+        as_row[j] = (j * 16 + row) * SCALE_PITCH;
+    // One 4-byte-per-lane direct-to-LDS load brings 64 consecutive groups of a row (lanes past the
+    // row's end, and rows past the matrix, read zeros from the bounded buffer; the table's pitch
+    // leaves room for whole loads). Issued before the first weight loads, complete with them.
+    {
+        const u32x4_t token_scales = uniform_descriptor(
+            p.a_scale + size_t(m0) * p.groups, unsigned(p.m - m0 < MT * 16 ? p.m - m0 : MT * 16) * unsigned(p.groups) * 4u);
+        const u32x4_t block_scales = uniform_descriptor(
+            p.w_scale + size_t(first_block) * p.groups,
+            unsigned(p.scale_blocks - first_block < 2 ? p.scale_blocks - first_block : 2) * unsigned(p.groups) * 4u);
+        for (int r = __builtin_amdgcn_readfirstlane(wave); r < SCALE_ROWS; r += WAVES) {
+            const bool token = r < MT * 16;
+            const unsigned row_bytes = unsigned(token ? r : r - MT * 16) * unsigned(p.groups) * 4u;
+            for (int g0 = 0; g0 < p.groups; g0 += 64)
+                load_word_to_lds_untracked(token ? token_scales : block_scales, unsigned(lane) * 4u,
+                                           row_bytes + unsigned(g0) * 4u, scale_table + r * SCALE_PITCH + g0);
+        }
     }
     // LDS patch of one tile: 16 rows x 8 pieces of 16 bytes, piece index XORed with row bits 1..3,
     // which makes both the line-shaped stores and the operand-shaped loads conflict-free
@@ -99,14 +119,15 @@ __global__ __launch_bounds__(WAVES * 64) void fp8_stream_kernel(Fp8StreamParams 
         return rotated * WAVES + wave;
     };
     u32x4_t raw[DEPTH][TILES][2];
-    float ws_reg[DEPTH][NT], as_reg[DEPTH][MT], live_reg[DEPTH];
+    int group_reg[DEPTH];
+    float live_reg[DEPTH];
     // Nothing in a fetch may use a loaded value (that would wait for the loads just issued): a dead
     // step is remembered as a zero factor and applied to the scale when the group is multiplied.
-    auto fetch = [&](int step, u32x4_t(&data)[TILES][2], float(&ws)[NT], float(&as)[MT],
-                     float &live) {
+    auto fetch = [&](int step, u32x4_t(&data)[TILES][2], int &group, float &live) {
         int g = group_of(step);
         live = step < steps && g < p.groups ? 1.f : 0.f;
         g = g < p.groups ? g : p.groups - 1;
+        group = g;
         const size_t offset = size_t(g) * GROUP;
 #pragma unroll
         for (int t = 0; t < TILES; ++t)
@@ -115,12 +136,6 @@ __global__ __launch_bounds__(WAVES * 64) void fp8_stream_kernel(Fp8StreamParams 
                 const u32x4_t *address = reinterpret_cast<const u32x4_t *>(source[t][h] + offset);
                 data[t][h] = t < NT ? __builtin_nontemporal_load(address) : *address;
             }
-#pragma unroll
-        for (int i = 0; i < NT; ++i)
-            ws[i] = ws_ptr[i][g];
-#pragma unroll
-        for (int j = 0; j < MT; ++j)
-            as[j] = as_ptr[j][g];
     };
 
     f32x4_t acc[NT][MT];
@@ -129,9 +144,15 @@ __global__ __launch_bounds__(WAVES * 64) void fp8_stream_kernel(Fp8StreamParams 
 #pragma unroll
         for (int j = 0; j < MT; ++j)
             acc[i][j] = f32x4_t{0.f, 0.f, 0.f, 0.f};
-    auto multiply = [&](const u32x4_t(&data)[TILES][2], const float(&ws)[NT], const float(&as)[MT],
-                        float live) {
+    auto multiply = [&](const u32x4_t(&data)[TILES][2], int group, float live) {
         u32x4_t *mine = &patch[wave][0][0];
+        float ws[NT], as[MT];
+#pragma unroll
+        for (int i = 0; i < NT; ++i)
+            ws[i] = scale_table[ws_row[i] + group];
+#pragma unroll
+        for (int j = 0; j < MT; ++j)
+            as[j] = scale_table[as_row[j] + group];
 #pragma unroll
         for (int t = 0; t < TILES; ++t) {
             mine[t * 128 + store_slot[0]] = data[t][0];
@@ -169,16 +190,21 @@ __global__ __launch_bounds__(WAVES * 64) void fp8_stream_kernel(Fp8StreamParams 
     // multiply covers only the oldest of the groups in flight
 #pragma unroll
     for (int d = 0; d < DEPTH; ++d) {
-        fetch(d, raw[d], ws_reg[d], as_reg[d], live_reg[d]);
+        fetch(d, raw[d], group_reg[d], live_reg[d]);
         __builtin_amdgcn_sched_barrier(0);
     }
+    // the scale table's loads are older than the DEPTH * TILES * 2 loads of the fetches above (the
+    // compiler does not count them, so the wait is explicit); the barrier shows every wavefront's
+    // part of the table to the others
+    wait_loads<DEPTH * TILES * 2>();
+    __syncthreads();
     for (int step = 0; step < steps; step += DEPTH) {
 #pragma unroll
         for (int d = 0; d < DEPTH; ++d) {
             __builtin_amdgcn_sched_barrier(0);
-            multiply(raw[d], ws_reg[d], as_reg[d], live_reg[d]);
+            multiply(raw[d], group_reg[d], live_reg[d]);
             __builtin_amdgcn_sched_barrier(0);
-            fetch(step + d + DEPTH, raw[d], ws_reg[d], as_reg[d], live_reg[d]);
+            fetch(step + d + DEPTH, raw[d], group_reg[d], live_reg[d]);
         }
     }
     // ---- every wavefront parks its partial sums in its own patches (nobody else reads those);
@@ -253,7 +279,7 @@ hipError_t launch_fp8_stream(hipStream_t stream, int row_tiles, int token_tiles,
                              int inner, const void *a, const float *a_scale, const void *w,
                              const float *w_scale, void *out)
 {
-    if (inner % GROUP || inner < GROUP || rows < 1 || outputs < 1)
+    if (inner % GROUP || inner < GROUP || inner / GROUP > STREAM_SCALE_GROUPS || rows < 1 || outputs < 1)
         return hipErrorInvalidValue;
     if ((rows + token_tiles * 16 - 1) / (token_tiles * 16) > 65535)
         return hipErrorInvalidValue;

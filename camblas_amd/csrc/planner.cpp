@@ -232,9 +232,17 @@ Plan make_plan(int dtype, int algorithm, bool trans_a, bool trans_b, int m, int 
     }
     // FP8 block-scaled: rows = n (tokens), outputs = m, always K-contiguous
     plan.counter = 4;
-    if (n > 8 && n <= 64) {
+    const bool tiles_apply = m % 4 == 0 && k < (1 << 24); // what the direct-to-LDS tiles need
+    // (the streaming kernel holds a row of K / 128 scales per token in LDS: K up to 24576; 33 to 64
+    // tokens go to the tiles when K is long enough to divide: measured at K = 1536 and 2048 the
+    // streaming kernel is 35 % faster there, at 7168 and 18432 the tiles are 10 to 35 % faster)
+    const bool streamable = k / 128 <= STREAM_SCALE_GROUPS;
+    if (n > 8 && streamable && (n <= 32 || (n <= 64 && (!tiles_apply || k < 4096)))) {
         // decode batches: one streaming pass over the weights, whole K per workgroup; the row
-        // tiles are limited by the operand registers (row_tiles * token_tiles <= 16, sum <= 10)
+        // tiles are limited by the operand registers (row_tiles * token_tiles <= 16, sum <= 10).
+        // From 33 tokens on the 64-token tiles below with divided K are faster (the streaming
+        // kernel's four token tiles gather four scale lines per lane and group: [18432, 7168] at
+        // 64 tokens 49 us against 33).
         const int token_tiles = n <= 16 ? 1 : n <= 32 ? 2 : 4;
         const int limit = std::min(16 / token_tiles, 10 - token_tiles);
         plan.family = FAMILY_FP8_STREAM;
@@ -250,7 +258,7 @@ Plan make_plan(int dtype, int algorithm, bool trans_a, bool trans_b, int m, int 
         plan.split_k = decode_split(ceil_div(m, v.block_n), ceil_div(k, v.block_k), compute_units);
         return plan;
     }
-    if (m % 4 != 0 || k >= (1 << 24)) {
+    if (!tiles_apply) {
         plan.family = FAMILY_FP8_BLOCK;
         plan.kernel = 0;
         return plan;
