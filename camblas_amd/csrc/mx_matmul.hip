@@ -49,16 +49,19 @@ struct MxParams {
 };
 
 constexpr int WAVES = 4, GROUP = 128;
-// Per-row weight scales (E2M1 weights) of a workgroup's rows are one contiguous byte range; when it
-// fits this many bytes it is copied to LDS once with coalesced loads instead of being gathered a
-// byte per lane and step (16 cache lines per gather for 64 useful bytes).
+// The weight scales of a workgroup's rows (E2M1: a scale row per weight row; E4M3: one per 32 weight
+// rows) are one contiguous byte range; when it fits this many bytes it is copied to LDS once with
+// whole 1 KB direct-to-LDS loads instead of being gathered a byte per lane and step (16 cache lines
+// per gather for 64 useful bytes).
 constexpr int STAGED_SCALE_BYTES = 32768;
-constexpr int STAGE_PIECES = STAGED_SCALE_BYTES / 16 / (WAVES * 64) + 1; // 16-byte pieces per thread
+// The scale bytes of a workgroup's tokens are one contiguous byte range too and are copied with it
+// when they fit this many bytes (a byte per lane, token tile and step from memory is a cache line
+// per lane; measured 14 to 17 % of the E2M1 launch at 1 to 16 tokens).
+constexpr int STAGED_TOKEN_BYTES = 16384;
 
 template <bool PACKED, bool GROUPED, bool STAGED, int NT, int MT>
 __global__ __launch_bounds__(WAVES * 64) void mx_stream_kernel(MxParams p)
 {
-    static_assert(PACKED || !STAGED, "only per-row scales are staged");
     // A step of a wavefront covers one 128-byte line of every weight row: one 128-input group of
     // E4M3 weights, two consecutive groups of packed E2M1 weights (a half-line step would leave the
     // other half of each line to another wavefront's request).
@@ -71,7 +74,9 @@ __global__ __launch_bounds__(WAVES * 64) void mx_stream_kernel(MxParams p)
     // same memory holds the wavefront's partial sums
     __shared__ __attribute__((aligned(16))) u32x4_t tiles[WAVES][NT + MT][128];
     static_assert(NT * MT * 64 <= (NT + MT) * 128, "partial sums must fit the wavefront's tile memory");
-    __shared__ __attribute__((aligned(16))) unsigned char staged[STAGED ? STAGED_SCALE_BYTES + 16 : 16];
+    // (direct-to-LDS loads write whole 1 KB pieces: a piece of slack behind each range)
+    __shared__ __attribute__((aligned(16))) unsigned char staged[STAGED ? STAGED_SCALE_BYTES + 1024 : 16];
+    __shared__ __attribute__((aligned(16))) unsigned char staged_tokens[STAGED ? STAGED_TOKEN_BYTES + 1024 : 16];
     const int thread = threadIdx.x, lane = thread % 64, wave = thread / 64;
     const int row = lane % 16, chunk = lane / 16; // operand row / token, 32-input chunk of the group
     const int n0 = blockIdx.x * (NT * 16), m0 = blockIdx.y * (MT * 16);
@@ -194,26 +199,50 @@ __global__ __launch_bounds__(WAVES * 64) void mx_stream_kernel(MxParams p)
 #pragma unroll
                 for (int h = 0; h < 2; ++h)
                     x[j][s][h] = *reinterpret_cast<const u32x4_t *>(x_source[j][h] + x_offset);
-                xs[j][s] = xs_source[j][block >> p.scale_shift];
+                if constexpr (STAGED)
+                    xs[j][s] = unsigned(block >> p.scale_shift); // read from LDS at multiply time
+                else
+                    xs[j][s] = xs_source[j][block >> p.scale_shift];
             }
         }
     };
 
-    // Staged scales: the byte range of rows n0 .. n0 + 16*NT - 1 (cut at the matrix end), widened to
-    // whole aligned 16-byte pieces (a piece holding one valid byte lies inside that byte's page).
-    // The loads go out before the first weight loads and are stored once those are in flight.
-    u32x4_t stage_raw[STAGE_PIECES];
-    int staged_shift = 0, stage_pieces = 0;
+    // Staged scales: two byte ranges, each copied into LDS by direct-to-LDS loads of 1 KB (16 bytes
+    // per lane) from the 4-byte aligned address at or below its start: the weight scales of rows
+    // n0 .. n0 + 16*NT - 1 (E2M1: a scale row per weight row; E4M3: a scale row per 32 weight rows),
+    // cut at the matrix end, and the scales of the workgroup's tokens. The loads go out before the
+    // first weight loads and are complete with them; bytes past a range's end are never read.
+    int staged_shift = 0, token_shift = 0;
+    int w_base[NT], x_base[MT]; // byte offset of this lane's scale row inside the staged ranges
     if constexpr (STAGED) {
-        const unsigned char *first = weight_scale + size_t(n0) * blocks;
-        const int length = min(NT * 16, p.outputs - n0) * blocks;
-        staged_shift = int(reinterpret_cast<uintptr_t>(first) & 15);
-        stage_pieces = (staged_shift + length + 15) / 16;
-        const u32x4_t *pieces = reinterpret_cast<const u32x4_t *>(first - staged_shift);
+        const int first_row = PACKED ? n0 : n0 / 32;
+        const int last = min(n0 + NT * 16, p.outputs) - 1;
+        const int staged_rows = (PACKED ? last : last / 32) - first_row + 1;
+        const unsigned char *first = weight_scale + size_t(first_row) * blocks;
+        staged_shift = int(reinterpret_cast<uintptr_t>(first) & 3);
+        const unsigned bytes = unsigned(staged_shift + staged_rows * blocks);
+        const u32x4_t range = uniform_descriptor(first - staged_shift, (bytes + 3u) & ~3u);
+        for (unsigned piece = __builtin_amdgcn_readfirstlane(wave); piece * 1024u < bytes; piece += WAVES)
+            load_to_lds_untracked(range, unsigned(lane) * 16u, piece * 1024u, staged + piece * 1024u);
 #pragma unroll
-        for (int e = 0; e < STAGE_PIECES; ++e) {
-            const int index = thread + e * (WAVES * 64);
-            stage_raw[e] = pieces[index < stage_pieces ? index : stage_pieces - 1];
+        for (int i = 0; i < NT; ++i) {
+            int n = n0 + i * 16 + (PACKED ? row : 0);
+            n = n < p.outputs ? n : p.outputs - 1;
+            w_base[i] = staged_shift + ((PACKED ? n : n / 32) - first_row) * blocks;
+        }
+        const int x_pitch = blocks >> p.scale_shift;
+        const int tokens = min(MT * 16, valid_rows - m0);
+        const unsigned char *first_token = input_scale + size_t(m0) * x_pitch;
+        token_shift = int(reinterpret_cast<uintptr_t>(first_token) & 3);
+        const unsigned token_bytes = unsigned(token_shift + tokens * x_pitch);
+        const u32x4_t token_range = uniform_descriptor(first_token - token_shift, (token_bytes + 3u) & ~3u);
+        for (unsigned piece = __builtin_amdgcn_readfirstlane(wave); piece * 1024u < token_bytes; piece += WAVES)
+            load_to_lds_untracked(token_range, unsigned(lane) * 16u, piece * 1024u, staged_tokens + piece * 1024u);
+#pragma unroll
+        for (int j = 0; j < MT; ++j) {
+            int m = m0 + j * 16 + row;
+            m = m < valid_rows ? m : valid_rows - 1;
+            x_base[j] = token_shift + (m - m0) * x_pitch;
         }
         __builtin_amdgcn_sched_barrier(0);
     }
@@ -264,8 +293,11 @@ __global__ __launch_bounds__(WAVES * 64) void mx_stream_kernel(MxParams p)
             unsigned w_scale[NT];
 #pragma unroll
             for (int i = 0; i < NT; ++i)
-                w_scale[i] = STAGED ? unsigned(staged[staged_shift + (i * 16 + row) * blocks + int(ws[i][s])])
-                                    : ws[i][s];
+                w_scale[i] = STAGED ? unsigned(staged[w_base[i] + int(ws[i][s])]) : ws[i][s];
+            unsigned x_scale[MT];
+#pragma unroll
+            for (int j = 0; j < MT; ++j)
+                x_scale[j] = STAGED ? unsigned(staged_tokens[x_base[j] + int(xs[j][s])]) : xs[j][s];
             // inputs past the end of K (and of dead steps) are zero
 #pragma unroll
             for (int j = 0; j < MT; ++j) {
@@ -276,7 +308,7 @@ __global__ __launch_bounds__(WAVES * 64) void mx_stream_kernel(MxParams p)
 #pragma unroll
                 for (int i = 0; i < NT; ++i)
                     acc[i][j] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(
-                        a[i], b, acc[i][j], PACKED ? 4 : 0, 0, 0, int(w_scale[i]), 0, int(xs[j][s]));
+                        a[i], b, acc[i][j], PACKED ? 4 : 0, 0, 0, int(w_scale[i]), 0, int(x_scale[j]));
             }
             // the patches are overwritten next: order the reads above before those stores
             __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
@@ -290,14 +322,12 @@ __global__ __launch_bounds__(WAVES * 64) void mx_stream_kernel(MxParams p)
         __builtin_amdgcn_sched_barrier(0);
     }
     if constexpr (STAGED) {
-#pragma unroll
-        for (int e = 0; e < STAGE_PIECES; ++e) {
-            const int index = thread + e * (WAVES * 64);
-            if (index < stage_pieces)
-                reinterpret_cast<u32x4_t *>(staged)[index] = stage_raw[e];
-        }
-        // not __syncthreads(): its fence would wait for every weight load issued above
-        pipeline_barrier<63>();
+        // the staged ranges' loads are older than the loads of the DEPTH fetches above (the compiler
+        // does not count them, so the wait is explicit; not __syncthreads(): its fence would wait
+        // for every weight load as well); the barrier shows every wavefront's pieces to the others
+        constexpr int FETCH_LOADS = 2 * (NT + MT * SUB);
+        static_assert(DEPTH * FETCH_LOADS < 64, "vmcnt holds 6 bits");
+        pipeline_barrier<DEPTH * FETCH_LOADS>();
     }
     for (int step = 0; step < steps; step += DEPTH) {
 #pragma unroll
@@ -357,8 +387,11 @@ hipError_t launch_one(hipStream_t stream, const MxParams &p, int groups)
     } else {
         dim3 grid(unsigned((p.outputs + NT * 16 - 1) / (NT * 16)),
                   unsigned((p.rows + MT * 16 - 1) / (MT * 16)), unsigned(groups));
-        if (PACKED && NT * 16 * (p.inner / 32) <= STAGED_SCALE_BYTES)
-            mx_stream_kernel<PACKED, GROUPED, PACKED, NT, MT><<<grid, WAVES * 64, 0, stream>>>(p);
+        const int blocks = p.inner / 32;
+        const int weight_scale_bytes = (PACKED ? NT * 16 : NT / 2 + 2) * blocks + 3;
+        const int token_scale_bytes = MT * 16 * (blocks >> p.scale_shift) + 3;
+        if (weight_scale_bytes <= STAGED_SCALE_BYTES && token_scale_bytes <= STAGED_TOKEN_BYTES)
+            mx_stream_kernel<PACKED, GROUPED, true, NT, MT><<<grid, WAVES * 64, 0, stream>>>(p);
         else
             mx_stream_kernel<PACKED, GROUPED, false, NT, MT><<<grid, WAVES * 64, 0, stream>>>(p);
         return launch_status();
