@@ -75,7 +75,8 @@ __device__ __forceinline__ u32x4_t uniform_descriptor(const void *base, unsigned
 }
 // load_to_lds / load_word_to_lds outside the compiler's bookkeeping of memory operations (it then
 // neither counts them nor makes later LDS reads wait for them): for data that is read with
-// lds_read_unordered after a wait the caller places. M0 is put back as it was. The loads still
+// lds_read_unordered after a wait the caller places. M0 is put back as it was, with the wait state a
+// direct-to-LDS load needs after a write of M0 on either side. The loads still
 // count in vmcnt, which only makes waits the compiler computes for its own loads stricter.
 __device__ __forceinline__ void load_to_lds_untracked(u32x4_t descriptor, unsigned lane_offset,
                                                       unsigned step_offset, const void *lds_base)
@@ -84,7 +85,7 @@ __device__ __forceinline__ void load_to_lds_untracked(u32x4_t descriptor, unsign
     const unsigned step = __builtin_amdgcn_readfirstlane(step_offset);
     unsigned saved;
     asm volatile("s_mov_b32 %0, m0\n\ts_mov_b32 m0, %1\n\ts_nop 0\n\t"
-                 "buffer_load_dwordx4 %2, %3, %4 offen lds\n\ts_mov_b32 m0, %0"
+                 "buffer_load_dwordx4 %2, %3, %4 offen lds\n\ts_mov_b32 m0, %0\n\ts_nop 0"
                  : "=&s"(saved)
                  : "s"(address), "v"(lane_offset), "s"(descriptor), "s"(step)
                  : "memory");
@@ -96,7 +97,7 @@ __device__ __forceinline__ void load_word_to_lds_untracked(u32x4_t descriptor, u
     const unsigned step = __builtin_amdgcn_readfirstlane(step_offset);
     unsigned saved;
     asm volatile("s_mov_b32 %0, m0\n\ts_mov_b32 m0, %1\n\ts_nop 0\n\t"
-                 "buffer_load_dword %2, %3, %4 offen lds\n\ts_mov_b32 m0, %0"
+                 "buffer_load_dword %2, %3, %4 offen lds\n\ts_mov_b32 m0, %0\n\ts_nop 0"
                  : "=&s"(saved)
                  : "s"(address), "v"(lane_offset), "s"(descriptor), "s"(step)
                  : "memory");
