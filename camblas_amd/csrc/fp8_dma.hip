@@ -206,7 +206,10 @@ __global__ __launch_bounds__(128 * WM) void fp8_dma_kernel(Fp8DmaParams p)
     auto multiply = [&](const u32x4_t *stage, u32x4_t *fill, const float (&as_now)[TM],
                         const float (&ws_now)[WS]) {
         constexpr int TILES = TN * TM, SHARE = (LOADS + TILES - 1) / TILES;
-        i32x8_t a_frag[2][2], b_frag[TM][2];
+        // (eight tiles per wavefront at two wavefronts per SIMD leave no registers for a second
+        // weight-fragment buffer: with it the 256 x 256 tile spilled 21 registers)
+        constexpr int A_BUFFERS = TILES >= 8 && WAVES == 8 ? 1 : 2;
+        i32x8_t a_frag[A_BUFFERS][2], b_frag[TM][2];
 #pragma unroll
         for (int j = 0; j < TM; ++j) {
             b_frag[j][0] = fragment(stage, b_frag_base + j * 32 * CH, 0);
@@ -226,9 +229,9 @@ __global__ __launch_bounds__(128 * WM) void fp8_dma_kernel(Fp8DmaParams p)
 #pragma unroll
             for (int r = 0; r < 16; ++r)
                 d[r] = 0.f;
-            d = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(a_frag[i & 1][0], b_frag[j][0], d, 0,
+            d = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(a_frag[i % A_BUFFERS][0], b_frag[j][0], d, 0,
                                                                 0, 0, UNIT, 0, UNIT);
-            d = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(a_frag[i & 1][1], b_frag[j][1], d, 0,
+            d = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(a_frag[i % A_BUFFERS][1], b_frag[j][1], d, 0,
                                                                 0, 0, UNIT, 0, UNIT);
         };
         auto accumulate = [&](int tile, const f32x16_t &d) {
@@ -240,10 +243,14 @@ __global__ __launch_bounds__(128 * WM) void fp8_dma_kernel(Fp8DmaParams p)
 #pragma unroll
         for (int tile = 0; tile < TILES; ++tile) {
             __builtin_amdgcn_sched_barrier(0);
-            if (tile % TM == 0 && tile / TM + 1 < TN) { // next weight tile into the other buffer
+            if (A_BUFFERS == 2 && tile % TM == 0 && tile / TM + 1 < TN) { // next weight tile into the other buffer
                 const int row = tile / TM + 1;
-                a_frag[row & 1][0] = fragment(stage, a_frag_base + row * 32 * CH, 0);
-                a_frag[row & 1][1] = fragment(stage, a_frag_base + row * 32 * CH, 1);
+                a_frag[row % A_BUFFERS][0] = fragment(stage, a_frag_base + row * 32 * CH, 0);
+                a_frag[row % A_BUFFERS][1] = fragment(stage, a_frag_base + row * 32 * CH, 1);
+            }
+            if (A_BUFFERS == 1 && tile % TM == 0 && tile > 0) { // this row's weight tile, the last row's MFMAs being issued
+                a_frag[0][0] = fragment(stage, a_frag_base + (tile / TM) * 32 * CH, 0);
+                a_frag[0][1] = fragment(stage, a_frag_base + (tile / TM) * 32 * CH, 1);
             }
             __builtin_amdgcn_sched_barrier(0);
             product(tile, dot[tile & 1]);

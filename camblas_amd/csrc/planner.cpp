@@ -276,7 +276,7 @@ Plan make_plan(int dtype, int algorithm, bool trans_a, bool trans_b, int m, int 
     const struct {
         int variant;
         double group_us;
-    } candidates[] = {{0, 2.10}, {8, 1.55}, {4, 1.12}, {7, 0.90}, {6, 0.80}, {9, 0.67}};
+    } candidates[] = {{0, 1.88}, {8, 1.55}, {4, 1.12}, {7, 0.90}, {6, 0.80}, {9, 0.67}};
     const int groups = k / 128;
     double best = 1e30;
     for (const auto &candidate : candidates) {
