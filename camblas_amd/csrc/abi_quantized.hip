@@ -30,6 +30,7 @@ Plan fp8_plan(const camblas_cuda_context *context, int rows, int outputs, int in
     if (forced < 0)
         return plan;
     plan.split_k = 1;
+    plan.tail_outputs = 0;
     if (forced >= 100) {
         plan.family = FAMILY_FP8_STREAM;
         plan.kernel = forced - 100;
@@ -99,7 +100,7 @@ extern "C" int camblas_cuda_fp8_block_matmul(camblas_cuda_context *context, int 
         context->counts[plan.counter]++;
         if (plan.family == FAMILY_FP8_DMA)
             return entry.finish(launch_fp8_dma(stream, plan.kernel, plan.split_k, rows, outputs, inner, a, a_scale,
-                                               w, w_scale, out, partials),
+                                               w, w_scale, out, partials, plan.tail_kernel, plan.tail_outputs),
                                 "FP8 block-scaled GEMM (direct LDS loads)");
         return entry.finish(launch_fp8_block(stream, plan.kernel, plan.split_k, rows, outputs, inner, a, a_scale,
                                              w, w_scale, out, partials),

@@ -87,6 +87,8 @@ struct Plan {
     int kernel = 0;   // variant index inside the family (stream family: 100*log2(K blocks per step) + 10*row_tiles + token_tiles)
     int split_k = 1;  // number of K partitions (partials reduced in fixed order)
     int counter = 0;  // stats slot incremented at launch
+    // FP8 prefill tiles: the last tail_outputs outputs run on variant tail_kernel in a second launch
+    int tail_kernel = 0, tail_outputs = 0;
 };
 
 // dtype: 0 FP32, 2 BF16, 3 FP8 block-scaled ('T','N' implied). aligned16: every operand pointer
@@ -209,7 +211,7 @@ hipError_t launch_fp8_block(hipStream_t stream, int variant, int split_k, int ro
 // ([split_k, rows, outputs]) summed in index order.
 hipError_t launch_fp8_dma(hipStream_t stream, int variant, int split_k, int rows, int outputs, int inner,
                           const void *a, const float *a_scale, const void *w, const float *w_scale,
-                          void *out, float *partials);
+                          void *out, float *partials, int tail_variant = 0, int tail_outputs = 0);
 hipError_t launch_fp8_split_sum(hipStream_t stream, int splits, size_t count, const float *partials, void *out);
 // row_tiles 1..8 (16 weight rows each), token_tiles 1, 2 or 4 (16 tokens each).
 hipError_t launch_fp8_stream(hipStream_t stream, int row_tiles, int token_tiles, int rows, int outputs,

@@ -33,6 +33,7 @@ struct Fp8DmaParams {
     unsigned short *out;
     float *partials; // FP32 [splits, m, n] when the K groups are divided over blockIdx.y, else null
     int n, m, k, groups, scale_blocks;
+    int out_pitch; // elements between tokens in `out` (the outputs of the whole product)
     int tiles_n, tiles_m;
     int split_groups; // K groups per blockIdx.y (all of them without a split)
 };
@@ -343,7 +344,7 @@ __global__ __launch_bounds__(128 * WM) void fp8_dma_kernel(Fp8DmaParams p)
 #pragma unroll
     for (int j = 0; j < TM; ++j) {
         const int m = m0 + (wm * TM + j) * 32 + frag_row;
-        unsigned short *row = p.out + size_t(m) * p.n + n0 + wn * TN * 32 + half * 4;
+        unsigned short *row = p.out + size_t(m) * p.out_pitch + n0 + wn * TN * 32 + half * 4;
 #pragma unroll
         for (int i = 0; i < TN; ++i) {
             __builtin_amdgcn_sched_barrier(0);
@@ -395,9 +396,32 @@ const TnVariant &fp8_dma_variant(int index) { return variants[index]; }
 // an FP32 plane of `partials` ([split_k, rows, outputs], 16-byte aligned) and the planes are summed
 // in index order before the one BF16 rounding: few tokens leave most compute units without a tile
 // otherwise (256 tokens by 18432 outputs are 72 tiles of 256 x 256).
+namespace
+{
+hipError_t launch_rows(hipStream_t stream, int variant, int splits, const Fp8DmaParams &p)
+{
+    switch (variant) {
+    case 0: return launch_one<2, 4, 2>(stream, p, splits);
+    case 1: return launch_one<1, 4, 2>(stream, p, splits);
+    case 2: return launch_one<2, 2, 2>(stream, p, splits);
+    case 3: return launch_one<1, 2, 2>(stream, p, splits);
+    case 4: return launch_one<1, 4, 3>(stream, p, splits);
+    case 5: return launch_one<2, 2, 3>(stream, p, splits);
+    case 6: return launch_one<1, 2, 3>(stream, p, splits);
+    case 7: return launch_one<1, 4, 3, 3>(stream, p, splits);
+    case 8: return launch_one<2, 4, 2, 3>(stream, p, splits);
+    case 9: return launch_one<1, 2, 3, 3>(stream, p, splits);
+    default: return hipErrorInvalidValue;
+    }
+}
+} // namespace
+
+// tail_outputs > 0 (undivided K only): the last tail_outputs outputs, starting at a multiple of 128,
+// run on tail_variant in a launch of their own, so that both launches are whole rounds of
+// workgroups where one tiling would end in a partly filled round.
 hipError_t launch_fp8_dma(hipStream_t stream, int variant, int split_k, int rows, int outputs, int inner,
                           const void *a, const float *a_scale, const void *w, const float *w_scale,
-                          void *out, float *partials)
+                          void *out, float *partials, int tail_variant, int tail_outputs)
 {
     if (outputs % 4 || inner % 128 || reinterpret_cast<uintptr_t>(out) % 8)
         return hipErrorInvalidValue;
@@ -406,35 +430,34 @@ hipError_t launch_fp8_dma(hipStream_t stream, int variant, int split_k, int rows
         return hipErrorInvalidValue;
     if (size_t(256) * size_t(inner) >= (size_t(1) << 32))
         return hipErrorInvalidValue;
+    if (tail_outputs < 0 || tail_outputs >= outputs || (tail_outputs && (split_k > 1 || (outputs - tail_outputs) % 128)))
+        return hipErrorInvalidValue;
     Fp8DmaParams p;
     p.w = static_cast<const unsigned char *>(w);
     p.a = static_cast<const unsigned char *>(a);
     p.w_scale = w_scale;
     p.a_scale = a_scale;
     p.out = static_cast<unsigned short *>(out);
-    p.n = outputs;
+    p.n = outputs - tail_outputs;
+    p.out_pitch = outputs;
     p.m = rows;
     p.k = inner;
     p.groups = inner / 128;
-    p.scale_blocks = (outputs + 127) / 128;
+    p.scale_blocks = (p.n + 127) / 128;
     p.tiles_n = p.tiles_m = 0;
     p.split_groups = (p.groups + split_k - 1) / split_k;
     // every blockIdx.y must own at least one group
     const int splits = (p.groups + p.split_groups - 1) / p.split_groups;
     p.partials = splits > 1 ? partials : nullptr;
-    hipError_t status;
-    switch (variant) {
-    case 0: status = launch_one<2, 4, 2>(stream, p, splits); break;
-    case 1: status = launch_one<1, 4, 2>(stream, p, splits); break;
-    case 2: status = launch_one<2, 2, 2>(stream, p, splits); break;
-    case 3: status = launch_one<1, 2, 2>(stream, p, splits); break;
-    case 4: status = launch_one<1, 4, 3>(stream, p, splits); break;
-    case 5: status = launch_one<2, 2, 3>(stream, p, splits); break;
-    case 6: status = launch_one<1, 2, 3>(stream, p, splits); break;
-    case 7: status = launch_one<1, 4, 3, 3>(stream, p, splits); break;
-    case 8: status = launch_one<2, 4, 2, 3>(stream, p, splits); break;
-    case 9: status = launch_one<1, 2, 3, 3>(stream, p, splits); break;
-    default: return hipErrorInvalidValue;
+    hipError_t status = launch_rows(stream, variant, splits, p);
+    if (status == hipSuccess && tail_outputs) {
+        const size_t first = size_t(p.n);
+        p.w += first * size_t(inner);
+        p.w_scale += (first / 128) * size_t(p.groups);
+        p.out += first;
+        p.n = tail_outputs;
+        p.scale_blocks = (tail_outputs + 127) / 128;
+        status = launch_rows(stream, tail_variant, 1, p);
     }
     if (status != hipSuccess || splits == 1)
         return status;
