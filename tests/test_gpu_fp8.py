@@ -78,6 +78,22 @@ def test_streaming_decode_variants(device, code, rows, outputs, inner):
     assert (np.abs(bf16_values(out) - wanted) <= bound).all()
 
 
+@pytest.mark.parametrize("rows,inner", [(16, 192 * 128), (24, 193 * 128), (5, 67 * 128)])
+def test_streaming_decode_scale_table_limits(device, rows, inner):
+    # the streaming kernel keeps a row of K / 128 scales per token in LDS: 192 groups is the most it
+    # takes (three whole 64-float loads per row), 193 goes to another kernel, 67 leaves a load with
+    # three live lanes; weight rows that straddle two 128-row scale blocks
+    outputs = 200
+    a, a_scale = oracle.fill_fp8_blocks(800 + rows, rows, inner, 1)
+    w, w_scale = oracle.fill_fp8_blocks(801, outputs, inner, 128)
+    out = run(device, a, a_scale, w, w_scale)
+    want64 = oracle.fp8_block_matmul_f64(a, a_scale, w, w_scale)
+    assert rel_frobenius(bf16_values(out), want64) <= TOLERANCE
+    wanted = oracle.bf16_to_f32(oracle.f32_to_bf16(want64.astype(np.float32)))
+    bound = 2.0**-7 * np.abs(wanted) + 1e-4 * np.abs(want64).max()
+    assert (np.abs(bf16_values(out) - wanted) <= bound).all()
+
+
 @pytest.mark.parametrize("code", list(range(20, 30)))
 @pytest.mark.parametrize("rows,outputs,inner", [(70, 300, 512), (256, 512, 128), (513, 260, 896)])
 def test_direct_lds_load_variants(device, code, rows, outputs, inner):
