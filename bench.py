@@ -688,7 +688,7 @@ def extras(torch, _kernels, _native, device, normal):
             counts = torch.full((experts,), fill, dtype=torch.int32, device=device)
             seconds = event_time(
                 torch, lambda i: _kernels.grouped_quantized_matmul(tokens, token_scale, table, order, counts,
-                                                                   outputs=features, packed=packed), 2, 5)
+                                                                   outputs=features, packed=packed), 10, 30)
             grouped[name + "_" + label] = {
                 "us": round(seconds * 1e6, 1),
                 "roofline": roofline_of("mfma fp8", 2.0 * experts * fill * features * inner, seconds)}
@@ -700,7 +700,7 @@ def extras(torch, _kernels, _native, device, normal):
     cache_v = normal((32, 8192, 8, 128))
     query = normal((32, 64, 128))
     live = torch.full((32,), 512, dtype=torch.int32, device=device)
-    seconds = event_time(torch, lambda i: _kernels.gqa_decode_attention(query, cache_k, cache_v, live), 3, 10)
+    seconds = event_time(torch, lambda i: _kernels.gqa_decode_attention(query, cache_k, cache_v, live), 20, 60)
     found["gqa_decode_512_live_of_8192"] = {
         "us": round(seconds * 1e6, 1), "roofline": roofline_of("hbm", 2 * 32 * 512 * 8 * 128 * 2, seconds)}
     del cache_k, cache_v, query
@@ -803,7 +803,7 @@ def extras(torch, _kernels, _native, device, normal):
             layer(0)
     stacked = event_time(torch, lambda i: stack.replay(), 5, 20) / layers
     traffic = LAYER_BYTES
-    seconds = event_time(torch, lambda i: attention(), 3, 20)
+    seconds = event_time(torch, lambda i: attention(), 20, 60)
     found["gqa_decode_attention_b32_ctx2048"] = {
         "us": round(seconds * 1e6, 1), "roofline": roofline_of("hbm", KV_BYTES, seconds),
     }
