@@ -242,7 +242,8 @@ bool mx_dma_supported(int outputs, int inner, const void *input, const void *wei
 hipError_t launch_mx_dma(hipStream_t stream, int variant, bool packed, int groups, int weight_groups,
                          int rows, int outputs, int inner, int activation_block, const void *input,
                          const void *input_scale, const void *weight, const void *weight_scale,
-                         const void *metadata, const void *active, const void *counts, void *out);
+                         const void *metadata, const void *active, const void *counts, void *out,
+                         int tail_variant = 0, int tail_outputs = 0);
 // Mixture-of-experts routing helpers.
 hipError_t launch_route_groups(hipStream_t stream, int tokens, int choices, int first_expert,
                                int groups, int rows, const void *experts, const void *active,

@@ -42,6 +42,7 @@ struct MxDmaParams {
     const unsigned long long *metadata;
     const int32_t *active, *counts;
     int weight_groups, groups;
+    int out_pitch; // elements between tokens in `out` (the outputs of the whole product)
 };
 
 __device__ __forceinline__ unsigned long long uniform(unsigned long long value)
@@ -185,12 +186,12 @@ __global__ __launch_bounds__(128 * WM) void mx_dma_kernel(MxDmaParams p)
         valid_rows = index >= 0 && index < p.weight_groups ? min(max(count, 0), p.rows) : 0;
         input += size_t(group) * p.rows * p.inner;
         input_scale += size_t(group) * p.rows * (WIDE_X ? p.steps : scale_pitch);
-        out += size_t(group) * p.rows * p.outputs;
+        out += size_t(group) * p.rows * p.out_pitch;
         if (m0 >= valid_rows) { // nothing to multiply: this tile of the output is zero
             for (int item = thread; item < BM * (BN / 4); item += 128 * WM) {
                 const int m = m0 + item / (BN / 4), n = n0 + (item % (BN / 4)) * 4;
                 if (m < p.rows && n < p.outputs)
-                    *reinterpret_cast<u32x2_t *>(out + size_t(m) * p.outputs + n) = u32x2_t{0u, 0u};
+                    *reinterpret_cast<u32x2_t *>(out + size_t(m) * p.out_pitch + n) = u32x2_t{0u, 0u};
             }
             return;
         }
@@ -479,7 +480,7 @@ __global__ __launch_bounds__(128 * WM) void mx_dma_kernel(MxDmaParams p)
     for (int j = 0; j < TM; ++j) {
         const int m = m0 + (wm * TM + j) * 32 + frag_row;
         const bool live = !GROUPED || m < valid_rows; // padding rows of a group are written as zeros
-        unsigned short *row = out + size_t(m) * p.outputs + n0 + wn * TN * 32 + half * 4;
+        unsigned short *row = out + size_t(m) * p.out_pitch + n0 + wn * TN * 32 + half * 4;
 #pragma unroll
         for (int i = 0; i < TN; ++i) {
             __builtin_amdgcn_sched_barrier(0);
@@ -548,14 +549,59 @@ bool mx_dma_supported(int outputs, int inner, const void *input, const void *wei
 }
 
 // groups == 0: plain product; >= 1: grouped (weights and their scales from the device table)
+namespace
+{
+// The plain product over outputs first .. first + count - 1 of `outputs` (first a multiple of 32).
+hipError_t launch_mx_dma_rows(hipStream_t stream, int variant, bool packed, int rows, int outputs, int first,
+                              int count, int inner, int activation_block, const void *input,
+                              const void *input_scale, const void *weight, const void *weight_scale, void *out)
+{
+    MxDmaParams p;
+    const size_t scale_pitch = size_t(inner / 32), weight_pitch = packed ? size_t(inner) / 2 : size_t(inner);
+    p.input = static_cast<const unsigned char *>(input);
+    p.input_scale = static_cast<const unsigned char *>(input_scale);
+    p.weight = static_cast<const unsigned char *>(weight) + size_t(first) * weight_pitch;
+    p.weight_scale = static_cast<const unsigned char *>(weight_scale) + size_t(packed ? first : first / 32) * scale_pitch;
+    p.out = static_cast<unsigned short *>(out) + first;
+    p.rows = rows;
+    p.outputs = count;
+    p.out_pitch = outputs;
+    p.inner = inner;
+    p.steps = inner / 128;
+    p.tiles_n = p.tiles_m = 0;
+    p.metadata = nullptr;
+    p.active = p.counts = nullptr;
+    p.weight_groups = 0;
+    if (!packed)
+        return launch_variant<false, false, false>(stream, p, 1, variant);
+    return activation_block == 128 ? launch_variant<true, true, false>(stream, p, 1, variant)
+                                   : launch_variant<true, false, false>(stream, p, 1, variant);
+}
+} // namespace
+
+// tail_outputs > 0 (plain product only): the last tail_outputs outputs, starting at a multiple of 256,
+// run on tail_variant in a launch of their own, so that both launches are whole rounds of
+// workgroups where one tiling would end in a partly filled round.
 hipError_t launch_mx_dma(hipStream_t stream, int variant, bool packed, int groups, int weight_groups,
                          int rows, int outputs, int inner, int activation_block, const void *input,
                          const void *input_scale, const void *weight, const void *weight_scale,
-                         const void *metadata, const void *active, const void *counts, void *out)
+                         const void *metadata, const void *active, const void *counts, void *out,
+                         int tail_variant, int tail_outputs)
 {
     if (!mx_dma_supported(outputs, inner, input, weight, out) ||
         (activation_block != 32 && !(packed && activation_block == 128)))
         return hipErrorInvalidValue;
+    if (tail_outputs) {
+        if (groups != 0 || tail_outputs < 0 || tail_outputs >= outputs || (outputs - tail_outputs) % 256)
+            return hipErrorInvalidValue;
+        const int first = outputs - tail_outputs;
+        hipError_t status = launch_mx_dma_rows(stream, variant, packed, rows, outputs, 0, first, inner, activation_block,
+                                               input, input_scale, weight, weight_scale, out);
+        if (status != hipSuccess)
+            return status;
+        return launch_mx_dma_rows(stream, tail_variant, packed, rows, outputs, first, tail_outputs, inner,
+                                  activation_block, input, input_scale, weight, weight_scale, out);
+    }
     MxDmaParams p;
     p.input = static_cast<const unsigned char *>(input);
     p.input_scale = static_cast<const unsigned char *>(input_scale);
@@ -564,6 +610,7 @@ hipError_t launch_mx_dma(hipStream_t stream, int variant, bool packed, int group
     p.out = static_cast<unsigned short *>(out);
     p.rows = rows;
     p.outputs = outputs;
+    p.out_pitch = outputs;
     p.inner = inner;
     p.steps = inner / 128;
     p.tiles_n = p.tiles_m = 0;

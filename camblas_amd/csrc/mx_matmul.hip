@@ -481,9 +481,40 @@ hipError_t launch_mx_matmul(hipStream_t stream, int kernel, int compute_units, b
         for (int candidate = 1; candidate < 4; ++candidate)
             if (cost[candidate] < cost[variant])
                 variant = candidate;
+        // A plain product whose 256 x 256 tiles end in a partly filled round: whole rounds over the
+        // first outputs, and the rest on the tile that covers them in the fewest weighted rounds
+        // (18432 outputs by 4096 tokens: four rounds, then 2048 outputs as one round of 256 x 128).
+        int tail_variant = 0, tail_outputs = 0;
+        if (groups == 0 && rows > 128) {
+            const long long token_tiles = (rows + 255) / 256;
+            const long long whole = tiles(256, 256) / compute_units;
+            const long long main_outputs = whole * compute_units / token_tiles * 256;
+            if (whole >= 1 && main_outputs > 0 && main_outputs < outputs) {
+                const int rest = outputs - int(main_outputs);
+                auto rest_tiles = [&](int tile_outputs, int tile_rows) {
+                    return static_cast<long long>((rest + tile_outputs - 1) / tile_outputs) * ((rows + tile_rows - 1) / tile_rows);
+                };
+                const double rest_cost[4] = {
+                    rounds(rest_tiles(256, 256)),
+                    rounds(rest_tiles(256, 128)) * (packed ? 0.6 : 0.57),
+                    !packed ? rounds(rest_tiles(192, 256)) * 0.84 : 1e30,
+                    rounds(rest_tiles(128, 128)) * (packed ? 0.45 : 0.43),
+                };
+                int best_rest = 0;
+                for (int candidate = 1; candidate < 4; ++candidate)
+                    if (rest_cost[candidate] < rest_cost[best_rest])
+                        best_rest = candidate;
+                // (a second launch costs about a twentieth of a round of large tiles)
+                if (double(whole) + rest_cost[best_rest] + 0.05 < 0.97 * cost[variant]) {
+                    variant = 0;
+                    tail_variant = best_rest;
+                    tail_outputs = rest;
+                }
+            }
+        }
         return launch_mx_dma(stream, variant, packed, groups, weight_groups, rows, outputs, inner,
                              activation_block, input, input_scale, weight, weight_scale, metadata,
-                             active, counts, out);
+                             active, counts, out, tail_variant, tail_outputs);
     }
     MxParams p;
     p.input = static_cast<const unsigned char *>(input);
