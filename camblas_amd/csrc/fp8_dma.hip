@@ -154,9 +154,9 @@ __global__ __launch_bounds__(128 * WM) void fp8_dma_kernel(Fp8DmaParams p)
         const int position = group % PERIOD;
         return lds_read_unordered(slab + as_index[j] + position / 4 * (TOKENS_PER_WAVE * 4) + position % 4);
     };
-    // The weight scales travel the same way: the tile's rows lie in at most four 128-row blocks,
-    // and lane l of one 4-byte-per-lane load brings group l % 8 of the slab for block l / 8 (every
-    // wavefront issues the same load: same bytes to the same place).
+    // The weight scales travel the same way: the tile's rows lie in two or three 128-row blocks
+    // (room for eight), and lane l of one 4-byte-per-lane load brings group l % 8 of the slab for
+    // block l / 8 (every wavefront issues the same load: same bytes to the same place).
     static_assert(SLAB_GROUPS == 8 && BN <= 7 * 128, "eight blocks of eight groups per load");
     auto weight_slab_at = [&](int index) {
         return reinterpret_cast<float *>(lds + STAGES * SLOTS + 2 * SLAB_SLOTS + (index & 1) * WEIGHT_SLAB_SLOTS);
