@@ -338,11 +338,23 @@ int launch_bf16_plan(const Entry &entry, Plan plan, const Product &p, float alph
         source = BetaSource{};
     }
     switch (plan.family) {
-    case FAMILY_DMA:
+    case FAMILY_DMA: {
         context->counts[plan.counter]++;
-        return entry.finish(launch_bgemm_dma(stream, plan.kernel, p.m, p.n, p.k, alpha, a, p.lda, b, p.ldb, beta,
-                                             c, p.ldc, source),
-                            "BF16 MFMA GEMM (direct LDS loads)");
+        // (a plan may end with a second launch over the last outputs, which would have made a
+        // partly filled last round of workgroups on the first tile)
+        const int first = p.m - plan.tail_outputs;
+        hipError_t status = launch_bgemm_dma(stream, plan.kernel, first, p.n, p.k, alpha, a, p.lda, b, p.ldb, beta,
+                                             c, p.ldc, source);
+        if (status == hipSuccess && plan.tail_outputs) {
+            const unsigned short *weights = static_cast<const unsigned short *>(a) + size_t(first) * p.lda;
+            BetaSource rest = source;
+            if (rest.z)
+                rest.z = static_cast<const unsigned short *>(rest.z) + first;
+            status = launch_bgemm_dma(stream, plan.tail_kernel, plan.tail_outputs, p.n, p.k, alpha, weights, p.lda,
+                                      b, p.ldb, beta, static_cast<unsigned short *>(c) + first, p.ldc, rest);
+        }
+        return entry.finish(status, "BF16 MFMA GEMM (direct LDS loads)");
+    }
     case FAMILY_STREAM: {
         StreamShares shares;
         if (plan.split_k > 1) {
@@ -469,6 +481,7 @@ int bf16_product(const Entry &entry, const Product &p, float alpha, const void *
         // tests: 0.. a register-staged tile variant (with override_split), 20..59 a direct-to-LDS
         // variant, 100 + 100*depth + 10*row_tiles + token_tiles the streaming kernel
         plan.split_k = 1;
+        plan.tail_outputs = 0;
         if (forced >= 100) {
             plan.family = FAMILY_STREAM;
             plan.kernel = forced - 100;

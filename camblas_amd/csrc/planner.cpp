@@ -211,6 +211,38 @@ Plan make_plan(int dtype, int algorithm, bool trans_a, bool trans_b, int m, int 
                         plan.kernel = candidate.variant;
                     }
                 }
+                // Two launches: whole rounds of one tile over the first outputs, then the outputs
+                // that would have made a partly filled last round on the tile that covers them
+                // cheapest. Costs in tile area per unit of efficiency; a second launch is priced
+                // like 5 us of a compute unit's work (0.38 ps per element of tile area and of K).
+                auto rounds_cost = [&](int rows, int variant, double weight) {
+                    const TnVariant &v = dma_variant(variant);
+                    const double tiles = double(ceil_div(rows, v.block_n)) * ceil_div(tokens, v.block_m);
+                    return std::ceil(tiles / compute_units) * v.block_n * v.block_m / weight;
+                };
+                double single = 1e300;
+                for (const auto &candidate : candidates)
+                    single = std::min(single, rounds_cost(outputs, candidate.variant, candidate.weight));
+                const double launch_cost = 5.0 / (3.8e-7 * k);
+                for (const auto &candidate : candidates) {
+                    const TnVariant &v = dma_variant(candidate.variant);
+                    const int token_tiles = ceil_div(tokens, v.block_m);
+                    const int whole = ceil_div(outputs, v.block_n) * token_tiles / compute_units;
+                    const int main_outputs = whole * compute_units / token_tiles * v.block_n;
+                    if (whole < 1 || main_outputs < 1 || main_outputs >= outputs)
+                        continue;
+                    const double main_cost = rounds_cost(main_outputs, candidate.variant, candidate.weight);
+                    for (const auto &tail : candidates) {
+                        const double cost =
+                            main_cost + rounds_cost(outputs - main_outputs, tail.variant, tail.weight) + launch_cost;
+                        if (cost < 0.97 * single) {
+                            single = cost / 0.97;
+                            plan.kernel = candidate.variant;
+                            plan.tail_kernel = tail.variant;
+                            plan.tail_outputs = outputs - main_outputs;
+                        }
+                    }
+                }
             } else {
                 const int candidates[3] = {0, 1, 2};
                 const int resident[3] = {1, 1, 2};
@@ -376,7 +408,11 @@ void describe_plan(const Plan &plan, int dtype, char *text, size_t bytes)
                       16 * (plan.kernel % 10));
         break;
     case FAMILY_DMA:
-        std::snprintf(text, bytes, "%s %s", type, dma_variant(plan.kernel).name);
+        if (plan.tail_outputs)
+            std::snprintf(text, bytes, "%s %s, last %d outputs %s", type, dma_variant(plan.kernel).name,
+                          plan.tail_outputs, dma_variant(plan.tail_kernel).name);
+        else
+            std::snprintf(text, bytes, "%s %s", type, dma_variant(plan.kernel).name);
         break;
     case FAMILY_STREAM:
         std::snprintf(text, bytes, "%s stream rows=%d tokens=%d k_step=%d k_shares=%d", type,

@@ -70,6 +70,9 @@ def test_planner_choices_for_the_baseline_shapes():
     # prefill: direct-to-LDS MFMA tile that divides 10240 x 4096 into exactly two waves of tiles
     code, text = describe(2, "T", "N", 10240, 4096, 8192, 8192, 8192, 10240)
     assert code // 1000 == 5 and "dma320x256" in text
+    # 2.8 rounds of 320 x 256 tiles: two whole rounds, and the last 4096 outputs as one round of 256 x 256
+    assert describe(2, "T", "N", 14336, 4096, 4096, 4096, 4096, 14336) == (
+        5010, "bf16 dma320x256x64s2w8, last 4096 outputs dma256x256x64s2w8")
     # K not a multiple of 64: register-staged MFMA tiles; unaligned operands and the other transpose
     # pairs: the layout-agnostic matrix-core kernel; slivers and the classical policy: vector-ALU tiles
     assert describe(2, "T", "N", 10240, 4096, 8200, 8200, 8200, 10240)[0] // 1000 == 2
