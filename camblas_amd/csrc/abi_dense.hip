@@ -322,6 +322,16 @@ template <typename T> struct BackwardPass {
     }
 };
 
+// The register-staged plan for a product whose output or addend the direct-to-LDS kernel cannot
+// take (8-byte stores and loads): the tile of the same shape, or the nearest one, one launch.
+void use_register_staged_tiles(Plan &plan)
+{
+    const TnVariant &tile = dma_variant(plan.kernel);
+    plan.family = FAMILY_MFMA_TN;
+    plan.kernel = tile.block_n >= 256 && tile.block_m >= 256 ? 0 : tile.block_n >= 256 ? 1 : 2;
+    plan.tail_outputs = 0;
+}
+
 // Launches one planned BF16 product. `reserved`: FP32 room for a split K that the caller already
 // holds inside the context's arena (null: reserve it here).
 int launch_bf16_plan(const Entry &entry, Plan plan, const Product &p, float alpha, const void *a, const void *b,
@@ -343,8 +353,18 @@ int launch_bf16_plan(const Entry &entry, Plan plan, const Product &p, float alph
         // (a plan may end with a second launch over the last outputs, which would have made a
         // partly filled last round of workgroups on the first tile)
         const int first = p.m - plan.tail_outputs;
+        float *partials = reserved;
+        if (plan.split_k > 1 && !partials) {
+            // without room for the partials (allocation failure, capture in progress) run undivided
+            if (reserve_scratch(context, size_t(plan.split_k) * size_t(p.m) * size_t(p.n) * 4) == hipSuccess) {
+                partials = static_cast<float *>(context->scratch);
+            } else {
+                context->counts[5]++;
+                plan.split_k = 1;
+            }
+        }
         hipError_t status = launch_bgemm_dma(stream, plan.kernel, first, p.n, p.k, alpha, a, p.lda, b, p.ldb, beta,
-                                             c, p.ldc, source);
+                                             c, p.ldc, source, plan.split_k, partials);
         if (status == hipSuccess && plan.tail_outputs) {
             const unsigned short *weights = static_cast<const unsigned short *>(a) + size_t(first) * p.lda;
             BetaSource rest = source;
@@ -427,9 +447,9 @@ int bf16_product_transposing(const Entry &entry, const Product &p, float alpha, 
     Plan plan = make_plan(2, context->algorithm, 1, 0, q.m, q.n, q.k, q.lda, q.ldb, q.ldc, aligned,
                           context->compute_units);
     if (plan.family == FAMILY_DMA && (!is_aligned(c, 8) || !is_aligned(source.z, 8) || source.ldz % 4))
-        plan.family = FAMILY_MFMA_TN;
+        use_register_staged_tiles(plan);
     size_t partial_bytes = 0; // room for a divided K, held in the same arena behind the copies
-    if (plan.split_k > 1 && plan.family == FAMILY_MFMA_TN)
+    if (plan.split_k > 1 && (plan.family == FAMILY_MFMA_TN || plan.family == FAMILY_DMA))
         partial_bytes = size_t(plan.split_k) * size_t(p.m) * size_t(p.n) * 4;
     else if (plan.split_k > 1 && plan.family == FAMILY_STREAM)
         partial_bytes = stream_partial_bytes(plan.kernel / 10 % 10, plan.kernel % 10, p.m, p.n, plan.split_k);
@@ -462,7 +482,7 @@ int bf16_product(const Entry &entry, const Product &p, float alpha, const void *
     Plan plan = make_plan(2, context->algorithm, p.trans_a, p.trans_b, p.m, p.n, p.k, p.lda, p.ldb, p.ldc,
                           is_aligned(a, 16) && is_aligned(b, 16), context->compute_units);
     if (plan.family == FAMILY_DMA && (!is_aligned(c, 8) || !is_aligned(source.z, 8) || source.ldz % 4))
-        plan.family = FAMILY_MFMA_TN; // same tile shapes, register-staged loads, scalar stores
+        use_register_staged_tiles(plan); // register-staged loads, scalar stores
     const int forced = context->override_kernel;
     if (plan.family == FAMILY_MFMA_BF16) {
         // tests: 60 keeps the layout-agnostic kernel, 61 takes the transposing route whatever the size
@@ -489,6 +509,7 @@ int bf16_product(const Entry &entry, const Product &p, float alpha, const void *
         } else if (forced >= 20 && forced < 60) {
             plan.family = FAMILY_DMA;
             plan.kernel = forced - 20;
+            plan.split_k = std::max(1, context->override_split);
         } else {
             plan.family = FAMILY_MFMA_TN;
             plan.kernel = forced;

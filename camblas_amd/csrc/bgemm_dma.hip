@@ -10,6 +10,9 @@
 // compiler can tell the in-flight stage from the one being read. Fragments of the next 16-deep
 // step are read while the current step's MFMAs issue. Workgroups are renumbered per XCD so the
 // tiles resident on one XCD share W and x panels through its L2.
+// With few tokens the tiles of a projection leave compute units idle; the K steps of a tile can then
+// be divided over gridDim.y workgroups, which leave FP32 planes that sum_shares_kernel adds in share
+// order and finishes with alpha, beta and the addend.
 // Shape requirements (the planner checks them): K % 64 == 0, N % 4 == 0, ldc % 4 == 0, 16-byte
 // aligned operands, 8-byte aligned y.
 // Contract: ref src/cuda/bfloat16.cuh:11-57 ('T','N' call of src/cuda/torch_bindings.cpp:155-199).
@@ -30,6 +33,10 @@ struct DmaParams {
     int n, m, k;
     float alpha, beta;
     int tiles_n, tiles_m;
+    // K divided over gridDim.y workgroups per tile: each takes `share_steps` steps of BK and leaves
+    // its FP32 sums in plane blockIdx.y of `partials` ([share][token][feature])
+    float *partials;
+    int share_steps;
 };
 
 // TN, TM: 32x32 MFMA tiles per wavefront along features / tokens; the workgroup has 2 x WM
@@ -59,7 +66,8 @@ __global__ __launch_bounds__(128 * WM) void bgemm_dma_kernel(DmaParams p)
     int tile_n, tile_m;
     xcd_tile(int(blockIdx.x), p.tiles_n, p.tiles_m, tile_n, tile_m);
     const int n0 = tile_n * BN, m0 = tile_m * BM;
-    const int k_tiles = p.k / BK;
+    const int first_step = int(blockIdx.y) * p.share_steps;
+    const int k_tiles = p.k / BK - first_step < p.share_steps ? p.k / BK - first_step : p.share_steps;
 
     const int thread = threadIdx.x, lane = thread % 64, wave = thread / 64;
     const int wn = wave % 2, wm = wave / 2; // 2 x WM wavefront grid
@@ -86,7 +94,7 @@ __global__ __launch_bounds__(128 * WM) void bgemm_dma_kernel(DmaParams p)
         p.w + size_t(n0) * p.lda, (unsigned(a_rows - 1) * unsigned(p.lda) + unsigned(p.k)) * 2u);
     const __amdgpu_buffer_rsrc_t b_resource = make_resource(
         p.x + size_t(m0) * p.ldb, (unsigned(b_rows - 1) * unsigned(p.ldb) + unsigned(p.k)) * 2u);
-    unsigned k_bytes = 0;
+    unsigned k_bytes = unsigned(first_step) * BK * 2;
     // Load number `index` (0 .. LOADS-1) of the K block at k_bytes.
     auto issue_one = [&](u32x4_t *stage, int index) {
         if (index < A_ITERS)
@@ -171,7 +179,7 @@ __global__ __launch_bounds__(128 * WM) void bgemm_dma_kernel(DmaParams p)
         mfma(a_frag[(KS - 1) & 1], b_frag[(KS - 1) & 1]);
         __builtin_amdgcn_sched_barrier(0);
     };
-    const unsigned last_k_bytes = unsigned(k_tiles - 1) * BK * 2;
+    const unsigned last_k_bytes = unsigned(first_step + k_tiles - 1) * BK * 2;
     auto clamp_k = [&]() { k_bytes = k_bytes < last_k_bytes ? k_bytes : last_k_bytes; };
 
     // prologue: STAGES - 1 steps in flight, the first one complete
@@ -221,6 +229,26 @@ __global__ __launch_bounds__(128 * WM) void bgemm_dma_kernel(DmaParams p)
 
     // ---- epilogue. Accumulator register 4q+e of lane l is feature 8q + 4*(l/32) + e, token l%32.
     const int first_feature = n0 + wn * TN * 32 + half * 4;
+    if (gridDim.y > 1) {
+        // a share of K: the plain sums, for sum_shares_kernel
+#pragma unroll
+        for (int j = 0; j < TM; ++j)
+#pragma unroll
+            for (int i = 0; i < TN; ++i) {
+                const int m = m0 + (wm * TM + j) * 32 + frag_row;
+                float *row = p.partials + (size_t(blockIdx.y) * p.m + m) * p.n + first_feature;
+#pragma unroll
+                for (int q = 0; q < 4; ++q) {
+                    const int offset = i * 32 + q * 8;
+                    if (m < p.m && first_feature + offset < p.n) {
+                        const f32x4_t sums = {acc[i][j][q * 4], acc[i][j][q * 4 + 1], acc[i][j][q * 4 + 2],
+                                              acc[i][j][q * 4 + 3]};
+                        *reinterpret_cast<f32x4_t *>(row + offset) = sums;
+                    }
+                }
+            }
+        return;
+    }
     auto store_tile = [&](int i, int j, const u32x2_t (&old)[4], bool with_beta) {
         const int m = m0 + (wm * TM + j) * 32 + frag_row;
         unsigned short *row = p.y + size_t(m) * p.ldc + first_feature;
@@ -282,8 +310,38 @@ __global__ __launch_bounds__(128 * WM) void bgemm_dma_kernel(DmaParams p)
     }
 }
 
+// y = alpha * (plane 0 + plane 1 + ...) + beta * z over the shares of a divided K, four features per
+// thread, the planes added in index order so that the result does not depend on scheduling.
+__global__ __launch_bounds__(256) void sum_shares_kernel(DmaParams p, int shares)
+{
+    const size_t quad = size_t(blockIdx.x) * 256 + threadIdx.x, per_row = size_t(p.n / 4);
+    if (quad >= per_row * size_t(p.m))
+        return;
+    const size_t m = quad / per_row, feature = quad % per_row * 4, plane = size_t(p.m) * p.n;
+    const float *source = p.partials + m * p.n + feature;
+    f32x4_t sum = *reinterpret_cast<const f32x4_t *>(source);
+    for (int share = 1; share < shares; ++share) {
+        const f32x4_t more = *reinterpret_cast<const f32x4_t *>(source + share * plane);
+#pragma unroll
+        for (int e = 0; e < 4; ++e)
+            sum[e] += more[e];
+    }
+#pragma unroll
+    for (int e = 0; e < 4; ++e)
+        sum[e] *= p.alpha;
+    if (p.beta != 0.f) {
+        const u32x2_t old = *reinterpret_cast<const u32x2_t *>(p.z + m * p.ldz + feature);
+        sum[0] = fmaf(p.beta, __uint_as_float(old[0] << 16), sum[0]);
+        sum[1] = fmaf(p.beta, __uint_as_float(old[0] & 0xffff0000u), sum[1]);
+        sum[2] = fmaf(p.beta, __uint_as_float(old[1] << 16), sum[2]);
+        sum[3] = fmaf(p.beta, __uint_as_float(old[1] & 0xffff0000u), sum[3]);
+    }
+    const u32x2_t packed = {pack_bf16x2(sum[0], sum[1]), pack_bf16x2(sum[2], sum[3])};
+    *reinterpret_cast<u32x2_t *>(p.y + m * p.ldc + feature) = packed;
+}
+
 template <int TN, int TM, int WM, int BK, int STAGES>
-hipError_t launch_dma(hipStream_t stream, DmaParams p)
+hipError_t launch_dma(hipStream_t stream, DmaParams p, int shares)
 {
     constexpr int BN = 64 * TN, BM = 32 * WM * TM;
     if (p.k % BK)
@@ -292,8 +350,16 @@ hipError_t launch_dma(hipStream_t stream, DmaParams p)
     p.tiles_m = (p.m + BM - 1) / BM;
     if (size_t(p.tiles_n) * size_t(p.tiles_m) > 0x7fffffffu)
         return hipErrorInvalidValue;
-    bgemm_dma_kernel<TN, TM, WM, BK, STAGES>
-        <<<unsigned(p.tiles_n) * unsigned(p.tiles_m), 128 * WM, 0, stream>>>(p);
+    const int steps = p.k / BK;
+    p.share_steps = (steps + shares - 1) / shares;
+    shares = (steps + p.share_steps - 1) / p.share_steps; // no empty share
+    const dim3 grid(unsigned(p.tiles_n) * unsigned(p.tiles_m), unsigned(shares));
+    bgemm_dma_kernel<TN, TM, WM, BK, STAGES><<<grid, 128 * WM, 0, stream>>>(p);
+    const hipError_t status = launch_status();
+    if (shares == 1 || status != hipSuccess)
+        return status;
+    const size_t quads = size_t(p.m) * size_t(p.n / 4);
+    sum_shares_kernel<<<unsigned((quads + 255) / 256), 256, 0, stream>>>(p, shares);
     return launch_status();
 }
 
@@ -312,9 +378,12 @@ const TnVariant &dma_variant(int index) { return variants[index]; }
 
 hipError_t launch_bgemm_dma(hipStream_t stream, int variant, int n_out, int m_rows, int k,
                             float alpha, const void *w, int lda, const void *x, int ldb, float beta,
-                            void *y, int ldc, const BetaSource &source)
+                            void *y, int ldc, const BetaSource &source, int shares, float *partials)
 {
     if (k % 64 || n_out % 4 || ldc % 4 || reinterpret_cast<uintptr_t>(y) % 8)
+        return hipErrorInvalidValue;
+    if (shares < 1 || shares > 64 || (shares > 1 && !partials) ||
+        size_t(m_rows) * size_t(n_out / 4) > size_t(0x7fffffff) * 256)
         return hipErrorInvalidValue;
     if (source.z && (source.ldz % 4 || reinterpret_cast<uintptr_t>(source.z) % 8))
         return hipErrorInvalidValue;
@@ -336,19 +405,21 @@ hipError_t launch_bgemm_dma(hipStream_t stream, int variant, int n_out, int m_ro
     p.alpha = alpha;
     p.beta = beta;
     p.tiles_n = p.tiles_m = 0;
+    p.partials = partials;
+    p.share_steps = 0;
     switch (variant) {
-    case 0: return launch_dma<4, 4, 2, 32, 4>(stream, p);
-    case 1: return launch_dma<4, 2, 2, 64, 3>(stream, p);
-    case 2: return launch_dma<2, 2, 2, 64, 2>(stream, p);
-    case 3: return launch_dma<4, 4, 2, 32, 3>(stream, p);
-    case 4: return launch_dma<4, 2, 2, 64, 2>(stream, p);
-    case 5: return launch_dma<2, 2, 2, 64, 3>(stream, p);
-    case 6: return launch_dma<4, 2, 4, 64, 2>(stream, p);
-    case 7: return launch_dma<4, 2, 4, 32, 4>(stream, p);
-    case 8: return launch_dma<4, 1, 4, 64, 3>(stream, p);
-    case 9: return launch_dma<2, 2, 4, 64, 3>(stream, p);
-    case 10: return launch_dma<5, 2, 4, 64, 2>(stream, p);
-    case 11: return launch_dma<3, 2, 4, 64, 2>(stream, p);
+    case 0: return launch_dma<4, 4, 2, 32, 4>(stream, p, shares);
+    case 1: return launch_dma<4, 2, 2, 64, 3>(stream, p, shares);
+    case 2: return launch_dma<2, 2, 2, 64, 2>(stream, p, shares);
+    case 3: return launch_dma<4, 4, 2, 32, 3>(stream, p, shares);
+    case 4: return launch_dma<4, 2, 2, 64, 2>(stream, p, shares);
+    case 5: return launch_dma<2, 2, 2, 64, 3>(stream, p, shares);
+    case 6: return launch_dma<4, 2, 4, 64, 2>(stream, p, shares);
+    case 7: return launch_dma<4, 2, 4, 32, 4>(stream, p, shares);
+    case 8: return launch_dma<4, 1, 4, 64, 3>(stream, p, shares);
+    case 9: return launch_dma<2, 2, 4, 64, 3>(stream, p, shares);
+    case 10: return launch_dma<5, 2, 4, 64, 2>(stream, p, shares);
+    case 11: return launch_dma<3, 2, 4, 64, 2>(stream, p, shares);
     default: return hipErrorInvalidValue;
     }
 }

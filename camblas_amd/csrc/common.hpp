@@ -174,7 +174,8 @@ hipError_t launch_bgemm_tn(hipStream_t stream, int variant, int split_k, int n_o
 // Needs k % 64 == 0, n_out % 4 == 0, ldc % 4 == 0, y 8-byte aligned (and the same of a beta source).
 hipError_t launch_bgemm_dma(hipStream_t stream, int variant, int n_out, int m_rows, int k,
                             float alpha, const void *w, int lda, const void *x, int ldb, float beta,
-                            void *y, int ldc, const BetaSource &source = {});
+                            void *y, int ldc, const BetaSource &source = {}, int shares = 1,
+                            float *partials = nullptr);
 // Decode-shaped BF16 linear: each workgroup streams 16*row_tiles weight rows over the whole K.
 // depth_log2: a K step is 2^depth_log2 blocks of 128 elements (0..3); row_tiles << depth_log2 <= 8
 // and (row_tiles + token_tiles) << depth_log2 <= 16 or the launch is refused.

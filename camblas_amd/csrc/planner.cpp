@@ -85,6 +85,37 @@ double occupancy_score(int n, int m, int block_n, int block_m, int resident, int
     double fill = (double(n) * m) / (tiles * block_n * block_m);
     return tiles / (rounds * slots) * fill;
 }
+
+// Estimated microseconds of one launch of a direct-to-LDS BF16 tile over `outputs` weight rows with
+// K divided over `shares` workgroups per tile, fitted to sweeps of six tiles and 1..8 shares over
+// ten projection shapes at 65..1536 tokens (the choice by this estimate is within 2 % of the best
+// measured kernel in the geometric mean, 20 % at worst). The longer of two terms: rounds of
+// workgroups times steps times the tile's time per 64-deep step; and the weights streamed at what
+// the workgroups in flight can draw (each keeps the stages it is not reading in flight for 2.6 us,
+// together at most 5.2 TB/s; a partly filled last round draws less). A divided K adds the second
+// kernel and the traffic of the FP32 planes.
+struct DmaPrice {
+    int variant;
+    double step_us, kilobytes_in_flight;
+};
+const DmaPrice dma_prices[] = {{5, 0.580, 64}, {9, 0.849, 96}, {6, 1.682, 64},
+                               {8, 0.943, 96}, {10, 1.878, 72}, {11, 1.281, 56}};
+double dma_launch_us(const DmaPrice &price, int outputs, int tokens, int k, int shares, int compute_units)
+{
+    const TnVariant &v = dma_variant(price.variant);
+    const double workgroups = double(ceil_div(outputs, v.block_n)) * ceil_div(tokens, v.block_m) * shares;
+    const double rounds = std::ceil(workgroups / compute_units);
+    const double steps = ceil_div(ceil_div(k, 64), shares);
+    const double bytes_per_us =
+        std::min(5.183e6, std::min(workgroups, double(compute_units)) * price.kilobytes_in_flight * 1024 / 2.601);
+    double stream_us = double(outputs) * k * 2 / bytes_per_us;
+    if (workgroups > compute_units)
+        stream_us *= rounds * compute_units / workgroups;
+    double us = 0.8 + std::max(rounds * steps * price.step_us, stream_us);
+    if (shares > 1)
+        us += 1.553 + 2.0 * shares * double(tokens) * outputs * 4 / 4.517e6;
+    return us;
+}
 } // namespace
 
 Plan make_plan(int dtype, int algorithm, bool trans_a, bool trans_b, int m, int n, int k, int lda,
@@ -176,6 +207,50 @@ Plan make_plan(int dtype, int algorithm, bool trans_a, bool trans_b, int m, int 
             while (plan.split_k < 16 && tiles * plan.split_k * 2 * 2 <= 5 * compute_units &&
                    k / (plan.split_k * 2) >= 512)
                 plan.split_k *= 2;
+        } else if (tokens <= 1536 && k % 64 == 0 && k >= 512 && outputs % 4 == 0 && ldc % 4 == 0 &&
+                   lda < (1 << 22) && ldb < (1 << 22)) {
+            // 65..1536 tokens: the direct-to-LDS tile, the number of workgroups K is divided over
+            // and, where a tile would end in a partly filled round, the tile of a second launch
+            // over the last outputs, all by estimated time. (Measured against the rules below,
+            // which this replaced: [8192, 8192] x 256 tokens 58 -> 47 us, [10240, 8192] x 256
+            // 77 -> 56, [4096, 14336] x 384 79 -> 59, [8192, 28672] x 384 305 -> 234.)
+            plan.family = FAMILY_DMA;
+            double best = 1e300;
+            const int shares[] = {1, 2, 3, 4, 6, 8};
+            for (const DmaPrice &price : dma_prices)
+                for (const int count : shares) {
+                    const TnVariant &v = dma_variant(price.variant);
+                    const double workgroups = double(ceil_div(outputs, v.block_n)) * ceil_div(tokens, v.block_m) * count;
+                    if (count > 1 && (k / count < 512 || workgroups > 2.0 * compute_units ||
+                                      double(count) * tokens * outputs * 4 > double(1 << 28)))
+                        continue;
+                    const double us = dma_launch_us(price, outputs, tokens, k, count, compute_units);
+                    if (us < best) {
+                        best = us;
+                        plan.kernel = price.variant;
+                        plan.split_k = count;
+                    }
+                }
+            for (const DmaPrice &main : dma_prices) {
+                const TnVariant &v = dma_variant(main.variant);
+                const int token_tiles = ceil_div(tokens, v.block_m);
+                const int whole = ceil_div(outputs, v.block_n) * token_tiles / compute_units;
+                const int main_outputs = whole * compute_units / token_tiles * v.block_n;
+                if (whole < 1 || main_outputs < 1 || main_outputs >= outputs)
+                    continue;
+                const double main_us = dma_launch_us(main, main_outputs, tokens, k, 1, compute_units);
+                for (const DmaPrice &tail : dma_prices) {
+                    const double us =
+                        main_us + dma_launch_us(tail, outputs - main_outputs, tokens, k, 1, compute_units) + 3.0;
+                    if (us < 0.97 * best) {
+                        best = us / 0.97;
+                        plan.kernel = main.variant;
+                        plan.split_k = 1;
+                        plan.tail_kernel = tail.variant;
+                        plan.tail_outputs = outputs - main_outputs;
+                    }
+                }
+            }
         } else if (ceil_div(outputs, 128) * ceil_div(tokens, 128) * 2 <= compute_units) {
             // few output tiles (a narrow projection, a small batch): 128 x 128 register-staged
             // tiles with K divided over workgroups, the largest power-of-two split that keeps the
@@ -411,6 +486,8 @@ void describe_plan(const Plan &plan, int dtype, char *text, size_t bytes)
         if (plan.tail_outputs)
             std::snprintf(text, bytes, "%s %s, last %d outputs %s", type, dma_variant(plan.kernel).name,
                           plan.tail_outputs, dma_variant(plan.tail_kernel).name);
+        else if (plan.split_k > 1)
+            std::snprintf(text, bytes, "%s %s split_k=%d", type, dma_variant(plan.kernel).name, plan.split_k);
         else
             std::snprintf(text, bytes, "%s %s", type, dma_variant(plan.kernel).name);
         break;

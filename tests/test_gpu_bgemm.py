@@ -119,6 +119,31 @@ def test_direct_lds_load_kernel(device, code, n_out, m_rows, k):
         assert np.array_equal(got2d[:, n_out:], c0.reshape(m_rows, ldc)[:, n_out:])
 
 
+@pytest.mark.parametrize("code", [22, 25, 29, 30])
+@pytest.mark.parametrize("shares", [2, 3, 7])
+def test_direct_lds_load_kernel_with_k_divided_over_workgroups(device, code, shares):
+    # 7 steps of 64 over 2 (4 + 3), 3 (3 + 3 + 1) and 7 workgroups per tile; FP32 planes summed in
+    # share order by a second kernel, which also applies alpha, beta and the addend
+    n_out, m_rows, k = 260, 513, 448
+    lda, ldb, ldc = k + 8, k + 16, n_out + 4
+    w = oracle.fill_normal_bf16(320 + code, (n_out * lda,))
+    x = oracle.fill_normal_bf16(340 + code, (m_rows * ldb,))
+    c0 = oracle.fill_normal_bf16(360, (m_rows * ldc,))
+    for alpha, beta in ((1.0, 0.0), (0.5, -1.5)):
+        got = run_bgemm(device, "T", "N", n_out, m_rows, k, alpha, w, lda, x, ldb, beta, c0, ldc,
+                        override=(code, shares))
+        want, want64 = reference("T", "N", n_out, m_rows, k, alpha, w, lda, x, ldb, beta, c0, ldc)
+        got2d = got.reshape(m_rows, ldc)
+        error = rel_frobenius(oracle.bf16_to_f32(got2d[:, :n_out]), want64.reshape(m_rows, n_out))
+        assert error <= TOLERANCE, (code, alpha, beta, error)
+        assert np.array_equal(got2d[:, n_out:], c0.reshape(m_rows, ldc)[:, n_out:])
+    # one share per step: each plane is an exact product of a 64-deep slice, so the sum in share
+    # order is reproducible run to run
+    again = run_bgemm(device, "T", "N", n_out, m_rows, k, 0.5, w, lda, x, ldb, -1.5, c0, ldc,
+                      override=(code, shares))
+    assert np.array_equal(got, again)
+
+
 @pytest.mark.parametrize("tokens", [1, 8, 32, 33, 64, 65, 200])
 def test_planned_linear_shapes(device, tokens):
     # aligned fast path as F.linear produces it; planner picks variant and split-K
@@ -367,6 +392,7 @@ def spread(z, ldz, m, n, c, ldc):
     ("T", "N", 300, 70, 328, (1, 3)),      # ... with a split K and the ordered reduction
     ("T", "N", 301, 9, 328, (121, 1)),     # streaming kernel, scalar stores
     ("T", "N", 512, 256, 320, (21, 1)),    # direct-to-LDS tiles
+    ("T", "N", 512, 256, 320, (25, 2)),    # ... with K divided and the planes summed by a second kernel
     ("T", "N", 1024, 40, 512, None),       # the planner's choice for a decode batch
     ("N", "N", 200, 150, 72, None),        # any-layout matrix-core kernel: addend spread first
     ("N", "T", 9, 7, 5, None),             # generic kernel: addend spread first
