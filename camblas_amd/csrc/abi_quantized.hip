@@ -225,9 +225,21 @@ extern "C" int camblas_cuda_quantized_matmul(camblas_cuda_context *context, int 
             !apart(output, {input, input_scale, weight, weight_scale}))
             return entry.refuse("invalid quantized matrix buffers");
         context->counts[4]++;
+        // K divided over several workgroups per tile needs FP32 planes; without them (allocation
+        // failure, capture in progress) the same tiles run with K undivided
+        const int shares = mx_matmul_shares(context->override_kernel, context->override_split, context->compute_units,
+                                            packed != 0, rows, outputs, inner, input, weight, output);
+        float *planes = nullptr;
+        if (shares > 1) {
+            if (reserve_scratch(context, size_t(shares) * size_t(rows) * size_t(outputs) * 4) == hipSuccess)
+                planes = static_cast<float *>(context->scratch);
+            else
+                context->counts[5]++;
+        }
         return entry.finish(launch_mx_matmul(context->stream, context->override_kernel, context->compute_units,
                                              packed != 0, 0, 0, rows, outputs, inner, activation_block, input,
-                                             input_scale, weight, weight_scale, nullptr, nullptr, nullptr, output),
+                                             input_scale, weight, weight_scale, nullptr, nullptr, nullptr, output,
+                                             context->override_split, planes),
                             "quantized matrix multiplication");
     });
 }

@@ -235,7 +235,12 @@ hipError_t launch_mx_matmul(hipStream_t stream, int kernel, int compute_units, b
                             int weight_groups, int rows, int outputs, int inner,
                             int activation_block, const void *input,
                             const void *input_scale, const void *weight, const void *weight_scale,
-                            const void *metadata, const void *active, const void *counts, void *out);
+                            const void *metadata, const void *active, const void *counts, void *out,
+                            int forced_shares = 0, float *planes = nullptr);
+// Workgroups that launch_mx_matmul would divide K over for a plain product (1: K is not divided);
+// `planes` then needs that many times rows * outputs floats, and without it K is not divided.
+int mx_matmul_shares(int kernel, int forced_shares, int compute_units, bool packed, int rows, int outputs,
+                     int inner, const void *input, const void *weight, const void *out);
 // Prefill-sized E8M0 product (hardware-scaled matrix instructions, operands loaded straight into
 // LDS); needs inner % 128 == 0, 16-byte aligned operands and an 8-byte aligned output.
 int mx_dma_variant_count();
@@ -244,7 +249,7 @@ hipError_t launch_mx_dma(hipStream_t stream, int variant, bool packed, int group
                          int rows, int outputs, int inner, int activation_block, const void *input,
                          const void *input_scale, const void *weight, const void *weight_scale,
                          const void *metadata, const void *active, const void *counts, void *out,
-                         int tail_variant = 0, int tail_outputs = 0);
+                         int tail_variant = 0, int tail_outputs = 0, int shares = 1, float *planes = nullptr);
 // Mixture-of-experts routing helpers.
 hipError_t launch_route_groups(hipStream_t stream, int tokens, int choices, int first_expert,
                                int groups, int rows, const void *experts, const void *active,

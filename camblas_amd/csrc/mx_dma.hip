@@ -43,6 +43,10 @@ struct MxDmaParams {
     const int32_t *active, *counts;
     int weight_groups, groups;
     int out_pitch; // elements between tokens in `out` (the outputs of the whole product)
+    // plain product with K divided over gridDim.y workgroups per tile: each takes `share_steps` steps
+    // and leaves its FP32 sums in plane blockIdx.y of `planes` ([share][token][output of this launch])
+    float *planes;
+    int share_steps;
 };
 
 __device__ __forceinline__ unsigned long long uniform(unsigned long long value)
@@ -199,6 +203,16 @@ __global__ __launch_bounds__(128 * WM) void mx_dma_kernel(MxDmaParams p)
         weight_scale = reinterpret_cast<const unsigned char *>(uniform(p.metadata[2 * size_t(index) + 1]));
     }
 
+    // a share of K: the same kernel over steps first_step .. first_step + steps - 1, by moving every
+    // operand to its first step (scale words are four bytes per step, so their alignment is kept)
+    constexpr unsigned W_STEP_BYTES = PACKED ? BK / 2 : BK;
+    const int first_step = GROUPED ? 0 : int(blockIdx.y) * p.share_steps;
+    const int steps = GROUPED ? p.steps : (p.steps - first_step < p.share_steps ? p.steps - first_step : p.share_steps);
+    weight += size_t(first_step) * W_STEP_BYTES;
+    input += size_t(first_step) * BK;
+    weight_scale += size_t(first_step) * 4;
+    input_scale += size_t(first_step) * (WIDE_X ? 1 : 4);
+
     // ---- operand loads. Lane -> (row inside one wavefront load, swizzled chunk); successive loads
     // of a thread are WAVES*rows apart, which leaves the swizzle unchanged, so one lane offset
     // serves all of them and the row advance goes into the wave-uniform offset.
@@ -212,12 +226,11 @@ __global__ __launch_bounds__(128 * WM) void mx_dma_kernel(MxDmaParams p)
     const unsigned x_row_step = unsigned(WAVES * X_ROWS) * unsigned(p.inner);
     const int w_rows = p.outputs - n0 < BN ? p.outputs - n0 : BN;
     const int x_rows = valid_rows - m0 < BM ? valid_rows - m0 : BM;
-    const __amdgpu_buffer_rsrc_t w_resource =
-        make_resource(weight + size_t(n0) * w_pitch, unsigned(w_rows) * w_pitch);
-    const __amdgpu_buffer_rsrc_t x_resource =
-        make_resource(input + size_t(m0) * p.inner, unsigned(x_rows) * unsigned(p.inner));
-    constexpr unsigned W_STEP_BYTES = PACKED ? BK / 2 : BK;
-    const int last_step = p.steps - 1;
+    const __amdgpu_buffer_rsrc_t w_resource = make_resource(
+        weight + size_t(n0) * w_pitch, unsigned(w_rows) * w_pitch - unsigned(first_step) * W_STEP_BYTES);
+    const __amdgpu_buffer_rsrc_t x_resource = make_resource(
+        input + size_t(m0) * p.inner, unsigned(x_rows) * unsigned(p.inner) - unsigned(first_step) * BK);
+    const int last_step = steps - 1;
     int load_step = 0;
     auto issue_one = [&](u32x4_t *stage, int index) {
         if (index < A_ITERS)
@@ -261,7 +274,8 @@ __global__ __launch_bounds__(128 * WM) void mx_dma_kernel(MxDmaParams p)
         slab_lane_off = unsigned(row) * unsigned(scale_pitch);
         const unsigned skew = piece_of_weights ? w_skew : x_skew;
         slab_resource = uniform_descriptor((piece_of_weights ? weight_scale : input_scale) - skew,
-                                           unsigned(rows) * unsigned(scale_pitch) + (skew ? 4u : 0u));
+                                           unsigned(rows) * unsigned(scale_pitch) + (skew ? 4u : 0u) -
+                                               unsigned(first_step) * 4u);
     }
     // E4M3 weights: one scale row per 32 weight rows; lane l brings word l % 4 of the slab for the
     // tile's block l / 4 (every wavefront issues the same load: same bytes to the same place)
@@ -269,7 +283,8 @@ __global__ __launch_bounds__(128 * WM) void mx_dma_kernel(MxDmaParams p)
     const int lane_block = n0 / 32 + lane / 4 < block_rows ? n0 / 32 + lane / 4 : block_rows - 1;
     const unsigned block_lane_off = unsigned(lane_block) * unsigned(scale_pitch) + unsigned(lane % 4) * 4u;
     const u32x4_t block_resource =
-        uniform_descriptor(weight_scale - w_skew, unsigned(block_rows) * unsigned(scale_pitch) + (w_skew ? 4u : 0u));
+        uniform_descriptor(weight_scale - w_skew, unsigned(block_rows) * unsigned(scale_pitch) + (w_skew ? 4u : 0u) -
+                                                      unsigned(first_step) * 4u);
     auto load_slabs = [&](int slab) {
         if constexpr (PIECES > 0)
             load_to_lds_untracked(slab_resource, slab_lane_off, unsigned(slab * PERIOD) * 4u,
@@ -460,9 +475,9 @@ __global__ __launch_bounds__(128 * WM) void mx_dma_kernel(MxDmaParams p)
         tie_after_wait(xs_now, xs_next);
     // whole rounds of STAGES steps run without a branch between the steps; the remainder follows
     int g = 0;
-    for (int slab = 1; g + STAGES <= p.steps; ++slab) {
+    for (int slab = 1; g + STAGES <= steps; ++slab) {
         load_slabs(slab);
-        const int end = slab * PERIOD < p.steps ? slab * PERIOD : p.steps;
+        const int end = slab * PERIOD < steps ? slab * PERIOD : steps;
         for (; g + STAGES <= end; g += STAGES) {
 #pragma unroll
             for (int s = 0; s < STAGES; ++s)
@@ -471,9 +486,29 @@ __global__ __launch_bounds__(128 * WM) void mx_dma_kernel(MxDmaParams p)
     }
 #pragma unroll
     for (int s = 0; s + 1 < STAGES; ++s)
-        if (g + s < p.steps)
+        if (g + s < steps)
             step(g + s, stage_at(s), stage_at((s + STAGES - 1) % STAGES));
     wait_loads<0>();
+
+    if constexpr (!GROUPED) {
+        if (gridDim.y > 1) { // a share of K: the plain sums, for sum_planes_kernel
+#pragma unroll
+            for (int j = 0; j < TM; ++j) {
+                const int m = m0 + (wm * TM + j) * 32 + frag_row;
+                float *row = p.planes + (size_t(blockIdx.y) * p.rows + m) * p.outputs + n0 + wn * TN * 32 + half * 4;
+#pragma unroll
+                for (int i = 0; i < TN; ++i)
+#pragma unroll
+                    for (int q = 0; q < 4; ++q) {
+                        const int offset = i * 32 + q * 8;
+                        if (m < p.rows && n0 + wn * TN * 32 + half * 4 + offset < p.outputs)
+                            *reinterpret_cast<f32x4_t *>(row + offset) = f32x4_t{
+                                acc[i][j][q * 4], acc[i][j][q * 4 + 1], acc[i][j][q * 4 + 2], acc[i][j][q * 4 + 3]};
+                    }
+            }
+            return;
+        }
+    }
 
     // ---- epilogue: accumulator register 4q+e of lane l is feature 8q + 4*(l/32) + e, token l%32
 #pragma unroll
@@ -499,19 +534,46 @@ __global__ __launch_bounds__(128 * WM) void mx_dma_kernel(MxDmaParams p)
     }
 }
 
+// out = plane 0 + plane 1 + ... of a divided K, four outputs per thread, the planes added in index
+// order so that the result does not depend on scheduling.
+__global__ __launch_bounds__(256) void sum_planes_kernel(MxDmaParams p, int shares)
+{
+    const size_t quad = size_t(blockIdx.x) * 256 + threadIdx.x, per_row = size_t(p.outputs / 4);
+    if (quad >= per_row * size_t(p.rows))
+        return;
+    const size_t m = quad / per_row, n = quad % per_row * 4, plane = size_t(p.rows) * p.outputs;
+    const float *source = p.planes + m * p.outputs + n;
+    f32x4_t sum = *reinterpret_cast<const f32x4_t *>(source);
+    for (int share = 1; share < shares; ++share) {
+        const f32x4_t more = *reinterpret_cast<const f32x4_t *>(source + share * plane);
+#pragma unroll
+        for (int e = 0; e < 4; ++e)
+            sum[e] += more[e];
+    }
+    const u32x2_t packed = {pack_bf16x2(sum[0], sum[1]), pack_bf16x2(sum[2], sum[3])};
+    *reinterpret_cast<u32x2_t *>(p.out + m * p.out_pitch + n) = packed;
+}
+
 template <bool PACKED, bool WIDE_X, bool GROUPED, int TN, int TM, int WM, int STAGES, int RING>
-hipError_t launch_one(hipStream_t stream, MxDmaParams p, int groups)
+hipError_t launch_one(hipStream_t stream, MxDmaParams p, int groups, int shares)
 {
     constexpr int BN = 64 * TN, BM = 32 * WM * TM;
     p.tiles_n = (p.outputs + BN - 1) / BN;
     p.tiles_m = (p.rows + BM - 1) / BM;
     const size_t tiles = size_t(p.tiles_n) * size_t(p.tiles_m) * size_t(GROUPED ? groups : 1);
-    if (tiles > 0x7fffffffu)
+    if (tiles > 0x7fffffffu || (GROUPED && shares != 1))
         return hipErrorInvalidValue;
     p.groups = groups;
-    dim3 grid{unsigned(tiles)};
+    p.share_steps = (p.steps + shares - 1) / shares;
+    shares = (p.steps + p.share_steps - 1) / p.share_steps; // no empty share
+    dim3 grid{unsigned(tiles), unsigned(shares)};
     mx_dma_kernel<PACKED, WIDE_X, GROUPED, TN, TM, WM, STAGES, RING>
         <<<grid, 128 * WM, 0, stream>>>(p);
+    const hipError_t status = launch_status();
+    if (shares == 1 || status != hipSuccess)
+        return status;
+    const size_t quads = size_t(p.rows) * size_t(p.outputs / 4);
+    sum_planes_kernel<<<unsigned((quads + 255) / 256), 256, 0, stream>>>(p, shares);
     return launch_status();
 }
 
@@ -520,16 +582,16 @@ hipError_t launch_one(hipStream_t stream, MxDmaParams p, int groups)
 // wavefront load covers 16 rows of packed weights: 192 rows are not a whole number of rounds);
 // variant 3: 128 x 128, three stages (twice the workgroups of variant 1 for small products)
 template <bool PACKED, bool WIDE_X, bool GROUPED>
-hipError_t launch_variant(hipStream_t stream, const MxDmaParams &p, int groups, int variant)
+hipError_t launch_variant(hipStream_t stream, const MxDmaParams &p, int groups, int variant, int shares = 1)
 {
     switch (variant) {
-    case 0: return launch_one<PACKED, WIDE_X, GROUPED, 4, 2, 4, PACKED ? 3 : 2, PACKED || GROUPED ? 2 : 3>(stream, p, groups);
-    case 1: return launch_one<PACKED, WIDE_X, GROUPED, 4, 1, 4, 3, 4>(stream, p, groups);
+    case 0: return launch_one<PACKED, WIDE_X, GROUPED, 4, 2, 4, PACKED ? 3 : 2, PACKED || GROUPED ? 2 : 3>(stream, p, groups, shares);
+    case 1: return launch_one<PACKED, WIDE_X, GROUPED, 4, 1, 4, 3, 4>(stream, p, groups, shares);
     case 2:
         if constexpr (!PACKED)
-            return launch_one<false, false, GROUPED, 3, 2, 4, 2, 3>(stream, p, groups);
+            return launch_one<false, false, GROUPED, 3, 2, 4, 2, 3>(stream, p, groups, shares);
         return hipErrorInvalidValue;
-    case 3: return launch_one<PACKED, WIDE_X, GROUPED, 2, 1, 4, 3, 4>(stream, p, groups);
+    case 3: return launch_one<PACKED, WIDE_X, GROUPED, 2, 1, 4, 3, 4>(stream, p, groups, shares);
     default: return hipErrorInvalidValue;
     }
 }
@@ -572,6 +634,8 @@ hipError_t launch_mx_dma_rows(hipStream_t stream, int variant, bool packed, int 
     p.metadata = nullptr;
     p.active = p.counts = nullptr;
     p.weight_groups = 0;
+    p.planes = nullptr;
+    p.share_steps = 0;
     if (!packed)
         return launch_variant<false, false, false>(stream, p, 1, variant);
     return activation_block == 128 ? launch_variant<true, true, false>(stream, p, 1, variant)
@@ -582,14 +646,19 @@ hipError_t launch_mx_dma_rows(hipStream_t stream, int variant, bool packed, int 
 // tail_outputs > 0 (plain product only): the last tail_outputs outputs, starting at a multiple of 256,
 // run on tail_variant in a launch of their own, so that both launches are whole rounds of
 // workgroups where one tiling would end in a partly filled round.
+// shares > 1 (plain product, one launch): K divided over that many workgroups per tile, with
+// `planes` holding shares * rows * outputs floats.
 hipError_t launch_mx_dma(hipStream_t stream, int variant, bool packed, int groups, int weight_groups,
                          int rows, int outputs, int inner, int activation_block, const void *input,
                          const void *input_scale, const void *weight, const void *weight_scale,
                          const void *metadata, const void *active, const void *counts, void *out,
-                         int tail_variant, int tail_outputs)
+                         int tail_variant, int tail_outputs, int shares, float *planes)
 {
     if (!mx_dma_supported(outputs, inner, input, weight, out) ||
         (activation_block != 32 && !(packed && activation_block == 128)))
+        return hipErrorInvalidValue;
+    if (shares < 1 || shares > 64 || (shares > 1 && (!planes || groups != 0 || tail_outputs)) ||
+        size_t(rows) * size_t(outputs / 4) > size_t(0x7fffffff) * 256)
         return hipErrorInvalidValue;
     if (tail_outputs) {
         if (groups != 0 || tail_outputs < 0 || tail_outputs >= outputs || (outputs - tail_outputs) % 256)
@@ -618,12 +687,14 @@ hipError_t launch_mx_dma(hipStream_t stream, int variant, bool packed, int group
     p.active = static_cast<const int32_t *>(active);
     p.counts = static_cast<const int32_t *>(counts);
     p.weight_groups = weight_groups;
+    p.planes = planes;
+    p.share_steps = 0;
     const bool wide = activation_block == 128;
     if (groups == 0) {
         if (!packed)
-            return launch_variant<false, false, false>(stream, p, 1, variant);
-        return wide ? launch_variant<true, true, false>(stream, p, 1, variant)
-                    : launch_variant<true, false, false>(stream, p, 1, variant);
+            return launch_variant<false, false, false>(stream, p, 1, variant, shares);
+        return wide ? launch_variant<true, true, false>(stream, p, 1, variant, shares)
+                    : launch_variant<true, false, false>(stream, p, 1, variant, shares);
     }
     if (!packed)
         return launch_variant<false, false, true>(stream, p, groups, variant);

@@ -443,13 +443,120 @@ hipError_t launch_shape(hipStream_t stream, const MxParams &p, int groups, int f
 }
 } // namespace
 
+namespace
+{
+// How a product of more than 32 rows runs on the tiled kernel: the tile, the workgroups K is divided
+// over, and for a product that would end in a partly filled round the tile of a second launch over
+// the last outputs.
+struct MxTilePlan {
+    int variant = 0, shares = 1, tail_variant = 0, tail_outputs = 0;
+};
+
+// {microseconds per 128-input step of one tile, kilobytes a workgroup keeps in flight} per variant
+struct MxTilePrice {
+    double step_us, kilobytes_in_flight;
+    int outputs, rows;
+};
+const MxTilePrice mx_prices[2][4] = {
+    {{1.60, 64, 256, 256}, {1.00, 96, 256, 128}, {1.35, 56, 192, 256}, {0.58, 64, 128, 128}},
+    {{1.60, 96, 256, 256}, {1.00, 64, 256, 128}, {1e30, 1, 192, 256}, {0.58, 48, 128, 128}},
+};
+
+// Estimated microseconds of one launch (as for the BF16 tiles: rounds of workgroups times steps
+// times the tile's time per step, or the weights streamed at what the workgroups in flight can
+// draw if that is longer; a divided K adds the second kernel and the traffic of the FP32 planes).
+// Prices from a sweep of every tile with 1..8 shares over seven projection shapes at 48..1536 rows,
+// both weight formats: the choice by this estimate is within 1 % of the best measured candidate in
+// the geometric mean.
+double mx_launch_us(const MxTilePrice &price, bool packed, long long batches, int rows, int outputs, int inner,
+                    int shares, int compute_units)
+{
+    const double workgroups =
+        double((outputs + price.outputs - 1) / price.outputs) * ((rows + price.rows - 1) / price.rows) * batches * shares;
+    const double rounds = std::ceil(workgroups / compute_units);
+    const double steps = (inner / 128 + shares - 1) / shares;
+    const double bytes_per_us =
+        std::min(5.2e6, std::min(workgroups, double(compute_units)) * price.kilobytes_in_flight * 1024 / 2.6);
+    double stream_us = double(batches) * outputs * inner / (packed ? 2 : 1) / bytes_per_us;
+    if (workgroups > compute_units)
+        stream_us *= rounds * compute_units / workgroups;
+    double us = 0.8 + std::max(rounds * steps * price.step_us, stream_us);
+    if (shares > 1)
+        us += 5.0 + 2.0 * shares * double(rows) * outputs * 4 / 4.5e6;
+    return us;
+}
+
+MxTilePlan mx_tile_plan(int compute_units, bool packed, int groups, int rows, int outputs, int inner)
+{
+    MxTilePlan plan;
+    const long long batches = groups > 0 ? groups : 1;
+    const MxTilePrice(&prices)[4] = mx_prices[packed ? 1 : 0];
+    double best = 1e300;
+    const int counts[] = {1, 2, 3, 4, 6, 8};
+    for (int variant = 0; variant < 4; ++variant) {
+        if (prices[variant].step_us > 1e29 || (prices[variant].rows > 128 && rows <= 128))
+            continue;
+        for (const int shares : counts) {
+            // a share has at least eight steps, the planes at most 256 MB; grouped products are not divided
+            if (shares > 1 && (groups > 0 || inner / 128 / shares < 8 ||
+                               double(shares) * rows * outputs * 4 > double(1 << 28)))
+                continue;
+            const double us = mx_launch_us(prices[variant], packed, batches, rows, outputs, inner, shares, compute_units);
+            if (us < best) {
+                best = us;
+                plan.variant = variant;
+                plan.shares = shares;
+            }
+        }
+    }
+    // A plain product whose 256 x 256 tiles end in a partly filled round: whole rounds over the
+    // first outputs, and the rest on the tile that covers them soonest
+    // (18432 outputs by 4096 tokens: four rounds, then 2048 outputs as one round of 256 x 128).
+    if (groups == 0 && rows > 128) {
+        const long long token_tiles = (rows + 255) / 256;
+        const long long whole = static_cast<long long>((outputs + 255) / 256) * token_tiles / compute_units;
+        const long long main_outputs = whole * compute_units / token_tiles * 256;
+        if (whole >= 1 && main_outputs > 0 && main_outputs < outputs) {
+            const double main_us = mx_launch_us(prices[0], packed, 1, rows, int(main_outputs), inner, 1, compute_units);
+            for (int variant = 0; variant < 4; ++variant) {
+                if (prices[variant].step_us > 1e29)
+                    continue;
+                const double us = main_us + 3.0 + mx_launch_us(prices[variant], packed, 1, rows, outputs - int(main_outputs),
+                                                               inner, 1, compute_units);
+                if (us < 0.97 * best) {
+                    best = us / 0.97;
+                    plan.variant = 0;
+                    plan.shares = 1;
+                    plan.tail_variant = variant;
+                    plan.tail_outputs = outputs - int(main_outputs);
+                }
+            }
+        }
+    }
+    return plan;
+}
+} // namespace
+
+int mx_matmul_shares(int kernel, int forced_shares, int compute_units, bool packed, int rows, int outputs,
+                     int inner, const void *input, const void *weight, const void *out)
+{
+    if (kernel >= 20)
+        return forced_shares > 1 ? forced_shares : 1;
+    if (kernel >= 0 || rows <= 32 || !mx_dma_supported(outputs, inner, input, weight, out))
+        return 1;
+    return mx_tile_plan(compute_units, packed, 0, rows, outputs, inner).shares;
+}
+
 // groups == 0: plain product (weight, weight_scale given); groups >= 1: grouped product (metadata,
-// active, counts given). activation_block 32 or 128. Weights 16-byte aligned.
+// active, counts given). activation_block 32 or 128. Weights 16-byte aligned. forced_shares: with a
+// forced tile variant (kernel >= 20), the workgroups K is divided over; planes: room for a divided K
+// (see mx_matmul_shares), without which K is not divided.
 hipError_t launch_mx_matmul(hipStream_t stream, int kernel, int compute_units, bool packed, int groups,
                             int weight_groups, int rows, int outputs, int inner,
                             int activation_block, const void *input,
                             const void *input_scale, const void *weight, const void *weight_scale,
-                            const void *metadata, const void *active, const void *counts, void *out)
+                            const void *metadata, const void *active, const void *counts, void *out,
+                            int forced_shares, float *planes)
 {
     // Above 32 rows the streaming kernel reads the weights once per 32-token slab; the tiled kernel
     // reads them once per 128 or 256 tokens (grouped weights come from the device table and are
@@ -459,62 +566,15 @@ hipError_t launch_mx_matmul(hipStream_t stream, int kernel, int compute_units, b
     if (kernel >= 20)
         return launch_mx_dma(stream, kernel - 20, packed, groups, weight_groups, rows, outputs, inner,
                              activation_block, input, input_scale, weight, weight_scale, metadata,
-                             active, counts, out);
+                             active, counts, out, 0, 0, planes && groups == 0 && forced_shares > 1 ? forced_shares : 1,
+                             planes);
     if (kernel < 0 && rows > 32 && mx_dma_supported(outputs, inner, input, checked_weight, out)) {
-        // 256 x 256 tiles do the most work per byte moved through LDS; the smaller tiles cost more
-        // per output (a 256 x 128 tile 0.57 of a large one, 0.6 with packed weights whose scales
-        // are gathered per row; a 192 x 256 tile, E4M3 weights only, 0.84; a 128 x 128 tile 0.43 /
-        // 0.45) but fill the chip when the large ones leave compute units idle: the fewest
-        // weighted rounds win (weights fitted to [18432, 7168] at 48 to 8192 rows).
-        const long long batches = groups > 0 ? groups : 1;
-        auto rounds = [&](long long tiles) { return double((tiles * batches + compute_units - 1) / compute_units); };
-        auto tiles = [&](int tile_outputs, int tile_rows) {
-            return static_cast<long long>((outputs + tile_outputs - 1) / tile_outputs) * ((rows + tile_rows - 1) / tile_rows);
-        };
-        const double cost[4] = {
-            rows > 128 ? rounds(tiles(256, 256)) : 1e30,
-            rounds(tiles(256, 128)) * (packed ? 0.6 : 0.57),
-            rows > 128 && !packed ? rounds(tiles(192, 256)) * 0.84 : 1e30,
-            rounds(tiles(128, 128)) * (packed ? 0.45 : 0.43),
-        };
-        int variant = 0;
-        for (int candidate = 1; candidate < 4; ++candidate)
-            if (cost[candidate] < cost[variant])
-                variant = candidate;
-        // A plain product whose 256 x 256 tiles end in a partly filled round: whole rounds over the
-        // first outputs, and the rest on the tile that covers them in the fewest weighted rounds
-        // (18432 outputs by 4096 tokens: four rounds, then 2048 outputs as one round of 256 x 128).
-        int tail_variant = 0, tail_outputs = 0;
-        if (groups == 0 && rows > 128) {
-            const long long token_tiles = (rows + 255) / 256;
-            const long long whole = tiles(256, 256) / compute_units;
-            const long long main_outputs = whole * compute_units / token_tiles * 256;
-            if (whole >= 1 && main_outputs > 0 && main_outputs < outputs) {
-                const int rest = outputs - int(main_outputs);
-                auto rest_tiles = [&](int tile_outputs, int tile_rows) {
-                    return static_cast<long long>((rest + tile_outputs - 1) / tile_outputs) * ((rows + tile_rows - 1) / tile_rows);
-                };
-                const double rest_cost[4] = {
-                    rounds(rest_tiles(256, 256)),
-                    rounds(rest_tiles(256, 128)) * (packed ? 0.6 : 0.57),
-                    !packed ? rounds(rest_tiles(192, 256)) * 0.84 : 1e30,
-                    rounds(rest_tiles(128, 128)) * (packed ? 0.45 : 0.43),
-                };
-                int best_rest = 0;
-                for (int candidate = 1; candidate < 4; ++candidate)
-                    if (rest_cost[candidate] < rest_cost[best_rest])
-                        best_rest = candidate;
-                // (a second launch costs about a twentieth of a round of large tiles)
-                if (double(whole) + rest_cost[best_rest] + 0.05 < 0.97 * cost[variant]) {
-                    variant = 0;
-                    tail_variant = best_rest;
-                    tail_outputs = rest;
-                }
-            }
-        }
-        return launch_mx_dma(stream, variant, packed, groups, weight_groups, rows, outputs, inner,
+        MxTilePlan plan = mx_tile_plan(compute_units, packed, groups, rows, outputs, inner);
+        if (plan.shares > 1 && !planes) // no room for the planes: the same tile with K undivided
+            plan.shares = 1;
+        return launch_mx_dma(stream, plan.variant, packed, groups, weight_groups, rows, outputs, inner,
                              activation_block, input, input_scale, weight, weight_scale, metadata,
-                             active, counts, out, tail_variant, tail_outputs);
+                             active, counts, out, plan.tail_variant, plan.tail_outputs, plan.shares, planes);
     }
     MxParams p;
     p.input = static_cast<const unsigned char *>(input);

@@ -38,13 +38,13 @@ def shifted(device, array, shift):
     return view
 
 
-def run(device, x, sx, weight, sw, packed, block, kernel="auto", shifts=(0, 0)):
+def run(device, x, sx, weight, sw, packed, block, kernel="auto", shifts=(0, 0), shares=0):
     xt = torch.from_numpy(x).to(device).view(torch.float8_e4m3fn)
     wt = torch.from_numpy(weight).to(device)
     if not packed:
         wt = wt.view(torch.float8_e4m3fn)
     native = _native.context(device)
-    native.call("hip_set_plan_override", KERNELS[kernel], 0)
+    native.call("hip_set_plan_override", KERNELS[kernel], shares)
     try:
         out = _kernels.quantized_matmul(xt, shifted(device, sx, shifts[0]), wt, shifted(device, sw, shifts[1]),
                                         activation_block=block)
@@ -115,6 +115,40 @@ def test_exact_products_with_every_scale_alignment(device, kernel, packed, block
     assert np.abs(want).max() < 2.0 ** 24 and (want * 64 == np.round(want * 64)).all()
     want = oracle.bf16_to_f32(oracle.f32_to_bf16(want.astype(np.float32)))
     assert np.array_equal(got, want)
+
+
+@pytest.mark.parametrize("kernel,packed,block", [f for f in FORMATS if f[0] != "auto"])
+@pytest.mark.parametrize("shares,shifts", [(2, (0, 0)), (4, (1, 3)), (9, (2, 1))])
+def test_exact_products_with_k_divided_over_workgroups(device, kernel, packed, block, shares, shifts):
+    # Nine steps of 128 inputs over 2 (5 + 4), 3 (asked for 4: 3 + 3 + 3) and 9 workgroups per tile, whose
+    # FP32 planes a second kernel adds in share order. Operands as in the test above, so that every
+    # plane and their sum are exact: the result must again be the BF16 rounding of the exact product,
+    # which pins the step at which each share starts in the operands and in both scale arrays.
+    rows, outputs, inner = 150, 328, 1152
+    rng = np.random.default_rng(57 + shares)
+    levels = np.array([0x00, 0x30, 0x38, 0x40, 0xB0, 0xB8, 0xC0], np.uint8)
+    x = levels[rng.integers(0, len(levels), (rows, inner))]
+    if packed:
+        nibbles = np.array([0, 1, 2, 3, 4, 9, 10, 11, 12], np.uint8)
+        pairs = nibbles[rng.integers(0, len(nibbles), (outputs, inner // 2, 2))]
+        weight = (pairs[..., 0] | (pairs[..., 1] << 4)).astype(np.uint8)
+    else:
+        weight = levels[rng.integers(0, len(levels), (outputs, inner))]
+    sx = rng.integers(125, 130, (rows, inner // block), dtype=np.uint8)
+    sw = rng.integers(125, 130, (outputs if packed else (outputs + 31) // 32, inner // 32), dtype=np.uint8)
+    got = run(device, x, sx, weight, sw, packed, block, kernel, shifts, shares)
+    want = oracle.mx_matmul_f64(x, sx, weight, sw, block, packed)
+    assert np.abs(want).max() < 2.0 ** 24 and (want * 64 == np.round(want * 64)).all()
+    want = oracle.bf16_to_f32(oracle.f32_to_bf16(want.astype(np.float32)))
+    assert np.array_equal(got, want)
+
+
+def test_planned_product_with_k_divided(device):
+    # a narrow projection with a long K at 96 rows: the planner divides K (56 tiles of 128 x 128 on 256
+    # compute units otherwise); random operands against the FP64 decoder
+    for packed in (False, True):
+        x, sx, weight, sw = operands(5, 96, 1024, 4096, packed, 32)
+        close(run(device, x, sx, weight, sw, packed, 32), x, sx, weight, sw, packed, 32)
 
 
 @pytest.mark.parametrize("packed", [False, True])
