@@ -228,7 +228,7 @@ extern "C" int camblas_cuda_quantized_matmul(camblas_cuda_context *context, int 
         // K divided over several workgroups per tile needs FP32 planes; without them (allocation
         // failure, capture in progress) the same tiles run with K undivided
         const int shares = mx_matmul_shares(context->override_kernel, context->override_split, context->compute_units,
-                                            packed != 0, rows, outputs, inner, input, weight, output);
+                                            packed != 0, rows, outputs, inner, activation_block, input, weight, output);
         float *planes = nullptr;
         if (shares > 1) {
             if (reserve_scratch(context, size_t(shares) * size_t(rows) * size_t(outputs) * 4) == hipSuccess)

@@ -240,7 +240,7 @@ hipError_t launch_mx_matmul(hipStream_t stream, int kernel, int compute_units, b
 // Workgroups that launch_mx_matmul would divide K over for a plain product (1: K is not divided);
 // `planes` then needs that many times rows * outputs floats, and without it K is not divided.
 int mx_matmul_shares(int kernel, int forced_shares, int compute_units, bool packed, int rows, int outputs,
-                     int inner, const void *input, const void *weight, const void *out);
+                     int inner, int activation_block, const void *input, const void *weight, const void *out);
 // Prefill-sized E8M0 product (hardware-scaled matrix instructions, operands loaded straight into
 // LDS); needs inner % 128 == 0, 16-byte aligned operands and an 8-byte aligned output.
 int mx_dma_variant_count();

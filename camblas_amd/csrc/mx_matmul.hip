@@ -537,12 +537,22 @@ MxTilePlan mx_tile_plan(int compute_units, bool packed, int groups, int rows, in
 }
 } // namespace
 
+// Rows from which the tiled kernel takes over: above 32 (the measured crossover), and from 17 on
+// when the streaming kernel could not hold the scale bytes of 32 tokens in its LDS table and would
+// gather them a byte per lane and step ([7168, 18432] x 32 rows: 34 us against 24 at 16 rows and 26 on
+// the tiles).
+static bool mx_rows_take_tiles(int rows, int inner, int activation_block)
+{
+    return rows > 32 || (rows > 16 && 32 * (inner / activation_block) + 3 > STAGED_TOKEN_BYTES);
+}
+
 int mx_matmul_shares(int kernel, int forced_shares, int compute_units, bool packed, int rows, int outputs,
-                     int inner, const void *input, const void *weight, const void *out)
+                     int inner, int activation_block, const void *input, const void *weight, const void *out)
 {
     if (kernel >= 20)
         return forced_shares > 1 ? forced_shares : 1;
-    if (kernel >= 0 || rows <= 32 || !mx_dma_supported(outputs, inner, input, weight, out))
+    if (kernel >= 0 || !mx_rows_take_tiles(rows, inner, activation_block) ||
+        !mx_dma_supported(outputs, inner, input, weight, out))
         return 1;
     return mx_tile_plan(compute_units, packed, 0, rows, outputs, inner).shares;
 }
@@ -560,15 +570,15 @@ hipError_t launch_mx_matmul(hipStream_t stream, int kernel, int compute_units, b
 {
     // Above 32 rows the streaming kernel reads the weights once per 32-token slab; the tiled kernel
     // reads them once per 128 or 256 tokens (grouped weights come from the device table and are
-    // 16-byte aligned by contract, so only the host-visible pointers are checked here). Measured
-    // crossover: 33 rows.
+    // 16-byte aligned by contract, so only the host-visible pointers are checked here).
     const void *checked_weight = groups == 0 ? weight : nullptr;
     if (kernel >= 20)
         return launch_mx_dma(stream, kernel - 20, packed, groups, weight_groups, rows, outputs, inner,
                              activation_block, input, input_scale, weight, weight_scale, metadata,
                              active, counts, out, 0, 0, planes && groups == 0 && forced_shares > 1 ? forced_shares : 1,
                              planes);
-    if (kernel < 0 && rows > 32 && mx_dma_supported(outputs, inner, input, checked_weight, out)) {
+    if (kernel < 0 && mx_rows_take_tiles(rows, inner, activation_block) &&
+        mx_dma_supported(outputs, inner, input, checked_weight, out)) {
         MxTilePlan plan = mx_tile_plan(compute_units, packed, groups, rows, outputs, inner);
         if (plan.shares > 1 && !planes) // no room for the planes: the same tile with K undivided
             plan.shares = 1;

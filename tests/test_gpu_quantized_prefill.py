@@ -152,6 +152,18 @@ def test_planned_product_with_k_divided(device):
 
 
 @pytest.mark.parametrize("packed", [False, True])
+def test_rows_17_to_32_with_a_long_k_take_the_tiles(device, packed):
+    # 24 rows x K = 18432: the scale bytes of 32 tokens (18 KB) exceed the streaming kernel's LDS table,
+    # so the product runs on the tiled kernel (with K divided: 3 tiles otherwise); the streaming
+    # kernel, forced, must agree with it
+    x, sx, weight, sw = operands(11, 24, 264, 18432, packed, 32)
+    planned = run(device, x, sx, weight, sw, packed, 32)
+    close(planned, x, sx, weight, sw, packed, 32)
+    streamed = run(device, x, sx, weight, sw, packed, 32, "stream")
+    close(streamed, x, sx, weight, sw, packed, 32)
+
+
+@pytest.mark.parametrize("packed", [False, True])
 def test_tiled_and_streaming_kernels_agree(device, packed):
     x, sx, weight, sw = operands(77, 200, 520, 512, packed, 32)
     tiled = run(device, x, sx, weight, sw, packed, 32, "tile256x256")
