@@ -380,10 +380,12 @@ Plan make_plan(int dtype, int algorithm, bool trans_a, bool trans_b, int m, int 
     // [2048, 7168], [7168, 2048] and [24576, 1536] from 72 to 4096 tokens: the choice is the
     // measured best or within a few per cent of it (e.g. [7168, 18432] at 256 tokens 60 us with
     // 256 x 128 tiles in four shares against 98 undivided; [4096, 7168] at 256 tokens 24 against 38).
+    // (The 64-token tiles are priced as measured with weights that come from memory, not from the
+    // last-level cache: every further token tile re-reads the weight rows.)
     const struct {
         int variant;
         double group_us;
-    } candidates[] = {{0, 1.88}, {8, 1.55}, {4, 1.12}, {7, 0.90}, {6, 0.80}, {9, 0.67}};
+    } candidates[] = {{0, 1.88}, {8, 1.55}, {4, 1.12}, {7, 0.90}, {6, 0.90}, {9, 0.72}};
     const int groups = k / 128;
     double best = 1e30;
     for (const auto &candidate : candidates) {
