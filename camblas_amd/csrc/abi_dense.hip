@@ -412,6 +412,22 @@ int launch_bf16_plan(const Entry &entry, Plan plan, const Product &p, float alph
                                             p.ldb, beta, c, p.ldc, partials, source),
                             "BF16 MFMA GEMM");
     }
+    case FAMILY_NN: {
+        float *partials = reserved;
+        if (plan.split_k > 1 && !partials) {
+            // without room for the partials (allocation failure, capture in progress) run undivided
+            if (reserve_scratch(context, size_t(plan.split_k) * size_t(p.m) * size_t(p.n) * 4) == hipSuccess) {
+                partials = static_cast<float *>(context->scratch);
+            } else {
+                context->counts[5]++;
+                plan.split_k = 1;
+            }
+        }
+        context->counts[plan.counter]++;
+        return entry.finish(launch_bgemm_nn(stream, p.m, p.n, p.k, alpha, a, p.lda, b, p.ldb, beta, c, p.ldc,
+                                            plan.split_k, partials),
+                            "BF16 GEMM (outputs contiguous)");
+    }
     case FAMILY_MFMA_BF16:
         context->counts[plan.counter]++;
         return entry.finish(launch_bgemm_any(stream, plan.kernel == 0, p.trans_a, p.trans_b, p.m, p.n, p.k, alpha,
@@ -431,32 +447,38 @@ int launch_bf16_plan(const Entry &entry, Plan plan, const Product &p, float alph
 // cost being one extra pass over each copied operand. Returns 1 when the arena could not hold the
 // copies.
 constexpr double TRANSPOSE_WORTHWHILE_FLOPS = 2.5e8; // about 512^3: below, the extra launches cost more
+// tokens_only: only the second operand (the tokens of a linear layer: few rows) is copied, and the
+// first stays as it lies, whichever way that is.
 int bf16_product_transposing(const Entry &entry, const Product &p, float alpha, const void *a, const void *b,
-                             float beta, void *c, const BetaSource &source)
+                             float beta, void *c, const BetaSource &source, bool tokens_only = false)
 {
     camblas_cuda_context *context = entry.context();
     hipStream_t stream = context->stream;
     const auto padded = [](size_t elements) { return (elements * 2 + 255) / 256 * 256; };
-    const size_t a_bytes = p.trans_a ? 0 : padded(size_t(p.m) * p.k);
+    const bool copy_a = !p.trans_a && !tokens_only;
+    const size_t a_bytes = copy_a ? padded(size_t(p.m) * p.k) : 0;
     const size_t b_bytes = p.trans_b ? padded(size_t(p.n) * p.k) : 0;
     Product q = p;
-    q.trans_a = 1, q.trans_b = 0;
-    q.lda = p.trans_a ? p.lda : p.k;
+    q.trans_a = copy_a ? 1 : p.trans_a, q.trans_b = 0;
+    q.lda = copy_a ? p.k : p.lda;
     q.ldb = p.trans_b ? p.k : p.ldb;
-    const bool aligned = (!p.trans_a || is_aligned(a, 16)) && (p.trans_b || is_aligned(b, 16));
-    Plan plan = make_plan(2, context->algorithm, 1, 0, q.m, q.n, q.k, q.lda, q.ldb, q.ldc, aligned,
+    const bool aligned = (copy_a || is_aligned(a, 16)) && (p.trans_b || is_aligned(b, 16));
+    Plan plan = make_plan(2, context->algorithm, q.trans_a, 0, q.m, q.n, q.k, q.lda, q.ldb, q.ldc, aligned,
                           context->compute_units);
     if (plan.family == FAMILY_DMA && (!is_aligned(c, 8) || !is_aligned(source.z, 8) || source.ldz % 4))
         use_register_staged_tiles(plan);
+    if (plan.family == FAMILY_NN && !is_aligned(c, 8))
+        plan = make_plan(2, context->algorithm, q.trans_a, 0, q.m, q.n, q.k, q.lda, q.ldb, q.ldc, false,
+                         context->compute_units);
     size_t partial_bytes = 0; // room for a divided K, held in the same arena behind the copies
-    if (plan.split_k > 1 && (plan.family == FAMILY_MFMA_TN || plan.family == FAMILY_DMA))
+    if (plan.split_k > 1 && (plan.family == FAMILY_MFMA_TN || plan.family == FAMILY_DMA || plan.family == FAMILY_NN))
         partial_bytes = size_t(plan.split_k) * size_t(p.m) * size_t(p.n) * 4;
     else if (plan.split_k > 1 && plan.family == FAMILY_STREAM)
         partial_bytes = stream_partial_bytes(plan.kernel / 10 % 10, plan.kernel % 10, p.m, p.n, plan.split_k);
     if (reserve_scratch(context, a_bytes + b_bytes + partial_bytes) != hipSuccess)
         return 1;
     char *arena = static_cast<char *>(context->scratch);
-    if (!p.trans_a) { // a[i + l*lda] -> [i*k + l]
+    if (copy_a) { // a[i + l*lda] -> [i*k + l]
         const hipError_t status = launch_transpose_bf16(stream, p.k, p.m, a, p.lda, arena, p.k);
         if (status != hipSuccess)
             return entry.finish(status, "BF16 operand transposition");
@@ -484,6 +506,24 @@ int bf16_product(const Entry &entry, const Product &p, float alpha, const void *
     if (plan.family == FAMILY_DMA && (!is_aligned(c, 8) || !is_aligned(source.z, 8) || source.ldz % 4))
         use_register_staged_tiles(plan); // register-staged loads, scalar stores
     const int forced = context->override_kernel;
+    // Tokens stored the other way round (K rows of tokens) and few of them: copying them transposed
+    // costs next to nothing, and the product then runs on the kernels for few tokens instead of the
+    // layout-agnostic tiles or, below 32 tokens, the vector-ALU kernel ([8192, 28672] x 16 tokens:
+    // 1760 us).
+    if (p.trans_b && p.n <= 512 && forced < 0 && context->algorithm != CAMBLAS_CUDA_CLASSICAL &&
+        2.0 * p.m * p.n * p.k >= 1e6) {
+        const int status = bf16_product_transposing(entry, p, alpha, a, b, beta, c, source, true);
+        if (status <= 0)
+            return status;
+        context->counts[5]++; // no room for the copy
+    }
+    // the outputs-contiguous kernel stores eight bytes at a time; tests: 60 and 61 ask for the
+    // layout-agnostic kernel or the transposing route instead, 62 sets the workgroups K is divided over
+    if (plan.family == FAMILY_NN && (!is_aligned(c, 8) || forced == 60 || forced == 61))
+        plan = make_plan(2, context->algorithm, p.trans_a, p.trans_b, p.m, p.n, p.k, p.lda, p.ldb, p.ldc, false,
+                         context->compute_units);
+    if (plan.family == FAMILY_NN && forced == 62)
+        plan.split_k = std::max(1, context->override_split);
     if (plan.family == FAMILY_MFMA_BF16) {
         // tests: 60 keeps the layout-agnostic kernel, 61 takes the transposing route whatever the size
         const bool worthwhile = 2.0 * p.m * p.n * p.k >= TRANSPOSE_WORTHWHILE_FLOPS;

@@ -373,6 +373,27 @@ const TnVariant variants[] = {
 };
 } // namespace
 
+hipError_t launch_sum_shares(hipStream_t stream, const float *partials, int shares, int n_out, int m_rows,
+                             float alpha, float beta, const void *z, int ldz, void *y, int ldc)
+{
+    if (n_out % 4 || ldc % 4 || ldz % 4 || reinterpret_cast<uintptr_t>(y) % 8 || reinterpret_cast<uintptr_t>(z) % 8 ||
+        size_t(m_rows) * size_t(n_out / 4) > size_t(0x7fffffff) * 256)
+        return hipErrorInvalidValue;
+    DmaParams p = {};
+    p.partials = const_cast<float *>(partials);
+    p.n = n_out;
+    p.m = m_rows;
+    p.alpha = alpha;
+    p.beta = beta;
+    p.z = static_cast<const unsigned short *>(z);
+    p.ldz = ldz;
+    p.y = static_cast<unsigned short *>(y);
+    p.ldc = ldc;
+    const size_t quads = size_t(m_rows) * size_t(n_out / 4);
+    sum_shares_kernel<<<unsigned((quads + 255) / 256), 256, 0, stream>>>(p, shares);
+    return launch_status();
+}
+
 int dma_variant_count() { return int(sizeof(variants) / sizeof(variants[0])); }
 const TnVariant &dma_variant(int index) { return variants[index]; }
 

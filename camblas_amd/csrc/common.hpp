@@ -79,7 +79,8 @@ enum KernelFamily {
     FAMILY_FP8_DMA = 6, // FP8 block-scaled prefill: the same structure with one scale group per step
     FAMILY_FP8_STREAM = 7, // FP8 block-scaled decode: weight-streaming kernel (10*row_tiles + token_tiles)
     FAMILY_MFMA_F32 = 8,   // FP32, any layout: 128 x 128 tiles on the FP32 matrix-core instruction
-    FAMILY_MFMA_BF16 = 9   // BF16, any layout: the same structure on the BF16 matrix-core instruction
+    FAMILY_MFMA_BF16 = 9,  // BF16, any layout: the same structure on the BF16 matrix-core instruction
+    FAMILY_NN = 10         // BF16 'N','N' with up to a few hundred tokens: one pass over a W that has its outputs contiguous
 };
 
 struct Plan {
@@ -176,6 +177,16 @@ hipError_t launch_bgemm_dma(hipStream_t stream, int variant, int n_out, int m_ro
                             float alpha, const void *w, int lda, const void *x, int ldb, float beta,
                             void *y, int ldc, const BetaSource &source = {}, int shares = 1,
                             float *partials = nullptr);
+// y = alpha * (plane 0 + ... + plane shares-1) + beta * z, planes [share][token][output] FP32, added in
+// index order; n_out, ldc, ldz multiples of four, y and z 8-byte aligned.
+hipError_t launch_sum_shares(hipStream_t stream, const float *partials, int shares, int n_out, int m_rows,
+                             float alpha, float beta, const void *z, int ldz, void *y, int ldc);
+// y[M,N] (ldc) = alpha * x[M,K] (ldb) * W[K,N] (lda: outputs contiguous) + beta * y for few tokens; needs
+// k % 64 == 0, n_out % 4 == 0, lda % 8 == 0, ldb % 8 == 0, ldc % 4 == 0, 16-byte aligned W and x, 8-byte
+// aligned y. partials: FP32 [shares, M, N] when shares > 1.
+hipError_t launch_bgemm_nn(hipStream_t stream, int n_out, int m_rows, int k, float alpha, const void *w, int lda,
+                           const void *x, int ldb, float beta, void *y, int ldc, int shares = 1,
+                           float *partials = nullptr);
 // Decode-shaped BF16 linear: each workgroup streams 16*row_tiles weight rows over the whole K.
 // depth_log2: a K step is 2^depth_log2 blocks of 128 elements (0..3); row_tiles << depth_log2 <= 8
 // and (row_tiles + token_tiles) << depth_log2 <= 16 or the launch is refused.

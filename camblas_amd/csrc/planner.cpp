@@ -149,6 +149,26 @@ Plan make_plan(int dtype, int algorithm, bool trans_a, bool trans_b, int m, int 
         bool matrix_path = algorithm != CAMBLAS_CUDA_CLASSICAL && trans_a && !trans_b &&
                            k % 8 == 0 && lda % 8 == 0 && ldb % 8 == 0 && aligned16 && lda < limit &&
                            ldb < limit;
+        // x @ W with a row-major W ('N','N') and up to 512 tokens: one pass over W per 256 tokens with
+        // its outputs contiguous (the layout-agnostic tiles below re-read operands through LDS in
+        // 32-deep steps and are 3 to 4 times slower at these sizes; below 32 tokens the product went
+        // to the vector-ALU kernel: [8192, 28672] x 16 tokens 1660 us). K divided over workgroups
+        // when the 128-output tiles leave compute units idle.
+        if (algorithm != CAMBLAS_CUDA_CLASSICAL && !trans_a && !trans_b && n <= 512 && k % 64 == 0 && k >= 64 &&
+            m % 4 == 0 && lda % 8 == 0 && ldb % 8 == 0 && ldc % 4 == 0 && aligned16 &&
+            double(k) * lda * 2 < 4294967296.0 && (256.0 * ldb + k) * 2 < 4294967296.0) {
+            plan.family = FAMILY_NN;
+            plan.counter = 4;
+            const int tiles = ceil_div(m, 128) * ceil_div(n, 256);
+            const int resident = n <= 64 ? 2 : 1; // workgroups a compute unit holds (LDS of three stages)
+            const int counts[] = {8, 6, 4, 3, 2};
+            for (const int shares : counts)
+                if (tiles * shares <= resident * compute_units && k / shares >= 512) {
+                    plan.split_k = shares;
+                    break;
+                }
+            return plan;
+        }
         if (!matrix_path) {
             // the other layouts (and 'T','N' operands the K-contiguous kernels cannot take): the
             // layout-agnostic matrix-core kernel unless the product is a sliver, tiles chosen as for
@@ -492,6 +512,9 @@ void describe_plan(const Plan &plan, int dtype, char *text, size_t bytes)
             std::snprintf(text, bytes, "%s %s split_k=%d", type, dma_variant(plan.kernel).name, plan.split_k);
         else
             std::snprintf(text, bytes, "%s %s", type, dma_variant(plan.kernel).name);
+        break;
+    case FAMILY_NN:
+        std::snprintf(text, bytes, "%s outputs-contiguous stream 128x64 split_k=%d", type, plan.split_k);
         break;
     case FAMILY_STREAM:
         std::snprintf(text, bytes, "%s stream rows=%d tokens=%d k_step=%d k_shares=%d", type,

@@ -84,7 +84,9 @@ def test_planner_choices_for_the_baseline_shapes():
     # pairs: the layout-agnostic matrix-core kernel; slivers and the classical policy: vector-ALU tiles
     assert describe(2, "T", "N", 10240, 4096, 8200, 8200, 8200, 10240)[0] // 1000 == 2
     assert describe(2, "T", "N", 1024, 64, 1001, 1001, 1001, 1024)[0] // 1000 == 9
-    assert describe(2, "N", "N", 1024, 64, 1024, 1024, 1024, 1024) == (9001, "bf16 mfma any-layout 128x64x32")
+    assert describe(2, "N", "N", 1024, 64, 1024, 1024, 1024, 1024) == (
+        10000, "bf16 outputs-contiguous stream 128x64 split_k=2")
+    assert describe(2, "N", "N", 1024, 600, 1024, 1024, 1024, 1024) == (9001, "bf16 mfma any-layout 128x64x32")
     assert describe(2, "N", "T", 8192, 8192, 4096, 8192, 8192, 8192) == (9000, "bf16 mfma any-layout 128x128x32")
     assert describe(2, "T", "N", 1024, 64, 1024, 1024, 1024, 1024, aligned16=False)[0] // 1000 == 9
     assert describe(2, "N", "N", 1024, 16, 1024, 1024, 1024, 1024)[0] // 1000 == 0

@@ -201,6 +201,52 @@ def test_every_layout_on_the_matrix_cores(device, ta, tb, m, n, k, pad):
         assert code // 1000 == 9
 
 
+@pytest.mark.parametrize("tokens", [1, 7, 32, 33, 64, 100, 129, 300, 513])
+@pytest.mark.parametrize("shares", [None, 2, 7])
+def test_outputs_contiguous_weights_with_few_tokens(device, tokens, shares):
+    # x @ W with W stored [K, N] ('N','N'): the kernel that streams W as it lies. 264 outputs (two
+    # tiles of 128, the second one ragged), 7 steps of 64, padded leading dimensions; up to 512 tokens
+    # (513 goes to the layout-agnostic kernel). With K divided over 2 (4 + 3 steps) and 7 workgroups.
+    outputs, k = 264, 448
+    lda, ldb, ldc = outputs + 8, k + 8, outputs + 4
+    w = oracle.fill_normal_bf16(501, (lda * k,))
+    x = oracle.fill_normal_bf16(502 + tokens, (ldb * tokens,))
+    c0 = oracle.fill_normal_bf16(503, (ldc * tokens,))
+    text = _native.plan_describe(2, "N", "N", outputs, tokens, k, lda, ldb, ldc)[1]
+    assert ("outputs-contiguous" in text) == (tokens <= 512)
+    for alpha, beta in ((1.0, 0.0), (0.5, -1.5)):
+        got = run_bgemm(device, "N", "N", outputs, tokens, k, alpha, w, lda, x, ldb, beta, c0, ldc,
+                        override=None if shares is None else (62, shares))
+        want, want64 = reference("N", "N", outputs, tokens, k, alpha, w, lda, x, ldb, beta, c0, ldc)
+        got2d = got.reshape(tokens, ldc)
+        error = rel_frobenius(oracle.bf16_to_f32(got2d[:, :outputs]), want64.reshape(tokens, outputs))
+        assert error <= TOLERANCE, (alpha, beta, error)
+        assert np.array_equal(got2d[:, outputs:], c0.reshape(tokens, ldc)[:, outputs:])
+
+
+def test_outputs_contiguous_weights_keep_nan_where_it_belongs(device):
+    # a NaN in one token reaches that token's outputs only, a NaN in one column of W that output
+    # only; what lies in the padding of W's rows (here NaN) reaches nothing
+    outputs, tokens, k = 260, 40, 128
+    lda, ldb, ldc = outputs + 12, k, outputs
+    nan = np.uint16(0x7FC0)
+    w = oracle.fill_normal_bf16(511, (k, lda))
+    w[:, outputs:] = nan
+    x = oracle.fill_normal_bf16(512, (tokens, ldb))
+    clean = run_bgemm(device, "N", "N", outputs, tokens, k, 1.0, w.ravel(), lda, x.ravel(), ldb, 0.0,
+                      np.zeros(ldc * tokens, np.uint16), ldc).reshape(tokens, ldc)
+    assert not np.isnan(oracle.bf16_to_f32(clean)).any()
+    x[5, 77] = nan
+    w[100, 9] = nan
+    got = oracle.bf16_to_f32(run_bgemm(device, "N", "N", outputs, tokens, k, 1.0, w.ravel(), lda, x.ravel(), ldb,
+                                       0.0, np.zeros(ldc * tokens, np.uint16), ldc).reshape(tokens, ldc))
+    expected = np.zeros((tokens, outputs), bool)
+    expected[5, :] = True
+    expected[:, 9] = True
+    assert np.array_equal(np.isnan(got), expected)
+    assert np.array_equal(got[~expected], oracle.bf16_to_f32(clean)[~expected])
+
+
 @pytest.mark.parametrize("ta,tb", [("N", "N"), ("N", "T"), ("T", "T")])
 @pytest.mark.parametrize("m,n,k,pad", [(200, 150, 72, 8), (130, 70, 33, 1), (300, 260, 320, 0)])
 def test_operands_transposed_into_the_linear_shape(device, ta, tb, m, n, k, pad):
