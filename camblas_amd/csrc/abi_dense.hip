@@ -139,6 +139,15 @@ int ordinary(const Entry &entry, const Product &p, float alpha, const float *a, 
         plan.family = context->override_kernel >= 1 ? FAMILY_MFMA_F32 : FAMILY_GENERIC;
         plan.kernel = context->override_kernel == 2 ? 1 : 0;
     }
+    if (plan.family == FAMILY_MFMA_F32 && plan.split_k > 1 && context->override_kernel < 0) {
+        // without room for the planes (allocation failure, capture in progress) K stays undivided
+        if (reserve_scratch(context, size_t(plan.split_k) * size_t(p.m) * size_t(p.n) * 4) == hipSuccess)
+            return entry.finish(launch_sgemm_mfma_divided(context->stream, p.trans_a, p.trans_b, p.m, p.n, p.k, alpha, a,
+                                                          p.lda, b, p.ldb, beta, c, p.ldc, plan.split_k,
+                                                          static_cast<float *>(context->scratch)),
+                                "classical GEMM");
+        context->counts[5]++;
+    }
     const hipError_t launched =
         plan.family == FAMILY_MFMA_F32
             ? launch_sgemm_mfma(context->stream, plan.kernel == 0, p.trans_a, p.trans_b, p.m, p.n, p.k, alpha,

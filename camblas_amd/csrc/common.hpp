@@ -128,6 +128,11 @@ hipError_t launch_sgemm_mfma(hipStream_t stream, bool wide, bool ta, bool tb, in
                              float alpha, const float *a, int lda, const float *b, int ldb, float beta,
                              float *c, int ldc, int batches = 1, size_t batch_stride = 0,
                              bool lower_only = false);
+// The FP32 product with K divided over `shares` workgroups per 128 x 64 tile (k % shares == 0; planes:
+// shares * m * n floats, summed in share order): few columns of C against a large A.
+hipError_t launch_sgemm_mfma_divided(hipStream_t stream, bool ta, bool tb, int m, int n, int k, float alpha,
+                                     const float *a, int lda, const float *b, int ldb, float beta, float *c,
+                                     int ldc, int shares, float *planes);
 hipError_t launch_dgemm_mfma(hipStream_t stream, bool ta, bool tb, int m, int n, int k, double alpha,
                              const double *a, int lda, const double *b, int ldb, double beta, double *c,
                              int ldc, int batches = 1, size_t batch_stride = 0, bool lower_only = false);

@@ -138,8 +138,26 @@ Plan make_plan(int dtype, int algorithm, bool trans_a, bool trans_b, int m, int 
         if (m >= 32 && n >= 32 && k >= 16) {
             plan.family = FAMILY_MFMA_F32;
             plan.kernel = double(ceil_div(m, 128)) * ceil_div(n, 128) >= 2.0 * compute_units ? 0 : 1;
+        } else if (algorithm != CAMBLAS_CUDA_CLASSICAL && m >= 256 && k >= 512) {
+            // a handful of columns against a large A (a linear layer at 2 to 31 tokens): the
+            // matrix-core tiles, mostly empty, still beat the vector-ALU kernel several times over
+            plan.family = FAMILY_MFMA_F32;
+            plan.kernel = 1;
         } else {
             plan.family = FAMILY_GENERIC;
+        }
+        // Few tiles and a long K (up to a few hundred tokens against a weight matrix): K divided
+        // over workgroups, about two per compute unit, FP32 planes summed in share order
+        // ([8192, 8192] x 16 tokens: 980 us on the vector-ALU kernel, 420 us at 32 tokens undivided).
+        if (plan.family == FAMILY_MFMA_F32 && plan.kernel == 1 && algorithm != CAMBLAS_CUDA_CLASSICAL && k >= 512) {
+            const int tiles = ceil_div(m, 128) * ceil_div(n, 64);
+            const int counts[] = {32, 16, 8, 4, 2};
+            for (const int shares : counts)
+                if (tiles * shares <= 2 * compute_units && k % shares == 0 && k / shares >= 256 &&
+                    double(shares) * m * n * 4 <= double(1 << 28)) {
+                    plan.split_k = shares;
+                    break;
+                }
         }
         plan.counter = algorithm == CAMBLAS_CUDA_LT || algorithm == CAMBLAS_CUDA_AUTO ? 4 : 0;
         return plan;
@@ -479,7 +497,10 @@ void describe_plan(const Plan &plan, int dtype, char *text, size_t bytes)
         std::snprintf(text, bytes, "%s gemv wave-per-row", type);
         break;
     case FAMILY_MFMA_F32:
-        std::snprintf(text, bytes, "%s mfma %s", type, plan.kernel == 0 ? "128x128x32" : "128x64x32");
+        if (plan.split_k > 1)
+            std::snprintf(text, bytes, "%s mfma 128x64x32 split_k=%d", type, plan.split_k);
+        else
+            std::snprintf(text, bytes, "%s mfma %s", type, plan.kernel == 0 ? "128x128x32" : "128x64x32");
         break;
     case FAMILY_MFMA_BF16:
         std::snprintf(text, bytes, "%s mfma any-layout %s", type, plan.kernel == 0 ? "128x128x32" : "128x64x32");

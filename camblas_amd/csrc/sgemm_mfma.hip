@@ -17,6 +17,9 @@ namespace camblas_hip
 namespace
 {
 constexpr int TILE = 128, DEPTH = 32, THREADS = 256;
+struct BatchStrides {
+    size_t a, b, c; // elements from one product of a batch to the next, per operand
+};
 constexpr int K_MAJOR_PITCH = TILE + 32, ROW_MAJOR_PITCH = DEPTH + 1;
 constexpr int TILE_WORDS = DEPTH * K_MAJOR_PITCH; // >= TILE * ROW_MAJOR_PITCH
 static_assert(TILE * ROW_MAJOR_PITCH <= TILE_WORDS, "one buffer serves both layouts");
@@ -34,15 +37,15 @@ template <bool TA, bool TB, int COLUMNS>
 __global__ __launch_bounds__(THREADS) void sgemm_mfma_kernel(int m, int n, int k, float alpha,
                                                              const float *a, int lda, const float *b,
                                                              int ldb, float beta, float *c, int ldc,
-                                                             size_t batch_stride, bool lower_only)
+                                                             BatchStrides strides, bool lower_only)
 {
     // a symmetric product: only the tiles that reach the diagonal, the rest is the mirroring pass
     int row0 = blockIdx.x * TILE, col0 = blockIdx.y * COLUMNS;
     if (lower_only && !lower_tile<TILE, COLUMNS>(blockIdx.x, n, row0, col0))
         return;
-    a += blockIdx.z * batch_stride; // one independent product per grid z-slice
-    b += blockIdx.z * batch_stride;
-    c += blockIdx.z * batch_stride;
+    a += blockIdx.z * strides.a; // one independent product per grid z-slice
+    b += blockIdx.z * strides.b;
+    c += blockIdx.z * strides.c;
     __shared__ float tile_a[TILE_WORDS];
     __shared__ float tile_b[TILE_WORDS];
     const int thread = threadIdx.x, lane = thread % 64, wave = thread / 64;
@@ -162,7 +165,7 @@ __global__ __launch_bounds__(THREADS) void sgemm_mfma_kernel(int m, int n, int k
 template <int COLUMNS>
 hipError_t launch_columns(hipStream_t stream, bool ta, bool tb, int m, int n, int k, float alpha,
                           const float *a, int lda, const float *b, int ldb, float beta, float *c, int ldc,
-                          int batches, size_t batch_stride, bool lower_only)
+                          int batches, BatchStrides strides, bool lower_only)
 {
     if (batches < 1 || batches > 65535)
         return hipErrorInvalidValue;
@@ -177,13 +180,13 @@ hipError_t launch_columns(hipStream_t stream, bool ta, bool tb, int m, int n, in
         if (lower_only)
             grid = dim3(lower_tile_count<TILE, COLUMNS>(n), 1, batches);
         if (!ta && !tb)
-            sgemm_mfma_kernel<false, false, COLUMNS><<<grid, THREADS, 0, stream>>>(m, columns, k, alpha, a, lda, bp, ldb, beta, cp, ldc, batch_stride, lower_only);
+            sgemm_mfma_kernel<false, false, COLUMNS><<<grid, THREADS, 0, stream>>>(m, columns, k, alpha, a, lda, bp, ldb, beta, cp, ldc, strides, lower_only);
         else if (!ta && tb)
-            sgemm_mfma_kernel<false, true, COLUMNS><<<grid, THREADS, 0, stream>>>(m, columns, k, alpha, a, lda, bp, ldb, beta, cp, ldc, batch_stride, lower_only);
+            sgemm_mfma_kernel<false, true, COLUMNS><<<grid, THREADS, 0, stream>>>(m, columns, k, alpha, a, lda, bp, ldb, beta, cp, ldc, strides, lower_only);
         else if (ta && !tb)
-            sgemm_mfma_kernel<true, false, COLUMNS><<<grid, THREADS, 0, stream>>>(m, columns, k, alpha, a, lda, bp, ldb, beta, cp, ldc, batch_stride, lower_only);
+            sgemm_mfma_kernel<true, false, COLUMNS><<<grid, THREADS, 0, stream>>>(m, columns, k, alpha, a, lda, bp, ldb, beta, cp, ldc, strides, lower_only);
         else
-            sgemm_mfma_kernel<true, true, COLUMNS><<<grid, THREADS, 0, stream>>>(m, columns, k, alpha, a, lda, bp, ldb, beta, cp, ldc, batch_stride, lower_only);
+            sgemm_mfma_kernel<true, true, COLUMNS><<<grid, THREADS, 0, stream>>>(m, columns, k, alpha, a, lda, bp, ldb, beta, cp, ldc, strides, lower_only);
         const hipError_t status = launch_status();
         if (status != hipSuccess)
             return status;
@@ -197,9 +200,52 @@ hipError_t launch_sgemm_mfma(hipStream_t stream, bool wide, bool ta, bool tb, in
                              float alpha, const float *a, int lda, const float *b, int ldb, float beta,
                              float *c, int ldc, int batches, size_t batch_stride, bool lower_only)
 {
+    const BatchStrides strides = {batch_stride, batch_stride, batch_stride};
     return wide ? launch_columns<128>(stream, ta, tb, m, n, k, alpha, a, lda, b, ldb, beta, c, ldc, batches,
-                                      batch_stride, lower_only)
+                                      strides, lower_only)
                 : launch_columns<64>(stream, ta, tb, m, n, k, alpha, a, lda, b, ldb, beta, c, ldc, batches,
-                                     batch_stride, lower_only);
+                                     strides, lower_only);
+}
+
+namespace
+{
+// c = alpha * (plane 0 + plane 1 + ...) + beta * c over the shares of a divided K, planes [share][n][m]
+// added in index order so that the result does not depend on scheduling.
+__global__ __launch_bounds__(256) void sum_planes_f32_kernel(int m, int n, int shares, float alpha, float beta,
+                                                             const float *planes, float *c, int ldc)
+{
+    const size_t index = size_t(blockIdx.x) * 256 + threadIdx.x, count = size_t(m) * n;
+    if (index >= count)
+        return;
+    float sum = planes[index];
+    for (int share = 1; share < shares; ++share)
+        sum += planes[size_t(share) * count + index];
+    float *out = c + (index / m) * size_t(ldc) + index % m;
+    const float value = alpha * sum;
+    *out = beta != 0.f ? fmaf(beta, *out, value) : value;
+}
+} // namespace
+
+// The same product with K divided over `shares` workgroups per 128 x 64 tile (k % shares == 0): for
+// a handful of columns of C against a large A, where the tiles alone would occupy a fraction of the
+// compute units. planes: shares * m * n floats.
+hipError_t launch_sgemm_mfma_divided(hipStream_t stream, bool ta, bool tb, int m, int n, int k, float alpha,
+                                     const float *a, int lda, const float *b, int ldb, float beta, float *c,
+                                     int ldc, int shares, float *planes)
+{
+    if (shares < 2 || shares > 65535 || k % shares || !planes)
+        return hipErrorInvalidValue;
+    const int part = k / shares;
+    const BatchStrides strides = {ta ? size_t(part) : size_t(part) * lda, tb ? size_t(part) * ldb : size_t(part),
+                                  size_t(m) * n};
+    const hipError_t status =
+        launch_columns<64>(stream, ta, tb, m, n, part, 1.f, a, lda, b, ldb, 0.f, planes, m, shares, strides, false);
+    if (status != hipSuccess)
+        return status;
+    const size_t count = size_t(m) * n;
+    if ((count + 255) / 256 > 0x7fffffffu)
+        return hipErrorInvalidValue;
+    sum_planes_f32_kernel<<<unsigned((count + 255) / 256), 256, 0, stream>>>(m, n, shares, alpha, beta, planes, c, ldc);
+    return launch_status();
 }
 } // namespace camblas_hip

@@ -62,6 +62,35 @@ def test_sgemm_padded_alpha_beta(device, kernel, ta, tb, shape):
     assert rel_frobenius(got2d[:, :m], scalar.reshape(n, ldc)[:, :m]) <= 5 * TOLERANCE
 
 
+@pytest.mark.parametrize("ta", "NT")
+@pytest.mark.parametrize("tb", "NT")
+@pytest.mark.parametrize("n", [1, 5, 31, 40])
+def test_sgemm_few_columns_against_a_large_matrix(device, ta, tb, n):
+    # a linear layer at a handful of tokens, every layout: matrix-core tiles with K divided over four
+    # workgroups per tile (k = 1024, five row tiles) and the planes summed in share order; padded
+    # leading dimensions, alpha and beta, untouched padding of C
+    m, k = 520, 1024
+    lda = (m if ta == "N" else k) + 3
+    ldb = (k if tb == "N" else n) + 2
+    ldc = m + 5
+    assert _native.plan_describe(0, ta, tb, m, n, k, lda, ldb, ldc)[1] == "f32 mfma 128x64x32 split_k=4" or (
+        n == 1 and ta == "T" and tb == "N")
+    a = oracle.fill_uniform(11, (lda * (k if ta == "N" else m),))
+    b = oracle.fill_uniform(12, (ldb * (n if tb == "N" else k),))
+    c0 = oracle.fill_uniform(13, (ldc * n,))
+    got = run_sgemm(device, ta, tb, m, n, k, 1.25, a, lda, b, ldb, -0.5, c0.copy(), ldc, algorithm="lt")
+    want64 = oracle.sgemm_f64(ta, tb, m, n, k, 1.25, a, lda, b, ldb, -0.5, c0.copy(), ldc, want64=True)
+    got2d, c2d = got.reshape(n, ldc), c0.reshape(n, ldc)
+    assert rel_frobenius(got2d[:, :m].ravel(), want64.reshape(n, m).ravel()) <= TOLERANCE
+    assert np.array_equal(got2d[:, m:], c2d[:, m:]), "padding rows of C were written"
+    # beta = 0 over a NaN-filled C
+    nan_c = np.full(ldc * n, np.nan, np.float32)
+    got = run_sgemm(device, ta, tb, m, n, k, 1.0, a, lda, b, ldb, 0.0, nan_c, ldc, algorithm="lt").reshape(n, ldc)
+    want64 = oracle.sgemm_f64(ta, tb, m, n, k, 1.0, a, lda, b, ldb, 0.0, np.zeros(ldc * n, np.float32), ldc,
+                              want64=True)
+    assert rel_frobenius(got[:, :m].ravel(), want64.reshape(n, m).ravel()) <= TOLERANCE
+
+
 def test_sgemm_beta_zero_ignores_nan_and_alpha_zero(device):
     m, n, k = 70, 33, 40
     a = oracle.fill_uniform(4, (m * k,))
