@@ -310,6 +310,208 @@ __global__ __launch_bounds__(128 * WM) void bgemm_dma_kernel(DmaParams p)
     }
 }
 
+// The same workgroup tile on v_mfma_f32_16x16x32_bf16. On operands with random bits the part sustains
+// 2.19 PFLOP/s with this instruction against 1.83 with the 32 x 32 x 16 one (it holds a higher clock:
+// measured with launches of nothing but matrix instructions), and the prefill kernel is limited by
+// that clock. A wavefront's (32*TN) x (32*TM) block is 2TN x 2TM tiles of 16 x 16 with four accumulator
+// registers each; a K step of 64 is two sub-steps of 32, in each of which every one of the 2TN
+// weight fragments (16 rows x 32 K: lane l holds K values 8*(l/16) .. +7 of row l%16) meets all 2TM
+// token fragments. The token fragments of a sub-step are read during the previous one, the weight
+// fragments travel RING-1 fragments ahead of their use in a ring of registers; the barrier of a step
+// lies RING-1 fragments before its end, so that the first fragments of the next stage are on their
+// way while the last matrix instructions of this one issue.
+template <int TN, int TM, int WM, int BK, int STAGES>
+__global__ __launch_bounds__(128 * WM) void bgemm_dma16_kernel(DmaParams p)
+{
+    constexpr int WAVES = 2 * WM;
+    constexpr int BN = 64 * TN, BM = 32 * WM * TM, CH = BK / 8;
+    constexpr int ROWS_PER_LOAD = 64 / CH;
+    constexpr int A_ITERS = BN / (WAVES * ROWS_PER_LOAD), B_ITERS = BM / (WAVES * ROWS_PER_LOAD);
+    static_assert(BK == 64 && BN % (WAVES * ROWS_PER_LOAD) == 0 && BM % (WAVES * ROWS_PER_LOAD) == 0,
+                  "every wavefront issues whole loads");
+    constexpr int LOADS = A_ITERS + B_ITERS;
+    constexpr int SLOTS = (BN + BM) * CH;
+    static_assert(STAGES >= 2 && STAGES <= 3, "pipeline shape");
+    __shared__ u32x4_t stage0[SLOTS];
+    __shared__ u32x4_t stage1[SLOTS];
+    __shared__ u32x4_t stage2[STAGES > 2 ? SLOTS : 1];
+
+    int tile_n, tile_m;
+    xcd_tile(int(blockIdx.x), p.tiles_n, p.tiles_m, tile_n, tile_m);
+    const int n0 = tile_n * BN, m0 = tile_m * BM;
+    const int first_step = int(blockIdx.y) * p.share_steps;
+    const int k_tiles = p.k / BK - first_step < p.share_steps ? p.k / BK - first_step : p.share_steps;
+
+    const int thread = threadIdx.x, lane = thread % 64, wave = thread / 64;
+    const int wn = wave % 2, wm = wave / 2;
+
+    // ---- fills: as in bgemm_dma_kernel
+    static_assert((WAVES * ROWS_PER_LOAD) % 16 == 0, "row step keeps the swizzle");
+    const int load_row = wave * ROWS_PER_LOAD + lane / CH;
+    const unsigned load_chunk = unsigned(((lane % CH) ^ lds_swizzle<CH>(load_row)) * 8);
+    const unsigned a_lane_off = (unsigned(load_row) * unsigned(p.lda) + load_chunk) * 2u;
+    const unsigned b_lane_off = (unsigned(load_row) * unsigned(p.ldb) + load_chunk) * 2u;
+    const unsigned a_row_step = unsigned(WAVES * ROWS_PER_LOAD) * unsigned(p.lda) * 2u;
+    const unsigned b_row_step = unsigned(WAVES * ROWS_PER_LOAD) * unsigned(p.ldb) * 2u;
+    const int a_rows = p.n - n0 < BN ? p.n - n0 : BN, b_rows = p.m - m0 < BM ? p.m - m0 : BM;
+    const __amdgpu_buffer_rsrc_t a_resource = make_resource(
+        p.w + size_t(n0) * p.lda, (unsigned(a_rows - 1) * unsigned(p.lda) + unsigned(p.k)) * 2u);
+    const __amdgpu_buffer_rsrc_t b_resource = make_resource(
+        p.x + size_t(m0) * p.ldb, (unsigned(b_rows - 1) * unsigned(p.ldb) + unsigned(p.k)) * 2u);
+    unsigned k_bytes = unsigned(first_step) * BK * 2;
+    const unsigned last_k_bytes = unsigned(first_step + k_tiles - 1) * BK * 2;
+    auto issue = [&](u32x4_t *stage) {
+#pragma unroll
+        for (int index = 0; index < LOADS; ++index) {
+            if (index < A_ITERS)
+                load_to_lds(a_resource, a_lane_off, k_bytes + unsigned(index) * a_row_step,
+                            stage + (index * WAVES + wave) * 64);
+            else
+                load_to_lds(b_resource, b_lane_off, k_bytes + unsigned(index - A_ITERS) * b_row_step,
+                            stage + BN * CH + ((index - A_ITERS) * WAVES + wave) * 64);
+        }
+        // (steps past the end re-read the last K block into a stage nobody multiplies)
+        k_bytes = k_bytes + BK * 2 < last_k_bytes ? k_bytes + BK * 2 : last_k_bytes;
+    };
+
+    // ---- fragments
+    constexpr int NA = 2 * TN, NB = 2 * TM, KS = BK / 32, ITEMS = KS * NA, RING = 4;
+    static_assert(ITEMS % RING == 0 && KS % 2 == 0, "ring slots and token buffers line up from step to step");
+    const int frag_row = lane % 16, group = lane / 16;
+    const int frag_swizzle = lds_swizzle<CH>(frag_row);
+    const int a_frag_base = (wn * TN * 32 + frag_row) * CH;
+    const int b_frag_base = BN * CH + (wm * TM * 32 + frag_row) * CH;
+    f32x4_t acc[NA][NB];
+#pragma unroll
+    for (int i = 0; i < NA; ++i)
+#pragma unroll
+        for (int j = 0; j < NB; ++j)
+            acc[i][j] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+    bf16x8_t a_ring[RING], b_buffer[2][NB];
+    auto read_a = [&](const u32x4_t *stage, int item) { // item = sub-step * NA + weight tile
+        const int ks = item / NA, i = item % NA;
+        a_ring[item % RING] =
+            __builtin_bit_cast(bf16x8_t, stage[a_frag_base + i * 16 * CH + ((ks * 4 + group) ^ frag_swizzle)]);
+    };
+    auto read_b = [&](const u32x4_t *stage, int ks) {
+#pragma unroll
+        for (int j = 0; j < NB; ++j)
+            b_buffer[ks & 1][j] =
+                __builtin_bit_cast(bf16x8_t, stage[b_frag_base + j * 16 * CH + ((ks * 4 + group) ^ frag_swizzle)]);
+    };
+    auto step = [&](u32x4_t *fill, const u32x4_t *current, const u32x4_t *next) {
+        __builtin_amdgcn_sched_barrier(0);
+        issue(fill);
+#pragma unroll
+        for (int item = 0; item < ITEMS; ++item) {
+            const int ks = item / NA, i = item % NA, ahead = item + RING - 1;
+            __builtin_amdgcn_sched_barrier(0);
+            if (item == ITEMS - (RING - 1)) {
+                pipeline_barrier<LOADS *(STAGES - 2)>();
+                read_b(next, 0);
+            }
+            if (ahead < ITEMS)
+                read_a(current, ahead);
+            else
+                read_a(next, ahead - ITEMS);
+            if (i == 0 && ks + 1 < KS)
+                read_b(current, ks + 1);
+            __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+            for (int j = 0; j < NB; ++j)
+                acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a_ring[item % RING], b_buffer[ks & 1][j],
+                                                                    acc[i][j], 0, 0, 0);
+        }
+        __builtin_amdgcn_sched_barrier(0);
+    };
+
+    issue(stage0);
+    if constexpr (STAGES > 2)
+        issue(stage1);
+    pipeline_barrier<LOADS *(STAGES - 2)>();
+    read_b(stage0, 0);
+#pragma unroll
+    for (int item = 0; item < RING - 1; ++item)
+        read_a(stage0, item);
+    for (int tile = 0; tile < k_tiles; tile += STAGES) {
+        if constexpr (STAGES == 2) {
+            step(stage1, stage0, stage1);
+            if (tile + 1 < k_tiles)
+                step(stage0, stage1, stage0);
+        } else {
+            step(stage2, stage0, stage1);
+            if (tile + 1 < k_tiles)
+                step(stage0, stage1, stage2);
+            if (tile + 2 < k_tiles)
+                step(stage1, stage2, stage0);
+        }
+    }
+    wait_loads<0>();
+
+    // ---- epilogue. Register e of lane l in tile (i, j) is feature 16 i + 4 (l / 16) + e, token 16 j + l % 16.
+    const int first_feature = n0 + wn * TN * 32 + group * 4;
+    const int first_token = m0 + wm * TM * 32 + frag_row;
+    if (gridDim.y > 1) { // a share of K: the plain sums, for sum_shares_kernel
+#pragma unroll
+        for (int j = 0; j < NB; ++j)
+#pragma unroll
+            for (int i = 0; i < NA; ++i) {
+                const int m = first_token + j * 16, n = first_feature + i * 16;
+                if (m < p.m && n < p.n)
+                    *reinterpret_cast<f32x4_t *>(p.partials + (size_t(blockIdx.y) * p.m + m) * p.n + n) = acc[i][j];
+            }
+        return;
+    }
+    auto store_tile = [&](int i, int j, u32x2_t old, bool with_beta) {
+        const int m = first_token + j * 16, n = first_feature + i * 16;
+        if (m < p.m && n < p.n) {
+            float v0 = p.alpha * acc[i][j][0], v1 = p.alpha * acc[i][j][1];
+            float v2 = p.alpha * acc[i][j][2], v3 = p.alpha * acc[i][j][3];
+            if (with_beta) {
+                v0 = fmaf(p.beta, __uint_as_float(old[0] << 16), v0);
+                v1 = fmaf(p.beta, __uint_as_float(old[0] & 0xffff0000u), v1);
+                v2 = fmaf(p.beta, __uint_as_float(old[1] << 16), v2);
+                v3 = fmaf(p.beta, __uint_as_float(old[1] & 0xffff0000u), v3);
+            }
+            *reinterpret_cast<u32x2_t *>(p.y + size_t(m) * p.ldc + n) = u32x2_t{pack_bf16x2(v0, v1), pack_bf16x2(v2, v3)};
+        }
+    };
+    if (p.beta == 0.f) {
+#pragma unroll
+        for (int j = 0; j < NB; ++j)
+#pragma unroll
+            for (int i = 0; i < NA; ++i)
+                store_tile(i, j, u32x2_t{0u, 0u}, false);
+        return;
+    }
+    // beta term: the addends of the next four tiles are fetched while four tiles are scaled and stored
+    // (unconditional loads: a position outside the matrix reads a valid element instead and is not used)
+    constexpr int TILES = NA * NB, AHEAD = 4;
+    u32x2_t old[2][AHEAD];
+    auto fetch = [&](int first, u32x2_t (&into)[AHEAD]) {
+#pragma unroll
+        for (int t = 0; t < AHEAD; ++t) {
+            const int tile = first + t < TILES ? first + t : TILES - 1;
+            int m = first_token + (tile / NA) * 16;
+            m = m < p.m ? m : p.m - 1;
+            const int n = first_feature + (tile % NA) * 16;
+            into[t] = *reinterpret_cast<const u32x2_t *>(p.z + size_t(m) * p.ldz + (n < p.n ? n : 0));
+        }
+    };
+    static_assert(TILES % AHEAD == 0, "whole groups of tiles");
+    fetch(0, old[0]);
+#pragma unroll
+    for (int first = 0; first < TILES; first += AHEAD) {
+        __builtin_amdgcn_sched_barrier(0);
+        if (first + AHEAD < TILES)
+            fetch(first + AHEAD, old[(first / AHEAD + 1) & 1]);
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int t = 0; t < AHEAD; ++t)
+            store_tile((first + t) % NA, (first + t) / NA, old[(first / AHEAD) & 1][t], true);
+    }
+}
+
 // y = alpha * (plane 0 + plane 1 + ...) + beta * z over the shares of a divided K, four features per
 // thread, the planes added in index order so that the result does not depend on scheduling.
 __global__ __launch_bounds__(256) void sum_shares_kernel(DmaParams p, int shares)
@@ -363,6 +565,29 @@ hipError_t launch_dma(hipStream_t stream, DmaParams p, int shares)
     return launch_status();
 }
 
+template <int TN, int TM, int WM, int BK, int STAGES>
+hipError_t launch_dma16(hipStream_t stream, DmaParams p, int shares)
+{
+    constexpr int BN = 64 * TN, BM = 32 * WM * TM;
+    if (p.k % BK)
+        return hipErrorInvalidValue;
+    p.tiles_n = (p.n + BN - 1) / BN;
+    p.tiles_m = (p.m + BM - 1) / BM;
+    if (size_t(p.tiles_n) * size_t(p.tiles_m) > 0x7fffffffu)
+        return hipErrorInvalidValue;
+    const int steps = p.k / BK;
+    p.share_steps = (steps + shares - 1) / shares;
+    shares = (steps + p.share_steps - 1) / p.share_steps; // no empty share
+    const dim3 grid(unsigned(p.tiles_n) * unsigned(p.tiles_m), unsigned(shares));
+    bgemm_dma16_kernel<TN, TM, WM, BK, STAGES><<<grid, 128 * WM, 0, stream>>>(p);
+    const hipError_t status = launch_status();
+    if (shares == 1 || status != hipSuccess)
+        return status;
+    const size_t quads = size_t(p.m) * size_t(p.n / 4);
+    sum_shares_kernel<<<unsigned((quads + 255) / 256), 256, 0, stream>>>(p, shares);
+    return launch_status();
+}
+
 const TnVariant variants[] = {
     {"dma256x256x32s4w4", 256, 256, 32, 256}, {"dma256x128x64s3w4", 256, 128, 64, 256},
     {"dma128x128x64s2w4", 128, 128, 64, 256}, {"dma256x256x32s3w4", 256, 256, 32, 256},
@@ -370,6 +595,10 @@ const TnVariant variants[] = {
     {"dma256x256x64s2w8", 256, 256, 64, 512}, {"dma256x256x32s4w8", 256, 256, 32, 512},
     {"dma256x128x64s3w8", 256, 128, 64, 512}, {"dma128x256x64s3w8", 128, 256, 64, 512},
     {"dma320x256x64s2w8", 320, 256, 64, 512}, {"dma192x256x64s2w8", 192, 256, 64, 512},
+    // the same tiles on the 16 x 16 x 32 matrix instruction
+    {"dma16-320x256x64s2w8", 320, 256, 64, 512}, {"dma16-256x256x64s2w8", 256, 256, 64, 512},
+    {"dma16-192x256x64s2w8", 192, 256, 64, 512}, {"dma16-128x256x64s3w8", 128, 256, 64, 512},
+    {"dma16-256x128x64s3w8", 256, 128, 64, 512}, {"dma16-128x128x64s3w4", 128, 128, 64, 256},
 };
 } // namespace
 
@@ -441,6 +670,12 @@ hipError_t launch_bgemm_dma(hipStream_t stream, int variant, int n_out, int m_ro
     case 9: return launch_dma<2, 2, 4, 64, 3>(stream, p, shares);
     case 10: return launch_dma<5, 2, 4, 64, 2>(stream, p, shares);
     case 11: return launch_dma<3, 2, 4, 64, 2>(stream, p, shares);
+    case 12: return launch_dma16<5, 2, 4, 64, 2>(stream, p, shares);
+    case 13: return launch_dma16<4, 2, 4, 64, 2>(stream, p, shares);
+    case 14: return launch_dma16<3, 2, 4, 64, 2>(stream, p, shares);
+    case 15: return launch_dma16<2, 2, 4, 64, 3>(stream, p, shares);
+    case 16: return launch_dma16<4, 1, 4, 64, 3>(stream, p, shares);
+    case 17: return launch_dma16<2, 2, 2, 64, 3>(stream, p, shares);
     default: return hipErrorInvalidValue;
     }
 }

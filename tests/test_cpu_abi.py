@@ -69,16 +69,16 @@ def test_planner_choices_for_the_baseline_shapes():
     assert "rows=32 tokens=16 k_step=256 k_shares=1" in describe(2, "T", "N", 8192, 1, 8192, 8192, 8192, 8192)[1]
     # prefill: direct-to-LDS MFMA tile that divides 10240 x 4096 into exactly two waves of tiles
     code, text = describe(2, "T", "N", 10240, 4096, 8192, 8192, 8192, 10240)
-    assert code // 1000 == 5 and "dma320x256" in text
+    assert code // 1000 == 5 and "dma16-320x256" in text
     # 2.8 rounds of 320 x 256 tiles: two whole rounds, and the last 4096 outputs as one round of 256 x 256
     assert describe(2, "T", "N", 14336, 4096, 4096, 4096, 4096, 14336) == (
-        5010, "bf16 dma320x256x64s2w8, last 4096 outputs dma256x256x64s2w8")
+        5012, "bf16 dma16-320x256x64s2w8, last 4096 outputs dma16-256x256x64s2w8")
     # 65..1536 tokens: tile, shares of K and a second launch by estimated time (one round of
     # workgroups where the tiles alone would leave compute units idle)
-    assert describe(2, "T", "N", 8192, 256, 8192, 8192, 8192, 8192) == (5009, "bf16 dma128x256x64s3w8 split_k=4")
-    assert describe(2, "T", "N", 10240, 128, 8192, 8192, 8192, 10240) == (5005, "bf16 dma128x128x64s3w4 split_k=3")
+    assert describe(2, "T", "N", 8192, 256, 8192, 8192, 8192, 8192) == (5015, "bf16 dma16-128x256x64s3w8 split_k=4")
+    assert describe(2, "T", "N", 10240, 128, 8192, 8192, 8192, 10240) == (5017, "bf16 dma16-128x128x64s3w4 split_k=3")
     assert describe(2, "T", "N", 28672, 1024, 8192, 8192, 8192, 28672) == (
-        5010, "bf16 dma320x256x64s2w8, last 8192 outputs dma128x256x64s3w8")
+        5012, "bf16 dma16-320x256x64s2w8, last 8192 outputs dma16-128x256x64s3w8")
     assert describe(2, "T", "N", 8192, 256, 8200, 8200, 8200, 8192) == (2002, "bf16 mfma128x128x64 split_k=4")
     # K not a multiple of 64: register-staged MFMA tiles; unaligned operands and the other transpose
     # pairs: the layout-agnostic matrix-core kernel; slivers and the classical policy: vector-ALU tiles

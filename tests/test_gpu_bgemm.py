@@ -100,7 +100,7 @@ def test_streaming_kernel_every_variant(device, code, n_out, m_rows, pad):
         assert np.array_equal(got2d[:, n_out:], c0.reshape(m_rows, ldc)[:, n_out:])
 
 
-@pytest.mark.parametrize("code", range(20, 32))
+@pytest.mark.parametrize("code", range(20, 38))
 @pytest.mark.parametrize("n_out,m_rows,k", [(300, 70, 320), (512, 256, 64), (260, 513, 448)])
 def test_direct_lds_load_kernel(device, code, n_out, m_rows, k):
     # direct global->LDS tiles: ragged N and M (partial tiles, clamped rows), odd and even numbers
@@ -119,7 +119,7 @@ def test_direct_lds_load_kernel(device, code, n_out, m_rows, k):
         assert np.array_equal(got2d[:, n_out:], c0.reshape(m_rows, ldc)[:, n_out:])
 
 
-@pytest.mark.parametrize("code", [22, 25, 29, 30])
+@pytest.mark.parametrize("code", [22, 25, 29, 30, 32, 35, 37])
 @pytest.mark.parametrize("shares", [2, 3, 7])
 def test_direct_lds_load_kernel_with_k_divided_over_workgroups(device, code, shares):
     # 7 steps of 64 over 2 (4 + 3), 3 (3 + 3 + 1) and 7 workgroups per tile; FP32 planes summed in
@@ -314,7 +314,7 @@ def test_classical_algorithm_uses_generic_kernel(device):
                          oracle.linear_bf16_f64(x, w)) <= TOLERANCE
 
 
-@pytest.mark.parametrize("override", [None, (0, 1), (4, 2), (172, 1), (20, 1), (22, 1)])
+@pytest.mark.parametrize("override", [None, (0, 1), (4, 2), (172, 1), (20, 1), (22, 1), (32, 1), (37, 1)])
 def test_exact_identity_and_fp32_accumulation(device, override):
     # identity placement (ref: tests/test_bfloat16.py:94-110): W = I gives y = x exactly
     size = 256
@@ -439,6 +439,7 @@ def spread(z, ldz, m, n, c, ldc):
     ("T", "N", 301, 9, 328, (121, 1)),     # streaming kernel, scalar stores
     ("T", "N", 512, 256, 320, (21, 1)),    # direct-to-LDS tiles
     ("T", "N", 512, 256, 320, (25, 2)),    # ... with K divided and the planes summed by a second kernel
+    ("T", "N", 512, 256, 320, (33, 1)),    # direct-to-LDS tiles on the 16 x 16 x 32 instruction
     ("T", "N", 1024, 40, 512, None),       # the planner's choice for a decode batch
     ("N", "N", 200, 150, 72, None),        # any-layout matrix-core kernel: addend spread first
     ("N", "T", 9, 7, 5, None),             # generic kernel: addend spread first
