@@ -38,7 +38,11 @@ struct Fp8DmaParams {
     int split_groups; // K groups per blockIdx.y (all of them without a split)
 };
 
-template <int TM, int WM, int STAGES, int TN>
+// NARROW: the products run on v_mfma_scale_f32_16x16x128_f8f6f4 (one instruction per 16 x 16 tile and
+// K group, four accumulator registers) instead of pairs of 32 x 32 x 64 ones: on operands with random
+// bits the part sustains 4.5 PFLOP/s with the former against 4.05 with the latter (it holds a higher
+// clock), and this kernel is limited by that clock.
+template <int TM, int WM, int STAGES, int TN, bool NARROW = false>
 __global__ __launch_bounds__(128 * WM) void fp8_dma_kernel(Fp8DmaParams p)
 {
     // (a fourth and a fifth stage were measured, with few and with many tokens: no gain, the kernel
@@ -120,7 +124,9 @@ __global__ __launch_bounds__(128 * WM) void fp8_dma_kernel(Fp8DmaParams p)
     // is older than the fills of the step that follows, so that step's wait covers it PERIOD - 1
     // steps before the slab is first read; a read is issued a few instructions before the step's
     // wait and its value is used after it.
-    const int frag_row = lane % 32, half = lane / 32;
+    // (32-wide instruction: operand row lane % 32, K half lane / 32; 16-wide: row lane % 16, K quarter lane / 16)
+    constexpr int FRAG_ROWS = NARROW ? 16 : 32, NJ = NARROW ? 2 * TM : TM; // token tiles per wavefront
+    const int frag_row = lane % FRAG_ROWS, half = lane / FRAG_ROWS;
     constexpr int LANES_PER_TOKEN = 2, SLAB_GROUPS = 4 * LANES_PER_TOKEN;
     constexpr int TOKENS_PER_WAVE = 64 / LANES_PER_TOKEN, LOADERS = BM / TOKENS_PER_WAVE;
     constexpr int PERIOD = SLAB_GROUPS / STAGES * STAGES;
@@ -141,10 +147,10 @@ __global__ __launch_bounds__(128 * WM) void fp8_dma_kernel(Fp8DmaParams p)
         load_to_lds_untracked(scale_resource, slab_lane_off, unsigned(first_group + slab * PERIOD) * 4u,
                               slab_at(slab) + loader * 64);
     };
-    int as_index[TM]; // float index of this lane's token inside a slab buffer (part 0, word 0)
+    int as_index[NJ]; // float index of this lane's token inside a slab buffer (part 0, word 0)
 #pragma unroll
-    for (int j = 0; j < TM; ++j) {
-        const int token = (wm * TM + j) * 32 + frag_row;
+    for (int j = 0; j < NJ; ++j) {
+        const int token = wm * TM * 32 + j * FRAG_ROWS + frag_row;
         as_index[j] = ((token / TOKENS_PER_WAVE) * 64 + token % TOKENS_PER_WAVE) * 4;
     }
     // (read with lds_read_unordered: the compiler would otherwise wait for every outstanding
@@ -183,14 +189,24 @@ __global__ __launch_bounds__(128 * WM) void fp8_dma_kernel(Fp8DmaParams p)
     const int frag_swizzle = lds_swizzle<CH>(frag_row);
     const int a_frag_base = (wn * TN * 32 + frag_row) * CH;
     const int b_frag_base = BN * CH + (wm * TM * 32 + frag_row) * CH;
-    f32x16_t acc[TN][TM];
+    f32x16_t acc[NARROW ? 1 : TN][NARROW ? 1 : TM];
+    constexpr int NI = 2 * TN; // 16-row weight tiles per wavefront
+    f32x4_t acc16[NARROW ? NI : 1][NARROW ? NJ : 1];
+    if constexpr (NARROW) {
 #pragma unroll
-    for (int i = 0; i < TN; ++i)
+        for (int i = 0; i < NI; ++i)
 #pragma unroll
-        for (int j = 0; j < TM; ++j)
+            for (int j = 0; j < NJ; ++j)
+                acc16[i][j] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+    } else {
 #pragma unroll
-            for (int r = 0; r < 16; ++r)
-                acc[i][j][r] = 0.f;
+        for (int i = 0; i < TN; ++i)
+#pragma unroll
+            for (int j = 0; j < TM; ++j)
+#pragma unroll
+                for (int r = 0; r < 16; ++r)
+                    acc[i][j][r] = 0.f;
+    }
 
     constexpr int UNIT = 0x7f7f7f7f; // E8M0 exponent 127 = scale 1.0 in every byte
     auto fragment = [&](const u32x4_t *stage, int base, int ks) {
@@ -199,12 +215,67 @@ __global__ __launch_bounds__(128 * WM) void fp8_dma_kernel(Fp8DmaParams p)
         return i32x8_t{int(lo[0]), int(lo[1]), int(lo[2]), int(lo[3]),
                        int(hi[0]), int(hi[1]), int(hi[2]), int(hi[3])};
     };
+    // operand of the 16-wide instruction: lane quarter c holds K positions 16c .. 16c+15 of its row in
+    // its first 16 bytes and 64+16c .. 64+16c+15 in its second 16 bytes
+    auto fragment16 = [&](const u32x4_t *stage, int base) {
+        u32x4_t lo = stage[base + (half ^ frag_swizzle)];
+        u32x4_t hi = stage[base + ((4 + half) ^ frag_swizzle)];
+        return i32x8_t{int(lo[0]), int(lo[1]), int(lo[2]), int(lo[3]),
+                       int(hi[0]), int(hi[1]), int(hi[2]), int(hi[3])};
+    };
+    // One K group on the 16-wide instruction. The token fragments are read once; the weight fragments
+    // travel one 16-row tile ahead in two register buffers; the tiles are walked in a software
+    // pipeline: the matrix instruction of tile t, a share of the LDS fills for the group STAGES-1
+    // ahead, then the four scaled accumulates of tile t-1.
+    auto multiply16 = [&](const u32x4_t *stage, u32x4_t *fill, const float (&as_now)[NJ], const float (&ws_now)[WS]) {
+        constexpr int TILES = NI * NJ, SHARE = (LOADS + TILES - 1) / TILES;
+        i32x8_t a_frag[2], b_frag[NJ];
+#pragma unroll
+        for (int j = 0; j < NJ; ++j)
+            b_frag[j] = fragment16(stage, b_frag_base + j * 16 * CH);
+        a_frag[0] = fragment16(stage, a_frag_base);
+        float scale[WS][NJ];
+#pragma unroll
+        for (int s = 0; s < WS; ++s)
+#pragma unroll
+            for (int j = 0; j < NJ; ++j)
+                scale[s][j] = __fmul_rn(as_now[j], ws_now[s]);
+        f32x4_t dot[2];
+#pragma unroll
+        for (int tile = 0; tile < TILES; ++tile) {
+            const int i = tile / NJ, j = tile % NJ;
+            __builtin_amdgcn_sched_barrier(0);
+            if (j == 0 && i + 1 < NI)
+                a_frag[(i + 1) & 1] = fragment16(stage, a_frag_base + (i + 1) * 16 * CH);
+            __builtin_amdgcn_sched_barrier(0);
+            dot[tile & 1] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(
+                a_frag[i & 1], b_frag[j], f32x4_t{0.f, 0.f, 0.f, 0.f}, 0, 0, 0, UNIT, 0, UNIT);
+            __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+            for (int index = tile * SHARE; index < (tile + 1) * SHARE && index < LOADS; ++index)
+                issue_one(fill, index);
+            __builtin_amdgcn_sched_barrier(0);
+            if (tile > 0) {
+                const int pi = (tile - 1) / NJ, pj = (tile - 1) % NJ;
+#pragma unroll
+                for (int r = 0; r < 4; ++r)
+                    acc16[pi][pj][r] = fmaf(dot[(tile - 1) & 1][r], scale[WS == 1 ? 0 : pi / 2][pj], acc16[pi][pj][r]);
+            }
+        }
+        __builtin_amdgcn_sched_barrier(0);
+        advance();
+#pragma unroll
+        for (int r = 0; r < 4; ++r)
+            acc16[NI - 1][NJ - 1][r] =
+                fmaf(dot[(TILES - 1) & 1][r], scale[WS == 1 ? 0 : (NI - 1) / 2][NJ - 1], acc16[NI - 1][NJ - 1][r]);
+        __builtin_amdgcn_sched_barrier(0);
+    };
     // One K group. The token fragments are read once; the weight fragments are streamed one
     // 32-row tile ahead (two register buffers), and the tiles are walked in a software pipeline: the
     // two MFMAs of tile t are issued, then a share of the LDS fills for the group STAGES-1 ahead,
     // then the 16 scaled accumulates of tile t-1, so that the vector ALU work and the load issue of
     // one tile run while the matrix cores execute the next (sched_barrier pins it).
-    auto multiply = [&](const u32x4_t *stage, u32x4_t *fill, const float (&as_now)[TM],
+    auto multiply = [&](const u32x4_t *stage, u32x4_t *fill, const float (&as_now)[NJ],
                         const float (&ws_now)[WS]) {
         constexpr int TILES = TN * TM, SHARE = (LOADS + TILES - 1) / TILES;
         // (eight tiles per wavefront at two wavefronts per SIMD leave no registers for a second
@@ -269,19 +340,22 @@ __global__ __launch_bounds__(128 * WM) void fp8_dma_kernel(Fp8DmaParams p)
         __builtin_amdgcn_sched_barrier(0);
     };
 
-    float ws_now[WS], as_now[TM];
+    float ws_now[WS], as_now[NJ];
     // One group: start the loads of the group STAGES-1 ahead into the stage that was read last,
     // multiply the current stage, read the next group's scales, then wait until only the newest
     // loads are still in flight (the wait also covers the scale reads).
     auto step = [&](int g, const u32x4_t *current, u32x4_t *fill) {
         const int next = g + 1 < group_count ? g + 1 : group_count - 1;
         __builtin_amdgcn_sched_barrier(0);
-        multiply(current, fill, as_now, ws_now);
+        if constexpr (NARROW)
+            multiply16(current, fill, as_now, ws_now);
+        else
+            multiply(current, fill, as_now, ws_now);
 #pragma unroll
         for (int s = 0; s < WS; ++s)
             ws_now[s] = weight_scale(s, next);
 #pragma unroll
-        for (int j = 0; j < TM; ++j)
+        for (int j = 0; j < NJ; ++j)
             as_now[j] = activation_scale(j, next);
         pipeline_barrier<(STAGES - 2) * LOADS>();
         tie_after_wait(ws_now, as_now);
@@ -299,7 +373,7 @@ __global__ __launch_bounds__(128 * WM) void fp8_dma_kernel(Fp8DmaParams p)
     for (int s = 0; s < WS; ++s)
         ws_now[s] = weight_scale(s, 0);
 #pragma unroll
-    for (int j = 0; j < TM; ++j)
+    for (int j = 0; j < NJ; ++j)
         as_now[j] = activation_scale(j, 0);
     __builtin_amdgcn_s_waitcnt(0xc07f); // lgkmcnt(0)
     tie_after_wait(ws_now, as_now);
@@ -322,6 +396,26 @@ __global__ __launch_bounds__(128 * WM) void fp8_dma_kernel(Fp8DmaParams p)
             step(g + s, stage_at(s), stage_at((s + STAGES - 1) % STAGES));
     wait_loads<0>();
 
+    if constexpr (NARROW) {
+        // register e of lane l in tile (i, j) is feature 16 i + 4 (l / 16) + e, token 16 j + l % 16
+        float *plane = p.partials ? p.partials + size_t(blockIdx.y) * size_t(p.m) * size_t(p.n) : nullptr;
+#pragma unroll
+        for (int j = 0; j < NJ; ++j) {
+            const int m = m0 + wm * TM * 32 + j * 16 + frag_row;
+#pragma unroll
+            for (int i = 0; i < NI; ++i) {
+                const int n = n0 + wn * TN * 32 + i * 16 + half * 4;
+                if (m >= p.m || n >= p.n)
+                    continue;
+                if (plane)
+                    *reinterpret_cast<f32x4_t *>(plane + size_t(m) * p.n + n) = acc16[i][j];
+                else
+                    *reinterpret_cast<u32x2_t *>(p.out + size_t(m) * p.out_pitch + n) =
+                        u32x2_t{pack_bf16x2(acc16[i][j][0], acc16[i][j][1]), pack_bf16x2(acc16[i][j][2], acc16[i][j][3])};
+            }
+        }
+        return;
+    }
     // ---- epilogue: accumulator register 4q+e of lane l is feature 8q + 4*(l/32) + e, token l%32
     if (p.partials) { // a share of the K groups: FP32 sums for the ordered reduction
         float *plane = p.partials + size_t(blockIdx.y) * size_t(p.m) * size_t(p.n);
@@ -361,7 +455,7 @@ __global__ __launch_bounds__(128 * WM) void fp8_dma_kernel(Fp8DmaParams p)
     }
 }
 
-template <int TM, int WM, int STAGES, int TN = 4>
+template <int TM, int WM, int STAGES, int TN = 4, bool NARROW = false>
 hipError_t launch_one(hipStream_t stream, Fp8DmaParams p, int splits)
 {
     constexpr int BN = 64 * TN, BM = 32 * WM * TM;
@@ -369,7 +463,7 @@ hipError_t launch_one(hipStream_t stream, Fp8DmaParams p, int splits)
     p.tiles_m = (p.m + BM - 1) / BM;
     if (size_t(p.tiles_n) * size_t(p.tiles_m) > 0x7fffffffu)
         return hipErrorInvalidValue;
-    fp8_dma_kernel<TM, WM, STAGES, TN>
+    fp8_dma_kernel<TM, WM, STAGES, TN, NARROW>
         <<<dim3(unsigned(p.tiles_n) * unsigned(p.tiles_m), unsigned(splits)), 128 * WM, 0, stream>>>(p);
     return launch_status();
 }
@@ -385,6 +479,13 @@ const TnVariant variants[] = {
     {"fp8dma192x128x128s3w8", 192, 128, 128, 512},
     {"fp8dma192x256x128w8", 192, 256, 128, 512},
     {"fp8dma192x64x128s3w4", 192, 64, 128, 256},
+    // the same tiles on the 16 x 16 x 128 matrix instruction (variants 0, 4, 6, 7, 8, 9)
+    {"fp8dma16-256x256x128w8", 256, 256, 128, 512},
+    {"fp8dma16-256x128x128s3w8", 256, 128, 128, 512},
+    {"fp8dma16-256x64x128s3w4", 256, 64, 128, 256},
+    {"fp8dma16-192x128x128s3w8", 192, 128, 128, 512},
+    {"fp8dma16-192x256x128w8", 192, 256, 128, 512},
+    {"fp8dma16-192x64x128s3w4", 192, 64, 128, 256},
 };
 } // namespace
 
@@ -411,6 +512,12 @@ hipError_t launch_rows(hipStream_t stream, int variant, int splits, const Fp8Dma
     case 7: return launch_one<1, 4, 3, 3>(stream, p, splits);
     case 8: return launch_one<2, 4, 2, 3>(stream, p, splits);
     case 9: return launch_one<1, 2, 3, 3>(stream, p, splits);
+    case 10: return launch_one<2, 4, 2, 4, true>(stream, p, splits);
+    case 11: return launch_one<1, 4, 3, 4, true>(stream, p, splits);
+    case 12: return launch_one<1, 2, 3, 4, true>(stream, p, splits);
+    case 13: return launch_one<1, 4, 3, 3, true>(stream, p, splits);
+    case 14: return launch_one<2, 4, 2, 3, true>(stream, p, splits);
+    case 15: return launch_one<1, 2, 3, 3, true>(stream, p, splits);
     default: return hipErrorInvalidValue;
     }
 }

@@ -494,6 +494,23 @@ Plan make_plan(int dtype, int algorithm, bool trans_a, bool trans_b, int m, int 
             }
         }
     }
+    // The 128-token and 256-token tiles also exist on the 16 x 16 x 128 matrix instruction, which the
+    // part runs at a higher clock on real data; that pays where the launch is bound by arithmetic
+    // (measured tile for tile: 256 x 256 at 4096 tokens 534 -> 509 us, 192 x 128 from 256 tokens on
+    // 2 to 6 % faster, 192 x 256 1 to 6 %; with fewer tokens, and on the 64-token tiles, the four
+    // times as many instructions per group cost more than the clock gives).
+    const auto narrow = [&](int variant) {
+        if (variant == 0 && n >= 2048)
+            return 10;
+        if (variant == 7 && n >= 256)
+            return 13;
+        if (variant == 8 && n >= 256)
+            return 14;
+        return variant;
+    };
+    plan.kernel = narrow(plan.kernel);
+    if (plan.tail_outputs)
+        plan.tail_kernel = narrow(plan.tail_kernel);
     return plan;
 }
 

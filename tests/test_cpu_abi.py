@@ -118,13 +118,13 @@ def test_planner_choices_for_the_baseline_shapes():
     assert "stream" not in describe(3, "T", "N", 7168, 16, 32768, 32768, 32768, 7168)[1]
     # 4.5 rounds of 256 x 256 tiles: four whole rounds, and the last 2048 outputs as one round of 256 x 128
     assert describe(3, "T", "N", 18432, 4096, 7168, 7168, 7168, 18432) == (
-        6000, "fp8-block128 fp8dma256x256x128w8 split_k=1, last 2048 outputs fp8dma256x128x128s3w8")
-    assert describe(3, "T", "N", 18432, 2048, 7168, 7168, 7168, 18432) == (6008, "fp8-block128 fp8dma192x256x128w8 split_k=1")
+        6010, "fp8-block128 fp8dma16-256x256x128w8 split_k=1, last 2048 outputs fp8dma256x128x128s3w8")
+    assert describe(3, "T", "N", 18432, 2048, 7168, 7168, 7168, 18432) == (6014, "fp8-block128 fp8dma16-192x256x128w8 split_k=1")
     # tiles and K shares are priced: 96 tiles of 192 rows fill the compute units at 256 tokens, a
     # narrow projection with a long K divides its groups, 256 x 256 tiles where 256 divides the outputs well
-    assert describe(3, "T", "N", 18432, 256, 7168, 7168, 7168, 18432)[1].endswith("fp8dma192x128x128s3w8 split_k=1")
-    assert describe(3, "T", "N", 7168, 256, 18432, 18432, 18432, 7168)[1].endswith("fp8dma192x128x128s3w8 split_k=3")
-    assert "fp8dma256x256x128w8 split_k=1" in describe(3, "T", "N", 7168, 4096, 18432, 18432, 18432, 7168)[1]
+    assert describe(3, "T", "N", 18432, 256, 7168, 7168, 7168, 18432)[1].endswith("fp8dma16-192x128x128s3w8 split_k=1")
+    assert describe(3, "T", "N", 7168, 256, 18432, 18432, 18432, 7168)[1].endswith("fp8dma16-192x128x128s3w8 split_k=3")
+    assert "fp8dma16-256x256x128w8 split_k=1" in describe(3, "T", "N", 7168, 4096, 18432, 18432, 18432, 7168)[1]
     assert describe(3, "T", "N", 24576, 512, 1536, 1536, 1536, 24576)[1].endswith("split_k=1")  # 12 groups: too few to divide
     # the plan is a pure function of its arguments
     assert describe(3, "T", "N", 18432, 16, 7168, 7168, 7168, 18432) == describe(

@@ -94,7 +94,7 @@ def test_streaming_decode_scale_table_limits(device, rows, inner):
     assert (np.abs(bf16_values(out) - wanted) <= bound).all()
 
 
-@pytest.mark.parametrize("code", list(range(20, 30)))
+@pytest.mark.parametrize("code", list(range(20, 36)))
 @pytest.mark.parametrize("rows,outputs,inner", [(70, 300, 512), (256, 512, 128), (513, 260, 896)])
 def test_direct_lds_load_variants(device, code, rows, outputs, inner):
     # partial tiles in both directions, a partial last weight-scale block, odd and even numbers of
@@ -109,7 +109,7 @@ def test_direct_lds_load_variants(device, code, rows, outputs, inner):
     assert (np.abs(bf16_values(out) - ordered) <= bound).all()
 
 
-@pytest.mark.parametrize("code,split", [(20, 2), (24, 3), (27, 2), (29, 7), (26, 64)])
+@pytest.mark.parametrize("code,split", [(20, 2), (24, 3), (27, 2), (29, 7), (26, 64), (30, 2), (31, 3), (35, 7)])
 @pytest.mark.parametrize("rows,outputs,inner", [(70, 300, 896), (129, 516, 1792)])
 def test_direct_lds_loads_with_divided_k_groups(device, code, split, rows, outputs, inner):
     # the K groups of a tile shared by several workgroups (uneven shares, more shares asked for than
@@ -152,7 +152,7 @@ def test_scale_indexing_is_bit_exact(device, override):
     assert np.array_equal(from_device_bf16(out), want)
 
 
-@pytest.mark.parametrize("override", [(code, 1) for code in range(20, 30)] + [(24, 3), (27, 2), (28, 5), (20, 4)])
+@pytest.mark.parametrize("override", [(code, 1) for code in range(20, 36)] + [(24, 3), (27, 2), (28, 5), (20, 4), (30, 4), (33, 2)])
 def test_scale_indexing_over_many_groups_is_bit_exact(device, override):
     # the same exact arithmetic over 29 K groups (an odd number: token rows of scales start at
     # every alignment; several rounds of the kernels' eight-group scale slabs, the last one partial),
