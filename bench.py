@@ -604,6 +604,29 @@ def extras(torch, _kernels, _native, device, normal):
     found["bf16_matmul_nn_4096"] = {"us": round(seconds * 1e6, 1),
                                     "roofline": roofline_of("mfma bf16", 2.0 * size**3, seconds)}
     del x, w, y
+    # BF16 linear at 256 tokens on a square projection (64 tiles of 128 x 256 for 256 compute units:
+    # K is divided over workgroups); five weight copies rotate so that the weights come from HBM
+    outputs, inner, tokens = 8192, 8192, 256
+    copies = [normal((outputs, inner), 0.02) for _ in range(5)]
+    x = normal((tokens, inner))
+    y = torch.empty((tokens, outputs), dtype=torch.bfloat16, device=device)
+    seconds = event_time(torch, lambda i: _kernels.matmul(x, copies[i % 5].t(), out=y), 10, 60)
+    found["bf16_linear_256_tokens_8192x8192"] = {
+        "us": round(seconds * 1e6, 1), "tflops": round(2.0 * tokens * outputs * inner / seconds / 1e12, 1),
+        "roofline": roofline_of("hbm", outputs * inner * 2 + tokens * (inner + outputs) * 2, seconds),
+        "plan": _native.plan_describe(2, "T", "N", outputs, tokens, inner, inner, inner, outputs)[1],
+    }
+    # x @ W with a row-major W [inner, outputs] ('N','N') and 16 tokens: the kernel that streams W as it lies
+    tokens = 16
+    x = normal((tokens, inner))
+    y = torch.empty((tokens, outputs), dtype=torch.bfloat16, device=device)
+    seconds = event_time(torch, lambda i: _kernels.matmul(x, copies[i % 5], out=y), 10, 60)
+    found["bf16_x_at_w_row_major_16_tokens_8192x8192"] = {
+        "us": round(seconds * 1e6, 1),
+        "roofline": roofline_of("hbm", outputs * inner * 2 + tokens * (inner + outputs) * 2, seconds),
+        "plan": _native.plan_describe(2, "N", "N", outputs, tokens, inner, outputs, inner, outputs)[1],
+    }
+    del copies, x, y
     # FP8 block-scaled linear; the decode sizes rotate three weight copies (396 MB) so that the
     # weights come from HBM rather than from the 256 MB last-level cache
     outputs, inner = 18432, 7168
@@ -672,6 +695,18 @@ def extras(torch, _kernels, _native, device, normal):
                     "roofline": roofline_of("mfma fp8", flops, seconds)}
         del w, scale, a, a_scale
     found["mx_quantized_matmul_m4096_18432x7168"] = mx
+    # a narrow projection with a long K at 128 rows (56 tiles of 128 x 128 for 256 compute units: K is
+    # divided over workgroups); five weight copies rotate so that the weights come from HBM
+    mx = {}
+    for name, packed in (("e4m3", False), ("e2m1", True)):
+        parts = [mx_operands(torch, device, packed, 128, 7168, 18432) for _ in range(5 if not packed else 8)]
+        a, a_scale = parts[0][2], parts[0][3]
+        seconds = event_time(
+            torch, lambda i: _kernels.quantized_matmul(a, a_scale, parts[i % len(parts)][0], parts[i % len(parts)][1]), 10, 60)
+        traffic = parts[0][0].numel() + parts[0][1].numel() + 128 * (18432 + 18432 // 32 + 7168 * 2)
+        mx[name] = {"us": round(seconds * 1e6, 1), "roofline": roofline_of("hbm", traffic, seconds)}
+        del parts, a, a_scale
+    found["mx_quantized_matmul_m128_7168x18432"] = mx
     # the grouped form as an MoE prefill meets it: 32 experts of [4096, 7168] with a capacity of 1024
     # rows each, every expert a quarter full (the rest of the capacity comes back as zeros)
     experts, capacity, features, inner = 32, 1024, 4096, 7168
