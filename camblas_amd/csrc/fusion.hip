@@ -66,6 +66,41 @@ __global__ void swiglu_kernel(size_t count, int width, float limit, const T *gat
     }
 }
 
+// Eight BF16 per thread per step; same arithmetic (a row is a whole number of such vectors, so one
+// routing factor serves a vector).
+__global__ void swiglu_bf16x8_kernel(size_t vectors, int row_vectors, float limit, const u32x4_t *gate,
+                                     const u32x4_t *up, const float *routing, u32x4_t *out)
+{
+    for (size_t index = size_t(blockIdx.x) * blockDim.x + threadIdx.x; index < vectors;
+         index += size_t(gridDim.x) * blockDim.x) {
+        const u32x4_t g = gate[index], u = up[index];
+        const float factor = routing ? routing[index / size_t(row_vectors)] : 1.f;
+        u32x4_t r;
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+            float value[2];
+#pragma unroll
+            for (int h = 0; h < 2; ++h) {
+                float gv = __uint_as_float(h ? g[e] & 0xffff0000u : g[e] << 16);
+                float uv = __uint_as_float(h ? u[e] & 0xffff0000u : u[e] << 16);
+                if (limit > 0) {
+                    if (gv > limit)
+                        gv = limit;
+                    if (uv > limit)
+                        uv = limit;
+                    if (uv < -limit)
+                        uv = -limit;
+                }
+                value[h] = __fmul_rn(gv / (1.f + expf(-gv)), uv);
+                if (routing)
+                    value[h] = __fmul_rn(factor, value[h]);
+            }
+            r[e] = pack_bf16x2(value[0], value[1]);
+        }
+        out[index] = r;
+    }
+}
+
 // ---------------------------------------------------------------- RMS normalisation rows
 // One workgroup per row. added = round_T(x + r) when a residual is given; scale = rsqrt(mean(v^2) +
 // eps); out = round_T(round_T(v*scale) * w) or, without intermediate rounding, round_T((v*scale)*w)
@@ -361,6 +396,10 @@ hipError_t launch_swiglu(hipStream_t stream, int dtype, uint64_t count, int widt
         swiglu_kernel<float><<<stride_blocks(count), 256, 0, stream>>>(
             count, width, limit, static_cast<const float *>(gate), static_cast<const float *>(up),
             routing, static_cast<float *>(out));
+    else if (width % 8 == 0 && count % 8 == 0 && aligned16(gate) && aligned16(up) && aligned16(out))
+        swiglu_bf16x8_kernel<<<stride_blocks(count / 8), 256, 0, stream>>>(
+            count / 8, width / 8, limit, static_cast<const u32x4_t *>(gate), static_cast<const u32x4_t *>(up), routing,
+            static_cast<u32x4_t *>(out));
     else
         swiglu_kernel<bf16_storage><<<stride_blocks(count), 256, 0, stream>>>(
             count, width, limit, static_cast<const bf16_storage *>(gate),

@@ -47,8 +47,9 @@ def test_silu_multiply_f32_and_in_place(device):
 
 @pytest.mark.parametrize("limit", [0.0, 1.5])
 @pytest.mark.parametrize("routed", [False, True])
-def test_swiglu_bf16(device, limit, routed):
-    rows, width = 7, 520
+@pytest.mark.parametrize("width", [520, 515])  # eight values per thread, or one by one
+def test_swiglu_bf16(device, limit, routed, width):
+    rows = 7
     gate = oracle.fill_normal_bf16(5, (rows, width), std=2.0)
     up = oracle.fill_normal_bf16(6, (rows, width), std=2.0)
     routing = oracle.fill_uniform(7, (rows,), 0.1, 1.0) if routed else None
