@@ -132,6 +132,66 @@ __global__ __launch_bounds__(THREADS) void reduce_groups_kernel(int choices, int
         output[size_t(token) * width + column] = sum;
     }
 }
+// The same with eight columns per thread (16-byte loads, all rows of a step's eight choices requested
+// before the first is added) and the columns of a token spread over gridDim.y workgroups: a token
+// summed one column and one choice at a time is a chain of 28 x 8 dependent 2-byte loads (36 us for
+// one token of 7168 columns; 2.2 TB/s at 8192 tokens).
+__global__ __launch_bounds__(THREADS) void reduce_groups_wide_kernel(int choices, int vectors, int grouped_rows,
+                                                                     const int64_t *experts, const int32_t *reverse,
+                                                                     const u32x4_t *input, f32x4_t *output)
+{
+    __shared__ int ordered_row[64];
+    __shared__ int ordered_count;
+    const int token = blockIdx.x, thread = threadIdx.x;
+    const int64_t *mine = experts + size_t(token) * choices;
+    if (thread < 64)
+        ordered_row[thread] = -1;
+    __syncthreads();
+    if (thread < choices) {
+        const int64_t expert = mine[thread];
+        const bool valid = expert >= 0 && expert < INT_MAX;
+        int rank = 0, valid_total = 0;
+        for (int other = 0; other < choices; ++other) {
+            const int64_t theirs = mine[other];
+            const bool theirs_valid = theirs >= 0 && theirs < INT_MAX;
+            valid_total += theirs_valid;
+            rank += theirs_valid && (theirs < expert || (theirs == expert && other < thread));
+        }
+        if (valid) {
+            const int row = reverse[size_t(token) * choices + thread];
+            ordered_row[rank] = row >= 0 && row < grouped_rows ? row : -1;
+        }
+        if (thread == 0)
+            ordered_count = valid_total;
+    }
+    __syncthreads();
+    const int count = ordered_count;
+    for (int vector = int(blockIdx.y) * THREADS + thread; vector < vectors; vector += int(gridDim.y) * THREADS) {
+        float sum[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+        for (int first = 0; first < count; first += 8) {
+            u32x4_t part[8];
+            bool present[8];
+#pragma unroll
+            for (int step = 0; step < 8; ++step) {
+                const int row = first + step < count ? ordered_row[first + step] : -1;
+                present[step] = row >= 0;
+                part[step] = input[size_t(present[step] ? row : 0) * vectors + vector];
+            }
+#pragma unroll
+            for (int step = 0; step < 8; ++step)
+                if (present[step]) {
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) {
+                        sum[2 * e] = __fadd_rn(sum[2 * e], __uint_as_float(part[step][e] << 16));
+                        sum[2 * e + 1] = __fadd_rn(sum[2 * e + 1], __uint_as_float(part[step][e] & 0xffff0000u));
+                    }
+                }
+        }
+        f32x4_t *out = output + (size_t(token) * vectors + vector) * 2;
+        out[0] = f32x4_t{sum[0], sum[1], sum[2], sum[3]};
+        out[1] = f32x4_t{sum[4], sum[5], sum[6], sum[7]};
+    }
+}
 } // namespace
 
 hipError_t launch_route_groups(hipStream_t stream, int tokens, int choices, int first_expert,
@@ -160,6 +220,16 @@ hipError_t launch_reduce_groups(hipStream_t stream, int tokens, int choices, int
                                 int grouped_rows, const void *experts, const void *reverse,
                                 const void *input, void *output)
 {
+    if (width % 8 == 0 && grouped_rows > 0 && reinterpret_cast<uintptr_t>(input) % 16 == 0 &&
+        reinterpret_cast<uintptr_t>(output) % 16 == 0) {
+        const int vectors = width / 8;
+        const int chunks = (vectors + THREADS - 1) / THREADS;
+        const dim3 grid(unsigned(tokens), unsigned(chunks < 8 ? chunks : 8));
+        reduce_groups_wide_kernel<<<grid, THREADS, 0, stream>>>(
+            choices, vectors, grouped_rows, static_cast<const int64_t *>(experts), static_cast<const int32_t *>(reverse),
+            static_cast<const u32x4_t *>(input), static_cast<f32x4_t *>(output));
+        return launch_status();
+    }
     reduce_groups_kernel<<<unsigned(tokens), THREADS, 0, stream>>>(
         choices, width, grouped_rows, static_cast<const int64_t *>(experts),
         static_cast<const int32_t *>(reverse), static_cast<const unsigned short *>(input),

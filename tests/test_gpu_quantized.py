@@ -233,7 +233,7 @@ def test_route_groups_is_exact(device, tokens, choices, groups, rows):
             assert experts.reshape(-1)[slot] - first == active[group]
 
 
-@pytest.mark.parametrize("tokens,choices,width", [(1, 8, 7168), (9, 4, 257), (3, 64, 40)])
+@pytest.mark.parametrize("tokens,choices,width", [(1, 8, 7168), (9, 4, 257), (3, 64, 40), (5, 12, 4104), (2, 3, 20480)])
 def test_reduce_groups_is_exact(device, tokens, choices, width):
     rng = np.random.default_rng(tokens + choices)
     grouped_rows = 50
