@@ -36,12 +36,18 @@ __global__ __launch_bounds__(THREADS) void route_fill_kernel(int groups, size_t 
         reverse[index] = -1;
 }
 
-__global__ __launch_bounds__(THREADS) void route_assign_kernel(int slot_count, int first_expert,
-                                                               int rows, const int64_t *experts,
-                                                               const int32_t *active, int32_t *counts,
-                                                               int32_t *slots, int32_t *reverse)
+// One workgroup of sixteen wavefronts per group. The slots are divided into sixteen contiguous
+// ranges, one per wavefront; a first pass counts each range's matches, one barrier turns the counts
+// into the row at which each range starts, and a second pass hands out the rows in ascending slot
+// order. (A workgroup-wide prefix sum per 256 slots, two barriers each, took 92 us for 65536 slots.)
+constexpr int ROUTE_THREADS = 1024;
+__global__ __launch_bounds__(ROUTE_THREADS) void route_assign_kernel(int slot_count, int first_expert,
+                                                                     int rows, const int64_t *experts,
+                                                                     const int32_t *active, int32_t *counts,
+                                                                     int32_t *slots, int32_t *reverse)
 {
-    __shared__ int wave_total[THREADS / 64];
+    constexpr int WAVES = ROUTE_THREADS / 64;
+    __shared__ int wave_total[WAVES];
     __shared__ int earlier;
     const int group = blockIdx.x, thread = threadIdx.x, lane = thread % 64, wave = thread / 64;
     const int local = active[group];
@@ -49,42 +55,47 @@ __global__ __launch_bounds__(THREADS) void route_assign_kernel(int slot_count, i
     if (thread == 0)
         earlier = 0;
     __syncthreads();
-    for (int other = thread; other < group; other += THREADS)
+    for (int other = thread; other < group; other += ROUTE_THREADS)
         if (active[other] == local)
             earlier = 1;
     __syncthreads();
     if (earlier)
         return; // counts[group] stays 0, slots stay -1
-    int assigned = 0; // uniform over the workgroup
-    for (int base = 0; base < slot_count; base += THREADS) {
-        const int slot = base + thread;
-        bool mine = false;
-        if (slot < slot_count) {
-            const int64_t expert = experts[slot];
-            mine = expert >= first_expert && expert < INT_MAX && int(expert) - first_expert == local;
-        }
-        const unsigned long long ballot = __ballot(mine);
-        const int before = __popcll(ballot & ((1ull << lane) - 1ull));
-        if (lane == 0)
-            wave_total[wave] = __popcll(ballot);
-        __syncthreads();
-        int offset = assigned, total = 0;
+    const int range = ((slot_count + WAVES - 1) / WAVES + 63) / 64 * 64;
+    const int begin = wave * range < slot_count ? wave * range : slot_count;
+    const int end = begin + range < slot_count ? begin + range : slot_count;
+    auto matches = [&](int slot) {
+        if (slot >= end)
+            return false;
+        const int64_t expert = experts[slot];
+        return expert >= first_expert && expert < INT_MAX && int(expert) - first_expert == local;
+    };
+    int found = 0;
+    for (int base = begin; base < end; base += 64)
+        found += __popcll(__ballot(matches(base + lane)));
+    if (lane == 0)
+        wave_total[wave] = found;
+    __syncthreads();
+    int row = 0, total = 0;
 #pragma unroll
-        for (int w = 0; w < THREADS / 64; ++w) {
-            if (w < wave)
-                offset += wave_total[w];
-            total += wave_total[w];
+    for (int w = 0; w < WAVES; ++w) {
+        if (w < wave)
+            row += wave_total[w];
+        total += wave_total[w];
+    }
+    for (int base = begin; base < end; base += 64) {
+        const int slot = base + lane;
+        const bool mine = matches(slot);
+        const unsigned long long ballot = __ballot(mine);
+        const int mine_row = row + __popcll(ballot & ((1ull << lane) - 1ull));
+        if (mine && mine_row < rows) {
+            slots[size_t(group) * rows + mine_row] = slot;
+            reverse[slot] = group * rows + mine_row;
         }
-        const int row = offset + before;
-        if (mine && row < rows) {
-            slots[size_t(group) * rows + row] = slot;
-            reverse[slot] = group * rows + row;
-        }
-        assigned += total;
-        __syncthreads();
+        row += __popcll(ballot);
     }
     if (thread == 0)
-        counts[group] = assigned;
+        counts[group] = total;
 }
 
 // One workgroup per token: the choices are ranked by (expert ID, choice) once, then every thread
@@ -209,7 +220,7 @@ hipError_t launch_route_groups(hipStream_t stream, int tokens, int choices, int 
     hipError_t status = launch_status();
     if (status != hipSuccess || !tokens)
         return status;
-    route_assign_kernel<<<unsigned(groups), THREADS, 0, stream>>>(
+    route_assign_kernel<<<unsigned(groups), ROUTE_THREADS, 0, stream>>>(
         tokens * choices, first_expert, rows, static_cast<const int64_t *>(experts),
         static_cast<const int32_t *>(active), static_cast<int32_t *>(counts),
         static_cast<int32_t *>(slots), static_cast<int32_t *>(reverse));
