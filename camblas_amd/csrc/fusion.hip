@@ -275,15 +275,25 @@ __global__ void rms_scale_kernel(size_t count, int width, float epsilon, const T
 // ---------------------------------------------------------------- rotary embedding
 // Rotate-half pairing (i, i + dim/2), angle = position * theta^(-2i/dim), FP32 sin/cos, one BF16
 // rounding per element. One thread per (token, head, i).
-__device__ __forceinline__ void rotate_pair(float position, int i, int dim, float theta, float lo,
-                                            float hi, unsigned short &out_lo, unsigned short &out_hi)
+__device__ __forceinline__ void pair_sincos(float position, int i, int dim, float theta, float &s, float &c)
 {
     float frequency = exp2f(-2.f * float(i) / float(dim) * log2f(theta));
     float angle = position * frequency;
-    float s, c;
     sincosf(angle, &s, &c);
-    out_lo = float_to_bf16_bits(lo * c - hi * s);
-    out_hi = float_to_bf16_bits(hi * c + lo * s);
+}
+__device__ __forceinline__ void rotate_by(float s, float c, float lo, float hi, unsigned short &out_lo,
+                                          unsigned short &out_hi)
+{
+    // (written out so that every kernel rounds in the same places whatever the compiler would contract)
+    out_lo = float_to_bf16_bits(__fmaf_rn(lo, c, -__fmul_rn(hi, s)));
+    out_hi = float_to_bf16_bits(__fmaf_rn(hi, c, __fmul_rn(lo, s)));
+}
+__device__ __forceinline__ void rotate_pair(float position, int i, int dim, float theta, float lo,
+                                            float hi, unsigned short &out_lo, unsigned short &out_hi)
+{
+    float s, c;
+    pair_sincos(position, i, dim, theta, s, c);
+    rotate_by(s, c, lo, hi, out_lo, out_hi);
 }
 
 __global__ void rope_kernel(int tokens, int heads, int dim, int token_stride, float theta,
@@ -300,6 +310,42 @@ __global__ void rope_kernel(int tokens, int heads, int dim, int token_stride, fl
     unsigned short *v = x + size_t(token) * token_stride + size_t(head) * dim;
     rotate_pair(float(positions[token]), i, dim, theta, bf16_bits_to_float(v[i]),
                 bf16_bits_to_float(v[i + half]), v[i], v[i + half]);
+}
+
+// Many tokens: one workgroup per token works out the sine and cosine of each pair index once (they
+// do not depend on the head; one thread per (token, head, i) repeats them for every head and runs at
+// the rate of the trigonometry, 2 TB/s) and then rotates eight pairs per thread with 16-byte
+// accesses. Same arithmetic per element as rope_kernel.
+__global__ __launch_bounds__(256) void rope_rows_kernel(int heads, int dim, int token_stride, float theta,
+                                                        const int32_t *positions, unsigned short *x)
+{
+    __shared__ float sines[512], cosines[512];
+    const int half = dim / 2, token = blockIdx.x, thread = threadIdx.x;
+    const float position = float(positions[token]);
+    for (int i = thread; i < half; i += 256)
+        pair_sincos(position, i, dim, theta, sines[i], cosines[i]);
+    __syncthreads();
+    const int chunks = half / 8; // 8 pairs per thread and step
+    unsigned short *row = x + size_t(token) * token_stride;
+    for (int item = thread; item < heads * chunks; item += 256) {
+        const int head = item / chunks, first = item % chunks * 8;
+        u32x4_t *lo_at = reinterpret_cast<u32x4_t *>(row + size_t(head) * dim + first);
+        u32x4_t *hi_at = reinterpret_cast<u32x4_t *>(row + size_t(head) * dim + half + first);
+        const u32x4_t lo = *lo_at, hi = *hi_at;
+        u32x4_t out_lo, out_hi;
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+            unsigned short l0, h0, l1, h1;
+            rotate_by(sines[first + 2 * e], cosines[first + 2 * e], __uint_as_float(lo[e] << 16),
+                      __uint_as_float(hi[e] << 16), l0, h0);
+            rotate_by(sines[first + 2 * e + 1], cosines[first + 2 * e + 1], __uint_as_float(lo[e] & 0xffff0000u),
+                      __uint_as_float(hi[e] & 0xffff0000u), l1, h1);
+            out_lo[e] = unsigned(l0) | (unsigned(l1) << 16);
+            out_hi[e] = unsigned(h0) | (unsigned(h1) << 16);
+        }
+        *lo_at = out_lo;
+        *hi_at = out_hi;
+    }
 }
 
 // Decode-step form of the two kernels above and below in one launch: a fused QKV activation row
@@ -507,6 +553,12 @@ hipError_t launch_rope_kv_append(hipStream_t stream, int batch, int q_heads, int
 hipError_t launch_rope(hipStream_t stream, int tokens, int heads, int dim, int token_stride,
                        float theta, const int32_t *positions, void *x)
 {
+    // (from 64 tokens on; fewer tokens are spread over more workgroups by the kernel below)
+    if (tokens >= 64 && dim % 16 == 0 && dim <= 1024 && token_stride % 8 == 0 && reinterpret_cast<uintptr_t>(x) % 16 == 0) {
+        rope_rows_kernel<<<unsigned(tokens), 256, 0, stream>>>(heads, dim, token_stride, theta, positions,
+                                                               static_cast<unsigned short *>(x));
+        return launch_status();
+    }
     size_t count = size_t(tokens) * heads * (dim / 2);
     rope_kernel<<<unsigned((count + 255) / 256), 256, 0, stream>>>(
         tokens, heads, dim, token_stride, theta, positions, static_cast<unsigned short *>(x));

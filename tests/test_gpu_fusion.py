@@ -137,6 +137,25 @@ def test_rope(device):
     assert rel_frobenius(bf16_values(out), oracle.bf16_to_f32(want)) <= 1e-2
 
 
+def test_rope_over_many_tokens_equals_rope_over_few(device):
+    # from 64 tokens on one workgroup per token works the angles out once for all heads; the result
+    # must equal, bit for bit, the same tokens rotated 50 at a time by the kernel with one thread per
+    # (token, head, pair); views with a token stride (the q and k heads of a fused activation) included
+    tokens, heads, dim = 150, 9, 128
+    x = oracle.fill_normal_bf16(21, (tokens, heads + 2, dim))
+    positions = torch.from_numpy(np.arange(tokens, dtype=np.int32) * 37 % 5000).to(device)
+    many, few = to_device_bf16(x, device), to_device_bf16(x, device)
+    _kernels.rope(many[:, :heads], positions)
+    for first in range(0, tokens, 50):
+        _kernels.rope(few[first:first + 50, :heads], positions[first:first + 50])
+    torch.cuda.synchronize()
+    differing = np.argwhere(from_device_bf16(many) != from_device_bf16(few))
+    assert len(differing) == 0, (len(differing), differing[:5])
+    assert np.array_equal(from_device_bf16(many)[:, heads:], x[:, heads:])
+    want = oracle.rope(x[:, :heads], positions.cpu().numpy(), 5e5)
+    assert rel_frobenius(bf16_values(many[:, :heads]), oracle.bf16_to_f32(want)) <= 1e-2
+
+
 @pytest.mark.parametrize("batch,q_heads,kv_heads,context", [(3, 16, 2, 700), (2, 8, 8, 256),
                                                             (2, 12, 4, 300), (1, 64, 8, 2048),
                                                             (3, 32, 2, 520), (2, 5, 5, 65)])
