@@ -98,7 +98,7 @@ struct DmaPrice {
     int variant;
     double step_us, kilobytes_in_flight;
 };
-const DmaPrice dma_prices[] = {{5, 0.580, 64}, {9, 0.849, 96}, {6, 1.682, 64},
+const DmaPrice dma_prices[] = {{5, 0.557, 64}, {9, 0.849, 96}, {6, 1.632, 64},
                                {8, 0.943, 96}, {10, 1.878, 72}, {11, 1.281, 56}};
 double dma_launch_us(const DmaPrice &price, int outputs, int tokens, int k, int shares, int compute_units)
 {
@@ -312,7 +312,7 @@ Plan make_plan(int dtype, int algorithm, bool trans_a, bool trans_b, int m, int 
                 const struct {
                     int variant, resident;
                     double weight;
-                } candidates[] = {{10, 1, 1.0}, {6, 1, 0.93}, {11, 1, 0.88}, {9, 1, 0.85}, {5, 1, 0.8}};
+                } candidates[] = {{10, 1, 1.0}, {6, 1, 0.96}, {11, 1, 0.88}, {9, 1, 0.85}, {5, 1, 0.83}};
                 plan.family = FAMILY_DMA;
                 for (const auto &candidate : candidates) {
                     const TnVariant &v = dma_variant(candidate.variant);
