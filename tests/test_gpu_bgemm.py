@@ -470,12 +470,12 @@ def test_addend_apart_from_the_output(device, ta, tb, m, n, k, override, ldz_kin
 
 @pytest.mark.parametrize("ldz_kind", [None, "row", "matrix"])
 def test_plan_that_ends_with_a_second_launch(device, ldz_kind):
-    # 14336 outputs x 2048 tokens is 1.4 rounds of 320 x 256 tiles: the planner covers the first
-    # 10240 outputs with one whole round and the last 4096 with a second launch of smaller tiles.
+    # 28672 outputs x 1024 tokens is 1.4 rounds of 320 x 256 tiles: the planner covers the first
+    # 20480 outputs with one whole round and the last 8192 with a second launch of smaller tiles.
     # Weights, output and addend of that launch start at an offset, with padded pitches.
-    m, n, k = 14336, 2048, 1024
+    m, n, k = 28672, 1024, 1024
     lda, ldb, ldc = k + 8, k + 16, m + 4
-    assert ", last 4096 outputs " in _native.plan_describe(2, "T", "N", m, n, k, lda, ldb, ldc)[1]
+    assert ", last 8192 outputs " in _native.plan_describe(2, "T", "N", m, n, k, lda, ldb, ldc)[1]
     a = oracle.fill_normal_bf16(51, (lda * m,), std=0.05)
     b = oracle.fill_normal_bf16(52, (ldb * n,))
     c = oracle.fill_normal_bf16(53, (ldc * n,))
@@ -490,7 +490,7 @@ def test_plan_that_ends_with_a_second_launch(device, ldz_kind):
         got = run_bgemm_add(device, "T", "N", m, n, k, alpha, a, lda, b, ldb, beta, z, ldz, c, ldc)
     want, want64 = reference("T", "N", m, n, k, alpha, a, lda, b, ldb, beta, start, ldc)
     got2d = got.reshape(n, ldc)
-    for first, last in ((0, 10240), (10240, m)):  # each launch's share holds the bar by itself
+    for first, last in ((0, 20480), (20480, m)):  # each launch's share holds the bar by itself
         error = rel_frobenius(oracle.bf16_to_f32(got2d[:, first:last]), want64.reshape(n, m)[:, first:last])
         assert error <= TOLERANCE, (first, error)
     assert np.array_equal(got2d[:, m:], c.reshape(n, ldc)[:, m:])
