@@ -156,16 +156,39 @@ int ordinary(const Entry &entry, const Product &p, float alpha, const float *a, 
     return entry.finish(launched, "classical GEMM");
 }
 
-// the ordinary FP64 product: matrix cores when every dimension holds a 16 x 16 x 4 tile
+// the ordinary FP64 product: matrix cores when every dimension holds a 16 x 16 x 4 tile, K divided
+// over workgroups when the tiles alone would leave most compute units idle
 // (ref: backend.cu:1066-1073)
 int ordinary(const Entry &entry, const Product &p, double alpha, const double *a, const double *b,
              double beta, double *c, bool)
 {
     camblas_cuda_context *context = entry.context();
     context->counts[0]++;
-    bool matrix = p.m >= 16 && p.n >= 16 && p.k >= 4;
+    // (fewer than 16 columns against a large A still go to the tiles: with K divided they run at
+    // five times the rate of the vector-ALU kernel, whose grid would be a few dozen workgroups)
+    bool matrix = p.m >= 16 && (p.n >= 16 || (p.m >= 256 && p.k >= 512)) && p.k >= 4;
     if (context->override_kernel >= 0) // tests: 0 vector-ALU tiles, else matrix-core tiles
         matrix = context->override_kernel >= 1;
+    // a handful of columns against a large A: the 128 x 128 tiles alone would occupy a fraction of
+    // the compute units, so K is divided over workgroups (the FP32 rule with this kernel's tile)
+    int shares = 1;
+    if (matrix && context->override_kernel < 0 && p.m >= 256 && p.k >= 512) {
+        const long long tiles = (long long)((p.m + 127) / 128) * ((p.n + 127) / 128);
+        for (int s : {32, 16, 8, 4, 2})
+            if (tiles * s <= 2LL * context->compute_units && p.k % s == 0 && p.k / s >= 256) {
+                shares = s;
+                break;
+            }
+    }
+    if (shares > 1) {
+        // without room for the planes (allocation failure, capture in progress) K stays undivided
+        if (reserve_scratch(context, size_t(shares) * size_t(p.m) * size_t(p.n) * 8) == hipSuccess)
+            return entry.finish(launch_dgemm_mfma_divided(context->stream, p.trans_a, p.trans_b, p.m, p.n, p.k, alpha,
+                                                          a, p.lda, b, p.ldb, beta, c, p.ldc, shares,
+                                                          static_cast<double *>(context->scratch)),
+                                "classical FP64 GEMM");
+        context->counts[5]++;
+    }
     const hipError_t launched =
         matrix ? launch_dgemm_mfma(context->stream, p.trans_a, p.trans_b, p.m, p.n, p.k, alpha, a, p.lda, b,
                                    p.ldb, beta, c, p.ldc)

@@ -136,6 +136,9 @@ hipError_t launch_sgemm_mfma_divided(hipStream_t stream, bool ta, bool tb, int m
 hipError_t launch_dgemm_mfma(hipStream_t stream, bool ta, bool tb, int m, int n, int k, double alpha,
                              const double *a, int lda, const double *b, int ldb, double beta, double *c,
                              int ldc, int batches = 1, size_t batch_stride = 0, bool lower_only = false);
+hipError_t launch_dgemm_mfma_divided(hipStream_t stream, bool ta, bool tb, int m, int n, int k, double alpha,
+                                     const double *a, int lda, const double *b, int ldb, double beta,
+                                     double *c, int ldc, int shares, double *planes);
 // c[row, column] = c[column, row] for row < column of a column-major n x n matrix (dtype 0 FP32, 1 FP64)
 hipError_t launch_mirror_lower(hipStream_t stream, int dtype, int n, void *c, int ldc);
 // Strassen policies for square 'N','N' products (strassen.hip). strassen_levels: recursion depth of

@@ -19,6 +19,9 @@ namespace
 typedef double f64x4_t __attribute__((ext_vector_type(4)));
 
 constexpr int TILE = 128, DEPTH = 16, THREADS = 256;
+struct BatchStrides {
+    size_t a, b, c; // elements from one product of a batch to the next, per operand
+};
 constexpr int K_MAJOR_PITCH = TILE + 16, ROW_MAJOR_PITCH = DEPTH + 1;
 constexpr int TILE_WORDS = DEPTH * K_MAJOR_PITCH; // >= TILE * ROW_MAJOR_PITCH
 static_assert(TILE * ROW_MAJOR_PITCH <= TILE_WORDS, "one buffer serves both layouts");
@@ -34,15 +37,15 @@ template <bool TA, bool TB>
 __global__ __launch_bounds__(THREADS, 2) void dgemm_mfma_kernel(int m, int n, int k, double alpha,
                                                              const double *a, int lda, const double *b,
                                                              int ldb, double beta, double *c, int ldc,
-                                                             size_t batch_stride, bool lower_only)
+                                                             BatchStrides batch_strides, bool lower_only)
 {
     // a symmetric product: only the tiles that reach the diagonal, the rest is the mirroring pass
     int row0 = blockIdx.x * TILE, col0 = blockIdx.y * TILE;
     if (lower_only && !lower_tile<TILE, TILE>(blockIdx.x, n, row0, col0))
         return;
-    a += blockIdx.z * batch_stride; // one independent product per grid z-slice
-    b += blockIdx.z * batch_stride;
-    c += blockIdx.z * batch_stride;
+    a += blockIdx.z * batch_strides.a; // one independent product per grid z-slice
+    b += blockIdx.z * batch_strides.b;
+    c += blockIdx.z * batch_strides.c;
     __shared__ double tile_a[TILE_WORDS];
     __shared__ double tile_b[TILE_WORDS];
     const int thread = threadIdx.x, lane = thread % 64, wave = thread / 64;
@@ -130,9 +133,11 @@ __global__ __launch_bounds__(THREADS, 2) void dgemm_mfma_kernel(int m, int n, in
 }
 } // namespace
 
-hipError_t launch_dgemm_mfma(hipStream_t stream, bool ta, bool tb, int m, int n, int k, double alpha,
-                             const double *a, int lda, const double *b, int ldb, double beta, double *c,
-                             int ldc, int batches, size_t batch_stride, bool lower_only)
+namespace
+{
+hipError_t launch_tiles(hipStream_t stream, bool ta, bool tb, int m, int n, int k, double alpha,
+                        const double *a, int lda, const double *b, int ldb, double beta, double *c, int ldc,
+                        int batches, BatchStrides batch_stride, bool lower_only)
 {
     if (batches < 1 || batches > 65535)
         return hipErrorInvalidValue;
@@ -159,5 +164,52 @@ hipError_t launch_dgemm_mfma(hipStream_t stream, bool ta, bool tb, int m, int n,
             return status;
     }
     return hipSuccess;
+}
+
+// c = alpha * (sum of the planes, in plane order) + beta * c
+__global__ __launch_bounds__(256) void sum_planes_f64_kernel(int m, int n, int shares, double alpha, double beta,
+                                                             const double *planes, double *c, int ldc)
+{
+    const size_t count = size_t(m) * n, at = size_t(blockIdx.x) * 256 + threadIdx.x;
+    if (at >= count)
+        return;
+    double sum = planes[at];
+    for (int s = 1; s < shares; ++s)
+        sum += planes[s * count + at];
+    double *out = c + at % m + at / m * ldc;
+    const double value = alpha * sum;
+    *out = beta != 0.0 ? fma(beta, *out, value) : value;
+}
+} // namespace
+
+hipError_t launch_dgemm_mfma(hipStream_t stream, bool ta, bool tb, int m, int n, int k, double alpha,
+                             const double *a, int lda, const double *b, int ldb, double beta, double *c,
+                             int ldc, int batches, size_t batch_stride, bool lower_only)
+{
+    return launch_tiles(stream, ta, tb, m, n, k, alpha, a, lda, b, ldb, beta, c, ldc, batches,
+                        BatchStrides{batch_stride, batch_stride, batch_stride}, lower_only);
+}
+
+// The same product with K divided over `shares` workgroups per 128 x 128 tile (k % shares == 0):
+// for a handful of columns of C against a large A, where the tiles alone would occupy a fraction
+// of the compute units. planes: shares * m * n doubles.
+hipError_t launch_dgemm_mfma_divided(hipStream_t stream, bool ta, bool tb, int m, int n, int k, double alpha,
+                                     const double *a, int lda, const double *b, int ldb, double beta,
+                                     double *c, int ldc, int shares, double *planes)
+{
+    if (shares < 2 || shares > 65535 || k % shares || !planes)
+        return hipErrorInvalidValue;
+    const int part = k / shares;
+    const BatchStrides strides = {ta ? size_t(part) : size_t(part) * lda, tb ? size_t(part) * ldb : size_t(part),
+                                  size_t(m) * n};
+    const hipError_t status =
+        launch_tiles(stream, ta, tb, m, n, part, 1.0, a, lda, b, ldb, 0.0, planes, m, shares, strides, false);
+    if (status != hipSuccess)
+        return status;
+    const size_t count = size_t(m) * n;
+    if ((count + 255) / 256 > 0x7fffffffu)
+        return hipErrorInvalidValue;
+    sum_planes_f64_kernel<<<unsigned((count + 255) / 256), 256, 0, stream>>>(m, n, shares, alpha, beta, planes, c, ldc);
+    return launch_status();
 }
 } // namespace camblas_hip

@@ -230,6 +230,41 @@ def test_dgemm_matches_float64_product(device, kernel, ta, tb, shape):
     assert np.array_equal(got[:, m:], c0.reshape(n, ldc)[:, m:])
 
 
+@pytest.mark.parametrize("ta", "NT")
+@pytest.mark.parametrize("tb", "NT")
+@pytest.mark.parametrize("n", [1, 5, 33, 130])
+def test_dgemm_few_columns_against_a_large_matrix(device, ta, tb, n):
+    # five (ten at n = 130) row tiles of 128 x 128 against 256 compute units: the planner divides
+    # K = 1024 over four workgroups per tile and sums the FP64 planes in share order. Small integers
+    # make every order of summation exact; random values are held to the tolerance of the test above.
+    m, k = 520, 1024
+    lda, ldb, ldc = (m if ta == "N" else k) + 1, (k if tb == "N" else n) + 2, m + 3
+    rng = np.random.default_rng(n)
+    for exact in (True, False):
+        if exact:
+            a = rng.integers(-8, 9, lda * (k if ta == "N" else m)).astype(np.float64)
+            b = rng.integers(-8, 9, ldb * (n if tb == "N" else k)).astype(np.float64)
+            c0 = rng.integers(-8, 9, ldc * n).astype(np.float64)
+        else:
+            a = oracle.fill_uniform(41, (lda * (k if ta == "N" else m),)).astype(np.float64)
+            b = oracle.fill_uniform(42, (ldb * (n if tb == "N" else k),)).astype(np.float64)
+            c0 = oracle.fill_uniform(43, (ldc * n,)).astype(np.float64)
+        got = run_dgemm(device, ta, tb, m, n, k, 0.5, a, lda, b, ldb, -2.0, c0.copy(), ldc).reshape(n, ldc)
+        left = a.reshape(-1, lda)[:, : (m if ta == "N" else k)]
+        left = left.T if ta == "N" else left
+        right = b.reshape(-1, ldb)[:, : (k if tb == "N" else n)]
+        right = right.T if tb == "N" else right
+        want = 0.5 * (left @ right) - 2.0 * c0.reshape(n, ldc)[:, :m].T
+        if exact:
+            assert np.array_equal(got[:, :m].T, want)
+        else:
+            assert rel_frobenius(got[:, :m].T, want) <= 1e-13
+        assert np.array_equal(got[:, m:], c0.reshape(n, ldc)[:, m:]), "padding rows of C were written"
+    nan_c = np.full(ldc * n, np.nan)
+    got = run_dgemm(device, ta, tb, m, n, k, 1.0, a, lda, b, ldb, 0.0, nan_c, ldc).reshape(n, ldc)
+    assert rel_frobenius(got[:, :m].T, left @ right) <= 1e-13
+
+
 @pytest.mark.parametrize("kernel", ["vector", "matrix"])
 def test_dgemm_beta_zero_ignores_nan_and_keeps_full_precision(device, kernel):
     # beta = 0 must not read C; 1 + 2^-40 squared keeps its 2^-39 term only in full FP64 arithmetic
