@@ -144,7 +144,7 @@ int ordinary(const Entry &entry, const Product &p, float alpha, const float *a, 
         if (reserve_scratch(context, size_t(plan.split_k) * size_t(p.m) * size_t(p.n) * 4) == hipSuccess)
             return entry.finish(launch_sgemm_mfma_divided(context->stream, p.trans_a, p.trans_b, p.m, p.n, p.k, alpha, a,
                                                           p.lda, b, p.ldb, beta, c, p.ldc, plan.split_k,
-                                                          static_cast<float *>(context->scratch)),
+                                                          static_cast<float *>(context->scratch), plan.kernel == 2),
                                 "classical GEMM");
         context->counts[5]++;
     }
@@ -171,11 +171,14 @@ int ordinary(const Entry &entry, const Product &p, double alpha, const double *a
         matrix = context->override_kernel >= 1;
     // a handful of columns against a large A: the 128 x 128 tiles alone would occupy a fraction of
     // the compute units, so K is divided over workgroups (the FP32 rule with this kernel's tile)
+    // (up to 32 columns: tiles of 128 x 16, to 64: 128 x 64, and four workgroups per compute unit)
     int shares = 1;
+    const int tile_columns = p.n <= 32 ? 16 : p.n <= 64 ? 64 : 128;
+    const bool narrow = tile_columns < 128;
     if (matrix && context->override_kernel < 0 && p.m >= 256 && p.k >= 512) {
-        const long long tiles = (long long)((p.m + 127) / 128) * ((p.n + 127) / 128);
+        const long long tiles = (long long)((p.m + 127) / 128) * ((p.n + tile_columns - 1) / tile_columns);
         for (int s : {32, 16, 8, 4, 2})
-            if (tiles * s <= 2LL * context->compute_units && p.k % s == 0 && p.k / s >= 256) {
+            if (tiles * s <= (narrow ? 4LL : 2LL) * context->compute_units && p.k % s == 0 && p.k / s >= 256) {
                 shares = s;
                 break;
             }
@@ -185,7 +188,7 @@ int ordinary(const Entry &entry, const Product &p, double alpha, const double *a
         if (reserve_scratch(context, size_t(shares) * size_t(p.m) * size_t(p.n) * 8) == hipSuccess)
             return entry.finish(launch_dgemm_mfma_divided(context->stream, p.trans_a, p.trans_b, p.m, p.n, p.k, alpha,
                                                           a, p.lda, b, p.ldb, beta, c, p.ldc, shares,
-                                                          static_cast<double *>(context->scratch)),
+                                                          static_cast<double *>(context->scratch), tile_columns),
                                 "classical FP64 GEMM");
         context->counts[5]++;
     }

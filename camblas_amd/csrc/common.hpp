@@ -132,13 +132,13 @@ hipError_t launch_sgemm_mfma(hipStream_t stream, bool wide, bool ta, bool tb, in
 // shares * m * n floats, summed in share order): few columns of C against a large A.
 hipError_t launch_sgemm_mfma_divided(hipStream_t stream, bool ta, bool tb, int m, int n, int k, float alpha,
                                      const float *a, int lda, const float *b, int ldb, float beta, float *c,
-                                     int ldc, int shares, float *planes);
+                                     int ldc, int shares, float *planes, bool narrow);
 hipError_t launch_dgemm_mfma(hipStream_t stream, bool ta, bool tb, int m, int n, int k, double alpha,
                              const double *a, int lda, const double *b, int ldb, double beta, double *c,
                              int ldc, int batches = 1, size_t batch_stride = 0, bool lower_only = false);
 hipError_t launch_dgemm_mfma_divided(hipStream_t stream, bool ta, bool tb, int m, int n, int k, double alpha,
                                      const double *a, int lda, const double *b, int ldb, double beta,
-                                     double *c, int ldc, int shares, double *planes);
+                                     double *c, int ldc, int shares, double *planes, int tile_columns);
 // c[row, column] = c[column, row] for row < column of a column-major n x n matrix (dtype 0 FP32, 1 FP64)
 hipError_t launch_mirror_lower(hipStream_t stream, int dtype, int n, void *c, int ldc);
 // Strassen policies for square 'N','N' products (strassen.hip). strassen_levels: recursion depth of

@@ -33,15 +33,17 @@ template <bool CONTIGUOUS_K> __device__ __forceinline__ int lds_index(int r, int
     return CONTIGUOUS_K ? r * ROW_MAJOR_PITCH + l : l * K_MAJOR_PITCH + r;
 }
 
-template <bool TA, bool TB>
+// COLUMNS: 128, or 64 / 16 for a product with a handful of columns (the four wavefronts then stack
+// along the rows, 32 x COLUMNS each; at 16 B brings one element per thread and step)
+template <bool TA, bool TB, int COLUMNS>
 __global__ __launch_bounds__(THREADS, 2) void dgemm_mfma_kernel(int m, int n, int k, double alpha,
                                                              const double *a, int lda, const double *b,
                                                              int ldb, double beta, double *c, int ldc,
                                                              BatchStrides batch_strides, bool lower_only)
 {
     // a symmetric product: only the tiles that reach the diagonal, the rest is the mirroring pass
-    int row0 = blockIdx.x * TILE, col0 = blockIdx.y * TILE;
-    if (lower_only && !lower_tile<TILE, TILE>(blockIdx.x, n, row0, col0))
+    int row0 = blockIdx.x * TILE, col0 = blockIdx.y * COLUMNS;
+    if (COLUMNS == TILE && lower_only && !lower_tile<TILE, TILE>(blockIdx.x, n, row0, col0))
         return;
     a += blockIdx.z * batch_strides.a; // one independent product per grid z-slice
     b += blockIdx.z * batch_strides.b;
@@ -49,11 +51,13 @@ __global__ __launch_bounds__(THREADS, 2) void dgemm_mfma_kernel(int m, int n, in
     __shared__ double tile_a[TILE_WORDS];
     __shared__ double tile_b[TILE_WORDS];
     const int thread = threadIdx.x, lane = thread % 64, wave = thread / 64;
-    constexpr int PER_THREAD = TILE * DEPTH / THREADS;
+    constexpr int PER_THREAD = TILE * DEPTH / THREADS, PER_THREAD_B = COLUMNS * DEPTH / THREADS;
+    constexpr int WAVES_DOWN = COLUMNS == TILE ? 2 : 4;           // wavefronts along the rows
+    constexpr int X = TILE / WAVES_DOWN / 16, Y = COLUMNS / (4 / WAVES_DOWN) / 16;
     // A(i, l) is a[i + l*lda] ('N', rows contiguous) or a[l + i*lda] ('T', K contiguous);
     // B(l, j) is b[l + j*ldb] ('N', K contiguous) or b[j + l*ldb] ('T', columns contiguous).
     // Element e of a step goes to the thread so that consecutive threads read consecutive memory.
-    double next_a[PER_THREAD], next_b[PER_THREAD];
+    double next_a[PER_THREAD], next_b[PER_THREAD_B];
     auto fetch = [&](int l0) {
 #pragma unroll
         for (int s = 0; s < PER_THREAD; ++s) {
@@ -61,7 +65,11 @@ __global__ __launch_bounds__(THREADS, 2) void dgemm_mfma_kernel(int m, int n, in
             const int ai = TA ? e / DEPTH : e % TILE, al = TA ? e % DEPTH : e / TILE;
             const int gi = row0 + ai, gl = l0 + al;
             next_a[s] = gi < m && gl < k ? (TA ? a[gl + size_t(gi) * lda] : a[gi + size_t(gl) * lda]) : 0.0;
-            const int bj = TB ? e % TILE : e / DEPTH, bl = TB ? e / TILE : e % DEPTH;
+        }
+#pragma unroll
+        for (int s = 0; s < PER_THREAD_B; ++s) {
+            const int e = s * THREADS + thread;
+            const int bj = TB ? e % COLUMNS : e / DEPTH, bl = TB ? e / COLUMNS : e % DEPTH;
             const int gj = col0 + bj, hl = l0 + bl;
             next_b[s] = gj < n && hl < k ? (TB ? b[gj + size_t(hl) * ldb] : b[hl + size_t(gj) * ldb]) : 0.0;
         }
@@ -72,18 +80,22 @@ __global__ __launch_bounds__(THREADS, 2) void dgemm_mfma_kernel(int m, int n, in
             const int e = s * THREADS + thread;
             const int ai = TA ? e / DEPTH : e % TILE, al = TA ? e % DEPTH : e / TILE;
             tile_a[lds_index<TA>(ai, al)] = next_a[s];
-            const int bj = TB ? e % TILE : e / DEPTH, bl = TB ? e / TILE : e % DEPTH;
+        }
+#pragma unroll
+        for (int s = 0; s < PER_THREAD_B; ++s) {
+            const int e = s * THREADS + thread;
+            const int bj = TB ? e % COLUMNS : e / DEPTH, bl = TB ? e / COLUMNS : e % DEPTH;
             tile_b[lds_index<!TB>(bj, bl)] = next_b[s];
         }
     };
 
-    const int wave_i = (wave % 2) * 64, wave_j = (wave / 2) * 64;
+    const int wave_i = (wave % WAVES_DOWN) * (X * 16), wave_j = (wave / WAVES_DOWN) * (Y * 16);
     const int frag_row = lane % 16, frag_k = lane / 16;
-    f64x4_t acc[4][4];
+    f64x4_t acc[X][Y];
 #pragma unroll
-    for (int x = 0; x < 4; ++x)
+    for (int x = 0; x < X; ++x)
 #pragma unroll
-        for (int y = 0; y < 4; ++y)
+        for (int y = 0; y < Y; ++y)
             acc[x][y] = f64x4_t{0.0, 0.0, 0.0, 0.0};
 
     fetch(0);
@@ -94,17 +106,17 @@ __global__ __launch_bounds__(THREADS, 2) void dgemm_mfma_kernel(int m, int n, in
             fetch(l0 + DEPTH);
 #pragma unroll
         for (int s = 0; s < DEPTH / 4; ++s) {
-            double av[4], bv[4];
+            double av[X], bv[Y];
 #pragma unroll
-            for (int x = 0; x < 4; ++x)
+            for (int x = 0; x < X; ++x)
                 av[x] = tile_a[lds_index<TA>(wave_i + x * 16 + frag_row, 4 * s + frag_k)];
 #pragma unroll
-            for (int y = 0; y < 4; ++y)
+            for (int y = 0; y < Y; ++y)
                 bv[y] = tile_b[lds_index<!TB>(wave_j + y * 16 + frag_row, 4 * s + frag_k)];
 #pragma unroll
-            for (int x = 0; x < 4; ++x)
+            for (int x = 0; x < X; ++x)
 #pragma unroll
-                for (int y = 0; y < 4; ++y)
+                for (int y = 0; y < Y; ++y)
                     acc[x][y] = __builtin_amdgcn_mfma_f64_16x16x4f64(av[x], bv[y], acc[x][y], 0, 0, 0);
         }
         __syncthreads();
@@ -113,12 +125,12 @@ __global__ __launch_bounds__(THREADS, 2) void dgemm_mfma_kernel(int m, int n, in
     // accumulator element e of lane l: row 4*e + l/16, column l%16 of the 16 x 16 tile (found with
     // an identity product; the FP32 16 x 16 instructions use 4*(l/16) + e instead)
 #pragma unroll
-    for (int y = 0; y < 4; ++y) {
+    for (int y = 0; y < Y; ++y) {
         const int j = col0 + wave_j + y * 16 + frag_row;
         if (j >= n)
             continue;
 #pragma unroll
-        for (int x = 0; x < 4; ++x) {
+        for (int x = 0; x < X; ++x) {
 #pragma unroll
             for (int e = 0; e < 4; ++e) {
                 const int i = row0 + wave_i + x * 16 + 4 * e + frag_k;
@@ -135,6 +147,7 @@ __global__ __launch_bounds__(THREADS, 2) void dgemm_mfma_kernel(int m, int n, in
 
 namespace
 {
+template <int COLUMNS>
 hipError_t launch_tiles(hipStream_t stream, bool ta, bool tb, int m, int n, int k, double alpha,
                         const double *a, int lda, const double *b, int ldb, double beta, double *c, int ldc,
                         int batches, BatchStrides batch_stride, bool lower_only)
@@ -143,22 +156,22 @@ hipError_t launch_tiles(hipStream_t stream, bool ta, bool tb, int m, int n, int 
         return hipErrorInvalidValue;
     // column tiles travel in grid.y (at most 65535): wider products go panel by panel; the
     // lower-triangle grid is one-dimensional
-    constexpr int PANEL = 65535 * TILE;
+    constexpr int PANEL = 65535 * COLUMNS;
     for (int first = 0; first < n; first += lower_only ? n : PANEL) {
         const int columns = lower_only ? n : (n - first < PANEL ? n - first : PANEL);
         const double *bp = b + (tb ? size_t(first) : size_t(first) * ldb);
         double *cp = c + size_t(first) * ldc;
-        dim3 grid((m + TILE - 1) / TILE, (columns + TILE - 1) / TILE, batches);
+        dim3 grid((m + TILE - 1) / TILE, (columns + COLUMNS - 1) / COLUMNS, batches);
         if (lower_only)
             grid = dim3(lower_tile_count<TILE, TILE>(n), 1, batches);
         if (!ta && !tb)
-            dgemm_mfma_kernel<false, false><<<grid, THREADS, 0, stream>>>(m, columns, k, alpha, a, lda, bp, ldb, beta, cp, ldc, batch_stride, lower_only);
+            dgemm_mfma_kernel<false, false, COLUMNS><<<grid, THREADS, 0, stream>>>(m, columns, k, alpha, a, lda, bp, ldb, beta, cp, ldc, batch_stride, lower_only);
         else if (!ta && tb)
-            dgemm_mfma_kernel<false, true><<<grid, THREADS, 0, stream>>>(m, columns, k, alpha, a, lda, bp, ldb, beta, cp, ldc, batch_stride, lower_only);
+            dgemm_mfma_kernel<false, true, COLUMNS><<<grid, THREADS, 0, stream>>>(m, columns, k, alpha, a, lda, bp, ldb, beta, cp, ldc, batch_stride, lower_only);
         else if (ta && !tb)
-            dgemm_mfma_kernel<true, false><<<grid, THREADS, 0, stream>>>(m, columns, k, alpha, a, lda, bp, ldb, beta, cp, ldc, batch_stride, lower_only);
+            dgemm_mfma_kernel<true, false, COLUMNS><<<grid, THREADS, 0, stream>>>(m, columns, k, alpha, a, lda, bp, ldb, beta, cp, ldc, batch_stride, lower_only);
         else
-            dgemm_mfma_kernel<true, true><<<grid, THREADS, 0, stream>>>(m, columns, k, alpha, a, lda, bp, ldb, beta, cp, ldc, batch_stride, lower_only);
+            dgemm_mfma_kernel<true, true, COLUMNS><<<grid, THREADS, 0, stream>>>(m, columns, k, alpha, a, lda, bp, ldb, beta, cp, ldc, batch_stride, lower_only);
         const hipError_t status = launch_status();
         if (status != hipSuccess)
             return status;
@@ -186,24 +199,29 @@ hipError_t launch_dgemm_mfma(hipStream_t stream, bool ta, bool tb, int m, int n,
                              const double *a, int lda, const double *b, int ldb, double beta, double *c,
                              int ldc, int batches, size_t batch_stride, bool lower_only)
 {
-    return launch_tiles(stream, ta, tb, m, n, k, alpha, a, lda, b, ldb, beta, c, ldc, batches,
-                        BatchStrides{batch_stride, batch_stride, batch_stride}, lower_only);
+    return launch_tiles<TILE>(stream, ta, tb, m, n, k, alpha, a, lda, b, ldb, beta, c, ldc, batches,
+                              BatchStrides{batch_stride, batch_stride, batch_stride}, lower_only);
 }
 
-// The same product with K divided over `shares` workgroups per 128 x 128 tile (k % shares == 0):
-// for a handful of columns of C against a large A, where the tiles alone would occupy a fraction
-// of the compute units. planes: shares * m * n doubles.
+// The same product with K divided over `shares` workgroups per tile (k % shares == 0): for a
+// handful of columns of C against a large A, where the tiles alone would occupy a fraction of the
+// compute units. tile_columns: 128, 64 or 16 columns of C per tile. planes: shares * m * n doubles.
 hipError_t launch_dgemm_mfma_divided(hipStream_t stream, bool ta, bool tb, int m, int n, int k, double alpha,
                                      const double *a, int lda, const double *b, int ldb, double beta,
-                                     double *c, int ldc, int shares, double *planes)
+                                     double *c, int ldc, int shares, double *planes, int tile_columns)
 {
-    if (shares < 2 || shares > 65535 || k % shares || !planes)
+    if (shares < 2 || shares > 65535 || k % shares || !planes ||
+        (tile_columns != 16 && tile_columns != 64 && tile_columns != TILE))
         return hipErrorInvalidValue;
     const int part = k / shares;
     const BatchStrides strides = {ta ? size_t(part) : size_t(part) * lda, tb ? size_t(part) * ldb : size_t(part),
                                   size_t(m) * n};
     const hipError_t status =
-        launch_tiles(stream, ta, tb, m, n, part, 1.0, a, lda, b, ldb, 0.0, planes, m, shares, strides, false);
+        tile_columns == 16
+            ? launch_tiles<16>(stream, ta, tb, m, n, part, 1.0, a, lda, b, ldb, 0.0, planes, m, shares, strides, false)
+        : tile_columns == 64
+            ? launch_tiles<64>(stream, ta, tb, m, n, part, 1.0, a, lda, b, ldb, 0.0, planes, m, shares, strides, false)
+            : launch_tiles<TILE>(stream, ta, tb, m, n, part, 1.0, a, lda, b, ldb, 0.0, planes, m, shares, strides, false);
     if (status != hipSuccess)
         return status;
     const size_t count = size_t(m) * n;

@@ -150,12 +150,16 @@ Plan make_plan(int dtype, int algorithm, bool trans_a, bool trans_b, int m, int 
         // over workgroups, about two per compute unit, FP32 planes summed in share order
         // ([8192, 8192] x 16 tokens: 980 us on the vector-ALU kernel, 420 us at 32 tokens undivided).
         if (plan.family == FAMILY_MFMA_F32 && plan.kernel == 1 && algorithm != CAMBLAS_CUDA_CLASSICAL && k >= 512) {
-            const int tiles = ceil_div(m, 128) * ceil_div(n, 64);
+            // (up to 32 columns: tiles of 128 x 32, kernel 2, and four workgroups per compute unit:
+            // [8192, 8192] x 16 tokens 100 us on the 64-column tiles)
+            const bool narrow = n <= 32;
+            const int tiles = ceil_div(m, 128) * ceil_div(n, narrow ? 32 : 64);
             const int counts[] = {32, 16, 8, 4, 2};
             for (const int shares : counts)
-                if (tiles * shares <= 2 * compute_units && k % shares == 0 && k / shares >= 256 &&
+                if (tiles * shares <= (narrow ? 4 : 2) * compute_units && k % shares == 0 && k / shares >= 256 &&
                     double(shares) * m * n * 4 <= double(1 << 28)) {
                     plan.split_k = shares;
+                    plan.kernel = narrow ? 2 : 1;
                     break;
                 }
         }
@@ -533,7 +537,8 @@ void describe_plan(const Plan &plan, int dtype, char *text, size_t bytes)
         break;
     case FAMILY_MFMA_F32:
         if (plan.split_k > 1)
-            std::snprintf(text, bytes, "%s mfma 128x64x32 split_k=%d", type, plan.split_k);
+            std::snprintf(text, bytes, "%s mfma %s split_k=%d", type, plan.kernel == 2 ? "128x32x32" : "128x64x32",
+                          plan.split_k);
         else
             std::snprintf(text, bytes, "%s mfma %s", type, plan.kernel == 0 ? "128x128x32" : "128x64x32");
         break;

@@ -32,7 +32,8 @@ template <bool CONTIGUOUS_K> __device__ __forceinline__ int lds_word(int r, int 
 }
 
 // COLUMNS: 128 or 64 columns of C per workgroup (64: twice the workgroups, for products whose
-// 128 x 128 tiles would leave one workgroup per compute unit with nothing to overlap with)
+// 128 x 128 tiles would leave one workgroup per compute unit with nothing to overlap with), or 32
+// for a handful of columns with K divided (the four wavefronts then stack along the rows)
 template <bool TA, bool TB, int COLUMNS>
 __global__ __launch_bounds__(THREADS) void sgemm_mfma_kernel(int m, int n, int k, float alpha,
                                                              const float *a, int lda, const float *b,
@@ -50,7 +51,9 @@ __global__ __launch_bounds__(THREADS) void sgemm_mfma_kernel(int m, int n, int k
     __shared__ float tile_b[TILE_WORDS];
     const int thread = threadIdx.x, lane = thread % 64, wave = thread / 64;
     constexpr int A_PER_THREAD = TILE * DEPTH / THREADS, B_PER_THREAD = COLUMNS * DEPTH / THREADS;
-    constexpr int WJ = COLUMNS / 64; // 32-column MFMA tiles per wavefront
+    constexpr int WAVES_DOWN = COLUMNS >= 64 ? 2 : 4;             // wavefronts along the rows
+    constexpr int WI = TILE / WAVES_DOWN / 32;                    // 32-row MFMA tiles per wavefront
+    constexpr int WJ = COLUMNS / (4 / WAVES_DOWN) / 32;           // 32-column MFMA tiles per wavefront
     // A(i, l) is a[i + l*lda] ('N', rows contiguous) or a[l + i*lda] ('T', K contiguous);
     // B(l, j) is b[l + j*ldb] ('N', K contiguous) or b[j + l*ldb] ('T', columns contiguous).
     // Element e of a step goes to the thread so that consecutive threads read consecutive memory.
@@ -86,11 +89,11 @@ __global__ __launch_bounds__(THREADS) void sgemm_mfma_kernel(int m, int n, int k
         }
     };
 
-    const int wave_i = (wave % 2) * 64, wave_j = (wave / 2) * (32 * WJ);
+    const int wave_i = (wave % WAVES_DOWN) * (32 * WI), wave_j = (wave / WAVES_DOWN) * (32 * WJ);
     const int frag_row = lane % 32, frag_k = lane / 32;
-    f32x16_t acc[2][WJ];
+    f32x16_t acc[WI][WJ];
 #pragma unroll
-    for (int x = 0; x < 2; ++x)
+    for (int x = 0; x < WI; ++x)
 #pragma unroll
         for (int y = 0; y < WJ; ++y)
 #pragma unroll
@@ -105,15 +108,15 @@ __global__ __launch_bounds__(THREADS) void sgemm_mfma_kernel(int m, int n, int k
             fetch(l0 + DEPTH);
 #pragma unroll
         for (int s = 0; s < DEPTH / 2; ++s) {
-            float av[2], bv[WJ];
+            float av[WI], bv[WJ];
 #pragma unroll
-            for (int x = 0; x < 2; ++x)
+            for (int x = 0; x < WI; ++x)
                 av[x] = tile_a[lds_word<TA>(wave_i + x * 32 + frag_row, 2 * s + frag_k)];
 #pragma unroll
             for (int y = 0; y < WJ; ++y)
                 bv[y] = tile_b[lds_word<!TB>(wave_j + y * 32 + frag_row, 2 * s + frag_k)];
 #pragma unroll
-            for (int x = 0; x < 2; ++x)
+            for (int x = 0; x < WI; ++x)
 #pragma unroll
                 for (int y = 0; y < WJ; ++y)
                     acc[x][y] = __builtin_amdgcn_mfma_f32_32x32x2f32(av[x], bv[y], acc[x][y], 0, 0, 0);
@@ -130,7 +133,7 @@ __global__ __launch_bounds__(THREADS) void sgemm_mfma_kernel(int m, int n, int k
         if (j >= n)
             continue;
 #pragma unroll
-        for (int x = 0; x < 2; ++x) {
+        for (int x = 0; x < WI; ++x) {
 #pragma unroll
             for (int q = 0; q < 4; ++q) {
                 const int i = row0 + wave_i + x * 32 + 8 * q + 4 * frag_k;
@@ -226,12 +229,12 @@ __global__ __launch_bounds__(256) void sum_planes_f32_kernel(int m, int n, int s
 }
 } // namespace
 
-// The same product with K divided over `shares` workgroups per 128 x 64 tile (k % shares == 0): for
-// a handful of columns of C against a large A, where the tiles alone would occupy a fraction of the
-// compute units. planes: shares * m * n floats.
+// The same product with K divided over `shares` workgroups per 128 x 64 tile (narrow: 128 x 32;
+// k % shares == 0): for a handful of columns of C against a large A, where the tiles alone would
+// occupy a fraction of the compute units. planes: shares * m * n floats.
 hipError_t launch_sgemm_mfma_divided(hipStream_t stream, bool ta, bool tb, int m, int n, int k, float alpha,
                                      const float *a, int lda, const float *b, int ldb, float beta, float *c,
-                                     int ldc, int shares, float *planes)
+                                     int ldc, int shares, float *planes, bool narrow)
 {
     if (shares < 2 || shares > 65535 || k % shares || !planes)
         return hipErrorInvalidValue;
@@ -239,7 +242,8 @@ hipError_t launch_sgemm_mfma_divided(hipStream_t stream, bool ta, bool tb, int m
     const BatchStrides strides = {ta ? size_t(part) : size_t(part) * lda, tb ? size_t(part) * ldb : size_t(part),
                                   size_t(m) * n};
     const hipError_t status =
-        launch_columns<64>(stream, ta, tb, m, n, part, 1.f, a, lda, b, ldb, 0.f, planes, m, shares, strides, false);
+        narrow ? launch_columns<32>(stream, ta, tb, m, n, part, 1.f, a, lda, b, ldb, 0.f, planes, m, shares, strides, false)
+               : launch_columns<64>(stream, ta, tb, m, n, part, 1.f, a, lda, b, ldb, 0.f, planes, m, shares, strides, false);
     if (status != hipSuccess)
         return status;
     const size_t count = size_t(m) * n;

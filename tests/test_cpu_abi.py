@@ -96,15 +96,16 @@ def test_planner_choices_for_the_baseline_shapes():
     assert describe(0, "T", "N", 4096, 1, 4096, 4096, 4096, 4096)[0] // 1000 == 1
     # (otherwise a handful of columns against a large A: matrix-core tiles with K divided over workgroups;
     # a small A stays on the vector-ALU tiles)
-    assert describe(0, "T", "N", 4096, 1, 4096, 4096, 4096, 4096, algorithm="lt") == (8001, "f32 mfma 128x64x32 split_k=16")
-    assert describe(0, "T", "N", 1000, 1, 4096, 4096, 4096, 1000) == (8001, "f32 mfma 128x64x32 split_k=16")
-    assert describe(0, "T", "N", 8192, 16, 8192, 8192, 8192, 8192) == (8001, "f32 mfma 128x64x32 split_k=8")
+    assert describe(0, "T", "N", 4096, 1, 4096, 4096, 4096, 4096, algorithm="lt") == (8002, "f32 mfma 128x32x32 split_k=16")
+    assert describe(0, "T", "N", 1000, 1, 4096, 4096, 4096, 1000) == (8002, "f32 mfma 128x32x32 split_k=16")
+    assert describe(0, "T", "N", 8192, 16, 8192, 8192, 8192, 8192) == (8002, "f32 mfma 128x32x32 split_k=16")
     assert describe(0, "T", "N", 200, 1, 4096, 4096, 4096, 200)[0] // 1000 == 0
     assert describe(0, "T", "N", 4096, 4, 4096, 4096, 4096, 4096, algorithm="classical")[0] // 1000 == 0
     # FP32 products: matrix-core tiles, 128 x 64 until every compute unit gets two 128 x 128 tiles
     assert describe(0, "N", "N", 2048, 2048, 2048, 2048, 2048, 2048) == (8001, "f32 mfma 128x64x32")
     assert describe(0, "T", "N", 4096, 4096, 4096, 4096, 4096, 4096) == (8000, "f32 mfma 128x128x32")
-    assert describe(0, "N", "N", 2048, 16, 2048, 2048, 2048, 2048) == (8001, "f32 mfma 128x64x32 split_k=8")
+    assert describe(0, "N", "N", 2048, 16, 2048, 2048, 2048, 2048) == (8002, "f32 mfma 128x32x32 split_k=8")
+    assert describe(0, "N", "N", 2048, 48, 2048, 2048, 2048, 2048) == (8001, "f32 mfma 128x64x32 split_k=8")
     assert describe(0, "N", "N", 128, 16, 2048, 128, 2048, 128)[0] // 1000 == 0
     # FP8: split-K tiles for a few tokens, the streaming kernel for decode batches, direct-to-LDS
     # tiles for prefill

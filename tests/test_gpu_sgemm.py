@@ -73,7 +73,8 @@ def test_sgemm_few_columns_against_a_large_matrix(device, ta, tb, n):
     lda = (m if ta == "N" else k) + 3
     ldb = (k if tb == "N" else n) + 2
     ldc = m + 5
-    assert _native.plan_describe(0, ta, tb, m, n, k, lda, ldb, ldc)[1] == "f32 mfma 128x64x32 split_k=4" or (
+    tile = "128x32x32" if n <= 32 else "128x64x32"
+    assert _native.plan_describe(0, ta, tb, m, n, k, lda, ldb, ldc)[1] == f"f32 mfma {tile} split_k=4" or (
         n == 1 and ta == "T" and tb == "N")
     a = oracle.fill_uniform(11, (lda * (k if ta == "N" else m),))
     b = oracle.fill_uniform(12, (ldb * (n if tb == "N" else k),))
@@ -232,10 +233,11 @@ def test_dgemm_matches_float64_product(device, kernel, ta, tb, shape):
 
 @pytest.mark.parametrize("ta", "NT")
 @pytest.mark.parametrize("tb", "NT")
-@pytest.mark.parametrize("n", [1, 5, 33, 130])
+@pytest.mark.parametrize("n", [1, 5, 20, 33, 130])
 def test_dgemm_few_columns_against_a_large_matrix(device, ta, tb, n):
-    # five (ten at n = 130) row tiles of 128 x 128 against 256 compute units: the planner divides
-    # K = 1024 over four workgroups per tile and sums the FP64 planes in share order. Small integers
+    # five (ten at n = 130) row tiles of 128 x 128 against 256 compute units, or of 128 x 16 up to 32
+    # columns (n = 20: two column tiles, the second ragged): the planner divides K = 1024 over four
+    # workgroups per tile and sums the FP64 planes in share order. Small integers
     # make every order of summation exact; random values are held to the tolerance of the test above.
     m, k = 520, 1024
     lda, ldb, ldc = (m if ta == "N" else k) + 1, (k if tb == "N" else n) + 2, m + 3
