@@ -65,6 +65,16 @@ hipError_t reserve_scratch(camblas_cuda_context *context, size_t bytes)
     return hipSuccess;
 }
 
+void *claim_scratch(camblas_cuda_context *context, size_t bytes)
+{
+    const size_t offset = (context->held_bytes + 255) / 256 * 256;
+    if (context->held_bytes && offset + bytes > context->scratch_bytes)
+        return nullptr;
+    if (reserve_scratch(context, offset + bytes) != hipSuccess)
+        return nullptr;
+    return static_cast<char *>(context->scratch) + offset;
+}
+
 hipError_t reserve_arrivals(camblas_cuda_context *context)
 {
     if (context->arrivals)

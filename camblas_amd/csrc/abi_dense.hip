@@ -124,27 +124,80 @@ template <> struct Kernels<double> {
     }
 };
 
+// The planner's choice for an ordinary FP32 product, with any forced kernel applied.
+Plan fp32_plan(const camblas_cuda_context *context, const Product &p, const float *a, const float *b)
+{
+    Plan plan = make_plan(0, context->algorithm, p.trans_a, p.trans_b, p.m, p.n, p.k, p.lda, p.ldb, p.ldc,
+                          is_aligned(a, 16) && is_aligned(b, 16), context->compute_units);
+    if (plan.family != FAMILY_GEMV_F32 && context->override_kernel >= 0) {
+        // tests: 0 vector-ALU tiles, 1 / 2 matrix-core tiles
+        plan.family = context->override_kernel >= 1 ? FAMILY_MFMA_F32 : FAMILY_GENERIC;
+        plan.kernel = context->override_kernel == 2 ? 1 : 0;
+        plan.split_k = 1;
+    }
+    if (plan.family != FAMILY_MFMA_F32)
+        plan.split_k = 1;
+    return plan;
+}
+
+// Into how many workgroups per tile an ordinary FP64 product divides K, and the tile width: a
+// handful of columns against a large A would occupy a fraction of the compute units with the
+// 128 x 128 tiles alone (the FP32 rule with this kernel's tiles: up to 32 columns tiles of
+// 128 x 16, up to 64 of 128 x 64, and four workgroups per compute unit).
+struct Fp64Plan {
+    bool matrix;
+    int shares, tile_columns;
+};
+Fp64Plan fp64_plan(const camblas_cuda_context *context, const Product &p)
+{
+    // (fewer than 16 columns against a large A still go to the tiles: with K divided they run at
+    // five times the rate of the vector-ALU kernel, whose grid would be a few dozen workgroups)
+    Fp64Plan plan{p.m >= 16 && (p.n >= 16 || (p.m >= 256 && p.k >= 512)) && p.k >= 4, 1,
+                  p.n <= 32 ? 16 : p.n <= 64 ? 64 : 128};
+    if (context->override_kernel >= 0) // tests: 0 vector-ALU tiles, else matrix-core tiles
+        plan.matrix = context->override_kernel >= 1;
+    const bool narrow = plan.tile_columns < 128;
+    if (plan.matrix && context->override_kernel < 0 && p.m >= 256 && p.k >= 512) {
+        const long long tiles =
+            (long long)((p.m + 127) / 128) * ((p.n + plan.tile_columns - 1) / plan.tile_columns);
+        for (int s : {32, 16, 8, 4, 2})
+            if (tiles * s <= (narrow ? 4LL : 2LL) * context->compute_units && p.k % s == 0 && p.k / s >= 256) {
+                plan.shares = s;
+                break;
+            }
+    }
+    return plan;
+}
+
+// Bytes of FP32 / FP64 planes the ordinary product of this shape would claim (0: K undivided).
+size_t plane_bytes(const camblas_cuda_context *context, const Product &p, const float *a, const float *b)
+{
+    const int shares = fp32_plan(context, p, a, b).split_k;
+    return shares > 1 ? size_t(shares) * size_t(p.m) * size_t(p.n) * sizeof(float) : 0;
+}
+size_t plane_bytes(const camblas_cuda_context *context, const Product &p, const double *, const double *)
+{
+    const int shares = fp64_plan(context, p).shares;
+    return shares > 1 ? size_t(shares) * size_t(p.m) * size_t(p.n) * sizeof(double) : 0;
+}
+
 // the ordinary FP32 product: the planner's choice (decode GEMV, matrix-core tiles, vector-ALU tiles)
 int ordinary(const Entry &entry, const Product &p, float alpha, const float *a, const float *b, float beta,
              float *c, bool classical_counter)
 {
     camblas_cuda_context *context = entry.context();
-    Plan plan = make_plan(0, context->algorithm, p.trans_a, p.trans_b, p.m, p.n, p.k, p.lda, p.ldb, p.ldc,
-                          is_aligned(a, 16) && is_aligned(b, 16), context->compute_units);
+    const Plan plan = fp32_plan(context, p, a, b);
     context->counts[classical_counter ? 0 : plan.counter]++;
     if (plan.family == FAMILY_GEMV_F32)
         return entry.finish(launch_gemv_f32(context->stream, p.m, p.k, alpha, a, p.lda, b, beta, c),
                             "FP32 native GEMV");
-    if (context->override_kernel >= 0) { // tests: 0 vector-ALU tiles, 1 / 2 matrix-core tiles
-        plan.family = context->override_kernel >= 1 ? FAMILY_MFMA_F32 : FAMILY_GENERIC;
-        plan.kernel = context->override_kernel == 2 ? 1 : 0;
-    }
-    if (plan.family == FAMILY_MFMA_F32 && plan.split_k > 1 && context->override_kernel < 0) {
-        // without room for the planes (allocation failure, capture in progress) K stays undivided
-        if (reserve_scratch(context, size_t(plan.split_k) * size_t(p.m) * size_t(p.n) * 4) == hipSuccess)
+    if (plan.split_k > 1) {
+        // without room for the planes (allocation failure, capture in progress, an enclosing
+        // helper holding the arena) K stays undivided
+        if (void *planes = claim_scratch(context, size_t(plan.split_k) * size_t(p.m) * size_t(p.n) * 4))
             return entry.finish(launch_sgemm_mfma_divided(context->stream, p.trans_a, p.trans_b, p.m, p.n, p.k, alpha, a,
                                                           p.lda, b, p.ldb, beta, c, p.ldc, plan.split_k,
-                                                          static_cast<float *>(context->scratch), plan.kernel == 2),
+                                                          static_cast<float *>(planes), plan.kernel == 2),
                                 "classical GEMM");
         context->counts[5]++;
     }
@@ -164,38 +217,21 @@ int ordinary(const Entry &entry, const Product &p, double alpha, const double *a
 {
     camblas_cuda_context *context = entry.context();
     context->counts[0]++;
-    // (fewer than 16 columns against a large A still go to the tiles: with K divided they run at
-    // five times the rate of the vector-ALU kernel, whose grid would be a few dozen workgroups)
-    bool matrix = p.m >= 16 && (p.n >= 16 || (p.m >= 256 && p.k >= 512)) && p.k >= 4;
-    if (context->override_kernel >= 0) // tests: 0 vector-ALU tiles, else matrix-core tiles
-        matrix = context->override_kernel >= 1;
-    // a handful of columns against a large A: the 128 x 128 tiles alone would occupy a fraction of
-    // the compute units, so K is divided over workgroups (the FP32 rule with this kernel's tile)
-    // (up to 32 columns: tiles of 128 x 16, to 64: 128 x 64, and four workgroups per compute unit)
-    int shares = 1;
-    const int tile_columns = p.n <= 32 ? 16 : p.n <= 64 ? 64 : 128;
-    const bool narrow = tile_columns < 128;
-    if (matrix && context->override_kernel < 0 && p.m >= 256 && p.k >= 512) {
-        const long long tiles = (long long)((p.m + 127) / 128) * ((p.n + tile_columns - 1) / tile_columns);
-        for (int s : {32, 16, 8, 4, 2})
-            if (tiles * s <= (narrow ? 4LL : 2LL) * context->compute_units && p.k % s == 0 && p.k / s >= 256) {
-                shares = s;
-                break;
-            }
-    }
-    if (shares > 1) {
-        // without room for the planes (allocation failure, capture in progress) K stays undivided
-        if (reserve_scratch(context, size_t(shares) * size_t(p.m) * size_t(p.n) * 8) == hipSuccess)
+    const Fp64Plan plan = fp64_plan(context, p);
+    if (plan.shares > 1) {
+        // without room for the planes (allocation failure, capture in progress, an enclosing
+        // helper holding the arena) K stays undivided
+        if (void *planes = claim_scratch(context, size_t(plan.shares) * size_t(p.m) * size_t(p.n) * 8))
             return entry.finish(launch_dgemm_mfma_divided(context->stream, p.trans_a, p.trans_b, p.m, p.n, p.k, alpha,
-                                                          a, p.lda, b, p.ldb, beta, c, p.ldc, shares,
-                                                          static_cast<double *>(context->scratch), tile_columns),
+                                                          a, p.lda, b, p.ldb, beta, c, p.ldc, plan.shares,
+                                                          static_cast<double *>(planes), plan.tile_columns),
                                 "classical FP64 GEMM");
         context->counts[5]++;
     }
     const hipError_t launched =
-        matrix ? launch_dgemm_mfma(context->stream, p.trans_a, p.trans_b, p.m, p.n, p.k, alpha, a, p.lda, b,
-                                   p.ldb, beta, c, p.ldc)
-               : Kernels<double>::vector(context->stream, p, alpha, a, b, beta, c);
+        plan.matrix ? launch_dgemm_mfma(context->stream, p.trans_a, p.trans_b, p.m, p.n, p.k, alpha, a, p.lda, b,
+                                        p.ldb, beta, c, p.ldc)
+                    : Kernels<double>::vector(context->stream, p, alpha, a, b, beta, c);
     return entry.finish(launched, "classical FP64 GEMM");
 }
 
@@ -269,20 +305,31 @@ int score_attention(const Entry &entry, int queries, int keys, int depth, int va
         return entry.refuse("attention scratch size overflow", 2);
     camblas_cuda_context *context = entry.context();
     context->counts[6]++;
-    const hipError_t grown = reserve_scratch(context, size_t(queries) * keys * sizeof(T));
+    const int depth_ld = std::max(1, depth), keys_ld = std::max(1, keys), values_ld = std::max(1, values);
+    const Product score('T', 'N', keys, queries, depth, depth_ld, depth_ld, keys_ld);
+    const Product mix('N', 'N', values, queries, keys, values_ld, keys_ld, values_ld);
+    // One reservation for the scores and, behind them, the planes of whichever of the two
+    // products divides K: the scores stay live across both, so the arena must not move or be
+    // handed out again in between. (If the larger request cannot be met, the scores alone are
+    // reserved and the products run undivided.)
+    const size_t own = size_t(queries) * keys * sizeof(T);
+    const size_t behind = std::max(plane_bytes(context, score, k, q), plane_bytes(context, mix, v, static_cast<const T *>(nullptr)));
+    hipError_t grown = hipErrorOutOfMemory;
+    if (behind)
+        grown = reserve_scratch(context, (own + 255) / 256 * 256 + behind);
+    if (grown != hipSuccess)
+        grown = reserve_scratch(context, own);
     if (grown != hipSuccess)
         return entry.refuse("attention scratch", int(grown));
     T *scores = static_cast<T *>(context->scratch);
-    const int depth_ld = std::max(1, depth), keys_ld = std::max(1, keys), values_ld = std::max(1, values);
+    const ScratchHold hold(context, std::max<size_t>(own, 1));
     // scores[queries, keys] = q k^T; with no keys the second product just writes zeros
-    const Product score('T', 'N', keys, queries, depth, depth_ld, depth_ld, keys_ld);
     if (const int status = dense_product(entry, score, T(1), k, q, T(0), scores))
         return status;
     const hipError_t softened =
         launch_softmax_rows(context->stream, Kernels<T>::dtype, scores, queries, keys, double(scale));
     if (softened != hipSuccess)
         return entry.refuse("attention softmax", int(softened));
-    const Product mix('N', 'N', values, queries, keys, values_ld, keys_ld, values_ld);
     return dense_product(entry, mix, T(1), v, scores, T(0), output);
 }
 
@@ -318,13 +365,35 @@ template <typename T> struct BackwardPass {
         context->counts[7]++;
         const int parts = chunks(), part_rows = std::max(1, int((int64_t(rows) + parts - 1) / parts));
         T *partial = nullptr;
+        size_t own = 0;
         if (parts > 1 && ((db2 && outputs > 0) || (db1 && hidden > 0))) {
-            const hipError_t grown =
-                reserve_scratch(context, size_t(parts) * std::max(hidden, outputs) * sizeof(T));
+            // the column-sum partials stay live across the products below: one reservation for
+            // them and, behind them, the largest set of planes any of those products divides K into
+            own = size_t(parts) * std::max(hidden, outputs) * sizeof(T);
+            size_t behind = 0;
+            auto planes = [&](char ta, char tb, int m, int n, int k, const T *a, int lda, const T *b, int ldb, int ldc) {
+                if (m > 0 && n > 0 && k > 0)
+                    behind = std::max(behind, plane_bytes(context, Product(ta, tb, m, n, k, std::max(1, lda), std::max(1, ldb), std::max(1, ldc)), a, b));
+            };
+            if (dw2)
+                planes('N', 'T', outputs, hidden, rows, grad, outputs, h, hidden, outputs);
+            if (first_layer) {
+                planes('T', 'N', hidden, rows, outputs, w2, outputs, grad, outputs, hidden);
+                if (dw1)
+                    planes('N', 'T', hidden, inputs, rows, dh, hidden, x, inputs, hidden);
+                if (dx)
+                    planes('T', 'N', inputs, rows, hidden, w1, hidden, dh, hidden, inputs);
+            }
+            hipError_t grown = hipErrorOutOfMemory;
+            if (behind)
+                grown = reserve_scratch(context, (own + 255) / 256 * 256 + behind);
+            if (grown != hipSuccess)
+                grown = reserve_scratch(context, own);
             if (grown != hipSuccess)
                 return entry.refuse("backward scratch", int(grown));
             partial = static_cast<T *>(context->scratch);
         }
+        const ScratchHold hold(context, own);
         // second layer: dw2[hidden, outputs] = h^T grad, db2 = column sums of grad
         if (dw2)
             if (const int status = product('N', 'T', outputs, hidden, rows, grad, outputs, h, hidden, dw2, outputs))

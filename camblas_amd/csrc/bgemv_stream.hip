@@ -231,8 +231,14 @@ __global__ __launch_bounds__(WAVES * 64) void bgemv_stream_kernel(StreamParams p
         // The planes are written and read with device-scope accesses, which go to the point where
         // all XCDs agree instead of staying in one XCD's L2, so no cache has to be written back or
         // invalidated (a device-scope fence per workgroup was measured at +20 us on a 70 us
-        // launch). The barrier waits until this workgroup's stores have been acknowledged there;
-        // only then is the arrival counted.
+        // launch). Order, written out: every wavefront waits until its own plane stores have been
+        // acknowledged at device scope (vmcnt counts a store until its acknowledgement returns),
+        // then the barrier collects all four wavefronts, and only then does thread 0 count the
+        // arrival; a barrier alone promises nothing about global stores still in flight. On the
+        // reading side the last arriver's plane loads are issued after the atomic has returned
+        // its value (the branch on it below depends on the returned value) and are device-scope
+        // too, so they cannot be served from a stale XCD-local line.
+        wait_loads<0>();
         __syncthreads(); // (also: every wavefront is done with `combine`)
         unsigned *flag = reinterpret_cast<unsigned *>(lds_bytes);
         if (thread == 0) {

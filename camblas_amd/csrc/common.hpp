@@ -19,6 +19,7 @@ struct camblas_cuda_context {
     int compute_units = 256;
     void *scratch = nullptr;       // split-K partials, attention partials
     size_t scratch_bytes = 0;
+    size_t held_bytes = 0;         // leading bytes of the arena an enclosing helper keeps live across nested products
     std::vector<void *> retired;   // superseded scratch kept alive for captured graphs
     size_t retired_bytes = 0;      // what those arenas hold together
     bool seen_capture = false;     // the arena has been used by a launch under stream capture
@@ -39,6 +40,19 @@ int fail(camblas_cuda_context *context, const char *operation, int code);
 // Ensures the context scratch holds at least `bytes`; refuses to grow while the stream is
 // capturing (ref: src/cuda/backend.cu:399-426). Returns hipSuccess or the failing status.
 hipError_t reserve_scratch(camblas_cuda_context *context, size_t bytes);
+// Room for `bytes` of temporaries of one product: from the arena's start, or, while an enclosing
+// helper holds the leading held_bytes of it (attention scores, column-sum partials), behind them
+// and only if the arena already has the room: growing would free what the helper holds. Null
+// when there is no room (the caller then runs the form that needs none).
+void *claim_scratch(camblas_cuda_context *context, size_t bytes);
+// Marks the leading `bytes` of the arena as held until the end of the scope.
+struct ScratchHold {
+    camblas_cuda_context *context;
+    ScratchHold(camblas_cuda_context *c, size_t bytes) : context(c) { c->held_bytes = bytes; }
+    ~ScratchHold() { context->held_bytes = 0; }
+    ScratchHold(const ScratchHold &) = delete;
+    ScratchHold &operator=(const ScratchHold &) = delete;
+};
 // The context's arrival counters (STREAM_ARRIVAL_SLOTS of them, zero between launches), made and
 // cleared on first use; never under stream capture.
 hipError_t reserve_arrivals(camblas_cuda_context *context);

@@ -160,8 +160,9 @@ int strassen_gemm(camblas_cuda_context *context, int levels, int n, T alpha, con
         const uintptr_t base = reinterpret_cast<uintptr_t>(context->scratch);
         return address >= base && address - base < context->scratch_bytes;
     };
+    // (an enclosing helper holds part of the arena: the workspace would move or overwrite it)
     if (levels < 1 || capture != hipStreamCaptureStatusNone || !std::isfinite(double(alpha)) ||
-        in_scratch(a) || in_scratch(b) || in_scratch(c))
+        context->held_bytes || in_scratch(a) || in_scratch(b) || in_scratch(c))
         return STRASSEN_NOT_ELIGIBLE;
 
     // scratch for L levels; an allocation failure drops a level (counted once as a guard fallback).

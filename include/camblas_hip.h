@@ -346,7 +346,11 @@ int camblas_hip_plan_describe(int dtype, int algorithm, char trans_a, char trans
  * this context (kernel < 0 restores the planner; split_k <= 0 lets the planner choose). For the
  * E8M0 products: 0 the weight-streaming kernel, 20 / 21 / 22 / 23 the tiled kernel with
  * 256 x 256, 256 x 128, (E4M3 weights only) 192 x 256 and 128 x 128 tiles; a forced kernel that
- * cannot run the call makes the call fail. */
+ * cannot run the call makes the call fail.
+ * TEST-ONLY: the override is state of the context it is set on (no other context sees it, and it
+ * ends with the context), it bypasses the planner's eligibility rules, and a forced variant may be
+ * far slower than the planner's choice or refuse shapes the planner would serve. Serving code never
+ * calls it; nothing in the library or its Python surface sets it outside the test suite. */
 int camblas_hip_set_plan_override(camblas_cuda_context *context, int kernel, int split_k);
 /* extension. Number of kernel variants `camblas_hip_set_plan_override` accepts for a dtype. */
 int camblas_hip_kernel_count(int dtype);

@@ -170,6 +170,59 @@ def test_mlp_backward_row_chunks_repeat_bitwise(device, dtype, rows):
     assert only[:3] == (None, None, None) and torch.equal(only[3], first[3]) and torch.equal(only[4], first[4])
 
 
+def _relative(actual, expected):
+    expected = expected.double().cpu()
+    return float((actual.double().cpu() - expected).norm() / expected.norm().clamp_min(1e-300))
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("queries,keys,depth,values",
+                         [(64, 2048, 64, 64), (64, 8192, 64, 1024), (64, 2048, 512, 64)])
+def test_attention_whose_products_divide_k_keeps_the_scores_intact(device, dtype, queries, keys, depth, values):
+    # The planner divides K of these products over workgroups (planes in the context's arena) while
+    # the score matrix lives in the same arena: first call on a context of its own (a new stream
+    # gets one, so the arena starts empty and must be sized for both at once), then warmed.
+    torch.manual_seed(queries + keys + depth + values)
+    q = torch.randn((queries, depth), dtype=dtype) * 0.3
+    k = torch.randn((keys, depth), dtype=dtype) * 0.3
+    v = torch.randn((keys, values), dtype=dtype)
+    expected = torch.softmax((q.double() @ k.double().T) * 0.25, dim=-1) @ v.double()
+    stream = torch.cuda.Stream(device)
+    with torch.cuda.stream(stream):
+        qd, kd, vd = q.to(device), k.to(device), v.to(device)
+        results = [_kernels.attention(qd, kd, vd, scale=0.25) for _ in range(3)]
+        stream.synchronize()
+    bar = 1e-5 if dtype == torch.float32 else 1e-13
+    for result in results:
+        assert _relative(result, expected) <= bar
+        assert torch.equal(result, results[0])
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_mlp_backward_whose_products_divide_k_keeps_the_partials_intact(device, dtype):
+    # rows=1024, hidden=256, outputs=64: dw2 = h^T grad divides K over workgroups while the bias
+    # gradients' row-chunk partials are held in the same arena
+    torch.manual_seed(1024)
+    rows, inputs, hidden_width, outputs = 1024, 96, 256, 64
+    stream = torch.cuda.Stream(device)
+    with torch.cuda.stream(stream):
+        x = torch.randn((rows, inputs), dtype=dtype, device=device)
+        w1 = torch.randn((inputs, hidden_width), dtype=dtype, device=device) * 0.1
+        w2 = torch.randn((hidden_width, outputs), dtype=dtype, device=device) * 0.1
+        hidden = torch.relu(torch.randn((rows, hidden_width), dtype=dtype, device=device))
+        gradient = torch.randn((rows, outputs), dtype=dtype, device=device)
+        runs = [_kernels.mlp_backward(x, w1, w2, hidden, gradient) for _ in range(3)]
+        stream.synchronize()
+    g, h = gradient.double().cpu(), hidden.double().cpu()
+    dh = (g @ w2.double().cpu().T) * (h > 0)
+    expected = (dh @ w1.double().cpu().T, x.double().cpu().T @ dh, dh.sum(0), h.T @ g, g.sum(0))
+    bar = 1e-5 if dtype == torch.float32 else 1e-13
+    for run in runs:
+        for got, first, want in zip(run, runs[0], expected):
+            assert torch.equal(got, first)
+            assert _relative(got, want) <= bar
+
+
 def test_c_abi_validation_counters_and_empty_shapes(device):
     native = _native.context(device)
     library = _native.library()

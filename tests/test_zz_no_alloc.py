@@ -67,3 +67,68 @@ def test_sizes_beyond_the_fixed_array_are_refused(device):
                     None, ct.c_float(1.0), ptr(q), q.stride(0), ptr(cache), ptr(cache[8:]), ptr(out))
     torch.cuda.synchronize()
     assert not out.any()
+
+
+CHILD = r"""
+import ctypes as ct
+import torch
+from camblas_amd import _native
+
+injector = ct.CDLL(None)
+injector.camblas_test_fail_next_allocation.restype = None
+injector.camblas_test_allocation_pending.restype = ct.c_int
+device = torch.device("cuda:0")
+lib = _native.library()
+P = lambda t: ct.c_void_p(t.data_ptr())
+Q, KV, D, batch, length = 16, 4, 128, 5, 1300
+torch.manual_seed(9300)
+q = torch.randn((batch, Q, D), device=device).to(torch.bfloat16)
+k = torch.randn((batch, length, KV, D), device=device).to(torch.bfloat16)
+v = torch.randn((batch, length, KV, D), device=device).to(torch.bfloat16)
+lengths = torch.tensor([1300, 1, 700, 257, 1299], dtype=torch.int32, device=device)
+resident = torch.full((batch, Q, D), float("nan"), dtype=torch.bfloat16, device=device)
+allocating = torch.full_like(resident, float("nan"))
+torch.cuda.synchronize()
+native = _native.context(device)                      # a context that has never grown its scratch
+def arguments(out):
+    return (native.handle, batch, Q, KV, D, length, P(lengths), ct.c_float(D ** -0.5), P(q), q.stride(0),
+            P(k), P(v), P(out))
+injector.camblas_test_fail_next_allocation()           # any hipMalloc from here on would fail
+assert lib.camblas_cuda_gqa_decode_attention_noalloc(*arguments(resident)) == 0
+assert injector.camblas_test_allocation_pending() == 1, "the allocation-free entry point allocated"
+# the allocating entry point on the same fresh context does ask for memory: it takes the armed failure
+assert lib.camblas_cuda_gqa_decode_attention(*arguments(allocating)) == -2
+assert injector.camblas_test_allocation_pending() == 0
+assert lib.camblas_cuda_gqa_decode_attention(*arguments(allocating)) == 0
+torch.cuda.synchronize()
+assert torch.equal(resident.view(torch.int16), allocating.view(torch.int16))
+assert not torch.isnan(resident.float()).any()
+_native.close()
+print("no allocation ok")
+"""
+
+
+def test_the_entry_point_allocates_nothing_on_a_fresh_context(tmp_path):
+    # A child process with the hipMalloc interposer of the allocation-failure tests preloaded: the
+    # call must succeed with a failure armed and leave it armed.
+    import os
+    import shutil
+    import subprocess
+    import sys
+    from pathlib import Path
+
+    root = Path(__file__).resolve().parents[1]
+    shim = root / "tests/support/fail_next_hipmalloc.so"
+    if not shim.is_file():
+        compiler = shutil.which("cc") or shutil.which("gcc")
+        if not compiler:
+            pytest.skip("no C compiler for the interposer")
+        shim = tmp_path / "fail_next_hipmalloc.so"
+        subprocess.run([compiler, "-shared", "-fPIC", str(root / "tests/support/fail_next_hipmalloc.c"), "-ldl",
+                        "-o", str(shim)], check=True, capture_output=True, text=True)
+    environment = dict(os.environ)
+    existing = environment.get("LD_PRELOAD", "")
+    environment["LD_PRELOAD"] = str(shim) + (":" + existing if existing else "")
+    result = subprocess.run([sys.executable, "-c", CHILD], cwd=root, env=environment, capture_output=True,
+                            text=True, timeout=240)
+    assert result.returncode == 0 and "no allocation ok" in result.stdout, result.stdout + result.stderr
