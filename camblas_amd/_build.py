@@ -32,6 +32,7 @@ CORE_SOURCES = (
     "bgemm_tn.hip",
     "bgemv_stream.hip",
     "bgemm_dma.hip",
+    "bgemm_wave4.hip",
     "bgemm_nn.hip",
     "fp8_block.hip",
     "fp8_dma.hip",

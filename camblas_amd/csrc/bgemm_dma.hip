@@ -19,26 +19,12 @@
 #include "common.hpp"
 #include "device.hpp"
 #include "dma.hpp"
+#include "bgemm_dma.hpp"
 
 namespace camblas_hip
 {
 namespace
 {
-struct DmaParams {
-    const unsigned short *w;
-    const unsigned short *x;
-    unsigned short *y;
-    const unsigned short *z; // what beta multiplies: z[token * ldz + feature] (y and ldc by default)
-    int lda, ldb, ldc, ldz;
-    int n, m, k;
-    float alpha, beta;
-    int tiles_n, tiles_m;
-    // K divided over gridDim.y workgroups per tile: each takes `share_steps` steps of BK and leaves
-    // its FP32 sums in plane blockIdx.y of `partials` ([share][token][feature])
-    float *partials;
-    int share_steps;
-};
-
 // TN, TM: 32x32 MFMA tiles per wavefront along features / tokens; the workgroup has 2 x WM
 // wavefronts and owns a (64*TN) x (32*WM*TM) tile; BK: K elements per step (32 or 64); STAGES: LDS
 // stages (STAGES - 1 steps are in flight).
@@ -606,8 +592,17 @@ const TnVariant variants[] = {
     {"dma16-320x256x64s2w8", 320, 256, 64, 512}, {"dma16-256x256x64s2w8", 256, 256, 64, 512},
     {"dma16-192x256x64s2w8", 192, 256, 64, 512}, {"dma16-128x256x64s3w8", 128, 256, 64, 512},
     {"dma16-256x128x64s3w8", 256, 128, 64, 512}, {"dma16-128x128x64s3w4", 128, 128, 64, 256},
+    // four wavefronts, one per SIMD, K loop in assembly (bgemm_wave4.hip); K % 128 == 0
+    {"wave4-256x256x64s2", 256, 256, 64, 256}, {"wave4-320x256x64s2", 320, 256, 64, 256},
 };
 } // namespace
+
+hipError_t launch_sum_shares(hipStream_t stream, const DmaParams &p, int shares)
+{
+    const size_t quads = size_t(p.m) * size_t(p.n / 4);
+    sum_shares_kernel<<<unsigned((quads + 255) / 256), 256, 0, stream>>>(p, shares);
+    return launch_status();
+}
 
 hipError_t launch_sum_shares(hipStream_t stream, const float *partials, int shares, int n_out, int m_rows,
                              float alpha, float beta, const void *z, int ldz, void *y, int ldc)
@@ -683,6 +678,8 @@ hipError_t launch_bgemm_dma(hipStream_t stream, int variant, int n_out, int m_ro
     case 15: return launch_dma16<2, 2, 4, 64, 3>(stream, p, shares);
     case 16: return launch_dma16<4, 1, 4, 64, 3>(stream, p, shares);
     case 17: return launch_dma16<2, 2, 2, 64, 3>(stream, p, shares);
+    case 18: return launch_bgemm_wave4(stream, 256, p, shares);
+    case 19: return launch_bgemm_wave4(stream, 320, p, shares);
     default: return hipErrorInvalidValue;
     }
 }

@@ -1,0 +1,266 @@
+#!/usr/bin/env python3
+"""Writes wave4_loop_<rows>x256.inc: the K loop of bgemm_wave4.hip as one inline-assembly statement.
+
+Why the loop is generated assembly and not HIP source: a workgroup of four wavefronts, one per SIMD,
+each owning a (16*NA) x 128 block of the output tile, keeps 4*NA*8 FP32 accumulators per lane. They
+fill the accumulation half of the register file (a0..a255; what does not fit goes to named
+architectural registers), and the operand fragments, double-buffered per 32-deep sub-step, take the
+low architectural registers. The compiler's allocator spreads such a kernel over both halves and
+spills; with every register named here it has nothing to decide inside the loop.
+
+One K step (64 elements) of a wavefront:
+  phase 1  NA*8 matrix instructions on fragment buffer 1 (second sub-step of the previous K step)
+           | direct-to-LDS fills of the K step after this one | LDS reads of this step's first
+           sub-step into buffer 0
+  phase 2  NA*8 matrix instructions on buffer 0 | LDS reads of the second sub-step into buffer 1
+  wait for the fills and the reads, barrier
+so the matrix pipe always has a full sub-step of independent instructions while the next operands
+travel, and the only point where the four wavefronts meet is one barrier per K step.
+
+The fragment file uses local variables of the including function by name: accs[] (f32x4_t outputs, tile (i, j) at 8 i + j),
+a_offset / b_offset (per-lane byte offsets of the fills, advanced by the loop), read_a0 / read_a1 /
+read_b0 / read_b1 (LDS byte addresses of the first weight / token fragment for sub-step 0 / 1 in
+stage 0), a_resource / b_resource (u32x4_t buffer descriptors), a_row_step / b_row_step (bytes
+between successive fill rows), fill_base (this wavefront's first LDS fill address in stage 0) and
+step_pairs ((K steps - 2) / 2).
+
+Usage: python gen_wave4_loop.py [--out DIR] [--drop fills,barrier,fillwait,reads]
+Without arguments it rewrites the .inc files beside this script. --drop leaves mechanisms out of the
+loop for timing-only builds that attribute the kernel's time (their results are wrong by design;
+such files are written somewhere else with --out and never shipped).
+"""
+
+import argparse
+from pathlib import Path
+
+DROP = set()
+
+NB = 8  # token tiles of 16 per wavefront: 128 tokens, two wavefronts across = 256
+
+
+class Layout:
+    def __init__(self, na):
+        self.na = na
+        self.rows = 32 * na  # weight rows of the workgroup tile (two wavefronts down)
+        self.stage_bytes = (self.rows + 256) * 128
+        self.frag = 4 * (na + NB)  # registers of one fragment buffer
+        self.buffers = (0, self.frag)
+        # accumulators beyond a0..a255 live in architectural registers behind the fragment buffers
+        self.extra_acc_base = 2 * self.frag
+        self.extra_acc = max(0, 4 * na * NB - 256)
+        self.scratch_v = self.extra_acc_base + self.extra_acc  # four stage-1 read addresses
+        self.clobbered_v = self.scratch_v + 4
+
+    def a_frag(self, buffer, i):
+        return self.buffers[buffer] + 4 * i
+
+    def b_frag(self, buffer, j):
+        return self.buffers[buffer] + 4 * (self.na + j)
+
+    def acc(self, i, j):
+        index = 4 * (i * NB + j)
+        if index < 256:
+            return f"a[{index}:{index + 3}]"
+        index = self.extra_acc_base + index - 256
+        return f"v[{index}:{index + 3}]"
+
+
+SAVED_M0, OFFSET, FILL1 = "s84", "s85", "s86"
+
+
+def fill_units(layout, target):
+    """Per direct-to-LDS load: (scalar set-up placed before a matrix instruction, the load after it).
+    M0 walks this wavefront's LDS slots in 4 KB strides through the weight rows and on into the
+    token rows; the row advance of successive loads is the scalar offset."""
+    units = []
+    for n in range(layout.na + NB):
+        weights = n < layout.na
+        first = n == 0 or n == layout.na
+        second = n == 1 or n == layout.na + 1
+        lane, resource, step = (("%[a_off]", "%[rsrc_a]", "%[a_step]") if weights
+                                else ("%[b_off]", "%[rsrc_b]", "%[b_step]"))
+        before = [f"s_mov_b32 m0, {target}" if n == 0 else "s_add_u32 m0, m0, 0x1000"]
+        if second:
+            before.append(f"s_mov_b32 {OFFSET}, {step}")
+        elif not first:
+            before.append(f"s_add_u32 {OFFSET}, {OFFSET}, {step}")
+        load = f"buffer_load_dwordx4 {lane}, {resource}, {'0' if first else OFFSET} offen lds"
+        if "fills" in DROP:
+            load = "s_nop 0"
+        # timing experiments: the same bytes fetched into registers instead of LDS, and / or written
+        # to LDS from registers
+        stage = layout.clobbered_v + 4 * n
+        offset = n * 4096
+        to_register = f"buffer_load_dwordx4 v[{stage}:{stage + 3}], {lane}, {resource}, {'0' if first else OFFSET} offen"
+        write = f"ds_write_b128 %[ra0], v[{stage}:{stage + 3}] offset:{offset}"
+        if "tovgpr" in DROP:
+            load = to_register
+        if "dswrite" in DROP:
+            load = write
+        if "staged" in DROP:
+            load = write + "\n" + to_register
+        units.append((before, load))
+    return units
+
+
+ADVANCE = ["v_add_u32_e32 %[a_off], 0x80, %[a_off]", "v_add_u32_e32 %[b_off], 0x80, %[b_off]"]
+
+
+def reads(layout, stage, sub_step, buffer):
+    """LDS reads of one sub-step's fragments: weight fragments first, token fragments after (the
+    token fragments of the buffer being overwritten are the last the previous phase still uses)."""
+    if stage == 0:
+        a_address, b_address = f"%[ra{sub_step}]", f"%[rb{sub_step}]"
+    else:
+        a_address = f"v{layout.scratch_v + sub_step}"
+        b_address = f"v{layout.scratch_v + 2 + sub_step}"
+    lines = []
+    for i in range(layout.na):
+        r = layout.a_frag(buffer, i)
+        lines.append(f"ds_read_b128 v[{r}:{r + 3}], {a_address} offset:{i * 2048}")
+    for j in range(NB):
+        r = layout.b_frag(buffer, j)
+        lines.append(f"ds_read_b128 v[{r}:{r + 3}], {b_address} offset:{j * 2048}")
+    if "reads" in DROP:
+        return []
+    return lines
+
+
+FILL_EVERY = 4  # a fill after every FILL_EVERY-th matrix instruction
+ORDER = "weights"  # consecutive matrix instructions share their weight fragment ("tokens", "snake": experiments)
+
+
+def tile_order(layout):
+    if ORDER == "tokens":
+        return [(i, j) for j in range(NB) for i in range(layout.na)]
+    if ORDER == "snake":
+        return [(i, j if i % 2 == 0 else NB - 1 - j) for i in range(layout.na) for j in range(NB)]
+    return [(i, j) for i in range(layout.na) for j in range(NB)]
+
+
+def phase(layout, buffer, read_lines, fills, zero=False, advance=False):
+    """NA*8 matrix instructions on one fragment buffer with the fills and LDS reads between them:
+    a fill after every FILL_EVERY-th instruction, a read after every odd one, until both run out."""
+    lines = []
+    count = layout.na * NB
+    fills = fills or []
+    assert len(fills) <= (count + FILL_EVERY - 1) // FILL_EVERY and len(read_lines) <= count // 2
+    for k, (i, j) in enumerate(tile_order(layout)):
+        unit = fills[k // FILL_EVERY] if k % FILL_EVERY == 0 and k // FILL_EVERY < len(fills) else None
+        if unit:
+            lines += unit[0]
+        a, b = layout.a_frag(buffer, i), layout.b_frag(buffer, j)
+        source = "0" if zero else layout.acc(i, j)
+        lines.append(f"v_mfma_f32_16x16x32_bf16 {layout.acc(i, j)}, v[{a}:{a + 3}], v[{b}:{b + 3}], {source}")
+        if unit:
+            lines.append(unit[1])
+            if advance and unit is fills[-1]:
+                lines += ADVANCE
+        if k % 2 == 1 and k // 2 < len(read_lines):
+            lines.append(read_lines[k // 2])
+    return lines
+
+
+def k_step(layout, stage, fill_target):
+    fills = fill_units(layout, fill_target) if fill_target else []
+    first = min(len(fills), (layout.na * NB + FILL_EVERY - 1) // FILL_EVERY)
+    lines = [f"; K step in stage {stage}" + (f", fills into {fill_target}" if fill_target else ", no fills")]
+    lines += phase(layout, 1, reads(layout, stage, 0, 0), fills[:first], advance=first == len(fills))
+    lines.append("s_waitcnt lgkmcnt(0)")
+    lines += phase(layout, 0, reads(layout, stage, 1, 1), fills[first:], advance=first < len(fills))
+    lines += ["s_waitcnt lgkmcnt(0)" if "fillwait" in DROP else "s_waitcnt vmcnt(0) lgkmcnt(0)"]
+    if "barrier" not in DROP:
+        lines.append("s_barrier")
+    return lines
+
+
+def program(layout):
+    v = layout.scratch_v
+    lines = [
+        f"s_mov_b32 {SAVED_M0}, m0",
+        f"s_add_u32 {FILL1}, %[fill0], {layout.stage_bytes:#x}",
+        f"v_add_u32_e32 v{v}, {layout.stage_bytes:#x}, %[ra0]",
+        f"v_add_u32_e32 v{v + 1}, {layout.stage_bytes:#x}, %[ra1]",
+        f"v_add_u32_e32 v{v + 2}, {layout.stage_bytes:#x}, %[rb0]",
+        f"v_add_u32_e32 v{v + 3}, {layout.stage_bytes:#x}, %[rb1]",
+        "; K step 0 into stage 0",
+    ]
+    for before, load in fill_units(layout, "%[fill0]"):
+        lines += before + ["s_nop 0", load]
+    lines += ADVANCE + ["s_waitcnt vmcnt(0)", "s_barrier", "; K step 1 into stage 1, first fragments of step 0"]
+    for before, load in fill_units(layout, FILL1):
+        lines += before + ["s_nop 0", load]
+    lines += ADVANCE + reads(layout, 0, 0, 0) + ["s_waitcnt lgkmcnt(0)"]
+    lines += phase(layout, 0, reads(layout, 0, 1, 1), None, zero=True)
+    lines += ["s_waitcnt vmcnt(0) lgkmcnt(0)", "s_barrier",
+              "s_cmp_eq_u32 %[pairs], 0", "s_cbranch_scc1 L_wave4_last%=", "L_wave4_loop%=:"]
+    lines += k_step(layout, 1, "%[fill0]")
+    lines += k_step(layout, 0, FILL1)
+    lines += ["s_sub_u32 %[pairs], %[pairs], 1", "s_cmp_lg_u32 %[pairs], 0", "s_cbranch_scc1 L_wave4_loop%=",
+              "L_wave4_last%=:"]
+    lines += k_step(layout, 1, None)
+    lines += ["; second sub-step of the last K step"]
+    lines += phase(layout, 1, [], None)
+    # the code after this statement reads accumulators: cover the longest matrix-instruction latency
+    lines += [f"s_mov_b32 m0, {SAVED_M0}", "s_nop 15", "s_nop 15"]
+    return lines
+
+
+def statement(layout):
+    text = ["// Generated by gen_wave4_loop.py; edit the generator, not this file.", "asm volatile("]
+    for line in "\n".join(program(layout)).split("\n"):
+        text.append(f'    "{line}\\n"')
+    # one four-wide output per accumulator tile (wider tuples of named accumulation registers trip the
+    # compiler when single elements are taken from them)
+    outputs = []
+    for t in range(layout.na * NB):
+        register = layout.acc(*divmod(t, NB))
+        # (accumulators in architectural registers are marked early-clobber: without it the compiler
+        # may hand the same registers to inputs, which the loop still reads after it has written them)
+        early = "&" if register.startswith("v") else ""
+        outputs.append(f'"={early}{{{register}}}"(accs[{t}])')
+    outputs += ['[a_off] "+v"(a_offset)', '[b_off] "+v"(b_offset)', '[pairs] "+s"(step_pairs)']
+    inputs = ['[ra0] "v"(read_a0)', '[ra1] "v"(read_a1)', '[rb0] "v"(read_b0)', '[rb1] "v"(read_b1)',
+              '[rsrc_a] "s"(a_resource)', '[rsrc_b] "s"(b_resource)', '[a_step] "s"(a_row_step)',
+              '[b_step] "s"(b_row_step)', '[fill0] "s"(fill_base)']
+    clobbers = ['"memory"', '"scc"', f'"{SAVED_M0}"', f'"{OFFSET}"', f'"{FILL1}"']
+    named = [n for n in range(layout.clobbered_v)
+             if not layout.extra_acc_base <= n < layout.extra_acc_base + layout.extra_acc]
+    clobbers += [f'"v{n}"' for n in named]
+    if DROP & {"tovgpr", "dswrite", "staged"}:
+        clobbers += [f'"v{n}"' for n in range(layout.clobbered_v, layout.clobbered_v + 4 * (layout.na + NB))]
+
+    def wrapped(items):
+        rows, row = [], "   "
+        for item in items:
+            if len(row) + len(item) > 108:
+                rows.append(row)
+                row = "   "
+            row += " " + item + ","
+        rows.append(row.rstrip(","))
+        return rows
+
+    text += ["    :"] + wrapped(outputs) + ["    :"] + wrapped(inputs) + ["    :"] + wrapped(clobbers) + [");", ""]
+    return "\n".join(text)
+
+
+def main():
+    parser = argparse.ArgumentParser(description=__doc__.split("\n")[0])
+    parser.add_argument("--out", type=Path, default=Path(__file__).resolve().parent)
+    parser.add_argument("--drop", default="")
+    parser.add_argument("--fill-every", type=int, default=FILL_EVERY)
+    parser.add_argument("--order", default=ORDER)
+    arguments = parser.parse_args()
+    DROP.update(item for item in arguments.drop.split(",") if item)
+    globals()["FILL_EVERY"] = arguments.fill_every
+    globals()["ORDER"] = arguments.order
+    experiments = DROP & {"tovgpr", "dswrite", "staged"}
+    for na in (8, 10):
+        if na == 10 and experiments:  # the register experiments need more registers than the 320-row tile leaves
+            DROP.difference_update(experiments)
+        layout = Layout(na)
+        (arguments.out / f"wave4_loop_{layout.rows}x256.inc").write_text(statement(layout))
+
+
+if __name__ == "__main__":
+    main()

@@ -313,10 +313,16 @@ Plan make_plan(int dtype, int algorithm, bool trans_a, bool trans_b, int m, int 
             double best = -1;
             if (direct) {
                 // direct-to-LDS tiles: {variant, resident workgroups per CU, relative efficiency}
-                const struct {
+                // (with K a multiple of 128 the two largest tiles run on four wavefronts with the K loop
+                // in assembly, 15-20 % and 5 % faster tile for tile, so the smaller tiles weigh less)
+                struct Candidate {
                     int variant, resident;
                     double weight;
-                } candidates[] = {{10, 1, 1.0}, {6, 1, 0.96}, {11, 1, 0.88}, {9, 1, 0.85}, {5, 1, 0.83}};
+                };
+                const bool four_wavefronts = k % 128 == 0 && k <= 16384;
+                const Candidate eight[] = {{10, 1, 1.0}, {6, 1, 0.96}, {11, 1, 0.88}, {9, 1, 0.85}, {5, 1, 0.83}};
+                const Candidate four[] = {{10, 1, 1.0}, {6, 1, 0.88}, {11, 1, 0.75}, {9, 1, 0.72}, {5, 1, 0.70}};
+                const Candidate(&candidates)[5] = four_wavefronts ? four : eight;
                 plan.family = FAMILY_DMA;
                 for (const auto &candidate : candidates) {
                     const TnVariant &v = dma_variant(candidate.variant);
@@ -381,10 +387,14 @@ Plan make_plan(int dtype, int algorithm, bool trans_a, bool trans_b, int m, int 
             // every tile above exists on the 16 x 16 x 32 matrix instruction as well, which the part
             // runs at a higher clock on real data: 3 to 11 % faster tile for tile (measured:
             // 4096 x 10240 x 8192 534 -> 481 us, 8192^3 on 256 x 256 tiles 862 -> 807)
-            const auto narrow = [](int variant) {
+            // (the 320 x 256 and 256 x 256 tiles: on four wavefronts, one per SIMD, when K allows)
+            // (measured round-robin on one box: 4096 x 10240 x 8192 478 -> 457 us, 8192^3 806 -> 757,
+            // 2048 x 8192 x 8192 204 -> 194; at K = 28672 the eight-wavefront tiles stay 3 % ahead)
+            const bool four_wavefronts = k % 128 == 0 && k <= 16384 && plan.split_k == 1;
+            const auto narrow = [four_wavefronts](int variant) {
                 switch (variant) {
-                case 10: return 12;
-                case 6: return 13;
+                case 10: return four_wavefronts ? 19 : 12;
+                case 6: return four_wavefronts ? 18 : 13;
                 case 11: return 14;
                 case 9: return 15;
                 case 8: return 16;

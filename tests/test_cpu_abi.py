@@ -67,18 +67,21 @@ def test_planner_choices_for_the_baseline_shapes():
     # a single token on a short K keeps the undivided 32-row tiles
     assert "rows=64 tokens=32 k_step=128 k_shares=2" in describe(2, "T", "N", 8192, 32, 28672, 28672, 28672, 8192)[1]
     assert "rows=32 tokens=16 k_step=256 k_shares=1" in describe(2, "T", "N", 8192, 1, 8192, 8192, 8192, 8192)[1]
-    # prefill: direct-to-LDS MFMA tile that divides 10240 x 4096 into exactly two waves of tiles
-    code, text = describe(2, "T", "N", 10240, 4096, 8192, 8192, 8192, 10240)
-    assert code // 1000 == 5 and "dma16-320x256" in text
-    # 2.8 rounds of 320 x 256 tiles: two whole rounds, and the last 4096 outputs as one round of 256 x 256
-    assert describe(2, "T", "N", 14336, 4096, 4096, 4096, 4096, 14336) == (
-        5012, "bf16 dma16-320x256x64s2w8, last 4096 outputs dma16-256x256x64s2w8")
+    # prefill: the 320 x 256 tile divides 10240 x 4096 into exactly two rounds of workgroups; with K a
+    # multiple of 128 it runs on four wavefronts with the K loop in assembly, else on eight
+    assert describe(2, "T", "N", 10240, 4096, 8192, 8192, 8192, 10240) == (5019, "bf16 wave4-320x256x64s2")
+    assert describe(2, "T", "N", 10240, 4096, 8256, 8256, 8256, 10240) == (5012, "bf16 dma16-320x256x64s2w8")
+    # 5.6 rounds of 320 x 256 tiles: five whole rounds, and the last 3072 outputs as one round of 192 x 256
+    assert describe(2, "T", "N", 28672, 4096, 8192, 8192, 8192, 28672) == (
+        5019, "bf16 wave4-320x256x64s2, last 3072 outputs dma16-192x256x64s2w8")
+    # a K beyond 16384 keeps the eight-wavefront tiles
+    assert describe(2, "T", "N", 8192, 4096, 28672, 28672, 28672, 8192) == (5013, "bf16 dma16-256x256x64s2w8")
     # 65..1536 tokens: tile, shares of K and a second launch by estimated time (one round of
     # workgroups where the tiles alone would leave compute units idle)
     assert describe(2, "T", "N", 8192, 256, 8192, 8192, 8192, 8192) == (5015, "bf16 dma16-128x256x64s3w8 split_k=4")
     assert describe(2, "T", "N", 10240, 128, 8192, 8192, 8192, 10240) == (5017, "bf16 dma16-128x128x64s3w4 split_k=3")
     assert describe(2, "T", "N", 28672, 1024, 8192, 8192, 8192, 28672) == (
-        5012, "bf16 dma16-320x256x64s2w8, last 8192 outputs dma16-128x256x64s3w8")
+        5019, "bf16 wave4-320x256x64s2, last 8192 outputs dma16-128x256x64s3w8")
     assert describe(2, "T", "N", 8192, 256, 8200, 8200, 8200, 8192) == (2002, "bf16 mfma128x128x64 split_k=4")
     # K not a multiple of 64: register-staged MFMA tiles; unaligned operands and the other transpose
     # pairs: the layout-agnostic matrix-core kernel; slivers and the classical policy: vector-ALU tiles
@@ -249,3 +252,16 @@ def test_plugin_entry_points_are_registered():
     assert ("sglang.srt.plugins", "camblas", "camblas_amd.sglang:install") in found
     text = (ROOT / "pyproject.toml").read_text()
     assert 'camblas = "camblas_amd:_autoload"' in text and 'camblas = "camblas_amd.sglang:install"' in text
+
+
+def test_generated_assembly_loops_are_in_step_with_their_generator(tmp_path):
+    # the K loops of the four-wavefront prefill tiles are committed as generated text: regenerate
+    # them and compare, so that an edit to one side alone is caught
+    import subprocess
+    import sys
+    from pathlib import Path
+
+    sources = Path(__file__).resolve().parents[1] / "camblas_amd" / "csrc"
+    subprocess.run([sys.executable, str(sources / "gen_wave4_loop.py"), "--out", str(tmp_path)], check=True)
+    for name in ("wave4_loop_256x256.inc", "wave4_loop_320x256.inc"):
+        assert (tmp_path / name).read_text() == (sources / name).read_text(), name

@@ -119,6 +119,63 @@ def test_direct_lds_load_kernel(device, code, n_out, m_rows, k):
         assert np.array_equal(got2d[:, n_out:], c0.reshape(m_rows, ldc)[:, n_out:])
 
 
+@pytest.mark.parametrize("code", [38, 39])
+@pytest.mark.parametrize("n_out,m_rows,k", [(300, 70, 384), (512, 256, 128), (260, 513, 512), (644, 300, 256)])
+def test_four_wavefront_tiles(device, code, n_out, m_rows, k):
+    # the four-wavefront 256 x 256 and 320 x 256 tiles with the K loop in assembly: an even number of
+    # 64-deep K steps (two steps: the loop body never runs; more: it does), ragged N and M over one
+    # and several tiles, padded operand rows
+    lda, ldb, ldc = k + 8, k + 16, n_out + 4
+    w = oracle.fill_normal_bf16(420 + code, (n_out * lda,))
+    x = oracle.fill_normal_bf16(440 + code, (m_rows * ldb,))
+    c0 = oracle.fill_normal_bf16(460, (m_rows * ldc,))
+    for alpha, beta in ((1.0, 0.0), (0.5, -1.5)):
+        got = run_bgemm(device, "T", "N", n_out, m_rows, k, alpha, w, lda, x, ldb, beta, c0, ldc,
+                        override=(code, 1))
+        want, want64 = reference("T", "N", n_out, m_rows, k, alpha, w, lda, x, ldb, beta, c0, ldc)
+        got2d = got.reshape(m_rows, ldc)
+        error = rel_frobenius(oracle.bf16_to_f32(got2d[:, :n_out]), want64.reshape(m_rows, n_out))
+        assert error <= TOLERANCE, (code, alpha, beta, error)
+        assert np.array_equal(got2d[:, n_out:], c0.reshape(m_rows, ldc)[:, n_out:])
+
+
+@pytest.mark.parametrize("code", [38, 39])
+def test_four_wavefront_tiles_place_every_output(device, code):
+    # x = one-hot rows select single weight columns: y[m, n] = W[n, hot(m)] exactly, so a fragment,
+    # accumulator or tile put in the wrong place shows as a wrong value at a known position
+    n_out, m_rows, k = 700, 520, 256
+    rng = np.random.default_rng(code)
+    w = oracle.f32_to_bf16(rng.integers(-64, 64, size=(n_out, k)).astype(np.float32))
+    hot = rng.integers(0, k, size=m_rows)
+    x32 = np.zeros((m_rows, k), np.float32)
+    x32[np.arange(m_rows), hot] = 1.0
+    x = oracle.f32_to_bf16(x32)
+    c0 = np.zeros((m_rows * n_out,), np.uint16)
+    got = run_bgemm(device, "T", "N", n_out, m_rows, k, 1.0, w.reshape(-1), k, x.reshape(-1), k, 0.0, c0, n_out,
+                    override=(code, 1))
+    want = oracle.bf16_to_f32(w)[:, hot].T
+    assert np.array_equal(oracle.bf16_to_f32(got.reshape(m_rows, n_out)), want)
+
+
+@pytest.mark.parametrize("code", [38, 39])
+@pytest.mark.parametrize("shares", [2, 3])
+def test_four_wavefront_tiles_with_k_divided_over_workgroups(device, code, shares):
+    # ten steps of 64 over 2 (6 + 4) and 3 (4 + 4 + 2) workgroups per tile: shares hold an even number of steps
+    n_out, m_rows, k = 260, 513, 640
+    lda, ldb, ldc = k + 8, k + 16, n_out + 4
+    w = oracle.fill_normal_bf16(520 + code, (n_out * lda,))
+    x = oracle.fill_normal_bf16(540 + code, (m_rows * ldb,))
+    c0 = oracle.fill_normal_bf16(560, (m_rows * ldc,))
+    for alpha, beta in ((1.0, 0.0), (0.5, -1.5)):
+        got = run_bgemm(device, "T", "N", n_out, m_rows, k, alpha, w, lda, x, ldb, beta, c0, ldc,
+                        override=(code, shares))
+        want, want64 = reference("T", "N", n_out, m_rows, k, alpha, w, lda, x, ldb, beta, c0, ldc)
+        got2d = got.reshape(m_rows, ldc)
+        error = rel_frobenius(oracle.bf16_to_f32(got2d[:, :n_out]), want64.reshape(m_rows, n_out))
+        assert error <= TOLERANCE, (code, alpha, beta, error)
+        assert np.array_equal(got2d[:, n_out:], c0.reshape(m_rows, ldc)[:, n_out:])
+
+
 @pytest.mark.parametrize("code", [22, 25, 29, 30, 32, 35, 37])
 @pytest.mark.parametrize("shares", [2, 3, 7])
 def test_direct_lds_load_kernel_with_k_divided_over_workgroups(device, code, shares):
