@@ -138,36 +138,75 @@ def tile_order(layout):
     return [(i, j) for i in range(layout.na) for j in range(NB)]
 
 
-def phase(layout, buffer, read_lines, fills, zero=False, advance=False):
+READS = "early"  # "late": an experiment, see k_step
+
+
+class LdsQueue:
+    """Counts this wavefront's LDS reads in issue order (they return in that order), so that a wait
+    for one of them can leave the later ones outstanding: s_waitcnt lgkmcnt(n) with n = reads
+    issued after it (the counter holds four bits)."""
+
+    def __init__(self):
+        self.issued = 0
+        self.sequence = {}
+
+    def issue(self, line):
+        self.sequence[line.split(",")[0]] = self.issued  # keyed by destination registers
+        self.issued += 1
+        return line
+
+    def wait_for(self, destination):
+        return f"s_waitcnt lgkmcnt({min(15, self.issued - self.sequence[destination] - 1)})"
+
+
+def phase(layout, buffer, read_lines, fills, zero=False, advance=False, read_every=2, queue=None, waits=False):
     """NA*8 matrix instructions on one fragment buffer with the fills and LDS reads between them:
-    a fill after every FILL_EVERY-th instruction, a read after every odd one, until both run out."""
+    a fill after every FILL_EVERY-th instruction, a read after every read_every-th one, until both
+    run out. waits: this buffer's fragments may still be on their way; wait for each weight
+    fragment before its first use (the token fragments were requested before all of them)."""
     lines = []
     count = layout.na * NB
     fills = fills or []
-    assert len(fills) <= (count + FILL_EVERY - 1) // FILL_EVERY and len(read_lines) <= count // 2
+    assert len(fills) <= (count + FILL_EVERY - 1) // FILL_EVERY and len(read_lines) * read_every <= count
     for k, (i, j) in enumerate(tile_order(layout)):
         unit = fills[k // FILL_EVERY] if k % FILL_EVERY == 0 and k // FILL_EVERY < len(fills) else None
         if unit:
             lines += unit[0]
         a, b = layout.a_frag(buffer, i), layout.b_frag(buffer, j)
+        if waits and j == 0:
+            lines.append(queue.wait_for(f"ds_read_b128 v[{a}:{a + 3}]"))
         source = "0" if zero else layout.acc(i, j)
         lines.append(f"v_mfma_f32_16x16x32_bf16 {layout.acc(i, j)}, v[{a}:{a + 3}], v[{b}:{b + 3}], {source}")
         if unit:
             lines.append(unit[1])
             if advance and unit is fills[-1]:
                 lines += ADVANCE
-        if k % 2 == 1 and k // 2 < len(read_lines):
-            lines.append(read_lines[k // 2])
+        if k % read_every == read_every - 1 and k // read_every < len(read_lines):
+            line = read_lines[k // read_every]
+            lines.append(queue.issue(line) if queue else line)
     return lines
 
 
 def k_step(layout, stage, fill_target):
     fills = fill_units(layout, fill_target) if fill_target else []
-    first = min(len(fills), (layout.na * NB + FILL_EVERY - 1) // FILL_EVERY)
+    count = layout.na * NB
+    first = min(len(fills), (count + FILL_EVERY - 1) // FILL_EVERY)
     lines = [f"; K step in stage {stage}" + (f", fills into {fill_target}" if fill_target else ", no fills")]
-    lines += phase(layout, 1, reads(layout, stage, 0, 0), fills[:first], advance=first == len(fills))
-    lines.append("s_waitcnt lgkmcnt(0)")
-    lines += phase(layout, 0, reads(layout, stage, 1, 1), fills[first:], advance=first < len(fills))
+    first_reads, second_reads = reads(layout, stage, 0, 0), reads(layout, stage, 1, 1)
+    if READS == "late" and first_reads:
+        # the first sub-step's fragments are requested over the whole of phase 1, token fragments
+        # first, and phase 2 waits for each weight fragment where it first needs it; phase 2's own
+        # requests are spread over its first three quarters (they must be back before the barrier)
+        queue = LdsQueue()
+        first_reads = first_reads[layout.na:] + first_reads[:layout.na]
+        lines += phase(layout, 1, first_reads, fills[:first], advance=first == len(fills),
+                       read_every=count // len(first_reads), queue=queue)
+        lines += phase(layout, 0, second_reads, fills[first:], advance=first < len(fills),
+                       read_every=max(2, (3 * count // 4) // len(second_reads)), queue=queue, waits=True)
+    else:
+        lines += phase(layout, 1, first_reads, fills[:first], advance=first == len(fills))
+        lines.append("s_waitcnt lgkmcnt(0)")
+        lines += phase(layout, 0, second_reads, fills[first:], advance=first < len(fills))
     lines += ["s_waitcnt lgkmcnt(0)" if "fillwait" in DROP else "s_waitcnt vmcnt(0) lgkmcnt(0)"]
     if "barrier" not in DROP:
         lines.append("s_barrier")
@@ -250,10 +289,12 @@ def main():
     parser.add_argument("--drop", default="")
     parser.add_argument("--fill-every", type=int, default=FILL_EVERY)
     parser.add_argument("--order", default=ORDER)
+    parser.add_argument("--reads", default=READS)
     arguments = parser.parse_args()
     DROP.update(item for item in arguments.drop.split(",") if item)
     globals()["FILL_EVERY"] = arguments.fill_every
     globals()["ORDER"] = arguments.order
+    globals()["READS"] = arguments.reads
     experiments = DROP & {"tovgpr", "dswrite", "staged"}
     for na in (8, 10):
         if na == 10 and experiments:  # the register experiments need more registers than the 320-row tile leaves

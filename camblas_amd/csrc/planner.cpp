@@ -314,14 +314,15 @@ Plan make_plan(int dtype, int algorithm, bool trans_a, bool trans_b, int m, int 
             if (direct) {
                 // direct-to-LDS tiles: {variant, resident workgroups per CU, relative efficiency}
                 // (with K a multiple of 128 the two largest tiles run on four wavefronts with the K loop
-                // in assembly, 15-20 % and 5 % faster tile for tile, so the smaller tiles weigh less)
+                // in assembly, 5 % faster tile for tile, so the smaller tiles weigh a little less; per
+                // round of workgroups at 8192 tokens: 320 x 256 230 us, 256 x 256 189 us)
                 struct Candidate {
                     int variant, resident;
                     double weight;
                 };
                 const bool four_wavefronts = k % 128 == 0 && k <= 16384;
                 const Candidate eight[] = {{10, 1, 1.0}, {6, 1, 0.96}, {11, 1, 0.88}, {9, 1, 0.85}, {5, 1, 0.83}};
-                const Candidate four[] = {{10, 1, 1.0}, {6, 1, 0.88}, {11, 1, 0.75}, {9, 1, 0.72}, {5, 1, 0.70}};
+                const Candidate four[] = {{10, 1, 1.0}, {6, 1, 0.96}, {11, 1, 0.84}, {9, 1, 0.81}, {5, 1, 0.79}};
                 const Candidate(&candidates)[5] = four_wavefronts ? four : eight;
                 plan.family = FAMILY_DMA;
                 for (const auto &candidate : candidates) {

@@ -71,9 +71,11 @@ def test_planner_choices_for_the_baseline_shapes():
     # multiple of 128 it runs on four wavefronts with the K loop in assembly, else on eight
     assert describe(2, "T", "N", 10240, 4096, 8192, 8192, 8192, 10240) == (5019, "bf16 wave4-320x256x64s2")
     assert describe(2, "T", "N", 10240, 4096, 8256, 8256, 8256, 10240) == (5012, "bf16 dma16-320x256x64s2w8")
-    # 5.6 rounds of 320 x 256 tiles: five whole rounds, and the last 3072 outputs as one round of 192 x 256
-    assert describe(2, "T", "N", 28672, 4096, 8192, 8192, 8192, 28672) == (
-        5019, "bf16 wave4-320x256x64s2, last 3072 outputs dma16-192x256x64s2w8")
+    # 2.8 rounds of 320 x 256 tiles: two whole rounds, and the last 4096 outputs as one round of 256 x 256
+    assert describe(2, "T", "N", 14336, 4096, 4096, 4096, 4096, 14336) == (
+        5019, "bf16 wave4-320x256x64s2, last 4096 outputs wave4-256x256x64s2")
+    # 28672 x 4096 outputs are exactly seven rounds of 256 x 256 tiles
+    assert describe(2, "T", "N", 28672, 4096, 8192, 8192, 8192, 28672) == (5018, "bf16 wave4-256x256x64s2")
     # a K beyond 16384 keeps the eight-wavefront tiles
     assert describe(2, "T", "N", 8192, 4096, 28672, 28672, 28672, 8192) == (5013, "bf16 dma16-256x256x64s2w8")
     # 65..1536 tokens: tile, shares of K and a second launch by estimated time (one round of
