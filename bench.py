@@ -8,8 +8,10 @@ camblas_cuda_bgemm('T','N') on resident operands. Three weight copies (3 x 470 M
 algorithmic HBM traffic of the timed steps divided by wall time (host clock around K steps with a
 device synchronisation on both sides).
 
-When the K timed steps last less than 200 ms the same loop is timed once more over enough steps to
-fill 200 ms and both figures are reported (`config.long_run`).
+When the K timed steps last less than 200 ms (a wall clock around a few milliseconds measures mostly
+the loop's start and the final synchronisation) the same loop is timed once more over enough steps
+to fill 200 ms, and `value`, `steps` and `ms_per_step` are those of the longer region; the K-step
+region is kept as `config.short_run`, K as `config.requested_steps`.
 
 The line also carries
   roofline      the dominant kernel (M=32 launch) timed with HIP events on the launch stream; its
@@ -18,7 +20,9 @@ The line also carries
   cpu_baseline  PyTorch's own CPU BF16 F.linear on the same shape, all host threads of this process,
   also          the other configurations (BF16 prefill linear and addmm, FP8 block-scaled linear,
                 E8M0 products, FP32 SGEMM, decode attention, decoder-layer decode step), each with
-                a `roofline` object of its own; PyTorch's CPU FP8 dequantise-then-mm; the CPU
+                a `roofline` object of its own (the matrix-bound ones also with the rate the
+                matrix instruction they run on sustains on varied operand bits, measured in the same
+                run, and the fraction of it they reach); PyTorch's CPU FP8 dequantise-then-mm; the CPU
                 oracle port; the reference's own CPU SGEMM when oracle/_ref is present.
 """
 
@@ -47,13 +51,61 @@ PEAKS = {"hbm": (HBM_PEAK, 1e9, "GB/s"), "mfma bf16": (BF16_PEAK, 1e12, "TFLOP/s
 LONG_REGION = 0.2  # seconds of wall clock the headline loop should fill
 
 
-def roofline_of(bound, amount, seconds):
+SUSTAINED = {}  # matrix instruction -> TFLOP/s it sustains on varied operands (filled by measure_sustained)
+
+
+def roofline_of(bound, amount, seconds, instruction=None):
     """The roofline object of one configuration: `amount` algorithmic bytes (bound "hbm") or flops
-    (bound "mfma <type>") per launch over the launch time measured with events."""
+    (bound "mfma <type>") per launch over the launch time measured with events. instruction: the
+    matrix instruction the kernel runs on; the object then also carries what that instruction
+    sustains on operands of varied bits with nothing else going on (measured in this run) and the
+    fraction of it that the kernel reaches."""
     peak, unit_scale, unit = PEAKS[bound]
-    return {"bound": bound.split()[0], "algorithmic": int(amount), "achieved": round(amount / seconds / unit_scale, 1),
-            "peak": peak / unit_scale, "unit": unit, "frac": round(amount / seconds / peak, 4),
-            "launch_us": round(seconds * 1e6, 2)}
+    found = {"bound": bound.split()[0], "algorithmic": int(amount), "achieved": round(amount / seconds / unit_scale, 1),
+             "peak": peak / unit_scale, "unit": unit, "frac": round(amount / seconds / peak, 4),
+             "launch_us": round(seconds * 1e6, 2)}
+    if instruction in SUSTAINED:
+        found["instruction"] = instruction
+        found["sustained"] = SUSTAINED[instruction]
+        found["frac_of_sustained"] = round(amount / seconds / 1e12 / SUSTAINED[instruction], 4)
+    return found
+
+
+def bf16_instruction(plan_text):
+    """The matrix instruction of a planned BF16 product, from the planner's description of it."""
+    if "wave4" in plan_text:
+        return "bf16_16x16x32_one_wavefront_per_simd"
+    return "bf16_16x16x32" if "dma16" in plan_text else "bf16_32x32x16"
+
+
+def measure_sustained(torch, device):
+    """What the matrix cores sustain: independent matrix instructions with no memory traffic (the
+    part's clock under matrix load included), per instruction the prefill kernels use, on constant
+    and on varied operand bits. Fills SUSTAINED and returns the table for the report."""
+    import ctypes as ct
+
+    units = torch.cuda.get_device_properties(device).multi_processor_count
+    sink = torch.empty(units * 512, dtype=torch.float32, device=device)
+    flops = ct.c_double(0.0)
+    table = {}
+    # (rounds sized for launches of 2-3 ms, long enough for the clock to settle)
+    for name, kind, rounds, single in (
+            ("bf16_32x32x16", 0, 16000, False), ("bf16_16x16x32", 4, 16000, False),
+            ("bf16_16x16x32_one_wavefront_per_simd", 4, 32000, True),
+            ("e4m3_scaled_32x32x64", 1, 8000, False), ("e4m3_scaled_16x16x128", 5, 8000, False),
+            ("e2m1_x_e4m3_scaled_32x32x64", 2, 8000, False), ("e2m1_x_e4m3_scaled_16x16x128", 6, 8000, False),
+            ("fp32_32x32x2", 3, 8000, False)):
+        launch = probes().camblas_probe_matrix_single if single else probes().camblas_probe_matrix
+        entry = {}
+        for operands, constant in (("varied", 0), ("constant", 1)):
+            seconds = event_time(
+                torch, lambda i: launch(ct.c_void_p(torch.cuda.current_stream(device).cuda_stream), kind, units,
+                                        rounds, constant, ct.c_void_p(sink.data_ptr()), sink.numel() * 4,
+                                        ct.byref(flops)), 2, 5)
+            entry[operands + "_operands_tflops"] = round(flops.value / seconds / 1e12, 1)
+        table[name] = entry
+        SUSTAINED[name] = entry["varied_operands_tflops"]
+    return table
 
 OUTPUTS, INNER = 28672, 8192
 BATCHES = (1, 8, 32)
@@ -250,13 +302,17 @@ def main():
         step(index)
     elapsed = timed(args.steps)
     step_bytes = sum(decode_bytes(m) for m in BATCHES)
-    value = step_bytes * args.steps / elapsed / 1e9
-    long_run = None
-    if elapsed < LONG_REGION:  # too short a region for a wall clock: time a longer one as well
-        long_steps = int(LONG_REGION * 1.1 / (elapsed / max(args.steps, 1))) + 1
-        long_elapsed = timed(long_steps)
-        long_run = {"steps": long_steps, "ms": round(long_elapsed * 1e3, 2),
-                    "value": round(step_bytes * long_steps / long_elapsed / 1e9, 1)}
+    steps = args.steps
+    short_run = None
+    if elapsed < LONG_REGION:
+        # too short a region for a wall clock (a few milliseconds are mostly the loop's start and the
+        # last synchronisation): enough steps to fill LONG_REGION are timed, and those are reported;
+        # the requested region is kept beside them
+        short_run = {"steps": args.steps, "ms": round(elapsed * 1e3, 2),
+                     "value": round(step_bytes * args.steps / elapsed / 1e9, 1)}
+        steps = int(LONG_REGION * 1.1 / (elapsed / max(args.steps, 1))) + 1
+        elapsed = timed(steps)
+    value = step_bytes * steps / elapsed / 1e9
 
     # dominant kernel: the M=32 launch, timed alone with events on the launch stream
     per_launch = {}
@@ -295,9 +351,9 @@ def main():
         "value": round(value, 1),
         "unit": "GB/s",
         "n_gpus": 1,
-        "steps": args.steps,
+        "steps": steps,
         "warmup": args.warmup,
-        "ms_per_step": round(elapsed / args.steps * 1e3, 4),
+        "ms_per_step": round(elapsed / steps * 1e3, 4),
         "higher_is_better": True,
         "scaling": "weak",
         "vs_baseline": None,
@@ -310,7 +366,8 @@ def main():
             "entry_point": "camblas_cuda_bgemm('T','N')",
             "peak_fraction": round(value * 1e9 / HBM_PEAK, 4),
             "timed_region_ms": round(elapsed * 1e3, 2),
-            "long_run": long_run,
+            "requested_steps": args.steps,
+            "short_run": short_run,
         },
         "roofline": roofline,
         "cpu_baseline": None if args.skip_cpu else cpu_torch_linear(),
@@ -337,6 +394,7 @@ def probes():
         lib.camblas_probe_copy.argtypes = [ct.c_void_p, ct.c_size_t, ct.c_void_p, ct.c_void_p]
         lib.camblas_probe_matrix.argtypes = [ct.c_void_p, ct.c_int, ct.c_int, ct.c_int, ct.c_int,
                                              ct.c_void_p, ct.c_size_t, ct.POINTER(ct.c_double)]
+        lib.camblas_probe_matrix_single.argtypes = lib.camblas_probe_matrix.argtypes
         probes.library = lib
     return probes.library
 
@@ -568,8 +626,11 @@ def layer_step(torch, _kernels, device, normal):
 def extras(torch, _kernels, _native, device, normal):
     """The other configurations, each as absolute rate and fraction of its roofline."""
     found = {}
+    found["matrix_instruction_issue_rate"] = measure_sustained(torch, device)
     # BF16 prefill linear and addmm (beta = 1)
     tokens, outputs, inner = 4096, 10240, 8192
+    prefill_instruction = bf16_instruction(
+        _native.plan_describe(2, "T", "N", outputs, tokens, inner, inner, inner, outputs)[1])
     x, w = normal((tokens, inner)), normal((outputs, inner), 0.02)
     y = torch.empty((tokens, outputs), dtype=torch.bfloat16, device=device)
     c = normal((tokens, outputs))
@@ -579,19 +640,20 @@ def extras(torch, _kernels, _native, device, normal):
     seconds = event_time(torch, lambda i: _kernels.matmul(x, w.t(), out=y), 50, 100)
     found["bf16_prefill_linear"] = {
         "shape": [tokens, outputs, inner], "us": round(seconds * 1e6, 1),
-        "tflops": round(flops / seconds / 1e12, 1), "roofline": roofline_of("mfma bf16", flops, seconds),
+        "tflops": round(flops / seconds / 1e12, 1),
+        "roofline": roofline_of("mfma bf16", flops, seconds, prefill_instruction),
     }
     seconds = event_time(torch, lambda i: _kernels.addmm(c, x, w.t(), beta=1.0), 10, 50)
     found["bf16_prefill_addmm_beta1"] = {
         "us": round(seconds * 1e6, 1), "tflops": round(flops / seconds / 1e12, 1),
-        "roofline": roofline_of("mfma bf16", flops, seconds),
+        "roofline": roofline_of("mfma bf16", flops, seconds, prefill_instruction),
         "note": "full [tokens, outputs] addend read by the product's epilogue (no expand+clone copy)",
     }
     row = normal((outputs,))
     seconds = event_time(torch, lambda i: _kernels.addmm(row, x, w.t(), beta=1.0), 10, 50)
     found["bf16_prefill_addmm_bias_row"] = {
         "us": round(seconds * 1e6, 1), "tflops": round(flops / seconds / 1e12, 1),
-        "roofline": roofline_of("mfma bf16", flops, seconds),
+        "roofline": roofline_of("mfma bf16", flops, seconds, prefill_instruction),
         "note": "[outputs] bias row of a linear layer, read by the product's epilogue",
     }
     del x, w, y, c, row
@@ -601,8 +663,10 @@ def extras(torch, _kernels, _native, device, normal):
     x, w = normal((size, size)), normal((size, size), 0.02)
     y = torch.empty((size, size), dtype=torch.bfloat16, device=device)
     seconds = event_time(torch, lambda i: _kernels.matmul(x, w, out=y), 10, 30)
-    found["bf16_matmul_nn_4096"] = {"us": round(seconds * 1e6, 1),
-                                    "roofline": roofline_of("mfma bf16", 2.0 * size**3, seconds)}
+    found["bf16_matmul_nn_4096"] = {
+        "us": round(seconds * 1e6, 1),
+        "roofline": roofline_of("mfma bf16", 2.0 * size**3, seconds, bf16_instruction(
+            _native.plan_describe(2, "T", "N", size, size, size, size, size, size)[1]))}
     del x, w, y
     # BF16 linear at 256 tokens on a square projection (64 tiles of 128 x 256 for 256 compute units:
     # K is divided over workgroups); five weight copies rotate so that the weights come from HBM
@@ -647,9 +711,12 @@ def extras(torch, _kernels, _native, device, normal):
         traffic = outputs * inner + w_scale.numel() * 4 + tokens * (inner + inner // 128 * 4 + outputs * 2)
         # few tokens stream the weights once (HBM roofline); 4096 tokens are matrix-core work
         bound = ("mfma fp8", flops) if flops / FP8_PEAK > traffic / HBM_PEAK else ("hbm", traffic)
+        plan_text = _native.plan_describe(3, "T", "N", outputs, tokens, inner, inner, inner, outputs)[1]
+        instruction = "e4m3_scaled_16x16x128" if "fp8dma16" in plan_text else "e4m3_scaled_32x32x64"
         fp8[str(tokens)] = {
             "us": round(seconds * 1e6, 1), "tflops": round(flops / seconds / 1e12, 1),
-            "gbps": round(traffic / seconds / 1e9, 1), "roofline": roofline_of(*bound, seconds),
+            "gbps": round(traffic / seconds / 1e9, 1),
+            "roofline": roofline_of(*bound, seconds, instruction if bound[0] != "hbm" else None),
         }
     found["fp8_block_linear_18432x7168"] = fp8
     # single-token block-32 product of the reference header (FP32 scales per 32 x 32 block)
@@ -692,7 +759,8 @@ def extras(torch, _kernels, _native, device, normal):
         seconds = event_time(torch, lambda i: _kernels.quantized_matmul(a, a_scale, w, scale), 50, 100)
         flops = 2.0 * 4096 * outputs * inner
         mx[name] = {"us": round(seconds * 1e6, 1), "tflops": round(flops / seconds / 1e12, 1),
-                    "roofline": roofline_of("mfma fp8", flops, seconds)}
+                    "roofline": roofline_of("mfma fp8", flops, seconds, "e2m1_x_e4m3_scaled_32x32x64" if packed
+                                            else "e4m3_scaled_32x32x64")}
         del w, scale, a, a_scale
     found["mx_quantized_matmul_m4096_18432x7168"] = mx
     # a narrow projection with a long K at 128 rows (56 tiles of 128 x 128 for 256 compute units: K is
@@ -747,7 +815,7 @@ def extras(torch, _kernels, _native, device, normal):
     c32 = torch.empty((size, size), device=device)
     seconds = event_time(torch, lambda i: _kernels.matmul(a32, b32, out=c32), 20, 60)
     found["fp32_sgemm_2048"] = {"us": round(seconds * 1e6, 1),
-                                "roofline": roofline_of("mfma fp32", 2.0 * size**3, seconds)}
+                                "roofline": roofline_of("mfma fp32", 2.0 * size**3, seconds, "fp32_32x32x2")}
     # single-token FP8 expert step (9 of 289 experts, rotating sets)
     experts, hidden, width, choices = MOE_SHAPE
     step = moe_step(torch, _kernels, device, normal)
@@ -757,28 +825,9 @@ def extras(torch, _kernels, _native, device, normal):
         "us": round(seconds * 1e6, 1), "roofline": roofline_of("hbm", traffic, seconds),
         "note": "two launches; bound by launch and latency, not bandwidth"}
     del step
-    # what the matrix cores sustain: independent matrix instructions with no memory traffic (the
-    # part's clock under matrix load included), the ceiling the prefill rates are read against
     import ctypes as ct
 
     native = _native.context(device)
-    units = torch.cuda.get_device_properties(device).multi_processor_count
-    sink = torch.empty(units * 512, dtype=torch.float32, device=device)
-    flops = ct.c_double(0.0)
-    sustained = {}
-    # (rounds sized for launches of 2-3 ms, long enough for the clock to settle)
-    for name, kind, rounds in (("bf16_32x32x16", 0, 16000), ("e4m3_scaled_32x32x64", 1, 8000),
-                               ("e2m1_x_e4m3_scaled_32x32x64", 2, 8000), ("fp32_32x32x2", 3, 8000)):
-        entry = {}
-        for operands, constant in (("varied", 0), ("constant", 1)):
-            seconds = event_time(
-                torch, lambda i: probes().camblas_probe_matrix(
-                    ct.c_void_p(torch.cuda.current_stream(device).cuda_stream), kind, units, rounds, constant,
-                    ct.c_void_p(sink.data_ptr()), sink.numel() * 4, ct.byref(flops)),
-                2, 5)
-            entry[operands + "_operands_tflops"] = round(flops.value / seconds / 1e12, 1)
-        sustained[name] = entry
-    found["matrix_instruction_issue_rate"] = sustained
     # FP64 DGEMM 4096^3 (plumbing), through the C entry point
 
     size = 4096

@@ -749,26 +749,156 @@ def rope_kv_append(qkv, positions, k_cache, v_cache, *, q_heads, kv_heads, theta
     return qkv
 
 
+def rope_angles(positions, dim=128, theta=500000.0):
+    """FP32 [batch, 2, dim / 2]: sines and cosines of positions * theta^(-2i/dim), the angles of one decode
+    step (the same for every layer), for rope_append_attention / decoder_layer_decode."""
+    _require(positions.is_cuda and positions.dtype == torch.int32 and positions.dim() == 1, "positions: int32 [batch]")
+    angles = torch.empty((positions.shape[0], 2, dim // 2), dtype=torch.float32, device=positions.device)
+    _native.context(positions.device).call("rope_angles", positions.shape[0], dim, ct.c_float(theta),
+                                           _pointer(positions), _pointer(angles))
+    return angles
+
+
+def rope_append_attention(qkv, positions, k_cache, v_cache, *, q_heads, kv_heads, theta=500000.0, scale=None,
+                          angles=None):
+    """rope_kv_append() and gqa_decode_attention() over positions + 1 entries in one call (two launches
+    instead of three): the attention's partition kernel rotates the queries and the new K row itself and
+    appends the new K and V rows to the caches. qkv [B, Hq + 2 Hkv, D] is left unrotated. Bit for bit the
+    result and the caches of the two separate calls."""
+    _require(qkv.dtype == torch.bfloat16 and qkv.is_cuda and qkv.dim() == 3
+             and qkv.shape[1] == q_heads + 2 * kv_heads, "qkv must be BF16 [B, Hq + 2 Hkv, D]")
+    _require(qkv.stride(2) == 1 and qkv.stride(1) == qkv.shape[2], "qkv heads must be dense")
+    _require(k_cache.is_contiguous() and v_cache.is_contiguous() and k_cache.shape == v_cache.shape
+             and k_cache.shape[2:] == (kv_heads, qkv.shape[2]), "caches must be [B, C, Hkv, D]")
+    batch, _, dim = qkv.shape
+    _require(angles is None or (angles.dtype == torch.float32 and angles.is_contiguous()
+                                and tuple(angles.shape) == (batch, 2, dim // 2)), "angles: what rope_angles returns")
+    scale = dim**-0.5 if scale is None else scale
+    out = torch.empty((batch, q_heads, dim), dtype=torch.bfloat16, device=qkv.device)
+    _native.context(qkv.device).call(
+        "rope_append_gqa_decode_attention", batch, q_heads, kv_heads, dim, k_cache.shape[1], _pointer(positions),
+        ct.c_float(theta), ct.c_float(scale), _pointer(qkv), qkv.stride(0), _pointer(k_cache), _pointer(v_cache),
+        _pointer(angles), _pointer(out))
+    return out
+
+
 def decoder_layer_decode(hidden, residual, weights, k_cache, v_cache, positions, lengths, *,
-                         q_heads, kv_heads, head_dim=128, epsilon=1e-5, theta=500000.0):
+                         q_heads, kv_heads, head_dim=128, epsilon=1e-5, theta=500000.0, angles=None):
     """One Llama-shaped decoder layer for one new token per sequence.
 
-    residual-add + RMSNorm -> fused QKV linear -> RoPE on q and k with cache append -> GQA decode
-    attention -> o-proj -> residual-add + RMSNorm -> SwiGLU MLP. Returns (mlp output, residual).
+    residual-add + RMSNorm -> fused QKV linear -> RoPE on q and k with cache append and GQA decode
+    attention (one call) -> o-proj -> residual-add + RMSNorm -> SwiGLU MLP. Returns (mlp output, residual).
     `weights` holds input_norm, qkv [ (Hq+2Hkv)*D, hidden ], o, post_norm, gate, up, down.
     `positions` (int32 [batch]) is the cache slot the new token is written to and rotated for;
     `lengths` (int32 [batch]) the number of valid cache positions afterwards (positions + 1).
+    `angles` (optional): rope_angles(positions, head_dim, theta), made once per decode step for all layers.
     Every step is a call into libcamblas_hip.so, so the whole function can be captured in a graph
     after one warm-up call on the capture stream.
     """
     batch = hidden.shape[0]
     residual, normed = add_rms_norm(hidden, residual, weights["input_norm"], epsilon)
     qkv = linear(normed, weights["qkv"]).view(batch, q_heads + 2 * kv_heads, head_dim)
-    rope_kv_append(qkv, positions, k_cache, v_cache, q_heads=q_heads, kv_heads=kv_heads, theta=theta)
-    attended = gqa_decode_attention(qkv[:, :q_heads], k_cache, v_cache, lengths)
+    # (rotary embedding, cache append and attention over positions + 1 entries: `lengths` is what that gives)
+    attended = rope_append_attention(qkv, positions, k_cache, v_cache, q_heads=q_heads, kv_heads=kv_heads,
+                                     theta=theta, angles=angles)
     projected = linear(attended.view(batch, q_heads * head_dim), weights["o"])
     residual, normed = add_rms_norm(projected, residual, weights["post_norm"], epsilon)
     return gated_mlp(normed, weights["gate"], weights["up"], weights["down"]), residual
+
+
+def add_residual_squares(x, residual):
+    """(added, squares, count): added = bf16(x + residual) and its rows' sums of squares, the state the
+    fused decode linears pass along (count partial sums per row; here one)."""
+    _require(x.is_cuda and x.dtype == residual.dtype == torch.bfloat16 and x.shape == residual.shape
+             and x.dim() == 2 and x.is_contiguous() and residual.is_contiguous(),
+             "add_residual_squares takes two contiguous BF16 [rows, width] device tensors")
+    rows, width = x.shape
+    added = torch.empty_like(x)
+    squares = torch.empty((1, rows), dtype=torch.float32, device=x.device)
+    _native.context(x.device).call("add_residual_squares", rows, width, _pointer(x), _pointer(residual),
+                                   _pointer(added), _pointer(squares))
+    return added, squares, 1
+
+
+def _fused_linear_takes(x, weight):
+    return (x.dtype == weight.dtype == torch.bfloat16 and x.is_cuda and x.dim() == 2 and weight.dim() == 2
+            and 0 < x.shape[0] <= 64 and x.shape[1] == weight.shape[1] and x.stride(1) == 1
+            and weight.stride(1) == 1 and x.shape[1] % 8 == 0 and x.stride(0) % 8 == 0
+            and weight.stride(0) % 8 == 0 and x.data_ptr() % 16 == 0 and weight.data_ptr() % 16 == 0)
+
+
+def linear_residual(x, weight, residual):
+    """(added, squares, count) with added = bf16(bf16(x weight^T) + residual): a decode linear with the
+    residual add of the RMSNorm that follows it in its epilogue, plus per-workgroup partial sums of
+    squares of the rows of `added` (squares[:count]) for the linear after that norm."""
+    _require(_fused_linear_takes(x, weight), "linear_residual takes a BF16 decode batch (at most 64 rows)")
+    rows, inner = x.shape
+    outputs = weight.shape[0]
+    _require(residual.dtype == torch.bfloat16 and tuple(residual.shape) == (rows, outputs)
+             and residual.stride(1) == 1, "residual must be BF16 [rows, outputs]")
+    added = torch.empty((rows, outputs), dtype=torch.bfloat16, device=x.device)
+    capacity = (outputs + 15) // 16
+    squares = torch.empty((capacity, rows), dtype=torch.float32, device=x.device)
+    count = ct.c_int(0)
+    _native.context(x.device).call(
+        "bf16_linear_residual", rows, outputs, inner, _pointer(x), x.stride(0), _pointer(weight), weight.stride(0),
+        _pointer(residual), residual.stride(0), _pointer(added), outputs, _pointer(squares), rows, capacity,
+        ct.byref(count))
+    return added, squares, count.value
+
+
+def rms_linear(x, squares, count, norm_weight, epsilon, weight):
+    """bf16(rms_norm(x) weight^T) for a BF16 decode batch, the normalisation done while the linear
+    stages its tokens; x, squares, count as linear_residual / add_residual_squares return them."""
+    _require(_fused_linear_takes(x, weight), "rms_linear takes a BF16 decode batch (at most 64 rows)")
+    rows, inner = x.shape
+    outputs = weight.shape[0]
+    _require(norm_weight.dtype == torch.bfloat16 and norm_weight.numel() == inner and norm_weight.is_contiguous()
+             and squares.dtype == torch.float32 and squares.dim() == 2 and squares.shape[1] >= rows
+             and squares.stride(1) == 1 and 1 <= count <= squares.shape[0], "rms_linear norm operands")
+    out = torch.empty((rows, outputs), dtype=torch.bfloat16, device=x.device)
+    _native.context(x.device).call(
+        "bf16_rms_linear", rows, outputs, inner, _pointer(x), x.stride(0), _pointer(squares), squares.stride(0),
+        count, _pointer(norm_weight), ct.c_float(epsilon), _pointer(weight), weight.stride(0), _pointer(out), outputs)
+    return out
+
+
+def rms_gated_linear(x, squares, count, norm_weight, epsilon, gate_weight, up_weight):
+    """gated_linear(rms_norm(x), gate, up) with the normalisation fused into the staging of x."""
+    _require(_gated_linear_takes(x, gate_weight, up_weight), "rms_gated_linear takes a BF16 decode batch")
+    rows, inner = x.shape
+    outputs = gate_weight.shape[0]
+    _require(norm_weight.dtype == torch.bfloat16 and norm_weight.numel() == inner and norm_weight.is_contiguous()
+             and squares.dtype == torch.float32 and squares.dim() == 2 and squares.shape[1] >= rows
+             and squares.stride(1) == 1 and 1 <= count <= squares.shape[0], "rms_gated_linear norm operands")
+    out = torch.empty((rows, outputs), dtype=torch.bfloat16, device=x.device)
+    _native.context(x.device).call(
+        "bf16_rms_gated_linear", rows, outputs, inner, _pointer(x), x.stride(0), _pointer(squares),
+        squares.stride(0), count, _pointer(norm_weight), ct.c_float(epsilon), _pointer(gate_weight),
+        _pointer(up_weight), gate_weight.stride(0), _pointer(out), outputs)
+    return out
+
+
+def decoder_layer_decode_fused(state, weights, k_cache, v_cache, positions, lengths, *,
+                               q_heads, kv_heads, head_dim=128, epsilon=1e-5, theta=500000.0, angles=None):
+    """decoder_layer_decode with both residual-add + RMSNorm steps fused into the linears around them.
+
+    `state` = (added, squares, count): the residual stream after the add that precedes this layer's
+    input norm, with its rows' partial sums of squares (add_residual_squares makes it for the first
+    layer; every layer returns the next one's). Six launches: QKV linear (normalising its input),
+    rotary embedding + cache append, attention (two), o-proj (adding the residual), gate + up +
+    SiLU-multiply (normalising its input), down projection (adding the residual). The values equal
+    decoder_layer_decode's up to the order in which the sums of squares are added.
+    """
+    added, squares, count = state
+    batch = added.shape[0]
+    qkv = rms_linear(added, squares, count, weights["input_norm"], epsilon, weights["qkv"])
+    qkv = qkv.view(batch, q_heads + 2 * kv_heads, head_dim)
+    attended = rope_append_attention(qkv, positions, k_cache, v_cache, q_heads=q_heads, kv_heads=kv_heads,
+                                     theta=theta, angles=angles)
+    added, squares, count = linear_residual(attended.view(batch, q_heads * head_dim), weights["o"], added)
+    hidden = rms_gated_linear(added, squares, count, weights["post_norm"], epsilon, weights["gate"], weights["up"])
+    return linear_residual(hidden, weights["down"], added)
 
 
 def __getattr__(name):

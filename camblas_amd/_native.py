@@ -86,6 +86,12 @@ SIGNATURES = {
     "gqa_decode_attention_noalloc": ([_P, _I, _I, _I, _I, _I, _P, _F, _P, _I, _P, _P, _P], _I),
     "gqa_decode_attention_noalloc_limit": ([], _SZ),
     "bf16_gated_linear": ([_P, _I, _I, _I, _P, _I, _P, _P, _I, _P, _I], _I),
+    "rope_append_gqa_decode_attention": ([_P, _I, _I, _I, _I, _I, _P, _F, _F, _P, _I, _P, _P, _P, _P], _I),
+    "rope_angles": ([_P, _I, _I, _F, _P, _P], _I),
+    "bf16_linear_residual": ([_P, _I, _I, _I, _P, _I, _P, _I, _P, _I, _P, _I, _P, _I, _I, ct.POINTER(_I)], _I),
+    "bf16_rms_linear": ([_P, _I, _I, _I, _P, _I, _P, _I, _I, _P, _F, _P, _I, _P, _I], _I),
+    "bf16_rms_gated_linear": ([_P, _I, _I, _I, _P, _I, _P, _I, _I, _P, _F, _P, _P, _I, _P, _I], _I),
+    "add_residual_squares": ([_P, _I, _I, _P, _P, _P, _P], _I),
     "fp8_moe_decode": ([_P, _I, _I, _I, _I, _I, _P, _P, _P, _P, _P, _P, _P, _F, _P], _I),
     "hip_plan_describe": ([_I, _I, _C, _C, _I, _I, _I, _I, _I, _I, _I, ct.c_char_p, _SZ], _I),
     "hip_set_plan_override": ([_P, _I, _I], _I),

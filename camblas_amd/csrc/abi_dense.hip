@@ -663,6 +663,47 @@ int bf16_product(const Entry &entry, const Product &p, float alpha, const void *
     return launch_bf16_plan(entry, plan, p, alpha, a, b, beta, c, source, nullptr);
 }
 
+// A decode linear (at most 64 tokens, weights [outputs, inner] with K contiguous) with one or both
+// halves of a residual-add + RMSNorm fused into it: always the weight-streaming kernel, planned like an
+// ordinary linear of that shape. workgroups (may be null): receives the number of workgroups along
+// the outputs, which is the number of partial sums of squares per token a residual epilogue writes.
+int fused_stream_linear(const Entry &entry, int tokens, int outputs, int inner, const void *x, int ldx,
+                        const void *w, int ldw, void *y, int ldy, StreamFusion fusion, int capacity, int *workgroups)
+{
+    camblas_cuda_context *context = entry.context();
+    Plan plan = make_plan(2, CAMBLAS_CUDA_AUTO, true, false, outputs, tokens, inner, ldw, ldx, ldy, true,
+                          context->compute_units);
+    if (plan.family != FAMILY_STREAM || plan.kernel / 100 > 1) {
+        // (33 to 64 tokens on a narrow projection plan other kernels: the undivided streaming kernel then)
+        plan.family = FAMILY_STREAM;
+        plan.kernel = undivided_stream_kernel(outputs, tokens, inner, context->compute_units);
+        plan.split_k = 1;
+        if (plan.kernel / 100 > 1)
+            plan.kernel %= 100;
+    }
+    StreamShares shares;
+    if (plan.split_k > 1) {
+        const size_t bytes = stream_partial_bytes(plan.kernel / 10 % 10, plan.kernel % 10, outputs, tokens, plan.split_k);
+        if (reserve_arrivals(context) == hipSuccess && reserve_scratch(context, bytes) == hipSuccess) {
+            shares = StreamShares{plan.split_k, static_cast<float *>(context->scratch), context->arrivals};
+        } else {
+            context->counts[5]++;
+            plan.kernel = undivided_stream_kernel(outputs, tokens, inner, context->compute_units) % 100;
+        }
+    }
+    const int row_tiles = plan.kernel / 10 % 10;
+    const int count = stream_workgroups_along_outputs(row_tiles, outputs);
+    if (workgroups)
+        *workgroups = count;
+    if (fusion.residual && count > capacity)
+        return entry.refuse("room for the partial sums of squares");
+    context->counts[plan.counter]++;
+    return entry.finish(launch_bgemv_stream(context->stream, plan.kernel / 100, row_tiles, plan.kernel % 10, outputs,
+                                            tokens, inner, 1.f, w, ldw, x, ldx, 0.f, y, ldy, BetaSource{}, shares,
+                                            fusion),
+                        "BF16 streaming linear with fused normalisation");
+}
+
 template <typename T>
 int typed_gemm(camblas_cuda_context *context, char ta, char tb, int m, int n, int k, T alpha, const T *a,
                int lda, const T *b, int ldb, T beta, T *c, int ldc)
@@ -836,3 +877,64 @@ extern "C" int camblas_cuda_mlp_backward(camblas_cuda_context *context, int dtyp
         }
     });
 }
+
+// ---- the residual-add + RMSNorm around the decode linears, fused into them (extensions; the norm's
+// arithmetic is the reference's, src/cuda/inference_fusion.cuh:136-191, binding
+// src/cuda/torch_bindings.cpp:675-701)
+
+extern "C" int camblas_cuda_bf16_linear_residual(camblas_cuda_context *context, int tokens, int outputs, int inner,
+                                                 const void *x, int ldx, const void *w, int ldw,
+                                                 const void *residual, int ld_residual, void *added, int ld_added,
+                                                 float *squares, int squares_ld, int squares_capacity,
+                                                 int *squares_count)
+{
+    Entry entry(context);
+    return entry.run([&] {
+        if (squares_count)
+            *squares_count = 0;
+        if (!within({{tokens, 0, 64, 1}, {outputs, 0, INT32_MAX, 1}, {inner, 8, (1 << 23) - 8, 8},
+                     {ldx, inner, (1 << 23) - 8, 8}, {ldw, inner, (1 << 23) - 8, 8},
+                     {ld_residual, outputs, INT32_MAX, 1}, {ld_added, outputs, INT32_MAX, 1},
+                     {squares_ld, tokens, INT32_MAX, 1}, {squares_capacity, 0, INT32_MAX, 1}}))
+            return entry.refuse("invalid fused linear dimensions");
+        if (tokens == 0 || outputs == 0)
+            return 0;
+        if (!usable({{x, 16}, {w, 16}, {residual, 2}, {added, 2}, {squares, 4}}) || !squares_count ||
+            !apart(added, {x, w}) || !apart(squares, {x, w, residual, added}))
+            return entry.refuse("invalid fused linear buffers");
+        StreamFusion fusion;
+        fusion.residual = residual;
+        fusion.ld_residual = ld_residual;
+        fusion.ssq_out = squares;
+        fusion.ssq_ld_out = squares_ld;
+        return fused_stream_linear(entry, tokens, outputs, inner, x, ldx, w, ldw, added, ld_added, fusion,
+                                   squares_capacity, squares_count);
+    });
+}
+
+extern "C" int camblas_cuda_bf16_rms_linear(camblas_cuda_context *context, int tokens, int outputs, int inner,
+                                            const void *x, int ldx, const float *squares, int squares_ld,
+                                            int squares_count, const void *norm_weight, float epsilon,
+                                            const void *w, int ldw, void *y, int ldy)
+{
+    Entry entry(context);
+    return entry.run([&] {
+        if (!within({{tokens, 0, 64, 1}, {outputs, 0, INT32_MAX, 1}, {inner, 8, (1 << 23) - 8, 8},
+                     {ldx, inner, (1 << 23) - 8, 8}, {ldw, inner, (1 << 23) - 8, 8}, {ldy, outputs, INT32_MAX, 1},
+                     {squares_ld, tokens, INT32_MAX, 1}, {squares_count, 1, INT32_MAX, 1}}) ||
+            !(epsilon >= 0.f) || !std::isfinite(epsilon))
+            return entry.refuse("invalid fused linear dimensions");
+        if (tokens == 0 || outputs == 0)
+            return 0;
+        if (!usable({{x, 16}, {w, 16}, {norm_weight, 16}, {squares, 4}, {y, 2}}) || !apart(y, {x, w, norm_weight, squares}))
+            return entry.refuse("invalid fused linear buffers");
+        StreamFusion fusion;
+        fusion.norm_weight = norm_weight;
+        fusion.ssq_in = squares;
+        fusion.ssq_count = squares_count;
+        fusion.ssq_ld = squares_ld;
+        fusion.epsilon = epsilon;
+        return fused_stream_linear(entry, tokens, outputs, inner, x, ldx, w, ldw, y, ldy, fusion, 0, nullptr);
+    });
+}
+

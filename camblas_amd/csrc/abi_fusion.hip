@@ -211,6 +211,64 @@ extern "C" int camblas_cuda_bf16_gated_linear(camblas_cuda_context *context, int
     });
 }
 
+// The same with the RMSNorm in front of it fused in: x holds the un-normalised rows, `squares`
+// [squares_count][squares_ld] partial sums of squares of each row (added in index order), and the
+// tokens are normalised while they are staged (round(round(x * scale) * norm_weight), the reference's
+// rounding points, src/cuda/inference_fusion.cuh:186-189).
+extern "C" int camblas_cuda_bf16_rms_gated_linear(camblas_cuda_context *context, int rows, int outputs, int inner,
+                                                  const void *x, int ldx, const float *squares, int squares_ld,
+                                                  int squares_count, const void *norm_weight, float epsilon,
+                                                  const void *gate, const void *up, int ldw, void *out, int ldo)
+{
+    Entry entry(context);
+    return entry.run([&] {
+        if (!within({{rows, 0, 64, 1}, {outputs, 0, INT32_MAX, 1}, {inner, 8, (1 << 23) - 8, 8}, {ldx, inner, (1 << 23) - 8, 8},
+                     {ldw, inner, (1 << 23) - 8, 8}, {ldo, outputs, INT32_MAX, 1}, {squares_ld, rows, INT32_MAX, 1},
+                     {squares_count, 1, INT32_MAX, 1}}) ||
+            !valid_epsilon(epsilon))
+            return entry.refuse("invalid gated linear dimensions");
+        if (rows == 0 || outputs == 0)
+            return 0;
+        if (!usable({{x, 16}, {gate, 16}, {up, 16}, {norm_weight, 16}, {squares, 4}, {out, 2}}) ||
+            !apart(out, {x, gate, up, norm_weight, squares}))
+            return entry.refuse("invalid gated linear buffers");
+        const int token_tiles = rows <= 16 ? 1 : rows <= 32 ? 2 : 4;
+        int pair_tiles = 4;
+        while (pair_tiles > 1 && (outputs + 16 * pair_tiles - 1) / (16 * pair_tiles) * 2 < 3 * context->compute_units)
+            --pair_tiles;
+        if (context->override_kernel >= 1 && context->override_kernel <= 4)
+            pair_tiles = context->override_kernel;
+        context->counts[4]++;
+        StreamFusion fusion;
+        fusion.norm_weight = norm_weight;
+        fusion.ssq_in = squares;
+        fusion.ssq_count = squares_count;
+        fusion.ssq_ld = squares_ld;
+        fusion.epsilon = epsilon;
+        return entry.finish(launch_gated_stream(context->stream, pair_tiles, token_tiles, outputs, rows, inner,
+                                                gate, up, ldw, x, ldx, out, ldo, fusion),
+                            "BF16 gated streaming linear with fused normalisation");
+    });
+}
+
+// added = round(x + residual) per element and squares[row] = the sum of added^2 over the row: the
+// state the fused linears pass along, made from scratch (a model's first layer).
+extern "C" int camblas_cuda_add_residual_squares(camblas_cuda_context *context, int rows, int width,
+                                                 const void *x, const void *residual, void *added, float *squares)
+{
+    Entry entry(context);
+    return entry.run([&] {
+        if (rows < 0 || !within({{width, 0, INT32_MAX, 1}}))
+            return entry.refuse("invalid residual squares arguments");
+        if (rows == 0)
+            return 0;
+        if (!usable({{x, 2}, {residual, 2}, {added, 2}, {squares, 4}}) || !apart(squares, {x, residual, added}))
+            return entry.refuse("invalid residual squares buffers");
+        return entry.finish(launch_add_residual_squares(entry.stream(), rows, width, x, residual, added, squares),
+                            "residual add with sums of squares");
+    });
+}
+
 // ---- decode-layer pieces (no counterpart in the reference)
 
 extern "C" int camblas_cuda_rope(camblas_cuda_context *context, int tokens, int heads, int dim,
@@ -328,6 +386,62 @@ extern "C" int camblas_cuda_gqa_decode_attention(camblas_cuda_context *context, 
                                     *where = context->scratch;
                                     return 0;
                                 });
+    });
+}
+
+// A decode step's rotary embedding, cache append and attention in one call (two launches instead
+// of three): qkv holds the step's un-rotated activation rows [q heads | k heads | v heads], token_stride
+// elements apart; positions[b] is the cache slot of sequence b's new token. Equals, bit for bit,
+// camblas_cuda_rope_kv_append followed by camblas_cuda_gqa_decode_attention with lengths = positions + 1,
+// except that qkv itself is left as it was (the rotated queries live in registers only).
+extern "C" int camblas_cuda_rope_append_gqa_decode_attention(camblas_cuda_context *context, int batch, int q_heads,
+                                                             int kv_heads, int dim, int context_length,
+                                                             const int32_t *positions, float theta, float scale,
+                                                             const void *qkv, int token_stride, void *k_cache,
+                                                             void *v_cache, const float *angles, void *output)
+{
+    Entry entry(context);
+    return entry.run([&] {
+        const bool shaped = batch >= 0 && q_heads >= 1 && kv_heads >= 1 && q_heads % kv_heads == 0 &&
+                            q_heads / kv_heads <= 16 && dim == 128 && context_length >= 1 &&
+                            token_stride >= (q_heads + 2 * kv_heads) * dim && token_stride % 8 == 0 &&
+                            std::isfinite(scale) && std::isfinite(theta) && theta > 0;
+        if (!shaped)
+            return entry.refuse("invalid decode attention arguments");
+        if (batch == 0)
+            return 0;
+        if (!usable({{qkv, 16}, {k_cache, 16}, {v_cache, 16}, {output, 16}, {positions, 4}}) ||
+            !is_aligned(angles, 4) || !apart(output, {qkv, k_cache, v_cache}) || !apart(k_cache, {qkv, v_cache}) || !apart(v_cache, {qkv}))
+            return entry.refuse("invalid decode attention buffers");
+        int splits = 1;
+        const size_t bytes = gqa_decode_scratch_bytes(batch, q_heads, dim, context_length, &splits);
+        const hipError_t grown = reserve_scratch(context, bytes);
+        if (grown != hipSuccess)
+            return entry.refuse("decode attention scratch", int(grown));
+        context->counts[6]++;
+        const unsigned short *rows = static_cast<const unsigned short *>(qkv);
+        return entry.finish(launch_gqa_decode(entry.stream(), batch, q_heads, kv_heads, dim, context_length, nullptr,
+                                              scale, rows, token_stride, k_cache, v_cache, output, context->scratch,
+                                              splits, positions, theta, rows + size_t(q_heads) * dim,
+                                              rows + size_t(q_heads + kv_heads) * dim, angles),
+                            "decode attention with rotary embedding and cache append");
+    });
+}
+
+// The angles of a decode step, once for all layers: angles[b][0][i] = sin, angles[b][1][i] = cos of
+// positions[b] * theta^(-2i/dim), i < dim / 2, FP32, the values the rotary kernels work out themselves.
+extern "C" int camblas_cuda_rope_angles(camblas_cuda_context *context, int batch, int dim, float theta,
+                                        const int32_t *positions, float *angles)
+{
+    Entry entry(context);
+    return entry.run([&] {
+        if (batch < 0 || batch > (1 << 20) || !within({{dim, 2, 1024, 2}}) || !std::isfinite(theta) || !(theta > 0))
+            return entry.refuse("invalid rotary embedding arguments");
+        if (batch == 0)
+            return 0;
+        if (!usable({{positions, 4}, {angles, 4}}))
+            return entry.refuse("invalid rotary embedding buffers");
+        return entry.finish(launch_rope_table(entry.stream(), batch, dim, theta, positions, angles), "rotary angles");
     });
 }
 

@@ -45,14 +45,56 @@ __device__ __forceinline__ float swap_lanes(float value, int mask)
     return __shfl_xor(value, mask, 64);
 }
 
-__global__ __launch_bounds__(WAVES * 64) void gqa_partition_kernel(
+// What the FRESH form of the partition kernel adds: the step's new token arrives un-rotated in a
+// fused activation row [q heads | k heads | v heads] per sequence and is rotated here (q in
+// registers, for every partition; k by the one wavefront whose positions hold the token's cache
+// slot), that wavefront takes the new K and V rows from the activation instead of the cache, and
+// writes them to the cache. This replaces a launch of the rotary-embedding + cache-append kernel.
+struct FreshToken {
+    const int32_t *positions; // cache slot of the new token per sequence; the sequence then has positions + 1 entries
+    float theta;
+    const unsigned short *k_new, *v_new; // rows of the activation, token_stride apart per sequence, head-major
+    int token_stride;
+    unsigned short *k_cache, *v_cache;
+    // optional: sines [batch][64] then cosines of the positions' angles, made once per decode step for all
+    // layers (rope_table_kernel); without it every workgroup works the angles out itself
+    const float *table;
+};
+
+// positions the attention covers: lengths[b], or, in the FRESH form, positions[b] + 1
+__device__ __forceinline__ int live_length(const int32_t *lengths, const int32_t *positions, int b, int context_length)
+{
+    if (positions)
+        return min(max(positions[b] + 1, 0), context_length);
+    return lengths ? min(max(lengths[b], 0), context_length) : context_length;
+}
+
+// rotates the pair (lo, hi) of packed BF16 vectors: element e of lo pairs with element e of hi; the
+// eight sines and cosines are read from LDS where they are used, so that they do not occupy registers
+// across the kernel
+__device__ __forceinline__ void rotate_vectors(const float *sines, const float *cosines, u32x4_t &lo, u32x4_t &hi)
+{
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+        unsigned short l0, h0, l1, h1;
+        rotate_by(sines[2 * e], cosines[2 * e], __uint_as_float(lo[e] << 16), __uint_as_float(hi[e] << 16), l0, h0);
+        rotate_by(sines[2 * e + 1], cosines[2 * e + 1], __uint_as_float(lo[e] & 0xffff0000u),
+                  __uint_as_float(hi[e] & 0xffff0000u), l1, h1);
+        lo[e] = unsigned(l0) | (unsigned(l1) << 16);
+        hi[e] = unsigned(h0) | (unsigned(h1) << 16);
+    }
+}
+
+template <bool FRESH>
+__device__ __forceinline__ void gqa_partition(
     int q_heads, int kv_heads, int context_length, const int32_t *lengths, float scale,
     const unsigned short *q, int q_stride, const unsigned short *k_cache,
     const unsigned short *v_cache, float *part_o, float *part_m, float *part_l, int splits,
-    int group)
+    int group, const FreshToken &fresh)
 {
     __shared__ __attribute__((aligned(16))) float wave_o[WAVES][HEADS][DIM];
     __shared__ float wave_m[WAVES][HEADS], wave_l[WAVES][HEADS];
+    __shared__ float trig[2][FRESH ? DIM / 2 : 1]; // FRESH: sines and cosines of the new token's position
     // Consecutive workgroups go to consecutive XCDs, so with the partition as the fast grid index
     // and a partition count that is a multiple of eight, partition s of every sequence and head
     // would run on XCD s % 8: sequences much shorter than the cache would keep one or two XCDs
@@ -61,7 +103,7 @@ __global__ __launch_bounds__(WAVES * 64) void gqa_partition_kernel(
     const int split = int((blockIdx.x + blockIdx.y + blockIdx.z * gridDim.y) % gridDim.x);
     const int thread = threadIdx.x, lane = thread % 64, wave = thread / 64;
     const int m = lane % 16, j = lane / 16;
-    const int length = lengths ? min(max(lengths[b], 0), context_length) : context_length;
+    const int length = live_length(lengths, FRESH ? fresh.positions : nullptr, b, context_length);
     if (split * CHUNK >= length)
         return; // past the sequence: the combine never reads this partition (uniform, before any barrier)
     const int begin = split * CHUNK + wave * WAVE_POSITIONS;
@@ -77,13 +119,21 @@ __global__ __launch_bounds__(WAVES * 64) void gqa_partition_kernel(
     for (int w = 0; w < 8; ++w)
         acc[w] = f32x4_t{0.f, 0.f, 0.f, 0.f};
     float top = -INFINITY, total = 0.f;
+    bf16x8_t q_frag[4], k_frag[4][4];
+    u32x4_t v_rows[2][8];
+    // FRESH: the new token's slot relative to this wavefront's first position (outside
+    // [0, count) when another wavefront or partition holds it, or when it lies outside the cache)
+    const int token = FRESH ? fresh.positions[b] : -1;
+    // (in scalar registers: the branches on it below are then branches, not predication, which keeps the
+    // rare path's loads and temporaries out of the common path's register allocation)
+    const int slot = __builtin_amdgcn_readfirstlane(FRESH && token >= 0 && token < context_length ? token - begin : -1);
+    const int wave_count = __builtin_amdgcn_readfirstlane(count);
+    const bool holds_token = slot >= 0 && slot < wave_count; // uniform over the wavefront
     if (count > 0) { // uniform over the wavefront
         // ---- loads: Q (head m, dims 32s + 8j ..), K (position 16t + m, same dims),
         // V (position 32u + 16(e/4) + 4j + e%4, dims 8m ..); rows past the end repeat the last one
         const int head = kvh * group + (m < group ? m : group - 1);
         const unsigned short *q_row = q + size_t(b) * q_stride + size_t(head) * DIM + 8 * j;
-        bf16x8_t q_frag[4], k_frag[4][4];
-        u32x4_t v_rows[2][8];
 #pragma unroll
         for (int s = 0; s < 4; ++s)
             q_frag[s] = *reinterpret_cast<const bf16x8_t *>(q_row + 32 * s);
@@ -107,6 +157,83 @@ __global__ __launch_bounds__(WAVES * 64) void gqa_partition_kernel(
                 v_rows[u][e] = __builtin_nontemporal_load(reinterpret_cast<const u32x4_t *>(
                     v_base + size_t(position) * row_stride + 8 * m));
             }
+    }
+    if constexpr (FRESH) {
+        // the sixty-four angles of the token's position, once per workgroup, while the loads travel
+        // (every lane working out its own sixteen doubled the kernel's time)
+        if (thread < DIM / 2) {
+            if (fresh.table) {
+                trig[0][thread] = fresh.table[(size_t(b) * 2) * (DIM / 2) + thread];
+                trig[1][thread] = fresh.table[(size_t(b) * 2 + 1) * (DIM / 2) + thread];
+            } else {
+                pair_sincos(float(token), thread, DIM, fresh.theta, trig[0][thread], trig[1][thread]);
+            }
+        }
+        __syncthreads();
+    }
+    if (count > 0) {
+        if constexpr (FRESH) {
+            // this lane's sixteen pair indices: dims 32 s + 8 j + e for s = 0, 1 pair with 64 + the same
+            // (fragments s and s + 2), for the queries and for the new K row alike
+#pragma unroll
+            for (int s = 0; s < 2; ++s) {
+                u32x4_t lo = __builtin_bit_cast(u32x4_t, q_frag[s]), hi = __builtin_bit_cast(u32x4_t, q_frag[s + 2]);
+                rotate_vectors(&trig[0][32 * s + 8 * j], &trig[1][32 * s + 8 * j], lo, hi);
+                q_frag[s] = __builtin_bit_cast(bf16x8_t, lo);
+                q_frag[s + 2] = __builtin_bit_cast(bf16x8_t, hi);
+            }
+            if (holds_token) {
+                const unsigned short *k_new = fresh.k_new + size_t(b) * fresh.token_stride + size_t(kvh) * DIM;
+                const unsigned short *v_new = fresh.v_new + size_t(b) * fresh.token_stride + size_t(kvh) * DIM;
+                unsigned short *k_slot = fresh.k_cache + (size_t(b) * context_length + begin + slot) * row_stride +
+                                         size_t(kvh) * DIM;
+                unsigned short *v_slot = fresh.v_cache + (size_t(b) * context_length + begin + slot) * row_stride +
+                                         size_t(kvh) * DIM;
+#pragma unroll
+                for (int t = 0; t < 4; ++t) {
+                    // (uniform: tile t holds the slot, or repeats it as the sequence's last row)
+                    if (!((slot >= 16 * t && slot < 16 * t + 16) || (slot == wave_count - 1 && 16 * t + 15 > slot)))
+                        continue;
+                    int position = 16 * t + m;
+                    position = position < count ? position : count - 1;
+                    if (position == slot) {
+                        // the token's cache slot is not written yet: what was loaded from it is replaced by
+                        // the activation's row, rotated (a second, dependent load, in this one wavefront only)
+#pragma unroll
+                        for (int s = 0; s < 4; ++s)
+                            k_frag[t][s] = *reinterpret_cast<const bf16x8_t *>(k_new + 32 * s + 8 * j);
+#pragma unroll
+                        for (int s = 0; s < 2; ++s) {
+                            u32x4_t lo = __builtin_bit_cast(u32x4_t, k_frag[t][s]);
+                            u32x4_t hi = __builtin_bit_cast(u32x4_t, k_frag[t][s + 2]);
+                            rotate_vectors(&trig[0][32 * s + 8 * j], &trig[1][32 * s + 8 * j], lo, hi);
+                            k_frag[t][s] = __builtin_bit_cast(bf16x8_t, lo);
+                            k_frag[t][s + 2] = __builtin_bit_cast(bf16x8_t, hi);
+                        }
+                        if (16 * t + m == slot) // the lanes that hold the row itself (not a repeat of it) append it
+#pragma unroll
+                            for (int s = 0; s < 4; ++s)
+                                *reinterpret_cast<bf16x8_t *>(k_slot + 32 * s + 8 * j) = k_frag[t][s];
+                    }
+                }
+#pragma unroll
+                for (int u = 0; u < 2; ++u)
+#pragma unroll
+                    for (int e = 0; e < 8; ++e) {
+                        // (uniform: some lane of this register holds the slot or repeats it)
+                        const int first = 32 * u + 16 * (e / 4) + e % 4, last = first + 12;
+                        if (!((slot >= first && slot <= last) || (slot == wave_count - 1 && last > slot)))
+                            continue;
+                        int position = 32 * u + 16 * (e / 4) + 4 * j + e % 4;
+                        const bool row_itself = position == slot;
+                        position = position < count ? position : count - 1;
+                        if (position == slot) // (also the lanes that repeat the last row: they must not keep stale data)
+                            v_rows[u][e] = *reinterpret_cast<const u32x4_t *>(v_new + 8 * m);
+                        if (row_itself)
+                            *reinterpret_cast<u32x4_t *>(v_slot + 8 * m) = v_rows[u][e];
+                    }
+            }
+        }
 
         // ---- scores: register r of tile t is position 16t + 4j + r, head m
         f32x4_t score[4];
@@ -202,17 +329,49 @@ __global__ __launch_bounds__(WAVES * 64) void gqa_partition_kernel(
     }
 }
 
+// table[b][0][i] = sin, table[b][1][i] = cos of positions[b] * theta^(-2i/dim), i < dim / 2: the angles of a
+// decode step, the same for every layer of a model
+__global__ void rope_table_kernel(int batch, int dim, float theta, const int32_t *positions, float *table)
+{
+    const int half = dim / 2, index = blockIdx.x * blockDim.x + threadIdx.x;
+    if (index >= batch * half)
+        return;
+    const int b = index / half, i = index % half;
+    pair_sincos(float(positions[b]), i, dim, theta, table[(size_t(b) * 2) * half + i], table[(size_t(b) * 2 + 1) * half + i]);
+}
+
+__global__ __launch_bounds__(WAVES * 64) void gqa_partition_kernel(
+    int q_heads, int kv_heads, int context_length, const int32_t *lengths, float scale,
+    const unsigned short *q, int q_stride, const unsigned short *k_cache,
+    const unsigned short *v_cache, float *part_o, float *part_m, float *part_l, int splits, int group)
+{
+    gqa_partition<false>(q_heads, kv_heads, context_length, lengths, scale, q, q_stride, k_cache, v_cache, part_o,
+                         part_m, part_l, splits, group, FreshToken{});
+}
+
+// (two wavefronts per SIMD, i.e. at most 256 registers, as the plain form has: two workgroups per
+// compute unit keep twice the cache rows in flight; left alone this form allocated 268 registers and
+// ran at half the rate)
+__global__ __launch_bounds__(WAVES * 64, 2) void gqa_fresh_partition_kernel(
+    int q_heads, int kv_heads, int context_length, float scale, const unsigned short *q, int q_stride,
+    const unsigned short *k_cache, const unsigned short *v_cache, float *part_o, float *part_m, float *part_l,
+    int splits, int group, FreshToken fresh)
+{
+    gqa_partition<true>(q_heads, kv_heads, context_length, nullptr, scale, q, q_stride, k_cache, v_cache, part_o,
+                        part_m, part_l, splits, group, fresh);
+}
+
 // out[b, head, :] = sum_s exp(m_s - M) o_s / sum_s exp(m_s - M) l_s, partitions in index order.
 // Only the partitions that hold positions of the sequence are read: the others were never written.
 __global__ __launch_bounds__(DIM) void gqa_combine_kernel(int partitions, int q_heads, int context_length,
-                                                          const int32_t *lengths, const float *part_o,
-                                                          const float *part_m, const float *part_l,
-                                                          unsigned short *out)
+                                                          const int32_t *lengths, const int32_t *positions,
+                                                          const float *part_o, const float *part_m,
+                                                          const float *part_l, unsigned short *out)
 {
     const size_t row = blockIdx.x; // b * q_heads + head
     const int d = threadIdx.x;
     const int b = int(row / q_heads);
-    const int length = lengths ? min(max(lengths[b], 0), context_length) : context_length;
+    const int length = live_length(lengths, positions, b, context_length);
     const int splits = min(partitions, (length + CHUNK - 1) / CHUNK);
     // Partitions are taken eight at a time with all loads of a batch issued before any is used
     // (a loop of dependent scalar loads would pay the memory latency once per partition); indices
@@ -266,6 +425,13 @@ size_t gqa_decode_scratch_bytes(int batch, int q_heads, int dim, int context_len
     return rows * (size_t(dim) + 2) * sizeof(float);
 }
 
+hipError_t launch_rope_table(hipStream_t stream, int batch, int dim, float theta, const int32_t *positions, float *table)
+{
+    const int count = batch * (dim / 2);
+    rope_table_kernel<<<unsigned((count + 255) / 256), 256, 0, stream>>>(batch, dim, theta, positions, table);
+    return launch_status();
+}
+
 size_t gqa_resident_scratch_bytes() { return RESIDENT_BYTES; }
 
 // Address of this device's copy of the fixed partials array. `device` must be the current device
@@ -294,7 +460,8 @@ hipError_t gqa_resident_scratch(int device, void **address)
 hipError_t launch_gqa_decode(hipStream_t stream, int batch, int q_heads, int kv_heads, int dim,
                              int context_length, const int32_t *lengths, float scale, const void *q,
                              int q_stride, const void *k, const void *v, void *out, void *partials,
-                             int splits)
+                             int splits, const int32_t *positions, float theta, const void *k_new,
+                             const void *v_new, const float *table)
 {
     const int group = kv_heads > 0 ? q_heads / kv_heads : 0;
     if (dim != DIM || splits > 65535 || kv_heads > 65535 || batch > 65535 || group < 1 ||
@@ -308,14 +475,24 @@ hipError_t launch_gqa_decode(hipStream_t stream, int batch, int q_heads, int kv_
     const unsigned short *qp = static_cast<const unsigned short *>(q);
     const unsigned short *kp = static_cast<const unsigned short *>(k);
     const unsigned short *vp = static_cast<const unsigned short *>(v);
-    gqa_partition_kernel<<<grid, WAVES * 64, 0, stream>>>(q_heads, kv_heads, context_length, lengths,
-                                                          scale, qp, q_stride, kp, vp, part_o, part_m,
-                                                          part_l, splits, group);
+    if (positions) {
+        // the new token's rows come with the queries (token stride q_stride) and go into the caches
+        const FreshToken fresh = {positions, theta, static_cast<const unsigned short *>(k_new),
+                                  static_cast<const unsigned short *>(v_new), q_stride,
+                                  const_cast<unsigned short *>(kp), const_cast<unsigned short *>(vp), table};
+        gqa_fresh_partition_kernel<<<grid, WAVES * 64, 0, stream>>>(q_heads, kv_heads, context_length, scale, qp,
+                                                                    q_stride, kp, vp, part_o, part_m, part_l, splits,
+                                                                    group, fresh);
+    } else {
+        gqa_partition_kernel<<<grid, WAVES * 64, 0, stream>>>(q_heads, kv_heads, context_length, lengths, scale, qp,
+                                                              q_stride, kp, vp, part_o, part_m, part_l, splits, group);
+    }
     hipError_t status = launch_status();
     if (status != hipSuccess)
         return status;
     gqa_combine_kernel<<<unsigned(size_t(batch) * q_heads), DIM, 0, stream>>>(
-        splits, q_heads, context_length, lengths, part_o, part_m, part_l, static_cast<unsigned short *>(out));
+        splits, q_heads, context_length, positions ? nullptr : lengths, positions, part_o, part_m, part_l,
+        static_cast<unsigned short *>(out));
     return launch_status();
 }
 } // namespace camblas_hip

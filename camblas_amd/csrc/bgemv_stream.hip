@@ -36,9 +36,31 @@ struct StreamParams {
     // arrival counter per (blockIdx.x, blockIdx.y), zero before and after every launch
     float *partials;
     unsigned *arrivals;
+    // ---- the FUSE instantiations only
+    // x is normalised while it is staged: round(round(x * scale[token]) * norm_weight[k]) with
+    // scale = rsqrt(sum / k + epsilon), sum = ssq_in[0][token] + ssq_in[1][token] + ... in index order
+    const unsigned short *norm_weight;
+    const float *ssq_in;
+    int ssq_count, ssq_ld;
+    float epsilon;
+    // y = round(round(alpha * x W^T) + residual[token * ld_residual + feature]), and workgroup
+    // blockIdx.x leaves the sums of squares of its features of every row of y in
+    // ssq_out[blockIdx.x * ssq_ld_out + token] (fixed order)
+    const unsigned short *residual;
+    int ld_residual;
+    float *ssq_out;
+    int ssq_ld_out;
 };
 
 constexpr int WAVES = 4, DEPTH = 2;
+
+typedef float f32x2_round_t __attribute__((ext_vector_type(2)));
+typedef __bf16 bf16x2_round_t __attribute__((ext_vector_type(2)));
+// two FP32 values rounded to nearest-even BF16 and packed, by the conversion instruction of gfx950
+__device__ __forceinline__ unsigned round_pack_bf16x2(float lo, float hi)
+{
+    return __builtin_bit_cast(unsigned, __builtin_convertvector(f32x2_round_t{lo, hi}, bf16x2_round_t));
+}
 
 // NT, MT: 16-row weight tiles and 16-token tiles per workgroup; a K step is KT blocks of 32*WAVES
 // elements, each block split over the WAVES wavefronts; DEPTH K steps are in flight in registers.
@@ -49,9 +71,20 @@ constexpr int WAVES = 4, DEPTH = 2;
 // linears and the SiLU-multiply of the reference's gated MLP (src/cuda/torch_bindings.cpp:703-723,
 // src/cuda/inference_fusion.cuh:19-28) with the same rounding points, without the two
 // activations' round trip through memory and without two of the three launches.
-template <int NT, int MT, int KT, bool GATED>
+//
+// FUSE: the residual-add + RMSNorm that surrounds a decode linear (ref src/cuda/inference_fusion.cuh:136-191:
+// added = round(x + r), scale = rsqrt(mean(added^2) + eps), out = round(round(added * scale) * w)) moved into
+// the linears on either side of it. The linear before the norm adds the residual to its rounded result in
+// the epilogue and leaves per-workgroup sums of squares; the linear after it adds those partial sums in
+// index order, forms the row scales and normalises the tokens on their way from registers to LDS (every
+// workgroup stages all of x anyway). Rounding points are the reference's; the sum of squares is taken
+// in a different (but fixed) order than a row kernel's, so the scale may differ in its last bit.
+// (FUSE: 0 none, 1 the normalised input, 2 the residual epilogue; compile-time, because a branch in
+// the loop keeps the compiler from counting the loads in flight and makes every wait a wait for all)
+template <int NT, int MT, int KT, bool GATED, int FUSE = 0>
 __global__ __launch_bounds__(WAVES * 64) void bgemv_stream_kernel(StreamParams p)
 {
+    constexpr bool NORMALISE = FUSE == 1, RESIDUAL = FUSE == 2 && !GATED;
     static_assert(!GATED || NT % 2 == 0, "gate and up tiles come in pairs");
     constexpr int HALF = GATED ? NT / 2 : NT; // distinct 16-row blocks of output rows
     constexpr int ROWS = HALF * 16, XROWS = MT * 16, CH = 4 * WAVES, BK = 32 * WAVES;
@@ -94,6 +127,7 @@ __global__ __launch_bounds__(WAVES * 64) void bgemv_stream_kernel(StreamParams p
     // flight. A K position past the end (the K tail, or the padding tile of an odd tile count) is
     // read from the last valid chunk instead and zeroed by a mask when it is stored to LDS.
     u32x4_t a_reg[DEPTH][KT][NT], b_reg[DEPTH][KT][MT];
+    u32x4_t norm_reg[DEPTH][NORMALISE ? KT : 1]; // the norm weights of a step's K positions
     // Workgroups start at different K tiles and wrap around: if all of them swept K in lock step
     // the chip would read one column block of every row at a time, a pattern strided by the row
     // pitch that lands on few HBM channels; staggering spreads the requests over all of them.
@@ -105,7 +139,7 @@ __global__ __launch_bounds__(WAVES * 64) void bgemv_stream_kernel(StreamParams p
     // W is read exactly once, so its loads are non-temporal: they bypass the cache allocation that
     // a 470 MB stream would otherwise keep evicting (measured: 5.7 -> 6.3 TB/s); x is re-read by
     // every workgroup and is loaded normally.
-    auto fetch = [&](int step, u32x4_t(&a)[KT][NT], u32x4_t(&b)[KT][MT]) {
+    auto fetch = [&](int step, u32x4_t(&a)[KT][NT], u32x4_t(&b)[KT][MT], u32x4_t(&norm)[NORMALISE ? KT : 1]) {
         // padding steps past the end (their data is masked away) all read one cached line
         const unsigned live = step < k_tiles ? 0xffffffffu : 0u;
         const int tile_k = rotated(step) * (BK * KT) + chunk * 8;
@@ -121,9 +155,25 @@ __global__ __launch_bounds__(WAVES * 64) void bgemv_stream_kernel(StreamParams p
 #pragma unroll
             for (int j = 0; j < MT; ++j)
                 b[t][j] = *reinterpret_cast<const u32x4_t *>(b_base + k0 + (b_off[j] & live));
+            if constexpr (NORMALISE)
+                norm[t] = *reinterpret_cast<const u32x4_t *>(p.norm_weight + k0);
         }
     };
-    auto stash = [&](int stage, int step, const u32x4_t(&a)[KT][NT], const u32x4_t(&b)[KT][MT]) {
+    float scale[MT] = {}; // NORMALISE: the row scales of this thread's tokens
+    auto normalised = [&](u32x4_t values, float row_scale, const u32x4_t &weights) {
+        u32x4_t result;
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+            const unsigned rounded = round_pack_bf16x2(__fmul_rn(__uint_as_float(values[e] << 16), row_scale),
+                                                       __fmul_rn(__uint_as_float(values[e] & 0xffff0000u), row_scale));
+            result[e] = round_pack_bf16x2(
+                __fmul_rn(__uint_as_float(rounded << 16), __uint_as_float(weights[e] << 16)),
+                __fmul_rn(__uint_as_float(rounded & 0xffff0000u), __uint_as_float(weights[e] & 0xffff0000u)));
+        }
+        return result;
+    };
+    auto stash = [&](int stage, int step, const u32x4_t(&a)[KT][NT], const u32x4_t(&b)[KT][MT],
+                     const u32x4_t(&norm)[NORMALISE ? KT : 1]) {
         const int tile_k = rotated(step) * (BK * KT) + chunk * 8;
 #pragma unroll
         for (int t = 0; t < KT; ++t) {
@@ -133,8 +183,12 @@ __global__ __launch_bounds__(WAVES * 64) void bgemv_stream_kernel(StreamParams p
             for (int i = 0; i < NT; ++i)
                 base[i * 16 * CH] = a[t][i] & mask;
 #pragma unroll
-            for (int j = 0; j < MT; ++j)
-                base[(NT + j) * 16 * CH] = b[t][j] & mask;
+            for (int j = 0; j < MT; ++j) {
+                u32x4_t tokens = b[t][j];
+                if constexpr (NORMALISE)
+                    tokens = normalised(tokens, scale[j], norm[t]);
+                base[(NT + j) * 16 * CH] = tokens & mask;
+            }
         }
     };
 
@@ -171,18 +225,44 @@ __global__ __launch_bounds__(WAVES * 64) void bgemv_stream_kernel(StreamParams p
     // loads" and only one tile stays in flight.
 #pragma unroll
     for (int d = 0; d < DEPTH; ++d) {
-        fetch(d, a_reg[d], b_reg[d]);
+        fetch(d, a_reg[d], b_reg[d], norm_reg[d]);
         __builtin_amdgcn_sched_barrier(0);
+    }
+    if constexpr (NORMALISE) {
+        {
+            // Row scales, with the first weight loads already on their way: the workgroup's tokens go
+            // round its threads, PARTS threads per token, each adding a contiguous range of the partial
+            // sums in index order; then the PARTS ranges in order. Fixed for a given count.
+            constexpr int PARTS = WAVES * 64 / XROWS;
+            float *table = reinterpret_cast<float *>(lds_bytes);
+            const int token = thread % XROWS, part = thread / XROWS;
+            const int row = m0 + token < p.m ? m0 + token : p.m - 1;
+            const int per = (p.ssq_count + PARTS - 1) / PARTS;
+            const int last = (part + 1) * per < p.ssq_count ? (part + 1) * per : p.ssq_count;
+            float sum = 0.f;
+            for (int q = part * per; q < last; ++q)
+                sum = __fadd_rn(sum, p.ssq_in[size_t(q) * p.ssq_ld + row]);
+            table[part * XROWS + token] = sum;
+            __syncthreads();
+#pragma unroll
+            for (int j = 0; j < MT; ++j) {
+                float total = table[j * 16 + pass_row];
+                for (int q = 1; q < PARTS; ++q)
+                    total = __fadd_rn(total, table[q * XROWS + j * 16 + pass_row]);
+                scale[j] = rsqrtf(__fadd_rn(total / float(p.k), p.epsilon));
+            }
+            __syncthreads(); // the table lies where the first stage is stashed
+        }
     }
     int stage = 0;
     for (int step = 0; step < k_tiles; step += DEPTH) {
 #pragma unroll
         for (int d = 0; d < DEPTH; ++d) {
             __builtin_amdgcn_sched_barrier(0);
-            stash(stage, step + d, a_reg[d], b_reg[d]);
+            stash(stage, step + d, a_reg[d], b_reg[d], norm_reg[d]);
             __syncthreads();
             __builtin_amdgcn_sched_barrier(0);
-            fetch(step + d + DEPTH, a_reg[d], b_reg[d]);
+            fetch(step + d + DEPTH, a_reg[d], b_reg[d], norm_reg[d]);
             __builtin_amdgcn_sched_barrier(0);
             multiply(stage);
             stage ^= 1;
@@ -253,6 +333,9 @@ __global__ __launch_bounds__(WAVES * 64) void bgemv_stream_kernel(StreamParams p
         if (*flag == 0)
             return;
     }
+    // (residual epilogue: per tile and lane, the squares of the four outputs the lane wrote; behind
+    // the region the wavefronts' sums were parked in, which the launcher sizes for)
+    float *square_table = reinterpret_cast<float *>(lds_bytes + size_t(WAVES) * NT * MT * 64 * 16);
 #pragma unroll
     for (int index = 0; index < HALF * MT; ++index) {
         if (index % WAVES != wave)
@@ -268,6 +351,31 @@ __global__ __launch_bounds__(WAVES * 64) void bgemv_stream_kernel(StreamParams p
                                               unsigned(index) * TILE_BYTES + unsigned(lane) * 16);
         } else {
             sum = summed(index);
+        }
+        if constexpr (RESIDUAL) {
+            {
+                // added = round(round(alpha * product) + residual), and this lane's share of the sums of
+                // squares of the rows of `added` (zero where the tile leaves the matrix)
+                float added[4] = {0.f, 0.f, 0.f, 0.f};
+                if (m < p.m && n < p.n) {
+                    const unsigned short *carried = p.residual + size_t(m) * p.ld_residual + n;
+                    unsigned short *out = p.y + size_t(m) * p.ldc + n;
+#pragma unroll
+                    for (int e = 0; e < 4; ++e)
+                        if (n + e < p.n) {
+                            const float product = bf16_bits_to_float(float_to_bf16_bits(p.alpha * sum[e]));
+                            const unsigned short bits = float_to_bf16_bits(__fadd_rn(product, bf16_bits_to_float(carried[e])));
+                            out[e] = bits;
+                            added[e] = bf16_bits_to_float(bits);
+                        }
+                }
+                float squares = __fmul_rn(added[0], added[0]);
+#pragma unroll
+                for (int e = 1; e < 4; ++e)
+                    squares = __fadd_rn(squares, __fmul_rn(added[e], added[e]));
+                square_table[index * 64 + lane] = squares;
+                continue;
+            }
         }
         if (m >= p.m || n >= p.n)
             continue;
@@ -319,19 +427,37 @@ __global__ __launch_bounds__(WAVES * 64) void bgemv_stream_kernel(StreamParams p
             }
         }
     }
+    if constexpr (RESIDUAL) {
+        {
+            // one thread per token adds the table's entries of that token in a fixed order: feature
+            // tiles ascending, inside a tile the four lane groups (features 0-3, 4-7, ...) ascending
+            __syncthreads();
+            if (thread < XROWS && m0 + thread < p.m) {
+                float total = 0.f;
+#pragma unroll
+                for (int i = 0; i < HALF; ++i)
+#pragma unroll
+                    for (int g = 0; g < 4; ++g)
+                        total = __fadd_rn(total, square_table[(i * MT + thread / 16) * 64 + g * 16 + thread % 16]);
+                p.ssq_out[size_t(blockIdx.x) * p.ssq_ld_out + m0 + thread] = total;
+            }
+        }
+    }
 }
 
-template <int NT, int MT, int KT, bool GATED = false>
+template <int NT, int MT, int KT, bool GATED = false, int FUSE = 0>
 hipError_t launch_one(hipStream_t stream, const StreamParams &p, int shares = 1)
 {
     constexpr size_t stage_bytes = size_t(2) * KT * (NT + MT) * 16 * (64 * WAVES);
-    constexpr size_t parked_bytes = size_t(WAVES) * NT * MT * 64 * 16; // partial sums at the end
+    // partial sums at the end (residual epilogue: and the table of squares behind them)
+    constexpr size_t parked_bytes =
+        size_t(WAVES) * NT * MT * 64 * 16 + (FUSE == 2 && !GATED ? size_t(NT) * MT * 64 * 4 : 0);
     constexpr size_t lds_bytes = stage_bytes > parked_bytes ? stage_bytes : parked_bytes;
     // combined limits: the tiles in flight fit the register file, a stage pair fits the LDS
     if constexpr (NT * KT > 8 || lds_bytes > 128 * 1024) {
         return hipErrorInvalidValue;
     } else {
-        auto kernel = bgemv_stream_kernel<NT, MT, KT, GATED>;
+        auto kernel = bgemv_stream_kernel<NT, MT, KT, GATED, FUSE>;
         static LdsLimitFlags limits; // (one per instantiation)
         const hipError_t status = raise_lds_limit(limits, reinterpret_cast<const void *>(kernel), lds_bytes);
         if (status != hipSuccess)
@@ -349,31 +475,52 @@ hipError_t launch_one(hipStream_t stream, const StreamParams &p, int shares = 1)
     }
 }
 
-template <int MT, int KT>
+template <int MT, int KT, int FUSE>
 hipError_t launch_rows(hipStream_t stream, int row_tiles, const StreamParams &p, int shares)
 {
     switch (row_tiles) {
-    case 1: return launch_one<1, MT, KT>(stream, p, shares);
-    case 2: return launch_one<2, MT, KT>(stream, p, shares);
-    case 3: return launch_one<3, MT, KT>(stream, p, shares);
-    case 4: return launch_one<4, MT, KT>(stream, p, shares);
-    case 5: return launch_one<5, MT, KT>(stream, p, shares);
-    case 6: return launch_one<6, MT, KT>(stream, p, shares);
-    case 7: return launch_one<7, MT, KT>(stream, p, shares);
-    case 8: return launch_one<8, MT, KT>(stream, p, shares);
+    case 1: return launch_one<1, MT, KT, false, FUSE>(stream, p, shares);
+    case 2: return launch_one<2, MT, KT, false, FUSE>(stream, p, shares);
+    case 3: return launch_one<3, MT, KT, false, FUSE>(stream, p, shares);
+    case 4: return launch_one<4, MT, KT, false, FUSE>(stream, p, shares);
+    case 5: return launch_one<5, MT, KT, false, FUSE>(stream, p, shares);
+    case 6: return launch_one<6, MT, KT, false, FUSE>(stream, p, shares);
+    case 7: return launch_one<7, MT, KT, false, FUSE>(stream, p, shares);
+    case 8: return launch_one<8, MT, KT, false, FUSE>(stream, p, shares);
     default: return hipErrorInvalidValue;
     }
 }
 
-template <int KT>
+template <int KT, int FUSE = 0>
 hipError_t launch_tokens(hipStream_t stream, int row_tiles, int token_tiles, const StreamParams &p, int shares)
 {
     switch (token_tiles) {
-    case 1: return launch_rows<1, KT>(stream, row_tiles, p, shares);
-    case 2: return launch_rows<2, KT>(stream, row_tiles, p, shares);
-    case 4: return launch_rows<4, KT>(stream, row_tiles, p, shares);
+    case 1: return launch_rows<1, KT, FUSE>(stream, row_tiles, p, shares);
+    case 2: return launch_rows<2, KT, FUSE>(stream, row_tiles, p, shares);
+    case 4: return launch_rows<4, KT, FUSE>(stream, row_tiles, p, shares);
     default: return hipErrorInvalidValue;
     }
+}
+
+// the fused halves of a launch, checked and copied into the kernel's parameters
+hipError_t apply_fusion(StreamParams &p, const StreamFusion &fusion, int token_tiles)
+{
+    p.norm_weight = static_cast<const unsigned short *>(fusion.norm_weight);
+    p.ssq_in = fusion.ssq_in;
+    p.ssq_count = fusion.ssq_count;
+    p.ssq_ld = fusion.ssq_ld;
+    p.epsilon = fusion.epsilon;
+    p.residual = static_cast<const unsigned short *>(fusion.residual);
+    p.ld_residual = fusion.ld_residual;
+    p.ssq_out = fusion.ssq_out;
+    p.ssq_ld_out = fusion.ssq_ld_out;
+    if (p.norm_weight && (!p.ssq_in || p.ssq_count < 1 || p.ssq_ld < p.m || p.k % 8 ||
+                          reinterpret_cast<uintptr_t>(p.norm_weight) % 16))
+        return hipErrorInvalidValue;
+    if (p.residual && (!p.ssq_out || p.ssq_ld_out < p.m || p.ld_residual < p.n || p.beta != 0.f))
+        return hipErrorInvalidValue;
+    (void)token_tiles;
+    return hipSuccess;
 }
 } // namespace
 
@@ -389,7 +536,7 @@ size_t stream_partial_bytes(int row_tiles, int token_tiles, int n_out, int m_row
 // whole K. pair_tiles 1..4, token_tiles 1, 2 or 4.
 hipError_t launch_gated_stream(hipStream_t stream, int pair_tiles, int token_tiles, int n_out, int m_rows,
                                int k, const void *gate, const void *up, int lda, const void *x, int ldb,
-                               void *y, int ldc)
+                               void *y, int ldc, const StreamFusion &fusion)
 {
     StreamParams p;
     p.w = static_cast<const unsigned short *>(gate);
@@ -411,27 +558,36 @@ hipError_t launch_gated_stream(hipStream_t stream, int pair_tiles, int token_til
     p.arrivals = nullptr;
     if ((m_rows + token_tiles * 16 - 1) / (token_tiles * 16) > 65535)
         return hipErrorInvalidValue;
+    const bool fused = fusion.norm_weight != nullptr;
+    if (fusion.residual)
+        return hipErrorInvalidValue; // the gated form has no residual epilogue
+    const hipError_t admitted = apply_fusion(p, fusion, token_tiles);
+    if (admitted != hipSuccess)
+        return admitted;
+#define CAMBLAS_GATED(NT, MT) \
+    return fused ? launch_one<NT, MT, 1, true, 1>(stream, p) : launch_one<NT, MT, 1, true, 0>(stream, p)
     switch (token_tiles * 10 + pair_tiles) {
-    case 11: return launch_one<2, 1, 1, true>(stream, p);
-    case 12: return launch_one<4, 1, 1, true>(stream, p);
-    case 13: return launch_one<6, 1, 1, true>(stream, p);
-    case 14: return launch_one<8, 1, 1, true>(stream, p);
-    case 21: return launch_one<2, 2, 1, true>(stream, p);
-    case 22: return launch_one<4, 2, 1, true>(stream, p);
-    case 23: return launch_one<6, 2, 1, true>(stream, p);
-    case 24: return launch_one<8, 2, 1, true>(stream, p);
-    case 41: return launch_one<2, 4, 1, true>(stream, p);
-    case 42: return launch_one<4, 4, 1, true>(stream, p);
-    case 43: return launch_one<6, 4, 1, true>(stream, p);
-    case 44: return launch_one<8, 4, 1, true>(stream, p);
+    case 11: CAMBLAS_GATED(2, 1);
+    case 12: CAMBLAS_GATED(4, 1);
+    case 13: CAMBLAS_GATED(6, 1);
+    case 14: CAMBLAS_GATED(8, 1);
+    case 21: CAMBLAS_GATED(2, 2);
+    case 22: CAMBLAS_GATED(4, 2);
+    case 23: CAMBLAS_GATED(6, 2);
+    case 24: CAMBLAS_GATED(8, 2);
+    case 41: CAMBLAS_GATED(2, 4);
+    case 42: CAMBLAS_GATED(4, 4);
+    case 43: CAMBLAS_GATED(6, 4);
+    case 44: CAMBLAS_GATED(8, 4);
     default: return hipErrorInvalidValue;
     }
+#undef CAMBLAS_GATED
 }
 
 hipError_t launch_bgemv_stream(hipStream_t stream, int depth_log2, int row_tiles, int token_tiles, int n_out,
                                int m_rows, int k, float alpha, const void *w, int lda,
                                const void *x, int ldb, float beta, void *y, int ldc,
-                               const BetaSource &source, const StreamShares &shares)
+                               const BetaSource &source, const StreamShares &shares, const StreamFusion &fusion)
 {
     StreamParams p;
     p.w = static_cast<const unsigned short *>(w);
@@ -454,6 +610,25 @@ hipError_t launch_bgemv_stream(hipStream_t stream, int depth_log2, int row_tiles
     p.arrivals = shares.arrivals;
     if ((m_rows + token_tiles * 16 - 1) / (token_tiles * 16) > 65535 || shares.count < 1 || shares.count > 64)
         return hipErrorInvalidValue;
+    const hipError_t admitted = apply_fusion(p, fusion, token_tiles);
+    if (admitted != hipSuccess)
+        return admitted;
+    if (fusion.norm_weight && fusion.residual)
+        return hipErrorInvalidValue; // one half per launch: no linear of a decoder layer needs both
+    if (fusion.norm_weight) { // the fused forms exist for K steps of one or two blocks
+        switch (depth_log2) {
+        case 0: return launch_tokens<1, 1>(stream, row_tiles, token_tiles, p, shares.count);
+        case 1: return launch_tokens<2, 1>(stream, row_tiles, token_tiles, p, shares.count);
+        default: return hipErrorInvalidValue;
+        }
+    }
+    if (fusion.residual) {
+        switch (depth_log2) {
+        case 0: return launch_tokens<1, 2>(stream, row_tiles, token_tiles, p, shares.count);
+        case 1: return launch_tokens<2, 2>(stream, row_tiles, token_tiles, p, shares.count);
+        default: return hipErrorInvalidValue;
+        }
+    }
     switch (depth_log2) {
     case 0: return launch_tokens<1>(stream, row_tiles, token_tiles, p, shares.count);
     case 1: return launch_tokens<2>(stream, row_tiles, token_tiles, p, shares.count);

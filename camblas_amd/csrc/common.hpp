@@ -227,16 +227,35 @@ struct StreamShares {
     unsigned *arrivals = nullptr;
 };
 int undivided_stream_kernel(int outputs, int tokens, int k, int compute_units);
+// The residual-add + RMSNorm around a decode linear, moved into the linears on either side of it.
+// norm_weight (BF16 [k], 16-byte aligned): x is normalised while it is staged, with the row scales
+// rsqrt(sum / k + epsilon), sum = ssq_in[0 * ssq_ld + token] + ssq_in[1 * ssq_ld + token] + ... over
+// ssq_count entries in index order. residual (BF16, ld_residual >= outputs): y = round(round(alpha *
+// x W^T) + residual) (beta must be 0), and every workgroup along the outputs leaves the sums of
+// squares of its features of each row of y in ssq_out[workgroup * ssq_ld_out + token]; the number of
+// such workgroups is stream_workgroups_along_outputs().
+struct StreamFusion {
+    const void *norm_weight = nullptr;
+    const float *ssq_in = nullptr;
+    int ssq_count = 0, ssq_ld = 0;
+    float epsilon = 0.f;
+    const void *residual = nullptr;
+    int ld_residual = 0;
+    float *ssq_out = nullptr;
+    int ssq_ld_out = 0;
+};
+inline int stream_workgroups_along_outputs(int row_tiles, int n_out) { return (n_out + row_tiles * 16 - 1) / (row_tiles * 16); }
 hipError_t launch_bgemv_stream(hipStream_t stream, int depth_log2, int row_tiles, int token_tiles, int n_out,
                                int m_rows, int k, float alpha, const void *w, int lda,
                                const void *x, int ldb, float beta, void *y, int ldc,
-                               const BetaSource &source = {}, const StreamShares &shares = {});
+                               const BetaSource &source = {}, const StreamShares &shares = {},
+                               const StreamFusion &fusion = {});
 // The gated-MLP front end for decode batches in one pass over both weight matrices:
 // y = round(round(silu(g)) * u), g = round(x gate^T), u = round(x up^T). pair_tiles 1..4 (16 output
 // rows each: that many gate rows and the same up rows per workgroup), token_tiles 1, 2 or 4.
 hipError_t launch_gated_stream(hipStream_t stream, int pair_tiles, int token_tiles, int n_out, int m_rows,
                                int k, const void *gate, const void *up, int lda, const void *x, int ldb,
-                               void *y, int ldc);
+                               void *y, int ldc, const StreamFusion &fusion = {});
 hipError_t launch_fp8_block(hipStream_t stream, int variant, int split_k, int rows, int outputs,
                             int inner, const void *a, const float *a_scale, const void *w,
                             const float *w_scale, void *out, float *partials);
@@ -309,6 +328,9 @@ hipError_t launch_swiglu(hipStream_t stream, int dtype, uint64_t count, int widt
 hipError_t launch_rms_rows(hipStream_t stream, int dtype, int weight_dtype, int rows, int width,
                            float epsilon, bool round_before_weight, const void *input,
                            const void *residual, const void *weight, void *added, void *out);
+// added[row] = round(x[row] + residual[row]) (BF16, contiguous rows of `width`), squares[row] = sum of added^2
+hipError_t launch_add_residual_squares(hipStream_t stream, int rows, int width, const void *x, const void *residual,
+                                       void *added, float *squares);
 hipError_t launch_bf16_square(hipStream_t stream, uint64_t count, const void *input, float *out);
 hipError_t launch_rms_scale(hipStream_t stream, int dtype, uint64_t count, int width, float epsilon,
                             const void *input, const void *weight, const float *means, void *out);
@@ -325,8 +347,15 @@ size_t gqa_decode_scratch_bytes(int batch, int q_heads, int dim, int context_len
 // `device` (which must be current; resolved with hipGetSymbolAddress on first use per device).
 size_t gqa_resident_scratch_bytes();
 hipError_t gqa_resident_scratch(int device, void **address);
+// positions (with theta, k_new, v_new) non-null: the step's new token arrives un-rotated, q / k_new /
+// v_new rows q_stride apart per sequence; the kernel rotates q and k_new, attends over positions + 1
+// entries and writes the new K and V rows into the caches (k and v are then written to); lengths unused.
 hipError_t launch_gqa_decode(hipStream_t stream, int batch, int q_heads, int kv_heads, int dim,
                              int context_length, const int32_t *lengths, float scale, const void *q,
                              int q_stride, const void *k, const void *v, void *out, void *partials,
-                             int splits);
+                             int splits, const int32_t *positions = nullptr, float theta = 0.f,
+                             const void *k_new = nullptr, const void *v_new = nullptr, const float *table = nullptr);
+// table[b][0][i] = sin, table[b][1][i] = cos of positions[b] * theta^(-2i/dim) for i < dim / 2
+hipError_t launch_rope_table(hipStream_t stream, int batch, int dim, float theta, const int32_t *positions,
+                             float *table);
 } // namespace camblas_hip

@@ -59,6 +59,28 @@ __device__ __forceinline__ unsigned f32x2_to_e4m3_sat(float first, float second)
     return codes;
 }
 
+// Rotary embedding, rotate-half pairing (i, i + dim/2): angle = position * theta^(-2i/dim) with FP32
+// sine and cosine, one BF16 rounding per element. Shared by every kernel that rotates, so that they
+// agree bit for bit.
+__device__ __forceinline__ void pair_sincos(float position, int i, int dim, float theta, float &s, float &c)
+{
+    float frequency = exp2f(-2.f * float(i) / float(dim) * log2f(theta));
+    float angle = position * frequency;
+    sincosf(angle, &s, &c);
+}
+__device__ __forceinline__ void rotate_by(float s, float c, float lo, float hi, unsigned short &out_lo,
+                                          unsigned short &out_hi)
+{
+    // (written out so that every kernel rounds in the same places whatever the compiler would contract;
+    // the two roundings to BF16 are one conversion instruction of gfx950, round to nearest even)
+    typedef float pair_f32 __attribute__((ext_vector_type(2)));
+    typedef __bf16 pair_bf16 __attribute__((ext_vector_type(2)));
+    const pair_f32 rotated = {__fmaf_rn(lo, c, -__fmul_rn(hi, s)), __fmaf_rn(hi, c, __fmul_rn(lo, s))};
+    const unsigned packed = __builtin_bit_cast(unsigned, __builtin_convertvector(rotated, pair_bf16));
+    out_lo = (unsigned short)(packed & 0xffffu);
+    out_hi = (unsigned short)(packed >> 16);
+}
+
 // Storage traits: T is float, double or bf16_storage (a 16-bit wrapper).
 struct bf16_storage {
     unsigned short bits;

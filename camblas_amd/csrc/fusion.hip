@@ -275,19 +275,6 @@ __global__ void rms_scale_kernel(size_t count, int width, float epsilon, const T
 // ---------------------------------------------------------------- rotary embedding
 // Rotate-half pairing (i, i + dim/2), angle = position * theta^(-2i/dim), FP32 sin/cos, one BF16
 // rounding per element. One thread per (token, head, i).
-__device__ __forceinline__ void pair_sincos(float position, int i, int dim, float theta, float &s, float &c)
-{
-    float frequency = exp2f(-2.f * float(i) / float(dim) * log2f(theta));
-    float angle = position * frequency;
-    sincosf(angle, &s, &c);
-}
-__device__ __forceinline__ void rotate_by(float s, float c, float lo, float hi, unsigned short &out_lo,
-                                          unsigned short &out_hi)
-{
-    // (written out so that every kernel rounds in the same places whatever the compiler would contract)
-    out_lo = float_to_bf16_bits(__fmaf_rn(lo, c, -__fmul_rn(hi, s)));
-    out_hi = float_to_bf16_bits(__fmaf_rn(hi, c, __fmul_rn(lo, s)));
-}
 __device__ __forceinline__ void rotate_pair(float position, int i, int dim, float theta, float lo,
                                             float hi, unsigned short &out_lo, unsigned short &out_hi)
 {
@@ -502,6 +489,42 @@ hipError_t launch_rms_rows(hipStream_t stream, int dtype, int weight_dtype, int 
             static_cast<const bf16_storage *>(residual), static_cast<const float *>(weight),
             static_cast<bf16_storage *>(added), static_cast<bf16_storage *>(out));
     }
+    return launch_status();
+}
+
+namespace
+{
+// One workgroup per row: added = round(x + r), and the row's sum of squares of `added` in a fixed
+// order (a thread's elements ascending, then the threads of a wavefront, then the wavefronts).
+__global__ __launch_bounds__(256) void add_residual_squares_kernel(int width, const unsigned short *x,
+                                                                   const unsigned short *residual,
+                                                                   unsigned short *added, float *squares)
+{
+    __shared__ float partial[4];
+    const size_t base = size_t(blockIdx.x) * width;
+    float sum = 0.f;
+    for (int column = threadIdx.x; column < width; column += 256) {
+        const unsigned short bits = float_to_bf16_bits(
+            __fadd_rn(bf16_bits_to_float(x[base + column]), bf16_bits_to_float(residual[base + column])));
+        added[base + column] = bits;
+        const float value = bf16_bits_to_float(bits);
+        sum = __fadd_rn(sum, __fmul_rn(value, value));
+    }
+    sum = wave_sum(sum);
+    if (threadIdx.x % 64 == 0)
+        partial[threadIdx.x / 64] = sum;
+    __syncthreads();
+    if (threadIdx.x == 0)
+        squares[blockIdx.x] = __fadd_rn(__fadd_rn(partial[0], partial[1]), __fadd_rn(partial[2], partial[3]));
+}
+} // namespace
+
+hipError_t launch_add_residual_squares(hipStream_t stream, int rows, int width, const void *x, const void *residual,
+                                       void *added, float *squares)
+{
+    add_residual_squares_kernel<<<rows, 256, 0, stream>>>(width, static_cast<const unsigned short *>(x),
+                                                          static_cast<const unsigned short *>(residual),
+                                                          static_cast<unsigned short *>(added), squares);
     return launch_status();
 }
 

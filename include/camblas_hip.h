@@ -277,6 +277,60 @@ int camblas_cuda_rope(camblas_cuda_context *context, int tokens, int heads, int 
 int camblas_cuda_bf16_gated_linear(camblas_cuda_context *context, int rows, int outputs, int inner,
                                    const void *x, int ldx, const void *gate, const void *up, int ldw,
                                    void *out, int ldo);
+/* extension (no reference counterpart). camblas_cuda_rope_kv_append and
+ * camblas_cuda_gqa_decode_attention in one call, two launches instead of three: qkv holds the step's
+ * un-rotated activation rows [q heads | k heads | v heads] (token_stride elements apart, a multiple
+ * of 8), positions[b] the cache slot of sequence b's new token. The queries are rotated in registers
+ * by every workgroup that needs them, the new K row is rotated by the workgroup whose positions
+ * hold its slot, which also writes it and the new V row into the caches and attends to them; the
+ * attention covers positions[b] + 1 entries. Output and caches equal the two separate calls bit for
+ * bit (lengths = positions + 1); qkv itself is left unrotated. A position outside [0, context_length)
+ * appends nothing (the attention then covers min(positions + 1, context_length) entries, none if
+ * negative). angles: NULL, or what camblas_cuda_rope_angles made for these positions and theta. */
+int camblas_cuda_rope_append_gqa_decode_attention(camblas_cuda_context *context, int batch, int q_heads,
+                                                  int kv_heads, int dim, int context_length,
+                                                  const int32_t *positions, float theta, float scale,
+                                                  const void *qkv_bf16, int token_stride, void *k_cache,
+                                                  void *v_cache, const float *angles, void *output);
+/* extension (no reference counterpart). The rotation angles of one decode step, which are the same
+ * for every layer of a model: angles[b][0][i] = sin, angles[b][1][i] = cos of positions[b] *
+ * theta^(-2i/dim) for i < dim / 2 (FP32 [batch][2][dim / 2]), exactly the values the rotary kernels
+ * work out themselves. camblas_cuda_rope_append_gqa_decode_attention takes them as `angles` (made with
+ * the same positions and theta; NULL: every workgroup works them out). */
+int camblas_cuda_rope_angles(camblas_cuda_context *context, int batch, int dim, float theta,
+                             const int32_t *positions, float *angles);
+/* extension. The residual-add + RMSNorm between two decode linears, moved into those linears (the
+ * arithmetic and its rounding points are the reference's norm, src/cuda/inference_fusion.cuh:136-191,
+ * binding src/cuda/torch_bindings.cpp:675-701: added = bf16(x + r), scale = rsqrt(mean(added^2) + eps),
+ * out = bf16(bf16(added * scale) * weight)). The linear BEFORE the norm:
+ *   added[tokens, outputs] = bf16(bf16(x w^T) + residual), and for every workgroup g along the outputs
+ *   squares[g * squares_ld + token] = the sum of added^2 over g's outputs (fixed order);
+ *   *squares_count (host) receives the number of such workgroups; it depends on the shape and the
+ *   device only. squares needs room for squares_capacity >= that many rows of squares_ld >= tokens
+ *   floats (ceil(outputs / 16) rows always suffice), else the call is refused.
+ * At most 64 tokens; inner, ldx, ldw multiples of 8; x and w 16-byte aligned. */
+int camblas_cuda_bf16_linear_residual(camblas_cuda_context *context, int tokens, int outputs, int inner,
+                                      const void *x, int ldx, const void *w, int ldw, const void *residual,
+                                      int ld_residual, void *added, int ld_added, float *squares, int squares_ld,
+                                      int squares_capacity, int *squares_count);
+/* extension. The linear AFTER the norm: y = bf16(normalised(x) w^T) where x holds the un-normalised
+ * rows (`added` above), squares [squares_count][squares_ld] their partial sums of squares (added in
+ * index order; mean = sum / inner) and norm_weight the BF16 norm weights [inner], 16-byte aligned. The
+ * tokens are normalised while the kernel stages them, so the normalised rows never exist in memory.
+ * Same shape limits as above. */
+int camblas_cuda_bf16_rms_linear(camblas_cuda_context *context, int tokens, int outputs, int inner, const void *x,
+                                 int ldx, const float *squares, int squares_ld, int squares_count,
+                                 const void *norm_weight, float epsilon, const void *w, int ldw, void *y, int ldy);
+/* extension. camblas_cuda_bf16_gated_linear with the same fused normalisation of its input. */
+int camblas_cuda_bf16_rms_gated_linear(camblas_cuda_context *context, int rows, int outputs, int inner,
+                                       const void *x, int ldx, const float *squares, int squares_ld,
+                                       int squares_count, const void *norm_weight, float epsilon, const void *gate,
+                                       const void *up, int ldw, void *out, int ldo);
+/* extension. The state those calls pass along, made from scratch (a model's first layer): added
+ * [rows, width] = bf16(x + residual), squares[row] = the sum of added^2 over the row (one partial
+ * sum per row: squares_count 1, squares_ld >= rows). BF16, contiguous rows. */
+int camblas_cuda_add_residual_squares(camblas_cuda_context *context, int rows, int width, const void *x,
+                                      const void *residual, void *added, float *squares);
 /* extension (no reference counterpart). Writes each sequence's new K and V heads, rows of k_new /
  * v_new [batch, kv_heads*dim] with row stride token_stride elements (e.g. slices of a fused QKV
  * activation), into the caches [batch, context, kv_heads, dim] at positions[batch]; positions

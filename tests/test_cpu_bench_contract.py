@@ -34,3 +34,18 @@ def test_roofline_object_arithmetic():
     assert bench.roofline_of("mfma bf16", 1.0, 1.0)["peak"] == 2500.0
     assert bench.roofline_of("mfma fp32", 1.0, 1.0)["peak"] == 157.3
     assert bench.roofline_of("mfma fp64", 1.0, 1.0)["peak"] == 78.6
+
+
+def test_roofline_object_carries_the_fraction_of_what_its_instruction_sustains():
+    assert "frac_of_sustained" not in bench.roofline_of("mfma bf16", 2.0e12, 1e-3, "bf16_16x16x32")  # not measured yet
+    bench.SUSTAINED["bf16_16x16x32"] = 2200.0
+    try:
+        found = bench.roofline_of("mfma bf16", 687.19e9, 450e-6, "bf16_16x16x32")
+        assert found["instruction"] == "bf16_16x16x32" and found["sustained"] == 2200.0
+        assert abs(found["frac_of_sustained"] - 687.19e9 / 450e-6 / 1e12 / 2200.0) < 1e-4
+        assert "frac_of_sustained" not in bench.roofline_of("hbm", 1.0, 1.0, None)
+    finally:
+        bench.SUSTAINED.clear()
+    assert bench.bf16_instruction("bf16 wave4-320x256x64s2") == "bf16_16x16x32_one_wavefront_per_simd"
+    assert bench.bf16_instruction("bf16 dma16-128x256x64s3w8 split_k=4") == "bf16_16x16x32"
+    assert bench.bf16_instruction("bf16 dma320x256x64s2w8") == "bf16_32x32x16"
