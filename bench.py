@@ -620,6 +620,16 @@ def layer_step(torch, _kernels, device, normal):
         turn[0] = (turn[0] + 1) % 3
         return _kernels.gqa_decode_attention(q, caches[turn[0]][0], caches[turn[0]][1], lengths)
 
+    # the same step with both residual-add + RMSNorm launches fused into the linears around them: it
+    # takes and returns the state the layers pass along (the added residual stream and its rows'
+    # partial sums of squares)
+    state = _kernels.add_residual_squares(hidden_in, residual)
+
+    def fused_step():
+        return _kernels.decoder_layer_decode_fused(
+            state, weights, k_cache, v_cache, positions, lengths, q_heads=q_heads, kv_heads=kv_heads, head_dim=dim)
+
+    step.fused = fused_step
     return step, attention
 
 
@@ -867,6 +877,7 @@ def extras(torch, _kernels, _native, device, normal):
         return step()
 
     eager = event_time(torch, layer, 10, 50)
+    fused_norms = event_time(torch, lambda i: step.fused(), 10, 50)
     # the same step replayed from a captured graph (capture on a side stream after a warm-up there)
     side = torch.cuda.Stream()
     side.wait_stream(torch.cuda.current_stream())
@@ -894,10 +905,14 @@ def extras(torch, _kernels, _native, device, normal):
     found["llama70b_layer_decode_b32_ctx2048"] = {
         "eager_us": round(eager * 1e6, 1), "graph_us": round(replayed * 1e6, 1),
         "graph_of_8_steps_us_per_step": round(stacked * 1e6, 1),
+        "fused_norms_eager_us": round(fused_norms * 1e6, 1),
         "roofline": roofline_of("hbm", traffic, min(eager, replayed, stacked)),
-        "note": "one layer, 9 library calls; rate from the fastest of stream launches, a one-step graph and an "
-                "eight-step graph (all device-bound); weights not rotated (1.7 GB per layer, beyond the "
-                "256 MB last-level cache)",
+        "note": "one layer, 8 launches (rotary embedding and cache append run inside the attention's first "
+                "kernel); rate from the fastest of stream launches, a one-step graph and an eight-step graph "
+                "(all device-bound); weights not rotated (1.7 GB per layer, beyond the 256 MB last-level "
+                "cache). fused_norms: the 6-launch form with both residual-add + RMSNorm steps inside the "
+                "linears around them, which pays up to 16 tokens and costs time at 32 (every workgroup "
+                "normalises all tokens)",
     }
     return found
 
