@@ -36,6 +36,7 @@ CORE_SOURCES = (
     "bgemm_nn.hip",
     "fp8_block.hip",
     "fp8_dma.hip",
+    "fp8_wave4.hip",
     "fp8_stream.hip",
     "fp8_block32.hip",
     "fp8_moe.hip",
@@ -76,6 +77,9 @@ def build_core(jobs=8, verbose=False):
     """Compile every HIP translation unit for gfx950 and link libcamblas_hip.so."""
     objects = LIB_DIR / "obj"
     objects.mkdir(parents=True, exist_ok=True)
+    # the K loop of fp8_wave4.hip is generated text of more than a megabyte: written here, not kept in
+    # the repository (the smaller loops of bgemm_wave4.hip are kept, and checked against their generator)
+    _run([sys.executable, CSRC / "gen_fp8_wave4_loop.py", "--out", CSRC])
 
     def compile_unit(name):
         source = CSRC / name
@@ -138,6 +142,9 @@ def build_tensor_binding(jobs=4):
     ]
     objects = LIB_DIR / "obj"
     objects.mkdir(parents=True, exist_ok=True)
+    # the K loop of fp8_wave4.hip is generated text of more than a megabyte: written here, not kept in
+    # the repository (the smaller loops of bgemm_wave4.hip are kept, and checked against their generator)
+    _run([sys.executable, CSRC / "gen_fp8_wave4_loop.py", "--out", CSRC])
 
     def compile_unit(name):
         unit = objects / (Path(name).stem + ".binding.o")

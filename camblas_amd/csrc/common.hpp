@@ -265,6 +265,10 @@ hipError_t launch_fp8_block(hipStream_t stream, int variant, int split_k, int ro
 hipError_t launch_fp8_dma(hipStream_t stream, int variant, int split_k, int rows, int outputs, int inner,
                           const void *a, const float *a_scale, const void *w, const float *w_scale,
                           void *out, float *partials, int tail_variant = 0, int tail_outputs = 0);
+// fp8_wave4.hip: the same product on four wavefronts per workgroup (192 x 256 tiles); inner % 1024 == 0,
+// inner >= 2048, undivided K only.
+hipError_t launch_fp8_wave4(hipStream_t stream, int rows, int outputs, int inner, const void *a, const float *a_scale,
+                            const void *w, const float *w_scale, void *out, int out_pitch);
 hipError_t launch_fp8_split_sum(hipStream_t stream, int splits, size_t count, const float *partials, void *out);
 // row_tiles 1..8 (16 weight rows each), token_tiles 1, 2 or 4 (16 tokens each).
 hipError_t launch_fp8_stream(hipStream_t stream, int row_tiles, int token_tiles, int rows, int outputs,

@@ -486,6 +486,8 @@ const TnVariant variants[] = {
     {"fp8dma16-192x128x128s3w8", 192, 128, 128, 512},
     {"fp8dma16-192x256x128w8", 192, 256, 128, 512},
     {"fp8dma16-192x64x128s3w4", 192, 64, 128, 256},
+    // four wavefronts, one per SIMD, K loop in generated assembly (fp8_wave4.hip)
+    {"fp8wave4-192x256x128", 192, 256, 128, 256},
 };
 } // namespace
 
@@ -518,6 +520,10 @@ hipError_t launch_rows(hipStream_t stream, int variant, int splits, const Fp8Dma
     case 13: return launch_one<1, 4, 3, 3, true>(stream, p, splits);
     case 14: return launch_one<2, 4, 2, 3, true>(stream, p, splits);
     case 15: return launch_one<1, 2, 3, 3, true>(stream, p, splits);
+    case 16:
+        if (splits != 1)
+            return hipErrorInvalidValue;
+        return launch_fp8_wave4(stream, p.m, p.n, p.k, p.a, p.a_scale, p.w, p.w_scale, p.out, p.out_pitch);
     default: return hipErrorInvalidValue;
     }
 }

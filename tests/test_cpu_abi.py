@@ -267,3 +267,23 @@ def test_generated_assembly_loops_are_in_step_with_their_generator(tmp_path):
     subprocess.run([sys.executable, str(sources / "gen_wave4_loop.py"), "--out", str(tmp_path)], check=True)
     for name in ("wave4_loop_256x256.inc", "wave4_loop_320x256.inc"):
         assert (tmp_path / name).read_text() == (sources / name).read_text(), name
+
+
+def test_fp8_four_wavefront_loop_generator_writes_whole_steps(tmp_path):
+    # the FP8 loop is generated at build time; its shape is fixed by the tile: three variants (where
+    # the wavefront's rows cross a scale block) x three slabs of eight K groups x 48 tiles, each tile
+    # one matrix instruction and four scaled accumulates, and the same number of barriers per variant
+    import subprocess
+    import sys
+    from pathlib import Path
+
+    sources = Path(__file__).resolve().parents[1] / "camblas_amd" / "csrc"
+    subprocess.run([sys.executable, str(sources / "gen_fp8_wave4_loop.py"), "--out", str(tmp_path)], check=True)
+    text = (tmp_path / "fp8_wave4_loop_192x256.inc").read_text()
+    variants = text.split("asm volatile(")[1:]
+    assert len(variants) == 3
+    for variant in variants:
+        assert variant.count("v_mfma_scale_f32_16x16x128_f8f6f4") == 3 * 8 * 48
+        assert variant.count("v_fmac_f32_e32") == 3 * 8 * 48 * 4
+        assert variant.count("s_barrier") == variants[0].count("s_barrier") == 2 + 3 * 8 - 1
+        assert "v_pk_" not in variant

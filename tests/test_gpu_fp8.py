@@ -125,6 +125,50 @@ def test_direct_lds_loads_with_divided_k_groups(device, code, split, rows, outpu
     assert (np.abs(bf16_values(out) - wanted) <= bound).all()
 
 
+@pytest.mark.parametrize("rows,outputs,inner", [(70, 300, 2048), (513, 452, 3072), (256, 1156, 4096)])
+def test_four_wavefront_tile(device, rows, outputs, inner):
+    # code 36: 192 x 256 tiles on four wavefronts with the K loop in generated assembly; partial tiles
+    # in both directions, a partial last weight-scale block, wavefronts whose 96 rows start at every
+    # offset inside a 128-row scale block (0, 32, 64, 96), two to four slabs of eight K groups.
+    # The chain is the ordered oracle's, so results agree to one BF16 unit.
+    a, a_scale = oracle.fill_fp8_blocks(740 + rows, rows, inner, 1)
+    w, w_scale = oracle.fill_fp8_blocks(741, outputs, inner, 128)
+    out = run(device, a, a_scale, w, w_scale, override=(36, 1))
+    want64 = oracle.fp8_block_matmul_f64(a, a_scale, w, w_scale)
+    assert rel_frobenius(bf16_values(out), want64) <= TOLERANCE
+    ordered = oracle.bf16_to_f32(oracle.fp8_block_matmul(a, a_scale, w, w_scale))
+    bound = 2.0**-7 * np.abs(ordered) + 1e-4 * np.abs(want64).max()
+    assert (np.abs(bf16_values(out) - ordered) <= bound).all()
+
+
+def test_four_wavefront_tile_scale_indexing_is_bit_exact(device):
+    # exact arithmetic (small-integer products, power-of-two scales, distinct per (token, group) and
+    # (block, group)) over 24 K groups = three slabs: a wrong scale index, a wrong slab buffer or a
+    # tile accumulated with the other block's scale changes bits
+    rows, outputs, inner = 300, 836, 24 * 128
+    groups, blocks = inner // 128, (outputs + 127) // 128
+    rng = np.random.default_rng(8)
+    small = np.array([0x00, 0x38, 0x40, 0x30, 0xB8, 0xC0], dtype=np.uint8)  # 0, 1, 2, .5, -1, -2
+    a = small[rng.integers(0, len(small), size=(rows, inner))]
+    w = small[rng.integers(0, len(small), size=(outputs, inner))]
+    a_scale = np.exp2(rng.integers(-5, 5, size=(rows, groups))).astype(np.float32)
+    w_scale = np.exp2(-((np.arange(blocks * groups).reshape(blocks, groups) * 5) % 7)).astype(np.float32)
+    out = run(device, a, a_scale, w, w_scale, override=(36, 1))
+    want = oracle.fp8_block_matmul(a, a_scale, w, w_scale)
+    assert np.array_equal(from_device_bf16(out), want)
+
+
+def test_four_wavefront_tile_matches_the_eight_wavefront_tile_bit_for_bit(device):
+    # the same K positions per lane quarter and the same chain: identical bits at the benchmark's
+    # inner dimension (56 groups = seven slabs), random data
+    rows, outputs, inner = 520, 772, 7168
+    a, a_scale = oracle.fill_fp8_blocks(750, rows, inner, 1)
+    w, w_scale = oracle.fill_fp8_blocks(751, outputs, inner, 128)
+    new = from_device_bf16(run(device, a, a_scale, w, w_scale, override=(36, 1)))
+    old = from_device_bf16(run(device, a, a_scale, w, w_scale, override=(34, 1)))
+    assert np.array_equal(new, old)
+
+
 @pytest.mark.parametrize("rows", [1, 16, 96, 256])
 def test_planned_shapes(device, rows):
     outputs, inner = 1536, 1024
