@@ -691,6 +691,8 @@ int fused_stream_linear(const Entry &entry, int tokens, int outputs, int inner, 
             plan.kernel = undivided_stream_kernel(outputs, tokens, inner, context->compute_units) % 100;
         }
     }
+    if (plan.kernel % 10 == 3) // (the fused forms exist with 1, 2 and 4 token tiles)
+        plan.kernel += 1;
     const int row_tiles = plan.kernel / 10 % 10;
     const int count = stream_workgroups_along_outputs(row_tiles, outputs);
     if (workgroups)

@@ -111,13 +111,20 @@ __global__ __launch_bounds__(WAVES * 64) void bgemv_stream_kernel(StreamParams p
     }
 #pragma unroll
     for (int j = 0; j < MT; ++j) {
-        int row = m0 + j * 16 + pass_row;
-        row = row < p.m ? row : p.m - 1;
-        b_off[j] = unsigned(row - m0) * unsigned(p.ldb);
+        // Byte offset inside the token descriptor below; a row past the end gets an offset outside it,
+        // which reads as zero without a memory request. (Reading an existing row in its place costs:
+        // a line that is requested again while its first request is in flight holds up the vector
+        // cache; [28672, 8192] at 33 tokens in a 48-token tile 106 us with every such lane on the
+        // last row, 96 us on distinct rows, 84 us with 48 real tokens.)
+        const int row = j * 16 + pass_row;
+        b_off[j] = m0 + row < p.m ? unsigned(row) * unsigned(p.ldb) * 2u : 0x80000000u;
     }
     const unsigned short *a_base = p.w + size_t(n0) * p.lda;
     const unsigned short *a2_base = GATED ? p.w2 + size_t(n0) * p.lda : a_base;
-    const unsigned short *b_base = p.x + size_t(m0) * p.ldb;
+    // (the launcher keeps 64 rows of x within 2 GB)
+    const int x_rows = p.m - m0 < XROWS ? p.m - m0 : XROWS;
+    const __amdgpu_buffer_rsrc_t x_resource =
+        make_resource(p.x + size_t(m0) * p.ldb, (unsigned(x_rows - 1) * unsigned(p.ldb) + unsigned(p.k)) * 2u);
     // LDS slot of this thread's chunk inside a 16-row pass; passes are 256 slots apart
     const int store_slot = pass_row * CH + (chunk ^ pass_row);
     static_assert(CH == 16 || CH == 32, "XOR swizzle covers the low four chunk bits");
@@ -154,7 +161,7 @@ __global__ __launch_bounds__(WAVES * 64) void bgemv_stream_kernel(StreamParams p
                     (i < HALF ? a_base : a2_base) + k0 + (a_off[i] & live)));
 #pragma unroll
             for (int j = 0; j < MT; ++j)
-                b[t][j] = *reinterpret_cast<const u32x4_t *>(b_base + k0 + (b_off[j] & live));
+                b[t][j] = __builtin_amdgcn_raw_buffer_load_b128(x_resource, int((b_off[j] & live) + unsigned(k0) * 2u), 0, 0);
             if constexpr (NORMALISE)
                 norm[t] = *reinterpret_cast<const u32x4_t *>(p.norm_weight + k0);
         }
@@ -497,6 +504,11 @@ hipError_t launch_tokens(hipStream_t stream, int row_tiles, int token_tiles, con
     switch (token_tiles) {
     case 1: return launch_rows<1, KT, FUSE>(stream, row_tiles, p, shares);
     case 2: return launch_rows<2, KT, FUSE>(stream, row_tiles, p, shares);
+    case 3: // (33 to 48 tokens; the fused forms keep to 1, 2 and 4 tiles)
+        if constexpr (FUSE == 0)
+            return launch_rows<3, KT, FUSE>(stream, row_tiles, p, shares);
+        else
+            return hipErrorInvalidValue;
     case 4: return launch_rows<4, KT, FUSE>(stream, row_tiles, p, shares);
     default: return hipErrorInvalidValue;
     }
@@ -558,6 +570,9 @@ hipError_t launch_gated_stream(hipStream_t stream, int pair_tiles, int token_til
     p.arrivals = nullptr;
     if ((m_rows + token_tiles * 16 - 1) / (token_tiles * 16) > 65535)
         return hipErrorInvalidValue;
+    // (a workgroup addresses its token rows with 31-bit byte offsets inside one descriptor)
+    if ((size_t(token_tiles * 16 - 1) * size_t(ldb) + size_t(k)) * 2 >= (size_t(1) << 31) || ldb < 1 || k < 1)
+        return hipErrorInvalidValue;
     const bool fused = fusion.norm_weight != nullptr;
     if (fusion.residual)
         return hipErrorInvalidValue; // the gated form has no residual epilogue
@@ -609,6 +624,9 @@ hipError_t launch_bgemv_stream(hipStream_t stream, int depth_log2, int row_tiles
     p.partials = shares.partials;
     p.arrivals = shares.arrivals;
     if ((m_rows + token_tiles * 16 - 1) / (token_tiles * 16) > 65535 || shares.count < 1 || shares.count > 64)
+        return hipErrorInvalidValue;
+    // (a workgroup addresses its token rows with 31-bit byte offsets inside one descriptor)
+    if ((size_t(token_tiles * 16 - 1) * size_t(ldb) + size_t(k)) * 2 >= (size_t(1) << 31) || ldb < 1 || k < 1)
         return hipErrorInvalidValue;
     const hipError_t admitted = apply_fusion(p, fusion, token_tiles);
     if (admitted != hipSuccess)

@@ -60,7 +60,12 @@ __global__ __launch_bounds__(WAVES * 64) void fp8_stream_kernel(Fp8StreamParams 
     const int steps = (p.groups + WAVES - 1) / WAVES; // groups per wavefront, padded
 
     // tile t < NT: weight rows n0 + 16 t ..; tile NT + j: tokens m0 + 16 j ..; half h: rows 8h ..
-    const unsigned char *source[TILES][2];
+    // Token rows are addressed by byte offsets inside a descriptor of the workgroup's existing token
+    // rows; a row past the end gets an offset outside it, which reads as zero without a memory
+    // request (lanes that all read one existing row instead request its lines again while the first
+    // request is in flight, which holds up the vector cache: measured on the BF16 sibling).
+    const unsigned char *source[NT][2];
+    unsigned token_offset[MT][2];
 #pragma unroll
     for (int h = 0; h < 2; ++h) {
 #pragma unroll
@@ -71,11 +76,12 @@ __global__ __launch_bounds__(WAVES * 64) void fp8_stream_kernel(Fp8StreamParams 
         }
 #pragma unroll
         for (int j = 0; j < MT; ++j) {
-            int m = m0 + j * 16 + h * 8 + load_row;
-            m = m < p.m ? m : p.m - 1;
-            source[NT + j][h] = p.a + size_t(m) * p.k + piece * 16;
+            const int m = j * 16 + h * 8 + load_row;
+            token_offset[j][h] = m0 + m < p.m ? unsigned(m) * unsigned(p.k) + unsigned(piece) * 16u : 0x80000000u;
         }
     }
+    const __amdgpu_buffer_rsrc_t token_resource = make_resource(
+        p.a + size_t(m0) * p.k, unsigned(p.m - m0 < MT * 16 ? p.m - m0 : MT * 16) * unsigned(p.k));
     // rows of the scale table: tokens m0 .., then the weight blocks first_block and first_block + 1
     const int first_block = n0 / 128;
     int ws_row[NT], as_row[MT];
@@ -133,8 +139,11 @@ __global__ __launch_bounds__(WAVES * 64) void fp8_stream_kernel(Fp8StreamParams 
         for (int t = 0; t < TILES; ++t)
 #pragma unroll
             for (int h = 0; h < 2; ++h) {
-                const u32x4_t *address = reinterpret_cast<const u32x4_t *>(source[t][h] + offset);
-                data[t][h] = t < NT ? __builtin_nontemporal_load(address) : *address;
+                if (t < NT)
+                    data[t][h] = __builtin_nontemporal_load(reinterpret_cast<const u32x4_t *>(source[t][h] + offset));
+                else
+                    data[t][h] = __builtin_amdgcn_raw_buffer_load_b128(
+                        token_resource, int(token_offset[t < NT ? 0 : t - NT][h] + unsigned(g) * GROUP), 0, 0);
             }
     };
 
@@ -282,6 +291,9 @@ hipError_t launch_fp8_stream(hipStream_t stream, int row_tiles, int token_tiles,
     if (inner % GROUP || inner < GROUP || inner / GROUP > STREAM_SCALE_GROUPS || rows < 1 || outputs < 1)
         return hipErrorInvalidValue;
     if ((rows + token_tiles * 16 - 1) / (token_tiles * 16) > 65535)
+        return hipErrorInvalidValue;
+    // (a workgroup addresses its token rows with 31-bit byte offsets inside one descriptor)
+    if (size_t(token_tiles) * 16 * size_t(inner) >= (size_t(1) << 31))
         return hipErrorInvalidValue;
     Fp8StreamParams p;
     p.w = static_cast<const unsigned char *>(w);

@@ -193,7 +193,8 @@ def step(buffer, split, *, fills, reads, first, last, scale_step):
         # (the results of the last two matrix instructions: more wait states than their latency)
         lines += ["s_nop 15", "s_nop 15"] + accumulate(TILES - 2, split) + accumulate(TILES - 1, split)
     else:
-        lines += ["s_waitcnt vmcnt(0) lgkmcnt(0)"] + ([] if "barrier" in DROP else ["s_barrier"])
+        lines += ["s_waitcnt lgkmcnt(0)" if "fillwait" in DROP else "s_waitcnt vmcnt(0) lgkmcnt(0)"]
+        lines += [] if "barrier" in DROP else ["s_barrier"]
     return lines
 
 
@@ -279,7 +280,7 @@ def statement(split):
 def main():
     parser = argparse.ArgumentParser(description=__doc__.split("\n")[0])
     parser.add_argument("--out", type=Path, default=Path(__file__).resolve().parent)
-    parser.add_argument("--drop", default="", help="experiments: comma list of fills, reads, scales, fmas, barrier")
+    parser.add_argument("--drop", default="", help="experiments: comma list of fills, reads, scales, fmas, barrier, fillwait")
     arguments = parser.parse_args()
     DROP.update(part for part in arguments.drop.split(",") if part)
     text = ["// Generated by gen_fp8_wave4_loop.py; edit the generator, not this file.",

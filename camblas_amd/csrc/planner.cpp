@@ -236,7 +236,7 @@ Plan make_plan(int dtype, int algorithm, bool trans_a, bool trans_b, int m, int 
             // (measured: [12288, 8192] 46-48 vs 55-58 us, [16384, 8192] 58-59 vs 71-74,
             // [12288, 16384] 79-81 vs 100-106) and from 40 tokens at 10240 rows (40-41 vs 43-48)
             plan.family = FAMILY_STREAM;
-            plan.kernel = 10 * std::min(8, ceil_div(2 * ceil_div(outputs, 16), compute_units)) + 4;
+            plan.kernel = 10 * std::min(8, ceil_div(2 * ceil_div(outputs, 16), compute_units)) + (tokens <= 48 ? 3 : 4);
             plan.split_k = 2;
         } else if (tokens <= 64) {
             // 33..64 tokens on a narrow projection: the undivided streaming kernel would have 32-48
@@ -415,7 +415,11 @@ Plan make_plan(int dtype, int algorithm, bool trans_a, bool trans_b, int m, int 
     // tokens go to the tiles when K is long enough to divide: measured at K = 1536 and 2048 the
     // streaming kernel is 35 % faster there, at 7168 and 18432 the tiles are 10 to 35 % faster)
     const bool streamable = k / 128 <= STREAM_SCALE_GROUPS;
-    if (n > 8 && streamable && (n <= 32 || (n <= 64 && (!tiles_apply || k < 4096)))) {
+    // (up to 8 tokens: only when the 16-row tiles alone fill the compute units; narrower projections
+    // keep the small tiles with divided K below. [18432, 7168] at 1 token: 24.2 us in this one launch
+    // against 24.5 in the two launches of the divided product, at 8 tokens 25.1 against 25.5 to 26.6)
+    const bool enough_rows = n > 8 || ceil_div(m, 16) >= compute_units;
+    if (enough_rows && streamable && (n <= 32 || (n <= 64 && (!tiles_apply || k < 4096)))) {
         // decode batches: one streaming pass over the weights, whole K per workgroup; the row
         // tiles are limited by the operand registers (row_tiles * token_tiles <= 16, sum <= 10).
         // From 33 tokens on the 64-token tiles below with divided K are faster (the streaming
@@ -533,7 +537,7 @@ Plan make_plan(int dtype, int algorithm, bool trans_a, bool trans_b, int m, int 
 int undivided_stream_kernel(int outputs, int tokens, int k, int compute_units)
 {
     const int row_tiles = stream_row_tiles(outputs, compute_units);
-    const int token_tiles = tokens <= 16 ? 1 : tokens <= 32 ? 2 : 4;
+    const int token_tiles = tokens <= 16 ? 1 : tokens <= 32 ? 2 : tokens <= 48 ? 3 : 4;
     return 100 * stream_depth_log2(row_tiles, token_tiles, k) + 10 * row_tiles + token_tiles;
 }
 

@@ -112,9 +112,11 @@ def test_planner_choices_for_the_baseline_shapes():
     assert describe(0, "N", "N", 2048, 16, 2048, 2048, 2048, 2048) == (8002, "f32 mfma 128x32x32 split_k=8")
     assert describe(0, "N", "N", 2048, 48, 2048, 2048, 2048, 2048) == (8001, "f32 mfma 128x64x32 split_k=8")
     assert describe(0, "N", "N", 128, 16, 2048, 128, 2048, 128)[0] // 1000 == 0
-    # FP8: split-K tiles for a few tokens, the streaming kernel for decode batches, direct-to-LDS
-    # tiles for prefill
-    assert describe(3, "T", "N", 18432, 1, 7168, 7168, 7168, 18432)[0] // 1000 == 3
+    # FP8: the streaming kernel for decode batches (one launch; up to 8 tokens only where the 16-row
+    # tiles fill the compute units, else small tiles with divided K), direct-to-LDS tiles for prefill
+    code, text = describe(3, "T", "N", 18432, 1, 7168, 7168, 7168, 18432)
+    assert code // 1000 == 7 and "stream rows=80 tokens=16" in text
+    assert describe(3, "T", "N", 2048, 1, 7168, 7168, 7168, 2048)[0] // 1000 == 3
     code, text = describe(3, "T", "N", 18432, 16, 7168, 7168, 7168, 18432)
     assert code // 1000 == 7 and "stream rows=80 tokens=16" in text
     # 33 to 64 tokens: tiles with divided K when K is long enough to divide, else the streaming kernel
