@@ -60,19 +60,19 @@ __global__ __launch_bounds__(WAVES * 64) void fp8_stream_kernel(Fp8StreamParams 
     const int steps = (p.groups + WAVES - 1) / WAVES; // groups per wavefront, padded
 
     // tile t < NT: weight rows n0 + 16 t ..; tile NT + j: tokens m0 + 16 j ..; half h: rows 8h ..
-    // Token rows are addressed by byte offsets inside a descriptor of the workgroup's existing token
-    // rows; a row past the end gets an offset outside it, which reads as zero without a memory
-    // request (lanes that all read one existing row instead request its lines again while the first
-    // request is in flight, which holds up the vector cache: measured on the BF16 sibling).
-    const unsigned char *source[NT][2];
-    unsigned token_offset[MT][2];
+    // Weight and token rows are addressed by byte offsets inside descriptors of the rows that exist
+    // for this workgroup; a row past the end, and every load of a step past the end of K, gets an
+    // offset outside the descriptor, which reads as zero without a memory request. (Reading existing
+    // bytes in their place costs: lanes that all read one existing row request its lines again while
+    // the first request is in flight, which holds up the vector cache, and the re-read last group of
+    // the prefetches beyond the loop came from HBM again: 11 % more bytes than the weights at one token.)
+    unsigned weight_offset[NT][2], token_offset[MT][2];
 #pragma unroll
     for (int h = 0; h < 2; ++h) {
 #pragma unroll
         for (int i = 0; i < NT; ++i) {
-            int n = n0 + i * 16 + h * 8 + load_row;
-            n = n < p.n ? n : p.n - 1;
-            source[i][h] = p.w + size_t(n) * p.k + piece * 16;
+            const int n = i * 16 + h * 8 + load_row;
+            weight_offset[i][h] = n0 + n < p.n ? unsigned(n) * unsigned(p.k) + unsigned(piece) * 16u : 0x80000000u;
         }
 #pragma unroll
         for (int j = 0; j < MT; ++j) {
@@ -80,6 +80,8 @@ __global__ __launch_bounds__(WAVES * 64) void fp8_stream_kernel(Fp8StreamParams 
             token_offset[j][h] = m0 + m < p.m ? unsigned(m) * unsigned(p.k) + unsigned(piece) * 16u : 0x80000000u;
         }
     }
+    const __amdgpu_buffer_rsrc_t weight_resource = make_resource(
+        p.w + size_t(n0) * p.k, unsigned(p.n - n0 < NT * 16 ? p.n - n0 : NT * 16) * unsigned(p.k));
     const __amdgpu_buffer_rsrc_t token_resource = make_resource(
         p.a + size_t(m0) * p.k, unsigned(p.m - m0 < MT * 16 ? p.m - m0 : MT * 16) * unsigned(p.k));
     // rows of the scale table: tokens m0 .., then the weight blocks first_block and first_block + 1
@@ -131,19 +133,22 @@ __global__ __launch_bounds__(WAVES * 64) void fp8_stream_kernel(Fp8StreamParams 
     // step is remembered as a zero factor and applied to the scale when the group is multiplied.
     auto fetch = [&](int step, u32x4_t(&data)[TILES][2], int &group, float &live) {
         int g = group_of(step);
-        live = step < steps && g < p.groups ? 1.f : 0.f;
+        const bool exists = step < steps && g < p.groups;
+        live = exists ? 1.f : 0.f;
         g = g < p.groups ? g : p.groups - 1;
         group = g;
-        const size_t offset = size_t(g) * GROUP;
+        const unsigned offset = unsigned(g) * GROUP, dead = exists ? 0u : 0x80000000u;
 #pragma unroll
         for (int t = 0; t < TILES; ++t)
 #pragma unroll
             for (int h = 0; h < 2; ++h) {
+                // (weights: read once, so non-temporal, cache policy bit 1)
                 if (t < NT)
-                    data[t][h] = __builtin_nontemporal_load(reinterpret_cast<const u32x4_t *>(source[t][h] + offset));
+                    data[t][h] = __builtin_amdgcn_raw_buffer_load_b128(weight_resource,
+                                                                       int((weight_offset[t < NT ? t : 0][h] + offset) | dead), 0, 2);
                 else
                     data[t][h] = __builtin_amdgcn_raw_buffer_load_b128(
-                        token_resource, int(token_offset[t < NT ? 0 : t - NT][h] + unsigned(g) * GROUP), 0, 0);
+                        token_resource, int((token_offset[t < NT ? 0 : t - NT][h] + offset) | dead), 0, 0);
             }
     };
 
@@ -293,7 +298,7 @@ hipError_t launch_fp8_stream(hipStream_t stream, int row_tiles, int token_tiles,
     if ((rows + token_tiles * 16 - 1) / (token_tiles * 16) > 65535)
         return hipErrorInvalidValue;
     // (a workgroup addresses its token rows with 31-bit byte offsets inside one descriptor)
-    if (size_t(token_tiles) * 16 * size_t(inner) >= (size_t(1) << 31))
+    if (size_t(std::max(token_tiles, row_tiles)) * 16 * size_t(inner) >= (size_t(1) << 31))
         return hipErrorInvalidValue;
     Fp8StreamParams p;
     p.w = static_cast<const unsigned char *>(w);
