@@ -114,29 +114,38 @@ __global__ __launch_bounds__(WAVES * 64) void mx_stream_kernel(MxParams p)
     // eight lanes per line, two loads per lane (rows r and r + 8), and transposed to the operand
     // layout through LDS: loading them straight in the operand layout would touch every line from
     // eight quarter-wave passes.
+    // Rows are addressed by byte offsets inside descriptors of the workgroup's existing weight rows
+    // and token rows; a row past the end, and every load of a step past the end of K, gets an offset
+    // outside the descriptor, which reads as zero without a memory request (an existing row read in
+    // its place is requested again while its first request is in flight, which holds up the vector
+    // cache; the re-read last span of the prefetches beyond the loop came from HBM a second time).
     const int load_row = lane / 8, piece = lane % 8;
-    const unsigned char *w_source[NT][2], *ws_source[NT];
+    unsigned w_source[NT][2];
+    const unsigned char *ws_source[NT];
+    const __amdgpu_buffer_rsrc_t weight_resource = make_resource(
+        weight + size_t(n0) * weight_pitch, unsigned(p.outputs - n0 < NT * 16 ? p.outputs - n0 : NT * 16) * unsigned(weight_pitch));
+    const __amdgpu_buffer_rsrc_t input_resource = make_resource(
+        input + size_t(m0) * p.inner, unsigned(valid_rows - m0 < MT * 16 ? valid_rows - m0 : MT * 16) * unsigned(p.inner));
 #pragma unroll
     for (int i = 0; i < NT; ++i) {
 #pragma unroll
         for (int h = 0; h < 2; ++h) {
-            int n = n0 + i * 16 + h * 8 + load_row;
-            n = n < p.outputs ? n : p.outputs - 1;
-            w_source[i][h] = weight + size_t(n) * weight_pitch;
+            const int n = i * 16 + h * 8 + load_row;
+            w_source[i][h] = n0 + n < p.outputs ? unsigned(n) * unsigned(weight_pitch) : 0x80000000u;
         }
         int n = n0 + i * 16 + row;
         n = n < p.outputs ? n : p.outputs - 1;
         // E4M3 weights: one scale per 32 x 32 block; E2M1 weights: one per row and 32 inputs
         ws_source[i] = weight_scale + size_t(PACKED ? n : n / 32) * blocks;
     }
-    const unsigned char *x_source[MT][2], *xs_source[MT];
+    unsigned x_source[MT][2];
+    const unsigned char *xs_source[MT];
 #pragma unroll
     for (int j = 0; j < MT; ++j) {
 #pragma unroll
         for (int h = 0; h < 2; ++h) {
-            int m = m0 + j * 16 + h * 8 + load_row;
-            m = m < valid_rows ? m : valid_rows - 1;
-            x_source[j][h] = input + size_t(m) * p.inner;
+            const int m = j * 16 + h * 8 + load_row;
+            x_source[j][h] = m0 + m < valid_rows ? unsigned(m) * unsigned(p.inner) : 0x80000000u;
         }
         int m = m0 + j * 16 + row;
         m = m < valid_rows ? m : valid_rows - 1;
@@ -168,14 +177,14 @@ __global__ __launch_bounds__(WAVES * 64) void mx_stream_kernel(MxParams p)
         const bool live = step < steps && g < spans;
         g = g < spans ? g : spans - 1;
         // bytes past the end of a row in a partial last span re-read the row's last 16 bytes
-        size_t w_offset = size_t(g) * 128 + piece * 16;
-        w_offset = w_offset < weight_pitch ? w_offset : weight_pitch - 16;
+        const unsigned dead = live ? 0u : 0x80000000u;
+        unsigned w_offset = unsigned(g) * 128u + unsigned(piece) * 16u;
+        w_offset = w_offset < unsigned(weight_pitch) ? w_offset : unsigned(weight_pitch) - 16u;
 #pragma unroll
         for (int i = 0; i < NT; ++i)
 #pragma unroll
-            for (int h = 0; h < 2; ++h)
-                w[i][h] = __builtin_nontemporal_load(
-                    reinterpret_cast<const u32x4_t *>(w_source[i][h] + w_offset));
+            for (int h = 0; h < 2; ++h) // (read once: non-temporal, cache policy bit 1)
+                w[i][h] = __builtin_amdgcn_raw_buffer_load_b128(weight_resource, int((w_source[i][h] + w_offset) | dead), 0, 2);
 #pragma unroll
         for (int s = 0; s < SUB; ++s) {
             const int first = g * STEP_INPUTS + s * GROUP; // first input of the 128-input group
@@ -198,7 +207,7 @@ __global__ __launch_bounds__(WAVES * 64) void mx_stream_kernel(MxParams p)
             for (int j = 0; j < MT; ++j) {
 #pragma unroll
                 for (int h = 0; h < 2; ++h)
-                    x[j][s][h] = *reinterpret_cast<const u32x4_t *>(x_source[j][h] + x_offset);
+                    x[j][s][h] = __builtin_amdgcn_raw_buffer_load_b128(input_resource, int((x_source[j][h] + unsigned(x_offset)) | dead), 0, 0);
                 if constexpr (STAGED)
                     xs[j][s] = unsigned(block >> p.scale_shift); // read from LDS at multiply time
                 else
@@ -385,6 +394,9 @@ hipError_t launch_one(hipStream_t stream, const MxParams &p, int groups)
     if constexpr (NT * MT > 16 || NT + MT * (PACKED ? 2 : 1) > 10) {
         return hipErrorInvalidValue;
     } else {
+        // (a workgroup addresses its weight rows and its token rows with 31-bit byte offsets)
+        if (size_t(NT > MT ? NT : MT) * 16 * size_t(p.inner) >= (size_t(1) << 31))
+            return hipErrorInvalidValue;
         dim3 grid(unsigned((p.outputs + NT * 16 - 1) / (NT * 16)),
                   unsigned((p.rows + MT * 16 - 1) / (MT * 16)), unsigned(groups));
         const int blocks = p.inner / 32;
