@@ -170,7 +170,18 @@ __device__ __forceinline__ void xcd_tile(int block, int tiles_n, int tiles_m, in
     const int total = tiles_n * tiles_m;
     const int per = total / 8, rem = total % 8, xcd = block % 8, local = block / 8;
     const int logical = xcd * per + (xcd < rem ? xcd : rem) + local;
-    constexpr int GROUP = 8;
+    // With few token tiles the weights are streamed once from memory and the token tiles of a feature
+    // tile must meet in one XCD's L2: the group is then the largest one (up to eight feature tiles)
+    // whose spans divide an XCD's range, so that no span straddles two XCDs (192 feature tiles by two
+    // token tiles in spans of 16 put a third of the siblings on different XCDs: 1.33 times the weight
+    // bytes fetched, measured; spans of 12 fit the 24 tiles of an XCD).
+    int GROUP = 8;
+    if (tiles_m > 1 && tiles_m <= 4 && rem == 0)
+        for (int g = 8; g >= 1; --g)
+            if (per % (g * tiles_m) == 0) {
+                GROUP = g;
+                break;
+            }
     const int span = GROUP * tiles_m;
     const int first_n = (logical / span) * GROUP;
     const int group_size = (tiles_n - first_n) < GROUP ? (tiles_n - first_n) : GROUP;
