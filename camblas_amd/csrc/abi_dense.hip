@@ -607,9 +607,20 @@ int bf16_product(const Entry &entry, const Product &p, float alpha, const void *
     camblas_cuda_context *context = entry.context();
     Plan plan = make_plan(2, context->algorithm, p.trans_a, p.trans_b, p.m, p.n, p.k, p.lda, p.ldb, p.ldc,
                           is_aligned(a, 16) && is_aligned(b, 16), context->compute_units);
+    const int forced = context->override_kernel;
+    // W as it lies (the planner's variant 20 for 'N','N'): the other kernels of that family assume
+    // K-contiguous weights, so neither the register-staged substitute nor a forced variant applies;
+    // tests: 60 and 61 ask for the layout-agnostic kernel or the transposing route instead
+    const bool as_it_lies = plan.family == FAMILY_DMA && plan.kernel == 20 && !p.trans_a;
+    if (as_it_lies) {
+        if (!is_aligned(c, 8) || !is_aligned(source.z, 8) || source.ldz % 4 || forced == 60 || forced == 61)
+            plan = make_plan(2, context->algorithm, p.trans_a, p.trans_b, p.m, p.n, p.k, p.lda, p.ldb, p.ldc, false,
+                             context->compute_units);
+        else
+            return launch_bf16_plan(entry, plan, p, alpha, a, b, beta, c, source, nullptr);
+    }
     if (plan.family == FAMILY_DMA && (!is_aligned(c, 8) || !is_aligned(source.z, 8) || source.ldz % 4))
         use_register_staged_tiles(plan); // register-staged loads, scalar stores
-    const int forced = context->override_kernel;
     // Tokens stored the other way round (K rows of tokens) and few of them: copying them transposed
     // costs next to nothing, and the product then runs on the kernels for few tokens instead of the
     // layout-agnostic tiles or, below 32 tokens, the vector-ALU kernel ([8192, 28672] x 16 tokens:

@@ -594,6 +594,8 @@ const TnVariant variants[] = {
     {"dma16-256x128x64s3w8", 256, 128, 64, 512}, {"dma16-128x128x64s3w4", 128, 128, 64, 256},
     // four wavefronts, one per SIMD, K loop in assembly (bgemm_wave4.hip); K % 128 == 0
     {"wave4-256x256x64s2", 256, 256, 64, 256}, {"wave4-320x256x64s2", 320, 256, 64, 256},
+    // the 256 x 256 tile for weights W[K, N] with the outputs contiguous ('N','N': w and lda describe W as it lies)
+    {"wave4-256x256x64s2-weights-as-they-lie", 256, 256, 64, 256},
 };
 } // namespace
 
@@ -680,6 +682,7 @@ hipError_t launch_bgemm_dma(hipStream_t stream, int variant, int n_out, int m_ro
     case 17: return launch_dma16<2, 2, 2, 64, 3>(stream, p, shares);
     case 18: return launch_bgemm_wave4(stream, 256, p, shares);
     case 19: return launch_bgemm_wave4(stream, 320, p, shares);
+    case 20: return launch_bgemm_wave4(stream, 256, p, shares, true);
     default: return hipErrorInvalidValue;
     }
 }

@@ -38,11 +38,26 @@ DROP = set()
 NB = 8  # token tiles of 16 per wavefront: 128 tokens, two wavefronts across = 256
 
 
+NN_PIECE = 1056  # bytes from one 1 KB piece of an as-it-lies weight tile to the next (see Layout)
+
+
 class Layout:
-    def __init__(self, na):
+    """na: 16-row weight tiles per wavefront. nn: the weights lie the other way round, K rows of
+    contiguous outputs (x @ W with a row-major W). A K step of such a tile is 64 rows of 512 bytes;
+    a direct-to-LDS load brings rows k and k + 4 (1 KB), pieces are placed 1056 bytes apart, and a lane
+    gathers its eight K values of one output with two ds_read_b64_tr_b16: within sixteen lanes, lane
+    4a + b receives element b of the four values at the addresses of lanes a, 4 + a, 8 + a, 12 + a,
+    so lane s points at row s / 4 of a four-row group, outputs 4 (s % 4) .. + 3, and receives four
+    K values of output s. The four rows of a group lie in four different pieces and the second group
+    of a 32-lane half (rows + 8) in four more: eight 32-byte runs in eight different bank windows."""
+
+    def __init__(self, na, nn=False):
         self.na = na
+        self.nn = nn
         self.rows = 32 * na  # weight rows of the workgroup tile (two wavefronts down)
-        self.stage_bytes = (self.rows + 256) * 128
+        assert not nn or na == 8, "a K row of 256 outputs is half a 1 KB load"
+        self.a_bytes = 32 * NN_PIECE if nn else self.rows * 128
+        self.stage_bytes = self.a_bytes + 256 * 128
         self.frag = 4 * (na + NB)  # registers of one fragment buffer
         self.buffers = (0, self.frag)
         # accumulators beyond a0..a255 live in architectural registers behind the fragment buffers
@@ -65,13 +80,14 @@ class Layout:
         return f"v[{index}:{index + 3}]"
 
 
-SAVED_M0, OFFSET, FILL1 = "s84", "s85", "s86"
+SAVED_M0, OFFSET, FILL1, FILL1B = "s84", "s85", "s86", "s87"
 
 
-def fill_units(layout, target):
+def fill_units(layout, target, target_b=None):
     """Per direct-to-LDS load: (scalar set-up placed before a matrix instruction, the load after it).
     M0 walks this wavefront's LDS slots in 4 KB strides through the weight rows and on into the
-    token rows; the row advance of successive loads is the scalar offset."""
+    token rows; the row advance of successive loads is the scalar offset. (As-it-lies weights: the
+    wavefront's pieces are four pieces, 4224 bytes, apart, and the token rows start at target_b.)"""
     units = []
     for n in range(layout.na + NB):
         weights = n < layout.na
@@ -79,7 +95,12 @@ def fill_units(layout, target):
         second = n == 1 or n == layout.na + 1
         lane, resource, step = (("%[a_off]", "%[rsrc_a]", "%[a_step]") if weights
                                 else ("%[b_off]", "%[rsrc_b]", "%[b_step]"))
-        before = [f"s_mov_b32 m0, {target}" if n == 0 else "s_add_u32 m0, m0, 0x1000"]
+        if n == 0:
+            before = [f"s_mov_b32 m0, {target}"]
+        elif layout.nn and n == layout.na:
+            before = [f"s_mov_b32 m0, {target_b}"]
+        else:
+            before = [f"s_add_u32 m0, m0, {4 * NN_PIECE:#x}" if layout.nn and weights else "s_add_u32 m0, m0, 0x1000"]
         if second:
             before.append(f"s_mov_b32 {OFFSET}, {step}")
         elif not first:
@@ -103,7 +124,11 @@ def fill_units(layout, target):
     return units
 
 
-ADVANCE = ["v_add_u32_e32 %[a_off], 0x80, %[a_off]", "v_add_u32_e32 %[b_off], 0x80, %[b_off]"]
+def advance(layout):
+    """The fills' per-lane offsets move on by one K step: 64 elements along a K-contiguous row, 64 rows
+    of an as-it-lies weight matrix."""
+    weights = "v_add_u32_e32 %[a_off], %[a_kstep], %[a_off]" if layout.nn else "v_add_u32_e32 %[a_off], 0x80, %[a_off]"
+    return [weights, "v_add_u32_e32 %[b_off], 0x80, %[b_off]"]
 
 
 def reads(layout, stage, sub_step, buffer):
@@ -117,7 +142,15 @@ def reads(layout, stage, sub_step, buffer):
     lines = []
     for i in range(layout.na):
         r = layout.a_frag(buffer, i)
-        lines.append(f"ds_read_b128 v[{r}:{r + 3}], {a_address} offset:{i * 2048}")
+        if layout.nn:
+            # K values 8 q .. + 3 and + 4 .. + 7 of the sub-step for lane group q: rows four apart are the
+            # two halves of a piece, a sub-step is sixteen pieces, the next sixteen outputs 32 bytes on
+            address = "%[ra0]" if stage == 0 else f"v{layout.scratch_v}"
+            offset = sub_step * 16 * NN_PIECE + i * 32
+            lines.append(f"ds_read_b64_tr_b16 v[{r}:{r + 1}], {address} offset:{offset}")
+            lines.append(f"ds_read_b64_tr_b16 v[{r + 2}:{r + 3}], {address} offset:{offset + 512}")
+        else:
+            lines.append(f"ds_read_b128 v[{r}:{r + 3}], {a_address} offset:{i * 2048}")
     for j in range(NB):
         r = layout.b_frag(buffer, j)
         lines.append(f"ds_read_b128 v[{r}:{r + 3}], {b_address} offset:{j * 2048}")
@@ -167,7 +200,8 @@ def phase(layout, buffer, read_lines, fills, zero=False, advance=False, read_eve
     lines = []
     count = layout.na * NB
     fills = fills or []
-    assert len(fills) <= (count + FILL_EVERY - 1) // FILL_EVERY and len(read_lines) * read_every <= count
+    assert len(fills) <= (count + FILL_EVERY - 1) // FILL_EVERY and len(read_lines) * read_every <= count, (
+        len(fills), len(read_lines), read_every, count)
     for k, (i, j) in enumerate(tile_order(layout)):
         unit = fills[k // FILL_EVERY] if k % FILL_EVERY == 0 and k // FILL_EVERY < len(fills) else None
         if unit:
@@ -180,15 +214,15 @@ def phase(layout, buffer, read_lines, fills, zero=False, advance=False, read_eve
         if unit:
             lines.append(unit[1])
             if advance and unit is fills[-1]:
-                lines += ADVANCE
+                lines += globals()["advance"](layout)
         if k % read_every == read_every - 1 and k // read_every < len(read_lines):
             line = read_lines[k // read_every]
             lines.append(queue.issue(line) if queue else line)
     return lines
 
 
-def k_step(layout, stage, fill_target):
-    fills = fill_units(layout, fill_target) if fill_target else []
+def k_step(layout, stage, fill_target, fill_target_b=None):
+    fills = fill_units(layout, fill_target, fill_target_b) if fill_target else []
     count = layout.na * NB
     first = min(len(fills), (count + FILL_EVERY - 1) // FILL_EVERY)
     lines = [f"; K step in stage {stage}" + (f", fills into {fill_target}" if fill_target else ", no fills")]
@@ -224,17 +258,19 @@ def program(layout):
         f"v_add_u32_e32 v{v + 3}, {layout.stage_bytes:#x}, %[rb1]",
         "; K step 0 into stage 0",
     ]
-    for before, load in fill_units(layout, "%[fill0]"):
+    if layout.nn:
+        lines.insert(2, f"s_add_u32 {FILL1B}, %[fill0b], {layout.stage_bytes:#x}")
+    for before, load in fill_units(layout, "%[fill0]", "%[fill0b]"):
         lines += before + ["s_nop 0", load]
-    lines += ADVANCE + ["s_waitcnt vmcnt(0)", "s_barrier", "; K step 1 into stage 1, first fragments of step 0"]
-    for before, load in fill_units(layout, FILL1):
+    lines += advance(layout) + ["s_waitcnt vmcnt(0)", "s_barrier", "; K step 1 into stage 1, first fragments of step 0"]
+    for before, load in fill_units(layout, FILL1, FILL1B):
         lines += before + ["s_nop 0", load]
-    lines += ADVANCE + reads(layout, 0, 0, 0) + ["s_waitcnt lgkmcnt(0)"]
+    lines += advance(layout) + reads(layout, 0, 0, 0) + ["s_waitcnt lgkmcnt(0)"]
     lines += phase(layout, 0, reads(layout, 0, 1, 1), None, zero=True)
     lines += ["s_waitcnt vmcnt(0) lgkmcnt(0)", "s_barrier",
               "s_cmp_eq_u32 %[pairs], 0", "s_cbranch_scc1 L_wave4_last%=", "L_wave4_loop%=:"]
-    lines += k_step(layout, 1, "%[fill0]")
-    lines += k_step(layout, 0, FILL1)
+    lines += k_step(layout, 1, "%[fill0]", "%[fill0b]")
+    lines += k_step(layout, 0, FILL1, FILL1B)
     lines += ["s_sub_u32 %[pairs], %[pairs], 1", "s_cmp_lg_u32 %[pairs], 0", "s_cbranch_scc1 L_wave4_loop%=",
               "L_wave4_last%=:"]
     lines += k_step(layout, 1, None)
@@ -262,7 +298,9 @@ def statement(layout):
     inputs = ['[ra0] "v"(read_a0)', '[ra1] "v"(read_a1)', '[rb0] "v"(read_b0)', '[rb1] "v"(read_b1)',
               '[rsrc_a] "s"(a_resource)', '[rsrc_b] "s"(b_resource)', '[a_step] "s"(a_row_step)',
               '[b_step] "s"(b_row_step)', '[fill0] "s"(fill_base)']
-    clobbers = ['"memory"', '"scc"', f'"{SAVED_M0}"', f'"{OFFSET}"', f'"{FILL1}"']
+    if layout.nn:
+        inputs += ['[fill0b] "s"(fill_base_b)', '[a_kstep] "s"(a_k_step)']
+    clobbers = ['"memory"', '"scc"', f'"{SAVED_M0}"', f'"{OFFSET}"', f'"{FILL1}"', f'"{FILL1B}"']
     named = [n for n in range(layout.clobbered_v)
              if not layout.extra_acc_base <= n < layout.extra_acc_base + layout.extra_acc]
     clobbers += [f'"v{n}"' for n in named]
@@ -301,6 +339,8 @@ def main():
             DROP.difference_update(experiments)
         layout = Layout(na)
         (arguments.out / f"wave4_loop_{layout.rows}x256.inc").write_text(statement(layout))
+    if not experiments:
+        (arguments.out / "wave4_loop_256x256_nn.inc").write_text(statement(Layout(8, nn=True)))
 
 
 if __name__ == "__main__":

@@ -191,6 +191,23 @@ Plan make_plan(int dtype, int algorithm, bool trans_a, bool trans_b, int m, int 
                 }
             return plan;
         }
+        // x @ W with a row-major W and many tokens: the four-wavefront 256 x 256 tile that copies W into
+        // LDS as it lies and transposes on the way to the registers, where its tiles fill at least nine
+        // tenths of the rounds of workgroups they make; other shapes are better served by a transposed
+        // copy of W and the tile the 'T','N' planner picks for it (measured, this kernel against the copy
+        // route: 8192^3 757 against 799 us, 8192 x 4096 x 4096 200 against 217, 4096^3 125 against 129;
+        // 4096 x 8192 x 10240, 2.5 rounds, 511 against 503 with the 320-row tile).
+        if (algorithm != CAMBLAS_CUDA_CLASSICAL && !trans_a && !trans_b && k % 128 == 0 && k >= 256 && m % 4 == 0 &&
+            lda % 8 == 0 && ldb % 8 == 0 && ldc % 4 == 0 && aligned16 && double(k) * lda * 2 < 4294967296.0 &&
+            (256.0 * ldb + k) * 2 < 4294967296.0) {
+            const int tiles = ceil_div(m, 256) * ceil_div(n, 256);
+            if (tiles * 10 >= ceil_div(tiles, compute_units) * compute_units * 9) {
+                plan.family = FAMILY_DMA;
+                plan.kernel = 20;
+                plan.counter = 4;
+                return plan;
+            }
+        }
         if (!matrix_path) {
             // the other layouts (and 'T','N' operands the K-contiguous kernels cannot take): the
             // layout-agnostic matrix-core kernel unless the product is a sliver, tiles chosen as for

@@ -267,7 +267,7 @@ def test_generated_assembly_loops_are_in_step_with_their_generator(tmp_path):
 
     sources = Path(__file__).resolve().parents[1] / "camblas_amd" / "csrc"
     subprocess.run([sys.executable, str(sources / "gen_wave4_loop.py"), "--out", str(tmp_path)], check=True)
-    for name in ("wave4_loop_256x256.inc", "wave4_loop_320x256.inc"):
+    for name in ("wave4_loop_256x256.inc", "wave4_loop_320x256.inc", "wave4_loop_256x256_nn.inc"):
         assert (tmp_path / name).read_text() == (sources / name).read_text(), name
 
 

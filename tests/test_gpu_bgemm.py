@@ -342,6 +342,32 @@ def test_large_product_of_another_layout_agrees_with_the_layout_agnostic_kernel(
     assert rel_frobenius(oracle.bf16_to_f32(routed).reshape(n, m)[:, rows], want) <= TOLERANCE
 
 
+@pytest.mark.parametrize("m,n,k,pad", [(4096, 4096, 256, 0), (3976, 3850, 640, 8)])
+def test_weights_as_they_lie_on_the_four_wavefront_tile(device, m, n, k, pad):
+    # x @ W with a row-major W and enough tokens that 256 x 256 tiles fill the chip: the planner sends it
+    # to the four-wavefront tile that copies W into LDS as it lies and gathers K through transposing LDS
+    # reads. Ragged edges in both directions, padded leading dimensions, alpha and beta; checked against
+    # the transposing route (a transposed copy of W, then the linear-layer tiles: the same products in
+    # the same K order, so the same bits) and, on sampled outputs, against FP64.
+    lda, ldb, ldc = m + pad, k + pad, m + (pad and 4)
+    text = _native.plan_describe(2, "N", "N", m, n, k, lda, ldb, ldc)[1]
+    assert "weights-as-they-lie" in text, text
+    a = oracle.fill_normal_bf16(111, (lda * k,))
+    b = oracle.fill_normal_bf16(112, (ldb * n,))
+    c0 = oracle.fill_normal_bf16(113, (ldc * n,))
+    for alpha, beta in ((1.0, 0.0), (0.75, -0.5)):
+        got = run_bgemm(device, "N", "N", m, n, k, alpha, a, lda, b, ldb, beta, c0, ldc)
+        routed = run_bgemm(device, "N", "N", m, n, k, alpha, a, lda, b, ldb, beta, c0, ldc, override=(61, 0))
+        assert np.array_equal(got, routed)
+        got2d = got.reshape(n, ldc)
+        assert np.array_equal(got2d[:, m:], c0.reshape(n, ldc)[:, m:])
+        rows = np.concatenate([np.arange(0, m, 211), [m - 1]])
+        a2 = oracle.bf16_to_f32(a).reshape(k, lda)[:, rows].astype(np.float64)
+        b2 = oracle.bf16_to_f32(b).reshape(n, ldb)[:, :k].astype(np.float64)
+        want = alpha * (b2 @ a2) + beta * oracle.bf16_to_f32(c0).reshape(n, ldc)[:, rows].astype(np.float64)
+        assert rel_frobenius(oracle.bf16_to_f32(got2d[:, rows]), want) <= TOLERANCE
+
+
 def test_layout_agnostic_kernel_counts_as_a_library_product(device):
     # row-major torch.mm(x, w) with a contiguous [in, out] weight arrives as 'N','N'
     native = _native.context(device)
