@@ -667,17 +667,21 @@ def extras(torch, _kernels, _native, device, normal):
         "note": "[outputs] bias row of a linear layer, read by the product's epilogue",
     }
     del x, w, y, c, row
-    # BF16 product with neither operand K-contiguous (row-major a @ b, 'N','N'): the layout-agnostic
-    # matrix-core kernel
-    size = 4096
-    x, w = normal((size, size)), normal((size, size), 0.02)
-    y = torch.empty((size, size), dtype=torch.bfloat16, device=device)
-    seconds = event_time(torch, lambda i: _kernels.matmul(x, w, out=y), 10, 30)
-    found["bf16_matmul_nn_4096"] = {
-        "us": round(seconds * 1e6, 1),
-        "roofline": roofline_of("mfma bf16", 2.0 * size**3, seconds, bf16_instruction(
-            _native.plan_describe(2, "T", "N", size, size, size, size, size, size)[1]))}
-    del x, w, y
+    # BF16 products of square operands: row-major a @ b with neither operand K-contiguous ('N','N': W is
+    # copied into LDS as it lies) at 4096^3, and the linear layout ('T','N') and 'N','N' at 8192^3, whose
+    # 256 x 256 tiles make four whole rounds of workgroups
+    for size in (4096, 8192):
+        x, w = normal((size, size)), normal((size, size), 0.02)
+        y = torch.empty((size, size), dtype=torch.bfloat16, device=device)
+        layouts = (("nn", lambda i: _kernels.matmul(x, w, out=y), "N"),) + (
+            (("tn", lambda i: _kernels.matmul(x, w.t(), out=y), "T"),) if size == 8192 else ())
+        for name, launch, trans_a in layouts:
+            seconds = event_time(torch, launch, 10, 30)
+            plan_text = _native.plan_describe(2, trans_a, "N", size, size, size, size, size, size)[1]
+            found[f"bf16_matmul_{name}_{size}"] = {
+                "us": round(seconds * 1e6, 1), "tflops": round(2.0 * size**3 / seconds / 1e12, 1), "plan": plan_text,
+                "roofline": roofline_of("mfma bf16", 2.0 * size**3, seconds, bf16_instruction(plan_text))}
+        del x, w, y
     # BF16 linear at 256 tokens on a square projection (64 tiles of 128 x 256 for 256 compute units:
     # K is divided over workgroups); five weight copies rotate so that the weights come from HBM
     outputs, inner, tokens = 8192, 8192, 256
