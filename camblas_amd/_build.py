@@ -42,6 +42,7 @@ CORE_SOURCES = (
     "fp8_moe.hip",
     "mx_matmul.hip",
     "mx_dma.hip",
+    "mx_wave4.hip",
     "routing.hip", "dense_ops.hip", "sgemm_mfma.hip", "dgemm_mfma.hip", "strassen.hip",
     "fusion.hip",
     "attention_decode.hip",
@@ -77,9 +78,10 @@ def build_core(jobs=8, verbose=False):
     """Compile every HIP translation unit for gfx950 and link libcamblas_hip.so."""
     objects = LIB_DIR / "obj"
     objects.mkdir(parents=True, exist_ok=True)
-    # the K loop of fp8_wave4.hip is generated text of more than a megabyte: written here, not kept in
+    # the K loops of fp8_wave4.hip and mx_wave4.hip are generated text of a megabyte and more: written here, not kept in
     # the repository (the smaller loops of bgemm_wave4.hip are kept, and checked against their generator)
     _run([sys.executable, CSRC / "gen_fp8_wave4_loop.py", "--out", CSRC])
+    _run([sys.executable, CSRC / "gen_mx_wave4_loop.py", "--out", CSRC])
 
     def compile_unit(name):
         source = CSRC / name
@@ -142,9 +144,10 @@ def build_tensor_binding(jobs=4):
     ]
     objects = LIB_DIR / "obj"
     objects.mkdir(parents=True, exist_ok=True)
-    # the K loop of fp8_wave4.hip is generated text of more than a megabyte: written here, not kept in
+    # the K loops of fp8_wave4.hip and mx_wave4.hip are generated text of a megabyte and more: written here, not kept in
     # the repository (the smaller loops of bgemm_wave4.hip are kept, and checked against their generator)
     _run([sys.executable, CSRC / "gen_fp8_wave4_loop.py", "--out", CSRC])
+    _run([sys.executable, CSRC / "gen_mx_wave4_loop.py", "--out", CSRC])
 
     def compile_unit(name):
         unit = objects / (Path(name).stem + ".binding.o")

@@ -597,7 +597,7 @@ hipError_t launch_variant(hipStream_t stream, const MxDmaParams &p, int groups, 
 }
 } // namespace
 
-int mx_dma_variant_count() { return 4; }
+int mx_dma_variant_count() { return 5; } // (4: the four-wavefront tile of mx_wave4.hip)
 
 // The prefill kernel's conditions: K a multiple of 128, 16-byte aligned operands, an 8-byte aligned
 // output (scale pointers may have any alignment).
@@ -618,8 +618,16 @@ hipError_t launch_mx_dma_rows(hipStream_t stream, int variant, bool packed, int 
                               int count, int inner, int activation_block, const void *input,
                               const void *input_scale, const void *weight, const void *weight_scale, void *out)
 {
-    MxDmaParams p;
     const size_t scale_pitch = size_t(inner / 32), weight_pitch = packed ? size_t(inner) / 2 : size_t(inner);
+    if (variant == 4) { // four wavefronts per workgroup, K loop in generated assembly
+        if (packed || activation_block != 32)
+            return hipErrorInvalidValue;
+        return launch_mx_wave4(stream, rows, count, inner, input, input_scale,
+                               static_cast<const unsigned char *>(weight) + size_t(first) * weight_pitch,
+                               static_cast<const unsigned char *>(weight_scale) + size_t(first / 32) * scale_pitch,
+                               static_cast<unsigned short *>(out) + first, outputs);
+    }
+    MxDmaParams p;
     p.input = static_cast<const unsigned char *>(input);
     p.input_scale = static_cast<const unsigned char *>(input_scale);
     p.weight = static_cast<const unsigned char *>(weight) + size_t(first) * weight_pitch;
@@ -670,6 +678,12 @@ hipError_t launch_mx_dma(hipStream_t stream, int variant, bool packed, int group
             return status;
         return launch_mx_dma_rows(stream, tail_variant, packed, rows, outputs, first, tail_outputs, inner,
                                   activation_block, input, input_scale, weight, weight_scale, out);
+    }
+    if (variant == 4) {
+        if (groups != 0 || shares != 1)
+            return hipErrorInvalidValue;
+        return launch_mx_dma_rows(stream, variant, packed, rows, outputs, 0, outputs, inner, activation_block, input,
+                                  input_scale, weight, weight_scale, out);
     }
     MxDmaParams p;
     p.input = static_cast<const unsigned char *>(input);

@@ -469,9 +469,11 @@ struct MxTilePrice {
     double step_us, kilobytes_in_flight;
     int outputs, rows;
 };
-const MxTilePrice mx_prices[2][4] = {
-    {{1.60, 64, 256, 256}, {1.00, 96, 256, 128}, {1.35, 56, 192, 256}, {0.58, 64, 128, 128}},
-    {{1.60, 96, 256, 256}, {1.00, 64, 256, 128}, {1e30, 1, 192, 256}, {0.58, 48, 128, 128}},
+// (variant 4: the four-wavefront 192 x 256 tile of mx_wave4.hip, unpacked weights and undivided K only;
+// [18432, 7168] at 4096 rows 403 us against 450 for the best plan of the other tiles, at 2048 rows 213 against 237)
+const MxTilePrice mx_prices[2][5] = {
+    {{1.60, 64, 256, 256}, {1.00, 96, 256, 128}, {1.35, 56, 192, 256}, {0.58, 64, 128, 128}, {1.20, 112, 192, 256}},
+    {{1.60, 96, 256, 256}, {1.00, 64, 256, 128}, {1e30, 1, 192, 256}, {0.58, 48, 128, 128}, {1e30, 1, 192, 256}},
 };
 
 // Estimated microseconds of one launch (as for the BF16 tiles: rounds of workgroups times steps
@@ -498,17 +500,23 @@ double mx_launch_us(const MxTilePrice &price, bool packed, long long batches, in
     return us;
 }
 
-MxTilePlan mx_tile_plan(int compute_units, bool packed, int groups, int rows, int outputs, int inner)
+// four_wavefronts: the call meets what the four-wavefront tile needs beyond the other tiles (see
+// mx_four_wavefront_tile_applies)
+MxTilePlan mx_tile_plan(int compute_units, bool packed, int groups, int rows, int outputs, int inner,
+                        bool four_wavefronts = false)
 {
     MxTilePlan plan;
     const long long batches = groups > 0 ? groups : 1;
-    const MxTilePrice(&prices)[4] = mx_prices[packed ? 1 : 0];
+    const MxTilePrice(&prices)[5] = mx_prices[packed ? 1 : 0];
     double best = 1e300;
     const int counts[] = {1, 2, 3, 4, 6, 8};
-    for (int variant = 0; variant < 4; ++variant) {
-        if (prices[variant].step_us > 1e29 || (prices[variant].rows > 128 && rows <= 128))
+    for (int variant = 0; variant < 5; ++variant) {
+        if (prices[variant].step_us > 1e29 || (prices[variant].rows > 128 && rows <= 128) ||
+            (variant == 4 && !(four_wavefronts && groups == 0)))
             continue;
         for (const int shares : counts) {
+            if (variant == 4 && shares > 1)
+                continue;
             // a share has at least eight steps, the planes at most 256 MB; grouped products are not divided
             if (shares > 1 && (groups > 0 || inner / 128 / shares < 8 ||
                                double(shares) * rows * outputs * 4 > double(1 << 28)))
@@ -553,6 +561,15 @@ MxTilePlan mx_tile_plan(int compute_units, bool packed, int groups, int rows, in
 // when the streaming kernel could not hold the scale bytes of 32 tokens in its LDS table and would
 // gather them a byte per lane and step ([7168, 18432] x 32 rows: 34 us against 24 at 16 rows and 26 on
 // the tiles).
+// What the four-wavefront tile needs beyond mx_dma_supported: the plain product of unpacked weights, a scale
+// per 32 inputs, whole slabs of eight 128-input groups (at least two), scale rows it can copy 16 and 4 bytes at a time.
+static bool mx_four_wavefront_tile_applies(bool packed, int groups, int inner, int activation_block,
+                                           const void *input_scale, const void *weight_scale)
+{
+    return !packed && groups == 0 && activation_block == 32 && inner % 1024 == 0 && inner >= 2048 &&
+           reinterpret_cast<uintptr_t>(input_scale) % 16 == 0 && reinterpret_cast<uintptr_t>(weight_scale) % 4 == 0;
+}
+
 static bool mx_rows_take_tiles(int rows, int inner, int activation_block)
 {
     return rows > 32 || (rows > 16 && 32 * (inner / activation_block) + 3 > STAGED_TOKEN_BYTES);
@@ -591,7 +608,9 @@ hipError_t launch_mx_matmul(hipStream_t stream, int kernel, int compute_units, b
                              planes);
     if (kernel < 0 && mx_rows_take_tiles(rows, inner, activation_block) &&
         mx_dma_supported(outputs, inner, input, checked_weight, out)) {
-        MxTilePlan plan = mx_tile_plan(compute_units, packed, groups, rows, outputs, inner);
+        MxTilePlan plan = mx_tile_plan(compute_units, packed, groups, rows, outputs, inner,
+                                       mx_four_wavefront_tile_applies(packed, groups, inner, activation_block, input_scale,
+                                                                      weight_scale));
         if (plan.shares > 1 && !planes) // no room for the planes: the same tile with K undivided
             plan.shares = 1;
         return launch_mx_dma(stream, plan.variant, packed, groups, weight_groups, rows, outputs, inner,

@@ -1,0 +1,147 @@
+// E8M0 block-scaled prefill product (E4M3 inputs with one scale byte per 32 inputs, E4M3 weights with
+// one scale byte per 32 x 32 block, BF16 out; contract: ref include/camblas_cuda.h:110-123,
+// src/cuda/backend.cu:1165-1191, value semantics tests/test_quantized.py:12-50 of the reference) on four
+// wavefronts per workgroup, one per SIMD: a workgroup owns 192 weight rows x 256 tokens, a wavefront
+// 96 x 128 = 6 x 8 tiles of v_mfma_scale_f32_16x16x128_f8f6f4 with the hardware applying both scales.
+// Against the eight-wavefront tiles of mx_dma.hip a wavefront reads each weight fragment from LDS once
+// per eight and each token fragment once per six matrix instructions, holds the fragments of two whole
+// K groups in the accumulation registers, and shares its SIMD's issue with nobody.
+//
+// The K loop is one inline-assembly statement with every register named, written by
+// gen_mx_wave4_loop.py into mx_wave4_loop_192x256.inc at build time (its header describes the
+// registers and the scale handling; the tile, fills and slabs are those of fp8_wave4.hip). Around it
+// this file is ordinary HIP.
+// Shape requirements: the plain product (no groups), unpacked E4M3 weights, one input scale per 32
+// inputs, K a multiple of 1024 and at least 2048, both scale pointers 4-byte aligned, outputs % 4 == 0.
+#include "common.hpp"
+#include "device.hpp"
+#include "dma.hpp"
+
+namespace camblas_hip
+{
+namespace
+{
+struct MxWave4Params {
+    const unsigned char *w, *a, *w_scale, *a_scale;
+    unsigned short *out;
+    int n, m, k, groups, block_rows, out_pitch, tiles_n, tiles_m;
+};
+
+constexpr int NA = 6, NB = 8, BN = 32 * NA, BM = 256, CH = 8;
+constexpr int STAGE_BYTES = (BN + BM) * 128, A_SLAB = 2 * STAGE_BYTES, W_SLAB = A_SLAB + 16384;
+constexpr int LDS_BYTES = W_SLAB + 512;
+
+__global__ __launch_bounds__(256) void mx_wave4_kernel(MxWave4Params p)
+{
+    // two stages of operands; two 8 KB buffers of token scale words [256 tokens][8 groups] 8 KB apart;
+    // two 256-byte buffers of weight scale words [8 block rows][8 groups]. The loop switches between the
+    // two buffers of a slab by flipping one address bit, which needs the array at LDS address 0 (it is
+    // the only LDS object of the kernel).
+    __shared__ u32x4_t lds[LDS_BYTES / 16];
+
+    int tile_n, tile_m;
+    xcd_tile(int(blockIdx.x), p.tiles_n, p.tiles_m, tile_n, tile_m);
+    const int n0 = tile_n * BN, m0 = tile_m * BM;
+    const int thread = threadIdx.x, lane = thread % 64;
+    const int wave = __builtin_amdgcn_readfirstlane(thread / 64);
+    const int wn = wave % 2, wm = wave / 2;
+
+    // ---- fills: wave instruction (it, wave) fills LDS slots [(it*4 + wave)*64, +64) of a stage with
+    // rows (it*4 + wave)*8 + lane/8, 16-byte chunk lane%8 holding logical chunk (lane%8) ^ swizzle(row);
+    // weight rows first, token rows behind them. Rows past the end of a matrix are outside the
+    // descriptor and read as zero.
+    const int load_row = wave * 8 + lane / CH;
+    unsigned a_offset = unsigned(load_row) * unsigned(p.k) + unsigned(((lane % CH) ^ lds_swizzle<CH>(load_row)) * 16);
+    unsigned b_offset = a_offset;
+    const unsigned row_step = __builtin_amdgcn_readfirstlane(32u * unsigned(p.k));
+    const int a_rows = p.n - n0 < BN ? p.n - n0 : BN, b_rows = p.m - m0 < BM ? p.m - m0 : BM;
+    const u32x4_t a_resource = uniform_descriptor(p.w + size_t(n0) * p.k, unsigned(a_rows) * unsigned(p.k));
+    const u32x4_t b_resource = uniform_descriptor(p.a + size_t(m0) * p.k, unsigned(b_rows) * unsigned(p.k));
+    const unsigned lds_base = static_cast<unsigned>(reinterpret_cast<uintptr_t>(lds));
+    const unsigned fill_base = __builtin_amdgcn_readfirstlane(lds_base + unsigned(wave) * 1024u);
+
+    // ---- scale slabs: the four scale bytes of a row and K group are one word. Token words: wavefront w
+    // copies pieces 2w and 2w + 1 of a slab (32 tokens each): lane l brings groups 4 (l % 2) .. + 3 of
+    // token l / 2 of the piece, 16 bytes, so that the piece lands as [token][8 groups]. Tokens that do
+    // not exist read as zero. Weight words: lane l of one 4-byte load brings group l % 8 of block row
+    // l / 8 from the tile's first 32-row block row (the tile's 192 rows are six of them).
+    const u32x4_t a_scale_resource =
+        uniform_descriptor(p.a_scale + size_t(m0) * p.groups * 4, unsigned(b_rows) * unsigned(p.groups) * 4u);
+    const unsigned slab_offset = (unsigned(wave * 64 + lane / 2) * unsigned(p.groups) + unsigned(lane % 2) * 4u) * 4u;
+    const unsigned slab_rows = __builtin_amdgcn_readfirstlane(32u * unsigned(p.groups) * 4u);
+    const unsigned slab_fill = __builtin_amdgcn_readfirstlane(lds_base + unsigned(A_SLAB) + unsigned(wave) * 2048u);
+    const int first_block = n0 / 32;
+    const int blocks = p.block_rows - first_block < 8 ? p.block_rows - first_block : 8;
+    const u32x4_t w_scale_resource = uniform_descriptor(p.w_scale + size_t(first_block) * p.groups * 4,
+                                                        unsigned(blocks) * unsigned(p.groups) * 4u);
+    const unsigned weight_slab_offset = (unsigned(lane / 8) * unsigned(p.groups) + unsigned(lane % 8)) * 4u;
+    const unsigned weight_slab_fill = __builtin_amdgcn_readfirstlane(lds_base + unsigned(W_SLAB));
+    unsigned slab_k = 0; // byte offset of the next slab along a row of scale words
+    unsigned middle_slabs = __builtin_amdgcn_readfirstlane(unsigned(p.groups / 8 - 2));
+
+    // ---- reads. Lane l holds row l % 16 of a 16-row tile and, of its 128 K positions, 16 c .. + 15 and
+    // 64 + 16 c .. + 15 with c = l / 16, and supplies the scale byte of inputs 32 c .. 32 c + 31: byte c
+    // of the row's word. Its eight tokens' words are 512 bytes apart in a slab.
+    const int frag_row = lane % 16, quarter = lane / 16;
+    const int frag_swizzle = lds_swizzle<CH>(frag_row);
+    const int wave_row = n0 + wn * NA * 16; // first weight row of the wavefront
+    const unsigned a_row_bytes = unsigned(wn * NA * 16 + frag_row) * 128u;
+    const unsigned b_row_bytes = unsigned(BN + wm * NB * 16 + frag_row) * 128u;
+    const unsigned read_a_lo = lds_base + a_row_bytes + unsigned(quarter ^ frag_swizzle) * 16u;
+    const unsigned read_a_hi = lds_base + a_row_bytes + unsigned((4 + quarter) ^ frag_swizzle) * 16u;
+    const unsigned read_b_lo = lds_base + b_row_bytes + unsigned(quarter ^ frag_swizzle) * 16u;
+    const unsigned read_b_hi = lds_base + b_row_bytes + unsigned((4 + quarter) ^ frag_swizzle) * 16u;
+    unsigned scale_address = lds_base + unsigned(A_SLAB) + unsigned(wm * NB * 16 + frag_row) * 32u + unsigned(quarter);
+    unsigned weight_scale_address = lds_base + unsigned(W_SLAB) + unsigned(wave_row / 32 - first_block) * 32u + unsigned(quarter);
+
+    // accumulator tile (i, j) (weight rows 16 i .., tokens 16 j ..) comes back as accs[8 i + j]
+    f32x4_t accs[NA * NB];
+#include "mx_wave4_loop_192x256.inc"
+
+    // ---- epilogue. Register e of lane l in tile (i, j) is feature 16 i + 4 (l / 16) + e, token 16 j + l % 16.
+#pragma unroll
+    for (int j = 0; j < NB; ++j) {
+        const int m = m0 + wm * NB * 16 + j * 16 + frag_row;
+#pragma unroll
+        for (int i = 0; i < NA; ++i) {
+            const int n = wave_row + i * 16 + quarter * 4;
+            const f32x4_t v = accs[NB * i + j];
+            if (m < p.m && n < p.n)
+                *reinterpret_cast<u32x2_t *>(p.out + size_t(m) * p.out_pitch + n) =
+                    u32x2_t{pack_bf16x2(v[0], v[1]), pack_bf16x2(v[2], v[3])};
+        }
+    }
+}
+} // namespace
+
+// `outputs` weight rows from `weight` on (scale rows from weight_scale on), written at `out` with `out_pitch`
+// elements between tokens.
+hipError_t launch_mx_wave4(hipStream_t stream, int rows, int outputs, int inner, const void *input,
+                           const void *input_scale, const void *weight, const void *weight_scale, void *out, int out_pitch)
+{
+    const auto misaligned = [](const void *pointer, uintptr_t to) { return reinterpret_cast<uintptr_t>(pointer) % to != 0; };
+    if (rows < 1 || outputs < 1 || outputs % 4 || out_pitch % 4 || inner % 1024 || inner < 2048 || misaligned(out, 8) ||
+        misaligned(input, 16) || misaligned(weight, 16) || misaligned(input_scale, 16) || misaligned(weight_scale, 4))
+        return hipErrorInvalidValue;
+    if (size_t(256) * size_t(inner) >= (size_t(1) << 32))
+        return hipErrorInvalidValue;
+    MxWave4Params p;
+    p.w = static_cast<const unsigned char *>(weight);
+    p.a = static_cast<const unsigned char *>(input);
+    p.w_scale = static_cast<const unsigned char *>(weight_scale);
+    p.a_scale = static_cast<const unsigned char *>(input_scale);
+    p.out = static_cast<unsigned short *>(out);
+    p.n = outputs;
+    p.m = rows;
+    p.k = inner;
+    p.groups = inner / 128;
+    p.block_rows = (outputs + 31) / 32;
+    p.out_pitch = out_pitch;
+    p.tiles_n = (outputs + BN - 1) / BN;
+    p.tiles_m = (rows + BM - 1) / BM;
+    if (size_t(p.tiles_n) * size_t(p.tiles_m) > 0x7fffffffu)
+        return hipErrorInvalidValue;
+    mx_wave4_kernel<<<unsigned(p.tiles_n) * unsigned(p.tiles_m), 256, 0, stream>>>(p);
+    return launch_status();
+}
+} // namespace camblas_hip

@@ -15,7 +15,8 @@ from helpers import bf16_values
 
 pytestmark = pytest.mark.gpu
 
-KERNELS = {"auto": -1, "stream": 0, "tile256x256": 20, "tile256x128": 21, "tile192x256": 22, "tile128x128": 23}
+KERNELS = {"auto": -1, "stream": 0, "tile256x256": 20, "tile256x128": 21, "tile192x256": 22, "tile128x128": 23,
+           "wave4-192x256": 24}
 
 
 def operands(seed, rows, outputs, inner, packed, block):
@@ -115,6 +116,50 @@ def test_exact_products_with_every_scale_alignment(device, kernel, packed, block
     assert np.abs(want).max() < 2.0 ** 24 and (want * 64 == np.round(want * 64)).all()
     want = oracle.bf16_to_f32(oracle.f32_to_bf16(want.astype(np.float32)))
     assert np.array_equal(got, want)
+
+
+@pytest.mark.parametrize("rows,outputs,inner", [(70, 296, 2048), (513, 456, 3072), (300, 840, 4096)])
+def test_four_wavefront_tile_random_operands(device, rows, outputs, inner):
+    # 192 x 256 tiles on four wavefronts with the K loop in generated assembly (E4M3 weights, a scale per 32
+    # inputs): partial tiles in both directions, a partial last 32-row scale block, two to four slabs of
+    # eight K groups, operands and scales mutated one at a time
+    x, sx, weight, sw = operands(950 + rows, rows, outputs, inner, False, 32)
+    for changed in ("original", "input", "weight", "input_scale", "weight_scale"):
+        if changed == "input":
+            x ^= 128
+        elif changed == "weight":
+            weight ^= 128
+            weight[(weight & 0x7F) == 0x7F] = 0x38  # keep the weights finite
+        elif changed == "input_scale":
+            sx -= 1
+        elif changed == "weight_scale":
+            sw += 1
+        close(run(device, x, sx, weight, sw, False, 32, "wave4-192x256"), x, sx, weight, sw, False, 32)
+
+
+def test_four_wavefront_tile_exact_products(device):
+    # exact arithmetic as in test_exact_products_with_every_scale_alignment over 24 K groups (three slabs):
+    # a scale byte of the wrong block, row, group or slab buffer changes the bits; and the eight-wavefront
+    # tile must give the same bits on random operands at the benchmark's inner dimension
+    rows, outputs, inner = 300, 840, 24 * 128
+    rng = np.random.default_rng(77)
+    levels = np.array([0x00, 0x30, 0x38, 0x40, 0xB0, 0xB8, 0xC0], np.uint8)
+    x = levels[rng.integers(0, len(levels), (rows, inner))]
+    weight = levels[rng.integers(0, len(levels), (outputs, inner))]
+    sx = rng.integers(125, 130, (rows, inner // 32), dtype=np.uint8)
+    sw = rng.integers(125, 130, ((outputs + 31) // 32, inner // 32), dtype=np.uint8)
+    got = run(device, x, sx, weight, sw, False, 32, "wave4-192x256")
+    want = oracle.mx_matmul_f64(x, sx, weight, sw, 32, False)
+    assert np.abs(want).max() < 2.0 ** 24 and (want * 64 == np.round(want * 64)).all()
+    assert np.array_equal(got, oracle.bf16_to_f32(oracle.f32_to_bf16(want.astype(np.float32))))
+
+
+def test_four_wavefront_tile_refuses_what_it_cannot_run(device):
+    # packed weights, a scale per 128 inputs, an inner dimension that is not whole slabs of eight groups
+    for packed, block, inner in ((True, 32, 2048), (True, 128, 2048), (False, 32, 1152)):
+        x, sx, weight, sw = operands(5, 64, 256, inner, packed, block)
+        with pytest.raises(RuntimeError):
+            run(device, x, sx, weight, sw, packed, block, "wave4-192x256")
 
 
 @pytest.mark.parametrize("kernel,packed,block", [f for f in FORMATS if f[0] != "auto"])
