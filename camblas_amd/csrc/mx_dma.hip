@@ -620,11 +620,11 @@ hipError_t launch_mx_dma_rows(hipStream_t stream, int variant, bool packed, int 
 {
     const size_t scale_pitch = size_t(inner / 32), weight_pitch = packed ? size_t(inner) / 2 : size_t(inner);
     if (variant == 4) { // four wavefronts per workgroup, K loop in generated assembly
-        if (packed || activation_block != 32)
+        if (activation_block != 32)
             return hipErrorInvalidValue;
-        return launch_mx_wave4(stream, rows, count, inner, input, input_scale,
+        return launch_mx_wave4(stream, packed, rows, count, inner, input, input_scale,
                                static_cast<const unsigned char *>(weight) + size_t(first) * weight_pitch,
-                               static_cast<const unsigned char *>(weight_scale) + size_t(first / 32) * scale_pitch,
+                               static_cast<const unsigned char *>(weight_scale) + size_t(packed ? first : first / 32) * scale_pitch,
                                static_cast<unsigned short *>(out) + first, outputs);
     }
     MxDmaParams p;

@@ -469,11 +469,12 @@ struct MxTilePrice {
     double step_us, kilobytes_in_flight;
     int outputs, rows;
 };
-// (variant 4: the four-wavefront 192 x 256 tile of mx_wave4.hip, unpacked weights and undivided K only;
-// [18432, 7168] at 4096 rows 403 us against 450 for the best plan of the other tiles, at 2048 rows 213 against 237)
+// (variant 4: the four-wavefront 192 x 256 tile of mx_wave4.hip, undivided K only; [18432, 7168] at 4096 rows
+// 403 us against 450 for the best plan of the other tiles (E2M1 weights: 379 against 435), at 2048 rows 213
+// against 237 (189 against 225), at 512 rows even (61 against 79))
 const MxTilePrice mx_prices[2][5] = {
     {{1.60, 64, 256, 256}, {1.00, 96, 256, 128}, {1.35, 56, 192, 256}, {0.58, 64, 128, 128}, {1.20, 112, 192, 256}},
-    {{1.60, 96, 256, 256}, {1.00, 64, 256, 128}, {1e30, 1, 192, 256}, {0.58, 48, 128, 128}, {1e30, 1, 192, 256}},
+    {{1.60, 96, 256, 256}, {1.00, 64, 256, 128}, {1e30, 1, 192, 256}, {0.58, 48, 128, 128}, {1.13, 88, 192, 256}},
 };
 
 // Estimated microseconds of one launch (as for the BF16 tiles: rounds of workgroups times steps
@@ -561,13 +562,15 @@ MxTilePlan mx_tile_plan(int compute_units, bool packed, int groups, int rows, in
 // when the streaming kernel could not hold the scale bytes of 32 tokens in its LDS table and would
 // gather them a byte per lane and step ([7168, 18432] x 32 rows: 34 us against 24 at 16 rows and 26 on
 // the tiles).
-// What the four-wavefront tile needs beyond mx_dma_supported: the plain product of unpacked weights, a scale
-// per 32 inputs, whole slabs of eight 128-input groups (at least two), scale rows it can copy 16 and 4 bytes at a time.
+// What the four-wavefront tile needs beyond mx_dma_supported: the plain product, a scale per 32 inputs, whole
+// slabs of eight 128-input groups (at least two), scale rows it can copy 16 bytes at a time (the block rows of
+// unpacked weights: 4).
 static bool mx_four_wavefront_tile_applies(bool packed, int groups, int inner, int activation_block,
                                            const void *input_scale, const void *weight_scale)
 {
-    return !packed && groups == 0 && activation_block == 32 && inner % 1024 == 0 && inner >= 2048 &&
-           reinterpret_cast<uintptr_t>(input_scale) % 16 == 0 && reinterpret_cast<uintptr_t>(weight_scale) % 4 == 0;
+    return groups == 0 && activation_block == 32 && inner % 1024 == 0 && inner >= 2048 &&
+           reinterpret_cast<uintptr_t>(input_scale) % 16 == 0 &&
+           reinterpret_cast<uintptr_t>(weight_scale) % (packed ? 16 : 4) == 0;
 }
 
 static bool mx_rows_take_tiles(int rows, int inner, int activation_block)

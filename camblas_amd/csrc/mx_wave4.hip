@@ -1,5 +1,6 @@
-// E8M0 block-scaled prefill product (E4M3 inputs with one scale byte per 32 inputs, E4M3 weights with
-// one scale byte per 32 x 32 block, BF16 out; contract: ref include/camblas_cuda.h:110-123,
+// E8M0 block-scaled prefill product (E4M3 inputs with one scale byte per 32 inputs; E4M3 weights with
+// one scale byte per 32 x 32 block, or packed E2M1 weights with one scale byte per row and 32 inputs;
+// BF16 out; contract: ref include/camblas_cuda.h:110-123,
 // src/cuda/backend.cu:1165-1191, value semantics tests/test_quantized.py:12-50 of the reference) on four
 // wavefronts per workgroup, one per SIMD: a workgroup owns 192 weight rows x 256 tokens, a wavefront
 // 96 x 128 = 6 x 8 tiles of v_mfma_scale_f32_16x16x128_f8f6f4 with the hardware applying both scales.
@@ -8,11 +9,12 @@
 // K groups in the accumulation registers, and shares its SIMD's issue with nobody.
 //
 // The K loop is one inline-assembly statement with every register named, written by
-// gen_mx_wave4_loop.py into mx_wave4_loop_192x256.inc at build time (its header describes the
+// gen_mx_wave4_loop.py into mx_wave4_loop_192x256*.inc at build time (its header describes the
 // registers and the scale handling; the tile, fills and slabs are those of fp8_wave4.hip). Around it
 // this file is ordinary HIP.
-// Shape requirements: the plain product (no groups), unpacked E4M3 weights, one input scale per 32
-// inputs, K a multiple of 1024 and at least 2048, both scale pointers 4-byte aligned, outputs % 4 == 0.
+// Shape requirements: the plain product (no groups), one input scale per 32 inputs, K a multiple of 1024
+// and at least 2048, scale rows the slab loads can copy (input scales 16-byte aligned; weight scales
+// 4-byte aligned for E4M3 weights, 16-byte for E2M1), outputs % 4 == 0.
 #include "common.hpp"
 #include "device.hpp"
 #include "dma.hpp"
@@ -28,15 +30,18 @@ struct MxWave4Params {
 };
 
 constexpr int NA = 6, NB = 8, BN = 32 * NA, BM = 256, CH = 8;
-constexpr int STAGE_BYTES = (BN + BM) * 128, A_SLAB = 2 * STAGE_BYTES, W_SLAB = A_SLAB + 16384;
-constexpr int LDS_BYTES = W_SLAB + 512;
 
-__global__ __launch_bounds__(256) void mx_wave4_kernel(MxWave4Params p)
+template <bool PACKED> __global__ __launch_bounds__(256) void mx_wave4_kernel(MxWave4Params p)
 {
-    // two stages of operands; two 8 KB buffers of token scale words [256 tokens][8 groups] 8 KB apart;
-    // two 256-byte buffers of weight scale words [8 block rows][8 groups]. The loop switches between the
-    // two buffers of a slab by flipping one address bit, which needs the array at LDS address 0 (it is
-    // the only LDS object of the kernel).
+    // Two stages of operands (weight rows of 128 bytes, or 64 when packed, then token rows); two 8 KB
+    // buffers of token scale words [256 tokens][8 groups] 8 KB apart; the weights' scale words likewise
+    // (E2M1: a word per row) or as two 256-byte buffers [8 block rows][8 groups] (E4M3). The loop switches
+    // between the two buffers of a slab by flipping one address bit, so the slabs start where that bit is
+    // clear, and the array lies at LDS address 0 (it is the only LDS object of the kernel).
+    constexpr int A_ROW = PACKED ? 64 : 128, A_BYTES = BN * A_ROW, STAGE_BYTES = A_BYTES + BM * 128;
+    constexpr int A_SLAB = PACKED ? 0x18000 : 2 * STAGE_BYTES, W_SLAB = A_SLAB + 0x4000;
+    constexpr int LDS_BYTES = W_SLAB + (PACKED ? 0x4000 : 512);
+    static_assert(2 * STAGE_BYTES <= A_SLAB && A_SLAB % 0x4000 == 0 && W_SLAB % 0x4000 == 0, "slab addresses");
     __shared__ u32x4_t lds[LDS_BYTES / 16];
 
     int tile_n, tile_m;
@@ -45,26 +50,34 @@ __global__ __launch_bounds__(256) void mx_wave4_kernel(MxWave4Params p)
     const int thread = threadIdx.x, lane = thread % 64;
     const int wave = __builtin_amdgcn_readfirstlane(thread / 64);
     const int wn = wave % 2, wm = wave / 2;
+    const unsigned pitch = PACKED ? unsigned(p.k) / 2u : unsigned(p.k); // bytes of a weight row
 
-    // ---- fills: wave instruction (it, wave) fills LDS slots [(it*4 + wave)*64, +64) of a stage with
-    // rows (it*4 + wave)*8 + lane/8, 16-byte chunk lane%8 holding logical chunk (lane%8) ^ swizzle(row);
-    // weight rows first, token rows behind them. Rows past the end of a matrix are outside the
-    // descriptor and read as zero.
+    // ---- fills: wave instruction (it, wave) fills LDS slots [(it*4 + wave)*64, +64) of a stage; rows of
+    // 128 bytes: rows (it*4 + wave)*8 + lane/8, chunk lane%8; rows of 64 bytes: rows (it*4 + wave)*16 +
+    // lane/4, chunk lane%4; the slot holds logical chunk (chunk ^ swizzle(row)). Weight rows first, token
+    // rows behind them. Rows past the end of a matrix are outside the descriptor and read as zero.
     const int load_row = wave * 8 + lane / CH;
-    unsigned a_offset = unsigned(load_row) * unsigned(p.k) + unsigned(((lane % CH) ^ lds_swizzle<CH>(load_row)) * 16);
-    unsigned b_offset = a_offset;
+    unsigned b_offset = unsigned(load_row) * unsigned(p.k) + unsigned(((lane % CH) ^ lds_swizzle<CH>(load_row)) * 16);
+    unsigned a_offset = b_offset;
     const unsigned row_step = __builtin_amdgcn_readfirstlane(32u * unsigned(p.k));
+    unsigned row_step_a = row_step;
+    if constexpr (PACKED) {
+        const int packed_row = wave * 16 + lane / 4;
+        a_offset = unsigned(packed_row) * pitch + unsigned(((lane % 4) ^ lds_swizzle<4>(packed_row)) * 16);
+        row_step_a = __builtin_amdgcn_readfirstlane(64u * pitch);
+    }
     const int a_rows = p.n - n0 < BN ? p.n - n0 : BN, b_rows = p.m - m0 < BM ? p.m - m0 : BM;
-    const u32x4_t a_resource = uniform_descriptor(p.w + size_t(n0) * p.k, unsigned(a_rows) * unsigned(p.k));
+    const u32x4_t a_resource = uniform_descriptor(p.w + size_t(n0) * pitch, unsigned(a_rows) * pitch);
     const u32x4_t b_resource = uniform_descriptor(p.a + size_t(m0) * p.k, unsigned(b_rows) * unsigned(p.k));
     const unsigned lds_base = static_cast<unsigned>(reinterpret_cast<uintptr_t>(lds));
     const unsigned fill_base = __builtin_amdgcn_readfirstlane(lds_base + unsigned(wave) * 1024u);
 
-    // ---- scale slabs: the four scale bytes of a row and K group are one word. Token words: wavefront w
-    // copies pieces 2w and 2w + 1 of a slab (32 tokens each): lane l brings groups 4 (l % 2) .. + 3 of
-    // token l / 2 of the piece, 16 bytes, so that the piece lands as [token][8 groups]. Tokens that do
-    // not exist read as zero. Weight words: lane l of one 4-byte load brings group l % 8 of block row
-    // l / 8 from the tile's first 32-row block row (the tile's 192 rows are six of them).
+    // ---- scale slabs: the four scale bytes of a row and K group are one word. Wavefront w copies pieces
+    // 2w and 2w + 1 of the token slab (32 tokens each): lane l brings groups 4 (l % 2) .. + 3 of token
+    // l / 2 of the piece, 16 bytes, so that the piece lands as [token][8 groups]. Rows that do not exist
+    // read as zero. Weight words, E2M1 (a word per row): pieces w and w + 4 of eight in the same way, of
+    // which six hold the tile's rows; E4M3: lane l of one 4-byte load brings group l % 8 of block row l / 8
+    // from the tile's first 32-row block row (the tile's 192 rows are six of them).
     const u32x4_t a_scale_resource =
         uniform_descriptor(p.a_scale + size_t(m0) * p.groups * 4, unsigned(b_rows) * unsigned(p.groups) * 4u);
     const unsigned slab_offset = (unsigned(wave * 64 + lane / 2) * unsigned(p.groups) + unsigned(lane % 2) * 4u) * 4u;
@@ -72,31 +85,44 @@ __global__ __launch_bounds__(256) void mx_wave4_kernel(MxWave4Params p)
     const unsigned slab_fill = __builtin_amdgcn_readfirstlane(lds_base + unsigned(A_SLAB) + unsigned(wave) * 2048u);
     const int first_block = n0 / 32;
     const int blocks = p.block_rows - first_block < 8 ? p.block_rows - first_block : 8;
-    const u32x4_t w_scale_resource = uniform_descriptor(p.w_scale + size_t(first_block) * p.groups * 4,
-                                                        unsigned(blocks) * unsigned(p.groups) * 4u);
-    const unsigned weight_slab_offset = (unsigned(lane / 8) * unsigned(p.groups) + unsigned(lane % 8)) * 4u;
-    const unsigned weight_slab_fill = __builtin_amdgcn_readfirstlane(lds_base + unsigned(W_SLAB));
+    const u32x4_t w_scale_resource =
+        PACKED ? uniform_descriptor(p.w_scale + size_t(n0) * p.groups * 4, unsigned(a_rows) * unsigned(p.groups) * 4u)
+               : uniform_descriptor(p.w_scale + size_t(first_block) * p.groups * 4, unsigned(blocks) * unsigned(p.groups) * 4u);
+    const unsigned weight_slab_offset =
+        PACKED ? (unsigned(wave * 32 + lane / 2) * unsigned(p.groups) + unsigned(lane % 2) * 4u) * 4u
+               : (unsigned(lane / 8) * unsigned(p.groups) + unsigned(lane % 8)) * 4u;
+    const unsigned weight_slab_rows = __builtin_amdgcn_readfirstlane(128u * unsigned(p.groups) * 4u);
+    const unsigned weight_slab_fill =
+        __builtin_amdgcn_readfirstlane(lds_base + unsigned(W_SLAB) + (PACKED ? unsigned(wave) * 1024u : 0u));
     unsigned slab_k = 0; // byte offset of the next slab along a row of scale words
     unsigned middle_slabs = __builtin_amdgcn_readfirstlane(unsigned(p.groups / 8 - 2));
 
-    // ---- reads. Lane l holds row l % 16 of a 16-row tile and, of its 128 K positions, 16 c .. + 15 and
-    // 64 + 16 c .. + 15 with c = l / 16, and supplies the scale byte of inputs 32 c .. 32 c + 31: byte c
-    // of the row's word. Its eight tokens' words are 512 bytes apart in a slab.
+    // ---- reads. Lane l holds row l % 16 of a 16-row tile. Of the 128 K positions of a group an 8-bit
+    // operand holds 16 c .. + 15 and 64 + 16 c .. + 15 with c = l / 16 (chunks c and 4 + c of its 128-byte
+    // row), a 4-bit operand 32 c .. + 31 (chunk c of its 64-byte row); either way the lane supplies the scale
+    // byte of inputs 32 c .. 32 c + 31: byte c of the row's word. Rows 16 apart are 512 bytes apart in a slab.
     const int frag_row = lane % 16, quarter = lane / 16;
     const int frag_swizzle = lds_swizzle<CH>(frag_row);
     const int wave_row = n0 + wn * NA * 16; // first weight row of the wavefront
-    const unsigned a_row_bytes = unsigned(wn * NA * 16 + frag_row) * 128u;
-    const unsigned b_row_bytes = unsigned(BN + wm * NB * 16 + frag_row) * 128u;
-    const unsigned read_a_lo = lds_base + a_row_bytes + unsigned(quarter ^ frag_swizzle) * 16u;
-    const unsigned read_a_hi = lds_base + a_row_bytes + unsigned((4 + quarter) ^ frag_swizzle) * 16u;
+    const unsigned a_row_bytes = unsigned(wn * NA * 16 + frag_row) * unsigned(A_ROW);
+    const unsigned b_row_bytes = unsigned(A_BYTES) + unsigned(wm * NB * 16 + frag_row) * 128u;
+    const unsigned read_a_lo =
+        lds_base + a_row_bytes + unsigned(PACKED ? quarter ^ lds_swizzle<4>(frag_row) : quarter ^ frag_swizzle) * 16u;
+    const unsigned read_a_hi = lds_base + a_row_bytes + unsigned((4 + quarter) ^ frag_swizzle) * 16u; // (E4M3 weights only)
     const unsigned read_b_lo = lds_base + b_row_bytes + unsigned(quarter ^ frag_swizzle) * 16u;
     const unsigned read_b_hi = lds_base + b_row_bytes + unsigned((4 + quarter) ^ frag_swizzle) * 16u;
     unsigned scale_address = lds_base + unsigned(A_SLAB) + unsigned(wm * NB * 16 + frag_row) * 32u + unsigned(quarter);
-    unsigned weight_scale_address = lds_base + unsigned(W_SLAB) + unsigned(wave_row / 32 - first_block) * 32u + unsigned(quarter);
+    unsigned weight_scale_address =
+        lds_base + unsigned(W_SLAB) + unsigned(quarter) +
+        (PACKED ? unsigned(wn * NA * 16 + frag_row) : unsigned(wave_row / 32 - first_block)) * 32u;
 
     // accumulator tile (i, j) (weight rows 16 i .., tokens 16 j ..) comes back as accs[8 i + j]
     f32x4_t accs[NA * NB];
+    if constexpr (PACKED) {
+#include "mx_wave4_loop_192x256_e2m1.inc"
+    } else {
 #include "mx_wave4_loop_192x256.inc"
+    }
 
     // ---- epilogue. Register e of lane l in tile (i, j) is feature 16 i + 4 (l / 16) + e, token 16 j + l % 16.
 #pragma unroll
@@ -115,13 +141,14 @@ __global__ __launch_bounds__(256) void mx_wave4_kernel(MxWave4Params p)
 } // namespace
 
 // `outputs` weight rows from `weight` on (scale rows from weight_scale on), written at `out` with `out_pitch`
-// elements between tokens.
-hipError_t launch_mx_wave4(hipStream_t stream, int rows, int outputs, int inner, const void *input,
+// elements between tokens. packed: E2M1 weights, two to a byte, a scale byte per row and 32 inputs.
+hipError_t launch_mx_wave4(hipStream_t stream, bool packed, int rows, int outputs, int inner, const void *input,
                            const void *input_scale, const void *weight, const void *weight_scale, void *out, int out_pitch)
 {
     const auto misaligned = [](const void *pointer, uintptr_t to) { return reinterpret_cast<uintptr_t>(pointer) % to != 0; };
     if (rows < 1 || outputs < 1 || outputs % 4 || out_pitch % 4 || inner % 1024 || inner < 2048 || misaligned(out, 8) ||
-        misaligned(input, 16) || misaligned(weight, 16) || misaligned(input_scale, 16) || misaligned(weight_scale, 4))
+        misaligned(input, 16) || misaligned(weight, 16) || misaligned(input_scale, 16) ||
+        misaligned(weight_scale, packed ? 16 : 4))
         return hipErrorInvalidValue;
     if (size_t(256) * size_t(inner) >= (size_t(1) << 32))
         return hipErrorInvalidValue;
@@ -141,7 +168,11 @@ hipError_t launch_mx_wave4(hipStream_t stream, int rows, int outputs, int inner,
     p.tiles_m = (rows + BM - 1) / BM;
     if (size_t(p.tiles_n) * size_t(p.tiles_m) > 0x7fffffffu)
         return hipErrorInvalidValue;
-    mx_wave4_kernel<<<unsigned(p.tiles_n) * unsigned(p.tiles_m), 256, 0, stream>>>(p);
+    const unsigned grid = unsigned(p.tiles_n) * unsigned(p.tiles_m);
+    if (packed)
+        mx_wave4_kernel<true><<<grid, 256, 0, stream>>>(p);
+    else
+        mx_wave4_kernel<false><<<grid, 256, 0, stream>>>(p);
     return launch_status();
 }
 } // namespace camblas_hip

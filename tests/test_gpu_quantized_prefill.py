@@ -118,45 +118,53 @@ def test_exact_products_with_every_scale_alignment(device, kernel, packed, block
     assert np.array_equal(got, want)
 
 
+@pytest.mark.parametrize("packed", [False, True])
 @pytest.mark.parametrize("rows,outputs,inner", [(70, 296, 2048), (513, 456, 3072), (300, 840, 4096)])
-def test_four_wavefront_tile_random_operands(device, rows, outputs, inner):
-    # 192 x 256 tiles on four wavefronts with the K loop in generated assembly (E4M3 weights, a scale per 32
-    # inputs): partial tiles in both directions, a partial last 32-row scale block, two to four slabs of
-    # eight K groups, operands and scales mutated one at a time
-    x, sx, weight, sw = operands(950 + rows, rows, outputs, inner, False, 32)
+def test_four_wavefront_tile_random_operands(device, packed, rows, outputs, inner):
+    # 192 x 256 tiles on four wavefronts with the K loop in generated assembly (a scale per 32 inputs; E4M3
+    # weights with a scale per 32 x 32 block, or packed E2M1 weights with a scale per row and 32 inputs):
+    # partial tiles in both directions, a partial last scale block, two to four slabs of eight K groups,
+    # operands and scales mutated one at a time
+    x, sx, weight, sw = operands(950 + rows, rows, outputs, inner, packed, 32)
     for changed in ("original", "input", "weight", "input_scale", "weight_scale"):
         if changed == "input":
             x ^= 128
         elif changed == "weight":
-            weight ^= 128
-            weight[(weight & 0x7F) == 0x7F] = 0x38  # keep the weights finite
+            weight ^= 17 if packed else 128
+            if not packed:
+                weight[(weight & 0x7F) == 0x7F] = 0x38  # keep the weights finite
         elif changed == "input_scale":
             sx -= 1
         elif changed == "weight_scale":
             sw += 1
-        close(run(device, x, sx, weight, sw, False, 32, "wave4-192x256"), x, sx, weight, sw, False, 32)
+        close(run(device, x, sx, weight, sw, packed, 32, "wave4-192x256"), x, sx, weight, sw, packed, 32)
 
 
-def test_four_wavefront_tile_exact_products(device):
+@pytest.mark.parametrize("packed", [False, True])
+def test_four_wavefront_tile_exact_products(device, packed):
     # exact arithmetic as in test_exact_products_with_every_scale_alignment over 24 K groups (three slabs):
-    # a scale byte of the wrong block, row, group or slab buffer changes the bits; and the eight-wavefront
-    # tile must give the same bits on random operands at the benchmark's inner dimension
+    # a scale byte of the wrong block, row, group or slab buffer changes the bits
     rows, outputs, inner = 300, 840, 24 * 128
     rng = np.random.default_rng(77)
     levels = np.array([0x00, 0x30, 0x38, 0x40, 0xB0, 0xB8, 0xC0], np.uint8)
     x = levels[rng.integers(0, len(levels), (rows, inner))]
-    weight = levels[rng.integers(0, len(levels), (outputs, inner))]
+    if packed:
+        nibbles = np.array([0, 1, 2, 3, 4, 9, 10, 11, 12], np.uint8)  # 0, .5, 1, 1.5, 2 and negatives
+        pairs = nibbles[rng.integers(0, len(nibbles), (outputs, inner // 2, 2))]
+        weight = (pairs[..., 0] | (pairs[..., 1] << 4)).astype(np.uint8)
+    else:
+        weight = levels[rng.integers(0, len(levels), (outputs, inner))]
     sx = rng.integers(125, 130, (rows, inner // 32), dtype=np.uint8)
-    sw = rng.integers(125, 130, ((outputs + 31) // 32, inner // 32), dtype=np.uint8)
-    got = run(device, x, sx, weight, sw, False, 32, "wave4-192x256")
-    want = oracle.mx_matmul_f64(x, sx, weight, sw, 32, False)
+    sw = rng.integers(125, 130, (outputs if packed else (outputs + 31) // 32, inner // 32), dtype=np.uint8)
+    got = run(device, x, sx, weight, sw, packed, 32, "wave4-192x256")
+    want = oracle.mx_matmul_f64(x, sx, weight, sw, 32, packed)
     assert np.abs(want).max() < 2.0 ** 24 and (want * 64 == np.round(want * 64)).all()
     assert np.array_equal(got, oracle.bf16_to_f32(oracle.f32_to_bf16(want.astype(np.float32))))
 
 
 def test_four_wavefront_tile_refuses_what_it_cannot_run(device):
-    # packed weights, a scale per 128 inputs, an inner dimension that is not whole slabs of eight groups
-    for packed, block, inner in ((True, 32, 2048), (True, 128, 2048), (False, 32, 1152)):
+    # a scale per 128 inputs, an inner dimension that is not whole slabs of eight groups
+    for packed, block, inner in ((True, 128, 2048), (False, 32, 1152), (True, 32, 1152)):
         x, sx, weight, sw = operands(5, 64, 256, inner, packed, block)
         with pytest.raises(RuntimeError):
             run(device, x, sx, weight, sw, packed, block, "wave4-192x256")
