@@ -79,13 +79,26 @@ class Form:
         return lines
 
     def scale_reads(self, into):
-        """The next group's scale bytes: the lane's eight tokens (512 bytes apart in a slab of
-        [row][8 groups] words) and its weight tiles' (E2M1: six rows 512 bytes apart in a slab of the same
-        shape; E4M3: the three 32-row blocks its 96 rows lie in, rows of 8 words)."""
+        """The next group's scale bytes: the lane's eight tokens and its weight tiles' (E2M1: six rows in a
+        slab of the tokens' shape; E4M3: the three 32-row blocks its 96 rows lie in, rows of 8 words). A slab
+        of rows is pieces of 32 rows, a piece two halves (groups 0-3, groups 4-7) of [row][4 words]: sixteen
+        rows in a row are sixteen different banks; rows 16 apart are 256 bytes apart, 32 apart a piece."""
         first = SCALES + self.set * into
-        lines = [f"ds_read_u8 v{first + j}, %[sa] offset:{512 * j}" for j in range(NB)]
-        pitch = 512 if self.packed else 32
-        lines += [f"ds_read_u8 v{first + NB + b}, %[sw] offset:{pitch * b}" for b in range(self.w_scales)]
+        rows = lambda index: (index // 2) * 1024 + (index % 2) * 256
+        lines = [f"ds_read_u8 v{first + j}, %[sa] offset:{rows(j)}" for j in range(NB)]
+        lines += [f"ds_read_u8 v{first + NB + b}, %[sw] offset:{rows(b) if self.packed else 32 * b}"
+                  for b in range(self.w_scales)]
+        return lines
+
+    def scale_advance(self, position):
+        """What the lane's slab addresses do after the reads of the step at `position` of a slab (which read
+        group position + 1): on to the next group's word: 4 bytes, from group 3 to group 4 into the piece's
+        second half, from group 7 to group 0 of the other buffer."""
+        rows = {2: ["v_add_u32_e32 {0}, 500, {0}"], 6: ["v_subrev_u32_e32 {0}, 524, {0}", "v_xor_b32_e32 {0}, 0x2000, {0}"]}
+        blocks = {6: ["v_subrev_u32_e32 {0}, 28, {0}", "v_xor_b32_e32 {0}, 0x100, {0}"]}
+        step = ["v_add_u32_e32 {0}, 4, {0}"]
+        lines = [line.format("%[sa]") for line in rows.get(position, step)]
+        lines += [line.format("%[sw]") for line in (rows if self.packed else blocks).get(position, step)]
         return lines
 
     def fill_units(self, target):
@@ -112,8 +125,8 @@ class Form:
 
     def slab_loads(self):
         """The next eight groups' scale words into the slab buffers that are not being read: two pieces of
-        the token slab per wavefront (32 tokens each, lanes 2t and 2t + 1 bring groups 0-3 and 4-7 of
-        token t); the weights' likewise (E2M1: pieces w and w + 4 of eight, of which six hold the tile's
+        the token slab per wavefront (32 tokens each, lane l brings groups 4 (l / 32) .. + 3 of token
+        l % 32); the weights' likewise (E2M1: pieces w and w + 4 of eight, of which six hold the tile's
         rows) or with one 4-byte-per-lane load (E4M3: every wavefront brings the same bytes to the same place)."""
         lines = [
             f"s_mov_b32 m0, {SLAB_TARGET}", "s_nop 0",
@@ -133,11 +146,10 @@ class Form:
                   f"s_xor_b32 {W_TARGET}, {W_TARGET}, {self.w_flip:#x}"]
         return lines
 
-    def step(self, buffer, *, fills, reads, first, last, scale_step):
+    def step(self, buffer, *, fills, reads, first, last, position):
         """One K group from fragment buffer `buffer` with scale set `buffer`. fills: LDS target of the group
         after the next, or None; reads: fetch the next group's fragments and scales into the other buffer
-        and set; first: the accumulators start from zero; scale_step: what the lane's slab addresses do
-        after its reads ("next": the next group of the slab; "wrap": the first group of the other buffers)."""
+        and set; first: the accumulators start from zero; position: of the step in its slab."""
         units = self.fill_units(fills) if fills else []
         pending = (self.scale_reads(1 - buffer) + self.fragment_reads(1 - buffer, 1 - buffer)) if reads else []
         assert len(pending) <= TILES and 3 * len(units) <= TILES
@@ -161,11 +173,7 @@ class Form:
             if t < len(pending):
                 lines.append(pending[t])
         if reads:
-            if scale_step == "next":
-                lines += ["v_add_u32_e32 %[sa], 4, %[sa]", "v_add_u32_e32 %[sw], 4, %[sw]"]
-            else:
-                lines += ["v_subrev_u32_e32 %[sa], 28, %[sa]", "v_xor_b32_e32 %[sa], 0x2000, %[sa]",
-                          "v_subrev_u32_e32 %[sw], 28, %[sw]", f"v_xor_b32_e32 %[sw], {self.w_flip:#x}, %[sw]"]
+            lines += self.scale_advance(position)
         if last:  # the code after the statement reads the accumulators: cover the longest instruction latency
             lines += ["s_nop 15", "s_nop 15"]
         else:
@@ -187,8 +195,7 @@ class Form:
         lines += self.advance() + ["s_waitcnt vmcnt(0)", "s_barrier", "; group 1 into stage 1"]
         for before, load in self.fill_units(FILL1):
             lines += before + ["s_nop 0", load]
-        lines += self.advance() + self.scale_reads(0) + self.fragment_reads(0, 0)
-        lines += ["v_add_u32_e32 %[sa], 4, %[sa]", "v_add_u32_e32 %[sw], 4, %[sw]"]
+        lines += self.advance() + self.scale_reads(0) + self.fragment_reads(0, 0) + self.scale_advance(7)
         # every wavefront has read stage 0 and group 1 has landed before stage 0 is filled again and stage 1 is read
         lines += ["s_waitcnt vmcnt(0) lgkmcnt(0)", "s_barrier"]
 
@@ -205,7 +212,7 @@ class Form:
                     body += self.slab_loads()
                 body += self.step(position % 2, fills=target, reads=not (last_slab and position == 7),
                                   first=first_slab and position == 0, last=last_slab and position == 7,
-                                  scale_step="wrap" if position == 6 else "next")
+                                  position=position)
             return body
 
         lines += ["; first slab"] + slab_steps(True, False)

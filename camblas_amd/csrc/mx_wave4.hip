@@ -73,14 +73,14 @@ template <bool PACKED> __global__ __launch_bounds__(256) void mx_wave4_kernel(Mx
     const unsigned fill_base = __builtin_amdgcn_readfirstlane(lds_base + unsigned(wave) * 1024u);
 
     // ---- scale slabs: the four scale bytes of a row and K group are one word. Wavefront w copies pieces
-    // 2w and 2w + 1 of the token slab (32 tokens each): lane l brings groups 4 (l % 2) .. + 3 of token
-    // l / 2 of the piece, 16 bytes, so that the piece lands as [token][8 groups]. Rows that do not exist
-    // read as zero. Weight words, E2M1 (a word per row): pieces w and w + 4 of eight in the same way, of
+    // 2w and 2w + 1 of the token slab (32 tokens each): lane l brings groups 4 (l / 32) .. + 3 of token
+    // l % 32 of the piece, 16 bytes, so that a piece lands as two halves of [token][4 groups] and sixteen
+    // tokens in a row lie in sixteen different banks. Rows that do not exist read as zero. Weight words, E2M1 (a word per row): pieces w and w + 4 of eight in the same way, of
     // which six hold the tile's rows; E4M3: lane l of one 4-byte load brings group l % 8 of block row l / 8
     // from the tile's first 32-row block row (the tile's 192 rows are six of them).
     const u32x4_t a_scale_resource =
         uniform_descriptor(p.a_scale + size_t(m0) * p.groups * 4, unsigned(b_rows) * unsigned(p.groups) * 4u);
-    const unsigned slab_offset = (unsigned(wave * 64 + lane / 2) * unsigned(p.groups) + unsigned(lane % 2) * 4u) * 4u;
+    const unsigned slab_offset = (unsigned(wave * 64 + lane % 32) * unsigned(p.groups) + unsigned(lane / 32) * 4u) * 4u;
     const unsigned slab_rows = __builtin_amdgcn_readfirstlane(32u * unsigned(p.groups) * 4u);
     const unsigned slab_fill = __builtin_amdgcn_readfirstlane(lds_base + unsigned(A_SLAB) + unsigned(wave) * 2048u);
     const int first_block = n0 / 32;
@@ -89,7 +89,7 @@ template <bool PACKED> __global__ __launch_bounds__(256) void mx_wave4_kernel(Mx
         PACKED ? uniform_descriptor(p.w_scale + size_t(n0) * p.groups * 4, unsigned(a_rows) * unsigned(p.groups) * 4u)
                : uniform_descriptor(p.w_scale + size_t(first_block) * p.groups * 4, unsigned(blocks) * unsigned(p.groups) * 4u);
     const unsigned weight_slab_offset =
-        PACKED ? (unsigned(wave * 32 + lane / 2) * unsigned(p.groups) + unsigned(lane % 2) * 4u) * 4u
+        PACKED ? (unsigned(wave * 32 + lane % 32) * unsigned(p.groups) + unsigned(lane / 32) * 4u) * 4u
                : (unsigned(lane / 8) * unsigned(p.groups) + unsigned(lane % 8)) * 4u;
     const unsigned weight_slab_rows = __builtin_amdgcn_readfirstlane(128u * unsigned(p.groups) * 4u);
     const unsigned weight_slab_fill =
@@ -100,7 +100,7 @@ template <bool PACKED> __global__ __launch_bounds__(256) void mx_wave4_kernel(Mx
     // ---- reads. Lane l holds row l % 16 of a 16-row tile. Of the 128 K positions of a group an 8-bit
     // operand holds 16 c .. + 15 and 64 + 16 c .. + 15 with c = l / 16 (chunks c and 4 + c of its 128-byte
     // row), a 4-bit operand 32 c .. + 31 (chunk c of its 64-byte row); either way the lane supplies the scale
-    // byte of inputs 32 c .. 32 c + 31: byte c of the row's word. Rows 16 apart are 512 bytes apart in a slab.
+    // byte of inputs 32 c .. 32 c + 31: byte c of the row's word.
     const int frag_row = lane % 16, quarter = lane / 16;
     const int frag_swizzle = lds_swizzle<CH>(frag_row);
     const int wave_row = n0 + wn * NA * 16; // first weight row of the wavefront
@@ -111,10 +111,11 @@ template <bool PACKED> __global__ __launch_bounds__(256) void mx_wave4_kernel(Mx
     const unsigned read_a_hi = lds_base + a_row_bytes + unsigned((4 + quarter) ^ frag_swizzle) * 16u; // (E4M3 weights only)
     const unsigned read_b_lo = lds_base + b_row_bytes + unsigned(quarter ^ frag_swizzle) * 16u;
     const unsigned read_b_hi = lds_base + b_row_bytes + unsigned((4 + quarter) ^ frag_swizzle) * 16u;
-    unsigned scale_address = lds_base + unsigned(A_SLAB) + unsigned(wm * NB * 16 + frag_row) * 32u + unsigned(quarter);
+    // (a wavefront's 128 tokens are four pieces of a slab, its 96 weight rows three)
+    unsigned scale_address = lds_base + unsigned(A_SLAB) + unsigned(wm * 4) * 1024u + unsigned(frag_row) * 16u + unsigned(quarter);
     unsigned weight_scale_address =
         lds_base + unsigned(W_SLAB) + unsigned(quarter) +
-        (PACKED ? unsigned(wn * NA * 16 + frag_row) : unsigned(wave_row / 32 - first_block)) * 32u;
+        (PACKED ? unsigned(wn * 3) * 1024u + unsigned(frag_row) * 16u : unsigned(wave_row / 32 - first_block) * 32u);
 
     // accumulator tile (i, j) (weight rows 16 i .., tokens 16 j ..) comes back as accs[8 i + j]
     f32x4_t accs[NA * NB];
