@@ -38,6 +38,12 @@ NA, NB = 6, 8  # 16-row weight tiles and 16-token tiles per wavefront
 TILES = NA * NB
 SCALES, STAGE1 = 192, 235
 SAVED_M0, OFFSET, FILL1, SLAB_TARGET, W_TARGET = "s84", "s85", "s86", "s87", "s88"
+# placement inside a step: a fill behind every FILL_EVERY-th matrix instruction from FILL_FROM on, an LDS read
+# behind every instruction from READ_FROM on. The fills are waited for at the end of the step they are issued
+# in, so they go first (measured, E4M3 weights at 4096 rows: fills every third instruction from the third on
+# and reads from the first 418 us; fills every second from the first 396-400 us wherever the reads start; all
+# fills in a burst 417 us)
+FILL_EVERY, FILL_FROM, READ_FROM = 2, 0, 8
 
 
 class Form:
@@ -152,8 +158,8 @@ class Form:
         and set; first: the accumulators start from zero; position: of the step in its slab."""
         units = self.fill_units(fills) if fills else []
         pending = (self.scale_reads(1 - buffer) + self.fragment_reads(1 - buffer, 1 - buffer)) if reads else []
-        assert len(pending) <= TILES and 3 * len(units) <= TILES
-        fill_at = {3 * n + 2: unit for n, unit in enumerate(units)}
+        assert len(pending) + READ_FROM <= TILES and FILL_EVERY * len(units) <= TILES
+        fill_at = {FILL_EVERY * n + FILL_FROM: unit for n, unit in enumerate(units)}
         scales = SCALES + self.set * buffer
         lines = []
         for t in range(TILES):
@@ -170,8 +176,8 @@ class Form:
                 lines.append(fill_at[t][1])
                 if fill_at[t] is units[-1]:
                     lines += self.advance()
-            if t < len(pending):
-                lines.append(pending[t])
+            if 0 <= t - READ_FROM < len(pending):
+                lines.append(pending[t - READ_FROM])
         if reads:
             lines += self.scale_advance(position)
         if last:  # the code after the statement reads the accumulators: cover the longest instruction latency
@@ -258,7 +264,10 @@ class Form:
 def main():
     parser = argparse.ArgumentParser(description=__doc__.split("\n")[0])
     parser.add_argument("--out", type=Path, default=Path(__file__).resolve().parent)
+    parser.add_argument("--placement", default="", help="experiments: FILL_EVERY,FILL_FROM,READ_FROM")
     arguments = parser.parse_args()
+    if arguments.placement:
+        globals()["FILL_EVERY"], globals()["FILL_FROM"], globals()["READ_FROM"] = (int(v) for v in arguments.placement.split(","))
     for packed in (False, True):
         form = Form(packed)
         (arguments.out / form.name).write_text(form.statement())
