@@ -144,6 +144,10 @@ def accumulate(tile, split):
 
 
 DROP = set()  # experiments only: parts of a step left out (results are then wrong), see --drop
+# a fill behind every FILL_EVERY-th matrix instruction of a step from FILL_FROM on (the fills are waited for
+# at the end of the step they are issued in, so they go first: every third from the third on 514 us at 4096
+# tokens, every second from the second on 489)
+FILL_EVERY, FILL_FROM = 2, 1
 
 
 def step(buffer, split, *, fills, reads, first, last, scale_step):
@@ -158,7 +162,7 @@ def step(buffer, split, *, fills, reads, first, last, scale_step):
         pending_reads = ([] if "scales" in DROP else scale_reads()) + (
             [] if "reads" in DROP else fragment_reads(1 - buffer, 1 - buffer))
     lines = []
-    fill_at = {3 * n + 2: unit for n, unit in enumerate(units)}  # tiles 2, 5, ..., 41
+    fill_at = {FILL_EVERY * n + FILL_FROM: unit for n, unit in enumerate(units)}
     for t in range(TILES):
         i, j = divmod(t, NB)
         if t in fill_at:
@@ -281,8 +285,11 @@ def main():
     parser = argparse.ArgumentParser(description=__doc__.split("\n")[0])
     parser.add_argument("--out", type=Path, default=Path(__file__).resolve().parent)
     parser.add_argument("--drop", default="", help="experiments: comma list of fills, reads, scales, fmas, barrier, fillwait")
+    parser.add_argument("--placement", default="", help="experiments: FILL_EVERY,FILL_FROM")
     arguments = parser.parse_args()
     DROP.update(part for part in arguments.drop.split(",") if part)
+    if arguments.placement:
+        globals()["FILL_EVERY"], globals()["FILL_FROM"] = (int(v) for v in arguments.placement.split(","))
     text = ["// Generated by gen_fp8_wave4_loop.py; edit the generator, not this file.",
             "// split: the first of the wavefront's six 16-row weight tiles that lies in its second scale block"]
     for index, split in enumerate((2, 4, 6)):
