@@ -611,7 +611,19 @@ int bf16_product(const Entry &entry, const Product &p, float alpha, const void *
     // W as it lies (the planner's variant 20 for 'N','N'): the other kernels of that family assume
     // K-contiguous weights, so neither the register-staged substitute nor a forced variant applies;
     // tests: 60 and 61 ask for the layout-agnostic kernel or the transposing route instead
-    const bool as_it_lies = plan.family == FAMILY_DMA && plan.kernel == 20 && !p.trans_a;
+    bool as_it_lies = plan.family == FAMILY_DMA && plan.kernel == 20 && !p.trans_a;
+    // tests: 40 forces that tile for an 'N','N' call of any size whose operands it can take (a launch that
+    // cannot run fails), and is refused for every other layout
+    if (forced == 40) {
+        if (p.trans_a || p.trans_b)
+            return entry.refuse("the forced tile takes 'N','N' operands only");
+        plan.family = FAMILY_DMA;
+        plan.kernel = 20;
+        plan.split_k = 1;
+        plan.tail_outputs = 0;
+        plan.counter = 4;
+        as_it_lies = true;
+    }
     if (as_it_lies) {
         if (!is_aligned(c, 8) || !is_aligned(source.z, 8) || source.ldz % 4 || forced == 60 || forced == 61)
             plan = make_plan(2, context->algorithm, p.trans_a, p.trans_b, p.m, p.n, p.k, p.lda, p.ldb, p.ldc, false,

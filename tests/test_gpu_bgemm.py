@@ -368,6 +368,24 @@ def test_weights_as_they_lie_on_the_four_wavefront_tile(device, m, n, k, pad):
         assert rel_frobenius(oracle.bf16_to_f32(got2d[:, rows]), want) <= TOLERANCE
 
 
+@pytest.mark.parametrize("m,n,k,pad", [(296, 260, 256, 8), (264, 70, 384, 0), (1000, 513, 128 * 5, 16)])
+def test_weights_as_they_lie_against_the_oracle(device, m, n, k, pad):
+    # the same tile forced (code 40) at sizes the oracle finishes: partial tiles in both directions, one to
+    # eight workgroups, two to five pairs of K steps, padded leading dimensions, alpha and beta
+    lda, ldb, ldc = m + pad, k + pad, m + (pad and 4)
+    a = oracle.fill_normal_bf16(121, (lda * k,))
+    b = oracle.fill_normal_bf16(122, (ldb * n,))
+    c0 = oracle.fill_normal_bf16(123, (ldc * n,))
+    for alpha, beta in ((1.0, 0.0), (0.5, -1.5)):
+        got = run_bgemm(device, "N", "N", m, n, k, alpha, a, lda, b, ldb, beta, c0, ldc, override=(40, 1))
+        want, want64 = reference("N", "N", m, n, k, alpha, a, lda, b, ldb, beta, c0, ldc)
+        got2d = got.reshape(n, ldc)
+        assert rel_frobenius(oracle.bf16_to_f32(got2d[:, :m]), want64.reshape(n, m)) <= TOLERANCE
+        assert np.array_equal(got2d[:, m:], c0.reshape(n, ldc)[:, m:])
+    with pytest.raises(RuntimeError):  # the tile is for 'N','N' operands only
+        run_bgemm(device, "T", "N", m, n, k, 1.0, a, k + pad, b, ldb, 0.0, c0, ldc, override=(40, 1))
+
+
 def test_layout_agnostic_kernel_counts_as_a_library_product(device):
     # row-major torch.mm(x, w) with a contiguous [in, out] weight arrives as 'N','N'
     native = _native.context(device)
