@@ -306,10 +306,13 @@ hipError_t launch_mx_dma(hipStream_t stream, int variant, bool packed, int group
                          const void *input_scale, const void *weight, const void *weight_scale,
                          const void *metadata, const void *active, const void *counts, void *out,
                          int tail_variant = 0, int tail_outputs = 0, int shares = 1, float *planes = nullptr);
-// mx_wave4.hip: the plain product on four wavefronts per workgroup (192 x 256 tiles); one input scale per 32
-// inputs, inner % 1024 == 0, inner >= 2048, input scales 16-byte aligned, weight scales 4-byte (packed: 16-byte) aligned.
+// mx_wave4.hip: the product on four wavefronts per workgroup (192 x 256 tiles); one input scale per 32 inputs,
+// inner % 1024 == 0, inner >= 2048, input scales 16-byte aligned, packed weights' scales 16-byte aligned.
+// metadata != nullptr: the grouped product (E4M3 weights only, out_pitch = outputs).
 hipError_t launch_mx_wave4(hipStream_t stream, bool packed, int rows, int outputs, int inner, const void *input,
-                           const void *input_scale, const void *weight, const void *weight_scale, void *out, int out_pitch);
+                           const void *input_scale, const void *weight, const void *weight_scale, void *out, int out_pitch,
+                           int groups = 0, int weight_groups = 0, const void *metadata = nullptr,
+                           const void *active = nullptr, const void *counts = nullptr);
 // Mixture-of-experts routing helpers.
 hipError_t launch_route_groups(hipStream_t stream, int tokens, int choices, int first_expert,
                                int groups, int rows, const void *experts, const void *active,

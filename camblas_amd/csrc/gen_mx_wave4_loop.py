@@ -86,13 +86,14 @@ class Form:
 
     def scale_reads(self, into):
         """The next group's scale bytes: the lane's eight tokens and its weight tiles' (E2M1: six rows in a
-        slab of the tokens' shape; E4M3: the three 32-row blocks its 96 rows lie in, rows of 8 words). A slab
+        slab of the tokens' shape; E4M3: the three 32-row blocks its 96 rows lie in, rows of 9 words: its
+        32 scale bytes from wherever they lie after the aligned address the row was copied from). A slab
         of rows is pieces of 32 rows, a piece two halves (groups 0-3, groups 4-7) of [row][4 words]: sixteen
         rows in a row are sixteen different banks; rows 16 apart are 256 bytes apart, 32 apart a piece."""
         first = SCALES + self.set * into
         rows = lambda index: (index // 2) * 1024 + (index % 2) * 256
         lines = [f"ds_read_u8 v{first + j}, %[sa] offset:{rows(j)}" for j in range(NB)]
-        lines += [f"ds_read_u8 v{first + NB + b}, %[sw] offset:{rows(b) if self.packed else 32 * b}"
+        lines += [f"ds_read_u8 v{first + NB + b}, %[sw] offset:{rows(b) if self.packed else 36 * b}"
                   for b in range(self.w_scales)]
         return lines
 

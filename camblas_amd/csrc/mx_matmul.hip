@@ -513,7 +513,7 @@ MxTilePlan mx_tile_plan(int compute_units, bool packed, int groups, int rows, in
     const int counts[] = {1, 2, 3, 4, 6, 8};
     for (int variant = 0; variant < 5; ++variant) {
         if (prices[variant].step_us > 1e29 || (prices[variant].rows > 128 && rows <= 128) ||
-            (variant == 4 && !(four_wavefronts && groups == 0)))
+            (variant == 4 && !four_wavefronts))
             continue;
         for (const int shares : counts) {
             if (variant == 4 && shares > 1)
@@ -562,15 +562,15 @@ MxTilePlan mx_tile_plan(int compute_units, bool packed, int groups, int rows, in
 // when the streaming kernel could not hold the scale bytes of 32 tokens in its LDS table and would
 // gather them a byte per lane and step ([7168, 18432] x 32 rows: 34 us against 24 at 16 rows and 26 on
 // the tiles).
-// What the four-wavefront tile needs beyond mx_dma_supported: the plain product, a scale per 32 inputs, whole
-// slabs of eight 128-input groups (at least two), scale rows it can copy 16 bytes at a time (the block rows of
-// unpacked weights: 4).
+// What the four-wavefront tile needs beyond mx_dma_supported: a scale per 32 inputs, whole slabs of eight
+// 128-input groups (at least two), input scale rows it can copy 16 bytes at a time, and the same of the
+// per-row scales of packed weights, whose address the host has to know: no grouped product of packed weights.
 static bool mx_four_wavefront_tile_applies(bool packed, int groups, int inner, int activation_block,
                                            const void *input_scale, const void *weight_scale)
 {
-    return groups == 0 && activation_block == 32 && inner % 1024 == 0 && inner >= 2048 &&
+    return activation_block == 32 && inner % 1024 == 0 && inner >= 2048 &&
            reinterpret_cast<uintptr_t>(input_scale) % 16 == 0 &&
-           reinterpret_cast<uintptr_t>(weight_scale) % (packed ? 16 : 4) == 0;
+           (packed ? groups == 0 && reinterpret_cast<uintptr_t>(weight_scale) % 16 == 0 : true);
 }
 
 static bool mx_rows_take_tiles(int rows, int inner, int activation_block)

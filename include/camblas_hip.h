@@ -400,7 +400,8 @@ int camblas_hip_plan_describe(int dtype, int algorithm, char trans_a, char trans
  * this context (kernel < 0 restores the planner; split_k <= 0 lets the planner choose). For the
  * E8M0 products: 0 the weight-streaming kernel, 20 / 21 / 22 / 23 the tiled kernel with
  * 256 x 256, 256 x 128, (E4M3 weights only) 192 x 256 and 128 x 128 tiles, 24 the four-wavefront
- * 192 x 256 tile; a forced kernel that cannot run the call makes the call fail. (BF16: 20 + n the
+ * 192 x 256 tile (grouped calls: E4M3 weights only); a forced kernel that cannot run the call makes
+ * the call fail. (BF16: 20 + n the
  * direct-to-LDS tile n, of which 38 / 39 are the four-wavefront 256- and 320-row tiles and 40 the
  * 256-row tile for weights stored with their outputs contiguous; FP8 with FP32 scales: 36 the
  * four-wavefront 192 x 256 tile.)

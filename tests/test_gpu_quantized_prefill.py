@@ -162,6 +162,22 @@ def test_four_wavefront_tile_exact_products(device, packed):
     assert np.array_equal(got, oracle.bf16_to_f32(oracle.f32_to_bf16(want.astype(np.float32))))
 
 
+@pytest.mark.parametrize("shift", [1, 2, 3])
+def test_four_wavefront_tile_block_scales_at_any_address(device, shift):
+    # the block scales of E4M3 weights need no alignment: the slab is copied from the aligned address below
+    # them with a ninth word per block row; exact products over three slabs show a byte taken from the wrong place
+    rows, outputs, inner = 100, 424, 24 * 128
+    rng = np.random.default_rng(78 + shift)
+    levels = np.array([0x00, 0x30, 0x38, 0x40, 0xB0, 0xB8, 0xC0], np.uint8)
+    x = levels[rng.integers(0, len(levels), (rows, inner))]
+    weight = levels[rng.integers(0, len(levels), (outputs, inner))]
+    sx = rng.integers(125, 130, (rows, inner // 32), dtype=np.uint8)
+    sw = rng.integers(125, 130, ((outputs + 31) // 32, inner // 32), dtype=np.uint8)
+    got = run(device, x, sx, weight, sw, False, 32, "wave4-192x256", shifts=(0, shift))
+    want = oracle.mx_matmul_f64(x, sx, weight, sw, 32, False)
+    assert np.array_equal(got, oracle.bf16_to_f32(oracle.f32_to_bf16(want.astype(np.float32))))
+
+
 def test_four_wavefront_tile_refuses_what_it_cannot_run(device):
     # a scale per 128 inputs, an inner dimension that is not whole slabs of eight groups
     for packed, block, inner in ((True, 128, 2048), (False, 32, 1152), (True, 32, 1152)):
@@ -261,10 +277,24 @@ def test_scale_extremes_and_nan(device, kernel, packed):
 @pytest.mark.parametrize("kernel", ["auto", "tile256x256", "tile256x128", "tile128x128"])
 @pytest.mark.parametrize("packed,block", [(False, 32), (True, 32), (True, 128)])
 def test_grouped_products(device, kernel, packed, block):
+    check_grouped_products(device, kernel, packed, block, inner=256, input_shift=1)
+
+
+def test_grouped_products_on_the_four_wavefront_tile(device):
+    # E4M3 weights only (the per-row scales of packed weights would have to be 16-byte aligned, which the
+    # host cannot see in a device table); each group's block scales at another alignment
+    check_grouped_products(device, "wave4-192x256", False, 32, inner=2048, input_shift=0)
+    with pytest.raises(RuntimeError):
+        check_grouped_products(device, "wave4-192x256", True, 32, inner=2048, input_shift=0)
+    with pytest.raises(RuntimeError):  # input scales that are not 16-byte aligned
+        check_grouped_products(device, "wave4-192x256", False, 32, inner=2048, input_shift=1)
+
+
+def check_grouped_products(device, kernel, packed, block, inner, input_shift):
     # ref: include/camblas_cuda.h:156-167 — weights chosen per group through a device table, an
     # invalid index gives zeros, counts clip the rows, padding rows are zero even where the
     # padding's scale bytes say NaN
-    groups, weight_groups, rows, outputs, inner = 6, 3, 300, 264, 256
+    groups, weight_groups, rows, outputs = 6, 3, 300, 264
     rng = np.random.default_rng(19)
     x = oracle.f32_to_e4m3((rng.standard_normal((groups, rows, inner)) * 8).astype(np.float32))
     sx = rng.integers(122, 129, (groups, rows, inner // block), dtype=np.uint8)
@@ -284,7 +314,7 @@ def test_grouped_products(device, kernel, packed, block):
     native.call("hip_set_plan_override", KERNELS[kernel], 0)
     try:
         out = _kernels.grouped_quantized_matmul(
-            torch.from_numpy(x).to(device).view(torch.float8_e4m3fn), shifted(device, sx, 1),
+            torch.from_numpy(x).to(device).view(torch.float8_e4m3fn), shifted(device, sx, input_shift),
             metadata, active, counts, outputs=outputs, packed=packed, activation_block=block)
         torch.cuda.synchronize()
     finally:
@@ -303,10 +333,18 @@ def test_grouped_products(device, kernel, packed, block):
 @pytest.mark.parametrize("kernel", ["tile256x128", "tile128x128"])
 @pytest.mark.parametrize("packed", [False, True])
 def test_grouped_products_many_groups_skewed_counts(device, kernel, packed):
+    check_many_groups_skewed_counts(device, kernel, packed, inner=128, compared=40)
+
+
+def test_many_groups_skewed_counts_on_the_four_wavefront_tile(device):
+    check_many_groups_skewed_counts(device, "wave4-192x256", False, inner=2048, compared=6)
+
+
+def check_many_groups_skewed_counts(device, kernel, packed, inner, compared):
     """150 groups (three 64-lane chunks of the tile numbering) with a capacity of several token tiles
     and counts from none to all of it, negative and oversized included: every tile with work is
     computed for the right group, every other tile of the capacity is zero."""
-    groups, weight_groups, rows, outputs, inner = 150, 5, 300, 136, 128
+    groups, weight_groups, rows, outputs = 150, 5, 300, 136
     rng = np.random.default_rng(23)
     x = oracle.f32_to_e4m3((rng.standard_normal((groups, rows, inner)) * 8).astype(np.float32))
     sx = rng.integers(124, 129, (groups, rows, inner // 32), dtype=np.uint8)
@@ -335,13 +373,13 @@ def test_grouped_products_many_groups_skewed_counts(device, kernel, packed):
     for g, (index, count) in enumerate(zip(active_host, counts_host)):
         count = min(max(count, 0), rows) if 0 <= index < weight_groups else 0
         assert not got[g, count:].any(), g
-        if count and checked < 40:  # the CPU product of every group would take minutes
+        if count and checked < compared:  # the CPU product of every group would take minutes
             close(got[g, :count], x[g, :count], sx[g, :count], weights[index].cpu().numpy(),
                   scales[index].cpu().numpy(), packed, 32)
             checked += 1
         elif count:
             assert got[g, :count].any(), g
-    assert checked == 40
+    assert checked == compared
 
 
 def test_forced_tile_kernel_refuses_what_it_cannot_run(device):
