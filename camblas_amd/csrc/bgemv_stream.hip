@@ -81,7 +81,14 @@ __device__ __forceinline__ unsigned round_pack_bf16x2(float lo, float hi)
 // in a different (but fixed) order than a row kernel's, so the scale may differ in its last bit.
 // (FUSE: 0 none, 1 the normalised input, 2 the residual epilogue; compile-time, because a branch in
 // the loop keeps the compiler from counting the loads in flight and makes every wait a wait for all)
-template <int NT, int MT, int KT, bool GATED, int FUSE = 0>
+//
+// EXACT: K is whole K steps. Then every load is a buffer load whose lane offset never changes (row and
+// chunk) with the K position in the scalar offset, and a step past the end reads through an empty
+// descriptor (zeros, no memory request), so a K step costs no address arithmetic and no masks on the
+// vector ALU. A workgroup has one wavefront per SIMD and its phases run one after another, so at three
+// and four token tiles those instructions were part of the step time ([28672, 8192] x 64 tokens: 203
+// vector-ALU instructions per wavefront and step, of which 28 are matrix instructions).
+template <int NT, int MT, int KT, bool GATED, int FUSE = 0, bool EXACT = false>
 __global__ __launch_bounds__(WAVES * 64) void bgemv_stream_kernel(StreamParams p)
 {
     constexpr bool NORMALISE = FUSE == 1, RESIDUAL = FUSE == 2 && !GATED;
@@ -123,8 +130,18 @@ __global__ __launch_bounds__(WAVES * 64) void bgemv_stream_kernel(StreamParams p
     const unsigned short *a2_base = GATED ? p.w2 + size_t(n0) * p.lda : a_base;
     // (the launcher keeps 64 rows of x within 2 GB)
     const int x_rows = p.m - m0 < XROWS ? p.m - m0 : XROWS;
-    const __amdgpu_buffer_rsrc_t x_resource =
-        make_resource(p.x + size_t(m0) * p.ldb, (unsigned(x_rows - 1) * unsigned(p.ldb) + unsigned(p.k)) * 2u);
+    const unsigned x_bytes = (unsigned(x_rows - 1) * unsigned(p.ldb) + unsigned(p.k)) * 2u;
+    const __amdgpu_buffer_rsrc_t x_resource = make_resource(p.x + size_t(m0) * p.ldb, x_bytes);
+    // EXACT: the weight rows of the workgroup (the launcher keeps them within 4 GB) and every lane's fixed offsets
+    const int w_rows = p.n - n0 < ROWS ? p.n - n0 : ROWS;
+    const unsigned w_bytes = (unsigned(w_rows - 1) * unsigned(p.lda) + unsigned(p.k)) * 2u;
+    unsigned a_lane[NT], b_lane[MT];
+#pragma unroll
+    for (int i = 0; i < NT; ++i)
+        a_lane[i] = (a_off[i] + unsigned(chunk) * 8u) * 2u;
+#pragma unroll
+    for (int j = 0; j < MT; ++j)
+        b_lane[j] = b_off[j] + unsigned(chunk) * 16u; // (a row past the end stays outside the descriptor)
     // LDS slot of this thread's chunk inside a 16-row pass; passes are 256 slots apart
     const int store_slot = pass_row * CH + (chunk ^ pass_row);
     static_assert(CH == 16 || CH == 32, "XOR swizzle covers the low four chunk bits");
@@ -147,6 +164,27 @@ __global__ __launch_bounds__(WAVES * 64) void bgemv_stream_kernel(StreamParams p
     // a 470 MB stream would otherwise keep evicting (measured: 5.7 -> 6.3 TB/s); x is re-read by
     // every workgroup and is loaded normally.
     auto fetch = [&](int step, u32x4_t(&a)[KT][NT], u32x4_t(&b)[KT][MT], u32x4_t(&norm)[NORMALISE ? KT : 1]) {
+        if constexpr (EXACT) {
+            const bool alive = step < k_tiles;
+            const __amdgpu_buffer_rsrc_t gate_rows = make_resource(a_base, alive ? w_bytes : 0u);
+            const __amdgpu_buffer_rsrc_t up_rows = make_resource(a2_base, alive ? w_bytes : 0u);
+            const __amdgpu_buffer_rsrc_t token_rows = make_resource(p.x + size_t(m0) * p.ldb, alive ? x_bytes : 0u);
+            const int step_bytes = rotated(step) * (BK * KT * 2);
+#pragma unroll
+            for (int t = 0; t < KT; ++t) {
+#pragma unroll
+                for (int i = 0; i < NT; ++i) // (cache policy 2: non-temporal, as below)
+                    a[t][i] = __builtin_amdgcn_raw_buffer_load_b128(i < HALF ? gate_rows : up_rows, int(a_lane[i]),
+                                                                    step_bytes + t * BK * 2, 2);
+#pragma unroll
+                for (int j = 0; j < MT; ++j)
+                    b[t][j] = __builtin_amdgcn_raw_buffer_load_b128(token_rows, int(b_lane[j]), step_bytes + t * BK * 2, 0);
+                if constexpr (NORMALISE)
+                    norm[t] = *reinterpret_cast<const u32x4_t *>(
+                        p.norm_weight + (alive ? rotated(step) * (BK * KT) + t * BK + chunk * 8 : 0));
+            }
+            return;
+        }
         // padding steps past the end (their data is masked away) all read one cached line
         const unsigned live = step < k_tiles ? 0xffffffffu : 0u;
         const int tile_k = rotated(step) * (BK * KT) + chunk * 8;
@@ -184,7 +222,8 @@ __global__ __launch_bounds__(WAVES * 64) void bgemv_stream_kernel(StreamParams p
         const int tile_k = rotated(step) * (BK * KT) + chunk * 8;
 #pragma unroll
         for (int t = 0; t < KT; ++t) {
-            const unsigned mask = step < k_tiles && tile_k + t * BK < p.k ? 0xffffffffu : 0u;
+            // (EXACT: what lies past the end was read as zeros)
+            const unsigned mask = EXACT || (step < k_tiles && tile_k + t * BK < p.k) ? 0xffffffffu : 0u;
             u32x4_t *base = lds + stage * STAGE_SLOTS + t * BLOCK_SLOTS + store_slot;
 #pragma unroll
             for (int i = 0; i < NT; ++i)
@@ -464,9 +503,12 @@ hipError_t launch_one(hipStream_t stream, const StreamParams &p, int shares = 1)
     if constexpr (NT * KT > 8 || lds_bytes > 128 * 1024) {
         return hipErrorInvalidValue;
     } else {
-        auto kernel = bgemv_stream_kernel<NT, MT, KT, GATED, FUSE>;
-        static LdsLimitFlags limits; // (one per instantiation)
-        const hipError_t status = raise_lds_limit(limits, reinterpret_cast<const void *>(kernel), lds_bytes);
+        // whole K steps and a workgroup's weight rows within one 4 GB descriptor: the variant without
+        // address arithmetic and masks in its K loop
+        const bool exact = p.k % (32 * WAVES * KT) == 0 && (size_t(NT * 16 - 1) * size_t(p.lda) + size_t(p.k)) * 2 < (size_t(1) << 32);
+        auto kernel = exact ? bgemv_stream_kernel<NT, MT, KT, GATED, FUSE, true> : bgemv_stream_kernel<NT, MT, KT, GATED, FUSE, false>;
+        static LdsLimitFlags limits[2]; // (one per instantiation)
+        const hipError_t status = raise_lds_limit(limits[exact ? 1 : 0], reinterpret_cast<const void *>(kernel), lds_bytes);
         if (status != hipSuccess)
             return status;
         constexpr int rows = (GATED ? NT / 2 : NT) * 16;

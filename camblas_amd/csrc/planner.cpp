@@ -70,6 +70,19 @@ int fp8_stream_row_tiles(int outputs, int token_tiles, int compute_units, int li
 // weight rows (projections with few outputs) take two blocks per step so that enough bytes are in
 // flight per compute unit; measured on 8192- and 10240-row projections, two blocks beat one by
 // 10-20 % up to three row tiles, and four blocks or more lose again.
+// 33..64 tokens on a projection too narrow for one workgroup per compute unit: the number of workgroups
+// K is divided over so that each takes 64 to 128 weight rows, if K is long enough for that many shares
+// (0: none is)
+int narrow_stream_shares(int outputs, int k, int compute_units)
+{
+    for (const int shares : {2, 4}) {
+        const int row_tiles = ceil_div(shares * ceil_div(outputs, 16), compute_units);
+        if (row_tiles >= 4 && row_tiles <= 8 && k >= (shares == 2 ? 8192 : 14336))
+            return shares;
+    }
+    return 0;
+}
+
 int stream_depth_log2(int row_tiles, int token_tiles, int k)
 {
     return row_tiles <= 3 && (row_tiles + token_tiles) * 2 <= 16 && k >= 2048 ? 1 : 0;
@@ -246,15 +259,25 @@ Plan make_plan(int dtype, int algorithm, bool trans_a, bool trans_b, int m, int 
                 plan.split_k = 2;
             }
         } else if (tokens <= 64 && k >= 8192 &&
-                   ceil_div(2 * ceil_div(outputs, 16), compute_units) >= (tokens >= 40 ? 5 : 6)) {
+                   ceil_div(2 * ceil_div(outputs, 16), compute_units) >= 5) {
             // 33..64 tokens on a projection of 10240 to 16384 rows: the streaming kernel with K
             // divided over two workgroups per tile and 80 to 128 rows each (one workgroup per
             // compute unit) beats the register-staged tiles below by 15-25 % from 12288 rows on
             // (measured: [12288, 8192] 46-48 vs 55-58 us, [16384, 8192] 58-59 vs 71-74,
-            // [12288, 16384] 79-81 vs 100-106) and from 40 tokens at 10240 rows (40-41 vs 43-48)
+            // [12288, 16384] 79-81 vs 100-106; [10240, 8192] 32 vs 41 at 33 tokens, 34.5 at 64)
             plan.family = FAMILY_STREAM;
             plan.kernel = 10 * std::min(8, ceil_div(2 * ceil_div(outputs, 16), compute_units)) + (tokens <= 48 ? 3 : 4);
             plan.split_k = 2;
+        } else if (const int shares = narrow_stream_shares(outputs, k, compute_units); tokens <= 64 && shares) {
+            // 33..64 tokens on a narrow projection with a long K: the streaming kernel again, K divided over
+            // two or four workgroups of 64 to 128 rows each, about one workgroup per compute unit (the
+            // token rows a workgroup re-reads through L2 are what costs here, and that traffic falls
+            // with the rows per workgroup). Measured against the register-staged tiles of the branch
+            // below at 33 / 48 / 64 tokens: [8192, 8192] 27 / 28 / 31 against 32 / 33 / 35 us,
+            // [8192, 28672] 78 / 83 / 95 against 88 / 92 / 97, [4096, 14336] 26 / 27 / 31 against 30 / 31 / 32.
+            plan.family = FAMILY_STREAM;
+            plan.kernel = 10 * ceil_div(shares * ceil_div(outputs, 16), compute_units) + (tokens <= 48 ? 3 : 4);
+            plan.split_k = shares;
         } else if (tokens <= 64) {
             // 33..64 tokens on a narrow projection: the undivided streaming kernel would have 32-48
             // weight rows per workgroup and re-read as many token rows through L2; 128 x 64

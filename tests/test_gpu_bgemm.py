@@ -82,10 +82,13 @@ STREAM_CODES = [
 
 @pytest.mark.parametrize("code", STREAM_CODES)
 @pytest.mark.parametrize("n_out,m_rows,pad", [(300, 70, 4), (301, 9, 4), (113, 1, 7)])
-def test_streaming_kernel_every_variant(device, code, n_out, m_rows, pad):
-    # ragged feature count, token counts that span and underfill the token tiles, K tail (328 is
-    # not a multiple of the 128-deep step), padded leading dimensions
-    k = 328
+@pytest.mark.parametrize("k", [328, 640, 3072])
+def test_streaming_kernel_every_variant(device, code, n_out, m_rows, pad, k):
+    # ragged feature count, token counts that span and underfill the token tiles, padded leading
+    # dimensions; K with a tail (328 is not a multiple of the 128-deep step), and K in whole steps, which
+    # takes the variant of the kernel whose loads need no masks (640: five steps of one block, a tail for
+    # the deeper steps; 3072: an even number of steps of one to four blocks and three of eight), so an odd
+    # number of steps, whose last pair ends with a step past the end, occurs in both
     lda, ldb, ldc = k + 8, k + 16, n_out + pad
     w = oracle.fill_normal_bf16(120 + code, (n_out * lda,))
     x = oracle.fill_normal_bf16(140 + code, (m_rows * ldb,))
@@ -738,6 +741,28 @@ def test_mid_width_projection_at_33_to_64_tokens(device, outputs, tokens):
     w = (torch.randn((outputs, inner), device=device, generator=generator) * 0.02).to(torch.bfloat16)
     x = torch.randn((tokens, inner), device=device, generator=generator).to(torch.bfloat16)
     y = _kernels.matmul(x, w.t())
+    rows = torch.cat([torch.arange(0, outputs, 509, device=device), torch.tensor([outputs - 1], device=device)])
+    want = x.double() @ w[rows].double().t()
+    got = y[:, rows].double()
+    assert float((got - want).norm() / want.norm()) <= TOLERANCE
+    bound = 2.0**-7 * want.abs() + 1e-4 * want.abs().max()
+    assert bool(((got - want).abs() <= bound).all())
+
+
+@pytest.mark.parametrize("outputs,inner,tokens,shares", [(8192, 8192, 33, 2), (8192, 28672, 48, 2), (4096, 14336, 64, 4),
+                                                         (10240, 8192, 33, 2)])
+def test_narrow_projection_at_33_to_64_tokens(device, outputs, inner, tokens, shares):
+    # projections with too few rows for a workgroup per compute unit: the streaming kernel with K divided
+    # over two or four workgroups of 64 to 128 rows (about one workgroup per compute unit in all); sampled
+    # output rows against FP64, and the same bits on every launch (the shares are added in index order)
+    text = _native.plan_describe(2, "T", "N", outputs, tokens, inner, inner, inner, outputs)[1]
+    assert "stream" in text and f"tokens={48 if tokens <= 48 else 64}" in text and f"k_shares={shares}" in text, text
+    generator = torch.Generator(device=device).manual_seed(outputs + tokens)
+    w = (torch.randn((outputs, inner), device=device, generator=generator) * 0.02).to(torch.bfloat16)
+    x = torch.randn((tokens, inner), device=device, generator=generator).to(torch.bfloat16)
+    y = _kernels.matmul(x, w.t())
+    for _ in range(20):
+        assert torch.equal(_kernels.matmul(x, w.t()), y)
     rows = torch.cat([torch.arange(0, outputs, 509, device=device), torch.tensor([outputs - 1], device=device)])
     want = x.double() @ w[rows].double().t()
     got = y[:, rows].double()
