@@ -705,6 +705,22 @@ def extras(torch, _kernels, _native, device, normal):
         "plan": _native.plan_describe(2, "N", "N", outputs, tokens, inner, outputs, inner, outputs)[1],
     }
     del copies, x, y
+    # decode batches between the streaming kernel's two- and four-tile forms, on the widest and on a narrow
+    # projection of the layer (three weight copies rotate)
+    mid = {}
+    for outputs, inner in ((28672, 8192), (8192, 8192)):
+        copies = [normal((outputs, inner), 0.02) for _ in range(3)]
+        for tokens in (48, 64):
+            x = normal((tokens, inner))
+            y = torch.empty((tokens, outputs), dtype=torch.bfloat16, device=device)
+            seconds = event_time(torch, lambda i: _kernels.matmul(x, copies[i % 3].t(), out=y), 10, 60)
+            mid["%dx%d_%d_tokens" % (outputs, inner, tokens)] = {
+                "us": round(seconds * 1e6, 1),
+                "roofline": roofline_of("hbm", outputs * inner * 2 + tokens * (inner + outputs) * 2, seconds),
+                "plan": _native.plan_describe(2, "T", "N", outputs, tokens, inner, inner, inner, outputs)[1],
+            }
+        del copies, x, y
+    found["bf16_linear_48_and_64_tokens"] = mid
     # FP8 block-scaled linear; the decode sizes rotate three weight copies (396 MB) so that the
     # weights come from HBM rather than from the 256 MB last-level cache
     outputs, inner = 18432, 7168
