@@ -31,6 +31,10 @@ CORE_SOURCES = (
     "gemv_f32.hip",
     "bgemm_tn.hip",
     "bgemv_stream.hip",
+    "bgemv_stream_deep.hip",
+    "bgemv_stream_norm.hip",
+    "bgemv_stream_residual.hip",
+    "bgemv_stream_gated.hip",
     "bgemm_dma.hip",
     "bgemm_wave4.hip",
     "bgemm_nn.hip",
