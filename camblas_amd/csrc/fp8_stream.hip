@@ -53,7 +53,7 @@ __global__ __launch_bounds__(WAVES * 64) void fp8_stream_kernel(Fp8StreamParams 
     __shared__ float scale_table[SCALE_ROWS * SCALE_PITCH];
     // after the last step the wavefront's patches hold its partial sums instead
     static_assert(NT * MT * 64 <= TILES * 128, "partial sums must fit the wavefront's patches");
-    const int thread = threadIdx.x, lane = thread % 64, wave = thread / 64;
+    const int thread = threadIdx.x, lane = thread % 64, wave = __builtin_amdgcn_readfirstlane(thread / 64);
     const int row = lane % 16, chunk = lane / 16; // operand row / token, 32-byte chunk of the group
     const int load_row = lane / 8, piece = lane % 8; // load layout: 8 lanes per 128-byte line
     const int n0 = blockIdx.x * (NT * 16), m0 = blockIdx.y * (MT * 16);
@@ -80,10 +80,8 @@ __global__ __launch_bounds__(WAVES * 64) void fp8_stream_kernel(Fp8StreamParams 
             token_offset[j][h] = m0 + m < p.m ? unsigned(m) * unsigned(p.k) + unsigned(piece) * 16u : 0x80000000u;
         }
     }
-    const __amdgpu_buffer_rsrc_t weight_resource = make_resource(
-        p.w + size_t(n0) * p.k, unsigned(p.n - n0 < NT * 16 ? p.n - n0 : NT * 16) * unsigned(p.k));
-    const __amdgpu_buffer_rsrc_t token_resource = make_resource(
-        p.a + size_t(m0) * p.k, unsigned(p.m - m0 < MT * 16 ? p.m - m0 : MT * 16) * unsigned(p.k));
+    const unsigned weight_bytes = unsigned(p.n - n0 < NT * 16 ? p.n - n0 : NT * 16) * unsigned(p.k);
+    const unsigned token_bytes = unsigned(p.m - m0 < MT * 16 ? p.m - m0 : MT * 16) * unsigned(p.k);
     // rows of the scale table: tokens m0 .., then the weight blocks first_block and first_block + 1
     const int first_block = n0 / 128;
     int ws_row[NT], as_row[MT];
@@ -137,18 +135,21 @@ __global__ __launch_bounds__(WAVES * 64) void fp8_stream_kernel(Fp8StreamParams 
         live = exists ? 1.f : 0.f;
         g = g < p.groups ? g : p.groups - 1;
         group = g;
-        const unsigned offset = unsigned(g) * GROUP, dead = exists ? 0u : 0x80000000u;
+        // The lane offsets never change: the group's position along K is the scalar offset, and a step past
+        // the end reads through descriptors of no bytes (zeros, no memory request), so a fetch costs the
+        // vector ALU nothing (a wavefront runs its fetches, LDS transposes and products one after another).
+        const int offset = g * GROUP;
+        const __amdgpu_buffer_rsrc_t weight_resource = make_resource(p.w + size_t(n0) * p.k, exists ? weight_bytes : 0u);
+        const __amdgpu_buffer_rsrc_t token_resource = make_resource(p.a + size_t(m0) * p.k, exists ? token_bytes : 0u);
 #pragma unroll
         for (int t = 0; t < TILES; ++t)
 #pragma unroll
             for (int h = 0; h < 2; ++h) {
                 // (weights: read once, so non-temporal, cache policy bit 1)
                 if (t < NT)
-                    data[t][h] = __builtin_amdgcn_raw_buffer_load_b128(weight_resource,
-                                                                       int((weight_offset[t < NT ? t : 0][h] + offset) | dead), 0, 2);
+                    data[t][h] = __builtin_amdgcn_raw_buffer_load_b128(weight_resource, int(weight_offset[t < NT ? t : 0][h]), offset, 2);
                 else
-                    data[t][h] = __builtin_amdgcn_raw_buffer_load_b128(
-                        token_resource, int((token_offset[t < NT ? 0 : t - NT][h] + offset) | dead), 0, 0);
+                    data[t][h] = __builtin_amdgcn_raw_buffer_load_b128(token_resource, int(token_offset[t < NT ? 0 : t - NT][h]), offset, 0);
             }
     };
 
