@@ -179,9 +179,11 @@ extern "C" int camblas_cuda_fp8_decode(camblas_cuda_context *context, int output
             !apart(output, {input, weight, input_scale, weight_scale}))
             return entry.refuse("invalid FP8 decode buffers");
         context->counts[4]++;
+        const int forced = context->override_kernel; // (tests: 301 / 302 / 304 force the wavefronts per workgroup)
         return entry.finish(launch_fp8_block32_decode(context->stream, outputs, inner, input, input_scale,
                                                       input_scale_stride, weight, weight_scale,
-                                                      weight_scale_row_stride, weight_scale_column_stride, output),
+                                                      weight_scale_row_stride, weight_scale_column_stride, output,
+                                                      forced == 301 || forced == 302 || forced == 304 ? forced - 300 : 0),
                             "FP8 block-32 decode");
     });
 }

@@ -275,9 +275,10 @@ hipError_t launch_fp8_stream(hipStream_t stream, int row_tiles, int token_tiles,
                              int inner, const void *a, const float *a_scale, const void *w,
                              const float *w_scale, void *out);
 // Single-token product with 32-wide FP32 scale blocks; sx null: x is BF16 and quantised on the fly.
+// forced_waves 1, 2 or 4: wavefronts per workgroup (0: by the number of outputs).
 hipError_t launch_fp8_block32_decode(hipStream_t stream, int outputs, int inner, const void *x,
                                      const float *sx, int sx_stride, const void *w, const float *sw,
-                                     int sw_row, int sw_col, void *out);
+                                     int sw_row, int sw_col, void *out, int forced_waves = 0);
 // One token through an FP8 (1x128 . 128x128 scales) mixture-of-experts layer: gate/up products,
 // clipped SiLU-multiply, down products, routed sum. scratch: fp8_moe_decode_scratch_bytes().
 size_t fp8_moe_decode_scratch_bytes(int choices, int width);

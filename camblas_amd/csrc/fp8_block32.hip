@@ -14,6 +14,11 @@
 // with row shifts (DPP) and chained there. W is loaded with eight lanes per 128-byte line
 // (non-temporal, eight steps in flight per wavefront) and transposed to the operand layout
 // through a private swizzled LDS patch, as in the 128-block streaming kernel.
+// A wavefront runs its steps one after another with few wavefronts per SIMD to hide them (16 rows per
+// wavefront: 1152 wavefronts for 18432 outputs), so the loop is kept short: the weight scales of the
+// wavefront's rows are copied to LDS once instead of being fetched per step, and when K is whole steps
+// (EXACT) the weight loads are buffer loads with fixed lane offsets and the K position in the scalar
+// offset, a step past the end reading through a descriptor of no bytes.
 #include "common.hpp"
 #include "device.hpp"
 #include "dma.hpp"
@@ -31,17 +36,23 @@ struct Block32Params {
     int n, k, sx_stride, sw_row, sw_col;
 };
 
-constexpr int WAVES = 4, DEPTH = 8, STEP = 128, MAX_K = 8192;
+constexpr int DEPTH = 8, STEP = 128, MAX_K = 8192;
 constexpr int UNIT = 0x7f7f7f7f; // E8M0 exponent 127 = scale 1.0 in every byte
 
-template <bool QUANTISE>
+// WAVES: wavefronts (of 16 rows each) per workgroup. Few outputs take fewer, so that the wavefronts spread
+// over more compute units: what a compute unit can draw is bounded by what it keeps in flight
+// ([4096, 7168]: 16.0 us on 64 workgroups of four wavefronts, measured below on 256 of one).
+template <bool QUANTISE, bool EXACT, int WAVES>
 __global__ __launch_bounds__(WAVES * 64) void fp8_block32_decode_kernel(Block32Params p)
 {
+    static_assert(!QUANTISE || WAVES == 4, "the quantiser takes one 32-value block per thread");
     // x and its scales, zero-padded to a whole number of DEPTH-step rounds
     __shared__ __attribute__((aligned(16))) unsigned x_words[MAX_K / 4];
     __shared__ __attribute__((aligned(16))) float x_scale[MAX_K / 32];
-    __shared__ __attribute__((aligned(16))) u32x4_t patch[WAVES][128];
-    const int thread = threadIdx.x, lane = thread % 64, wave = thread / 64;
+    __shared__ __attribute__((aligned(16))) u32x4_t patch[WAVES][2 * 128]; // two steps' tiles
+    // the scales of each wavefront's rows (16 rows lie in one 32-row block: one scale per 32-input block)
+    __shared__ float w_scale[WAVES][MAX_K / 32];
+    const int thread = threadIdx.x, lane = thread % 64, wave = __builtin_amdgcn_readfirstlane(thread / 64);
     const int blocks = p.k / 32, steps = (p.k + STEP - 1) / STEP;
     const int rounds = (steps + DEPTH - 1) / DEPTH, padded_steps = rounds * DEPTH;
 
@@ -62,15 +73,20 @@ __global__ __launch_bounds__(WAVES * 64) void fp8_block32_decode_kernel(Block32P
     // Loads only (nothing here may use a loaded value). Bytes past the end of a row in a partial
     // last step, and whole steps past the end, re-read the row's last 16 bytes: x is zero there.
     u32x4_t raw[DEPTH][2];
-    float sw_reg[DEPTH];
-    auto fetch = [&](int step, u32x4_t(&data)[2], float &scale) {
-        int offset = step * STEP + piece * 16;
-        offset = offset < p.k ? offset : p.k - 16;
-        data[0] = __builtin_nontemporal_load(reinterpret_cast<const u32x4_t *>(row_base[0] + offset));
-        data[1] = __builtin_nontemporal_load(reinterpret_cast<const u32x4_t *>(row_base[1] + offset));
-        int b = step * 4 + (column & 3);
-        b = b < blocks ? b : blocks - 1;
-        scale = sw_row[size_t(b) * p.sw_col];
+    const unsigned lane_offset[2] = {unsigned(load_row) * unsigned(p.k) + unsigned(piece) * 16u,
+                                     unsigned(load_row + 8) * unsigned(p.k) + unsigned(piece) * 16u};
+    auto fetch = [&](int step, u32x4_t(&data)[2]) {
+        if constexpr (EXACT) { // (cache policy 2: non-temporal)
+            const __amdgpu_buffer_rsrc_t rows =
+                make_resource(p.w + size_t(first_row) * p.k, step < steps ? 16u * unsigned(p.k) : 0u);
+            data[0] = __builtin_amdgcn_raw_buffer_load_b128(rows, int(lane_offset[0]), step * STEP, 2);
+            data[1] = __builtin_amdgcn_raw_buffer_load_b128(rows, int(lane_offset[1]), step * STEP, 2);
+        } else {
+            int offset = step * STEP + piece * 16;
+            offset = offset < p.k ? offset : p.k - 16;
+            data[0] = __builtin_nontemporal_load(reinterpret_cast<const u32x4_t *>(row_base[0] + offset));
+            data[1] = __builtin_nontemporal_load(reinterpret_cast<const u32x4_t *>(row_base[1] + offset));
+        }
     };
 
     // ---- the token: its loads are issued first, the first DEPTH weight steps right behind them,
@@ -78,11 +94,10 @@ __global__ __launch_bounds__(WAVES * 64) void fp8_block32_decode_kernel(Block32P
     // does not wait for the weights): the weight stream's first latency overlaps the staging.
     // Every loop below has a fixed trip count (MAX_K bounds it) so that the compiler can count the
     // loads in flight instead of waiting for all of them.
-    static_assert(MAX_K / 32 <= WAVES * 64, "one 32-value block per thread");
-    constexpr int WORDS_PER_THREAD = MAX_K / 4 / (WAVES * 64);
+    constexpr int WORDS_PER_THREAD = MAX_K / 4 / (WAVES * 64), BLOCKS_PER_THREAD = MAX_K / 32 / (WAVES * 64);
     const unsigned *source = static_cast<const unsigned *>(p.x);
     unsigned staged[QUANTISE ? 16 : WORDS_PER_THREAD];
-    float staged_scale = 0.f;
+    float staged_scale[BLOCKS_PER_THREAD] = {};
     if constexpr (QUANTISE) {
         const int b = thread < blocks ? thread : blocks - 1; // BF16 pairs of block `thread`
 #pragma unroll
@@ -94,14 +109,29 @@ __global__ __launch_bounds__(WAVES * 64) void fp8_block32_decode_kernel(Block32P
             const int word = thread + i * WAVES * 64;
             staged[i] = source[word < p.k / 4 ? word : p.k / 4 - 1];
         }
-        staged_scale = p.sx[size_t(thread < blocks ? thread : blocks - 1) * p.sx_stride];
+#pragma unroll
+        for (int i = 0; i < BLOCKS_PER_THREAD; ++i) {
+            const int b = thread + i * WAVES * 64;
+            staged_scale[i] = p.sx[size_t(b < blocks ? b : blocks - 1) * p.sx_stride];
+        }
+    }
+    // the wavefront's weight scales, block lane + 64 i (past the end: the last one again; x is zero there)
+    constexpr int SCALES_PER_LANE = MAX_K / 32 / 64;
+    float staged_weight_scale[SCALES_PER_LANE];
+#pragma unroll
+    for (int i = 0; i < SCALES_PER_LANE; ++i) {
+        const int b = lane + 64 * i;
+        staged_weight_scale[i] = sw_row[size_t(b < blocks ? b : blocks - 1) * p.sw_col];
     }
     __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
     for (int d = 0; d < DEPTH; ++d) {
-        fetch(d, raw[d], sw_reg[d]);
+        fetch(d, raw[d]);
         __builtin_amdgcn_sched_barrier(0);
     }
+#pragma unroll
+    for (int i = 0; i < SCALES_PER_LANE; ++i)
+        w_scale[wave][lane + 64 * i] = staged_weight_scale[i];
     if constexpr (QUANTISE) {
         const int b = thread;
         if (b < padded_steps * 4) {
@@ -144,8 +174,12 @@ __global__ __launch_bounds__(WAVES * 64) void fp8_block32_decode_kernel(Block32P
             if (word < padded_steps * 32)
                 x_words[word] = word < p.k / 4 ? staged[i] : 0u;
         }
-        if (thread < padded_steps * 4)
-            x_scale[thread] = thread < blocks ? staged_scale : 0.f;
+#pragma unroll
+        for (int i = 0; i < BLOCKS_PER_THREAD; ++i) {
+            const int b = thread + i * WAVES * 64;
+            if (b < padded_steps * 4)
+                x_scale[b] = b < blocks ? staged_scale[i] : 0.f;
+        }
     }
     // (not __syncthreads(): its fence would wait for every weight load issued above; the LDS
     // stores are waited for explicitly, the weight loads stay in flight)
@@ -154,47 +188,66 @@ __global__ __launch_bounds__(WAVES * 64) void fp8_block32_decode_kernel(Block32P
         return; // no barrier below this point
 
     float sum[4] = {0.f, 0.f, 0.f, 0.f};
-    auto multiply = [&](int step, const u32x4_t(&data)[2], float scale) {
-        mine[store_slot[0]] = data[0];
-        mine[store_slot[1]] = data[1];
+    // Two steps at a time: their LDS round trips, matrix instructions and row shifts overlap, and only the
+    // chains of fused multiply-adds run in the order of the blocks (a wavefront has nobody to hide a step's
+    // latencies behind: [4096, 7168] took 56 steps x 0.24 us whatever the memory system did).
+    auto multiply = [&](int step, const u32x4_t(&first)[2], const u32x4_t(&second)[2]) {
+        mine[store_slot[0]] = first[0];
+        mine[store_slot[1]] = first[1];
+        mine[128 + store_slot[0]] = second[0];
+        mine[128 + store_slot[1]] = second[1];
         // other lanes' stores are read below: keep the compiler from moving the loads up (the
         // hardware executes one wavefront's LDS operations in order)
         __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
         __builtin_amdgcn_wave_barrier();
         __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
-        u32x4_t lo = mine[read_slot[0]], hi = mine[read_slot[1]];
-        const u32x4_t *x_step = reinterpret_cast<const u32x4_t *>(x_words) + step * 8 + chunk * 2;
-        u32x4_t x_lo = x_step[0], x_hi = x_step[1];
         const unsigned keep = column == chunk ? 0xffffffffu : 0u; // block c only in column c
-        i32x8_t a = {int(lo[0]), int(lo[1]), int(lo[2]), int(lo[3]),
-                     int(hi[0]), int(hi[1]), int(hi[2]), int(hi[3])};
-        i32x8_t b = {int(x_lo[0] & keep), int(x_lo[1] & keep), int(x_lo[2] & keep), int(x_lo[3] & keep),
-                     int(x_hi[0] & keep), int(x_hi[1] & keep), int(x_hi[2] & keep), int(x_hi[3] & keep)};
-        f32x4_t dot = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(
-            a, b, f32x4_t{0.f, 0.f, 0.f, 0.f}, 0, 0, 0, UNIT, 0, UNIT);
-        const f32x4_t scales = *reinterpret_cast<const f32x4_t *>(x_scale + step * 4);
+        float scaled[2][4];
+        f32x4_t scales[2];
 #pragma unroll
-        for (int r = 0; r < 4; ++r) {
-            // column c holds block c of row 4*chunk + r; bring blocks 1..3 to column 0 and chain
-            const float scaled = __fmul_rn(dot[r], scale);
-            const float block1 = dpp_move<0x101>(scaled), block2 = dpp_move<0x102>(scaled),
-                        block3 = dpp_move<0x103>(scaled);
-            sum[r] = fmaf(scaled, scales[0], sum[r]);
-            sum[r] = fmaf(block1, scales[1], sum[r]);
-            sum[r] = fmaf(block2, scales[2], sum[r]);
-            sum[r] = fmaf(block3, scales[3], sum[r]);
+        for (int half = 0; half < 2; ++half) {
+            const u32x4_t lo = mine[128 * half + read_slot[0]], hi = mine[128 * half + read_slot[1]];
+            const u32x4_t *x_step = reinterpret_cast<const u32x4_t *>(x_words) + (step + half) * 8 + chunk * 2;
+            const u32x4_t x_lo = x_step[0], x_hi = x_step[1];
+            const i32x8_t a = {int(lo[0]), int(lo[1]), int(lo[2]), int(lo[3]),
+                               int(hi[0]), int(hi[1]), int(hi[2]), int(hi[3])};
+            const i32x8_t b = {int(x_lo[0] & keep), int(x_lo[1] & keep), int(x_lo[2] & keep), int(x_lo[3] & keep),
+                               int(x_hi[0] & keep), int(x_hi[1] & keep), int(x_hi[2] & keep), int(x_hi[3] & keep)};
+            const f32x4_t dot = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(
+                a, b, f32x4_t{0.f, 0.f, 0.f, 0.f}, 0, 0, 0, UNIT, 0, UNIT);
+            const float scale = w_scale[wave][(step + half) * 4 + (column & 3)];
+            scales[half] = *reinterpret_cast<const f32x4_t *>(x_scale + (step + half) * 4);
+#pragma unroll
+            for (int r = 0; r < 4; ++r)
+                scaled[half][r] = __fmul_rn(dot[r], scale);
         }
+#pragma unroll
+        for (int half = 0; half < 2; ++half)
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+                // column c holds block c of row 4*chunk + r; bring blocks 1..3 to column 0 and chain
+                const float value = scaled[half][r];
+                const float block1 = dpp_move<0x101>(value), block2 = dpp_move<0x102>(value),
+                            block3 = dpp_move<0x103>(value);
+                sum[r] = fmaf(value, scales[half][0], sum[r]);
+                sum[r] = fmaf(block1, scales[half][1], sum[r]);
+                sum[r] = fmaf(block2, scales[half][2], sum[r]);
+                sum[r] = fmaf(block3, scales[half][3], sum[r]);
+            }
         __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
         __builtin_amdgcn_wave_barrier();
     };
 
+    static_assert(DEPTH % 2 == 0, "steps go in pairs");
     for (int step = 0; step < padded_steps; step += DEPTH) {
 #pragma unroll
-        for (int d = 0; d < DEPTH; ++d) {
+        for (int d = 0; d < DEPTH; d += 2) {
             __builtin_amdgcn_sched_barrier(0);
-            multiply(step + d, raw[d], sw_reg[d]);
+            multiply(step + d, raw[d], raw[d + 1]);
             __builtin_amdgcn_sched_barrier(0);
-            fetch(step + d + DEPTH, raw[d], sw_reg[d]);
+            fetch(step + d + DEPTH, raw[d]);
+            __builtin_amdgcn_sched_barrier(0);
+            fetch(step + d + 1 + DEPTH, raw[d + 1]);
         }
     }
     if (column == 0) {
@@ -211,7 +264,7 @@ __global__ __launch_bounds__(WAVES * 64) void fp8_block32_decode_kernel(Block32P
 // and x 4-byte aligned.
 hipError_t launch_fp8_block32_decode(hipStream_t stream, int outputs, int inner, const void *x,
                                      const float *sx, int sx_stride, const void *w, const float *sw,
-                                     int sw_row, int sw_col, void *out)
+                                     int sw_row, int sw_col, void *out, int forced_waves)
 {
     if (outputs < 16 || outputs % 16 || inner < 32 || inner > MAX_K || inner % 32)
         return hipErrorInvalidValue;
@@ -226,11 +279,21 @@ hipError_t launch_fp8_block32_decode(hipStream_t stream, int outputs, int inner,
     p.sx_stride = sx_stride;
     p.sw_row = sw_row;
     p.sw_col = sw_col;
-    const unsigned grid = unsigned((outputs + WAVES * 16 - 1) / (WAVES * 16));
-    if (sx)
-        fp8_block32_decode_kernel<false><<<grid, WAVES * 64, 0, stream>>>(p);
-    else
-        fp8_block32_decode_kernel<true><<<grid, WAVES * 64, 0, stream>>>(p);
+    const bool exact = inner % STEP == 0; // (16 rows of at most 8192 bytes fit any descriptor)
+    const auto grid_of = [outputs](int waves) { return unsigned((outputs + waves * 16 - 1) / (waves * 16)); };
+    if (!sx) {
+        (exact ? fp8_block32_decode_kernel<true, true, 4> : fp8_block32_decode_kernel<true, false, 4>)<<<grid_of(4), 256, 0, stream>>>(p);
+        return launch_status();
+    }
+    // (one wavefront per workgroup spreads the wavefronts evenly over the compute units: [18432, 7168] 25.1 us
+    // against 29.9 with four, [4096, 7168] 13.6 against 16.2; the others are kept for tests)
+    const int waves = forced_waves ? forced_waves : 1;
+    switch (waves) {
+    case 1: (exact ? fp8_block32_decode_kernel<false, true, 1> : fp8_block32_decode_kernel<false, false, 1>)<<<grid_of(1), 64, 0, stream>>>(p); break;
+    case 2: (exact ? fp8_block32_decode_kernel<false, true, 2> : fp8_block32_decode_kernel<false, false, 2>)<<<grid_of(2), 128, 0, stream>>>(p); break;
+    case 4: (exact ? fp8_block32_decode_kernel<false, true, 4> : fp8_block32_decode_kernel<false, false, 4>)<<<grid_of(4), 256, 0, stream>>>(p); break;
+    default: return hipErrorInvalidValue;
+    }
     return launch_status();
 }
 } // namespace camblas_hip

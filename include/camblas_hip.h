@@ -404,7 +404,8 @@ int camblas_hip_plan_describe(int dtype, int algorithm, char trans_a, char trans
  * the call fail. (BF16: 20 + n the
  * direct-to-LDS tile n, of which 38 / 39 are the four-wavefront 256- and 320-row tiles and 40 the
  * 256-row tile for weights stored with their outputs contiguous; FP8 with FP32 scales: 36 the
- * four-wavefront 192 x 256 tile.)
+ * four-wavefront 192 x 256 tile; the single-token product with 32-wide scale blocks: 301 / 302 / 304
+ * one, two or four wavefronts per workgroup.)
  * TEST-ONLY: the override is state of the context it is set on (no other context sees it, and it
  * ends with the context), it bypasses the planner's eligibility rules, and a forced variant may be
  * far slower than the planner's choice or refuse shapes the planner would serve. Serving code never

@@ -317,6 +317,16 @@ def test_block32_decode_matches_ordered_oracle(device, outputs, inner):
     strided = _kernels.fp8_decode(fp8_tensor(x, device).view(1, -1), storage[:, 0].view(1, -1),
                                   fp8_tensor(w, device), torch.from_numpy(sw).to(device).T.contiguous().T)
     assert torch.equal(strided.view(torch.int16), out.view(torch.int16))
+    # the forms with two and four wavefronts per workgroup (the planned one has one) give the same bits
+    native = _native.context(device)
+    for code in (302, 304):
+        native.call("hip_set_plan_override", code, 0)
+        try:
+            forced = _kernels.fp8_decode(fp8_tensor(x, device).view(1, -1), torch.from_numpy(sx).to(device).view(1, -1),
+                                         fp8_tensor(w, device), torch.from_numpy(sw).to(device))
+        finally:
+            native.call("hip_set_plan_override", -1, 0)
+        assert torch.equal(forced.view(torch.int16), out.view(torch.int16)), code
 
 
 def test_block32_known_answers_graph_and_nan(device):
