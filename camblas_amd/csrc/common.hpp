@@ -270,7 +270,7 @@ hipError_t launch_fp8_dma(hipStream_t stream, int variant, int split_k, int rows
 hipError_t launch_fp8_wave4(hipStream_t stream, int rows, int outputs, int inner, const void *a, const float *a_scale,
                             const void *w, const float *w_scale, void *out, int out_pitch);
 hipError_t launch_fp8_split_sum(hipStream_t stream, int splits, size_t count, const float *partials, void *out);
-// row_tiles 1..8 (16 weight rows each), token_tiles 1, 2 or 4 (16 tokens each).
+// row_tiles 1..8 (16 weight rows each), token_tiles 1 to 4 (16 tokens each); product <= 20, sum <= 10.
 hipError_t launch_fp8_stream(hipStream_t stream, int row_tiles, int token_tiles, int rows, int outputs,
                              int inner, const void *a, const float *a_scale, const void *w,
                              const float *w_scale, void *out);

@@ -44,7 +44,9 @@ __global__ __launch_bounds__(WAVES * 64) void fp8_stream_kernel(Fp8StreamParams 
     // groups in flight per wavefront: three while the operand registers allow it
     constexpr int DEPTH = NT + MT <= 6 ? 3 : 2;
     constexpr int TILES = NT + MT; // weight tiles, then token tiles
-    __shared__ __attribute__((aligned(16))) u32x4_t patch[WAVES][TILES][128];
+    // (per wavefront: the 2 KB patches of its tiles, or, after the last step, its NT * MT partial tiles of 1 KB)
+    constexpr int PATCH = TILES * 128 > NT * MT * 64 ? TILES * 128 : NT * MT * 64;
+    __shared__ __attribute__((aligned(16))) u32x4_t patch[WAVES][PATCH];
     // The scales of the workgroup's tokens (one row of `groups` floats per token) and of the two
     // 128-row weight blocks its rows can lie in, copied to LDS once: a lane that fetched its
     // token's scale for every group itself would request a cache line per lane and group, the same
@@ -52,7 +54,6 @@ __global__ __launch_bounds__(WAVES * 64) void fp8_stream_kernel(Fp8StreamParams 
     constexpr int SCALE_ROWS = MT * 16 + 2, SCALE_PITCH = STREAM_SCALE_PITCH;
     __shared__ float scale_table[SCALE_ROWS * SCALE_PITCH];
     // after the last step the wavefront's patches hold its partial sums instead
-    static_assert(NT * MT * 64 <= TILES * 128, "partial sums must fit the wavefront's patches");
     const int thread = threadIdx.x, lane = thread % 64, wave = __builtin_amdgcn_readfirstlane(thread / 64);
     const int row = lane % 16, chunk = lane / 16; // operand row / token, 32-byte chunk of the group
     const int load_row = lane / 8, piece = lane % 8; // load layout: 8 lanes per 128-byte line
@@ -160,7 +161,7 @@ __global__ __launch_bounds__(WAVES * 64) void fp8_stream_kernel(Fp8StreamParams 
         for (int j = 0; j < MT; ++j)
             acc[i][j] = f32x4_t{0.f, 0.f, 0.f, 0.f};
     auto multiply = [&](const u32x4_t(&data)[TILES][2], int group, float live) {
-        u32x4_t *mine = &patch[wave][0][0];
+        u32x4_t *mine = &patch[wave][0];
         float ws[NT], as[MT];
 #pragma unroll
         for (int i = 0; i < NT; ++i)
@@ -224,7 +225,7 @@ __global__ __launch_bounds__(WAVES * 64) void fp8_stream_kernel(Fp8StreamParams 
     }
     // ---- every wavefront parks its partial sums in its own patches (nobody else reads those);
     // after one barrier tile t is summed in wavefront order 0, 1, 2, 3 by wavefront t % 4
-    f32x4_t *parked = reinterpret_cast<f32x4_t *>(&patch[wave][0][0]);
+    f32x4_t *parked = reinterpret_cast<f32x4_t *>(&patch[wave][0]);
 #pragma unroll
     for (int i = 0; i < NT; ++i)
 #pragma unroll
@@ -243,10 +244,10 @@ __global__ __launch_bounds__(WAVES * 64) void fp8_stream_kernel(Fp8StreamParams 
         const int n = n0 + i * 16 + chunk * 4;
         if (m >= p.m || n >= p.n)
             continue;
-        f32x4_t sum = reinterpret_cast<const f32x4_t *>(&patch[0][0][0])[index * 64 + lane];
+        f32x4_t sum = reinterpret_cast<const f32x4_t *>(&patch[0][0])[index * 64 + lane];
 #pragma unroll
         for (int w = 1; w < WAVES; ++w)
-            sum = sum + reinterpret_cast<const f32x4_t *>(&patch[w][0][0])[index * 64 + lane];
+            sum = sum + reinterpret_cast<const f32x4_t *>(&patch[w][0])[index * 64 + lane];
         unsigned short *out = p.out + size_t(m) * p.n + n;
         if (n + 3 < p.n && vector_store) {
             u32x2_t packed = {pack_bf16x2(sum[0], sum[1]), pack_bf16x2(sum[2], sum[3])};
@@ -263,7 +264,7 @@ __global__ __launch_bounds__(WAVES * 64) void fp8_stream_kernel(Fp8StreamParams 
 template <int NT, int MT> hipError_t launch_one(hipStream_t stream, const Fp8StreamParams &p)
 {
     // the prefetch registers grow with NT + MT: keep both groups in flight inside the register file
-    if constexpr (NT * MT > 16 || NT + MT > 10) {
+    if constexpr (NT * MT > 20 || NT + MT > 10) {
         return hipErrorInvalidValue;
     } else {
         dim3 grid(unsigned((p.n + NT * 16 - 1) / (NT * 16)), unsigned((p.m + MT * 16 - 1) / (MT * 16)));
@@ -288,7 +289,8 @@ template <int MT> hipError_t launch_rows(hipStream_t stream, int row_tiles, cons
 }
 } // namespace
 
-// row_tiles 1..8 (16 weight rows each), token_tiles 1, 2 or 4 (16 tokens each); a, w 16-byte
+// row_tiles 1..8 (16 weight rows each), token_tiles 1 to 4 (16 tokens each), their product at most 20 and
+// their sum at most 10; a, w 16-byte
 // aligned, inner a multiple of 128.
 hipError_t launch_fp8_stream(hipStream_t stream, int row_tiles, int token_tiles, int rows, int outputs,
                              int inner, const void *a, const float *a_scale, const void *w,
@@ -315,6 +317,7 @@ hipError_t launch_fp8_stream(hipStream_t stream, int row_tiles, int token_tiles,
     switch (token_tiles) {
     case 1: return launch_rows<1>(stream, row_tiles, p);
     case 2: return launch_rows<2>(stream, row_tiles, p);
+    case 3: return launch_rows<3>(stream, row_tiles, p);
     case 4: return launch_rows<4>(stream, row_tiles, p);
     default: return hipErrorInvalidValue;
     }

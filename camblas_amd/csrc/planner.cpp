@@ -462,15 +462,30 @@ Plan make_plan(int dtype, int algorithm, bool trans_a, bool trans_b, int m, int 
     if (enough_rows && streamable && (n <= 32 || (n <= 64 && (!tiles_apply || k < 4096)))) {
         // decode batches: one streaming pass over the weights, whole K per workgroup; the row
         // tiles are limited by the operand registers (row_tiles * token_tiles <= 16, sum <= 10).
-        // From 33 tokens on the 64-token tiles below with divided K are faster (the streaming
-        // kernel's four token tiles gather four scale lines per lane and group: [18432, 7168] at
-        // 64 tokens 49 us against 33).
+        // From 33 tokens on the 64-token tiles below with divided K are faster, but for the wide
+        // projections of the rule that follows this one.
         const int token_tiles = n <= 16 ? 1 : n <= 32 ? 2 : 4;
         const int limit = std::min(16 / token_tiles, 10 - token_tiles);
         plan.family = FAMILY_FP8_STREAM;
         plan.kernel =
             10 * fp8_stream_row_tiles(m, token_tiles, compute_units, std::min(8, limit)) + token_tiles;
         return plan;
+    }
+    if (n > 32 && n <= 64 && streamable && enough_rows) {
+        // 33 to 64 tokens on a projection whose 16-row tiles come to about one workgroup of five or six per
+        // compute unit: the streaming kernel again, with three token tiles up to 48 tokens, four above
+        // ([18432, 7168] in 231 workgroups of 80 rows: 27.0 / 28.2 / 32.2 us at 33 / 48 / 64 tokens against
+        // 30.6 / 31.5 / 33.6 on the tiles with K divided; with fewer rows per workgroup, or a number of
+        // workgroups just above the compute units, the tiles stay ahead: [7168, 18432] 32 against 46 to 63)
+        const int token_tiles = n <= 48 ? 3 : 4;
+        const int row_tiles = ceil_div(ceil_div(m, 16), compute_units);
+        const int workgroups = ceil_div(ceil_div(m, 16), row_tiles);
+        if (row_tiles >= 5 && row_tiles * token_tiles <= 20 && row_tiles + token_tiles <= 10 &&
+            workgroups * 100 >= compute_units * 85) {
+            plan.family = FAMILY_FP8_STREAM;
+            plan.kernel = 10 * row_tiles + token_tiles;
+            return plan;
+        }
     }
     if (n <= 8) {
         // a handful of tokens: small tiles with split-K put the most workgroups on the weight stream

@@ -119,8 +119,11 @@ def test_planner_choices_for_the_baseline_shapes():
     assert describe(3, "T", "N", 2048, 1, 7168, 7168, 7168, 2048)[0] // 1000 == 3
     code, text = describe(3, "T", "N", 18432, 16, 7168, 7168, 7168, 18432)
     assert code // 1000 == 7 and "stream rows=80 tokens=16" in text
-    # 33 to 64 tokens: tiles with divided K when K is long enough to divide, else the streaming kernel
-    assert "split_k=3" in describe(3, "T", "N", 18432, 64, 7168, 7168, 7168, 18432)[1]
+    # 33 to 64 tokens: the streaming kernel where its workgroups of five or six row tiles come to about one per
+    # compute unit; otherwise tiles with divided K when K is long enough to divide, else the streaming kernel
+    assert "stream rows=80 tokens=48" in describe(3, "T", "N", 18432, 33, 7168, 7168, 7168, 18432)[1]
+    assert "stream rows=80 tokens=64" in describe(3, "T", "N", 18432, 64, 7168, 7168, 7168, 18432)[1]
+    assert "split_k=6" in describe(3, "T", "N", 7168, 64, 18432, 18432, 18432, 7168)[1]
     assert "tokens=64" in describe(3, "T", "N", 7168, 64, 2048, 2048, 2048, 7168)[1]
     # the streaming kernel holds K / 128 scales per token in LDS: K beyond 24576 goes to the tiles
     assert "stream" not in describe(3, "T", "N", 7168, 16, 32768, 32768, 32768, 7168)[1]

@@ -57,8 +57,8 @@ def test_random_blocks_every_variant(device, variant, split, rows):
 
 
 # 100 + 10*row_tiles + token_tiles: the weight-streaming decode kernel
-FP8_STREAM_CODES = [100 + 10 * rows + tokens for rows in range(1, 9) for tokens in (1, 2, 4)
-                    if rows * tokens <= 16 and rows + tokens <= 10]
+FP8_STREAM_CODES = [100 + 10 * rows + tokens for rows in range(1, 9) for tokens in (1, 2, 3, 4)
+                    if rows * tokens <= 20 and rows + tokens <= 10]
 
 
 @pytest.mark.parametrize("code", FP8_STREAM_CODES)
