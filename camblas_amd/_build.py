@@ -35,6 +35,7 @@ CORE_SOURCES = (
     "bgemv_stream_norm.hip",
     "bgemv_stream_residual.hip",
     "bgemv_stream_gated.hip",
+    "bgemv_stream_many.hip",
     "bgemm_dma.hip",
     "bgemm_wave4.hip",
     "bgemm_nn.hip",

@@ -113,6 +113,10 @@ hipError_t launch_bgemv_stream(hipStream_t stream, int depth_log2, int row_tiles
         return admitted;
     if (fusion.norm_weight && fusion.residual)
         return hipErrorInvalidValue; // one half per launch: no linear of a decoder layer needs both
+    if (token_tiles > 4)
+        return fusion.norm_weight || fusion.residual || depth_log2 != 0
+                   ? hipErrorInvalidValue
+                   : stream_many_tokens(stream, row_tiles, token_tiles, p, shares.count);
     if (fusion.norm_weight) // (the fused forms exist for K steps of one or two blocks)
         return stream_normalising(stream, depth_log2, row_tiles, token_tiles, p, shares.count);
     if (fusion.residual)

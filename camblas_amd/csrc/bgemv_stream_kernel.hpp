@@ -18,7 +18,8 @@
 // This header holds the kernel and its launch templates; the instantiations are spread over several
 // translation units that compile side by side (bgemv_stream.hip: one K block per step;
 // bgemv_stream_deep.hip: two to eight; bgemv_stream_norm.hip and bgemv_stream_residual.hip: the fused
-// halves; bgemv_stream_gated.hip: the gated form), each behind one of the functions declared at the end.
+// halves; bgemv_stream_gated.hip: the gated form; bgemv_stream_many.hip: more than four token tiles), each
+// behind one of the functions declared at the end.
 #pragma once
 #include "common.hpp"
 #include "device.hpp"
@@ -59,6 +60,8 @@ struct StreamParams {
 namespace
 {
 constexpr int WAVES = 4, DEPTH = 2;
+// passes in which the wavefronts' partial tiles (1 KB each) go through LDS at the end of a workgroup
+constexpr int stream_combine_passes(int row_tiles, int token_tiles) { return WAVES * row_tiles * token_tiles > 144 ? 2 : 1; }
 
 typedef float f32x2_round_t __attribute__((ext_vector_type(2)));
 typedef __bf16 bf16x2_round_t __attribute__((ext_vector_type(2)));
@@ -322,23 +325,29 @@ __global__ __launch_bounds__(WAVES * 64) void bgemv_stream_kernel(StreamParams p
     }
 
     // ---- combine the K partitions of the wavefronts: each parks its partial sums in a region of
-    // its own, and after one barrier tile t is summed in wavefront order 0, 1, 2, 3 by wavefront t % 4
-    __syncthreads();
+    // its own, and after one barrier tile t is summed in wavefront order 0, 1, 2, 3 by wavefront t % 4.
+    // The sums of more than 36 tiles do not fit the LDS at once: they go in two passes of half the tiles.
     // (the launcher sizes the dynamic LDS for the larger of the two uses)
+    constexpr int PASSES = stream_combine_passes(NT, MT), PASS_TILES = (NT * MT + PASSES - 1) / PASSES;
+    static_assert(PASSES == 1 || (!GATED && FUSE == 0), "passes of the plain form");
     f32x4_t *combine = reinterpret_cast<f32x4_t *>(lds_bytes);
+    auto park = [&](int pass) {
+        __syncthreads(); // (every wavefront is done with the stages, or with the previous pass)
 #pragma unroll
-    for (int i = 0; i < NT; ++i)
+        for (int i = 0; i < NT; ++i)
 #pragma unroll
-        for (int j = 0; j < MT; ++j)
-            combine[((wave * NT + i) * MT + j) * 64 + lane] = acc[i][j];
-    __syncthreads();
+            for (int j = 0; j < MT; ++j)
+                if ((i * MT + j) / PASS_TILES == pass)
+                    combine[(wave * PASS_TILES + (i * MT + j) % PASS_TILES) * 64 + lane] = acc[i][j];
+        __syncthreads();
+    };
     // ---- epilogue: wavefront w writes tiles w, w+4, ...; register r of lane l is feature
     // 4*(l/16) + r and token l%16 inside the 16x16 tile
-    auto summed = [&](int index) {
-        f32x4_t sum = combine[index * 64 + lane];
+    auto summed = [&](int index) { // (of the pass that is parked)
+        f32x4_t sum = combine[(index % PASS_TILES) * 64 + lane];
 #pragma unroll
         for (int w = 1; w < WAVES; ++w)
-            sum = sum + combine[(w * NT * MT + index) * 64 + lane];
+            sum = sum + combine[(w * PASS_TILES + index % PASS_TILES) * 64 + lane];
         return sum;
     };
     // ---- K divided over several workgroups: every workgroup parks its sums in its own FP32 plane;
@@ -354,11 +363,15 @@ __global__ __launch_bounds__(WAVES * 64) void bgemv_stream_kernel(StreamParams p
     if (divided) {
         const __amdgpu_buffer_rsrc_t mine = make_resource(group + blockIdx.z * plane_bytes, GROUP_BYTES);
 #pragma unroll
-        for (int index = 0; index < HALF * MT; ++index) {
-            if (index % WAVES != wave)
-                continue;
-            const f32x4_t sum = summed(index);
-            store_device_scope(mine, unsigned(index) * TILE_BYTES + unsigned(lane) * 16, sum);
+        for (int pass = 0; pass < PASSES; ++pass) {
+            park(pass);
+#pragma unroll
+            for (int index = pass * PASS_TILES; index < (pass + 1) * PASS_TILES && index < NT * MT; ++index) {
+                if (index % WAVES != wave)
+                    continue;
+                const f32x4_t sum = summed(index);
+                store_device_scope(mine, unsigned(index) * TILE_BYTES + unsigned(lane) * 16, sum);
+            }
         }
         // The planes are written and read with device-scope accesses, which go to the point where
         // all XCDs agree instead of staying in one XCD's L2, so no cache has to be written back or
@@ -389,7 +402,11 @@ __global__ __launch_bounds__(WAVES * 64) void bgemv_stream_kernel(StreamParams p
     // the region the wavefronts' sums were parked in, which the launcher sizes for)
     float *square_table = reinterpret_cast<float *>(lds_bytes + size_t(WAVES) * NT * MT * 64 * 16);
 #pragma unroll
-    for (int index = 0; index < HALF * MT; ++index) {
+    for (int pass = 0; pass < PASSES; ++pass) {
+    if (!divided) // (a divided product parked its sums above and reads the planes here)
+        park(pass);
+#pragma unroll
+    for (int index = pass * PASS_TILES; index < (pass + 1) * PASS_TILES && index < HALF * MT; ++index) {
         if (index % WAVES != wave)
             continue;
         const int i = index / MT, j = index % MT;
@@ -479,6 +496,7 @@ __global__ __launch_bounds__(WAVES * 64) void bgemv_stream_kernel(StreamParams p
             }
         }
     }
+    } // passes
     if constexpr (RESIDUAL) {
         {
             // one thread per token adds the table's entries of that token in a fixed order: feature
@@ -502,11 +520,11 @@ hipError_t launch_one(hipStream_t stream, const StreamParams &p, int shares = 1)
 {
     constexpr size_t stage_bytes = size_t(2) * KT * (NT + MT) * 16 * (64 * WAVES);
     // partial sums at the end (residual epilogue: and the table of squares behind them)
-    constexpr size_t parked_bytes =
-        size_t(WAVES) * NT * MT * 64 * 16 + (FUSE == 2 && !GATED ? size_t(NT) * MT * 64 * 4 : 0);
+    constexpr size_t parked_bytes = size_t(WAVES) * ((NT * MT + stream_combine_passes(NT, MT) - 1) / stream_combine_passes(NT, MT)) * 64 * 16 +
+                                    (FUSE == 2 && !GATED ? size_t(NT) * MT * 64 * 4 : 0);
     constexpr size_t lds_bytes = stage_bytes > parked_bytes ? stage_bytes : parked_bytes;
     // combined limits: the tiles in flight fit the register file, a stage pair fits the LDS
-    if constexpr (NT * KT > 8 || lds_bytes > 128 * 1024) {
+    if constexpr (NT * KT > 8 || lds_bytes > 160 * 1024) {
         return hipErrorInvalidValue;
     } else {
         // whole K steps and a workgroup's weight rows within one 4 GB descriptor: the variant without
@@ -569,4 +587,6 @@ hipError_t stream_plain_deep(hipStream_t stream, int depth_log2, int row_tiles, 
 hipError_t stream_normalising(hipStream_t stream, int depth_log2, int row_tiles, int token_tiles, const StreamParams &p, int shares);
 hipError_t stream_residual(hipStream_t stream, int depth_log2, int row_tiles, int token_tiles, const StreamParams &p, int shares);
 hipError_t stream_gated(hipStream_t stream, int pair_tiles, int token_tiles, bool normalising, const StreamParams &p);
+// five to eight token tiles (65 to 128 tokens): the plain form with one K block per step
+hipError_t stream_many_tokens(hipStream_t stream, int row_tiles, int token_tiles, const StreamParams &p, int shares);
 } // namespace camblas_hip

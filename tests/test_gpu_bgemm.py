@@ -78,6 +78,9 @@ STREAM_CODES = [
     for depth in (0, 1, 2, 3) for rows in range(1, 9) for tokens in (1, 2, 3, 4)
     if (rows << depth) <= 8 and ((rows + tokens) << depth) <= 16
 ]
+# five to eight token tiles (65 to 128 tokens): one K block per step; from 37 tiles on the wavefronts' partial
+# tiles are combined in two passes (an odd number of tiles, 7 x 7, included)
+MANY_TOKEN_CODES = [100 + 10 * rows + tokens for rows in range(1, 9) for tokens in (5, 6, 7, 8)]
 
 
 @pytest.mark.parametrize("code", STREAM_CODES)
@@ -96,6 +99,25 @@ def test_streaming_kernel_every_variant(device, code, n_out, m_rows, pad, k):
     for alpha, beta in ((1.0, 0.0), (0.5, -1.5)):
         got = run_bgemm(device, "T", "N", n_out, m_rows, k, alpha, w, lda, x, ldb, beta, c0, ldc,
                         override=(code, 1))
+        want, want64 = reference("T", "N", n_out, m_rows, k, alpha, w, lda, x, ldb, beta, c0, ldc)
+        got2d = got.reshape(m_rows, ldc)
+        error = rel_frobenius(oracle.bf16_to_f32(got2d[:, :n_out]), want64.reshape(m_rows, n_out))
+        assert error <= TOLERANCE, (code, alpha, beta, error)
+        assert np.array_equal(got2d[:, n_out:], c0.reshape(m_rows, ldc)[:, n_out:])
+
+
+@pytest.mark.parametrize("code", MANY_TOKEN_CODES)
+@pytest.mark.parametrize("n_out,m_rows,k,shares", [(300, 120, 328, 1), (301, 65, 640, 1), (264, 128, 1024, 2)])
+def test_streaming_kernel_with_many_token_tiles(device, code, n_out, m_rows, k, shares):
+    # ragged feature counts, token counts that fill, underfill and (120 tokens in a tile of 80) span the
+    # token tiles, K with and without a tail, K divided over two workgroups
+    lda, ldb, ldc = k + 8, k + 16, n_out + 4
+    w = oracle.fill_normal_bf16(620 + code, (n_out * lda,))
+    x = oracle.fill_normal_bf16(640 + code, (m_rows * ldb,))
+    c0 = oracle.fill_normal_bf16(660, (m_rows * ldc,))
+    for alpha, beta in ((1.0, 0.0), (0.5, -1.5)):
+        got = run_bgemm(device, "T", "N", n_out, m_rows, k, alpha, w, lda, x, ldb, beta, c0, ldc,
+                        override=(code, shares))
         want, want64 = reference("T", "N", n_out, m_rows, k, alpha, w, lda, x, ldb, beta, c0, ldc)
         got2d = got.reshape(m_rows, ldc)
         error = rel_frobenius(oracle.bf16_to_f32(got2d[:, :n_out]), want64.reshape(m_rows, n_out))
