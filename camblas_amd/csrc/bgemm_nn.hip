@@ -5,13 +5,17 @@
 // The matrix instruction wants, per lane, eight consecutive K values of one output column, which in
 // this layout lie a whole row of W apart. A workgroup of four wavefronts owns 128 outputs for up to
 // 256 tokens and streams W once: each step copies 64 rows x 128 outputs (256-byte pieces of rows:
-// whole cache lines) straight into LDS as they lie, and a lane gathers its eight values with eight
-// 2-byte LDS reads whose addresses differ by constants. Four rows of the tile are one 1 KB
-// direct-to-LDS load; successive loads are placed 1056 bytes apart, so that the two halves of a
-// wavefront (rows r and r + 8 of the same columns) read from different banks. The tokens go through
-// LDS as in the linear-layer kernels (128-byte rows, 16-byte chunks XOR-swizzled). At decode sizes
-// the kernel is bound by the W stream, and the eight-fold LDS reads stay below what a compute unit's
-// share of that stream needs.
+// whole cache lines) straight into LDS, and a lane gathers its eight K values of one output with two
+// transposing LDS reads (ds_read_b64_tr_b16: within sixteen lanes, lane 4a + b receives element b of
+// the four 8-byte values at the addresses of lanes a, 4 + a, 8 + a, 12 + a; so lane s points at row
+// s / 4 of four consecutive rows, outputs 4 (s % 4) .. + 3, and receives four K values of output s). A
+// 1 KB direct-to-LDS load (a piece) brings rows j, j + 16, j + 32 and j + 48 of the step, 256 contiguous
+// bytes of each, and successive pieces are placed 1056 bytes apart: four consecutive rows lie in four
+// pieces, 32 bytes of bank offset apart, so the sixteen lanes of a transposing read touch sixteen
+// different 8-byte bank pairs. The
+// tokens go through LDS as in the linear-layer kernels (128-byte rows, 16-byte chunks XOR-swizzled).
+// At decode sizes the kernel is bound by the W stream. (Eight 2-byte reads per fragment, which these
+// two replace, were a third of a step's LDS time: [8192, 8192] x 16 tokens 31.7 us.)
 // K can be divided over gridDim.y workgroups per tile (few outputs): FP32 planes, summed in share
 // order by the same kernel that serves the linear-layer tiles.
 // Needs K % 64 == 0, N % 4 == 0, lda % 8 == 0, ldb % 8 == 0, ldc % 4 == 0, 16-byte aligned W and x, an
@@ -36,6 +40,16 @@ struct NnParams {
     int share_steps;
 };
 
+typedef short i16x4_t __attribute__((ext_vector_type(4)));
+typedef short i16x8_t __attribute__((ext_vector_type(8)));
+// ds_read_b64_tr_b16 at a byte address inside a __shared__ array
+__device__ __forceinline__ i16x4_t read_transposed(const unsigned char *address)
+{
+    // (a pointer-to-pointer cast: through an integer the compiler would lose which LDS object is read and make
+    // the read wait for every direct-to-LDS load in flight)
+    return __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) i16x4_t *)(address));
+}
+
 constexpr int NN_BN = 128, NN_BK = 64, NN_STAGES = 3;
 constexpr int NN_PIECE = 66;                      // 16-byte slots from one 4-row piece of W to the next (1 KB + 32 B)
 constexpr int NN_W_SLOTS = (NN_BK / 4) * NN_PIECE; // per stage
@@ -57,14 +71,14 @@ template <int TM> __global__ __launch_bounds__(256) void bgemm_nn_kernel(NnParam
     const int first_step = int(blockIdx.y) * p.share_steps;
     const int steps = steps_all - first_step < p.share_steps ? steps_all - first_step : p.share_steps;
 
-    // ---- fills. W piece q of a stage (rows 4q .. 4q+3 of the step) is loaded by wavefront q % 4:
-    // lane l brings the 16 bytes at row l / 16, outputs 8 * (l % 16) .. + 7. Rows past K and outputs
+    // ---- fills. W piece j of a stage (rows j, j + 16, j + 32, j + 48 of the step) is loaded by wavefront
+    // j % 4: lane l brings the 16 bytes at row j + 16 * (l / 16), outputs 8 * (l % 16) .. + 7. Rows past K and outputs
     // past the end of the last row lie outside the buffer resource and read as zero; outputs past N
     // inside a row are whatever lies there and only reach accumulators that are never stored.
     const __amdgpu_buffer_rsrc_t w_resource =
         make_resource(p.w + n0, (unsigned(p.k - 1) * unsigned(p.lda) + unsigned(p.n - n0)) * 2u);
-    const unsigned w_lane_off = (unsigned(wave * 4 + lane / 16) * unsigned(p.lda) + unsigned(lane % 16) * 8u) * 2u;
-    const unsigned w_piece_step = unsigned(WAVES * 4) * unsigned(p.lda) * 2u; // successive pieces of a wavefront
+    const unsigned w_lane_off = (unsigned(wave + 16 * (lane / 16)) * unsigned(p.lda) + unsigned(lane % 16) * 8u) * 2u;
+    const unsigned w_piece_step = unsigned(WAVES) * unsigned(p.lda) * 2u; // successive pieces of a wavefront
     const unsigned w_k_step = unsigned(NN_BK) * unsigned(p.lda) * 2u;
     // token rows: eight 128-byte rows per load, lane l row l / 8, the chunk that belongs in its slot
     const int x_rows = p.m - m0 < BM ? p.m - m0 : BM;
@@ -93,7 +107,11 @@ template <int TM> __global__ __launch_bounds__(256) void bgemm_nn_kernel(NnParam
     // ---- operand reads. Output column of this lane: 32 * wave + lane % 32; lane half h = lane / 32
     // holds K values 8h .. 8h+7 of every 16-deep sub-step.
     const int column = lane % 32, half = lane / 32;
-    const int w_lane_bytes = half * 2 * NN_PIECE * 16 + (wave * 32 + column) * 2;
+    // the transposing reads: for the sub-step's rows 8 h .. 8 h + 3 this lane points at row 8 h + (lane % 16) / 4
+    // (piece of that number; 256 bytes further per 16-deep sub-step) and at four outputs from `pointed` on;
+    // the value it receives is of output `column`. Rows 8 h + 4 .. lie four pieces on.
+    const int pointed = wave * 32 + (lane / 16 % 2) * 16 + 4 * (lane % 4);
+    const int w_lane_bytes = (half * 8 + (lane % 16) / 4) * NN_PIECE * 16 + pointed * 2;
     const int x_swizzle = lds_swizzle<8>(column);
     f32x16_t acc[TM];
 #pragma unroll
@@ -106,18 +124,10 @@ template <int TM> __global__ __launch_bounds__(256) void bgemm_nn_kernel(NnParam
         const unsigned char *bytes = reinterpret_cast<const unsigned char *>(stage) + w_lane_bytes;
 #pragma unroll
         for (int ks = 0; ks < NN_BK / 16; ++ks) {
-            unsigned packed[4];
-#pragma unroll
-            for (int pair = 0; pair < 4; ++pair) {
-                // rows 16 ks + 8 h + 2 pair and the next one: piece (row / 4), row (row % 4) inside it
-                const int lo = 2 * pair, hi = 2 * pair + 1;
-                const unsigned short a =
-                    *reinterpret_cast<const unsigned short *>(bytes + (ks * 4 + lo / 4) * NN_PIECE * 16 + (lo % 4) * 256);
-                const unsigned short b =
-                    *reinterpret_cast<const unsigned short *>(bytes + (ks * 4 + hi / 4) * NN_PIECE * 16 + (hi % 4) * 256);
-                packed[pair] = unsigned(a) | (unsigned(b) << 16);
-            }
-            const bf16x8_t w_frag = __builtin_bit_cast(bf16x8_t, u32x4_t{packed[0], packed[1], packed[2], packed[3]});
+            const i16x4_t lower = read_transposed(bytes + ks * 256);
+            const i16x4_t upper = read_transposed(bytes + ks * 256 + 4 * NN_PIECE * 16);
+            const bf16x8_t w_frag = __builtin_bit_cast(bf16x8_t, i16x8_t{lower[0], lower[1], lower[2], lower[3],
+                                                                        upper[0], upper[1], upper[2], upper[3]});
 #pragma unroll
             for (int j = 0; j < TM; ++j) {
                 const bf16x8_t x_frag = __builtin_bit_cast(
