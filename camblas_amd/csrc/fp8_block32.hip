@@ -45,7 +45,6 @@ constexpr int UNIT = 0x7f7f7f7f; // E8M0 exponent 127 = scale 1.0 in every byte
 template <bool QUANTISE, bool EXACT, int WAVES>
 __global__ __launch_bounds__(WAVES * 64) void fp8_block32_decode_kernel(Block32Params p)
 {
-    static_assert(!QUANTISE || WAVES == 4, "the quantiser takes one 32-value block per thread");
     // x and its scales, zero-padded to a whole number of DEPTH-step rounds
     __shared__ __attribute__((aligned(16))) unsigned x_words[MAX_K / 4];
     __shared__ __attribute__((aligned(16))) float x_scale[MAX_K / 32];
@@ -96,13 +95,17 @@ __global__ __launch_bounds__(WAVES * 64) void fp8_block32_decode_kernel(Block32P
     // loads in flight instead of waiting for all of them.
     constexpr int WORDS_PER_THREAD = MAX_K / 4 / (WAVES * 64), BLOCKS_PER_THREAD = MAX_K / 32 / (WAVES * 64);
     const unsigned *source = static_cast<const unsigned *>(p.x);
-    unsigned staged[QUANTISE ? 16 : WORDS_PER_THREAD];
+    unsigned staged[QUANTISE ? 16 * BLOCKS_PER_THREAD : WORDS_PER_THREAD];
     float staged_scale[BLOCKS_PER_THREAD] = {};
     if constexpr (QUANTISE) {
-        const int b = thread < blocks ? thread : blocks - 1; // BF16 pairs of block `thread`
 #pragma unroll
-        for (int e = 0; e < 16; ++e)
-            staged[e] = source[b * 16 + e];
+        for (int i = 0; i < BLOCKS_PER_THREAD; ++i) {
+            const int block = thread + i * WAVES * 64;
+            const int b = block < blocks ? block : blocks - 1; // BF16 pairs of a 32-value block
+#pragma unroll
+            for (int e = 0; e < 16; ++e)
+                staged[16 * i + e] = source[b * 16 + e];
+        }
     } else {
 #pragma unroll
         for (int i = 0; i < WORDS_PER_THREAD; ++i) {
@@ -133,14 +136,16 @@ __global__ __launch_bounds__(WAVES * 64) void fp8_block32_decode_kernel(Block32P
     for (int i = 0; i < SCALES_PER_LANE; ++i)
         w_scale[wave][lane + 64 * i] = staged_weight_scale[i];
     if constexpr (QUANTISE) {
-        const int b = thread;
+#pragma unroll
+        for (int i = 0; i < BLOCKS_PER_THREAD; ++i) {
+        const int b = thread + i * WAVES * 64;
         if (b < padded_steps * 4) {
             float value[32];
             float amax = 1e-10f;
             if (b < blocks) {
 #pragma unroll
                 for (int e = 0; e < 16; ++e) {
-                    const unsigned pair = staged[e];
+                    const unsigned pair = staged[16 * i + e];
                     value[2 * e] = __uint_as_float(pair << 16);
                     value[2 * e + 1] = __uint_as_float(pair & 0xffff0000u);
                     amax = fmaxf(amax, fmaxf(fabsf(value[2 * e]), fabsf(value[2 * e + 1])));
@@ -167,6 +172,7 @@ __global__ __launch_bounds__(WAVES * 64) void fp8_block32_decode_kernel(Block32P
                     x_words[b * 8 + word] = 0u;
             }
         }
+        } // blocks of this thread
     } else {
 #pragma unroll
         for (int i = 0; i < WORDS_PER_THREAD; ++i) {
@@ -281,19 +287,24 @@ hipError_t launch_fp8_block32_decode(hipStream_t stream, int outputs, int inner,
     p.sw_col = sw_col;
     const bool exact = inner % STEP == 0; // (16 rows of at most 8192 bytes fit any descriptor)
     const auto grid_of = [outputs](int waves) { return unsigned((outputs + waves * 16 - 1) / (waves * 16)); };
-    if (!sx) {
-        (exact ? fp8_block32_decode_kernel<true, true, 4> : fp8_block32_decode_kernel<true, false, 4>)<<<grid_of(4), 256, 0, stream>>>(p);
-        return launch_status();
-    }
     // (one wavefront per workgroup spreads the wavefronts evenly over the compute units: [18432, 7168] 25.1 us
     // against 29.9 with four, [4096, 7168] 13.6 against 16.2; the others are kept for tests)
-    const int waves = forced_waves ? forced_waves : 1;
-    switch (waves) {
-    case 1: (exact ? fp8_block32_decode_kernel<false, true, 1> : fp8_block32_decode_kernel<false, false, 1>)<<<grid_of(1), 64, 0, stream>>>(p); break;
-    case 2: (exact ? fp8_block32_decode_kernel<false, true, 2> : fp8_block32_decode_kernel<false, false, 2>)<<<grid_of(2), 128, 0, stream>>>(p); break;
-    case 4: (exact ? fp8_block32_decode_kernel<false, true, 4> : fp8_block32_decode_kernel<false, false, 4>)<<<grid_of(4), 256, 0, stream>>>(p); break;
+    // (the quantising form keeps four: every workgroup quantises the whole token first, and with one
+    // wavefront that takes four times as long: [18432, 7168] 28.6 us with four, 29.2 with one)
+    const int waves = forced_waves ? forced_waves : sx ? 1 : 4;
+#define CAMBLAS_BLOCK32(QUANTISE, WAVES) \
+    (exact ? fp8_block32_decode_kernel<QUANTISE, true, WAVES> : fp8_block32_decode_kernel<QUANTISE, false, WAVES>) \
+        <<<grid_of(WAVES), WAVES * 64, 0, stream>>>(p)
+    switch (waves * 2 + (sx ? 0 : 1)) {
+    case 2: CAMBLAS_BLOCK32(false, 1); break;
+    case 3: CAMBLAS_BLOCK32(true, 1); break;
+    case 4: CAMBLAS_BLOCK32(false, 2); break;
+    case 5: CAMBLAS_BLOCK32(true, 2); break;
+    case 8: CAMBLAS_BLOCK32(false, 4); break;
+    case 9: CAMBLAS_BLOCK32(true, 4); break;
     default: return hipErrorInvalidValue;
     }
+#undef CAMBLAS_BLOCK32
     return launch_status();
 }
 } // namespace camblas_hip

@@ -327,6 +327,16 @@ def test_block32_decode_matches_ordered_oracle(device, outputs, inner):
         finally:
             native.call("hip_set_plan_override", -1, 0)
         assert torch.equal(forced.view(torch.int16), out.view(torch.int16)), code
+    # the quantising form (BF16 token in, four wavefronts per workgroup planned) likewise
+    token = torch.from_numpy(oracle.bf16_to_f32(oracle.fill_normal_bf16(77, (inner,)))).to(device).to(torch.bfloat16).view(1, -1)
+    planned = _kernels.fp8_linear(token, fp8_tensor(w, device), torch.from_numpy(sw).to(device))
+    for code in (301, 302):
+        native.call("hip_set_plan_override", code, 0)
+        try:
+            forced = _kernels.fp8_linear(token, fp8_tensor(w, device), torch.from_numpy(sw).to(device))
+        finally:
+            native.call("hip_set_plan_override", -1, 0)
+        assert torch.equal(forced.view(torch.int16), planned.view(torch.int16)), code
 
 
 def test_block32_known_answers_graph_and_nan(device):
