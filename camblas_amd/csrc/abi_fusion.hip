@@ -197,7 +197,7 @@ extern "C" int camblas_cuda_bf16_gated_linear(camblas_cuda_context *context, int
             return 0;
         if (!usable({{x, 16}, {gate, 16}, {up, 16}, {out, 2}}) || !apart(out, {x, gate, up}))
             return entry.refuse("invalid gated linear buffers");
-        const int token_tiles = rows <= 16 ? 1 : rows <= 32 ? 2 : 4;
+        const int token_tiles = rows <= 16 ? 1 : rows <= 32 ? 2 : rows <= 48 ? 3 : 4;
         // the widest workgroups that still leave one and a half per compute unit (or a test's choice)
         int pair_tiles = 4;
         while (pair_tiles > 1 && (outputs + 16 * pair_tiles - 1) / (16 * pair_tiles) * 2 < 3 * context->compute_units)

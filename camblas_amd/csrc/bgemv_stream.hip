@@ -42,7 +42,7 @@ size_t stream_partial_bytes(int row_tiles, int token_tiles, int n_out, int m_row
 
 // Gated form: out[m, n] = round(round(silu(g)) * u) with g = round(x Wg^T), u = round(x Wu^T); a
 // workgroup owns 16 * pair_tiles output rows (that many gate rows and the same up rows) over the
-// whole K. pair_tiles 1..4, token_tiles 1, 2 or 4.
+// whole K. pair_tiles 1..4, token_tiles 1 to 4 (three: without the fused normalisation only).
 hipError_t launch_gated_stream(hipStream_t stream, int pair_tiles, int token_tiles, int n_out, int m_rows,
                                int k, const void *gate, const void *up, int lda, const void *x, int ldb,
                                void *y, int ldc, const StreamFusion &fusion)

@@ -17,6 +17,11 @@ hipError_t stream_gated(hipStream_t stream, int pair_tiles, int token_tiles, boo
     case 22: CAMBLAS_GATED(4, 2);
     case 23: CAMBLAS_GATED(6, 2);
     case 24: CAMBLAS_GATED(8, 2);
+    // (33 to 48 tokens; the form with the normalisation keeps to one, two and four token tiles)
+    case 31: return fused ? hipErrorInvalidValue : launch_one<2, 3, 1, true, 0>(stream, p);
+    case 32: return fused ? hipErrorInvalidValue : launch_one<4, 3, 1, true, 0>(stream, p);
+    case 33: return fused ? hipErrorInvalidValue : launch_one<6, 3, 1, true, 0>(stream, p);
+    case 34: return fused ? hipErrorInvalidValue : launch_one<8, 3, 1, true, 0>(stream, p);
     case 41: CAMBLAS_GATED(2, 4);
     case 42: CAMBLAS_GATED(4, 4);
     case 43: CAMBLAS_GATED(6, 4);

@@ -245,7 +245,9 @@ def test_rope_kv_append_equals_rope_then_append(device):
 
 
 @pytest.mark.parametrize("rows,outputs,inner,pairs", [(1, 100, 256, None), (7, 130, 264, 1), (32, 300, 512, 2),
-                                                        (33, 70, 136, 3), (64, 257, 1024, 4), (32, 1024, 2048, None)])
+                                                        (33, 70, 136, 3), (64, 257, 1024, 4), (32, 1024, 2048, None),
+                                                        (40, 130, 264, 1), (48, 300, 512, 2), (47, 257, 1024, 4),
+                                                        (48, 1024, 2048, None)])
 def test_gated_linear_equals_the_three_call_composition(device, rows, outputs, inner, pairs):
     # one pass over both weight matrices against linear, linear, silu_multiply: the rounding points
     # are the same and only the order of the FP32 sums inside a product may differ (the planner is
