@@ -25,7 +25,7 @@ def bf16_linear(x_bits, w_bits):
     return oracle.f32_to_bf16(oracle.linear_bf16_f64(x_bits, w_bits).astype(np.float32))
 
 
-def make_inputs(seed):
+def make_inputs(seed, batch=BATCH):
     weights = {
         "input_norm": oracle.fill_normal_bf16(seed + 1, (HIDDEN,), mean=1.0, std=0.02),
         "post_norm": oracle.fill_normal_bf16(seed + 2, (HIDDEN,), mean=1.0, std=0.02),
@@ -35,11 +35,13 @@ def make_inputs(seed):
         "up": oracle.fill_normal_bf16(seed + 6, (FFN, HIDDEN), std=0.03),
         "down": oracle.fill_normal_bf16(seed + 7, (HIDDEN, FFN), std=0.03),
     }
-    hidden = oracle.fill_normal_bf16(seed + 8, (BATCH, HIDDEN))
-    residual = oracle.fill_normal_bf16(seed + 9, (BATCH, HIDDEN))
-    k_cache = oracle.fill_normal_bf16(seed + 10, (BATCH, CONTEXT, KV_HEADS, DIM))
-    v_cache = oracle.fill_normal_bf16(seed + 11, (BATCH, CONTEXT, KV_HEADS, DIM))
+    hidden = oracle.fill_normal_bf16(seed + 8, (batch, HIDDEN))
+    residual = oracle.fill_normal_bf16(seed + 9, (batch, HIDDEN))
+    k_cache = oracle.fill_normal_bf16(seed + 10, (batch, CONTEXT, KV_HEADS, DIM))
+    v_cache = oracle.fill_normal_bf16(seed + 11, (batch, CONTEXT, KV_HEADS, DIM))
     positions = np.array([CONTEXT - 1, 0, 17, 256], np.int32)
+    if batch != BATCH:
+        positions = np.random.default_rng(seed).integers(0, CONTEXT, batch).astype(np.int32)
     return weights, hidden, residual, k_cache, v_cache, positions
 
 
@@ -77,16 +79,18 @@ def device_layer(device, weights, hidden, residual, k_cache, v_cache, positions)
     return out, res, kc, vc
 
 
-def test_layer_matches_oracle_pipeline(device):
-    inputs = make_inputs(3000)
+@pytest.mark.parametrize("batch", [BATCH, 17, 40, 64])
+def test_layer_matches_oracle_pipeline(device, batch):
+    # (the batches take the streaming linears with one to four token tiles, the gated launch included)
+    inputs = make_inputs(3000 + batch, batch)
     want_out, want_res, want_k, want_v = oracle_layer(*inputs)
     out, res, kc, vc = device_layer(device, *inputs)
     assert rel_frobenius(bf16_values(res), oracle.bf16_to_f32(want_res)) <= 1e-2
     assert rel_frobenius(bf16_values(out), oracle.bf16_to_f32(want_out)) <= 2e-2
     # the cache rows that were not appended are untouched; the appended V row is a pure copy of a
     # linear output and the K row a rotation of one
-    untouched = np.ones((BATCH, CONTEXT), bool)
-    untouched[np.arange(BATCH), inputs[5]] = False
+    untouched = np.ones((batch, CONTEXT), bool)
+    untouched[np.arange(batch), inputs[5]] = False
     assert np.array_equal(from_device_bf16(kc)[untouched], inputs[3][untouched])
     assert np.array_equal(from_device_bf16(vc)[untouched], inputs[4][untouched])
     assert rel_frobenius(bf16_values(vc), oracle.bf16_to_f32(want_v)) <= 1e-2
