@@ -79,7 +79,7 @@ def device_layer(device, weights, hidden, residual, k_cache, v_cache, positions)
     return out, res, kc, vc
 
 
-@pytest.mark.parametrize("batch", [BATCH, 17, 40, 64])
+@pytest.mark.parametrize("batch", [BATCH, 17, 40, 64, 80])
 def test_layer_matches_oracle_pipeline(device, batch):
     # (the batches take the streaming linears with one to four token tiles, the gated launch included)
     inputs = make_inputs(3000 + batch, batch)
