@@ -401,7 +401,8 @@ int camblas_hip_plan_describe(int dtype, int algorithm, char trans_a, char trans
  * E8M0 products: 0 the weight-streaming kernel, 20 / 21 / 22 / 23 the tiled kernel with
  * 256 x 256, 256 x 128, (E4M3 weights only) 192 x 256 and 128 x 128 tiles, 24 the four-wavefront
  * 192 x 256 tile (grouped calls: E4M3 weights only); a forced kernel that cannot run the call makes
- * the call fail. (BF16: 20 + n the
+ * the call fail. (BF16: 100 + 100 d + 10 r + t the weight-streaming kernel with 2^d K blocks per
+ * step, r row tiles and t token tiles of 16 (t up to 8, above 4 with d = 0 only); 20 + n the
  * direct-to-LDS tile n, of which 38 / 39 are the four-wavefront 256- and 320-row tiles and 40 the
  * 256-row tile for weights stored with their outputs contiguous; FP8 with FP32 scales: 36 the
  * four-wavefront 192 x 256 tile; the single-token product with 32-wide scale blocks: 301 / 302 / 304
